@@ -1,0 +1,215 @@
+"""Attention over paged KV, restated on the CPU. Test infrastructure only.
+
+Conventions: query head h reads KV head h // (HQ // HKV); a token at position p sees positions n <= p of its sequence
+(and, with a sliding window w, only n > p - w); softmax in the natural base over scores q.k * scale; a row that sees no
+position gives output 0 and log-sum-exp -inf.
+"""
+import math
+
+import torch
+
+from . import append
+
+
+# -- the float64 reference over stored values (test_paged_kv_attention.py:71-81) ---------------------------------------
+def reference(q, keys, values, seen, scale):
+    """q [HQ][D] float64 over keys [n][HKV][D], values [n][HKV][DV] where seen [n] (bool) -> (out [HQ][DV], lse [HQ]).
+    A head that sees nothing gets zeros and -inf."""
+    hq, hkv = q.shape[0], keys.shape[1]
+    group = hq // hkv
+    out, lse = [], []
+    neg = torch.tensor(float("-inf"), dtype=torch.float64)
+    for h in range(hq):
+        k, v = keys[:, h // group], values[:, h // group]
+        s = (k @ q[h]) * scale
+        s = torch.where(seen, s, neg)
+        if not bool(seen.any()):
+            out.append(torch.zeros(values.shape[-1], dtype=torch.float64))
+            lse.append(neg.clone())
+            continue
+        lse.append(torch.logsumexp(s, 0))
+        out.append(torch.softmax(s, 0) @ v)
+    return torch.stack(out), torch.stack(lse)
+
+
+def stored_rows(key_pages, value_pages, table, n, page, kind, key_scales=None, value_scales=None,
+                multipliers=(1.0, 1.0)):
+    """Positions 0..n-1 of the sequence with page table `table`, decoded to float64: keys [n][HKV][D], values
+    [n][HKV][DV] (test_paged_kv_attention.py:50-60)."""
+    hkv, d, dv = key_pages.shape[-2], key_pages.shape[-1], value_pages.shape[-1]
+    ids = append.slots(table, torch.arange(n), page)
+    k = key_pages.reshape(-1, hkv, d)[ids]
+    v = value_pages.reshape(-1, hkv, dv)[ids]
+    ks = key_scales.reshape(-1, hkv)[ids] if key_scales is not None else None
+    vs = value_scales.reshape(-1, hkv)[ids] if value_scales is not None else None
+    return (append.decode_rows(k, ks, kind, multipliers[0]), append.decode_rows(v, vs, kind, multipliers[1]))
+
+
+def window_reference(q, key_pages, value_pages, kind, table, first, count, page, scale, key_scales=None,
+                     value_scales=None, multipliers=(1.0, 1.0), sliding=0, q_dtype=torch.bfloat16):
+    """One window row in float64: q [count][HQ][D] (rounded to q_dtype first, as the kernels read it) at positions
+    first .. first + count - 1 -> (out [count][HQ][DV], lse [count][HQ])."""
+    n = first + count
+    keys, values = stored_rows(key_pages, value_pages, table, n, page, kind, key_scales, value_scales, multipliers)
+    qd = q.to(q_dtype).double()
+    positions = torch.arange(n)
+    outs, lses = [], []
+    for c in range(count):
+        seen = positions <= first + c
+        if sliding:
+            seen = seen & (positions > first + c - sliding)
+        o, l = reference(qd[c], keys, values, seen, scale)
+        outs.append(o)
+        lses.append(l)
+    return torch.stack(outs), torch.stack(lses)
+
+
+# -- the reference's CPU/torch path: gather, then SDPA (pages.py:455-477, device_attention.py:1148-1166) ---------------
+def gather(key_pages, value_pages, table, count, page, kind, compute, key_scales=None, value_scales=None,
+           multipliers=(1.0, 1.0)):
+    """A sequence's first `count` positions as contiguous rows in the compute dtype, dequantised (pages.py:455-477):
+    index_select of whole pages, reshape, cut."""
+    index = torch.as_tensor(table, dtype=torch.int64)[:math.ceil(count / page)]
+    n = index.numel() * page
+    hkv, d, dv = key_pages.shape[-2], key_pages.shape[-1], value_pages.shape[-1]
+    k = key_pages.index_select(0, index).reshape(n, hkv, d)[:count]
+    v = value_pages.index_select(0, index).reshape(n, hkv, dv)[:count]
+    if kind == "fp8":
+        return (k.float() * multipliers[0]).to(compute), (v.float() * multipliers[1]).to(compute)
+    if kind in append.ROW_SCALED:
+        ks = key_scales.index_select(0, index).reshape(n, hkv)[:count]
+        vs = value_scales.index_select(0, index).reshape(n, hkv)[:count]
+        return (k.float() * ks[..., None]).to(compute), (v.float() * vs[..., None]).to(compute)
+    return k.to(compute), v.to(compute)
+
+
+def sdpa_rows(queries, rows, gather_row, scale, out):
+    """The reference's CPU attention path (device_attention.py:1148-1166): per batch row (first token, count, first
+    position) gather its KV with gather_row(r, n) and run torch's scaled_dot_product_attention with GQA; one token sees
+    everything held, a chunk from position 0 is plain causal, a later chunk takes the offset mask."""
+    heads = queries.shape[1]
+    for r, (first, count, position) in enumerate(rows):
+        keys, values = gather_row(r, position + count)
+        q = queries[first:first + count].transpose(0, 1).unsqueeze(0).to(keys.dtype)
+        k, v = keys.transpose(0, 1).unsqueeze(0), values.transpose(0, 1).unsqueeze(0)
+        mask, causal = None, count > 1 and position == 0
+        if count > 1 and position > 0:
+            seen = torch.arange(position + count)
+            mask = seen[None, :] <= (position + torch.arange(count))[:, None]
+        found = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask, is_causal=causal,
+                                                                 scale=scale, enable_gqa=heads != keys.shape[1])
+        out[first:first + count] = found[0].transpose(0, 1).to(out.dtype)
+    return out
+
+
+def windows_dense(q, keys, values, position, scale, sliding=0, sinks=None):
+    """One row of tokens at positions position.. over its gathered keys [n][HKV][D] and values in FP32, causal
+    (device_attention.py:1301-1335 without trees and block lists) -> (out [count][HQ][DV] FP32, lse [count][HQ])."""
+    count, hq, d = q.shape
+    hkv = keys.shape[1]
+    g = hq // hkv
+    n = torch.arange(keys.shape[0])
+    seen = (n[None, :] <= (position + torch.arange(count))[:, None])
+    if sliding:
+        seen = seen & (n[None, :] > (position + torch.arange(count))[:, None] - sliding)
+    qq = q.float().view(count, hkv, g, d)
+    s = torch.einsum("ckgd,nkd->ckgn", qq, keys.float()) * scale
+    s = s.masked_fill(~seen[:, None, None, :], float("-inf"))
+    top = s.amax(-1)
+    if sinks is not None:
+        top = torch.maximum(top, sinks.view(1, hkv, g))
+    sub = torch.where(top == float("-inf"), 0.0, top)
+    p = torch.exp(s - sub[..., None])
+    total = p.sum(-1)
+    if sinks is not None:
+        total = total + torch.exp(sinks.view(1, hkv, g) - sub)
+    o = torch.einsum("ckgn,nkd->ckgd", p, values.float()) / total.clamp(min=1e-30)[..., None]
+    out = torch.where(total[..., None] > 0, o, 0.0).view(count, hq, -1)
+    lse = torch.where(total > 0, top + torch.log(total.clamp(min=1e-30)), float("-inf")).view(count, hq)
+    return out, lse
+
+
+# -- online softmax steps (kernels/core/python/crit_kcore/attention_softmax.py:37-101), natural base --------------------
+def step(s, m):
+    """One block of scores s [rows][positions] (masked ones -inf) against running maxima m [rows] -> (p, alpha,
+    m_new); a row that has seen nothing keeps -inf and gets p = 0, alpha = 0."""
+    m_new = torch.maximum(m, s.amax(dim=1))
+    m_sub = torch.where(m_new == float("-inf"), torch.zeros_like(m_new), m_new)
+    return torch.exp(s - m_sub[:, None]), torch.exp(m - m_sub), m_new
+
+
+def fold(m_run, l_run, m, l):
+    """A partial state (m, l) into the running one -> (m_new, l_new, keep, take): out = out * keep + partial * take."""
+    m_new = torch.maximum(m_run, m)
+    m_sub = torch.where(m_new == float("-inf"), torch.zeros_like(m_new), m_new)
+    keep, take = torch.exp(m_run - m_sub), torch.exp(m - m_sub)
+    return m_new, l_run * keep + l * take, keep, take
+
+
+def finish(acc, l):
+    """acc / l per row, 0 where l == 0."""
+    ok = l != 0
+    return torch.where(ok[:, None], acc / torch.where(ok, l, torch.ones_like(l))[:, None], torch.zeros_like(acc))
+
+
+def lse(m, l):
+    """m + log l, -inf where l == 0."""
+    return torch.where(l != 0, m + torch.log(torch.where(l != 0, l, torch.ones_like(l))), torch.full_like(m, -math.inf))
+
+
+# -- log-sum-exp merge across parts (inference/partitioned-attention/plugin.py:52-64) ------------------------------------
+def merge(outs, lses):
+    """Partials of the same queries over disjoint keys: outs [parts][T][HQ][DV], lses [parts][T][HQ] (-inf: the part
+    saw no key) -> (out FP32, lse FP32); a token no part saw gets zeros and -inf."""
+    outs, lses = torch.stack(list(outs)).float(), torch.stack(list(lses)).float()
+    top = lses.amax(0)
+    sub = torch.where(top == float("-inf"), 0.0, top)
+    weights = torch.where(lses == float("-inf"), 0.0, torch.exp(lses - sub))
+    total = weights.sum(0)
+    out = (weights[..., None] * outs).sum(0) / total.clamp(min=1e-30)[..., None]
+    out = torch.where(total[..., None] > 0, out, 0.0)
+    return out, torch.where(total > 0, sub + torch.log(total.clamp(min=1e-30)), float("-inf"))
+
+
+# -- the host technique (inference/partitioned-attention/code/implementation.py:22-138), Python floats -------------------
+def owner(position, world):
+    """The rank that owns a position: position mod world (implementation.py:34-35)."""
+    return position % world
+
+
+def global_position(local, world, rank):
+    """implementation.py:42-43."""
+    return local * world + rank
+
+
+def attention_partial(query, rows, value_width, query_position, scale=None):
+    """rows of (global position, key, value) one rank holds -> (output tuple, log normalizer); positions past the
+    query are masked; an empty shard gives zeros and -inf (implementation.py:71-116)."""
+    scale = 1 / math.sqrt(len(query)) if scale is None else scale
+    logits, values = [], []
+    for position, key, value in rows:
+        if position > query_position:
+            continue
+        logits.append(math.fsum(a * b for a, b in zip(query, key)) * scale)
+        values.append(value)
+    if not logits:
+        return (0.0,) * value_width, -math.inf
+    top = max(logits)
+    weights = [math.exp(x - top) for x in logits]
+    total = math.fsum(weights)
+    output = tuple(math.fsum((w / total) * row[c] for w, row in zip(weights, values)) for c in range(value_width))
+    return output, top + math.log(total)
+
+
+def merge_partials(partials):
+    """(output, log normalizer) pairs of disjoint shards -> the whole's; all-empty input raises
+    (implementation.py:119-138)."""
+    partials = list(partials)
+    top = max(l for _, l in partials)
+    if top == -math.inf:
+        raise ValueError("attention has no visible keys")
+    weights = [math.exp(l - top) for _, l in partials]
+    total = math.fsum(weights)
+    width = len(partials[0][0])
+    output = tuple(math.fsum((w / total) * o[c] for w, (o, _) in zip(weights, partials)) for c in range(width))
+    return output, top + math.log(total)

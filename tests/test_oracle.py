@@ -1,0 +1,358 @@
+"""Pins the CPU oracle before anything is checked against it: reference-held golden vectors, closed forms,
+library routines and brute force on tiny inputs. Runs without a GPU."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import append, attend, e4m3
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _vectors():
+    pairs = []
+    with open(os.path.join(GOLDEN, "e4m3_scale_vectors.txt"), encoding="utf-8") as f:
+        for line in f:
+            fields = line.split("#", 1)[0].split()
+            if fields:
+                pairs.append((int(fields[0], 16), int(fields[1], 16)))
+    return pairs
+
+
+# -- E4M3 ----------------------------------------------------------------------------------------------------------------
+def test_the_golden_file_holds_the_24_reference_vectors():
+    assert len(_vectors()) == 24
+
+
+def test_integer_encoder_reproduces_every_reference_vector():
+    bits = np.array([b for b, _ in _vectors()], dtype=np.uint32).view(np.float32)
+    want = np.array([c for _, c in _vectors()], dtype=np.uint8)
+    assert np.array_equal(e4m3.encode(bits), want)
+
+
+def test_torch_cast_with_the_clamp_reproduces_every_reference_vector_and_needs_the_clamp():
+    bits = torch.from_numpy(np.array([b for b, _ in _vectors()], dtype=np.uint32).view(np.float32).copy())
+    want = torch.tensor([c for _, c in _vectors()], dtype=torch.uint8)
+    got = bits.clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8)
+    assert torch.equal(got, want)
+    unclamped = bits.to(torch.float8_e4m3fn).view(torch.uint8)
+    assert not torch.equal(unclamped, want)        # 1e30 and +inf become NaN codes without it
+
+
+def test_decoder_matches_the_closed_form_on_every_code():
+    codes = np.arange(256, dtype=np.uint8)
+    got = e4m3.decode(codes)
+    for b in range(256):
+        mag = e4m3.magnitude(b)
+        if mag is None:
+            assert math.isnan(got[b])
+        else:
+            assert got[b] == (-mag if b & 0x80 else mag), b
+    assert e4m3.magnitude(0x7E) == 448.0 and e4m3.magnitude(0x08) == 2.0 ** -6 and e4m3.magnitude(0x01) == 2.0 ** -9
+
+
+def test_decoder_matches_torchs_cast_back():
+    codes = torch.arange(256, dtype=torch.uint8)
+    want = codes.view(torch.float8_e4m3fn).float().numpy()
+    got = e4m3.decode(codes.numpy())
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.array_equal(got[~np.isnan(got)], want[~np.isnan(want)])
+
+
+def test_encode_of_every_finite_code_value_is_the_code():
+    codes = np.array([b for b in range(256) if (b & 0x7F) != 0x7F], dtype=np.uint8)
+    assert np.array_equal(e4m3.encode(e4m3.decode(codes)), codes)      # -0.0 keeps 0x80
+
+
+def test_integer_encoder_equals_torch_on_every_97th_bit_pattern_in_range():
+    # The reference's own check of its encoder (kernels/core/tests/test_core_triton.py:68-77), both signs.
+    top = np.float32(448.0).view(np.uint32)
+    pos = np.arange(0, int(top) + 1, 97, dtype=np.uint32)
+    bits = np.concatenate([pos, pos | np.uint32(0x80000000)])
+    x = bits.view(np.float32)
+    want = torch.from_numpy(x.copy()).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(e4m3.encode(x), want)
+
+
+def test_special_values():
+    x = np.array([-0.0, -(2.0 ** -10), 2.0 ** -10, 1e-30, 448.0, -448.0, 1e30, -np.inf, np.nan], dtype=np.float32)
+    assert e4m3.encode(x).tolist() == [0x80, 0x80, 0x00, 0x00, 0x7E, 0xFE, 0x7E, 0xFE, 0x7F]
+    t = torch.from_numpy(x.copy()).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8)
+    assert t.tolist() == [0x80, 0x80, 0x00, 0x00, 0x7E, 0xFE, 0x7E, 0xFE, 0x7F]
+
+
+# -- append ----------------------------------------------------------------------------------------------------------------
+def test_slot_math_closed_form_and_known_answers():
+    table = [7, 2, 9]
+    assert append.slot(table, 0, 16) == 112 and append.slot(table, 15, 16) == 127
+    assert append.slot(table, 16, 16) == 32 and append.slot(table, 37, 16) == 9 * 16 + 5
+    got = append.slots(torch.tensor(table), torch.arange(48), 16).tolist()
+    assert got == [table[p // 16] * 16 + p % 16 for p in range(48)]      # test_rounds.py:34-36's rule
+    assert len(set(got)) == 48
+
+
+def test_bf16_and_fp16_appends_are_round_to_nearest_even():
+    x = torch.tensor([1.00390625, 1.01171875, 3.3895313892515355e38, -1.00390625]).view(1, 1, 4)
+    bits = append.encode(x, "bf16")[0].view(torch.int16).flatten().tolist()
+    assert [b & 0xFFFF for b in bits] == [0x3F80, 0x3F82, 0x7F7F, 0xBF80]
+    h = append.encode(torch.tensor([1.00048828125, 1.00146484375]).view(1, 1, 2), "fp16")[0]
+    assert [b & 0xFFFF for b in h.view(torch.int16).flatten().tolist()] == [0x3C00, 0x3C02]
+
+
+@pytest.mark.parametrize("mult", [0.05, 0.07, 1.0, 3.0])
+def test_fp8_append_torch_cast_equals_the_integer_encoder(mult):
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(64, 3, 128, generator=g) * 3
+    x[0, 0, :8] = torch.tensor([0.0, -0.0, 1e30, -1e30, 448.0 * mult, 2.0 ** -10 * mult, float("inf"), 1e-30])
+    a = append.encode(x, "fp8", mult)[0].view(torch.uint8)
+    b = append.encode_fp8_integer(x, mult)
+    assert torch.equal(a, b)
+
+
+def test_fp8_append_with_one_multiplier_per_head_is_the_scalar_rule_head_by_head():
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(10, 4, 64, generator=g) * 2
+    mults = torch.tensor([0.01, 0.02, 0.5, 1.5])
+    got = append.encode(x, "fp8", mults)[0].view(torch.uint8)
+    for h in range(4):
+        want = append.encode(x[:, h:h + 1], "fp8", float(mults[h]))[0].view(torch.uint8)
+        assert torch.equal(got[:, h:h + 1], want)
+
+
+def test_division_is_ieee_a_reciprocal_multiply_gives_other_codes():
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(100_000, generator=g)
+    s = torch.full_like(x, 0.05)
+    exact, approx = x / s, x * (1.0 / s)
+    assert float((exact != approx).float().mean()) > 0.05
+    # The stored FP32 row scales show it directly: amax / 448 is not amax * (1 / 448) for many rows.
+    amax = x.abs()
+    assert not torch.equal(amax / torch.full_like(amax, 448.0), amax * (1.0 / 448.0))
+    assert torch.equal(append.row_scales(x.view(-1, 1), 448.0), (amax / torch.full_like(amax, 448.0)).clamp(min=1e-30))
+
+
+def test_row_scaled_encodings_follow_their_rules():
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(12, 2, 64, generator=g) * 4
+    x[3] = 0.0
+    codes, scale = append.fp8_rows(x)
+    amax = x.abs().amax(-1)
+    assert torch.equal(scale, torch.maximum(amax / 448.0, torch.tensor(1e-30)))    # x / 448.0 on CPU is IEEE too
+    assert float(scale[3, 0]) == pytest.approx(1e-30) and not bool(codes[3].view(torch.uint8).any())
+    back = torch.from_numpy(e4m3.decode(codes.view(torch.uint8).numpy())) * scale[..., None]
+    assert float((back - x).abs().max()) <= float(amax.max()) / 16 + 1e-6       # 3 mantissa bits: half a step of 1/8
+    # the row's largest magnitude lands on +-448 exactly
+    top = codes.view(torch.uint8).view(12, 2, 64)[torch.arange(12) != 3] & 0x7F
+    assert bool((top.amax(-1) == 0x7E).all())
+    icodes, iscale = append.int8_rows(x)
+    assert torch.equal(iscale, torch.maximum(amax / 127.0, torch.tensor(1e-30)))
+    assert int(icodes.abs().max()) == 127
+    want = torch.round(x / iscale[..., None]).clamp(-127, 127).to(torch.int8)
+    assert torch.equal(icodes, want)
+    assert torch.round(torch.tensor([0.5, 1.5, 2.5, -0.5])).tolist() == [0.0, 2.0, 2.0, -0.0]    # ties to even
+
+
+@pytest.mark.parametrize("kind", ["bf16", "fp16", "fp8", "fp8:row", "int8"])
+def test_write_places_rows_at_their_slots_and_skips_negative_ones(kind):
+    g = torch.Generator().manual_seed(1)
+    keys, values = torch.randn(40, 3, 32, generator=g) * 3, torch.randn(40, 3, 16, generator=g)
+    k = torch.zeros(4, 16, 3, 32, dtype=append.STORAGE[kind])
+    v = torch.zeros(4, 16, 3, 16, dtype=append.STORAGE[kind])
+    ks = vs = None
+    if kind in append.ROW_SCALED:
+        ks, vs = torch.zeros(4, 16, 3), torch.zeros(4, 16, 3)
+    ids = torch.randperm(64, generator=g)[:40]
+    ids[7] = -1
+    append.write(keys, values, ids, k, v, kind, ks, vs, multipliers=(0.05, 0.07))
+    keep = ids >= 0
+    for x, store, scales, m in ((keys, k, ks, 0.05), (values, v, vs, 0.07)):
+        want, want_scale = append.encode(x[keep], kind, m)
+        got = store.view(-1, 3, store.shape[-1])[ids[keep]]
+        assert torch.equal(append._bytes(got), append._bytes(want))
+        if want_scale is not None:
+            assert torch.equal(scales.view(-1, 3)[ids[keep]], want_scale)
+        untouched = torch.ones(64, dtype=torch.bool)
+        untouched[ids[keep]] = False
+        assert not bool(store.view(-1, 3, store.shape[-1])[untouched].float().abs().sum())
+    # the torch path sends a skipped token to the dump slot instead
+    k2 = torch.zeros_like(k)
+    append.write(keys, None, ids, k2, None, kind, torch.zeros(4, 16, 3) if ks is not None else None, None,
+                 multipliers=(0.05, 0.07), dump_slot=63)
+    assert bool(k2.view(-1, 3, 32)[63].float().abs().sum()) or bool((ids == 63).any())
+
+
+# -- attention ---------------------------------------------------------------------------------------------------------------
+def _brute(q, keys, values, seen, scale, group):
+    out, lse = [], []
+    for h in range(len(q)):
+        kv = h // group
+        scores = [sum(a * b for a, b in zip(q[h], keys[n][kv])) * scale for n in range(len(keys)) if seen[n]]
+        vals = [values[n][kv] for n in range(len(keys)) if seen[n]]
+        top = max(scores)
+        w = [math.exp(s - top) for s in scores]
+        total = sum(w)
+        out.append([sum(wi / total * v[c] for wi, v in zip(w, vals)) for c in range(len(vals[0]))])
+        lse.append(top + math.log(total))
+    return out, lse
+
+
+def test_reference_attention_equals_brute_force_and_maps_gqa_heads_by_division():
+    g = torch.Generator().manual_seed(2)
+    q = torch.randn(4, 8, generator=g, dtype=torch.float64)
+    keys = torch.randn(9, 2, 8, generator=g, dtype=torch.float64)
+    values = torch.randn(9, 2, 5, generator=g, dtype=torch.float64)
+    seen = torch.tensor([True] * 6 + [False] * 3)
+    out, lse = attend.reference(q, keys, values, seen, 0.3)
+    want, want_lse = _brute(q.tolist(), keys.tolist(), values.tolist(), seen.tolist(), 0.3, 2)
+    assert torch.allclose(out, torch.tensor(want, dtype=torch.float64), atol=1e-12)
+    assert torch.allclose(lse, torch.tensor(want_lse, dtype=torch.float64), atol=1e-12)
+    # heads 0,1 read KV head 0 and heads 2,3 read KV head 1: changing KV head 1 moves only heads 2 and 3
+    keys2 = keys.clone()
+    keys2[:, 1] += 1.0
+    out2, _ = attend.reference(q, keys2, values, seen, 0.3)
+    assert torch.equal(out2[:2], out[:2]) and not torch.equal(out2[2:], out[2:])
+
+
+def test_zero_queries_average_the_values_and_unseen_rows_give_zero_and_minus_infinity():
+    keys = torch.randn(7, 1, 4, dtype=torch.float64)
+    values = torch.arange(14, dtype=torch.float64).view(7, 1, 2)
+    out, lse = attend.reference(torch.zeros(2, 4, dtype=torch.float64), keys, values, torch.ones(7, dtype=torch.bool), 1.0)
+    assert torch.allclose(out[0], values[:, 0].mean(0)) and float(lse[0]) == pytest.approx(math.log(7))
+    out, lse = attend.reference(torch.zeros(2, 4, dtype=torch.float64), keys, values, torch.zeros(7, dtype=torch.bool), 1.0)
+    assert not bool(out.any()) and bool(torch.isinf(lse).all()) and bool((lse < 0).all())
+    # the attention-state README's worked example (README.md:224-238): zero query over values 2 and 10 -> 6, then 2
+    kv = torch.tensor([[[1.0, 0.0]], [[0.0, 1.0]]], dtype=torch.float64)
+    vv = torch.tensor([[[2.0]], [[10.0]]], dtype=torch.float64)
+    z = torch.zeros(1, 2, dtype=torch.float64)
+    assert float(attend.reference(z, kv, vv, torch.tensor([True, True]), 1.0)[0]) == 6.0
+    assert float(attend.reference(z, kv, vv, torch.tensor([True, False]), 1.0)[0]) == 2.0
+
+
+def _pool(kind, hkv, d, dv, page, lengths, seed=0, multipliers=(0.02, 0.03)):
+    """One layer's pages over shuffled page tables, written by the oracle's append."""
+    g = torch.Generator().manual_seed(seed)
+    width = max(math.ceil(n / page) for n in lengths) + 1
+    n_pages = width * len(lengths) + 3
+    k = torch.zeros(n_pages, page, hkv, d, dtype=append.STORAGE[kind])
+    v = torch.zeros(n_pages, page, hkv, dv, dtype=append.STORAGE[kind])
+    ks = vs = None
+    if kind in append.ROW_SCALED:
+        ks, vs = torch.zeros(n_pages, page, hkv), torch.zeros(n_pages, page, hkv)
+    tables = torch.randperm(n_pages, generator=g)[:width * len(lengths)].view(len(lengths), width).to(torch.int32)
+    raw = []
+    for s, n in enumerate(lengths):
+        keys, values = torch.randn(n, hkv, d, generator=g), torch.randn(n, hkv, dv, generator=g)
+        append.write(keys, values, append.slots(tables[s], torch.arange(n), page), k, v, kind, ks, vs, multipliers)
+        raw.append((keys, values))
+    return k, v, ks, vs, tables, raw
+
+
+@pytest.mark.parametrize("kind", ["fp32", "bf16", "fp8", "fp8:row", "int8"])
+def test_the_sdpa_cpu_path_and_the_dense_window_agree_with_float64_over_the_stored_values(kind):
+    hq, hkv, d, page = 8, 2, 128, 16
+    lengths = [64, 200, 333, 512]
+    mult = (0.02, 0.03) if kind == "fp8" else (1.0, 1.0)
+    k, v, ks, vs, tables, _ = _pool(kind, hkv, d, d, page, lengths, multipliers=mult)
+    compute = torch.float32 if kind == "fp32" else torch.bfloat16
+    g = torch.Generator().manual_seed(3)
+    rows = [(0, 1, 63), (1, 1, 199), (2, 3, 330), (5, 2, 510)]          # (first token, count, first position)
+    q = torch.randn(7, hq, d, generator=g)
+    scale = d ** -0.5
+
+    def gather_row(r, n):
+        return attend.gather(k, v, tables[r], n, page, kind, compute, ks, vs, mult)
+    out = attend.sdpa_rows(q, rows, gather_row, scale, torch.empty(7, hq, d))
+    tol = 1e-5 if kind == "fp32" else 2e-2
+    for r, (first, count, position) in enumerate(rows):
+        want, want_lse = attend.window_reference(q[first:first + count], k, v, kind, tables[r], position, count, page,
+                                                 scale, ks, vs, mult, q_dtype=compute)
+        assert torch.allclose(out[first:first + count].double(), want, atol=tol, rtol=tol)
+        keys, values = attend.stored_rows(k, v, tables[r], position + count, page, kind, ks, vs, mult)
+        dense, dense_lse = attend.windows_dense(q[first:first + count].to(compute), keys.float(), values.float(),
+                                                position, scale)
+        assert torch.allclose(dense.double(), want, atol=1e-4, rtol=1e-4)
+        assert torch.allclose(dense_lse.double(), want_lse, atol=1e-4, rtol=1e-5)
+
+
+def test_a_sliding_window_sees_only_its_last_positions():
+    k, v, ks, vs, tables, _ = _pool("bf16", 1, 16, 16, 16, [100])
+    q = torch.randn(2, 2, 16, generator=torch.Generator().manual_seed(4))
+    out, _ = attend.window_reference(q, k, v, "bf16", tables[0], 98, 2, 16, 0.25, sliding=8)
+    keys, values = attend.stored_rows(k, v, tables[0], 100, 16, "bf16")
+    for c in range(2):
+        seen = torch.zeros(100, dtype=torch.bool)
+        seen[98 + c - 7:98 + c + 1] = True
+        want, _ = attend.reference(q[c].bfloat16().double(), keys, values, seen, 0.25)
+        assert torch.equal(out[c], want)
+    dense, _ = attend.windows_dense(q.bfloat16(), keys.float(), values.float(), 98, 0.25, sliding=8)
+    assert torch.allclose(dense.double(), out, atol=1e-5)
+
+
+# -- online softmax steps and merges -------------------------------------------------------------------------------------
+@pytest.mark.parametrize("cuts", [[5], [1, 2, 3], [0, 7], [3, 3]])
+def test_folding_any_cut_of_the_scores_equals_one_pass(cuts):
+    g = torch.Generator().manual_seed(9)
+    s = torch.randn(3, 11, generator=g, dtype=torch.float64) * 4
+    s[1, :] = float("-inf")                                       # a row that sees nothing
+    s[2, 4:] = float("-inf")
+    vals = torch.randn(11, 5, generator=g, dtype=torch.float64)
+    bounds = [0] + cuts + [11]
+    m_run = torch.full((3,), float("-inf"), dtype=torch.float64)
+    l_run = torch.zeros(3, dtype=torch.float64)
+    acc_run = torch.zeros(3, 5, dtype=torch.float64)
+    for a, b in zip(bounds[:-1], bounds[1:]):
+        m = torch.full((3,), float("-inf"), dtype=torch.float64)
+        if b > a:
+            p, alpha, m = attend.step(s[:, a:b], m)
+            l, acc = p.sum(1), p @ vals[a:b]
+        else:
+            l, acc = torch.zeros(3, dtype=torch.float64), torch.zeros(3, 5, dtype=torch.float64)
+        m_run, l_run, keep, take = attend.fold(m_run, l_run, m, l)
+        acc_run = acc_run * keep[:, None] + acc * take[:, None]
+    out, lse = attend.finish(acc_run, l_run), attend.lse(m_run, l_run)
+    want = torch.softmax(s[[0, 2]], 1) @ vals
+    assert torch.allclose(out[[0, 2]], want, atol=1e-12)
+    assert torch.allclose(lse[[0, 2]], torch.logsumexp(s[[0, 2]], 1), atol=1e-12)
+    assert not bool(out[1].any()) and float(lse[1]) == float("-inf") and not bool(torch.isnan(out).any())
+
+
+def test_merge_reproduces_the_readme_worked_example_and_the_host_oracle():
+    # inference/partitioned-attention/README.md:48-62: four ranks share two tokens, two are empty -> 5.0
+    rows = ((0, (1., 0.), (2.,)), (1, (0., 1.), (8.,)))
+    parts = [attend.attention_partial((1., 1.), [r for r in rows if attend.owner(r[0], 4) == rank], 1, 1)
+             for rank in range(4)]
+    assert attend.merge_partials(parts)[0] == (5.,)
+    assert attend.global_position(3, 4, 1) == 13
+    assert attend.attention_partial((1., 1.), rows, 1, 0)[0] == (2.,)
+    with pytest.raises(ValueError):
+        attend.merge_partials([((0.0,), -math.inf)] * 2)
+    outs = [torch.tensor(o).view(1, 1, 1) for o, _ in parts]
+    lses = [torch.tensor(l).view(1, 1) for _, l in parts]
+    out, lse = attend.merge(outs, lses)
+    assert float(out) == pytest.approx(5.0) and float(lse) == pytest.approx(attend.merge_partials(parts)[1])
+
+
+def test_merge_skips_parts_without_keys_and_gives_zero_for_a_token_no_part_saw():
+    # inference/partitioned-attention/tests/test_device.py:70-77
+    outs = [torch.ones(2, 1, 3), torch.zeros(2, 1, 3)]
+    lses = [torch.tensor([[0.5], [float("-inf")]]), torch.full((2, 1), float("-inf"))]
+    out, lse = attend.merge(outs, lses)
+    assert out[0].tolist() == [[1.0, 1.0, 1.0]]
+    assert (out[1].tolist(), lse[1].tolist()) == ([[0.0, 0.0, 0.0]], [float("-inf")])
+    assert float(lse[0, 0]) == pytest.approx(0.5, abs=1e-6)
+
+
+@pytest.mark.parametrize("cut", [1, 120, 299])
+def test_merged_shards_equal_attention_over_the_whole_whatever_the_cut(cut):
+    g = torch.Generator().manual_seed(1)
+    keys, values = torch.randn(300, 2, 64, generator=g).double(), torch.randn(300, 2, 64, generator=g).double()
+    q = torch.randn(4, 64, generator=g).double()
+    every = torch.ones(300, dtype=torch.bool)
+    want, want_lse = attend.reference(q, keys, values, every, 0.125)
+    a = attend.reference(q, keys[:cut], values[:cut], every[:cut], 0.125)
+    b = attend.reference(q, keys[cut:], values[cut:], every[cut:], 0.125)
+    out, lse = attend.merge([a[0][None].float(), b[0][None].float()], [a[1][None].float(), b[1][None].float()])
+    assert torch.allclose(out[0].double(), want, atol=1e-5) and torch.allclose(lse[0].double(), want_lse, atol=1e-5)
