@@ -1,0 +1,50 @@
+// The C ABI: argument checks live in the launchers; this file only forwards and names errors.
+#include "pkv_launch.hpp"
+
+extern "C" {
+
+int crit_pkv_write(const crit_pkv_write_params* p, void* stream) {
+    return pkv::launch_write(p, reinterpret_cast<hipStream_t>(stream));
+}
+
+int crit_pkv_attend(const crit_pkv_attend_params* p, void* stream) {
+    return pkv::launch_attend(p, reinterpret_cast<hipStream_t>(stream));
+}
+
+int crit_pkv_merge(const crit_pkv_merge_params* p, void* stream) {
+    return pkv::launch_merge(p, reinterpret_cast<hipStream_t>(stream));
+}
+
+int crit_pkv_prefill(const crit_pkv_prefill_params* p, void* stream) {
+    return pkv::launch_prefill(p, reinterpret_cast<hipStream_t>(stream));
+}
+
+int crit_pkv_stream_read(const void* data, int64_t bytes, float* sink, void* stream) {
+    return pkv::launch_stream_read(data, bytes, sink, reinterpret_cast<hipStream_t>(stream));
+}
+
+int crit_pkv_abi_version(void) { return CRIT_PKV_ABI_VERSION; }
+
+int crit_pkv_params_size(int which) {
+    switch (which) {
+        case 0: return (int)sizeof(crit_pkv_write_params);
+        case 1: return (int)sizeof(crit_pkv_attend_params);
+        case 2: return (int)sizeof(crit_pkv_merge_params);
+        case 3: return (int)sizeof(crit_pkv_prefill_params);
+    }
+    return -1;
+}
+
+const char* crit_pkv_error(int code) {
+    switch (code) {
+        case 0: return "ok";
+        case CRIT_PKV_E_GEOMETRY: return "crit_pkv: a shape the kernels do not take (head dims 64/128/256 with keys and values of one width, query heads a multiple of the KV heads, 1..64 columns, 16-byte aligned rows)";
+        case CRIT_PKV_E_DTYPE: return "crit_pkv: a dtype or page kind the kernels do not take";
+        case CRIT_PKV_E_NULL: return "crit_pkv: a required pointer is NULL";
+        case CRIT_PKV_E_WORKSPACE: return "crit_pkv: partitions, piece or the partial arrays do not fit the launch";
+    }
+    if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
+    return "crit_pkv: unknown error";
+}
+
+}   // extern "C"

@@ -1,0 +1,131 @@
+// Device helpers shared by the paged-KV kernels (gfx950 only): 16-bit float bit casts, the E4M3FN codec, DPP
+// reductions inside a 16-lane row, and the online-softmax fold.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/crit_pkv.h"
+
+namespace pkv {
+
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+
+#define PKV_DEV __device__ __forceinline__
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+PKV_DEV uint32_t f2u(float x) { return __builtin_bit_cast(uint32_t, x); }
+PKV_DEV float u2f(uint32_t x) { return __builtin_bit_cast(float, x); }
+
+// -- bf16 / f16 ---------------------------------------------------------------------------------------------------------
+PKV_DEV float bf16_lo(uint32_t w) { return u2f(w << 16); }
+PKV_DEV float bf16_hi(uint32_t w) { return u2f(w & 0xffff0000u); }
+
+// FP32 -> BF16 bits, round to nearest even; NaN -> 0x7FC0 (what torch's CPU cast stores).
+PKV_DEV uint32_t bf16_rne(float x) {
+    uint32_t u = f2u(x);
+    uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    return (x != x) ? 0x7fc0u : r;
+}
+PKV_DEV uint32_t pack_bf16(float a, float b) { return bf16_rne(a) | (bf16_rne(b) << 16); }
+
+PKV_DEV float f16_lo(uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu)); }
+PKV_DEV float f16_hi(uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16)); }
+PKV_DEV uint32_t f16_bits(float x) { return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)x); }   // RNE
+PKV_DEV uint32_t pack_f16(float a, float b) { return f16_bits(a) | (f16_bits(b) << 16); }
+
+// -- E4M3FN -------------------------------------------------------------------------------------------------------------
+// FP32 -> code: clamp to [-448, 448], round to nearest code, ties to even; sign from the sign bit (-0.0 -> 0x80);
+// NaN -> 0x7F | sign. Integer arithmetic only, so the bytes do not depend on any conversion mode of the hardware.
+PKV_DEV uint32_t e4m3_encode(float x) {
+    const uint32_t bits = f2u(x);
+    const uint32_t sign = (bits >> 24) & 0x80u;
+    float a = __builtin_fabsf(x);
+    const bool nan = x != x;
+    a = a > 448.0f ? 448.0f : a;
+    const uint32_t ab = f2u(a);
+    int ex = (int)(ab >> 23) - 127;
+    int sex = ex < -126 ? -126 : ex;
+    const float frac = a * u2f((uint32_t)(127 - sex) << 23);               // exact scaling into [1, 2)
+    int mant = (int)__builtin_rintf((frac - 1.0f) * 8.0f);                  // ties to even
+    const bool carry = mant == 8;
+    ex = carry ? ex + 1 : ex;
+    mant = carry ? 0 : mant;
+    const uint32_t normal = ((uint32_t)(ex + 7) << 3) | (uint32_t)mant;
+    const uint32_t sub = (uint32_t)(int)__builtin_rintf(a * 512.0f);       // below 2^-6: multiples of 2^-9
+    uint32_t code = a < 0.015625f ? sub : normal;
+    code = nan ? 0x7fu : code;
+    return code | sign;
+}
+
+// Two E4M3FN codes (bytes 0,1 or 2,3 of w) -> FP32, by the hardware conversion (OCP E4M3 on gfx950).
+template <bool HI>
+PKV_DEV f32x2 e4m3_pair(uint32_t w) { return __builtin_amdgcn_cvt_pk_f32_fp8((int)w, HI); }
+
+// -- cross-lane ------------------------------------------------------------------------------------------------------------
+// DPP controls: quad_perm [1,0,3,2] = 0xB1 (xor 1), quad_perm [2,3,0,1] = 0x4E (xor 2), row_half_mirror = 0x141
+// (lane i <-> 7 - i inside each 8), row_mirror = 0x140 (lane i <-> 15 - i inside each 16).
+template <int CTRL>
+PKV_DEV float dpp(float x) {
+    return u2f((uint32_t)__builtin_amdgcn_update_dpp(0, (int)f2u(x), CTRL, 0xf, 0xf, true));
+}
+
+// Sum over the LANES (8, 16 or 32, a power of two) lanes of each aligned group; every lane gets the same bits.
+template <int LANES>
+PKV_DEV float group_sum(float x) {
+    x += dpp<0xB1>(x);
+    x += dpp<0x4E>(x);
+    x += dpp<0x141>(x);
+    if constexpr (LANES >= 16) x += dpp<0x140>(x);
+    if constexpr (LANES >= 32) x += __shfl_xor(x, 16);
+    if constexpr (LANES >= 64) x += __shfl_xor(x, 32);
+    return x;
+}
+template <int LANES>
+PKV_DEV float group_max(float x) {
+    x = __builtin_fmaxf(x, dpp<0xB1>(x));
+    x = __builtin_fmaxf(x, dpp<0x4E>(x));
+    x = __builtin_fmaxf(x, dpp<0x141>(x));
+    if constexpr (LANES >= 16) x = __builtin_fmaxf(x, dpp<0x140>(x));
+    if constexpr (LANES >= 32) x = __builtin_fmaxf(x, __shfl_xor(x, 16));
+    if constexpr (LANES >= 64) x = __builtin_fmaxf(x, __shfl_xor(x, 32));
+    return x;
+}
+
+// -- online softmax, base 2 -----------------------------------------------------------------------------------------------
+PKV_DEV float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }   // v_exp_f32; exp2(-inf) = 0
+
+// A partial state (m, l) into the running one, in the caller's order: out = out * keep + partial * take.
+struct Fold {
+    float m, l, keep, take;
+};
+PKV_DEV Fold fold(float m_run, float l_run, float m, float l) {
+    Fold f;
+    f.m = __builtin_fmaxf(m_run, m);
+    const float sub = f.m == -INFINITY ? 0.0f : f.m;
+    f.keep = exp2_fast(m_run - sub);
+    f.take = exp2_fast(m - sub);
+    f.l = __builtin_fmaf(l_run, f.keep, l * f.take);
+    return f;
+}
+
+PKV_DEV void store_out(void* out, int dtype, int64_t index, float x) {
+    if (dtype == CRIT_PKV_BF16) {
+        reinterpret_cast<uint16_t*>(out)[index] = (uint16_t)bf16_rne(x);
+    } else if (dtype == CRIT_PKV_F16) {
+        reinterpret_cast<uint16_t*>(out)[index] = (uint16_t)f16_bits(x);
+    } else {
+        reinterpret_cast<float*>(out)[index] = x;
+    }
+}
+
+inline int hip_code(hipError_t e) { return e == hipSuccess ? 0 : (int)e; }
+
+}   // namespace pkv

@@ -1,0 +1,13 @@
+// Host-side launchers, one per translation unit of kernels; the C ABI (pkv_abi.hip) forwards to them.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "../../include/crit_pkv.h"
+
+namespace pkv {
+int launch_write(const crit_pkv_write_params* p, hipStream_t stream);
+int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream);
+int launch_merge(const crit_pkv_merge_params* p, hipStream_t stream);
+int launch_prefill(const crit_pkv_prefill_params* p, hipStream_t stream);
+int launch_stream_read(const void* data, int64_t bytes, float* sink, hipStream_t stream);
+}   // namespace pkv

@@ -1,0 +1,262 @@
+// KV append: a step's keys and values scattered into their slots of one layer's pages, encoded for the page kind.
+// HBM-bound: every lane moves 16 bytes of page row per store, a wave covers 64/LPR whole rows per pass, rows of one
+// token are consecutive in the grid so the reads of a token's heads are contiguous too.
+#include "pkv_common.hpp"
+#include "pkv_launch.hpp"
+
+namespace pkv {
+
+struct WriteArgs {
+    const void* src[2];
+    void* pages[2];
+    float* scales[2];
+    const int64_t* slots;
+    const float* head_mult;
+    int64_t stride_t[2], stride_h[2];
+    int64_t tokens;
+    int dim[2];
+    int hkv;
+    int heads;      // hkv (keys only) or 2 * hkv
+    float mult[2];
+};
+
+template <int IN>
+PKV_DEV float load_in(const void* base, int64_t i) {
+    if constexpr (IN == CRIT_PKV_F32) return reinterpret_cast<const float*>(base)[i];
+    if constexpr (IN == CRIT_PKV_BF16) return u2f((uint32_t)reinterpret_cast<const uint16_t*>(base)[i] << 16);
+    return (float)reinterpret_cast<const _Float16*>(base)[i];
+}
+
+// EPL consecutive input elements as FP32, by 16-byte loads (the caller checked the alignment).
+template <int IN, int EPL>
+PKV_DEV void load_vec(const void* base, int64_t i, float (&x)[EPL]) {
+    if constexpr (IN == CRIT_PKV_F32) {
+        const float4* p = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(base) + i);
+#pragma unroll
+        for (int j = 0; j < EPL / 4; ++j) {
+            float4 v = p[j];
+            x[4 * j] = v.x, x[4 * j + 1] = v.y, x[4 * j + 2] = v.z, x[4 * j + 3] = v.w;
+        }
+    } else {
+        const uint4* p = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(base) + i);
+#pragma unroll
+        for (int j = 0; j < EPL / 8; ++j) {
+            uint4 v = p[j];
+            uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                if constexpr (IN == CRIT_PKV_BF16) {
+                    x[8 * j + 2 * k] = bf16_lo(w[k]), x[8 * j + 2 * k + 1] = bf16_hi(w[k]);
+                } else {
+                    x[8 * j + 2 * k] = f16_lo(w[k]), x[8 * j + 2 * k + 1] = f16_hi(w[k]);
+                }
+            }
+        }
+    }
+}
+
+// One row = (token, head) with head in [0, heads): keys' heads first, then values'. LPR lanes hold one row, EPL
+// elements each (16 bytes of page row). KIND as in the ABI; F16: 16-bit pages are fp16, not bf16.
+template <int KIND, bool F16, int IN, int LPR>
+__global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
+    constexpr int EPL = KIND == 0 ? 8 : 16;
+    const int lane_in_row = threadIdx.x % LPR;
+    const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPR;
+    if (row >= a.tokens * a.heads) return;
+    const int64_t t = row / a.heads;
+    int head = (int)(row % a.heads);
+    const int which = head >= a.hkv ? 1 : 0;
+    head -= which * a.hkv;
+    const int64_t slot = a.slots[t];
+    if (slot < 0) return;
+    const int dim = a.dim[which];
+    const int i0 = lane_in_row * EPL;
+    const bool live = i0 < dim;
+    float x[EPL];
+    if (live) {
+        load_vec<IN, EPL>(a.src[which], t * a.stride_t[which] + head * a.stride_h[which] + i0, x);
+    } else {
+#pragma unroll
+        for (int j = 0; j < EPL; ++j) x[j] = 0.0f;
+    }
+    const int64_t dst = (slot * a.hkv + head) * dim + i0;
+    if constexpr (KIND == 0) {
+        uint4 v;
+        if constexpr (F16) {
+            v = make_uint4(pack_f16(x[0], x[1]), pack_f16(x[2], x[3]), pack_f16(x[4], x[5]), pack_f16(x[6], x[7]));
+        } else {
+            v = make_uint4(pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]), pack_bf16(x[6], x[7]));
+        }
+        if (live) *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(a.pages[which]) + dst) = v;
+    } else {
+        float div;
+        if constexpr (KIND == 1) {
+            div = a.head_mult ? a.head_mult[which * a.hkv + head] : a.mult[which];
+        } else {
+            float amax = 0.0f;
+#pragma unroll
+            for (int j = 0; j < EPL; ++j) {
+                const float m = __builtin_fabsf(x[j]);
+                amax = (m > amax || m != m) ? m : amax;       // a NaN in the row makes the scale NaN, as torch's amax
+            }
+#pragma unroll
+            for (int o = 1; o < LPR; o <<= 1) {
+                const float other = __shfl_xor(amax, o);
+                amax = (other > amax || other != other) ? other : amax;
+            }
+            const float top = KIND == 2 ? 448.0f : 127.0f;
+            div = __fdiv_rn(amax, top);
+            div = div < 1e-30f ? 1e-30f : div;               // clamp(min=1e-30); NaN stays NaN
+            if (lane_in_row == 0) a.scales[which][slot * a.hkv + head] = div;
+        }
+        uint32_t w[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            uint32_t packed = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float q = __fdiv_rn(x[4 * k + j], div);
+                uint32_t code;
+                if constexpr (KIND == 3) {
+                    float r = __builtin_rintf(q);            // ties to even
+                    r = r < -127.0f ? -127.0f : (r > 127.0f ? 127.0f : r);
+                    code = (uint32_t)(int)r & 0xffu;
+                } else {
+                    code = e4m3_encode(q);
+                }
+                packed |= code << (8 * j);
+            }
+            w[k] = packed;
+        }
+        if (live) *reinterpret_cast<uint4*>(reinterpret_cast<uint8_t*>(a.pages[which]) + dst) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+}
+
+// Any width and alignment: one lane per row element group of one (scalar loads and stores); the row scale by a
+// loop. Used when a row is not a whole number of 16-byte lanes or a stride breaks the alignment.
+template <int KIND, bool F16, int IN>
+__global__ __launch_bounds__(256) void write_rows_scalar(WriteArgs a) {
+    const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (row >= a.tokens * a.heads) return;
+    const int64_t t = row / a.heads;
+    int head = (int)(row % a.heads);
+    const int which = head >= a.hkv ? 1 : 0;
+    head -= which * a.hkv;
+    const int64_t slot = a.slots[t];
+    if (slot < 0) return;
+    const int dim = a.dim[which];
+    const int64_t src = t * a.stride_t[which] + head * a.stride_h[which];
+    const int64_t dst = (slot * a.hkv + head) * dim;
+    float div = 1.0f;
+    if constexpr (KIND == 1) div = a.head_mult ? a.head_mult[which * a.hkv + head] : a.mult[which];
+    if constexpr (KIND >= 2) {
+        float amax = 0.0f;
+        for (int i = 0; i < dim; ++i) {
+            const float m = __builtin_fabsf(load_in<IN>(a.src[which], src + i));
+            amax = (m > amax || m != m) ? m : amax;
+        }
+        div = __fdiv_rn(amax, KIND == 2 ? 448.0f : 127.0f);
+        div = div < 1e-30f ? 1e-30f : div;
+        a.scales[which][slot * a.hkv + head] = div;
+    }
+    for (int i = 0; i < dim; ++i) {
+        const float x = load_in<IN>(a.src[which], src + i);
+        if constexpr (KIND == 0) {
+            reinterpret_cast<uint16_t*>(a.pages[which])[dst + i] = (uint16_t)(F16 ? f16_bits(x) : bf16_rne(x));
+        } else {
+            const float q = __fdiv_rn(x, div);
+            uint32_t code;
+            if constexpr (KIND == 3) {
+                float r = __builtin_rintf(q);
+                r = r < -127.0f ? -127.0f : (r > 127.0f ? 127.0f : r);
+                code = (uint32_t)(int)r & 0xffu;
+            } else {
+                code = e4m3_encode(q);
+            }
+            reinterpret_cast<uint8_t*>(a.pages[which])[dst + i] = (uint8_t)code;
+        }
+    }
+}
+
+template <int KIND, bool F16, int IN>
+static int launch_kind(const WriteArgs& a, int lpr, bool vector, hipStream_t stream) {
+    const int64_t rows = a.tokens * a.heads;
+    if (!vector) {
+        const int64_t blocks = (rows + 255) / 256;
+        hipLaunchKernelGGL((write_rows_scalar<KIND, F16, IN>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+        return hip_code(hipGetLastError());
+    }
+    const int64_t blocks = (rows * lpr + 255) / 256;
+    switch (lpr) {
+#define PKV_CASE(L)                                                                                              \
+    case L:                                                                                                      \
+        hipLaunchKernelGGL((write_rows<KIND, F16, IN, L>), dim3((unsigned)blocks), dim3(256), 0, stream, a);     \
+        break;
+        PKV_CASE(1) PKV_CASE(2) PKV_CASE(4) PKV_CASE(8) PKV_CASE(16) PKV_CASE(32) PKV_CASE(64)
+#undef PKV_CASE
+        default:
+            return CRIT_PKV_E_GEOMETRY;
+    }
+    return hip_code(hipGetLastError());
+}
+
+template <int KIND, bool F16>
+static int launch_in(const WriteArgs& a, int in_dtype, int lpr, bool vector, hipStream_t stream) {
+    switch (in_dtype) {
+        case CRIT_PKV_F32: return launch_kind<KIND, F16, CRIT_PKV_F32>(a, lpr, vector, stream);
+        case CRIT_PKV_BF16: return launch_kind<KIND, F16, CRIT_PKV_BF16>(a, lpr, vector, stream);
+        case CRIT_PKV_F16: return launch_kind<KIND, F16, CRIT_PKV_F16>(a, lpr, vector, stream);
+    }
+    return CRIT_PKV_E_DTYPE;
+}
+
+static int next_pow2(int n) {
+    int p = 1;
+    while (p < n) p <<= 1;
+    return p;
+}
+
+int launch_write(const crit_pkv_write_params* p, hipStream_t stream) {
+    if (!p || !p->keys || !p->key_pages || !p->slots) return CRIT_PKV_E_NULL;
+    if ((p->values == nullptr) != (p->value_pages == nullptr)) return CRIT_PKV_E_NULL;
+    if (p->tokens < 0 || p->kv_heads < 1 || p->head_dim < 1 || (p->values && p->value_dim < 1)) return CRIT_PKV_E_GEOMETRY;
+    if (p->kind < 0 || p->kind > 3) return CRIT_PKV_E_DTYPE;
+    if (p->kind >= 2 && (!p->key_scales || (p->values && !p->value_scales))) return CRIT_PKV_E_NULL;
+    if (p->kind == 0 && p->page_dtype != CRIT_PKV_BF16 && p->page_dtype != CRIT_PKV_F16) return CRIT_PKV_E_DTYPE;
+    if (p->tokens == 0) return 0;
+    WriteArgs a;
+    a.src[0] = p->keys, a.src[1] = p->values;
+    a.pages[0] = p->key_pages, a.pages[1] = p->value_pages;
+    a.scales[0] = p->key_scales, a.scales[1] = p->value_scales;
+    a.slots = p->slots;
+    a.head_mult = p->kind == 1 ? p->head_multipliers : nullptr;
+    a.stride_t[0] = p->key_stride_t, a.stride_t[1] = p->value_stride_t;
+    a.stride_h[0] = p->key_stride_h, a.stride_h[1] = p->value_stride_h;
+    a.tokens = p->tokens;
+    a.dim[0] = p->head_dim, a.dim[1] = p->values ? p->value_dim : p->head_dim;
+    a.hkv = p->kv_heads;
+    a.heads = p->values ? 2 * p->kv_heads : p->kv_heads;
+    a.mult[0] = p->key_multiplier, a.mult[1] = p->value_multiplier;
+    // The vector path: rows are whole 16-byte lanes on both sides and every row start is 16-byte aligned.
+    const int epl = p->kind == 0 ? 8 : 16;
+    const int in_bytes = p->in_dtype == CRIT_PKV_F32 ? 4 : 2;
+    const int in_align = 16 / in_bytes;
+    const int widest = a.dim[0] > a.dim[1] ? a.dim[0] : a.dim[1];
+    const int lpr = next_pow2((widest + epl - 1) / epl);
+    bool vector = lpr <= 64;
+    for (int w = 0; w < (p->values ? 2 : 1); ++w) {
+        vector = vector && a.dim[w] % epl == 0 && a.stride_t[w] % in_align == 0 && a.stride_h[w] % in_align == 0 &&
+                 (reinterpret_cast<uintptr_t>(a.src[w]) % 16) == 0 && (reinterpret_cast<uintptr_t>(a.pages[w]) % 16) == 0;
+    }
+    const bool f16 = p->kind == 0 && p->page_dtype == CRIT_PKV_F16;
+    switch (p->kind) {
+        case 0: return f16 ? launch_in<0, true>(a, p->in_dtype, lpr, vector, stream)
+                           : launch_in<0, false>(a, p->in_dtype, lpr, vector, stream);
+        case 1: return launch_in<1, false>(a, p->in_dtype, lpr, vector, stream);
+        case 2: return launch_in<2, false>(a, p->in_dtype, lpr, vector, stream);
+        case 3: return launch_in<3, false>(a, p->in_dtype, lpr, vector, stream);
+    }
+    return CRIT_PKV_E_DTYPE;
+}
+
+}   // namespace pkv

@@ -1,0 +1,530 @@
+"""Attention over paged KV caches on one MI355X (gfx950): the kernels module crit's KVPool and DeviceAttention call.
+
+The same module interface as crit's `paged_kv_attention` package (reference kernels/techniques/attention/
+paged-kv-attention/torch-ext/paged_kv_attention/__init__.py): write(), attend(), prefill(), partitions(), piece_size(),
+tile_for(), workspace_floats(), the flash_* and cuda_* rules, owner()/release(), KINDS and MAX_COLUMNS, with the same
+argument names, meaning and errors, so `KVPool(kernels=this_module)` and `DeviceAttention(kernels=this_module)` work
+unchanged. Behind it are hand-written HIP kernels in libcrit_pkv.so, reached through a C ABI with ctypes (_abi.py);
+torch is used for device memory and streams only. There is no fallback: a missing library is an error.
+
+Pages. A cache layer is keys [pages][page][kv_heads][dim] and values [pages][page][kv_heads][value_dim]; position p of
+a sequence lives at slot table[p // page] * page + p % page. Page kinds: "bf16", "fp16"; "fp8" (E4M3 codes, value =
+code * multiplier, one multiplier per layer for keys and one for values, or with a [2][kv_heads] FP32 tensor one per
+KV head); "fp8:row" and "int8" (codes with an FP32 scale per position and KV head).
+
+Windows (attend). Row r is counts[r] <= columns tokens of one sequence: tokens starts[r].. of q, column c at position
+firsts[r] + c (its keys and values written already), page table tables[rows[r]]. Column c sees positions up to its own.
+Keys are read in pieces of `piece` positions; piece i belongs to partition i mod P. Each partition's unnormalised
+output, running maximum and sum go to the partials and a merge folds a column's partitions in order. A column's bits
+depend on its own query and keys, P, the piece and the page kind only: not on the rows beside it nor on the launch's
+width. With flash=True (or "cuda") the pieces are contiguous splits of `chunk` positions, one per partition, so the
+bits depend on the chunk only.
+
+Everything a launch reads about lengths (firsts, counts, position) is read on the device; after the first call of a
+shape nothing is allocated when `out` and `workspace` are given, so launches can be captured in a HIP graph.
+"""
+import contextlib
+import math
+import threading
+from typing import NamedTuple
+
+import torch
+
+from . import _abi
+
+__all__ = ["KINDS", "PIECE", "MAX_COLUMNS", "Derive", "attend", "derive", "cuda_block", "cuda_chunk", "cuda_parts",
+           "cuda_prompt", "cuda_ramp", "cuda_splits", "flash_block", "flash_chunk", "flash_parts", "flash_tile",
+           "merge_shards", "owner", "partitions", "piece_size", "prefill", "prefill_rows", "release", "stream_read",
+           "tile_for", "workspace_floats", "write"]
+
+KINDS = {"bf16": 0, "fp16": 0, "fp8": 1, "fp8:row": 2, "int8": 3}
+PIECE = 512          # positions per piece of FP8 or INT8 pages at a 128-wide head (piece_size)
+MAX_COLUMNS = 64     # columns of one row a launch reads
+MAX_QUERY_ROWS = 8   # query rows (columns x group heads) one workgroup holds; wider windows take more tiles
+
+_DTYPE = {torch.float32: _abi.F32, torch.bfloat16: _abi.BF16, torch.float16: _abi.F16}
+
+
+class Derive(NamedTuple):
+    """Keys derived from the value rows on read (the reference's derive=). Not served by these kernels: attend() and
+    prefill() refuse it."""
+    weight: object
+    eps: float
+    freqs: object
+    rotary_dim: int
+    table: object = None
+
+
+def derive(weight, eps, freqs, rotary_dim):
+    return Derive(weight, float(eps), freqs, int(rotary_dim))
+
+
+def _unsupported(what):
+    return NotImplementedError(f"paged_kv_attention (gfx950): {what} is not served by these kernels")
+
+
+# -- owners and module workspaces (reference __init__.py:129-171) --------------------------------------------------------
+_workspaces = {}
+_retired = []      # workspaces a launch outgrew: a captured graph may still replay into them, so they are kept
+_owner = threading.local()
+
+
+@contextlib.contextmanager
+def owner(key):
+    """Launches inside this block take module workspaces of their own, apart from every other owner's."""
+    before = getattr(_owner, "key", None)
+    _owner.key = key
+    try:
+        yield
+    finally:
+        _owner.key = before
+
+
+def release(key):
+    """Drop an owner's module workspaces (its captured graphs must be gone)."""
+    for at in [at for at in _workspaces if at[1] == key]:
+        del _workspaces[at]
+    _retired[:] = [(k, found) for k, found in _retired if k != key]
+
+
+def _held(device):
+    return (str(device), getattr(_owner, "key", None))
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _require_device(t, what):
+    if not t.is_cuda:
+        raise ValueError(f"{what} lives on the GPU (these are HIP kernels; there is no CPU path)")
+
+
+def _check_kind(kind, key_scales):
+    if kind not in KINDS:
+        raise ValueError(f"page kinds are {', '.join(KINDS)}, not {kind!r}")
+    if (KINDS[kind] >= 2) != (key_scales is not None):
+        raise ValueError(f"{kind} pages {'take' if KINDS[kind] >= 2 else 'have no'} scales per position and head")
+    return KINDS[kind]
+
+
+def _check_sliding(sliding, blocks):
+    sliding = int(sliding or 0)
+    if sliding < 0:
+        raise ValueError("a sliding window is 0 (none) or a number of positions")
+    if sliding and blocks is not None:
+        raise ValueError("a sliding window reads windows without block lists")
+    return sliding
+
+
+def _check_sinks(sinks, q):
+    if sinks is not None and (sinks.dtype != torch.float32 or sinks.dim() != 1 or sinks.shape[0] != q.shape[1] or
+                              not sinks.is_contiguous() or sinks.device != q.device):
+        raise ValueError(f"sinks are contiguous FP32 [{q.shape[1]}] (one a query head) on q's device")
+
+
+def _multipliers(multipliers, kv_heads, device):
+    """(key multiplier, value multiplier, per-head tensor or None): a pair of numbers, or a [2][kv_heads] FP32 tensor
+    on the device (one multiplier per KV head: keys' row then values')."""
+    if torch.is_tensor(multipliers):
+        if multipliers.dtype != torch.float32 or tuple(multipliers.shape) != (2, kv_heads) or \
+                not multipliers.is_contiguous() or multipliers.device != device:
+            raise ValueError(f"per-head multipliers are a contiguous FP32 [2][{kv_heads}] tensor on the pages' device")
+        return 1.0, 1.0, multipliers
+    return float(multipliers[0]), float(multipliers[1]), None
+
+
+def _page_dtype(pages, kind):
+    if KINDS[kind] == 0:
+        want = torch.float16 if kind == "fp16" else torch.bfloat16
+        if pages.dtype != want:
+            raise ValueError(f"{kind} pages are {want}, not {pages.dtype}")
+        return _abi.F16 if kind == "fp16" else _abi.BF16
+    return _abi.BF16
+
+
+def _cus(device):
+    return torch.cuda.get_device_properties(device).multi_processor_count
+
+
+# -- the split's order knobs -----------------------------------------------------------------------------------------------
+def partitions(device, kv_heads, kind, head_dim=None, value_dim=None):
+    """The partition count for a cache of `kv_heads` heads on `device`: about two workgroups per compute unit for one
+    long row (a power of two within 8..64). A column's bits depend on it: one count per cache."""
+    if kind not in KINDS:
+        raise ValueError(f"page kinds are {', '.join(KINDS)}, not {kind!r}")
+    programs = 2 * _cus(torch.device(device))
+    wanted = max(1, programs // max(1, int(kv_heads)))
+    return max(8, min(64, 1 << (wanted - 1).bit_length()))
+
+
+def piece_size(head_dim, value_dim, kind="bf16", kv_heads=None):
+    """Positions per piece: 32 Ki head values for 16-bit pages, 64 Ki for 8-bit ones (128 KiB of keys and values of
+    one KV head either way), within 64..512. A column's bits depend on it; it follows the cache's geometry and page
+    kind only."""
+    if kind not in KINDS:
+        raise ValueError(f"page kinds are {', '.join(KINDS)}, not {kind!r}")
+    values = 32768 if KINDS[kind] == 0 else 65536
+    return max(64, min(512, values // max(int(head_dim), int(value_dim))))
+
+
+def tile_for(columns, group, capability, fused=False):
+    """(rows, waves, stages) of a window launch's query tile: up to MAX_QUERY_ROWS rows of the flattened (column, group
+    head) list in a workgroup of four wavefronts, two steps in flight. rows // group never exceeds `columns`, so a
+    launch keeps the width its rows have."""
+    rows = max(1, min(int(columns) * int(group), MAX_QUERY_ROWS))
+    return rows, 4, 2
+
+
+def workspace_floats(tokens, heads, partitions, value_dim):
+    """FP32 floats of the partials a launch needs for `tokens` partial rows."""
+    return tokens * heads * partitions * (value_dim + 2)
+
+
+def _workspace(device, tokens, heads, parts, dv, given=None):
+    need = tokens * heads * parts
+    if given is not None:
+        if given.dtype != torch.float32 or given.numel() < need * (dv + 2) or not given.is_contiguous():
+            raise ValueError(f"attend's workspace holds {given.numel()} floats; this launch needs {need * (dv + 2)} "
+                             "(workspace_floats)")
+        return given[:need * dv], given[need * dv:need * (dv + 1)], given[need * (dv + 1):need * (dv + 2)]
+    found = _workspaces.get(_held(device))
+    if found is None or found.numel() < need * (dv + 2):
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("paged_kv_attention.attend: run a launch of this size once before capturing it (its "
+                               "partials' workspace is allocated outside the capture)")
+        if found is not None:
+            _retired.append((getattr(_owner, "key", None), found))
+        found = _workspaces[_held(device)] = torch.empty(max(need, 4096) * (dv + 2), dtype=torch.float32,
+                                                         device=device)
+    return found[:need * dv], found[need * dv:need * (dv + 1)], found[need * (dv + 1):need * (dv + 2)]
+
+
+# -- writes ----------------------------------------------------------------------------------------------------------------
+def write(keys, values, slots, key_pages, value_pages, kind, key_scales=None, value_scales=None,
+          multipliers=(1.0, 1.0)):
+    """A step's keys [tokens][kv_heads][dim] and values [tokens][kv_heads][value_dim] (FP32, BF16 or FP16) into their
+    slots ([tokens] int64; a slot below 0 is skipped) of one layer's pages (any view whose storage is
+    [slots][kv_heads][dim]), encoded for the page kind, in one launch; the bytes torch's own casts would store
+    (x.float() / multiplier clamped to +-448 then E4M3 for "fp8"; the row rules for "fp8:row" and "int8", their scales
+    written beside the codes). values and value_pages None: keys only. keys and key_pages None: values only."""
+    if keys is None:
+        if values is None:
+            raise ValueError("write takes keys, values or both")
+        if torch.is_tensor(multipliers):
+            multipliers = torch.stack([multipliers[1], multipliers[1]])
+        else:
+            multipliers = (multipliers[1], multipliers[1])
+        return write(values, None, slots, value_pages, None, kind, value_scales, None, multipliers=multipliers)
+    k_kind = _check_kind(kind, key_scales)
+    _require_device(keys, "write's keys")
+    T, hkv, d = keys.shape
+    if T == 0:
+        return
+    if keys.dtype not in _DTYPE:
+        keys = keys.float()
+    if keys.stride(-1) != 1:
+        keys = keys.contiguous()
+    if values is not None:
+        if values.dtype != keys.dtype:
+            values = values.to(keys.dtype)
+        if values.stride(-1) != 1:
+            values = values.contiguous()
+        if value_pages is None or (k_kind >= 2 and value_scales is None):
+            raise ValueError("values come with their pages (and their scales for fp8:row and int8)")
+    if slots.dtype != torch.int64 or not slots.is_contiguous():
+        slots = slots.to(torch.int64).contiguous()
+    if not key_pages.is_contiguous() or (value_pages is not None and not value_pages.is_contiguous()):
+        raise ValueError("a layer's pages are contiguous ([slots][kv_heads][dim] storage)")
+    km, vm, per_head = _multipliers(multipliers, hkv, keys.device)
+    p = _abi.WriteParams()
+    p.keys, p.values, p.slots = keys.data_ptr(), _ptr(values), slots.data_ptr()
+    p.key_pages, p.value_pages = key_pages.data_ptr(), _ptr(value_pages)
+    p.key_scales, p.value_scales = _ptr(key_scales), _ptr(value_scales)
+    p.head_multipliers = _ptr(per_head)
+    p.tokens = T
+    p.key_stride_t, p.key_stride_h = keys.stride(0), keys.stride(1)
+    if values is not None:
+        p.value_stride_t, p.value_stride_h = values.stride(0), values.stride(1)
+    p.kv_heads, p.head_dim = hkv, d
+    p.value_dim = values.shape[-1] if values is not None else 0
+    p.kind, p.page_dtype, p.in_dtype = k_kind, _page_dtype(key_pages, kind), _DTYPE[keys.dtype]
+    p.key_multiplier, p.value_multiplier = km, vm
+    with torch.cuda.device(keys.device):
+        _abi.check(_abi.load().crit_pkv_write(p, _stream(keys.device)), "paged_kv_attention.write")
+
+
+# -- windows ---------------------------------------------------------------------------------------------------------------
+FLASH_CHUNK = 1024        # positions a split of a contiguous-split launch over a cache (flash_chunk's rule)
+
+
+def flash_block(head_dim, value_dim, heads, kv_heads, page, kind="bf16"):
+    """Positions a wavefront's step covers (the granule a chunk is a multiple of): four loads of 64 / (dim / 8) rows."""
+    return 4 * (64 // max(1, max(int(head_dim), int(value_dim)) // 8)) if max(head_dim, value_dim) <= 512 else 4
+
+
+def flash_chunk(head_dim, value_dim, heads, kv_heads, page, kind="bf16"):
+    """Positions a split of every contiguous-split launch over a cache of this geometry: FLASH_CHUNK, a multiple of
+    the block. A column's bits depend on it: one per cache."""
+    block = flash_block(head_dim, value_dim, heads, kv_heads, page, kind)
+    return max(block, FLASH_CHUNK // block * block)
+
+
+def flash_parts(positions, chunk):
+    """Splits a contiguous-split launch's partial row takes over page tables holding `positions` positions a row."""
+    return max(1, -(-int(positions) // int(chunk)))
+
+
+def flash_tile(head_dim, value_dim, heads, kv_heads, page, kind, capability):
+    return MAX_QUERY_ROWS, 4
+
+
+# The reference's hand-written CUDA tile has no counterpart of its own here: reader "cuda" runs the same contiguous-split
+# kernels as reader "flash".
+cuda_block, cuda_chunk = flash_block, flash_chunk
+
+
+def cuda_ramp(*args, **kwargs):
+    return (1, 0)
+
+
+def cuda_splits(*args, **kwargs):
+    return 1
+
+
+def cuda_parts(head_dim, value_dim, heads, kv_heads, page, kind, positions, chunk=None, ramp=None):
+    chunk = chunk or cuda_chunk(head_dim, value_dim, heads, kv_heads, page, kind)
+    return flash_parts(positions, chunk)
+
+
+def cuda_prompt(head_dim, value_dim, dtype, kind, device):
+    """Whether the CUDA flash prompt chunk serves a pool: never (prompt chunks go through prefill())."""
+    return False
+
+
+def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, columns, page, *, counts=None,
+           offsets=None, tokens=None, key_scales=None, value_scales=None, multipliers=(1.0, 1.0), scale=None,
+           partitions=None, parents=None, blocks=None, block_size=None, out=None, lse=None, workspace=None, piece=None,
+           fused=False, fresh=None, vsplit=None, tile=None, num_warps=None, num_stages=None, maxnreg=None,
+           flash=False, chunk=None, ramp=None, sinks=None, sliding=0, derive=None, phases=0):
+    """Decode and verify windows over paged KV (see the module's description).
+
+    q [tokens][heads][dim] BF16 or FP16 (FP16 for "fp16" pages); key_pages/value_pages one layer's pages, key_scales/
+    value_scales their scales for "fp8:row" and "int8"; tables [S][width] int32 page tables; rows [R] int32 the table
+    row of each batch row; starts [R] int32 its first token in q; firsts [R] int64 its column 0's position; counts [R]
+    int32 its columns (None: `columns` each; more than `columns` read as `columns`); columns the widest row
+    (<= MAX_COLUMNS), a Python int. offsets [R] int32 and tokens: each row's first partial row and the partial rows
+    the launch takes from offsets[0] on. Writes out [tokens][heads][value_dim] (BF16, FP16 or FP32; q's dtype when
+    not given) at the rows' tokens, and lse [tokens][heads] FP32 when given; returns out. workspace: an FP32 tensor of
+    workspace_floats(partial rows, heads, partitions, value_dim) or more (default: one the module keeps per device and
+    owner, grown outside a capture). fused: one launch folds every partition itself, the same bits, no workspace.
+    flash (True or "cuda"): contiguous splits of `chunk` positions (default flash_chunk()), one per partition.
+    sinks: FP32 [heads] sink logits folded into each row's final state; sliding: a sliding window in positions.
+    multipliers: an "fp8" layer's (key, value) multipliers, or a [2][kv_heads] FP32 tensor (one per KV head).
+    parents, blocks, fresh and derive are not served. phases (a measurement's): 1 runs the split launch only, 2 the
+    merge only."""
+    if derive is not None:
+        raise _unsupported("derive= (keys derived from value rows)")
+    if parents is not None:
+        raise _unsupported("parents= (draft trees)")
+    if blocks is not None:
+        raise _unsupported("blocks= (block-sparse lists)")
+    if fresh is not None:
+        raise _unsupported("fresh= (a prompt chunk's own rows)")
+    k_kind = _check_kind(kind, key_scales)
+    _require_device(q, "attend's q")
+    T, hq, d = q.shape
+    _check_sinks(sinks, q)
+    sliding = _check_sliding(sliding, blocks)
+    hkv, dv = key_pages.shape[-2], value_pages.shape[-1]
+    R = int(starts.shape[0])
+    if hq % hkv or not 1 <= columns <= MAX_COLUMNS or R == 0:
+        raise ValueError("query heads a multiple of the KV heads, 1..64 columns a row, one row or more")
+    if q.stride(-1) != 1:
+        raise ValueError("q's last dimension is contiguous")
+    if d != dv or d not in (64, 128, 256):
+        raise ValueError("head dims are 64, 128 or 256, keys and values of one width")
+    want_q = torch.float16 if kind == "fp16" else torch.bfloat16
+    if q.dtype != want_q:
+        raise ValueError(f"q is {want_q} over {kind} pages, not {q.dtype}")
+    if (offsets is None) != (tokens is None):
+        raise ValueError("offsets come with the partial rows they take (tokens)")
+    if tables.dtype != torch.int32 or tables.stride(-1) != 1 or rows.dtype != torch.int32 or \
+            starts.dtype != torch.int32 or firsts.dtype != torch.int64:
+        raise ValueError("tables, rows and starts are int32 and firsts int64")
+    if counts is not None and counts.dtype != torch.int32 or offsets is not None and offsets.dtype != torch.int32:
+        raise ValueError("counts and offsets are int32")
+    partial_rows = R * columns if offsets is None else int(tokens)
+    device = q.device
+    block = flash_block(d, dv, hq, hkv, page, kind)
+    if flash:
+        piece = int(chunk or flash_chunk(d, dv, hq, hkv, page, kind))
+        if piece % block:
+            raise ValueError(f"a contiguous split ({piece} positions) is a multiple of the block ({block})")
+        parts = flash_parts(tables.shape[1] * page, piece)
+    else:
+        parts = int(partitions or globals()["partitions"](device, hkv, kind, d, dv))
+        piece = int(piece or piece_size(d, dv, kind, hkv))
+        if piece % block:
+            raise ValueError(f"a piece ({piece} positions) is a multiple of {block} at this head width")
+    scale = float(scale if scale is not None else d ** -0.5)
+    if fused:
+        po = pm = pl = None
+    else:
+        po, pm, pl = _workspace(device, partial_rows, hq, parts, dv, workspace)
+    if out is None:
+        out = torch.empty(T, hq, dv, dtype=q.dtype, device=device)
+    if out.dtype not in _DTYPE or out.stride(-1) != 1 or out.shape[-1] != dv:
+        raise ValueError("out is [tokens][heads][value_dim] BF16, FP16 or FP32, its last dimension contiguous")
+    if lse is not None and (lse.dtype != torch.float32 or not lse.is_contiguous()):
+        raise ValueError("lse is contiguous FP32 [tokens][heads]")
+    km, vm, per_head = _multipliers(multipliers, hkv, device)
+    p = _abi.AttendParams()
+    p.q, p.key_pages, p.value_pages = q.data_ptr(), key_pages.data_ptr(), value_pages.data_ptr()
+    p.key_scales, p.value_scales, p.head_multipliers = _ptr(key_scales), _ptr(value_scales), _ptr(per_head)
+    p.tables, p.rows, p.starts, p.counts = tables.data_ptr(), rows.data_ptr(), starts.data_ptr(), _ptr(counts)
+    p.firsts, p.offsets = firsts.data_ptr(), _ptr(offsets)
+    p.partial_out, p.partial_max, p.partial_sum = _ptr(po), _ptr(pm), _ptr(pl)
+    p.out, p.lse, p.sinks = out.data_ptr(), _ptr(lse), _ptr(sinks)
+    p.q_stride_t, p.q_stride_h, p.out_stride_t, p.out_stride_h = q.stride(0), q.stride(1), out.stride(0), out.stride(1)
+    p.table_stride, p.table_width = tables.stride(0), tables.shape[1]
+    p.n_rows, p.columns, p.heads, p.kv_heads, p.head_dim, p.value_dim, p.page = R, int(columns), hq, hkv, d, dv, int(page)
+    p.kind, p.page_dtype, p.out_dtype = k_kind, _page_dtype(key_pages, kind), _DTYPE[out.dtype]
+    p.partitions, p.piece, p.fused, p.sliding, p.phases = parts, piece, int(bool(fused)), sliding, int(phases)
+    p.scale, p.key_multiplier, p.value_multiplier = scale, km, vm
+    with torch.cuda.device(device):
+        _abi.check(_abi.load().crit_pkv_attend(p, _stream(device)), "paged_kv_attention.attend")
+    return out
+
+
+def merge_shards(outs, lses):
+    """Partials of the same queries over disjoint keys (outs [parts][tokens][heads][dim], lses [parts][tokens][heads]
+    FP32, -inf for a part with no key) -> (out FP32, lse FP32), the parts weighted by exp(lse - max): the device twin
+    of the partitioned-attention plugin's merge() (reference inference/partitioned-attention/plugin.py:52-64). A token
+    no part saw gets zeros and -inf. Not part of the reference module's interface."""
+    outs = outs if torch.is_tensor(outs) else torch.stack(list(outs))
+    lses = lses if torch.is_tensor(lses) else torch.stack(list(lses))
+    _require_device(outs, "merge_shards' outs")
+    if outs.dtype not in _DTYPE:
+        outs = outs.float()
+    outs, lses = outs.contiguous(), lses.float().contiguous()
+    parts, tokens, heads, dim = outs.shape
+    out = torch.empty(tokens, heads, dim, dtype=torch.float32, device=outs.device)
+    lse = torch.empty(tokens, heads, dtype=torch.float32, device=outs.device)
+    p = _abi.MergeParams()
+    p.outs, p.lses, p.out, p.lse = outs.data_ptr(), lses.data_ptr(), out.data_ptr(), lse.data_ptr()
+    p.rows, p.parts, p.value_dim, p.in_dtype = tokens * heads, parts, dim, _DTYPE[outs.dtype]
+    with torch.cuda.device(outs.device):
+        _abi.check(_abi.load().crit_pkv_merge(p, _stream(outs.device)), "paged_kv_attention.merge_shards")
+    return out, lse
+
+
+# -- prompt chunks -----------------------------------------------------------------------------------------------------------
+def _prefill_launch(q, key_pages, value_pages, kind, tables, table_rows, starts, counts, positions, max_count, chunks,
+                    page, key_scales, value_scales, multipliers, scale, out, lse, sinks, sliding):
+    k_kind = _check_kind(kind, key_scales)
+    _require_device(q, "prefill's q")
+    T, hq, d = q.shape
+    hkv = key_pages.shape[-2]
+    if value_pages.shape[-1] != d:
+        raise ValueError("prompt chunks read keys and values of one width")
+    if hq % hkv or q.stride(-1) != 1:
+        raise ValueError("query heads a multiple of the KV heads, q's last dimension contiguous")
+    want_q = torch.float16 if kind == "fp16" else torch.bfloat16
+    if q.dtype != want_q:
+        raise ValueError(f"q is {want_q} over {kind} pages, not {q.dtype}")
+    device = q.device
+    out = torch.empty_like(q) if out is None else out
+    if out.dtype not in _DTYPE or out.stride(-1) != 1:
+        raise ValueError("out is [tokens][heads][dim] BF16, FP16 or FP32, its last dimension contiguous")
+    if lse is not None and (lse.dtype != torch.float32 or lse.stride(-1) != 1 or lse.stride(0) != hq):
+        raise ValueError("lse is contiguous FP32 [tokens][heads]")
+    km, vm, per_head = _multipliers(multipliers, hkv, device)
+    p = _abi.PrefillParams()
+    p.q, p.key_pages, p.value_pages = q.data_ptr(), key_pages.data_ptr(), value_pages.data_ptr()
+    p.key_scales, p.value_scales, p.head_multipliers = _ptr(key_scales), _ptr(value_scales), _ptr(per_head)
+    if tables.dtype == torch.int32:
+        p.tables = tables.data_ptr()
+    elif tables.dtype == torch.int64:
+        p.tables64 = tables.data_ptr()
+    else:
+        raise ValueError("a page table is int32 or int64")
+    p.table_rows, p.starts, p.counts, p.positions = _ptr(table_rows), _ptr(starts), _ptr(counts), positions.data_ptr()
+    p.out, p.lse, p.sinks = out.data_ptr(), _ptr(lse), _ptr(sinks)
+    p.q_stride_t, p.q_stride_h, p.out_stride_t, p.out_stride_h = q.stride(0), q.stride(1), out.stride(0), out.stride(1)
+    p.table_stride = tables.stride(0) if tables.dim() == 2 else 0
+    p.table_width = tables.shape[-1]
+    p.chunks, p.max_count, p.heads, p.kv_heads, p.head_dim, p.page = chunks, max_count, hq, hkv, d, int(page)
+    p.kind, p.page_dtype, p.out_dtype = k_kind, _page_dtype(key_pages, kind), _DTYPE[out.dtype]
+    p.sliding = sliding
+    p.scale = float(scale if scale is not None else d ** -0.5)
+    p.key_multiplier, p.value_multiplier = km, vm
+    with torch.cuda.device(device):
+        _abi.check(_abi.load().crit_pkv_prefill(p, _stream(device)), "paged_kv_attention.prefill")
+    return out
+
+
+_positions = {}
+
+
+def prefill(q, key_pages, value_pages, kind, table, position, page, *, key_scales=None, value_scales=None,
+            multipliers=(1.0, 1.0), scale=None, out=None, lse=None, int8_qk=False, fresh=None, flash=False,
+            sinks=None, sliding=0, splits=None, workspace=None, derive=None):
+    """A prompt chunk of one sequence: q [T][heads][dim] at positions position.. (their keys and values written),
+    table [pages] int32 or int64 -> out [T][heads][dim] (and lse [T][heads] FP32 when given), causal. position: an
+    int, or a one-element int64 device tensor read on the device. One matrix-core launch whatever `flash` says; a
+    token's bits follow its own positions only. int8_qk, fresh and derive are not served."""
+    if derive is not None:
+        raise _unsupported("derive= (keys derived from value rows)")
+    if fresh is not None:
+        raise _unsupported("fresh= (a prompt chunk's own rows)")
+    if int8_qk:
+        raise _unsupported("int8_qk")
+    _check_sinks(sinks, q)
+    sliding = _check_sliding(sliding, None)
+    T = q.shape[0]
+    if T == 0:
+        return torch.empty_like(q) if out is None else out
+    if torch.is_tensor(position):
+        positions = position.reshape(1)
+        if positions.dtype != torch.int64 or positions.device != q.device:
+            raise ValueError("a device position is a one-element int64 tensor on q's device")
+    else:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("paged_kv_attention.prefill: a captured chunk takes its position as a device tensor")
+        positions = torch.tensor([int(position)], dtype=torch.int64, device=q.device)
+    return _prefill_launch(q, key_pages, value_pages, kind, table.reshape(1, -1), None, None, None, positions, T, 1,
+                           page, key_scales, value_scales, multipliers, scale, out, lse, sinks, sliding)
+
+
+def prefill_rows(q, key_pages, value_pages, kind, tables, table_rows, starts, counts, positions, max_count, page, *,
+                 key_scales=None, value_scales=None, multipliers=(1.0, 1.0), scale=None, out=None, lse=None,
+                 sinks=None, sliding=0):
+    """Several prompt chunks in one launch (where the reference launches prefill() once per row): chunk i is counts[i]
+    <= max_count tokens from token starts[i] of q at positions positions[i].. of the sequence whose page table is
+    tables[table_rows[i]]; tables [S][width] int32, table_rows/starts/counts [chunks] int32, positions [chunks] int64,
+    all on the device and read there. Not part of the reference module's interface."""
+    _check_sinks(sinks, q)
+    sliding = _check_sliding(sliding, None)
+    chunks = int(positions.shape[0])
+    if chunks == 0:
+        return torch.empty_like(q) if out is None else out
+    return _prefill_launch(q, key_pages, value_pages, kind, tables, table_rows, starts, counts, positions,
+                           int(max_count), chunks, page, key_scales, value_scales, multipliers, scale, out, lse, sinks,
+                           sliding)
+
+
+def stream_read(data, sink=None):
+    """Reads every byte of `data` (a contiguous device tensor, a multiple of 16 bytes) once with 16-byte loads: the
+    streaming-read yardstick the benchmark times beside the nominal HBM peak."""
+    _require_device(data, "stream_read's data")
+    nbytes = data.numel() * data.element_size()
+    sink = torch.zeros(64, dtype=torch.float32, device=data.device) if sink is None else sink
+    with torch.cuda.device(data.device):
+        _abi.check(_abi.load().crit_pkv_stream_read(data.data_ptr(), nbytes, sink.data_ptr(), _stream(data.device)),
+                   "paged_kv_attention.stream_read")
+    return sink

@@ -1,0 +1,129 @@
+"""ctypes mirror of include/crit_pkv.h and the loader of libcrit_pkv.so.
+
+The library is looked for at $CRIT_PKV_LIB, beside this package (a staged copy inside a crit kernel cache) and in
+crit_amd/lib (the in-tree build). If none exists and hipcc is on PATH it is built once, in-tree; otherwise loading
+fails: there is no other implementation behind this module.
+"""
+import ctypes
+import os
+import shutil
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+NAME = "libcrit_pkv.so"
+ABI_VERSION = 1
+
+KIND_16BIT, KIND_FP8, KIND_FP8_ROW, KIND_INT8 = 0, 1, 2, 3
+F32, BF16, F16 = 0, 1, 2
+
+_p, _i64, _i32, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_float
+
+
+class WriteParams(ctypes.Structure):
+    _fields_ = [("keys", _p), ("values", _p), ("slots", _p), ("key_pages", _p), ("value_pages", _p),
+                ("key_scales", _p), ("value_scales", _p), ("head_multipliers", _p),
+                ("tokens", _i64), ("key_stride_t", _i64), ("key_stride_h", _i64), ("value_stride_t", _i64),
+                ("value_stride_h", _i64),
+                ("kv_heads", _i32), ("head_dim", _i32), ("value_dim", _i32), ("kind", _i32), ("page_dtype", _i32),
+                ("in_dtype", _i32), ("key_multiplier", _f32), ("value_multiplier", _f32)]
+
+
+class AttendParams(ctypes.Structure):
+    _fields_ = [("q", _p), ("key_pages", _p), ("value_pages", _p), ("key_scales", _p), ("value_scales", _p),
+                ("head_multipliers", _p), ("tables", _p), ("rows", _p), ("starts", _p), ("counts", _p), ("firsts", _p),
+                ("offsets", _p), ("partial_out", _p), ("partial_max", _p), ("partial_sum", _p), ("out", _p),
+                ("lse", _p), ("sinks", _p),
+                ("q_stride_t", _i64), ("q_stride_h", _i64), ("out_stride_t", _i64), ("out_stride_h", _i64),
+                ("table_stride", _i64),
+                ("table_width", _i32), ("n_rows", _i32), ("columns", _i32), ("heads", _i32), ("kv_heads", _i32),
+                ("head_dim", _i32), ("value_dim", _i32), ("page", _i32), ("kind", _i32), ("page_dtype", _i32),
+                ("out_dtype", _i32), ("partitions", _i32), ("piece", _i32), ("fused", _i32), ("sliding", _i32), ("phases", _i32),
+                ("scale", _f32), ("key_multiplier", _f32), ("value_multiplier", _f32)]
+
+
+class MergeParams(ctypes.Structure):
+    _fields_ = [("outs", _p), ("lses", _p), ("out", _p), ("lse", _p), ("rows", _i64), ("parts", _i32),
+                ("value_dim", _i32), ("in_dtype", _i32)]
+
+
+class PrefillParams(ctypes.Structure):
+    _fields_ = [("q", _p), ("key_pages", _p), ("value_pages", _p), ("key_scales", _p), ("value_scales", _p),
+                ("head_multipliers", _p), ("tables", _p), ("tables64", _p), ("table_rows", _p), ("starts", _p),
+                ("counts", _p), ("positions", _p), ("out", _p), ("lse", _p), ("sinks", _p),
+                ("q_stride_t", _i64), ("q_stride_h", _i64), ("out_stride_t", _i64), ("out_stride_h", _i64),
+                ("table_stride", _i64),
+                ("table_width", _i32), ("chunks", _i32), ("max_count", _i32), ("heads", _i32), ("kv_heads", _i32),
+                ("head_dim", _i32), ("page", _i32), ("kind", _i32), ("page_dtype", _i32), ("out_dtype", _i32),
+                ("sliding", _i32), ("scale", _f32), ("key_multiplier", _f32), ("value_multiplier", _f32)]
+
+
+SYMBOLS = ("crit_pkv_write", "crit_pkv_attend", "crit_pkv_merge", "crit_pkv_prefill", "crit_pkv_abi_version",
+           "crit_pkv_params_size", "crit_pkv_error", "crit_pkv_stream_read")
+
+_lib = None
+
+
+def candidates():
+    found = []
+    if os.environ.get("CRIT_PKV_LIB"):
+        found.append(os.environ["CRIT_PKV_LIB"])
+    found.append(os.path.join(_HERE, NAME))
+    found.append(os.path.join(os.path.dirname(_HERE), "lib", NAME))
+    return found
+
+
+def _build_in_tree():
+    """The in-tree build (crit_amd/build.py), when this package sits inside crit_amd and hipcc exists."""
+    script = os.path.join(os.path.dirname(_HERE), "build.py")
+    if not os.path.exists(script) or shutil.which("hipcc") is None:
+        return None
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("_crit_pkv_build", script)
+    module = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(module)
+    return module.build(verbose=False)
+
+
+def load():
+    """The loaded library (a ctypes.CDLL with typed entry points); raises RuntimeError when it cannot be had."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = next((c for c in candidates() if os.path.exists(c)), None)
+    if path is None:
+        path = _build_in_tree()
+    if path is None:
+        raise RuntimeError(f"{NAME} is not built (looked in {', '.join(candidates())}) and hipcc is not available: "
+                           "run `python -m crit_amd.build`; this module has no other implementation")
+    lib = ctypes.CDLL(path)
+    for name in SYMBOLS:
+        if not hasattr(lib, name):
+            raise RuntimeError(f"{path} does not export {name}")
+    lib.crit_pkv_error.restype = ctypes.c_char_p
+    lib.crit_pkv_error.argtypes = [ctypes.c_int]
+    lib.crit_pkv_params_size.argtypes = [ctypes.c_int]
+    for name, struct in (("crit_pkv_write", WriteParams), ("crit_pkv_attend", AttendParams),
+                         ("crit_pkv_merge", MergeParams), ("crit_pkv_prefill", PrefillParams)):
+        fn = getattr(lib, name)
+        fn.restype = ctypes.c_int
+        fn.argtypes = [ctypes.POINTER(struct), ctypes.c_void_p]
+    lib.crit_pkv_stream_read.restype = ctypes.c_int
+    lib.crit_pkv_stream_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
+    if lib.crit_pkv_abi_version() != ABI_VERSION:
+        raise RuntimeError(f"{path} speaks ABI {lib.crit_pkv_abi_version()}, this package {ABI_VERSION}: rebuild it")
+    for which, struct in enumerate((WriteParams, AttendParams, MergeParams, PrefillParams)):
+        if lib.crit_pkv_params_size(which) != ctypes.sizeof(struct):
+            raise RuntimeError(f"{path}: parameter struct {which} is {lib.crit_pkv_params_size(which)} bytes, the "
+                               f"Python mirror {ctypes.sizeof(struct)}: rebuild the library")
+    lib.path = path
+    _lib = lib
+    return lib
+
+
+def check(code, what):
+    """Raise for a non-zero return of an entry point: ValueError for a refused launch, RuntimeError for a HIP error."""
+    if code == 0:
+        return
+    text = load().crit_pkv_error(code).decode()
+    if code < 0:
+        raise ValueError(f"{what}: {text}")
+    raise RuntimeError(f"{what}: HIP error {code}: {text}")

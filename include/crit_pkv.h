@@ -1,0 +1,174 @@
+/* crit_pkv: C ABI of the MI355X (gfx950) paged-KV kernels.
+ *
+ * The boundary a host binds (ctypes, cgo, JNI ...): plain pointers and sizes, one POD parameter struct per entry
+ * point, the caller's HIP stream. Every buffer is caller-owned device memory; the library owns none. Nothing here
+ * allocates, synchronises or reads a length on the host: row lengths and positions are read on the device, so one
+ * launch shape (a captured HIP graph) serves every length.
+ *
+ * Each entry point replaces the kernel launches behind one function of the reference's kernels module
+ * (kernels/techniques/attention/paged-kv-attention/torch-ext/paged_kv_attention/__init__.py); the pattern of the ABI
+ * (parameter struct mirrored by the host, int error codes, an error-string function, a params-size cross-check)
+ * follows the reference's own C ABI for its CUDA tile (cuda_window.cu:1482-1535).
+ *
+ * Return value of every launch: 0 = launched; > 0 = a HIP runtime error code; < 0 = one of CRIT_PKV_E_* (the launch
+ * was refused before anything ran). crit_pkv_error() names any of them.
+ */
+#ifndef CRIT_PKV_H
+#define CRIT_PKV_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CRIT_PKV_ABI_VERSION 1
+
+/* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
+#define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
+#define CRIT_PKV_KIND_FP8 1     /* E4M3FN codes, value = code * multiplier (per layer, or per KV head) */
+#define CRIT_PKV_KIND_FP8_ROW 2 /* E4M3FN codes, one FP32 scale per (slot, KV head) */
+#define CRIT_PKV_KIND_INT8 3    /* INT8 codes, one FP32 scale per (slot, KV head) */
+
+/* Element types of 16-bit/32-bit float buffers. */
+#define CRIT_PKV_F32 0
+#define CRIT_PKV_BF16 1
+#define CRIT_PKV_F16 2
+
+#define CRIT_PKV_E_GEOMETRY (-1)    /* shapes the kernels do not take (head dims, group size, columns, page, piece) */
+#define CRIT_PKV_E_DTYPE (-2)       /* a dtype/kind combination the kernels do not take */
+#define CRIT_PKV_E_NULL (-3)        /* a required pointer is NULL */
+#define CRIT_PKV_E_WORKSPACE (-4)   /* partitions/piece/workspace pointers inconsistent */
+
+#define CRIT_PKV_MAX_COLUMNS 64
+
+/* ---- append ------------------------------------------------------------------------------------------------------
+ * Replaces write() -> _write_kernel (__init__.py:289-324, _kernels.py:112-150); the torch rule it must reproduce
+ * bit for bit is KVPool.write (inference/attention-state/code/pages.py:439-453, 872-895).
+ * keys [tokens][kv_heads][head_dim], values [tokens][kv_heads][value_dim]: element (t, h, i) at
+ * base + t*stride_t + h*stride_h + i (strides in elements, last dimension contiguous). Pages: any storage laid out
+ * [slots][kv_heads][dim]; row (slot, head) starts at (slot*kv_heads + head)*dim. A slot below 0 is skipped.
+ * values/value_pages NULL: keys only. */
+typedef struct crit_pkv_write_params {
+    const void* keys;
+    const void* values;             /* NULL: keys only */
+    const int64_t* slots;           /* [tokens] */
+    void* key_pages;
+    void* value_pages;              /* NULL with values NULL */
+    float* key_scales;              /* [slots][kv_heads], kinds FP8_ROW and INT8; else NULL */
+    float* value_scales;
+    const float* head_multipliers;  /* optional [2][kv_heads] FP32 (keys' then values'), kind FP8: overrides the two
+                                       scalars below with one multiplier per KV head; NULL: the scalars */
+    int64_t tokens;
+    int64_t key_stride_t, key_stride_h, value_stride_t, value_stride_h;
+    int32_t kv_heads, head_dim, value_dim;
+    int32_t kind;                   /* CRIT_PKV_KIND_* */
+    int32_t page_dtype;             /* kind 16BIT: CRIT_PKV_BF16 or CRIT_PKV_F16 */
+    int32_t in_dtype;               /* CRIT_PKV_F32, _BF16 or _F16: the dtype of keys and values */
+    float key_multiplier, value_multiplier;   /* kind FP8: code = e4m3(clamp(x / multiplier, -448, 448)) */
+} crit_pkv_write_params;
+
+int crit_pkv_write(const crit_pkv_write_params* p, void* stream);
+
+/* ---- decode / verify windows ---------------------------------------------------------------------------------------
+ * Replaces attend() -> _window_kernel + _merge_kernel (__init__.py:396-576, _kernels.py:359-478, 558-604) and, with
+ * piece = the chunk and partitions = ceil(table positions / chunk), attend(flash=...) (__init__.py:641-712).
+ * Row r is counts[r] (<= columns) tokens of one sequence: tokens starts[r].. of q/out, column c at position
+ * firsts[r] + c, page table tables[rows[r]]; column c sees positions n <= firsts[r] + c (and n > firsts[r] + c -
+ * sliding when sliding > 0). Positions are read in pieces of `piece` positions; piece i belongs to partition
+ * i % partitions. Partition b of (row, column, head) writes its unnormalised output, running maximum and sum at
+ * index ((prow + c)*heads + head)*partitions + b of the three partial arrays, prow = offsets ? offsets[r] -
+ * offsets[0] : r*columns; the merge folds partitions 0 .. min(partitions, ceil((firsts[r]+c+1)/piece)) - 1 in order and
+ * writes out (and lse). fused != 0: one launch folds the partitions itself, same bits, no partial arrays. */
+typedef struct crit_pkv_attend_params {
+    const void* q;                  /* [tokens][heads][head_dim] bf16 or f16 */
+    const void* key_pages;
+    const void* value_pages;
+    const float* key_scales;        /* row-scaled kinds */
+    const float* value_scales;
+    const float* head_multipliers;  /* optional [2][kv_heads], kind FP8 */
+    const int32_t* tables;          /* [S][table_width] */
+    const int32_t* rows;            /* [n_rows] */
+    const int32_t* starts;          /* [n_rows] */
+    const int32_t* counts;          /* [n_rows] or NULL: `columns` each */
+    const int64_t* firsts;          /* [n_rows] */
+    const int32_t* offsets;         /* [n_rows] or NULL */
+    float* partial_out;             /* [partial rows * heads * partitions][value_dim] */
+    float* partial_max;             /* [partial rows * heads * partitions] (base-2 units) */
+    float* partial_sum;
+    void* out;                      /* [tokens][heads][value_dim], out_dtype */
+    float* lse;                     /* [tokens][heads] or NULL */
+    const float* sinks;             /* [heads] or NULL */
+    int64_t q_stride_t, q_stride_h, out_stride_t, out_stride_h, table_stride;
+    int32_t table_width, n_rows, columns, heads, kv_heads, head_dim, value_dim, page;
+    int32_t kind, page_dtype, out_dtype;
+    int32_t partitions, piece;
+    int32_t fused;
+    int32_t sliding;
+    int32_t phases;                 /* 0: the split launch then the merge; 1: the split launch only; 2: the merge only
+                                       (for timing one kernel; ignored when fused) */
+    float scale, key_multiplier, value_multiplier;
+} crit_pkv_attend_params;
+
+int crit_pkv_attend(const crit_pkv_attend_params* p, void* stream);
+
+/* ---- merge of shard partials ---------------------------------------------------------------------------------------
+ * Replaces PartitionedAttention.merge (inference/partitioned-attention/plugin.py:52-64): outs [parts][n][value_dim]
+ * (in_dtype), lses [parts][n] FP32 (-inf: the part saw no key) -> out [n][value_dim] FP32, lse [n] FP32, n = tokens
+ * * heads. A row no part saw gets zeros and -inf. */
+typedef struct crit_pkv_merge_params {
+    const void* outs;
+    const float* lses;
+    float* out;
+    float* lse;
+    int64_t rows;                   /* tokens * heads */
+    int32_t parts, value_dim, in_dtype;
+} crit_pkv_merge_params;
+
+int crit_pkv_merge(const crit_pkv_merge_params* p, void* stream);
+
+/* ---- prompt chunks ---------------------------------------------------------------------------------------------------
+ * Replaces prefill() -> _prefill_kernel (__init__.py:1245-1332, _kernels.py:610-726), and a batch of them in one
+ * launch (the reference launches one per row, device_attention.py:901-916).
+ * Chunk i is counts[i] tokens starting at token starts[i] of q/out, at positions positions[i] .. of the sequence whose
+ * page table is tables + table_rows[i]*table_stride; token t sees positions n <= positions[i] + t (causal). All
+ * metadata is on the device. max_count bounds counts[] (it sizes the grid). */
+typedef struct crit_pkv_prefill_params {
+    const void* q;
+    const void* key_pages;
+    const void* value_pages;
+    const float* key_scales;
+    const float* value_scales;
+    const float* head_multipliers;
+    const int32_t* tables;          /* int32 page tables, or ... */
+    const int64_t* tables64;        /* ... int64 ones (exactly one of the two is non-NULL) */
+    const int32_t* table_rows;      /* [chunks] or NULL: chunk i reads table row i */
+    const int32_t* starts;          /* [chunks] or NULL: 0 */
+    const int32_t* counts;          /* [chunks] or NULL: max_count */
+    const int64_t* positions;       /* [chunks] */
+    void* out;
+    float* lse;                     /* or NULL */
+    const float* sinks;             /* or NULL */
+    int64_t q_stride_t, q_stride_h, out_stride_t, out_stride_h, table_stride;
+    int32_t table_width, chunks, max_count, heads, kv_heads, head_dim, page;
+    int32_t kind, page_dtype, out_dtype;
+    int32_t sliding;
+    float scale, key_multiplier, value_multiplier;
+} crit_pkv_prefill_params;
+
+int crit_pkv_prefill(const crit_pkv_prefill_params* p, void* stream);
+
+/* ---- housekeeping ------------------------------------------------------------------------------------------------- */
+int crit_pkv_abi_version(void);
+/* sizeof() of the parameter structs as the library was compiled, for the host's mirror to cross-check
+ * (which: 0 write, 1 attend, 2 merge, 3 prefill), as crit_cw_params_size() does (cuda_window.cu:1502). */
+int crit_pkv_params_size(int which);
+const char* crit_pkv_error(int code);
+/* A streaming-read probe: sums `bytes` (a multiple of 16) of device memory into sink[0..63]; the achievable-HBM-read
+ * yardstick the benchmark prints beside the nominal peak. No counterpart in the reference. */
+int crit_pkv_stream_read(const void* data, int64_t bytes, float* sink, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

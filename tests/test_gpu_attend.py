@@ -1,0 +1,348 @@
+"""Paged decode / verify-window attention on the GPU against the CPU oracle (float64 attention over the stored values),
+and the bit-for-bit invariances the reference demands of its split-KV reader. Mirrors the reference's
+kernels/techniques/attention/paged-kv-attention/tests/test_paged_kv_attention.py:132-188, 275-297, 401-456, 501-512,
+tests/test_nonfinite.py, tests/test_sinks.py and tests/test_sliding.py. Tolerances: the reference's own (8e-3 abs +
+2e-2 rel, lse 1e-3), tighter than the 2e-2 (bf16) / 5e-2 (fp8) the task allows."""
+import pytest
+import torch
+
+from tests.support import KINDS, Cache, kernels, rand_q
+
+pytestmark = pytest.mark.gpu
+dev = "cuda"
+ATOL, RTOL = 8e-3, 2e-2
+
+
+def _close(got, want, what=None):
+    torch.testing.assert_close(got.double().cpu(), want, atol=ATOL, rtol=RTOL, msg=None if what is None else str(what))
+
+
+def _close_lse(got, want, what=None):
+    torch.testing.assert_close(got.double().cpu(), want, atol=1e-3, rtol=1e-4, msg=None if what is None else str(what))
+
+
+SHAPES = [(8, 2, 128, 128), (32, 8, 128, 128), (40, 8, 128, 128), (24, 4, 256, 256), (12, 2, 64, 64), (56, 8, 128, 128)]
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("hq,hkv,d,dv", SHAPES)
+@pytest.mark.parametrize("page", [16, 48])
+def test_windows_match_float64_attention(kind, hq, hkv, d, dv, page):
+    cache = Cache(kind, hkv, d, dv, page, [130, 64, 1, 517])
+    cols = 5
+    rows, starts, firsts, counts = [0, 1, 2, 3], [0, 5, 10, 15], [125, 59, 0, 400], [5, 5, 1, 3]
+    q = rand_q(20, hq, d, 3)
+    lse = torch.full((20, hq), 7.0, device=dev)
+    out = cache.attend(q, rows, starts, firsts, cols, lse=lse,
+                       counts=torch.tensor(counts, dtype=torch.int32, device=dev))
+    for s, start, first, count in zip(rows, starts, firsts, counts):
+        want, want_lse = cache.want(q[start:start + count], s, first, count)
+        _close(out[start:start + count], want, (s, first))
+        _close_lse(lse[start:start + count], want_lse, (s, first))
+    assert bool((lse[11:15] == 7.0).all()) and bool((lse[18:] == 7.0).all())      # only the rows' tokens are written
+
+
+def test_the_cpu_reference_configuration():
+    # batch 4, 8 query heads, 2 KV heads, head_dim 128, page 16, contexts {64, 200, 333, 512}, a seeded permutation of
+    # 128 physical pages, scale 1/sqrt(128); one new token appended per sequence, then attended.
+    pk = kernels()
+    g = torch.Generator().manual_seed(0)
+    lengths = [64, 200, 333, 512]
+    hq, hkv, d, page, n_pages = 8, 2, 128, 16, 128
+    perm = torch.randperm(n_pages, generator=g)
+    widths = [-(-(n + 1) // page) for n in lengths]
+    tables = torch.full((4, 48), n_pages, dtype=torch.int32)          # unused entries: the dump page
+    at = 0
+    for s, w in enumerate(widths):
+        tables[s, :w] = perm[at:at + w].to(torch.int32)
+        at += w
+    for kind, tol in (("bf16", 2e-2), ("fp8", 5e-2)):
+        store = torch.bfloat16 if kind == "bf16" else torch.float8_e4m3fn
+        k = torch.zeros(n_pages + 1, page, hkv, d, dtype=store, device=dev)
+        v = torch.zeros_like(k)
+        mult = (1.0, 1.0) if kind == "bf16" else (4.5 / 448, 4.5 / 448)
+        raw = []
+        from oracle import append as oa
+        for s, n in enumerate(lengths):
+            keys, values = torch.randn(n + 1, hkv, d, generator=g), torch.randn(n + 1, hkv, d, generator=g)
+            raw.append((keys, values))
+            slots = oa.slots(tables[s], torch.arange(n), page)
+            pk.write(keys[:n].to(dev), values[:n].to(dev), slots.to(dev), k, v, kind, multipliers=mult)
+        # the step: one new token per sequence
+        new_slots = torch.stack([oa.slots(tables[s], torch.tensor([n]), page)[0] for s, n in enumerate(lengths)])
+        pk.write(torch.stack([r[0][-1] for r in raw]).to(dev), torch.stack([r[1][-1] for r in raw]).to(dev),
+                 new_slots.to(dev), k, v, kind, multipliers=mult)
+        q = torch.randn(4, hq, d, generator=g)
+        out = pk.attend(q.to(dev).bfloat16(), k, v, kind, tables.to(dev), torch.arange(4, dtype=torch.int32, device=dev),
+                        torch.arange(4, dtype=torch.int32, device=dev),
+                        torch.tensor(lengths, dtype=torch.int64, device=dev), 1, page, multipliers=mult, scale=d ** -0.5)
+        from oracle import attend as oatt
+        for s, n in enumerate(lengths):
+            want, _ = oatt.window_reference(q[s:s + 1], k.cpu(), v.cpu(), kind, tables[s], n, 1, page, d ** -0.5,
+                                            multipliers=mult)
+            torch.testing.assert_close(out[s:s + 1].double().cpu(), want, atol=tol, rtol=tol)
+            # and against the raw (unquantised) FP32 inputs through the reference's CPU path: gather + SDPA in FP32
+            exact = torch.nn.functional.scaled_dot_product_attention(
+                q[s].view(1, hq, 1, d), raw[s][0].transpose(0, 1).unsqueeze(0), raw[s][1].transpose(0, 1).unsqueeze(0),
+                scale=d ** -0.5, enable_gqa=True)[0, :, 0]
+            torch.testing.assert_close(out[s].float().cpu(), exact, atol=tol, rtol=tol)
+
+
+@pytest.mark.parametrize("kind", ["bf16", "fp8", "fp8:row", "int8"])
+def test_rows_and_columns_are_invariant_bit_for_bit(kind):
+    pk = kernels()
+    cache = Cache(kind, 4, 128, 128, 16, [700, 300, 2100])
+    q = rand_q(24, 16, 128, 5)
+    together = cache.attend(q, [0, 1, 2], [0, 8, 16], [690, 290, 2090], 8)
+    for s, start, first in zip([0, 1, 2], [0, 8, 16], [690, 290, 2090]):
+        alone = cache.attend(q[start:start + 8], [s], [0], [first], 8)
+        assert torch.equal(alone, together[start:start + 8])
+        for c in range(8):    # each column decoded alone, in a launch of one column
+            one = cache.attend(q[start + c:start + c + 1], [s], [0], [first + c], 1)
+            assert torch.equal(one[0], together[start + c]), (s, c)
+        wide = cache.attend(q[start:start + 8], [s], [0], [first], 16,
+                            counts=torch.tensor([8], dtype=torch.int32, device=dev))
+        assert torch.equal(wide, together[start:start + 8])
+    counts = torch.tensor([3, 1, 4], dtype=torch.int32, device=dev)
+    offsets = torch.tensor([0, 3, 4], dtype=torch.int32, device=dev)
+    floats = pk.workspace_floats(8, 16, pk.partitions(dev, 4, kind), 128)
+    packed = cache.attend(q, [0, 1, 2], [0, 8, 16], [690, 290, 2090], 8, counts=counts, offsets=offsets, tokens=8,
+                          workspace=torch.full((floats,), float("nan"), dtype=torch.float32, device=dev))
+    for start, count in zip([0, 8, 16], [3, 1, 4]):
+        assert torch.equal(packed[start:start + count], together[start:start + count])
+
+
+def test_a_count_past_the_columns_reads_as_the_columns():
+    cache = Cache("bf16", 2, 128, 128, 16, [300, 300])
+    q = rand_q(8, 8, 128, 11)
+    want = cache.attend(q, [0, 1], [0, 4], [290, 280], 4)
+    got = cache.attend(q, [0, 1], [0, 4], [290, 280], 4, counts=torch.tensor([9, 4], dtype=torch.int32, device=dev))
+    assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("kind", ["bf16", "fp8", "int8"])
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (24, 4, 256)])
+def test_a_fused_launch_gives_a_column_the_split_launchs_bits(kind, hq, hkv, d):
+    for length in (40, 700, 5000):
+        cache = Cache(kind, hkv, d, d, 64, [length], seed=1)
+        T = min(130, length)
+        pos0 = length - T
+        q = rand_q(T, hq, d, 2)
+        starts = list(range(0, T, 64))
+        counts = torch.tensor([min(64, T - s) for s in starts], dtype=torch.int32, device=dev)
+        lse, one_lse = torch.empty(T, hq, device=dev), torch.empty(T, hq, device=dev)
+        fused = cache.attend(q, [0] * len(starts), starts, [pos0 + s for s in starts], 64, counts=counts, fused=True,
+                             lse=lse)
+        alone = cache.attend(q, [0] * T, list(range(T)), [pos0 + i for i in range(T)], 1, lse=one_lse)
+        assert torch.equal(fused, alone), (kind, length)
+        assert torch.equal(lse, one_lse), (kind, length)
+        want, want_lse = cache.want(q[:3], 0, pos0, 3)
+        _close(fused[:3], want)
+        _close_lse(lse[:3], want_lse)
+
+
+def test_a_given_workspace_holds_the_partials_and_a_small_one_is_refused():
+    pk = kernels()
+    cache = Cache("bf16", 2, 128, 128, 16, [300])
+    q = rand_q(4, 8, 128, 9)
+    floats = pk.workspace_floats(4, 8, 16, 128)
+    own = cache.attend(q, [0], [0], [296], 4, partitions=16)
+    given = cache.attend(q, [0], [0], [296], 4, partitions=16,
+                         workspace=torch.full((floats,), float("nan"), dtype=torch.float32, device=dev))
+    assert torch.equal(own, given)
+    with pytest.raises(ValueError, match="workspace"):
+        cache.attend(q, [0], [0], [296], 4, partitions=16,
+                     workspace=torch.empty(floats - 1, dtype=torch.float32, device=dev))
+
+
+@pytest.mark.parametrize("kind,chunk", [("bf16", 512), ("bf16", 1024), ("fp8", 2048)])
+def test_contiguous_splits_match_float64_and_do_not_depend_on_the_table_width(kind, chunk):
+    cache = Cache(kind, 8, 128, 128, 16, [5000, 900])
+    q = rand_q(2, 40, 128, 21)
+    lse = torch.empty(2, 40, device=dev)
+    out = cache.attend(q, [0, 1], [0, 1], [4999, 899], 1, flash=True, chunk=chunk, lse=lse)
+    for s, first in ((0, 4999), (1, 899)):
+        want, want_lse = cache.want(q[s:s + 1], s, first, 1)
+        _close(out[s:s + 1], want)
+        _close_lse(lse[s:s + 1], want_lse)
+    # a wider table (more splits in the grid, none of them holding a position) changes no bit
+    wider = torch.cat([cache.tables, torch.zeros(2, 4096, dtype=torch.int32, device=dev)], 1).contiguous()
+    narrow, cache.tables = cache.tables, wider
+    again = cache.attend(q, [0, 1], [0, 1], [4999, 899], 1, flash=True, chunk=chunk)
+    cache.tables = narrow
+    assert torch.equal(again, out)
+
+
+def test_one_graph_replays_at_every_length():
+    pk = kernels()
+    cache = Cache("fp8:row", 4, 128, 128, 16, [5000, 5000])
+    q = rand_q(10, 16, 128, 8).to(torch.bfloat16)
+    rows = torch.tensor([0, 1], dtype=torch.int32, device=dev)
+    starts = torch.tensor([0, 5], dtype=torch.int32, device=dev)
+    firsts = torch.tensor([10, 20], dtype=torch.int64, device=dev)
+    out = torch.empty(10, 16, 128, dtype=torch.bfloat16, device=dev)
+    workspace = torch.empty(pk.workspace_floats(10, 16, pk.partitions(dev, 4, "fp8:row"), 128), dtype=torch.float32,
+                            device=dev)
+
+    def launch(into):
+        return pk.attend(q, cache.k, cache.v, "fp8:row", cache.tables, rows, starts, firsts, 5, 16,
+                         key_scales=cache.ks, value_scales=cache.vs, out=into, workspace=workspace)
+    launch(out)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        launch(out)
+    for a, b in ((10, 20), (4000, 63), (64, 4990), (1, 2)):
+        firsts.copy_(torch.tensor([a, b], device=dev))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        eager = launch(torch.empty_like(out))
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), (a, b)
+
+
+def test_work_follows_the_rows_length_not_the_capacity():
+    # Every position past the row's own is poisoned (NaN scales) before the launch: a read of any would show.
+    pk = kernels()
+    cache = Cache("fp8:row", 4, 128, 128, 64, [20_000])
+    q = rand_q(1, 16, 128, 1).to(torch.bfloat16)
+    args = lambda firsts: (q, cache.k, cache.v, "fp8:row", cache.tables, torch.zeros(1, dtype=torch.int32, device=dev),
+                           torch.zeros(1, dtype=torch.int32, device=dev), firsts, 1, 64)
+    kw = dict(key_scales=cache.ks, value_scales=cache.vs)
+    for first in (19_000, 4_000):
+        firsts = torch.tensor([first], device=dev)
+        want = pk.attend(*args(firsts), **kw).clone()
+        past = cache.slots(0, torch.arange(first + 1, 20_000, device=dev))
+        cache.ks.view(-1, 4)[past] = float("nan")
+        cache.vs.view(-1, 4)[past] = float("nan")
+        got = pk.attend(*args(firsts), **kw)
+        assert bool(torch.isfinite(got).all()), first
+        assert torch.equal(got, want), first
+
+
+def test_a_nan_query_poisons_only_its_own_token_and_head():
+    cache = Cache("bf16", 2, 128, 128, 16, [300, 300])
+    q = rand_q(4, 8, 128, 4)
+    clean = cache.attend(q, [0, 1], [0, 2], [298, 298], 2)
+    q[1, 3, 7] = float("nan")
+    dirty = cache.attend(q, [0, 1], [0, 2], [298, 298], 2)
+    assert bool(torch.isnan(dirty[1, 3]).all())
+    mask = torch.ones(4, 8, dtype=torch.bool, device=dev)
+    mask[1, 3] = False
+    assert torch.equal(dirty[mask], clean[mask])
+
+
+def test_a_window_of_one_position_returns_that_positions_value():
+    cache = Cache("bf16", 2, 128, 128, 16, [40])
+    q = rand_q(1, 8, 128, 4)
+    one = cache.attend(q, [0], [0], [5], 1, sliding=1)
+    stored = cache.v.view(-1, 2, 128)[cache.slots(0, torch.tensor([5]))][0]         # [hkv][dv]
+    assert torch.equal(one[0], stored.repeat_interleave(4, 0))
+    zero = cache.attend(q, [0], [0], [0], 1)                                       # position 0 sees itself only
+    stored = cache.v.view(-1, 2, 128)[cache.slots(0, torch.tensor([0]))][0]
+    assert torch.equal(zero[0], stored.repeat_interleave(4, 0))
+
+
+@pytest.mark.parametrize("kind", ["bf16", "fp8:row"])
+@pytest.mark.parametrize("window", [1, 100, 128, 1000])
+def test_a_sliding_window_sees_only_its_last_positions(kind, window):
+    cache = Cache(kind, 2, 128, 128, 16, [3000])
+    q = rand_q(4, 8, 128, 4)
+    lse = torch.empty(4, 8, device=dev)
+    out = cache.attend(q, [0], [0], [2996], 4, sliding=window, lse=lse)
+    want, want_lse = cache.want(q, 0, 2996, 4, sliding=window)
+    _close(out, want)
+    _close_lse(lse, want_lse)
+    for c in range(4):
+        one = cache.attend(q[c:c + 1], [0], [0], [2996 + c], 1, sliding=window)
+        assert torch.equal(one[0], out[c])
+
+
+def test_sinks_add_one_valueless_position_to_every_softmax():
+    cache = Cache("bf16", 2, 128, 128, 16, [500])
+    q = rand_q(2, 8, 128, 4)
+    sinks = torch.tensor([0.0, 1.0, -1.0, float("-inf"), 3.0, 0.5, -0.5, 2.0], device=dev)
+    lse, plain_lse = torch.empty(2, 8, device=dev), torch.empty(2, 8, device=dev)
+    out = cache.attend(q, [0], [0], [498], 2, sinks=sinks, lse=lse)
+    plain = cache.attend(q, [0], [0], [498], 2, lse=plain_lse)
+    # out = plain * sum / (sum + e^sink); lse = log(e^plain_lse + e^sink)
+    weight = torch.exp(plain_lse) / (torch.exp(plain_lse) + torch.exp(sinks)[None, :])
+    torch.testing.assert_close(out.float(), plain.float() * weight[..., None], atol=8e-3, rtol=2e-2)
+    torch.testing.assert_close(lse, torch.logaddexp(plain_lse, sinks[None, :].expand(2, 8)), atol=1e-3, rtol=1e-4)
+    assert torch.equal(out[:, 3], plain[:, 3])
+    fused = cache.attend(q, [0], [0], [498], 2, sinks=sinks, fused=True)
+    assert torch.equal(fused, out)
+
+
+def test_outputs_in_fp32_and_fp16_pages():
+    cache = Cache("fp16", 2, 128, 128, 16, [333])
+    q = rand_q(1, 8, 128, 4)
+    out32 = torch.empty(1, 8, 128, dtype=torch.float32, device=dev)
+    cache.attend(q, [0], [0], [332], 1, out=out32)
+    want, _ = cache.want(q, 0, 332, 1)
+    _close(out32, want)
+    out16 = cache.attend(q, [0], [0], [332], 1)
+    assert out16.dtype == torch.float16
+    assert torch.equal(out32.half(), out16)
+
+
+def test_later_launches_of_a_step_take_absolute_offsets():
+    # DeviceAttention hands a later launch cloned slices whose offsets keep their absolute values: the partial rows
+    # count from the launch's first row (inference/attention-state/code/device_attention.py:692-699).
+    cache = Cache("bf16", 2, 128, 128, 16, [300, 300, 300])
+    q = rand_q(3, 8, 128, 4)
+    whole = cache.attend(q, [0, 1, 2], [0, 1, 2], [299, 299, 299], 1,
+                         counts=torch.ones(3, dtype=torch.int32, device=dev),
+                         offsets=torch.tensor([0, 1, 2], dtype=torch.int32, device=dev), tokens=3)
+    out = torch.zeros_like(whole)
+    pk = kernels()
+    floats = pk.workspace_floats(2, 8, pk.partitions(dev, 2, "bf16"), 128)
+    cache.attend(q, [1, 2], [1, 2], [299, 299], 1, counts=torch.ones(2, dtype=torch.int32, device=dev),
+                 offsets=torch.tensor([1, 2], dtype=torch.int32, device=dev), tokens=2, out=out,
+                 workspace=torch.empty(floats, dtype=torch.float32, device=dev))
+    assert torch.equal(out[1:], whole[1:]) and not bool(out[0].any())
+
+
+def test_merge_shards_equals_attention_over_the_whole_sequence():
+    # inference/partitioned-attention/tests/test_device.py:44-77
+    pk = kernels()
+    g = torch.Generator().manual_seed(1)
+    keys, values = torch.randn(300, 2, 128, generator=g), torch.randn(300, 2, 128, generator=g)
+    q = torch.randn(1, 4, 128, generator=g).to(dev)
+    caches = {}
+    for name, (a, b) in {"s": (0, 300), "a": (0, 120), "b": (120, 300)}.items():
+        c = Cache("bf16", 2, 128, 128, 16, [b - a], seed=7)
+        c.write(0, 0, keys[a:b].to(dev), values[a:b].to(dev))
+        caches[name] = c
+
+    def step(c, n):
+        lse = torch.empty(1, 4, device=dev)
+        return c.attend(q, [0], [0], [n - 1], 1, lse=lse), lse
+    out, lse = step(caches["s"], 300)
+    parts = [step(caches["a"], 120), step(caches["b"], 180)]
+    merged, merged_lse = pk.merge_shards([o for o, _ in parts], [x for _, x in parts])
+    torch.testing.assert_close(merged, out.float(), atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(merged_lse, lse, atol=2e-3, rtol=1e-4)
+    from oracle import attend as oatt
+    want, want_lse = oatt.merge([o.cpu() for o, _ in parts], [x.cpu() for _, x in parts])
+    torch.testing.assert_close(merged.cpu(), want, atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(merged_lse.cpu(), want_lse, atol=1e-5, rtol=1e-5)
+    outs = [torch.ones(2, 1, 128, device=dev), torch.zeros(2, 1, 128, device=dev)]
+    lses = [torch.tensor([[0.5], [float("-inf")]], device=dev), torch.full((2, 1), float("-inf"), device=dev)]
+    o, l = pk.merge_shards(outs, lses)
+    assert bool((o[0] == 1).all()) and not bool(o[1].any()) and float(l[1, 0]) == float("-inf")
+    assert abs(float(l[0, 0]) - 0.5) < 1e-6
+
+
+def test_bad_geometry_is_refused():
+    cache = Cache("bf16", 2, 128, 128, 16, [100])
+    q = rand_q(1, 8, 128, 4)
+    with pytest.raises(ValueError):
+        cache.attend(q, [0], [0], [99], 65)
+    with pytest.raises(ValueError):
+        cache.attend(q[:, :7], [0], [0], [99], 1)
+    with pytest.raises(ValueError, match="offsets"):
+        cache.attend(q, [0], [0], [99], 1, offsets=torch.zeros(1, dtype=torch.int32, device=dev))
+    with pytest.raises(NotImplementedError):
+        cache.attend(q, [0], [0], [99], 1, parents=torch.tensor([-1], device=dev))

@@ -1,0 +1,162 @@
+"""KV append on the GPU against the CPU oracle: every stored byte (and row scale) equal, skipped slots untouched.
+Mirrors the reference's kernels/techniques/attention/paged-kv-attention/tests/test_paged_kv_attention.py:88-126,
+482-498. Calls go through the kernels module, which reaches the HIP kernels through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import append as oracle_append
+from oracle import e4m3
+from tests.support import KINDS, STORE, bits, expected_pages, kernels
+
+pytestmark = pytest.mark.gpu
+dev = "cuda"
+
+
+def _check(kind, got, want):
+    for name, g, w in zip(("keys", "values", "key scales", "value scales"), got, want):
+        if w is None:
+            continue
+        assert torch.equal(bits(g.cpu()).reshape(-1), bits(w).reshape(-1)), (kind, name)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("d,dv", [(128, 128), (64, 128), (256, 256)])
+@pytest.mark.parametrize("in_dtype", [torch.float32, torch.bfloat16])
+def test_writes_encode_as_torch_does_and_skip_negative_slots(kind, d, dv, in_dtype):
+    pk = kernels()
+    g = torch.Generator().manual_seed(1)
+    keys = (torch.randn(40, 3, d, generator=g) * 3).to(in_dtype)
+    values = torch.randn(40, 3, dv, generator=g).to(in_dtype)
+    keys[5] = 0.0
+    k = torch.zeros(64, 3, d, dtype=STORE[kind], device=dev)
+    v = torch.zeros(64, 3, dv, dtype=STORE[kind], device=dev)
+    ks = vs = None
+    if kind in ("fp8:row", "int8"):
+        ks, vs = torch.zeros(64, 3, device=dev), torch.zeros(64, 3, device=dev)
+    slots = torch.randperm(64, generator=g)[:40]
+    slots[7] = -1
+    mult = (0.05, 0.07)
+    pk.write(keys.to(dev), values.to(dev), slots.to(dev), k, v, kind, ks, vs, multipliers=mult)
+    _check(kind, (k, v, ks, vs), expected_pages(kind, keys, values, slots, 64, mult))
+
+
+@pytest.mark.parametrize("kind", ["bf16", "fp8", "fp8:row", "int8"])
+def test_a_large_append_with_edge_values_is_bit_exact(kind):
+    # 4,152 tokens (the mixed prefill + decode batch's append), 8 KV heads, with the values that break sloppy
+    # encoders: signed zeros, the subnormal ties, saturation, infinities, 1% outliers x20.
+    pk = kernels()
+    g = torch.Generator().manual_seed(2)
+    T, hkv, d = 4152, 8, 128
+    keys, values = torch.randn(T, hkv, d, generator=g), torch.randn(T, hkv, d, generator=g)
+    hot = torch.rand(T, hkv, d, generator=g) < 0.01
+    keys = torch.where(hot, keys * 20, keys)
+    mult = (0.04, 0.06)
+    edge = torch.tensor([0.0, -0.0, 2.0 ** -10, -(2.0 ** -10), 2.0 ** -9, 448.0, -448.0, 449.0, 1e30, -1e30,
+                         float("inf"), float("-inf"), 1e-30, 0.0146484375, 432.0, 248.0])
+    keys[0, 0, :16] = edge * mult[0]
+    values[1, 2, :16] = edge * mult[1]
+    n_slots = 8192
+    slots = torch.randperm(n_slots, generator=g)[:T]
+    slots[100] = -1
+    slots[4000] = -5
+    k = torch.zeros(n_slots, hkv, d, dtype=STORE[kind], device=dev)
+    v = torch.zeros(n_slots, hkv, d, dtype=STORE[kind], device=dev)
+    ks = vs = None
+    if kind in ("fp8:row", "int8"):
+        ks, vs = torch.zeros(n_slots, hkv, device=dev), torch.zeros(n_slots, hkv, device=dev)
+    if kind in ("fp8:row", "int8"):      # an infinite row maximum makes every quotient NaN: keep the rows finite there
+        keys = torch.nan_to_num(keys, posinf=3e4, neginf=-3e4)
+        values = torch.nan_to_num(values, posinf=3e4, neginf=-3e4)
+    pk.write(keys.to(dev), values.to(dev), slots.to(dev), k, v, kind, ks, vs, multipliers=mult)
+    _check(kind, (k, v, ks, vs), expected_pages(kind, keys, values, slots, n_slots, mult))
+
+
+def test_fp8_codes_on_every_97th_bit_pattern_equal_torchs_cast_and_the_reference_vectors():
+    # The reference's own check of its encoder (kernels/core/tests/test_core_triton.py:68-77), through write().
+    pk = kernels()
+    top = int(np.float32(448.0).view(np.uint32))
+    pos = np.arange(0, top + 1, 97, dtype=np.uint32)
+    allbits = np.concatenate([pos, pos | np.uint32(0x80000000)])
+    allbits = np.concatenate([allbits, np.zeros((-len(allbits)) % 128, dtype=np.uint32)])
+    x = torch.from_numpy(allbits.view(np.float32).copy()).view(-1, 1, 128)
+    T = x.shape[0]
+    k = torch.zeros(T, 1, 128, dtype=torch.float8_e4m3fn, device=dev)
+    pk.write(x.to(dev), None, torch.arange(T, device=dev), k, None, "fp8", multipliers=(1.0, 1.0))
+    want = x.clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8)
+    assert torch.equal(k.cpu().view(torch.uint8), want)
+    assert np.array_equal(e4m3.encode(x.numpy().reshape(-1)), want.numpy().reshape(-1))
+
+
+@pytest.mark.parametrize("kind", ["bf16", "fp8:row", "int8"])
+def test_key_only_writes_leave_no_values(kind):
+    pk = kernels()
+    g = torch.Generator().manual_seed(3)
+    keys = torch.randn(20, 1, 64, generator=g).to(dev)
+    k = torch.zeros(32, 1, 64, dtype=STORE[kind], device=dev)
+    ks = torch.zeros(32, 1, device=dev) if kind != "bf16" else None
+    slots = torch.arange(20, device=dev) + 5
+    pk.write(keys, None, slots, k, None, kind, ks, None)
+    both = torch.zeros_like(k)
+    other = torch.zeros(32, 1, 64, dtype=STORE[kind], device=dev)
+    both_s = torch.zeros(32, 1, device=dev) if ks is not None else None
+    pk.write(keys, keys, slots, both, other, kind, both_s, torch.zeros_like(both_s) if ks is not None else None)
+    assert torch.equal(bits(k), bits(both))
+    if ks is not None:
+        assert torch.equal(ks, both_s)
+    want = expected_pages(kind, keys.cpu(), keys.cpu(), slots.cpu(), 32, (1.0, 1.0))
+    assert torch.equal(bits(k.cpu()), bits(want[0]))
+
+
+def test_values_only_writes_use_the_value_multiplier():
+    pk = kernels()
+    g = torch.Generator().manual_seed(4)
+    values = torch.randn(9, 2, 128, generator=g)
+    v = torch.zeros(16, 2, 128, dtype=torch.float8_e4m3fn, device=dev)
+    slots = torch.arange(9)
+    pk.write(None, values.to(dev), slots.to(dev), None, v, "fp8", multipliers=(0.5, 0.03))
+    want = oracle_append.encode(values, "fp8", 0.03)[0]
+    assert torch.equal(v.cpu().view(torch.uint8)[:9], want.view(torch.uint8))
+
+
+def test_one_multiplier_per_kv_head():
+    pk = kernels()
+    g = torch.Generator().manual_seed(5)
+    keys, values = torch.randn(33, 8, 128, generator=g), torch.randn(33, 8, 128, generator=g)
+    mults = torch.rand(2, 8, generator=g) * 0.1 + 0.01
+    k = torch.zeros(64, 8, 128, dtype=torch.float8_e4m3fn, device=dev)
+    v = torch.zeros_like(k)
+    slots = torch.randperm(64, generator=g)[:33]
+    pk.write(keys.to(dev), values.to(dev), slots.to(dev), k, v, "fp8", multipliers=mults.to(dev))
+    want = expected_pages("fp8", keys, values, slots, 64, (mults[0], mults[1]))
+    _check("fp8", (k, v, None, None), want)
+
+
+def test_odd_widths_and_strided_inputs_take_the_scalar_path():
+    pk = kernels()
+    g = torch.Generator().manual_seed(6)
+    big = torch.randn(12, 2, 3, 80, generator=g)
+    keys, values = big[:, :, 0], big[:, :, 2, :40]            # head stride 240, token stride 480; widths 80 and 40
+    for kind in ("bf16", "fp8", "int8"):
+        k = torch.zeros(16, 2, 80, dtype=STORE[kind], device=dev)
+        v = torch.zeros(16, 2, 40, dtype=STORE[kind], device=dev)
+        ks = vs = None
+        if kind == "int8":
+            ks, vs = torch.zeros(16, 2, device=dev), torch.zeros(16, 2, device=dev)
+        slots = torch.randperm(16, generator=g)[:12]
+        bigd = big.to(dev)
+        pk.write(bigd[:, :, 0], bigd[:, :, 2, :40], slots.to(dev), k, v, kind, ks, vs, multipliers=(0.1, 0.2))
+        _check(kind, (k, v, ks, vs), expected_pages(kind, keys, values, slots, 16, (0.1, 0.2)))
+
+
+def test_bad_arguments_are_refused():
+    pk = kernels()
+    k = torch.zeros(4, 1, 64, dtype=torch.bfloat16, device=dev)
+    x = torch.zeros(2, 1, 64, device=dev)
+    with pytest.raises(ValueError):
+        pk.write(None, None, torch.zeros(2, dtype=torch.int64, device=dev), None, None, "bf16")
+    with pytest.raises(ValueError, match="page kinds"):
+        pk.write(x, None, torch.zeros(2, dtype=torch.int64, device=dev), k, None, "fp4")
+    with pytest.raises(ValueError, match="scales"):
+        pk.write(x, None, torch.zeros(2, dtype=torch.int64, device=dev), k, None, "int8")
+    pk.write(x[:0], None, torch.zeros(0, dtype=torch.int64, device=dev), k, None, "bf16")     # no tokens: nothing
