@@ -1,0 +1,300 @@
+"""Benchmark of the paged-KV hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3] [--no-extras] [--no-cpu]
+
+A step is one pass of the hot path over one synthetic batch: for each of 32 layers, one KV append (one new token per
+sequence) and one paged decode attention over the whole context. The default workload is the Llama-3-8B-shaped bf16
+configuration (32 query heads, 8 KV heads, head_dim 128, page 16, batch 64, contexts uniform in [1024, 8192], pages
+randomly permuted in a pool 1.25x the needed size). Inputs are resident in HBM before the timed region starts.
+
+Prints ONE JSON line on stdout (everything else goes to stderr): the whole-step rate in algorithmic GB/s, the decode
+kernel's roofline fraction from HIP-event timing of that kernel alone, and the reference's CPU path (gather + SDPA and
+index_copy append, FP32, restated in oracle/) timed on this host on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, vendor figure
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+WORKLOADS = {
+    # name: (kind, batch, ctx_lo, ctx_hi, hq, hkv, d, layers, value scale, outliers)
+    "c2": dict(kind="bf16", batch=64, lo=1024, hi=8192, hq=32, hkv=8, d=128, layers=32, std=0.5, outliers=False,
+               name="llama3-8b-shaped paged decode, bf16 KV: B=64, ctx~U[1024,8192], 32q/8kv x128, page 16, 32 layers x (append + attend)"),
+    "c3": dict(kind="fp8", batch=128, lo=2048, hi=16384, hq=32, hkv=8, d=128, layers=32, std=1.0, outliers=True,
+               name="llama3-8b-shaped paged decode, FP8 E4M3 KV (per-(layer, kv-head) scales): B=128, ctx~U[2048,16384], 32 layers x (append + attend)"),
+}
+
+
+class Workload:
+    def __init__(self, spec, device, seed=0, layers=None):
+        import crit_amd.paged_kv_attention as pk
+        self.pk, self.spec, self.device = pk, spec, device
+        g = torch.Generator().manual_seed(seed)
+        B, page = spec["batch"], 16
+        self.page, self.kind = page, spec["kind"]
+        self.layers = layers or spec["layers"]
+        hkv, d, hq = spec["hkv"], spec["d"], spec["hq"]
+        # ctx = positions already in the cache; the step appends position ctx and attends over ctx + 1 positions
+        self.ctx = torch.randint(spec["lo"], spec["hi"] + 1, (B,), generator=g)
+        need = int(((self.ctx + 1 + page - 1) // page).sum())
+        self.n_pages = int(need * 1.25)
+        perm = torch.randperm(self.n_pages, generator=g)
+        width = int(((self.ctx.max() + 1 + page - 1) // page + 15) // 16 * 16)
+        tables = torch.full((B, width), self.n_pages, dtype=torch.int32)      # unused entries: the dump page
+        at = 0
+        for s in range(B):
+            w = int((self.ctx[s] + 1 + page - 1) // page)
+            tables[s, :w] = perm[at:at + w].to(torch.int32)
+            at += w
+        self.tables = tables.to(device)
+        store = torch.bfloat16 if self.kind == "bf16" else torch.float8_e4m3fn
+        self.k, self.v = [], []
+        gen = torch.Generator(device=device).manual_seed(seed)
+        self.mult = []
+        for layer in range(self.layers):
+            shape = (self.n_pages + 1, page, hkv, d)
+            pages = []
+            for _ in range(2):
+                x = torch.randn(shape, device=device, dtype=torch.bfloat16, generator=gen) * spec["std"]
+                if spec["outliers"]:
+                    hot = torch.rand(shape, device=device, generator=gen) < 0.01
+                    x = torch.where(hot, x * 20, x)
+                pages.append(x)
+            if self.kind == "fp8":
+                # per-(layer, kv-head) scales: amax / 448 over the rows (keys' row, then values')
+                m = torch.stack([p.float().abs().amax(dim=(0, 1, 3)) / 448.0 for p in pages]).contiguous()
+                self.mult.append(m)
+                pages = [(p.float() / m[i][None, None, :, None]).clamp(-448, 448).to(store) for i, p in enumerate(pages)]
+            else:
+                self.mult.append((1.0, 1.0))
+            self.k.append(pages[0])
+            self.v.append(pages[1])
+        self.rows = torch.arange(B, dtype=torch.int32, device=device)
+        self.starts = torch.arange(B, dtype=torch.int32, device=device)
+        self.counts = torch.ones(B, dtype=torch.int32, device=device)
+        self.firsts = self.ctx.to(torch.int64).to(device)
+        slots = torch.stack([tables[s, int(self.ctx[s]) // page].long() * page + int(self.ctx[s]) % page for s in range(B)])
+        self.slots = slots.to(device)
+        self.q = (torch.randn(B, hq, d, device=device, generator=gen) * spec["std"]).to(torch.bfloat16)
+        self.new_k = (torch.randn(B, hkv, d, device=device, generator=gen) * spec["std"]).to(torch.bfloat16)
+        self.new_v = (torch.randn(B, hkv, d, device=device, generator=gen) * spec["std"]).to(torch.bfloat16)
+        self.out = torch.empty(B, hq, d, dtype=torch.bfloat16, device=device)
+        self.parts = pk.partitions(device, hkv, self.kind, d, d)
+        self.piece = pk.piece_size(d, d, self.kind, hkv)
+        self.workspace = torch.empty(pk.workspace_floats(B, hq, self.parts, d), dtype=torch.float32, device=device)
+        e = 2 if self.kind == "bf16" else 1
+        tokens = int((self.ctx + 1).sum())
+        self.decode_bytes = tokens * hkv * (d + d) * e            # per layer: K and V of every visible position
+        self.append_bytes = B * hkv * (d + d) * (e + 2)           # per layer: page bytes written + bf16 inputs read
+        self.tokens = tokens
+
+    def append(self, layer):
+        self.pk.write(self.new_k, self.new_v, self.slots, self.k[layer], self.v[layer], self.kind,
+                      multipliers=self.mult[layer])
+
+    def attend(self, layer, phases=0):
+        self.pk.attend(self.q, self.k[layer], self.v[layer], self.kind, self.tables, self.rows, self.starts, self.firsts,
+                       1, self.page, counts=self.counts, offsets=self.starts, tokens=self.q.shape[0],
+                       multipliers=self.mult[layer], partitions=self.parts, piece=self.piece, out=self.out,
+                       workspace=self.workspace, phases=phases)
+
+    def step(self):
+        for layer in range(self.layers):
+            self.append(layer)
+            self.attend(layer)
+
+
+def timed(fn, reps, warmup=1):
+    """Average milliseconds of fn() over reps calls, by HIP events on the current stream (the launch stream)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps
+
+
+def kernel_ms(w, phases):
+    """Average duration of one launch phase over every layer (cold: each layer's pages are different memory)."""
+    w.attend(0, phases)
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for layer in range(w.layers):
+        w.attend(layer, phases)
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / w.layers
+
+
+def cpu_baseline(spec, seconds=20.0):
+    """The reference's CPU path (FP32 pages: index_copy append, then per row gather + SDPA) restated in oracle/,
+    timed on this host over ONE layer and the first 8 sequences of the workload; the rate counts the same algorithmic
+    bytes as the GPU figure (the GPU configuration's element size) for those sequences."""
+    from oracle import append as oa
+    from oracle import attend as oatt
+    g = torch.Generator().manual_seed(0)
+    B, page, hkv, d, hq = 8, 16, spec["hkv"], spec["d"], spec["hq"]
+    ctx = torch.randint(spec["lo"], spec["hi"] + 1, (spec["batch"],), generator=g)[:B]
+    need = int(((ctx + 1 + page - 1) // page).sum())
+    n_pages = int(need * 1.25)
+    perm = torch.randperm(n_pages, generator=g)
+    tables, at = [], 0
+    for s in range(B):
+        wd = int((ctx[s] + 1 + page - 1) // page)
+        tables.append(perm[at:at + wd])
+        at += wd
+    k = torch.randn(n_pages + 1, page, hkv, d, generator=g) * spec["std"]
+    v = torch.randn(n_pages + 1, page, hkv, d, generator=g) * spec["std"]
+    q = torch.randn(B, hq, d, generator=g)
+    nk, nv = torch.randn(B, hkv, d, generator=g), torch.randn(B, hkv, d, generator=g)
+    slots = torch.stack([oa.slots(tables[s], torch.tensor([int(ctx[s])]), page)[0] for s in range(B)])
+    rows = [(s, 1, int(ctx[s])) for s in range(B)]
+    out = torch.empty(B, hq, d)
+
+    def one():
+        oa.write(nk, nv, slots, k, v, "fp32", dump_slot=n_pages * page)
+        oatt.sdpa_rows(q, rows, lambda r, n: oatt.gather(k, v, tables[r], n, page, "fp32", torch.float32), d ** -0.5, out)
+    one()
+    reps, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < seconds or reps < 2:
+        one()
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    e = 2 if spec["kind"] == "bf16" else 1
+    nbytes = int((ctx + 1).sum()) * hkv * 2 * d * e + B * hkv * 2 * d * (e + 2)
+    return {"value": round(nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"1 layer x first 8 of {spec['batch']} sequences ({int((ctx + 1).sum())} positions), FP32 pages, "
+                      f"{reps} reps, {dt * 1e3:.1f} ms each; bytes counted at the GPU configuration's element size",
+            "host_cpus": os.cpu_count()}
+
+
+def append_sweep(pk, device, kind):
+    """KV append GB/s against the token count (algorithmic bytes: page bytes written + bf16 inputs read)."""
+    hkv, d, found = 8, 128, {}
+    store = torch.bfloat16 if kind == "bf16" else torch.float8_e4m3fn
+    e = 2 if kind == "bf16" else 1
+    n_slots = 1 << 20
+    k = torch.zeros(n_slots, hkv, d, dtype=store, device=device)
+    v = torch.zeros_like(k)
+    g = torch.Generator(device=device).manual_seed(1)
+    for T in (64, 1024, 4152, 65536, 262144):
+        keys = torch.randn(T, hkv, d, device=device, generator=g).to(torch.bfloat16)
+        values = torch.randn(T, hkv, d, device=device, generator=g).to(torch.bfloat16)
+        slots = torch.randperm(n_slots, device=device, generator=g)[:T]
+        ms = timed(lambda: pk.write(keys, values, slots, k, v, kind, multipliers=(0.02, 0.03)), 20, 3)
+        nbytes = T * hkv * 2 * d * (e + 2)
+        found[str(T)] = {"us": round(ms * 1e3, 2), "GB/s": round(nbytes / ms / 1e6, 1)}
+    return found
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this path has no cross-GPU part (run with --gpus 1)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU (the CPU oracle is a checker, not a product path)")
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    import crit_amd.paged_kv_attention as pk
+    spec = WORKLOADS[args.workload]
+    log(f"[bench] building workload {args.workload}: {spec['name']}")
+    w = Workload(spec, device)
+    log(f"[bench] {w.tokens} positions, pool {w.n_pages} pages/layer, decode {w.decode_bytes / 1e9:.3f} GB/layer, "
+        f"partitions {w.parts}, piece {w.piece}")
+    for _ in range(args.warmup):
+        w.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        w.step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    step_bytes = (w.decode_bytes + w.append_bytes) * w.layers
+    value = step_bytes / ms_per_step / 1e6
+
+    split_ms = kernel_ms(w, 1)
+    merge_ms = kernel_ms(w, 2)
+    append_ms = timed(lambda: w.append(0), 50, 5)
+    achieved = w.decode_bytes / split_ms / 1e6
+    sink = torch.zeros(64, device=device)
+    read_ms, read_bytes = None, 0
+    for layer in range(min(4, w.layers)):
+        flat = w.k[layer].view(torch.uint8).reshape(-1)
+        flat = flat[:flat.numel() // 16 * 16]
+        ms = timed(lambda: pk.stream_read(flat, sink), 1, 0)
+        read_ms, read_bytes = (ms if read_ms is None else min(read_ms, ms)), flat.numel()
+    stream_gbps = read_bytes / read_ms / 1e6
+    result = {
+        "metric": "paged decode attention + KV append, algorithmic HBM GB/s over one 32-layer decode step",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if w.kind == "bf16" else "fp8_e4m3 KV, bf16 q, f32 accumulate", "data": "synthetic",
+        "config": {"workload": spec["name"], "positions": w.tokens, "partitions": w.parts, "piece": w.piece},
+        "roofline": {"bound": "hbm", "kernel": "attend_kernel (split launch)", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "launch_ms": round(split_ms, 4), "merge_ms": round(merge_ms, 4),
+                     "algorithmic_bytes_per_launch": w.decode_bytes,
+                     "stream_read_GB/s": round(stream_gbps, 1)},
+        "append": {"us_per_launch": round(append_ms * 1e3, 2), "tokens": spec["batch"],
+                   "GB/s": round(w.append_bytes / append_ms / 1e6, 2)},
+        "fraction_of_peak": round(value / HBM_PEAK_GBPS, 4),
+    }
+    log(f"[bench] step {ms_per_step:.3f} ms; split launch {split_ms:.4f} ms = {achieved:.0f} GB/s; merge {merge_ms:.4f} ms; "
+        f"append {append_ms * 1e3:.1f} us; stream read {stream_gbps:.0f} GB/s")
+    del w
+    torch.cuda.empty_cache()
+    if not args.no_extras:
+        extras = {}
+        other = "c3" if args.workload == "c2" else "c2"
+        ospec = WORKLOADS[other]
+        log(f"[bench] extra: {other} on 8 layers")
+        ow = Workload(ospec, device, layers=8)
+        for _ in range(2):
+            ow.step()
+        ms = timed(ow.step, 3, 0)
+        osplit = kernel_ms(ow, 1)
+        extras[other] = {"workload": ospec["name"] + " (8 of 32 layers resident; per-layer figures)",
+                         "ms_per_layer": round(ms / ow.layers, 4),
+                         "GB/s": round((ow.decode_bytes + ow.append_bytes) * ow.layers / ms / 1e6, 1),
+                         "split_launch_ms": round(osplit, 4), "split_launch_GB/s": round(ow.decode_bytes / osplit / 1e6, 1),
+                         "frac": round(ow.decode_bytes / osplit / 1e6 / HBM_PEAK_GBPS, 4)}
+        log(f"[bench] {other}: {extras[other]}")
+        del ow
+        torch.cuda.empty_cache()
+        extras["append_GB/s_by_tokens"] = {kind: append_sweep(pk, device, kind) for kind in ("bf16", "fp8")}
+        log(f"[bench] append sweep: {extras['append_GB/s_by_tokens']}")
+        result["extra"] = extras
+    if not args.no_cpu:
+        log("[bench] timing the CPU reference path (about 20 s)")
+        result["cpu_baseline"] = cpu_baseline(spec)
+        log(f"[bench] cpu: {result['cpu_baseline']}")
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()
