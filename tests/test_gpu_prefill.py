@@ -1,0 +1,154 @@
+"""Chunked prefill over paged KV (the matrix-core path) on the GPU against the CPU oracle. Mirrors the reference's
+kernels/techniques/attention/paged-kv-attention/tests/test_paged_kv_attention.py:459-480, 515-536 and the prompt-row
+call sites of inference/attention-state/code/device_attention.py:901-916 (int64 tables, sliced outputs)."""
+import pytest
+import torch
+
+from tests.support import KINDS, Cache, kernels, rand_q
+
+pytestmark = pytest.mark.gpu
+dev = "cuda"
+ATOL, RTOL = 8e-3, 2e-2
+
+
+def _check(cache, q, out, lse, position, tokens, sliding=0):
+    for t in tokens:
+        want, want_lse = cache.want(q[t:t + 1], 0, position + t, 1, sliding=sliding)
+        torch.testing.assert_close(out[t:t + 1].double().cpu(), want, atol=ATOL, rtol=RTOL, msg=f"token {t}")
+        if lse is not None:
+            torch.testing.assert_close(lse[t:t + 1].double().cpu(), want_lse, atol=1e-3, rtol=1e-4, msg=f"lse {t}")
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 128), (32, 8, 128), (40, 8, 128), (12, 2, 64)])
+def test_prompt_chunks_match_float64_attention(kind, hq, hkv, d):
+    pk = kernels()
+    cache = Cache(kind, hkv, d, d, 16, [300])
+    q = rand_q(100, hq, d, 4)
+    lse = torch.empty(100, hq, device=dev)
+    q_dtype = torch.float16 if kind == "fp16" else torch.bfloat16
+    out = pk.prefill(q.to(q_dtype), cache.k, cache.v, kind, cache.tables[0], 200, 16, key_scales=cache.ks,
+                     value_scales=cache.vs, multipliers=cache.multipliers, lse=lse)
+    _check(cache, q, out, lse, 200, (0, 37, 63, 64, 99))
+
+
+@pytest.mark.parametrize("position,T", [(0, 1), (0, 512), (1, 17), (1000, 512), (8191, 33)])
+def test_chunks_at_any_position_and_length(position, T):
+    pk = kernels()
+    cache = Cache("bf16", 8, 128, 128, 16, [position + T], seed=3, scale=0.5)
+    q = rand_q(T, 32, 128, 5)
+    lse = torch.empty(T, 32, device=dev)
+    out = pk.prefill(q.bfloat16(), cache.k, cache.v, "bf16", cache.tables[0].long(), position, 16, lse=lse)
+    picks = sorted({0, T // 3, T - 1})
+    _check(cache, q, out, lse, position, picks)
+
+
+def test_a_tokens_bits_follow_its_own_positions_only():
+    # The same tokens read as one chunk, as two chunks, and at a device position: every bit equal.
+    pk = kernels()
+    cache = Cache("bf16", 2, 128, 128, 16, [700])
+    q = rand_q(200, 8, 128, 6).bfloat16()
+    table = cache.tables[0]
+    whole = pk.prefill(q, cache.k, cache.v, "bf16", table, 500, 16)
+    first = pk.prefill(q[:77], cache.k, cache.v, "bf16", table, 500, 16)
+    second = pk.prefill(q[77:], cache.k, cache.v, "bf16", table, 577, 16)
+    assert torch.equal(torch.cat([first, second]), whole)
+    position = torch.tensor([500], dtype=torch.int64, device=dev)
+    assert torch.equal(pk.prefill(q, cache.k, cache.v, "bf16", table, position, 16), whole)
+    sliced = torch.zeros(300, 8, 128, dtype=torch.bfloat16, device=dev)
+    pk.prefill(q, cache.k, cache.v, "bf16", table, 500, 16, out=sliced[50:250])
+    assert torch.equal(sliced[50:250], whole) and not bool(sliced[:50].any()) and not bool(sliced[250:].any())
+
+
+def test_a_chunk_at_a_device_position_replays_from_one_graph():
+    pk = kernels()
+    cache = Cache("fp8:row", 4, 128, 128, 16, [700])
+    q = rand_q(64, 16, 128, 12).to(torch.bfloat16)
+    table = cache.tables[0]
+    position = torch.zeros(1, dtype=torch.int64, device=dev)
+    out = torch.empty_like(q)
+
+    def launch(into, at):
+        pk.prefill(q, cache.k, cache.v, "fp8:row", table, at, 16, key_scales=cache.ks, value_scales=cache.vs, out=into)
+    launch(out, position)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        launch(out, position)
+    for at in (0, 5, 300, 636):
+        position.fill_(at)
+        graph.replay()
+        torch.cuda.synchronize()
+        want = torch.empty_like(q)
+        launch(want, at)
+        assert torch.equal(out, want), at
+
+
+def test_several_chunks_in_one_launch_equal_one_launch_each():
+    # the mixed batch's prefill part: chunks of different lengths on prefixes of different lengths, one launch
+    pk = kernels()
+    lengths = [512 + 0, 512 + 1000, 300 + 4097, 512 + 8192]
+    counts = [512, 512, 300, 512]
+    cache = Cache("bf16", 8, 128, 128, 16, lengths, seed=9, scale=0.5)
+    starts = [0, 512, 1024, 1324]
+    q = rand_q(sum(counts), 32, 128, 7).bfloat16()
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    positions = torch.tensor([n - c for n, c in zip(lengths, counts)], dtype=torch.int64, device=dev)
+    lse = torch.empty(q.shape[0], 32, device=dev)
+    out = pk.prefill_rows(q, cache.k, cache.v, "bf16", cache.tables, i32([0, 1, 2, 3]), i32(starts), i32(counts),
+                          positions, 512, 16, lse=lse)
+    for s, (start, count, n) in enumerate(zip(starts, counts, lengths)):
+        one = pk.prefill(q[start:start + count], cache.k, cache.v, "bf16", cache.tables[s], n - count, 16)
+        assert torch.equal(out[start:start + count], one), s
+    want, want_lse = cache.want(q[1324 + 511:1324 + 512].float(), 3, lengths[3] - 1, 1)
+    torch.testing.assert_close(out[-1:].double().cpu(), want, atol=ATOL, rtol=RTOL)
+    torch.testing.assert_close(lse[-1:].double().cpu(), want_lse, atol=1e-3, rtol=1e-4)
+
+
+def test_prefill_agrees_with_the_decode_reader_within_the_readers_rounding():
+    pk = kernels()
+    cache = Cache("bf16", 2, 128, 128, 16, [400])
+    q = rand_q(64, 8, 128, 8)
+    chunk = pk.prefill(q.bfloat16(), cache.k, cache.v, "bf16", cache.tables[0], 336, 16)
+    decode = cache.attend(q, [0], [0], [336], 64)
+    torch.testing.assert_close(chunk.float(), decode.float(), atol=1.6e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("window", [1, 100, 1000])
+def test_a_sliding_window_and_sinks(window):
+    pk = kernels()
+    cache = Cache("bf16", 2, 128, 128, 16, [1500])
+    q = rand_q(130, 8, 128, 9)
+    lse = torch.empty(130, 8, device=dev)
+    out = pk.prefill(q.bfloat16(), cache.k, cache.v, "bf16", cache.tables[0], 1370, 16, sliding=window, lse=lse)
+    _check(cache, q, out, lse, 1370, (0, 64, 129), sliding=window)
+    sinks = torch.linspace(-2, 2, 8, device=dev)
+    with_sinks = pk.prefill(q.bfloat16(), cache.k, cache.v, "bf16", cache.tables[0], 1370, 16, sliding=window, sinks=sinks)
+    weight = torch.exp(lse) / (torch.exp(lse) + torch.exp(sinks)[None, :])
+    torch.testing.assert_close(with_sinks.float(), out.float() * weight[..., None], atol=8e-3, rtol=2e-2)
+
+
+def test_fp32_outputs_and_warm_up_shapes():
+    pk = kernels()
+    cache = Cache("bf16", 2, 128, 128, 16, [40])
+    q = rand_q(9, 8, 128, 2)
+    out = torch.empty(9, 8, 128, dtype=torch.float32, device=dev)
+    pk.prefill(q.bfloat16(), cache.k, cache.v, "bf16", cache.tables[0], 31, 16, out=out)
+    _check(cache, q, out, None, 31, (0, 8))
+    # DeviceAttention's load-time call: one token at position 0 over a one-entry int64 table of the dump page
+    dump = torch.full((1,), cache.k.shape[0] - 1, dtype=torch.int64, device=dev)
+    one = pk.prefill(q[:1].bfloat16(), cache.k, cache.v, "bf16", dump, 0, 16)
+    assert one.shape == (1, 8, 128)
+
+
+def test_what_the_prompt_reader_does_not_take_is_refused():
+    pk = kernels()
+    cache = Cache("int8", 2, 128, 128, 16, [40])
+    q = rand_q(4, 8, 128, 2).bfloat16()
+    kw = dict(key_scales=cache.ks, value_scales=cache.vs)
+    with pytest.raises(NotImplementedError):
+        pk.prefill(q, cache.k, cache.v, "int8", cache.tables[0], 36, 16, int8_qk=True, **kw)
+    with pytest.raises(NotImplementedError):
+        pk.prefill(q, cache.k, cache.v, "int8", cache.tables[0], 36, 16, fresh=(q, q), **kw)
+    with pytest.raises(ValueError):
+        pk.prefill(q.float(), cache.k, cache.v, "int8", cache.tables[0], 36, 16, **kw)
