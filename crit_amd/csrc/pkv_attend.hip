@@ -1,397 +1,15 @@
-// Paged decode / verify-window attention, split over KV partitions, and the merge of the partitions.
-//
-// Work unit: one workgroup of 4 wavefronts per (row, KV head, query tile, partition). A query tile is QR rows of the
-// flattened (column, query head of the KV head's group) list, so the group's heads share every K/V row read.
-// Inside a wavefront LPR = D/8 lanes hold one K (or V) row, 16 bytes each (8 bytes for 8-bit pages), so one
-// load instruction fetches 64/LPR whole rows; a step is four such loads for K and four for V. Each 16-lane group keeps
-// its own online-softmax state over the positions it reads; the groups and the four wavefronts are folded at the
-// end in a fixed order, then the partition's state goes to the partials (or, fused, into the running state).
-// No matrix cores: the kernel is bound by HBM reads of K and V.
-//
-// A column's bits depend on its own query, its own keys, `piece`, `partitions` and the page kind only: position n is
-// always read by the same wavefront, lane group and step whatever the launch, masked positions contribute exact
-// zeros, and every sum is an explicit FMA chain in a fixed order (built with -ffp-contract=off).
-#include <type_traits>
-
-#include "pkv_common.hpp"
+// Host side of the decode / verify-window launches (argument checks, grid, the choice of kernel) and the small
+// kernels around the split launch: the merge of the partitions, the merge of shard partials, a streaming-read probe.
+#include "pkv_attend_args.hpp"
 #include "pkv_launch.hpp"
 
 namespace pkv {
 
-struct AttendArgs {
-    const uint8_t* q;
-    const uint8_t* kp;
-    const uint8_t* vp;
-    const float* ks;
-    const float* vs;
-    const float* hm;
-    const int32_t* tables;
-    const int32_t* rows;
-    const int32_t* starts;
-    const int32_t* counts;
-    const int64_t* firsts;
-    const int32_t* offsets;
-    float* po;
-    float* pm;
-    float* pl;
-    void* out;
-    float* lse;
-    const float* sinks;
-    int64_t q_st, q_sh, o_st, o_sh, tab_stride;
-    int tab_width, n_rows, columns, hq, hkv, g, page, page_shift, parts, piece, sliding, out_dtype, tiles;
-    float sscale, k_mult, v_mult;
-};
-
-template <int KIND>
-struct StepBuf {
-    using Vec = typename std::conditional<KIND == 0, uint4, uint2>::type;
-    Vec k[4], v[4];
-    float ks[4], vs[4];
-};
-
-template <int KIND, bool F16, int LPR, int QR, bool FUSED>
-__global__ __launch_bounds__(256) void attend_kernel(AttendArgs a) {
-    constexpr int D = LPR * 8;
-    constexpr int PPI = 64 / LPR;      // positions one load instruction of a wavefront covers
-    constexpr int SP = 4 * PPI;        // positions a wavefront's step covers
-    constexpr int EB = KIND == 0 ? 2 : 1;
-    constexpr int EPT = (QR * D + 255) / 256;   // output elements a thread folds
-    __shared__ __align__(16) float s_acc[4][QR][D];
-    __shared__ float s_m[4][QR], s_l[4][QR];
-
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lg = lane / LPR, li = lane % LPR;
-    int bx = blockIdx.x;
-    const int tile = bx % a.tiles;
-    bx /= a.tiles;
-    const int kvh = bx % a.hkv;
-    const int r = bx / a.hkv;
-    const int b = blockIdx.y;
-    int count = a.columns;
-    if (a.counts) count = min(a.counts[r], a.columns);
-    const int j0 = tile * QR;
-    if (j0 >= count * a.g) return;
-    const int64_t first64 = a.firsts[r];
-    const int c_lo = j0 / a.g;
-    const int c_hi = min(count, (j0 + QR - 1) / a.g + 1);
-    int64_t nk64 = first64 + c_hi;
-    nk64 = nk64 < 0 ? 0 : (nk64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : nk64);
-    const int n_keys = (int)nk64;
-    const int first = (int)(first64 < 0 ? 0 : (first64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first64));
-    const int n_pieces = (n_keys + a.piece - 1) / a.piece;
-    if (!FUSED && b >= n_pieces) return;
-    const int64_t trow = (int64_t)a.rows[r] * a.tab_stride;
-    const int start = a.starts[r];
-
-    // The tile's rows: column, query head, last visible position.
-    int lim[QR];
-    bool live[QR];
-    int qhead[QR], col[QR];
-#pragma unroll
-    for (int rr = 0; rr < QR; ++rr) {
-        const int j = j0 + rr;
-        col[rr] = j / a.g;
-        qhead[rr] = kvh * a.g + j % a.g;
-        live[rr] = col[rr] < count;
-        lim[rr] = first + col[rr];
-    }
-    // The lane's slice of each query row: packed 16-bit pairs for 16-bit pages, FP32 for 8-bit pages.
-    uint32_t qp[QR][4];
-    float qf[KIND == 0 ? 1 : QR][8];
-#pragma unroll
-    for (int rr = 0; rr < QR; ++rr) {
-        uint4 w = make_uint4(0, 0, 0, 0);
-        if (live[rr]) {
-            w = *reinterpret_cast<const uint4*>(a.q + ((int64_t)(start + col[rr]) * a.q_st + (int64_t)qhead[rr] * a.q_sh + li * 8) * 2);
-        }
-        qp[rr][0] = w.x, qp[rr][1] = w.y, qp[rr][2] = w.z, qp[rr][3] = w.w;
-        if constexpr (KIND != 0) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                qf[rr][2 * j] = F16 ? f16_lo(qp[rr][j]) : bf16_lo(qp[rr][j]);
-                qf[rr][2 * j + 1] = F16 ? f16_hi(qp[rr][j]) : bf16_hi(qp[rr][j]);
-            }
-        }
-    }
-    float k_mult = a.k_mult, v_mult = a.v_mult;
-    if (KIND == 1 && a.hm) k_mult = a.hm[kvh], v_mult = a.hm[a.hkv + kvh];
-    const float sscale = a.sscale * (KIND == 1 ? k_mult : 1.0f);
-    if (KIND != 1) v_mult = 1.0f;
-    const int win = a.sliding;
-
-    const uint8_t* kbase = a.kp + ((int64_t)kvh * D + li * 8) * EB;
-    const uint8_t* vbase = a.vp + ((int64_t)kvh * D + li * 8) * EB;
-    const int64_t slot_bytes = (int64_t)a.hkv * D * EB;
-
-    auto fetch_tab = [&](int base, int (&tab)[4]) {
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            int n = base + k * PPI + lg;
-            n = n < n_keys ? n : n_keys - 1;
-            int pidx = a.page_shift >= 0 ? (n >> a.page_shift) : (n / a.page);
-            pidx = pidx < a.tab_width ? pidx : a.tab_width - 1;
-            tab[k] = a.tables[trow + pidx];
-        }
-    };
-    auto fetch_kv = [&](int base, const int (&tab)[4], StepBuf<KIND>& buf) {
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            int n = base + k * PPI + lg;
-            n = n < n_keys ? n : n_keys - 1;
-            const int in_page = a.page_shift >= 0 ? (n & (a.page - 1)) : (n % a.page);
-            const int64_t slot = (int64_t)tab[k] * a.page + in_page;
-            buf.k[k] = *reinterpret_cast<const typename StepBuf<KIND>::Vec*>(kbase + slot * slot_bytes);
-            buf.v[k] = *reinterpret_cast<const typename StepBuf<KIND>::Vec*>(vbase + slot * slot_bytes);
-            if constexpr (KIND >= 2) {
-                buf.ks[k] = a.ks[slot * a.hkv + kvh];
-                buf.vs[k] = a.vs[slot * a.hkv + kvh];
-            }
-        }
-    };
-
-    // Running state of the fused fold (one per output element of this thread).
-    float run_m[EPT], run_l[EPT], run_a[EPT];
-#pragma unroll
-    for (int e = 0; e < EPT; ++e) run_m[e] = -INFINITY, run_l[e] = 0.0f, run_a[e] = 0.0f;
-
-    const int part_lo = FUSED ? 0 : b;
-    const int part_hi = FUSED ? min(a.parts, n_pieces) : b + 1;
-    for (int part = part_lo; part < part_hi; ++part) {
-        float m[QR], l[QR], acc[QR][8];
-#pragma unroll
-        for (int rr = 0; rr < QR; ++rr) {
-            m[rr] = -INFINITY, l[rr] = 0.0f;
-#pragma unroll
-            for (int d = 0; d < 8; ++d) acc[rr][d] = 0.0f;
-        }
-        // This wavefront's steps: steps wave, wave + 4, ... of pieces part, part + parts, ...
-        int pi = part, st = wave;
-        if (win > 0) {   // pieces wholly below the tile's window are skipped (no row sees them)
-            const int wlo = first + c_lo - win + 1;
-            const int below = (wlo > 0 ? wlo : 0) / a.piece - part;
-            if (below > 0) pi = part + (below + a.parts - 1) / a.parts * a.parts;
-        }
-        auto base_of = [&]() -> int {
-            if (st * SP >= a.piece) return -1;
-            const int64_t base = (int64_t)pi * a.piece + st * SP;
-            return base < n_keys ? (int)base : -1;
-        };
-        auto advance = [&]() -> int {
-            st += 4;
-            if (st * SP >= a.piece) pi += a.parts, st = wave;
-            return base_of();
-        };
-
-        auto compute = [&](int base, const StepBuf<KIND>& buf) {
-            float s[4][QR];
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                uint32_t kw[4];
-                float kf[8];
-                if constexpr (KIND == 0) {
-                    kw[0] = buf.k[k].x, kw[1] = buf.k[k].y, kw[2] = buf.k[k].z, kw[3] = buf.k[k].w;
-                } else if constexpr (KIND == 3) {
-                    const uint32_t w2[2] = {buf.k[k].x, buf.k[k].y};
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) kf[j] = (float)(int8_t)(w2[j / 4] >> (8 * (j % 4)));
-                } else {
-                    const f32x2 a0 = e4m3_pair<false>(buf.k[k].x), a1 = e4m3_pair<true>(buf.k[k].x);
-                    const f32x2 a2 = e4m3_pair<false>(buf.k[k].y), a3 = e4m3_pair<true>(buf.k[k].y);
-                    kf[0] = a0.x, kf[1] = a0.y, kf[2] = a1.x, kf[3] = a1.y;
-                    kf[4] = a2.x, kf[5] = a2.y, kf[6] = a3.x, kf[7] = a3.y;
-                }
-#pragma unroll
-                for (int rr = 0; rr < QR; ++rr) {
-                    float d = 0.0f;
-                    if constexpr (KIND == 0) {
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            if constexpr (F16) {
-                                d = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, qp[rr][j]), __builtin_bit_cast(f16x2, kw[j]), d, false);
-                            } else {
-                                d = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, qp[rr][j]), __builtin_bit_cast(bf16x2, kw[j]), d, false);
-                            }
-                        }
-                    } else {
-#pragma unroll
-                        for (int j = 0; j < 8; ++j) d = __builtin_fmaf(qf[rr][j], kf[j], d);
-                    }
-                    s[k][rr] = group_sum<LPR>(d);
-                }
-            }
-            // Scale, mask, and one online-softmax update per row over the step's four positions of this lane group.
-#pragma unroll
-            for (int rr = 0; rr < QR; ++rr) {
-                float top = -INFINITY;
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const int n = base + k * PPI + lg;
-                    float x = s[k][rr] * (KIND >= 2 ? sscale * buf.ks[k] : sscale);
-                    bool vis = n <= lim[rr] && n < n_keys;
-                    if (win > 0) vis = vis && n > lim[rr] - win;
-                    x = vis ? x : -INFINITY;
-                    s[k][rr] = x;
-                    top = __builtin_fmaxf(top, x);
-                }
-                const float m_new = __builtin_fmaxf(m[rr], top);
-                const float sub = m_new == -INFINITY ? 0.0f : m_new;
-                const float alpha = exp2_fast(m[rr] - sub);
-                float sum = 0.0f;
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const float p = exp2_fast(s[k][rr] - sub);
-                    sum += p;
-                    s[k][rr] = KIND >= 2 ? p * buf.vs[k] : p;
-                }
-                l[rr] = __builtin_fmaf(l[rr], alpha, sum);
-                m[rr] = m_new;
-#pragma unroll
-                for (int d = 0; d < 8; ++d) acc[rr][d] *= alpha;
-            }
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                float vf[8];
-                if constexpr (KIND == 0) {
-                    const uint32_t vw[4] = {buf.v[k].x, buf.v[k].y, buf.v[k].z, buf.v[k].w};
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        vf[2 * j] = F16 ? f16_lo(vw[j]) : bf16_lo(vw[j]);
-                        vf[2 * j + 1] = F16 ? f16_hi(vw[j]) : bf16_hi(vw[j]);
-                    }
-                } else if constexpr (KIND == 3) {
-                    const uint32_t w2[2] = {buf.v[k].x, buf.v[k].y};
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) vf[j] = (float)(int8_t)(w2[j / 4] >> (8 * (j % 4)));
-                } else {
-                    const f32x2 a0 = e4m3_pair<false>(buf.v[k].x), a1 = e4m3_pair<true>(buf.v[k].x);
-                    const f32x2 a2 = e4m3_pair<false>(buf.v[k].y), a3 = e4m3_pair<true>(buf.v[k].y);
-                    vf[0] = a0.x, vf[1] = a0.y, vf[2] = a1.x, vf[3] = a1.y;
-                    vf[4] = a2.x, vf[5] = a2.y, vf[6] = a3.x, vf[7] = a3.y;
-                }
-#pragma unroll
-                for (int rr = 0; rr < QR; ++rr) {
-#pragma unroll
-                    for (int d = 0; d < 8; ++d) acc[rr][d] = __builtin_fmaf(s[k][rr], vf[d], acc[rr][d]);
-                }
-            }
-        };
-
-        // Three-stage software pipeline: table entries two steps ahead, K/V one step ahead, compute.
-        StepBuf<KIND> bufA, bufB;
-        int tabA[4], tabB[4];
-        int base0 = base_of();
-        if (base0 >= 0) fetch_tab(base0, tabA);
-        int base1 = base0 >= 0 ? advance() : -1;
-        if (base0 >= 0) fetch_kv(base0, tabA, bufA);
-        if (base1 >= 0) fetch_tab(base1, tabB);
-        while (base0 >= 0) {
-            int base2 = base1 >= 0 ? advance() : -1;
-            if (base1 >= 0) fetch_kv(base1, tabB, bufB);
-            if (base2 >= 0) fetch_tab(base2, tabA);
-            compute(base0, bufA);
-            if (base1 < 0) break;
-            base0 = base2 >= 0 ? advance() : -1;
-            if (base2 >= 0) fetch_kv(base2, tabA, bufA);
-            if (base0 >= 0) fetch_tab(base0, tabB);
-            compute(base1, bufB);
-            base1 = base0;
-            base0 = base2;
-            // now base0 is loaded in bufA, base1's table entries are in tabB
-        }
-
-        // Fold the wavefront's lane groups (butterfly: every lane ends with the same bits), then the four wavefronts
-        // through LDS in wavefront order.
-#pragma unroll
-        for (int rr = 0; rr < QR; ++rr) {
-            float top = m[rr];
-#pragma unroll
-            for (int o = LPR; o < 64; o <<= 1) top = __builtin_fmaxf(top, __shfl_xor(top, o));
-            const float sub = top == -INFINITY ? 0.0f : top;
-            const float w = exp2_fast(m[rr] - sub);
-            float lw = l[rr] * w;
-#pragma unroll
-            for (int o = LPR; o < 64; o <<= 1) lw += __shfl_xor(lw, o);
-#pragma unroll
-            for (int d = 0; d < 8; ++d) {
-                float x = acc[rr][d] * w;
-#pragma unroll
-                for (int o = LPR; o < 64; o <<= 1) x += __shfl_xor(x, o);
-                acc[rr][d] = x;
-            }
-            m[rr] = top, l[rr] = lw;
-        }
-        if (FUSED) __syncthreads();      // the previous partition's fold has read the LDS
-        if (lg == 0) {
-#pragma unroll
-            for (int rr = 0; rr < QR; ++rr) {
-                *reinterpret_cast<float4*>(&s_acc[wave][rr][li * 8]) = make_float4(acc[rr][0], acc[rr][1], acc[rr][2], acc[rr][3]);
-                *reinterpret_cast<float4*>(&s_acc[wave][rr][li * 8 + 4]) = make_float4(acc[rr][4], acc[rr][5], acc[rr][6], acc[rr][7]);
-                if (li == 0) s_m[wave][rr] = m[rr], s_l[wave][rr] = l[rr];
-            }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int e = 0; e < EPT; ++e) {
-            const int idx = tid + e * 256;
-            if (idx < QR * D) {
-                const int rr = idx / D, d = idx % D;
-                float M = s_m[0][rr];
-#pragma unroll
-                for (int w = 1; w < 4; ++w) M = __builtin_fmaxf(M, s_m[w][rr]);
-                const float sub = M == -INFINITY ? 0.0f : M;
-                float L = 0.0f, A = 0.0f;
-#pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    const float f = exp2_fast(s_m[w][rr] - sub);
-                    L = __builtin_fmaf(s_l[w][rr], f, L);
-                    A = __builtin_fmaf(s_acc[w][rr][d], f, A);
-                }
-                A *= v_mult;
-                const int j = j0 + rr;
-                const int c = j / a.g;
-                if (c < count) {
-                    if constexpr (FUSED) {
-                        // A column folds the partitions that hold its positions, as the merge does.
-                        const int held = min(a.parts, (first + c + a.piece) / a.piece);
-                        if (part < held) {
-                            const Fold f = fold(run_m[e], run_l[e], M, L);
-                            run_a[e] = __builtin_fmaf(run_a[e], f.keep, A * f.take);
-                            run_m[e] = f.m, run_l[e] = f.l;
-                        }
-                    } else {
-                        const int64_t prow = a.offsets ? (int64_t)(a.offsets[r] - a.offsets[0]) : (int64_t)r * a.columns;
-                        const int64_t at = ((prow + c) * a.hq + kvh * a.g + j % a.g) * a.parts + b;
-                        a.po[at * D + d] = A;
-                        if (d == 0) a.pm[at] = M, a.pl[at] = L;
-                    }
-                }
-            }
-        }
-    }
-    if constexpr (FUSED) {
-#pragma unroll
-        for (int e = 0; e < EPT; ++e) {
-            const int idx = tid + e * 256;
-            if (idx < QR * D) {
-                const int rr = idx / D, d = idx % D;
-                const int j = j0 + rr;
-                const int c = j / a.g;
-                if (c < count) {
-                    const int head = kvh * a.g + j % a.g;
-                    float M = run_m[e], L = run_l[e], A = run_a[e];
-                    if (a.sinks) {
-                        const Fold f = fold(M, L, a.sinks[head] * kLog2e, 1.0f);
-                        A *= f.keep, M = f.m, L = f.l;
-                    }
-                    const float o = L != 0.0f ? A / L : 0.0f;
-                    store_out(a.out, a.out_dtype, (int64_t)(start + c) * a.o_st + (int64_t)head * a.o_sh + d, o);
-                    if (a.lse && d == 0) {
-                        a.lse[(int64_t)(start + c) * a.hq + head] = L != 0.0f ? __builtin_fmaf(M, kLn2, __logf(L)) : -INFINITY;
-                    }
-                }
-            }
-        }
-    }
-}
+int launch_attend_bf16(const AttendArgs& a, int lpr, int qr, bool fused, bool page16, dim3 grid, hipStream_t stream);
+int launch_attend_f16(const AttendArgs& a, int lpr, int qr, bool fused, bool page16, dim3 grid, hipStream_t stream);
+int launch_attend_fp8(const AttendArgs& a, int lpr, int qr, bool fused, bool page16, dim3 grid, hipStream_t stream);
+int launch_attend_fp8row(const AttendArgs& a, int lpr, int qr, bool fused, bool page16, dim3 grid, hipStream_t stream);
+int launch_attend_int8(const AttendArgs& a, int lpr, int qr, bool fused, bool page16, dim3 grid, hipStream_t stream);
 
 // One wavefront per (column, head, row): folds the partitions that hold the column's positions, in order.
 template <int DV>
@@ -501,42 +119,6 @@ static int pick_qr(int live_rows) {
     return 8;
 }
 
-template <int KIND, bool F16, int LPR, bool FUSED>
-static int launch_qr(const AttendArgs& a, int qr, dim3 grid, hipStream_t stream) {
-    switch (qr) {
-#define PKV_CASE(Q)                                                                                                  \
-    case Q:                                                                                                          \
-        hipLaunchKernelGGL((attend_kernel<KIND, F16, LPR, Q, FUSED>), grid, dim3(256), 0, stream, a);               \
-        break;
-        PKV_CASE(1) PKV_CASE(2) PKV_CASE(4) PKV_CASE(5) PKV_CASE(6) PKV_CASE(8)
-#undef PKV_CASE
-        default:
-            return CRIT_PKV_E_GEOMETRY;
-    }
-    return hip_code(hipGetLastError());
-}
-
-template <int KIND, bool F16, bool FUSED>
-static int launch_lpr(const AttendArgs& a, int lpr, int qr, dim3 grid, hipStream_t stream) {
-    switch (lpr) {
-        case 8: return launch_qr<KIND, F16, 8, FUSED>(a, qr, grid, stream);
-        case 16: return launch_qr<KIND, F16, 16, FUSED>(a, qr, grid, stream);
-        case 32: return launch_qr<KIND, F16, 32, FUSED>(a, qr, grid, stream);
-    }
-    return CRIT_PKV_E_GEOMETRY;
-}
-
-template <bool FUSED>
-static int launch_kind(const AttendArgs& a, int kind, bool f16, int lpr, int qr, dim3 grid, hipStream_t stream) {
-    switch (kind) {
-        case 0: return f16 ? launch_lpr<0, true, FUSED>(a, lpr, qr, grid, stream) : launch_lpr<0, false, FUSED>(a, lpr, qr, grid, stream);
-        case 1: return launch_lpr<1, false, FUSED>(a, lpr, qr, grid, stream);
-        case 2: return launch_lpr<2, false, FUSED>(a, lpr, qr, grid, stream);
-        case 3: return launch_lpr<3, false, FUSED>(a, lpr, qr, grid, stream);
-    }
-    return CRIT_PKV_E_DTYPE;
-}
-
 int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     if (!p || !p->q || !p->key_pages || !p->value_pages || !p->tables || !p->rows || !p->starts || !p->firsts || !p->out)
         return CRIT_PKV_E_NULL;
@@ -580,9 +162,20 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     const int64_t gx = (int64_t)p->n_rows * p->kv_heads * a.tiles;
     if (gx > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
     const dim3 grid((unsigned)gx, p->fused ? 1u : (unsigned)p->partitions);
+    const bool page16 = p->page % 16 == 0;
+    auto split = [&](bool fused) -> int {
+        switch (p->kind) {
+            case 0: return f16 ? launch_attend_f16(a, lpr, qr, fused, page16, grid, stream)
+                               : launch_attend_bf16(a, lpr, qr, fused, page16, grid, stream);
+            case 1: return launch_attend_fp8(a, lpr, qr, fused, page16, grid, stream);
+            case 2: return launch_attend_fp8row(a, lpr, qr, fused, page16, grid, stream);
+            case 3: return launch_attend_int8(a, lpr, qr, fused, page16, grid, stream);
+        }
+        return CRIT_PKV_E_DTYPE;
+    };
     int rc = 0;
-    if (p->fused) return launch_kind<true>(a, p->kind, f16, lpr, qr, grid, stream);
-    if (p->phases != 2) rc = launch_kind<false>(a, p->kind, f16, lpr, qr, grid, stream);
+    if (p->fused) return split(true);
+    if (p->phases != 2) rc = split(false);
     if (rc || p->phases == 1) return rc;
     if (p->heads > 65535 || p->n_rows > 65535) return CRIT_PKV_E_GEOMETRY;
     const dim3 mgrid((unsigned)p->columns, (unsigned)p->heads, (unsigned)p->n_rows);

@@ -1,0 +1,37 @@
+// Launch of the split (or fused) kernels for ONE page kind; each pkv_attend_k*.hip instantiates one kind so the
+// kinds compile in parallel.
+#pragma once
+#include "pkv_attend128.hpp"
+#include "pkv_attend_generic.hpp"
+
+namespace pkv {
+
+template <int KIND, bool F16, int QR, bool FUSED>
+static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipStream_t stream) {
+    if (lpr == 16) {
+        if (page16) hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, FUSED, true>), grid, dim3(256), 0, stream, a);
+        else hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, FUSED, false>), grid, dim3(256), 0, stream, a);
+    } else if (lpr == 8) {
+        hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 8, QR, FUSED>), grid, dim3(256), 0, stream, a);
+    } else if (lpr == 32) {
+        hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 32, QR, FUSED>), grid, dim3(256), 0, stream, a);
+    } else {
+        return CRIT_PKV_E_GEOMETRY;
+    }
+    return hip_code(hipGetLastError());
+}
+
+template <int KIND, bool F16>
+static int launch_kind_impl(const AttendArgs& a, int lpr, int qr, bool fused, bool page16, dim3 grid, hipStream_t stream) {
+    switch (qr) {
+#define PKV_CASE(Q)                                                                               \
+    case Q:                                                                                       \
+        return fused ? launch_one<KIND, F16, Q, true>(a, lpr, page16, grid, stream)               \
+                     : launch_one<KIND, F16, Q, false>(a, lpr, page16, grid, stream);
+        PKV_CASE(1) PKV_CASE(2) PKV_CASE(4) PKV_CASE(5) PKV_CASE(6) PKV_CASE(8)
+#undef PKV_CASE
+    }
+    return CRIT_PKV_E_GEOMETRY;
+}
+
+}   // namespace pkv
