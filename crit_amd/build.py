@@ -26,7 +26,7 @@ def sources():
 
 def _compile(src):
     obj = os.path.join(OBJ_DIR, os.path.basename(src)[:-4] + ".o")
-    cmd = ["hipcc", *FLAGS, "-c", src, "-o", obj]
+    cmd = ["hipcc", *FLAGS, *os.environ.get("CRIT_PKV_EXTRA_FLAGS", "").split(), "-c", src, "-o", obj]
     done = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(line for line in done.stderr.splitlines() if noise not in line)
@@ -44,13 +44,14 @@ def build(verbose=True, jobs=None):
     for _, err in found:
         if err.strip() and verbose:
             print(err, file=sys.stderr)
-    link = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *[obj for obj, _ in found]]
+    out = os.environ.get("CRIT_PKV_OUT", LIB)
+    link = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out, *[obj for obj, _ in found]]
     done = subprocess.run(link, capture_output=True, text=True)
     if done.returncode:
         raise RuntimeError(f"link failed:\n{done.stderr}")
     if verbose:
-        print(f"built {LIB}")
-    return LIB
+        print(f"built {out}")
+    return out
 
 
 if __name__ == "__main__":

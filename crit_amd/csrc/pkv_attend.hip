@@ -21,7 +21,8 @@ __global__ __launch_bounds__(64) void merge_kernel(AttendArgs a) {
     if (c >= count) return;
     int64_t first = a.firsts[r];
     first = first < 0 ? 0 : (first > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first);
-    const int nb = (int)min((int64_t)a.parts, (first + c + a.piece) / a.piece);
+    const int64_t seen = min(first + c + 1, (int64_t)a.max_keys);
+    const int nb = (int)min((int64_t)a.parts, (seen + a.piece - 1) / a.piece);
     const int64_t prow = a.offsets ? (int64_t)(a.offsets[r] - a.offsets[0]) : (int64_t)r * a.columns;
     const int64_t at = ((prow + c) * a.hq + head) * a.parts;
     float M = -INFINITY, L = 0.0f, A[EPL];
@@ -159,10 +160,22 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     const int live_rows = p->columns * a.g;
     const int qr = pick_qr(live_rows);
     a.tiles = (live_rows + qr - 1) / qr;
-    const int64_t gx = (int64_t)p->n_rows * p->kv_heads * a.tiles;
-    if (gx > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
-    const dim3 grid((unsigned)gx, p->fused ? 1u : (unsigned)p->partitions);
+    // The 128-wide kernel serves two adjacent KV heads per wavefront where the head count is even, so every position
+    // is read in segments of two rows (512 bytes of 16-bit pages, 256 of 8-bit ones): measured best on MI355X against
+    // one and four heads. Fixed by the cache's geometry, never by the launch: a column's bits depend on it.
     const bool page16 = p->page % 16 == 0;
+    a.heads_per_wave = 1;
+    if (lpr == 16 && page16) {
+        if (p->kv_heads % 2 == 0) a.heads_per_wave = 2;
+    }
+    const int64_t gx = (int64_t)p->n_rows * (p->kv_heads / a.heads_per_wave) * a.tiles;
+    if (gx > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
+    // Positions past the page tables do not exist: partitions that could only hold such pieces are not launched.
+    const int64_t table_keys = (int64_t)p->table_width * p->page;
+    a.max_keys = (int)(table_keys < 0x3fffffff ? table_keys : 0x3fffffff);
+    const int64_t live_parts = (a.max_keys + (int64_t)p->piece - 1) / p->piece;
+    const unsigned gy = (unsigned)(live_parts < p->partitions ? live_parts : p->partitions);
+    const dim3 grid((unsigned)gx, p->fused ? 1u : gy);
     auto split = [&](bool fused) -> int {
         switch (p->kind) {
             case 0: return f16 ? launch_attend_f16(a, lpr, qr, fused, page16, grid, stream)

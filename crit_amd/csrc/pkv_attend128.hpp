@@ -10,6 +10,10 @@
 //           per lane.
 //   values  16 lanes (one DPP row) hold one V row, 16 bytes (8 for 8-bit pages) each; a DPP row owns four of the
 //           step's positions and keeps its own online-softmax state and its own output accumulators for them.
+// A wavefront serves HW adjacent KV heads at once (DPP row rho: head rho % HW, position block rho / HW), so every
+// load instruction fetches HW x 128 contiguous bytes per position: 512-byte segments (2 heads of 16-bit pages, 4
+// heads of 8-bit pages) are what the HBM system streams at full rate from randomly placed pages; 128-byte and
+// 256-byte segments measurably are not.
 // The probabilities cross from the first layout to the second through LDS as 16-bit pairs of adjacent positions,
 // which is exactly the operand v_dot2 wants against the matching pairs of V values (built with v_perm_b32), so P.V
 // costs one dot2 per two multiply-adds. At the end the four DPP rows and the four wavefronts are folded in a fixed
@@ -73,11 +77,20 @@ struct Step128 {
     float ks, vs;      // row-scaled kinds: the scales of this lane's score position
 };
 
-template <int KIND, bool F16, int QR, bool FUSED, bool PAGE16>
-__global__ __launch_bounds__(256) void attend128_kernel(AttendArgs a) {
+// Wavefronts per SIMD the register allocation leaves room for: the keys' and values' register buffers of 16-bit pages
+// are twice those of 8-bit pages, and the query slices and accumulators grow with the tile's rows; more resident
+// workgroups hide each other's start-up latency, spills cost more than they give.
+constexpr int attend_waves(int kind, int qr) { return qr <= 2 ? 4 : (qr <= 4 && kind != 0 ? 3 : 2); }
+
+// Pages are a multiple of 16 positions, so the 16 positions of a step share one page table entry, which is uniform
+// over the wavefront: a step's addresses are a scalar base plus per-lane offsets that do not change from step to step.
+template <int KIND, bool F16, int QR, int HW, bool FUSED>
+__global__ __launch_bounds__(256, attend_waves(KIND, QR)) void attend128_kernel(AttendArgs a) {
     constexpr int D = 128;
     constexpr int RB = (QR + 3) / 4;            // blocks of four query rows
     constexpr int EB = KIND == 0 ? 2 : 1;
+    constexpr int PB = 4 / HW;                  // position blocks (of 4 positions) a wavefront's step holds
+    constexpr int SPW = 4 * PB;                 // positions a wavefront's step covers
     constexpr int EPT = (QR * D + 255) / 256;
     __shared__ __align__(16) float s_acc[4][QR][D];
     __shared__ float s_m[4][QR], s_l[4][QR];
@@ -89,13 +102,15 @@ __global__ __launch_bounds__(256) void attend128_kernel(AttendArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int rho = lane >> 4, lam = lane & 15;
     const int b3 = (lane >> 3) & 1, b2 = (lane >> 2) & 1, b1 = (lane >> 1) & 1, b0 = lane & 1;
-    const int g8 = lane >> 3, li8 = lane & 7;
+    const int li8 = lane & 7;
     const int q4 = 2 * b2 + b3;                 // which of the DPP row's four positions this lane's score is of
+    const int hw = rho % HW, pb = rho / HW;     // the DPP row's head (of the wavefront's HW) and position block
     int bx = blockIdx.x;
     const int tile = bx % a.tiles;
     bx /= a.tiles;
-    const int kvh = bx % a.hkv;
-    const int r = bx / a.hkv;
+    const int hgroups = a.hkv / HW;
+    const int kvh = (bx % hgroups) * HW + hw;   // this lane's KV head
+    const int r = bx / hgroups;
     const int b = blockIdx.y;
     int count = a.columns;
     if (a.counts) count = min(a.counts[r], a.columns);
@@ -105,7 +120,7 @@ __global__ __launch_bounds__(256) void attend128_kernel(AttendArgs a) {
     const int c_lo = j0 / a.g;
     const int c_hi = min(count, (j0 + QR - 1) / a.g + 1);
     int64_t nk64 = first64 + c_hi;
-    nk64 = nk64 < 0 ? 0 : (nk64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : nk64);
+    nk64 = nk64 < 0 ? 0 : (nk64 > (int64_t)a.max_keys ? (int64_t)a.max_keys : nk64);
     const int n_keys = (int)nk64;
     const int first = (int)(first64 < 0 ? 0 : (first64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first64));
     const int n_pieces = (n_keys + a.piece - 1) / a.piece;
@@ -142,76 +157,76 @@ __global__ __launch_bounds__(256) void attend128_kernel(AttendArgs a) {
         const int c = j / a.g;
         my_lim[blk] = (4 * blk + 2 * b1 + b0 < QR && c < count) ? first + c : -1;
     }
-    float k_mult = a.k_mult, v_mult = a.v_mult;
-    if (KIND == 1 && a.hm) k_mult = a.hm[kvh], v_mult = a.hm[a.hkv + kvh];
+    float k_mult = a.k_mult;
+    if (KIND == 1 && a.hm) k_mult = a.hm[kvh];
     const float sscale = a.sscale * (KIND == 1 ? k_mult : 1.0f);
-    if (KIND != 1) v_mult = 1.0f;
     const int win = a.sliding;
 
-    const int64_t slot_bytes = (int64_t)a.hkv * D * EB;
-    const uint8_t* kbase = a.kp + (int64_t)kvh * D * EB + li8 * 16;
-    const uint8_t* vbase = a.vp + (int64_t)kvh * D * EB + lam * (8 * EB);
+    // Offsets of the positions this lane reads within a step (its two K rows, its DPP row's four V rows, its score),
+    // and their byte offsets from the step's first slot: the same every step but the row's last.
+    const int slot_bytes = a.hkv * D * EB;
+    const int koff[2] = {4 * pb + b3, 4 * pb + 2 + b3};
+    const int voff[4] = {4 * pb, 4 * pb + 1, 4 * pb + 2, 4 * pb + 3};
+    const int soff = 4 * pb + q4;
+    const uint32_t klane = (uint32_t)(kvh * D * EB + li8 * 16);
+    const uint32_t vlane = (uint32_t)(kvh * D * EB + lam * 8 * EB);
+    uint32_t kvo[2], vvo[4];
+#pragma unroll
+    for (int pr = 0; pr < 2; ++pr) kvo[pr] = (uint32_t)(koff[pr] * slot_bytes) + klane;
+#pragma unroll
+    for (int kv = 0; kv < 4; ++kv) vvo[kv] = (uint32_t)(voff[kv] * slot_bytes) + vlane;
+    const uint32_t svo = (uint32_t)(soff * a.hkv + kvh);
 
-    // Offsets of the positions this lane reads within a step: its two K rows, its row's four V rows, its score.
-    const int koff[2] = {g8, 8 + g8};
-    const int soff = 8 * b2 + 2 * rho + b3;
-
-    struct Tab {
-        int k[2], v[4], s;      // page table entries (PAGE16: one entry serves the step, in k[0])
-    };
-    auto clampn = [&](int n) { return n < n_keys ? n : n_keys - 1; };
-    auto entry = [&](int n) -> int {
-        int pidx = a.page_shift >= 0 ? (n >> a.page_shift) : (n / a.page);
+    auto entry = [&](int base) -> int {     // the page table entry of a step (uniform over the wavefront)
+        int pidx = a.page_shift >= 0 ? (base >> a.page_shift) : (base / a.page);
         pidx = pidx < a.tab_width ? pidx : a.tab_width - 1;
         return a.tables[trow + pidx];
     };
-    auto fetch_tab = [&](int base, Tab& t) {
-        if constexpr (PAGE16) {
-            t.k[0] = entry(base);      // the step's 16 positions share a page (page is a multiple of 16)
-        } else {
-            t.k[0] = entry(clampn(base + koff[0])), t.k[1] = entry(clampn(base + koff[1]));
+    // The step's first slot (uniform): page entry * page + base's offset in its page.
+    auto first_slot = [&](int base, int e) -> int64_t {
+        const int pidx = a.page_shift >= 0 ? (base >> a.page_shift) : (base / a.page);
+        return (int64_t)__builtin_amdgcn_readfirstlane(e) * a.page + (base - pidx * a.page);
+    };
+    auto fetch_k = [&](int base, int e, Step128<KIND>& buf) {
+        const int64_t slot0 = first_slot(base, e);
+        const uint8_t* sbase = a.kp + slot0 * slot_bytes;
+        uint32_t o[2] = {kvo[0], kvo[1]};
+        uint32_t so = svo;
+        if (base + SPW > n_keys) {      // the row's last step: positions past its keys read its last key instead
 #pragma unroll
-            for (int kv = 0; kv < 4; ++kv) t.v[kv] = entry(clampn(base + 8 * (kv >> 1) + 2 * rho + (kv & 1)));
-            if constexpr (KIND >= 2) t.s = entry(clampn(base + soff));
+            for (int pr = 0; pr < 2; ++pr) o[pr] = (uint32_t)(min(koff[pr], n_keys - 1 - base) * slot_bytes) + klane;
+            so = (uint32_t)(min(soff, n_keys - 1 - base) * a.hkv + kvh);
         }
-    };
-    auto slot_of = [&](int base, int off, int page_entry) -> int64_t {
-        const int n = clampn(base + off);
-        int in_page;
-        if constexpr (PAGE16) {
-            const int pidx = a.page_shift >= 0 ? (base >> a.page_shift) : (base / a.page);
-            in_page = n - pidx * a.page;
-        } else {
-            in_page = a.page_shift >= 0 ? (n & (a.page - 1)) : (n % a.page);
-        }
-        return (int64_t)page_entry * a.page + in_page;
-    };
-    auto fetch_kv = [&](int base, const Tab& t, Step128<KIND>& buf) {
 #pragma unroll
         for (int pr = 0; pr < 2; ++pr) {
-            const uint8_t* row = kbase + slot_of(base, koff[pr], PAGE16 ? t.k[0] : t.k[pr]) * slot_bytes;
             if constexpr (KIND == 0) {
-                buf.k[2 * pr] = *reinterpret_cast<const uint4*>(row);
-                buf.k[2 * pr + 1] = *reinterpret_cast<const uint4*>(row + 128);
+                buf.k[2 * pr] = *reinterpret_cast<const uint4*>(sbase + o[pr]);
+                buf.k[2 * pr + 1] = *reinterpret_cast<const uint4*>(sbase + o[pr] + 128);
             } else {
-                buf.k[pr] = *reinterpret_cast<const uint4*>(row);
+                buf.k[pr] = *reinterpret_cast<const uint4*>(sbase + o[pr]);
             }
         }
-#pragma unroll
-        for (int kv = 0; kv < 4; ++kv) {
-            const int64_t slot = slot_of(base, 8 * (kv >> 1) + 2 * rho + (kv & 1), PAGE16 ? t.k[0] : t.v[kv]);
-            buf.v[kv] = *reinterpret_cast<const typename Step128<KIND>::VVec*>(vbase + slot * slot_bytes);
-        }
         if constexpr (KIND >= 2) {
-            const int64_t slot = slot_of(base, soff, PAGE16 ? t.k[0] : t.s);
-            buf.ks = a.ks[slot * a.hkv + kvh];
-            buf.vs = a.vs[slot * a.hkv + kvh];
+            buf.ks = (a.ks + slot0 * a.hkv)[so];
+            buf.vs = (a.vs + slot0 * a.hkv)[so];
         }
     };
-
-    float run_m[EPT], run_l[EPT], run_a[EPT];
+    auto fetch_v = [&](int base, int e, Step128<KIND>& buf) {
+        const uint8_t* sbase = a.vp + first_slot(base, e) * slot_bytes;
+        uint32_t o[4] = {vvo[0], vvo[1], vvo[2], vvo[3]};
+        if (base + SPW > n_keys) {
 #pragma unroll
-    for (int e = 0; e < EPT; ++e) run_m[e] = -INFINITY, run_l[e] = 0.0f, run_a[e] = 0.0f;
+            for (int kv = 0; kv < 4; ++kv) o[kv] = (uint32_t)(min(voff[kv], n_keys - 1 - base) * slot_bytes) + vlane;
+        }
+#pragma unroll
+        for (int kv = 0; kv < 4; ++kv) buf.v[kv] = *reinterpret_cast<const typename Step128<KIND>::VVec*>(sbase + o[kv]);
+    };
+
+    float run_m[FUSED ? HW : 1][EPT], run_l[FUSED ? HW : 1][EPT], run_a[FUSED ? HW : 1][EPT];
+#pragma unroll
+    for (int i = 0; i < (FUSED ? HW : 1); ++i)
+#pragma unroll
+        for (int e = 0; e < EPT; ++e) run_m[i][e] = -INFINITY, run_l[i][e] = 0.0f, run_a[i][e] = 0.0f;
 
     const int part_lo = FUSED ? 0 : b;
     const int part_hi = FUSED ? min(a.parts, n_pieces) : b + 1;
@@ -233,18 +248,19 @@ __global__ __launch_bounds__(256) void attend128_kernel(AttendArgs a) {
             if (below > 0) pi = part + (below + a.parts - 1) / a.parts * a.parts;
         }
         auto base_of = [&]() -> int {
-            if (st * 16 >= a.piece) return -1;
-            const int64_t base = (int64_t)pi * a.piece + st * 16;
+            if (st * SPW >= a.piece) return -1;
+            const int64_t base = (int64_t)pi * a.piece + st * SPW;
             return base < n_keys ? (int)base : -1;
         };
         auto advance = [&]() -> int {
             st += 4;
-            if (st * 16 >= a.piece) pi += a.parts, st = wave;
+            if (st * SPW >= a.piece) pi += a.parts, st = wave;
             return base_of();
         };
 
-        auto compute = [&](int base, const Step128<KIND>& buf) {
-            // -- scores: each lane's partial dots of its K slices with every query row, pairs A and B
+        // Scores and softmax of one step: leaves the step's probabilities (pairs of adjacent positions per query row)
+        // in pp and has rescaled the accumulators where a row's maximum moved.
+        auto scores = [&](int base, const Step128<KIND>& buf, uint32_t (&pp)[RB * 4][2]) {
             float dpart[2][RB * 4];
 #pragma unroll
             for (int pr = 0; pr < 2; ++pr) {
@@ -269,11 +285,10 @@ __global__ __launch_bounds__(256) void attend128_kernel(AttendArgs a) {
                     dpart[pr][rr] = d;
                 }
             }
-            // -- per block of four query rows: transposing reduction over the 8 lanes of a K row, then the softmax
-            //    update of the one score the lane is left with
             float alpha_any = 1.0f;
 #pragma unroll
             for (int blk = 0; blk < RB; ++blk) {
+                // transposing reduction over the 8 lanes of a K row: 8 partial sums in, 1 finished score out
                 float t2[2][2];
 #pragma unroll
                 for (int pr = 0; pr < 2; ++pr) {
@@ -313,8 +328,6 @@ __global__ __launch_bounds__(256) void attend128_kernel(AttendArgs a) {
                 if (q4 == 0) s_alpha[wave][rho][4 * blk + 2 * b1 + b0] = alpha;
             }
             __builtin_amdgcn_wave_barrier();
-            // -- probabilities back, as pairs of adjacent positions per query row
-            uint32_t pp[RB * 4][2];
 #pragma unroll
             for (int h2 = 0; h2 < RB * 2; ++h2) {
                 const uint4 w = *reinterpret_cast<const uint4*>(&s_p[wave][rho][2 * h2][0]);
@@ -335,7 +348,9 @@ __global__ __launch_bounds__(256) void attend128_kernel(AttendArgs a) {
                 }
             }
             __builtin_amdgcn_wave_barrier();
-            // -- P.V: pairs of positions (0,1) and (2,3) of the row against the matching pairs of V values
+        };
+        // P.V of one step: pairs of positions (0,1) and (2,3) of the DPP row against the matching pairs of V values.
+        auto values = [&](const Step128<KIND>& buf, const uint32_t (&pp)[RB * 4][2]) {
 #pragma unroll
             for (int kp = 0; kp < 2; ++kp) {
                 uint32_t pv[8];
@@ -367,29 +382,45 @@ __global__ __launch_bounds__(256) void attend128_kernel(AttendArgs a) {
             }
         };
 
-        // Three-stage software pipeline: table entries two steps ahead, K/V one step ahead, compute.
+        // Software pipeline over two register buffers: a step's keys are reloaded (for two steps ahead) as soon as its
+        // scores are done, its values as soon as its P.V is done, so between one and two steps are in flight; the page
+        // table entries run one step further ahead. Every load of the loop is issued unconditionally (past the
+        // wavefront's last step it re-reads its first step, which the caches hold): with straight-line loads the
+        // compiler counts the outstanding ones exactly and waits only for the step it is about to use.
         Step128<KIND> bufA, bufB;
-        Tab tabA, tabB;
+        uint32_t pp[RB * 4][2];
         int base0 = base_of();
-        if (base0 >= 0) fetch_tab(base0, tabA);
-        int base1 = base0 >= 0 ? advance() : -1;
-        if (base0 >= 0) fetch_kv(base0, tabA, bufA);
-        if (base1 >= 0) fetch_tab(base1, tabB);
-        while (base0 >= 0) {
+        if (base0 >= 0) {
+            const int again = base0;
+            auto safe = [&](int base) { return base >= 0 ? base : again; };
+            int e0 = entry(base0);
+            int base1 = advance();
+            int e1 = entry(safe(base1));
             int base2 = base1 >= 0 ? advance() : -1;
-            if (base1 >= 0) fetch_kv(base1, tabB, bufB);
-            if (base2 >= 0) fetch_tab(base2, tabA);
-            compute(base0, bufA);
-            if (base1 < 0) break;
-            base0 = base2 >= 0 ? advance() : -1;
-            if (base2 >= 0) fetch_kv(base2, tabA, bufA);
-            if (base0 >= 0) fetch_tab(base0, tabB);
-            compute(base1, bufB);
-            base1 = base0;
-            base0 = base2;
+            int e2 = entry(safe(base2));
+            fetch_k(base0, e0, bufA), fetch_v(base0, e0, bufA);
+            fetch_k(safe(base1), e1, bufB), fetch_v(safe(base1), e1, bufB);
+            for (;;) {
+                const int base3 = base2 >= 0 ? advance() : -1;
+                const int e3 = entry(safe(base3));
+                scores(base0, bufA, pp);
+                fetch_k(safe(base2), e2, bufA);
+                values(bufA, pp);
+                fetch_v(safe(base2), e2, bufA);
+                if (base1 < 0) break;
+                const int base4 = base3 >= 0 ? advance() : -1;
+                const int e4 = entry(safe(base4));
+                scores(base1, bufB, pp);
+                fetch_k(safe(base3), e3, bufB);
+                values(bufB, pp);
+                fetch_v(safe(base3), e3, bufB);
+                if (base2 < 0) break;
+                base0 = base2, base1 = base3, base2 = base4, e2 = e4;
+            }
         }
 
-        // Fold the wavefront's four DPP rows: every lane needs each query row's maximum and sum of every DPP row.
+        // Fold the DPP rows that served the same head (its position blocks): every lane needs each query row's
+        // maximum and sum of those rows.
 #pragma unroll
         for (int blk = 0; blk < RB; ++blk) {
             if (q4 == 0) s_rm[wave][rho][4 * blk + 2 * b1 + b0] = m[blk], s_rl[wave][rho][4 * blk + 2 * b1 + b0] = l[blk];
@@ -398,65 +429,75 @@ __global__ __launch_bounds__(256) void attend128_kernel(AttendArgs a) {
         float wm[QR], wl[QR];
 #pragma unroll
         for (int rr = 0; rr < QR; ++rr) {
-            float top = s_rm[wave][0][rr];
+            float top = s_rm[wave][hw][rr];
 #pragma unroll
-            for (int o = 1; o < 4; ++o) top = __builtin_fmaxf(top, s_rm[wave][o][rr]);
+            for (int o = 1; o < PB; ++o) top = __builtin_fmaxf(top, s_rm[wave][hw + HW * o][rr]);
             const float sub = top == -INFINITY ? 0.0f : top;
             float lsum = 0.0f;
 #pragma unroll
-            for (int o = 0; o < 4; ++o) lsum = __builtin_fmaf(s_rl[wave][o][rr], exp2_fast(s_rm[wave][o][rr] - sub), lsum);
-            const float w = exp2_fast(s_rm[wave][rho][rr] - sub);
+            for (int o = 0; o < PB; ++o) lsum = __builtin_fmaf(s_rl[wave][hw + HW * o][rr], exp2_fast(s_rm[wave][hw + HW * o][rr] - sub), lsum);
+            if constexpr (PB > 1) {
+                const float w = exp2_fast(s_rm[wave][rho][rr] - sub);
 #pragma unroll
-            for (int d = 0; d < 8; ++d) {
-                float x = acc[rr][d] * w;
-                x += __shfl_xor(x, 16);
-                x += __shfl_xor(x, 32);
-                acc[rr][d] = x;
+                for (int d = 0; d < 8; ++d) {
+                    float x = acc[rr][d] * w;
+#pragma unroll
+                    for (int o = 16 * HW; o < 64; o <<= 1) x += __shfl_xor(x, o);
+                    acc[rr][d] = x;
+                }
             }
             wm[rr] = top, wl[rr] = lsum;
         }
-        if (FUSED) __syncthreads();      // the previous partition's fold has read the LDS
-        if (rho == 0) {
+        // Then the four wavefronts, one head of the wavefront at a time through LDS, in wavefront order.
 #pragma unroll
-            for (int rr = 0; rr < QR; ++rr) {
-                *reinterpret_cast<float4*>(&s_acc[wave][rr][lam * 8]) = make_float4(acc[rr][0], acc[rr][1], acc[rr][2], acc[rr][3]);
-                *reinterpret_cast<float4*>(&s_acc[wave][rr][lam * 8 + 4]) = make_float4(acc[rr][4], acc[rr][5], acc[rr][6], acc[rr][7]);
-                if (lam == 0) s_m[wave][rr] = wm[rr], s_l[wave][rr] = wl[rr];
-            }
-        }
-        __syncthreads();
+        for (int head_i = 0; head_i < HW; ++head_i) {
+            if (FUSED || head_i > 0) __syncthreads();      // the previous fold has read the LDS
+            if (rho == head_i) {
 #pragma unroll
-        for (int e = 0; e < EPT; ++e) {
-            const int idx = tid + e * 256;
-            if (idx < QR * D) {
-                const int rr = idx / D, d = idx % D;
-                float M = s_m[0][rr];
-#pragma unroll
-                for (int w = 1; w < 4; ++w) M = __builtin_fmaxf(M, s_m[w][rr]);
-                const float sub = M == -INFINITY ? 0.0f : M;
-                float L = 0.0f, A = 0.0f;
-#pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    const float f = exp2_fast(s_m[w][rr] - sub);
-                    L = __builtin_fmaf(s_l[w][rr], f, L);
-                    A = __builtin_fmaf(s_acc[w][rr][d], f, A);
+                for (int rr = 0; rr < QR; ++rr) {
+                    *reinterpret_cast<float4*>(&s_acc[wave][rr][lam * 8]) = make_float4(acc[rr][0], acc[rr][1], acc[rr][2], acc[rr][3]);
+                    *reinterpret_cast<float4*>(&s_acc[wave][rr][lam * 8 + 4]) = make_float4(acc[rr][4], acc[rr][5], acc[rr][6], acc[rr][7]);
+                    if (lam == 0) s_m[wave][rr] = wm[rr], s_l[wave][rr] = wl[rr];
                 }
-                A *= v_mult;
-                const int j = j0 + rr;
-                const int c = j / a.g;
-                if (c < count) {
-                    if constexpr (FUSED) {
-                        const int held = min(a.parts, (first + c + a.piece) / a.piece);
-                        if (part < held) {
-                            const Fold f = fold(run_m[e], run_l[e], M, L);
-                            run_a[e] = __builtin_fmaf(run_a[e], f.keep, A * f.take);
-                            run_m[e] = f.m, run_l[e] = f.l;
+            }
+            __syncthreads();
+            const int head_kv = (kvh - hw) + head_i;      // the KV head being folded (uniform)
+            float vm = a.v_mult;
+            if (KIND == 1 && a.hm) vm = a.hm[a.hkv + head_kv];
+            if (KIND != 1) vm = 1.0f;
+#pragma unroll
+            for (int e = 0; e < EPT; ++e) {
+                const int idx = tid + e * 256;
+                if (idx < QR * D) {
+                    const int rr = idx / D, d = idx % D;
+                    float M = s_m[0][rr];
+#pragma unroll
+                    for (int w = 1; w < 4; ++w) M = __builtin_fmaxf(M, s_m[w][rr]);
+                    const float sub = M == -INFINITY ? 0.0f : M;
+                    float L = 0.0f, A = 0.0f;
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        const float f = exp2_fast(s_m[w][rr] - sub);
+                        L = __builtin_fmaf(s_l[w][rr], f, L);
+                        A = __builtin_fmaf(s_acc[w][rr][d], f, A);
+                    }
+                    A *= vm;
+                    const int j = j0 + rr;
+                    const int c = j / a.g;
+                    if (c < count) {
+                        if constexpr (FUSED) {
+                            const int held = min(a.parts, (min(first + c + 1, a.max_keys) + a.piece - 1) / a.piece);
+                            if (part < held) {
+                                const Fold f = fold(run_m[head_i][e], run_l[head_i][e], M, L);
+                                run_a[head_i][e] = __builtin_fmaf(run_a[head_i][e], f.keep, A * f.take);
+                                run_m[head_i][e] = f.m, run_l[head_i][e] = f.l;
+                            }
+                        } else {
+                            const int64_t prow = a.offsets ? (int64_t)(a.offsets[r] - a.offsets[0]) : (int64_t)r * a.columns;
+                            const int64_t at = ((prow + c) * a.hq + head_kv * a.g + j % a.g) * a.parts + b;
+                            a.po[at * D + d] = A;
+                            if (d == 0) a.pm[at] = M, a.pl[at] = L;
                         }
-                    } else {
-                        const int64_t prow = a.offsets ? (int64_t)(a.offsets[r] - a.offsets[0]) : (int64_t)r * a.columns;
-                        const int64_t at = ((prow + c) * a.hq + kvh * a.g + j % a.g) * a.parts + b;
-                        a.po[at * D + d] = A;
-                        if (d == 0) a.pm[at] = M, a.pl[at] = L;
                     }
                 }
             }
@@ -464,23 +505,27 @@ __global__ __launch_bounds__(256) void attend128_kernel(AttendArgs a) {
     }
     if constexpr (FUSED) {
 #pragma unroll
-        for (int e = 0; e < EPT; ++e) {
-            const int idx = tid + e * 256;
-            if (idx < QR * D) {
-                const int rr = idx / D, d = idx % D;
-                const int j = j0 + rr;
-                const int c = j / a.g;
-                if (c < count) {
-                    const int head = kvh * a.g + j % a.g;
-                    float M = run_m[e], L = run_l[e], A = run_a[e];
-                    if (a.sinks) {
-                        const Fold f = fold(M, L, a.sinks[head] * kLog2e, 1.0f);
-                        A *= f.keep, M = f.m, L = f.l;
-                    }
-                    const float o = L != 0.0f ? A / L : 0.0f;
-                    store_out(a.out, a.out_dtype, (int64_t)(start + c) * a.o_st + (int64_t)head * a.o_sh + d, o);
-                    if (a.lse && d == 0) {
-                        a.lse[(int64_t)(start + c) * a.hq + head] = L != 0.0f ? __builtin_fmaf(M, kLn2, __logf(L)) : -INFINITY;
+        for (int head_i = 0; head_i < HW; ++head_i) {
+            const int head_kv = (kvh - hw) + head_i;
+#pragma unroll
+            for (int e = 0; e < EPT; ++e) {
+                const int idx = tid + e * 256;
+                if (idx < QR * D) {
+                    const int rr = idx / D, d = idx % D;
+                    const int j = j0 + rr;
+                    const int c = j / a.g;
+                    if (c < count) {
+                        const int head = head_kv * a.g + j % a.g;
+                        float M = run_m[head_i][e], L = run_l[head_i][e], A = run_a[head_i][e];
+                        if (a.sinks) {
+                            const Fold f = fold(M, L, a.sinks[head] * kLog2e, 1.0f);
+                            A *= f.keep, M = f.m, L = f.l;
+                        }
+                        const float o = L != 0.0f ? A / L : 0.0f;
+                        store_out(a.out, a.out_dtype, (int64_t)(start + c) * a.o_st + (int64_t)head * a.o_sh + d, o);
+                        if (a.lse && d == 0) {
+                            a.lse[(int64_t)(start + c) * a.hq + head] = L != 0.0f ? __builtin_fmaf(M, kLn2, __logf(L)) : -INFINITY;
+                        }
                     }
                 }
             }

@@ -26,7 +26,7 @@ struct AttendArgs {
     float* lse;
     const float* sinks;
     int64_t q_st, q_sh, o_st, o_sh, tab_stride;
-    int tab_width, n_rows, columns, hq, hkv, g, page, page_shift, parts, piece, sliding, out_dtype, tiles;
+    int tab_width, n_rows, columns, hq, hkv, g, page, page_shift, parts, piece, sliding, out_dtype, tiles, max_keys, heads_per_wave;
     float sscale, k_mult, v_mult;
 };
 

@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
     const int c_lo = j0 / a.g;
     const int c_hi = min(count, (j0 + QR - 1) / a.g + 1);
     int64_t nk64 = first64 + c_hi;
-    nk64 = nk64 < 0 ? 0 : (nk64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : nk64);
+    nk64 = nk64 < 0 ? 0 : (nk64 > (int64_t)a.max_keys ? (int64_t)a.max_keys : nk64);
     const int n_keys = (int)nk64;
     const int first = (int)(first64 < 0 ? 0 : (first64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first64));
     const int n_pieces = (n_keys + a.piece - 1) / a.piece;
@@ -325,7 +325,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
                 if (c < count) {
                     if constexpr (FUSED) {
                         // A column folds the partitions that hold its positions, as the merge does.
-                        const int held = min(a.parts, (first + c + a.piece) / a.piece);
+                        const int held = min(a.parts, (min(first + c + 1, a.max_keys) + a.piece - 1) / a.piece);
                         if (part < held) {
                             const Fold f = fold(run_m[e], run_l[e], M, L);
                             run_a[e] = __builtin_fmaf(run_a[e], f.keep, A * f.take);

@@ -8,9 +8,15 @@ namespace pkv {
 
 template <int KIND, bool F16, int QR, bool FUSED>
 static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipStream_t stream) {
-    if (lpr == 16) {
-        if (page16) hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, FUSED, true>), grid, dim3(256), 0, stream, a);
-        else hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, FUSED, false>), grid, dim3(256), 0, stream, a);
+    if (lpr == 16 && page16) {       // pages of a multiple of 16 positions: the bandwidth path
+        switch (a.heads_per_wave) {
+            case 1: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 1, FUSED>), grid, dim3(256), 0, stream, a); break;
+            case 2: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 2, FUSED>), grid, dim3(256), 0, stream, a); break;
+            case 4: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 4, FUSED>), grid, dim3(256), 0, stream, a); break;
+            default: return CRIT_PKV_E_GEOMETRY;
+        }
+    } else if (lpr == 16) {
+        hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 16, QR, FUSED>), grid, dim3(256), 0, stream, a);
     } else if (lpr == 8) {
         hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 8, QR, FUSED>), grid, dim3(256), 0, stream, a);
     } else if (lpr == 32) {

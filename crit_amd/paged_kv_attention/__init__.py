@@ -38,7 +38,7 @@ __all__ = ["KINDS", "PIECE", "MAX_COLUMNS", "Derive", "attend", "derive", "cuda_
            "tile_for", "workspace_floats", "write"]
 
 KINDS = {"bf16": 0, "fp16": 0, "fp8": 1, "fp8:row": 2, "int8": 3}
-PIECE = 512          # positions per piece of FP8 or INT8 pages at a 128-wide head (piece_size)
+PIECE = 2048         # positions per piece of FP8 or INT8 pages at a 128-wide head (piece_size)
 MAX_COLUMNS = 64     # columns of one row a launch reads
 MAX_QUERY_ROWS = 8   # query rows (columns x group heads) one workgroup holds; wider windows take more tiles
 
@@ -154,22 +154,24 @@ def _cus(device):
 # -- the split's order knobs -----------------------------------------------------------------------------------------------
 def partitions(device, kv_heads, kind, head_dim=None, value_dim=None):
     """The partition count for a cache of `kv_heads` heads on `device`: about two workgroups per compute unit for one
-    long row (a power of two within 8..64). A column's bits depend on it: one count per cache."""
+    long row, a workgroup serving two KV heads (a power of two within 8..64; partitions past a launch's page tables
+    are never launched, so a large count costs short rows nothing). A column's bits depend on it: one count per
+    cache."""
     if kind not in KINDS:
         raise ValueError(f"page kinds are {', '.join(KINDS)}, not {kind!r}")
     programs = 2 * _cus(torch.device(device))
-    wanted = max(1, programs // max(1, int(kv_heads)))
+    wanted = max(1, programs // max(1, int(kv_heads) // 2))
     return max(8, min(64, 1 << (wanted - 1).bit_length()))
 
 
 def piece_size(head_dim, value_dim, kind="bf16", kv_heads=None):
-    """Positions per piece: 32 Ki head values for 16-bit pages, 64 Ki for 8-bit ones (128 KiB of keys and values of
-    one KV head either way), within 64..512. A column's bits depend on it; it follows the cache's geometry and page
-    kind only."""
+    """Positions per piece: 128 Ki head values for 16-bit pages, 256 Ki for 8-bit ones (512 KiB of keys and values of
+    one KV head either way: measured on MI355X, a workgroup's start-up is then a few percent of its streaming),
+    within 256..2048. A column's bits depend on it; it follows the cache's geometry and page kind only."""
     if kind not in KINDS:
         raise ValueError(f"page kinds are {', '.join(KINDS)}, not {kind!r}")
-    values = 32768 if KINDS[kind] == 0 else 65536
-    return max(64, min(512, values // max(int(head_dim), int(value_dim))))
+    values = 131072 if KINDS[kind] == 0 else 262144
+    return max(256, min(2048, values // max(int(head_dim), int(value_dim))))
 
 
 def tile_for(columns, group, capability, fused=False):
