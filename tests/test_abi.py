@@ -1,0 +1,87 @@
+"""The C-ABI library loads on a machine without a GPU and exports every entry point include/crit_pkv.h declares; the
+Python mirror of the parameter structs has the library's sizes. No compute call is made here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "crit_pkv.h")
+
+
+def _declared():
+    text = open(HEADER, encoding="utf-8").read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(crit_pkv_\w+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from crit_amd.paged_kv_attention import _abi
+    return _abi.load()
+
+
+def test_the_header_declares_the_entry_points():
+    names = _declared()
+    for want in ("crit_pkv_write", "crit_pkv_attend", "crit_pkv_merge", "crit_pkv_prefill", "crit_pkv_error",
+                 "crit_pkv_params_size", "crit_pkv_abi_version", "crit_pkv_stream_read"):
+        assert want in names
+
+
+def test_the_library_exports_every_declared_symbol(lib):
+    for name in _declared():
+        assert hasattr(lib, name), name
+
+
+def test_struct_mirrors_match_the_library(lib):
+    from crit_amd.paged_kv_attention import _abi
+    assert lib.crit_pkv_abi_version() == _abi.ABI_VERSION
+    for which, struct in enumerate((_abi.WriteParams, _abi.AttendParams, _abi.MergeParams, _abi.PrefillParams)):
+        assert lib.crit_pkv_params_size(which) == ctypes.sizeof(struct)
+    assert lib.crit_pkv_params_size(99) == -1
+
+
+def test_error_strings(lib):
+    assert lib.crit_pkv_error(0) == b"ok"
+    for code in (-1, -2, -3, -4):
+        assert lib.crit_pkv_error(code).startswith(b"crit_pkv:")
+    from crit_amd.paged_kv_attention import _abi
+    with pytest.raises(ValueError, match="crit_pkv"):
+        _abi.check(-1, "x")
+    _abi.check(0, "x")
+
+
+def test_null_parameters_are_refused_without_touching_a_gpu(lib):
+    from crit_amd.paged_kv_attention import _abi
+    for fn, struct in ((lib.crit_pkv_write, _abi.WriteParams), (lib.crit_pkv_attend, _abi.AttendParams),
+                       (lib.crit_pkv_merge, _abi.MergeParams), (lib.crit_pkv_prefill, _abi.PrefillParams)):
+        assert fn(ctypes.byref(struct()), None) == -3          # CRIT_PKV_E_NULL: nothing was launched
+
+
+def test_the_module_keeps_the_reference_interface():
+    # names and signatures crit's KVPool and DeviceAttention call (reference __init__.py:74-80, 260-362, 396-400, 1245)
+    import inspect
+    import crit_amd.paged_kv_attention as pk
+    assert pk.MAX_COLUMNS == 64 and pk.KINDS == {"bf16": 0, "fp16": 0, "fp8": 1, "fp8:row": 2, "int8": 3}
+    for name in ("write", "attend", "prefill", "partitions", "piece_size", "tile_for", "workspace_floats", "flash_chunk",
+                 "flash_parts", "flash_block", "flash_tile", "cuda_chunk", "cuda_parts", "cuda_prompt", "owner", "release"):
+        assert callable(getattr(pk, name)), name
+    assert list(inspect.signature(pk.write).parameters) == [
+        "keys", "values", "slots", "key_pages", "value_pages", "kind", "key_scales", "value_scales", "multipliers"]
+    attend = inspect.signature(pk.attend).parameters
+    assert list(attend)[:10] == ["q", "key_pages", "value_pages", "kind", "tables", "rows", "starts", "firsts", "columns",
+                                 "page"]
+    for name in ("counts", "offsets", "tokens", "key_scales", "value_scales", "multipliers", "scale", "partitions",
+                 "parents", "blocks", "block_size", "out", "lse", "workspace", "piece", "fused", "fresh", "flash", "chunk",
+                 "sinks", "sliding", "derive"):
+        assert attend[name].kind is inspect.Parameter.KEYWORD_ONLY, name
+    prefill = inspect.signature(pk.prefill).parameters
+    assert list(prefill)[:7] == ["q", "key_pages", "value_pages", "kind", "table", "position", "page"]
+    assert pk.workspace_floats(3, 8, 16, 128) == 3 * 8 * 16 * 130
+    assert pk.tile_for(1, 4, (9, 5))[0] // 4 == 1 and pk.tile_for(5, 4, (9, 5))[0] // 4 <= 5
+    assert pk.piece_size(128, 128, "bf16") % 16 == 0 and pk.flash_chunk(128, 128, 32, 8, 16) % pk.flash_block(128, 128, 32, 8, 16) == 0
+    assert pk.flash_parts(200_000, 1024) == 196 and pk.cuda_prompt(128, 128, None, "bf16", "cuda") is False
+    with pk.owner("a"):
+        pass
+    pk.release("a")
