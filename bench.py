@@ -205,6 +205,95 @@ def append_sweep(pk, device, kind):
     return found
 
 
+def long_context(pk, device):
+    """Split-K partitioned decode over long contexts (40 query heads, 8 KV heads, bf16, random page placement in a
+    200k-token pool): contiguous splits of `chunk` positions, then the log-sum-exp merge. One layer, one token a row."""
+    hq, hkv, d, page, found = 40, 8, 128, 16, {}
+    pool_tokens = 200_000 * 4 + 64
+    n_pages = pool_tokens // page
+    g = torch.Generator(device=device).manual_seed(3)
+    k = torch.randn(n_pages + 1, page, hkv, d, device=device, dtype=torch.bfloat16, generator=g)
+    v = torch.randn(n_pages + 1, page, hkv, d, device=device, dtype=torch.bfloat16, generator=g)
+    for batch in (1, 4):
+        for ctx in (32_768, 131_072, 200_000):
+            width = (ctx + page - 1) // page
+            perm = torch.randperm(n_pages, device=device, generator=g)[:batch * width].view(batch, width).to(torch.int32)
+            tables = torch.full((batch, (width + 15) // 16 * 16), n_pages, dtype=torch.int32, device=device)
+            tables[:, :width] = perm
+            q = torch.randn(batch, hq, d, device=device, generator=g).to(torch.bfloat16)
+            rows = torch.arange(batch, dtype=torch.int32, device=device)
+            firsts = torch.full((batch,), ctx - 1, dtype=torch.int64, device=device)
+            out = torch.empty(batch, hq, d, dtype=torch.bfloat16, device=device)
+            nbytes = batch * ctx * hkv * 2 * d * 2
+            for chunk in (512, 1024, 2048):
+                parts = pk.flash_parts(tables.shape[1] * page, chunk)
+                ws = torch.empty(pk.workspace_floats(batch, hq, parts, d), dtype=torch.float32, device=device)
+                call = lambda phases=0: pk.attend(q, k, v, "bf16", tables, rows, rows, firsts, 1, page, flash=True,
+                                                  chunk=chunk, out=out, workspace=ws, phases=phases)
+                total = timed(call, 10, 2)
+                split = timed(lambda: call(1), 10, 2)
+                found[f"B{batch}_ctx{ctx}_chunk{chunk}"] = {
+                    "us": round(total * 1e3, 1), "split_us": round(split * 1e3, 1), "merge_us": round((total - split) * 1e3, 1),
+                    "GB/s": round(nbytes / total / 1e6, 1), "split_GB/s": round(nbytes / split / 1e6, 1)}
+    return found
+
+
+def mixed_prefill(pk, device):
+    """Chunked prefill over paged KV mixed with decode in one batch (32 query heads, 8 KV heads, bf16): 8 chunks of 512
+    new tokens on seeded prefixes in [0, 8192] plus 56 decode rows; one layer: append of all 4,152 tokens, one
+    prefill launch for the 8 chunks, one decode launch for the 56 rows."""
+    hq, hkv, d, page = 32, 8, 128, 16
+    gcpu = torch.Generator().manual_seed(5)
+    prefixes = torch.randint(0, 8193, (8,), generator=gcpu).tolist()
+    ctxs = torch.randint(1024, 8193, (56,), generator=gcpu).tolist()
+    lengths = [p + 512 for p in prefixes] + [c + 1 for c in ctxs]
+    widths = [(n + page - 1) // page for n in lengths]
+    n_pages = int(sum(widths) * 1.25)
+    g = torch.Generator(device=device).manual_seed(5)
+    k = torch.randn(n_pages + 1, page, hkv, d, device=device, dtype=torch.bfloat16, generator=g)
+    v = torch.randn(n_pages + 1, page, hkv, d, device=device, dtype=torch.bfloat16, generator=g)
+    perm = torch.randperm(n_pages, generator=gcpu)
+    tables = torch.full((64, (max(widths) + 15) // 16 * 16), n_pages, dtype=torch.int32)
+    at = 0
+    for s, w in enumerate(widths):
+        tables[s, :w] = perm[at:at + w].to(torch.int32)
+        at += w
+    T = 8 * 512 + 56
+    slots = []
+    for s in range(8):
+        pos = torch.arange(prefixes[s], prefixes[s] + 512)
+        slots.append(tables[s][pos // page].long() * page + pos % page)
+    for i, c in enumerate(ctxs):
+        slots.append(tables[8 + i][c // page].long().view(1) * page + c % page)
+    slots = torch.cat(slots).to(device)
+    tables = tables.to(device)
+    q = torch.randn(T, hq, d, device=device, generator=g).to(torch.bfloat16)
+    nk = torch.randn(T, hkv, d, device=device, generator=g).to(torch.bfloat16)
+    nv = torch.randn(T, hkv, d, device=device, generator=g).to(torch.bfloat16)
+    out = torch.empty(T, hq, d, dtype=torch.bfloat16, device=device)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=device)
+    chunk_rows, chunk_starts, chunk_counts = i32(list(range(8))), i32([512 * s for s in range(8)]), i32([512] * 8)
+    positions = torch.tensor(prefixes, dtype=torch.int64, device=device)
+    d_rows, d_starts = i32(list(range(8, 64))), i32([4096 + i for i in range(56)])
+    d_firsts = torch.tensor(ctxs, dtype=torch.int64, device=device)
+    parts, piece = pk.partitions(device, hkv, "bf16", d, d), pk.piece_size(d, d, "bf16", hkv)
+    ws = torch.empty(pk.workspace_floats(56, hq, parts, d), dtype=torch.float32, device=device)
+    append = lambda: pk.write(nk, nv, slots, k, v, "bf16")
+    prefill = lambda: pk.prefill_rows(q, k, v, "bf16", tables, chunk_rows, chunk_starts, chunk_counts, positions, 512,
+                                      page, out=out)
+    decode = lambda: pk.attend(q, k, v, "bf16", tables, d_rows, d_starts, d_firsts, 1, page, partitions=parts,
+                               piece=piece, out=out, workspace=ws)
+    flops = sum(4 * hq * d * sum(p + t + 1 for t in range(512)) for p in prefixes)
+    t_append, t_prefill, t_decode = timed(append, 20, 3), timed(prefill, 10, 2), timed(decode, 20, 3)
+    step = timed(lambda: (append(), prefill(), decode()), 10, 2)
+    return {"prefixes": prefixes, "prefill_GFLOP": round(flops / 1e9, 1), "prefill_us": round(t_prefill * 1e3, 1),
+            "prefill_TFLOP/s": round(flops / t_prefill / 1e9, 1),
+            "prefill_frac_of_bf16_mfma_peak": round(flops / t_prefill / 1e9 / 2500.0, 4),
+            "append_us": round(t_append * 1e3, 1), "append_tokens": T,
+            "append_GB/s": round(T * hkv * 2 * d * 4 / t_append / 1e6, 1),
+            "decode_us": round(t_decode * 1e3, 1), "step_us": round(step * 1e3, 1)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -288,6 +377,11 @@ def main():
         torch.cuda.empty_cache()
         extras["append_GB/s_by_tokens"] = {kind: append_sweep(pk, device, kind) for kind in ("bf16", "fp8")}
         log(f"[bench] append sweep: {extras['append_GB/s_by_tokens']}")
+        extras["long_context_splitk_bf16"] = long_context(pk, device)
+        log(f"[bench] long context: {extras['long_context_splitk_bf16']}")
+        torch.cuda.empty_cache()
+        extras["mixed_prefill_decode_bf16"] = mixed_prefill(pk, device)
+        log(f"[bench] mixed prefill + decode: {extras['mixed_prefill_decode_bf16']}")
         result["extra"] = extras
     if not args.no_cpu:
         log("[bench] timing the CPU reference path (about 20 s)")

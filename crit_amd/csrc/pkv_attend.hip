@@ -28,11 +28,27 @@ __global__ __launch_bounds__(64) void merge_kernel(AttendArgs a) {
     float M = -INFINITY, L = 0.0f, A[EPL];
 #pragma unroll
     for (int e = 0; e < EPL; ++e) A[e] = 0.0f;
-    for (int b = 0; b < nb; ++b) {
-        const Fold f = fold(M, L, a.pm[at + b], a.pl[at + b]);
+    // Folded strictly in partition order (the fused launch folds the same way), but loaded U partitions at a time so
+    // the loads of a long row's hundreds of partials overlap instead of chaining their latencies.
+    constexpr int U = 32;
+    for (int b0 = 0; b0 < nb; b0 += U) {
+        float pm[U], pl[U], po[U][EPL];
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) A[e] = __builtin_fmaf(A[e], f.keep, a.po[(at + b) * DV + e * 64 + lane] * f.take);
-        M = f.m, L = f.l;
+        for (int u = 0; u < U; ++u) {
+            const int b = b0 + u < nb ? b0 + u : nb - 1;
+            pm[u] = a.pm[at + b], pl[u] = a.pl[at + b];
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) po[u][e] = a.po[(at + b) * DV + e * 64 + lane];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (b0 + u < nb) {
+                const Fold f = fold(M, L, pm[u], pl[u]);
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) A[e] = __builtin_fmaf(A[e], f.keep, po[u][e] * f.take);
+                M = f.m, L = f.l;
+            }
+        }
     }
     if (a.sinks) {
         const Fold f = fold(M, L, a.sinks[head] * kLog2e, 1.0f);

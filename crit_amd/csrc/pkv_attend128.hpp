@@ -177,17 +177,17 @@ __global__ __launch_bounds__(256, attend_waves(KIND, QR)) void attend128_kernel(
     for (int kv = 0; kv < 4; ++kv) vvo[kv] = (uint32_t)(voff[kv] * slot_bytes) + vlane;
     const uint32_t svo = (uint32_t)(soff * a.hkv + kvh);
 
-    auto entry = [&](int base) -> int {     // the page table entry of a step (uniform over the wavefront)
+    auto entry = [&](int base) __attribute__((always_inline)) -> int {     // the page table entry of a step (uniform over the wavefront)
         int pidx = a.page_shift >= 0 ? (base >> a.page_shift) : (base / a.page);
         pidx = pidx < a.tab_width ? pidx : a.tab_width - 1;
         return a.tables[trow + pidx];
     };
     // The step's first slot (uniform): page entry * page + base's offset in its page.
-    auto first_slot = [&](int base, int e) -> int64_t {
+    auto first_slot = [&](int base, int e) __attribute__((always_inline)) -> int64_t {
         const int pidx = a.page_shift >= 0 ? (base >> a.page_shift) : (base / a.page);
         return (int64_t)__builtin_amdgcn_readfirstlane(e) * a.page + (base - pidx * a.page);
     };
-    auto fetch_k = [&](int base, int e, Step128<KIND>& buf) {
+    auto fetch_k = [&](int base, int e, Step128<KIND>& buf) __attribute__((always_inline)) {
         const int64_t slot0 = first_slot(base, e);
         const uint8_t* sbase = a.kp + slot0 * slot_bytes;
         uint32_t o[2] = {kvo[0], kvo[1]};
@@ -211,7 +211,7 @@ __global__ __launch_bounds__(256, attend_waves(KIND, QR)) void attend128_kernel(
             buf.vs = (a.vs + slot0 * a.hkv)[so];
         }
     };
-    auto fetch_v = [&](int base, int e, Step128<KIND>& buf) {
+    auto fetch_v = [&](int base, int e, Step128<KIND>& buf) __attribute__((always_inline)) {
         const uint8_t* sbase = a.vp + first_slot(base, e) * slot_bytes;
         uint32_t o[4] = {vvo[0], vvo[1], vvo[2], vvo[3]};
         if (base + SPW > n_keys) {
@@ -247,12 +247,12 @@ __global__ __launch_bounds__(256, attend_waves(KIND, QR)) void attend128_kernel(
             const int below = (wlo > 0 ? wlo : 0) / a.piece - part;
             if (below > 0) pi = part + (below + a.parts - 1) / a.parts * a.parts;
         }
-        auto base_of = [&]() -> int {
+        auto base_of = [&]() __attribute__((always_inline)) -> int {
             if (st * SPW >= a.piece) return -1;
             const int64_t base = (int64_t)pi * a.piece + st * SPW;
             return base < n_keys ? (int)base : -1;
         };
-        auto advance = [&]() -> int {
+        auto advance = [&]() __attribute__((always_inline)) -> int {
             st += 4;
             if (st * SPW >= a.piece) pi += a.parts, st = wave;
             return base_of();
@@ -392,7 +392,7 @@ __global__ __launch_bounds__(256, attend_waves(KIND, QR)) void attend128_kernel(
         int base0 = base_of();
         if (base0 >= 0) {
             const int again = base0;
-            auto safe = [&](int base) { return base >= 0 ? base : again; };
+            auto safe = [&](int base) __attribute__((always_inline)) { return base >= 0 ? base : again; };
             int e0 = entry(base0);
             int base1 = advance();
             int e1 = entry(safe(base1));

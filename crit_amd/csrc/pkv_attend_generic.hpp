@@ -144,18 +144,18 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
             const int below = (wlo > 0 ? wlo : 0) / a.piece - part;
             if (below > 0) pi = part + (below + a.parts - 1) / a.parts * a.parts;
         }
-        auto base_of = [&]() -> int {
+        auto base_of = [&]() __attribute__((always_inline)) -> int {
             if (st * SP >= a.piece) return -1;
             const int64_t base = (int64_t)pi * a.piece + st * SP;
             return base < n_keys ? (int)base : -1;
         };
-        auto advance = [&]() -> int {
+        auto advance = [&]() __attribute__((always_inline)) -> int {
             st += 4;
             if (st * SP >= a.piece) pi += a.parts, st = wave;
             return base_of();
         };
 
-        auto compute = [&](int base, const StepBuf<KIND>& buf) {
+        auto compute = [&](int base, const StepBuf<KIND>& buf) __attribute__((always_inline)) {
             float s[4][QR];
 #pragma unroll
             for (int k = 0; k < 4; ++k) {

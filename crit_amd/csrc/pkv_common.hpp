@@ -4,10 +4,17 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+#include <utility>
+
 #include "../../include/crit_pkv.h"
 
 namespace pkv {
 
+// Native vectors for values that live in register arrays: the compiler promotes arrays of these to registers, which
+// it does not always do for arrays of the runtime's uint4 / uint2 classes copied whole.
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
@@ -17,6 +24,17 @@ typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 
 #define PKV_DEV __device__ __forceinline__
+
+// A loop unrolled by template expansion: f(std::integral_constant<int, 0>{}), ..., f(<N - 1>). Register arrays indexed
+// through it are indexed by constants whatever the optimiser makes of the body.
+template <class F, int... I>
+PKV_DEV void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+PKV_DEV void static_for(F&& f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;

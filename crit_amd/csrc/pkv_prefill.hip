@@ -69,26 +69,43 @@ PKV_DEV f32x16 mfma(uint4 a, uint4 b, f32x16 c) {
     }
 }
 
+// Two probabilities as a 16-bit pair by the hardware conversions (round to nearest even).
 template <bool F16>
-PKV_DEV uint32_t pack16(float a, float b) {
+PKV_DEV uint32_t to_pair(float a, float b) {
     if constexpr (F16) return pack_f16(a, b);
-    // round to nearest even by the hardware path: the values are probabilities, never NaN unless the query is
-    return pack_bf16(a, b);
+    typedef __attribute__((ext_vector_type(2))) __bf16 pair_t;
+    pair_t r = {(__bf16)a, (__bf16)b};
+    return __builtin_bit_cast(uint32_t, r);
 }
 
+template <bool F16>
+PKV_DEV float dot2_acc(uint32_t a, uint32_t b, float c) {
+    if constexpr (F16) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
+    } else {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
+    }
+}
+
+// V^T in LDS is [dim][64 keys], rows of 128 bytes without padding; the 8-byte group of four keys g of row `row` sits
+// at group g ^ swz(row): the stores (lanes vary the dim chunk and the key group) and the operand reads (lanes vary
+// the dim and the half-wave's key group) both spread over all banks.
+PKV_DEV int swz(int row) { return (row & 15) ^ ((row >> 3) & 15); }
+
 template <int KIND, bool F16, int D>
-__global__ __launch_bounds__(256) void prefill_kernel(PrefillArgs a) {
+__global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
     constexpr int KS = D / 16;          // k-steps of the first product
     constexpr int NB = D / 32;          // 32-wide output blocks of the second product
     constexpr int KSTR = D + 8;         // K row stride in LDS (16-bit elements): 16 bytes of padding
-    constexpr int VSTR = BN + 4;        // V^T row stride in LDS: 8 bytes of padding
     constexpr int EB = KIND == 0 ? 2 : 1;
     constexpr int CH = D * EB / 16;     // 16-byte chunks of one K or V row in the pages
     constexpr int KPASS = BN * CH / 256;   // passes of 256 threads over a K block, rows contiguous over lanes
-    constexpr int VPASS = CH / 4;          // passes over a V block: lane = key, wavefront = chunk
-    __shared__ __align__(16) uint16_t k_lds[BN * KSTR];
-    __shared__ __align__(16) uint16_t v_lds[D * VSTR];
-    __shared__ float ks_lds[BN], vs_lds[BN];
+    constexpr int VGROUPS = 16 * CH;    // 16-bit pages: (group of four keys, 16-byte chunk) pairs of a V block
+    constexpr int VGP = (VGROUPS + 255) / 256;
+    constexpr int VPASS = KIND == 0 ? 4 * VGP : CH / 4;
+    __shared__ __align__(16) uint16_t k_lds[2][BN * KSTR];
+    __shared__ __align__(16) uint16_t v_lds[2][D * BN];
+    __shared__ float ks_lds[2][BN], vs_lds[2][BN];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n32 = lane & 31, h = lane >> 5;
     const int tile = gridDim.x - 1 - blockIdx.x;      // later tiles see more keys: start them first
@@ -115,6 +132,10 @@ __global__ __launch_bounds__(256) void prefill_kernel(PrefillArgs a) {
             qreg[ks] = *reinterpret_cast<const uint4*>(a.q + ((int64_t)(start + t) * a.q_st + (int64_t)head * a.q_sh + 16 * ks + 8 * h) * 2);
         }
     }
+    // The lowest limit among the wavefront's live rows: key blocks wholly at or below it need no mask.
+    int wave_lo = live ? lim : 0x7fffffff;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) wave_lo = min(wave_lo, __shfl_xor(wave_lo, o));
     float k_mult = a.k_mult, v_mult = a.v_mult;
     if (KIND == 1 && a.hm) k_mult = a.hm[kvh], v_mult = a.hm[a.hkv + kvh];
     const float sscale = a.sscale * (KIND == 1 ? k_mult : 1.0f);
@@ -128,7 +149,7 @@ __global__ __launch_bounds__(256) void prefill_kernel(PrefillArgs a) {
     int kt_lo = 0;
     if (win > 0) kt_lo = max(0, pos + t_lo - win + 1) / BN;
 
-    auto slot_of = [&](int n) -> int64_t {
+    auto slot_of = [&](int n) __attribute__((always_inline)) -> int64_t {
         n = n < n_max ? n : n_max;
         int pidx = a.page_shift >= 0 ? (n >> a.page_shift) : (n / a.page);
         const int in_page = n - pidx * a.page;
@@ -140,20 +161,34 @@ __global__ __launch_bounds__(256) void prefill_kernel(PrefillArgs a) {
     const uint8_t* kbase = a.kp + (int64_t)kvh * D * EB;
     const uint8_t* vbase = a.vp + (int64_t)kvh * D * EB;
 
-    uint4 kreg[KPASS], vreg[VPASS];
+    // Global -> registers -> LDS. K: rows contiguous over lanes. V, 16-bit pages: a thread takes one 16-byte chunk of
+    // four adjacent keys and stores it transposed as eight 8-byte groups; 8-bit pages: lane = key, wavefront = chunk.
+    u32x4 kreg[KPASS], vreg[VPASS];
     float ksreg = 1.0f, vsreg = 1.0f;
-    auto load_block = [&](int kt) {
+    auto load_block = [&](int kt) __attribute__((always_inline)) {
         const int n0 = kt * BN;
-#pragma unroll
-        for (int p = 0; p < KPASS; ++p) {
+        static_for<KPASS>([&](auto pc) __attribute__((always_inline)) {
+            constexpr int p = decltype(pc)::value;
             const int idx = p * 256 + tid;
             const int kk = idx / CH, c = idx % CH;
-            kreg[p] = *reinterpret_cast<const uint4*>(kbase + slot_of(n0 + kk) * slot_bytes + c * 16);
-        }
-        const int64_t vslot = slot_of(n0 + lane);
-#pragma unroll
-        for (int p = 0; p < VPASS; ++p) {
-            vreg[p] = *reinterpret_cast<const uint4*>(vbase + vslot * slot_bytes + (4 * p + wave) * 16);
+            kreg[p] = *reinterpret_cast<const u32x4*>(kbase + slot_of(n0 + kk) * slot_bytes + c * 16);
+        });
+        if constexpr (KIND == 0) {
+            static_for<VGP>([&](auto pc) __attribute__((always_inline)) {
+                constexpr int p = decltype(pc)::value;
+                const int idx = (p * 256 + tid) % VGROUPS;      // D = 64: the upper half of the workgroup repeats the lower
+                const int kg = idx / CH, c = idx % CH;
+                static_for<4>([&](auto jc) __attribute__((always_inline)) {
+                    constexpr int jj = decltype(jc)::value;
+                    vreg[4 * p + jj] = *reinterpret_cast<const u32x4*>(vbase + slot_of(n0 + 4 * kg + jj) * slot_bytes + c * 16);
+                });
+            });
+        } else {
+            const int64_t vslot = slot_of(n0 + lane);
+            static_for<VPASS>([&](auto pc) __attribute__((always_inline)) {
+                constexpr int p = decltype(pc)::value;
+                vreg[p] = *reinterpret_cast<const u32x4*>(vbase + vslot * slot_bytes + (4 * p + wave) * 16);
+            });
         }
         if constexpr (KIND >= 2) {
             if (tid < BN) {
@@ -162,40 +197,56 @@ __global__ __launch_bounds__(256) void prefill_kernel(PrefillArgs a) {
             }
         }
     };
-    auto store_block = [&]() {
-#pragma unroll
-        for (int p = 0; p < KPASS; ++p) {
+    auto store_block = [&](int buf) __attribute__((always_inline)) {
+        uint16_t* kl = k_lds[buf];
+        uint16_t* vl = v_lds[buf];
+        static_for<KPASS>([&](auto pc) __attribute__((always_inline)) {
+            constexpr int p = decltype(pc)::value;
             const int idx = p * 256 + tid;
             const int kk = idx / CH, c = idx % CH;
             if constexpr (KIND == 0) {
-                *reinterpret_cast<uint4*>(&k_lds[kk * KSTR + c * 8]) = kreg[p];
+                *reinterpret_cast<u32x4*>(&kl[kk * KSTR + c * 8]) = kreg[p];
             } else {
-                *reinterpret_cast<uint4*>(&k_lds[kk * KSTR + c * 16]) = codes_to_bf16<KIND>(kreg[p].x, kreg[p].y);
-                *reinterpret_cast<uint4*>(&k_lds[kk * KSTR + c * 16 + 8]) = codes_to_bf16<KIND>(kreg[p].z, kreg[p].w);
+                *reinterpret_cast<uint4*>(&kl[kk * KSTR + c * 16]) = codes_to_bf16<KIND>(kreg[p].x, kreg[p].y);
+                *reinterpret_cast<uint4*>(&kl[kk * KSTR + c * 16 + 8]) = codes_to_bf16<KIND>(kreg[p].z, kreg[p].w);
             }
-        }
+        });
+        if constexpr (KIND == 0) {
+            static_for<VGP>([&](auto pc) __attribute__((always_inline)) {
+                constexpr int p = decltype(pc)::value;
+                const int idx = (p * 256 + tid) % VGROUPS;      // repeated groups store the same bytes twice
+                const int kg = idx / CH, c = idx % CH;
+                const uint32_t w0[4] = {vreg[4 * p].x, vreg[4 * p].y, vreg[4 * p].z, vreg[4 * p].w};
+                const uint32_t w1[4] = {vreg[4 * p + 1].x, vreg[4 * p + 1].y, vreg[4 * p + 1].z, vreg[4 * p + 1].w};
+                const uint32_t w2[4] = {vreg[4 * p + 2].x, vreg[4 * p + 2].y, vreg[4 * p + 2].z, vreg[4 * p + 2].w};
+                const uint32_t w3[4] = {vreg[4 * p + 3].x, vreg[4 * p + 3].y, vreg[4 * p + 3].z, vreg[4 * p + 3].w};
 #pragma unroll
-        for (int p = 0; p < VPASS; ++p) {
-            const int c = 4 * p + wave;
-            if constexpr (KIND == 0) {
-                const uint32_t w[4] = {vreg[p].x, vreg[p].y, vreg[p].z, vreg[p].w};
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    v_lds[(c * 8 + 2 * i) * VSTR + lane] = (uint16_t)(w[i] & 0xffffu);
-                    v_lds[(c * 8 + 2 * i + 1) * VSTR + lane] = (uint16_t)(w[i] >> 16);
+                for (int i = 0; i < 8; ++i) {
+                    const int row = c * 8 + i;
+                    const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
+                    const uint32_t k01 = __builtin_amdgcn_perm(w1[i / 2], w0[i / 2], sel);
+                    const uint32_t k23 = __builtin_amdgcn_perm(w3[i / 2], w2[i / 2], sel);
+                    *reinterpret_cast<uint2*>(&vl[row * BN + 4 * (kg ^ swz(row))]) = make_uint2(k01, k23);
                 }
-            } else {
+            });
+        } else {
+            static_for<VPASS>([&](auto pc) __attribute__((always_inline)) {
+                constexpr int p = decltype(pc)::value;
+                const int c = 4 * p + wave;
                 const uint4 lo = codes_to_bf16<KIND>(vreg[p].x, vreg[p].y), hi = codes_to_bf16<KIND>(vreg[p].z, vreg[p].w);
                 const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    v_lds[(c * 16 + 2 * i) * VSTR + lane] = (uint16_t)(w[i] & 0xffffu);
-                    v_lds[(c * 16 + 2 * i + 1) * VSTR + lane] = (uint16_t)(w[i] >> 16);
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+                        const int row = c * 16 + 2 * i + half;
+                        vl[row * BN + 4 * ((lane >> 2) ^ swz(row)) + (lane & 3)] = (uint16_t)(half ? w[i] >> 16 : w[i] & 0xffffu);
+                    }
                 }
-            }
+            });
         }
         if constexpr (KIND >= 2) {
-            if (tid < BN) ks_lds[tid] = ksreg, vs_lds[tid] = vsreg;
+            if (tid < BN) ks_lds[buf][tid] = ksreg, vs_lds[buf][tid] = vsreg;
         }
     };
 
@@ -206,13 +257,16 @@ __global__ __launch_bounds__(256) void prefill_kernel(PrefillArgs a) {
         for (int v = 0; v < 16; ++v) o[nb][v] = 0.0f;
     float m = -INFINITY, l = 0.0f;
 
+    // Double-buffered LDS, one barrier a block: block kt is multiplied from buffer kt & 1 while block kt + 1 (already
+    // in registers) is stored into the other buffer and block kt + 2 is fetched from the pages.
     load_block(kt_lo);
+    store_block(kt_lo & 1);
+    if (kt_lo < kt_hi) load_block(kt_lo + 1);
+    __syncthreads();
     for (int kt = kt_lo; kt <= kt_hi; ++kt) {
-        __syncthreads();          // the previous block's products have read the LDS
-        store_block();
-        __syncthreads();
-        if (kt < kt_hi) load_block(kt + 1);     // in flight while this block is multiplied
-
+        const int buf = kt & 1;
+        const uint16_t* kl = k_lds[buf];
+        const uint16_t* vl = v_lds[buf];
         // S^T = K Q^T: two blocks of 32 keys x this wavefront's 32 rows.
         f32x16 s[2];
 #pragma unroll
@@ -221,22 +275,31 @@ __global__ __launch_bounds__(256) void prefill_kernel(PrefillArgs a) {
             for (int v = 0; v < 16; ++v) s[kb][v] = 0.0f;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const uint4 kop = *reinterpret_cast<const uint4*>(&k_lds[(32 * kb + n32) * KSTR + 16 * ks + 8 * h]);
+                const uint4 kop = *reinterpret_cast<const uint4*>(&kl[(32 * kb + n32) * KSTR + 16 * ks + 8 * h]);
                 s[kb] = mfma<F16>(kop, qreg[ks], s[kb]);
             }
         }
-        // Scale and mask; the lane holds keys 32 kb + 8 (v / 4) + 4 h + v % 4 of its own row.
+        // The next block goes into the other buffer while this one is multiplied (its readers passed the barrier).
+        if (kt < kt_hi) {
+            store_block(buf ^ 1);
+            if (kt + 1 < kt_hi) load_block(kt + 2);
+        }
+        // Scale (and mask where the block is not wholly visible); the lane holds keys 32 kb + 8 (v / 4) + 4 h + v % 4
+        // of its own row.
+        const bool masked = win > 0 || kt * BN + BN - 1 > wave_lo;
         float top = -INFINITY;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int kin = 32 * kb + 8 * (v / 4) + 4 * h + v % 4;
-                const int n = kt * BN + kin;
-                float x = s[kb][v] * (KIND >= 2 ? sscale * ks_lds[kin] : sscale);
-                bool vis = n <= lim;
-                if (win > 0) vis = vis && n > lim - win;
-                x = vis ? x : -INFINITY;
+                float x = s[kb][v] * (KIND >= 2 ? sscale * ks_lds[buf][kin] : sscale);
+                if (masked) {
+                    const int n = kt * BN + kin;
+                    bool vis = n <= lim;
+                    if (win > 0) vis = vis && n > lim - win;
+                    x = vis ? x : -INFINITY;
+                }
                 s[kb][v] = x;
                 top = __builtin_fmaxf(top, x);
             }
@@ -250,18 +313,19 @@ __global__ __launch_bounds__(256) void prefill_kernel(PrefillArgs a) {
         uint4 pop[2][2];      // P^T as the second product's B operand: [32-key block][half of it]
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
-            float p[16];
+            uint32_t pw[8];
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                p[v] = exp2_fast(s[kb][v] - sub);
-                sum += p[v];
-                if constexpr (KIND >= 2) p[v] *= vs_lds[32 * kb + 8 * (v / 4) + 4 * h + v % 4];
+            for (int v2 = 0; v2 < 8; ++v2) {
+                float p0 = exp2_fast(s[kb][2 * v2] - sub), p1 = exp2_fast(s[kb][2 * v2 + 1] - sub);
+                sum += p0 + p1;
+                if constexpr (KIND >= 2) {     // the values' scales ride on the operand, not on the sum
+                    p0 *= vs_lds[buf][32 * kb + 8 * ((2 * v2) / 4) + 4 * h + (2 * v2) % 4];
+                    p1 *= vs_lds[buf][32 * kb + 8 * ((2 * v2 + 1) / 4) + 4 * h + (2 * v2 + 1) % 4];
+                }
+                pw[v2] = to_pair<F16>(p0, p1);
             }
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                pop[kb][half] = make_uint4(pack16<F16>(p[8 * half], p[8 * half + 1]), pack16<F16>(p[8 * half + 2], p[8 * half + 3]),
-                                           pack16<F16>(p[8 * half + 4], p[8 * half + 5]), pack16<F16>(p[8 * half + 6], p[8 * half + 7]));
-            }
+            pop[kb][0] = make_uint4(pw[0], pw[1], pw[2], pw[3]);
+            pop[kb][1] = make_uint4(pw[4], pw[5], pw[6], pw[7]);
         }
         l = __builtin_fmaf(l, alpha, sum);
         // wave-uniform: skip the rescale when no row's maximum moved (alpha == 1 everywhere)
@@ -274,16 +338,20 @@ __global__ __launch_bounds__(256) void prefill_kernel(PrefillArgs a) {
         // O^T += V^T P^T: the lane feeds V^T[dim 32 nb + n32][keys of its half] and its own probabilities.
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
+            const int row = 32 * nb + n32;
+            const int sw = swz(row);
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {
-                    const uint16_t* row = &v_lds[(32 * nb + n32) * VSTR + 32 * kb + 16 * half + 4 * h];
-                    const uint2 lo = *reinterpret_cast<const uint2*>(row), hi = *reinterpret_cast<const uint2*>(row + 8);
+                    const int g0 = 8 * kb + 4 * half + h;
+                    const uint2 lo = *reinterpret_cast<const uint2*>(&vl[row * BN + 4 * (g0 ^ sw)]);
+                    const uint2 hi = *reinterpret_cast<const uint2*>(&vl[row * BN + 4 * ((g0 + 2) ^ sw)]);
                     o[nb] = mfma<F16>(make_uint4(lo.x, lo.y, hi.x, hi.y), pop[kb][half], o[nb]);
                 }
             }
         }
+        __syncthreads();          // every wavefront is done with this buffer; the other one is stored
     }
     // The two half-waves hold the same row's sums over different keys.
     l += __shfl_xor(l, 32);
