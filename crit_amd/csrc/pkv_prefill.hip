@@ -149,13 +149,20 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
     int kt_lo = 0;
     if (win > 0) kt_lo = max(0, pos + t_lo - win + 1) / BN;
 
-    auto slot_of = [&](int n) __attribute__((always_inline)) -> int64_t {
+    // The page table entry and the slot of a position (positions past the chunk's last written one read that one).
+    // One 4-byte load whatever the table's type: an int64 entry's low word holds the page number (little endian).
+    const uint8_t* tab_bytes = a.tables ? reinterpret_cast<const uint8_t*>(a.tables) : reinterpret_cast<const uint8_t*>(a.tables64);
+    const int tab_shift = a.tables ? 2 : 3;
+    auto entry_of = [&](int n) __attribute__((always_inline)) -> int {
         n = n < n_max ? n : n_max;
         int pidx = a.page_shift >= 0 ? (n >> a.page_shift) : (n / a.page);
-        const int in_page = n - pidx * a.page;
         pidx = pidx < a.tab_width ? pidx : a.tab_width - 1;
-        const int64_t pg = a.tables ? (int64_t)a.tables[trow + pidx] : a.tables64[trow + pidx];
-        return pg * a.page + in_page;
+        return *reinterpret_cast<const int*>(tab_bytes + ((trow + pidx) << tab_shift));
+    };
+    auto slot_at = [&](int n, int pg) __attribute__((always_inline)) -> int64_t {
+        n = n < n_max ? n : n_max;
+        const int pidx = a.page_shift >= 0 ? (n >> a.page_shift) : (n / a.page);
+        return (int64_t)pg * a.page + (n - pidx * a.page);
     };
     const int64_t slot_bytes = (int64_t)a.hkv * D * EB;
     const uint8_t* kbase = a.kp + (int64_t)kvh * D * EB;
@@ -163,38 +170,54 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
 
     // Global -> registers -> LDS. K: rows contiguous over lanes. V, 16-bit pages: a thread takes one 16-byte chunk of
     // four adjacent keys and stores it transposed as eight 8-byte groups; 8-bit pages: lane = key, wavefront = chunk.
+    // The page table entries of a block are fetched one block before its rows (load_entries, then load_block): a
+    // row's address depends on its entry, and a wait on an entry would also wait on every row load issued before it.
+    constexpr int NENT = KPASS + (KIND == 0 ? VGP * 4 : 1) + (KIND >= 2 ? 1 : 0);
     u32x4 kreg[KPASS], vreg[VPASS];
+    int ent[NENT];
     float ksreg = 1.0f, vsreg = 1.0f;
+    auto load_entries = [&](int kt) __attribute__((always_inline)) {
+        const int n0 = kt * BN;
+        static_for<KPASS>([&](auto pc) __attribute__((always_inline)) {
+            constexpr int p = decltype(pc)::value;
+            ent[p] = entry_of(n0 + (p * 256 + tid) / CH);
+        });
+        if constexpr (KIND == 0) {
+            static_for<VGP * 4>([&](auto ic) __attribute__((always_inline)) {
+                constexpr int i = decltype(ic)::value;
+                const int kg = ((i / 4) * 256 + tid) % VGROUPS / CH;
+                ent[KPASS + i] = entry_of(n0 + 4 * kg + i % 4);
+            });
+        } else {
+            ent[KPASS] = entry_of(n0 + lane);
+        }
+        if constexpr (KIND >= 2) ent[NENT - 1] = entry_of(n0 + (tid & (BN - 1)));
+    };
     auto load_block = [&](int kt) __attribute__((always_inline)) {
         const int n0 = kt * BN;
         static_for<KPASS>([&](auto pc) __attribute__((always_inline)) {
             constexpr int p = decltype(pc)::value;
             const int idx = p * 256 + tid;
             const int kk = idx / CH, c = idx % CH;
-            kreg[p] = *reinterpret_cast<const u32x4*>(kbase + slot_of(n0 + kk) * slot_bytes + c * 16);
+            kreg[p] = *reinterpret_cast<const u32x4*>(kbase + slot_at(n0 + kk, ent[p]) * slot_bytes + c * 16);
         });
         if constexpr (KIND == 0) {
-            static_for<VGP>([&](auto pc) __attribute__((always_inline)) {
-                constexpr int p = decltype(pc)::value;
-                const int idx = (p * 256 + tid) % VGROUPS;      // D = 64: the upper half of the workgroup repeats the lower
+            static_for<VGP * 4>([&](auto ic) __attribute__((always_inline)) {
+                constexpr int i = decltype(ic)::value;
+                const int idx = ((i / 4) * 256 + tid) % VGROUPS;      // D = 64: the upper half of the workgroup repeats the lower
                 const int kg = idx / CH, c = idx % CH;
-                static_for<4>([&](auto jc) __attribute__((always_inline)) {
-                    constexpr int jj = decltype(jc)::value;
-                    vreg[4 * p + jj] = *reinterpret_cast<const u32x4*>(vbase + slot_of(n0 + 4 * kg + jj) * slot_bytes + c * 16);
-                });
+                vreg[i] = *reinterpret_cast<const u32x4*>(vbase + slot_at(n0 + 4 * kg + i % 4, ent[KPASS + i]) * slot_bytes + c * 16);
             });
         } else {
-            const int64_t vslot = slot_of(n0 + lane);
+            const int64_t vslot = slot_at(n0 + lane, ent[KPASS]);
             static_for<VPASS>([&](auto pc) __attribute__((always_inline)) {
                 constexpr int p = decltype(pc)::value;
                 vreg[p] = *reinterpret_cast<const u32x4*>(vbase + vslot * slot_bytes + (4 * p + wave) * 16);
             });
         }
         if constexpr (KIND >= 2) {
-            if (tid < BN) {
-                const int64_t s = slot_of(n0 + tid);
-                ksreg = a.ks[s * a.hkv + kvh], vsreg = a.vs[s * a.hkv + kvh];
-            }
+            const int64_t s = slot_at(n0 + (tid & (BN - 1)), ent[NENT - 1]);
+            ksreg = a.ks[s * a.hkv + kvh], vsreg = a.vs[s * a.hkv + kvh];
         }
     };
     auto store_block = [&](int buf) __attribute__((always_inline)) {
@@ -258,10 +281,16 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
     float m = -INFINITY, l = 0.0f;
 
     // Double-buffered LDS, one barrier a block: block kt is multiplied from buffer kt & 1 while block kt + 1 (already
-    // in registers) is stored into the other buffer and block kt + 2 is fetched from the pages.
+    // in registers) is stored into the other buffer, block kt + 2 is fetched from the pages and the table entries of
+    // block kt + 3 are read. Every load of the loop is unconditional (past the last block it repeats the last one), so
+    // the compiler counts the outstanding loads exactly instead of waiting for all of them.
+    auto upto = [&](int kt) __attribute__((always_inline)) { return kt < kt_hi ? kt : kt_hi; };
+    load_entries(kt_lo);
     load_block(kt_lo);
+    load_entries(upto(kt_lo + 1));
     store_block(kt_lo & 1);
-    if (kt_lo < kt_hi) load_block(kt_lo + 1);
+    load_block(upto(kt_lo + 1));
+    load_entries(upto(kt_lo + 2));
     __syncthreads();
     for (int kt = kt_lo; kt <= kt_hi; ++kt) {
         const int buf = kt & 1;
@@ -280,10 +309,9 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
             }
         }
         // The next block goes into the other buffer while this one is multiplied (its readers passed the barrier).
-        if (kt < kt_hi) {
-            store_block(buf ^ 1);
-            if (kt + 1 < kt_hi) load_block(kt + 2);
-        }
+        store_block(buf ^ 1);
+        load_block(upto(kt + 2));
+        load_entries(upto(kt + 3));
         // Scale (and mask where the block is not wholly visible); the lane holds keys 32 kb + 8 (v / 4) + 4 h + v % 4
         // of its own row.
         const bool masked = win > 0 || kt * BN + BN - 1 > wave_lo;
