@@ -34,10 +34,21 @@ struct PrefillArgs {
     float* lse;
     const float* sinks;
     int64_t q_st, q_sh, o_st, o_sh, tab_stride;
-    int tab_width, chunks, max_count, hq, hkv, g, page, page_shift, sliding, out_dtype;
+    int tab_width, chunks, max_count, hq, hkv, g, page, page_l, sliding, out_dtype, tiles;
+    uint32_t page_magic;     // n / page == (mulhi(page_magic, n) + n) >> page_l for 0 <= n < 2^31
     float sscale, k_mult, v_mult;
 };
 
+#ifndef PKV_NO_PRIO
+#define PKV_PRIO(x) __builtin_amdgcn_s_setprio(x)
+#else
+#define PKV_PRIO(x)
+#endif
+#ifdef PKV_NO_SB
+#define PKV_SB()
+#else
+#define PKV_SB() __builtin_amdgcn_sched_barrier(0)
+#endif
 constexpr int BM = 128;   // query rows a workgroup holds
 constexpr int BN = 64;    // keys a block holds
 
@@ -60,6 +71,16 @@ PKV_DEV uint4 codes_to_bf16(uint32_t w0, uint32_t w1) {
     return r;
 }
 
+template <bool F16>
+PKV_DEV f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
+    if constexpr (F16) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+}
+template <bool F16>
+PKV_DEV f32x16 mfma(u32x4 a, uint4 b, f32x16 c) { return mfma<F16>(a, u32x4{b.x, b.y, b.z, b.w}, c); }
 template <bool F16>
 PKV_DEV f32x16 mfma(uint4 a, uint4 b, f32x16 c) {
     if constexpr (F16) {
@@ -88,9 +109,10 @@ PKV_DEV float dot2_acc(uint32_t a, uint32_t b, float c) {
 }
 
 // V^T in LDS is [dim][64 keys], rows of 128 bytes without padding; the 8-byte group of four keys g of row `row` sits
-// at group g ^ swz(row): the stores (lanes vary the dim chunk and the key group) and the operand reads (lanes vary
-// the dim and the half-wave's key group) both spread over all banks.
-PKV_DEV int swz(int row) { return (row & 15) ^ ((row >> 3) & 15); }
+// at group g ^ swz(row). The stores (16 lanes: 16 dim chunks of 8 rows, one row of each) and the operand reads (16
+// lanes: 16 adjacent rows) both spread over all banks, and the swizzle is a XOR of bit fields, so an address is one
+// per-thread value XOR a compile-time constant plus a compile-time offset.
+PKV_DEV int swz(int row) { return ((row >> 3) & 15) ^ ((row & 7) << 1); }
 
 template <int KIND, bool F16, int D>
 __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
@@ -108,8 +130,14 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
     __shared__ float ks_lds[2][BN], vs_lds[2][BN];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n32 = lane & 31, h = lane >> 5;
-    const int tile = gridDim.x - 1 - blockIdx.x;      // later tiles see more keys: start them first
-    const int kvh = blockIdx.y, z = blockIdx.z;
+    // Workgroups go to the 8 XCDs round robin by linear id, and each XCD has its own L2: all tiles of one (chunk, KV
+    // head) read the same keys, so they take ids of one residue mod 8 and share that XCD's L2. Later tiles see more
+    // keys: they start first.
+    const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
+    const int group = xcd + 8 * (q / a.tiles);
+    if (group >= a.hkv * a.chunks) return;
+    const int tile = a.tiles - 1 - q % a.tiles;
+    const int kvh = group % a.hkv, z = group / a.hkv;
     int count = a.max_count;
     if (a.counts) count = min(a.counts[z], a.max_count);
     if ((int64_t)tile * BM >= (int64_t)count * a.g) return;
@@ -132,15 +160,23 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
             qreg[ks] = *reinterpret_cast<const uint4*>(a.q + ((int64_t)(start + t) * a.q_st + (int64_t)head * a.q_sh + 16 * ks + 8 * h) * 2);
         }
     }
+    if (a.sscale < 0.0f && KIND < 2) {      // a negative scale: its sign goes into the queries, |scale| into the exponent
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            qreg[ks].x ^= 0x80008000u, qreg[ks].y ^= 0x80008000u, qreg[ks].z ^= 0x80008000u, qreg[ks].w ^= 0x80008000u;
+        }
+    }
     // The lowest limit among the wavefront's live rows: key blocks wholly at or below it need no mask.
     int wave_lo = live ? lim : 0x7fffffff;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) wave_lo = min(wave_lo, __shfl_xor(wave_lo, o));
+    wave_lo = __builtin_amdgcn_readfirstlane(wave_lo);
     float k_mult = a.k_mult, v_mult = a.v_mult;
     if (KIND == 1 && a.hm) k_mult = a.hm[kvh], v_mult = a.hm[a.hkv + kvh];
     const float sscale = a.sscale * (KIND == 1 ? k_mult : 1.0f);
     if (KIND != 1) v_mult = 1.0f;
     const int win = a.sliding;
+    const float sabs = __builtin_fabsf(sscale);
 
     const int t_lo = tile * BM / a.g;
     const int t_hi = min(count - 1, (tile * BM + BM - 1) / a.g);
@@ -149,80 +185,78 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
     int kt_lo = 0;
     if (win > 0) kt_lo = max(0, pos + t_lo - win + 1) / BN;
 
-    // The page table entry and the slot of a position (positions past the chunk's last written one read that one).
-    // One 4-byte load whatever the table's type: an int64 entry's low word holds the page number (little endian).
-    const uint8_t* tab_bytes = a.tables ? reinterpret_cast<const uint8_t*>(a.tables) : reinterpret_cast<const uint8_t*>(a.tables64);
+    // A block's 64 keys map onto the 64 lanes: lane i looks up the page table entry and the slot of position 64 kt + i
+    // (positions past the chunk's last written one read that one), every wavefront for itself, and a thread then takes
+    // the slots of the rows it loads from the lanes that hold them (ds_bpermute). One 4-byte table load whatever the
+    // table's type: an int64 entry's low word holds the page number (little endian). Slots fit 32 unsigned bits: a
+    // row is at least 64 bytes and a pool at most the card's memory.
+    const uint8_t* tab_row = (a.tables ? reinterpret_cast<const uint8_t*>(a.tables) : reinterpret_cast<const uint8_t*>(a.tables64)) +
+                             (trow << (a.tables ? 2 : 3));
     const int tab_shift = a.tables ? 2 : 3;
-    auto entry_of = [&](int n) __attribute__((always_inline)) -> int {
-        n = n < n_max ? n : n_max;
-        int pidx = a.page_shift >= 0 ? (n >> a.page_shift) : (n / a.page);
-        pidx = pidx < a.tab_width ? pidx : a.tab_width - 1;
-        return *reinterpret_cast<const int*>(tab_bytes + ((trow + pidx) << tab_shift));
-    };
-    auto slot_at = [&](int n, int pg) __attribute__((always_inline)) -> int64_t {
-        n = n < n_max ? n : n_max;
-        const int pidx = a.page_shift >= 0 ? (n >> a.page_shift) : (n / a.page);
-        return (int64_t)pg * a.page + (n - pidx * a.page);
-    };
-    const int64_t slot_bytes = (int64_t)a.hkv * D * EB;
+    const uint32_t slot_bytes = (uint32_t)a.hkv * D * EB;
     const uint8_t* kbase = a.kp + (int64_t)kvh * D * EB;
     const uint8_t* vbase = a.vp + (int64_t)kvh * D * EB;
-
     // Global -> registers -> LDS. K: rows contiguous over lanes. V, 16-bit pages: a thread takes one 16-byte chunk of
     // four adjacent keys and stores it transposed as eight 8-byte groups; 8-bit pages: lane = key, wavefront = chunk.
-    // The page table entries of a block are fetched one block before its rows (load_entries, then load_block): a
+    // The page table entries of a block are fetched one block before its rows (load_entries, then take_slots, then load_k and load_v): a
     // row's address depends on its entry, and a wait on an entry would also wait on every row load issued before it.
-    constexpr int NENT = KPASS + (KIND == 0 ? VGP * 4 : 1) + (KIND >= 2 ? 1 : 0);
     u32x4 kreg[KPASS], vreg[VPASS];
-    int ent[NENT];
+    int ent = 0, inp = 0;
     float ksreg = 1.0f, vsreg = 1.0f;
     auto load_entries = [&](int kt) __attribute__((always_inline)) {
-        const int n0 = kt * BN;
-        static_for<KPASS>([&](auto pc) __attribute__((always_inline)) {
-            constexpr int p = decltype(pc)::value;
-            ent[p] = entry_of(n0 + (p * 256 + tid) / CH);
-        });
-        if constexpr (KIND == 0) {
-            static_for<VGP * 4>([&](auto ic) __attribute__((always_inline)) {
-                constexpr int i = decltype(ic)::value;
-                const int kg = ((i / 4) * 256 + tid) % VGROUPS / CH;
-                ent[KPASS + i] = entry_of(n0 + 4 * kg + i % 4);
-            });
-        } else {
-            ent[KPASS] = entry_of(n0 + lane);
-        }
-        if constexpr (KIND >= 2) ent[NENT - 1] = entry_of(n0 + (tid & (BN - 1)));
+        int n = kt * BN + lane;
+        n = n < n_max ? n : n_max;
+        uint32_t pidx = (__umulhi(a.page_magic, (uint32_t)n) + (uint32_t)n) >> a.page_l;
+        inp = n - (int)pidx * a.page;
+        pidx = pidx < (uint32_t)a.tab_width ? pidx : (uint32_t)a.tab_width - 1u;
+        ent = *reinterpret_cast<const int*>(tab_row + (pidx << tab_shift));
     };
-    auto load_block = [&](int kt) __attribute__((always_inline)) {
-        const int n0 = kt * BN;
+    // take_slots turns the entries into slots and hands every thread the slots of its rows; it runs during the second
+    // product of the iteration before the loads that use them, so the exchange's latency passes behind the products
+    // and load_k / load_v issue their row loads back to back.
+    constexpr int NROW = KPASS + (KIND == 0 ? 4 : 0);
+    uint32_t rowslot[NROW], myslot = 0;
+    auto take_slots = [&]() __attribute__((always_inline)) {
+        myslot = (uint32_t)ent * (uint32_t)a.page + (uint32_t)inp;
         static_for<KPASS>([&](auto pc) __attribute__((always_inline)) {
             constexpr int p = decltype(pc)::value;
-            const int idx = p * 256 + tid;
-            const int kk = idx / CH, c = idx % CH;
-            kreg[p] = *reinterpret_cast<const u32x4*>(kbase + slot_at(n0 + kk, ent[p]) * slot_bytes + c * 16);
+            rowslot[p] = (uint32_t)__builtin_amdgcn_ds_bpermute(((p * 256 + tid) / CH) << 2, (int)myslot);
         });
         if constexpr (KIND == 0) {
-            static_for<VGP * 4>([&](auto ic) __attribute__((always_inline)) {
+            const int kg = tid % VGROUPS / CH;      // D = 64: the upper half of the workgroup repeats the lower
+            static_for<4>([&](auto ic) __attribute__((always_inline)) {
                 constexpr int i = decltype(ic)::value;
-                const int idx = ((i / 4) * 256 + tid) % VGROUPS;      // D = 64: the upper half of the workgroup repeats the lower
-                const int kg = idx / CH, c = idx % CH;
-                vreg[i] = *reinterpret_cast<const u32x4*>(vbase + slot_at(n0 + 4 * kg + i % 4, ent[KPASS + i]) * slot_bytes + c * 16);
+                rowslot[KPASS + i] = (uint32_t)__builtin_amdgcn_ds_bpermute((4 * kg + i) << 2, (int)myslot);
+            });
+        }
+    };
+    auto load_k = [&]() __attribute__((always_inline)) {
+        const uint8_t* kthread = kbase + (tid % CH) * 16;
+        static_for<KPASS>([&](auto pc) __attribute__((always_inline)) {
+            constexpr int p = decltype(pc)::value;
+            kreg[p] = *reinterpret_cast<const u32x4*>(kthread + (uint64_t)rowslot[p] * slot_bytes);
+        });
+        if constexpr (KIND >= 2) {
+            ksreg = a.ks[(uint64_t)myslot * a.hkv + kvh], vsreg = a.vs[(uint64_t)myslot * a.hkv + kvh];
+        }
+    };
+    auto load_v = [&]() __attribute__((always_inline)) {
+        if constexpr (KIND == 0) {
+            const uint8_t* vthread = vbase + (tid % VGROUPS % CH) * 16;
+            static_for<4>([&](auto ic) __attribute__((always_inline)) {
+                constexpr int i = decltype(ic)::value;
+                vreg[i] = *reinterpret_cast<const u32x4*>(vthread + (uint64_t)rowslot[KPASS + i] * slot_bytes);
             });
         } else {
-            const int64_t vslot = slot_at(n0 + lane, ent[KPASS]);
+            const uint8_t* vrow = vbase + (uint64_t)myslot * slot_bytes;
             static_for<VPASS>([&](auto pc) __attribute__((always_inline)) {
                 constexpr int p = decltype(pc)::value;
-                vreg[p] = *reinterpret_cast<const u32x4*>(vbase + vslot * slot_bytes + (4 * p + wave) * 16);
+                vreg[p] = *reinterpret_cast<const u32x4*>(vrow + (4 * p + wave) * 16);
             });
         }
-        if constexpr (KIND >= 2) {
-            const int64_t s = slot_at(n0 + (tid & (BN - 1)), ent[NENT - 1]);
-            ksreg = a.ks[s * a.hkv + kvh], vsreg = a.vs[s * a.hkv + kvh];
-        }
     };
-    auto store_block = [&](int buf) __attribute__((always_inline)) {
+    auto store_k = [&](int buf) __attribute__((always_inline)) {
         uint16_t* kl = k_lds[buf];
-        uint16_t* vl = v_lds[buf];
         static_for<KPASS>([&](auto pc) __attribute__((always_inline)) {
             constexpr int p = decltype(pc)::value;
             const int idx = p * 256 + tid;
@@ -234,6 +268,12 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
                 *reinterpret_cast<uint4*>(&kl[kk * KSTR + c * 16 + 8]) = codes_to_bf16<KIND>(kreg[p].z, kreg[p].w);
             }
         });
+        if constexpr (KIND >= 2) {
+            if (tid < BN) ks_lds[buf][tid] = ksreg, vs_lds[buf][tid] = vsreg;
+        }
+    };
+    auto store_v = [&](int buf) __attribute__((always_inline)) {
+        uint16_t* vl = v_lds[buf];
         if constexpr (KIND == 0) {
             static_for<VGP>([&](auto pc) __attribute__((always_inline)) {
                 constexpr int p = decltype(pc)::value;
@@ -243,13 +283,15 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
                 const uint32_t w1[4] = {vreg[4 * p + 1].x, vreg[4 * p + 1].y, vreg[4 * p + 1].z, vreg[4 * p + 1].w};
                 const uint32_t w2[4] = {vreg[4 * p + 2].x, vreg[4 * p + 2].y, vreg[4 * p + 2].z, vreg[4 * p + 2].w};
                 const uint32_t w3[4] = {vreg[4 * p + 3].x, vreg[4 * p + 3].y, vreg[4 * p + 3].z, vreg[4 * p + 3].w};
+                // row 8 c + i, group kg ^ swz(row): byte offset (1024 c + 8 (kg ^ c)) ^ (16 i), plus 128 i
+                uint8_t* vb = reinterpret_cast<uint8_t*>(vl);
+                const uint32_t v_write = 1024u * (uint32_t)c + 8u * (uint32_t)(kg ^ c);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    const int row = c * 8 + i;
                     const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
                     const uint32_t k01 = __builtin_amdgcn_perm(w1[i / 2], w0[i / 2], sel);
                     const uint32_t k23 = __builtin_amdgcn_perm(w3[i / 2], w2[i / 2], sel);
-                    *reinterpret_cast<uint2*>(&vl[row * BN + 4 * (kg ^ swz(row))]) = make_uint2(k01, k23);
+                    *reinterpret_cast<u32x2*>(vb + (v_write ^ (16u * i)) + 128 * i) = u32x2{k01, k23};
                 }
             });
         } else {
@@ -268,8 +310,28 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
                 }
             });
         }
-        if constexpr (KIND >= 2) {
-            if (tid < BN) ks_lds[buf][tid] = ksreg, vs_lds[buf][tid] = vsreg;
+    };
+    // Operand reads, two operands a step. K, step i: k-step i of both 32-key halves. V, step i: keys
+    // 16 (i / (NB / 2)) .. + 15 of the 32-dim blocks 2 (i % (NB / 2)) and the next one.
+    auto read_k = [&](const uint16_t* kl, auto ic, u32x4 (&dst)[2]) __attribute__((always_inline)) {
+        constexpr int i = decltype(ic)::value;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+            dst[kb] = *reinterpret_cast<const u32x4*>(&kl[(32 * kb + n32) * KSTR + 16 * i + 8 * h]);
+    };
+    // Byte offset of the lane's V^T operand inside a buffer: row (32 nb + n32), group (4 g + 2 j + h) ^ swz(row)
+    //   = v_read ^ (8 * ((4 g + 2 j) ^ (4 nb))) + 4096 nb.
+    const uint32_t v_read = (uint32_t)n32 * (BN * 2) + 8u * (uint32_t)(h ^ (n32 >> 3) ^ ((n32 & 7) << 1));
+    auto read_v = [&](const uint16_t* vl, auto ic, u32x4 (&dst)[2]) __attribute__((always_inline)) {
+        constexpr int i = decltype(ic)::value;
+        constexpr int g = i / (NB / 2);      // keys 16 g .. 16 g + 15: 32-key half g / 2, half of it g % 2
+        const uint8_t* vb = reinterpret_cast<const uint8_t*>(vl);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int nb = 2 * (i % (NB / 2)) + j;
+            const u32x2 lo = *reinterpret_cast<const u32x2*>(vb + (v_read ^ (8u * ((4 * g) ^ (4 * nb & 15)))) + 32 * BN * 2 * nb);
+            const u32x2 hi = *reinterpret_cast<const u32x2*>(vb + (v_read ^ (8u * ((4 * g + 2) ^ (4 * nb & 15)))) + 32 * BN * 2 * nb);
+            dst[j] = u32x4{lo.x, lo.y, hi.x, hi.y};
         }
     };
 
@@ -281,105 +343,158 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
     float m = -INFINITY, l = 0.0f;
 
     // Double-buffered LDS, one barrier a block: block kt is multiplied from buffer kt & 1 while block kt + 1 (already
-    // in registers) is stored into the other buffer, block kt + 2 is fetched from the pages and the table entries of
-    // block kt + 3 are read. Every load of the loop is unconditional (past the last block it repeats the last one), so
+    // in registers) is stored into the other buffer and its registers are at once reloaded with block kt + 2 (a whole
+    // iteration before they are stored); the slots of block kt + 3 and the table entries of block kt + 4 follow
+    // during the second product. Every load of the loop is unconditional (past the last block it repeats the last one), so
     // the compiler counts the outstanding loads exactly instead of waiting for all of them.
     auto upto = [&](int kt) __attribute__((always_inline)) { return kt < kt_hi ? kt : kt_hi; };
     load_entries(kt_lo);
-    load_block(kt_lo);
+    take_slots();
+    load_k();
+    load_v();
     load_entries(upto(kt_lo + 1));
-    store_block(kt_lo & 1);
-    load_block(upto(kt_lo + 1));
+    store_k(kt_lo & 1);
+    store_v(kt_lo & 1);
+    take_slots();
+    load_k();
+    load_v();
     load_entries(upto(kt_lo + 2));
+    take_slots();
+    load_entries(upto(kt_lo + 3));
     __syncthreads();
-    for (int kt = kt_lo; kt <= kt_hi; ++kt) {
+    // One key block; MASK: 0 = every key is visible to every row of the workgroup, 1 = causal limit and sliding window.
+    auto block = [&](int kt, auto mask_c) __attribute__((always_inline)) {
+        constexpr int MASK = decltype(mask_c)::value;
         const int buf = kt & 1;
         const uint16_t* kl = k_lds[buf];
         const uint16_t* vl = v_lds[buf];
-        // S^T = K Q^T: two blocks of 32 keys x this wavefront's 32 rows.
+        // S^T = K Q^T: two blocks of 32 keys x this wavefront's 32 rows. The operands of a group of four products are
+        // read while the group before is multiplied, and the next block goes into the other LDS buffer (its readers
+        // passed the barrier) in the shadow of the products.
         f32x16 s[2];
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
+        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int v = 0; v < 16; ++v) s[kb][v] = 0.0f;
+        constexpr int RING = 3;      // operands are read RING - 1 steps before their products
+        u32x4 ka[RING][2];
+        static_for<RING - 1>([&](auto ic) __attribute__((always_inline)) { read_k(kl, ic, ka[decltype(ic)::value]); });
+        PKV_PRIO(1);
+        static_for<KS>([&](auto ic) __attribute__((always_inline)) {
+            constexpr int i = decltype(ic)::value;
+            if constexpr (i + RING - 1 < KS) read_k(kl, std::integral_constant<int, i + RING - 1>{}, ka[(i + RING - 1) % RING]);
+            s[0] = mfma<F16>(ka[i % RING][0], qreg[i], s[0]);
+            s[1] = mfma<F16>(ka[i % RING][1], qreg[i], s[1]);
+            if constexpr (i == 0) store_k(buf ^ 1), load_k();
+            if constexpr (i == KS / 2 - 1) store_v(buf ^ 1), load_v();
+            PKV_SB();
+        });
+        PKV_PRIO(0);
+        u32x4 va[RING][2];
+        static_for<RING - 1>([&](auto ic) __attribute__((always_inline)) { read_v(vl, ic, va[decltype(ic)::value]); });
+        PKV_SB();
+        // Mask where the block is not wholly visible; the lane holds keys 32 kb + 8 (v / 4) + 4 h + v % 4 of its own
+        // row. With one scale for all keys (sscale > 0 after the sign went into the scores) the maximum is taken over
+        // the raw scores and the scale rides on the exponent's fused multiply-add; with per-key scales (row-scaled
+        // pages) each score is scaled first.
+        if constexpr (KIND >= 2) {
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const uint4 kop = *reinterpret_cast<const uint4*>(&kl[(32 * kb + n32) * KSTR + 16 * ks + 8 * h]);
-                s[kb] = mfma<F16>(kop, qreg[ks], s[kb]);
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) s[kb][v] *= sscale * ks_lds[buf][32 * kb + 8 * (v / 4) + 4 * h + v % 4];
+        }
+        if constexpr (MASK > 0) {
+            // key 32 kb + 8 (v / 4) + v % 4 + 4 h is visible iff that constant is in (rel_lo, rel]
+            const int rel = lim - kt * BN - 4 * h;
+            const int rel_lo = win > 0 ? rel - win : -0x40000000;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int c = 32 * kb + 8 * (v / 4) + v % 4;
+                    const bool vis = c <= rel && c > rel_lo;
+                    s[kb][v] = vis ? s[kb][v] : -INFINITY;
+                }
             }
         }
-        // The next block goes into the other buffer while this one is multiplied (its readers passed the barrier).
-        store_block(buf ^ 1);
-        load_block(upto(kt + 2));
-        load_entries(upto(kt + 3));
-        // Scale (and mask where the block is not wholly visible); the lane holds keys 32 kb + 8 (v / 4) + 4 h + v % 4
-        // of its own row.
-        const bool masked = win > 0 || kt * BN + BN - 1 > wave_lo;
         float top = -INFINITY;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int kin = 32 * kb + 8 * (v / 4) + 4 * h + v % 4;
-                float x = s[kb][v] * (KIND >= 2 ? sscale * ks_lds[buf][kin] : sscale);
-                if (masked) {
-                    const int n = kt * BN + kin;
-                    bool vis = n <= lim;
-                    if (win > 0) vis = vis && n > lim - win;
-                    x = vis ? x : -INFINITY;
-                }
-                s[kb][v] = x;
-                top = __builtin_fmaxf(top, x);
+                top = __builtin_fmaxf(top, s[kb][v]);
             }
         }
+        if constexpr (KIND < 2) top = top == -INFINITY ? -INFINITY : top * sabs;
         top = __builtin_fmaxf(top, __shfl_xor(top, 32));
         const float m_new = __builtin_fmaxf(m, top);
         const float sub = m_new == -INFINITY ? 0.0f : m_new;
         const float alpha = exp2_fast(m - sub);
         m = m_new;
         float sum = 0.0f;
-        uint4 pop[2][2];      // P^T as the second product's B operand: [32-key block][half of it]
+        // P^T as the second product's B operand, 16 keys at a time: the probabilities of keys 32 kb + 16 half .. + 15.
+        auto probs = [&](int kb, int half) __attribute__((always_inline)) -> u32x4 {
+            uint32_t pw[4];
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-            uint32_t pw[8];
-#pragma unroll
-            for (int v2 = 0; v2 < 8; ++v2) {
-                float p0 = exp2_fast(s[kb][2 * v2] - sub), p1 = exp2_fast(s[kb][2 * v2 + 1] - sub);
+            for (int j = 0; j < 4; ++j) {
+                const int v = 8 * half + 2 * j;
+                float p0, p1;
+                if constexpr (KIND >= 2) {
+                    p0 = exp2_fast(s[kb][v] - sub), p1 = exp2_fast(s[kb][v + 1] - sub);
+                } else {
+                    p0 = exp2_fast(__builtin_fmaf(s[kb][v], sabs, -sub)), p1 = exp2_fast(__builtin_fmaf(s[kb][v + 1], sabs, -sub));
+                }
                 sum += p0 + p1;
                 if constexpr (KIND >= 2) {     // the values' scales ride on the operand, not on the sum
-                    p0 *= vs_lds[buf][32 * kb + 8 * ((2 * v2) / 4) + 4 * h + (2 * v2) % 4];
-                    p1 *= vs_lds[buf][32 * kb + 8 * ((2 * v2 + 1) / 4) + 4 * h + (2 * v2 + 1) % 4];
+                    p0 *= vs_lds[buf][32 * kb + 8 * (v / 4) + 4 * h + v % 4];
+                    p1 *= vs_lds[buf][32 * kb + 8 * ((v + 1) / 4) + 4 * h + (v + 1) % 4];
                 }
-                pw[v2] = to_pair<F16>(p0, p1);
+                pw[j] = to_pair<F16>(p0, p1);
             }
-            pop[kb][0] = make_uint4(pw[0], pw[1], pw[2], pw[3]);
-            pop[kb][1] = make_uint4(pw[4], pw[5], pw[6], pw[7]);
-        }
-        l = __builtin_fmaf(l, alpha, sum);
+            return u32x4{pw[0], pw[1], pw[2], pw[3]};
+        };
+        u32x4 pop[4];
+        pop[0] = probs(0, 0);
+        pop[1] = probs(0, 1);
         // wave-uniform: skip the rescale when no row's maximum moved (alpha == 1 everywhere)
         if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+            asm volatile("s_nop 0");      // pins the branch: an unconditional rescale by 1 is what the optimiser would make of it
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) o[nb][v] *= alpha;
         }
-        // O^T += V^T P^T: the lane feeds V^T[dim 32 nb + n32][keys of its half] and its own probabilities.
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-            const int row = 32 * nb + n32;
-            const int sw = swz(row);
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-                for (int half = 0; half < 2; ++half) {
-                    const int g0 = 8 * kb + 4 * half + h;
-                    const uint2 lo = *reinterpret_cast<const uint2*>(&vl[row * BN + 4 * (g0 ^ sw)]);
-                    const uint2 hi = *reinterpret_cast<const uint2*>(&vl[row * BN + 4 * ((g0 + 2) ^ sw)]);
-                    o[nb] = mfma<F16>(make_uint4(lo.x, lo.y, hi.x, hi.y), pop[kb][half], o[nb]);
-                }
+        PKV_SB();
+        // O^T += V^T P^T: the lane feeds V^T[dim 32 nb + n32][keys of its half] and its own probabilities. The second
+        // half's exponentials run in the shadow of the first half's products.
+        PKV_PRIO(1);
+        constexpr int VSTEPS = 2 * NB;
+        static_for<VSTEPS>([&](auto ic) __attribute__((always_inline)) {
+            constexpr int i = decltype(ic)::value;
+            constexpr int g = i / (NB / 2), nb = 2 * (i % (NB / 2));
+            if constexpr (i + RING - 1 < VSTEPS) read_v(vl, std::integral_constant<int, i + RING - 1>{}, va[(i + RING - 1) % RING]);
+            o[nb] = mfma<F16>(va[i % RING][0], pop[g], o[nb]);
+            o[nb + 1] = mfma<F16>(va[i % RING][1], pop[g], o[nb + 1]);
+            if constexpr (i == 0) pop[2] = probs(1, 0);
+            if constexpr (i == NB / 2) pop[3] = probs(1, 1);
+            if constexpr (i == VSTEPS - 2) {      // the slots of block kt + 3 for the next iteration's loads, the entries of kt + 4
+                take_slots();
+                load_entries(upto(kt + 4));
             }
-        }
+            PKV_SB();
+        });
+        PKV_PRIO(0);
+        l = __builtin_fmaf(l, alpha, sum);
+    };
+    // Blocks wholly visible to every row of the workgroup first (none under a sliding window), then the masked ones.
+    const int kt_full = win > 0 ? kt_lo : max(kt_lo, min(kt_hi + 1, (pos + t_lo + 1) / BN));
+    for (int kt = kt_lo; kt < kt_full; ++kt) {
+        block(kt, std::integral_constant<int, 0>{});
         __syncthreads();          // every wavefront is done with this buffer; the other one is stored
+    }
+    for (int kt = kt_full; kt <= kt_hi; ++kt) {
+        block(kt, std::integral_constant<int, 1>{});
+        __syncthreads();
     }
     // The two half-waves hold the same row's sums over different keys.
     l += __shfl_xor(l, 32);
@@ -430,7 +545,7 @@ int launch_prefill(const crit_pkv_prefill_params* p, hipStream_t stream) {
     const bool f16 = p->page_dtype == CRIT_PKV_F16;
     if (f16 && p->kind != 0) return CRIT_PKV_E_DTYPE;
     if (p->out_dtype != CRIT_PKV_F32 && p->out_dtype != CRIT_PKV_BF16 && p->out_dtype != CRIT_PKV_F16) return CRIT_PKV_E_DTYPE;
-    if (p->chunks < 1 || p->chunks > 65535 || p->max_count < 1 || p->kv_heads < 1 || p->kv_heads > 65535 || p->heads < 1 ||
+    if (p->chunks < 1 || p->chunks > 65535 || p->max_count < 1 || p->max_count > (1 << 30) || p->kv_heads < 1 || p->kv_heads > 65535 || p->heads < 1 ||
         p->heads % p->kv_heads || p->page < 1 || p->table_width < 1 || p->sliding < 0)
         return CRIT_PKV_E_GEOMETRY;
     if (p->head_dim != 64 && p->head_dim != 128) return CRIT_PKV_E_GEOMETRY;
@@ -452,14 +567,16 @@ int launch_prefill(const crit_pkv_prefill_params* p, hipStream_t stream) {
     a.tab_width = p->table_width, a.chunks = p->chunks, a.max_count = p->max_count, a.hq = p->heads, a.hkv = p->kv_heads;
     a.g = p->heads / p->kv_heads;
     a.page = p->page;
-    a.page_shift = -1;
-    for (int s = 0; s < 31; ++s)
-        if ((1 << s) == p->page) a.page_shift = s;
+    a.page_l = 0;
+    while ((1ll << a.page_l) < p->page) ++a.page_l;
+    a.page_magic = (uint32_t)((((1ull << a.page_l) - (uint64_t)p->page) << 32) / (uint64_t)p->page + 1);
     a.sliding = p->sliding, a.out_dtype = p->out_dtype;
     a.sscale = p->scale * kLog2e, a.k_mult = p->key_multiplier, a.v_mult = p->value_multiplier;
     const int64_t tiles = ((int64_t)p->max_count * a.g + BM - 1) / BM;
-    if (tiles > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
-    const dim3 grid((unsigned)tiles, (unsigned)p->kv_heads, (unsigned)p->chunks);
+    const int64_t groups8 = ((int64_t)p->kv_heads * p->chunks + 7) / 8;
+    if (tiles * groups8 * 8 > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
+    a.tiles = (int)tiles;
+    const dim3 grid((unsigned)(tiles * groups8 * 8));
     switch (p->kind) {
         case 0: return f16 ? launch_d<0, true>(a, p->head_dim, grid, stream) : launch_d<0, false>(a, p->head_dim, grid, stream);
         case 1: return launch_d<1, false>(a, p->head_dim, grid, stream);
