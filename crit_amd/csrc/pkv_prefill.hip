@@ -387,8 +387,18 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
             s[1] = mfma<F16>(ka[i % RING][1], qreg[i], s[1]);
             if constexpr (i == 0) store_k(buf ^ 1), load_k();
             if constexpr (i == KS / 2 - 1) store_v(buf ^ 1), load_v();
-            PKV_SB();
         });
+        // one product, then a share of the staging work (LDS reads of later operands, the stores' permutes and
+        // writes, the row loads) in its shadow
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * (RING - 1), 0);
+        static_for<2 * KS>([&](auto) __attribute__((always_inline)) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        });
+        PKV_SB();
         PKV_PRIO(0);
         u32x4 va[RING][2];
         static_for<RING - 1>([&](auto ic) __attribute__((always_inline)) { read_v(vl, ic, va[decltype(ic)::value]); });
