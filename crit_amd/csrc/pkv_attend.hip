@@ -1,5 +1,7 @@
 // Host side of the decode / verify-window launches (argument checks, grid, the choice of kernel) and the small
 // kernels around the split launch: the merge of the partitions, the merge of shard partials, a streaming-read probe.
+#include <atomic>
+
 #include "pkv_attend_args.hpp"
 #include "pkv_launch.hpp"
 
@@ -136,6 +138,50 @@ static int pick_qr(int live_rows) {
     return 8;
 }
 
+// -- the unit-pulling launches' counters ------------------------------------------------------------------------------------
+constexpr int kTicketPairs = 64;
+static __device__ __align__(256) unsigned pkv_tickets[2 * kTicketPairs];      // zero at load; every device has its own copy
+
+namespace {
+constexpr int kMaxDevices = 64;
+struct DeviceState {
+    std::atomic<int> cus{-1};
+    std::atomic<unsigned*> tickets{nullptr};
+    std::atomic<unsigned> next{0};
+};
+DeviceState g_devices[kMaxDevices];
+DeviceState* device_state() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    return &g_devices[dev];
+}
+}   // namespace
+
+int compute_units() {
+    DeviceState* st = device_state();
+    if (!st) return 0;
+    int n = st->cus.load(std::memory_order_relaxed);
+    if (n < 0) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        st->cus.store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
+unsigned* next_ticket() {
+    DeviceState* st = device_state();
+    if (!st) return nullptr;
+    unsigned* base = st->tickets.load(std::memory_order_acquire);
+    if (!base) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(pkv_tickets)) != hipSuccess || !ptr) return nullptr;
+        base = static_cast<unsigned*>(ptr);
+        st->tickets.store(base, std::memory_order_release);
+    }
+    return base + 2 * (st->next.fetch_add(1, std::memory_order_relaxed) % kTicketPairs);
+}
+
 int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     if (!p || !p->q || !p->key_pages || !p->value_pages || !p->tables || !p->rows || !p->starts || !p->firsts || !p->out)
         return CRIT_PKV_E_NULL;
@@ -192,6 +238,12 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     const int64_t live_parts = (a.max_keys + (int64_t)p->piece - 1) / p->piece;
     const unsigned gy = (unsigned)(live_parts < p->partitions ? live_parts : p->partitions);
     const dim3 grid((unsigned)gx, p->fused ? 1u : gy);
+    a.units_x = a.units_y = 0;
+    a.ticket = nullptr;
+    if (lpr == 16 && page16) {
+        a.ticket = next_ticket();
+        if (!a.ticket || compute_units() < 1) return CRIT_PKV_E_GEOMETRY;
+    }
     auto split = [&](bool fused) -> int {
         switch (p->kind) {
             case 0: return f16 ? launch_attend_f16(a, lpr, qr, fused, page16, grid, stream)

@@ -84,8 +84,9 @@ constexpr int attend_waves(int kind, int qr) { return qr <= 2 ? 4 : (qr <= 4 && 
 
 // Pages are a multiple of 16 positions, so the 16 positions of a step share one page table entry, which is uniform
 // over the wavefront: a step's addresses are a scalar base plus per-lane offsets that do not change from step to step.
+// One unit of work: (ux, uy) of a units_x x units_y list, what a workgroup of a plain launch would get as blockIdx.
 template <int KIND, bool F16, int QR, int HW, bool FUSED>
-__global__ __launch_bounds__(256, attend_waves(KIND, QR)) void attend128_kernel(AttendArgs a) {
+PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
     constexpr int D = 128;
     constexpr int RB = (QR + 3) / 4;            // blocks of four query rows
     constexpr int EB = KIND == 0 ? 2 : 1;
@@ -105,18 +106,22 @@ __global__ __launch_bounds__(256, attend_waves(KIND, QR)) void attend128_kernel(
     const int li8 = lane & 7;
     const int q4 = 2 * b2 + b3;                 // which of the DPP row's four positions this lane's score is of
     const int hw = rho % HW, pb = rho / HW;     // the DPP row's head (of the wavefront's HW) and position block
-    int bx = blockIdx.x;
+    int bx = ux;
     const int tile = bx % a.tiles;
     bx /= a.tiles;
     const int hgroups = a.hkv / HW;
     const int kvh = (bx % hgroups) * HW + hw;   // this lane's KV head
     const int r = bx / hgroups;
-    const int b = blockIdx.y;
-    int count = a.columns;
-    if (a.counts) count = min(a.counts[r], a.columns);
+    int b = uy;
+    // The row's four descriptors are read together, ahead of every test that could end the unit: one memory round
+    // trip instead of a chain of them at the start of every unit.
+    const int count_in = a.counts ? a.counts[r] : a.columns;
+    const int64_t first64 = a.firsts[r];
+    const int64_t trow = (int64_t)a.rows[r] * a.tab_stride;
+    const int start = a.starts[r];
+    const int count = min(count_in, a.columns);
     const int j0 = tile * QR;
     if (j0 >= count * a.g) return;
-    const int64_t first64 = a.firsts[r];
     const int c_lo = j0 / a.g;
     const int c_hi = min(count, (j0 + QR - 1) / a.g + 1);
     int64_t nk64 = first64 + c_hi;
@@ -124,9 +129,14 @@ __global__ __launch_bounds__(256, attend_waves(KIND, QR)) void attend128_kernel(
     const int n_keys = (int)nk64;
     const int first = (int)(first64 < 0 ? 0 : (first64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first64));
     const int n_pieces = (n_keys + a.piece - 1) / a.piece;
-    if (!FUSED && b >= n_pieces) return;
-    const int64_t trow = (int64_t)a.rows[r] * a.tab_stride;
-    const int start = a.starts[r];
+    if constexpr (!FUSED) {
+        // Units are taken in list order, y slowest: the row's last partition (usually a partial piece, the smallest
+        // unit of work) takes the last y, so the small units start last and fill the launch's tail.
+        const int np = min(n_pieces, a.parts);
+        if (np <= 0) return;
+        if (b == a.units_y - 1) b = np - 1;
+        else if (b >= np - 1) return;
+    }
 
     // The lane's slices of the tile's query rows (packed 16-bit pairs): dims 8 li8 .. +7 and 64 + 8 li8 .. +7 over
     // 16-bit pages, dims 16 li8 .. +15 over 8-bit pages (the dims its K loads cover).
@@ -529,6 +539,35 @@ __global__ __launch_bounds__(256, attend_waves(KIND, QR)) void attend128_kernel(
                     }
                 }
             }
+        }
+    }
+}
+
+// The launch: as many workgroups as the card holds at once, each taking units from a ticket counter until the list is
+// exhausted. The hardware's own dispatcher binds a workgroup to an XCD by its id and starts workgroups strictly in
+// order, so with units as uneven as ragged contexts make them it leaves slots idle behind a busy one; resident
+// workgroups that pull the next unit themselves keep every slot busy to the end. The last workgroup to finish zeroes
+// the counters for the next launch that uses them.
+template <int KIND, bool F16, int QR, int HW, bool FUSED>
+__global__ __launch_bounds__(256, attend_waves(KIND, QR)) void attend128_kernel(AttendArgs a) {
+    __shared__ unsigned s_unit;
+    const unsigned total = (unsigned)a.units_x * (unsigned)a.units_y;
+    if (threadIdx.x == 0) s_unit = atomicAdd(a.ticket, 1u);
+    __syncthreads();
+    unsigned u = s_unit;
+    while (u < total) {
+        // (the next ticket is drawn after the unit, not during it: a returning atomic in flight makes every wait on
+        // the unit's loads a wait for all of them, which costs more than the ticket's round trip)
+        attend128_unit<KIND, F16, QR, HW, FUSED>(a, (int)(u % (unsigned)a.units_x), (int)(u / (unsigned)a.units_x));
+        __syncthreads();      // the unit is done with the shared arrays, and every thread has read s_unit
+        if (threadIdx.x == 0) s_unit = atomicAdd(a.ticket, 1u);
+        __syncthreads();
+        u = s_unit;
+    }
+    if (threadIdx.x == 0) {
+        if (atomicAdd(a.ticket + 1, 1u) == gridDim.x - 1) {
+            atomicExch(a.ticket, 0u);
+            atomicExch(a.ticket + 1, 0u);
         }
     }
 }

@@ -25,8 +25,9 @@ struct AttendArgs {
     void* out;
     float* lse;
     const float* sinks;
+    unsigned* ticket;      // two zeroed counters of the unit-pulling launches: next unit, workgroups done
     int64_t q_st, q_sh, o_st, o_sh, tab_stride;
-    int tab_width, n_rows, columns, hq, hkv, g, page, page_shift, parts, piece, sliding, out_dtype, tiles, max_keys, heads_per_wave;
+    int tab_width, n_rows, columns, hq, hkv, g, page, page_shift, parts, piece, sliding, out_dtype, tiles, max_keys, heads_per_wave, units_x, units_y;
     float sscale, k_mult, v_mult;
 };
 

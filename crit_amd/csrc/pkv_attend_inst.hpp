@@ -3,16 +3,23 @@
 #pragma once
 #include "pkv_attend128.hpp"
 #include "pkv_attend_generic.hpp"
+#include "pkv_launch.hpp"
 
 namespace pkv {
 
 template <int KIND, bool F16, int QR, bool FUSED>
 static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipStream_t stream) {
-    if (lpr == 16 && page16) {       // pages of a multiple of 16 positions: the bandwidth path
+    if (lpr == 16 && page16) {       // pages of a multiple of 16 positions: the bandwidth path, resident workgroups pulling units
+        AttendArgs u = a;
+        u.units_x = (int)grid.x, u.units_y = (int)grid.y;
+        const int64_t units = (int64_t)grid.x * grid.y;
+        if (units > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
+        const int64_t resident = (int64_t)compute_units() * attend_waves(KIND, QR);
+        const dim3 pgrid((unsigned)(units < resident ? units : resident));
         switch (a.heads_per_wave) {
-            case 1: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 1, FUSED>), grid, dim3(256), 0, stream, a); break;
-            case 2: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 2, FUSED>), grid, dim3(256), 0, stream, a); break;
-            case 4: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 4, FUSED>), grid, dim3(256), 0, stream, a); break;
+            case 1: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 1, FUSED>), pgrid, dim3(256), 0, stream, u); break;
+            case 2: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 2, FUSED>), pgrid, dim3(256), 0, stream, u); break;
+            case 4: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 4, FUSED>), pgrid, dim3(256), 0, stream, u); break;
             default: return CRIT_PKV_E_GEOMETRY;
         }
     } else if (lpr == 16) {
