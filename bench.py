@@ -24,6 +24,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, vendor figure
 
+# HBM bytes one split launch moves, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this file (each counter in
+# a run of its own, scaled by what it reads for the stream-read probe and for a 262,144-token append, kernels of
+# known size: factors 0.5000 and 1.000). Measured for the default workload only.
+MEASURED_TRAFFIC_BYTES = {"c2": 1_436_963_942}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -302,6 +307,9 @@ def main():
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also launch one KV append of 262,144 tokens: with the stream-read probe, two kernels of known "
+                         "read and write sizes against which FETCH_SIZE / WRITE_SIZE counters are scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no cross-GPU part (run with --gpus 1)")
@@ -345,7 +353,8 @@ def main():
         "dtype": "bf16" if w.kind == "bf16" else "fp8_e4m3 KV, bf16 q, f32 accumulate", "data": "synthetic",
         "config": {"workload": spec["name"], "positions": w.tokens, "partitions": w.parts, "piece": w.piece},
         "roofline": {"bound": "hbm", "kernel": "attend_kernel (split launch)", "achieved": round(achieved, 1),
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "launch_ms": round(split_ms, 4), "merge_ms": round(merge_ms, 4),
                      "algorithmic_bytes_per_launch": w.decode_bytes,
                      "stream_read_GB/s": round(stream_gbps, 1)},
@@ -357,6 +366,19 @@ def main():
         f"append {append_ms * 1e3:.1f} us; stream read {stream_gbps:.0f} GB/s")
     del w
     torch.cuda.empty_cache()
+    if args.calibrate:
+        T, hkv, d = 262144, 8, 128
+        ck = torch.zeros(1 << 20, hkv, d, dtype=torch.bfloat16, device=device)
+        cv = torch.zeros_like(ck)
+        keys = torch.randn(T, hkv, d, device=device).to(torch.bfloat16)
+        values = torch.randn(T, hkv, d, device=device).to(torch.bfloat16)
+        slots = torch.randperm(1 << 20, device=device)[:T]
+        pk.write(keys, values, slots, ck, cv, "bf16")
+        torch.cuda.synchronize()
+        log(f"[bench] calibration: stream_read_kernel reads {read_bytes} bytes a launch; write_rows of {T} tokens reads "
+            f"{2 * T * hkv * d * 2 + T * 8} bytes and writes {2 * T * hkv * d * 2} bytes")
+        del ck, cv, keys, values, slots
+        torch.cuda.empty_cache()
     if not args.no_extras:
         extras = {}
         other = "c3" if args.workload == "c2" else "c2"
