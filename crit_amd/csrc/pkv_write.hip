@@ -56,79 +56,117 @@ PKV_DEV void load_vec(const void* base, int64_t i, float (&x)[EPL]) {
 }
 
 // One row = (token, head) with head in [0, heads): keys' heads first, then values'. LPR lanes hold one row, EPL
-// elements each (16 bytes of page row). KIND as in the ABI; F16: 16-bit pages are fp16, not bf16.
-template <int KIND, bool F16, int IN, int LPR>
+// elements each (16 bytes of page row). KIND as in the ABI; F16: 16-bit pages are fp16, not bf16. A thread takes U rows,
+// 256 / LPR apart (so a workgroup's accesses stay contiguous per pass), and issues all their loads before the first
+// store: U times the bytes in flight per thread, which is what a streaming copy on this card needs.
+template <int KIND, bool F16, int IN, int LPR, int U>
 __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
     constexpr int EPL = KIND == 0 ? 8 : 16;
+    constexpr int RPP = 256 / LPR;      // rows a workgroup covers per pass
     const int lane_in_row = threadIdx.x % LPR;
-    const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPR;
-    if (row >= a.tokens * a.heads) return;
-    const int64_t t = row / a.heads;
-    int head = (int)(row % a.heads);
-    const int which = head >= a.hkv ? 1 : 0;
-    head -= which * a.hkv;
-    const int64_t slot = a.slots[t];
-    if (slot < 0) return;
-    const int dim = a.dim[which];
+    const int64_t row0 = (int64_t)blockIdx.x * (RPP * U) + threadIdx.x / LPR;
+    const int64_t n_rows = a.tokens * a.heads;
     const int i0 = lane_in_row * EPL;
-    const bool live = i0 < dim;
-    float x[EPL];
-    if (live) {
-        load_vec<IN, EPL>(a.src[which], t * a.stride_t[which] + head * a.stride_h[which] + i0, x);
-    } else {
+    float x[U][EPL];
+    int64_t slot[U];
+    int head[U], which[U];
+    bool live[U];
 #pragma unroll
-        for (int j = 0; j < EPL; ++j) x[j] = 0.0f;
+    for (int u = 0; u < U; ++u) {
+        const int64_t row = row0 + u * RPP;
+        const bool in = row < n_rows;
+        const int64_t t = in ? row / a.heads : 0;
+        head[u] = in ? (int)(row % a.heads) : 0;
+        which[u] = head[u] >= a.hkv ? 1 : 0;
+        head[u] -= which[u] * a.hkv;
+        slot[u] = in ? a.slots[t] : -1;
+        live[u] = in && i0 < a.dim[which[u]];
+        if (live[u]) {
+            load_vec<IN, EPL>(a.src[which[u]], t * a.stride_t[which[u]] + head[u] * a.stride_h[which[u]] + i0, x[u]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < EPL; ++j) x[u][j] = 0.0f;
+        }
     }
-    const int64_t dst = (slot * a.hkv + head) * dim + i0;
-    if constexpr (KIND == 0) {
-        uint4 v;
-        if constexpr (F16) {
-            v = make_uint4(pack_f16(x[0], x[1]), pack_f16(x[2], x[3]), pack_f16(x[4], x[5]), pack_f16(x[6], x[7]));
-        } else {
-            v = make_uint4(pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]), pack_bf16(x[6], x[7]));
-        }
-        if (live) *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(a.pages[which]) + dst) = v;
-    } else {
-        float div;
-        if constexpr (KIND == 1) {
-            div = a.head_mult ? a.head_mult[which * a.hkv + head] : a.mult[which];
-        } else {
-            float amax = 0.0f;
 #pragma unroll
-            for (int j = 0; j < EPL; ++j) {
-                const float m = __builtin_fabsf(x[j]);
-                amax = (m > amax || m != m) ? m : amax;       // a NaN in the row makes the scale NaN, as torch's amax
+    for (int u = 0; u < U; ++u) {
+        // (a whole row's lanes agree on slot[u] < 0, so the row-scale exchange below stays among participating lanes)
+        if (slot[u] < 0) continue;
+        const int dim = a.dim[which[u]];
+        const int64_t dst = (slot[u] * a.hkv + head[u]) * dim + i0;
+        if constexpr (KIND == 0) {
+            uint4 v;
+            if constexpr (F16) {
+                v = make_uint4(pack_f16(x[u][0], x[u][1]), pack_f16(x[u][2], x[u][3]), pack_f16(x[u][4], x[u][5]), pack_f16(x[u][6], x[u][7]));
+            } else {
+                v = make_uint4(pack_bf16(x[u][0], x[u][1]), pack_bf16(x[u][2], x[u][3]), pack_bf16(x[u][4], x[u][5]), pack_bf16(x[u][6], x[u][7]));
             }
+            if (live[u]) *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(a.pages[which[u]]) + dst) = v;
+        } else {
+            float div;
+            if constexpr (KIND == 1) {
+                div = a.head_mult ? a.head_mult[which[u] * a.hkv + head[u]] : a.mult[which[u]];
+            } else {
+                float amax = 0.0f;
 #pragma unroll
-            for (int o = 1; o < LPR; o <<= 1) {
-                const float other = __shfl_xor(amax, o);
-                amax = (other > amax || other != other) ? other : amax;
-            }
-            const float top = KIND == 2 ? 448.0f : 127.0f;
-            div = __fdiv_rn(amax, top);
-            div = div < 1e-30f ? 1e-30f : div;               // clamp(min=1e-30); NaN stays NaN
-            if (lane_in_row == 0) a.scales[which][slot * a.hkv + head] = div;
-        }
-        uint32_t w[4];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            uint32_t packed = 0;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float q = __fdiv_rn(x[4 * k + j], div);
-                uint32_t code;
-                if constexpr (KIND == 3) {
-                    float r = __builtin_rintf(q);            // ties to even
-                    r = r < -127.0f ? -127.0f : (r > 127.0f ? 127.0f : r);
-                    code = (uint32_t)(int)r & 0xffu;
-                } else {
-                    code = e4m3_encode(q);
+                for (int j = 0; j < EPL; ++j) {
+                    const float m = __builtin_fabsf(x[u][j]);
+                    amax = (m > amax || m != m) ? m : amax;       // a NaN in the row makes the scale NaN, as torch's amax
                 }
-                packed |= code << (8 * j);
+#pragma unroll
+                for (int o = 1; o < LPR; o <<= 1) {
+                    const float other = __shfl_xor(amax, o);
+                    amax = (other > amax || other != other) ? other : amax;
+                }
+                const float top = KIND == 2 ? 448.0f : 127.0f;
+                div = __fdiv_rn(amax, top);
+                div = div < 1e-30f ? 1e-30f : div;               // clamp(min=1e-30); NaN stays NaN
+                if (lane_in_row == 0) a.scales[which[u]][slot[u] * a.hkv + head[u]] = div;
             }
-            w[k] = packed;
+            uint32_t w[4];
+            float q[16];
+#pragma unroll
+            for (int j = 0; j < 16; ++j) q[j] = __fdiv_rn(x[u][j], div);
+            if constexpr (KIND == 3) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    uint32_t packed = 0;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        float r = __builtin_rintf(q[4 * k + j]);            // ties to even
+                        r = r < -127.0f ? -127.0f : (r > 127.0f ? 127.0f : r);
+                        packed |= ((uint32_t)(int)r & 0xffu) << (8 * j);
+                    }
+                    w[k] = packed;
+                }
+            } else {
+                // Finite quotients (all but the rarest rows): clamp, then the hardware's round-to-nearest-even
+                // conversion, two codes an instruction; a NaN anywhere in the lane's 16 (or infinities of both signs,
+                // whose sum is NaN too) sends the lane through the integer encoder, which fixes the NaN code and sign.
+                float sum = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 16; ++j) sum += q[j];
+                if (sum == sum) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const float c0 = __builtin_amdgcn_fmed3f(q[4 * k], -448.0f, 448.0f), c1 = __builtin_amdgcn_fmed3f(q[4 * k + 1], -448.0f, 448.0f);
+                        const float c2 = __builtin_amdgcn_fmed3f(q[4 * k + 2], -448.0f, 448.0f), c3 = __builtin_amdgcn_fmed3f(q[4 * k + 3], -448.0f, 448.0f);
+                        int packed = __builtin_amdgcn_cvt_pk_fp8_f32(c0, c1, 0, false);
+                        packed = __builtin_amdgcn_cvt_pk_fp8_f32(c2, c3, packed, true);
+                        w[k] = (uint32_t)packed;
+                    }
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        uint32_t packed = 0;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) packed |= e4m3_encode(q[4 * k + j]) << (8 * j);
+                        w[k] = packed;
+                    }
+                }
+            }
+            if (live[u]) *reinterpret_cast<uint4*>(reinterpret_cast<uint8_t*>(a.pages[which[u]]) + dst) = make_uint4(w[0], w[1], w[2], w[3]);
         }
-        if (live) *reinterpret_cast<uint4*>(reinterpret_cast<uint8_t*>(a.pages[which]) + dst) = make_uint4(w[0], w[1], w[2], w[3]);
     }
 }
 
@@ -186,11 +224,16 @@ static int launch_kind(const WriteArgs& a, int lpr, bool vector, hipStream_t str
         hipLaunchKernelGGL((write_rows_scalar<KIND, F16, IN>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
         return hip_code(hipGetLastError());
     }
-    const int64_t blocks = (rows * lpr + 255) / 256;
+    // Four rows a thread once there is work for every compute unit several times over; one row a thread below that,
+    // where the launch is latency-bound and more workgroups finish sooner.
+    const bool wide = rows * lpr >= (int64_t)1 << 19;
+    const int rows_per_block = 256 / lpr * (wide ? 4 : 1);
+    const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
     switch (lpr) {
-#define PKV_CASE(L)                                                                                              \
-    case L:                                                                                                      \
-        hipLaunchKernelGGL((write_rows<KIND, F16, IN, L>), dim3((unsigned)blocks), dim3(256), 0, stream, a);     \
+#define PKV_CASE(L)                                                                                                 \
+    case L:                                                                                                         \
+        if (wide) hipLaunchKernelGGL((write_rows<KIND, F16, IN, L, 4>), dim3((unsigned)blocks), dim3(256), 0, stream, a); \
+        else hipLaunchKernelGGL((write_rows<KIND, F16, IN, L, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, a);      \
         break;
         PKV_CASE(1) PKV_CASE(2) PKV_CASE(4) PKV_CASE(8) PKV_CASE(16) PKV_CASE(32) PKV_CASE(64)
 #undef PKV_CASE
