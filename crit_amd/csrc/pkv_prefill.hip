@@ -12,45 +12,10 @@
 // the B operand it must feed to the second product: no shuffle, no LDS round trip for P.
 //
 // A token's bits follow its own positions only: the key blocks are absolute, masked keys contribute exact zeros.
-#include "pkv_common.hpp"
 #include "pkv_launch.hpp"
+#include "pkv_prefill.hpp"
 
 namespace pkv {
-
-struct PrefillArgs {
-    const uint8_t* q;
-    const uint8_t* kp;
-    const uint8_t* vp;
-    const float* ks;
-    const float* vs;
-    const float* hm;
-    const int32_t* tables;
-    const int64_t* tables64;
-    const int32_t* table_rows;
-    const int32_t* starts;
-    const int32_t* counts;
-    const int64_t* positions;
-    void* out;
-    float* lse;
-    const float* sinks;
-    int64_t q_st, q_sh, o_st, o_sh, tab_stride;
-    int tab_width, chunks, max_count, hq, hkv, g, page, page_l, sliding, out_dtype, tiles;
-    uint32_t page_magic;     // n / page == (mulhi(page_magic, n) + n) >> page_l for 0 <= n < 2^31
-    float sscale, k_mult, v_mult;
-};
-
-#ifndef PKV_NO_PRIO
-#define PKV_PRIO(x) __builtin_amdgcn_s_setprio(x)
-#else
-#define PKV_PRIO(x)
-#endif
-#ifdef PKV_NO_SB
-#define PKV_SB()
-#else
-#define PKV_SB() __builtin_amdgcn_sched_barrier(0)
-#endif
-constexpr int BM = 128;   // query rows a workgroup holds
-constexpr int BN = 64;    // keys a block holds
 
 // 8 codes (two words of E4M3 or INT8) -> 8 BF16 values packed in a uint4, exactly.
 template <int KIND>
@@ -72,34 +37,6 @@ PKV_DEV uint4 codes_to_bf16(uint32_t w0, uint32_t w1) {
 }
 
 template <bool F16>
-PKV_DEV f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
-    if constexpr (F16) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-    } else {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-    }
-}
-template <bool F16>
-PKV_DEV f32x16 mfma(u32x4 a, uint4 b, f32x16 c) { return mfma<F16>(a, u32x4{b.x, b.y, b.z, b.w}, c); }
-template <bool F16>
-PKV_DEV f32x16 mfma(uint4 a, uint4 b, f32x16 c) {
-    if constexpr (F16) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-    } else {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-    }
-}
-
-// Two probabilities as a 16-bit pair by the hardware conversions (round to nearest even).
-template <bool F16>
-PKV_DEV uint32_t to_pair(float a, float b) {
-    if constexpr (F16) return pack_f16(a, b);
-    typedef __attribute__((ext_vector_type(2))) __bf16 pair_t;
-    pair_t r = {(__bf16)a, (__bf16)b};
-    return __builtin_bit_cast(uint32_t, r);
-}
-
-template <bool F16>
 PKV_DEV float dot2_acc(uint32_t a, uint32_t b, float c) {
     if constexpr (F16) {
         return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
@@ -107,12 +44,6 @@ PKV_DEV float dot2_acc(uint32_t a, uint32_t b, float c) {
         return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
     }
 }
-
-// V^T in LDS is [dim][64 keys], rows of 128 bytes without padding; the 8-byte group of four keys g of row `row` sits
-// at group g ^ swz(row). The stores (16 lanes: 16 dim chunks of 8 rows, one row of each) and the operand reads (16
-// lanes: 16 adjacent rows) both spread over all banks, and the swizzle is a XOR of bit fields, so an address is one
-// per-thread value XOR a compile-time constant plus a compile-time offset.
-PKV_DEV int swz(int row) { return ((row >> 3) & 15) ^ ((row & 7) << 1); }
 
 template <int KIND, bool F16, int D>
 __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
@@ -137,7 +68,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
     const int group = xcd + 8 * (q / a.tiles);
     if (group >= a.hkv * a.chunks) return;
     const int tile = a.tiles - 1 - q % a.tiles;
-    const int kvh = group % a.hkv, z = group / a.hkv;
+    const int kvh = group % a.hkv, z = chunk_by_rank(a, group / a.hkv, lane);
     int count = a.max_count;
     if (a.counts) count = min(a.counts[z], a.max_count);
     if ((int64_t)tile * BM >= (int64_t)count * a.g) return;
@@ -437,7 +368,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
         }
         if constexpr (KIND < 2) top = top == -INFINITY ? -INFINITY : top * sabs;
         top = __builtin_fmaxf(top, __shfl_xor(top, 32));
-        const float m_new = __builtin_fmaxf(m, top);
+        const float m_new = top > m + kMaxSlack ? top : m;
         const float sub = m_new == -INFINITY ? 0.0f : m_new;
         const float alpha = exp2_fast(m - sub);
         m = m_new;

@@ -1,0 +1,103 @@
+// Declarations of the chunked-prefill kernel: the launch arguments, the MFMA wrappers, the LDS swizzle of V^T, the
+// order in which chunks are taken.
+#pragma once
+#include "pkv_common.hpp"
+
+namespace pkv {
+
+struct PrefillArgs {
+    const uint8_t* q;
+    const uint8_t* kp;
+    const uint8_t* vp;
+    const float* ks;
+    const float* vs;
+    const float* hm;
+    const int32_t* tables;
+    const int64_t* tables64;
+    const int32_t* table_rows;
+    const int32_t* starts;
+    const int32_t* counts;
+    const int64_t* positions;
+    void* out;
+    float* lse;
+    const float* sinks;
+    int64_t q_st, q_sh, o_st, o_sh, tab_stride;
+    int tab_width, chunks, max_count, hq, hkv, g, page, page_l, sliding, out_dtype, tiles;
+    uint32_t page_magic;     // n / page == (mulhi(page_magic, n) + n) >> page_l for 0 <= n < 2^31
+    float sscale, k_mult, v_mult;
+};
+
+#ifndef PKV_NO_PRIO
+#define PKV_PRIO(x) __builtin_amdgcn_s_setprio(x)
+#else
+#define PKV_PRIO(x)
+#endif
+#ifdef PKV_NO_SB
+#define PKV_SB()
+#else
+#define PKV_SB() __builtin_amdgcn_sched_barrier(0)
+#endif
+// The running maximum a row's exponentials are taken against moves only when a block's maximum exceeds it by more
+// than this (in log2 units): probabilities then reach 2^8 at most, far inside the range of the 16-bit operand and the
+// FP32 sums, the final division by the row's sum (taken against the same reference) cancels the factor, and the
+// accumulators are rescaled on a handful of blocks instead of most of them. A row's own data decide, nothing else.
+constexpr float kMaxSlack = 8.0f;
+constexpr int BM = 128;   // query rows a workgroup holds
+constexpr int BN = 64;    // keys a block holds
+
+template <bool F16>
+PKV_DEV f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
+    if constexpr (F16) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+}
+template <bool F16>
+PKV_DEV f32x16 mfma(u32x4 a, uint4 b, f32x16 c) { return mfma<F16>(a, u32x4{b.x, b.y, b.z, b.w}, c); }
+template <bool F16>
+PKV_DEV f32x16 mfma(uint4 a, uint4 b, f32x16 c) {
+    if constexpr (F16) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+}
+
+// Two probabilities as a 16-bit pair by the hardware conversions (round to nearest even).
+template <bool F16>
+PKV_DEV uint32_t to_pair(float a, float b) {
+    if constexpr (F16) return pack_f16(a, b);
+    typedef __attribute__((ext_vector_type(2))) __bf16 pair_t;
+    pair_t r = {(__bf16)a, (__bf16)b};
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+// V^T in LDS is [dim][64 keys], rows of 128 bytes without padding; the 8-byte group of four keys g of row `row` sits
+// at group g ^ swz(row). The stores (16 lanes: 16 dim chunks of 8 rows, one row of each) and the operand reads (16
+// lanes: 16 adjacent rows) both spread over all banks, and the swizzle is a XOR of bit fields, so an address is one
+// per-thread value XOR a compile-time constant plus a compile-time offset.
+PKV_DEV int swz(int row) { return ((row >> 3) & 15) ^ ((row & 7) << 1); }
+
+// Workgroups start in grid order, and a launch's tail is as long as the last ones to start: the chunks are taken
+// longest first (most keys to walk; ties by index). Every wavefront ranks the chunks for itself, lane i holding chunk
+// i: launches of up to 64 chunks, larger ones keep the caller's order.
+PKV_DEV int chunk_by_rank(const PrefillArgs& a, int rank, int lane) {
+    if (a.chunks > 64 || a.chunks < 2) return rank;
+    int len = -1;
+    if (lane < a.chunks) {
+        const int count = a.counts ? min(a.counts[lane], a.max_count) : a.max_count;
+        int64_t pos = a.positions[lane];
+        pos = pos < 0 ? 0 : (pos > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : pos);
+        len = (int)pos + (count > 0 ? count : 0);
+    }
+    int ahead = 0;      // chunks that go before this lane's
+    for (int j = 0; j < a.chunks; ++j) {
+        const int other = __shfl(len, j);
+        ahead += (other > len || (other == len && j < lane)) ? 1 : 0;
+    }
+    const unsigned long long hit = __ballot(lane < a.chunks && ahead == rank);
+    return __ffsll(hit) - 1;
+}
+
+}   // namespace pkv
