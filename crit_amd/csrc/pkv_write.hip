@@ -41,7 +41,7 @@ PKV_DEV void load_vec(const void* base, int64_t i, float (&x)[EPL]) {
         const uint4* p = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(base) + i);
 #pragma unroll
         for (int j = 0; j < EPL / 8; ++j) {
-            uint4 v = p[j];
+            const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p) + j);      // read once
             uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
@@ -101,7 +101,7 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
             } else {
                 v = make_uint4(pack_bf16(x[u][0], x[u][1]), pack_bf16(x[u][2], x[u][3]), pack_bf16(x[u][4], x[u][5]), pack_bf16(x[u][6], x[u][7]));
             }
-            if (live[u]) *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(a.pages[which[u]]) + dst) = v;
+            if (live[u]) __builtin_nontemporal_store(u32x4{v.x, v.y, v.z, v.w}, reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(a.pages[which[u]]) + dst));
         } else {
             float div;
             if constexpr (KIND == 1) {
@@ -165,7 +165,7 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
                     }
                 }
             }
-            if (live[u]) *reinterpret_cast<uint4*>(reinterpret_cast<uint8_t*>(a.pages[which[u]]) + dst) = make_uint4(w[0], w[1], w[2], w[3]);
+            if (live[u]) __builtin_nontemporal_store(u32x4{w[0], w[1], w[2], w[3]}, reinterpret_cast<u32x4*>(reinterpret_cast<uint8_t*>(a.pages[which[u]]) + dst));
         }
     }
 }

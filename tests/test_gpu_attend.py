@@ -346,3 +346,40 @@ def test_bad_geometry_is_refused():
         cache.attend(q, [0], [0], [99], 1, offsets=torch.zeros(1, dtype=torch.int32, device=dev))
     with pytest.raises(NotImplementedError):
         cache.attend(q, [0], [0], [99], 1, parents=torch.tensor([-1], device=dev))
+
+
+def test_launches_that_overlap_on_two_streams_do_not_share_counters():
+    # The split launch's workgroups pull their units from a counter pair the launch takes from a ring: launches in
+    # flight together (two streams here, many each) must not disturb one another, and every one must leave its pair
+    # zeroed for the launch that gets it next (130 launches go round the ring of 64 twice).
+    caches = [Cache("bf16", 4, 128, 128, 16, [3000, 1700, 900], seed=s) for s in (1, 2)]
+    qs = [rand_q(3, 16, 128, 20 + s) for s in range(2)]
+    want = [c.attend(q, [0, 1, 2], [0, 1, 2], [2999, 1699, 899], 1) for c, q in zip(caches, qs)]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(2)]
+    outs = [[], []]
+    for rep in range(65):
+        for i, stream in enumerate(streams):
+            with torch.cuda.stream(stream):
+                outs[i].append(caches[i].attend(qs[i], [0, 1, 2], [0, 1, 2], [2999, 1699, 899], 1))
+    torch.cuda.synchronize()
+    for i in range(2):
+        for got in outs[i]:
+            assert torch.equal(got, want[i])
+
+
+def test_more_units_than_resident_workgroups_and_ragged_rows():
+    # 96 rows of very different lengths over 8 KV heads: several thousand units for a few hundred resident
+    # workgroups, most of the list's (row, partition) slots empty; every row against its own launch, bit for bit.
+    g = torch.Generator().manual_seed(9)
+    lengths = [int(x) for x in torch.randint(1, 6000, (96,), generator=g)]
+    lengths[5], lengths[50] = 1, 5999
+    cache = Cache("fp8", 8, 128, 128, 16, lengths, seed=4)
+    q = rand_q(96, 32, 128, 6)
+    firsts = [n - 1 for n in lengths]
+    together = cache.attend(q, list(range(96)), list(range(96)), firsts, 1)
+    for s in (0, 5, 17, 50, 95):
+        alone = cache.attend(q[s:s + 1], [s], [0], [firsts[s]], 1)
+        assert torch.equal(alone[0], together[s]), s
+        want, _ = cache.want(q[s:s + 1].to(torch.bfloat16), s, firsts[s], 1)
+        _close(together[s:s + 1], want, s)

@@ -152,3 +152,24 @@ def test_what_the_prompt_reader_does_not_take_is_refused():
         pk.prefill(q, cache.k, cache.v, "int8", cache.tables[0], 36, 16, fresh=(q, q), **kw)
     with pytest.raises(ValueError):
         pk.prefill(q.float(), cache.k, cache.v, "int8", cache.tables[0], 36, 16, **kw)
+
+
+@pytest.mark.parametrize("n_chunks", [5, 70])
+def test_chunks_are_taken_in_any_order_with_equal_lengths_and_past_the_ranked_limit(n_chunks):
+    # Workgroups take the chunks longest first (ranked on the device for up to 64 chunks, ties by index; the caller's
+    # order beyond that): whatever the order, every chunk gets its own rows. Equal lengths make every rank a tie.
+    pk = kernels()
+    lengths = [40 + 16 * (i % 3) for i in range(n_chunks)]
+    lengths[1] = lengths[3] = lengths[0]
+    counts = [min(n, 24) for n in lengths]
+    cache = Cache("bf16", 2, 128, 128, 16, lengths, seed=3, scale=0.5)
+    starts = [sum(counts[:i]) for i in range(n_chunks)]
+    q = rand_q(sum(counts), 8, 128, 13).bfloat16()
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    positions = torch.tensor([n - c for n, c in zip(lengths, counts)], dtype=torch.int64, device=dev)
+    out = pk.prefill_rows(q, cache.k, cache.v, "bf16", cache.tables, i32(list(range(n_chunks))), i32(starts),
+                          i32(counts), positions, 32, 16)
+    for s in range(n_chunks):
+        one = pk.prefill(q[starts[s]:starts[s] + counts[s]], cache.k, cache.v, "bf16", cache.tables[s],
+                         lengths[s] - counts[s], 16)
+        assert torch.equal(out[starts[s]:starts[s] + counts[s]], one), s
