@@ -201,6 +201,8 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     const int sp = 4 * (64 / lpr);
     if (p->partitions < 1 || p->partitions > 65535 || p->piece < 1 || p->piece % sp) return CRIT_PKV_E_WORKSPACE;
     if (!p->fused && (!p->partial_out || !p->partial_max || !p->partial_sum)) return CRIT_PKV_E_WORKSPACE;
+    if (p->parents && p->parents64) return CRIT_PKV_E_NULL;
+    if ((p->parents || p->parents64) && p->columns > 64) return CRIT_PKV_E_GEOMETRY;      // an ancestor set is a 64-bit mask
     AttendArgs a;
     a.q = reinterpret_cast<const uint8_t*>(p->q);
     a.kp = reinterpret_cast<const uint8_t*>(p->key_pages);
@@ -210,6 +212,7 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     a.tables = p->tables, a.rows = p->rows, a.starts = p->starts, a.counts = p->counts, a.firsts = p->firsts, a.offsets = p->offsets;
     a.po = p->partial_out, a.pm = p->partial_max, a.pl = p->partial_sum;
     a.out = p->out, a.lse = p->lse, a.sinks = p->sinks;
+    a.parents = p->parents, a.parents64 = p->parents64;
     a.q_st = p->q_stride_t, a.q_sh = p->q_stride_h, a.o_st = p->out_stride_t, a.o_sh = p->out_stride_h, a.tab_stride = p->table_stride;
     a.tab_width = p->table_width, a.n_rows = p->n_rows, a.columns = p->columns, a.hq = p->heads, a.hkv = p->kv_heads;
     a.g = p->heads / p->kv_heads;

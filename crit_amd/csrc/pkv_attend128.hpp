@@ -167,6 +167,11 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
         const int c = j / a.g;
         my_lim[blk] = (4 * blk + 2 * b1 + b0 < QR && c < count) ? first + c : -1;
     }
+    // With a draft tree the window positions that row sees are those of its ancestors and itself.
+    const bool tree = a.parents != nullptr || a.parents64 != nullptr;
+    unsigned long long my_anc[RB];
+#pragma unroll
+    for (int blk = 0; blk < RB; ++blk) my_anc[blk] = (tree && my_lim[blk] >= 0) ? ancestors(a, start, my_lim[blk] - first) : 0ull;
     float k_mult = a.k_mult;
     if (KIND == 1 && a.hm) k_mult = a.hm[kvh];
     const float sscale = a.sscale * (KIND == 1 ? k_mult : 1.0f);
@@ -321,6 +326,7 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
                 const int n = base + soff;
                 x *= KIND >= 2 ? sscale * buf.ks : sscale;
                 bool vis = n <= my_lim[blk] && n < n_keys;
+                if (tree) vis = vis && (n < first || ((my_anc[blk] >> ((n - first) & 63)) & 1ull) != 0);
                 if (win > 0) vis = vis && n > my_lim[blk] - win;
                 x = vis ? x : -INFINITY;
                 float top = __builtin_fmaxf(x, dpp<kRor4>(x));

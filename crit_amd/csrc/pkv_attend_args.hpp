@@ -25,10 +25,27 @@ struct AttendArgs {
     void* out;
     float* lse;
     const float* sinks;
+    const int32_t* parents;      // draft trees: each token's parent column, int32 ...
+    const int64_t* parents64;    // ... or int64; both null: plain causal windows
     unsigned* ticket;      // two zeroed counters of the unit-pulling launches: next unit, workgroups done
     int64_t q_st, q_sh, o_st, o_sh, tab_stride;
     int tab_width, n_rows, columns, hq, hkv, g, page, page_shift, parts, piece, sliding, out_dtype, tiles, max_keys, heads_per_wave, units_x, units_y;
     float sscale, k_mult, v_mult;
 };
+
+// Draft trees: the set of window columns column `c` of the row whose first token is `start` sees (its ancestors and
+// itself) as a 64-bit mask, by walking the parent links (parents come before children, so at most c links; a link that
+// does not point at an earlier column ends the walk).
+PKV_DEV unsigned long long ancestors(const AttendArgs& a, int start, int c) {
+    unsigned long long set = 1ull << c;
+    int at = c;
+    for (int hop = 0; hop < 64 && at > 0; ++hop) {
+        const int64_t par = a.parents ? (int64_t)a.parents[start + at] : a.parents64[start + at];
+        if (par < 0 || par >= at) break;
+        at = (int)par;
+        set |= 1ull << at;
+    }
+    return set;
+}
 
 }   // namespace pkv

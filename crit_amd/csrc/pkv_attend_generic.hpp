@@ -68,6 +68,11 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
         live[rr] = col[rr] < count;
         lim[rr] = first + col[rr];
     }
+    // With a draft tree the window positions a row sees are those of its ancestors and itself.
+    const bool tree = a.parents != nullptr || a.parents64 != nullptr;
+    unsigned long long anc[QR];
+#pragma unroll
+    for (int rr = 0; rr < QR; ++rr) anc[rr] = (tree && live[rr]) ? ancestors(a, start, col[rr]) : 0ull;
     // The lane's slice of each query row: packed 16-bit pairs for 16-bit pages, FP32 for 8-bit pages.
     uint32_t qp[QR][4];
     float qf[KIND == 0 ? 1 : QR][8];
@@ -201,6 +206,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
                     const int n = base + k * PPI + lg;
                     float x = s[k][rr] * (KIND >= 2 ? sscale * buf.ks[k] : sscale);
                     bool vis = n <= lim[rr] && n < n_keys;
+                    if (tree) vis = vis && (n < first || ((anc[rr] >> ((n - first) & 63)) & 1ull) != 0);
                     if (win > 0) vis = vis && n > lim[rr] - win;
                     x = vis ? x : -INFINITY;
                     s[k][rr] = x;

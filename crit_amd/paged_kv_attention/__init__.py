@@ -327,12 +327,20 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
     flash (True or "cuda"): contiguous splits of `chunk` positions (default flash_chunk()), one per partition.
     sinks: FP32 [heads] sink logits folded into each row's final state; sliding: a sliding window in positions.
     multipliers: an "fp8" layer's (key, value) multipliers, or a [2][kv_heads] FP32 tensor (one per KV head).
-    parents, blocks, fresh and derive are not served. phases (a measurement's): 1 runs the split launch only, 2 the
+    parents: draft trees, one int32 or int64 per token of q: its parent's column in its row's window, -1 for none,
+    parents before children; a column then sees every position below its row's first and, of the window, its ancestors'
+    positions and its own (a chain -1, 0, 1, ... is the plain causal window, bit for bit).
+    blocks, fresh and derive are not served. phases (a measurement's): 1 runs the split launch only, 2 the
     merge only."""
     if derive is not None:
         raise _unsupported("derive= (keys derived from value rows)")
     if parents is not None:
-        raise _unsupported("parents= (draft trees)")
+        _require_device(parents, "attend's parents")
+        parents = parents.reshape(-1)
+        if parents.dtype not in (torch.int32, torch.int64) or parents.stride(0) != 1 or parents.numel() < q.shape[0]:
+            raise ValueError("parents holds one int32 or int64 parent column per token of q, contiguous")
+        if int(columns) > 64:
+            raise ValueError("a draft tree's row has at most 64 columns (a column's ancestors are a 64-bit set)")
     if blocks is not None:
         raise _unsupported("blocks= (block-sparse lists)")
     if fresh is not None:
@@ -392,6 +400,8 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
     p.firsts, p.offsets = firsts.data_ptr(), _ptr(offsets)
     p.partial_out, p.partial_max, p.partial_sum = _ptr(po), _ptr(pm), _ptr(pl)
     p.out, p.lse, p.sinks = out.data_ptr(), _ptr(lse), _ptr(sinks)
+    if parents is not None:
+        p.parents, p.parents64 = (parents.data_ptr(), None) if parents.dtype == torch.int32 else (None, parents.data_ptr())
     p.q_stride_t, p.q_stride_h, p.out_stride_t, p.out_stride_h = q.stride(0), q.stride(1), out.stride(0), out.stride(1)
     p.table_stride, p.table_width = tables.stride(0), tables.shape[1]
     p.n_rows, p.columns, p.heads, p.kv_heads, p.head_dim, p.value_dim, p.page = R, int(columns), hq, hkv, d, dv, int(page)

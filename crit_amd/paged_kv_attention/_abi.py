@@ -10,7 +10,7 @@ import shutil
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 NAME = "libcrit_pkv.so"
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 KIND_16BIT, KIND_FP8, KIND_FP8_ROW, KIND_INT8 = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
@@ -31,7 +31,7 @@ class AttendParams(ctypes.Structure):
     _fields_ = [("q", _p), ("key_pages", _p), ("value_pages", _p), ("key_scales", _p), ("value_scales", _p),
                 ("head_multipliers", _p), ("tables", _p), ("rows", _p), ("starts", _p), ("counts", _p), ("firsts", _p),
                 ("offsets", _p), ("partial_out", _p), ("partial_max", _p), ("partial_sum", _p), ("out", _p),
-                ("lse", _p), ("sinks", _p),
+                ("lse", _p), ("sinks", _p), ("parents", _p), ("parents64", _p),
                 ("q_stride_t", _i64), ("q_stride_h", _i64), ("out_stride_t", _i64), ("out_stride_h", _i64),
                 ("table_stride", _i64),
                 ("table_width", _i32), ("n_rows", _i32), ("columns", _i32), ("heads", _i32), ("kv_heads", _i32),

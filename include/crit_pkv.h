@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 1
+#define CRIT_PKV_ABI_VERSION 2
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -99,6 +99,12 @@ typedef struct crit_pkv_attend_params {
     void* out;                      /* [tokens][heads][value_dim], out_dtype */
     float* lse;                     /* [tokens][heads] or NULL */
     const float* sinks;             /* [heads] or NULL */
+    const int32_t* parents;         /* draft trees (_kernels.py:155-165, 325-329): [tokens] int32 ... */
+    const int64_t* parents64;       /* ... or int64 (at most one of the two non-NULL): token starts[r] + c holds the
+                                       column of its parent in row r's window, -1 for none, parents before children.
+                                       Column c then sees every position below firsts[r] and, of the window, the
+                                       positions firsts[r] + a of its ancestors a and itself. NULL, NULL: column c
+                                       sees positions <= firsts[r] + c. */
     int64_t q_stride_t, q_stride_h, out_stride_t, out_stride_h, table_stride;
     int32_t table_width, n_rows, columns, heads, kv_heads, head_dim, value_dim, page;
     int32_t kind, page_dtype, out_dtype;

@@ -45,19 +45,35 @@ def stored_rows(key_pages, value_pages, table, n, page, kind, key_scales=None, v
     return (append.decode_rows(k, ks, kind, multipliers[0]), append.decode_rows(v, vs, kind, multipliers[1]))
 
 
+def seen_by(first, count, c, n, parents=None, sliding=0):
+    """Which of positions 0 .. n - 1 column c of a window row at `first` sees (_kernels.py:325-333): without parents
+    the positions <= first + c; with parents (each column's parent column, -1 for none, parents before children)
+    every position below first and, of the window, the positions of c's ancestors and c's own. A sliding window of w
+    positions drops positions <= first + c - w either way."""
+    positions = torch.arange(n)
+    if parents is None:
+        seen = positions <= first + c
+    else:
+        mine, at = {c}, int(parents[c])
+        while at >= 0:
+            mine.add(at)
+            at = int(parents[at])
+        seen = torch.tensor([p < first or (p - first) in mine for p in range(n)], dtype=torch.bool)
+    if sliding:
+        seen = seen & (positions > first + c - sliding)
+    return seen
+
+
 def window_reference(q, key_pages, value_pages, kind, table, first, count, page, scale, key_scales=None,
-                     value_scales=None, multipliers=(1.0, 1.0), sliding=0, q_dtype=torch.bfloat16):
+                     value_scales=None, multipliers=(1.0, 1.0), sliding=0, q_dtype=torch.bfloat16, parents=None):
     """One window row in float64: q [count][HQ][D] (rounded to q_dtype first, as the kernels read it) at positions
-    first .. first + count - 1 -> (out [count][HQ][DV], lse [count][HQ])."""
+    first .. first + count - 1 -> (out [count][HQ][DV], lse [count][HQ]). parents: the row's draft tree (seen_by)."""
     n = first + count
     keys, values = stored_rows(key_pages, value_pages, table, n, page, kind, key_scales, value_scales, multipliers)
     qd = q.to(q_dtype).double()
-    positions = torch.arange(n)
     outs, lses = [], []
     for c in range(count):
-        seen = positions <= first + c
-        if sliding:
-            seen = seen & (positions > first + c - sliding)
+        seen = seen_by(first, count, c, n, parents, sliding)
         o, l = reference(qd[c], keys, values, seen, scale)
         outs.append(o)
         lses.append(l)

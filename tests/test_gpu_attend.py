@@ -345,7 +345,7 @@ def test_bad_geometry_is_refused():
     with pytest.raises(ValueError, match="offsets"):
         cache.attend(q, [0], [0], [99], 1, offsets=torch.zeros(1, dtype=torch.int32, device=dev))
     with pytest.raises(NotImplementedError):
-        cache.attend(q, [0], [0], [99], 1, parents=torch.tensor([-1], device=dev))
+        cache.attend(q, [0], [0], [99], 1, blocks=torch.zeros(1, 1, dtype=torch.int32, device=dev), block_size=16)
 
 
 def test_launches_that_overlap_on_two_streams_do_not_share_counters():
@@ -383,3 +383,33 @@ def test_more_units_than_resident_workgroups_and_ragged_rows():
         assert torch.equal(alone[0], together[s]), s
         want, _ = cache.want(q[s:s + 1].to(torch.bfloat16), s, firsts[s], 1)
         _close(together[s:s + 1], want, s)
+
+
+@pytest.mark.parametrize("kind,hq,hkv,d,page", [("bf16", 8, 2, 128, 16), ("int8", 8, 2, 128, 16), ("fp8", 32, 8, 128, 16),
+                                                 ("bf16", 12, 2, 64, 16), ("fp8:row", 8, 2, 128, 48)])
+def test_a_tree_sees_its_ancestors_and_a_chain_is_causal(kind, hq, hkv, d, page):
+    # the reference's tree test (tests/test_cuda.py:110-129, tests/test_flash.py:74-92)
+    cache = Cache(kind, hkv, d, d, page, [400, 300])
+    parents = torch.tensor([-1, 0, 0, 1, 1, 2, 5, 3], dtype=torch.int64, device=dev)
+    q = rand_q(8, hq, d, 6)
+    out = cache.attend(q, [0], [0], [392], 8, parents=parents)
+    want, _ = cache.want(q.to(torch.bfloat16), 0, 392, 8, parents=parents.tolist())
+    _close(out, want)
+    chain = cache.attend(q, [0], [0], [392], 8, parents=torch.arange(-1, 7, device=dev))
+    assert torch.equal(chain, cache.attend(q, [0], [0], [392], 8))
+    assert not torch.equal(chain, out)
+    assert torch.equal(cache.attend(q, [0], [0], [392], 8, parents=parents.int(), fused=True), out)
+    assert torch.equal(cache.attend(q, [0], [0], [392], 8, parents=parents, flash=True, chunk=128),
+                       cache.attend(q, [0], [0], [392], 8, parents=parents, flash=True, chunk=128, fused=True))
+    # two rows in one launch, the second a shorter tree behind the first row's tokens: each as alone
+    both = torch.cat([parents, torch.tensor([-1, 0, 1, 1, 0], dtype=torch.int64, device=dev)])
+    q2 = rand_q(13, hq, d, 7)
+    together = cache.attend(q2, [0, 1], [0, 8], [392, 295], 8, parents=both,
+                            counts=torch.tensor([8, 5], dtype=torch.int32, device=dev))
+    alone = cache.attend(q2[8:13], [1], [0], [295], 8, parents=both[8:13].contiguous(),
+                         counts=torch.tensor([5], dtype=torch.int32, device=dev))
+    assert torch.equal(together[8:13], alone)
+    want2, _ = cache.want(q2[8:13].to(torch.bfloat16), 1, 295, 5, parents=both[8:13].tolist())
+    _close(together[8:13], want2)
+    with pytest.raises(ValueError):
+        cache.attend(q, [0], [0], [392], 8, parents=parents.float())

@@ -356,3 +356,31 @@ def test_merged_shards_equal_attention_over_the_whole_whatever_the_cut(cut):
     b = attend.reference(q, keys[cut:], values[cut:], every[cut:], 0.125)
     out, lse = attend.merge([a[0][None].float(), b[0][None].float()], [a[1][None].float(), b[1][None].float()])
     assert torch.allclose(out[0].double(), want, atol=1e-5) and torch.allclose(lse[0].double(), want_lse, atol=1e-5)
+
+
+def test_a_draft_tree_column_sees_what_its_path_alone_would_hold():
+    # Pins seen_by(): the reference's tree of its own tests (tests/test_cuda.py:113) against an independent statement
+    # of the rule. A column's attention over the tree equals plain causal attention over a sequence that holds the
+    # prefix and then only the column's path (root .. column) at consecutive positions, which is what the reference's
+    # pool makes of an accepted path (pages.py:662-684); a chain is the causal window; a star sees the root and itself.
+    k, v, ks, vs, tables, _ = _pool("bf16", 1, 16, 16, 16, [48])
+    q = torch.randn(8, 2, 16, generator=torch.Generator().manual_seed(5))
+    parents = [-1, 0, 0, 1, 1, 2, 5, 3]
+    first = 40
+    out, lse = attend.window_reference(q, k, v, "bf16", tables[0], first, 8, 16, 0.25, parents=parents)
+    keys, values = attend.stored_rows(k, v, tables[0], 48, 16, "bf16")
+    paths = {0: [0], 1: [0, 1], 2: [0, 2], 3: [0, 1, 3], 4: [0, 1, 4], 5: [0, 2, 5], 6: [0, 2, 5, 6], 7: [0, 1, 3, 7]}
+    for c, path in paths.items():
+        index = torch.tensor(list(range(first)) + [first + a for a in path])
+        want, want_lse = attend.reference(q[c].bfloat16().double(), keys[index], values[index],
+                                          torch.ones(len(index), dtype=torch.bool), 0.25)
+        assert torch.allclose(out[c], want, atol=1e-12, rtol=1e-12), c
+        assert torch.allclose(lse[c], want_lse, atol=1e-12, rtol=1e-12), c
+        assert attend.seen_by(first, 8, c, 48, parents).sum() == first + len(path)
+    chain, _ = attend.window_reference(q, k, v, "bf16", tables[0], first, 8, 16, 0.25, parents=list(range(-1, 7)))
+    plain, _ = attend.window_reference(q, k, v, "bf16", tables[0], first, 8, 16, 0.25)
+    assert torch.equal(chain, plain)
+    star = attend.seen_by(first, 8, 5, 48, [-1, 0, 0, 0, 0, 0, 0, 0])
+    assert star.nonzero().flatten().tolist() == list(range(first)) + [first, first + 5]
+    slid = attend.seen_by(first, 8, 6, 48, parents, sliding=3)       # positions > 40 + 6 - 3 of the path 0, 2, 5, 6
+    assert slid.nonzero().flatten().tolist() == [first + 5, first + 6]
