@@ -27,7 +27,7 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, vendor figure
 # HBM bytes one split launch moves, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this file (each counter in
 # a run of its own, scaled by what it reads for the stream-read probe and for a 262,144-token append, kernels of
 # known size: factors 0.5000 and 1.000). Measured for the default workload only.
-MEASURED_TRAFFIC_BYTES = {"c2": 1_436_963_942}
+MEASURED_TRAFFIC_BYTES = {"c2": 1_437_029_273}
 
 
 def log(*a):
@@ -307,6 +307,8 @@ def main():
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run only the mixed prefill + decode batch of the extras (for counter runs on prefill_kernel)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch one KV append of 262,144 tokens: with the stream-read probe, two kernels of known "
                          "read and write sizes against which FETCH_SIZE / WRITE_SIZE counters are scaled")
@@ -318,6 +320,11 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     import crit_amd.paged_kv_attention as pk
+    if args.prefill_only:
+        found = mixed_prefill(pk, device)
+        log(f"[bench] mixed prefill + decode: {found}")
+        print(json.dumps({"mixed_prefill_decode_bf16": found}), flush=True)
+        return
     spec = WORKLOADS[args.workload]
     log(f"[bench] building workload {args.workload}: {spec['name']}")
     w = Workload(spec, device)
