@@ -41,13 +41,15 @@ def test_writes_encode_as_torch_does_and_skip_negative_slots(kind, d, dv, in_dty
     _check(kind, (k, v, ks, vs), expected_pages(kind, keys, values, slots, 64, mult))
 
 
+@pytest.mark.parametrize("T", [4152, 33001])
 @pytest.mark.parametrize("kind", ["bf16", "fp8", "fp8:row", "int8"])
-def test_a_large_append_with_edge_values_is_bit_exact(kind):
-    # 4,152 tokens (the mixed prefill + decode batch's append), 8 KV heads, with the values that break sloppy
-    # encoders: signed zeros, the subnormal ties, saturation, infinities, 1% outliers x20.
+def test_a_large_append_with_edge_values_is_bit_exact(kind, T):
+    # 4,152 tokens (the mixed prefill + decode batch's append) and 33,001 (a launch large enough for the kernel that
+    # gives a thread four rows; an odd count, so its last workgroups are ragged), 8 KV heads, with the values that
+    # break sloppy encoders: signed zeros, the subnormal ties, saturation, infinities, 1% outliers x20.
     pk = kernels()
     g = torch.Generator().manual_seed(2)
-    T, hkv, d = 4152, 8, 128
+    hkv, d = 8, 128
     keys, values = torch.randn(T, hkv, d, generator=g), torch.randn(T, hkv, d, generator=g)
     hot = torch.rand(T, hkv, d, generator=g) < 0.01
     keys = torch.where(hot, keys * 20, keys)
@@ -56,7 +58,7 @@ def test_a_large_append_with_edge_values_is_bit_exact(kind):
                          float("inf"), float("-inf"), 1e-30, 0.0146484375, 432.0, 248.0])
     keys[0, 0, :16] = edge * mult[0]
     values[1, 2, :16] = edge * mult[1]
-    n_slots = 8192
+    n_slots = 8192 if T < 8192 else 40000
     slots = torch.randperm(n_slots, generator=g)[:T]
     slots[100] = -1
     slots[4000] = -5
