@@ -91,12 +91,6 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
             qreg[ks] = *reinterpret_cast<const uint4*>(a.q + ((int64_t)(start + t) * a.q_st + (int64_t)head * a.q_sh + 16 * ks + 8 * h) * 2);
         }
     }
-    if (a.sscale < 0.0f && KIND < 2) {      // a negative scale: its sign goes into the queries, |scale| into the exponent
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            qreg[ks].x ^= 0x80008000u, qreg[ks].y ^= 0x80008000u, qreg[ks].z ^= 0x80008000u, qreg[ks].w ^= 0x80008000u;
-        }
-    }
     // The lowest limit among the wavefront's live rows: key blocks wholly at or below it need no mask.
     int wave_lo = live ? lim : 0x7fffffff;
 #pragma unroll
@@ -108,6 +102,12 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
     if (KIND != 1) v_mult = 1.0f;
     const int win = a.sliding;
     const float sabs = __builtin_fabsf(sscale);
+    if (sscale < 0.0f && KIND < 2) {      // a negative scale: its sign goes into the queries, |scale| into the exponent
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            qreg[ks].x ^= 0x80008000u, qreg[ks].y ^= 0x80008000u, qreg[ks].z ^= 0x80008000u, qreg[ks].w ^= 0x80008000u;
+        }
+    }
 
     const int t_lo = tile * BM / a.g;
     const int t_hi = min(count - 1, (tile * BM + BM - 1) / a.g);
@@ -335,7 +335,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
         static_for<RING - 1>([&](auto ic) __attribute__((always_inline)) { read_v(vl, ic, va[decltype(ic)::value]); });
         PKV_SB();
         // Mask where the block is not wholly visible; the lane holds keys 32 kb + 8 (v / 4) + 4 h + v % 4 of its own
-        // row. With one scale for all keys (sscale > 0 after the sign went into the scores) the maximum is taken over
+        // row. With one scale for all keys (positive once its sign went into the queries) the maximum is taken over
         // the raw scores and the scale rides on the exponent's fused multiply-add; with per-key scales (row-scaled
         // pages) each score is scaled first.
         if constexpr (KIND >= 2) {

@@ -27,16 +27,11 @@ struct PrefillArgs {
     float sscale, k_mult, v_mult;
 };
 
-#ifndef PKV_NO_PRIO
+// A wavefront raises its priority while it issues matrix instructions, so the other wavefront of its SIMD fills the
+// gaps with vector work instead of delaying them.
 #define PKV_PRIO(x) __builtin_amdgcn_s_setprio(x)
-#else
-#define PKV_PRIO(x)
-#endif
-#ifdef PKV_NO_SB
-#define PKV_SB()
-#else
+// Nothing is scheduled across this point: it fixes the order of the phases the kernel lays out by hand.
 #define PKV_SB() __builtin_amdgcn_sched_barrier(0)
-#endif
 // The running maximum a row's exponentials are taken against moves only when a block's maximum exceeds it by more
 // than this (in log2 units): probabilities then reach 2^8 at most, far inside the range of the 16-bit operand and the
 // FP32 sums, the final division by the row's sum (taken against the same reference) cancels the factor, and the

@@ -173,3 +173,20 @@ def test_chunks_are_taken_in_any_order_with_equal_lengths_and_past_the_ranked_li
         one = pk.prefill(q[starts[s]:starts[s] + counts[s]], cache.k, cache.v, "bf16", cache.tables[s],
                          lengths[s] - counts[s], 16)
         assert torch.equal(out[starts[s]:starts[s] + counts[s]], one), s
+
+
+@pytest.mark.parametrize("kind", ["bf16", "fp8", "fp8:row"])
+def test_a_negative_or_large_scale_and_a_far_running_maximum(kind):
+    # A negative softmax scale (its sign goes into the queries for pages with one scale, into the per-key scales
+    # otherwise) and a scale large enough that a row's maximum moves by far more than the slack between key blocks.
+    pk = kernels()
+    cache = Cache(kind, 2, 128, 128, 16, [300])
+    q = rand_q(70, 8, 128, 21)
+    for scale in (-0.09, 0.9):
+        lse = torch.empty(70, 8, device=dev)
+        out = pk.prefill(q.bfloat16(), cache.k, cache.v, kind, cache.tables[0], 230, 16, key_scales=cache.ks,
+                         value_scales=cache.vs, multipliers=cache.multipliers, lse=lse, scale=scale)
+        for t in (0, 33, 69):
+            want, want_lse = cache.want(q[t:t + 1], 0, 230 + t, 1, scale=scale)
+            torch.testing.assert_close(out[t:t + 1].double().cpu(), want, atol=ATOL, rtol=RTOL, msg=f"{scale} token {t}")
+            torch.testing.assert_close(lse[t:t + 1].double().cpu(), want_lse, atol=2e-3, rtol=1e-4, msg=f"{scale} lse {t}")
