@@ -17,23 +17,21 @@
 
 namespace pkv {
 
-// 8 codes (two words of E4M3 or INT8) -> 8 BF16 values packed in a uint4, exactly.
-template <int KIND>
-PKV_DEV uint4 codes_to_bf16(uint32_t w0, uint32_t w1) {
-    float f[8];
+// Two codes (bytes 0,1 or 2,3 of a word of E4M3 or INT8 codes) -> two BF16 values in one word, exactly.
+template <int KIND, bool HI>
+PKV_DEV uint32_t code_pair(uint32_t w) {
     if constexpr (KIND == 3) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) f[j] = (float)(int8_t)(w0 >> (8 * j)), f[4 + j] = (float)(int8_t)(w1 >> (8 * j));
+        const float f0 = (float)(int8_t)(w >> (HI ? 16 : 0)), f1 = (float)(int8_t)(w >> (HI ? 24 : 8));
+        return __builtin_amdgcn_perm(f2u(f1), f2u(f0), 0x07060302u);
     } else {
-        const f32x2 a0 = e4m3_pair<false>(w0), a1 = e4m3_pair<true>(w0), a2 = e4m3_pair<false>(w1), a3 = e4m3_pair<true>(w1);
-        f[0] = a0.x, f[1] = a0.y, f[2] = a1.x, f[3] = a1.y, f[4] = a2.x, f[5] = a2.y, f[6] = a3.x, f[7] = a3.y;
+        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)w, 1.0f, HI));
     }
-    uint4 r;
-    r.x = (f2u(f[0]) >> 16) | (f2u(f[1]) & 0xffff0000u);
-    r.y = (f2u(f[2]) >> 16) | (f2u(f[3]) & 0xffff0000u);
-    r.z = (f2u(f[4]) >> 16) | (f2u(f[5]) & 0xffff0000u);
-    r.w = (f2u(f[6]) >> 16) | (f2u(f[7]) & 0xffff0000u);
-    return r;
+}
+
+// 8 codes (two words) -> 8 BF16 values packed in a uint4, exactly.
+template <int KIND>
+PKV_DEV u32x4 codes_to_bf16(uint32_t w0, uint32_t w1) {
+    return u32x4{code_pair<KIND, false>(w0), code_pair<KIND, true>(w0), code_pair<KIND, false>(w1), code_pair<KIND, true>(w1)};
 }
 
 template <bool F16>
@@ -53,9 +51,10 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
     constexpr int EB = KIND == 0 ? 2 : 1;
     constexpr int CH = D * EB / 16;     // 16-byte chunks of one K or V row in the pages
     constexpr int KPASS = BN * CH / 256;   // passes of 256 threads over a K block, rows contiguous over lanes
-    constexpr int VGROUPS = 16 * CH;    // 16-bit pages: (group of four keys, 16-byte chunk) pairs of a V block
-    constexpr int VGP = (VGROUPS + 255) / 256;
-    constexpr int VPASS = KIND == 0 ? 4 * VGP : CH / 4;
+    // V staging: a thread takes 8 dims (one 16-byte chunk of 16-bit pages, half a chunk of 8-bit ones) of four adjacent
+    // keys; D / 8 such pieces a key, 16 groups of four keys a block.
+    constexpr int VC = D / 8;           // 8-dim pieces of one V row
+    constexpr int VGROUPS = 16 * VC;    // (group of four keys, 8-dim piece) pairs of a V block: 256 (D = 128) or 128
     __shared__ __align__(16) uint16_t k_lds[2][BN * KSTR];
     __shared__ __align__(16) uint16_t v_lds[2][D * BN];
     __shared__ float ks_lds[2][BN], vs_lds[2][BN];
@@ -127,11 +126,11 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
     const uint32_t slot_bytes = (uint32_t)a.hkv * D * EB;
     const uint8_t* kbase = a.kp + (int64_t)kvh * D * EB;
     const uint8_t* vbase = a.vp + (int64_t)kvh * D * EB;
-    // Global -> registers -> LDS. K: rows contiguous over lanes. V, 16-bit pages: a thread takes one 16-byte chunk of
-    // four adjacent keys and stores it transposed as eight 8-byte groups; 8-bit pages: lane = key, wavefront = chunk.
+    // Global -> registers -> LDS. K: rows contiguous over lanes. V: a thread takes eight dims of four adjacent keys and
+    // stores them transposed as eight 8-byte groups (8-bit codes become 16-bit values on the way, exactly).
     // The page table entries of a block are fetched one block before its rows (load_entries, then take_slots, then load_k and load_v): a
     // row's address depends on its entry, and a wait on an entry would also wait on every row load issued before it.
-    u32x4 kreg[KPASS], vreg[VPASS];
+    u32x4 kreg[KPASS], vreg[4];      // vreg[i]: key 4 kg + i; 8-bit pages fill .x and .y only
     int ent = 0, inp = 0;
     float ksreg = 1.0f, vsreg = 1.0f;
     auto load_entries = [&](int kt) __attribute__((always_inline)) {
@@ -145,7 +144,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
     // take_slots turns the entries into slots and hands every thread the slots of its rows; it runs during the second
     // product of the iteration before the loads that use them, so the exchange's latency passes behind the products
     // and load_k / load_v issue their row loads back to back.
-    constexpr int NROW = KPASS + (KIND == 0 ? 4 : 0);
+    constexpr int NROW = KPASS + 4;
     uint32_t rowslot[NROW], myslot = 0;
     auto take_slots = [&]() __attribute__((always_inline)) {
         myslot = (uint32_t)ent * (uint32_t)a.page + (uint32_t)inp;
@@ -153,13 +152,11 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
             constexpr int p = decltype(pc)::value;
             rowslot[p] = (uint32_t)__builtin_amdgcn_ds_bpermute(((p * 256 + tid) / CH) << 2, (int)myslot);
         });
-        if constexpr (KIND == 0) {
-            const int kg = tid % VGROUPS / CH;      // D = 64: the upper half of the workgroup repeats the lower
-            static_for<4>([&](auto ic) __attribute__((always_inline)) {
-                constexpr int i = decltype(ic)::value;
-                rowslot[KPASS + i] = (uint32_t)__builtin_amdgcn_ds_bpermute((4 * kg + i) << 2, (int)myslot);
-            });
-        }
+        const int kg = tid % VGROUPS / VC;      // D = 64: the upper half of the workgroup repeats the lower
+        static_for<4>([&](auto ic) __attribute__((always_inline)) {
+            constexpr int i = decltype(ic)::value;
+            rowslot[KPASS + i] = (uint32_t)__builtin_amdgcn_ds_bpermute((4 * kg + i) << 2, (int)myslot);
+        });
     };
     auto load_k = [&]() __attribute__((always_inline)) {
         const uint8_t* kthread = kbase + (tid % CH) * 16;
@@ -172,19 +169,17 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
         }
     };
     auto load_v = [&]() __attribute__((always_inline)) {
-        if constexpr (KIND == 0) {
-            const uint8_t* vthread = vbase + (tid % VGROUPS % CH) * 16;
-            static_for<4>([&](auto ic) __attribute__((always_inline)) {
-                constexpr int i = decltype(ic)::value;
-                vreg[i] = *reinterpret_cast<const u32x4*>(vthread + (uint64_t)rowslot[KPASS + i] * slot_bytes);
-            });
-        } else {
-            const uint8_t* vrow = vbase + (uint64_t)myslot * slot_bytes;
-            static_for<VPASS>([&](auto pc) __attribute__((always_inline)) {
-                constexpr int p = decltype(pc)::value;
-                vreg[p] = *reinterpret_cast<const u32x4*>(vrow + (4 * p + wave) * 16);
-            });
-        }
+        const uint8_t* vthread = vbase + (tid % VGROUPS % VC) * (8 * EB);
+        static_for<4>([&](auto ic) __attribute__((always_inline)) {
+            constexpr int i = decltype(ic)::value;
+            const uint8_t* row = vthread + (uint64_t)rowslot[KPASS + i] * slot_bytes;
+            if constexpr (KIND == 0) {
+                vreg[i] = *reinterpret_cast<const u32x4*>(row);
+            } else {
+                const u32x2 w = *reinterpret_cast<const u32x2*>(row);
+                vreg[i].x = w.x, vreg[i].y = w.y;
+            }
+        });
     };
     auto store_k = [&](int buf) __attribute__((always_inline)) {
         uint16_t* kl = k_lds[buf];
@@ -195,8 +190,10 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
             if constexpr (KIND == 0) {
                 *reinterpret_cast<u32x4*>(&kl[kk * KSTR + c * 8]) = kreg[p];
             } else {
-                *reinterpret_cast<uint4*>(&kl[kk * KSTR + c * 16]) = codes_to_bf16<KIND>(kreg[p].x, kreg[p].y);
-                *reinterpret_cast<uint4*>(&kl[kk * KSTR + c * 16 + 8]) = codes_to_bf16<KIND>(kreg[p].z, kreg[p].w);
+                *reinterpret_cast<u32x4*>(&kl[kk * KSTR + c * 16]) = codes_to_bf16<KIND>(kreg[p].x, kreg[p].y);
+                PKV_SB();      // one 16-byte group converted and stored at a time keeps the conversions' temporaries few
+                *reinterpret_cast<u32x4*>(&kl[kk * KSTR + c * 16 + 8]) = codes_to_bf16<KIND>(kreg[p].z, kreg[p].w);
+                PKV_SB();
             }
         });
         if constexpr (KIND >= 2) {
@@ -204,43 +201,33 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
         }
     };
     auto store_v = [&](int buf) __attribute__((always_inline)) {
-        uint16_t* vl = v_lds[buf];
-        if constexpr (KIND == 0) {
-            static_for<VGP>([&](auto pc) __attribute__((always_inline)) {
-                constexpr int p = decltype(pc)::value;
-                const int idx = (p * 256 + tid) % VGROUPS;      // repeated groups store the same bytes twice
-                const int kg = idx / CH, c = idx % CH;
-                const uint32_t w0[4] = {vreg[4 * p].x, vreg[4 * p].y, vreg[4 * p].z, vreg[4 * p].w};
-                const uint32_t w1[4] = {vreg[4 * p + 1].x, vreg[4 * p + 1].y, vreg[4 * p + 1].z, vreg[4 * p + 1].w};
-                const uint32_t w2[4] = {vreg[4 * p + 2].x, vreg[4 * p + 2].y, vreg[4 * p + 2].z, vreg[4 * p + 2].w};
-                const uint32_t w3[4] = {vreg[4 * p + 3].x, vreg[4 * p + 3].y, vreg[4 * p + 3].z, vreg[4 * p + 3].w};
-                // row 8 c + i, group kg ^ swz(row): byte offset (1024 c + 8 (kg ^ c)) ^ (16 i), plus 128 i
-                uint8_t* vb = reinterpret_cast<uint8_t*>(vl);
-                const uint32_t v_write = 1024u * (uint32_t)c + 8u * (uint32_t)(kg ^ c);
+        // The thread's four keys x eight dims as 16-bit pairs of adjacent dims (8-bit codes converted, exactly), then
+        // transposed: dim row 8 c + i gets the four keys' values as one 8-byte group at group kg ^ swz(row), byte
+        // offset (1024 c + 8 (kg ^ c)) ^ (16 i), plus 128 i.
+        const int idx = tid % VGROUPS;      // repeated pairs store the same bytes twice
+        const int kg = idx / VC, c = idx % VC;
+        uint8_t* vb = reinterpret_cast<uint8_t*>(v_lds[buf]);
+        const uint32_t v_write = 1024u * (uint32_t)c + 8u * (uint32_t)(kg ^ c);
+        static_for<4>([&](auto jc) __attribute__((always_inline)) {
+            constexpr int j = decltype(jc)::value;      // dims 2 j and 2 j + 1 of the thread's eight
+            uint32_t w[4];
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
-                    const uint32_t k01 = __builtin_amdgcn_perm(w1[i / 2], w0[i / 2], sel);
-                    const uint32_t k23 = __builtin_amdgcn_perm(w3[i / 2], w2[i / 2], sel);
-                    *reinterpret_cast<u32x2*>(vb + (v_write ^ (16u * i)) + 128 * i) = u32x2{k01, k23};
+            for (int k = 0; k < 4; ++k) {
+                if constexpr (KIND == 0) {
+                    w[k] = vreg[k][j];
+                } else {
+                    w[k] = code_pair<KIND, j % 2 == 1>(vreg[k][j / 2]);
                 }
-            });
-        } else {
-            static_for<VPASS>([&](auto pc) __attribute__((always_inline)) {
-                constexpr int p = decltype(pc)::value;
-                const int c = 4 * p + wave;
-                const uint4 lo = codes_to_bf16<KIND>(vreg[p].x, vreg[p].y), hi = codes_to_bf16<KIND>(vreg[p].z, vreg[p].w);
-                const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            }
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-#pragma unroll
-                    for (int half = 0; half < 2; ++half) {
-                        const int row = c * 16 + 2 * i + half;
-                        vl[row * BN + 4 * ((lane >> 2) ^ swz(row)) + (lane & 3)] = (uint16_t)(half ? w[i] >> 16 : w[i] & 0xffffu);
-                    }
-                }
-            });
-        }
+            for (int i = 2 * j; i < 2 * j + 2; ++i) {
+                const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
+                const uint32_t k01 = __builtin_amdgcn_perm(w[1], w[0], sel);
+                const uint32_t k23 = __builtin_amdgcn_perm(w[3], w[2], sel);
+                *reinterpret_cast<u32x2*>(vb + (v_write ^ (16u * i)) + 128 * i) = u32x2{k01, k23};
+            }
+            if constexpr (KIND != 0) PKV_SB();      // (as in store_k)
+        });
     };
     // Operand reads, two operands a step. K, step i: k-step i of both 32-key halves. V, step i: keys
     // 16 (i / (NB / 2)) .. + 15 of the 32-dim blocks 2 (i % (NB / 2)) and the next one.
@@ -318,17 +305,20 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
             s[1] = mfma<F16>(ka[i % RING][1], qreg[i], s[1]);
             if constexpr (i == 0) store_k(buf ^ 1), load_k();
             if constexpr (i == KS / 2 - 1) store_v(buf ^ 1), load_v();
+            if constexpr (KIND != 0) PKV_SB();
         });
         // one product, then a share of the staging work (LDS reads of later operands, the stores' permutes and
         // writes, the row loads) in its shadow
-        __builtin_amdgcn_sched_group_barrier(0x100, 2 * (RING - 1), 0);
-        static_for<2 * KS>([&](auto) __attribute__((always_inline)) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
-            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        });
+        if constexpr (KIND == 0) {      // (8-bit pages: the conversions' temporaries make this order spill)
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 * (RING - 1), 0);
+            static_for<2 * KS>([&](auto) __attribute__((always_inline)) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            });
+        }
         PKV_SB();
         PKV_PRIO(0);
         u32x4 va[RING][2];
