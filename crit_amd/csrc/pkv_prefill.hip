@@ -363,11 +363,15 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
         const float alpha = exp2_fast(m - sub);
         m = m_new;
         float sum = 0.0f;
-        // P^T as the second product's B operand, 16 keys at a time: the probabilities of keys 32 kb + 16 half .. + 15.
-        auto probs = [&](int kb, int half) __attribute__((always_inline)) -> u32x4 {
-            uint32_t pw[4];
+        // P^T as the second product's B operand: pop[g] holds the probabilities of keys 16 g .. 16 g + 15 (32-key half
+        // g / 2, half of it g % 2), four 16-bit pairs, taken two pairs at a time so that only the first two pairs'
+        // exponentials run before the second product starts and the rest in the shadow of its matrix instructions.
+        u32x4 pop[4];
+        auto pairs = [&](auto gc, auto partc) __attribute__((always_inline)) {
+            constexpr int g = decltype(gc)::value, part = decltype(partc)::value;
+            constexpr int kb = g / 2, half = g % 2;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 2 * part; j < 2 * part + 2; ++j) {
                 const int v = 8 * half + 2 * j;
                 float p0, p1;
                 if constexpr (KIND >= 2) {
@@ -380,13 +384,13 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
                     p0 *= vs_lds[buf][32 * kb + 8 * (v / 4) + 4 * h + v % 4];
                     p1 *= vs_lds[buf][32 * kb + 8 * ((v + 1) / 4) + 4 * h + (v + 1) % 4];
                 }
-                pw[j] = to_pair<F16>(p0, p1);
+                pop[g][j] = to_pair<F16>(p0, p1);
             }
-            return u32x4{pw[0], pw[1], pw[2], pw[3]};
         };
-        u32x4 pop[4];
-        pop[0] = probs(0, 0);
-        pop[1] = probs(0, 1);
+        const std::integral_constant<int, 0> c0;
+        const std::integral_constant<int, 1> c1;
+        pairs(c0, c0);
+        pairs(c0, c1);
         // wave-uniform: skip the rescale when no row's maximum moved (alpha == 1 everywhere)
         if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
             asm volatile("s_nop 0");      // pins the branch: an unconditional rescale by 1 is what the optimiser would make of it
@@ -406,8 +410,15 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
             if constexpr (i + RING - 1 < VSTEPS) read_v(vl, std::integral_constant<int, i + RING - 1>{}, va[(i + RING - 1) % RING]);
             o[nb] = mfma<F16>(va[i % RING][0], pop[g], o[nb]);
             o[nb + 1] = mfma<F16>(va[i % RING][1], pop[g], o[nb + 1]);
-            if constexpr (i == 0) pop[2] = probs(1, 0);
-            if constexpr (i == NB / 2) pop[3] = probs(1, 1);
+            // steps 0 .. 5 take the pairs of pop[1], pop[2], pop[3] in order, each a step (D = 128) or more (D = 64:
+            // two at a time) before the step that multiplies by them
+            if constexpr (NB == 4) {
+                if constexpr (i < 6) pairs(std::integral_constant<int, 1 + i / 2>{}, std::integral_constant<int, i % 2>{});
+            } else {
+                if constexpr (i == 0) pairs(c1, c0), pairs(c1, c1);
+                if constexpr (i == 1) pairs(std::integral_constant<int, 2>{}, c0), pairs(std::integral_constant<int, 2>{}, c1);
+                if constexpr (i == 2) pairs(std::integral_constant<int, 3>{}, c0), pairs(std::integral_constant<int, 3>{}, c1);
+            }
             if constexpr (i == VSTEPS - 2) {      // the slots of block kt + 3 for the next iteration's loads, the entries of kt + 4
                 take_slots();
                 load_entries(upto(kt + 4));
