@@ -31,27 +31,32 @@ __global__ __launch_bounds__(64) void merge_kernel(AttendArgs a) {
 #pragma unroll
     for (int e = 0; e < EPL; ++e) A[e] = 0.0f;
     // Folded strictly in partition order (the fused launch folds the same way), but loaded U partitions at a time so
-    // the loads of a long row's hundreds of partials overlap instead of chaining their latencies.
-    constexpr int U = 32;
-    for (int b0 = 0; b0 < nb; b0 += U) {
-        float pm[U], pl[U], po[U][EPL];
+    // the loads of a long row's hundreds of partials overlap instead of chaining their latencies: 8 at a time for the
+    // few partitions of an ordinary decode row, 32 at a time beyond that.
+    auto fold_from = [&](int b_lo, auto uc) __attribute__((always_inline)) {
+        constexpr int U = decltype(uc)::value;
+        for (int b0 = b_lo; b0 < nb; b0 += U) {
+            float pm[U], pl[U], po[U][EPL];
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int b = b0 + u < nb ? b0 + u : nb - 1;
-            pm[u] = a.pm[at + b], pl[u] = a.pl[at + b];
+            for (int u = 0; u < U; ++u) {
+                const int b = b0 + u < nb ? b0 + u : nb - 1;
+                pm[u] = a.pm[at + b], pl[u] = a.pl[at + b];
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) po[u][e] = a.po[(at + b) * DV + e * 64 + lane];
-        }
+                for (int e = 0; e < EPL; ++e) po[u][e] = a.po[(at + b) * DV + e * 64 + lane];
+            }
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            if (b0 + u < nb) {
-                const Fold f = fold(M, L, pm[u], pl[u]);
+            for (int u = 0; u < U; ++u) {
+                if (b0 + u < nb) {
+                    const Fold f = fold(M, L, pm[u], pl[u]);
 #pragma unroll
-                for (int e = 0; e < EPL; ++e) A[e] = __builtin_fmaf(A[e], f.keep, po[u][e] * f.take);
-                M = f.m, L = f.l;
+                    for (int e = 0; e < EPL; ++e) A[e] = __builtin_fmaf(A[e], f.keep, po[u][e] * f.take);
+                    M = f.m, L = f.l;
+                }
             }
         }
-    }
+    };
+    if (nb <= 8) fold_from(0, std::integral_constant<int, 8>{});
+    else fold_from(0, std::integral_constant<int, 32>{});
     if (a.sinks) {
         const Fold f = fold(M, L, a.sinks[head] * kLog2e, 1.0f);
 #pragma unroll

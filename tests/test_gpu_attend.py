@@ -356,12 +356,16 @@ def test_launches_that_overlap_on_two_streams_do_not_share_counters():
     qs = [rand_q(3, 16, 128, 20 + s) for s in range(2)]
     want = [c.attend(q, [0, 1, 2], [0, 1, 2], [2999, 1699, 899], 1) for c, q in zip(caches, qs)]
     torch.cuda.synchronize()
+    pk = kernels()
+    floats = pk.workspace_floats(3, 16, pk.partitions(dev, 4, "bf16"), 128)
+    # (each stream its own partials: the module's default workspace is one per device and owner, as the reference's)
+    spaces = [torch.empty(floats, dtype=torch.float32, device=dev) for _ in range(2)]
     streams = [torch.cuda.Stream() for _ in range(2)]
     outs = [[], []]
     for rep in range(65):
         for i, stream in enumerate(streams):
             with torch.cuda.stream(stream):
-                outs[i].append(caches[i].attend(qs[i], [0, 1, 2], [0, 1, 2], [2999, 1699, 899], 1))
+                outs[i].append(caches[i].attend(qs[i], [0, 1, 2], [0, 1, 2], [2999, 1699, 899], 1, workspace=spaces[i]))
     torch.cuda.synchronize()
     for i in range(2):
         for got in outs[i]:
