@@ -558,15 +558,13 @@ template <int KIND, bool F16, int QR, int HW, bool FUSED>
 __global__ __launch_bounds__(256, attend_waves(KIND, QR)) void attend128_kernel(AttendArgs a) {
     __shared__ unsigned s_unit;
     const unsigned total = (unsigned)a.units_x * (unsigned)a.units_y;
-    if (threadIdx.x == 0) s_unit = atomicAdd(a.ticket, 1u);
-    __syncthreads();
-    unsigned u = s_unit;
+    unsigned u = blockIdx.x;      // the first gridDim.x units need no ticket: tickets number the units after them
     while (u < total) {
         // (the next ticket is drawn after the unit, not during it: a returning atomic in flight makes every wait on
         // the unit's loads a wait for all of them, which costs more than the ticket's round trip)
         attend128_unit<KIND, F16, QR, HW, FUSED>(a, (int)(u % (unsigned)a.units_x), (int)(u / (unsigned)a.units_x));
         __syncthreads();      // the unit is done with the shared arrays, and every thread has read s_unit
-        if (threadIdx.x == 0) s_unit = atomicAdd(a.ticket, 1u);
+        if (threadIdx.x == 0) s_unit = gridDim.x + atomicAdd(a.ticket, 1u);
         __syncthreads();
         u = s_unit;
     }
