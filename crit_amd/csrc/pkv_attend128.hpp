@@ -130,12 +130,19 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
     const int first = (int)(first64 < 0 ? 0 : (first64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first64));
     const int n_pieces = (n_keys + a.piece - 1) / a.piece;
     if constexpr (!FUSED) {
-        // Units are taken in list order, y slowest: the row's last partition (usually a partial piece, the smallest
-        // unit of work) takes the last y, so the small units start last and fill the launch's tail.
+        // Units are taken in list order, y slowest, and a launch's tail is as long as its last units: the row's last
+        // partition (usually a partial piece, the smallest unit of work) is listed after every other partition, at
+        // the last y but one if it holds half a piece or more and at the very last y if it holds less, so the units
+        // that start last are the smallest.
         const int np = min(n_pieces, a.parts);
         if (np <= 0) return;
-        if (b == a.units_y - 1) b = np - 1;
-        else if (b >= np - 1) return;
+        const bool small = np == n_pieces && n_keys - (np - 1) * a.piece < a.piece / 2;
+        if (b >= a.units_y - 2) {
+            if ((b == a.units_y - 1) != small) return;
+            b = np - 1;
+        } else if (b >= np - 1) {
+            return;
+        }
     }
 
     // The lane's slices of the tile's query rows (packed 16-bit pairs): dims 8 li8 .. +7 and 64 + 8 li8 .. +7 over

@@ -11,8 +11,9 @@ template <int KIND, bool F16, int QR, bool FUSED>
 static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipStream_t stream) {
     if (lpr == 16 && page16) {       // pages of a multiple of 16 positions: the bandwidth path, resident workgroups pulling units
         AttendArgs u = a;
-        u.units_x = (int)grid.x, u.units_y = (int)grid.y;
-        const int64_t units = (int64_t)grid.x * grid.y;
+        // (a split launch lists a row's last partition twice, for the one of two size classes it falls in)
+        u.units_x = (int)grid.x, u.units_y = FUSED ? (int)grid.y : (int)grid.y + 1;
+        const int64_t units = (int64_t)u.units_x * u.units_y;
         if (units > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
         const int64_t resident = (int64_t)compute_units() * attend_waves(KIND, QR);
         const dim3 pgrid((unsigned)(units < resident ? units : resident));
