@@ -42,6 +42,42 @@ constexpr float kLn2 = 0.6931471805599453f;
 PKV_DEV uint32_t f2u(float x) { return __builtin_bit_cast(uint32_t, x); }
 PKV_DEV float u2f(uint32_t x) { return __builtin_bit_cast(float, x); }
 
+// -- division by a value fixed per launch ------------------------------------------------------------------------------------
+// n / d for 0 <= n < 2^31 by a multiply and a shift (d >= 1): l = ceil(log2 d), magic = floor(2^32 (2^l - d) / d) + 1.
+struct Div32 {
+    uint32_t magic, shift;
+};
+inline Div32 make_div32(uint32_t d) {
+    uint32_t l = 0;
+    while ((1ull << l) < d) ++l;
+    return {(uint32_t)((((1ull << l) - (uint64_t)d) << 32) / (uint64_t)d + 1), l};
+}
+PKV_DEV uint32_t div32(Div32 m, uint32_t n) { return (__umulhi(m.magic, n) + n) >> m.shift; }
+
+// x / d, correctly rounded, for many x and one d: the steps of the compiler's own FP32 division (a reciprocal refined
+// once, the quotient refined twice through exact residuals) with everything that depends on d alone computed once.
+// Those steps give the correctly rounded quotient wherever none of them overflows or loses bits to underflow, which
+// `plain` guarantees for the quotients a page code can tell apart (|x / d| from 2^-12 up, below 2^127): d in
+// 2^-60 .. 2^60, where the reciprocal, the residuals of such quotients (2^-24 of x) and their products stay normal.
+// Smaller quotients may come out a few steps off and still round to the same (zero) code; a quotient that overflows
+// comes out NaN, which the callers send through the exact division. The residuals are taken negated, d q - x, and
+// subtracted: the same bits, and a zero x keeps its sign through every step (-0 + +0 would be +0).
+struct Quotients {
+    float d, r;
+    bool plain;
+    PKV_DEV explicit Quotients(float div) : d(div) {
+        plain = div >= 0x1p-60f && div <= 0x1p60f;
+        const float r0 = __builtin_amdgcn_rcpf(div);
+        r = __builtin_fmaf(__builtin_fmaf(-div, r0, 1.0f), r0, r0);
+    }
+    PKV_DEV float of(float x) const {
+        float q = x * r;
+        q = __builtin_fmaf(-__builtin_fmaf(d, q, -x), r, q);
+        q = __builtin_fmaf(-__builtin_fmaf(d, q, -x), r, q);
+        return q;
+    }
+};
+
 // -- bf16 / f16 ---------------------------------------------------------------------------------------------------------
 PKV_DEV float bf16_lo(uint32_t w) { return u2f(w << 16); }
 PKV_DEV float bf16_hi(uint32_t w) { return u2f(w & 0xffff0000u); }

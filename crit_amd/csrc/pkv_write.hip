@@ -17,6 +17,7 @@ struct WriteArgs {
     int dim[2];
     int hkv;
     int heads;      // hkv (keys only) or 2 * hkv
+    Div32 heads_div;
     float mult[2];
 };
 
@@ -27,29 +28,79 @@ PKV_DEV float load_in(const void* base, int64_t i) {
     return (float)reinterpret_cast<const _Float16*>(base)[i];
 }
 
-// EPL consecutive input elements as FP32, by 16-byte loads (the caller checked the alignment).
+// EPL consecutive input elements of one lane as they lie in memory, fetched by 16-byte loads (the caller checked the
+// alignment) and widened to FP32 only where they are used: a row waits in a quarter to half of the registers its FP32
+// values would take, which is what lets twice the wavefronts be resident.
 template <int IN, int EPL>
-PKV_DEV void load_vec(const void* base, int64_t i, float (&x)[EPL]) {
-    if constexpr (IN == CRIT_PKV_F32) {
-        const float4* p = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(base) + i);
+struct RawRow {
+    static constexpr int N = EPL * (IN == CRIT_PKV_F32 ? 4 : 2) / 16;
+    u32x4 v[N];
+    PKV_DEV void load(const void* base, int64_t i) {
+        const u32x4* p = reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(base) + i * (IN == CRIT_PKV_F32 ? 4 : 2));
 #pragma unroll
-        for (int j = 0; j < EPL / 4; ++j) {
-            float4 v = p[j];
-            x[4 * j] = v.x, x[4 * j + 1] = v.y, x[4 * j + 2] = v.z, x[4 * j + 3] = v.w;
+        for (int j = 0; j < N; ++j) v[j] = __builtin_nontemporal_load(p + j);      // read once
+    }
+    PKV_DEV void zero() {
+#pragma unroll
+        for (int j = 0; j < N; ++j) v[j] = u32x4{0, 0, 0, 0};
+    }
+    template <int J>
+    PKV_DEV float at() const {
+        if constexpr (IN == CRIT_PKV_F32) {
+            return u2f(v[J / 4][J % 4]);
+        } else {
+            const uint32_t w = v[J / 8][(J % 8) / 2];
+            if constexpr (IN == CRIT_PKV_BF16) return (J & 1) ? bf16_hi(w) : bf16_lo(w);
+            return (J & 1) ? f16_hi(w) : f16_lo(w);
+        }
+    }
+    PKV_DEV void widen(float (&x)[EPL]) const {
+        static_for<EPL>([&](auto j) { x[j] = at<j>(); });
+    }
+};
+
+// 16 codes of one lane from exact divisions: the reference's arithmetic step by step, for the lanes whose quotients
+// the shared-step division cannot vouch for.
+template <int KIND>
+PKV_DEV void exact_codes(const float (&x)[16], float div, uint32_t (&w)[4]) {
+    float q[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) q[j] = __fdiv_rn(x[j], div);
+    if constexpr (KIND == 3) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            uint32_t packed = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float r = __builtin_rintf(q[4 * k + j]);            // ties to even
+                r = r < -127.0f ? -127.0f : (r > 127.0f ? 127.0f : r);
+                packed |= ((uint32_t)(int)r & 0xffu) << (8 * j);
+            }
+            w[k] = packed;
         }
     } else {
-        const uint4* p = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(base) + i);
+        // Finite quotients: clamp, then the hardware's round-to-nearest-even conversion, two codes an instruction; a NaN
+        // anywhere in the lane's 16 (or infinities of both signs, whose sum is NaN too) sends the lane through the
+        // integer encoder, which fixes the NaN code and sign.
+        float sum = 0.0f;
 #pragma unroll
-        for (int j = 0; j < EPL / 8; ++j) {
-            const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p) + j);      // read once
-            uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        for (int j = 0; j < 16; ++j) sum += q[j];
+        if (sum == sum) {
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                if constexpr (IN == CRIT_PKV_BF16) {
-                    x[8 * j + 2 * k] = bf16_lo(w[k]), x[8 * j + 2 * k + 1] = bf16_hi(w[k]);
-                } else {
-                    x[8 * j + 2 * k] = f16_lo(w[k]), x[8 * j + 2 * k + 1] = f16_hi(w[k]);
-                }
+                const float c0 = __builtin_amdgcn_fmed3f(q[4 * k], -448.0f, 448.0f), c1 = __builtin_amdgcn_fmed3f(q[4 * k + 1], -448.0f, 448.0f);
+                const float c2 = __builtin_amdgcn_fmed3f(q[4 * k + 2], -448.0f, 448.0f), c3 = __builtin_amdgcn_fmed3f(q[4 * k + 3], -448.0f, 448.0f);
+                int packed = __builtin_amdgcn_cvt_pk_fp8_f32(c0, c1, 0, false);
+                packed = __builtin_amdgcn_cvt_pk_fp8_f32(c2, c3, packed, true);
+                w[k] = (uint32_t)packed;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                uint32_t packed = 0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) packed |= e4m3_encode(q[4 * k + j]) << (8 * j);
+                w[k] = packed;
             }
         }
     }
@@ -64,53 +115,60 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
     constexpr int EPL = KIND == 0 ? 8 : 16;
     constexpr int RPP = 256 / LPR;      // rows a workgroup covers per pass
     const int lane_in_row = threadIdx.x % LPR;
-    const int64_t row0 = (int64_t)blockIdx.x * (RPP * U) + threadIdx.x / LPR;
-    const int64_t n_rows = a.tokens * a.heads;
+    // (a launch holds fewer than 2^31 rows, the launcher sees to that: 32-bit row arithmetic, and the token of a row
+    // by a multiply and a shift; a 64-bit division here costs more instructions than the rest of the kernel)
+    const uint32_t row0 = blockIdx.x * (uint32_t)(RPP * U) + threadIdx.x / LPR;
+    const uint32_t n_rows = (uint32_t)(a.tokens * a.heads);
     const int i0 = lane_in_row * EPL;
-    float x[U][EPL];
+    RawRow<IN, EPL> raw[U];
     int64_t slot[U];
     int head[U], which[U];
     bool live[U];
+    float mult[U];      // "fp8" pages: the row's divisor, fetched with its inputs
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-        const int64_t row = row0 + u * RPP;
+        const uint32_t row = row0 + u * RPP;
         const bool in = row < n_rows;
-        const int64_t t = in ? row / a.heads : 0;
-        head[u] = in ? (int)(row % a.heads) : 0;
+        const int64_t t = in ? (int64_t)div32(a.heads_div, row) : 0;
+        head[u] = in ? (int)(row - (uint32_t)t * (uint32_t)a.heads) : 0;
         which[u] = head[u] >= a.hkv ? 1 : 0;
         head[u] -= which[u] * a.hkv;
         slot[u] = in ? a.slots[t] : -1;
         live[u] = in && i0 < a.dim[which[u]];
+        mult[u] = 1.0f;
+        if constexpr (KIND == 1) mult[u] = a.head_mult ? a.head_mult[which[u] * a.hkv + head[u]] : a.mult[which[u]];
         if (live[u]) {
-            load_vec<IN, EPL>(a.src[which[u]], t * a.stride_t[which[u]] + head[u] * a.stride_h[which[u]] + i0, x[u]);
+            raw[u].load(a.src[which[u]], t * a.stride_t[which[u]] + head[u] * a.stride_h[which[u]] + i0);
         } else {
-#pragma unroll
-            for (int j = 0; j < EPL; ++j) x[u][j] = 0.0f;
+            raw[u].zero();
         }
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         // (a whole row's lanes agree on slot[u] < 0, so the row-scale exchange below stays among participating lanes)
         if (slot[u] < 0) continue;
+        float x[EPL];
+        raw[u].widen(x);
         const int dim = a.dim[which[u]];
         const int64_t dst = (slot[u] * a.hkv + head[u]) * dim + i0;
         if constexpr (KIND == 0) {
             uint4 v;
             if constexpr (F16) {
-                v = make_uint4(pack_f16(x[u][0], x[u][1]), pack_f16(x[u][2], x[u][3]), pack_f16(x[u][4], x[u][5]), pack_f16(x[u][6], x[u][7]));
+                v = make_uint4(pack_f16(x[0], x[1]), pack_f16(x[2], x[3]), pack_f16(x[4], x[5]), pack_f16(x[6], x[7]));
             } else {
-                v = make_uint4(pack_bf16(x[u][0], x[u][1]), pack_bf16(x[u][2], x[u][3]), pack_bf16(x[u][4], x[u][5]), pack_bf16(x[u][6], x[u][7]));
+                v = make_uint4(pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]), pack_bf16(x[6], x[7]));
             }
             if (live[u]) __builtin_nontemporal_store(u32x4{v.x, v.y, v.z, v.w}, reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(a.pages[which[u]]) + dst));
         } else {
             float div;
+            bool zero_row = false;
             if constexpr (KIND == 1) {
-                div = a.head_mult ? a.head_mult[which[u] * a.hkv + head[u]] : a.mult[which[u]];
+                div = mult[u];
             } else {
                 float amax = 0.0f;
 #pragma unroll
                 for (int j = 0; j < EPL; ++j) {
-                    const float m = __builtin_fabsf(x[u][j]);
+                    const float m = __builtin_fabsf(x[j]);
                     amax = (m > amax || m != m) ? m : amax;       // a NaN in the row makes the scale NaN, as torch's amax
                 }
 #pragma unroll
@@ -121,50 +179,40 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
                 const float top = KIND == 2 ? 448.0f : 127.0f;
                 div = __fdiv_rn(amax, top);
                 div = div < 1e-30f ? 1e-30f : div;               // clamp(min=1e-30); NaN stays NaN
+                zero_row = amax == 0.0f;
                 if (lane_in_row == 0) a.scales[which[u]][slot[u] * a.hkv + head[u]] = div;
             }
+            // The quotients by the shared steps of one division, straight through to the codes; where the divisor does
+            // not allow that (an all-zero row's does, the 1e-30 floor: its quotients are zeros of the inputs' signs
+            // either way) or a quotient came out NaN (a NaN or infinite input, a quotient past FP32), the lane's codes
+            // are made again from exact divisions.
             uint32_t w[4];
-            float q[16];
+            const Quotients quot(div);
+            bool coded = quot.plain || zero_row;
+            float sum = 0.0f;
 #pragma unroll
-            for (int j = 0; j < 16; ++j) q[j] = __fdiv_rn(x[u][j], div);
-            if constexpr (KIND == 3) {
+            for (int k = 0; k < 4; ++k) {
+                float c[4];
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    uint32_t packed = 0;
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        float r = __builtin_rintf(q[4 * k + j]);            // ties to even
-                        r = r < -127.0f ? -127.0f : (r > 127.0f ? 127.0f : r);
-                        packed |= ((uint32_t)(int)r & 0xffu) << (8 * j);
+                for (int j = 0; j < 4; ++j) {
+                    const float q = quot.of(x[4 * k + j]);
+                    if constexpr (KIND == 3) {
+                        c[j] = __builtin_amdgcn_fmed3f(__builtin_rintf(q), -127.0f, 127.0f);      // ties to even
+                    } else {
+                        if constexpr (KIND == 1) sum += q;      // (a row's own scale keeps its quotients finite)
+                        c[j] = __builtin_amdgcn_fmed3f(q, -448.0f, 448.0f);
                     }
-                    w[k] = packed;
                 }
-            } else {
-                // Finite quotients (all but the rarest rows): clamp, then the hardware's round-to-nearest-even
-                // conversion, two codes an instruction; a NaN anywhere in the lane's 16 (or infinities of both signs,
-                // whose sum is NaN too) sends the lane through the integer encoder, which fixes the NaN code and sign.
-                float sum = 0.0f;
-#pragma unroll
-                for (int j = 0; j < 16; ++j) sum += q[j];
-                if (sum == sum) {
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        const float c0 = __builtin_amdgcn_fmed3f(q[4 * k], -448.0f, 448.0f), c1 = __builtin_amdgcn_fmed3f(q[4 * k + 1], -448.0f, 448.0f);
-                        const float c2 = __builtin_amdgcn_fmed3f(q[4 * k + 2], -448.0f, 448.0f), c3 = __builtin_amdgcn_fmed3f(q[4 * k + 3], -448.0f, 448.0f);
-                        int packed = __builtin_amdgcn_cvt_pk_fp8_f32(c0, c1, 0, false);
-                        packed = __builtin_amdgcn_cvt_pk_fp8_f32(c2, c3, packed, true);
-                        w[k] = (uint32_t)packed;
-                    }
+                if constexpr (KIND == 3) {
+                    w[k] = ((uint32_t)(int)c[0] & 0xffu) | (((uint32_t)(int)c[1] & 0xffu) << 8) | (((uint32_t)(int)c[2] & 0xffu) << 16) |
+                           ((uint32_t)(int)c[3] << 24);
                 } else {
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        uint32_t packed = 0;
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) packed |= e4m3_encode(q[4 * k + j]) << (8 * j);
-                        w[k] = packed;
-                    }
+                    int packed = __builtin_amdgcn_cvt_pk_fp8_f32(c[0], c[1], 0, false);
+                    w[k] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], packed, true);
                 }
             }
+            coded = coded && sum == sum;
+            if (__builtin_expect(!coded, 0)) exact_codes<KIND>(x, div, w);
             if (live[u]) __builtin_nontemporal_store(u32x4{w[0], w[1], w[2], w[3]}, reinterpret_cast<u32x4*>(reinterpret_cast<uint8_t*>(a.pages[which[u]]) + dst));
         }
     }
@@ -218,12 +266,28 @@ __global__ __launch_bounds__(256) void write_rows_scalar(WriteArgs a) {
 
 template <int KIND, bool F16, int IN>
 static int launch_kind(const WriteArgs& a, int lpr, bool vector, hipStream_t stream) {
-    const int64_t rows = a.tokens * a.heads;
     if (!vector) {
-        const int64_t blocks = (rows + 255) / 256;
+        const int64_t blocks = (a.tokens * a.heads + 255) / 256;
         hipLaunchKernelGGL((write_rows_scalar<KIND, F16, IN>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
         return hip_code(hipGetLastError());
     }
+    // The vector kernels count rows in 32 bits: more tokens than 2^31 rows hold go in several launches.
+    const int64_t most = (((int64_t)1 << 31) - (1 << 16)) / a.heads;
+    if (a.tokens > most) {
+        const int in_bytes = IN == CRIT_PKV_F32 ? 4 : 2;
+        for (int64_t t0 = 0; t0 < a.tokens; t0 += most) {
+            WriteArgs part = a;
+            part.tokens = a.tokens - t0 < most ? a.tokens - t0 : most;
+            part.slots = a.slots + t0;
+            for (int w = 0; w < 2; ++w) {
+                if (a.src[w]) part.src[w] = reinterpret_cast<const char*>(a.src[w]) + t0 * a.stride_t[w] * in_bytes;
+            }
+            const int code = launch_kind<KIND, F16, IN>(part, lpr, vector, stream);
+            if (code) return code;
+        }
+        return 0;
+    }
+    const int64_t rows = a.tokens * a.heads;
     // Four rows a thread once there is work for every compute unit many times over (2^21 lane-rows: 16,384 tokens of
     // 8 KV heads of 16-bit pages); one row a thread below that, where the launch is latency-bound and more workgroups
     // finish sooner (at 4,152 tokens: 10.4 us against 14.2).
@@ -280,6 +344,7 @@ int launch_write(const crit_pkv_write_params* p, hipStream_t stream) {
     a.dim[0] = p->head_dim, a.dim[1] = p->values ? p->value_dim : p->head_dim;
     a.hkv = p->kv_heads;
     a.heads = p->values ? 2 * p->kv_heads : p->kv_heads;
+    a.heads_div = make_div32((uint32_t)a.heads);
     a.mult[0] = p->key_multiplier, a.mult[1] = p->value_multiplier;
     // The vector path: rows are whole 16-byte lanes on both sides and every row start is 16-byte aligned.
     const int epl = p->kind == 0 ? 8 : 16;

@@ -134,6 +134,62 @@ def test_one_multiplier_per_kv_head():
     _check("fp8", (k, v, None, None), want)
 
 
+def _codes_between(kind, n, g):
+    """n values halfway between two neighbouring codes of the kind (in the codes' own units)."""
+    if kind == "int8":
+        return torch.randint(-127, 127, (n,), generator=g).double() + 0.5
+    c = torch.randint(0, 126, (n,), generator=g).to(torch.uint8)          # 0 .. 448's code - 1
+    lo, hi = c.view(torch.float8_e4m3fn).double(), (c + 1).view(torch.float8_e4m3fn).double()
+    sign = torch.randint(0, 2, (n,), generator=g).double() * 2 - 1
+    return sign * (lo + hi) / 2
+
+
+def test_fp8_quotients_at_rounding_boundaries_under_awkward_multipliers():
+    # Inputs within a few FP32 steps of (a tie between two codes) x (the head's multiplier): any division that is not the
+    # correctly rounded one lands on the wrong side of some of them. Multipliers that are no powers of two, negative,
+    # and far enough out that the reciprocal is subnormal or the quotient overflows.
+    pk = kernels()
+    g = torch.Generator().manual_seed(11)
+    T, hkv, d = 257, 8, 128
+    mults = torch.tensor([[0.03, 1.0 / 3.0, 3.7e-5, -0.7, 1e-35, 1e35, 0.999999, 1234.567],
+                          [7e-3, -1.1e-4, 2.5, 1e-37, 0.1, 5e30, 3.0, 0.06]], dtype=torch.float32)
+    rows = []
+    for which in range(2):
+        mid = _codes_between("fp8", T * hkv * d, g).view(T, hkv, d)
+        steps = torch.randint(-6, 7, (T, hkv, d), generator=g).double() * 2.0 ** -24
+        rows.append((mid * mults[which].double()[None, :, None] * (1 + steps)).float())
+    keys, values = rows
+    k = torch.zeros(512, hkv, d, dtype=torch.float8_e4m3fn, device=dev)
+    v = torch.zeros_like(k)
+    slots = torch.randperm(512, generator=g)[:T]
+    pk.write(keys.to(dev), values.to(dev), slots.to(dev), k, v, "fp8", multipliers=mults.to(dev))
+    _check("fp8", (k, v, None, None), expected_pages("fp8", keys, values, slots, 512, (mults[0], mults[1])))
+
+
+@pytest.mark.parametrize("kind", ["fp8:row", "int8"])
+def test_row_scaled_quotients_at_rounding_boundaries(kind):
+    # Each row holds its maximum once and otherwise values within a few FP32 steps of (a tie between two codes) x (the
+    # scale that maximum gives the row).
+    pk = kernels()
+    g = torch.Generator().manual_seed(12)
+    T, hkv, d = 300, 4, 128
+    top = 448.0 if kind == "fp8:row" else 127.0
+    amax = (torch.rand(T, hkv, generator=g) * 40 + 0.01).float()
+    scale = (amax / torch.full_like(amax, top)).clamp(min=1e-30)
+    mid = _codes_between("fp8" if kind == "fp8:row" else "int8", T * hkv * d, g).view(T, hkv, d)
+    steps = torch.randint(-6, 7, (T, hkv, d), generator=g).double() * 2.0 ** -24
+    keys = (mid * scale.double()[..., None] * (1 + steps)).float()
+    keys = torch.where(keys.abs() >= amax[..., None], keys * 0.5, keys)
+    keys[:, :, 5] = amax * (torch.randint(0, 2, (T, hkv), generator=g).float() * 2 - 1)
+    values = keys.flip(0).contiguous()
+    k = torch.zeros(512, hkv, d, dtype=STORE[kind], device=dev)
+    v = torch.zeros_like(k)
+    ks, vs = torch.zeros(512, hkv, device=dev), torch.zeros(512, hkv, device=dev)
+    slots = torch.randperm(512, generator=g)[:T]
+    pk.write(keys.to(dev), values.to(dev), slots.to(dev), k, v, kind, ks, vs)
+    _check(kind, (k, v, ks, vs), expected_pages(kind, keys, values, slots, 512, (1.0, 1.0)))
+
+
 def test_odd_widths_and_strided_inputs_take_the_scalar_path():
     pk = kernels()
     g = torch.Generator().manual_seed(6)
