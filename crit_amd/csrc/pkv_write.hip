@@ -4,6 +4,13 @@
 #include "pkv_common.hpp"
 #include "pkv_launch.hpp"
 
+#ifndef PKV_WIDE_U16
+#define PKV_WIDE_U16 4
+#endif
+#ifndef PKV_WIDE_U8
+#define PKV_WIDE_U8 2
+#endif
+
 namespace pkv {
 
 struct WriteArgs {
@@ -60,50 +67,36 @@ struct RawRow {
 };
 
 // 16 codes of one lane from exact divisions: the reference's arithmetic step by step, for the lanes whose quotients
-// the shared-step division cannot vouch for.
-template <int KIND>
-PKV_DEV void exact_codes(const float (&x)[16], float div, uint32_t (&w)[4]) {
-    float q[16];
-#pragma unroll
-    for (int j = 0; j < 16; ++j) q[j] = __fdiv_rn(x[j], div);
-    if constexpr (KIND == 3) {
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            uint32_t packed = 0;
+// the shared-step division cannot vouch for. Four codes at a time, so the rare path needs few registers of its own.
+template <int KIND, class Row>
+PKV_DEV void exact_codes(const Row& row, float div, uint32_t (&w)[4]) {
+    static_for<4>([&](auto k) {
+        const float q[4] = {__fdiv_rn(row.template at<4 * k>(), div), __fdiv_rn(row.template at<4 * k + 1>(), div),
+                            __fdiv_rn(row.template at<4 * k + 2>(), div), __fdiv_rn(row.template at<4 * k + 3>(), div)};
+        uint32_t packed = 0;
+        if constexpr (KIND == 3) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                float r = __builtin_rintf(q[4 * k + j]);            // ties to even
+                float r = __builtin_rintf(q[j]);            // ties to even
                 r = r < -127.0f ? -127.0f : (r > 127.0f ? 127.0f : r);
                 packed |= ((uint32_t)(int)r & 0xffu) << (8 * j);
             }
-            w[k] = packed;
-        }
-    } else {
-        // Finite quotients: clamp, then the hardware's round-to-nearest-even conversion, two codes an instruction; a NaN
-        // anywhere in the lane's 16 (or infinities of both signs, whose sum is NaN too) sends the lane through the
-        // integer encoder, which fixes the NaN code and sign.
-        float sum = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 16; ++j) sum += q[j];
-        if (sum == sum) {
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const float c0 = __builtin_amdgcn_fmed3f(q[4 * k], -448.0f, 448.0f), c1 = __builtin_amdgcn_fmed3f(q[4 * k + 1], -448.0f, 448.0f);
-                const float c2 = __builtin_amdgcn_fmed3f(q[4 * k + 2], -448.0f, 448.0f), c3 = __builtin_amdgcn_fmed3f(q[4 * k + 3], -448.0f, 448.0f);
-                int packed = __builtin_amdgcn_cvt_pk_fp8_f32(c0, c1, 0, false);
-                packed = __builtin_amdgcn_cvt_pk_fp8_f32(c2, c3, packed, true);
-                w[k] = (uint32_t)packed;
-            }
         } else {
+            // Finite quotients: clamp, then the hardware's round-to-nearest-even conversion, two codes an instruction;
+            // a NaN among the four (or infinities of both signs, whose sum is NaN too) sends them through the integer
+            // encoder, which fixes the NaN code and sign and agrees with the hardware on everything else.
+            const float sum = (q[0] + q[1]) + (q[2] + q[3]);
+            if (sum == sum) {
+                const float c0 = __builtin_amdgcn_fmed3f(q[0], -448.0f, 448.0f), c1 = __builtin_amdgcn_fmed3f(q[1], -448.0f, 448.0f);
+                const float c2 = __builtin_amdgcn_fmed3f(q[2], -448.0f, 448.0f), c3 = __builtin_amdgcn_fmed3f(q[3], -448.0f, 448.0f);
+                packed = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(c2, c3, __builtin_amdgcn_cvt_pk_fp8_f32(c0, c1, 0, false), true);
+            } else {
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                uint32_t packed = 0;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) packed |= e4m3_encode(q[4 * k + j]) << (8 * j);
-                w[k] = packed;
+                for (int j = 0; j < 4; ++j) packed |= e4m3_encode(q[j]) << (8 * j);
             }
         }
-    }
+        w[k] = packed;
+    });
 }
 
 // One row = (token, head) with head in [0, heads): keys' heads first, then values'. LPR lanes hold one row, EPL
@@ -122,34 +115,45 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
     const int i0 = lane_in_row * EPL;
     RawRow<IN, EPL> raw[U];
     int64_t slot[U];
-    int head[U], which[U];
-    bool live[U];
-    float mult[U];      // "fp8" pages: the row's divisor, fetched with its inputs
+    int head[U];
+    bool second[U], in[U], live[U];      // second: a row of the values; live: this lane holds elements of the row
+    float mult[U];                       // "fp8" pages: the row's divisor, fetched with its inputs
+    // Every load of the U rows is issued before anything waits for one: no load sits under a condition (a row past the
+    // end reads row 0, a lane past a narrow row's width reads the row's start) and nothing indexes the launch arguments
+    // by a value a lane computes (which would fetch them from memory): the choice between the keys' and the values'
+    // arguments is a select between scalars.
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const uint32_t row = row0 + u * RPP;
-        const bool in = row < n_rows;
-        const int64_t t = in ? (int64_t)div32(a.heads_div, row) : 0;
-        head[u] = in ? (int)(row - (uint32_t)t * (uint32_t)a.heads) : 0;
-        which[u] = head[u] >= a.hkv ? 1 : 0;
-        head[u] -= which[u] * a.hkv;
-        slot[u] = in ? a.slots[t] : -1;
-        live[u] = in && i0 < a.dim[which[u]];
-        mult[u] = 1.0f;
-        if constexpr (KIND == 1) mult[u] = a.head_mult ? a.head_mult[which[u] * a.hkv + head[u]] : a.mult[which[u]];
-        if (live[u]) {
-            raw[u].load(a.src[which[u]], t * a.stride_t[which[u]] + head[u] * a.stride_h[which[u]] + i0);
-        } else {
-            raw[u].zero();
+        in[u] = row < n_rows;
+        const uint32_t rowc = in[u] ? row : 0;
+        const uint32_t t = div32(a.heads_div, rowc);
+        const int h = (int)(rowc - t * (uint32_t)a.heads);
+        second[u] = h >= a.hkv;
+        head[u] = second[u] ? h - a.hkv : h;
+        live[u] = in[u] && i0 < (second[u] ? a.dim[1] : a.dim[0]);
+        slot[u] = a.slots[t];
+        mult[u] = second[u] ? a.mult[1] : a.mult[0];
+        if constexpr (KIND == 1) {
+            if (a.head_mult) mult[u] = a.head_mult[(second[u] ? a.hkv : 0) + head[u]];
         }
+        const void* src = second[u] ? a.src[1] : a.src[0];
+        const int64_t st = second[u] ? a.stride_t[1] : a.stride_t[0], sh = second[u] ? a.stride_h[1] : a.stride_h[0];
+        raw[u].load(src, (int64_t)t * st + head[u] * sh + (live[u] ? i0 : 0));
     }
+    __builtin_amdgcn_sched_barrier(0);      // (nothing that waits for a load moves up among the loads)
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-        // (a whole row's lanes agree on slot[u] < 0, so the row-scale exchange below stays among participating lanes)
-        if (slot[u] < 0) continue;
+        // (a whole row's lanes agree on these, so the row-scale exchange below stays among participating lanes)
+        if (!in[u] || slot[u] < 0) continue;
+        if constexpr (KIND >= 2) {
+            if (!live[u]) raw[u].zero();      // the row's maximum is over its own elements
+        }
         float x[EPL];
         raw[u].widen(x);
-        const int dim = a.dim[which[u]];
+        const int dim = second[u] ? a.dim[1] : a.dim[0];
+        void* const pages = second[u] ? a.pages[1] : a.pages[0];
+        float* const scales = second[u] ? a.scales[1] : a.scales[0];
         const int64_t dst = (slot[u] * a.hkv + head[u]) * dim + i0;
         if constexpr (KIND == 0) {
             uint4 v;
@@ -158,7 +162,7 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
             } else {
                 v = make_uint4(pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]), pack_bf16(x[6], x[7]));
             }
-            if (live[u]) __builtin_nontemporal_store(u32x4{v.x, v.y, v.z, v.w}, reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(a.pages[which[u]]) + dst));
+            if (live[u]) __builtin_nontemporal_store(u32x4{v.x, v.y, v.z, v.w}, reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(pages) + dst));
         } else {
             float div;
             bool zero_row = false;
@@ -180,7 +184,7 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
                 div = __fdiv_rn(amax, top);
                 div = div < 1e-30f ? 1e-30f : div;               // clamp(min=1e-30); NaN stays NaN
                 zero_row = amax == 0.0f;
-                if (lane_in_row == 0) a.scales[which[u]][slot[u] * a.hkv + head[u]] = div;
+                if (lane_in_row == 0) scales[slot[u] * a.hkv + head[u]] = div;
             }
             // The quotients by the shared steps of one division, straight through to the codes; where the divisor does
             // not allow that (an all-zero row's does, the 1e-30 floor: its quotients are zeros of the inputs' signs
@@ -210,10 +214,15 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
                     int packed = __builtin_amdgcn_cvt_pk_fp8_f32(c[0], c[1], 0, false);
                     w[k] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], packed, true);
                 }
+                // (four independent chains are enough to fill the pipeline; interleaving all sixteen costs the registers
+                // of two more resident wavefronts)
+                __builtin_amdgcn_sched_barrier(0);
             }
             coded = coded && sum == sum;
-            if (__builtin_expect(!coded, 0)) exact_codes<KIND>(x, div, w);
-            if (live[u]) __builtin_nontemporal_store(u32x4{w[0], w[1], w[2], w[3]}, reinterpret_cast<u32x4*>(reinterpret_cast<uint8_t*>(a.pages[which[u]]) + dst));
+#ifndef NO_COLD
+            if (__builtin_expect(!coded, 0)) exact_codes<KIND>(raw[u], div, w);
+#endif
+            if (live[u]) __builtin_nontemporal_store(u32x4{w[0], w[1], w[2], w[3]}, reinterpret_cast<u32x4*>(reinterpret_cast<uint8_t*>(pages) + dst));
         }
     }
 }
@@ -292,12 +301,13 @@ static int launch_kind(const WriteArgs& a, int lpr, bool vector, hipStream_t str
     // 8 KV heads of 16-bit pages); one row a thread below that, where the launch is latency-bound and more workgroups
     // finish sooner (at 4,152 tokens: 10.4 us against 14.2).
     const bool wide = rows * lpr >= (int64_t)1 << 21;
-    const int rows_per_block = 256 / lpr * (wide ? 4 : 1);
+    constexpr int WIDE_U = KIND == 0 ? PKV_WIDE_U16 : PKV_WIDE_U8;
+    const int rows_per_block = 256 / lpr * (wide ? WIDE_U : 1);
     const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
     switch (lpr) {
 #define PKV_CASE(L)                                                                                                 \
     case L:                                                                                                         \
-        if (wide) hipLaunchKernelGGL((write_rows<KIND, F16, IN, L, 4>), dim3((unsigned)blocks), dim3(256), 0, stream, a); \
+        if (wide) hipLaunchKernelGGL((write_rows<KIND, F16, IN, L, WIDE_U>), dim3((unsigned)blocks), dim3(256), 0, stream, a); \
         else hipLaunchKernelGGL((write_rows<KIND, F16, IN, L, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, a);      \
         break;
         PKV_CASE(1) PKV_CASE(2) PKV_CASE(4) PKV_CASE(8) PKV_CASE(16) PKV_CASE(32) PKV_CASE(64)
