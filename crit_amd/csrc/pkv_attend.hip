@@ -24,7 +24,7 @@ __global__ __launch_bounds__(64) void merge_kernel(AttendArgs a) {
     int64_t first = a.firsts[r];
     first = first < 0 ? 0 : (first > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first);
     const int64_t seen = min(first + c + 1, (int64_t)a.max_keys);
-    const int nb = (int)min((int64_t)a.parts, (seen + a.piece - 1) / a.piece);
+    const int nb = (int)min((uint32_t)a.parts, ((uint32_t)seen + (uint32_t)a.piece - 1u) / (uint32_t)a.piece);      // (32-bit: seen <= max_keys)
     const int64_t prow = a.offsets ? (int64_t)(a.offsets[r] - a.offsets[0]) : (int64_t)r * a.columns;
     const int64_t at = ((prow + c) * a.hq + head) * a.parts;
     float M = -INFINITY, L = 0.0f, A[EPL];
@@ -105,12 +105,20 @@ __global__ __launch_bounds__(64) void shard_merge_kernel(crit_pkv_merge_params p
 __global__ __launch_bounds__(256) void stream_read_kernel(const uint4* data, int64_t vecs, float* sink) {
     uint32_t acc = 0;
     const int64_t stride = (int64_t)gridDim.x * 256 * 4;
-    for (int64_t i = (int64_t)blockIdx.x * 256 * 4 + threadIdx.x; i < vecs; i += stride) {
-        uint4 v0 = data[i], v1 = make_uint4(0, 0, 0, 0), v2 = v1, v3 = v1;
-        if (i + 256 < vecs) v1 = data[i + 256];
-        if (i + 512 < vecs) v2 = data[i + 512];
-        if (i + 768 < vecs) v3 = data[i + 768];
+    int64_t i = (int64_t)blockIdx.x * 256 * 4 + threadIdx.x;
+    // Whole passes: four loads a thread, none under a condition, so all four are in flight together.
+    for (; i + 768 < vecs; i += stride) {
+        const u32x4* p = reinterpret_cast<const u32x4*>(data) + i;
+        const u32x4 v0 = __builtin_nontemporal_load(p), v1 = __builtin_nontemporal_load(p + 256);
+        const u32x4 v2 = __builtin_nontemporal_load(p + 512), v3 = __builtin_nontemporal_load(p + 768);
         acc ^= v0.x ^ v0.y ^ v0.z ^ v0.w ^ v1.x ^ v1.y ^ v1.z ^ v1.w ^ v2.x ^ v2.y ^ v2.z ^ v2.w ^ v3.x ^ v3.y ^ v3.z ^ v3.w;
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {      // the last, partial pass of the workgroup that holds the end
+        if (i + 256 * k < vecs) {
+            const uint4 v = data[i + 256 * k];
+            acc ^= v.x ^ v.y ^ v.z ^ v.w;
+        }
     }
     if (acc == 0x12345678u) sink[threadIdx.x & 63] = 1.0f;    // keeps the loads alive; practically never taken
 }

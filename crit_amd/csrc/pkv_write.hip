@@ -4,13 +4,6 @@
 #include "pkv_common.hpp"
 #include "pkv_launch.hpp"
 
-#ifndef PKV_WIDE_U16
-#define PKV_WIDE_U16 4
-#endif
-#ifndef PKV_WIDE_U8
-#define PKV_WIDE_U8 2
-#endif
-
 namespace pkv {
 
 struct WriteArgs {
@@ -102,7 +95,9 @@ PKV_DEV void exact_codes(const Row& row, float div, uint32_t (&w)[4]) {
 // One row = (token, head) with head in [0, heads): keys' heads first, then values'. LPR lanes hold one row, EPL
 // elements each (16 bytes of page row). KIND as in the ABI; F16: 16-bit pages are fp16, not bf16. A thread takes U rows,
 // 256 / LPR apart (so a workgroup's accesses stay contiguous per pass), and issues all their loads before the first
-// store: U times the bytes in flight per thread, which is what a streaming copy on this card needs.
+// store. The launcher gives every thread one row: with the loads free of conditions and 46-52 registers a thread, eight
+// wavefronts a SIMD are resident, and more, shorter workgroups measured faster than more rows a thread at every size
+// (262,144 tokens of 8 KV heads, bf16: 389 us with one row, 397 with two, 413 with four).
 template <int KIND, bool F16, int IN, int LPR, int U>
 __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
     constexpr int EPL = KIND == 0 ? 8 : 16;
@@ -297,18 +292,12 @@ static int launch_kind(const WriteArgs& a, int lpr, bool vector, hipStream_t str
         return 0;
     }
     const int64_t rows = a.tokens * a.heads;
-    // Four rows a thread once there is work for every compute unit many times over (2^21 lane-rows: 16,384 tokens of
-    // 8 KV heads of 16-bit pages); one row a thread below that, where the launch is latency-bound and more workgroups
-    // finish sooner (at 4,152 tokens: 10.4 us against 14.2).
-    const bool wide = rows * lpr >= (int64_t)1 << 21;
-    constexpr int WIDE_U = KIND == 0 ? PKV_WIDE_U16 : PKV_WIDE_U8;
-    const int rows_per_block = 256 / lpr * (wide ? WIDE_U : 1);
+    const int rows_per_block = 256 / lpr;
     const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
     switch (lpr) {
 #define PKV_CASE(L)                                                                                                 \
     case L:                                                                                                         \
-        if (wide) hipLaunchKernelGGL((write_rows<KIND, F16, IN, L, WIDE_U>), dim3((unsigned)blocks), dim3(256), 0, stream, a); \
-        else hipLaunchKernelGGL((write_rows<KIND, F16, IN, L, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, a);      \
+        hipLaunchKernelGGL((write_rows<KIND, F16, IN, L, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, a);       \
         break;
         PKV_CASE(1) PKV_CASE(2) PKV_CASE(4) PKV_CASE(8) PKV_CASE(16) PKV_CASE(32) PKV_CASE(64)
 #undef PKV_CASE

@@ -44,9 +44,9 @@ def test_writes_encode_as_torch_does_and_skip_negative_slots(kind, d, dv, in_dty
 @pytest.mark.parametrize("T", [4152, 33001])
 @pytest.mark.parametrize("kind", ["bf16", "fp8", "fp8:row", "int8"])
 def test_a_large_append_with_edge_values_is_bit_exact(kind, T):
-    # 4,152 tokens (the mixed prefill + decode batch's append) and 33,001 (a launch large enough for the kernel that
-    # gives a thread four rows; an odd count, so its last workgroups are ragged), 8 KV heads, with the values that
-    # break sloppy encoders: signed zeros, the subnormal ties, saturation, infinities, 1% outliers x20.
+    # 4,152 tokens (the mixed prefill + decode batch's append) and 33,001 (an odd count, so the last workgroup is
+    # ragged, over thousands of workgroups), 8 KV heads, with the values that break sloppy encoders: signed zeros, the
+    # subnormal ties, saturation, infinities, 1% outliers x20.
     pk = kernels()
     g = torch.Generator().manual_seed(2)
     hkv, d = 8, 128
