@@ -27,6 +27,22 @@
 
 namespace pkv {
 
+// A 16-byte (or 8-byte) load of value rows, which are read once: nontemporal, so the caches do not keep them (measured
+// +4 % on the decode launch; the same hint on the key rows measured -1 %, so those stay plain loads).
+PKV_DEV uint4 load_once16(const uint8_t* p) {
+    const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+PKV_DEV uint2 load_once8(const uint8_t* p) {
+    const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
+    return make_uint2(v.x, v.y);
+}
+
+// A workgroup barrier that orders the shared arrays only: a wavefront waits for its own LDS traffic, then for the
+// others. __syncthreads() would also wait until the wavefront's global stores (a unit's partials, which only the next
+// kernel reads) have drained, a memory round trip at every barrier of a unit's end.
+PKV_DEV void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // DPP controls inside a row of 16 lanes.
 constexpr int kXor1 = 0xB1, kXor2 = 0x4E, kRor4 = 0x124, kRor8 = 0x128, kRor12 = 0x12C;
 
@@ -115,10 +131,17 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
     int b = uy;
     // The row's four descriptors are read together, ahead of every test that could end the unit: one memory round
     // trip instead of a chain of them at the start of every unit.
-    const int count_in = a.counts ? a.counts[r] : a.columns;
-    const int64_t first64 = a.firsts[r];
-    const int64_t trow = (int64_t)a.rows[r] * a.tab_stride;
-    const int start = a.starts[r];
+    int count_raw = *(a.counts ? a.counts + r : a.starts + r);      // (no load under a condition)
+    int64_t first64 = a.firsts[r];
+    int table_row = a.rows[r];
+    int start = a.starts[r];
+    int off_r = *(a.offsets ? a.offsets + r : a.starts + r), off_0 = *(a.offsets ? a.offsets : a.starts);
+    // (the values are taken together here, which keeps the compiler from sinking some of the loads below the tests
+    // that follow, or down to the unit's end where the partials' rows are computed: one round trip, not several)
+    asm volatile("" : "+v"(count_raw), "+v"(first64), "+v"(table_row), "+v"(start), "+v"(off_r), "+v"(off_0));
+    const int64_t prow = a.offsets ? (int64_t)(off_r - off_0) : (int64_t)r * a.columns;      // the row's first partial row
+    const int count_in = a.counts ? count_raw : a.columns;
+    const int64_t trow = (int64_t)table_row * a.tab_stride;
     const int count = min(count_in, a.columns);
     const int j0 = tile * QR;
     if (j0 >= count * a.g) return;
@@ -145,27 +168,6 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
         }
     }
 
-    // The lane's slices of the tile's query rows (packed 16-bit pairs): dims 8 li8 .. +7 and 64 + 8 li8 .. +7 over
-    // 16-bit pages, dims 16 li8 .. +15 over 8-bit pages (the dims its K loads cover).
-    uint32_t qp[QR][8];
-#pragma unroll
-    for (int rr = 0; rr < QR; ++rr) {
-        const int j = j0 + rr;
-        const int c = j / a.g;
-        uint4 w0 = make_uint4(0, 0, 0, 0), w1 = w0;
-        if (c < count) {
-            const uint8_t* row = a.q + ((int64_t)(start + c) * a.q_st + (int64_t)(kvh * a.g + j % a.g) * a.q_sh) * 2;
-            if constexpr (KIND == 0) {
-                w0 = *reinterpret_cast<const uint4*>(row + li8 * 16);
-                w1 = *reinterpret_cast<const uint4*>(row + 128 + li8 * 16);
-            } else {
-                w0 = *reinterpret_cast<const uint4*>(row + li8 * 32);
-                w1 = *reinterpret_cast<const uint4*>(row + li8 * 32 + 16);
-            }
-        }
-        qp[rr][0] = w0.x, qp[rr][1] = w0.y, qp[rr][2] = w0.z, qp[rr][3] = w0.w;
-        qp[rr][4] = w1.x, qp[rr][5] = w1.y, qp[rr][6] = w1.z, qp[rr][7] = w1.w;
-    }
     // The query row of this lane's score in each block, and the last position it sees.
     int my_lim[RB];
 #pragma unroll
@@ -241,17 +243,80 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
             for (int kv = 0; kv < 4; ++kv) o[kv] = (uint32_t)(min(voff[kv], n_keys - 1 - base) * slot_bytes) + vlane;
         }
 #pragma unroll
-        for (int kv = 0; kv < 4; ++kv) buf.v[kv] = *reinterpret_cast<const typename Step128<KIND>::VVec*>(sbase + o[kv]);
+        for (int kv = 0; kv < 4; ++kv) {
+            if constexpr (KIND == 0) buf.v[kv] = load_once16(sbase + o[kv]);
+            else buf.v[kv] = load_once8(sbase + o[kv]);
+        }
     };
 
+    // A wavefront's walk over a partition's steps, and the first three steps of the unit's first partition with their
+    // page table entries: those loads go out ahead of the query loads, so the keys and values wait for one memory round
+    // trip after the descriptors, not for the queries' and then the entries'.
+    int pi, st;
+    auto start_part = [&](int part) __attribute__((always_inline)) {
+        pi = part, st = wave;
+        if (win > 0) {
+            const int wlo = first + c_lo - win + 1;
+            const int below = (wlo > 0 ? wlo : 0) / a.piece - part;
+            if (below > 0) pi = part + (below + a.parts - 1) / a.parts * a.parts;
+        }
+    };
+    auto base_of = [&]() __attribute__((always_inline)) -> int {
+        if (st * SPW >= a.piece) return -1;
+        const int64_t base = (int64_t)pi * a.piece + st * SPW;
+        return base < n_keys ? (int)base : -1;
+    };
+    auto advance = [&]() __attribute__((always_inline)) -> int {
+        st += 4;
+        if (st * SPW >= a.piece) pi += a.parts, st = wave;
+        return base_of();
+    };
+    struct Lead {
+        int base0, base1, base2, e0, e1, e2;
+    };
+    auto lead_of = [&](int part) __attribute__((always_inline)) -> Lead {
+        Lead f;
+        start_part(part);
+        f.base0 = base_of();
+        const int again = f.base0 >= 0 ? f.base0 : 0;      // (a wavefront without a step reads position 0's entry)
+        f.e0 = entry(again);
+        f.base1 = f.base0 >= 0 ? advance() : -1;
+        f.e1 = entry(f.base1 >= 0 ? f.base1 : again);
+        f.base2 = f.base1 >= 0 ? advance() : -1;
+        f.e2 = entry(f.base2 >= 0 ? f.base2 : again);
+        return f;
+    };
+    const int part_lo = FUSED ? 0 : b;
+    const int part_hi = FUSED ? min(a.parts, n_pieces) : b + 1;
+    const Lead lead_first = lead_of(part_lo);
+
+    // The lane's slices of the tile's query rows (packed 16-bit pairs): dims 8 li8 .. +7 and 64 + 8 li8 .. +7 over
+    // 16-bit pages, dims 16 li8 .. +15 over 8-bit pages (the dims its K loads cover).
+    uint32_t qp[QR][8];
+#pragma unroll
+    for (int rr = 0; rr < QR; ++rr) {
+        const int j = j0 + rr;
+        const int c = j / a.g;
+        uint4 w0 = make_uint4(0, 0, 0, 0), w1 = w0;
+        if (c < count) {
+            const uint8_t* row = a.q + ((int64_t)(start + c) * a.q_st + (int64_t)(kvh * a.g + j % a.g) * a.q_sh) * 2;
+            if constexpr (KIND == 0) {
+                w0 = *reinterpret_cast<const uint4*>(row + li8 * 16);
+                w1 = *reinterpret_cast<const uint4*>(row + 128 + li8 * 16);
+            } else {
+                w0 = *reinterpret_cast<const uint4*>(row + li8 * 32);
+                w1 = *reinterpret_cast<const uint4*>(row + li8 * 32 + 16);
+            }
+        }
+        qp[rr][0] = w0.x, qp[rr][1] = w0.y, qp[rr][2] = w0.z, qp[rr][3] = w0.w;
+        qp[rr][4] = w1.x, qp[rr][5] = w1.y, qp[rr][6] = w1.z, qp[rr][7] = w1.w;
+    }
     float run_m[FUSED ? HW : 1][EPT], run_l[FUSED ? HW : 1][EPT], run_a[FUSED ? HW : 1][EPT];
 #pragma unroll
     for (int i = 0; i < (FUSED ? HW : 1); ++i)
 #pragma unroll
         for (int e = 0; e < EPT; ++e) run_m[i][e] = -INFINITY, run_l[i][e] = 0.0f, run_a[i][e] = 0.0f;
 
-    const int part_lo = FUSED ? 0 : b;
-    const int part_hi = FUSED ? min(a.parts, n_pieces) : b + 1;
     for (int part = part_lo; part < part_hi; ++part) {
         // Per DPP row: the running maximum and sum of the query row this lane's score belongs to (per block), and the
         // row's output accumulators for the lane's 8 value dims.
@@ -262,23 +327,6 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
         for (int rr = 0; rr < QR; ++rr)
 #pragma unroll
             for (int d = 0; d < 8; ++d) acc[rr][d] = 0.0f;
-
-        int pi = part, st = wave;
-        if (win > 0) {
-            const int wlo = first + c_lo - win + 1;
-            const int below = (wlo > 0 ? wlo : 0) / a.piece - part;
-            if (below > 0) pi = part + (below + a.parts - 1) / a.parts * a.parts;
-        }
-        auto base_of = [&]() __attribute__((always_inline)) -> int {
-            if (st * SPW >= a.piece) return -1;
-            const int64_t base = (int64_t)pi * a.piece + st * SPW;
-            return base < n_keys ? (int)base : -1;
-        };
-        auto advance = [&]() __attribute__((always_inline)) -> int {
-            st += 4;
-            if (st * SPW >= a.piece) pi += a.parts, st = wave;
-            return base_of();
-        };
 
         // Scores and softmax of one step: leaves the step's probabilities (pairs of adjacent positions per query row)
         // in pp and has rescaled the accumulators where a row's maximum moved.
@@ -412,15 +460,13 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
         // compiler counts the outstanding ones exactly and waits only for the step it is about to use.
         Step128<KIND> bufA, bufB;
         uint32_t pp[RB * 4][2];
-        int base0 = base_of();
+        const Lead f = part == part_lo ? lead_first : lead_of(part);
+        int base0 = f.base0, base1 = f.base1, base2 = f.base2;
         if (base0 >= 0) {
             const int again = base0;
             auto safe = [&](int base) __attribute__((always_inline)) { return base >= 0 ? base : again; };
-            int e0 = entry(base0);
-            int base1 = advance();
-            int e1 = entry(safe(base1));
-            int base2 = base1 >= 0 ? advance() : -1;
-            int e2 = entry(safe(base2));
+            const int e0 = f.e0, e1 = f.e1;
+            int e2 = f.e2;
             fetch_k(base0, e0, bufA), fetch_v(base0, e0, bufA);
             fetch_k(safe(base1), e1, bufB), fetch_v(safe(base1), e1, bufB);
             for (;;) {
@@ -474,7 +520,7 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
         // Then the four wavefronts, one head of the wavefront at a time through LDS, in wavefront order.
 #pragma unroll
         for (int head_i = 0; head_i < HW; ++head_i) {
-            if (FUSED || head_i > 0) __syncthreads();      // the previous fold has read the LDS
+            if (FUSED || head_i > 0) lds_barrier();      // the previous fold has read the LDS
             if (rho == head_i) {
 #pragma unroll
                 for (int rr = 0; rr < QR; ++rr) {
@@ -483,7 +529,7 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
                     if (lam == 0) s_m[wave][rr] = wm[rr], s_l[wave][rr] = wl[rr];
                 }
             }
-            __syncthreads();
+            lds_barrier();
             const int head_kv = (kvh - hw) + head_i;      // the KV head being folded (uniform)
             float vm = a.v_mult;
             if (KIND == 1 && a.hm) vm = a.hm[a.hkv + head_kv];
@@ -516,7 +562,6 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
                                 run_m[head_i][e] = f.m, run_l[head_i][e] = f.l;
                             }
                         } else {
-                            const int64_t prow = a.offsets ? (int64_t)(a.offsets[r] - a.offsets[0]) : (int64_t)r * a.columns;
                             const int64_t at = ((prow + c) * a.hq + head_kv * a.g + j % a.g) * a.parts + b;
                             a.po[at * D + d] = A;
                             if (d == 0) a.pm[at] = M, a.pl[at] = L;
@@ -570,9 +615,9 @@ __global__ __launch_bounds__(256, attend_waves(KIND, QR)) void attend128_kernel(
         // (the next ticket is drawn after the unit, not during it: a returning atomic in flight makes every wait on
         // the unit's loads a wait for all of them, which costs more than the ticket's round trip)
         attend128_unit<KIND, F16, QR, HW, FUSED>(a, (int)(u % (unsigned)a.units_x), (int)(u / (unsigned)a.units_x));
-        __syncthreads();      // the unit is done with the shared arrays, and every thread has read s_unit
+        lds_barrier();      // the unit is done with the shared arrays, and every thread has read s_unit
         if (threadIdx.x == 0) s_unit = gridDim.x + atomicAdd(a.ticket, 1u);
-        __syncthreads();
+        lds_barrier();
         u = s_unit;
     }
     if (threadIdx.x == 0) {
