@@ -139,6 +139,12 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
     // (the values are taken together here, which keeps the compiler from sinking some of the loads below the tests
     // that follow, or down to the unit's end where the partials' rows are computed: one round trip, not several)
     asm volatile("" : "+v"(count_raw), "+v"(first64), "+v"(table_row), "+v"(start), "+v"(off_r), "+v"(off_0));
+    // (they are the same in every lane, which the compiler cannot see through the line above: as scalars again, the
+    // walk over the row's steps and its page table entries stays on the scalar unit)
+    count_raw = __builtin_amdgcn_readfirstlane(count_raw), table_row = __builtin_amdgcn_readfirstlane(table_row);
+    start = __builtin_amdgcn_readfirstlane(start), off_r = __builtin_amdgcn_readfirstlane(off_r), off_0 = __builtin_amdgcn_readfirstlane(off_0);
+    first64 = (int64_t)(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(first64 >> 32)) << 32) |
+                        (uint32_t)__builtin_amdgcn_readfirstlane((int)first64));
     const int64_t prow = a.offsets ? (int64_t)(off_r - off_0) : (int64_t)r * a.columns;      // the row's first partial row
     const int count_in = a.counts ? count_raw : a.columns;
     const int64_t trow = (int64_t)table_row * a.tab_stride;
