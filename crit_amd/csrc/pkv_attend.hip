@@ -24,7 +24,9 @@ __global__ __launch_bounds__(64) void merge_kernel(AttendArgs a) {
     int64_t first = a.firsts[r];
     first = first < 0 ? 0 : (first > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first);
     const int64_t seen = min(first + c + 1, (int64_t)a.max_keys);
-    const int nb = (int)min((uint32_t)a.parts, ((uint32_t)seen + (uint32_t)a.piece - 1u) / (uint32_t)a.piece);      // (32-bit: seen <= max_keys)
+    // (32-bit: seen <= max_keys; with block lists the partitions divide the list's run, the same for every column)
+    const uint32_t run = a.blocks ? (uint32_t)a.listed_keys : (uint32_t)seen;
+    const int nb = (int)min((uint32_t)a.parts, (run + (uint32_t)a.piece - 1u) / (uint32_t)a.piece);
     const int64_t prow = a.offsets ? (int64_t)(a.offsets[r] - a.offsets[0]) : (int64_t)r * a.columns;
     const int64_t at = ((prow + c) * a.hq + head) * a.parts;
     float M = -INFINITY, L = 0.0f, A[EPL];
@@ -215,6 +217,12 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     if (p->partitions < 1 || p->partitions > 65535 || p->piece < 1 || p->piece % sp) return CRIT_PKV_E_WORKSPACE;
     if (!p->fused && (!p->partial_out || !p->partial_max || !p->partial_sum)) return CRIT_PKV_E_WORKSPACE;
     if (p->parents && p->parents64) return CRIT_PKV_E_NULL;
+    if (p->blocks) {
+        if (p->fused || p->sliding) return CRIT_PKV_E_GEOMETRY;
+        if (p->blocks_k < 1 || p->blocks_k > kMaxListedBlocks || p->block_size < 1 || p->blocks_stride < p->blocks_k ||
+            (int64_t)p->blocks_k * p->block_size > 0x3fffffff)
+            return CRIT_PKV_E_GEOMETRY;
+    }
     if ((p->parents || p->parents64) && p->columns > 64) return CRIT_PKV_E_GEOMETRY;      // an ancestor set is a 64-bit mask
     AttendArgs a;
     a.q = reinterpret_cast<const uint8_t*>(p->q);
@@ -226,6 +234,9 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     a.po = p->partial_out, a.pm = p->partial_max, a.pl = p->partial_sum;
     a.out = p->out, a.lse = p->lse, a.sinks = p->sinks;
     a.parents = p->parents, a.parents64 = p->parents64;
+    a.blocks = p->blocks, a.blocks_stride = p->blocks_stride, a.blocks_k = p->blocks_k, a.block_size = p->block_size;
+    a.listed_keys = p->blocks ? p->blocks_k * p->block_size : 0;
+    a.block_div = make_div32(p->blocks ? (uint32_t)p->block_size : 1u);
     a.q_st = p->q_stride_t, a.q_sh = p->q_stride_h, a.o_st = p->out_stride_t, a.o_sh = p->out_stride_h, a.tab_stride = p->table_stride;
     a.tab_width = p->table_width, a.n_rows = p->n_rows, a.columns = p->columns, a.hq = p->heads, a.hkv = p->kv_heads;
     a.g = p->heads / p->kv_heads;
@@ -236,12 +247,17 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     a.parts = p->partitions, a.piece = p->piece, a.sliding = p->sliding, a.out_dtype = p->out_dtype;
     a.sscale = p->scale * kLog2e, a.k_mult = p->key_multiplier, a.v_mult = p->value_multiplier;
     const int live_rows = p->columns * a.g;
-    const int qr = pick_qr(live_rows);
+    int qr = pick_qr(live_rows);
+    if (p->blocks) {      // a tile of one column's rows: the largest tile height that divides the group
+        qr = 1;
+        for (int q : {2, 4, 5, 6, 8})
+            if (a.g % q == 0) qr = q;
+    }
     a.tiles = (live_rows + qr - 1) / qr;
     // The 128-wide kernel serves two adjacent KV heads per wavefront where the head count is even, so every position
     // is read in segments of two rows (512 bytes of 16-bit pages, 256 of 8-bit ones): measured best on MI355X against
     // one and four heads. Fixed by the cache's geometry, never by the launch: a column's bits depend on it.
-    const bool page16 = p->page % 16 == 0;
+    const bool page16 = p->page % 16 == 0 && !p->blocks;      // (block lists: the generic kernel, positions looked up one by one)
     a.heads_per_wave = 1;
     if (lpr == 16 && page16) {
         if (p->kv_heads % 2 == 0) a.heads_per_wave = 2;
@@ -251,7 +267,7 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     // Positions past the page tables do not exist: partitions that could only hold such pieces are not launched.
     const int64_t table_keys = (int64_t)p->table_width * p->page;
     a.max_keys = (int)(table_keys < 0x3fffffff ? table_keys : 0x3fffffff);
-    const int64_t live_parts = (a.max_keys + (int64_t)p->piece - 1) / p->piece;
+    const int64_t live_parts = ((p->blocks ? (int64_t)a.listed_keys : (int64_t)a.max_keys) + (int64_t)p->piece - 1) / p->piece;
     const unsigned gy = (unsigned)(live_parts < p->partitions ? live_parts : p->partitions);
     const dim3 grid((unsigned)gx, p->fused ? 1u : gy);
     a.units_x = a.units_y = 0;

@@ -6,6 +6,8 @@
 
 namespace pkv {
 
+constexpr int kMaxListedBlocks = 1024;      // block ids a token's list may hold (they are copied to LDS)
+
 struct AttendArgs {
     const uint8_t* q;
     const uint8_t* kp;
@@ -27,9 +29,12 @@ struct AttendArgs {
     const float* sinks;
     const int32_t* parents;      // draft trees: each token's parent column, int32 ...
     const int64_t* parents64;    // ... or int64; both null: plain causal windows
+    const int32_t* blocks;       // block-sparse lists [tokens][blocks_k], or null: every position
     unsigned* ticket;      // two zeroed counters of the unit-pulling launches: next unit, workgroups done
-    int64_t q_st, q_sh, o_st, o_sh, tab_stride;
+    int64_t q_st, q_sh, o_st, o_sh, tab_stride, blocks_stride;
     int tab_width, n_rows, columns, hq, hkv, g, page, page_shift, parts, piece, sliding, out_dtype, tiles, max_keys, heads_per_wave, units_x, units_y;
+    int blocks_k, block_size, listed_keys;      // listed_keys = blocks_k * block_size: the positions a list's run holds
+    Div32 block_div;
     float sscale, k_mult, v_mult;
 };
 

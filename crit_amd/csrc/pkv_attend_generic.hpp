@@ -8,6 +8,12 @@
 // its own online-softmax state over the positions it reads; the groups and the four wavefronts are folded at the
 // end in a fixed order, then the partition's state goes to the partials (or, fused, into the running state).
 //
+// SPARSE: block lists. A tile then holds rows of ONE column (the launcher picks QR dividing the group), whose list of
+// block ids is copied to LDS; the positions read are the run u = 0 .. blocks_k * block_size - 1 of the list, position
+// n(u) = blocks[u / block_size] * block_size + u % block_size, cut into pieces and partitions like an ordinary row's
+// positions; an id of -1, a position past the column's own or past the page tables is masked. Only listed blocks are
+// read. (Not fused, no sliding window: the launcher refuses those.)
+//
 // A column's bits depend on its own query, its own keys, `piece`, `partitions` and the page kind only: position n is
 // always read by the same wavefront, lane group and step whatever the launch, masked positions contribute exact
 // zeros, and every sum is an explicit FMA chain in a fixed order (built with -ffp-contract=off).
@@ -21,10 +27,13 @@ struct StepBuf {
     using Vec = typename std::conditional<KIND == 0, uint4, uint2>::type;
     Vec k[4], v[4];
     float ks[4], vs[4];
+    int pos[4];      // SPARSE: the position each of the lane group's four rows holds, -1 for none
 };
 
-template <int KIND, bool F16, int LPR, int QR, bool FUSED>
+
+template <int KIND, bool F16, int LPR, int QR, bool FUSED, bool SPARSE = false>
 __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
+    static_assert(!(SPARSE && FUSED), "block lists are read by the split launch");
     constexpr int D = LPR * 8;
     constexpr int PPI = 64 / LPR;      // positions one load instruction of a wavefront covers
     constexpr int SP = 4 * PPI;        // positions a wavefront's step covers
@@ -32,6 +41,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
     constexpr int EPT = (QR * D + 255) / 256;   // output elements a thread folds
     __shared__ __align__(16) float s_acc[4][QR][D];
     __shared__ float s_m[4][QR], s_l[4][QR];
+    __shared__ int s_blocks[SPARSE ? kMaxListedBlocks : 1];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lg = lane / LPR, li = lane % LPR;
     int bx = blockIdx.x;
@@ -51,10 +61,24 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
     nk64 = nk64 < 0 ? 0 : (nk64 > (int64_t)a.max_keys ? (int64_t)a.max_keys : nk64);
     const int n_keys = (int)nk64;
     const int first = (int)(first64 < 0 ? 0 : (first64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first64));
-    const int n_pieces = (n_keys + a.piece - 1) / a.piece;
+    const int n_run = SPARSE ? a.listed_keys : n_keys;      // the positions the partitions divide among them
+    const int n_pieces = (n_run + a.piece - 1) / a.piece;
     if (!FUSED && b >= n_pieces) return;
     const int64_t trow = (int64_t)a.rows[r] * a.tab_stride;
     const int start = a.starts[r];
+    if constexpr (SPARSE) {      // the tile's column's list (QR divides the group: one column a tile)
+        const int32_t* list = a.blocks + (int64_t)(start + c_lo) * a.blocks_stride;
+        for (int i = tid; i < a.blocks_k; i += 256) s_blocks[i] = list[i];
+        __syncthreads();
+    }
+    // SPARSE: the position behind place u of the list's run, -1 for none.
+    auto listed = [&](int u) __attribute__((always_inline)) -> int {
+        if (u >= a.listed_keys) return -1;
+        const int e = (int)div32(a.block_div, (uint32_t)u);
+        const int id = s_blocks[e];
+        const int64_t n = (int64_t)id * a.block_size + (u - e * a.block_size);
+        return (id >= 0 && n < n_keys) ? (int)n : -1;
+    };
 
     // The tile's rows: column, query head, last visible position.
     int lim[QR];
@@ -101,21 +125,31 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
     const uint8_t* vbase = a.vp + ((int64_t)kvh * D + li * 8) * EB;
     const int64_t slot_bytes = (int64_t)a.hkv * D * EB;
 
-    auto fetch_tab = [&](int base, int (&tab)[4]) {
+    auto fetch_tab = [&](int base, int (&tab)[4], int (&pos)[4]) {
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             int n = base + k * PPI + lg;
-            n = n < n_keys ? n : n_keys - 1;
+            if constexpr (SPARSE) {
+                pos[k] = listed(n);
+                n = pos[k] >= 0 ? pos[k] : 0;      // (a masked place reads position 0: any valid address)
+            } else {
+                n = n < n_keys ? n : n_keys - 1;
+            }
             int pidx = a.page_shift >= 0 ? (n >> a.page_shift) : (n / a.page);
             pidx = pidx < a.tab_width ? pidx : a.tab_width - 1;
             tab[k] = a.tables[trow + pidx];
         }
     };
-    auto fetch_kv = [&](int base, const int (&tab)[4], StepBuf<KIND>& buf) {
+    auto fetch_kv = [&](int base, const int (&tab)[4], const int (&pos)[4], StepBuf<KIND>& buf) {
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             int n = base + k * PPI + lg;
-            n = n < n_keys ? n : n_keys - 1;
+            if constexpr (SPARSE) {
+                buf.pos[k] = pos[k];
+                n = pos[k] >= 0 ? pos[k] : 0;
+            } else {
+                n = n < n_keys ? n : n_keys - 1;
+            }
             const int in_page = a.page_shift >= 0 ? (n & (a.page - 1)) : (n % a.page);
             const int64_t slot = (int64_t)tab[k] * a.page + in_page;
             buf.k[k] = *reinterpret_cast<const typename StepBuf<KIND>::Vec*>(kbase + slot * slot_bytes);
@@ -152,7 +186,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
         auto base_of = [&]() __attribute__((always_inline)) -> int {
             if (st * SP >= a.piece) return -1;
             const int64_t base = (int64_t)pi * a.piece + st * SP;
-            return base < n_keys ? (int)base : -1;
+            return base < n_run ? (int)base : -1;
         };
         auto advance = [&]() __attribute__((always_inline)) -> int {
             st += 4;
@@ -203,9 +237,10 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
                 float top = -INFINITY;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    const int n = base + k * PPI + lg;
+                    const int n = SPARSE ? buf.pos[k] : base + k * PPI + lg;
                     float x = s[k][rr] * (KIND >= 2 ? sscale * buf.ks[k] : sscale);
                     bool vis = n <= lim[rr] && n < n_keys;
+                    if constexpr (SPARSE) vis = vis && n >= 0;
                     if (tree) vis = vis && (n < first || ((anc[rr] >> ((n - first) & 63)) & 1ull) != 0);
                     if (win > 0) vis = vis && n > lim[rr] - win;
                     x = vis ? x : -INFINITY;
@@ -257,21 +292,21 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
 
         // Three-stage software pipeline: table entries two steps ahead, K/V one step ahead, compute.
         StepBuf<KIND> bufA, bufB;
-        int tabA[4], tabB[4];
+        int tabA[4], tabB[4], posA[4], posB[4];
         int base0 = base_of();
-        if (base0 >= 0) fetch_tab(base0, tabA);
+        if (base0 >= 0) fetch_tab(base0, tabA, posA);
         int base1 = base0 >= 0 ? advance() : -1;
-        if (base0 >= 0) fetch_kv(base0, tabA, bufA);
-        if (base1 >= 0) fetch_tab(base1, tabB);
+        if (base0 >= 0) fetch_kv(base0, tabA, posA, bufA);
+        if (base1 >= 0) fetch_tab(base1, tabB, posB);
         while (base0 >= 0) {
             int base2 = base1 >= 0 ? advance() : -1;
-            if (base1 >= 0) fetch_kv(base1, tabB, bufB);
-            if (base2 >= 0) fetch_tab(base2, tabA);
+            if (base1 >= 0) fetch_kv(base1, tabB, posB, bufB);
+            if (base2 >= 0) fetch_tab(base2, tabA, posA);
             compute(base0, bufA);
             if (base1 < 0) break;
             base0 = base2 >= 0 ? advance() : -1;
-            if (base2 >= 0) fetch_kv(base2, tabA, bufA);
-            if (base0 >= 0) fetch_tab(base0, tabB);
+            if (base2 >= 0) fetch_kv(base2, tabA, posA, bufA);
+            if (base0 >= 0) fetch_tab(base0, tabB, posB);
             compute(base1, bufB);
             base1 = base0;
             base0 = base2;

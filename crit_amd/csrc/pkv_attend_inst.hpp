@@ -9,6 +9,17 @@ namespace pkv {
 
 template <int KIND, bool F16, int QR, bool FUSED>
 static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipStream_t stream) {
+    if constexpr (!FUSED) {
+        if (a.blocks) {      // block lists: the generic kernel reading each column's listed blocks only
+            switch (lpr) {
+                case 8: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 8, QR, false, true>), grid, dim3(256), 0, stream, a); break;
+                case 16: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 16, QR, false, true>), grid, dim3(256), 0, stream, a); break;
+                case 32: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 32, QR, false, true>), grid, dim3(256), 0, stream, a); break;
+                default: return CRIT_PKV_E_GEOMETRY;
+            }
+            return hip_code(hipGetLastError());
+        }
+    }
     if (lpr == 16 && page16) {       // pages of a multiple of 16 positions: the bandwidth path, resident workgroups pulling units
         AttendArgs u = a;
         // (a split launch lists a row's last partition twice, for the one of two size classes it falls in)

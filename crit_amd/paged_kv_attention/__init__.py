@@ -40,6 +40,7 @@ __all__ = ["KINDS", "PIECE", "MAX_COLUMNS", "Derive", "attend", "derive", "cuda_
 KINDS = {"bf16": 0, "fp16": 0, "fp8": 1, "fp8:row": 2, "int8": 3}
 PIECE = 2048         # positions per piece of FP8 or INT8 pages at a 128-wide head (piece_size)
 MAX_COLUMNS = 64     # columns of one row a launch reads
+MAX_LISTED_BLOCKS = 1024      # block ids a token's list holds at most (attend's blocks=)
 MAX_QUERY_ROWS = 8   # query rows (columns x group heads) one workgroup holds; wider windows take more tiles
 
 _DTYPE = {torch.float32: _abi.F32, torch.bfloat16: _abi.BF16, torch.float16: _abi.F16}
@@ -330,7 +331,10 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
     parents: draft trees, one int32 or int64 per token of q: its parent's column in its row's window, -1 for none,
     parents before children; a column then sees every position below its row's first and, of the window, its ancestors'
     positions and its own (a chain -1, 0, 1, ... is the plain causal window, bit for bit).
-    blocks, fresh and derive are not served. phases (a measurement's): 1 runs the split launch only, 2 the
+    blocks [tokens][k] int32 and block_size: each token's list of KV block ids (block_size positions each, -1 for none,
+    no id twice): the token sees, of its positions, only those of its listed blocks, and only they are read (a list is
+    one run of k x block_size positions cut into pieces and partitions; up to MAX_LISTED_BLOCKS ids; not with fused,
+    flash or sliding). fresh and derive are not served. phases (a measurement's): 1 runs the split launch only, 2 the
     merge only."""
     if derive is not None:
         raise _unsupported("derive= (keys derived from value rows)")
@@ -342,7 +346,18 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
         if int(columns) > 64:
             raise ValueError("a draft tree's row has at most 64 columns (a column's ancestors are a 64-bit set)")
     if blocks is not None:
-        raise _unsupported("blocks= (block-sparse lists)")
+        _require_device(blocks, "attend's blocks")
+        if fused:
+            raise ValueError("a fused launch reads windows without block lists")
+        if not block_size or int(block_size) < 1:
+            raise ValueError("block-sparse attention takes the blocks' size in positions")
+        if blocks.dtype != torch.int32 or blocks.dim() != 2 or blocks.shape[0] < q.shape[0]:
+            raise ValueError("blocks holds one list of int32 KV block ids per token of q: [tokens][k]")
+        if not 1 <= blocks.shape[1] <= MAX_LISTED_BLOCKS:
+            raise ValueError(f"a token lists 1 .. {MAX_LISTED_BLOCKS} blocks, not {blocks.shape[1]}")
+        if blocks.stride(-1) != 1:
+            blocks = blocks.contiguous()
+        flash = False      # (block lists: the split launch, as in the reference)
     if fresh is not None:
         raise _unsupported("fresh= (a prompt chunk's own rows)")
     k_kind = _check_kind(kind, key_scales)
@@ -402,6 +417,9 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
     p.out, p.lse, p.sinks = out.data_ptr(), _ptr(lse), _ptr(sinks)
     if parents is not None:
         p.parents, p.parents64 = (parents.data_ptr(), None) if parents.dtype == torch.int32 else (None, parents.data_ptr())
+    if blocks is not None:
+        p.blocks, p.blocks_stride = blocks.data_ptr(), blocks.stride(0)
+        p.blocks_k, p.block_size = int(blocks.shape[1]), int(block_size)
     p.q_stride_t, p.q_stride_h, p.out_stride_t, p.out_stride_h = q.stride(0), q.stride(1), out.stride(0), out.stride(1)
     p.table_stride, p.table_width = tables.stride(0), tables.shape[1]
     p.n_rows, p.columns, p.heads, p.kv_heads, p.head_dim, p.value_dim, p.page = R, int(columns), hq, hkv, d, dv, int(page)

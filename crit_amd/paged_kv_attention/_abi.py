@@ -10,7 +10,7 @@ import shutil
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 NAME = "libcrit_pkv.so"
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 KIND_16BIT, KIND_FP8, KIND_FP8_ROW, KIND_INT8 = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
@@ -31,12 +31,13 @@ class AttendParams(ctypes.Structure):
     _fields_ = [("q", _p), ("key_pages", _p), ("value_pages", _p), ("key_scales", _p), ("value_scales", _p),
                 ("head_multipliers", _p), ("tables", _p), ("rows", _p), ("starts", _p), ("counts", _p), ("firsts", _p),
                 ("offsets", _p), ("partial_out", _p), ("partial_max", _p), ("partial_sum", _p), ("out", _p),
-                ("lse", _p), ("sinks", _p), ("parents", _p), ("parents64", _p),
+                ("lse", _p), ("sinks", _p), ("parents", _p), ("parents64", _p), ("blocks", _p),
                 ("q_stride_t", _i64), ("q_stride_h", _i64), ("out_stride_t", _i64), ("out_stride_h", _i64),
-                ("table_stride", _i64),
+                ("table_stride", _i64), ("blocks_stride", _i64),
                 ("table_width", _i32), ("n_rows", _i32), ("columns", _i32), ("heads", _i32), ("kv_heads", _i32),
                 ("head_dim", _i32), ("value_dim", _i32), ("page", _i32), ("kind", _i32), ("page_dtype", _i32),
                 ("out_dtype", _i32), ("partitions", _i32), ("piece", _i32), ("fused", _i32), ("sliding", _i32), ("phases", _i32),
+                ("blocks_k", _i32), ("block_size", _i32),
                 ("scale", _f32), ("key_multiplier", _f32), ("value_multiplier", _f32)]
 
 

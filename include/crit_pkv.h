@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 2
+#define CRIT_PKV_ABI_VERSION 3
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -105,7 +105,15 @@ typedef struct crit_pkv_attend_params {
                                        Column c then sees every position below firsts[r] and, of the window, the
                                        positions firsts[r] + a of its ancestors a and itself. NULL, NULL: column c
                                        sees positions <= firsts[r] + c. */
+    const int32_t* blocks;          /* block-sparse lists (attend's blocks=, _kernels.py:483-556): [tokens][blocks_k] KV
+                                       block ids of block_size positions each, -1 for none, no id twice in a list. A
+                                       token then sees, of the positions above, only those of its listed blocks, which
+                                       are all the launch reads: a list is read as one run of blocks_k * block_size
+                                       positions, in pieces of `piece`, piece i in partition i % partitions, and the
+                                       merge folds min(partitions, ceil(blocks_k * block_size / piece)) partials.
+                                       NULL: every position. Not with fused or sliding. */
     int64_t q_stride_t, q_stride_h, out_stride_t, out_stride_h, table_stride;
+    int64_t blocks_stride;          /* elements between two tokens' lists */
     int32_t table_width, n_rows, columns, heads, kv_heads, head_dim, value_dim, page;
     int32_t kind, page_dtype, out_dtype;
     int32_t partitions, piece;
@@ -113,6 +121,7 @@ typedef struct crit_pkv_attend_params {
     int32_t sliding;
     int32_t phases;                 /* 0: the split launch then the merge; 1: the split launch only; 2: the merge only
                                        (for timing one kernel; ignored when fused) */
+    int32_t blocks_k, block_size;   /* ids a list (1 .. 1024), positions a block (>= 1) */
     float scale, key_multiplier, value_multiplier;
 } crit_pkv_attend_params;
 

@@ -64,16 +64,28 @@ def seen_by(first, count, c, n, parents=None, sliding=0):
     return seen
 
 
+def listed(blocks, block_size, n):
+    """Which of positions 0 .. n - 1 lie in one of a token's listed KV blocks (device_attention.py:1315-1317, the test at
+    test_paged_kv_attention.py:391-392): block ids of block_size positions each, -1 for none."""
+    ids = torch.as_tensor(blocks, dtype=torch.int64)
+    ids = ids[ids >= 0]
+    return (torch.arange(n) // block_size)[:, None].eq(ids[None, :]).any(1)
+
+
 def window_reference(q, key_pages, value_pages, kind, table, first, count, page, scale, key_scales=None,
-                     value_scales=None, multipliers=(1.0, 1.0), sliding=0, q_dtype=torch.bfloat16, parents=None):
+                     value_scales=None, multipliers=(1.0, 1.0), sliding=0, q_dtype=torch.bfloat16, parents=None,
+                     blocks=None, block_size=None):
     """One window row in float64: q [count][HQ][D] (rounded to q_dtype first, as the kernels read it) at positions
-    first .. first + count - 1 -> (out [count][HQ][DV], lse [count][HQ]). parents: the row's draft tree (seen_by)."""
+    first .. first + count - 1 -> (out [count][HQ][DV], lse [count][HQ]). parents: the row's draft tree (seen_by);
+    blocks [count][k] with block_size: each column's listed KV blocks (listed)."""
     n = first + count
     keys, values = stored_rows(key_pages, value_pages, table, n, page, kind, key_scales, value_scales, multipliers)
     qd = q.to(q_dtype).double()
     outs, lses = [], []
     for c in range(count):
         seen = seen_by(first, count, c, n, parents, sliding)
+        if blocks is not None:
+            seen = seen & listed(blocks[c], block_size, n)
         o, l = reference(qd[c], keys, values, seen, scale)
         outs.append(o)
         lses.append(l)

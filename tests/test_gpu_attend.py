@@ -3,6 +3,8 @@ and the bit-for-bit invariances the reference demands of its split-KV reader. Mi
 kernels/techniques/attention/paged-kv-attention/tests/test_paged_kv_attention.py:132-188, 275-297, 401-456, 501-512,
 tests/test_nonfinite.py, tests/test_sinks.py and tests/test_sliding.py. Tolerances: the reference's own (8e-3 abs +
 2e-2 rel, lse 1e-3), tighter than the 2e-2 (bf16) / 5e-2 (fp8) the task allows."""
+import math
+
 import pytest
 import torch
 
@@ -345,7 +347,8 @@ def test_bad_geometry_is_refused():
     with pytest.raises(ValueError, match="offsets"):
         cache.attend(q, [0], [0], [99], 1, offsets=torch.zeros(1, dtype=torch.int32, device=dev))
     with pytest.raises(NotImplementedError):
-        cache.attend(q, [0], [0], [99], 1, blocks=torch.zeros(1, 1, dtype=torch.int32, device=dev), block_size=16)
+        cache.attend(q, [0], [0], [99], 1, fresh=(q, q, torch.zeros(1, dtype=torch.int64, device=dev),
+                                                    torch.zeros(1, dtype=torch.int64, device=dev)))
 
 
 def test_launches_that_overlap_on_two_streams_do_not_share_counters():
@@ -417,3 +420,59 @@ def test_a_tree_sees_its_ancestors_and_a_chain_is_causal(kind, hq, hkv, d, page)
     _close(together[8:13], want2)
     with pytest.raises(ValueError):
         cache.attend(q, [0], [0], [392], 8, parents=parents.float())
+
+
+@pytest.mark.parametrize("kind,hq,hkv,d,page", [("bf16", 8, 2, 128, 16), ("int8", 8, 2, 128, 16), ("fp8", 32, 8, 128, 16),
+                                                 ("bf16", 12, 2, 64, 16), ("fp8:row", 10, 2, 128, 48), ("fp16", 6, 2, 256, 16)])
+@pytest.mark.parametrize("block_size", [4, 16, 80])
+def test_block_lists_see_only_their_blocks(kind, hq, hkv, d, page, block_size):
+    # the reference's test (tests/test_paged_kv_attention.py:372-397): four tokens of one row, each with its own list
+    # of 10 - t blocks out of the sequence's, -1 behind them; a token sees its listed blocks' positions up to its own.
+    cache = Cache(kind, hkv, d, d, page, [1000])
+    g = torch.Generator().manual_seed(9)
+    q = rand_q(4, hq, d, 7)
+    nblk = math.ceil(1000 / block_size)
+    blocks = torch.full((4, 12), -1, dtype=torch.int32)
+    for t in range(4):
+        chosen = torch.randperm(nblk, generator=g)[:10 - t].sort().values
+        blocks[t, :len(chosen)] = chosen.to(torch.int32)
+    lse = torch.empty(4, hq, device=dev)
+    out = cache.attend(q, [0], [0], [996], 4, blocks=blocks.to(dev), block_size=block_size, lse=lse, partitions=4)
+    q_dtype = torch.float16 if kind == "fp16" else torch.bfloat16
+    want, want_lse = cache.want(q.to(q_dtype), 0, 996, 4, blocks=blocks, block_size=block_size)
+    _close(out, want)
+    _close_lse(lse, want_lse)
+    # the lists in another order, and in a wider tensor of lists: the same positions (sums in another order)
+    wide = torch.full((4, 40), -1, dtype=torch.int32)
+    wide[:, 5:17] = blocks.flip(1)
+    again = cache.attend(q, [0], [0], [996], 4, blocks=wide.to(dev)[:, 5:17], block_size=block_size, partitions=4)
+    _close(again, want)
+
+
+def test_block_lists_rows_are_their_own_and_empty_lists_see_nothing():
+    cache = Cache("bf16", 4, 128, 128, 16, [3000, 700])
+    q = rand_q(3, 16, 128, 8)
+    blocks = torch.full((3, 6), -1, dtype=torch.int32)
+    blocks[0, :4] = torch.tensor([0, 7, 20, 46])        # row 0: two columns at 2998, 2999; block 46 = positions 2944 .. 3007
+    blocks[1, :3] = torch.tensor([46, 3, 11])
+    # token 2 (row 1, position 699) lists nothing: zeros and -inf
+    lse = torch.empty(3, 16, device=dev)
+    both = cache.attend(q, [0, 1], [0, 2], [2998, 699], 2, blocks=blocks.to(dev), block_size=64, lse=lse,
+                        counts=torch.tensor([2, 1], dtype=torch.int32, device=dev))
+    want, _ = cache.want(q[:2].to(torch.bfloat16), 0, 2998, 2, blocks=blocks[:2], block_size=64)
+    _close(both[:2], want)
+    assert bool((both[2] == 0).all()) and bool(torch.isinf(lse[2]).all())
+    alone = cache.attend(q[:2], [0], [0], [2998], 2, blocks=blocks[:2].to(dev), block_size=64)
+    assert torch.equal(alone, both[:2])
+    # a block past the token's own position, or past the page table, is masked: listing it changes nothing
+    more = blocks.clone()
+    more[0, 4], more[0, 5] = 47, 100000
+    assert torch.equal(cache.attend(q[:2], [0], [0], [2998], 2, blocks=more[:2].to(dev), block_size=64)[0], alone[0])
+    with pytest.raises(ValueError):
+        cache.attend(q[:2], [0], [0], [2998], 2, blocks=blocks[:2].to(dev), block_size=64, fused=True)
+    with pytest.raises(ValueError):
+        cache.attend(q[:2], [0], [0], [2998], 2, blocks=blocks[:2].to(dev), block_size=64, sliding=8)
+    with pytest.raises(ValueError):
+        cache.attend(q[:2], [0], [0], [2998], 2, blocks=blocks[:2].to(dev))
+    with pytest.raises(ValueError):
+        cache.attend(q[:2], [0], [0], [2998], 2, blocks=blocks[:2].long().to(dev), block_size=64)

@@ -384,3 +384,34 @@ def test_a_draft_tree_column_sees_what_its_path_alone_would_hold():
     assert star.nonzero().flatten().tolist() == list(range(first)) + [first, first + 5]
     slid = attend.seen_by(first, 8, 6, 48, parents, sliding=3)       # positions > 40 + 6 - 3 of the path 0, 2, 5, 6
     assert slid.nonzero().flatten().tolist() == [first + 5, first + 6]
+
+
+def test_a_block_list_sees_what_a_sequence_of_only_its_blocks_would_hold():
+    # Pins listed() and its use in window_reference(): a token with a list of KV blocks attends as a plain token would
+    # over a sequence that holds only the listed blocks' positions up to the token's own, in any order of the list;
+    # ids of -1, blocks past the token's position and blocks past the sequence add nothing; every block listed is
+    # plain causal attention; an empty list gives zeros and -inf. Block sizes that divide the page, that do not, and
+    # one larger than a page (the reference tests 4, 16 and 80: test_paged_kv_attention.py:374).
+    k, v, ks, vs, tables, _ = _pool("bf16", 1, 16, 16, 16, [200])
+    q = torch.randn(2, 2, 16, generator=torch.Generator().manual_seed(6))
+    keys, values = attend.stored_rows(k, v, tables[0], 200, 16, "bf16")
+    first = 150
+    for bs in (4, 16, 80, 7):
+        nblk = math.ceil(200 / bs)
+        lists = [[nblk - 1, 0, -1, (first + 1) // bs, 2, 10 ** 6, -1], [1, (first // bs), nblk + 3, -1, -1, -1, -1]]
+        out, lse = attend.window_reference(q, k, v, "bf16", tables[0], first, 2, 16, 0.25, blocks=lists, block_size=bs)
+        for c in range(2):
+            own = first + c
+            index = sorted({n for b in lists[c] if b >= 0 for n in range(b * bs, (b + 1) * bs) if n <= own and n < 200})
+            assert attend.listed(lists[c], bs, 200).nonzero().flatten().tolist() == \
+                sorted({n for b in lists[c] if b >= 0 for n in range(b * bs, (b + 1) * bs) if n < 200})
+            want, want_lse = attend.reference(q[c].bfloat16().double(), keys[index], values[index],
+                                              torch.ones(len(index), dtype=torch.bool), 0.25)
+            assert torch.allclose(out[c], want, atol=1e-12, rtol=1e-12), (bs, c)
+            assert torch.allclose(lse[c], want_lse, atol=1e-12, rtol=1e-12), (bs, c)
+        every = [list(range(nblk)), list(range(nblk))[::-1]]
+        full, _ = attend.window_reference(q, k, v, "bf16", tables[0], first, 2, 16, 0.25, blocks=every, block_size=bs)
+        plain, _ = attend.window_reference(q, k, v, "bf16", tables[0], first, 2, 16, 0.25)
+        assert torch.equal(full, plain)
+    none, none_lse = attend.window_reference(q, k, v, "bf16", tables[0], first, 2, 16, 0.25, blocks=[[-1], [-1]], block_size=16)
+    assert bool((none == 0).all()) and bool(torch.isinf(none_lse).all())
