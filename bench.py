@@ -243,6 +243,35 @@ def long_context(pk, device):
     return found
 
 
+def block_sparse(pk, device):
+    """Block-sparse decode (attend's blocks=): every row lists k KV blocks of 64 positions, sorted and distinct, out of a
+    65,536-token context (32 query heads, 8 KV heads, bf16, random page placement); only the listed blocks are read,
+    so the algorithmic bytes are rows x k x 64 positions x KV heads x (D + DV) x 2. One layer, one token a row; the
+    caller's 4 partitions (the reference's PIECE_PARTITIONS) and the most the list's pieces allow."""
+    hq, hkv, d, page, ctx, bs, found = 32, 8, 128, 16, 65_536, 64, {}
+    batch = 64
+    width = ctx // page
+    n_pages = batch * width
+    g = torch.Generator(device=device).manual_seed(5)
+    k = torch.randn(n_pages + 1, page, hkv, d, device=device, dtype=torch.bfloat16, generator=g)
+    v = torch.randn(n_pages + 1, page, hkv, d, device=device, dtype=torch.bfloat16, generator=g)
+    tables = torch.randperm(n_pages, device=device, generator=g).view(batch, width).to(torch.int32)
+    q = torch.randn(batch, hq, d, device=device, generator=g).to(torch.bfloat16)
+    rows = torch.arange(batch, dtype=torch.int32, device=device)
+    firsts = torch.full((batch,), ctx - 1, dtype=torch.int64, device=device)
+    out = torch.empty(batch, hq, d, dtype=torch.bfloat16, device=device)
+    for listed in (16, 64, 256):
+        ids = torch.stack([torch.randperm(ctx // bs, device=device, generator=g)[:listed].sort().values for _ in range(batch)])
+        blocks = ids.to(torch.int32)
+        nbytes = batch * listed * bs * hkv * 2 * d * 2
+        for parts in (4, 32):
+            ws = torch.empty(pk.workspace_floats(batch, hq, parts, d), dtype=torch.float32, device=device)
+            ms = timed(lambda: pk.attend(q, k, v, "bf16", tables, rows, rows, firsts, 1, page, blocks=blocks, block_size=bs,
+                                         partitions=parts, out=out, workspace=ws), 10, 2)
+            found[f"k{listed}_partitions{parts}"] = {"us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1)}
+    return found
+
+
 def mixed_prefill(pk, device):
     """Chunked prefill over paged KV mixed with decode in one batch (32 query heads, 8 KV heads, bf16): 8 chunks of 512
     new tokens on seeded prefixes in [0, 8192] plus 56 decode rows; one layer: append of all 4,152 tokens, one
@@ -409,6 +438,8 @@ def main():
         extras["long_context_splitk_bf16"] = long_context(pk, device)
         log(f"[bench] long context: {extras['long_context_splitk_bf16']}")
         torch.cuda.empty_cache()
+        extras["block_sparse_decode_bf16"] = block_sparse(pk, device)
+        log(f"[bench] block-sparse decode: {extras['block_sparse_decode_bf16']}")
         extras["mixed_prefill_decode_bf16"] = mixed_prefill(pk, device)
         log(f"[bench] mixed prefill + decode: {extras['mixed_prefill_decode_bf16']}")
         result["extra"] = extras

@@ -27,17 +27,6 @@
 
 namespace pkv {
 
-// A 16-byte (or 8-byte) load of value rows, which are read once: nontemporal, so the caches do not keep them (measured
-// +4 % on the decode launch; the same hint on the key rows measured -1 %, so those stay plain loads).
-PKV_DEV uint4 load_once16(const uint8_t* p) {
-    const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
-    return make_uint4(v.x, v.y, v.z, v.w);
-}
-PKV_DEV uint2 load_once8(const uint8_t* p) {
-    const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
-    return make_uint2(v.x, v.y);
-}
-
 // A workgroup barrier that orders the shared arrays only: a wavefront waits for its own LDS traffic, then for the
 // others. __syncthreads() would also wait until the wavefront's global stores (a unit's partials, which only the next
 // kernel reads) have drained, a memory round trip at every barrier of a unit's end.

@@ -153,7 +153,8 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
             const int in_page = a.page_shift >= 0 ? (n & (a.page - 1)) : (n % a.page);
             const int64_t slot = (int64_t)tab[k] * a.page + in_page;
             buf.k[k] = *reinterpret_cast<const typename StepBuf<KIND>::Vec*>(kbase + slot * slot_bytes);
-            buf.v[k] = *reinterpret_cast<const typename StepBuf<KIND>::Vec*>(vbase + slot * slot_bytes);
+            if constexpr (KIND == 0) buf.v[k] = load_once16(vbase + slot * slot_bytes);
+            else buf.v[k] = load_once8(vbase + slot * slot_bytes);
             if constexpr (KIND >= 2) {
                 buf.ks[k] = a.ks[slot * a.hkv + kvh];
                 buf.vs[k] = a.vs[slot * a.hkv + kvh];
@@ -290,27 +291,32 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
             }
         };
 
-        // Three-stage software pipeline: table entries two steps ahead, K/V one step ahead, compute.
+        // Three-stage software pipeline: table entries two steps ahead, K/V one step ahead, compute. Every load of the
+        // loop is issued unconditionally (past the wavefront's last step it re-reads its first step, which the caches
+        // hold): with loads under conditions the compiler waits for all outstanding loads at every use.
         StepBuf<KIND> bufA, bufB;
         int tabA[4], tabB[4], posA[4], posB[4];
         int base0 = base_of();
-        if (base0 >= 0) fetch_tab(base0, tabA, posA);
-        int base1 = base0 >= 0 ? advance() : -1;
-        if (base0 >= 0) fetch_kv(base0, tabA, posA, bufA);
-        if (base1 >= 0) fetch_tab(base1, tabB, posB);
-        while (base0 >= 0) {
-            int base2 = base1 >= 0 ? advance() : -1;
-            if (base1 >= 0) fetch_kv(base1, tabB, posB, bufB);
-            if (base2 >= 0) fetch_tab(base2, tabA, posA);
-            compute(base0, bufA);
-            if (base1 < 0) break;
-            base0 = base2 >= 0 ? advance() : -1;
-            if (base2 >= 0) fetch_kv(base2, tabA, posA, bufA);
-            if (base0 >= 0) fetch_tab(base0, tabB, posB);
-            compute(base1, bufB);
-            base1 = base0;
-            base0 = base2;
-            // now base0 is loaded in bufA, base1's table entries are in tabB
+        if (base0 >= 0) {
+            const int again = base0;
+            auto safe = [&](int base) __attribute__((always_inline)) { return base >= 0 ? base : again; };
+            fetch_tab(base0, tabA, posA);
+            int base1 = advance();
+            fetch_tab(safe(base1), tabB, posB);
+            fetch_kv(base0, tabA, posA, bufA);
+            for (;;) {
+                const int base2 = base1 >= 0 ? advance() : -1;
+                fetch_kv(safe(base1), tabB, posB, bufB);
+                fetch_tab(safe(base2), tabA, posA);
+                compute(base0, bufA);
+                if (base1 < 0) break;
+                const int base3 = base2 >= 0 ? advance() : -1;
+                fetch_kv(safe(base2), tabA, posA, bufA);
+                fetch_tab(safe(base3), tabB, posB);
+                compute(base1, bufB);
+                if (base2 < 0) break;
+                base0 = base2, base1 = base3;
+            }
         }
 
         // Fold the wavefront's lane groups (butterfly: every lane ends with the same bits), then the four wavefronts
