@@ -257,9 +257,12 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     // The 128-wide kernel serves two adjacent KV heads per wavefront where the head count is even, so every position
     // is read in segments of two rows (512 bytes of 16-bit pages, 256 of 8-bit ones): measured best on MI355X against
     // one and four heads. Fixed by the cache's geometry, never by the launch: a column's bits depend on it.
-    const bool page16 = p->page % 16 == 0 && !p->blocks;      // (block lists: the generic kernel, positions looked up one by one)
+    // (block lists of blocks that are a multiple of 16 positions walk their lists in the 128-wide kernel, others in
+    // the generic one, each position looked up on its own)
+    const bool fast_lists = p->blocks && lpr == 16 && p->page % 16 == 0 && p->block_size % 16 == 0;
+    const bool page16 = p->page % 16 == 0 && !p->blocks;
     a.heads_per_wave = 1;
-    if (lpr == 16 && page16) {
+    if (lpr == 16 && (page16 || fast_lists)) {
         if (p->kv_heads % 2 == 0) a.heads_per_wave = 2;
     }
     const int64_t gx = (int64_t)p->n_rows * (p->kv_heads / a.heads_per_wave) * a.tiles;
@@ -272,7 +275,7 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     const dim3 grid((unsigned)gx, p->fused ? 1u : gy);
     a.units_x = a.units_y = 0;
     a.ticket = nullptr;
-    if (lpr == 16 && page16) {
+    if (lpr == 16 && (page16 || fast_lists)) {
         a.ticket = next_ticket();
         if (!a.ticket || compute_units() < 1) return CRIT_PKV_E_GEOMETRY;
     }

@@ -90,8 +90,14 @@ constexpr int attend_waves(int kind, int qr) { return qr <= 2 ? 4 : (qr <= 4 && 
 // Pages are a multiple of 16 positions, so the 16 positions of a step share one page table entry, which is uniform
 // over the wavefront: a step's addresses are a scalar base plus per-lane offsets that do not change from step to step.
 // One unit of work: (ux, uy) of a units_x x units_y list, what a workgroup of a plain launch would get as blockIdx.
-template <int KIND, bool F16, int QR, int HW, bool FUSED>
+// SPARSE: block lists of blocks that are a multiple of 16 positions. A tile then holds the rows of one column (the
+// launcher picks QR dividing the group); the unit walks the run of the column's list, place u at position
+// blocks[u / block_size] * block_size + u % block_size, cut into pieces and partitions like an ordinary row's positions;
+// a step's places lie in one block and one page, so the walk stays scalar: a step of an unlisted place (id -1) or past
+// the column's positions is skipped, every other step is read exactly as an ordinary row's.
+template <int KIND, bool F16, int QR, int HW, bool FUSED, bool SPARSE = false>
 PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
+    static_assert(!(SPARSE && FUSED), "block lists are read by the split launch");
     constexpr int D = 128;
     constexpr int RB = (QR + 3) / 4;            // blocks of four query rows
     constexpr int EB = KIND == 0 ? 2 : 1;
@@ -103,6 +109,7 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
     __shared__ __align__(16) uint16_t s_p[4][4][RB * 4][4];   // [wavefront][DPP row][query row][position of the row]
     __shared__ __align__(16) float s_alpha[4][4][RB * 4];
     __shared__ __align__(16) float s_rm[4][4][RB * 4], s_rl[4][4][RB * 4];
+    __shared__ int s_blocks[SPARSE ? kMaxListedBlocks : 1];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -146,7 +153,8 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
     nk64 = nk64 < 0 ? 0 : (nk64 > (int64_t)a.max_keys ? (int64_t)a.max_keys : nk64);
     const int n_keys = (int)nk64;
     const int first = (int)(first64 < 0 ? 0 : (first64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first64));
-    const int n_pieces = (n_keys + a.piece - 1) / a.piece;
+    const int n_run = SPARSE ? a.listed_keys : n_keys;      // the positions (or places of a list) the partitions divide
+    const int n_pieces = (n_run + a.piece - 1) / a.piece;
     if constexpr (!FUSED) {
         // Units are taken in list order, y slowest, and a launch's tail is as long as its last units: the row's last
         // partition (usually a partial piece, the smallest unit of work) is listed after every other partition, at
@@ -154,7 +162,7 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
         // that start last are the smallest.
         const int np = min(n_pieces, a.parts);
         if (np <= 0) return;
-        const bool small = np == n_pieces && n_keys - (np - 1) * a.piece < a.piece / 2;
+        const bool small = np == n_pieces && n_run - (np - 1) * a.piece < a.piece / 2;
         if (b >= a.units_y - 2) {
             if ((b == a.units_y - 1) != small) return;
             b = np - 1;
@@ -256,14 +264,35 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
             if (below > 0) pi = part + (below + a.parts - 1) / a.parts * a.parts;
         }
     };
+    if constexpr (SPARSE) {      // the tile's column's list, for the walk below (the unit's callers order the reuse)
+        const int32_t* list = a.blocks + (int64_t)(start + c_lo) * a.blocks_stride;
+        for (int i = tid; i < a.blocks_k; i += 256) s_blocks[i] = list[i];
+        lds_barrier();
+    }
     auto base_of = [&]() __attribute__((always_inline)) -> int {
-        if (st * SPW >= a.piece) return -1;
-        const int64_t base = (int64_t)pi * a.piece + st * SPW;
-        return base < n_keys ? (int)base : -1;
+        if constexpr (SPARSE) {      // the cursor's step if its block is listed and holds a position of the column, else the next such
+            if (wave * SPW >= a.piece) return -1;
+            for (;;) {
+                if (st * SPW >= a.piece) pi += a.parts, st = wave;
+                const int64_t place = (int64_t)pi * a.piece + st * SPW;
+                if (place >= n_run) return -1;
+                const int e = (int)div32(a.block_div, (uint32_t)place);
+                const int id = __builtin_amdgcn_readfirstlane(s_blocks[e]);
+                const int64_t base = (int64_t)id * a.block_size + ((int)place - e * a.block_size);
+                if (id >= 0 && base < n_keys) return (int)base;
+                st += 4;
+            }
+        } else {
+            if (st * SPW >= a.piece) return -1;
+            const int64_t base = (int64_t)pi * a.piece + st * SPW;
+            return base < n_keys ? (int)base : -1;
+        }
     };
     auto advance = [&]() __attribute__((always_inline)) -> int {
         st += 4;
-        if (st * SPW >= a.piece) pi += a.parts, st = wave;
+        if constexpr (!SPARSE) {
+            if (st * SPW >= a.piece) pi += a.parts, st = wave;
+        }
         return base_of();
     };
     struct Lead {
@@ -601,7 +630,7 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
 // order, so with units as uneven as ragged contexts make them it leaves slots idle behind a busy one; resident
 // workgroups that pull the next unit themselves keep every slot busy to the end. The last workgroup to finish zeroes
 // the counters for the next launch that uses them.
-template <int KIND, bool F16, int QR, int HW, bool FUSED>
+template <int KIND, bool F16, int QR, int HW, bool FUSED, bool SPARSE = false>
 __global__ __launch_bounds__(256, attend_waves(KIND, QR)) void attend128_kernel(AttendArgs a) {
     __shared__ unsigned s_unit;
     const unsigned total = (unsigned)a.units_x * (unsigned)a.units_y;
@@ -609,7 +638,7 @@ __global__ __launch_bounds__(256, attend_waves(KIND, QR)) void attend128_kernel(
     while (u < total) {
         // (the next ticket is drawn after the unit, not during it: a returning atomic in flight makes every wait on
         // the unit's loads a wait for all of them, which costs more than the ticket's round trip)
-        attend128_unit<KIND, F16, QR, HW, FUSED>(a, (int)(u % (unsigned)a.units_x), (int)(u / (unsigned)a.units_x));
+        attend128_unit<KIND, F16, QR, HW, FUSED, SPARSE>(a, (int)(u % (unsigned)a.units_x), (int)(u / (unsigned)a.units_x));
         lds_barrier();      // the unit is done with the shared arrays, and every thread has read s_unit
         if (threadIdx.x == 0) s_unit = gridDim.x + atomicAdd(a.ticket, 1u);
         lds_barrier();

@@ -10,7 +10,22 @@ namespace pkv {
 template <int KIND, bool F16, int QR, bool FUSED>
 static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipStream_t stream) {
     if constexpr (!FUSED) {
-        if (a.blocks) {      // block lists: the generic kernel reading each column's listed blocks only
+        if (a.blocks && lpr == 16 && a.page % 16 == 0 && a.block_size % 16 == 0) {
+            // block lists whose steps lie in one block and one page: the bandwidth path walking each column's list
+            AttendArgs u = a;
+            u.units_x = (int)grid.x, u.units_y = (int)grid.y + 1;
+            const int64_t units = (int64_t)u.units_x * u.units_y;
+            if (units > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
+            const int64_t resident = (int64_t)compute_units() * attend_waves(KIND, QR);
+            const dim3 pgrid((unsigned)(units < resident ? units : resident));
+            switch (a.heads_per_wave) {
+                case 1: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 1, false, true>), pgrid, dim3(256), 0, stream, u); break;
+                case 2: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 2, false, true>), pgrid, dim3(256), 0, stream, u); break;
+                default: return CRIT_PKV_E_GEOMETRY;
+            }
+            return hip_code(hipGetLastError());
+        }
+        if (a.blocks) {      // other block lists: the generic kernel, each position looked up on its own
             switch (lpr) {
                 case 8: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 8, QR, false, true>), grid, dim3(256), 0, stream, a); break;
                 case 16: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 16, QR, false, true>), grid, dim3(256), 0, stream, a); break;

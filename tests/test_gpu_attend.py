@@ -476,3 +476,26 @@ def test_block_lists_rows_are_their_own_and_empty_lists_see_nothing():
         cache.attend(q[:2], [0], [0], [2998], 2, blocks=blocks[:2].to(dev))
     with pytest.raises(ValueError):
         cache.attend(q[:2], [0], [0], [2998], 2, blocks=blocks[:2].long().to(dev), block_size=64)
+
+
+@pytest.mark.parametrize("kind,block_size", [("bf16", 64), ("fp8", 32), ("bf16", 24)])
+def test_block_lists_with_a_draft_tree_over_long_lists(kind, block_size):
+    # Lists long enough for several pieces and partitions (blocks of 64 and 32 walk their lists in the 128-wide kernel,
+    # blocks of 24 in the generic one), a draft tree on top: a column sees its listed blocks' positions below the
+    # window and, of the window, its ancestors' and its own where listed.
+    cache = Cache(kind, 2, 128, 128, 16, [6000])
+    g = torch.Generator().manual_seed(13)
+    parents = torch.tensor([-1, 0, 0, 1, 2], dtype=torch.int32, device=dev)
+    first = 5990
+    q = rand_q(5, 8, 128, 11)
+    nblk = math.ceil(6000 / block_size)
+    blocks = torch.full((5, 70), -1, dtype=torch.int32)
+    for t in range(5):
+        chosen = torch.randperm(nblk - 1, generator=g)[:60 - 7 * t]
+        blocks[t, :len(chosen)] = chosen.to(torch.int32)
+        blocks[t, 65] = nblk - 1                      # the window's own block, behind a gap of -1
+    out = cache.attend(q, [0], [0], [first], 5, parents=parents, blocks=blocks.to(dev), block_size=block_size, partitions=3)
+    want, _ = cache.want(q.to(torch.bfloat16), 0, first, 5, parents=parents.tolist(), blocks=blocks, block_size=block_size)
+    _close(out, want)
+    more = cache.attend(q, [0], [0], [first], 5, parents=parents, blocks=blocks.to(dev), block_size=block_size, partitions=16)
+    _close(more, want)
