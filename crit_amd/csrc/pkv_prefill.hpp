@@ -68,6 +68,32 @@ PKV_DEV uint32_t to_pair(float a, float b) {
     return __builtin_bit_cast(uint32_t, r);
 }
 
+// Two codes (bytes 0,1 or 2,3 of a word of E4M3 or INT8 codes) -> two BF16 values in one word, exactly.
+template <int KIND, bool HI>
+PKV_DEV uint32_t code_pair(uint32_t w) {
+    if constexpr (KIND == 3) {
+        const float f0 = (float)(int8_t)(w >> (HI ? 16 : 0)), f1 = (float)(int8_t)(w >> (HI ? 24 : 8));
+        return __builtin_amdgcn_perm(f2u(f1), f2u(f0), 0x07060302u);
+    } else {
+        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)w, 1.0f, HI));
+    }
+}
+
+// 8 codes (two words) -> 8 BF16 values packed in a uint4, exactly.
+template <int KIND>
+PKV_DEV u32x4 codes_to_bf16(uint32_t w0, uint32_t w1) {
+    return u32x4{code_pair<KIND, false>(w0), code_pair<KIND, true>(w0), code_pair<KIND, false>(w1), code_pair<KIND, true>(w1)};
+}
+
+template <bool F16>
+PKV_DEV float dot2_acc(uint32_t a, uint32_t b, float c) {
+    if constexpr (F16) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
+    } else {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
+    }
+}
+
 // V^T in LDS is [dim][64 keys], rows of 128 bytes without padding; the 8-byte group of four keys g of row `row` sits
 // at group g ^ swz(row). The stores (16 lanes: 16 dim chunks of 8 rows, one row of each) and the operand reads (16
 // lanes: 16 adjacent rows) both spread over all banks, and the swizzle is a XOR of bit fields, so an address is one
