@@ -17,21 +17,28 @@
 
 namespace pkv {
 
-template <int KIND, bool F16, int D>
-__global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
+template <int KIND, bool F16, int D, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillArgs a) {
+    static_assert(WAVES == 4 || (WAVES == 8 && D == 128), "eight wavefronts: 128-wide heads only");
+    constexpr int NT = 64 * WAVES;      // threads of the workgroup
+    constexpr int BMW = 32 * WAVES;     // query rows it holds
     constexpr int KS = D / 16;          // k-steps of the first product
     constexpr int NB = D / 32;          // 32-wide output blocks of the second product
     constexpr int KSTR = D + 8;         // K row stride in LDS (16-bit elements): 16 bytes of padding
     constexpr int EB = KIND == 0 ? 2 : 1;
     constexpr int CH = D * EB / 16;     // 16-byte chunks of one K or V row in the pages
-    constexpr int KPASS = BN * CH / 256;   // passes of 256 threads over a K block, rows contiguous over lanes
-    // V staging: a thread takes 8 dims (one 16-byte chunk of 16-bit pages, half a chunk of 8-bit ones) of four adjacent
-    // keys; D / 8 such pieces a key, 16 groups of four keys a block.
-    constexpr int VC = D / 8;           // 8-dim pieces of one V row
-    constexpr int VGROUPS = 16 * VC;    // (group of four keys, 8-dim piece) pairs of a V block: 256 (D = 128) or 128
+    constexpr int KPASS = BN * CH / NT;    // passes of the workgroup over a K block, rows contiguous over lanes
+    // V staging: a thread takes DPT dims (eight, or four where eight wavefronts share the block) of four adjacent keys;
+    // D / DPT such pieces a key, 16 groups of four keys a block.
+    constexpr int DPT = WAVES == 8 ? 4 : 8;
+    constexpr int VC = D / DPT;         // pieces of one V row
+    constexpr int VGROUPS = 16 * VC;    // (group of four keys, piece) pairs of a V block: the workgroup's threads, or half of them (D = 64)
+    // K blocks alternate between two buffers. V blocks too with four wavefronts; with eight, half of the wavefronts
+    // multiply by a block's values one iteration after the other half (below), so V blocks go round three buffers.
+    constexpr int VBUFS = WAVES == 8 ? 3 : 2;
     __shared__ __align__(16) uint16_t k_lds[2][BN * KSTR];
-    __shared__ __align__(16) uint16_t v_lds[2][D * BN];
-    __shared__ float ks_lds[2][BN], vs_lds[2][BN];
+    __shared__ __align__(16) uint16_t v_lds[VBUFS][D * BN];
+    __shared__ float ks_lds[2][BN], vs_lds[VBUFS][BN];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n32 = lane & 31, h = lane >> 5;
     // Workgroups go to the 8 XCDs round robin by linear id, and each XCD has its own L2: all tiles of one (chunk, KV
@@ -44,7 +51,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
     const int kvh = group % a.hkv, z = chunk_by_rank(a, group / a.hkv, lane);
     int count = a.max_count;
     if (a.counts) count = min(a.counts[z], a.max_count);
-    if ((int64_t)tile * BM >= (int64_t)count * a.g) return;
+    if ((int64_t)tile * BMW >= (int64_t)count * a.g) return;
     const int start = a.starts ? a.starts[z] : 0;
     int64_t pos64 = a.positions[z];
     pos64 = pos64 < 0 ? 0 : (pos64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : pos64);
@@ -52,7 +59,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
     const int64_t trow = (int64_t)(a.table_rows ? a.table_rows[z] : z) * a.tab_stride;
 
     // This lane's query row.
-    const int j = tile * BM + wave * 32 + n32;
+    const int j = tile * BMW + wave * 32 + n32;
     const int t = j / a.g, head = kvh * a.g + j % a.g;
     const bool live = t < count;
     const int lim = live ? pos + t : -1;
@@ -82,8 +89,8 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
         }
     }
 
-    const int t_lo = tile * BM / a.g;
-    const int t_hi = min(count - 1, (tile * BM + BM - 1) / a.g);
+    const int t_lo = tile * BMW / a.g;
+    const int t_hi = min(count - 1, (tile * BMW + BMW - 1) / a.g);
     const int n_max = pos + count - 1;                 // the chunk's last written position
     const int kt_hi = (pos + t_hi) / BN;
     int kt_lo = 0;
@@ -124,7 +131,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
         myslot = (uint32_t)ent * (uint32_t)a.page + (uint32_t)inp;
         static_for<KPASS>([&](auto pc) __attribute__((always_inline)) {
             constexpr int p = decltype(pc)::value;
-            rowslot[p] = (uint32_t)__builtin_amdgcn_ds_bpermute(((p * 256 + tid) / CH) << 2, (int)myslot);
+            rowslot[p] = (uint32_t)__builtin_amdgcn_ds_bpermute(((p * NT + tid) / CH) << 2, (int)myslot);
         });
         const int kg = tid % VGROUPS / VC;      // D = 64: the upper half of the workgroup repeats the lower
         static_for<4>([&](auto ic) __attribute__((always_inline)) {
@@ -138,28 +145,29 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
             constexpr int p = decltype(pc)::value;
             kreg[p] = *reinterpret_cast<const u32x4*>(kthread + (uint64_t)rowslot[p] * slot_bytes);
         });
-        if constexpr (KIND >= 2) {
-            ksreg = a.ks[(uint64_t)myslot * a.hkv + kvh], vsreg = a.vs[(uint64_t)myslot * a.hkv + kvh];
-        }
+        if constexpr (KIND >= 2) ksreg = a.ks[(uint64_t)myslot * a.hkv + kvh];
     };
     auto load_v = [&]() __attribute__((always_inline)) {
-        const uint8_t* vthread = vbase + (tid % VGROUPS % VC) * (8 * EB);
+        const uint8_t* vthread = vbase + (tid % VGROUPS % VC) * (DPT * EB);
         static_for<4>([&](auto ic) __attribute__((always_inline)) {
             constexpr int i = decltype(ic)::value;
             const uint8_t* row = vthread + (uint64_t)rowslot[KPASS + i] * slot_bytes;
-            if constexpr (KIND == 0) {
+            if constexpr (DPT * EB == 16) {
                 vreg[i] = *reinterpret_cast<const u32x4*>(row);
-            } else {
+            } else if constexpr (DPT * EB == 8) {
                 const u32x2 w = *reinterpret_cast<const u32x2*>(row);
                 vreg[i].x = w.x, vreg[i].y = w.y;
+            } else {
+                vreg[i].x = *reinterpret_cast<const uint32_t*>(row);
             }
         });
+        if constexpr (KIND >= 2) vsreg = a.vs[(uint64_t)myslot * a.hkv + kvh];
     };
     auto store_k = [&](int buf) __attribute__((always_inline)) {
         uint16_t* kl = k_lds[buf];
         static_for<KPASS>([&](auto pc) __attribute__((always_inline)) {
             constexpr int p = decltype(pc)::value;
-            const int idx = p * 256 + tid;
+            const int idx = p * NT + tid;
             const int kk = idx / CH, c = idx % CH;
             if constexpr (KIND == 0) {
                 *reinterpret_cast<u32x4*>(&kl[kk * KSTR + c * 8]) = kreg[p];
@@ -171,18 +179,23 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
             }
         });
         if constexpr (KIND >= 2) {
-            if (tid < BN) ks_lds[buf][tid] = ksreg, vs_lds[buf][tid] = vsreg;
+            if (tid < BN) ks_lds[buf][tid] = ksreg;
         }
     };
     auto store_v = [&](int buf) __attribute__((always_inline)) {
-        // The thread's four keys x eight dims as 16-bit pairs of adjacent dims (8-bit codes converted, exactly), then
-        // transposed: dim row 8 c + i gets the four keys' values as one 8-byte group at group kg ^ swz(row), byte
-        // offset (1024 c + 8 (kg ^ c)) ^ (16 i), plus 128 i.
+        // The thread's four keys x DPT dims as 16-bit pairs of adjacent dims (8-bit codes converted, exactly), then
+        // transposed: dim row 8 c + i gets the four keys' values as one 8-byte group at the place v_place gives, byte
+        // offset v_place(kg, 8 c) ^ (16 i), plus 128 i. A thread with four dims holds i = 4 up + 0 .. 3 of them: 64 up
+        // goes into the XOR and 512 up into the sum (bits 7 to 9 of the first term are clear, so the sum carries nothing).
         const int idx = tid % VGROUPS;      // repeated pairs store the same bytes twice
-        const int kg = idx / VC, c = idx % VC;
+        const int kg = idx / VC, piece = idx % VC;
+        const int c = piece / (8 / DPT), up = piece % (8 / DPT);
         uint8_t* vb = reinterpret_cast<uint8_t*>(v_lds[buf]);
-        const uint32_t v_write = 1024u * (uint32_t)c + 8u * (uint32_t)(kg ^ c);
-        static_for<4>([&](auto jc) __attribute__((always_inline)) {
+        if constexpr (KIND >= 2) {
+            if (tid < BN) vs_lds[buf][tid] = vsreg;
+        }
+        const uint32_t v_write = ((uint32_t)v_place(kg, 8 * c) ^ (64u * (uint32_t)up)) + 512u * (uint32_t)up;
+        static_for<DPT / 2>([&](auto jc) __attribute__((always_inline)) {
             constexpr int j = decltype(jc)::value;      // dims 2 j and 2 j + 1 of the thread's eight
             uint32_t w[4];
 #pragma unroll
@@ -211,9 +224,10 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
         for (int kb = 0; kb < 2; ++kb)
             dst[kb] = *reinterpret_cast<const u32x4*>(&kl[(32 * kb + n32) * KSTR + 16 * i + 8 * h]);
     };
-    // Byte offset of the lane's V^T operand inside a buffer: row (32 nb + n32), group (4 g + 2 j + h) ^ swz(row)
-    //   = v_read ^ (8 * ((4 g + 2 j) ^ (4 nb))) + 4096 nb.
-    const uint32_t v_read = (uint32_t)n32 * (BN * 2) + 8u * (uint32_t)(h ^ (n32 >> 3) ^ ((n32 & 7) << 1));
+    // Byte offset of the lane's V^T operand inside a buffer: row 32 nb + n32, the 16-byte slot of groups 4 g + h and
+    // 4 g + 2 + h = v_place(4 g + h, 32 nb + n32) less its half bit = v_read ^ (16 (2 g ^ 4 (nb & 1))) + 4096 nb; the
+    // two groups come in that order in rows below 64 and swapped above.
+    const uint32_t v_read = (uint32_t)v_place(h, n32);
     auto read_v = [&](const uint16_t* vl, auto ic, u32x4 (&dst)[2]) __attribute__((always_inline)) {
         constexpr int i = decltype(ic)::value;
         constexpr int g = i / (NB / 2);      // keys 16 g .. 16 g + 15: 32-key half g / 2, half of it g % 2
@@ -221,9 +235,8 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int nb = 2 * (i % (NB / 2)) + j;
-            const u32x2 lo = *reinterpret_cast<const u32x2*>(vb + (v_read ^ (8u * ((4 * g) ^ (4 * nb & 15)))) + 32 * BN * 2 * nb);
-            const u32x2 hi = *reinterpret_cast<const u32x2*>(vb + (v_read ^ (8u * ((4 * g + 2) ^ (4 * nb & 15)))) + 32 * BN * 2 * nb);
-            dst[j] = u32x4{lo.x, lo.y, hi.x, hi.y};
+            const u32x4 w = *reinterpret_cast<const u32x4*>(vb + (v_read ^ (16u * ((2 * g) ^ (4 * (nb & 1))))) + 32 * BN * 2 * nb);
+            dst[j] = (nb >> 1) ? u32x4{w.z, w.w, w.x, w.y} : w;
         }
     };
 
@@ -236,9 +249,9 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
 
     // Double-buffered LDS, one barrier a block: block kt is multiplied from buffer kt & 1 while block kt + 1 (already
     // in registers) is stored into the other buffer and its registers are at once reloaded with block kt + 2 (a whole
-    // iteration before they are stored); the slots of block kt + 3 and the table entries of block kt + 4 follow
-    // during the second product. Every load of the loop is unconditional (past the last block it repeats the last one), so
-    // the compiler counts the outstanding loads exactly instead of waiting for all of them.
+    // iteration before they are stored); the slots of block kt + 3 and the table entries of block kt + 4 follow. Every
+    // load of the loop is unconditional (past the last block it repeats the last one), so the compiler counts the
+    // outstanding loads exactly instead of waiting for all of them.
     auto upto = [&](int kt) __attribute__((always_inline)) { return kt < kt_hi ? kt : kt_hi; };
     load_entries(kt_lo);
     take_slots();
@@ -246,7 +259,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
     load_v();
     load_entries(upto(kt_lo + 1));
     store_k(kt_lo & 1);
-    store_v(kt_lo & 1);
+    store_v(WAVES == 8 ? 0 : kt_lo & 1);
     take_slots();
     load_k();
     load_v();
@@ -254,21 +267,27 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
     take_slots();
     load_entries(upto(kt_lo + 3));
     __syncthreads();
-    // One key block; MASK: 0 = every key is visible to every row of the workgroup, 1 = causal limit and sliding window.
-    auto block = [&](int kt, auto mask_c) __attribute__((always_inline)) {
-        constexpr int MASK = decltype(mask_c)::value;
+
+    // A key block in three phases. scores: S^T = K Q^T on the matrix cores, with the staging of the next block in its
+    // shadow. weigh: mask, running maximum, the first exponentials (vector work). values: O^T += V^T P^T on the matrix
+    // cores, the remaining exponentials in its shadow.
+    constexpr int RING = 3;      // operands are read RING - 1 steps before their products
+    f32x16 s[2];
+    u32x4 va[RING][2], pop[4];
+    float alpha = 1.0f, sum = 0.0f, sub = 0.0f;
+    const std::integral_constant<int, 0> c0;
+    const std::integral_constant<int, 1> c1;
+    // kt: the block; vnext: the V buffer block kt + 1 goes to.
+    auto scores = [&](int kt, int vnext) __attribute__((always_inline)) {
         const int buf = kt & 1;
         const uint16_t* kl = k_lds[buf];
-        const uint16_t* vl = v_lds[buf];
-        // S^T = K Q^T: two blocks of 32 keys x this wavefront's 32 rows. The operands of a group of four products are
-        // read while the group before is multiplied, and the next block goes into the other LDS buffer (its readers
-        // passed the barrier) in the shadow of the products.
-        f32x16 s[2];
+        // Two blocks of 32 keys x this wavefront's 32 rows. The operands of a step are read RING - 1 steps before it,
+        // and the next block goes into the other LDS buffers (their readers passed the barrier) in the shadow of the
+        // products.
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int v = 0; v < 16; ++v) s[kb][v] = 0.0f;
-        constexpr int RING = 3;      // operands are read RING - 1 steps before their products
         u32x4 ka[RING][2];
         static_for<RING - 1>([&](auto ic) __attribute__((always_inline)) { read_k(kl, ic, ka[decltype(ic)::value]); });
         PKV_PRIO(1);
@@ -278,7 +297,11 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
             s[0] = mfma<F16>(ka[i % RING][0], qreg[i], s[0]);
             s[1] = mfma<F16>(ka[i % RING][1], qreg[i], s[1]);
             if constexpr (i == 0) store_k(buf ^ 1), load_k();
-            if constexpr (i == KS / 2 - 1) store_v(buf ^ 1), load_v();
+            if constexpr (i == KS / 2 - 1) store_v(vnext), load_v();
+            if constexpr (WAVES == 8 && i == KS - 2) {      // the slots of block kt + 3 for the next iteration's loads, the entries of kt + 4
+                take_slots();
+                load_entries(upto(kt + 4));
+            }
             if constexpr (KIND != 0) PKV_SB();
         });
         // one product, then a share of the staging work (LDS reads of later operands, the stores' permutes and
@@ -295,19 +318,45 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
         }
         PKV_SB();
         PKV_PRIO(0);
-        u32x4 va[RING][2];
-        static_for<RING - 1>([&](auto ic) __attribute__((always_inline)) { read_v(vl, ic, va[decltype(ic)::value]); });
-        PKV_SB();
-        // Mask where the block is not wholly visible; the lane holds keys 32 kb + 8 (v / 4) + 4 h + v % 4 of its own
-        // row. With one scale for all keys (positive once its sign went into the queries) the maximum is taken over
-        // the raw scores and the scale rides on the exponent's fused multiply-add; with per-key scales (row-scaled
-        // pages) each score is scaled first.
+        // With one scale for all keys (positive once its sign went into the queries) the maximum is taken over the raw
+        // scores and the scale rides on the exponent's fused multiply-add; with per-key scales (row-scaled pages) each
+        // score is scaled first. The lane holds keys 32 kb + 8 (v / 4) + 4 h + v % 4 of its own row.
         if constexpr (KIND >= 2) {
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) s[kb][v] *= sscale * ks_lds[buf][32 * kb + 8 * (v / 4) + 4 * h + v % 4];
         }
+    };
+    // P^T as the second product's B operand: pop[g] holds the probabilities of keys 16 g .. 16 g + 15 (32-key half
+    // g / 2, half of it g % 2), four 16-bit pairs, taken two pairs at a time so that only the first two pairs'
+    // exponentials run before the second product starts and the rest in the shadow of its matrix instructions.
+    auto pairs = [&](int vbuf, auto gc, auto partc) __attribute__((always_inline)) {
+        constexpr int g = decltype(gc)::value, part = decltype(partc)::value;
+        constexpr int kb = g / 2, half = g % 2;
+#pragma unroll
+        for (int j = 2 * part; j < 2 * part + 2; ++j) {
+            const int v = 8 * half + 2 * j;
+            float p0, p1;
+            if constexpr (KIND >= 2) {
+                p0 = exp2_fast(s[kb][v] - sub), p1 = exp2_fast(s[kb][v + 1] - sub);
+            } else {
+                p0 = exp2_fast(__builtin_fmaf(s[kb][v], sabs, -sub)), p1 = exp2_fast(__builtin_fmaf(s[kb][v + 1], sabs, -sub));
+            }
+            sum += p0 + p1;
+            if constexpr (KIND >= 2) {     // the values' scales ride on the operand, not on the sum
+                p0 *= vs_lds[vbuf][32 * kb + 8 * (v / 4) + 4 * h + v % 4];
+                p1 *= vs_lds[vbuf][32 * kb + 8 * ((v + 1) / 4) + 4 * h + (v + 1) % 4];
+            }
+            pop[g][j] = to_pair<F16>(p0, p1);
+        }
+    };
+    // MASK: 0 = every key of the block is visible to every row of the workgroup, 1 = causal limit and sliding window.
+    auto weigh = [&](int kt, int vbuf, auto mask_c) __attribute__((always_inline)) {
+        constexpr int MASK = decltype(mask_c)::value;
+        const uint16_t* vl = v_lds[vbuf];
+        static_for<RING - 1>([&](auto ic) __attribute__((always_inline)) { read_v(vl, ic, va[decltype(ic)::value]); });
+        PKV_SB();
         if constexpr (MASK > 0) {
             // key 32 kb + 8 (v / 4) + v % 4 + 4 h is visible iff that constant is in (rel_lo, rel]
             const int rel = lim - kt * BN - 4 * h;
@@ -333,38 +382,12 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
         if constexpr (KIND < 2) top = top == -INFINITY ? -INFINITY : top * sabs;
         top = __builtin_fmaxf(top, __shfl_xor(top, 32));
         const float m_new = top > m + kMaxSlack ? top : m;
-        const float sub = m_new == -INFINITY ? 0.0f : m_new;
-        const float alpha = exp2_fast(m - sub);
+        sub = m_new == -INFINITY ? 0.0f : m_new;
+        alpha = exp2_fast(m - sub);
         m = m_new;
-        float sum = 0.0f;
-        // P^T as the second product's B operand: pop[g] holds the probabilities of keys 16 g .. 16 g + 15 (32-key half
-        // g / 2, half of it g % 2), four 16-bit pairs, taken two pairs at a time so that only the first two pairs'
-        // exponentials run before the second product starts and the rest in the shadow of its matrix instructions.
-        u32x4 pop[4];
-        auto pairs = [&](auto gc, auto partc) __attribute__((always_inline)) {
-            constexpr int g = decltype(gc)::value, part = decltype(partc)::value;
-            constexpr int kb = g / 2, half = g % 2;
-#pragma unroll
-            for (int j = 2 * part; j < 2 * part + 2; ++j) {
-                const int v = 8 * half + 2 * j;
-                float p0, p1;
-                if constexpr (KIND >= 2) {
-                    p0 = exp2_fast(s[kb][v] - sub), p1 = exp2_fast(s[kb][v + 1] - sub);
-                } else {
-                    p0 = exp2_fast(__builtin_fmaf(s[kb][v], sabs, -sub)), p1 = exp2_fast(__builtin_fmaf(s[kb][v + 1], sabs, -sub));
-                }
-                sum += p0 + p1;
-                if constexpr (KIND >= 2) {     // the values' scales ride on the operand, not on the sum
-                    p0 *= vs_lds[buf][32 * kb + 8 * (v / 4) + 4 * h + v % 4];
-                    p1 *= vs_lds[buf][32 * kb + 8 * ((v + 1) / 4) + 4 * h + (v + 1) % 4];
-                }
-                pop[g][j] = to_pair<F16>(p0, p1);
-            }
-        };
-        const std::integral_constant<int, 0> c0;
-        const std::integral_constant<int, 1> c1;
-        pairs(c0, c0);
-        pairs(c0, c1);
+        sum = 0.0f;
+        pairs(vbuf, c0, c0);
+        pairs(vbuf, c0, c1);
         // wave-uniform: skip the rescale when no row's maximum moved (alpha == 1 everywhere)
         if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
             asm volatile("s_nop 0");      // pins the branch: an unconditional rescale by 1 is what the optimiser would make of it
@@ -374,8 +397,11 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
                 for (int v = 0; v < 16; ++v) o[nb][v] *= alpha;
         }
         PKV_SB();
-        // O^T += V^T P^T: the lane feeds V^T[dim 32 nb + n32][keys of its half] and its own probabilities. The second
-        // half's exponentials run in the shadow of the first half's products.
+    };
+    // The lane feeds V^T[dim 32 nb + n32][keys of its half] and its own probabilities. The second half's exponentials
+    // run in the shadow of the first half's products.
+    auto values = [&](int kt, int vbuf) __attribute__((always_inline)) {
+        const uint16_t* vl = v_lds[vbuf];
         PKV_PRIO(1);
         constexpr int VSTEPS = 2 * NB;
         static_for<VSTEPS>([&](auto ic) __attribute__((always_inline)) {
@@ -387,13 +413,13 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
             // steps 0 .. 5 take the pairs of pop[1], pop[2], pop[3] in order, each a step (D = 128) or more (D = 64:
             // two at a time) before the step that multiplies by them
             if constexpr (NB == 4) {
-                if constexpr (i < 6) pairs(std::integral_constant<int, 1 + i / 2>{}, std::integral_constant<int, i % 2>{});
+                if constexpr (i < 6) pairs(vbuf, std::integral_constant<int, 1 + i / 2>{}, std::integral_constant<int, i % 2>{});
             } else {
-                if constexpr (i == 0) pairs(c1, c0), pairs(c1, c1);
-                if constexpr (i == 1) pairs(std::integral_constant<int, 2>{}, c0), pairs(std::integral_constant<int, 2>{}, c1);
-                if constexpr (i == 2) pairs(std::integral_constant<int, 3>{}, c0), pairs(std::integral_constant<int, 3>{}, c1);
+                if constexpr (i == 0) pairs(vbuf, c1, c0), pairs(vbuf, c1, c1);
+                if constexpr (i == 1) pairs(vbuf, std::integral_constant<int, 2>{}, c0), pairs(vbuf, std::integral_constant<int, 2>{}, c1);
+                if constexpr (i == 2) pairs(vbuf, std::integral_constant<int, 3>{}, c0), pairs(vbuf, std::integral_constant<int, 3>{}, c1);
             }
-            if constexpr (i == VSTEPS - 2) {      // the slots of block kt + 3 for the next iteration's loads, the entries of kt + 4
+            if constexpr (WAVES == 4 && i == VSTEPS - 2) {      // the slots of block kt + 3 for the next iteration's loads, the entries of kt + 4
                 take_slots();
                 load_entries(upto(kt + 4));
             }
@@ -404,13 +430,54 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
     };
     // Blocks wholly visible to every row of the workgroup first (none under a sliding window), then the masked ones.
     const int kt_full = win > 0 ? kt_lo : max(kt_lo, min(kt_hi + 1, (pos + t_lo + 1) / BN));
-    for (int kt = kt_lo; kt < kt_full; ++kt) {
-        block(kt, std::integral_constant<int, 0>{});
-        __syncthreads();          // every wavefront is done with this buffer; the other one is stored
-    }
-    for (int kt = kt_full; kt <= kt_hi; ++kt) {
-        block(kt, std::integral_constant<int, 1>{});
-        __syncthreads();
+    if constexpr (WAVES == 4) {
+        for (int kt = kt_lo; kt < kt_full; ++kt) {
+            scores(kt, (kt & 1) ^ 1), weigh(kt, kt & 1, c0), values(kt, kt & 1);
+            __syncthreads();          // every wavefront is done with this buffer; the other one is stored
+        }
+        for (int kt = kt_full; kt <= kt_hi; ++kt) {
+            scores(kt, (kt & 1) ^ 1), weigh(kt, kt & 1, c1), values(kt, kt & 1);
+            __syncthreads();
+        }
+    } else {
+        // Eight wavefronts, two a SIMD, and the barrier keeps them in step: were both of a SIMD in the same phase, its
+        // matrix pipe would idle while they weigh and its vector pipe while they multiply. So wavefronts 4 to 7 run a
+        // block's phases rotated by one iteration: between two barriers they weigh and multiply the values of block
+        // kt - 1 and then take the scores of block kt, while wavefronts 0 to 3 take the scores of block kt, weigh it
+        // and multiply its values: whenever one of a SIMD's two is in a matrix phase the other is in vector work or in the
+        // other matrix phase's complement. Both kinds stage block kt + 1 during their scores of block kt, so a K buffer
+        // is read in one iteration by all (two buffers) and a V buffer in two successive ones (three).
+        auto after = [](int b) { return b == 2 ? 0 : b + 1; };
+        const bool behind = __builtin_amdgcn_readfirstlane(wave >> 2) != 0;
+        if (!behind) {
+            int vcur = 0;
+            for (int kt = kt_lo; kt < kt_full; ++kt) {
+                scores(kt, after(vcur)), weigh(kt, vcur, c0), values(kt, vcur);
+                __syncthreads();
+                vcur = after(vcur);
+            }
+            for (int kt = kt_full; kt <= kt_hi; ++kt) {
+                scores(kt, after(vcur)), weigh(kt, vcur, c1), values(kt, vcur);
+                __syncthreads();
+                vcur = after(vcur);
+            }
+        } else {
+            scores(kt_lo, 1);
+            __syncthreads();
+            int vprev = 0, vcur = 1;
+            const int kt_mid = min(kt_full, kt_hi);      // iterations up to here weigh a wholly visible block (kt - 1)
+            for (int kt = kt_lo + 1; kt <= kt_mid; ++kt) {
+                weigh(kt - 1, vprev, c0), values(kt - 1, vprev), scores(kt, after(vcur));
+                __syncthreads();
+                vprev = vcur, vcur = after(vcur);
+            }
+            for (int kt = max(kt_lo, kt_mid) + 1; kt <= kt_hi; ++kt) {
+                weigh(kt - 1, vprev, c1), values(kt - 1, vprev), scores(kt, after(vcur));
+                __syncthreads();
+                vprev = vcur, vcur = after(vcur);
+            }
+            weigh(kt_hi, vprev, c1), values(kt_hi, vprev);      // (a mask over a wholly visible block changes nothing)
+        }
     }
     // The two half-waves hold the same row's sums over different keys.
     l += __shfl_xor(l, 32);
@@ -444,10 +511,16 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a) {
 }
 
 template <int KIND, bool F16>
-static int launch_d(const PrefillArgs& a, int d, dim3 grid, hipStream_t stream) {
+static int launch_d(const PrefillArgs& a, int d, bool wide, dim3 grid, hipStream_t stream) {
     switch (d) {
-        case 64: hipLaunchKernelGGL((prefill_kernel<KIND, F16, 64>), grid, dim3(256), 0, stream, a); break;
-        case 128: hipLaunchKernelGGL((prefill_kernel<KIND, F16, 128>), grid, dim3(256), 0, stream, a); break;
+        case 64: hipLaunchKernelGGL((prefill_kernel<KIND, F16, 64, 4>), grid, dim3(256), 0, stream, a); break;
+        case 128:
+            if (wide) {
+                hipLaunchKernelGGL((prefill_kernel<KIND, F16, 128, 8>), grid, dim3(512), 0, stream, a);
+            } else {
+                hipLaunchKernelGGL((prefill_kernel<KIND, F16, 128, 4>), grid, dim3(256), 0, stream, a);
+            }
+            break;
         default: return CRIT_PKV_E_GEOMETRY;
     }
     return hip_code(hipGetLastError());
@@ -488,16 +561,20 @@ int launch_prefill(const crit_pkv_prefill_params* p, hipStream_t stream) {
     a.page_magic = (uint32_t)((((1ull << a.page_l) - (uint64_t)p->page) << 32) / (uint64_t)p->page + 1);
     a.sliding = p->sliding, a.out_dtype = p->out_dtype;
     a.sscale = p->scale * kLog2e, a.k_mult = p->key_multiplier, a.v_mult = p->value_multiplier;
-    const int64_t tiles = ((int64_t)p->max_count * a.g + BM - 1) / BM;
+    // 128-wide heads: eight wavefronts on 256 rows stage each key block once for twice the rows, which pays where the
+    // launch still has a workgroup or more for every compute unit.
     const int64_t groups8 = ((int64_t)p->kv_heads * p->chunks + 7) / 8;
+    int64_t tiles = ((int64_t)p->max_count * a.g + 2 * BM - 1) / (2 * BM);
+    const bool wide = p->head_dim == 128 && tiles * p->kv_heads * p->chunks >= compute_units();
+    if (!wide) tiles = ((int64_t)p->max_count * a.g + BM - 1) / BM;
     if (tiles * groups8 * 8 > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
     a.tiles = (int)tiles;
     const dim3 grid((unsigned)(tiles * groups8 * 8));
     switch (p->kind) {
-        case 0: return f16 ? launch_d<0, true>(a, p->head_dim, grid, stream) : launch_d<0, false>(a, p->head_dim, grid, stream);
-        case 1: return launch_d<1, false>(a, p->head_dim, grid, stream);
-        case 2: return launch_d<2, false>(a, p->head_dim, grid, stream);
-        case 3: return launch_d<3, false>(a, p->head_dim, grid, stream);
+        case 0: return f16 ? launch_d<0, true>(a, p->head_dim, wide, grid, stream) : launch_d<0, false>(a, p->head_dim, wide, grid, stream);
+        case 1: return launch_d<1, false>(a, p->head_dim, wide, grid, stream);
+        case 2: return launch_d<2, false>(a, p->head_dim, wide, grid, stream);
+        case 3: return launch_d<3, false>(a, p->head_dim, wide, grid, stream);
     }
     return CRIT_PKV_E_DTYPE;
 }
