@@ -225,8 +225,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
             dst[kb] = *reinterpret_cast<const u32x4*>(&kl[(32 * kb + n32) * KSTR + 16 * i + 8 * h]);
     };
     // Byte offset of the lane's V^T operand inside a buffer: row 32 nb + n32, the 16-byte slot of groups 4 g + h and
-    // 4 g + 2 + h = v_place(4 g + h, 32 nb + n32) less its half bit = v_read ^ (16 (2 g ^ 4 (nb & 1))) + 4096 nb; the
-    // two groups come in that order in rows below 64 and swapped above.
+    // 4 g + 2 + h = v_place(4 g + h, 32 nb + n32) = v_read ^ (16 (2 g ^ 4 (nb & 1))) + 4096 nb.
     const uint32_t v_read = (uint32_t)v_place(h, n32);
     auto read_v = [&](const uint16_t* vl, auto ic, u32x4 (&dst)[2]) __attribute__((always_inline)) {
         constexpr int i = decltype(ic)::value;
@@ -236,7 +235,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
         for (int j = 0; j < 2; ++j) {
             const int nb = 2 * (i % (NB / 2)) + j;
             const u32x4 w = *reinterpret_cast<const u32x4*>(vb + (v_read ^ (16u * ((2 * g) ^ (4 * (nb & 1))))) + 32 * BN * 2 * nb);
-            dst[j] = (nb >> 1) ? u32x4{w.z, w.w, w.x, w.y} : w;
+            dst[j] = w;
         }
     };
 

@@ -97,15 +97,15 @@ PKV_DEV float dot2_acc(uint32_t a, uint32_t b, float c) {
 // V^T in LDS is [dim][64 keys], rows of 128 bytes without padding, in 8-byte groups of four keys. The second product's
 // lane (row, h) multiplies, in its step over keys 16 g .. 16 g + 15, the groups 4 g + h and 4 g + 2 + h (the keys whose
 // probabilities the first product left in that lane), so a row keeps those two side by side in one 16-byte slot, slot
-// 2 g + h, and the operand is ONE 16-byte read. Slots are swizzled by the row, slot ^ (row & 7) ^ ((row >> 3) & 7), and
-// the two halves of a slot swap in rows 64 and up: the stores (16 lanes: 16 dim chunks of 8 rows, one row of each, 8
-// bytes a lane) and the operand reads (16 lanes: 16 adjacent rows, 16 bytes a lane) both spread evenly over the banks,
-// and every term is a XOR of bit fields, so an address is one per-thread value XOR a compile-time constant plus a
-// compile-time offset. v_place: the byte offset of key group kg in row `row`.
+// 2 g + h, and the operand is ONE 16-byte read. Slots are swizzled by the row, slot ^ (row & 7) ^ ((row >> 3) & 7): the
+// operand reads (16 lanes: 16 adjacent rows, 16 bytes a lane) spread evenly over the banks, the stores (16 lanes: 16
+// dim chunks of 8 rows, one row of each, 8 bytes a lane) two to a bank (rows 64 apart meet; a store is a small share
+// of the traffic, and swapping the halves of a slot in the upper rows instead would cost the reads a register
+// shuffle). Every term is a XOR of bit fields, so an address is one per-thread value XOR a compile-time constant plus
+// a compile-time offset. v_place: the byte offset of key group kg in row `row`.
 PKV_DEV int v_place(int kg, int row) {
     const int slot = (2 * (kg >> 2) + (kg & 1)) ^ (row & 7) ^ ((row >> 3) & 7);
-    const int half = ((kg >> 1) & 1) ^ ((row >> 6) & 1);
-    return 128 * row + 16 * slot + 8 * half;
+    return 128 * row + 16 * slot + 8 * ((kg >> 1) & 1);
 }
 
 // Workgroups start in grid order, and a launch's tail is as long as the last ones to start: the chunks are taken
