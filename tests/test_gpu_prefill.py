@@ -105,6 +105,41 @@ def test_several_chunks_in_one_launch_equal_one_launch_each():
     torch.testing.assert_close(lse[-1:].double().cpu(), want_lse, atol=1e-3, rtol=1e-4)
 
 
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("window", [0, 300])
+def test_launches_that_fill_the_chip_equal_one_launch_per_chunk(kind, window):
+    # 128-wide heads: a launch with 256-row tiles for every compute unit or more (here 8 chunks x 8 KV heads x 4 tiles
+    # = 256) runs eight wavefronts a workgroup, half of them a phase behind; a chunk launched alone runs four on
+    # 128-row tiles. Every bit equal, every kind, ragged counts, with and without a window and sinks; and the oracle.
+    pk = kernels()
+    counts = [256, 255, 256, 129, 256, 1, 200, 256]
+    prefixes = [0, 7, 64, 500, 1023, 1100, 63, 128]
+    lengths = [p + c for p, c in zip(prefixes, counts)]
+    cache = Cache(kind, 8, 128, 128, 16, lengths, seed=17, scale=0.5)
+    starts = [sum(counts[:i]) for i in range(8)]
+    q32 = rand_q(sum(counts), 32, 128, 19)
+    q = q32.to(torch.float16 if kind == "fp16" else torch.bfloat16)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    positions = torch.tensor(prefixes, dtype=torch.int64, device=dev)
+    sinks = torch.linspace(-1, 1, 32, device=dev) if window else None
+    kw = dict(key_scales=cache.ks, value_scales=cache.vs, multipliers=cache.multipliers, sliding=window, sinks=sinks)
+    lse = torch.empty(q.shape[0], 32, device=dev)
+    out = pk.prefill_rows(q, cache.k, cache.v, kind, cache.tables, i32(list(range(8))), i32(starts), i32(counts),
+                          positions, 256, 16, lse=lse, **kw)
+    for s in range(8):
+        rows = slice(starts[s], starts[s] + counts[s])
+        one_lse = torch.empty(counts[s], 32, device=dev)
+        one = pk.prefill(q[rows], cache.k, cache.v, kind, cache.tables[s], prefixes[s], 16, lse=one_lse, **kw)
+        assert torch.equal(out[rows], one), s
+        assert torch.equal(lse[rows], one_lse), s
+    if not window:
+        for s, t in ((0, 0), (3, 128), (4, 255), (5, 0), (7, 100)):
+            row = starts[s] + t
+            want, want_lse = cache.want(q32[row:row + 1], s, prefixes[s] + t, 1)
+            torch.testing.assert_close(out[row:row + 1].double().cpu(), want, atol=ATOL, rtol=RTOL, msg=f"chunk {s} token {t}")
+            torch.testing.assert_close(lse[row:row + 1].double().cpu(), want_lse, atol=1e-3, rtol=1e-4, msg=f"lse {s} {t}")
+
+
 def test_prefill_agrees_with_the_decode_reader_within_the_readers_rounding():
     pk = kernels()
     cache = Cache("bf16", 2, 128, 128, 16, [400])
