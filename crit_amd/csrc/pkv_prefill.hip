@@ -17,8 +17,10 @@
 
 namespace pkv {
 
-template <int KIND, bool F16, int D, int WAVES>
+// RESUME: the launch that continues rows from their states over a chunk's fresh rows (PrefillArgs::mode 2; 16-bit only).
+template <int KIND, bool F16, int D, int WAVES, bool RESUME = false>
 __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillArgs a) {
+    static_assert(!RESUME || KIND == 0, "fresh rows are 16-bit");
     static_assert(WAVES == 4 || (WAVES == 8 && D == 128), "eight wavefronts: 128-wide heads only");
     constexpr int NT = 64 * WAVES;      // threads of the workgroup
     constexpr int BMW = 32 * WAVES;     // query rows it holds
@@ -56,6 +58,14 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
     int64_t pos64 = a.positions[z];
     pos64 = pos64 < 0 ? 0 : (pos64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : pos64);
     const int pos = (int)pos64;
+    // Positions from `first` on belong to the other launch of a chunk with fresh rows (between the chunk's position
+    // and its end, as the reference clamps it).
+    int first = 0;
+    if (a.mode != 0) {
+        int64_t f = a.firsts ? a.firsts[z] : pos64;
+        f = f < pos64 ? pos64 : (f > pos64 + count ? pos64 + count : f);
+        first = (int)f;
+    }
     const int64_t trow = (int64_t)(a.table_rows ? a.table_rows[z] : z) * a.tab_stride;
 
     // This lane's query row.
@@ -91,10 +101,16 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
 
     const int t_lo = tile * BMW / a.g;
     const int t_hi = min(count - 1, (tile * BMW + BMW - 1) / a.g);
-    const int n_max = pos + count - 1;                 // the chunk's last written position
-    const int kt_hi = (pos + t_hi) / BN;
+    const int n_max = a.mode == 1 ? first - 1 : pos + count - 1;      // the last position whose row is read
+    int kt_hi = (pos + t_hi) / BN;
     int kt_lo = 0;
     if (win > 0) kt_lo = max(0, pos + t_lo - win + 1) / BN;
+    if (a.mode == 1) kt_hi = first > 0 ? min(kt_hi, (first - 1) / BN) : -1;
+    if (RESUME) kt_lo = max(kt_lo, first / BN);
+    const bool any_block = kt_hi >= kt_lo;      // (always with mode 0)
+    // The lowest and highest position this launch reads for any row.
+    const int cap = a.mode == 1 ? first - 1 : 0x3fffffff;
+    const int floor_excl = RESUME ? first - 1 : -0x20000000;
 
     // A block's 64 keys map onto the 64 lanes: lane i looks up the page table entry and the slot of position 64 kt + i
     // (positions past the chunk's last written one read that one), every wavefront for itself, and a thread then takes
@@ -104,7 +120,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
     const uint8_t* tab_row = (a.tables ? reinterpret_cast<const uint8_t*>(a.tables) : reinterpret_cast<const uint8_t*>(a.tables64)) +
                              (trow << (a.tables ? 2 : 3));
     const int tab_shift = a.tables ? 2 : 3;
-    const uint32_t slot_bytes = (uint32_t)a.hkv * D * EB;
+    const uint32_t k_slot_bytes = a.k_slot_bytes, v_slot_bytes = a.v_slot_bytes;
     const uint8_t* kbase = a.kp + (int64_t)kvh * D * EB;
     const uint8_t* vbase = a.vp + (int64_t)kvh * D * EB;
     // Global -> registers -> LDS. K: rows contiguous over lanes. V: a thread takes eight dims of four adjacent keys and
@@ -114,13 +130,16 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
     u32x4 kreg[KPASS], vreg[4];      // vreg[i]: key 4 kg + i; 8-bit pages fill .x and .y only
     int ent = 0, inp = 0;
     float ksreg = 1.0f, vsreg = 1.0f;
+    constexpr bool direct = RESUME;      // fresh rows: the chunk's tokens in order, no table (the launcher sets page = 1)
     auto load_entries = [&](int kt) __attribute__((always_inline)) {
         int n = kt * BN + lane;
         n = n < n_max ? n : n_max;
         uint32_t pidx = (__umulhi(a.page_magic, (uint32_t)n) + (uint32_t)n) >> a.page_l;
-        inp = n - (int)pidx * a.page;
+        const int in_page = n - (int)pidx * a.page;
         pidx = pidx < (uint32_t)a.tab_width ? pidx : (uint32_t)a.tab_width - 1u;
-        ent = *reinterpret_cast<const int*>(tab_row + (pidx << tab_shift));
+        const int got = *reinterpret_cast<const int*>(tab_row + ((direct ? 0u : pidx) << tab_shift));      // (unconditional: entry 0 when unused)
+        ent = direct ? start + max(n - pos, 0) : got;
+        inp = direct ? 0 : in_page;
     };
     // take_slots turns the entries into slots and hands every thread the slots of its rows; it runs during the second
     // product of the iteration before the loads that use them, so the exchange's latency passes behind the products
@@ -143,7 +162,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
         const uint8_t* kthread = kbase + (tid % CH) * 16;
         static_for<KPASS>([&](auto pc) __attribute__((always_inline)) {
             constexpr int p = decltype(pc)::value;
-            kreg[p] = *reinterpret_cast<const u32x4*>(kthread + (uint64_t)rowslot[p] * slot_bytes);
+            kreg[p] = *reinterpret_cast<const u32x4*>(kthread + (uint64_t)rowslot[p] * k_slot_bytes);
         });
         if constexpr (KIND >= 2) ksreg = a.ks[(uint64_t)myslot * a.hkv + kvh];
     };
@@ -151,7 +170,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
         const uint8_t* vthread = vbase + (tid % VGROUPS % VC) * (DPT * EB);
         static_for<4>([&](auto ic) __attribute__((always_inline)) {
             constexpr int i = decltype(ic)::value;
-            const uint8_t* row = vthread + (uint64_t)rowslot[KPASS + i] * slot_bytes;
+            const uint8_t* row = vthread + (uint64_t)rowslot[KPASS + i] * v_slot_bytes;
             if constexpr (DPT * EB == 16) {
                 vreg[i] = *reinterpret_cast<const u32x4*>(row);
             } else if constexpr (DPT * EB == 8) {
@@ -245,6 +264,19 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
 #pragma unroll
         for (int v = 0; v < 16; ++v) o[nb][v] = 0.0f;
     float m = -INFINITY, l = 0.0f;
+    if (RESUME && live) {
+        const int64_t state_at = ((int64_t)(start + t) * a.hq + head) * (D + kStatePad);      // the state the launch over the pages left: this lane's dims, the row's maximum, its sum once
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+            for (int v4 = 0; v4 < 4; ++v4) {
+                const float4 x = *reinterpret_cast<const float4*>(a.state + state_at + 32 * nb + 8 * v4 + 4 * h);
+                o[nb][4 * v4] = x.x, o[nb][4 * v4 + 1] = x.y, o[nb][4 * v4 + 2] = x.z, o[nb][4 * v4 + 3] = x.w;
+            }
+        }
+        m = a.state[state_at + D];
+        l = h == 0 ? a.state[state_at + D + 1] : 0.0f;
+    }
 
     // Double-buffered LDS, one barrier a block: block kt is multiplied from buffer kt & 1 while block kt + 1 (already
     // in registers) is stored into the other buffer and its registers are at once reloaded with block kt + 2 (a whole
@@ -252,20 +284,22 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
     // load of the loop is unconditional (past the last block it repeats the last one), so the compiler counts the
     // outstanding loads exactly instead of waiting for all of them.
     auto upto = [&](int kt) __attribute__((always_inline)) { return kt < kt_hi ? kt : kt_hi; };
-    load_entries(kt_lo);
-    take_slots();
-    load_k();
-    load_v();
-    load_entries(upto(kt_lo + 1));
-    store_k(kt_lo & 1);
-    store_v(WAVES == 8 ? 0 : kt_lo & 1);
-    take_slots();
-    load_k();
-    load_v();
-    load_entries(upto(kt_lo + 2));
-    take_slots();
-    load_entries(upto(kt_lo + 3));
-    __syncthreads();
+    if (any_block) {
+        load_entries(kt_lo);
+        take_slots();
+        load_k();
+        load_v();
+        load_entries(upto(kt_lo + 1));
+        store_k(kt_lo & 1);
+        store_v(WAVES == 8 ? 0 : kt_lo & 1);
+        take_slots();
+        load_k();
+        load_v();
+        load_entries(upto(kt_lo + 2));
+        take_slots();
+        load_entries(upto(kt_lo + 3));
+        __syncthreads();
+    }
 
     // A key block in three phases. scores: S^T = K Q^T on the matrix cores, with the staging of the next block in its
     // shadow. weigh: mask, running maximum, the first exponentials (vector work). values: O^T += V^T P^T on the matrix
@@ -358,8 +392,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
         PKV_SB();
         if constexpr (MASK > 0) {
             // key 32 kb + 8 (v / 4) + v % 4 + 4 h is visible iff that constant is in (rel_lo, rel]
-            const int rel = lim - kt * BN - 4 * h;
-            const int rel_lo = win > 0 ? rel - win : -0x40000000;
+            const int rel = min(lim, cap) - kt * BN - 4 * h;
+            const int rel_lo = max(win > 0 ? lim - win : -0x20000000, floor_excl) - kt * BN - 4 * h;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
@@ -428,8 +462,12 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
         l = __builtin_fmaf(l, alpha, sum);
     };
     // Blocks wholly visible to every row of the workgroup first (none under a sliding window), then the masked ones.
-    const int kt_full = win > 0 ? kt_lo : max(kt_lo, min(kt_hi + 1, (pos + t_lo + 1) / BN));
-    if constexpr (WAVES == 4) {
+    int kt_full = win > 0 ? kt_lo : max(kt_lo, min(kt_hi + 1, (pos + t_lo + 1) / BN));
+    if (a.mode == 1) kt_full = max(kt_lo, min(kt_full, first / BN));      // blocks wholly below the first fresh position
+    if (RESUME) kt_full = kt_lo;
+    if (!any_block) {
+        // no position of this launch for these rows: the state passes through
+    } else if constexpr (WAVES == 4) {
         for (int kt = kt_lo; kt < kt_full; ++kt) {
             scores(kt, (kt & 1) ^ 1), weigh(kt, kt & 1, c0), values(kt, kt & 1);
             __syncthreads();          // every wavefront is done with this buffer; the other one is stored
@@ -481,6 +519,21 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
     // The two half-waves hold the same row's sums over different keys.
     l += __shfl_xor(l, 32);
     if (!live) return;
+    if (a.mode == 1) {
+        const int64_t state_at = ((int64_t)(start + t) * a.hq + head) * (D + kStatePad);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+            for (int v4 = 0; v4 < 4; ++v4) {
+                // (the values' one multiplier, which a launch of its own applies with the final division, goes in here:
+                // the fresh rows that follow count as given)
+                *reinterpret_cast<float4*>(a.state + state_at + 32 * nb + 8 * v4 + 4 * h) =
+                    make_float4(o[nb][4 * v4] * v_mult, o[nb][4 * v4 + 1] * v_mult, o[nb][4 * v4 + 2] * v_mult, o[nb][4 * v4 + 3] * v_mult);
+            }
+        }
+        if (h == 0) a.state[state_at + D] = m, a.state[state_at + D + 1] = l;
+        return;
+    }
     if (a.sinks) {
         const Fold f = fold(m, l, a.sinks[head] * kLog2e, 1.0f);
 #pragma unroll
@@ -509,20 +562,42 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
     if (a.lse && h == 0) a.lse[(int64_t)(start + t) * a.hq + head] = l != 0.0f ? __builtin_fmaf(m, kLn2, __logf(l)) : -INFINITY;
 }
 
-template <int KIND, bool F16>
+template <int KIND, bool F16, bool RESUME = false>
 static int launch_d(const PrefillArgs& a, int d, bool wide, dim3 grid, hipStream_t stream) {
     switch (d) {
-        case 64: hipLaunchKernelGGL((prefill_kernel<KIND, F16, 64, 4>), grid, dim3(256), 0, stream, a); break;
+        case 64: hipLaunchKernelGGL((prefill_kernel<KIND, F16, 64, 4, RESUME>), grid, dim3(256), 0, stream, a); break;
         case 128:
             if (wide) {
-                hipLaunchKernelGGL((prefill_kernel<KIND, F16, 128, 8>), grid, dim3(512), 0, stream, a);
+                hipLaunchKernelGGL((prefill_kernel<KIND, F16, 128, 8, RESUME>), grid, dim3(512), 0, stream, a);
             } else {
-                hipLaunchKernelGGL((prefill_kernel<KIND, F16, 128, 4>), grid, dim3(256), 0, stream, a);
+                hipLaunchKernelGGL((prefill_kernel<KIND, F16, 128, 4, RESUME>), grid, dim3(256), 0, stream, a);
             }
             break;
         default: return CRIT_PKV_E_GEOMETRY;
     }
     return hip_code(hipGetLastError());
+}
+
+// One launch: the grid for the shape the launch takes, then the kernel of its kind.
+static int launch_one(PrefillArgs a, int kind, bool f16, int head_dim, int kv_heads, int chunks, int max_count, hipStream_t stream) {
+    // 128-wide heads: eight wavefronts on 256 rows stage each key block once for twice the rows, which pays where the
+    // launch still has a workgroup or more for every compute unit.
+    const int64_t groups8 = ((int64_t)kv_heads * chunks + 7) / 8;
+    int64_t tiles = ((int64_t)max_count * a.g + 2 * BM - 1) / (2 * BM);
+    const bool wide = head_dim == 128 && tiles * kv_heads * chunks >= compute_units();
+    if (!wide) tiles = ((int64_t)max_count * a.g + BM - 1) / BM;
+    if (tiles * groups8 * 8 > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
+    a.tiles = (int)tiles;
+    const dim3 grid((unsigned)(tiles * groups8 * 8));
+    switch (kind) {
+        case 0:
+            if (a.mode == 2) return f16 ? launch_d<0, true, true>(a, head_dim, wide, grid, stream) : launch_d<0, false, true>(a, head_dim, wide, grid, stream);
+            return f16 ? launch_d<0, true>(a, head_dim, wide, grid, stream) : launch_d<0, false>(a, head_dim, wide, grid, stream);
+        case 1: return launch_d<1, false>(a, head_dim, wide, grid, stream);
+        case 2: return launch_d<2, false>(a, head_dim, wide, grid, stream);
+        case 3: return launch_d<3, false>(a, head_dim, wide, grid, stream);
+    }
+    return CRIT_PKV_E_DTYPE;
 }
 
 int launch_prefill(const crit_pkv_prefill_params* p, hipStream_t stream) {
@@ -542,6 +617,16 @@ int launch_prefill(const crit_pkv_prefill_params* p, hipStream_t stream) {
         (reinterpret_cast<uintptr_t>(p->q) % 16) || (reinterpret_cast<uintptr_t>(p->out) % 16) ||
         (reinterpret_cast<uintptr_t>(p->key_pages) % 16) || (reinterpret_cast<uintptr_t>(p->value_pages) % 16))
         return CRIT_PKV_E_GEOMETRY;
+    const bool fresh = p->fresh_keys != nullptr || p->fresh_values != nullptr;
+    if (fresh) {
+        if (!p->fresh_keys || !p->fresh_values || !p->fresh_state) return CRIT_PKV_E_NULL;
+        const int64_t row = (int64_t)p->kv_heads * p->head_dim;
+        if (p->fresh_stride_k < row || p->fresh_stride_v < row || p->fresh_stride_k % 8 || p->fresh_stride_v % 8 ||
+            p->fresh_stride_k > 0x3fffffff || p->fresh_stride_v > 0x3fffffff ||
+            (reinterpret_cast<uintptr_t>(p->fresh_keys) % 16) || (reinterpret_cast<uintptr_t>(p->fresh_values) % 16) ||
+            (reinterpret_cast<uintptr_t>(p->fresh_state) % 16))
+            return CRIT_PKV_E_GEOMETRY;
+    }
     PrefillArgs a;
     a.q = reinterpret_cast<const uint8_t*>(p->q);
     a.kp = reinterpret_cast<const uint8_t*>(p->key_pages);
@@ -560,22 +645,22 @@ int launch_prefill(const crit_pkv_prefill_params* p, hipStream_t stream) {
     a.page_magic = (uint32_t)((((1ull << a.page_l) - (uint64_t)p->page) << 32) / (uint64_t)p->page + 1);
     a.sliding = p->sliding, a.out_dtype = p->out_dtype;
     a.sscale = p->scale * kLog2e, a.k_mult = p->key_multiplier, a.v_mult = p->value_multiplier;
-    // 128-wide heads: eight wavefronts on 256 rows stage each key block once for twice the rows, which pays where the
-    // launch still has a workgroup or more for every compute unit.
-    const int64_t groups8 = ((int64_t)p->kv_heads * p->chunks + 7) / 8;
-    int64_t tiles = ((int64_t)p->max_count * a.g + 2 * BM - 1) / (2 * BM);
-    const bool wide = p->head_dim == 128 && tiles * p->kv_heads * p->chunks >= compute_units();
-    if (!wide) tiles = ((int64_t)p->max_count * a.g + BM - 1) / BM;
-    if (tiles * groups8 * 8 > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
-    a.tiles = (int)tiles;
-    const dim3 grid((unsigned)(tiles * groups8 * 8));
-    switch (p->kind) {
-        case 0: return f16 ? launch_d<0, true>(a, p->head_dim, wide, grid, stream) : launch_d<0, false>(a, p->head_dim, wide, grid, stream);
-        case 1: return launch_d<1, false>(a, p->head_dim, wide, grid, stream);
-        case 2: return launch_d<2, false>(a, p->head_dim, wide, grid, stream);
-        case 3: return launch_d<3, false>(a, p->head_dim, wide, grid, stream);
-    }
-    return CRIT_PKV_E_DTYPE;
+    a.firsts = nullptr, a.state = nullptr, a.mode = 0;
+    a.k_slot_bytes = a.v_slot_bytes = (uint32_t)p->kv_heads * p->head_dim * (p->kind == 0 ? 2 : 1);
+    a.tiles = 0;
+    if (!fresh) return launch_one(a, p->kind, f16, p->head_dim, p->kv_heads, p->chunks, p->max_count, stream);
+    // The positions below each chunk's first fresh one from the pages, then the rest from the fresh rows (16-bit, in
+    // q's type, no scales), through the rows' states.
+    a.firsts = p->fresh_firsts, a.state = p->fresh_state, a.mode = 1;
+    const int err = launch_one(a, p->kind, f16, p->head_dim, p->kv_heads, p->chunks, p->max_count, stream);
+    if (err != 0) return err;
+    a.mode = 2;
+    a.kp = reinterpret_cast<const uint8_t*>(p->fresh_keys), a.vp = reinterpret_cast<const uint8_t*>(p->fresh_values);
+    a.k_slot_bytes = (uint32_t)(p->fresh_stride_k * 2), a.v_slot_bytes = (uint32_t)(p->fresh_stride_v * 2);
+    a.ks = a.vs = a.hm = nullptr;
+    a.k_mult = a.v_mult = 1.0f;
+    a.page = 1, a.page_l = 0, a.page_magic = 1;
+    return launch_one(a, 0, f16, p->head_dim, p->kv_heads, p->chunks, p->max_count, stream);
 }
 
 }   // namespace pkv

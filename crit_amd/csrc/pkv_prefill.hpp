@@ -25,7 +25,17 @@ struct PrefillArgs {
     int tab_width, chunks, max_count, hq, hkv, g, page, page_l, sliding, out_dtype, tiles;
     uint32_t page_magic;     // n / page == (mulhi(page_magic, n) + n) >> page_l for 0 <= n < 2^31
     float sscale, k_mult, v_mult;
+    // A chunk whose own positions from `first` on are read from fresh 16-bit rows takes two launches that hand a row's
+    // running state (unnormalised output, maximum, sum) through `state`: mode 1 reads the positions below the chunk's
+    // first fresh one from the pages and writes the state; mode 2 starts from it, reads the positions from the first
+    // fresh one on as rows of kp / vp (row = the chunk's first token + position - the chunk's position, no page table) and
+    // finishes the rows. Mode 0: one launch over the pages.
+    const int64_t* firsts;   // [chunks], or null: the chunk's position (all of its own positions are fresh)
+    float* state;            // [token][head][kStateRow] FP32
+    int mode;
+    uint32_t k_slot_bytes, v_slot_bytes;     // bytes from one slot's (or fresh row's) K / V row to the next
 };
+constexpr int kStatePad = 4;      // a row of the state is head_dim + 4 floats: the output, the maximum, the sum, 16-byte rows
 
 // A wavefront raises its priority while it issues matrix instructions, so the other wavefront of its SIMD fills the
 // gaps with vector work instead of delaying them.

@@ -34,7 +34,8 @@ from . import _abi
 
 __all__ = ["KINDS", "PIECE", "MAX_COLUMNS", "Derive", "attend", "derive", "cuda_block", "cuda_chunk", "cuda_parts",
            "cuda_prompt", "cuda_ramp", "cuda_splits", "flash_block", "flash_chunk", "flash_parts", "flash_tile",
-           "merge_shards", "owner", "partitions", "piece_size", "prefill", "prefill_rows", "release", "stream_read",
+           "merge_shards", "owner", "partitions", "piece_size", "prefill", "prefill_rows", "prefill_state_floats", "release",
+           "stream_read",
            "tile_for", "workspace_floats", "write"]
 
 KINDS = {"bf16": 0, "fp16": 0, "fp8": 1, "fp8:row": 2, "int8": 3}
@@ -83,8 +84,9 @@ def owner(key):
 
 def release(key):
     """Drop an owner's module workspaces (its captured graphs must be gone)."""
-    for at in [at for at in _workspaces if at[1] == key]:
-        del _workspaces[at]
+    for held in (_workspaces, _states):
+        for at in [at for at in held if at[1] == key]:
+            del held[at]
     _retired[:] = [(k, found) for k, found in _retired if k != key]
 
 
@@ -454,8 +456,55 @@ def merge_shards(outs, lses):
 
 
 # -- prompt chunks -----------------------------------------------------------------------------------------------------------
+def prefill_state_floats(tokens, heads, dim):
+    """FP32 floats of the scratch a prompt launch with fresh rows hands its rows' states through (prefill's and
+    prefill_rows' workspace=), for q of `tokens` rows."""
+    return tokens * heads * (dim + 4)
+
+
+_states = {}
+
+
+def _prefill_state(device, tokens, heads, dim, given):
+    need = prefill_state_floats(tokens, heads, dim)
+    if given is not None:
+        if given.dtype != torch.float32 or given.numel() < need or not given.is_contiguous() or given.device != device \
+                or given.data_ptr() % 16:
+            raise ValueError(f"a prompt chunk with fresh rows needs {need} contiguous FP32 floats of workspace on its "
+                             "device, 16-byte aligned (prefill_state_floats)")
+        return given
+    found = _states.get(_held(device))
+    if found is None or found.numel() < need:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("paged_kv_attention.prefill: run a chunk of this size with fresh rows once before "
+                               "capturing it, or pass workspace= (the rows' states are allocated outside the capture)")
+        if found is not None:
+            _retired.append((getattr(_owner, "key", None), found))
+        found = _states[_held(device)] = torch.empty(max(need, 1 << 16), dtype=torch.float32, device=device)
+    return found
+
+
+def _check_fresh(fresh, q, hkv, d, chunks):
+    """(keys, values, firsts or None) of a prompt launch's fresh rows, checked as the reference checks them
+    (__init__.py:1301-1308): [tokens][kv_heads][dim] each in q's dtype, head rows contiguous."""
+    fk, fv, firsts = fresh
+    T = q.shape[0]
+    for name, x in (("keys", fk), ("values", fv)):
+        if not torch.is_tensor(x) or x.shape != (T, hkv, d) or x.stride(-1) != 1 or x.stride(1) != d:
+            raise ValueError(f"fresh keys and values are [{T}][{hkv}][{d}], each head row contiguous")
+        if x.dtype != q.dtype or x.device != q.device:
+            raise ValueError("fresh rows in q's dtype on q's device")
+        if x.stride(0) % 8 or x.data_ptr() % 16:
+            raise ValueError("fresh rows 16-byte aligned, their token stride a multiple of 8 elements")
+    if firsts is not None and (not torch.is_tensor(firsts) or firsts.dtype != torch.int64 or firsts.device != q.device
+                               or firsts.numel() != chunks or not firsts.is_contiguous()):
+        raise ValueError("the first fresh positions are int64, one a chunk, on q's device")
+    return fk, fv, firsts
+
+
 def _prefill_launch(q, key_pages, value_pages, kind, tables, table_rows, starts, counts, positions, max_count, chunks,
-                    page, key_scales, value_scales, multipliers, scale, out, lse, sinks, sliding):
+                    page, key_scales, value_scales, multipliers, scale, out, lse, sinks, sliding, fresh=None,
+                    workspace=None):
     k_kind = _check_kind(kind, key_scales)
     _require_device(q, "prefill's q")
     T, hq, d = q.shape
@@ -493,6 +542,11 @@ def _prefill_launch(q, key_pages, value_pages, kind, tables, table_rows, starts,
     p.sliding = sliding
     p.scale = float(scale if scale is not None else d ** -0.5)
     p.key_multiplier, p.value_multiplier = km, vm
+    if fresh is not None:
+        fk, fv, firsts = _check_fresh(fresh, q, hkv, d, chunks)
+        state = _prefill_state(device, T, hq, d, workspace)
+        p.fresh_keys, p.fresh_values, p.fresh_firsts, p.fresh_state = fk.data_ptr(), fv.data_ptr(), _ptr(firsts), state.data_ptr()
+        p.fresh_stride_k, p.fresh_stride_v = fk.stride(0), fv.stride(0)
     with torch.cuda.device(device):
         _abi.check(_abi.load().crit_pkv_prefill(p, _stream(device)), "paged_kv_attention.prefill")
     return out
@@ -507,11 +561,14 @@ def prefill(q, key_pages, value_pages, kind, table, position, page, *, key_scale
     """A prompt chunk of one sequence: q [T][heads][dim] at positions position.. (their keys and values written),
     table [pages] int32 or int64 -> out [T][heads][dim] (and lse [T][heads] FP32 when given), causal. position: an
     int, or a one-element int64 device tensor read on the device. One matrix-core launch whatever `flash` says; a
-    token's bits follow its own positions only. int8_qk, fresh and derive are not served."""
+    token's bits follow its own positions only. fresh: (keys, values) [T][kv_heads][dim] in q's dtype, the chunk's own
+    as the projections gave them, or (keys, values, first): the chunk reads its own positions from `first` on (default:
+    all of them; an int or a one-element int64 device tensor, clamped to the chunk's positions) from them, unscaled,
+    and the earlier ones from the pages: two launches (the pages' positions, then the fresh rows) that hand the rows'
+    states through `workspace` (FP32, prefill_state_floats(T, heads, dim); default: one the module keeps per device,
+    grown outside a capture); a token's bits follow its own positions and `first`. int8_qk and derive are not served."""
     if derive is not None:
         raise _unsupported("derive= (keys derived from value rows)")
-    if fresh is not None:
-        raise _unsupported("fresh= (a prompt chunk's own rows)")
     if int8_qk:
         raise _unsupported("int8_qk")
     _check_sinks(sinks, q)
@@ -527,25 +584,44 @@ def prefill(q, key_pages, value_pages, kind, table, position, page, *, key_scale
         if torch.cuda.is_current_stream_capturing():
             raise RuntimeError("paged_kv_attention.prefill: a captured chunk takes its position as a device tensor")
         positions = torch.tensor([int(position)], dtype=torch.int64, device=q.device)
+    if fresh is not None:
+        if len(fresh) not in (2, 3):
+            raise ValueError("fresh is (keys, values) or (keys, values, first)")
+        first = fresh[2] if len(fresh) == 3 else None
+        if first is not None and not torch.is_tensor(first):
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError("paged_kv_attention.prefill: a captured chunk takes its first fresh position as a "
+                                   "device tensor")
+            first = torch.tensor([int(first)], dtype=torch.int64, device=q.device)
+        elif first is not None:
+            first = first.reshape(1)
+        fresh = (fresh[0], fresh[1], first)
     return _prefill_launch(q, key_pages, value_pages, kind, table.reshape(1, -1), None, None, None, positions, T, 1,
-                           page, key_scales, value_scales, multipliers, scale, out, lse, sinks, sliding)
+                           page, key_scales, value_scales, multipliers, scale, out, lse, sinks, sliding, fresh,
+                           workspace)
 
 
 def prefill_rows(q, key_pages, value_pages, kind, tables, table_rows, starts, counts, positions, max_count, page, *,
                  key_scales=None, value_scales=None, multipliers=(1.0, 1.0), scale=None, out=None, lse=None,
-                 sinks=None, sliding=0):
+                 sinks=None, sliding=0, fresh=None, workspace=None):
     """Several prompt chunks in one launch (where the reference launches prefill() once per row): chunk i is counts[i]
     <= max_count tokens from token starts[i] of q at positions positions[i].. of the sequence whose page table is
     tables[table_rows[i]]; tables [S][width] int32, table_rows/starts/counts [chunks] int32, positions [chunks] int64,
-    all on the device and read there. Not part of the reference module's interface."""
+    all on the device and read there. fresh: (keys, values, firsts) parallel to q's tokens as prefill() takes them,
+    firsts [chunks] int64 on the device or None (every chunk's own positions). Not part of the reference module's
+    interface."""
     _check_sinks(sinks, q)
     sliding = _check_sliding(sliding, None)
     chunks = int(positions.shape[0])
     if chunks == 0:
         return torch.empty_like(q) if out is None else out
+    if fresh is not None:
+        if len(fresh) not in (2, 3):
+            raise ValueError("fresh is (keys, values) or (keys, values, firsts)")
+        fresh = (fresh[0], fresh[1], fresh[2] if len(fresh) == 3 else None)
     return _prefill_launch(q, key_pages, value_pages, kind, tables, table_rows, starts, counts, positions,
                            int(max_count), chunks, page, key_scales, value_scales, multipliers, scale, out, lse, sinks,
-                           sliding)
+                           sliding, fresh, workspace)
 
 
 def stream_read(data, sink=None):

@@ -10,7 +10,7 @@ import shutil
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 NAME = "libcrit_pkv.so"
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 KIND_16BIT, KIND_FP8, KIND_FP8_ROW, KIND_INT8 = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
@@ -54,7 +54,9 @@ class PrefillParams(ctypes.Structure):
                 ("table_stride", _i64),
                 ("table_width", _i32), ("chunks", _i32), ("max_count", _i32), ("heads", _i32), ("kv_heads", _i32),
                 ("head_dim", _i32), ("page", _i32), ("kind", _i32), ("page_dtype", _i32), ("out_dtype", _i32),
-                ("sliding", _i32), ("scale", _f32), ("key_multiplier", _f32), ("value_multiplier", _f32)]
+                ("sliding", _i32), ("scale", _f32), ("key_multiplier", _f32), ("value_multiplier", _f32),
+                ("fresh_keys", _p), ("fresh_values", _p), ("fresh_firsts", _p), ("fresh_state", _p),
+                ("fresh_stride_k", _i64), ("fresh_stride_v", _i64)]
 
 
 SYMBOLS = ("crit_pkv_write", "crit_pkv_attend", "crit_pkv_merge", "crit_pkv_prefill", "crit_pkv_abi_version",

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 3
+#define CRIT_PKV_ABI_VERSION 4
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -169,6 +169,18 @@ typedef struct crit_pkv_prefill_params {
     int32_t kind, page_dtype, out_dtype;
     int32_t sliding;
     float scale, key_multiplier, value_multiplier;
+    /* A chunk's own keys and values as the projections gave them (the reference's fresh=, __init__.py:1250-1255,
+     * 1301-1308; _kernels.py:616-650): [tokens][kv_heads][head_dim] in q's type, parallel to q's tokens, each head row
+     * contiguous, token rows fresh_stride_k / fresh_stride_v elements apart. Chunk i then reads its positions from
+     * fresh_firsts[i] on (clamped to the chunk's own positions; NULL: all of them) from these rows, unscaled, and the
+     * earlier ones from the pages. Both NULL: every position from the pages. With them, fresh_state is FP32 scratch of
+     * tokens x heads x (head_dim + 4) floats (tokens: q's rows the chunks cover, counted from row 0), 16-byte
+     * aligned, that the call's two launches hand the rows' running states through. */
+    const void* fresh_keys;
+    const void* fresh_values;
+    const int64_t* fresh_firsts;
+    float* fresh_state;
+    int64_t fresh_stride_k, fresh_stride_v;
 } crit_pkv_prefill_params;
 
 int crit_pkv_prefill(const crit_pkv_prefill_params* p, void* stream);

@@ -72,14 +72,32 @@ def listed(blocks, block_size, n):
     return (torch.arange(n) // block_size)[:, None].eq(ids[None, :]).any(1)
 
 
+def with_fresh(keys, values, fresh, q_dtype):
+    """Positions from `first` on take their keys and values from the fresh rows (row = position - shift), 16-bit in
+    q's dtype and unscaled, instead of the pages' decoded ones (_kernels.py:272-274, 291-345: the scores of a fresh
+    position times the scale only, its probability times 1; device_attention.py:1136-1145 says the same of the torch
+    path). fresh = (fresh keys [N][HKV][D], fresh values [N][HKV][DV], shift, first)."""
+    fk, fv, shift, first = fresh
+    n = keys.shape[0]
+    lo = max(int(first), 0)
+    if lo >= n:
+        return keys, values
+    keys, values = keys.clone(), values.clone()
+    keys[lo:] = fk[lo - shift:n - shift].to(q_dtype).double()
+    values[lo:] = fv[lo - shift:n - shift].to(q_dtype).double()
+    return keys, values
+
+
 def window_reference(q, key_pages, value_pages, kind, table, first, count, page, scale, key_scales=None,
                      value_scales=None, multipliers=(1.0, 1.0), sliding=0, q_dtype=torch.bfloat16, parents=None,
-                     blocks=None, block_size=None):
+                     blocks=None, block_size=None, fresh=None):
     """One window row in float64: q [count][HQ][D] (rounded to q_dtype first, as the kernels read it) at positions
     first .. first + count - 1 -> (out [count][HQ][DV], lse [count][HQ]). parents: the row's draft tree (seen_by);
-    blocks [count][k] with block_size: each column's listed KV blocks (listed)."""
+    blocks [count][k] with block_size: each column's listed KV blocks (listed); fresh: with_fresh's tuple."""
     n = first + count
     keys, values = stored_rows(key_pages, value_pages, table, n, page, kind, key_scales, value_scales, multipliers)
+    if fresh is not None:
+        keys, values = with_fresh(keys, values, fresh, q_dtype)
     qd = q.to(q_dtype).double()
     outs, lses = [], []
     for c in range(count):

@@ -176,6 +176,114 @@ def test_fp32_outputs_and_warm_up_shapes():
     assert one.shape == (1, 8, 128)
 
 
+def _fresh_rows(T, hkv, d, seed, dtype):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(T, hkv, d, generator=g).to(dtype).to(dev), torch.randn(T, hkv, d, generator=g).to(dtype).to(dev))
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_a_chunk_reads_its_own_positions_from_fresh_rows(kind):
+    # fresh=(keys, values[, first]): the chunk's positions from `first` on (default: all its own) come from the 16-bit
+    # rows given, unscaled, the earlier ones from the pages (the reference's prefill(fresh=), __init__.py:1250-1255):
+    # against the oracle for every kind, a first at the chunk's start, inside a key block, at a block's edge, before
+    # the chunk (clamped to it) and past it (no fresh position: the bits of the launch without fresh rows, up to the
+    # place of FP8 pages' value multiplier); lse too.
+    pk = kernels()
+    position, T = 200, 150
+    cache = Cache(kind, 2, 128, 128, 16, [position + T], seed=23)
+    q = rand_q(T, 8, 128, 24)
+    q_dtype = torch.float16 if kind == "fp16" else torch.bfloat16
+    fk, fv = _fresh_rows(T, 2, 128, 25, q_dtype)
+    kw = dict(key_scales=cache.ks, value_scales=cache.vs, multipliers=cache.multipliers)
+    plain_lse = torch.empty(T, 8, device=dev)
+    plain = pk.prefill(q.to(q_dtype), cache.k, cache.v, kind, cache.tables[0], position, 16, lse=plain_lse, **kw)
+    for first in (None, position + 37, 256, 3, position + T, 10 ** 9):
+        lse = torch.empty(T, 8, device=dev)
+        fresh = (fk, fv) if first is None else (fk, fv, first)
+        out = pk.prefill(q.to(q_dtype), cache.k, cache.v, kind, cache.tables[0], position, 16, lse=lse, fresh=fresh, **kw)
+        at = position if first is None else min(max(first, position), position + T)
+        if at >= position + T:
+            if kind == "fp8":      # (the values' multiplier goes into the state, not into the final division: other roundings)
+                torch.testing.assert_close(out.float(), plain.float(), atol=ATOL, rtol=RTOL)
+            else:
+                assert torch.equal(out, plain), first
+            assert torch.equal(lse, plain_lse), first
+            continue
+        for t in (0, 36, 37, 56, 149):
+            want, want_lse = cache.want(q[t:t + 1], 0, position + t, 1, fresh=(fk.cpu(), fv.cpu(), position, at))
+            torch.testing.assert_close(out[t:t + 1].double().cpu(), want, atol=ATOL, rtol=RTOL, msg=f"first {first} token {t}")
+            torch.testing.assert_close(lse[t:t + 1].double().cpu(), want_lse, atol=1e-3, rtol=1e-4, msg=f"first {first} lse {t}")
+    on_device = torch.tensor([position + 37], dtype=torch.int64, device=dev)
+    a = pk.prefill(q.to(q_dtype), cache.k, cache.v, kind, cache.tables[0], position, 16, fresh=(fk, fv, on_device), **kw)
+    b = pk.prefill(q.to(q_dtype), cache.k, cache.v, kind, cache.tables[0], position, 16, fresh=(fk, fv, position + 37), **kw)
+    assert torch.equal(a, b)
+
+
+def test_fresh_rows_from_position_zero_with_a_window_and_sinks_and_a_workspace_of_the_callers():
+    # A first chunk (nothing in the pages below it), a sliding window that cuts into the fresh positions and below
+    # them, sink logits, and the rows' states in a workspace the caller gives (too small a one is refused).
+    pk = kernels()
+    cache = Cache("fp8", 2, 128, 128, 16, [700], seed=29)
+    q = rand_q(300, 8, 128, 30)
+    fk, fv = _fresh_rows(300, 2, 128, 31, torch.bfloat16)
+    kw = dict(multipliers=cache.multipliers)
+    out = pk.prefill(q.bfloat16(), cache.k, cache.v, "fp8", cache.tables[0], 0, 16, fresh=(fk, fv), **kw)
+    for t in (0, 63, 64, 299):
+        want, _ = cache.want(q[t:t + 1], 0, t, 1, fresh=(fk.cpu(), fv.cpu(), 0, 0))
+        torch.testing.assert_close(out[t:t + 1].double().cpu(), want, atol=ATOL, rtol=RTOL, msg=f"token {t}")
+    ws = torch.empty(pk.prefill_state_floats(300, 8, 128), dtype=torch.float32, device=dev)
+    for window in (50, 250):
+        lse = torch.empty(300, 8, device=dev)
+        out = pk.prefill(q.bfloat16(), cache.k, cache.v, "fp8", cache.tables[0], 400, 16, fresh=(fk, fv, 500),
+                         sliding=window, lse=lse, workspace=ws, **kw)
+        for t in (0, 99, 100, 149, 151, 299):
+            want, want_lse = cache.want(q[t:t + 1], 0, 400 + t, 1, sliding=window, fresh=(fk.cpu(), fv.cpu(), 400, 500))
+            torch.testing.assert_close(out[t:t + 1].double().cpu(), want, atol=ATOL, rtol=RTOL, msg=f"window {window} token {t}")
+            torch.testing.assert_close(lse[t:t + 1].double().cpu(), want_lse, atol=1e-3, rtol=1e-4)
+        sinks = torch.linspace(-2, 2, 8, device=dev)
+        with_sinks = pk.prefill(q.bfloat16(), cache.k, cache.v, "fp8", cache.tables[0], 400, 16, fresh=(fk, fv, 500),
+                                sliding=window, sinks=sinks, workspace=ws, **kw)
+        weight = torch.exp(lse) / (torch.exp(lse) + torch.exp(sinks)[None, :])
+        torch.testing.assert_close(with_sinks.float(), out.float() * weight[..., None], atol=8e-3, rtol=2e-2)
+    with pytest.raises(ValueError):
+        pk.prefill(q.bfloat16(), cache.k, cache.v, "fp8", cache.tables[0], 400, 16, fresh=(fk, fv), workspace=ws[:1000], **kw)
+    with pytest.raises(ValueError):
+        pk.prefill(q.bfloat16(), cache.k, cache.v, "fp8", cache.tables[0], 400, 16, fresh=(fk[:10], fv[:10]), **kw)
+    with pytest.raises(ValueError):
+        pk.prefill(q.bfloat16(), cache.k, cache.v, "fp8", cache.tables[0], 400, 16, fresh=(fk.float(), fv.float()), **kw)
+
+
+@pytest.mark.parametrize("kind", ["bf16", "fp8", "int8"])
+def test_several_chunks_with_fresh_rows_equal_one_launch_each(kind):
+    # prefill_rows(fresh=(keys, values, firsts)): the rows parallel to q's tokens, a first per chunk on the device; a
+    # launch that fills the chip (eight wavefronts a workgroup in both of its passes) equals one launch per chunk bit
+    # for bit, and firsts of None every chunk's own positions.
+    pk = kernels()
+    counts = [256, 255, 256, 129, 256, 1, 200, 256]
+    prefixes = [0, 7, 64, 500, 1023, 1100, 63, 128]
+    firsts = [0, 100, 64, 10 ** 6, 1023 + 255, 1100, 0, 200]
+    lengths = [p + c for p, c in zip(prefixes, counts)]
+    cache = Cache(kind, 8, 128, 128, 16, lengths, seed=37, scale=0.5)
+    starts = [sum(counts[:i]) for i in range(8)]
+    q = rand_q(sum(counts), 32, 128, 38).bfloat16()
+    fk, fv = _fresh_rows(sum(counts), 8, 128, 39, torch.bfloat16)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    positions = torch.tensor(prefixes, dtype=torch.int64, device=dev)
+    kw = dict(key_scales=cache.ks, value_scales=cache.vs, multipliers=cache.multipliers)
+    for given in (torch.tensor(firsts, dtype=torch.int64, device=dev), None):
+        lse = torch.empty(q.shape[0], 32, device=dev)
+        out = pk.prefill_rows(q, cache.k, cache.v, kind, cache.tables, i32(list(range(8))), i32(starts), i32(counts),
+                              positions, 256, 16, lse=lse, fresh=(fk, fv, given), **kw)
+        for s in range(8):
+            rows = slice(starts[s], starts[s] + counts[s])
+            one_lse = torch.empty(counts[s], 32, device=dev)
+            first = prefixes[s] if given is None else firsts[s]
+            one = pk.prefill(q[rows], cache.k, cache.v, kind, cache.tables[s], prefixes[s], 16, lse=one_lse,
+                             fresh=(fk[rows], fv[rows], first), **kw)
+            assert torch.equal(out[rows], one), s
+            assert torch.equal(lse[rows], one_lse), s
+
+
 def test_what_the_prompt_reader_does_not_take_is_refused():
     pk = kernels()
     cache = Cache("int8", 2, 128, 128, 16, [40])
@@ -184,7 +292,7 @@ def test_what_the_prompt_reader_does_not_take_is_refused():
     with pytest.raises(NotImplementedError):
         pk.prefill(q, cache.k, cache.v, "int8", cache.tables[0], 36, 16, int8_qk=True, **kw)
     with pytest.raises(NotImplementedError):
-        pk.prefill(q, cache.k, cache.v, "int8", cache.tables[0], 36, 16, fresh=(q, q), **kw)
+        pk.prefill(q, cache.k, cache.v, "int8", cache.tables[0], 36, 16, derive=(None, 1e-6, None, 0), **kw)
     with pytest.raises(ValueError):
         pk.prefill(q.float(), cache.k, cache.v, "int8", cache.tables[0], 36, 16, **kw)
 

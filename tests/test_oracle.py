@@ -415,3 +415,44 @@ def test_a_block_list_sees_what_a_sequence_of_only_its_blocks_would_hold():
         assert torch.equal(full, plain)
     none, none_lse = attend.window_reference(q, k, v, "bf16", tables[0], first, 2, 16, 0.25, blocks=[[-1], [-1]], block_size=16)
     assert bool((none == 0).all()) and bool(torch.isinf(none_lse).all())
+
+
+def test_fresh_rows_replace_the_positions_from_their_first_on_unscaled():
+    # Pins with_fresh() and its use in window_reference(): a chunk that reads its positions from `first` on from fresh
+    # 16-bit rows attends as a plain chunk would over a 16-bit pool whose pages hold, at those positions, the fresh rows
+    # (written by hand below, not through with_fresh) and elsewhere the pages' decoded values; the page scales do not
+    # touch a fresh position (FP8 pages with multipliers 0.5 / 0.25: a fresh row counts as given); fresh rows that
+    # equal the stored ones, and a first past the chunk, change nothing; the worked case of one key: a token that sees
+    # only a fresh position returns that row's value whatever the pages hold.
+    gen = torch.Generator().manual_seed(11)
+    k, v, ks, vs, tables, _ = _pool("fp8", 1, 16, 16, 16, [100])
+    position, T = 60, 40
+    q = torch.randn(T, 2, 16, generator=gen)
+    fk = torch.randn(T, 1, 16, generator=gen).bfloat16()
+    fv = torch.randn(T, 1, 16, generator=gen).bfloat16()
+    mult = (0.5, 0.25)
+    keys, values = attend.stored_rows(k, v, tables[0], 100, 16, "fp8", multipliers=mult)
+    for first in (position, position + 13, 0, 10 ** 6):
+        out, lse = attend.window_reference(q, k, v, "fp8", tables[0], position, T, 16, 0.25, multipliers=mult,
+                                           fresh=(fk, fv, position, max(first, position)))
+        kk, vv = keys.clone(), values.clone()
+        for n in range(max(first, position), 100):
+            kk[n], vv[n] = fk[n - position].double(), fv[n - position].double()
+        for c in (0, 12, 13, 39):
+            seen = torch.arange(100) <= position + c
+            want, want_lse = attend.reference(q[c].bfloat16().double(), kk, vv, seen, 0.25)
+            assert torch.allclose(out[c], want, atol=1e-12, rtol=1e-12), (first, c)
+            assert torch.allclose(lse[c], want_lse, atol=1e-12, rtol=1e-12), (first, c)
+    plain, plain_lse = attend.window_reference(q, k, v, "fp8", tables[0], position, T, 16, 0.25, multipliers=mult)
+    none, none_lse = attend.window_reference(q, k, v, "fp8", tables[0], position, T, 16, 0.25, multipliers=mult,
+                                             fresh=(fk, fv, position, 10 ** 6))
+    assert torch.equal(plain, none) and torch.equal(plain_lse, none_lse)
+    k16, v16, _, _, t16, _ = _pool("bf16", 1, 16, 16, 16, [100])
+    own_k, own_v = attend.stored_rows(k16, v16, t16[0], 100, 16, "bf16")
+    same, _ = attend.window_reference(q, k16, v16, "bf16", t16[0], position, T, 16, 0.25,
+                                      fresh=(own_k[position:].bfloat16(), own_v[position:].bfloat16(), position, position))
+    assert torch.equal(same, attend.window_reference(q, k16, v16, "bf16", t16[0], position, T, 16, 0.25)[0])
+    one, one_lse = attend.window_reference(q[:1], k, v, "fp8", tables[0], 0, 1, 16, 0.25, multipliers=mult,
+                                           fresh=(fk, fv, 0, 0))
+    assert torch.allclose(one[0], fv[0, 0].double().expand(2, 16), atol=1e-12)
+    assert torch.allclose(one_lse[0], (q[0].bfloat16().double() @ fk[0, 0].double()) * 0.25, atol=1e-12)
