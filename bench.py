@@ -328,6 +328,43 @@ def mixed_prefill(pk, device):
             "decode_us": round(t_decode * 1e3, 1), "step_us": round(step * 1e3, 1)}
 
 
+def prefill_fresh(pk, device):
+    """The mixed batch's 8 prompt chunks over FP8 pages (one multiplier pair), once reading every position from the
+    pages and once with fresh=: each chunk's own 512 positions from 16-bit rows as the projections gave them, its
+    prefix from the pages (two launches through the rows' states)."""
+    hq, hkv, d, page = 32, 8, 128, 16
+    gcpu = torch.Generator().manual_seed(5)
+    prefixes = torch.randint(0, 8193, (8,), generator=gcpu).tolist()
+    widths = [(p + 512 + page - 1) // page for p in prefixes]
+    n_pages = int(sum(widths) * 1.25)
+    g = torch.Generator(device=device).manual_seed(7)
+    k = (torch.randn(n_pages + 1, page, hkv, d, device=device, generator=g) / 0.02).clamp(-448, 448).to(torch.float8_e4m3fn)
+    v = (torch.randn(n_pages + 1, page, hkv, d, device=device, generator=g) / 0.02).clamp(-448, 448).to(torch.float8_e4m3fn)
+    perm = torch.randperm(n_pages, generator=gcpu)
+    tables = torch.full((8, (max(widths) + 15) // 16 * 16), n_pages, dtype=torch.int32)
+    at = 0
+    for s, w in enumerate(widths):
+        tables[s, :w] = perm[at:at + w].to(torch.int32)
+        at += w
+    tables = tables.to(device)
+    q = torch.randn(4096, hq, d, device=device, generator=g).to(torch.bfloat16)
+    fk = torch.randn(4096, hkv, d, device=device, generator=g).to(torch.bfloat16)
+    fv = torch.randn(4096, hkv, d, device=device, generator=g).to(torch.bfloat16)
+    out = torch.empty_like(q)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=device)
+    rows, starts, counts = i32(list(range(8))), i32([512 * s for s in range(8)]), i32([512] * 8)
+    positions = torch.tensor(prefixes, dtype=torch.int64, device=device)
+    flops = sum(4 * hq * d * sum(p + t + 1 for t in range(512)) for p in prefixes)
+    ws = torch.empty(pk.prefill_state_floats(4096, hq, d), dtype=torch.float32, device=device)
+    call = lambda fresh: pk.prefill_rows(q, k, v, "fp8", tables, rows, starts, counts, positions, 512, page,
+                                         multipliers=(0.02, 0.02), out=out, fresh=fresh, workspace=ws)
+    t_pages, t_fresh = timed(lambda: call(None), 10, 2), timed(lambda: call((fk, fv, None)), 10, 2)
+    return {"prefill_GFLOP": round(flops / 1e9, 1), "pages_only_us": round(t_pages * 1e3, 1),
+            "pages_only_TFLOP/s": round(flops / t_pages / 1e9, 1), "with_fresh_rows_us": round(t_fresh * 1e3, 1),
+            "with_fresh_rows_TFLOP/s": round(flops / t_fresh / 1e9, 1),
+            "state_bytes": 2 * 4096 * hq * (d + 4) * 4}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -442,6 +479,8 @@ def main():
         log(f"[bench] block-sparse decode: {extras['block_sparse_decode_bf16']}")
         extras["mixed_prefill_decode_bf16"] = mixed_prefill(pk, device)
         log(f"[bench] mixed prefill + decode: {extras['mixed_prefill_decode_bf16']}")
+        extras["prefill_fp8_pages_fresh_rows"] = prefill_fresh(pk, device)
+        log(f"[bench] prefill over FP8 pages, with fresh rows: {extras['prefill_fp8_pages_fresh_rows']}")
         result["extra"] = extras
     if not args.no_cpu:
         log("[bench] timing the CPU reference path (about 20 s)")
