@@ -157,14 +157,14 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
     const int n_pieces = (n_run + a.piece - 1) / a.piece;
     if constexpr (!FUSED) {
         // Units are taken in list order, y slowest, and a launch's tail is as long as its last units: the row's last
-        // partition (usually a partial piece, the smallest unit of work) is listed after every other partition, at
-        // the last y but one if it holds half a piece or more and at the very last y if it holds less, so the units
-        // that start last are the smallest.
+        // partition (usually a partial piece, the smallest unit of work) is listed after every other partition, in
+        // kTailClasses rows of y by its size (a whole piece or more first, the smallest remainders last).
         const int np = min(n_pieces, a.parts);
         if (np <= 0) return;
-        const bool small = np == n_pieces && n_run - (np - 1) * a.piece < a.piece / 2;
-        if (b >= a.units_y - 2) {
-            if ((b == a.units_y - 1) != small) return;
+        int cls = 0;
+        if (np == n_pieces) cls = min(kTailClasses - 1, (np * a.piece - n_run) * kTailClasses / a.piece);
+        if (b >= a.units_y - kTailClasses) {
+            if (b - (a.units_y - kTailClasses) != cls) return;
             b = np - 1;
         } else if (b >= np - 1) {
             return;

@@ -7,6 +7,9 @@
 namespace pkv {
 
 constexpr int kMaxListedBlocks = 1024;      // block ids a token's list may hold (they are copied to LDS)
+// A split launch lists every row's last partition (usually a partial piece, the smallest unit of work) after all other
+// partitions, in this many classes of decreasing size, so that the units that start last are the smallest.
+constexpr int kTailClasses = 4;
 
 struct AttendArgs {
     const uint8_t* q;

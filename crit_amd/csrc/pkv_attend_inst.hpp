@@ -13,7 +13,7 @@ static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipS
         if (a.blocks && lpr == 16 && a.page % 16 == 0 && a.block_size % 16 == 0) {
             // block lists whose steps lie in one block and one page: the bandwidth path walking each column's list
             AttendArgs u = a;
-            u.units_x = (int)grid.x, u.units_y = (int)grid.y + 1;
+            u.units_x = (int)grid.x, u.units_y = (int)grid.y + kTailClasses - 1;
             const int64_t units = (int64_t)u.units_x * u.units_y;
             if (units > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
             const int64_t resident = (int64_t)compute_units() * attend_waves(KIND, QR);
@@ -38,7 +38,7 @@ static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipS
     if (lpr == 16 && page16) {       // pages of a multiple of 16 positions: the bandwidth path, resident workgroups pulling units
         AttendArgs u = a;
         // (a split launch lists a row's last partition twice, for the one of two size classes it falls in)
-        u.units_x = (int)grid.x, u.units_y = FUSED ? (int)grid.y : (int)grid.y + 1;
+        u.units_x = (int)grid.x, u.units_y = FUSED ? (int)grid.y : (int)grid.y + kTailClasses - 1;
         const int64_t units = (int64_t)u.units_x * u.units_y;
         if (units > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
         const int64_t resident = (int64_t)compute_units() * attend_waves(KIND, QR);
