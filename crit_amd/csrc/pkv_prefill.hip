@@ -18,9 +18,13 @@
 namespace pkv {
 
 // RESUME: the launch that continues rows from their states over a chunk's fresh rows (PrefillArgs::mode 2; 16-bit only).
-template <int KIND, bool F16, int D, int WAVES, bool RESUME = false>
+// IQK: INT8 pages with the first product in integers (the reference's int8_qk): each query row becomes INT8 codes at its
+// own scale, the keys' codes go to LDS as they are, and S^T = K Q^T is v_mfma_i32_32x32x32_i8 (32 dims a step).
+template <int KIND, bool F16, int D, int WAVES, bool RESUME = false, bool IQK = false>
 __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillArgs a) {
     static_assert(!RESUME || KIND == 0, "fresh rows are 16-bit");
+    static_assert(!IQK || KIND == 3, "integer scores: INT8 pages");
+    constexpr int KSTR8 = D + 16;       // IQK: K row stride in LDS (bytes)
     static_assert(WAVES == 4 || (WAVES == 8 && D == 128), "eight wavefronts: 128-wide heads only");
     constexpr int NT = 64 * WAVES;      // threads of the workgroup
     constexpr int BMW = 32 * WAVES;     // query rows it holds
@@ -73,12 +77,50 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
     const int t = j / a.g, head = kvh * a.g + j % a.g;
     const bool live = t < count;
     const int lim = live ? pos + t : -1;
+    // 16-bit scores: the lane's B operand of k-step ks is dims 16 ks + 8 h .. + 7 of its row. Integer scores: of step
+    // ks (32 dims) dims 32 ks + 16 h .. + 15, as codes; qreg[ks] for ks < D / 32 then holds 16 codes.
     uint4 qreg[KS];
+    float q_scale = 1.0f;      // IQK: the row's scale, amax / 127
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         qreg[ks] = make_uint4(0, 0, 0, 0);
         if (live) {
-            qreg[ks] = *reinterpret_cast<const uint4*>(a.q + ((int64_t)(start + t) * a.q_st + (int64_t)head * a.q_sh + 16 * ks + 8 * h) * 2);
+            const int dim = IQK ? 32 * (ks / 2) + 16 * h + 8 * (ks % 2) : 16 * ks + 8 * h;
+            qreg[ks] = *reinterpret_cast<const uint4*>(a.q + ((int64_t)(start + t) * a.q_st + (int64_t)head * a.q_sh + dim) * 2);
+        }
+    }
+    if constexpr (IQK) {
+        // Each query row to INT8 at its own scale (amax / 127, at least 1e-30), rounded half away from zero
+        // (_kernels.py:637-643); the two half-waves hold the two halves of the row's dims.
+        float x[KS][8];
+        float amax = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const uint32_t w[4] = {qreg[ks].x, qreg[ks].y, qreg[ks].z, qreg[ks].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                x[ks][2 * i] = u2f(w[i] << 16), x[ks][2 * i + 1] = u2f(w[i] & 0xffff0000u);
+                amax = __builtin_fmaxf(amax, __builtin_fmaxf(__builtin_fabsf(x[ks][2 * i]), __builtin_fabsf(x[ks][2 * i + 1])));
+            }
+        }
+        amax = __builtin_fmaxf(amax, __shfl_xor(amax, 32));
+        q_scale = __builtin_fmaxf(__fdiv_rn(amax, 127.0f), 1e-30f);
+#pragma unroll
+        for (int s2 = 0; s2 < KS / 2; ++s2) {
+            uint32_t code[4];
+#pragma unroll
+            for (int wd = 0; wd < 4; ++wd) {
+                uint32_t packed = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int e = 4 * wd + i;      // element 0 .. 15 of the step: registers 2 s2 (0 .. 7) and 2 s2 + 1 (8 .. 15)
+                    const float f = __fdiv_rn(x[2 * s2 + e / 8][e % 8], q_scale);
+                    const int c = (int)(f >= 0.0f ? f + 0.5f : f - 0.5f);      // (a NaN row gives codes of 0, as the cast does)
+                    packed |= ((uint32_t)c & 0xffu) << (8 * i);
+                }
+                code[wd] = packed;
+            }
+            qreg[s2] = make_uint4(code[0], code[1], code[2], code[3]);
         }
     }
     // The lowest limit among the wavefront's live rows: key blocks wholly at or below it need no mask.
@@ -88,7 +130,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
     wave_lo = __builtin_amdgcn_readfirstlane(wave_lo);
     float k_mult = a.k_mult, v_mult = a.v_mult;
     if (KIND == 1 && a.hm) k_mult = a.hm[kvh], v_mult = a.hm[a.hkv + kvh];
-    const float sscale = a.sscale * (KIND == 1 ? k_mult : 1.0f);
+    const float sscale = a.sscale * (KIND == 1 ? k_mult : 1.0f) * q_scale;
     if (KIND != 1) v_mult = 1.0f;
     const int win = a.sliding;
     const float sabs = __builtin_fabsf(sscale);
@@ -190,6 +232,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
             const int kk = idx / CH, c = idx % CH;
             if constexpr (KIND == 0) {
                 *reinterpret_cast<u32x4*>(&kl[kk * KSTR + c * 8]) = kreg[p];
+            } else if constexpr (IQK) {
+                *reinterpret_cast<u32x4*>(reinterpret_cast<uint8_t*>(kl) + kk * KSTR8 + c * 16) = kreg[p];
             } else {
                 *reinterpret_cast<u32x4*>(&kl[kk * KSTR + c * 16]) = codes_to_bf16<KIND>(kreg[p].x, kreg[p].y);
                 PKV_SB();      // one 16-byte group converted and stored at a time keeps the conversions' temporaries few
@@ -240,8 +284,13 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
     auto read_k = [&](const uint16_t* kl, auto ic, u32x4 (&dst)[2]) __attribute__((always_inline)) {
         constexpr int i = decltype(ic)::value;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-            dst[kb] = *reinterpret_cast<const u32x4*>(&kl[(32 * kb + n32) * KSTR + 16 * i + 8 * h]);
+        for (int kb = 0; kb < 2; ++kb) {
+            if constexpr (IQK) {
+                dst[kb] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint8_t*>(kl) + (32 * kb + n32) * KSTR8 + 32 * i + 16 * h);
+            } else {
+                dst[kb] = *reinterpret_cast<const u32x4*>(&kl[(32 * kb + n32) * KSTR + 16 * i + 8 * h]);
+            }
+        }
     };
     // Byte offset of the lane's V^T operand inside a buffer: row 32 nb + n32, the 16-byte slot of groups 4 g + h and
     // 4 g + 2 + h = v_place(4 g + h, 32 nb + n32) = v_read ^ (16 (2 g ^ 4 (nb & 1))) + 4096 nb.
@@ -323,20 +372,40 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
             for (int v = 0; v < 16; ++v) s[kb][v] = 0.0f;
         u32x4 ka[RING][2];
         static_for<RING - 1>([&](auto ic) __attribute__((always_inline)) { read_k(kl, ic, ka[decltype(ic)::value]); });
+        constexpr int KSTEPS = IQK ? D / 32 : KS;      // steps of 32 dims with integer scores, of 16 otherwise
+        i32x16 si[2];
+        if constexpr (IQK) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) si[kb][v] = 0;
+        }
         PKV_PRIO(1);
-        static_for<KS>([&](auto ic) __attribute__((always_inline)) {
+        static_for<KSTEPS>([&](auto ic) __attribute__((always_inline)) {
             constexpr int i = decltype(ic)::value;
-            if constexpr (i + RING - 1 < KS) read_k(kl, std::integral_constant<int, i + RING - 1>{}, ka[(i + RING - 1) % RING]);
-            s[0] = mfma<F16>(ka[i % RING][0], qreg[i], s[0]);
-            s[1] = mfma<F16>(ka[i % RING][1], qreg[i], s[1]);
+            if constexpr (i + RING - 1 < KSTEPS) read_k(kl, std::integral_constant<int, i + RING - 1>{}, ka[(i + RING - 1) % RING]);
+            if constexpr (IQK) {
+                const i32x4 qi = {(int)qreg[i].x, (int)qreg[i].y, (int)qreg[i].z, (int)qreg[i].w};
+                si[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, ka[i % RING][0]), qi, si[0], 0, 0, 0);
+                si[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, ka[i % RING][1]), qi, si[1], 0, 0, 0);
+            } else {
+                s[0] = mfma<F16>(ka[i % RING][0], qreg[i], s[0]);
+                s[1] = mfma<F16>(ka[i % RING][1], qreg[i], s[1]);
+            }
             if constexpr (i == 0) store_k(buf ^ 1), load_k();
-            if constexpr (i == KS / 2 - 1) store_v(vnext), load_v();
-            if constexpr (WAVES == 8 && i == KS - 2) {      // the slots of block kt + 3 for the next iteration's loads, the entries of kt + 4
+            if constexpr (i == KSTEPS / 2 - 1) store_v(vnext), load_v();
+            if constexpr (WAVES == 8 && i == KSTEPS - 2) {      // the slots of block kt + 3 for the next iteration's loads, the entries of kt + 4
                 take_slots();
                 load_entries(upto(kt + 4));
             }
             if constexpr (KIND != 0) PKV_SB();
         });
+        if constexpr (IQK) {      // exact integer dot products of the codes; the rows' and keys' scales follow below
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) s[kb][v] = (float)si[kb][v];
+        }
         // one product, then a share of the staging work (LDS reads of later operands, the stores' permutes and
         // writes, the row loads) in its shadow
         if constexpr (KIND == 0) {      // (8-bit pages: the conversions' temporaries make this order spill)
@@ -562,15 +631,15 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
     if (a.lse && h == 0) a.lse[(int64_t)(start + t) * a.hq + head] = l != 0.0f ? __builtin_fmaf(m, kLn2, __logf(l)) : -INFINITY;
 }
 
-template <int KIND, bool F16, bool RESUME = false>
+template <int KIND, bool F16, bool RESUME = false, bool IQK = false>
 static int launch_d(const PrefillArgs& a, int d, bool wide, dim3 grid, hipStream_t stream) {
     switch (d) {
-        case 64: hipLaunchKernelGGL((prefill_kernel<KIND, F16, 64, 4, RESUME>), grid, dim3(256), 0, stream, a); break;
+        case 64: hipLaunchKernelGGL((prefill_kernel<KIND, F16, 64, 4, RESUME, IQK>), grid, dim3(256), 0, stream, a); break;
         case 128:
             if (wide) {
-                hipLaunchKernelGGL((prefill_kernel<KIND, F16, 128, 8, RESUME>), grid, dim3(512), 0, stream, a);
+                hipLaunchKernelGGL((prefill_kernel<KIND, F16, 128, 8, RESUME, IQK>), grid, dim3(512), 0, stream, a);
             } else {
-                hipLaunchKernelGGL((prefill_kernel<KIND, F16, 128, 4, RESUME>), grid, dim3(256), 0, stream, a);
+                hipLaunchKernelGGL((prefill_kernel<KIND, F16, 128, 4, RESUME, IQK>), grid, dim3(256), 0, stream, a);
             }
             break;
         default: return CRIT_PKV_E_GEOMETRY;
@@ -595,7 +664,9 @@ static int launch_one(PrefillArgs a, int kind, bool f16, int head_dim, int kv_he
             return f16 ? launch_d<0, true>(a, head_dim, wide, grid, stream) : launch_d<0, false>(a, head_dim, wide, grid, stream);
         case 1: return launch_d<1, false>(a, head_dim, wide, grid, stream);
         case 2: return launch_d<2, false>(a, head_dim, wide, grid, stream);
-        case 3: return launch_d<3, false>(a, head_dim, wide, grid, stream);
+        case 3:
+            if (a.iqk) return launch_d<3, false, false, true>(a, head_dim, wide, grid, stream);
+            return launch_d<3, false>(a, head_dim, wide, grid, stream);
     }
     return CRIT_PKV_E_DTYPE;
 }
@@ -605,6 +676,7 @@ int launch_prefill(const crit_pkv_prefill_params* p, hipStream_t stream) {
     if ((p->tables == nullptr) == (p->tables64 == nullptr)) return CRIT_PKV_E_NULL;
     if (p->kind < 0 || p->kind > 3) return CRIT_PKV_E_DTYPE;
     if (p->kind >= 2 && (!p->key_scales || !p->value_scales)) return CRIT_PKV_E_NULL;
+    if (p->int8_qk && p->kind != 3) return CRIT_PKV_E_DTYPE;
     const bool f16 = p->page_dtype == CRIT_PKV_F16;
     if (f16 && p->kind != 0) return CRIT_PKV_E_DTYPE;
     if (p->out_dtype != CRIT_PKV_F32 && p->out_dtype != CRIT_PKV_BF16 && p->out_dtype != CRIT_PKV_F16) return CRIT_PKV_E_DTYPE;
@@ -646,6 +718,7 @@ int launch_prefill(const crit_pkv_prefill_params* p, hipStream_t stream) {
     a.sliding = p->sliding, a.out_dtype = p->out_dtype;
     a.sscale = p->scale * kLog2e, a.k_mult = p->key_multiplier, a.v_mult = p->value_multiplier;
     a.firsts = nullptr, a.state = nullptr, a.mode = 0;
+    a.iqk = p->int8_qk != 0;
     a.k_slot_bytes = a.v_slot_bytes = (uint32_t)p->kv_heads * p->head_dim * (p->kind == 0 ? 2 : 1);
     a.tiles = 0;
     if (!fresh) return launch_one(a, p->kind, f16, p->head_dim, p->kv_heads, p->chunks, p->max_count, stream);
@@ -660,6 +733,7 @@ int launch_prefill(const crit_pkv_prefill_params* p, hipStream_t stream) {
     a.ks = a.vs = a.hm = nullptr;
     a.k_mult = a.v_mult = 1.0f;
     a.page = 1, a.page_l = 0, a.page_magic = 1;
+    a.iqk = 0;      // (fresh rows are multiplied in q's type, as the reference's are)
     return launch_one(a, 0, f16, p->head_dim, p->kv_heads, p->chunks, p->max_count, stream);
 }
 

@@ -33,6 +33,7 @@ struct PrefillArgs {
     const int64_t* firsts;   // [chunks], or null: the chunk's position (all of its own positions are fresh)
     float* state;            // [token][head][kStateRow] FP32
     int mode;
+    int iqk;                 // INT8 pages: integer scores from INT8 query codes (the reference's int8_qk)
     uint32_t k_slot_bytes, v_slot_bytes;     // bytes from one slot's (or fresh row's) K / V row to the next
 };
 constexpr int kStatePad = 4;      // a row of the state is head_dim + 4 floats: the output, the maximum, the sum, 16-byte rows

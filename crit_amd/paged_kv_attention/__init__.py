@@ -504,8 +504,10 @@ def _check_fresh(fresh, q, hkv, d, chunks):
 
 def _prefill_launch(q, key_pages, value_pages, kind, tables, table_rows, starts, counts, positions, max_count, chunks,
                     page, key_scales, value_scales, multipliers, scale, out, lse, sinks, sliding, fresh=None,
-                    workspace=None):
+                    workspace=None, int8_qk=False):
     k_kind = _check_kind(kind, key_scales)
+    if int8_qk and k_kind != 3:
+        raise ValueError("int8_qk multiplies INT8 queries with INT8 keys: int8 pages only")
     _require_device(q, "prefill's q")
     T, hq, d = q.shape
     hkv = key_pages.shape[-2]
@@ -542,6 +544,7 @@ def _prefill_launch(q, key_pages, value_pages, kind, tables, table_rows, starts,
     p.sliding = sliding
     p.scale = float(scale if scale is not None else d ** -0.5)
     p.key_multiplier, p.value_multiplier = km, vm
+    p.int8_qk = int(bool(int8_qk))
     if fresh is not None:
         fk, fv, firsts = _check_fresh(fresh, q, hkv, d, chunks)
         state = _prefill_state(device, T, hq, d, workspace)
@@ -566,11 +569,12 @@ def prefill(q, key_pages, value_pages, kind, table, position, page, *, key_scale
     all of them; an int or a one-element int64 device tensor, clamped to the chunk's positions) from them, unscaled,
     and the earlier ones from the pages: two launches (the pages' positions, then the fresh rows) that hand the rows'
     states through `workspace` (FP32, prefill_state_floats(T, heads, dim); default: one the module keeps per device,
-    grown outside a capture); a token's bits follow its own positions and `first`. int8_qk and derive are not served."""
+    grown outside a capture); a token's bits follow its own positions and `first`. int8_qk (INT8 pages): each query
+    row rounded to INT8 codes at its own scale (amax / 127, half away from zero) and the scores taken as exact integer
+    products of the codes on the matrix cores (v_mfma_i32_32x32x32_i8) times the row's and the keys' scales; fresh rows
+    are still read in q's type. derive is not served."""
     if derive is not None:
         raise _unsupported("derive= (keys derived from value rows)")
-    if int8_qk:
-        raise _unsupported("int8_qk")
     _check_sinks(sinks, q)
     sliding = _check_sliding(sliding, None)
     T = q.shape[0]
@@ -598,12 +602,12 @@ def prefill(q, key_pages, value_pages, kind, table, position, page, *, key_scale
         fresh = (fresh[0], fresh[1], first)
     return _prefill_launch(q, key_pages, value_pages, kind, table.reshape(1, -1), None, None, None, positions, T, 1,
                            page, key_scales, value_scales, multipliers, scale, out, lse, sinks, sliding, fresh,
-                           workspace)
+                           workspace, int8_qk)
 
 
 def prefill_rows(q, key_pages, value_pages, kind, tables, table_rows, starts, counts, positions, max_count, page, *,
                  key_scales=None, value_scales=None, multipliers=(1.0, 1.0), scale=None, out=None, lse=None,
-                 sinks=None, sliding=0, fresh=None, workspace=None):
+                 sinks=None, sliding=0, fresh=None, workspace=None, int8_qk=False):
     """Several prompt chunks in one launch (where the reference launches prefill() once per row): chunk i is counts[i]
     <= max_count tokens from token starts[i] of q at positions positions[i].. of the sequence whose page table is
     tables[table_rows[i]]; tables [S][width] int32, table_rows/starts/counts [chunks] int32, positions [chunks] int64,
@@ -621,7 +625,7 @@ def prefill_rows(q, key_pages, value_pages, kind, tables, table_rows, starts, co
         fresh = (fresh[0], fresh[1], fresh[2] if len(fresh) == 3 else None)
     return _prefill_launch(q, key_pages, value_pages, kind, tables, table_rows, starts, counts, positions,
                            int(max_count), chunks, page, key_scales, value_scales, multipliers, scale, out, lse, sinks,
-                           sliding, fresh, workspace)
+                           sliding, fresh, workspace, int8_qk)
 
 
 def stream_read(data, sink=None):

@@ -56,7 +56,7 @@ class PrefillParams(ctypes.Structure):
                 ("head_dim", _i32), ("page", _i32), ("kind", _i32), ("page_dtype", _i32), ("out_dtype", _i32),
                 ("sliding", _i32), ("scale", _f32), ("key_multiplier", _f32), ("value_multiplier", _f32),
                 ("fresh_keys", _p), ("fresh_values", _p), ("fresh_firsts", _p), ("fresh_state", _p),
-                ("fresh_stride_k", _i64), ("fresh_stride_v", _i64)]
+                ("fresh_stride_k", _i64), ("fresh_stride_v", _i64), ("int8_qk", _i32)]
 
 
 SYMBOLS = ("crit_pkv_write", "crit_pkv_attend", "crit_pkv_merge", "crit_pkv_prefill", "crit_pkv_abi_version",

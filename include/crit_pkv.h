@@ -181,6 +181,10 @@ typedef struct crit_pkv_prefill_params {
     const int64_t* fresh_firsts;
     float* fresh_state;
     int64_t fresh_stride_k, fresh_stride_v;
+    /* INT8 pages only (the reference's int8_qk, __init__.py:1245, _kernels.py:637-643, 668-671): each query row is
+     * rounded to INT8 codes at its own scale (amax / 127, half away from zero) and the scores are exact integer
+     * products of query and key codes times the two scales. Fresh rows, where given, are still read in q's type. */
+    int32_t int8_qk;
 } crit_pkv_prefill_params;
 
 int crit_pkv_prefill(const crit_pkv_prefill_params* p, void* stream);

@@ -88,17 +88,32 @@ def with_fresh(keys, values, fresh, q_dtype):
     return keys, values
 
 
+def int8_rows(q):
+    """Each query row [.., D] (FP32 values of the 16-bit queries) to INT8 codes at its own scale and back, in float64
+    (_kernels.py:637-643): scale = max(amax / 127, 1e-30) in FP32, codes = q / scale rounded half away from zero
+    (|code| <= 127). The scores of an int8_qk chunk are the exact products of these codes and the keys' codes times
+    both scales (_kernels.py:668-671), i.e. attention with the queries replaced by codes x scale."""
+    qf = q.float()
+    scale = (qf.abs().amax(-1, keepdim=True) / 127.0).clamp(min=1e-30)
+    x = qf / scale
+    codes = torch.where(x >= 0, x + 0.5, x - 0.5).trunc().clamp(-128, 127)
+    return codes.double() * scale.double()
+
+
 def window_reference(q, key_pages, value_pages, kind, table, first, count, page, scale, key_scales=None,
                      value_scales=None, multipliers=(1.0, 1.0), sliding=0, q_dtype=torch.bfloat16, parents=None,
-                     blocks=None, block_size=None, fresh=None):
+                     blocks=None, block_size=None, fresh=None, int8_qk=False):
     """One window row in float64: q [count][HQ][D] (rounded to q_dtype first, as the kernels read it) at positions
     first .. first + count - 1 -> (out [count][HQ][DV], lse [count][HQ]). parents: the row's draft tree (seen_by);
-    blocks [count][k] with block_size: each column's listed KV blocks (listed); fresh: with_fresh's tuple."""
+    blocks [count][k] with block_size: each column's listed KV blocks (listed); fresh: with_fresh's tuple; int8_qk: the
+    queries as int8_rows gives them (pages only: not with fresh)."""
     n = first + count
     keys, values = stored_rows(key_pages, value_pages, table, n, page, kind, key_scales, value_scales, multipliers)
     if fresh is not None:
         keys, values = with_fresh(keys, values, fresh, q_dtype)
     qd = q.to(q_dtype).double()
+    if int8_qk:
+        qd = int8_rows(q.to(q_dtype))
     outs, lses = [], []
     for c in range(count):
         seen = seen_by(first, count, c, n, parents, sliding)

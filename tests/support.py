@@ -63,7 +63,8 @@ class Cache:
         c = lambda t: None if t is None else t.cpu()
         return c(self.k), c(self.v), c(self.ks), c(self.vs), self.tables.cpu()
 
-    def want(self, q, s, first, count, scale=None, sliding=0, parents=None, blocks=None, block_size=None, fresh=None):
+    def want(self, q, s, first, count, scale=None, sliding=0, parents=None, blocks=None, block_size=None, fresh=None,
+             int8_qk=False):
         """The oracle's float64 (out, lse) of one window row over the STORED values."""
         k, v, ks, vs, tables = self.cpu()
         q_dtype = torch.float16 if self.kind == "fp16" else torch.bfloat16
@@ -73,7 +74,7 @@ class Cache:
         return oracle_attend.window_reference(q.cpu().float(), k, v, self.kind, tables[s], first, count, self.page,
                                               scale if scale is not None else self.d ** -0.5, ks, vs, m,
                                               sliding=sliding, q_dtype=q_dtype, parents=parents, blocks=blocks,
-                                              block_size=block_size, fresh=fresh)
+                                              block_size=block_size, fresh=fresh, int8_qk=int8_qk)
 
     def attend(self, q, rows, starts, firsts, columns, **kw):
         q_dtype = torch.float16 if self.kind == "fp16" else torch.bfloat16

@@ -284,15 +284,73 @@ def test_several_chunks_with_fresh_rows_equal_one_launch_each(kind):
             assert torch.equal(lse[rows], one_lse), s
 
 
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 128), (12, 2, 64)])
+def test_int8_queries_against_int8_keys(hq, hkv, d):
+    # int8_qk over INT8 pages: the scores are exact integer products of the query rows' INT8 codes (their own scale,
+    # amax / 127, half away from zero) and the keys' codes, times both scales: against the oracle with the queries
+    # rounded the same way, and within the reference's own bound of the launch that keeps the queries' 16 bits
+    # (0.06, test_paged_kv_attention.py:476-479); with a negative scale, a sliding window and sinks; with fresh rows
+    # (read in q's type after the pages' integer scores).
+    pk = kernels()
+    cache = Cache("int8", hkv, d, d, 16, [500], seed=41)
+    q = rand_q(150, hq, d, 42)
+    kw = dict(key_scales=cache.ks, value_scales=cache.vs)
+    lse = torch.empty(150, hq, device=dev)
+    out = pk.prefill(q.bfloat16(), cache.k, cache.v, "int8", cache.tables[0], 350, 16, int8_qk=True, lse=lse, **kw)
+    exact = pk.prefill(q.bfloat16(), cache.k, cache.v, "int8", cache.tables[0], 350, 16, **kw)
+    assert float((out.float() - exact.float()).abs().max()) < 0.06
+    for t in (0, 63, 64, 149):
+        want, want_lse = cache.want(q[t:t + 1], 0, 350 + t, 1, int8_qk=True)
+        torch.testing.assert_close(out[t:t + 1].double().cpu(), want, atol=ATOL, rtol=RTOL, msg=f"token {t}")
+        torch.testing.assert_close(lse[t:t + 1].double().cpu(), want_lse, atol=1e-3, rtol=1e-4, msg=f"lse {t}")
+    sinks = torch.linspace(-1, 1, hq, device=dev)
+    out = pk.prefill(q.bfloat16(), cache.k, cache.v, "int8", cache.tables[0], 350, 16, int8_qk=True, scale=-0.11,
+                     sliding=70, lse=lse, **kw)
+    for t in (0, 100):
+        want, want_lse = cache.want(q[t:t + 1], 0, 350 + t, 1, int8_qk=True, scale=-0.11, sliding=70)
+        torch.testing.assert_close(out[t:t + 1].double().cpu(), want, atol=ATOL, rtol=RTOL, msg=f"negative scale, token {t}")
+        torch.testing.assert_close(lse[t:t + 1].double().cpu(), want_lse, atol=2e-3, rtol=1e-4)
+    with_sinks = pk.prefill(q.bfloat16(), cache.k, cache.v, "int8", cache.tables[0], 350, 16, int8_qk=True, scale=-0.11,
+                            sliding=70, sinks=sinks, **kw)
+    weight = torch.exp(lse) / (torch.exp(lse) + torch.exp(sinks)[None, :])
+    torch.testing.assert_close(with_sinks.float(), out.float() * weight[..., None], atol=8e-3, rtol=2e-2)
+    # the chunk's own positions fresh: the pages' part in integers, the fresh part in 16 bits; with every position
+    # fresh nothing is left of the integers and the launch equals the one without int8_qk
+    fk, fv = _fresh_rows(150, hkv, d, 43, torch.bfloat16)
+    mixed = pk.prefill(q.bfloat16(), cache.k, cache.v, "int8", cache.tables[0], 350, 16, int8_qk=True, fresh=(fk, fv), **kw)
+    plain = pk.prefill(q.bfloat16(), cache.k, cache.v, "int8", cache.tables[0], 350, 16, fresh=(fk, fv), **kw)
+    assert float((mixed.float() - plain.float()).abs().max()) < 0.06
+    first = pk.prefill(q.bfloat16(), cache.k, cache.v, "int8", cache.tables[0], 0, 16, int8_qk=True, fresh=(fk, fv), **kw)
+    assert torch.equal(first, pk.prefill(q.bfloat16(), cache.k, cache.v, "int8", cache.tables[0], 0, 16, fresh=(fk, fv), **kw))
+
+
+def test_int8_queries_in_a_launch_that_fills_the_chip_equal_one_launch_per_chunk():
+    pk = kernels()
+    counts = [256, 255, 256, 129, 256, 1, 200, 256]
+    prefixes = [0, 7, 64, 500, 1023, 1100, 63, 128]
+    cache = Cache("int8", 8, 128, 128, 16, [p + c for p, c in zip(prefixes, counts)], seed=47, scale=0.5)
+    starts = [sum(counts[:i]) for i in range(8)]
+    q = rand_q(sum(counts), 32, 128, 48).bfloat16()
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    positions = torch.tensor(prefixes, dtype=torch.int64, device=dev)
+    kw = dict(key_scales=cache.ks, value_scales=cache.vs, int8_qk=True)
+    out = pk.prefill_rows(q, cache.k, cache.v, "int8", cache.tables, i32(list(range(8))), i32(starts), i32(counts),
+                          positions, 256, 16, **kw)
+    for s in range(8):
+        rows = slice(starts[s], starts[s] + counts[s])
+        assert torch.equal(out[rows], pk.prefill(q[rows], cache.k, cache.v, "int8", cache.tables[s], prefixes[s], 16, **kw)), s
+
+
 def test_what_the_prompt_reader_does_not_take_is_refused():
     pk = kernels()
     cache = Cache("int8", 2, 128, 128, 16, [40])
     q = rand_q(4, 8, 128, 2).bfloat16()
     kw = dict(key_scales=cache.ks, value_scales=cache.vs)
     with pytest.raises(NotImplementedError):
-        pk.prefill(q, cache.k, cache.v, "int8", cache.tables[0], 36, 16, int8_qk=True, **kw)
-    with pytest.raises(NotImplementedError):
         pk.prefill(q, cache.k, cache.v, "int8", cache.tables[0], 36, 16, derive=(None, 1e-6, None, 0), **kw)
+    row = Cache("fp8:row", 2, 128, 128, 16, [40])
+    with pytest.raises(ValueError):      # INT8 queries against INT8 keys only
+        pk.prefill(q, row.k, row.v, "fp8:row", row.tables[0], 36, 16, int8_qk=True, key_scales=row.ks, value_scales=row.vs)
     with pytest.raises(ValueError):
         pk.prefill(q.float(), cache.k, cache.v, "int8", cache.tables[0], 36, 16, **kw)
 

@@ -456,3 +456,28 @@ def test_fresh_rows_replace_the_positions_from_their_first_on_unscaled():
                                            fresh=(fk, fv, 0, 0))
     assert torch.allclose(one[0], fv[0, 0].double().expand(2, 16), atol=1e-12)
     assert torch.allclose(one_lse[0], (q[0].bfloat16().double() @ fk[0, 0].double()) * 0.25, atol=1e-12)
+
+
+def test_int8_query_rows_are_their_codes_times_their_scale():
+    # Pins int8_rows(): known answers (amax maps to +-127; halves round away from zero; a zero row stays zero at the
+    # floor scale), the closed form codes = round_half_away(q * 127 / amax) on random rows, |codes| <= 127, an error of
+    # at most half a step, and its use in window_reference(): the same as attending with the rounded queries.
+    q = torch.tensor([[127.0, -127.0, 63.5, -63.5, 0.4, -0.6, 0.0, 1.0], [0.0] * 8, [2.0, 1.0, 0.5, 0.25, -2.0, 0.0, 0.0, 0.0]])
+    got = attend.int8_rows(q)
+    assert got[0].tolist() == [127.0, -127.0, 64.0, -64.0, 0.0, -1.0, 0.0, 1.0]
+    assert got[1].tolist() == [0.0] * 8
+    step = 2.0 / 127.0
+    assert torch.allclose(got[2], torch.tensor([127, 64, 32, 16, -127, 0, 0, 0], dtype=torch.float64) * float(torch.tensor(step)), atol=1e-12)
+    x = torch.randn(64, 128, generator=torch.Generator().manual_seed(3)).bfloat16().float()
+    amax = x.abs().amax(-1, keepdim=True)
+    scale = (amax / 127.0).double()
+    codes = attend.int8_rows(x) / scale
+    assert bool((codes == codes.round()).all()) and float(codes.abs().max()) <= 127
+    assert float((attend.int8_rows(x) - x.double()).abs().max() / scale.max()) <= 0.5 + 1e-6
+    k, v, ks, vs, tables, _ = _pool("int8", 1, 16, 16, 16, [60])
+    q = torch.randn(3, 2, 16, generator=torch.Generator().manual_seed(4))
+    out, lse = attend.window_reference(q, k, v, "int8", tables[0], 57, 3, 16, 0.25, ks, vs, int8_qk=True)
+    keys, values = attend.stored_rows(k, v, tables[0], 60, 16, "int8", ks, vs)
+    for c in range(3):
+        want, want_lse = attend.reference(attend.int8_rows(q[c].bfloat16()), keys, values, torch.arange(60) <= 57 + c, 0.25)
+        assert torch.allclose(out[c], want, atol=1e-12) and torch.allclose(lse[c], want_lse, atol=1e-12)
