@@ -328,6 +328,50 @@ def mixed_prefill(pk, device):
             "decode_us": round(t_decode * 1e3, 1), "step_us": round(step * 1e3, 1)}
 
 
+def prefill_by_kind(pk, device):
+    """The mixed batch's 8 prompt chunks (512 tokens each on prefixes in [0, 8192]) over pages of every 8-bit kind,
+    and over INT8 pages with int8_qk (integer scores)."""
+    hq, hkv, d, page = 32, 8, 128, 16
+    gcpu = torch.Generator().manual_seed(5)
+    prefixes = torch.randint(0, 8193, (8,), generator=gcpu).tolist()
+    widths = [(p + 512 + page - 1) // page for p in prefixes]
+    n_pages = int(sum(widths) * 1.25)
+    perm = torch.randperm(n_pages, generator=gcpu)
+    tables = torch.full((8, (max(widths) + 15) // 16 * 16), n_pages, dtype=torch.int32)
+    at = 0
+    for s, w in enumerate(widths):
+        tables[s, :w] = perm[at:at + w].to(torch.int32)
+        at += w
+    tables = tables.to(device)
+    g = torch.Generator(device=device).manual_seed(9)
+    q = torch.randn(4096, hq, d, device=device, generator=g).to(torch.bfloat16)
+    out = torch.empty_like(q)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=device)
+    rows, starts, counts = i32(list(range(8))), i32([512 * s for s in range(8)]), i32([512] * 8)
+    positions = torch.tensor(prefixes, dtype=torch.int64, device=device)
+    flops = sum(4 * hq * d * sum(p + t + 1 for t in range(512)) for p in prefixes)
+    found = {}
+    for kind in ("fp8", "fp8:row", "int8"):
+        store = torch.int8 if kind == "int8" else torch.float8_e4m3fn
+        kf = torch.randn(n_pages + 1, page, hkv, d, device=device, generator=g)
+        vf = torch.randn(n_pages + 1, page, hkv, d, device=device, generator=g)
+        ks = vs = None
+        if kind == "fp8":
+            k, v = (kf / 0.02).clamp(-448, 448).to(store), (vf / 0.02).clamp(-448, 448).to(store)
+        else:
+            top = 448.0 if kind == "fp8:row" else 127.0
+            ks, vs = kf.abs().amax(-1) / top, vf.abs().amax(-1) / top
+            k, v = kf / ks[..., None], vf / vs[..., None]
+            k, v = (k.round().to(store), v.round().to(store)) if kind == "int8" else (k.to(store), v.to(store))
+        del kf, vf
+        for iqk in ((False, True) if kind == "int8" else (False,)):
+            call = lambda: pk.prefill_rows(q, k, v, kind, tables, rows, starts, counts, positions, 512, page,
+                                           key_scales=ks, value_scales=vs, multipliers=(0.02, 0.02), out=out, int8_qk=iqk)
+            t = timed(call, 10, 2)
+            found[kind + (" int8_qk" if iqk else "")] = {"us": round(t * 1e3, 1), "TFLOP/s": round(flops / t / 1e9, 1)}
+    return found
+
+
 def prefill_fresh(pk, device):
     """The mixed batch's 8 prompt chunks over FP8 pages (one multiplier pair), once reading every position from the
     pages and once with fresh=: each chunk's own 512 positions from 16-bit rows as the projections gave them, its
@@ -479,6 +523,8 @@ def main():
         log(f"[bench] block-sparse decode: {extras['block_sparse_decode_bf16']}")
         extras["mixed_prefill_decode_bf16"] = mixed_prefill(pk, device)
         log(f"[bench] mixed prefill + decode: {extras['mixed_prefill_decode_bf16']}")
+        extras["prefill_8bit_pages"] = prefill_by_kind(pk, device)
+        log(f"[bench] prefill over 8-bit pages: {extras['prefill_8bit_pages']}")
         extras["prefill_fp8_pages_fresh_rows"] = prefill_fresh(pk, device)
         log(f"[bench] prefill over FP8 pages, with fresh rows: {extras['prefill_fp8_pages_fresh_rows']}")
         result["extra"] = extras
