@@ -533,15 +533,25 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
     // Blocks wholly visible to every row of the workgroup first (none under a sliding window), then the masked ones.
     int kt_full = win > 0 ? kt_lo : max(kt_lo, min(kt_hi + 1, (pos + t_lo + 1) / BN));
     if (a.mode == 1) kt_full = max(kt_lo, min(kt_full, first / BN));      // blocks wholly below the first fresh position
-    if (RESUME) kt_full = kt_lo;
+    // A resuming launch's first block may begin below the first fresh position: blocks up to kt_lead take the mask too.
+    int kt_lead = kt_lo;
+    if (RESUME && win == 0) kt_lead = min(max(kt_lo, (first + BN - 1) / BN), kt_hi + 1);
+    kt_full = max(kt_full, kt_lead);
     if (!any_block) {
         // no position of this launch for these rows: the state passes through
     } else if constexpr (WAVES == 4) {
-        for (int kt = kt_lo; kt < kt_full; ++kt) {
+        int kt = kt_lo;
+        if constexpr (RESUME) {
+            for (; kt < kt_lead; ++kt) {
+                scores(kt, (kt & 1) ^ 1), weigh(kt, kt & 1, c1), values(kt, kt & 1);
+                __syncthreads();
+            }
+        }
+        for (; kt < kt_full; ++kt) {
             scores(kt, (kt & 1) ^ 1), weigh(kt, kt & 1, c0), values(kt, kt & 1);
             __syncthreads();          // every wavefront is done with this buffer; the other one is stored
         }
-        for (int kt = kt_full; kt <= kt_hi; ++kt) {
+        for (; kt <= kt_hi; ++kt) {
             scores(kt, (kt & 1) ^ 1), weigh(kt, kt & 1, c1), values(kt, kt & 1);
             __syncthreads();
         }
@@ -556,28 +566,42 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
         auto after = [](int b) { return b == 2 ? 0 : b + 1; };
         const bool behind = __builtin_amdgcn_readfirstlane(wave >> 2) != 0;
         if (!behind) {
-            int vcur = 0;
-            for (int kt = kt_lo; kt < kt_full; ++kt) {
+            int vcur = 0, kt = kt_lo;
+            if constexpr (RESUME) {
+                for (; kt < kt_lead; ++kt) {
+                    scores(kt, after(vcur)), weigh(kt, vcur, c1), values(kt, vcur);
+                    __syncthreads();
+                    vcur = after(vcur);
+                }
+            }
+            for (; kt < kt_full; ++kt) {
                 scores(kt, after(vcur)), weigh(kt, vcur, c0), values(kt, vcur);
                 __syncthreads();
                 vcur = after(vcur);
             }
-            for (int kt = kt_full; kt <= kt_hi; ++kt) {
+            for (; kt <= kt_hi; ++kt) {
                 scores(kt, after(vcur)), weigh(kt, vcur, c1), values(kt, vcur);
                 __syncthreads();
                 vcur = after(vcur);
             }
         } else {
+            // iteration kt weighs block kt - 1: masked while that block is below kt_lead or from kt_full on
             scores(kt_lo, 1);
             __syncthreads();
-            int vprev = 0, vcur = 1;
-            const int kt_mid = min(kt_full, kt_hi);      // iterations up to here weigh a wholly visible block (kt - 1)
-            for (int kt = kt_lo + 1; kt <= kt_mid; ++kt) {
+            int vprev = 0, vcur = 1, kt = kt_lo + 1;
+            if constexpr (RESUME) {
+                for (; kt <= min(kt_lead, kt_hi); ++kt) {
+                    weigh(kt - 1, vprev, c1), values(kt - 1, vprev), scores(kt, after(vcur));
+                    __syncthreads();
+                    vprev = vcur, vcur = after(vcur);
+                }
+            }
+            for (; kt <= min(kt_full, kt_hi); ++kt) {
                 weigh(kt - 1, vprev, c0), values(kt - 1, vprev), scores(kt, after(vcur));
                 __syncthreads();
                 vprev = vcur, vcur = after(vcur);
             }
-            for (int kt = max(kt_lo, kt_mid) + 1; kt <= kt_hi; ++kt) {
+            for (; kt <= kt_hi; ++kt) {
                 weigh(kt - 1, vprev, c1), values(kt - 1, vprev), scores(kt, after(vcur));
                 __syncthreads();
                 vprev = vcur, vcur = after(vcur);
@@ -636,9 +660,13 @@ static int launch_d(const PrefillArgs& a, int d, bool wide, dim3 grid, hipStream
     switch (d) {
         case 64: hipLaunchKernelGGL((prefill_kernel<KIND, F16, 64, 4, RESUME, IQK>), grid, dim3(256), 0, stream, a); break;
         case 128:
-            if (wide) {
-                hipLaunchKernelGGL((prefill_kernel<KIND, F16, 128, 8, RESUME, IQK>), grid, dim3(512), 0, stream, a);
-            } else {
+            if constexpr (!RESUME) {
+                if (wide) {
+                    hipLaunchKernelGGL((prefill_kernel<KIND, F16, 128, 8, RESUME, IQK>), grid, dim3(512), 0, stream, a);
+                    break;
+                }
+            }
+            {
                 hipLaunchKernelGGL((prefill_kernel<KIND, F16, 128, 4, RESUME, IQK>), grid, dim3(256), 0, stream, a);
             }
             break;
@@ -653,7 +681,9 @@ static int launch_one(PrefillArgs a, int kind, bool f16, int head_dim, int kv_he
     // launch still has a workgroup or more for every compute unit.
     const int64_t groups8 = ((int64_t)kv_heads * chunks + 7) / 8;
     int64_t tiles = ((int64_t)max_count * a.g + 2 * BM - 1) / (2 * BM);
-    const bool wide = head_dim == 128 && tiles * kv_heads * chunks >= compute_units();
+    // (The launch that resumes rows over their fresh positions is short and takes the four-wavefront shape: with its
+    // three loops per wavefront group the eight-wavefront one spills.)
+    const bool wide = head_dim == 128 && a.mode != 2 && tiles * kv_heads * chunks >= compute_units();
     if (!wide) tiles = ((int64_t)max_count * a.g + BM - 1) / BM;
     if (tiles * groups8 * 8 > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
     a.tiles = (int)tiles;
