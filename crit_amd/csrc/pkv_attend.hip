@@ -14,6 +14,9 @@ int launch_attend_fp8row(const AttendArgs& a, int lpr, int qr, bool fused, bool 
 int launch_attend_int8(const AttendArgs& a, int lpr, int qr, bool fused, bool page16, dim3 grid, hipStream_t stream);
 
 // One wavefront per (column, head, row): folds the partitions that hold the column's positions, in order.
+// Lane `at`'s value of x (at: the same in every lane).
+PKV_DEV float lane_value(float x, int at) { return u2f((uint32_t)__builtin_amdgcn_readlane((int)f2u(x), at)); }
+
 template <int DV>
 __global__ __launch_bounds__(64) void merge_kernel(AttendArgs a) {
     constexpr int EPL = DV / 64;
@@ -32,33 +35,90 @@ __global__ __launch_bounds__(64) void merge_kernel(AttendArgs a) {
     float M = -INFINITY, L = 0.0f, A[EPL];
 #pragma unroll
     for (int e = 0; e < EPL; ++e) A[e] = 0.0f;
-    // Folded strictly in partition order (the fused launch folds the same way), but loaded U partitions at a time so
-    // the loads of a long row's hundreds of partials overlap instead of chaining their latencies: 8 at a time for the
-    // few partitions of an ordinary decode row, 32 at a time beyond that.
-    auto fold_from = [&](int b_lo, auto uc) __attribute__((always_inline)) {
-        constexpr int U = decltype(uc)::value;
-        for (int b0 = b_lo; b0 < nb; b0 += U) {
-            float pm[U], pl[U], po[U][EPL];
+    // Folded strictly in partition order (the fused launch folds the same way: fold()). Few partitions (an ordinary
+    // decode row): their states loaded 8 at a time so the loads overlap, then folded one by one.
+    if (nb <= 8) {
+        float pm[8], pl[8], po[8][EPL];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int b = u < nb ? u : nb - 1;
+            pm[u] = a.pm[at + b], pl[u] = a.pl[at + b];
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) po[u][e] = a.po[(at + b) * DV + e * 64 + lane];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            if (u < nb) {
+                const Fold f = fold(M, L, pm[u], pl[u]);
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) A[e] = __builtin_fmaf(A[e], f.keep, po[u][e] * f.take);
+                M = f.m, L = f.l;
+            }
+        }
+    } else {
+        // Many partitions (a long row's hundreds): a fold's maximum, its two exponentials and the product l * take
+        // depend only on the maxima before it, so a batch of U partitions takes them on U lanes at once, the same
+        // operations on the same values as fold() one by one: the running maximum as a prefix maximum over the lanes
+        // (exact in any order), then keep, take and l * take a lane each. What stays in order is one fused
+        // multiply-add for the sum and one multiply and one fused multiply-add a value dim, their factors read from
+        // the lane that holds them. The next batch's states are loaded while this one is folded.
+        constexpr int U = EPL > 2 ? 16 : 32;
+        float po[2][U][EPL], pm_next, pl_next;
+        auto load_scalars = [&](int b0) __attribute__((always_inline)) {
+            const int b = min(b0 + (lane & (U - 1)), nb - 1);
+            pm_next = a.pm[at + b], pl_next = a.pl[at + b];
+        };
+        auto load_values = [&](int b0, float (&dst)[U][EPL]) __attribute__((always_inline)) {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const int b = b0 + u < nb ? b0 + u : nb - 1;
-                pm[u] = a.pm[at + b], pl[u] = a.pl[at + b];
+                const int b = min(b0 + u, nb - 1);
 #pragma unroll
-                for (int e = 0; e < EPL; ++e) po[u][e] = a.po[(at + b) * DV + e * 64 + lane];
+                for (int e = 0; e < EPL; ++e) dst[u][e] = a.po[(at + b) * DV + e * 64 + lane];
             }
+        };
+        auto fold_batch = [&](int b0, float pm, float pl, const float (&val)[U][EPL]) __attribute__((always_inline)) {
+            const int u_lane = lane & (U - 1);
+            if (b0 + u_lane >= nb) pm = -INFINITY, pl = 0.0f;      // (lanes past the last partition are not folded below)
+            float upto = pm;      // the maximum of this batch's partitions up to the lane's
+#pragma unroll
+            for (int o = 1; o < U; o <<= 1) {
+                const float other = __shfl_up(upto, o, U);
+                if (u_lane >= o) upto = __builtin_fmaxf(upto, other);
+            }
+            const float m_new = __builtin_fmaxf(M, upto);
+            float m_old = __shfl_up(m_new, 1, U);
+            if (u_lane == 0) m_old = M;
+            const float sub = m_new == -INFINITY ? 0.0f : m_new;
+            const float keep = exp2_fast(m_old - sub), take = exp2_fast(pm - sub);
+            const float l_take = pl * take;
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 if (b0 + u < nb) {
-                    const Fold f = fold(M, L, pm[u], pl[u]);
+                    const float k_u = lane_value(keep, u), t_u = lane_value(take, u);
+                    L = __builtin_fmaf(L, k_u, lane_value(l_take, u));
 #pragma unroll
-                    for (int e = 0; e < EPL; ++e) A[e] = __builtin_fmaf(A[e], f.keep, po[u][e] * f.take);
-                    M = f.m, L = f.l;
+                    for (int e = 0; e < EPL; ++e) A[e] = __builtin_fmaf(A[e], k_u, val[u][e] * t_u);
                 }
             }
+            M = lane_value(m_new, min(nb - b0, U) - 1);
+        };
+        load_scalars(0);
+        load_values(0, po[0]);
+        for (int b0 = 0;;) {
+            float pm = pm_next, pl = pl_next;
+            load_scalars(b0 + U);      // (past the last partition the loads repeat it and are not folded)
+            load_values(b0 + U, po[1]);
+            fold_batch(b0, pm, pl, po[0]);
+            b0 += U;
+            if (b0 >= nb) break;
+            pm = pm_next, pl = pl_next;
+            load_scalars(b0 + U);
+            load_values(b0 + U, po[0]);
+            fold_batch(b0, pm, pl, po[1]);
+            b0 += U;
+            if (b0 >= nb) break;
         }
-    };
-    if (nb <= 8) fold_from(0, std::integral_constant<int, 8>{});
-    else fold_from(0, std::integral_constant<int, 32>{});
+    }
     if (a.sinks) {
         const Fold f = fold(M, L, a.sinks[head] * kLog2e, 1.0f);
 #pragma unroll

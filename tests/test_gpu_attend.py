@@ -143,6 +143,31 @@ def test_a_fused_launch_gives_a_column_the_split_launchs_bits(kind, hq, hkv, d):
         _close_lse(lse[:3], want_lse)
 
 
+@pytest.mark.parametrize("kind,hq,hkv,d", [("bf16", 8, 2, 128), ("fp8", 24, 4, 256), ("bf16", 8, 2, 64)])
+def test_a_row_of_many_partitions_merges_to_the_fused_launchs_bits(kind, hq, hkv, d):
+    # Long rows cut into many partitions (the long-context split): the merge takes the maxima and exponentials of a
+    # batch of partitions on as many lanes and keeps only the sums in order; the fused launch folds one partition
+    # after another. The same bits for 9 partitions (the first count past the one-by-one merge), one batch exactly,
+    # a few batches with a ragged last one, a count no row fills; with sinks; and the oracle.
+    pk = kernels()
+    block = pk.flash_block(d, d, hq, hkv, 16, kind)
+    cache = Cache(kind, hkv, d, d, 16, [40 * block * 5 + 7], seed=51)
+    n = cache.lengths[0] if hasattr(cache, "lengths") else 40 * block * 5 + 7
+    q = rand_q(3, hq, d, 52)
+    sinks = torch.linspace(-1, 1, hq, device=dev)
+    for parts, piece in ((9, block * 23), (32, block * 6), (16, block * 6), (77, block * 2), (500, block)):
+        lse, fused_lse = torch.empty(3, hq, device=dev), torch.empty(3, hq, device=dev)
+        split = cache.attend(q, [0], [0], [n - 3], 3, partitions=parts, piece=piece, lse=lse)
+        fused = cache.attend(q, [0], [0], [n - 3], 3, partitions=parts, piece=piece, lse=fused_lse, fused=True)
+        assert torch.equal(split, fused), (parts, piece)
+        assert torch.equal(lse, fused_lse), (parts, piece)
+        want, want_lse = cache.want(q, 0, n - 3, 3)
+        _close(split, want)
+        _close_lse(lse, want_lse)
+        assert torch.equal(cache.attend(q, [0], [0], [n - 3], 3, partitions=parts, piece=piece, sinks=sinks),
+                           cache.attend(q, [0], [0], [n - 3], 3, partitions=parts, piece=piece, sinks=sinks, fused=True))
+
+
 def test_a_given_workspace_holds_the_partials_and_a_small_one_is_refused():
     pk = kernels()
     cache = Cache("bf16", 2, 128, 128, 16, [300])
