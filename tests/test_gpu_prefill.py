@@ -140,6 +140,27 @@ def test_launches_that_fill_the_chip_equal_one_launch_per_chunk(kind, window):
             torch.testing.assert_close(lse[row:row + 1].double().cpu(), want_lse, atol=1e-3, rtol=1e-4, msg=f"lse {s} {t}")
 
 
+def test_a_group_of_five_query_heads_in_a_launch_that_fills_the_chip():
+    # 40 query heads on 8 KV heads: a token's five rows straddle the 256-row tiles' edges (256 is no multiple of 5).
+    pk = kernels()
+    counts, prefixes = [256, 200, 256, 77, 256, 256, 13, 256], [0, 70, 64, 900, 511, 1100, 63, 128]
+    cache = Cache("bf16", 8, 128, 128, 16, [p + c for p, c in zip(prefixes, counts)], seed=61, scale=0.5)
+    starts = [sum(counts[:i]) for i in range(8)]
+    q32 = rand_q(sum(counts), 40, 128, 62)
+    q = q32.bfloat16()
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    positions = torch.tensor(prefixes, dtype=torch.int64, device=dev)
+    out = pk.prefill_rows(q, cache.k, cache.v, "bf16", cache.tables, i32(list(range(8))), i32(starts), i32(counts),
+                          positions, 256, 16)
+    for s in range(8):
+        rows = slice(starts[s], starts[s] + counts[s])
+        assert torch.equal(out[rows], pk.prefill(q[rows], cache.k, cache.v, "bf16", cache.tables[s], prefixes[s], 16)), s
+    for s, t in ((0, 51), (3, 76), (5, 255)):
+        row = starts[s] + t
+        want, _ = cache.want(q32[row:row + 1], s, prefixes[s] + t, 1)
+        torch.testing.assert_close(out[row:row + 1].double().cpu(), want, atol=ATOL, rtol=RTOL, msg=f"chunk {s} token {t}")
+
+
 def test_prefill_agrees_with_the_decode_reader_within_the_readers_rounding():
     pk = kernels()
     cache = Cache("bf16", 2, 128, 128, 16, [400])
