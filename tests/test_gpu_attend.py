@@ -166,6 +166,12 @@ def test_a_row_of_many_partitions_merges_to_the_fused_launchs_bits(kind, hq, hkv
         _close_lse(lse, want_lse)
         assert torch.equal(cache.attend(q, [0], [0], [n - 3], 3, partitions=parts, piece=piece, sinks=sinks),
                            cache.attend(q, [0], [0], [n - 3], 3, partitions=parts, piece=piece, sinks=sinks, fused=True))
+        # a sliding window that leaves most partitions without a visible position (empty states between live ones)
+        window = 5 * block + 3
+        slid = cache.attend(q, [0], [0], [n - 3], 3, partitions=parts, piece=piece, sliding=window)
+        assert torch.equal(slid, cache.attend(q, [0], [0], [n - 3], 3, partitions=parts, piece=piece, sliding=window, fused=True))
+        want, _ = cache.want(q, 0, n - 3, 3, sliding=window)
+        _close(slid, want)
 
 
 def test_a_given_workspace_holds_the_partials_and_a_small_one_is_refused():
