@@ -284,6 +284,15 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
             return CRIT_PKV_E_GEOMETRY;
     }
     if ((p->parents || p->parents64) && p->columns > 64) return CRIT_PKV_E_GEOMETRY;      // an ancestor set is a 64-bit mask
+    const bool fresh = p->fresh_keys != nullptr || p->fresh_values != nullptr;
+    if (fresh) {
+        if (!p->fresh_keys || !p->fresh_values || !p->fresh_shifts || !p->fresh_firsts) return CRIT_PKV_E_NULL;
+        if (p->blocks) return CRIT_PKV_E_GEOMETRY;      // (block lists read the pages only, as the reference's)
+        const int64_t row = (int64_t)p->kv_heads * p->head_dim;
+        if (p->fresh_rows < 1 || p->fresh_stride_k < row || p->fresh_stride_v < row || p->fresh_stride_k % 8 || p->fresh_stride_v % 8 ||
+            (reinterpret_cast<uintptr_t>(p->fresh_keys) % 16) || (reinterpret_cast<uintptr_t>(p->fresh_values) % 16))
+            return CRIT_PKV_E_GEOMETRY;
+    }
     AttendArgs a;
     a.q = reinterpret_cast<const uint8_t*>(p->q);
     a.kp = reinterpret_cast<const uint8_t*>(p->key_pages);
@@ -295,6 +304,10 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     a.out = p->out, a.lse = p->lse, a.sinks = p->sinks;
     a.parents = p->parents, a.parents64 = p->parents64;
     a.blocks = p->blocks, a.blocks_stride = p->blocks_stride, a.blocks_k = p->blocks_k, a.block_size = p->block_size;
+    a.fk = reinterpret_cast<const uint8_t*>(p->fresh_keys), a.fv = reinterpret_cast<const uint8_t*>(p->fresh_values);
+    a.f_shifts = p->fresh_shifts, a.f_firsts = p->fresh_firsts;
+    a.f_stride_k = p->fresh_stride_k, a.f_stride_v = p->fresh_stride_v, a.f_rows = p->fresh_rows;
+    a.f_per_row = p->fresh_per_row ? 1 : 0;
     a.listed_keys = p->blocks ? p->blocks_k * p->block_size : 0;
     a.block_div = make_div32(p->blocks ? (uint32_t)p->block_size : 1u);
     a.q_st = p->q_stride_t, a.q_sh = p->q_stride_h, a.o_st = p->out_stride_t, a.o_sh = p->out_stride_h, a.tab_stride = p->table_stride;
@@ -320,7 +333,7 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     // (block lists of blocks that are a multiple of 16 positions walk their lists in the 128-wide kernel, others in
     // the generic one, each position looked up on its own)
     const bool fast_lists = p->blocks && lpr == 16 && p->page % 16 == 0 && p->block_size % 16 == 0;
-    const bool page16 = p->page % 16 == 0 && !p->blocks;
+    const bool page16 = p->page % 16 == 0 && !p->blocks && !fresh;      // (rows with fresh positions take the generic kernel)
     a.heads_per_wave = 1;
     if (lpr == 16 && (page16 || fast_lists)) {
         if (p->kv_heads % 2 == 0) a.heads_per_wave = 2;

@@ -39,6 +39,15 @@ struct AttendArgs {
     int blocks_k, block_size, listed_keys;      // listed_keys = blocks_k * block_size: the positions a list's run holds
     Div32 block_div;
     float sscale, k_mult, v_mult;
+    // Fresh rows (attend's fresh=): row r reads its positions from f_firsts[r * f_per_row] on from rows
+    // position - f_shifts[r * f_per_row] of fk / fv ([f_rows][kv_heads][dim], q's 16-bit type, unscaled) instead of the
+    // pages. fk null: every position from the pages.
+    const uint8_t* fk;
+    const uint8_t* fv;
+    const int64_t* f_shifts;
+    const int64_t* f_firsts;
+    int64_t f_stride_k, f_stride_v, f_rows;
+    int f_per_row;
 };
 
 // A 16-byte (or 8-byte) load of value rows, which are read once: nontemporal, so the caches do not keep them (measured

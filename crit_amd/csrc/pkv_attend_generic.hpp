@@ -22,18 +22,28 @@
 
 namespace pkv {
 
-template <int KIND>
+struct NoFreshRows {};
+struct FreshRows {
+    uint4 k[4], v[4];      // the lane's 8 elements of the four positions' fresh rows, 16-bit
+};
+template <int KIND, bool FRESH = false>
 struct StepBuf {
     using Vec = typename std::conditional<KIND == 0, uint4, uint2>::type;
     Vec k[4], v[4];
     float ks[4], vs[4];
     int pos[4];      // SPARSE: the position each of the lane group's four rows holds, -1 for none
+    typename std::conditional<FRESH, FreshRows, NoFreshRows>::type f;
 };
 
 
-template <int KIND, bool F16, int LPR, int QR, bool FUSED, bool SPARSE = false>
+// FRESH: positions from the row's first fresh one on are read from 16-bit rows given beside the pages (row = position -
+// the row's shift), unscaled: a score times the softmax scale only, a probability times 1 (_kernels.py:272-274, 291-345).
+// A lane holds the same 8 elements of a row either way (16 bytes of a fresh row, 8 or 16 of a page's), so both rows are
+// loaded for every position and the position picks one.
+template <int KIND, bool F16, int LPR, int QR, bool FUSED, bool SPARSE = false, bool FRESH = false>
 __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
     static_assert(!(SPARSE && FUSED), "block lists are read by the split launch");
+    static_assert(!(SPARSE && FRESH), "block lists read the pages only");
     constexpr int D = LPR * 8;
     constexpr int PPI = 64 / LPR;      // positions one load instruction of a wavefront covers
     constexpr int SP = 4 * PPI;        // positions a wavefront's step covers
@@ -66,6 +76,13 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
     if (!FUSED && b >= n_pieces) return;
     const int64_t trow = (int64_t)a.rows[r] * a.tab_stride;
     const int start = a.starts[r];
+    int f_first = 0x7fffffff;
+    int64_t f_shift = 0;
+    if constexpr (FRESH) {
+        const int64_t ff = a.f_firsts[(int64_t)r * a.f_per_row];
+        f_first = (int)(ff < 0 ? 0 : (ff > (int64_t)0x7fffffff ? (int64_t)0x7fffffff : ff));
+        f_shift = a.f_shifts[(int64_t)r * a.f_per_row];
+    }
     if constexpr (SPARSE) {      // the tile's column's list (QR divides the group: one column a tile)
         const int32_t* list = a.blocks + (int64_t)(start + c_lo) * a.blocks_stride;
         for (int i = tid; i < a.blocks_k; i += 256) s_blocks[i] = list[i];
@@ -140,7 +157,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
             tab[k] = a.tables[trow + pidx];
         }
     };
-    auto fetch_kv = [&](int base, const int (&tab)[4], const int (&pos)[4], StepBuf<KIND>& buf) {
+    auto fetch_kv = [&](int base, const int (&tab)[4], const int (&pos)[4], StepBuf<KIND, FRESH>& buf) {
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             int n = base + k * PPI + lg;
@@ -158,6 +175,12 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
             if constexpr (KIND >= 2) {
                 buf.ks[k] = a.ks[slot * a.hkv + kvh];
                 buf.vs[k] = a.vs[slot * a.hkv + kvh];
+            }
+            if constexpr (FRESH) {      // (unconditional too: a position below the first fresh one reads row 0 or its own clamped)
+                int64_t row = (int64_t)n - f_shift;
+                row = row < 0 ? 0 : (row >= a.f_rows ? a.f_rows - 1 : row);
+                buf.f.k[k] = *reinterpret_cast<const uint4*>(a.fk + (row * a.f_stride_k + (int64_t)kvh * D + li * 8) * 2);
+                buf.f.v[k] = load_once16(a.fv + (row * a.f_stride_v + (int64_t)kvh * D + li * 8) * 2);
             }
         }
     };
@@ -195,8 +218,11 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
             return base_of();
         };
 
-        auto compute = [&](int base, const StepBuf<KIND>& buf) __attribute__((always_inline)) {
+        auto compute = [&](int base, const StepBuf<KIND, FRESH>& buf) __attribute__((always_inline)) {
             float s[4][QR];
+            bool isf[4];      // FRESH: the position's row is a fresh one
+#pragma unroll
+            for (int k = 0; k < 4; ++k) isf[k] = FRESH && base + k * PPI + lg >= f_first;
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 uint32_t kw[4];
@@ -212,6 +238,18 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
                     const f32x2 a2 = e4m3_pair<false>(buf.k[k].y), a3 = e4m3_pair<true>(buf.k[k].y);
                     kf[0] = a0.x, kf[1] = a0.y, kf[2] = a1.x, kf[3] = a1.y;
                     kf[4] = a2.x, kf[5] = a2.y, kf[6] = a3.x, kf[7] = a3.y;
+                }
+                if constexpr (FRESH) {
+                    const uint32_t fw[4] = {buf.f.k[k].x, buf.f.k[k].y, buf.f.k[k].z, buf.f.k[k].w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if constexpr (KIND == 0) {
+                            kw[j] = isf[k] ? fw[j] : kw[j];
+                        } else {
+                            kf[2 * j] = isf[k] ? (F16 ? f16_lo(fw[j]) : bf16_lo(fw[j])) : kf[2 * j];
+                            kf[2 * j + 1] = isf[k] ? (F16 ? f16_hi(fw[j]) : bf16_hi(fw[j])) : kf[2 * j + 1];
+                        }
+                    }
                 }
 #pragma unroll
                 for (int rr = 0; rr < QR; ++rr) {
@@ -239,7 +277,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const int n = SPARSE ? buf.pos[k] : base + k * PPI + lg;
-                    float x = s[k][rr] * (KIND >= 2 ? sscale * buf.ks[k] : sscale);
+                    float x = s[k][rr] * (isf[k] ? a.sscale : (KIND >= 2 ? sscale * buf.ks[k] : sscale));
                     bool vis = n <= lim[rr] && n < n_keys;
                     if constexpr (SPARSE) vis = vis && n >= 0;
                     if (tree) vis = vis && (n < first || ((anc[rr] >> ((n - first) & 63)) & 1ull) != 0);
@@ -256,7 +294,11 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
                 for (int k = 0; k < 4; ++k) {
                     const float p = exp2_fast(s[k][rr] - sub);
                     sum += p;
-                    s[k][rr] = KIND >= 2 ? p * buf.vs[k] : p;
+                    if constexpr (FRESH && KIND != 0) {      // (FP8 pages' one value multiplier rides here too: a fresh row counts as given)
+                        s[k][rr] = isf[k] ? p : p * (KIND >= 2 ? buf.vs[k] : v_mult);
+                    } else {
+                        s[k][rr] = KIND >= 2 ? p * buf.vs[k] : p;
+                    }
                 }
                 l[rr] = __builtin_fmaf(l[rr], alpha, sum);
                 m[rr] = m_new;
@@ -283,6 +325,14 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
                     vf[0] = a0.x, vf[1] = a0.y, vf[2] = a1.x, vf[3] = a1.y;
                     vf[4] = a2.x, vf[5] = a2.y, vf[6] = a3.x, vf[7] = a3.y;
                 }
+                if constexpr (FRESH) {
+                    const uint32_t fw[4] = {buf.f.v[k].x, buf.f.v[k].y, buf.f.v[k].z, buf.f.v[k].w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        vf[2 * j] = isf[k] ? (F16 ? f16_lo(fw[j]) : bf16_lo(fw[j])) : vf[2 * j];
+                        vf[2 * j + 1] = isf[k] ? (F16 ? f16_hi(fw[j]) : bf16_hi(fw[j])) : vf[2 * j + 1];
+                    }
+                }
 #pragma unroll
                 for (int rr = 0; rr < QR; ++rr) {
 #pragma unroll
@@ -294,7 +344,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
         // Three-stage software pipeline: table entries two steps ahead, K/V one step ahead, compute. Every load of the
         // loop is issued unconditionally (past the wavefront's last step it re-reads its first step, which the caches
         // hold): with loads under conditions the compiler waits for all outstanding loads at every use.
-        StepBuf<KIND> bufA, bufB;
+        StepBuf<KIND, FRESH> bufA, bufB;
         int tabA[4], tabB[4], posA[4], posB[4];
         int base0 = base_of();
         if (base0 >= 0) {
@@ -366,7 +416,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
                     L = __builtin_fmaf(s_l[w][rr], f, L);
                     A = __builtin_fmaf(s_acc[w][rr][d], f, A);
                 }
-                A *= v_mult;
+                if constexpr (!(FRESH && KIND == 1)) A *= v_mult;      // (with fresh rows the multiplier went in a position at a time)
                 const int j = j0 + rr;
                 const int c = j / a.g;
                 if (c < count) {

@@ -49,6 +49,13 @@ static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipS
             case 4: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 4, FUSED>), pgrid, dim3(256), 0, stream, u); break;
             default: return CRIT_PKV_E_GEOMETRY;
         }
+    } else if (a.fk) {       // fresh rows beside the pages: the generic kernel's variant that reads both (any head width)
+        switch (lpr) {
+            case 8: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 8, QR, FUSED, false, true>), grid, dim3(256), 0, stream, a); break;
+            case 16: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 16, QR, FUSED, false, true>), grid, dim3(256), 0, stream, a); break;
+            case 32: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 32, QR, FUSED, false, true>), grid, dim3(256), 0, stream, a); break;
+            default: return CRIT_PKV_E_GEOMETRY;
+        }
     } else if (lpr == 16) {
         hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 16, QR, FUSED>), grid, dim3(256), 0, stream, a);
     } else if (lpr == 8) {

@@ -336,8 +336,12 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
     blocks [tokens][k] int32 and block_size: each token's list of KV block ids (block_size positions each, -1 for none,
     no id twice): the token sees, of its positions, only those of its listed blocks, and only they are read (a list is
     one run of k x block_size positions cut into pieces and partitions; up to MAX_LISTED_BLOCKS ids; not with fused,
-    flash or sliding). fresh and derive are not served. phases (a measurement's): 1 runs the split launch only, 2 the
-    merge only."""
+    flash or sliding). fresh: (keys [N][kv_heads][dim], values [N][kv_heads][value_dim] in q's dtype, shift, first):
+    each row's positions from `first` on are read from those rows instead of the pages (row = position - shift; a
+    prompt chunk's own keys and values as the projections gave them, unscaled), shift and first int64 device tensors
+    of one element a row, or of one element for every row; not with block lists; such launches take the generic
+    kernel, split or fused, the same bits either way. derive is not served. phases (a measurement's): 1 runs the split
+    launch only, 2 the merge only."""
     if derive is not None:
         raise _unsupported("derive= (keys derived from value rows)")
     if parents is not None:
@@ -360,8 +364,8 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
         if blocks.stride(-1) != 1:
             blocks = blocks.contiguous()
         flash = False      # (block lists: the split launch, as in the reference)
-    if fresh is not None:
-        raise _unsupported("fresh= (a prompt chunk's own rows)")
+    if fresh is not None and blocks is not None:
+        raise ValueError("fresh rows are not read through block lists")
     k_kind = _check_kind(kind, key_scales)
     _require_device(q, "attend's q")
     T, hq, d = q.shape
@@ -428,6 +432,25 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
     p.kind, p.page_dtype, p.out_dtype = k_kind, _page_dtype(key_pages, kind), _DTYPE[out.dtype]
     p.partitions, p.piece, p.fused, p.sliding, p.phases = parts, piece, int(bool(fused)), sliding, int(phases)
     p.scale, p.key_multiplier, p.value_multiplier = scale, km, vm
+    if fresh is not None:
+        fk, fv, fshift, ffirst = fresh
+        if not (torch.is_tensor(fk) and torch.is_tensor(fv)) or fk.dim() != 3 or fk.shape[1:] != (hkv, d) or \
+                fv.shape[1:] != (hkv, dv) or fk.shape[0] != fv.shape[0] or fk.shape[0] < 1 or fk.stride(-1) != 1 or \
+                fv.stride(-1) != 1 or fk.stride(1) != d or fv.stride(1) != dv or not torch.is_tensor(fshift) or \
+                not torch.is_tensor(ffirst) or fshift.numel() != ffirst.numel() or fshift.numel() not in (1, R):
+            raise ValueError(f"fresh rows are [N][{hkv}][dim] each, head rows contiguous, with one shift and first "
+                             "a row or one for every row")
+        if fk.dtype != q.dtype or fv.dtype != q.dtype or fk.device != device or fv.device != device:
+            raise ValueError("fresh rows in q's dtype on q's device")
+        if fshift.dtype != torch.int64 or ffirst.dtype != torch.int64 or fshift.device != device or \
+                ffirst.device != device or not fshift.is_contiguous() or not ffirst.is_contiguous():
+            raise ValueError("a fresh row's shift and first are contiguous int64 tensors on q's device")
+        if fk.stride(0) % 8 or fv.stride(0) % 8 or fk.data_ptr() % 16 or fv.data_ptr() % 16:
+            raise ValueError("fresh rows 16-byte aligned, their token stride a multiple of 8 elements")
+        p.fresh_keys, p.fresh_values = fk.data_ptr(), fv.data_ptr()
+        p.fresh_shifts, p.fresh_firsts = fshift.data_ptr(), ffirst.data_ptr()
+        p.fresh_stride_k, p.fresh_stride_v, p.fresh_rows = fk.stride(0), fv.stride(0), int(fk.shape[0])
+        p.fresh_per_row = int(fshift.numel() != 1)
     with torch.cuda.device(device):
         _abi.check(_abi.load().crit_pkv_attend(p, _stream(device)), "paged_kv_attention.attend")
     return out

@@ -10,7 +10,7 @@ import shutil
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 NAME = "libcrit_pkv.so"
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 KIND_16BIT, KIND_FP8, KIND_FP8_ROW, KIND_INT8 = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
@@ -38,7 +38,9 @@ class AttendParams(ctypes.Structure):
                 ("head_dim", _i32), ("value_dim", _i32), ("page", _i32), ("kind", _i32), ("page_dtype", _i32),
                 ("out_dtype", _i32), ("partitions", _i32), ("piece", _i32), ("fused", _i32), ("sliding", _i32), ("phases", _i32),
                 ("blocks_k", _i32), ("block_size", _i32),
-                ("scale", _f32), ("key_multiplier", _f32), ("value_multiplier", _f32)]
+                ("scale", _f32), ("key_multiplier", _f32), ("value_multiplier", _f32),
+                ("fresh_keys", _p), ("fresh_values", _p), ("fresh_shifts", _p), ("fresh_firsts", _p),
+                ("fresh_stride_k", _i64), ("fresh_stride_v", _i64), ("fresh_rows", _i64), ("fresh_per_row", _i32)]
 
 
 class MergeParams(ctypes.Structure):

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 4
+#define CRIT_PKV_ABI_VERSION 5
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -123,6 +123,17 @@ typedef struct crit_pkv_attend_params {
                                        (for timing one kernel; ignored when fused) */
     int32_t blocks_k, block_size;   /* ids a list (1 .. 1024), positions a block (>= 1) */
     float scale, key_multiplier, value_multiplier;
+    /* Fresh rows (attend's fresh=, __init__.py:417-421, _kernels.py:272-274, 291-345): row r reads its positions from
+     * fresh_firsts[i] on from rows `position - fresh_shifts[i]` of fresh_keys / fresh_values ([fresh_rows][kv_heads][dim]
+     * in q's type, each head row contiguous, token rows fresh_stride_k / _v elements apart) instead of the pages,
+     * unscaled; i = r with fresh_per_row, else 0 (one shift and first for every row). All four pointers or none. Not
+     * with block lists. Such launches take the generic kernel whatever the head width. */
+    const void* fresh_keys;
+    const void* fresh_values;
+    const int64_t* fresh_shifts;
+    const int64_t* fresh_firsts;
+    int64_t fresh_stride_k, fresh_stride_v, fresh_rows;
+    int32_t fresh_per_row;
 } crit_pkv_attend_params;
 
 int crit_pkv_attend(const crit_pkv_attend_params* p, void* stream);

@@ -174,6 +174,73 @@ def test_a_row_of_many_partitions_merges_to_the_fused_launchs_bits(kind, hq, hkv
         _close(slid, want)
 
 
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 128), (24, 4, 256), (12, 2, 64)])
+def test_rows_read_their_fresh_positions_beside_the_pages(kind, hq, hkv, d):
+    # attend(fresh=(keys, values, shift, first)): a prompt chunk of 130 tokens at position 300 as window rows of up to
+    # 64 columns (DeviceAttention._decode_rows' pieces, device_attention.py:751-783), its own positions from 16-bit
+    # rows as the projections gave them (row = position - shift, unscaled), the prefix from the pages: against the
+    # oracle, one shift and first for every row and one a row (a row whose first lies past every position reads the
+    # pages only); split = fused = each row alone, bit for bit; with a sliding window and sinks.
+    position, T = 300, 130
+    cache = Cache(kind, hkv, d, d, 16, [position + T], seed=71)
+    q = rand_q(T, hq, d, 72)
+    q_dtype = torch.float16 if kind == "fp16" else torch.bfloat16
+    g = torch.Generator().manual_seed(73)
+    fk, fv = torch.randn(T, hkv, d, generator=g).to(q_dtype).to(dev), torch.randn(T, hkv, d, generator=g).to(q_dtype).to(dev)
+    starts = [0, 64, 128]
+    counts = torch.tensor([64, 64, 2], dtype=torch.int32, device=dev)
+    firsts = [position + s for s in starts]
+    i64 = lambda x: torch.tensor(x, dtype=torch.int64, device=dev)
+    one = (fk, fv, i64([position]), i64([position]))
+    lse, fused_lse = torch.empty(T, hq, device=dev), torch.empty(T, hq, device=dev)
+    out = cache.attend(q, [0, 0, 0], starts, firsts, 64, counts=counts, fresh=one, lse=lse)
+    fused = cache.attend(q, [0, 0, 0], starts, firsts, 64, counts=counts, fresh=one, lse=fused_lse, fused=True)
+    assert torch.equal(out, fused) and torch.equal(lse, fused_lse)
+    for t in (0, 1, 63, 64, 129):
+        want, want_lse = cache.want(q[t:t + 1], 0, position + t, 1, fresh=(fk.cpu(), fv.cpu(), position, position))
+        _close(out[t:t + 1], want, f"token {t}")
+        _close_lse(lse[t:t + 1], want_lse, f"lse {t}")
+    alone = cache.attend(q[64:128], [0], [0], [position + 64], 64, fresh=one)
+    assert torch.equal(alone, out[64:128])
+    # a shift and a first for each row: the second row's own positions only (its first 64 positions back in the
+    # pages), the third row none
+    each = (fk, fv, i64([position] * 3), i64([position, position + 64, 1 << 62]))
+    mixed = cache.attend(q, [0, 0, 0], starts, firsts, 64, counts=counts, fresh=each)
+    assert torch.equal(mixed[:64], out[:64])
+    want, _ = cache.want(q[100:101], 0, position + 100, 1, fresh=(fk.cpu(), fv.cpu(), position, position + 64))
+    _close(mixed[100:101], want, "second row")
+    want, _ = cache.want(q[129:130], 0, position + 129, 1)
+    _close(mixed[129:130], want, "third row")
+    sinks = torch.linspace(-1, 1, hq, device=dev)
+    slid = cache.attend(q, [0, 0, 0], starts, firsts, 64, counts=counts, fresh=one, sliding=90, sinks=sinks, lse=lse)
+    assert torch.equal(slid, cache.attend(q, [0, 0, 0], starts, firsts, 64, counts=counts, fresh=one, sliding=90,
+                                          sinks=sinks, fused=True))
+    plain_lse = torch.empty(T, hq, device=dev)
+    plain = cache.attend(q, [0, 0, 0], starts, firsts, 64, counts=counts, fresh=one, sliding=90, lse=plain_lse)
+    want, want_lse = cache.want(q[70:71], 0, position + 70, 1, sliding=90, fresh=(fk.cpu(), fv.cpu(), position, position))
+    _close(plain[70:71], want, "window")
+    _close_lse(plain_lse[70:71], want_lse, "window lse")
+    weight = torch.exp(plain_lse) / (torch.exp(plain_lse) + torch.exp(sinks)[None, :])
+    torch.testing.assert_close(slid.float(), plain.float() * weight[..., None], atol=8e-3, rtol=2e-2)
+
+
+def test_fresh_rows_that_do_not_fit_are_refused():
+    cache = Cache("bf16", 2, 128, 128, 16, [100])
+    q = rand_q(4, 8, 128, 1)
+    fk = torch.zeros(4, 2, 128, dtype=torch.bfloat16, device=dev)
+    i64 = lambda x: torch.tensor(x, dtype=torch.int64, device=dev)
+    with pytest.raises(ValueError):
+        cache.attend(q, [0], [0], [96], 4, fresh=(fk[:, :1], fk, i64([96]), i64([96])))
+    with pytest.raises(ValueError):
+        cache.attend(q, [0], [0], [96], 4, fresh=(fk.float(), fk.float(), i64([96]), i64([96])))
+    with pytest.raises(ValueError):
+        cache.attend(q, [0], [0], [96], 4, fresh=(fk, fk, i64([96, 96]), i64([96, 96])))
+    with pytest.raises(ValueError):
+        cache.attend(q, [0], [0], [96], 4, fresh=(fk, fk, i64([96]), i64([96])),
+                     blocks=torch.zeros(4, 2, dtype=torch.int32, device=dev), block_size=16)
+
+
 def test_a_given_workspace_holds_the_partials_and_a_small_one_is_refused():
     pk = kernels()
     cache = Cache("bf16", 2, 128, 128, 16, [300])
@@ -378,8 +445,7 @@ def test_bad_geometry_is_refused():
     with pytest.raises(ValueError, match="offsets"):
         cache.attend(q, [0], [0], [99], 1, offsets=torch.zeros(1, dtype=torch.int32, device=dev))
     with pytest.raises(NotImplementedError):
-        cache.attend(q, [0], [0], [99], 1, fresh=(q, q, torch.zeros(1, dtype=torch.int64, device=dev),
-                                                    torch.zeros(1, dtype=torch.int64, device=dev)))
+        cache.attend(q, [0], [0], [99], 1, derive=(q, 0))
 
 
 def test_launches_that_overlap_on_two_streams_do_not_share_counters():
