@@ -19,6 +19,18 @@ int crit_pkv_prefill(const crit_pkv_prefill_params* p, void* stream) {
     return pkv::launch_prefill(p, reinterpret_cast<hipStream_t>(stream));
 }
 
+int crit_pkv_slots_at(const crit_pkv_slots_params* p, void* stream) {
+    return pkv::launch_slots_at(p, reinterpret_cast<hipStream_t>(stream));
+}
+
+int crit_pkv_compact(const crit_pkv_compact_params* p, void* stream) {
+    return pkv::launch_compact(p, reinterpret_cast<hipStream_t>(stream));
+}
+
+int crit_pkv_copy_pages(const crit_pkv_copy_pages_params* p, void* stream) {
+    return pkv::launch_copy_pages(p, reinterpret_cast<hipStream_t>(stream));
+}
+
 int crit_pkv_stream_read(const void* data, int64_t bytes, float* sink, void* stream) {
     return pkv::launch_stream_read(data, bytes, sink, reinterpret_cast<hipStream_t>(stream));
 }
@@ -31,6 +43,9 @@ int crit_pkv_params_size(int which) {
         case 1: return (int)sizeof(crit_pkv_attend_params);
         case 2: return (int)sizeof(crit_pkv_merge_params);
         case 3: return (int)sizeof(crit_pkv_prefill_params);
+        case 4: return (int)sizeof(crit_pkv_slots_params);
+        case 5: return (int)sizeof(crit_pkv_compact_params);
+        case 6: return (int)sizeof(crit_pkv_copy_pages_params);
     }
     return -1;
 }
@@ -38,7 +53,7 @@ int crit_pkv_params_size(int which) {
 const char* crit_pkv_error(int code) {
     switch (code) {
         case 0: return "ok";
-        case CRIT_PKV_E_GEOMETRY: return "crit_pkv: a shape the kernels do not take (head dims 64/128/256 with keys and values of one width, query heads a multiple of the KV heads, 1..64 columns, 16-byte aligned rows)";
+        case CRIT_PKV_E_GEOMETRY: return "crit_pkv: a shape the kernels do not take (head dims 64/128/256 with keys and values of one width, query heads a multiple of the KV heads, 1..64 columns, 16-byte aligned rows; pool stores in multiples of 4 bytes, tree paths of up to 256 columns)";
         case CRIT_PKV_E_DTYPE: return "crit_pkv: a dtype or page kind the kernels do not take";
         case CRIT_PKV_E_NULL: return "crit_pkv: a required pointer is NULL";
         case CRIT_PKV_E_WORKSPACE: return "crit_pkv: partitions, piece or the partial arrays do not fit the launch";

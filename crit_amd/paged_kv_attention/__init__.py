@@ -35,7 +35,7 @@ from . import _abi
 __all__ = ["KINDS", "PIECE", "MAX_COLUMNS", "Derive", "attend", "derive", "cuda_block", "cuda_chunk", "cuda_parts",
            "cuda_prompt", "cuda_ramp", "cuda_splits", "flash_block", "flash_chunk", "flash_parts", "flash_tile",
            "merge_shards", "owner", "partitions", "piece_size", "prefill", "prefill_rows", "prefill_state_floats", "release",
-           "stream_read",
+           "stream_read", "slots_at", "compact", "copy_pages",
            "tile_for", "workspace_floats", "write"]
 
 KINDS = {"bf16": 0, "fp16": 0, "fp8": 1, "fp8:row": 2, "int8": 3}
@@ -661,3 +661,115 @@ def stream_read(data, sink=None):
         _abi.check(_abi.load().crit_pkv_stream_read(data.data_ptr(), nbytes, sink.data_ptr(), _stream(data.device)),
                    "paged_kv_attention.stream_read")
     return sink
+
+
+# -- pool bookkeeping on the device (reference: inference/attention-state/code/pages.py:646-684, 861-869) ----------------
+def _i64_on(t, device, what, n=None):
+    if not torch.is_tensor(t) or t.dtype != torch.int64 or t.device != device or not t.is_contiguous() or \
+            (n is not None and t.numel() < n):
+        raise ValueError(f"{what} is a contiguous int64 tensor on the tables' device" + (f" of {n} or more" if n else ""))
+    return t
+
+
+def _tables(round_tables, round_capacity):
+    _require_device(round_tables, "the round tables")
+    if round_tables.dtype != torch.int32 or round_tables.dim() != 2 or round_tables.stride(1) != 1 or \
+            round_tables.shape[0] < 1 or round_tables.shape[1] < 1:
+        raise ValueError("round tables are [round slots][table pages] int32, a row contiguous")
+    _i64_on(round_capacity, round_tables.device, "the round slots' capacity", round_tables.shape[0])
+
+
+def _stores(p, stores, layers, slots):
+    """Fills p.stores from tensors [layers][...] whose layer holds `slots` rows back to back (keys, values, scales)."""
+    stores = [s for s in stores if s is not None]
+    if not 1 <= len(stores) <= _abi.MAX_STORES:
+        raise ValueError(f"1 to {_abi.MAX_STORES} stores (keys, values, their scales)")
+    device = stores[0].device
+    for i, s in enumerate(stores):
+        _require_device(s, "a store")
+        if s.device != device or s.dim() < 2 or s.shape[0] != layers or not s[0].is_contiguous():
+            raise ValueError(f"a store is [{layers} layers][...] on one device, each layer contiguous")
+        layer_bytes = s[0].numel() * s.element_size()
+        if slots < 1 or layer_bytes % slots:
+            raise ValueError(f"a layer of a store holds {slots} rows of one size")
+        p.stores[i].base, p.stores[i].layer_stride = s.data_ptr(), s.stride(0) * s.element_size()
+        p.stores[i].row_bytes = layer_bytes // slots
+    p.n_stores, p.layers = len(stores), layers
+    return device
+
+
+def slots_at(round_tables, round_capacity, slot, positions, page, dump, *, rows=None, out=None):
+    """The KV slots of `positions` of the sequences bound to round slots `slot` (any shape, both int64): KVPool._slots_at
+    (pages.py:655-660) in one launch: table[min(p // page, pages - 1)] * page + p % page where 0 <= p < the slot's
+    capacity, the dump page's first slot (dump * page) elsewhere. rows: `slot` holds one entry a row and rows [n] names
+    each position's row (the index_select of _reserve_round, pages.py:652-653). A round slot that does not exist reads
+    as one without capacity. Returns out (int64, positions' shape)."""
+    _tables(round_tables, round_capacity)
+    device = round_tables.device
+    _i64_on(slot, device, "slots_at's slot")
+    _i64_on(positions, device, "slots_at's positions")
+    if rows is not None:
+        _i64_on(rows, device, "slots_at's rows", positions.numel())
+    elif slot.numel() != positions.numel():
+        raise ValueError("one round slot a position (or rows=)")
+    if out is None:
+        out = torch.empty_like(positions)
+    else:
+        _i64_on(out, device, "slots_at's out", positions.numel())
+    p = _abi.SlotsParams()
+    p.round_tables, p.round_capacity, p.slots, p.rows = round_tables.data_ptr(), round_capacity.data_ptr(), slot.data_ptr(), _ptr(rows)
+    p.positions, p.out, p.n, p.n_slots = positions.data_ptr(), out.data_ptr(), positions.numel(), slot.numel()
+    p.round_slots, p.table_stride, p.table_pages = round_tables.shape[0], round_tables.stride(0), round_tables.shape[1]
+    p.page, p.dump = int(page), int(dump)
+    with torch.cuda.device(device):
+        _abi.check(_abi.load().crit_pkv_slots_at(p, _stream(device)), "paged_kv_attention.slots_at")
+    return out
+
+
+def compact(stores, slots, round_tables, round_capacity, start, emitted, path, moved, page, dump):
+    """An accepted draft-tree path's rows to consecutive positions, KVPool._compact (pages.py:662-684) in one launch
+    over every layer and store: for round row r (round slot r) where moved[r] == 0, node path[r][j] at position
+    start[r] + path[r][j] moves to start[r] + j for 0 < j < emitted[r] with path[r][j] >= 0; then moved[:rows] = 1.
+    stores: the pool's tensors [layers][...] (keys, values, row scales; None entries skipped), each layer `slots` rows;
+    path [rows][width] int64 or int32 (up to 256 columns); start, emitted, moved int64 [rows or more]."""
+    _tables(round_tables, round_capacity)
+    device = round_tables.device
+    if not torch.is_tensor(path) or path.dim() != 2 or path.dtype not in (torch.int64, torch.int32) or \
+            path.device != device or path.stride(1) != 1 or not 1 <= path.shape[1] <= _abi.MAX_PATH:
+        raise ValueError(f"a tree path is [rows][1 .. {_abi.MAX_PATH} columns] int64 or int32 on the tables' device")
+    rows = path.shape[0]
+    if rows > round_tables.shape[0]:
+        raise ValueError(f"{rows} rows read round slots 0 .. {rows - 1}; the tables hold {round_tables.shape[0]}")
+    if rows == 0:
+        return
+    p = _abi.CompactParams()
+    live = [s for s in stores if s is not None]
+    if not live:
+        raise ValueError("compact moves the rows of one store at least")
+    if _stores(p, live, live[0].shape[0], int(slots)) != device:
+        raise ValueError("stores on the tables' device")
+    p.round_tables, p.round_capacity = round_tables.data_ptr(), round_capacity.data_ptr()
+    p.start, p.emitted = _i64_on(start, device, "start", rows).data_ptr(), _i64_on(emitted, device, "emitted", rows).data_ptr()
+    p.moved, p.path = _i64_on(moved, device, "moved", rows).data_ptr(), path.data_ptr()
+    p.rows, p.round_slots, p.table_stride, p.path_stride = rows, round_tables.shape[0], round_tables.stride(0), path.stride(0)
+    p.width, p.path_is_32, p.table_pages, p.page, p.dump = path.shape[1], int(path.dtype == torch.int32), round_tables.shape[1], int(page), int(dump)
+    with torch.cuda.device(device):
+        _abi.check(_abi.load().crit_pkv_compact(p, _stream(device)), "paged_kv_attention.compact")
+
+
+def copy_pages(stores, slots, source, target, page):
+    """Pages source[i] copied to pages target[i] in every layer of every store (the copies of KVPool._copy,
+    pages.py:861-869, for all of a step's shared pages at once): source, target int64 [n] on the device, a pair with a
+    negative id skipped; no target is another pair's source or target. stores and slots as compact() takes them."""
+    live = [s for s in stores if s is not None]
+    if not live:
+        raise ValueError("copy_pages copies the pages of one store at least")
+    p = _abi.CopyPagesParams()
+    device = _stores(p, live, live[0].shape[0], int(slots))
+    _i64_on(source, device, "copy_pages' source")
+    _i64_on(target, device, "copy_pages' target", source.numel())
+    if source.numel() == 0:
+        return
+    p.source, p.target, p.n, p.page = source.data_ptr(), target.data_ptr(), source.numel(), int(page)
+    with torch.cuda.device(device):
+        _abi.check(_abi.load().crit_pkv_copy_pages(p, _stream(device)), "paged_kv_attention.copy_pages")

@@ -10,7 +10,7 @@ import shutil
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 NAME = "libcrit_pkv.so"
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 KIND_16BIT, KIND_FP8, KIND_FP8_ROW, KIND_INT8 = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
@@ -61,8 +61,35 @@ class PrefillParams(ctypes.Structure):
                 ("fresh_stride_k", _i64), ("fresh_stride_v", _i64), ("int8_qk", _i32)]
 
 
-SYMBOLS = ("crit_pkv_write", "crit_pkv_attend", "crit_pkv_merge", "crit_pkv_prefill", "crit_pkv_abi_version",
-           "crit_pkv_params_size", "crit_pkv_error", "crit_pkv_stream_read")
+class Store(ctypes.Structure):
+    _fields_ = [("base", _p), ("layer_stride", _i64), ("row_bytes", _i64)]
+
+
+MAX_STORES, MAX_PATH = 4, 256
+
+
+class SlotsParams(ctypes.Structure):
+    _fields_ = [("round_tables", _p), ("round_capacity", _p), ("slots", _p), ("rows", _p), ("positions", _p), ("out", _p),
+                ("n", _i64), ("round_slots", _i64), ("table_stride", _i64), ("n_slots", _i64),
+                ("table_pages", _i32), ("page", _i32), ("dump", _i32)]
+
+
+class CompactParams(ctypes.Structure):
+    _fields_ = [("round_tables", _p), ("round_capacity", _p), ("start", _p), ("emitted", _p), ("path", _p), ("moved", _p),
+                ("stores", Store * MAX_STORES),
+                ("rows", _i64), ("round_slots", _i64), ("table_stride", _i64), ("path_stride", _i64),
+                ("n_stores", _i32), ("layers", _i32), ("width", _i32), ("path_is_32", _i32), ("table_pages", _i32),
+                ("page", _i32), ("dump", _i32)]
+
+
+class CopyPagesParams(ctypes.Structure):
+    _fields_ = [("source", _p), ("target", _p), ("stores", Store * MAX_STORES), ("n", _i64),
+                ("n_stores", _i32), ("layers", _i32), ("page", _i32)]
+
+
+SYMBOLS = ("crit_pkv_write", "crit_pkv_attend", "crit_pkv_merge", "crit_pkv_prefill", "crit_pkv_slots_at",
+           "crit_pkv_compact", "crit_pkv_copy_pages", "crit_pkv_abi_version", "crit_pkv_params_size", "crit_pkv_error",
+           "crit_pkv_stream_read")
 
 _lib = None
 
@@ -107,7 +134,9 @@ def load():
     lib.crit_pkv_error.argtypes = [ctypes.c_int]
     lib.crit_pkv_params_size.argtypes = [ctypes.c_int]
     for name, struct in (("crit_pkv_write", WriteParams), ("crit_pkv_attend", AttendParams),
-                         ("crit_pkv_merge", MergeParams), ("crit_pkv_prefill", PrefillParams)):
+                         ("crit_pkv_merge", MergeParams), ("crit_pkv_prefill", PrefillParams),
+                         ("crit_pkv_slots_at", SlotsParams), ("crit_pkv_compact", CompactParams),
+                         ("crit_pkv_copy_pages", CopyPagesParams)):
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(struct), ctypes.c_void_p]
@@ -115,7 +144,8 @@ def load():
     lib.crit_pkv_stream_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
     if lib.crit_pkv_abi_version() != ABI_VERSION:
         raise RuntimeError(f"{path} speaks ABI {lib.crit_pkv_abi_version()}, this package {ABI_VERSION}: rebuild it")
-    for which, struct in enumerate((WriteParams, AttendParams, MergeParams, PrefillParams)):
+    for which, struct in enumerate((WriteParams, AttendParams, MergeParams, PrefillParams, SlotsParams, CompactParams,
+                                    CopyPagesParams)):
         if lib.crit_pkv_params_size(which) != ctypes.sizeof(struct):
             raise RuntimeError(f"{path}: parameter struct {which} is {lib.crit_pkv_params_size(which)} bytes, the "
                                f"Python mirror {ctypes.sizeof(struct)}: rebuild the library")

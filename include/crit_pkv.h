@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 5
+#define CRIT_PKV_ABI_VERSION 6
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -200,10 +200,80 @@ typedef struct crit_pkv_prefill_params {
 
 int crit_pkv_prefill(const crit_pkv_prefill_params* p, void* stream);
 
+/* ---- pool bookkeeping on the device --------------------------------------------------------------------------------
+ * What KVPool does with torch indexing for rounds that run without the host (inference/attention-state/code/
+ * pages.py): the slots of positions through the bound page tables, the move of an accepted draft-tree path's rows,
+ * and the copy of a shared page before it is written. One launch each, nothing read on the host, so a decode step's
+ * slots -> append -> attention chain is captured as one HIP graph. */
+
+/* A store of rows the pool holds per layer: a layer's rows start at base + layer * layer_stride (bytes); row `slot`
+ * is row_bytes bytes at slot * row_bytes (keys: kv_heads * head_dim elements; row scales: kv_heads floats).
+ * row_bytes and layer_stride are multiples of 4; stores whose base, stride and row_bytes are multiples of 16 move
+ * 16 bytes a lane. */
+typedef struct crit_pkv_store {
+    void* base;
+    int64_t layer_stride;
+    int64_t row_bytes;
+} crit_pkv_store;
+
+#define CRIT_PKV_MAX_STORES 4       /* keys, values, key scales, value scales */
+#define CRIT_PKV_MAX_PATH 256       /* columns of a tree path */
+
+/* Replaces KVPool._slots_at and the index_select before it in _reserve_round (pages.py:646-660):
+ *   s = rows ? slots[rows[i]] : slots[i];   p = positions[i]
+ *   out[i] = 0 <= p < round_capacity[s] ? round_tables[s][min(p / page, table_pages - 1)] * page + p % page
+ *                                       : dump * page
+ * A round slot outside 0 .. round_slots - 1 (the reference's indexing would raise) reads as capacity 0. */
+typedef struct crit_pkv_slots_params {
+    const int32_t* round_tables;    /* [round_slots][table_stride >= table_pages] */
+    const int64_t* round_capacity;  /* [round_slots] */
+    const int64_t* slots;           /* the round slot of each token, or of each row with `rows` */
+    const int64_t* rows;            /* optional [n]: the row of each token */
+    const int64_t* positions;       /* [n] */
+    int64_t* out;                   /* [n] */
+    int64_t n, round_slots, table_stride, n_slots;   /* n_slots: entries of `slots` (bounds rows[i]) */
+    int32_t table_pages, page, dump;
+} crit_pkv_slots_params;
+
+int crit_pkv_slots_at(const crit_pkv_slots_params* p, void* stream);
+
+/* Replaces KVPool._compact (pages.py:662-684), called by commit_round for a draft tree: for round row r (round slot
+ * r) and column 0 < j < min(width, emitted[r]) with path[r][j] >= 0, where moved[r] == 0, the row of every store and
+ * layer at position start[r] + path[r][j] is copied to position start[r] + j (slots as crit_pkv_slots_at finds them:
+ * a position outside the slot's capacity is the dump page's first slot). All of a row's sources are read before any
+ * of its targets is written, as index_copy_(index_select()) does. Then moved[r] = 1 for every r < rows (a second
+ * launch on the same stream). */
+typedef struct crit_pkv_compact_params {
+    const int32_t* round_tables;
+    const int64_t* round_capacity;
+    const int64_t* start;           /* [rows] */
+    const int64_t* emitted;         /* [rows] */
+    const void* path;               /* [rows][path_stride >= width], int64, or int32 with path_is_32 */
+    int64_t* moved;                 /* [rows] */
+    crit_pkv_store stores[CRIT_PKV_MAX_STORES];
+    int64_t rows, round_slots, table_stride, path_stride;
+    int32_t n_stores, layers, width, path_is_32, table_pages, page, dump;
+} crit_pkv_compact_params;
+
+int crit_pkv_compact(const crit_pkv_compact_params* p, void* stream);
+
+/* Replaces the copies of KVPool._copy (pages.py:861-869: a page shared with a fork is copied before it is written),
+ * for n pages at once: every store's rows source[i] * page .. + page - 1 of every layer are copied to the rows of
+ * target[i]. A pair with a negative id is skipped. No target may be another pair's source or target. */
+typedef struct crit_pkv_copy_pages_params {
+    const int64_t* source;          /* [n] page ids */
+    const int64_t* target;          /* [n] */
+    crit_pkv_store stores[CRIT_PKV_MAX_STORES];
+    int64_t n;
+    int32_t n_stores, layers, page;
+} crit_pkv_copy_pages_params;
+
+int crit_pkv_copy_pages(const crit_pkv_copy_pages_params* p, void* stream);
+
 /* ---- housekeeping ------------------------------------------------------------------------------------------------- */
 int crit_pkv_abi_version(void);
 /* sizeof() of the parameter structs as the library was compiled, for the host's mirror to cross-check
- * (which: 0 write, 1 attend, 2 merge, 3 prefill), as crit_cw_params_size() does (cuda_window.cu:1502). */
+ * (which: 0 write, 1 attend, 2 merge, 3 prefill, 4 slots_at, 5 compact, 6 copy_pages), as crit_cw_params_size() does (cuda_window.cu:1502). */
 int crit_pkv_params_size(int which);
 const char* crit_pkv_error(int code);
 /* A streaming-read probe: sums `bytes` (a multiple of 16) of device memory into sink[0..63]; the achievable-HBM-read

@@ -1,0 +1,237 @@
+"""The pool's device-side bookkeeping on the GPU against the CPU oracle, bit for bit: slots of positions through bound
+page tables, the move of an accepted draft-tree path's rows, copies of whole pages; and a decode step (slots -> append
+-> attention) captured once and replayed as the sequences grow. Mirrors the reference's
+inference/attention-state/tests/test_rounds.py:45-60, 190-215, 275-291. Calls go through the kernels module, which
+reaches the HIP kernels through the C ABI."""
+import pytest
+import torch
+
+from oracle import pool as oracle_pool
+from tests.support import STORE, bits, kernels
+
+pytestmark = pytest.mark.gpu
+dev = "cuda"
+
+
+def _round_pool(page, table_pages, lengths, round_slots, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    pages = round_slots * table_pages
+    order = torch.randperm(pages, generator=g).tolist()
+    tables = torch.full((round_slots, table_pages), pages, dtype=torch.int32)
+    capacity = torch.zeros(round_slots, dtype=torch.int64)
+    for s, n in lengths:
+        held = -(-n // page)
+        tables[s, :held] = torch.tensor([order.pop() for _ in range(held)], dtype=torch.int32)
+        capacity[s] = n
+    return tables, capacity, pages
+
+
+def test_slots_are_the_closed_form_inside_capacity_and_the_dump_page_outside():
+    pk = kernels()
+    page = 16
+    tables, capacity, dump = _round_pool(page, 40, [(0, 600), (1, 17), (3, 640), (5, 1)], 6)
+    wide = torch.full((6, 48), -5, dtype=torch.int32, device=dev)      # the tables as a view of wider rows
+    wide[:, :40] = tables.to(dev)
+    tables_dev = wide[:, :40]
+    g = torch.Generator().manual_seed(3)
+    n = 70001      # more than one workgroup's, not a multiple of anything
+    slot = torch.randint(0, 6, (n,), generator=g)
+    where = torch.randint(-3, 700, (n,), generator=g)
+    where[:4] = torch.tensor([0, 599, 600, -1])
+    slot[:4] = 0
+    want = oracle_pool.slots_at(tables, capacity, slot, where, page, dump)
+    got = pk.slots_at(tables_dev, capacity.to(dev), slot.to(dev), where.to(dev), page, dump)
+    assert torch.equal(got.cpu(), want)
+    # any shape, and an output given (test_rounds.py:283-289)
+    out = torch.full((10, 7), -7, dtype=torch.int64, device=dev)
+    pk.slots_at(tables_dev, capacity.to(dev), slot[:70].view(10, 7).to(dev), where[:70].view(10, 7).to(dev), page, dump,
+                out=out)
+    assert torch.equal(out.cpu(), want[:70].view(10, 7))
+    # a round's reserve: each token's row's slot first (pages.py:652-653)
+    slots_t = torch.tensor([3, 0, 5, 2])
+    rows_t = torch.randint(0, 4, (300,), generator=g)
+    positions = torch.randint(0, 660, (300,), generator=g)
+    want = oracle_pool.reserve_round(tables, capacity, slots_t, rows_t, positions, page, dump)
+    got = pk.slots_at(tables_dev, capacity.to(dev), slots_t.to(dev), positions.to(dev), page, dump, rows=rows_t.to(dev))
+    assert torch.equal(got.cpu(), want)
+    # round slots that do not exist read as slots without capacity
+    got = pk.slots_at(tables_dev, capacity.to(dev), torch.tensor([6, -1, 0], device=dev),
+                      torch.tensor([0, 0, 0], device=dev), page, dump)
+    assert got.tolist() == [dump * page, dump * page, int(tables[0, 0]) * page]
+    assert pk.slots_at(tables_dev, capacity.to(dev), slot[:0].to(dev), where[:0].to(dev), page, dump).numel() == 0
+
+
+def _stores(kind, layers, slots, hkv, d, seed, one_allocation=False):
+    g = torch.Generator().manual_seed(seed)
+    if kind in ("bf16", "fp16"):
+        make = lambda: torch.randn(layers, slots, hkv, d, generator=g).to(STORE[kind])
+    else:
+        make = lambda: torch.randint(0, 256, (layers, slots, hkv, d), generator=g, dtype=torch.uint8).view(
+            torch.int8 if kind == "int8" else torch.float8_e4m3fn)
+    found = [make(), make()]
+    if kind in ("fp8:row", "int8"):
+        found += [torch.rand(layers, slots, hkv, generator=g), torch.rand(layers, slots, hkv, generator=g)]
+    return found
+
+
+def _on_device(stores, interleaved):
+    """The stores on the GPU; interleaved: keys and values as two views of one allocation, a layer's keys followed by its
+    values (a layer stride that is not the layer's size)."""
+    if not interleaved:
+        return [s.to(dev) for s in stores]
+    k, v = stores[0], stores[1]
+    both = torch.stack([bits(k), bits(v)], dim=1).to(dev).contiguous()      # [layers][2][slots][hkv][d]
+    return [both[:, 0].view(k.dtype), both[:, 1].view(v.dtype)] + [s.to(dev) for s in stores[2:]]
+
+
+def _same(got, want, what=""):
+    for i, (a, b) in enumerate(zip(got, want)):
+        assert torch.equal(bits(a).cpu(), bits(b)), f"{what} store {i}"
+
+
+@pytest.mark.parametrize("kind,hkv,d", [("bf16", 2, 16), ("bf16", 8, 128), ("fp8:row", 8, 128), ("int8", 2, 64), ("fp8", 3, 20)])
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_compact_moves_accepted_paths_as_index_copy_of_index_select_does(kind, hkv, d, interleaved):
+    pk = kernels()
+    page, layers, rows = 16, 3, 5
+    tables, capacity, dump = _round_pool(page, 12, [(0, 80), (1, 190), (2, 100), (3, 64), (4, 33)], 6, seed=4)
+    slots = (dump + 1) * page
+    stores = _stores(kind, layers, slots, hkv, d, 5)
+    start = torch.tensor([30, 100, 7, 50, 20, 0])
+    emitted = torch.tensor([3, 6, 0, 9, 4, 0])
+    # row 0: the reference's own case (test_rounds.py:208); row 1: a deeper path; row 2 held; row 3: no tree, a
+    # permutation whose targets are later sources; row 4: moved already
+    path = torch.full((rows, 12), -1, dtype=torch.int64)
+    path[0, :3] = torch.tensor([0, 2, 5])
+    path[1, :6] = torch.tensor([0, 3, 4, 7, 10, 11])
+    path[2, :4] = torch.tensor([0, 1, 2, 3])
+    path[3, :9] = torch.tensor([0, 2, 1, 4, 3, 8, 7, 6, 5])
+    path[4, :4] = torch.tensor([0, 2, 4, 6])
+    moved = torch.tensor([0, 0, 0, 0, 1, 0])
+    for dtype in (torch.int64, torch.int32):
+        want = [s.clone() for s in stores]
+        want_moved = moved.clone()
+        oracle_pool.compact(want, slots, tables, capacity, start, emitted, path, want_moved, page, dump)
+        got = _on_device(stores, interleaved)
+        got_moved = moved.to(dev)
+        pk.compact(got, slots, tables.to(dev), capacity.to(dev), start.to(dev), emitted.to(dev), path.to(dtype).to(dev),
+                   got_moved, page, dump)
+        _same(got, want, f"path {dtype}")
+        assert got_moved.tolist() == want_moved.tolist() == [1, 1, 1, 1, 1, 0]
+        assert not torch.equal(bits(want[0]), bits(stores[0]))
+        # a second commit of the round finds the paths moved (test_rounds.py:211)
+        pk.compact(got, slots, tables.to(dev), capacity.to(dev), start.to(dev), emitted.to(dev), path.to(dtype).to(dev),
+                   got_moved, page, dump)
+        _same(got, want, "second commit")
+
+
+def test_compact_of_the_widest_path_and_of_sources_past_capacity():
+    pk = kernels()
+    page, layers = 16, 2
+    tables, capacity, dump = _round_pool(page, 40, [(0, 600), (1, 300)], 2, seed=6)
+    slots = (dump + 1) * page
+    stores = _stores("fp8:row", layers, slots, 8, 128, 7)
+    g = torch.Generator().manual_seed(8)
+    # 256 columns: a random increasing path (a tree's) in row 0; in row 1 every second accepted node lies past the
+    # slot's capacity, whose source is then the dump page's first slot
+    path = torch.full((2, 256), -1, dtype=torch.int64)
+    path[0] = torch.cat([torch.zeros(1, dtype=torch.int64), torch.sort(torch.randperm(330, generator=g)[:255] + 1).values])
+    path[1, :40] = torch.arange(40) * 2
+    path[1, 1:40:2] += 400
+    start, emitted, moved = torch.tensor([200, 100]), torch.tensor([256, 40]), torch.zeros(2, dtype=torch.int64)
+    want = [s.clone() for s in stores]
+    oracle_pool.compact(want, slots, tables, capacity, start, emitted, path, moved.clone(), page, dump)
+    got = [s.to(dev) for s in stores]
+    pk.compact(got, slots, tables.to(dev), capacity.to(dev), start.to(dev), emitted.to(dev), path.to(dev), moved.to(dev),
+               page, dump)
+    _same(got, want)
+    with pytest.raises(ValueError):
+        pk.compact(got, slots, tables.to(dev), capacity.to(dev), start.to(dev), emitted.to(dev),
+                   torch.zeros(2, 257, dtype=torch.int64, device=dev), moved.to(dev), page, dump)
+    with pytest.raises(ValueError):      # more rows than round slots
+        pk.compact(got, slots, tables.to(dev), capacity.to(dev), start.to(dev), emitted.to(dev),
+                   torch.zeros(3, 4, dtype=torch.int64, device=dev), moved.to(dev), page, dump)
+    with pytest.raises(ValueError):      # rows of 6 bytes
+        pk.compact([torch.zeros(layers, slots, 3, dtype=torch.bfloat16, device=dev)], slots, tables.to(dev), capacity.to(dev),
+                   start.to(dev), emitted.to(dev), path.to(dev), moved.to(dev), page, dump)
+
+
+@pytest.mark.parametrize("kind,hkv,d,page", [("bf16", 8, 128, 16), ("fp8:row", 8, 128, 16), ("int8", 2, 64, 4), ("fp16", 1, 6, 2)])
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_pages_are_copied_whole_in_every_layer_and_store(kind, hkv, d, page, interleaved):
+    pk = kernels()
+    pages, layers = 40, 3
+    stores = _stores(kind, layers, pages * page, hkv, d, 9)
+    source = torch.tensor([3, -1, 7, 39, 12, 3])
+    target = torch.tensor([0, 5, 9, 1, -1, 38])
+    want = [s.clone() for s in stores]
+    oracle_pool.copy_pages(want, pages * page, source, target, page)
+    got = _on_device(stores, interleaved)
+    pk.copy_pages(got, pages * page, source.to(dev), target.to(dev), page)
+    _same(got, want)
+    assert not torch.equal(bits(want[0]), bits(stores[0]))
+    pk.copy_pages(got, pages * page, source[:0].to(dev), target[:0].to(dev), page)
+    _same(got, want, "no pages")
+
+
+def test_a_decode_step_from_positions_on_the_device_replays_from_one_graph():
+    # The hot loop without the host (pages.py:646-660 and the step's kernels): slots of each row's next position from the
+    # bound tables, the token's keys and values appended there, attention over the row up to it, for two layers, captured
+    # once; every replay after the lengths moved on the device equals the same step launched eagerly, bit for bit, and
+    # the oracle over the pool as the eager launches left it.
+    from oracle import attend as oracle_attend
+    pk = kernels()
+    page, layers, hq, hkv, d, B = 16, 2, 8, 2, 128, 3
+    tables, capacity, dump = _round_pool(page, 32, [(0, 500), (1, 500), (2, 500)], 4, seed=10)
+    tables, capacity = tables.contiguous().to(dev), capacity.to(dev)
+    g = torch.Generator().manual_seed(11)
+
+    def fresh_pool():
+        g2 = torch.Generator().manual_seed(12)
+        k = (torch.randn(layers, dump + 1, page, hkv, d, generator=g2) * 0.5).bfloat16().to(dev)
+        v = (torch.randn(layers, dump + 1, page, hkv, d, generator=g2) * 0.5).bfloat16().to(dev)
+        return k, v
+    pools = {"graph": fresh_pool(), "eager": fresh_pool()}
+    lengths = torch.tensor([40, 333, 7], dtype=torch.int64, device=dev)
+    slot_ids = torch.arange(B, dtype=torch.int64, device=dev)
+    rows = torch.arange(B, dtype=torch.int32, device=dev)
+    starts = torch.arange(B, dtype=torch.int32, device=dev)
+    keys = torch.randn(layers, B, hkv, d, generator=g).bfloat16().to(dev)
+    values = torch.randn(layers, B, hkv, d, generator=g).bfloat16().to(dev)
+    q = torch.randn(layers, B, hq, d, generator=g).bfloat16().to(dev)
+    parts = pk.partitions(torch.device(dev), hkv, "bf16")
+    workspace = torch.empty(pk.workspace_floats(B, hq, parts, d), dtype=torch.float32, device=dev)
+
+    def step(which, slots, out):
+        k, v = pools[which]
+        pk.slots_at(tables, capacity, slot_ids, lengths, page, dump, out=slots)
+        for layer in range(layers):
+            pk.write(keys[layer], values[layer], slots, k[layer], v[layer], "bf16")
+            pk.attend(q[layer], k[layer], v[layer], "bf16", tables, rows, starts, lengths, 1, page, out=out[layer],
+                      workspace=workspace)
+    slots_g, out_g = torch.empty(B, dtype=torch.int64, device=dev), torch.empty(layers, B, hq, d, dtype=torch.bfloat16, device=dev)
+    slots_e, out_e = torch.empty_like(slots_g), torch.empty_like(out_g)
+    step("graph", slots_g, out_g)      # (the first launches on a device look addresses up: outside the capture)
+    torch.cuda.synchronize()
+    pools["graph"] = fresh_pool()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step("graph", slots_g, out_g)
+    pools["graph"][0].copy_(pools["eager"][0]), pools["graph"][1].copy_(pools["eager"][1])
+    for n in range(6):
+        graph.replay()
+        torch.cuda.synchronize()
+        step("eager", slots_e, out_e)
+        torch.cuda.synchronize()
+        assert torch.equal(slots_g, slots_e), n
+        assert torch.equal(out_g, out_e), n
+        assert torch.equal(pools["graph"][0], pools["eager"][0]) and torch.equal(pools["graph"][1], pools["eager"][1]), n
+        at = lengths.tolist()
+        want_slots = [int(tables[s, p // page]) * page + p % page for s, p in enumerate(at)]
+        assert slots_g.tolist() == want_slots
+        k_cpu, v_cpu = pools["eager"][0][1].cpu(), pools["eager"][1][1].cpu()
+        for s in range(B):
+            want, _ = oracle_attend.window_reference(q[1, s:s + 1].float().cpu(), k_cpu, v_cpu, "bf16", tables[s].cpu(), at[s], 1,
+                                                     page, d ** -0.5)
+            torch.testing.assert_close(out_g[1, s:s + 1].double().cpu(), want, atol=2e-2, rtol=2e-2)
+        lengths += torch.tensor([1, 16, 3], device=dev)      # the sequences grow on the device

@@ -481,3 +481,118 @@ def test_int8_query_rows_are_their_codes_times_their_scale():
     for c in range(3):
         want, want_lse = attend.reference(attend.int8_rows(q[c].bfloat16()), keys, values, torch.arange(60) <= 57 + c, 0.25)
         assert torch.allclose(out[c], want, atol=1e-12) and torch.allclose(lse[c], want_lse, atol=1e-12)
+
+
+# -- the pool's device-side bookkeeping ------------------------------------------------------------------------------------
+def _round_pool(page=4, table_pages=6, lengths=((0, 17), (1, 9), (3, 24)), round_slots=4, seed=0):
+    """Round tables of a few bound sequences over shuffled pages; unbound slots and the entries past a sequence's pages
+    at the dump page (test_rounds.py:52-54)."""
+    g = torch.Generator().manual_seed(seed)
+    pages = round_slots * table_pages
+    order = torch.randperm(pages, generator=g).tolist()
+    tables = torch.full((round_slots, table_pages), pages, dtype=torch.int32)
+    capacity = torch.zeros(round_slots, dtype=torch.int64)
+    for s, n in lengths:
+        held = -(-n // page)
+        tables[s, :held] = torch.tensor([order.pop() for _ in range(held)], dtype=torch.int32)
+        capacity[s] = n
+    return tables, capacity, pages
+
+
+def test_slots_at_is_the_closed_form_inside_a_slots_capacity_and_the_dump_page_outside():
+    from oracle import pool
+    page = 4
+    tables, capacity, dump = _round_pool(page)
+    slot = torch.tensor([[0, 0, 0, 0], [1, 1, 1, 1], [2, 2, 3, 3]])
+    where = torch.tensor([[0, 5, 16, 17], [8, 9, -1, 400], [0, 3, 23, 24]])
+    got = pool.slots_at(tables, capacity, slot, where, page, dump)
+    for s, p, found in zip(slot.reshape(-1).tolist(), where.reshape(-1).tolist(), got.reshape(-1).tolist()):
+        if 0 <= p < int(capacity[s]):
+            assert found == int(tables[s, p // page]) * page + p % page      # test_rounds.py:34-36
+        else:
+            assert found == dump * page      # past capacity, before 0, an unbound slot: test_rounds.py:58-60, 289
+    inside = got[(where >= 0) & (where < capacity[slot])]
+    assert len(set(inside.tolist())) == inside.numel() and int(inside.max()) < dump * page
+    # a round's reserve: each token's row's slot first (pages.py:652-653)
+    slots_t, rows_t = torch.tensor([3, 0]), torch.tensor([0, 0, 1, 1, 1])
+    positions = torch.tensor([22, 23, 15, 16, 17])
+    got = pool.reserve_round(tables, capacity, slots_t, rows_t, positions, page, dump).tolist()
+    want = [int(tables[3, 5]) * 4 + 2, int(tables[3, 5]) * 4 + 3, int(tables[0, 3]) * 4 + 3, int(tables[0, 4]) * 4, dump * 4]
+    assert got == want
+
+
+def _sequence_rows(store, table, positions, page):
+    at = torch.tensor([int(table[p // page]) * page + p % page for p in positions])
+    return store[:, at]
+
+
+def test_compact_moves_an_accepted_path_to_consecutive_positions_once():
+    from oracle import pool
+    page, layers = 4, 2
+    # one sequence of 30 tokens bound with room for 80 (test_rounds.py:190-215): a window of 6 at 30, the nodes 0, 2
+    # and 5 accepted
+    tables, capacity, dump = _round_pool(page, table_pages=20, lengths=((0, 80),), round_slots=2)
+    slots = (dump + 1) * page
+    g = torch.Generator().manual_seed(1)
+    keys = torch.randn(layers, slots, 2, 16, generator=g).bfloat16()
+    scales = torch.rand(layers, slots, 2, generator=g)
+    before_k, before_s = keys.clone(), scales.clone()
+    start, emitted, moved = torch.tensor([30, 0]), torch.tensor([3, 0]), torch.zeros(2, dtype=torch.int64)
+    path = torch.tensor([[0, 2, 5, -1, -1, -1]])
+    pool.compact([keys, None, scales], slots, tables, capacity, start, emitted, path, moved, page, dump)
+    for now, was in ((keys, before_k), (scales, before_s)):
+        got, old = _sequence_rows(now, tables[0], range(36), page), _sequence_rows(was, tables[0], range(36), page)
+        assert torch.equal(got[:, :30], old[:, :30])
+        assert torch.equal(got[:, 30:33], old[:, [30, 32, 35]])
+        assert torch.equal(got[:, 33:], old[:, 33:])      # what lies past the new frontier is left as it was
+    assert moved.tolist() == [1, 0]
+    again = keys.clone()
+    pool.compact([keys, None, scales], slots, tables, capacity, start, emitted, path, moved, page, dump)
+    assert torch.equal(keys, again)      # a second commit finds the path moved (test_rounds.py:211)
+    # a held row (nothing emitted) moves nothing
+    moved.zero_()
+    pool.compact([keys], slots, tables, capacity, start, torch.tensor([0, 0]), path, moved, page, dump)
+    assert torch.equal(keys, again)
+
+
+def test_compact_reads_every_source_before_it_writes_a_target():
+    from oracle import pool
+    # path [0, 1, 3, 2 ...] would be no tree, but the rule is index_copy_(index_select()): position 2 is column 2's
+    # target and column 3's source, and column 3 must still deliver position 2's old row. A model that moves one row
+    # after the other in column order delivers the new one and must differ.
+    page = 4
+    tables, capacity, dump = _round_pool(page, table_pages=8, lengths=((0, 30), (1, 30)), round_slots=2)
+    slots = (dump + 1) * page
+    values = torch.arange(slots, dtype=torch.float32).view(1, slots, 1).repeat(1, 1, 3).contiguous()
+    before = values.clone()
+    start, emitted, moved = torch.tensor([8, 5]), torch.tensor([4, 3]), torch.zeros(2, dtype=torch.int64)
+    path = torch.tensor([[0, 1, 3, 2, 4], [0, 4, 1, 3, -1]])
+    pool.compact([values], slots, tables, capacity, start, emitted, path, moved, page, dump)
+    old0 = _sequence_rows(before, tables[0], range(14), page)
+    got0 = _sequence_rows(values, tables[0], range(14), page)
+    assert torch.equal(got0[:, 8:12], old0[:, [8, 9, 11, 10]])
+    assert torch.equal(got0[:, 12:], old0[:, 12:])
+    old1 = _sequence_rows(before, tables[1], range(10), page)
+    got1 = _sequence_rows(values, tables[1], range(10), page)
+    assert torch.equal(got1[:, 5:8], old1[:, [5, 9, 6]])      # column 3 lies at emitted: not moved
+    assert torch.equal(got1[:, 8:], old1[:, 8:])
+    one_by_one = before.clone()
+    for j, node in ((1, 1), (2, 3), (3, 2)):
+        src, dst = int(tables[0, (8 + node) // 4]) * 4 + (8 + node) % 4, int(tables[0, (8 + j) // 4]) * 4 + (8 + j) % 4
+        one_by_one[:, dst] = one_by_one[:, src]
+    assert not torch.equal(_sequence_rows(one_by_one, tables[0], range(14), page), got0)
+
+
+def test_copy_pages_copies_whole_pages_in_every_layer_and_store():
+    from oracle import pool
+    page, pages, layers = 4, 10, 3
+    g = torch.Generator().manual_seed(2)
+    keys = torch.randn(layers, pages * page, 2, 8, generator=g)
+    codes = torch.randint(0, 255, (layers, pages * page, 2, 8), generator=g, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    before_k, before_c = keys.clone(), codes.clone()
+    pool.copy_pages([keys, codes], pages * page, torch.tensor([3, -1, 7]), torch.tensor([0, 5, 9]), page)
+    for now, was in ((keys, before_k), (codes.view(torch.uint8), before_c.view(torch.uint8))):
+        paged, old = now.view(layers, pages, -1), was.view(layers, pages, -1)
+        assert torch.equal(paged[:, 0], old[:, 3]) and torch.equal(paged[:, 9], old[:, 7])
+        rest = [1, 2, 3, 4, 5, 6, 7, 8]
+        assert torch.equal(paged[:, rest], old[:, rest])
