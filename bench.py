@@ -372,6 +372,68 @@ def prefill_by_kind(pk, device):
     return found
 
 
+def pool_bookkeeping(pk, device):
+    """The pool's device-side bookkeeping at the 8B shape (32 layers, 8 KV heads x 128, page 16, bf16): a decode step's
+    slots, a draft-tree round's move of accepted rows (64 rows, 5 of 8 columns emitted), and copies of 256 shared pages;
+    the torch indexing the reference runs for the last two (pages.py:676-683, 861-869) timed beside them. Bytes are those
+    read plus those written."""
+    layers, hkv, d, page, pages, B, width = 32, 8, 128, 16, 4096, 64, 8
+    g = torch.Generator(device=device).manual_seed(5)
+    slots = (pages + 1) * page
+    k = torch.randn(layers, slots, hkv, d, device=device, generator=g).to(torch.bfloat16)
+    v = torch.randn(layers, slots, hkv, d, device=device, generator=g).to(torch.bfloat16)
+    table_pages = pages // B
+    tables = torch.randperm(pages, device=device, generator=g).to(torch.int32).view(B, table_pages).contiguous()
+    capacity = torch.full((B,), table_pages * page, dtype=torch.int64, device=device)
+    lengths = torch.randint(100, 900, (B,), device=device, generator=g)
+    slot_ids = torch.arange(B, device=device)
+    found = {}
+    out = torch.empty(B, dtype=torch.int64, device=device)
+    ms = timed(lambda: pk.slots_at(tables, capacity, slot_ids, lengths, page, pages, out=out), 50, 3)
+    found["slots_at_64_positions_us"] = round(ms * 1e3, 2)
+    many = torch.randint(0, table_pages * page, (4152,), device=device, generator=g)
+    rows = torch.randint(0, B, (4152,), device=device, generator=g)
+    ms = timed(lambda: pk.slots_at(tables, capacity, slot_ids, many, page, pages, rows=rows), 50, 3)
+    found["slots_at_4152_positions_us"] = round(ms * 1e3, 2)
+    path = torch.tensor([0, 2, 3, 5, 6, -1, -1, -1], device=device).repeat(B, 1)
+    emitted = torch.full((B,), 5, dtype=torch.int64, device=device)
+    moved = torch.zeros(B, dtype=torch.int64, device=device)
+
+    def compact():
+        moved.zero_()
+        pk.compact([k, v], slots, tables, capacity, lengths, emitted, path, moved, page, pages)
+    nbytes = B * 4 * hkv * d * 2 * layers * 2 * 2
+    ms = timed(compact, 20, 3)
+    found["compact_64_rows_4_moves"] = {"us": round(ms * 1e3, 2), "GB/s": round(nbytes / ms / 1e6, 1)}
+    columns = torch.arange(width, device=device)
+    keep = (columns[None, :] < emitted[:, None]) & (columns[None, :] > 0) & (path >= 0)
+    where = lambda p: pk.slots_at(tables, capacity, slot_ids[:, None].expand(B, width).contiguous(), p.contiguous(), page, pages)
+    source = where(torch.where(keep, lengths[:, None] + path, -1)).reshape(-1)
+    target = where(torch.where(keep, lengths[:, None] + columns[None, :], -1)).reshape(-1)
+
+    def torch_compact():
+        for flat in (k, v):
+            flat.index_copy_(1, target, flat.index_select(1, source))
+    ms = timed(torch_compact, 5, 1)
+    found["compact_64_rows_4_moves"]["torch_indexing_us"] = round(ms * 1e3, 2)
+    n = 256
+    ids = torch.randperm(pages, device=device, generator=g)
+    source, target = ids[:n].contiguous(), ids[n:2 * n].contiguous()
+    nbytes = n * page * hkv * d * 2 * layers * 2 * 2
+    ms = timed(lambda: pk.copy_pages([k, v], slots, source, target, page), 20, 3)
+    found["copy_256_pages"] = {"us": round(ms * 1e3, 2), "GB/s": round(nbytes / ms / 1e6, 1)}
+    kp, vp = k.view(layers, pages + 1, page, hkv, d), v.view(layers, pages + 1, page, hkv, d)
+    pairs = list(zip(source.tolist(), target.tolist()))
+
+    def torch_copies():
+        for a, b in pairs:
+            kp[:, b].copy_(kp[:, a])
+            vp[:, b].copy_(vp[:, a])
+    ms = timed(torch_copies, 3, 1)
+    found["copy_256_pages"]["torch_page_by_page_us"] = round(ms * 1e3, 2)
+    return found
+
+
 def prefill_fresh(pk, device):
     """The mixed batch's 8 prompt chunks over FP8 pages (one multiplier pair), once reading every position from the
     pages and once with fresh=: each chunk's own 512 positions from 16-bit rows as the projections gave them, its
@@ -419,6 +481,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the mixed prefill + decode batch of the extras (for counter runs on prefill_kernel)")
+    ap.add_argument("--pool-only", action="store_true",
+                    help="run only the pool bookkeeping of the extras (slots, the move of accepted rows, page copies)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch one KV append of 262,144 tokens: with the stream-read probe, two kernels of known "
                          "read and write sizes against which FETCH_SIZE / WRITE_SIZE counters are scaled")
@@ -434,6 +498,11 @@ def main():
         found = mixed_prefill(pk, device)
         log(f"[bench] mixed prefill + decode: {found}")
         print(json.dumps({"mixed_prefill_decode_bf16": found}), flush=True)
+        return
+    if args.pool_only:
+        found = pool_bookkeeping(pk, device)
+        log(f"[bench] pool bookkeeping: {found}")
+        print(json.dumps({"pool_bookkeeping_bf16": found}), flush=True)
         return
     spec = WORKLOADS[args.workload]
     log(f"[bench] building workload {args.workload}: {spec['name']}")
@@ -527,6 +596,9 @@ def main():
         log(f"[bench] prefill over 8-bit pages: {extras['prefill_8bit_pages']}")
         extras["prefill_fp8_pages_fresh_rows"] = prefill_fresh(pk, device)
         log(f"[bench] prefill over FP8 pages, with fresh rows: {extras['prefill_fp8_pages_fresh_rows']}")
+        torch.cuda.empty_cache()
+        extras["pool_bookkeeping_bf16"] = pool_bookkeeping(pk, device)
+        log(f"[bench] pool bookkeeping: {extras['pool_bookkeeping_bf16']}")
         result["extra"] = extras
     if not args.no_cpu:
         log("[bench] timing the CPU reference path (about 20 s)")

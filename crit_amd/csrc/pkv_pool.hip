@@ -7,6 +7,8 @@
 namespace pkv {
 namespace {
 
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
+
 struct Tables {
     const int32_t* tables;
     const int64_t* capacity;
@@ -43,7 +45,7 @@ struct Stores {
     int wide[CRIT_PKV_MAX_STORES];      // the store moves 16 bytes a lane (its base, stride and unit allow it), else 4
 };
 
-constexpr int kStageBytes = 32768;
+constexpr int kStageBytes = 16384;      // (with the lists: six workgroups a compute unit)
 
 // One workgroup: one round row, one layer, one store. The kept columns' source and target slots are listed first; then
 // the rows move through LDS a slice of their bytes at a time, every source of the slice read before a target is
@@ -75,8 +77,7 @@ __global__ __launch_bounds__(256) void compact_kernel(Tables t, Stores stores, c
                                                       const void* path, int path_is_32, int64_t path_stride, int width,
                                                       const int64_t* moved) {
     __shared__ int64_t s_src[CRIT_PKV_MAX_PATH], s_dst[CRIT_PKV_MAX_PATH];
-    __shared__ int s_keep[CRIT_PKV_MAX_PATH];
-    __shared__ int s_n;
+    __shared__ int s_kept[4];
     __shared__ uint4 stage[kStageBytes / sizeof(uint4)];
     const int tid = threadIdx.x;
     const int64_t r = blockIdx.x;
@@ -95,15 +96,16 @@ __global__ __launch_bounds__(256) void compact_kernel(Tables t, Stores stores, c
             dst = slot_at(t, r, first + tid);
         }
     }
-    s_keep[tid] = keep;
+    // (a column's place in the list: the kept columns before it, counted a wavefront at a time)
+    const unsigned long long kept = __ballot(keep);
+    const int lane = tid & 63, wave = tid >> 6;
+    if (lane == 0) s_kept[wave] = __popcll(kept);
     __syncthreads();
-    // (a column's place in the list: the kept columns before it)
-    int at = 0;
-    for (int j = 0; j < tid; ++j) at += s_keep[j];
+    int at = __popcll(kept & ((1ull << lane) - 1ull));
+    for (int w = 0; w < wave; ++w) at += s_kept[w];
     if (keep) s_src[at] = src, s_dst[at] = dst;
-    if (tid == 255) s_n = at + keep;
+    const int n = s_kept[0] + s_kept[1] + s_kept[2] + s_kept[3];
     __syncthreads();
-    const int n = s_n;
     if (n == 0) return;
     uint8_t* base = reinterpret_cast<uint8_t*>(st.base) + (int64_t)layer * st.layer_stride;
     if (stores.wide[blockIdx.z])
@@ -124,16 +126,16 @@ __device__ __forceinline__ void copy_piece(uint8_t* base, int64_t page_bytes, in
     G* dst = reinterpret_cast<G*>(base + to * page_bytes);
     const int64_t total = page_bytes / (int64_t)sizeof(G);
     const int64_t lo = (int64_t)piece * 1024;
-    G held[4];
+    G held[4];      // (read once, written once: nontemporal both ways, the caches keep neither)
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const int64_t i = lo + k * 256 + threadIdx.x;
-        if (i < total) held[k] = src[i];
+        if (i < total) held[k] = __builtin_nontemporal_load(src + i);
     }
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const int64_t i = lo + k * 256 + threadIdx.x;
-        if (i < total) dst[i] = held[k];
+        if (i < total) __builtin_nontemporal_store(held[k], dst + i);
     }
 }
 
@@ -145,7 +147,7 @@ __global__ __launch_bounds__(256) void copy_pages_kernel(Stores stores, const in
     if (from < 0 || to < 0) return;
     uint8_t* base = reinterpret_cast<uint8_t*>(st.base) + (int64_t)blockIdx.y * st.layer_stride;
     if (stores.wide[blockIdx.z])
-        copy_piece<uint4>(base, st.row_bytes * page, from, to, piece);
+        copy_piece<u32x4>(base, st.row_bytes * page, from, to, piece);
     else
         copy_piece<uint32_t>(base, st.row_bytes * page, from, to, piece);
 }
