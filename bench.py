@@ -431,6 +431,20 @@ def pool_bookkeeping(pk, device):
             vp[:, b].copy_(vp[:, a])
     ms = timed(torch_copies, 3, 1)
     found["copy_256_pages"]["torch_page_by_page_us"] = round(ms * 1e3, 2)
+    # rows read back (KVPool.gather / rows_at): 262,144 rows of one layer at random slots, bf16 pages to bf16 and FP8
+    # pages to bf16 and FP32; bytes read + written
+    del kp, vp, v
+    n = 262144
+    where = torch.randint(0, slots, (n,), device=device, generator=g)
+    k16, v16 = k[0], k[1]
+    k8, v8 = k[2].view(torch.float8_e4m3fn)[:, :, :d].contiguous(), k[3].view(torch.float8_e4m3fn)[:, :, :d].contiguous()
+    for name, kk, vv, kind, e, dtype in (("bf16_to_bf16", k16, v16, "bf16", 2, torch.bfloat16),
+                                         ("fp8_to_bf16", k8, v8, "fp8", 1, torch.bfloat16),
+                                         ("fp8_to_fp32", k8, v8, "fp8", 1, torch.float32)):
+        out = (torch.empty(n, hkv, d, dtype=dtype, device=device), torch.empty(n, hkv, d, dtype=dtype, device=device))
+        ms = timed(lambda: pk.rows_at(kk, vv, kind, where, multipliers=(0.02, 0.03), dtype=dtype, out=out), 20, 3)
+        nbytes = n * hkv * 2 * d * (e + out[0].element_size())
+        found[f"rows_at_262144_{name}"] = {"us": round(ms * 1e3, 2), "GB/s": round(nbytes / ms / 1e6, 1)}
     return found
 
 

@@ -31,6 +31,10 @@ int crit_pkv_copy_pages(const crit_pkv_copy_pages_params* p, void* stream) {
     return pkv::launch_copy_pages(p, reinterpret_cast<hipStream_t>(stream));
 }
 
+int crit_pkv_read_rows(const crit_pkv_read_params* p, void* stream) {
+    return pkv::launch_read_rows(p, reinterpret_cast<hipStream_t>(stream));
+}
+
 int crit_pkv_stream_read(const void* data, int64_t bytes, float* sink, void* stream) {
     return pkv::launch_stream_read(data, bytes, sink, reinterpret_cast<hipStream_t>(stream));
 }
@@ -46,6 +50,7 @@ int crit_pkv_params_size(int which) {
         case 4: return (int)sizeof(crit_pkv_slots_params);
         case 5: return (int)sizeof(crit_pkv_compact_params);
         case 6: return (int)sizeof(crit_pkv_copy_pages_params);
+        case 7: return (int)sizeof(crit_pkv_read_params);
     }
     return -1;
 }

@@ -35,7 +35,7 @@ from . import _abi
 __all__ = ["KINDS", "PIECE", "MAX_COLUMNS", "Derive", "attend", "derive", "cuda_block", "cuda_chunk", "cuda_parts",
            "cuda_prompt", "cuda_ramp", "cuda_splits", "flash_block", "flash_chunk", "flash_parts", "flash_tile",
            "merge_shards", "owner", "partitions", "piece_size", "prefill", "prefill_rows", "prefill_state_floats", "release",
-           "stream_read", "slots_at", "compact", "copy_pages",
+           "stream_read", "slots_at", "compact", "copy_pages", "rows_at", "gather",
            "tile_for", "workspace_floats", "write"]
 
 KINDS = {"bf16": 0, "fp16": 0, "fp8": 1, "fp8:row": 2, "int8": 3}
@@ -773,3 +773,63 @@ def copy_pages(stores, slots, source, target, page):
     p.source, p.target, p.n, p.page = source.data_ptr(), target.data_ptr(), source.numel(), int(page)
     with torch.cuda.device(device):
         _abi.check(_abi.load().crit_pkv_copy_pages(p, _stream(device)), "paged_kv_attention.copy_pages")
+
+
+# -- rows read back (reference: inference/attention-state/code/pages.py:455-493) -----------------------------------------
+def _read(key_pages, value_pages, kind, n, shape, dtype, key_scales, value_scales, multipliers, slots=None, table=None,
+          page=0, out=None):
+    k_kind = _check_kind(kind, key_scales)
+    _require_device(key_pages, "the key pages")
+    device = key_pages.device
+    if dtype not in _DTYPE:
+        raise ValueError("rows are read back as float32, bfloat16 or float16")
+    if key_pages.dim() < 2 or not key_pages.is_contiguous() or (value_pages is not None and (
+            not value_pages.is_contiguous() or value_pages.device != device or value_pages.shape[-2] != key_pages.shape[-2])):
+        raise ValueError("pages are contiguous [...][kv_heads][dim] on one device")
+    hkv, d = key_pages.shape[-2], key_pages.shape[-1]
+    dv = 0 if value_pages is None else value_pages.shape[-1]
+    if d % 8 or dv % 8:
+        raise ValueError("head widths are multiples of 8")
+    km, vm, heads = _multipliers(multipliers, hkv, device)
+    if out is None:
+        out = (torch.empty(*shape, hkv, d, dtype=dtype, device=device),
+               None if value_pages is None else torch.empty(*shape, hkv, dv, dtype=dtype, device=device))
+    else:
+        for o, width in zip(out, (d, dv)):
+            if o is not None and (o.dtype != dtype or o.device != device or not o.is_contiguous() or
+                                  o.numel() != n * hkv * width):
+                raise ValueError("out holds (keys, values) [n][kv_heads][dim], contiguous, in the dtype asked for")
+    p = _abi.ReadParams()
+    p.key_pages, p.value_pages, p.key_scales, p.value_scales = key_pages.data_ptr(), _ptr(value_pages), _ptr(key_scales), _ptr(value_scales)
+    p.head_multipliers, p.slots = _ptr(heads), _ptr(slots)
+    if table is not None:
+        p.table, p.table64 = (table.data_ptr(), None) if table.dtype == torch.int32 else (None, table.data_ptr())
+    p.out_keys, p.out_values, p.n = out[0].data_ptr(), _ptr(out[1]), n
+    p.kv_heads, p.head_dim, p.value_dim, p.page, p.kind = hkv, d, dv, int(page), k_kind
+    p.page_dtype, p.out_dtype, p.key_multiplier, p.value_multiplier = _page_dtype(key_pages, kind), _DTYPE[dtype], km, vm
+    with torch.cuda.device(device):
+        _abi.check(_abi.load().crit_pkv_read_rows(p, _stream(device)), "paged_kv_attention.rows_at")
+    return out
+
+
+def rows_at(key_pages, value_pages, kind, slots, *, key_scales=None, value_scales=None, multipliers=(1.0, 1.0),
+            dtype=torch.float32, out=None):
+    """The keys and values at `slots` (any shape, int64, on the device) dequantised: KVPool.rows_at (pages.py:479-493)
+    in one launch: float(stored) * the layer's multiplier or the row's scale, one FP32 product, in `dtype` (FP32 as the
+    reference's). A negative slot reads as zeros. value_pages None: keys only. Returns (keys [..., kv_heads, dim],
+    values)."""
+    if not torch.is_tensor(slots) or slots.dtype != torch.int64 or slots.device != key_pages.device or not slots.is_contiguous():
+        raise ValueError("slots are a contiguous int64 tensor on the pages' device")
+    return _read(key_pages, value_pages, kind, slots.numel(), tuple(slots.shape), dtype, key_scales, value_scales,
+                 multipliers, slots=slots, out=out)
+
+
+def gather(key_pages, value_pages, kind, table, count, page, *, key_scales=None, value_scales=None,
+           multipliers=(1.0, 1.0), dtype=torch.bfloat16, out=None):
+    """A sequence's first `count` positions as contiguous rows in the compute dtype, dequantised: KVPool.gather
+    (pages.py:455-477) in one launch; table [ceil(count / page) or more] int32 or int64 on the device."""
+    if not torch.is_tensor(table) or table.dtype not in (torch.int32, torch.int64) or table.device != key_pages.device or \
+            table.dim() != 1 or not table.is_contiguous() or table.numel() * page < count or count < 0 or page < 1:
+        raise ValueError("a page table is a contiguous int32 or int64 tensor on the pages' device that covers `count` positions")
+    return _read(key_pages, value_pages, kind, int(count), (int(count),), dtype, key_scales, value_scales, multipliers,
+                 table=table, page=page, out=out)

@@ -10,7 +10,7 @@ import shutil
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 NAME = "libcrit_pkv.so"
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 KIND_16BIT, KIND_FP8, KIND_FP8_ROW, KIND_INT8 = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
@@ -87,8 +87,15 @@ class CopyPagesParams(ctypes.Structure):
                 ("n_stores", _i32), ("layers", _i32), ("page", _i32)]
 
 
+class ReadParams(ctypes.Structure):
+    _fields_ = [("key_pages", _p), ("value_pages", _p), ("key_scales", _p), ("value_scales", _p), ("head_multipliers", _p),
+                ("slots", _p), ("table", _p), ("table64", _p), ("out_keys", _p), ("out_values", _p), ("n", _i64),
+                ("kv_heads", _i32), ("head_dim", _i32), ("value_dim", _i32), ("page", _i32), ("kind", _i32),
+                ("page_dtype", _i32), ("out_dtype", _i32), ("key_multiplier", _f32), ("value_multiplier", _f32)]
+
+
 SYMBOLS = ("crit_pkv_write", "crit_pkv_attend", "crit_pkv_merge", "crit_pkv_prefill", "crit_pkv_slots_at",
-           "crit_pkv_compact", "crit_pkv_copy_pages", "crit_pkv_abi_version", "crit_pkv_params_size", "crit_pkv_error",
+           "crit_pkv_compact", "crit_pkv_copy_pages", "crit_pkv_read_rows", "crit_pkv_abi_version", "crit_pkv_params_size", "crit_pkv_error",
            "crit_pkv_stream_read")
 
 _lib = None
@@ -136,7 +143,7 @@ def load():
     for name, struct in (("crit_pkv_write", WriteParams), ("crit_pkv_attend", AttendParams),
                          ("crit_pkv_merge", MergeParams), ("crit_pkv_prefill", PrefillParams),
                          ("crit_pkv_slots_at", SlotsParams), ("crit_pkv_compact", CompactParams),
-                         ("crit_pkv_copy_pages", CopyPagesParams)):
+                         ("crit_pkv_copy_pages", CopyPagesParams), ("crit_pkv_read_rows", ReadParams)):
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(struct), ctypes.c_void_p]
@@ -145,7 +152,7 @@ def load():
     if lib.crit_pkv_abi_version() != ABI_VERSION:
         raise RuntimeError(f"{path} speaks ABI {lib.crit_pkv_abi_version()}, this package {ABI_VERSION}: rebuild it")
     for which, struct in enumerate((WriteParams, AttendParams, MergeParams, PrefillParams, SlotsParams, CompactParams,
-                                    CopyPagesParams)):
+                                    CopyPagesParams, ReadParams)):
         if lib.crit_pkv_params_size(which) != ctypes.sizeof(struct):
             raise RuntimeError(f"{path}: parameter struct {which} is {lib.crit_pkv_params_size(which)} bytes, the "
                                f"Python mirror {ctypes.sizeof(struct)}: rebuild the library")

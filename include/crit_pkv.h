@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 6
+#define CRIT_PKV_ABI_VERSION 7
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -270,10 +270,35 @@ typedef struct crit_pkv_copy_pages_params {
 
 int crit_pkv_copy_pages(const crit_pkv_copy_pages_params* p, void* stream);
 
+/* ---- rows read back ----------------------------------------------------------------------------------------------
+ * Replaces the index_select, cast and multiply of KVPool.gather and KVPool.rows_at (pages.py:455-493): row i of the
+ * output is the pool's row at slots[i], or, with a page table instead (exactly one of slots, table, table64), at
+ * table[i / page] * page + i % page (a sequence's first n positions); value = float(stored) * scale in FP32 (the
+ * layer's multiplier, or the row's scale), rounded once to out_dtype. A negative slot reads as zeros. out_keys
+ * [n][kv_heads][head_dim], out_values [n][kv_heads][value_dim], contiguous; value_pages / out_values NULL: keys only.
+ * Head widths are multiples of 8. */
+typedef struct crit_pkv_read_params {
+    const void* key_pages;
+    const void* value_pages;
+    const float* key_scales;        /* kinds FP8_ROW and INT8 */
+    const float* value_scales;
+    const float* head_multipliers;  /* optional [2][kv_heads], kind FP8 */
+    const int64_t* slots;           /* [n] */
+    const int32_t* table;           /* [ceil(n / page)] */
+    const int64_t* table64;
+    void* out_keys;
+    void* out_values;
+    int64_t n;
+    int32_t kv_heads, head_dim, value_dim, page, kind, page_dtype, out_dtype;
+    float key_multiplier, value_multiplier;
+} crit_pkv_read_params;
+
+int crit_pkv_read_rows(const crit_pkv_read_params* p, void* stream);
+
 /* ---- housekeeping ------------------------------------------------------------------------------------------------- */
 int crit_pkv_abi_version(void);
 /* sizeof() of the parameter structs as the library was compiled, for the host's mirror to cross-check
- * (which: 0 write, 1 attend, 2 merge, 3 prefill, 4 slots_at, 5 compact, 6 copy_pages), as crit_cw_params_size() does (cuda_window.cu:1502). */
+ * (which: 0 write, 1 attend, 2 merge, 3 prefill, 4 slots_at, 5 compact, 6 copy_pages, 7 read_rows), as crit_cw_params_size() does (cuda_window.cu:1502). */
 int crit_pkv_params_size(int which);
 const char* crit_pkv_error(int code);
 /* A streaming-read probe: sums `bytes` (a multiple of 16) of device memory into sink[0..63]; the achievable-HBM-read

@@ -144,6 +144,22 @@ def gather(key_pages, value_pages, table, count, page, kind, compute, key_scales
     return k.to(compute), v.to(compute)
 
 
+def rows_at(key_pages, value_pages, slots, kind, key_scales=None, value_scales=None, multipliers=(1.0, 1.0)):
+    """The keys and values at `slots` (any shape, int64) dequantised to FP32 (pages.py:479-493): index_select of the
+    rows, .float(), times the layer's multiplier (fp8) or the row's scale. Pages [pages][page][HKV][dim]."""
+    hkv, d, dv = key_pages.shape[-2], key_pages.shape[-1], value_pages.shape[-1]
+    flat = slots.reshape(-1)
+    k = key_pages.reshape(-1, hkv, d).index_select(0, flat).float()
+    v = value_pages.reshape(-1, hkv, dv).index_select(0, flat).float()
+    if kind == "fp8":
+        k, v = k * multipliers[0], v * multipliers[1]
+    elif kind in append.ROW_SCALED:
+        k = k * key_scales.reshape(-1, hkv).index_select(0, flat)[..., None]
+        v = v * value_scales.reshape(-1, hkv).index_select(0, flat)[..., None]
+    shape = tuple(slots.shape)
+    return k.view(*shape, hkv, d), v.view(*shape, hkv, dv)
+
+
 def sdpa_rows(queries, rows, gather_row, scale, out):
     """The reference's CPU attention path (device_attention.py:1148-1166): per batch row (first token, count, first
     position) gather its KV with gather_row(r, n) and run torch's scaled_dot_product_attention with GQA; one token sees

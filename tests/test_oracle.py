@@ -596,3 +596,47 @@ def test_copy_pages_copies_whole_pages_in_every_layer_and_store():
         assert torch.equal(paged[:, 0], old[:, 3]) and torch.equal(paged[:, 9], old[:, 7])
         rest = [1, 2, 3, 4, 5, 6, 7, 8]
         assert torch.equal(paged[:, rest], old[:, rest])
+
+
+# -- rows read back ------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("kind", ["bf16", "fp16", "fp8", "fp8:row", "int8"])
+def test_rows_read_back_are_the_codes_times_their_scale_one_fp32_product(kind):
+    # Pins rows_at() and gather(): each element against the closed-form decoder (e4m3.decode: every code's value from
+    # its bit fields) or the integer code, times the scale as one IEEE FP32 product (numpy float32, no torch); gather of
+    # a sequence's first positions is rows_at of the slots its table gives (the slot closed form), in the compute dtype.
+    g = torch.Generator().manual_seed(21)
+    pages, page, hkv, d = 9, 4, 2, 8
+    slots_n = pages * page
+    ks = vs = None
+    if kind in ("bf16", "fp16"):
+        k = torch.randn(pages, page, hkv, d, generator=g).to(append.STORAGE[kind])
+        v = torch.randn(pages, page, hkv, d, generator=g).to(append.STORAGE[kind])
+    else:
+        raw = lambda: torch.randint(0, 256, (pages, page, hkv, d), generator=g, dtype=torch.uint8)
+        k, v = raw(), raw()
+        k[k == 0x7f], k[k == 0xff], v[v == 0x7f], v[v == 0xff] = 0, 0, 0, 0      # (E4M3's NaN codes aside)
+        k, v = k.view(append.STORAGE[kind]), v.view(append.STORAGE[kind])
+    if kind in append.ROW_SCALED:
+        ks, vs = torch.rand(pages, page, hkv, generator=g) + 0.01, torch.rand(pages, page, hkv, generator=g) + 0.01
+    mult = (0.37, 1.9)
+    slots = torch.tensor([[5, 0, 35], [17, 17, 8]])
+    got_k, got_v = attend.rows_at(k, v, slots, kind, ks, vs, mult)
+    assert got_k.shape == (2, 3, hkv, d) and got_k.dtype == torch.float32
+    for store, scales, m, got in ((k, ks, mult[0], got_k), (v, vs, mult[1], got_v)):
+        flat = store.reshape(slots_n, hkv, d)
+        for a, row in enumerate(slots.tolist()):
+            for b, s in enumerate(row):
+                for h in range(hkv):
+                    if kind in ("bf16", "fp16"):
+                        want = flat[s, h].float().numpy()
+                    else:
+                        codes = flat[s, h].view(torch.uint8).numpy()
+                        real = e4m3.decode(codes).astype(np.float32) if kind != "int8" else codes.view(np.int8).astype(np.float32)
+                        scale = np.float32(m) if kind == "fp8" else scales.reshape(slots_n, hkv)[s, h].numpy()
+                        want = real * scale
+                    assert np.array_equal(got[a, b, h].numpy(), want), (kind, s, h)
+    table = torch.tensor([7, 2, 8, 0])
+    for compute in (torch.bfloat16, torch.float32):
+        gk, gv = attend.gather(k, v, table, 13, page, kind, compute, ks, vs, mult)
+        rk, rv = attend.rows_at(k, v, append.slots(table, torch.arange(13), page), kind, ks, vs, mult)
+        assert gk.dtype == compute and torch.equal(gk, rk.to(compute)) and torch.equal(gv, rv.to(compute))
