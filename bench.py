@@ -210,6 +210,36 @@ def append_sweep(pk, device, kind):
     return found
 
 
+def append_rope(pk, device):
+    """KV append with the keys' rotary embedding fused in (write's rope=) beside the plain append of the same rows:
+    8 KV heads x 128, bf16 inputs; bytes as the plain append's (the table's rows are read besides: 512 B a token)."""
+    hkv, d, found = 8, 128, {}
+    n_slots = 1 << 20
+    g = torch.Generator(device=device).manual_seed(2)
+    angle = torch.arange(8192, dtype=torch.float64, device=device)[:, None] / \
+        (10000.0 ** (torch.arange(d // 2, dtype=torch.float64, device=device) / (d // 2)))[None, :]
+    table = torch.cat([angle.cos(), angle.sin()], 1).float().contiguous()
+    for kind in ("bf16", "fp8"):
+        store = torch.bfloat16 if kind == "bf16" else torch.float8_e4m3fn
+        e = 2 if kind == "bf16" else 1
+        k = torch.zeros(n_slots, hkv, d, dtype=store, device=device)
+        v = torch.zeros_like(k)
+        found[kind] = {}
+        for T in (64, 4152, 262144):
+            keys = torch.randn(T, hkv, d, device=device, generator=g).to(torch.bfloat16)
+            values = torch.randn(T, hkv, d, device=device, generator=g).to(torch.bfloat16)
+            slots = torch.randperm(n_slots, device=device, generator=g)[:T]
+            positions = torch.randint(0, 8192, (T,), device=device, generator=g)
+            plain = timed(lambda: pk.write(keys, values, slots, k, v, kind, multipliers=(0.02, 0.03)), 20, 3)
+            fused = timed(lambda: pk.write(keys, values, slots, k, v, kind, multipliers=(0.02, 0.03),
+                                           rope=(table, positions)), 20, 3)
+            nbytes = T * hkv * 2 * d * (e + 2)
+            found[kind][str(T)] = {"plain_us": round(plain * 1e3, 2), "with_rope_us": round(fused * 1e3, 2),
+                                   "with_rope_GB/s": round(nbytes / fused / 1e6, 1)}
+        del k, v
+    return found
+
+
 def long_context(pk, device):
     """Split-K partitioned decode over long contexts (40 query heads, 8 KV heads, bf16, random page placement in a
     200k-token pool): contiguous splits of `chunk` positions, then the log-sum-exp merge. One layer, one token a row."""
@@ -599,6 +629,8 @@ def main():
         torch.cuda.empty_cache()
         extras["append_GB/s_by_tokens"] = {kind: append_sweep(pk, device, kind) for kind in ("bf16", "fp8")}
         log(f"[bench] append sweep: {extras['append_GB/s_by_tokens']}")
+        extras["append_with_rope"] = append_rope(pk, device)
+        log(f"[bench] append with the keys' rope fused in: {extras['append_with_rope']}")
         extras["long_context_splitk_bf16"] = long_context(pk, device)
         log(f"[bench] long context: {extras['long_context_splitk_bf16']}")
         torch.cuda.empty_cache()

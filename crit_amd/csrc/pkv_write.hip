@@ -19,6 +19,13 @@ struct WriteArgs {
     int heads;      // hkv (keys only) or 2 * hkv
     Div32 heads_div;
     float mult[2];
+    // Rotary embedding of the key rows on their way in (rope_table null: none): cos of pair j of position p at
+    // rope_table[p * dim[0] + j], sin at [p * dim[0] + dim[0] / 2 + j]; positions clamped to the table's rows.
+    const float* rope_table;
+    const int64_t* positions;
+    int64_t rope_rows;
+    int rope_interleaved;
+    float rope_scale;
 };
 
 template <int IN>
@@ -56,6 +63,32 @@ struct RawRow {
     }
     PKV_DEV void widen(float (&x)[EPL]) const {
         static_for<EPL>([&](auto j) { x[j] = at<j>(); });
+    }
+    // The row of the lane `delta` lanes away (xor).
+    PKV_DEV RawRow across(int delta) const {
+        RawRow r;
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            r.v[j] = u32x4{(unsigned)__shfl_xor((int)v[j].x, delta), (unsigned)__shfl_xor((int)v[j].y, delta),
+                           (unsigned)__shfl_xor((int)v[j].z, delta), (unsigned)__shfl_xor((int)v[j].w, delta)};
+        }
+        return r;
+    }
+    // x rounded to the input type (nearest even) and packed as the row.
+    PKV_DEV void pack(const float (&x)[EPL]) {
+        if constexpr (IN == CRIT_PKV_F32) {
+            static_for<N>([&](auto j) { v[j] = u32x4{f2u(x[4 * j]), f2u(x[4 * j + 1]), f2u(x[4 * j + 2]), f2u(x[4 * j + 3])}; });
+        } else if constexpr (IN == CRIT_PKV_BF16) {
+            static_for<N>([&](auto j) {
+                v[j] = u32x4{pack_bf16(x[8 * j], x[8 * j + 1]), pack_bf16(x[8 * j + 2], x[8 * j + 3]),
+                             pack_bf16(x[8 * j + 4], x[8 * j + 5]), pack_bf16(x[8 * j + 6], x[8 * j + 7])};
+            });
+        } else {
+            static_for<N>([&](auto j) {
+                v[j] = u32x4{pack_f16(x[8 * j], x[8 * j + 1]), pack_f16(x[8 * j + 2], x[8 * j + 3]),
+                             pack_f16(x[8 * j + 4], x[8 * j + 5]), pack_f16(x[8 * j + 6], x[8 * j + 7])};
+            });
+        }
     }
 };
 
@@ -98,7 +131,12 @@ PKV_DEV void exact_codes(const Row& row, float div, uint32_t (&w)[4]) {
 // store. The launcher gives every thread one row: with the loads free of conditions and 46-52 registers a thread, eight
 // wavefronts a SIMD are resident, and more, shorter workgroups measured faster than more rows a thread at every size
 // (262,144 tokens of 8 KV heads, bf16: 389 us with one row, 397 with two, 413 with four).
-template <int KIND, bool F16, int IN, int LPR, int U>
+// ROPE: the key rows are rotated at their tokens' positions first (the reference's rope() before write(),
+// inference/fused-norms/code/torch_norms.py:89-147, over the whole head width): pairs (j, j + dim / 2) (style half: the
+// partner element sits dim / 2 further, in the lane LPR / 2 away) or (2j, 2j + 1) (interleaved: both in the lane);
+// a cos - b sin and b cos + a sin as separate FP32 products and a sum, rounded to the input's type as rope() rounds
+// to its output's, and packed back into the row, which then goes through the append unchanged.
+template <int KIND, bool F16, int IN, int LPR, int U, bool ROPE = false>
 __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
     constexpr int EPL = KIND == 0 ? 8 : 16;
     constexpr int RPP = 256 / LPR;      // rows a workgroup covers per pass
@@ -137,6 +175,49 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
         raw[u].load(src, (int64_t)t * st + head[u] * sh + (live[u] ? i0 : 0));
     }
     __builtin_amdgcn_sched_barrier(0);      // (nothing that waits for a load moves up among the loads)
+    if constexpr (ROPE) {
+        static_assert(U == 1 && LPR >= 2, "one row a thread, a row over two lanes or more");
+        const uint32_t rowc = in[0] ? row0 : 0;
+        const uint32_t t = div32(a.heads_div, rowc);
+        int64_t pos = a.positions[t];
+        pos = pos < 0 ? 0 : (pos > a.rope_rows - 1 ? a.rope_rows - 1 : pos);
+        const int half = a.dim[0] >> 1;
+        const bool upper = lane_in_row >= LPR / 2;
+        // (every lane takes part in the exchange and loads a row of the table: a values' row is left as it was)
+        const int j0 = a.rope_interleaved ? i0 >> 1 : (upper ? i0 - half : i0);
+        constexpr int PAIRS = EPL;      // style half: one pair an element; interleaved: EPL / 2 pairs
+        float cs[PAIRS], sn[PAIRS];
+        // (16-byte loads: the table's rows and a lane's first pair are multiples of four floats)
+        const float4* line = reinterpret_cast<const float4*>(a.rope_table + pos * a.dim[0] + j0);
+        const float4* line_sin = reinterpret_cast<const float4*>(a.rope_table + pos * a.dim[0] + half + j0);
+        const int quads = a.rope_interleaved ? EPL / 8 : EPL / 4;
+#pragma unroll
+        for (int j = 0; j < PAIRS / 4; ++j) {
+            const float4 c = j < quads ? line[j] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            const float4 z = j < quads ? line_sin[j] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            cs[4 * j] = c.x, cs[4 * j + 1] = c.y, cs[4 * j + 2] = c.z, cs[4 * j + 3] = c.w;
+            sn[4 * j] = z.x, sn[4 * j + 1] = z.y, sn[4 * j + 2] = z.z, sn[4 * j + 3] = z.w;
+        }
+        if (a.rope_scale != 1.0f) {
+#pragma unroll
+            for (int j = 0; j < PAIRS; ++j) cs[j] = cs[j] * a.rope_scale, sn[j] = sn[j] * a.rope_scale;
+        }
+        float mine[EPL], other[EPL], y[EPL];
+        raw[0].widen(mine);
+        raw[0].across(LPR / 2).widen(other);
+        if (a.rope_interleaved) {
+#pragma unroll
+            for (int j = 0; j < EPL / 2; ++j) {
+                const float x0 = mine[2 * j], x1 = mine[2 * j + 1];
+                y[2 * j] = x0 * cs[j] - x1 * sn[j];
+                y[2 * j + 1] = x1 * cs[j] + x0 * sn[j];
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < EPL; ++j) y[j] = upper ? mine[j] * cs[j] + other[j] * sn[j] : mine[j] * cs[j] - other[j] * sn[j];
+        }
+        if (!second[0]) raw[0].pack(y);
+    }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         // (a whole row's lanes agree on these, so the row-scale exchange below stays among participating lanes)
@@ -271,6 +352,7 @@ __global__ __launch_bounds__(256) void write_rows_scalar(WriteArgs a) {
 template <int KIND, bool F16, int IN>
 static int launch_kind(const WriteArgs& a, int lpr, bool vector, hipStream_t stream) {
     if (!vector) {
+        if (a.rope_table) return CRIT_PKV_E_GEOMETRY;      // (the rotation lives in the vector kernel)
         const int64_t blocks = (a.tokens * a.heads + 255) / 256;
         hipLaunchKernelGGL((write_rows_scalar<KIND, F16, IN>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
         return hip_code(hipGetLastError());
@@ -283,6 +365,7 @@ static int launch_kind(const WriteArgs& a, int lpr, bool vector, hipStream_t str
             WriteArgs part = a;
             part.tokens = a.tokens - t0 < most ? a.tokens - t0 : most;
             part.slots = a.slots + t0;
+            if (a.positions) part.positions = a.positions + t0;
             for (int w = 0; w < 2; ++w) {
                 if (a.src[w]) part.src[w] = reinterpret_cast<const char*>(a.src[w]) + t0 * a.stride_t[w] * in_bytes;
             }
@@ -294,6 +377,19 @@ static int launch_kind(const WriteArgs& a, int lpr, bool vector, hipStream_t str
     const int64_t rows = a.tokens * a.heads;
     const int rows_per_block = 256 / lpr;
     const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
+    if (a.rope_table) {      // (head widths 64, 128 and 256: 4 to 32 lanes a row)
+        switch (lpr) {
+#define PKV_CASE(L)                                                                                                 \
+    case L:                                                                                                         \
+        hipLaunchKernelGGL((write_rows<KIND, F16, IN, L, 1, true>), dim3((unsigned)blocks), dim3(256), 0, stream, a); \
+        break;
+            PKV_CASE(4) PKV_CASE(8) PKV_CASE(16) PKV_CASE(32)
+#undef PKV_CASE
+            default:
+                return CRIT_PKV_E_GEOMETRY;
+        }
+        return hip_code(hipGetLastError());
+    }
     switch (lpr) {
 #define PKV_CASE(L)                                                                                                 \
     case L:                                                                                                         \
@@ -345,6 +441,16 @@ int launch_write(const crit_pkv_write_params* p, hipStream_t stream) {
     a.heads = p->values ? 2 * p->kv_heads : p->kv_heads;
     a.heads_div = make_div32((uint32_t)a.heads);
     a.mult[0] = p->key_multiplier, a.mult[1] = p->value_multiplier;
+    a.rope_table = p->rope_table, a.positions = p->rope_positions, a.rope_rows = p->rope_rows;
+    a.rope_interleaved = p->rope_interleaved ? 1 : 0, a.rope_scale = p->rope_scale;
+    if (p->rope_table) {
+        // the whole head width rotates, a power of two of whole lanes; the lanes of a values' row of another width
+        // would not line up with the keys' in the exchange
+        if (!p->rope_positions) return CRIT_PKV_E_NULL;
+        if (p->rope_rows < 1 || (p->head_dim != 64 && p->head_dim != 128 && p->head_dim != 256) ||
+            (p->values && p->value_dim > p->head_dim) || (reinterpret_cast<uintptr_t>(p->rope_table) % 16))
+            return CRIT_PKV_E_GEOMETRY;
+    }
     // The vector path: rows are whole 16-byte lanes on both sides and every row start is 16-byte aligned.
     const int epl = p->kind == 0 ? 8 : 16;
     const int in_bytes = p->in_dtype == CRIT_PKV_F32 ? 4 : 2;

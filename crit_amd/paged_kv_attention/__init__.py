@@ -211,13 +211,20 @@ def _workspace(device, tokens, heads, parts, dv, given=None):
 
 # -- writes ----------------------------------------------------------------------------------------------------------------
 def write(keys, values, slots, key_pages, value_pages, kind, key_scales=None, value_scales=None,
-          multipliers=(1.0, 1.0)):
+          multipliers=(1.0, 1.0), *, rope=None):
     """A step's keys [tokens][kv_heads][dim] and values [tokens][kv_heads][value_dim] (FP32, BF16 or FP16) into their
     slots ([tokens] int64; a slot below 0 is skipped) of one layer's pages (any view whose storage is
     [slots][kv_heads][dim]), encoded for the page kind, in one launch; the bytes torch's own casts would store
     (x.float() / multiplier clamped to +-448 then E4M3 for "fp8"; the row rules for "fp8:row" and "int8", their scales
-    written beside the codes). values and value_pages None: keys only. keys and key_pages None: values only."""
+    written beside the codes). values and value_pages None: keys only. keys and key_pages None: values only.
+    rope (no counterpart in the reference's write: the rope() its model plugins call on the keys just before,
+    inference/fused-norms/code/torch_norms.py:89-147, fused into this launch): (table, positions) or (table, positions,
+    style, scale): table FP32 [rows][dim] (cos of every pair, then sin), positions [tokens] int64 (clamped to the table's
+    rows), style "half" (pairs j, j + dim / 2) or "interleaved" (2j, 2j + 1), scale on cos and sin; the keys go in as
+    rope() would have returned them in their own dtype. Head widths 64, 128, 256, values no wider than keys."""
     if keys is None:
+        if rope is not None:
+            raise ValueError("rope rotates keys")
         if values is None:
             raise ValueError("write takes keys, values or both")
         if torch.is_tensor(multipliers):
@@ -259,6 +266,22 @@ def write(keys, values, slots, key_pages, value_pages, kind, key_scales=None, va
     p.value_dim = values.shape[-1] if values is not None else 0
     p.kind, p.page_dtype, p.in_dtype = k_kind, _page_dtype(key_pages, kind), _DTYPE[keys.dtype]
     p.key_multiplier, p.value_multiplier = km, vm
+    if rope is not None:
+        if not 2 <= len(rope) <= 4:
+            raise ValueError("rope is (table, positions), with a style and a scale if not half and 1")
+        table, positions, style, scale = tuple(rope) + ("half", 1.0)[len(rope) - 2:]
+        if style not in ("half", "interleaved"):
+            raise ValueError(f"rope's style is half or interleaved, not {style!r}")
+        if not torch.is_tensor(table) or table.dtype != torch.float32 or table.dim() != 2 or table.shape[1] != d or \
+                table.shape[0] < 1 or not table.is_contiguous() or table.device != keys.device:
+            raise ValueError(f"rope's table is a contiguous FP32 [rows][{d}] tensor (cos, then sin) on the keys' device")
+        if not torch.is_tensor(positions) or positions.dtype != torch.int64 or tuple(positions.shape) != (T,) or \
+                not positions.is_contiguous() or positions.device != keys.device:
+            raise ValueError(f"rope's positions are a contiguous int64 [{T}] tensor on the keys' device")
+        if d not in (64, 128, 256) or p.value_dim > d:
+            raise ValueError("rope in the append takes head widths 64, 128 and 256, values no wider than keys")
+        p.rope_table, p.rope_positions, p.rope_rows = table.data_ptr(), positions.data_ptr(), table.shape[0]
+        p.rope_interleaved, p.rope_scale = int(style == "interleaved"), float(scale)
     with torch.cuda.device(keys.device):
         _abi.check(_abi.load().crit_pkv_write(p, _stream(keys.device)), "paged_kv_attention.write")
 

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 7
+#define CRIT_PKV_ABI_VERSION 8
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -66,6 +66,18 @@ typedef struct crit_pkv_write_params {
     int32_t page_dtype;             /* kind 16BIT: CRIT_PKV_BF16 or CRIT_PKV_F16 */
     int32_t in_dtype;               /* CRIT_PKV_F32, _BF16 or _F16: the dtype of keys and values */
     float key_multiplier, value_multiplier;   /* kind FP8: code = e4m3(clamp(x / multiplier, -448, 448)) */
+    /* Rotary embedding of the keys on their way in: the reference's rope() (inference/fused-norms/code/
+     * torch_norms.py:89-147; called as rope_pair before write by the model plugins) over the whole head width, fused
+     * into the append. rope_table NULL: none. Else a [rope_rows][head_dim] FP32 table, cos of every pair then sin
+     * (torch_norms.py:104-106), read at rope_positions[t] clamped to its rows; pairs (j, j + head_dim / 2), or
+     * (2j, 2j + 1) with rope_interleaved; rope_scale multiplies cos and sin. a cos - b sin and b cos + a sin in
+     * FP32, rounded to in_dtype as rope() rounds to its output's type, then appended as given keys would be. Head
+     * widths 64, 128, 256; rows 16-byte aligned; values no wider than keys. */
+    const float* rope_table;
+    const int64_t* rope_positions;  /* [tokens] */
+    int64_t rope_rows;
+    int32_t rope_interleaved;
+    float rope_scale;
 } crit_pkv_write_params;
 
 int crit_pkv_write(const crit_pkv_write_params* p, void* stream);

@@ -116,3 +116,27 @@ def decode_rows(store, scales, kind, multiplier=1.0, dtype=torch.float64):
     if kind in ROW_SCALED:
         x = x * scales.to(dtype)[..., None]
     return x
+
+
+def rope(x, positions, table, style="half", scale=1.0):
+    """Each token's heads [tokens][heads][dim] rotated at its position over the whole head width, as the reference's
+    rope() with a [positions][dim] table (cos of every pair, then sin; inference/fused-norms/code/torch_norms.py:89-147):
+    FP32 inside (a cos - b sin, b cos + a sin as separate products and a sum), positions clamped to the table's rows,
+    scale on cos and sin, one rounding to x's dtype. Pairs (j, j + dim / 2) for style half, (2j, 2j + 1) interleaved."""
+    dim = x.shape[-1]
+    half = dim // 2
+    rows = table.float().index_select(0, torch.as_tensor(positions, dtype=torch.int64).clamp(0, table.shape[0] - 1))
+    cos, sin = rows[:, :half], rows[:, half:]
+    if scale != 1.0:
+        cos, sin = cos * scale, sin * scale
+    cos, sin = cos[:, None, :], sin[:, None, :]
+    x32 = x.float()
+    if style == "half":
+        a, b = x32[..., :half], x32[..., half:]
+        turned = torch.cat([a * cos - b * sin, b * cos + a * sin], -1)
+    elif style == "interleaved":
+        a, b = x32[..., 0::2], x32[..., 1::2]
+        turned = torch.stack([a * cos - b * sin, b * cos + a * sin], -1).flatten(-2)
+    else:
+        raise ValueError(style)
+    return turned.to(x.dtype)

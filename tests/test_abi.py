@@ -67,8 +67,11 @@ def test_the_module_keeps_the_reference_interface():
     for name in ("write", "attend", "prefill", "partitions", "piece_size", "tile_for", "workspace_floats", "flash_chunk",
                  "flash_parts", "flash_block", "flash_tile", "cuda_chunk", "cuda_parts", "cuda_prompt", "owner", "release"):
         assert callable(getattr(pk, name)), name
-    assert list(inspect.signature(pk.write).parameters) == [
+    write = inspect.signature(pk.write).parameters
+    assert list(write)[:9] == [
         "keys", "values", "slots", "key_pages", "value_pages", "kind", "key_scales", "value_scales", "multipliers"]
+    # (beyond the reference's: the keys' rotary embedding fused into the append, by keyword only)
+    assert list(write)[9:] == ["rope"] and write["rope"].kind is inspect.Parameter.KEYWORD_ONLY and write["rope"].default is None
     attend = inspect.signature(pk.attend).parameters
     assert list(attend)[:10] == ["q", "key_pages", "value_pages", "kind", "tables", "rows", "starts", "firsts", "columns",
                                  "page"]

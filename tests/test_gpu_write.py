@@ -218,3 +218,49 @@ def test_bad_arguments_are_refused():
     with pytest.raises(ValueError, match="scales"):
         pk.write(x, None, torch.zeros(2, dtype=torch.int64, device=dev), k, None, "int8")
     pk.write(x[:0], None, torch.zeros(0, dtype=torch.int64, device=dev), k, None, "bf16")     # no tokens: nothing
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("d,dv,in_dtype", [(128, 128, torch.bfloat16), (64, 64, torch.float32), (256, 128, torch.bfloat16),
+                                           (128, 64, torch.float16)])
+@pytest.mark.parametrize("style", ["half", "interleaved"])
+def test_keys_rotated_on_their_way_in_are_the_bytes_of_rope_then_write(kind, d, dv, in_dtype, style):
+    # write(rope=(table, positions, style, scale)): the reference's rope() on the keys (inference/fused-norms/code/
+    # torch_norms.py:89-147, what its model plugins run just before the append) fused into the launch: every stored byte
+    # and row scale equals the oracle's rope() followed by its write(), the values untouched by the rotation; positions
+    # past the table read its last row; a skipped slot stays zero.
+    pk = kernels()
+    g = torch.Generator().manual_seed(51)
+    T, hkv, P = 70, 3, 200
+    keys = (torch.randn(T, hkv, d, generator=g) * 2).to(in_dtype)
+    values = torch.randn(T, hkv, dv, generator=g).to(in_dtype)
+    half = d // 2
+    angle = torch.arange(P, dtype=torch.float64)[:, None] / (10000.0 ** (torch.arange(half, dtype=torch.float64) / half))[None, :]
+    table = torch.cat([angle.cos(), angle.sin()], 1).float()
+    positions = torch.randint(0, P, (T,), generator=g)
+    positions[:3] = torch.tensor([0, P + 5, -1])
+    slots = torch.randperm(96, generator=g)[:T]
+    slots[9] = -1
+    mult = (0.05, 0.07)
+    for scale in (1.0, 0.75):
+        k = torch.zeros(96, hkv, d, dtype=STORE[kind], device=dev)
+        v = torch.zeros(96, hkv, dv, dtype=STORE[kind], device=dev)
+        ks = vs = None
+        if kind in ("fp8:row", "int8"):
+            ks, vs = torch.zeros(96, hkv, device=dev), torch.zeros(96, hkv, device=dev)
+        pk.write(keys.to(dev), values.to(dev), slots.to(dev), k, v, kind, ks, vs, multipliers=mult,
+                 rope=(table.to(dev), positions.to(dev), style, scale))
+        turned = oracle_append.rope(keys, positions, table, style, scale)
+        want = expected_pages(kind, turned, values, slots, 96, mult)
+        _check(kind, (k, v, ks, vs), want)
+    if kind == "bf16":      # keys only; a table or positions that do not fit are refused
+        k = torch.zeros(96, hkv, d, dtype=STORE[kind], device=dev)
+        pk.write(keys.to(dev), None, slots.to(dev), k, None, kind, rope=(table.to(dev), positions.to(dev), style))
+        want = expected_pages(kind, oracle_append.rope(keys, positions, table, style), values, slots, 96, mult)
+        assert torch.equal(bits(k.cpu()).reshape(-1), bits(want[0]).reshape(-1))
+        with pytest.raises(ValueError):
+            pk.write(keys.to(dev), None, slots.to(dev), k, None, kind, rope=(table[:, :half].contiguous().to(dev), positions.to(dev)))
+        with pytest.raises(ValueError):
+            pk.write(keys.to(dev), None, slots.to(dev), k, None, kind, rope=(table.to(dev), positions[:5].to(dev)))
+        with pytest.raises(ValueError):
+            pk.write(keys.to(dev), None, slots.to(dev), k, None, kind, rope=(table.to(dev), positions.to(dev), "pairs"))

@@ -640,3 +640,46 @@ def test_rows_read_back_are_the_codes_times_their_scale_one_fp32_product(kind):
         gk, gv = attend.gather(k, v, table, 13, page, kind, compute, ks, vs, mult)
         rk, rv = attend.rows_at(k, v, append.slots(table, torch.arange(13), page), kind, ks, vs, mult)
         assert gk.dtype == compute and torch.equal(gk, rk.to(compute)) and torch.equal(gv, rv.to(compute))
+
+
+# -- rotary embedding before the append -----------------------------------------------------------------------------------
+@pytest.mark.parametrize("style", ["half", "interleaved"])
+def test_rope_turns_each_pair_by_its_positions_angle(style):
+    # Pins append.rope(): against the rotation as complex numbers in float64 ((a + ib) e^{i theta}, to FP32 rounding),
+    # against a scalar loop in numpy float32 with the same separate roundings (bit for bit), by what a rotation
+    # preserves (each pair's norm), by the angle sum (turning by p then by r equals turning by p + r, to rounding), and
+    # at position 0 (the identity); positions outside the table read its first and last rows.
+    g = torch.Generator().manual_seed(41)
+    T, H, D, P = 7, 3, 16, 50
+    half = D // 2
+    freqs = 1.0 / (10000.0 ** (torch.arange(half, dtype=torch.float64) / half))
+    angle = torch.arange(P, dtype=torch.float64)[:, None] * freqs[None, :]
+    table = torch.cat([angle.cos(), angle.sin()], 1).float()
+    x = torch.randn(T, H, D, generator=g)
+    positions = torch.tensor([0, 3, 49, 17, 5, 60, -2])
+    got = append.rope(x, positions, table, style)
+    at = positions.clamp(0, P - 1)
+    pair = (lambda t: (t[..., :half], t[..., half:])) if style == "half" else (lambda t: (t[..., 0::2], t[..., 1::2]))
+    a, b = pair(x.double())
+    turned = torch.complex(a, b) * torch.polar(torch.ones(T, 1, half, dtype=torch.float64), angle[at][:, None, :])
+    ga, gb = pair(got.double())
+    torch.testing.assert_close(ga, turned.real, atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(gb, turned.imag, atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(ga ** 2 + gb ** 2, a ** 2 + b ** 2, atol=1e-5, rtol=1e-5)
+    assert torch.equal(got[0], x[0]) and torch.equal(got[6], x[6])      # position 0 (and -2, clamped to it)
+    xn, tn = x.numpy(), table.numpy()
+    for t in range(T):
+        for h in range(H):
+            for j in range(half):
+                ia, ib = (j, j + half) if style == "half" else (2 * j, 2 * j + 1)
+                c, s = tn[int(at[t]), j], tn[int(at[t]), half + j]
+                wa = np.float32(np.float32(xn[t, h, ia] * c) - np.float32(xn[t, h, ib] * s))
+                wb = np.float32(np.float32(xn[t, h, ib] * c) + np.float32(xn[t, h, ia] * s))
+                assert got[t, h, ia].item() == wa and got[t, h, ib].item() == wb
+    twice = append.rope(append.rope(x, torch.full((T,), 11), table, style), torch.full((T,), 6), table, style)
+    torch.testing.assert_close(twice, append.rope(x, torch.full((T,), 17), table, style), atol=2e-6, rtol=1e-5)
+    # scale multiplies cos and sin first; 16-bit inputs come back in their dtype, rounded once
+    scaled = append.rope(x, positions, table, style, scale=0.5)
+    torch.testing.assert_close(scaled, got * 0.5, atol=1e-6, rtol=1e-6)
+    low = append.rope(x.bfloat16(), positions, table, style)
+    assert low.dtype == torch.bfloat16 and torch.equal(low, append.rope(x.bfloat16().float(), positions, table, style).bfloat16())
