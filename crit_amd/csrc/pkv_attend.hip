@@ -299,7 +299,7 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     a.vp = reinterpret_cast<const uint8_t*>(p->value_pages);
     a.ks = p->key_scales, a.vs = p->value_scales;
     a.hm = p->kind == 1 ? p->head_multipliers : nullptr;
-    a.tables = p->tables, a.rows = p->rows, a.starts = p->starts, a.counts = p->counts, a.firsts = p->firsts, a.offsets = p->offsets;
+    a.tables = p->tables, a.rows = reinterpret_cast<const int32_t*>(p->rows), a.rows_step = p->rows_are_64 ? 2 : 1, a.starts = p->starts, a.counts = p->counts, a.firsts = p->firsts, a.offsets = p->offsets;
     a.po = p->partial_out, a.pm = p->partial_max, a.pl = p->partial_sum;
     a.out = p->out, a.lse = p->lse, a.sinks = p->sinks;
     a.parents = p->parents, a.parents64 = p->parents64;

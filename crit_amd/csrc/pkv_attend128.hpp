@@ -129,7 +129,7 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
     // trip instead of a chain of them at the start of every unit.
     int count_raw = *(a.counts ? a.counts + r : a.starts + r);      // (no load under a condition)
     int64_t first64 = a.firsts[r];
-    int table_row = a.rows[r];
+    int table_row = a.rows[(int64_t)r * a.rows_step];
     int start = a.starts[r];
     int off_r = *(a.offsets ? a.offsets + r : a.starts + r), off_0 = *(a.offsets ? a.offsets : a.starts);
     // (the values are taken together here, which keeps the compiler from sinking some of the loads below the tests

@@ -19,7 +19,8 @@ struct AttendArgs {
     const float* vs;
     const float* hm;
     const int32_t* tables;
-    const int32_t* rows;
+    const int32_t* rows;      // entry r at rows[r * rows_step]: int32 entries (step 1) or the low words of int64 ones (step 2)
+    int rows_step;
     const int32_t* starts;
     const int32_t* counts;
     const int64_t* firsts;

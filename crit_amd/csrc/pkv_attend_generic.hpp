@@ -74,7 +74,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
     const int n_run = SPARSE ? a.listed_keys : n_keys;      // the positions the partitions divide among them
     const int n_pieces = (n_run + a.piece - 1) / a.piece;
     if (!FUSED && b >= n_pieces) return;
-    const int64_t trow = (int64_t)a.rows[r] * a.tab_stride;
+    const int64_t trow = (int64_t)a.rows[(int64_t)r * a.rows_step] * a.tab_stride;
     const int start = a.starts[r];
     int f_first = 0x7fffffff;
     int64_t f_shift = 0;

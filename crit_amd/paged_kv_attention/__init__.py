@@ -342,7 +342,7 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
     """Decode and verify windows over paged KV (see the module's description).
 
     q [tokens][heads][dim] BF16 or FP16 (FP16 for "fp16" pages); key_pages/value_pages one layer's pages, key_scales/
-    value_scales their scales for "fp8:row" and "int8"; tables [S][width] int32 page tables; rows [R] int32 the table
+    value_scales their scales for "fp8:row" and "int8"; tables [S][width] int32 page tables; rows [R] int32 (or int64: a round's slots as they are) the table
     row of each batch row; starts [R] int32 its first token in q; firsts [R] int64 its column 0's position; counts [R]
     int32 its columns (None: `columns` each; more than `columns` read as `columns`); columns the widest row
     (<= MAX_COLUMNS), a Python int. offsets [R] int32 and tokens: each row's first partial row and the partial rows
@@ -407,9 +407,9 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
         raise ValueError(f"q is {want_q} over {kind} pages, not {q.dtype}")
     if (offsets is None) != (tokens is None):
         raise ValueError("offsets come with the partial rows they take (tokens)")
-    if tables.dtype != torch.int32 or tables.stride(-1) != 1 or rows.dtype != torch.int32 or \
+    if tables.dtype != torch.int32 or tables.stride(-1) != 1 or rows.dtype not in (torch.int32, torch.int64) or \
             starts.dtype != torch.int32 or firsts.dtype != torch.int64:
-        raise ValueError("tables, rows and starts are int32 and firsts int64")
+        raise ValueError("tables and starts are int32, rows int32 or int64 and firsts int64")
     if counts is not None and counts.dtype != torch.int32 or offsets is not None and offsets.dtype != torch.int32:
         raise ValueError("counts and offsets are int32")
     partial_rows = R * columns if offsets is None else int(tokens)
@@ -441,6 +441,7 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
     p.q, p.key_pages, p.value_pages = q.data_ptr(), key_pages.data_ptr(), value_pages.data_ptr()
     p.key_scales, p.value_scales, p.head_multipliers = _ptr(key_scales), _ptr(value_scales), _ptr(per_head)
     p.tables, p.rows, p.starts, p.counts = tables.data_ptr(), rows.data_ptr(), starts.data_ptr(), _ptr(counts)
+    p.rows_are_64 = int(rows.dtype == torch.int64)
     p.firsts, p.offsets = firsts.data_ptr(), _ptr(offsets)
     p.partial_out, p.partial_max, p.partial_sum = _ptr(po), _ptr(pm), _ptr(pl)
     p.out, p.lse, p.sinks = out.data_ptr(), _ptr(lse), _ptr(sinks)

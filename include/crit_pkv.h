@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 8
+#define CRIT_PKV_ABI_VERSION 9
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -100,7 +100,7 @@ typedef struct crit_pkv_attend_params {
     const float* value_scales;
     const float* head_multipliers;  /* optional [2][kv_heads], kind FP8 */
     const int32_t* tables;          /* [S][table_width] */
-    const int32_t* rows;            /* [n_rows] */
+    const void* rows;               /* [n_rows] int32, or int64 with rows_are_64: the table row of each batch row */
     const int32_t* starts;          /* [n_rows] */
     const int32_t* counts;          /* [n_rows] or NULL: `columns` each */
     const int64_t* firsts;          /* [n_rows] */
@@ -146,6 +146,9 @@ typedef struct crit_pkv_attend_params {
     const int64_t* fresh_firsts;
     int64_t fresh_stride_k, fresh_stride_v, fresh_rows;
     int32_t fresh_per_row;
+    /* rows holds int64 entries (a captured round hands the reader its round slots as they are, int64:
+     * inference/attention-state/code/device_attention.py:573, core/python/crit_plugins/device.py:661,681). */
+    int32_t rows_are_64;
 } crit_pkv_attend_params;
 
 int crit_pkv_attend(const crit_pkv_attend_params* p, void* stream);

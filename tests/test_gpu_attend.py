@@ -596,3 +596,23 @@ def test_block_lists_with_a_draft_tree_over_long_lists(kind, block_size):
     _close(out, want)
     more = cache.attend(q, [0], [0], [first], 5, parents=parents, blocks=blocks.to(dev), block_size=block_size, partitions=16)
     _close(more, want)
+
+
+@pytest.mark.parametrize("kind", ["bf16", "fp8:row"])
+def test_a_round_hands_its_slots_over_as_int64_rows(kind):
+    # A captured round's launch (device_attention.py:561-576): the pool's round tables, the batch's round slots as they
+    # are (int64, device.py:661, 681), starts int32, the frontier int64, no counts: the same bits as int32 rows, through
+    # the 128-wide kernel, the generic one (a head width of 64) and the fused launch.
+    for hq, hkv, d in ((8, 2, 128), (4, 2, 64)):
+        cache = Cache(kind, hkv, d, d, 16, [700, 90, 300], seed=81)
+        cols = 4
+        q = rand_q(3 * cols, hq, d, 82)
+        slots_t = torch.tensor([2, 0, 1], dtype=torch.int64, device=dev)
+        starts_t = (torch.arange(4, dtype=torch.int32, device=dev) * cols)[:3]
+        frontier = torch.tensor([290, 640, 70], dtype=torch.int64, device=dev)
+        for fused in (False, True):
+            got = cache.attend(q, slots_t, starts_t, frontier, cols, fused=fused)
+            want = cache.attend(q, slots_t.to(torch.int32), starts_t, frontier, cols, fused=fused)
+            assert torch.equal(got, want)
+        ref, _ = cache.want(q[cols:2 * cols], 0, 640, cols)
+        _close(got[cols:2 * cols], ref)
