@@ -1,0 +1,194 @@
+"""The benchmark configurations at their full sizes (Llama-3-8B-shaped bf16 decode, FP8 decode at batch 128, 200k-token
+split-K decode, chunked prefill mixed with decode): every row of every launch against textbook float64 attention over
+the STORED values, computed densely by torch on the GPU (the oracle's reference() formula; anchored here against the
+CPU oracle on sampled rows), plus what does not depend on size: a fused launch and each row alone give the split
+launch's bits, every chunk size of the contiguous splits agrees, appended bytes read back equal the oracle's encoding.
+Tolerances: 2e-2 for 16-bit pages, 5e-2 for FP8 pages (outputs), 2e-3 for the log-sum-exp."""
+import math
+
+import pytest
+import torch
+
+from oracle import append as oracle_append
+from oracle import attend as oracle_attend
+from tests.support import kernels
+
+pytestmark = pytest.mark.gpu
+dev = "cuda"
+PAGE, HKV, D = 16, 8, 128
+
+
+class Pool:
+    """One layer's pages for sequences of the given lengths over a seeded permutation of a pool 1.25 times the pages
+    needed, filled on the GPU."""
+
+    def __init__(self, kind, lengths, seed, outliers=False, room=1):
+        self.pk = kernels()
+        self.kind, self.lengths = kind, list(lengths)
+        g = torch.Generator(device=dev).manual_seed(seed)
+        held = [math.ceil((n + room) / PAGE) for n in lengths]
+        self.width = (max(held) + 15) // 16 * 16
+        self.pages = int(sum(held) * 1.25) + 1
+        order = torch.randperm(self.pages, device=dev, generator=g).to(torch.int32)
+        self.tables = torch.full((len(lengths), self.width), self.pages, dtype=torch.int32, device=dev)      # (the dump page)
+        at = 0
+        for s, w in enumerate(held):
+            self.tables[s, :w] = order[at:at + w]
+            at += w
+        store = torch.bfloat16 if kind == "bf16" else torch.float8_e4m3fn
+        self.k = torch.zeros(self.pages + 1, PAGE, HKV, D, dtype=store, device=dev)
+        self.v = torch.zeros(self.pages + 1, PAGE, HKV, D, dtype=store, device=dev)
+        self.mult = (1.0, 1.0)
+        if kind == "fp8":      # per-(layer, KV head) multipliers: amax / 448 over what is appended (N(0,1), 1 % x 20)
+            self.mult = torch.tensor([[20.0 * 4.5 / 448.0] * HKV, [20.0 * 4.4 / 448.0] * HKV], device=dev)
+        for s, n in enumerate(lengths):
+            keys = torch.randn(n, HKV, D, device=dev, generator=g)
+            values = torch.randn(n, HKV, D, device=dev, generator=g)
+            if outliers:
+                keys = torch.where(torch.rand(n, HKV, D, device=dev, generator=g) < 0.01, keys * 20, keys)
+                values = torch.where(torch.rand(n, HKV, D, device=dev, generator=g) < 0.01, values * 20, values)
+            else:
+                keys, values = keys * 0.5, values * 0.5
+            self.pk.write(keys.bfloat16(), values.bfloat16(), self.slots(s, 0, n), self.k, self.v, kind, multipliers=self.mult)
+
+    def slots(self, s, start, n):
+        p = torch.arange(start, start + n, device=dev)
+        return self.tables[s][p // PAGE].long() * PAGE + p % PAGE
+
+    def stored(self, s, n):
+        """Positions 0 .. n - 1 of sequence s as float64 (keys, values) [n][HKV][D]: the codes times their multiplier."""
+        at = self.slots(s, 0, n)
+        k = self.k.view(-1, HKV, D)[at].double()
+        v = self.v.view(-1, HKV, D)[at].double()
+        if self.kind == "fp8":
+            k, v = k * self.mult[0].double()[None, :, None], v * self.mult[1].double()[None, :, None]
+        return k, v
+
+
+def dense(q, keys, values, position, scale):
+    """Float64 attention of a chunk q [T][HQ][D] whose token t sits at position + t and sees positions 0 .. position + t
+    of keys / values [n][HKV][D] (n >= position + T): (out [T][HQ][D], lse [T][HQ]); the oracle's reference(), all
+    heads at once."""
+    T, hq, _ = q.shape
+    g = hq // HKV
+    n = position + T
+    qq = q.double().view(T, HKV, g, D)
+    s = torch.einsum("thgd,nhd->thgn", qq, keys[:n]) * scale
+    seen = torch.arange(n, device=q.device)[None, :] <= (position + torch.arange(T, device=q.device))[:, None]
+    s = s.masked_fill(~seen[:, None, None, :], float("-inf"))
+    lse = torch.logsumexp(s, -1)
+    out = torch.einsum("thgn,nhd->thgd", torch.softmax(s, -1), values[:n])
+    return out.reshape(T, hq, D), lse.reshape(T, hq)
+
+
+def check(out, lse, want, want_lse, tol, what):
+    torch.testing.assert_close(out.double(), want, atol=tol, rtol=tol, msg=lambda m: f"{what}: {m}")
+    torch.testing.assert_close(lse.double(), want_lse, atol=2e-3, rtol=1e-3, msg=lambda m: f"{what} lse: {m}")
+
+
+def decode_all(pool, q, firsts, **kw):
+    B = len(pool.lengths)
+    rows = torch.arange(B, dtype=torch.int32, device=dev)
+    lse = torch.empty(B, q.shape[1], device=dev)
+    out = pool.pk.attend(q, pool.k, pool.v, pool.kind, pool.tables, rows, rows.clone(), firsts, 1, PAGE,
+                         multipliers=pool.mult, lse=lse, **kw)
+    return out, lse
+
+
+@pytest.mark.parametrize("kind,B,low,high,tol", [("bf16", 64, 1024, 8192, 2e-2), ("fp8", 128, 2048, 16384, 5e-2)])
+def test_a_decode_step_of_the_8b_shape_at_its_batch_and_lengths(kind, B, low, high, tol):
+    pk = kernels()
+    hq = 32
+    lengths = torch.randint(low, high + 1, (B,), generator=torch.Generator().manual_seed(7)).tolist()
+    lengths[0], lengths[1] = low, high
+    pool = Pool(kind, lengths, 8, outliers=kind == "fp8")
+    g = torch.Generator(device=dev).manual_seed(9)
+    # the step's append: one token a sequence at its length; the bytes read back equal the oracle's encoding
+    keys = torch.randn(B, HKV, D, device=dev, generator=g).bfloat16()
+    values = torch.randn(B, HKV, D, device=dev, generator=g).bfloat16()
+    slots = torch.stack([pool.slots(s, n, 1)[0] for s, n in enumerate(lengths)])
+    pk.write(keys, values, slots, pool.k, pool.v, kind, multipliers=pool.mult)
+    for given, pages, which in ((keys, pool.k, 0), (values, pool.v, 1)):
+        m = 1.0 if kind == "bf16" else pool.mult[which].cpu()
+        want, _ = oracle_append.encode(given.cpu(), kind, m)
+        got = pages.view(-1, HKV, D)[slots].cpu()
+        assert torch.equal(got.view(torch.uint8), want.view(torch.uint8)), "appended bytes"
+    q = torch.randn(B, hq, D, device=dev, generator=g).bfloat16()
+    firsts = torch.tensor(lengths, dtype=torch.int64, device=dev)
+    out, lse = decode_all(pool, q, firsts)
+    scale = D ** -0.5
+    for s, n in enumerate(lengths):
+        k, v = pool.stored(s, n + 1)
+        want, want_lse = dense(q[s:s + 1], k, v, n, scale)
+        check(out[s:s + 1], lse[s:s + 1], want, want_lse, tol, f"row {s} of {n + 1} positions")
+    # the dense reference itself against the CPU oracle, on the shortest row
+    k, v = pool.stored(0, lengths[0] + 1)
+    want, want_lse = dense(q[:1], k, v, lengths[0], scale)
+    seen = torch.ones(lengths[0] + 1, dtype=torch.bool)
+    ref, ref_lse = oracle_attend.reference(q[0].double().cpu(), k.cpu(), v.cpu(), seen, scale)
+    # (the GPU library's float64 products agree with the CPU's to about 1e-6 of the values here, four orders below
+    # the bound the kernels are held to)
+    torch.testing.assert_close(want[0].cpu(), ref, atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(want_lse[0].cpu(), ref_lse, atol=1e-5, rtol=1e-5)
+    # what does not depend on size: the fused launch and a row alone give the split launch's bits
+    fused, fused_lse = decode_all(pool, q, firsts, fused=True)
+    assert torch.equal(out, fused) and torch.equal(lse, fused_lse)
+    for s in (1, B - 1):
+        alone = pk.attend(q[s:s + 1], pool.k, pool.v, kind, pool.tables, torch.tensor([s], dtype=torch.int32, device=dev),
+                          torch.zeros(1, dtype=torch.int32, device=dev), firsts[s:s + 1], 1, PAGE, multipliers=pool.mult)
+        assert torch.equal(alone, out[s:s + 1])
+
+
+@pytest.mark.parametrize("B,context", [(1, 200000), (4, 131072), (2, 32768)])
+def test_long_contexts_through_contiguous_splits_and_their_merge(B, context):
+    hq = 40
+    pool = Pool("bf16", [context - 1] * B, 10)
+    g = torch.Generator(device=dev).manual_seed(11)
+    q = torch.randn(B, hq, D, device=dev, generator=g).bfloat16()
+    firsts = torch.full((B,), context - 1, dtype=torch.int64, device=dev)
+    scale = D ** -0.5
+    wants = [dense(q[s:s + 1], *pool.stored(s, context), context - 1, scale) for s in range(B)]
+    found = {}
+    for chunk in (None, 512, 1024, 2048):
+        out, lse = decode_all(pool, q, firsts, **({} if chunk is None else dict(flash=True, chunk=chunk)))
+        for s in range(B):
+            check(out[s:s + 1], lse[s:s + 1], wants[s][0], wants[s][1], 2e-2, f"chunk {chunk} row {s}")
+        found[chunk] = (out, lse)
+    # every cut of the positions gives the same sum to rounding: the log-sum-exp of any two chunk sizes agrees far
+    # inside the bound against the reference
+    for chunk in (512, 2048):
+        torch.testing.assert_close(found[chunk][1], found[1024][1], atol=1e-4, rtol=1e-5)
+
+
+def test_prompt_chunks_on_prefixes_mixed_with_decode_rows():
+    pk = kernels()
+    hq, T = 32, 512
+    prefixes = [1229, 6096, 6373, 0, 1175, 5023, 8192, 4769]
+    decodes = torch.randint(1024, 8193, (56,), generator=torch.Generator().manual_seed(12)).tolist()
+    pool = Pool("bf16", [p + T for p in prefixes] + [n + 1 for n in decodes], 13, room=0)
+    g = torch.Generator(device=dev).manual_seed(14)
+    tokens = 8 * T + 56
+    q = torch.randn(tokens, hq, D, device=dev, generator=g).bfloat16()
+    out = torch.empty(tokens, hq, D, dtype=torch.bfloat16, device=dev)
+    lse = torch.empty(tokens, hq, device=dev)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    pk.prefill_rows(q, pool.k, pool.v, "bf16", pool.tables, i32(list(range(8))), i32([c * T for c in range(8)]),
+                    i32([T] * 8), torch.tensor(prefixes, dtype=torch.int64, device=dev), T, PAGE, out=out, lse=lse)
+    rows = i32(list(range(8, 64)))
+    pk.attend(q, pool.k, pool.v, "bf16", pool.tables, rows, i32([8 * T + r for r in range(56)]),
+              torch.tensor(decodes, dtype=torch.int64, device=dev), 1, PAGE, out=out, lse=lse)
+    scale = D ** -0.5
+    for c, p in enumerate(prefixes):
+        k, v = pool.stored(c, p + T)
+        want, want_lse = dense(q[c * T:(c + 1) * T], k, v, p, scale)
+        check(out[c * T:(c + 1) * T], lse[c * T:(c + 1) * T], want, want_lse, 2e-2, f"chunk {c} on a prefix of {p}")
+    for r, n in enumerate(decodes):
+        k, v = pool.stored(8 + r, n + 1)
+        t = 8 * T + r
+        want, want_lse = dense(q[t:t + 1], k, v, n, scale)
+        check(out[t:t + 1], lse[t:t + 1], want, want_lse, 2e-2, f"decode row {r}")
+    # a prompt token's output is the same position decoded, to the readers' rounding
+    c, t = 2, 300
+    one = pk.attend(q[c * T + t:c * T + t + 1], pool.k, pool.v, "bf16", pool.tables, i32([c]), i32([0]),
+                    torch.tensor([prefixes[c] + t], dtype=torch.int64, device=dev), 1, PAGE)
+    torch.testing.assert_close(one.float(), out[c * T + t:c * T + t + 1].float(), atol=8e-3, rtol=2e-2)
