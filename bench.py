@@ -624,6 +624,11 @@ def main():
                          "GB/s": round((ow.decode_bytes + ow.append_bytes) * ow.layers / ms / 1e6, 1),
                          "split_launch_ms": round(osplit, 4), "split_launch_GB/s": round(ow.decode_bytes / osplit / 1e6, 1),
                          "frac": round(ow.decode_bytes / osplit / 1e6 / HBM_PEAK_GBPS, 4)}
+        # the same launches with pieces twice as long (attend's piece=, a deployment's choice through the plugin's
+        # `piece` option: fixed per pool like the default; halves the units' fixed costs, and a small batch's units)
+        ow.piece *= 2
+        olong = kernel_ms(ow, 1)
+        extras[other]["split_launch_GB/s_with_pieces_twice_as_long"] = round(ow.decode_bytes / olong / 1e6, 1)
         log(f"[bench] {other}: {extras[other]}")
         del ow
         torch.cuda.empty_cache()
