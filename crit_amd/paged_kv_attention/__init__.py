@@ -102,6 +102,26 @@ def _stream(device):
     return torch.cuda.current_stream(device).cuda_stream
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)      # (the stream's handle without a Stream object)
+
+
+def _launch(device, name, what, *args):
+    """Calls entry point `name` with args and the caller's current stream of `device` as its last argument, with
+    `device` current (a decode step calls this about a hundred times: the device is switched only where it is not the
+    current one already); raises what _abi.check raises."""
+    index = device.index
+    current = torch.cuda.current_device()
+    entry = getattr(_abi.load(), name)
+    if index is None or index == current:
+        stream = _raw_stream(current) if _raw_stream is not None else torch.cuda.current_stream(device).cuda_stream
+        code = entry(*args, stream)
+    else:
+        with torch.cuda.device(device):
+            code = entry(*args, _stream(device))
+    if code:
+        _abi.check(code, what)
+
+
 def _require_device(t, what):
     if not t.is_cuda:
         raise ValueError(f"{what} lives on the GPU (these are HIP kernels; there is no CPU path)")
@@ -150,8 +170,14 @@ def _page_dtype(pages, kind):
     return _abi.BF16
 
 
+_cu_count = {}
+
+
 def _cus(device):
-    return torch.cuda.get_device_properties(device).multi_processor_count
+    found = _cu_count.get(device)
+    if found is None:
+        found = _cu_count[device] = torch.cuda.get_device_properties(device).multi_processor_count
+    return found
 
 
 # -- the split's order knobs -----------------------------------------------------------------------------------------------
@@ -282,8 +308,7 @@ def write(keys, values, slots, key_pages, value_pages, kind, key_scales=None, va
             raise ValueError("rope in the append takes head widths 64, 128 and 256, values no wider than keys")
         p.rope_table, p.rope_positions, p.rope_rows = table.data_ptr(), positions.data_ptr(), table.shape[0]
         p.rope_interleaved, p.rope_scale = int(style == "interleaved"), float(scale)
-    with torch.cuda.device(keys.device):
-        _abi.check(_abi.load().crit_pkv_write(p, _stream(keys.device)), "paged_kv_attention.write")
+    _launch(keys.device, "crit_pkv_write", "paged_kv_attention.write", p)
 
 
 # -- windows ---------------------------------------------------------------------------------------------------------------
@@ -475,8 +500,7 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
         p.fresh_shifts, p.fresh_firsts = fshift.data_ptr(), ffirst.data_ptr()
         p.fresh_stride_k, p.fresh_stride_v, p.fresh_rows = fk.stride(0), fv.stride(0), int(fk.shape[0])
         p.fresh_per_row = int(fshift.numel() != 1)
-    with torch.cuda.device(device):
-        _abi.check(_abi.load().crit_pkv_attend(p, _stream(device)), "paged_kv_attention.attend")
+    _launch(device, "crit_pkv_attend", "paged_kv_attention.attend", p)
     return out
 
 
@@ -497,8 +521,7 @@ def merge_shards(outs, lses):
     p = _abi.MergeParams()
     p.outs, p.lses, p.out, p.lse = outs.data_ptr(), lses.data_ptr(), out.data_ptr(), lse.data_ptr()
     p.rows, p.parts, p.value_dim, p.in_dtype = tokens * heads, parts, dim, _DTYPE[outs.dtype]
-    with torch.cuda.device(outs.device):
-        _abi.check(_abi.load().crit_pkv_merge(p, _stream(outs.device)), "paged_kv_attention.merge_shards")
+    _launch(outs.device, "crit_pkv_merge", "paged_kv_attention.merge_shards", p)
     return out, lse
 
 
@@ -597,8 +620,7 @@ def _prefill_launch(q, key_pages, value_pages, kind, tables, table_rows, starts,
         state = _prefill_state(device, T, hq, d, workspace)
         p.fresh_keys, p.fresh_values, p.fresh_firsts, p.fresh_state = fk.data_ptr(), fv.data_ptr(), _ptr(firsts), state.data_ptr()
         p.fresh_stride_k, p.fresh_stride_v = fk.stride(0), fv.stride(0)
-    with torch.cuda.device(device):
-        _abi.check(_abi.load().crit_pkv_prefill(p, _stream(device)), "paged_kv_attention.prefill")
+    _launch(device, "crit_pkv_prefill", "paged_kv_attention.prefill", p)
     return out
 
 
@@ -681,9 +703,7 @@ def stream_read(data, sink=None):
     _require_device(data, "stream_read's data")
     nbytes = data.numel() * data.element_size()
     sink = torch.zeros(64, dtype=torch.float32, device=data.device) if sink is None else sink
-    with torch.cuda.device(data.device):
-        _abi.check(_abi.load().crit_pkv_stream_read(data.data_ptr(), nbytes, sink.data_ptr(), _stream(data.device)),
-                   "paged_kv_attention.stream_read")
+    _launch(data.device, "crit_pkv_stream_read", "paged_kv_attention.stream_read", data.data_ptr(), nbytes, sink.data_ptr())
     return sink
 
 
@@ -745,8 +765,7 @@ def slots_at(round_tables, round_capacity, slot, positions, page, dump, *, rows=
     p.positions, p.out, p.n, p.n_slots = positions.data_ptr(), out.data_ptr(), positions.numel(), slot.numel()
     p.round_slots, p.table_stride, p.table_pages = round_tables.shape[0], round_tables.stride(0), round_tables.shape[1]
     p.page, p.dump = int(page), int(dump)
-    with torch.cuda.device(device):
-        _abi.check(_abi.load().crit_pkv_slots_at(p, _stream(device)), "paged_kv_attention.slots_at")
+    _launch(device, "crit_pkv_slots_at", "paged_kv_attention.slots_at", p)
     return out
 
 
@@ -777,8 +796,7 @@ def compact(stores, slots, round_tables, round_capacity, start, emitted, path, m
     p.moved, p.path = _i64_on(moved, device, "moved", rows).data_ptr(), path.data_ptr()
     p.rows, p.round_slots, p.table_stride, p.path_stride = rows, round_tables.shape[0], round_tables.stride(0), path.stride(0)
     p.width, p.path_is_32, p.table_pages, p.page, p.dump = path.shape[1], int(path.dtype == torch.int32), round_tables.shape[1], int(page), int(dump)
-    with torch.cuda.device(device):
-        _abi.check(_abi.load().crit_pkv_compact(p, _stream(device)), "paged_kv_attention.compact")
+    _launch(device, "crit_pkv_compact", "paged_kv_attention.compact", p)
 
 
 def copy_pages(stores, slots, source, target, page):
@@ -795,8 +813,7 @@ def copy_pages(stores, slots, source, target, page):
     if source.numel() == 0:
         return
     p.source, p.target, p.n, p.page = source.data_ptr(), target.data_ptr(), source.numel(), int(page)
-    with torch.cuda.device(device):
-        _abi.check(_abi.load().crit_pkv_copy_pages(p, _stream(device)), "paged_kv_attention.copy_pages")
+    _launch(device, "crit_pkv_copy_pages", "paged_kv_attention.copy_pages", p)
 
 
 # -- rows read back (reference: inference/attention-state/code/pages.py:455-493) -----------------------------------------
@@ -831,8 +848,7 @@ def _read(key_pages, value_pages, kind, n, shape, dtype, key_scales, value_scale
     p.out_keys, p.out_values, p.n = out[0].data_ptr(), _ptr(out[1]), n
     p.kv_heads, p.head_dim, p.value_dim, p.page, p.kind = hkv, d, dv, int(page), k_kind
     p.page_dtype, p.out_dtype, p.key_multiplier, p.value_multiplier = _page_dtype(key_pages, kind), _DTYPE[dtype], km, vm
-    with torch.cuda.device(device):
-        _abi.check(_abi.load().crit_pkv_read_rows(p, _stream(device)), "paged_kv_attention.rows_at")
+    _launch(device, "crit_pkv_read_rows", "paged_kv_attention.rows_at", p)
     return out
 
 
