@@ -478,6 +478,82 @@ def pool_bookkeeping(pk, device):
     return found
 
 
+def small_batches(pk, device):
+    """What a piece costs a batch that does not fill the chip: one layer's decode launch (split + merge, 8B shape) for
+    4 sequences of about 2,000 positions and for one of 8,000, at the default piece and at pieces of 256 positions
+    (attend's piece=, the plugin's `piece` option: fixed per pool either way). Microseconds a launch over four layers of
+    different memory; the launches are queued without waits, so a figure near the host's cost of a call is bound by it."""
+    hq, hkv, d, page, found = 32, 8, 128, 16, {}
+    g = torch.Generator(device=device).manual_seed(3)
+    for kind in ("bf16", "fp8"):
+        store = torch.bfloat16 if kind == "bf16" else torch.float8_e4m3fn
+        for name, lengths in (("4_rows_of_2000", [1900, 2000, 2100, 2048]), ("1_row_of_8000", [8000])):
+            B = len(lengths)
+            width = ((max(lengths) + page) // page + 15) // 16 * 16
+            pages = B * width
+            k = (torch.randn(4, pages + 1, page, hkv, d, device=device, generator=g) * 0.5).to(store)
+            v = (torch.randn(4, pages + 1, page, hkv, d, device=device, generator=g) * 0.5).to(store)
+            tables = torch.randperm(pages, device=device, generator=g).to(torch.int32).view(B, width).contiguous()
+            rows = torch.arange(B, dtype=torch.int32, device=device)
+            firsts = torch.tensor(lengths, dtype=torch.int64, device=device)
+            q = torch.randn(B, hq, d, device=device, generator=g).to(torch.bfloat16)
+            out = torch.empty_like(q)
+            at = [0]
+
+            def launch(piece):
+                at[0] = (at[0] + 1) % 4
+                pk.attend(q, k[at[0]], v[at[0]], kind, tables, rows, rows, firsts, 1, page, out=out, piece=piece,
+                          multipliers=(0.02, 0.03))
+            default = pk.piece_size(d, d, kind, hkv)
+            found[f"{kind}_{name}"] = {f"piece_{default}_us": round(timed(lambda: launch(default), 40, 4) * 1e3, 1),
+                                       "piece_256_us": round(timed(lambda: launch(256), 40, 4) * 1e3, 1)}
+    return found
+
+
+def captured_step(pk, device):
+    """A decode step of a small batch (4 sequences of about 2,000 positions, 32 layers, 8B shape, bf16) launched eagerly
+    and replayed from one HIP graph: slots of the next positions from the bound tables, then append + attention a
+    layer, nothing read on the host; the lengths grow on the device between steps. At the default piece and at pieces of
+    256 positions (small_batches())."""
+    layers, hq, hkv, d, page, B = 32, 32, 8, 128, 16, 4
+    pages_each = 160
+    pages = B * pages_each
+    g = torch.Generator(device=device).manual_seed(6)
+    k = (torch.randn(layers, pages + 1, page, hkv, d, device=device, generator=g) * 0.5).to(torch.bfloat16)
+    v = (torch.randn(layers, pages + 1, page, hkv, d, device=device, generator=g) * 0.5).to(torch.bfloat16)
+    tables = torch.randperm(pages, device=device, generator=g).to(torch.int32).view(B, pages_each).contiguous()
+    capacity = torch.full((B,), pages_each * page, dtype=torch.int64, device=device)
+    lengths = torch.tensor([1900, 2000, 2100, 2048], dtype=torch.int64, device=device)
+    slot_ids = torch.arange(B, dtype=torch.int64, device=device)
+    starts = torch.arange(B, dtype=torch.int32, device=device)
+    keys = torch.randn(layers, B, hkv, d, device=device, generator=g).to(torch.bfloat16)
+    values = torch.randn(layers, B, hkv, d, device=device, generator=g).to(torch.bfloat16)
+    q = torch.randn(layers, B, hq, d, device=device, generator=g).to(torch.bfloat16)
+    out = torch.empty(layers, B, hq, d, dtype=torch.bfloat16, device=device)
+    slots = torch.empty(B, dtype=torch.int64, device=device)
+    parts = pk.partitions(device, hkv, "bf16", d, d)
+    workspace = torch.empty(pk.workspace_floats(B, hq, parts, d), dtype=torch.float32, device=device)
+    one = torch.ones(B, dtype=torch.int64, device=device)
+
+    found = {"layers": layers, "batch": B, "launches": 1 + layers * 3 + 1}
+    for piece in (pk.piece_size(d, d, "bf16", hkv), 256):
+        def step():
+            pk.slots_at(tables, capacity, slot_ids, lengths, page, pages, out=slots)
+            for layer in range(layers):
+                pk.write(keys[layer], values[layer], slots, k[layer], v[layer], "bf16")
+                pk.attend(q[layer], k[layer], v[layer], "bf16", tables, slot_ids, starts, lengths, 1, page,
+                          out=out[layer], workspace=workspace, piece=piece)
+            lengths.add_(one)
+        step()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        found[f"piece_{piece}"] = {"eager_ms": round(timed(step, 20, 2), 3), "graph_replay_ms": round(timed(graph.replay, 20, 2), 3)}
+        del graph
+    return found
+
+
 def prefill_fresh(pk, device):
     """The mixed batch's 8 prompt chunks over FP8 pages (one multiplier pair), once reading every position from the
     pages and once with fresh=: each chunk's own 512 positions from 16-bit rows as the projections gave them, its
@@ -648,6 +724,10 @@ def main():
         extras["prefill_fp8_pages_fresh_rows"] = prefill_fresh(pk, device)
         log(f"[bench] prefill over FP8 pages, with fresh rows: {extras['prefill_fp8_pages_fresh_rows']}")
         torch.cuda.empty_cache()
+        extras["small_batches_by_piece"] = small_batches(pk, device)
+        log(f"[bench] small batches, default piece and 256: {extras['small_batches_by_piece']}")
+        extras["captured_decode_step_bf16"] = captured_step(pk, device)
+        log(f"[bench] a small batch's decode step, eager and from one graph: {extras['captured_decode_step_bf16']}")
         extras["pool_bookkeeping_bf16"] = pool_bookkeeping(pk, device)
         log(f"[bench] pool bookkeeping: {extras['pool_bookkeeping_bf16']}")
         result["extra"] = extras
