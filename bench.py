@@ -26,8 +26,8 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, vendor figure
 
 # HBM bytes one split launch moves, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this file (each counter in
 # a run of its own, scaled by what it reads for the stream-read probe and for a 262,144-token append, kernels of
-# known size: factors 0.5000 and 1.000). Measured for the default workload only.
-MEASURED_TRAFFIC_BYTES = {"c2": 1_453_522_329}
+# known size: factors 0.5000 and 1.000).
+MEASURED_TRAFFIC_BYTES = {"c2": 1_453_522_329, "c3": 2_661_386_240}
 
 
 def log(*a):
