@@ -17,7 +17,7 @@ struct ReadArgs {
     const int64_t* slots;         // [n], or null: through the table
     const int32_t* table;
     const int64_t* table64;
-    int64_t n;
+    int64_t n, pool_slots;        // pool_slots: a slot at or past it reads as zeros (0: not checked)
     int hkv, dim[2], page, kind, f16_pages, out_dtype;
 };
 
@@ -45,7 +45,7 @@ __global__ __launch_bounds__(256) void read_rows_kernel(ReadArgs a) {
         slot = (a.table ? (int64_t)a.table[entry] : a.table64[entry]) * a.page + i % a.page;
     }
     float x[E];
-    if (slot < 0) {
+    if (slot < 0 || (a.pool_slots > 0 && slot >= a.pool_slots)) {
 #pragma unroll
         for (int j = 0; j < E; ++j) x[j] = 0.0f;
     } else {
@@ -118,7 +118,7 @@ int launch_read_rows(const crit_pkv_read_params* p, hipStream_t stream) {
     const int sources = (p->slots != nullptr) + (p->table != nullptr) + (p->table64 != nullptr);
     if (sources != 1) return CRIT_PKV_E_NULL;
     const int dv = p->value_pages ? p->value_dim : 0;
-    if (p->n < 0 || p->kv_heads < 1 || p->head_dim < 8 || p->head_dim % 8 || dv % 8 || (p->value_pages && dv < 8) ||
+    if (p->n < 0 || p->pool_slots < 0 || p->kv_heads < 1 || p->head_dim < 8 || p->head_dim % 8 || dv % 8 || (p->value_pages && dv < 8) ||
         (!p->slots && p->page < 1))
         return CRIT_PKV_E_GEOMETRY;
     if (p->kind < 0 || p->kind > 3 || p->out_dtype < 0 || p->out_dtype > 2) return CRIT_PKV_E_DTYPE;
@@ -132,7 +132,7 @@ int launch_read_rows(const crit_pkv_read_params* p, hipStream_t stream) {
     a.scales[0] = p->key_scales, a.scales[1] = p->value_scales;
     a.head_mult = p->head_multipliers, a.mult[0] = p->key_multiplier, a.mult[1] = p->value_multiplier;
     a.out[0] = p->out_keys, a.out[1] = p->out_values;
-    a.slots = p->slots, a.table = p->table, a.table64 = p->table64, a.n = p->n;
+    a.slots = p->slots, a.table = p->table, a.table64 = p->table64, a.n = p->n, a.pool_slots = p->pool_slots;
     a.hkv = p->kv_heads, a.dim[0] = p->head_dim, a.dim[1] = dv, a.page = p->page, a.kind = p->kind;
     a.f16_pages = p->page_dtype == CRIT_PKV_F16, a.out_dtype = p->out_dtype;
     const int widest = p->head_dim > dv ? p->head_dim : dv;

@@ -846,6 +846,7 @@ def _read(key_pages, value_pages, kind, n, shape, dtype, key_scales, value_scale
     if table is not None:
         p.table, p.table64 = (table.data_ptr(), None) if table.dtype == torch.int32 else (None, table.data_ptr())
     p.out_keys, p.out_values, p.n = out[0].data_ptr(), _ptr(out[1]), n
+    p.pool_slots = key_pages.numel() // (hkv * d)
     p.kv_heads, p.head_dim, p.value_dim, p.page, p.kind = hkv, d, dv, int(page), k_kind
     p.page_dtype, p.out_dtype, p.key_multiplier, p.value_multiplier = _page_dtype(key_pages, kind), _DTYPE[dtype], km, vm
     _launch(device, "crit_pkv_read_rows", "paged_kv_attention.rows_at", p)
@@ -856,7 +857,7 @@ def rows_at(key_pages, value_pages, kind, slots, *, key_scales=None, value_scale
             dtype=torch.float32, out=None):
     """The keys and values at `slots` (any shape, int64, on the device) dequantised: KVPool.rows_at (pages.py:479-493)
     in one launch: float(stored) * the layer's multiplier or the row's scale, one FP32 product, in `dtype` (FP32 as the
-    reference's). A negative slot reads as zeros. value_pages None: keys only. Returns (keys [..., kv_heads, dim],
+    reference's). A negative slot, or one past the pages, reads as zeros. value_pages None: keys only. Returns (keys [..., kv_heads, dim],
     values)."""
     if not torch.is_tensor(slots) or slots.dtype != torch.int64 or slots.device != key_pages.device or not slots.is_contiguous():
         raise ValueError("slots are a contiguous int64 tensor on the pages' device")

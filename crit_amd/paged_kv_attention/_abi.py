@@ -10,7 +10,7 @@ import shutil
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 NAME = "libcrit_pkv.so"
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 KIND_16BIT, KIND_FP8, KIND_FP8_ROW, KIND_INT8 = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
@@ -92,7 +92,7 @@ class CopyPagesParams(ctypes.Structure):
 
 class ReadParams(ctypes.Structure):
     _fields_ = [("key_pages", _p), ("value_pages", _p), ("key_scales", _p), ("value_scales", _p), ("head_multipliers", _p),
-                ("slots", _p), ("table", _p), ("table64", _p), ("out_keys", _p), ("out_values", _p), ("n", _i64),
+                ("slots", _p), ("table", _p), ("table64", _p), ("out_keys", _p), ("out_values", _p), ("n", _i64), ("pool_slots", _i64),
                 ("kv_heads", _i32), ("head_dim", _i32), ("value_dim", _i32), ("page", _i32), ("kind", _i32),
                 ("page_dtype", _i32), ("out_dtype", _i32), ("key_multiplier", _f32), ("value_multiplier", _f32)]
 

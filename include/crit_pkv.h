@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 9
+#define CRIT_PKV_ABI_VERSION 10
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -304,6 +304,8 @@ typedef struct crit_pkv_read_params {
     void* out_keys;
     void* out_values;
     int64_t n;
+    int64_t pool_slots;             /* slots a layer holds: a slot at or past it reads as zeros, like a negative one
+                                       (the reference's index_select would raise); 0: not checked */
     int32_t kv_heads, head_dim, value_dim, page, kind, page_dtype, out_dtype;
     float key_multiplier, value_multiplier;
 } crit_pkv_read_params;

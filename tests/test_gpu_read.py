@@ -56,12 +56,12 @@ def test_rows_at_slots_and_a_sequences_first_positions_read_back_as_torch_does(k
                                      multipliers=mult, dtype=compute)
             _equal(got_k, want_k, f"gathered keys {compute} {count}")
             _equal(got_v, want_v, f"gathered values {compute} {count}")
-    # keys only (a pool without values), into a buffer given, a negative slot as zeros
+    # keys only (a pool without values), into a buffer given, a negative slot and one past the pages as zeros
     out = (torch.full((5, hkv, d), 9.0, device=dev), None)
-    some = torch.tensor([3, -1, 0, 639, 17])
+    some = torch.tensor([3, -1, 0, 639, 640])      # (640: the first slot past the pages)
     pk.rows_at(on(k), None, kind, some.to(dev), key_scales=on(ks), multipliers=mult, out=out)
-    want_k, _ = oracle_attend.rows_at(k, v, some.clamp(min=0), kind, ks, vs, mult)
-    want_k[1] = 0
+    want_k, _ = oracle_attend.rows_at(k, v, some.clamp(0, 639), kind, ks, vs, mult)
+    want_k[1], want_k[4] = 0, 0
     _equal(out[0], want_k, "keys only")
 
 
