@@ -140,11 +140,11 @@ __device__ __forceinline__ void copy_piece(uint8_t* base, int64_t page_bytes, in
 }
 
 __global__ __launch_bounds__(256) void copy_pages_kernel(Stores stores, const int64_t* source, const int64_t* target, int page,
-                                                         int pieces) {
+                                                         int pieces, int64_t pool_pages) {
     const int which = blockIdx.x / pieces, piece = blockIdx.x - which * pieces;
     const crit_pkv_store st = stores.s[blockIdx.z];
     const int64_t from = source[which], to = target[which];
-    if (from < 0 || to < 0) return;
+    if (from < 0 || to < 0 || (pool_pages > 0 && (from >= pool_pages || to >= pool_pages))) return;
     uint8_t* base = reinterpret_cast<uint8_t*>(st.base) + (int64_t)blockIdx.y * st.layer_stride;
     if (stores.wide[blockIdx.z])
         copy_piece<u32x4>(base, st.row_bytes * page, from, to, piece);
@@ -216,7 +216,8 @@ int launch_copy_pages(const crit_pkv_copy_pages_params* p, hipStream_t stream) {
     if (!p) return CRIT_PKV_E_NULL;
     if (p->n == 0) return 0;
     if (!p->source || !p->target) return CRIT_PKV_E_NULL;
-    if (p->n < 0 || p->page < 1 || p->layers < 1 || p->layers > 65535 || p->n_stores < 1 || p->n_stores > CRIT_PKV_MAX_STORES)
+    if (p->n < 0 || p->pool_pages < 0 || p->page < 1 || p->layers < 1 || p->layers > 65535 || p->n_stores < 1 ||
+        p->n_stores > CRIT_PKV_MAX_STORES)
         return CRIT_PKV_E_GEOMETRY;
     Stores stores;
     if (const int bad = take_stores(p->stores, p->n_stores, p->page, stores)) return bad;
@@ -227,7 +228,8 @@ int launch_copy_pages(const crit_pkv_copy_pages_params* p, hipStream_t stream) {
     }
     if (pieces * p->n > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
     const dim3 grid((unsigned)(pieces * p->n), (unsigned)p->layers, (unsigned)p->n_stores);
-    hipLaunchKernelGGL(copy_pages_kernel, grid, dim3(256), 0, stream, stores, p->source, p->target, p->page, (int)pieces);
+    hipLaunchKernelGGL(copy_pages_kernel, grid, dim3(256), 0, stream, stores, p->source, p->target, p->page, (int)pieces,
+                       p->pool_pages);
     return (int)hipGetLastError();
 }
 

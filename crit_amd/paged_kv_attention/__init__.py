@@ -802,7 +802,7 @@ def compact(stores, slots, round_tables, round_capacity, start, emitted, path, m
 def copy_pages(stores, slots, source, target, page):
     """Pages source[i] copied to pages target[i] in every layer of every store (the copies of KVPool._copy,
     pages.py:861-869, for all of a step's shared pages at once): source, target int64 [n] on the device, a pair with a
-    negative id skipped; no target is another pair's source or target. stores and slots as compact() takes them."""
+    negative id (or one past the layer's pages) skipped; no target is another pair's source or target. stores and slots as compact() takes them."""
     live = [s for s in stores if s is not None]
     if not live:
         raise ValueError("copy_pages copies the pages of one store at least")
@@ -813,6 +813,7 @@ def copy_pages(stores, slots, source, target, page):
     if source.numel() == 0:
         return
     p.source, p.target, p.n, p.page = source.data_ptr(), target.data_ptr(), source.numel(), int(page)
+    p.pool_pages = int(slots) // int(page)
     _launch(device, "crit_pkv_copy_pages", "paged_kv_attention.copy_pages", p)
 
 

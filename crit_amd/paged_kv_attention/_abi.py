@@ -10,7 +10,7 @@ import shutil
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 NAME = "libcrit_pkv.so"
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 KIND_16BIT, KIND_FP8, KIND_FP8_ROW, KIND_INT8 = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
@@ -86,7 +86,7 @@ class CompactParams(ctypes.Structure):
 
 
 class CopyPagesParams(ctypes.Structure):
-    _fields_ = [("source", _p), ("target", _p), ("stores", Store * MAX_STORES), ("n", _i64),
+    _fields_ = [("source", _p), ("target", _p), ("stores", Store * MAX_STORES), ("n", _i64), ("pool_pages", _i64),
                 ("n_stores", _i32), ("layers", _i32), ("page", _i32)]
 
 

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 10
+#define CRIT_PKV_ABI_VERSION 11
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -274,12 +274,13 @@ int crit_pkv_compact(const crit_pkv_compact_params* p, void* stream);
 
 /* Replaces the copies of KVPool._copy (pages.py:861-869: a page shared with a fork is copied before it is written),
  * for n pages at once: every store's rows source[i] * page .. + page - 1 of every layer are copied to the rows of
- * target[i]. A pair with a negative id is skipped. No target may be another pair's source or target. */
+ * target[i]. A pair with a negative id (or one past pool_pages) is skipped. No target may be another pair's source or target. */
 typedef struct crit_pkv_copy_pages_params {
     const int64_t* source;          /* [n] page ids */
     const int64_t* target;          /* [n] */
     crit_pkv_store stores[CRIT_PKV_MAX_STORES];
     int64_t n;
+    int64_t pool_pages;             /* pages a layer holds: a pair with an id at or past it is skipped; 0: not checked */
     int32_t n_stores, layers, page;
 } crit_pkv_copy_pages_params;
 

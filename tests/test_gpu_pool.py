@@ -162,10 +162,10 @@ def test_pages_are_copied_whole_in_every_layer_and_store(kind, hkv, d, page, int
     pk = kernels()
     pages, layers = 40, 3
     stores = _stores(kind, layers, pages * page, hkv, d, 9)
-    source = torch.tensor([3, -1, 7, 39, 12, 3])
-    target = torch.tensor([0, 5, 9, 1, -1, 38])
+    source = torch.tensor([3, -1, 7, 39, 12, 3, 40, 2])      # (40: the first id past the pages)
+    target = torch.tensor([0, 5, 9, 1, -1, 38, 4, 41])
     want = [s.clone() for s in stores]
-    oracle_pool.copy_pages(want, pages * page, source, target, page)
+    oracle_pool.copy_pages(want, pages * page, source[:6], target[:6], page)      # (the last two pairs are skipped)
     got = _on_device(stores, interleaved)
     pk.copy_pages(got, pages * page, source.to(dev), target.to(dev), page)
     _same(got, want)
