@@ -88,3 +88,29 @@ def test_the_module_keeps_the_reference_interface():
     with pk.owner("a"):
         pass
     pk.release("a")
+
+
+def test_the_pool_functions_refuse_host_tensors_and_bad_shapes_before_any_launch():
+    # (host logic only: every check below fails before a kernel could be launched, so it runs without a GPU)
+    import pytest
+    import torch
+    import crit_amd.paged_kv_attention as pk
+    tables = torch.zeros(2, 4, dtype=torch.int32)
+    capacity = torch.zeros(2, dtype=torch.int64)
+    i64 = torch.zeros(3, dtype=torch.int64)
+    with pytest.raises(ValueError, match="GPU"):
+        pk.slots_at(tables, capacity, i64, i64, 16, 8)
+    with pytest.raises(ValueError, match="GPU"):
+        pk.compact([torch.zeros(1, 8, 2, 16)], 8, tables, capacity, i64, i64, torch.zeros(1, 4, dtype=torch.int64), i64, 16, 8)
+    with pytest.raises(ValueError):
+        pk.copy_pages([], 8, i64, i64, 4)
+    with pytest.raises(ValueError, match="GPU"):
+        pk.copy_pages([torch.zeros(1, 8, 2, 16)], 8, i64, i64, 4)
+    with pytest.raises(ValueError):
+        pk.rows_at(torch.zeros(8, 2, 16, dtype=torch.bfloat16), None, "bf16", i64.to(torch.int32))
+    with pytest.raises(ValueError, match="GPU"):
+        pk.rows_at(torch.zeros(8, 2, 16, dtype=torch.bfloat16), None, "bf16", i64)
+    with pytest.raises(ValueError):
+        pk.gather(torch.zeros(8, 2, 16, dtype=torch.bfloat16), None, "bf16", torch.zeros(1, dtype=torch.int32), 40, 16)
+    with pytest.raises(ValueError, match="rope rotates keys"):
+        pk.write(None, torch.zeros(1, 2, 16), i64[:1], None, torch.zeros(8, 2, 16), "bf16", rope=(None, None))
