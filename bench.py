@@ -270,6 +270,9 @@ def long_context(pk, device):
                 found[f"B{batch}_ctx{ctx}_chunk{chunk}"] = {
                     "us": round(total * 1e3, 1), "split_us": round(split * 1e3, 1), "merge_us": round((total - split) * 1e3, 1),
                     "GB/s": round(nbytes / total / 1e6, 1), "split_GB/s": round(nbytes / split / 1e6, 1)}
+            # (the default reader beside them: partitions x pieces, a partition's pieces b, b + P, ... one unit)
+            total = timed(lambda: pk.attend(q, k, v, "bf16", tables, rows, rows, firsts, 1, page, out=out), 10, 2)
+            found[f"B{batch}_ctx{ctx}_default_reader"] = {"us": round(total * 1e3, 1), "GB/s": round(nbytes / total / 1e6, 1)}
     return found
 
 
