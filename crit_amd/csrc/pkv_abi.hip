@@ -39,6 +39,16 @@ int crit_pkv_stream_read(const void* data, int64_t bytes, float* sink, void* str
     return pkv::launch_stream_read(data, bytes, sink, reinterpret_cast<hipStream_t>(stream));
 }
 
+int crit_pkv_stream_capture(void* stream, unsigned long long* id) {
+    if (!id) return CRIT_PKV_E_NULL;
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    unsigned long long found = 0;
+    const hipError_t e = hipStreamGetCaptureInfo(reinterpret_cast<hipStream_t>(stream), &status, &found);
+    if (e != hipSuccess) return (int)e;
+    *id = status == hipStreamCaptureStatusActive ? (found ? found : ~0ull) : 0;
+    return 0;
+}
+
 int crit_pkv_abi_version(void) { return CRIT_PKV_ABI_VERSION; }
 
 int crit_pkv_params_size(int which) {
@@ -58,7 +68,7 @@ int crit_pkv_params_size(int which) {
 const char* crit_pkv_error(int code) {
     switch (code) {
         case 0: return "ok";
-        case CRIT_PKV_E_GEOMETRY: return "crit_pkv: a shape the kernels do not take (head dims 64/128/256 with keys and values of one width, query heads a multiple of the KV heads, 1..64 columns, 16-byte aligned rows; pool stores in multiples of 4 bytes, tree paths of up to 256 columns)";
+        case CRIT_PKV_E_GEOMETRY: return "crit_pkv: a shape the kernels do not take (head dims 16 to 256 in powers of two (prompt chunks: 64 or 128, keys and values of one width), query heads a multiple of the KV heads, 1..64 columns, 16-byte aligned rows; pool stores in multiples of 4 bytes, tree paths of up to 256 columns)";
         case CRIT_PKV_E_DTYPE: return "crit_pkv: a dtype or page kind the kernels do not take";
         case CRIT_PKV_E_NULL: return "crit_pkv: a required pointer is NULL";
         case CRIT_PKV_E_WORKSPACE: return "crit_pkv: partitions, piece or the partial arrays do not fit the launch";

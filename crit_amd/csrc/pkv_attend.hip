@@ -19,8 +19,9 @@ PKV_DEV float lane_value(float x, int at) { return u2f((uint32_t)__builtin_amdgc
 
 template <int DV>
 __global__ __launch_bounds__(64) void merge_kernel(AttendArgs a) {
-    constexpr int EPL = DV / 64;
-    const int c = blockIdx.x, head = blockIdx.y, r = blockIdx.z, lane = threadIdx.x;
+    constexpr int EPL = DV < 64 ? 1 : DV / 64;      // (value rows narrower than a wavefront: the lanes past them idle)
+    const int c = blockIdx.x, head = blockIdx.y, r = blockIdx.z;
+    const int lane = DV < 64 ? min((int)threadIdx.x, DV - 1) : (int)threadIdx.x;
     int count = a.columns;
     if (a.counts) count = min(a.counts[r], a.columns);
     if (c >= count) return;
@@ -129,9 +130,9 @@ __global__ __launch_bounds__(64) void merge_kernel(AttendArgs a) {
 #pragma unroll
     for (int e = 0; e < EPL; ++e) {
         const float o = L != 0.0f ? A[e] / L : 0.0f;
-        store_out(a.out, a.out_dtype, token * a.o_st + (int64_t)head * a.o_sh + e * 64 + lane, o);
+        if (DV >= 64 || (int)threadIdx.x < DV) store_out(a.out, a.out_dtype, token * a.o_st + (int64_t)head * a.o_sh + e * 64 + lane, o);
     }
-    if (a.lse && lane == 0) a.lse[token * a.hq + head] = L != 0.0f ? __builtin_fmaf(M, kLn2, __logf(L)) : -INFINITY;
+    if (a.lse && threadIdx.x == 0) a.lse[token * a.hq + head] = L != 0.0f ? __builtin_fmaf(M, kLn2, __logf(L)) : -INFINITY;
 }
 
 // Shard merge: outs [parts][rows][DV], lses [parts][rows] (natural log) -> out FP32, lse; one wavefront per row.
@@ -213,48 +214,21 @@ static int pick_qr(int live_rows) {
     return 8;
 }
 
-// -- the unit-pulling launches' counters ------------------------------------------------------------------------------------
-constexpr int kTicketPairs = 64;
-static __device__ __align__(256) unsigned pkv_tickets[2 * kTicketPairs];      // zero at load; every device has its own copy
-
+// -- compute units of the current device (cached: the query is a driver call) ----------------------------------------------
 namespace {
 constexpr int kMaxDevices = 64;
-struct DeviceState {
-    std::atomic<int> cus{-1};
-    std::atomic<unsigned*> tickets{nullptr};
-    std::atomic<unsigned> next{0};
-};
-DeviceState g_devices[kMaxDevices];
-DeviceState* device_state() {
-    int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
-    return &g_devices[dev];
-}
+std::atomic<int> g_cus[kMaxDevices];      // 0: not asked yet
 }   // namespace
 
 int compute_units() {
-    DeviceState* st = device_state();
-    if (!st) return 0;
-    int n = st->cus.load(std::memory_order_relaxed);
-    if (n < 0) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-        st->cus.store(n, std::memory_order_relaxed);
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+    int n = g_cus[dev].load(std::memory_order_relaxed);
+    if (n <= 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        g_cus[dev].store(n, std::memory_order_relaxed);
     }
     return n;
-}
-
-unsigned* next_ticket() {
-    DeviceState* st = device_state();
-    if (!st) return nullptr;
-    unsigned* base = st->tickets.load(std::memory_order_acquire);
-    if (!base) {
-        void* ptr = nullptr;
-        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(pkv_tickets)) != hipSuccess || !ptr) return nullptr;
-        base = static_cast<unsigned*>(ptr);
-        st->tickets.store(base, std::memory_order_release);
-    }
-    return base + 2 * (st->next.fetch_add(1, std::memory_order_relaxed) % kTicketPairs);
 }
 
 int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
@@ -268,11 +242,13 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     if (p->n_rows < 1 || p->columns < 1 || p->columns > CRIT_PKV_MAX_COLUMNS || p->kv_heads < 1 || p->heads < 1 ||
         p->heads % p->kv_heads || p->page < 1 || p->table_width < 1 || p->sliding < 0)
         return CRIT_PKV_E_GEOMETRY;
-    if (p->head_dim != p->value_dim || (p->head_dim != 64 && p->head_dim != 128 && p->head_dim != 256)) return CRIT_PKV_E_GEOMETRY;
+    auto width_ok = [](int d) { return d == 16 || d == 32 || d == 64 || d == 128 || d == 256; };
+    if (!width_ok(p->head_dim) || !width_ok(p->value_dim)) return CRIT_PKV_E_GEOMETRY;
     if (p->q_stride_t % 8 || p->q_stride_h % 8 || (reinterpret_cast<uintptr_t>(p->q) % 16) ||
         (reinterpret_cast<uintptr_t>(p->key_pages) % 16) || (reinterpret_cast<uintptr_t>(p->value_pages) % 16))
         return CRIT_PKV_E_GEOMETRY;
-    const int lpr = p->head_dim / 8;
+    const int lpr = (p->head_dim > p->value_dim ? p->head_dim : p->value_dim) / 8;      // lanes that hold the wider row
+    const bool wide128 = p->head_dim == 128 && p->value_dim == 128;
     const int sp = 4 * (64 / lpr);
     if (p->partitions < 1 || p->partitions > 65535 || p->piece < 1 || p->piece % sp) return CRIT_PKV_E_WORKSPACE;
     if (!p->fused && (!p->partial_out || !p->partial_max || !p->partial_sum)) return CRIT_PKV_E_WORKSPACE;
@@ -288,8 +264,8 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     if (fresh) {
         if (!p->fresh_keys || !p->fresh_values || !p->fresh_shifts || !p->fresh_firsts) return CRIT_PKV_E_NULL;
         if (p->blocks) return CRIT_PKV_E_GEOMETRY;      // (block lists read the pages only, as the reference's)
-        const int64_t row = (int64_t)p->kv_heads * p->head_dim;
-        if (p->fresh_rows < 1 || p->fresh_stride_k < row || p->fresh_stride_v < row || p->fresh_stride_k % 8 || p->fresh_stride_v % 8 ||
+        const int64_t row = (int64_t)p->kv_heads * p->head_dim, row_v = (int64_t)p->kv_heads * p->value_dim;
+        if (p->fresh_rows < 1 || p->fresh_stride_k < row || p->fresh_stride_v < row_v || p->fresh_stride_k % 8 || p->fresh_stride_v % 8 ||
             (reinterpret_cast<uintptr_t>(p->fresh_keys) % 16) || (reinterpret_cast<uintptr_t>(p->fresh_values) % 16))
             return CRIT_PKV_E_GEOMETRY;
     }
@@ -313,6 +289,7 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     a.q_st = p->q_stride_t, a.q_sh = p->q_stride_h, a.o_st = p->out_stride_t, a.o_sh = p->out_stride_h, a.tab_stride = p->table_stride;
     a.tab_width = p->table_width, a.n_rows = p->n_rows, a.columns = p->columns, a.hq = p->heads, a.hkv = p->kv_heads;
     a.g = p->heads / p->kv_heads;
+    a.dk = p->head_dim, a.dv = p->value_dim;
     a.page = p->page;
     a.page_shift = -1;
     for (int s = 0; s < 31; ++s)
@@ -332,12 +309,11 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     // one and four heads. Fixed by the cache's geometry, never by the launch: a column's bits depend on it.
     // (block lists of blocks that are a multiple of 16 positions walk their lists in the 128-wide kernel, others in
     // the generic one, each position looked up on its own)
-    const bool fast_lists = p->blocks && lpr == 16 && p->page % 16 == 0 && p->block_size % 16 == 0;
+    const bool fast_lists = p->blocks && wide128 && p->page % 16 == 0 && p->block_size % 16 == 0;
     const bool page16 = p->page % 16 == 0 && !p->blocks && !fresh;      // (rows with fresh positions take the generic kernel)
     a.heads_per_wave = 1;
-    if (lpr == 16 && (page16 || fast_lists)) {
-        if (p->kv_heads % 2 == 0) a.heads_per_wave = 2;
-    }
+    a.fast128 = wide128 && (page16 || fast_lists);
+    if (a.fast128 && p->kv_heads % 2 == 0) a.heads_per_wave = 2;
     const int64_t gx = (int64_t)p->n_rows * (p->kv_heads / a.heads_per_wave) * a.tiles;
     if (gx > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
     // Positions past the page tables do not exist: partitions that could only hold such pieces are not launched.
@@ -347,11 +323,10 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     const unsigned gy = (unsigned)(live_parts < p->partitions ? live_parts : p->partitions);
     const dim3 grid((unsigned)gx, p->fused ? 1u : gy);
     a.units_x = a.units_y = 0;
-    a.ticket = nullptr;
-    if (lpr == 16 && (page16 || fast_lists)) {
-        a.ticket = next_ticket();
-        if (!a.ticket || compute_units() < 1) return CRIT_PKV_E_GEOMETRY;
-    }
+    // The unit-pulling launches draw their units from the caller's two counters; without them units are dealt in turn.
+    a.ticket = p->launch_state;
+    if (reinterpret_cast<uintptr_t>(p->launch_state) % 8) return CRIT_PKV_E_GEOMETRY;
+    if (a.fast128 && compute_units() < 1) return CRIT_PKV_E_GEOMETRY;
     auto split = [&](bool fused) -> int {
         switch (p->kind) {
             case 0: return f16 ? launch_attend_f16(a, lpr, qr, fused, page16, grid, stream)
@@ -369,6 +344,8 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     if (p->heads > 65535 || p->n_rows > 65535) return CRIT_PKV_E_GEOMETRY;
     const dim3 mgrid((unsigned)p->columns, (unsigned)p->heads, (unsigned)p->n_rows);
     switch (p->value_dim) {
+        case 16: hipLaunchKernelGGL((merge_kernel<16>), mgrid, dim3(64), 0, stream, a); break;
+        case 32: hipLaunchKernelGGL((merge_kernel<32>), mgrid, dim3(64), 0, stream, a); break;
         case 64: hipLaunchKernelGGL((merge_kernel<64>), mgrid, dim3(64), 0, stream, a); break;
         case 128: hipLaunchKernelGGL((merge_kernel<128>), mgrid, dim3(64), 0, stream, a); break;
         case 256: hipLaunchKernelGGL((merge_kernel<256>), mgrid, dim3(64), 0, stream, a); break;

@@ -625,25 +625,31 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
     }
 }
 
-// The launch: as many workgroups as the card holds at once, each taking units from a ticket counter until the list is
-// exhausted. The hardware's own dispatcher binds a workgroup to an XCD by its id and starts workgroups strictly in
-// order, so with units as uneven as ragged contexts make them it leaves slots idle behind a busy one; resident
-// workgroups that pull the next unit themselves keep every slot busy to the end. The last workgroup to finish zeroes
-// the counters for the next launch that uses them.
+// The launch: as many workgroups as the card holds at once, each taking units from the launch's counter (the caller's
+// memory) until the list is exhausted. The hardware's own dispatcher binds a workgroup to an XCD by its id and starts
+// workgroups strictly in order, so with units as uneven as ragged contexts make them it leaves slots idle behind a
+// busy one; resident workgroups that pull the next unit themselves keep every slot busy to the end. The last workgroup
+// to finish zeroes the counters for the next launch that uses them. Without counters the units are dealt in turn.
 template <int KIND, bool F16, int QR, int HW, bool FUSED, bool SPARSE = false>
 __global__ __launch_bounds__(256, attend_waves(KIND, QR)) void attend128_kernel(AttendArgs a) {
     __shared__ unsigned s_unit;
     const unsigned total = (unsigned)a.units_x * (unsigned)a.units_y;
     unsigned u = blockIdx.x;      // the first gridDim.x units need no ticket: tickets number the units after them
+    const bool pulled = a.ticket != nullptr;
     while (u < total) {
         // (the next ticket is drawn after the unit, not during it: a returning atomic in flight makes every wait on
         // the unit's loads a wait for all of them, which costs more than the ticket's round trip)
         attend128_unit<KIND, F16, QR, HW, FUSED, SPARSE>(a, (int)(u % (unsigned)a.units_x), (int)(u / (unsigned)a.units_x));
         lds_barrier();      // the unit is done with the shared arrays, and every thread has read s_unit
-        if (threadIdx.x == 0) s_unit = gridDim.x + atomicAdd(a.ticket, 1u);
-        lds_barrier();
-        u = s_unit;
+        if (pulled) {
+            if (threadIdx.x == 0) s_unit = gridDim.x + atomicAdd(a.ticket, 1u);
+            lds_barrier();
+            u = s_unit;
+        } else {
+            u += gridDim.x;
+        }
     }
+    if (!pulled) return;
     if (threadIdx.x == 0) {
         if (atomicAdd(a.ticket + 1, 1u) == gridDim.x - 1) {
             atomicExch(a.ticket, 0u);

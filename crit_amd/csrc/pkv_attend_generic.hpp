@@ -1,10 +1,12 @@
-// Paged decode / verify-window attention, generic head widths (64, 128, 256): the first, plain form of the split
-// launch, kept for the widths the 128-wide kernel does not cover.
+// Paged decode / verify-window attention, generic head widths (16 to 256, keys and values of different widths too):
+// the first, plain form of the split launch, kept for what the 128-wide kernel does not cover.
 //
 // Work unit: one workgroup of 4 wavefronts per (row, KV head, query tile, partition). A query tile is QR rows of the
 // flattened (column, query head of the KV head's group) list, so the group's heads share every K/V row read.
-// Inside a wavefront LPR = D/8 lanes hold one K (or V) row, 16 bytes each (8 bytes for 8-bit pages), so one
-// load instruction fetches 64/LPR whole rows; a step is four such loads for K and four for V. Each lane group keeps
+// Inside a wavefront LPR = max(key width, value width) / 8 lanes hold one K (or V) row, 16 bytes each (8 bytes for
+// 8-bit pages), so one load instruction fetches 64/LPR whole rows; a step is four such loads for K and four for V.
+// Where one of the two is narrower, the group's lanes past its width read its last 8 elements again and count for
+// nothing (their query slice is zero; the outputs they accumulate are not stored). Each lane group keeps
 // its own online-softmax state over the positions it reads; the groups and the four wavefronts are folded at the
 // end in a fixed order, then the partition's state goes to the partials (or, fused, into the running state).
 //
@@ -44,7 +46,7 @@ template <int KIND, bool F16, int LPR, int QR, bool FUSED, bool SPARSE = false, 
 __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
     static_assert(!(SPARSE && FUSED), "block lists are read by the split launch");
     static_assert(!(SPARSE && FRESH), "block lists read the pages only");
-    constexpr int D = LPR * 8;
+    constexpr int D = LPR * 8;         // the wider of the key and value rows
     constexpr int PPI = 64 / LPR;      // positions one load instruction of a wavefront covers
     constexpr int SP = 4 * PPI;        // positions a wavefront's step covers
     constexpr int EB = KIND == 0 ? 2 : 1;
@@ -54,6 +56,8 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
     __shared__ int s_blocks[SPARSE ? kMaxListedBlocks : 1];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lg = lane / LPR, li = lane % LPR;
+    const int dk = a.dk, dv = a.dv;                     // the rows' own widths (multiples of 8, D the wider)
+    const int lik = min(li * 8, dk - 8), liv = min(li * 8, dv - 8);      // the lane's first element of a K row and of a V row
     int bx = blockIdx.x;
     const int tile = bx % a.tiles;
     bx /= a.tiles;
@@ -120,7 +124,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
 #pragma unroll
     for (int rr = 0; rr < QR; ++rr) {
         uint4 w = make_uint4(0, 0, 0, 0);
-        if (live[rr]) {
+        if (live[rr] && li * 8 < dk) {
             w = *reinterpret_cast<const uint4*>(a.q + ((int64_t)(start + col[rr]) * a.q_st + (int64_t)qhead[rr] * a.q_sh + li * 8) * 2);
         }
         qp[rr][0] = w.x, qp[rr][1] = w.y, qp[rr][2] = w.z, qp[rr][3] = w.w;
@@ -138,9 +142,9 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
     if (KIND != 1) v_mult = 1.0f;
     const int win = a.sliding;
 
-    const uint8_t* kbase = a.kp + ((int64_t)kvh * D + li * 8) * EB;
-    const uint8_t* vbase = a.vp + ((int64_t)kvh * D + li * 8) * EB;
-    const int64_t slot_bytes = (int64_t)a.hkv * D * EB;
+    const uint8_t* kbase = a.kp + ((int64_t)kvh * dk + lik) * EB;
+    const uint8_t* vbase = a.vp + ((int64_t)kvh * dv + liv) * EB;
+    const int64_t slot_bytes_k = (int64_t)a.hkv * dk * EB, slot_bytes_v = (int64_t)a.hkv * dv * EB;
 
     auto fetch_tab = [&](int base, int (&tab)[4], int (&pos)[4]) {
 #pragma unroll
@@ -169,9 +173,9 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
             }
             const int in_page = a.page_shift >= 0 ? (n & (a.page - 1)) : (n % a.page);
             const int64_t slot = (int64_t)tab[k] * a.page + in_page;
-            buf.k[k] = *reinterpret_cast<const typename StepBuf<KIND>::Vec*>(kbase + slot * slot_bytes);
-            if constexpr (KIND == 0) buf.v[k] = load_once16(vbase + slot * slot_bytes);
-            else buf.v[k] = load_once8(vbase + slot * slot_bytes);
+            buf.k[k] = *reinterpret_cast<const typename StepBuf<KIND>::Vec*>(kbase + slot * slot_bytes_k);
+            if constexpr (KIND == 0) buf.v[k] = load_once16(vbase + slot * slot_bytes_v);
+            else buf.v[k] = load_once8(vbase + slot * slot_bytes_v);
             if constexpr (KIND >= 2) {
                 buf.ks[k] = a.ks[slot * a.hkv + kvh];
                 buf.vs[k] = a.vs[slot * a.hkv + kvh];
@@ -179,8 +183,8 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
             if constexpr (FRESH) {      // (unconditional too: a position below the first fresh one reads row 0 or its own clamped)
                 int64_t row = (int64_t)n - f_shift;
                 row = row < 0 ? 0 : (row >= a.f_rows ? a.f_rows - 1 : row);
-                buf.f.k[k] = *reinterpret_cast<const uint4*>(a.fk + (row * a.f_stride_k + (int64_t)kvh * D + li * 8) * 2);
-                buf.f.v[k] = load_once16(a.fv + (row * a.f_stride_v + (int64_t)kvh * D + li * 8) * 2);
+                buf.f.k[k] = *reinterpret_cast<const uint4*>(a.fk + (row * a.f_stride_k + (int64_t)kvh * dk + lik) * 2);
+                buf.f.v[k] = load_once16(a.fv + (row * a.f_stride_v + (int64_t)kvh * dv + liv) * 2);
             }
         }
     };
@@ -419,7 +423,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
                 if constexpr (!(FRESH && KIND == 1)) A *= v_mult;      // (with fresh rows the multiplier went in a position at a time)
                 const int j = j0 + rr;
                 const int c = j / a.g;
-                if (c < count) {
+                if (c < count && d < dv) {
                     if constexpr (FUSED) {
                         // A column folds the partitions that hold its positions, as the merge does.
                         const int held = min(a.parts, (min(first + c + 1, a.max_keys) + a.piece - 1) / a.piece);
@@ -431,7 +435,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
                     } else {
                         const int64_t prow = a.offsets ? (int64_t)(a.offsets[r] - a.offsets[0]) : (int64_t)r * a.columns;
                         const int64_t at = ((prow + c) * a.hq + kvh * a.g + j % a.g) * a.parts + b;
-                        a.po[at * D + d] = A;
+                        a.po[at * dv + d] = A;
                         if (d == 0) a.pm[at] = M, a.pl[at] = L;
                     }
                 }
@@ -446,7 +450,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
                 const int rr = idx / D, d = idx % D;
                 const int j = j0 + rr;
                 const int c = j / a.g;
-                if (c < count) {
+                if (c < count && d < dv) {
                     const int head = kvh * a.g + j % a.g;
                     float M = run_m[e], L = run_l[e], A = run_a[e];
                     if (a.sinks) {

@@ -10,7 +10,7 @@ namespace pkv {
 template <int KIND, bool F16, int QR, bool FUSED>
 static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipStream_t stream) {
     if constexpr (!FUSED) {
-        if (a.blocks && lpr == 16 && a.page % 16 == 0 && a.block_size % 16 == 0) {
+        if (a.blocks && a.fast128) {
             // block lists whose steps lie in one block and one page: the bandwidth path walking each column's list
             AttendArgs u = a;
             u.units_x = (int)grid.x, u.units_y = (int)grid.y + kTailClasses - 1;
@@ -27,6 +27,8 @@ static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipS
         }
         if (a.blocks) {      // other block lists: the generic kernel, each position looked up on its own
             switch (lpr) {
+                case 2: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 2, QR, false, true>), grid, dim3(256), 0, stream, a); break;
+                case 4: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 4, QR, false, true>), grid, dim3(256), 0, stream, a); break;
                 case 8: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 8, QR, false, true>), grid, dim3(256), 0, stream, a); break;
                 case 16: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 16, QR, false, true>), grid, dim3(256), 0, stream, a); break;
                 case 32: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 32, QR, false, true>), grid, dim3(256), 0, stream, a); break;
@@ -35,7 +37,7 @@ static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipS
             return hip_code(hipGetLastError());
         }
     }
-    if (lpr == 16 && page16) {       // pages of a multiple of 16 positions: the bandwidth path, resident workgroups pulling units
+    if (a.fast128 && !a.blocks) {       // 128-wide heads, pages of a multiple of 16 positions: the bandwidth path, resident workgroups pulling units
         AttendArgs u = a;
         // (a split launch lists a row's last partition twice, for the one of two size classes it falls in)
         u.units_x = (int)grid.x, u.units_y = FUSED ? (int)grid.y : (int)grid.y + kTailClasses - 1;
@@ -46,11 +48,12 @@ static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipS
         switch (a.heads_per_wave) {
             case 1: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 1, FUSED>), pgrid, dim3(256), 0, stream, u); break;
             case 2: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 2, FUSED>), pgrid, dim3(256), 0, stream, u); break;
-            case 4: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 4, FUSED>), pgrid, dim3(256), 0, stream, u); break;
             default: return CRIT_PKV_E_GEOMETRY;
         }
     } else if (a.fk) {       // fresh rows beside the pages: the generic kernel's variant that reads both (any head width)
         switch (lpr) {
+            case 2: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 2, QR, FUSED, false, true>), grid, dim3(256), 0, stream, a); break;
+            case 4: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 4, QR, FUSED, false, true>), grid, dim3(256), 0, stream, a); break;
             case 8: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 8, QR, FUSED, false, true>), grid, dim3(256), 0, stream, a); break;
             case 16: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 16, QR, FUSED, false, true>), grid, dim3(256), 0, stream, a); break;
             case 32: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 32, QR, FUSED, false, true>), grid, dim3(256), 0, stream, a); break;
@@ -62,6 +65,10 @@ static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipS
         hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 8, QR, FUSED>), grid, dim3(256), 0, stream, a);
     } else if (lpr == 32) {
         hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 32, QR, FUSED>), grid, dim3(256), 0, stream, a);
+    } else if (lpr == 4) {
+        hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 4, QR, FUSED>), grid, dim3(256), 0, stream, a);
+    } else if (lpr == 2) {
+        hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 2, QR, FUSED>), grid, dim3(256), 0, stream, a);
     } else {
         return CRIT_PKV_E_GEOMETRY;
     }

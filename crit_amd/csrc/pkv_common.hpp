@@ -133,12 +133,12 @@ PKV_DEV float dpp(float x) {
     return u2f((uint32_t)__builtin_amdgcn_update_dpp(0, (int)f2u(x), CTRL, 0xf, 0xf, true));
 }
 
-// Sum over the LANES (8, 16 or 32, a power of two) lanes of each aligned group; every lane gets the same bits.
+// Sum over the LANES (2 to 64, a power of two) lanes of each aligned group; every lane gets the same bits.
 template <int LANES>
 PKV_DEV float group_sum(float x) {
     x += dpp<0xB1>(x);
-    x += dpp<0x4E>(x);
-    x += dpp<0x141>(x);
+    if constexpr (LANES >= 4) x += dpp<0x4E>(x);
+    if constexpr (LANES >= 8) x += dpp<0x141>(x);
     if constexpr (LANES >= 16) x += dpp<0x140>(x);
     if constexpr (LANES >= 32) x += __shfl_xor(x, 16);
     if constexpr (LANES >= 64) x += __shfl_xor(x, 32);
@@ -147,8 +147,8 @@ PKV_DEV float group_sum(float x) {
 template <int LANES>
 PKV_DEV float group_max(float x) {
     x = __builtin_fmaxf(x, dpp<0xB1>(x));
-    x = __builtin_fmaxf(x, dpp<0x4E>(x));
-    x = __builtin_fmaxf(x, dpp<0x141>(x));
+    if constexpr (LANES >= 4) x = __builtin_fmaxf(x, dpp<0x4E>(x));
+    if constexpr (LANES >= 8) x = __builtin_fmaxf(x, dpp<0x141>(x));
     if constexpr (LANES >= 16) x = __builtin_fmaxf(x, dpp<0x140>(x));
     if constexpr (LANES >= 32) x = __builtin_fmaxf(x, __shfl_xor(x, 16));
     if constexpr (LANES >= 64) x = __builtin_fmaxf(x, __shfl_xor(x, 32));

@@ -16,8 +16,4 @@ int launch_read_rows(const crit_pkv_read_params* p, hipStream_t stream);
 int launch_stream_read(const void* data, int64_t bytes, float* sink, hipStream_t stream);
 // Compute units of the current device (cached per device), or 0 if the query fails.
 int compute_units();
-// Two zeroed device counters for one unit-pulling launch on the current device, from a ring of 64 pairs the library
-// holds per device (launches that are in flight together use different pairs as long as fewer than 64 overlap; the
-// kernel zeroes its pair again when its last workgroup finishes). Null if the device query fails.
-unsigned* next_ticket();
 }   // namespace pkv

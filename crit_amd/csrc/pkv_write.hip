@@ -295,9 +295,7 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
                 __builtin_amdgcn_sched_barrier(0);
             }
             coded = coded && sum == sum;
-#ifndef NO_COLD
             if (__builtin_expect(!coded, 0)) exact_codes<KIND>(raw[u], div, w);
-#endif
             if (live[u]) __builtin_nontemporal_store(u32x4{w[0], w[1], w[2], w[3]}, reinterpret_cast<u32x4*>(reinterpret_cast<uint8_t*>(pages) + dst));
         }
     }

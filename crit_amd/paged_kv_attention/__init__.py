@@ -43,6 +43,7 @@ PIECE = 2048         # positions per piece of FP8 or INT8 pages at a 128-wide he
 MAX_COLUMNS = 64     # columns of one row a launch reads
 MAX_LISTED_BLOCKS = 1024      # block ids a token's list holds at most (attend's blocks=)
 MAX_QUERY_ROWS = 8   # query rows (columns x group heads) one workgroup holds; wider windows take more tiles
+HEAD_WIDTHS = (16, 32, 64, 128, 256)      # key and value head widths attend() reads, in any pairing
 
 _DTYPE = {torch.float32: _abi.F32, torch.bfloat16: _abi.BF16, torch.float16: _abi.F16}
 
@@ -65,59 +66,121 @@ def _unsupported(what):
     return NotImplementedError(f"paged_kv_attention (gfx950): {what} is not served by these kernels")
 
 
-# -- owners and module workspaces (reference __init__.py:129-171) --------------------------------------------------------
-_workspaces = {}
-_retired = []      # workspaces a launch outgrew: a captured graph may still replay into them, so they are kept
-_owner = threading.local()
+# -- owners: what the module itself keeps on a device (reference __init__.py:129-171 keeps its workspaces the same way) --
+class _Holding:
+    """One owner's memory on one device: the partials of its split launches, the row states of its prompt chunks with
+    fresh rows, and the counters its unit-pulling launches draw from. Buffers a launch outgrew stay in `kept`: a
+    captured graph may still replay into them."""
+    __slots__ = ("partials", "states", "counters", "pairs_used", "pair_of", "kept")
+
+    def __init__(self):
+        self.partials = self.states = self.counters = None
+        self.pairs_used, self.pair_of, self.kept = 0, {}, []
 
 
-@contextlib.contextmanager
-def owner(key):
-    """Launches inside this block take module workspaces of their own, apart from every other owner's."""
-    before = getattr(_owner, "key", None)
-    _owner.key = key
-    try:
-        yield
-    finally:
-        _owner.key = before
+COUNTER_PAIRS = 512      # counter pairs an owner's block holds (one a stream that launches, one a capture)
+_holdings = {}           # (device index, owner key) -> _Holding
+_local = threading.local()
+
+
+class owner:
+    """`with owner(key):` — the launches inside take module memory of their own (partials, prompt-row states, launch
+    counters), apart from every other owner's and from launches outside any block; a graph captured inside replays
+    into its owner's memory. Nests; per thread. release(key) drops the memory."""
+
+    def __init__(self, key):
+        self.key = key
+
+    def __enter__(self):
+        stack = _local.__dict__.setdefault("owners", [])
+        stack.append(self.key)
+        return self
+
+    def __exit__(self, *exc):
+        _local.owners.pop()
+        return False
+
+
+def _owner_key():
+    stack = getattr(_local, "owners", None)
+    return stack[-1] if stack else None
 
 
 def release(key):
-    """Drop an owner's module workspaces (its captured graphs must be gone)."""
-    for held in (_workspaces, _states):
-        for at in [at for at in held if at[1] == key]:
-            del held[at]
-    _retired[:] = [(k, found) for k, found in _retired if k != key]
+    """Forget everything the module holds for owner `key`, on every device (its captured graphs must be gone first:
+    they replay into that memory)."""
+    for at in [at for at in _holdings if at[1] == key]:
+        _holdings.pop(at)
 
 
-def _held(device):
-    return (str(device), getattr(_owner, "key", None))
+def _holding(device):
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    at = (index, _owner_key())
+    found = _holdings.get(at)
+    if found is None:
+        found = _holdings[at] = _Holding()
+    return found
+
+
+def _grown(holding, name, floats, device, floor, what):
+    """The holding's FP32 buffer `name`, at least `floats` long; grown (never under a capture) by replacing it."""
+    found = getattr(holding, name)
+    if found is None or found.numel() < floats:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError(f"paged_kv_attention.{what} (the module allocates outside a capture only)")
+        if found is not None:
+            holding.kept.append(found)
+        found = torch.empty(max(floats, floor), dtype=torch.float32, device=device)
+        setattr(holding, name, found)
+    return found
+
+
+def _launch_state(device, stream):
+    """The address of the two counters a unit-pulling launch on `stream` draws from: one pair per (owner, device,
+    stream) for eager launches, which run one after another there, and one per (capture, stream) for captured ones, so
+    a replaying graph never meets an eager launch or another graph in its counters, whatever streams they run on.
+    The pairs come from a zeroed block the owner holds; a launch leaves its pair zero."""
+    holding = _holding(device)
+    capture = _abi.capture_id(stream)
+    at = holding.pair_of.get((stream, capture))
+    if at is None:
+        if holding.counters is None or holding.pairs_used == COUNTER_PAIRS:
+            if capture:
+                raise RuntimeError("paged_kv_attention.attend: run a launch once on this device before capturing one "
+                                   "(its launch counters are allocated, zeroed, outside a capture)")
+            if holding.counters is not None:
+                holding.kept.append(holding.counters)
+            holding.counters, holding.pairs_used = torch.zeros(2 * COUNTER_PAIRS, dtype=torch.int32, device=device), 0
+        at = holding.pair_of[(stream, capture)] = holding.counters.data_ptr() + 8 * holding.pairs_used
+        holding.pairs_used += 1
+    return at
 
 
 def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
-def _stream(device):
-    return torch.cuda.current_stream(device).cuda_stream
-
-
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)      # (the stream's handle without a Stream object)
 
 
-def _launch(device, name, what, *args):
-    """Calls entry point `name` with args and the caller's current stream of `device` as its last argument, with
-    `device` current (a decode step calls this about a hundred times: the device is switched only where it is not the
-    current one already); raises what _abi.check raises."""
-    index = device.index
-    current = torch.cuda.current_device()
+def _stream_of(device):
+    """The handle of the caller's current stream on `device`."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    return _raw_stream(index) if _raw_stream is not None else torch.cuda.current_stream(device).cuda_stream
+
+
+def _launch(device, name, what, *args, stream=None):
+    """Calls entry point `name` with args and the caller's current stream of `device` (or `stream`, its handle) as its
+    last argument, with `device` current (a decode step calls this about a hundred times: the device is switched only
+    where it is not the current one already); raises what _abi.check raises."""
     entry = getattr(_abi.load(), name)
-    if index is None or index == current:
-        stream = _raw_stream(current) if _raw_stream is not None else torch.cuda.current_stream(device).cuda_stream
+    if stream is None:
+        stream = _stream_of(device)
+    if device.index is None or device.index == torch.cuda.current_device():
         code = entry(*args, stream)
     else:
         with torch.cuda.device(device):
-            code = entry(*args, _stream(device))
+            code = entry(*args, stream)
     if code:
         _abi.check(code, what)
 
@@ -128,26 +191,35 @@ def _require_device(t, what):
 
 
 def _check_kind(kind, key_scales):
-    if kind not in KINDS:
-        raise ValueError(f"page kinds are {', '.join(KINDS)}, not {kind!r}")
-    if (KINDS[kind] >= 2) != (key_scales is not None):
-        raise ValueError(f"{kind} pages {'take' if KINDS[kind] >= 2 else 'have no'} scales per position and head")
-    return KINDS[kind]
+    """The kind's number; row-scaled kinds come with their scales, the others without."""
+    number = KINDS.get(kind)
+    if number is None:
+        raise ValueError(f"{kind!r} is no page kind ({', '.join(KINDS)})")
+    row_scaled, given = number >= 2, key_scales is not None
+    if row_scaled and not given:
+        raise ValueError(f"{kind} pages are read with their scales (one per position and KV head)")
+    if given and not row_scaled:
+        raise ValueError(f"{kind} pages carry no scales per position")
+    return number
 
 
 def _check_sliding(sliding, blocks):
-    sliding = int(sliding or 0)
-    if sliding < 0:
-        raise ValueError("a sliding window is 0 (none) or a number of positions")
-    if sliding and blocks is not None:
-        raise ValueError("a sliding window reads windows without block lists")
-    return sliding
+    width = int(sliding) if sliding else 0
+    if width < 0:
+        raise ValueError(f"sliding={sliding}: a window's width in positions, or 0 for none")
+    if width > 0 and blocks is not None:
+        raise ValueError("sliding windows and block lists do not combine")
+    return width
 
 
 def _check_sinks(sinks, q):
-    if sinks is not None and (sinks.dtype != torch.float32 or sinks.dim() != 1 or sinks.shape[0] != q.shape[1] or
-                              not sinks.is_contiguous() or sinks.device != q.device):
-        raise ValueError(f"sinks are contiguous FP32 [{q.shape[1]}] (one a query head) on q's device")
+    if sinks is None:
+        return
+    heads = q.shape[1]
+    ok = (sinks.dtype == torch.float32 and tuple(sinks.shape) == (heads,) and sinks.is_contiguous()
+          and sinks.device == q.device)
+    if not ok:
+        raise ValueError(f"sinks: one FP32 logit per query head ([{heads}], contiguous, on q's device)")
 
 
 def _multipliers(multipliers, kv_heads, device):
@@ -217,22 +289,18 @@ def workspace_floats(tokens, heads, partitions, value_dim):
 
 
 def _workspace(device, tokens, heads, parts, dv, given=None):
-    need = tokens * heads * parts
-    if given is not None:
-        if given.dtype != torch.float32 or given.numel() < need * (dv + 2) or not given.is_contiguous():
-            raise ValueError(f"attend's workspace holds {given.numel()} floats; this launch needs {need * (dv + 2)} "
-                             "(workspace_floats)")
-        return given[:need * dv], given[need * dv:need * (dv + 1)], given[need * (dv + 1):need * (dv + 2)]
-    found = _workspaces.get(_held(device))
-    if found is None or found.numel() < need * (dv + 2):
-        if torch.cuda.is_current_stream_capturing():
-            raise RuntimeError("paged_kv_attention.attend: run a launch of this size once before capturing it (its "
-                               "partials' workspace is allocated outside the capture)")
-        if found is not None:
-            _retired.append((getattr(_owner, "key", None), found))
-        found = _workspaces[_held(device)] = torch.empty(max(need, 4096) * (dv + 2), dtype=torch.float32,
-                                                         device=device)
-    return found[:need * dv], found[need * dv:need * (dv + 1)], found[need * (dv + 1):need * (dv + 2)]
+    """(partial outputs, maxima, sums) of a split launch: three views of the caller's FP32 workspace, or of the one the
+    current owner holds on the device."""
+    states = tokens * heads * parts
+    floats = states * (dv + 2)
+    if given is None:
+        given = _grown(_holding(device), "partials", floats, device, 4096 * (dv + 2),
+                       "attend: run a launch of this size once before capturing it")
+    elif given.dtype != torch.float32 or not given.is_contiguous() or given.numel() < floats:
+        raise ValueError(f"workspace: {floats} contiguous FP32 floats for this launch (workspace_floats()), "
+                         f"{given.numel()} given")
+    outs, rest = given[:states * dv], given[states * dv:]
+    return outs, rest[:states], rest[states:2 * states]
 
 
 # -- writes ----------------------------------------------------------------------------------------------------------------
@@ -425,8 +493,8 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
         raise ValueError("query heads a multiple of the KV heads, 1..64 columns a row, one row or more")
     if q.stride(-1) != 1:
         raise ValueError("q's last dimension is contiguous")
-    if d != dv or d not in (64, 128, 256):
-        raise ValueError("head dims are 64, 128 or 256, keys and values of one width")
+    if d not in HEAD_WIDTHS or dv not in HEAD_WIDTHS or key_pages.shape[-1] != d:
+        raise ValueError(f"head widths are powers of two from 16 to 256 (q's, keys' and values'), not {d} and {dv}")
     want_q = torch.float16 if kind == "fp16" else torch.bfloat16
     if q.dtype != want_q:
         raise ValueError(f"q is {want_q} over {kind} pages, not {q.dtype}")
@@ -439,6 +507,8 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
         raise ValueError("counts and offsets are int32")
     partial_rows = R * columns if offsets is None else int(tokens)
     device = q.device
+    if key_pages.device != device or value_pages.device != device or tables.device != device:
+        raise ValueError("q, the pages and the page tables live on one device")
     block = flash_block(d, dv, hq, hkv, page, kind)
     if flash:
         piece = int(chunk or flash_chunk(d, dv, hq, hkv, page, kind))
@@ -448,8 +518,11 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
     else:
         parts = int(partitions or globals()["partitions"](device, hkv, kind, d, dv))
         piece = int(piece or piece_size(d, dv, kind, hkv))
-        if piece % block:
-            raise ValueError(f"a piece ({piece} positions) is a multiple of {block} at this head width")
+        if piece < 1:
+            raise ValueError(f"a piece is a number of positions, not {piece}")
+        # A piece is a whole number of the wavefronts' steps: one that is not (crit's piece option admits 16 to 128,
+        # a step at narrow heads is up to 128 positions) is read as the next multiple. Still one piece per cache.
+        piece = -(-piece // block) * block
     scale = float(scale if scale is not None else d ** -0.5)
     if fused:
         po = pm = pl = None
@@ -500,7 +573,9 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
         p.fresh_shifts, p.fresh_firsts = fshift.data_ptr(), ffirst.data_ptr()
         p.fresh_stride_k, p.fresh_stride_v, p.fresh_rows = fk.stride(0), fv.stride(0), int(fk.shape[0])
         p.fresh_per_row = int(fshift.numel() != 1)
-    _launch(device, "crit_pkv_attend", "paged_kv_attention.attend", p)
+    stream = _stream_of(device)
+    p.launch_state = _launch_state(device, stream)
+    _launch(device, "crit_pkv_attend", "paged_kv_attention.attend", p, stream=stream)
     return out
 
 
@@ -532,26 +607,16 @@ def prefill_state_floats(tokens, heads, dim):
     return tokens * heads * (dim + 4)
 
 
-_states = {}
-
-
 def _prefill_state(device, tokens, heads, dim, given):
     need = prefill_state_floats(tokens, heads, dim)
-    if given is not None:
-        if given.dtype != torch.float32 or given.numel() < need or not given.is_contiguous() or given.device != device \
-                or given.data_ptr() % 16:
-            raise ValueError(f"a prompt chunk with fresh rows needs {need} contiguous FP32 floats of workspace on its "
-                             "device, 16-byte aligned (prefill_state_floats)")
-        return given
-    found = _states.get(_held(device))
-    if found is None or found.numel() < need:
-        if torch.cuda.is_current_stream_capturing():
-            raise RuntimeError("paged_kv_attention.prefill: run a chunk of this size with fresh rows once before "
-                               "capturing it, or pass workspace= (the rows' states are allocated outside the capture)")
-        if found is not None:
-            _retired.append((getattr(_owner, "key", None), found))
-        found = _states[_held(device)] = torch.empty(max(need, 1 << 16), dtype=torch.float32, device=device)
-    return found
+    if given is None:
+        return _grown(_holding(device), "states", need, device, 1 << 16,
+                      "prefill: run a chunk of this size with fresh rows once before capturing it, or pass workspace=")
+    if given.dtype != torch.float32 or given.numel() < need or not given.is_contiguous() or given.device != device \
+            or given.data_ptr() % 16:
+        raise ValueError(f"a prompt chunk with fresh rows needs {need} contiguous FP32 floats of workspace on its "
+                         "device, 16-byte aligned (prefill_state_floats)")
+    return given
 
 
 def _check_fresh(fresh, q, hkv, d, chunks):
@@ -589,6 +654,10 @@ def _prefill_launch(q, key_pages, value_pages, kind, tables, table_rows, starts,
     if q.dtype != want_q:
         raise ValueError(f"q is {want_q} over {kind} pages, not {q.dtype}")
     device = q.device
+    if d not in (64, 128):
+        return _prefill_as_windows(q, key_pages, value_pages, kind, tables, table_rows, starts, counts, positions,
+                                   max_count, chunks, page, key_scales, value_scales, multipliers, scale, out, lse,
+                                   sinks, sliding, fresh, int8_qk)
     out = torch.empty_like(q) if out is None else out
     if out.dtype not in _DTYPE or out.stride(-1) != 1:
         raise ValueError("out is [tokens][heads][dim] BF16, FP16 or FP32, its last dimension contiguous")
@@ -624,7 +693,42 @@ def _prefill_launch(q, key_pages, value_pages, kind, tables, table_rows, starts,
     return out
 
 
-_positions = {}
+def _prefill_as_windows(q, key_pages, value_pages, kind, tables, table_rows, starts, counts, positions, max_count,
+                        chunks, page, key_scales, value_scales, multipliers, scale, out, lse, sinks, sliding, fresh,
+                        int8_qk):
+    """Prompt chunks at the head widths the matrix-core kernel does not take (16, 32, 256): every chunk cut into window
+    rows of up to MAX_COLUMNS tokens and read by attend()'s fused launch, as crit itself reads prompt rows with
+    prompt_reader decode (device_attention.py:751-783). The rows' metadata is computed on the device from the chunks'
+    (no length is read on the host)."""
+    if int8_qk:
+        raise _unsupported(f"int8_qk at head width {q.shape[-1]}")
+    device, hq = q.device, q.shape[1]
+    if q.shape[-1] not in HEAD_WIDTHS:
+        raise ValueError(f"head widths are powers of two from 16 to 256, not {q.shape[-1]}")
+    per = -(-int(max_count) // MAX_COLUMNS)                                   # window rows a chunk
+    step = torch.arange(per, dtype=torch.int64, device=device) * MAX_COLUMNS   # each one's first column in its chunk
+    zero = torch.zeros(chunks, dtype=torch.int64, device=device)
+    first_token = zero if starts is None else starts.to(torch.int64)
+    length = torch.full((chunks,), int(max_count), dtype=torch.int64, device=device) if counts is None else counts.to(torch.int64)
+    table_of = torch.arange(chunks, dtype=torch.int64, device=device) if table_rows is None else table_rows.to(torch.int64)
+    w_starts = (first_token[:, None] + step[None, :]).reshape(-1).to(torch.int32)
+    w_firsts = (positions[:, None] + step[None, :]).reshape(-1).contiguous()
+    w_counts = (length[:, None] - step[None, :]).clamp(0, MAX_COLUMNS).reshape(-1).to(torch.int32)
+    w_rows = table_of[:, None].expand(chunks, per).reshape(-1).to(torch.int32)
+    given = None
+    if fresh is not None:      # a chunk's own rows sit beside q's tokens: row = position - (chunk position - first token)
+        fk, fv, firsts = _check_fresh(fresh, q, key_pages.shape[-2], q.shape[-1], chunks)
+        shift = positions - first_token
+        own = positions if firsts is None else torch.maximum(firsts, positions)
+        given = (fk, fv, shift[:, None].expand(chunks, per).reshape(-1).contiguous(),
+                 own[:, None].expand(chunks, per).reshape(-1).contiguous())
+    if tables.dtype != torch.int32:
+        tables = tables.to(torch.int32)
+    if out is None:
+        out = torch.empty(q.shape[0], hq, value_pages.shape[-1], dtype=q.dtype, device=device)
+    return attend(q, key_pages, value_pages, kind, tables, w_rows, w_starts, w_firsts, MAX_COLUMNS, page,
+                  counts=w_counts, key_scales=key_scales, value_scales=value_scales, multipliers=multipliers,
+                  scale=scale, out=out, lse=lse, fused=True, fresh=given, sinks=sinks, sliding=sliding)
 
 
 def prefill(q, key_pages, value_pages, kind, table, position, page, *, key_scales=None, value_scales=None,

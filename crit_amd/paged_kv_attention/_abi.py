@@ -10,7 +10,7 @@ import shutil
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 NAME = "libcrit_pkv.so"
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 KIND_16BIT, KIND_FP8, KIND_FP8_ROW, KIND_INT8 = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
@@ -43,7 +43,7 @@ class AttendParams(ctypes.Structure):
                 ("scale", _f32), ("key_multiplier", _f32), ("value_multiplier", _f32),
                 ("fresh_keys", _p), ("fresh_values", _p), ("fresh_shifts", _p), ("fresh_firsts", _p),
                 ("fresh_stride_k", _i64), ("fresh_stride_v", _i64), ("fresh_rows", _i64), ("fresh_per_row", _i32),
-                ("rows_are_64", _i32)]
+                ("rows_are_64", _i32), ("launch_state", _p)]
 
 
 class MergeParams(ctypes.Structure):
@@ -99,7 +99,7 @@ class ReadParams(ctypes.Structure):
 
 SYMBOLS = ("crit_pkv_write", "crit_pkv_attend", "crit_pkv_merge", "crit_pkv_prefill", "crit_pkv_slots_at",
            "crit_pkv_compact", "crit_pkv_copy_pages", "crit_pkv_read_rows", "crit_pkv_abi_version", "crit_pkv_params_size", "crit_pkv_error",
-           "crit_pkv_stream_read")
+           "crit_pkv_stream_read", "crit_pkv_stream_capture")
 
 _lib = None
 
@@ -150,6 +150,8 @@ def load():
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(struct), ctypes.c_void_p]
+    lib.crit_pkv_stream_capture.restype = ctypes.c_int
+    lib.crit_pkv_stream_capture.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_ulonglong)]
     lib.crit_pkv_stream_read.restype = ctypes.c_int
     lib.crit_pkv_stream_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
     if lib.crit_pkv_abi_version() != ABI_VERSION:
@@ -162,6 +164,17 @@ def load():
     lib.path = path
     _lib = lib
     return lib
+
+
+_capture = ctypes.c_ulonglong()
+
+
+def capture_id(stream):
+    """The id of the capture `stream` (a handle) is recording into, 0 when it is not capturing."""
+    code = load().crit_pkv_stream_capture(stream, ctypes.byref(_capture))
+    if code:
+        check(code, "crit_pkv_stream_capture")
+    return _capture.value
 
 
 def check(code, what):

@@ -1,9 +1,11 @@
 /* crit_pkv: C ABI of the MI355X (gfx950) paged-KV kernels.
  *
  * The boundary a host binds (ctypes, cgo, JNI ...): plain pointers and sizes, one POD parameter struct per entry
- * point, the caller's HIP stream. Every buffer is caller-owned device memory; the library owns none. Nothing here
- * allocates, synchronises or reads a length on the host: row lengths and positions are read on the device, so one
- * launch shape (a captured HIP graph) serves every length.
+ * point, the caller's HIP stream. Every buffer is caller-owned device memory, the counters of a launch included
+ * (crit_pkv_attend_params.launch_state): the library keeps no state between calls, so two owners' launches, eager or
+ * replayed from captured graphs, never meet in memory neither of them passed. Nothing here allocates, synchronises or
+ * reads a length on the host: row lengths and positions are read on the device, so one launch shape (a captured HIP
+ * graph) serves every length.
  *
  * Each entry point replaces the kernel launches behind one function of the reference's kernels module
  * (kernels/techniques/attention/paged-kv-attention/torch-ext/paged_kv_attention/__init__.py); the pattern of the ABI
@@ -22,7 +24,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 11
+#define CRIT_PKV_ABI_VERSION 12
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -149,6 +151,14 @@ typedef struct crit_pkv_attend_params {
     /* rows holds int64 entries (a captured round hands the reader its round slots as they are, int64:
      * inference/attention-state/code/device_attention.py:573, core/python/crit_plugins/device.py:661,681). */
     int32_t rows_are_64;
+    /* The launch's two counters (next unit, workgroups done): 8 bytes of device memory, 8-byte aligned, zero before the
+     * first launch that uses them; a launch leaves them zero when its last workgroup ends. Resident workgroups draw
+     * their units of work from them, which keeps every compute unit busy when the rows' lengths differ. Launches that
+     * may run at the same time (other streams, another owner's captured graph replaying) take different counters;
+     * launches one after another on a stream share theirs. The reference keeps such state per owner in its module
+     * (__init__.py:141-171); here it is the caller's, like every other buffer. NULL: units are dealt to the
+     * workgroups in turn, no counters (the same bits; slower on ragged batches). */
+    uint32_t* launch_state;
 } crit_pkv_attend_params;
 
 int crit_pkv_attend(const crit_pkv_attend_params* p, void* stream);
@@ -319,6 +329,10 @@ int crit_pkv_abi_version(void);
  * (which: 0 write, 1 attend, 2 merge, 3 prefill, 4 slots_at, 5 compact, 6 copy_pages, 7 read_rows), as crit_cw_params_size() does (cuda_window.cu:1502). */
 int crit_pkv_params_size(int which);
 const char* crit_pkv_error(int code);
+/* *id = the id of the capture `stream` is recording into (never 0), or 0 when it is not capturing; returns 0 or a HIP
+ * error code. For hosts that key a launch's counters (crit_pkv_attend_params.launch_state) by capture, so that a
+ * replaying graph never shares them with an eager launch. No counterpart in the reference. */
+int crit_pkv_stream_capture(void* stream, unsigned long long* id);
 /* A streaming-read probe: sums `bytes` (a multiple of 16) of device memory into sink[0..63]; the achievable-HBM-read
  * yardstick the benchmark prints beside the nominal peak. No counterpart in the reference. */
 int crit_pkv_stream_read(const void* data, int64_t bytes, float* sink, void* stream);

@@ -23,7 +23,12 @@ def _close_lse(got, want, what=None):
     torch.testing.assert_close(got.double().cpu(), want, atol=1e-3, rtol=1e-4, msg=None if what is None else str(what))
 
 
-SHAPES = [(8, 2, 128, 128), (32, 8, 128, 128), (40, 8, 128, 128), (24, 4, 256, 256), (12, 2, 64, 64), (56, 8, 128, 128)]
+# The reference's own shapes (test_paged_kv_attention.py:129, keys and values of different widths among them), the
+# benchmark's, one and three KV heads (a wavefront of the 128-wide kernel then serves one head, not two), and the
+# narrowest heads.
+SHAPES = [(8, 2, 128, 128), (32, 8, 128, 128), (40, 8, 128, 128), (24, 4, 256, 256), (12, 2, 64, 128), (12, 2, 64, 64),
+          (56, 8, 128, 128), (6, 1, 128, 128), (12, 3, 128, 128), (8, 2, 128, 64), (4, 2, 16, 32), (6, 1, 32, 16),
+          (5, 1, 256, 64)]
 
 
 @pytest.mark.parametrize("kind", KINDS)
@@ -91,10 +96,11 @@ def test_the_cpu_reference_configuration():
 
 
 @pytest.mark.parametrize("kind", ["bf16", "fp8", "fp8:row", "int8"])
-def test_rows_and_columns_are_invariant_bit_for_bit(kind):
+@pytest.mark.parametrize("hkv,d,dv", [(4, 128, 128), (1, 128, 128), (3, 128, 128), (2, 64, 128)])
+def test_rows_and_columns_are_invariant_bit_for_bit(kind, hkv, d, dv):
     pk = kernels()
-    cache = Cache(kind, 4, 128, 128, 16, [700, 300, 2100])
-    q = rand_q(24, 16, 128, 5)
+    cache = Cache(kind, hkv, d, dv, 16, [700, 300, 2100])
+    q = rand_q(24, 4 * hkv, d, 5)
     together = cache.attend(q, [0, 1, 2], [0, 8, 16], [690, 290, 2090], 8)
     for s, start, first in zip([0, 1, 2], [0, 8, 16], [690, 290, 2090]):
         alone = cache.attend(q[start:start + 8], [s], [0], [first], 8)
@@ -107,7 +113,7 @@ def test_rows_and_columns_are_invariant_bit_for_bit(kind):
         assert torch.equal(wide, together[start:start + 8])
     counts = torch.tensor([3, 1, 4], dtype=torch.int32, device=dev)
     offsets = torch.tensor([0, 3, 4], dtype=torch.int32, device=dev)
-    floats = pk.workspace_floats(8, 16, pk.partitions(dev, 4, kind), 128)
+    floats = pk.workspace_floats(8, 4 * hkv, pk.partitions(dev, hkv, kind), dv)
     packed = cache.attend(q, [0, 1, 2], [0, 8, 16], [690, 290, 2090], 8, counts=counts, offsets=offsets, tokens=8,
                           workspace=torch.full((floats,), float("nan"), dtype=torch.float32, device=dev))
     for start, count in zip([0, 8, 16], [3, 1, 4]):
@@ -123,10 +129,11 @@ def test_a_count_past_the_columns_reads_as_the_columns():
 
 
 @pytest.mark.parametrize("kind", ["bf16", "fp8", "int8"])
-@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (24, 4, 256)])
-def test_a_fused_launch_gives_a_column_the_split_launchs_bits(kind, hq, hkv, d):
+@pytest.mark.parametrize("hq,hkv,d,dv", [(32, 8, 128, 128), (24, 4, 256, 256), (6, 1, 128, 128), (12, 3, 128, 128),
+                                         (12, 2, 64, 128)])
+def test_a_fused_launch_gives_a_column_the_split_launchs_bits(kind, hq, hkv, d, dv):
     for length in (40, 700, 5000):
-        cache = Cache(kind, hkv, d, d, 64, [length], seed=1)
+        cache = Cache(kind, hkv, d, dv, 64, [length], seed=1)
         T = min(130, length)
         pos0 = length - T
         q = rand_q(T, hq, d, 2)
@@ -449,9 +456,9 @@ def test_bad_geometry_is_refused():
 
 
 def test_launches_that_overlap_on_two_streams_do_not_share_counters():
-    # The split launch's workgroups pull their units from a counter pair the launch takes from a ring: launches in
-    # flight together (two streams here, many each) must not disturb one another, and every one must leave its pair
-    # zeroed for the launch that gets it next (130 launches go round the ring of 64 twice).
+    # The split launch's workgroups pull their units from two counters the module hands the launch, one pair per
+    # stream: launches in flight together (two streams here, many each) must not disturb one another, and every one
+    # must leave its pair zeroed for the next launch on its stream.
     caches = [Cache("bf16", 4, 128, 128, 16, [3000, 1700, 900], seed=s) for s in (1, 2)]
     qs = [rand_q(3, 16, 128, 20 + s) for s in range(2)]
     want = [c.attend(q, [0, 1, 2], [0, 1, 2], [2999, 1699, 899], 1) for c, q in zip(caches, qs)]
@@ -470,6 +477,82 @@ def test_launches_that_overlap_on_two_streams_do_not_share_counters():
     for i in range(2):
         for got in outs[i]:
             assert torch.equal(got, want[i])
+
+
+def test_an_owners_graph_replays_beside_another_owners_eager_launches():
+    # Owner A captures a step of 32 launches and replays it on one stream while owner B issues more than 64 eager
+    # launches on another: each owner's launch counters and partials are its own (a captured launch bakes its counters'
+    # address in, so it must never be an address an eager launch or another graph is handed), and both get the bits
+    # of their launches run alone.
+    pk = kernels()
+    lengths = [3000, 1700, 900, 2500]
+    caches = [Cache("bf16", 4, 128, 128, 16, lengths, seed=s) for s in (31, 32)]
+    qs = [rand_q(4, 16, 128, 40 + s) for s in range(2)]
+    firsts = [n - 1 for n in lengths]
+    rows = torch.arange(4, dtype=torch.int32, device=dev)
+    firsts_t = torch.tensor(firsts, dtype=torch.int64, device=dev)
+    want = [c.attend(q, rows, rows, firsts_t, 1) for c, q in zip(caches, qs)]
+    torch.cuda.synchronize()
+    layers = 32
+    out_a = torch.zeros(layers, 4, 16, 128, dtype=torch.bfloat16, device=dev)
+
+    def step_a():
+        for layer in range(layers):
+            caches[0].attend(qs[0], rows, rows, firsts_t, 1, out=out_a[layer])
+    with pk.owner("a"):
+        step_a()      # (the owner's partials and counters are allocated outside the capture)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step_a()
+    streams = [torch.cuda.Stream() for _ in range(2)]
+    got_b = []
+    for rep in range(3):
+        out_a.zero_()
+        torch.cuda.synchronize()
+        with torch.cuda.stream(streams[0]):
+            graph.replay()
+        with torch.cuda.stream(streams[1]), pk.owner("b"):
+            for i in range(70):
+                got_b.append(caches[1].attend(qs[1], rows, rows, firsts_t, 1))
+        torch.cuda.synchronize()
+        for layer in range(layers):
+            assert torch.equal(out_a[layer], want[0]), (rep, layer)
+    for got in got_b:
+        assert torch.equal(got, want[1])
+    # the two owners hold different counters, and a capture's are not the eager stream's
+    held = {key: h for key, h in pk._holdings.items() if key[1] in ("a", "b")}
+    assert len(held) == 2
+    pairs = [at for h in held.values() for at in h.pair_of.values()]
+    assert len(pairs) == len(set(pairs)) >= 3
+    pk.release("a"), pk.release("b")
+    assert not [key for key in pk._holdings if key[1] in ("a", "b")]
+
+
+def test_a_launch_without_counters_deals_its_units_in_turn():
+    # The C ABI with launch_state NULL (a host that keeps no counters): units are dealt to the workgroups in turn,
+    # the same bits as the pulled launch.
+    from crit_amd.paged_kv_attention import _abi
+    cache = Cache("fp8", 8, 128, 128, 16, [5000, 300, 1200, 64, 2048, 4097], seed=33)
+    q = rand_q(6, 32, 128, 34)
+    rows = torch.arange(6, dtype=torch.int32, device=dev)
+    firsts = torch.tensor([n - 1 for n in cache.lengths], dtype=torch.int64, device=dev)
+    want = cache.attend(q, rows, rows, firsts, 1)
+    lib, seen = _abi.load(), []
+    real = lib.crit_pkv_attend
+
+    def without_counters(params, stream):
+        params.launch_state = None
+        seen.append(1)
+        return real(params, stream)
+    lib.crit_pkv_attend = without_counters
+    try:
+        got = cache.attend(q, rows, rows, firsts, 1)
+    finally:
+        lib.crit_pkv_attend = real
+    torch.cuda.synchronize()
+    assert len(seen) == 1
+    assert torch.equal(got, want)
 
 
 def test_more_units_than_resident_workgroups_and_ragged_rows():

@@ -1,7 +1,8 @@
 """The benchmark configurations at their full sizes (Llama-3-8B-shaped bf16 decode, FP8 decode at batch 128, 200k-token
 split-K decode, chunked prefill mixed with decode): every row of every launch against textbook float64 attention over
-the STORED values, computed densely by torch on the GPU (the oracle's reference() formula; anchored here against the
-CPU oracle on sampled rows), plus what does not depend on size: a fused launch and each row alone give the split
+the STORED values, computed densely by torch on the GPU (the oracle's reference() formula), and in every configuration
+sampled rows of the launch directly against the CPU oracle (oracle.attend.window_reference over the pages copied
+back), plus what does not depend on size: a fused launch and each row alone give the split
 launch's bits, every chunk size of the contiguous splits agrees, appended bytes read back equal the oracle's encoding.
 Tolerances: 2e-2 for 16-bit pages, 5e-2 for FP8 pages (outputs), 2e-3 for the log-sum-exp."""
 import math
@@ -39,21 +40,44 @@ class Pool:
         self.k = torch.zeros(self.pages + 1, PAGE, HKV, D, dtype=store, device=dev)
         self.v = torch.zeros(self.pages + 1, PAGE, HKV, D, dtype=store, device=dev)
         self.mult = (1.0, 1.0)
-        if kind == "fp8":      # per-(layer, KV head) multipliers: amax / 448 over what is appended (N(0,1), 1 % x 20)
-            self.mult = torch.tensor([[20.0 * 4.5 / 448.0] * HKV, [20.0 * 4.4 / 448.0] * HKV], device=dev)
-        for s, n in enumerate(lengths):
-            keys = torch.randn(n, HKV, D, device=dev, generator=g)
-            values = torch.randn(n, HKV, D, device=dev, generator=g)
+
+        def rows_of(s, n):      # sequence s's keys and values, the same at every call
+            gs = torch.Generator(device=dev).manual_seed(seed * 100003 + s)
+            keys = torch.randn(n, HKV, D, device=dev, generator=gs)
+            values = torch.randn(n, HKV, D, device=dev, generator=gs)
             if outliers:
-                keys = torch.where(torch.rand(n, HKV, D, device=dev, generator=g) < 0.01, keys * 20, keys)
-                values = torch.where(torch.rand(n, HKV, D, device=dev, generator=g) < 0.01, values * 20, values)
+                keys = torch.where(torch.rand(n, HKV, D, device=dev, generator=gs) < 0.01, keys * 20, keys)
+                values = torch.where(torch.rand(n, HKV, D, device=dev, generator=gs) < 0.01, values * 20, values)
             else:
                 keys, values = keys * 0.5, values * 0.5
-            self.pk.write(keys.bfloat16(), values.bfloat16(), self.slots(s, 0, n), self.k, self.v, kind, multipliers=self.mult)
+            return keys.bfloat16(), values.bfloat16()
+        if kind == "fp8":      # per-(layer, KV head) multipliers: amax / 448 over the rows appended (N(0,1), 1 % x 20)
+            top = torch.zeros(2, HKV, device=dev)
+            for s, n in enumerate(lengths):
+                keys, values = rows_of(s, n)
+                top[0] = torch.maximum(top[0], keys.float().abs().amax((0, 2)))
+                top[1] = torch.maximum(top[1], values.float().abs().amax((0, 2)))
+            self.mult = (top / 448.0).contiguous()
+        for s, n in enumerate(lengths):
+            keys, values = rows_of(s, n)
+            self.pk.write(keys, values, self.slots(s, 0, n), self.k, self.v, kind, multipliers=self.mult)
 
     def slots(self, s, start, n):
         p = torch.arange(start, start + n, device=dev)
         return self.tables[s][p // PAGE].long() * PAGE + p % PAGE
+
+    def oracle_rows(self, q, tokens, s, first, tol, out, lse, what):
+        """Tokens `tokens` of q / out / lse (consecutive columns of one window row of sequence s, the first at position
+        `first`) against the CPU oracle over the pages as they are stored."""
+        if not hasattr(self, "_cpu"):
+            self._cpu = (self.k.cpu(), self.v.cpu(), self.tables.cpu())
+        k, v, tables = self._cpu
+        mult = (1.0, 1.0) if self.kind != "fp8" else (self.mult[0].cpu(), self.mult[1].cpu())
+        count = tokens.stop - tokens.start
+        want, want_lse = oracle_attend.window_reference(q[tokens].float().cpu(), k, v, self.kind, tables[s], first, count,
+                                                        PAGE, D ** -0.5, multipliers=mult)
+        torch.testing.assert_close(out[tokens].double().cpu(), want, atol=tol, rtol=tol, msg=lambda m: f"{what} vs the oracle: {m}")
+        torch.testing.assert_close(lse[tokens].double().cpu(), want_lse, atol=2e-3, rtol=1e-3, msg=lambda m: f"{what} lse vs the oracle: {m}")
 
     def stored(self, s, n):
         """Positions 0 .. n - 1 of sequence s as float64 (keys, values) [n][HKV][D]: the codes times their multiplier."""
@@ -121,15 +145,9 @@ def test_a_decode_step_of_the_8b_shape_at_its_batch_and_lengths(kind, B, low, hi
         k, v = pool.stored(s, n + 1)
         want, want_lse = dense(q[s:s + 1], k, v, n, scale)
         check(out[s:s + 1], lse[s:s + 1], want, want_lse, tol, f"row {s} of {n + 1} positions")
-    # the dense reference itself against the CPU oracle, on the shortest row
-    k, v = pool.stored(0, lengths[0] + 1)
-    want, want_lse = dense(q[:1], k, v, lengths[0], scale)
-    seen = torch.ones(lengths[0] + 1, dtype=torch.bool)
-    ref, ref_lse = oracle_attend.reference(q[0].double().cpu(), k.cpu(), v.cpu(), seen, scale)
-    # (the GPU library's float64 products agree with the CPU's to about 1e-6 of the values here, four orders below
-    # the bound the kernels are held to)
-    torch.testing.assert_close(want[0].cpu(), ref, atol=1e-5, rtol=1e-5)
-    torch.testing.assert_close(want_lse[0].cpu(), ref_lse, atol=1e-5, rtol=1e-5)
+    # the launch's shortest and longest rows and one between, directly against the CPU oracle
+    for s in (0, 1, B // 2):
+        pool.oracle_rows(q, slice(s, s + 1), s, lengths[s], tol, out, lse, f"row {s}")
     # what does not depend on size: the fused launch and a row alone give the split launch's bits
     fused, fused_lse = decode_all(pool, q, firsts, fused=True)
     assert torch.equal(out, fused) and torch.equal(lse, fused_lse)
@@ -153,6 +171,8 @@ def test_long_contexts_through_contiguous_splits_and_their_merge(B, context):
         out, lse = decode_all(pool, q, firsts, **({} if chunk is None else dict(flash=True, chunk=chunk)))
         for s in range(B):
             check(out[s:s + 1], lse[s:s + 1], wants[s][0], wants[s][1], 2e-2, f"chunk {chunk} row {s}")
+        if B == 1 or chunk is None:      # a row of each context directly against the CPU oracle (200k: every reader)
+            pool.oracle_rows(q, slice(B - 1, B), B - 1, context - 1, 2e-2, out, lse, f"chunk {chunk} row {B - 1}")
         found[chunk] = (out, lse)
     # every cut of the positions gives the same sum to rounding: the log-sum-exp of any two chunk sizes agrees far
     # inside the bound against the reference
@@ -187,6 +207,11 @@ def test_prompt_chunks_on_prefixes_mixed_with_decode_rows():
         t = 8 * T + r
         want, want_lse = dense(q[t:t + 1], k, v, n, scale)
         check(out[t:t + 1], lse[t:t + 1], want, want_lse, 2e-2, f"decode row {r}")
+    # directly against the CPU oracle: the chunk that starts its sequence, the last columns of the one on the longest
+    # prefix, and a decode row
+    pool.oracle_rows(q, slice(3 * T, 3 * T + T), 3, 0, 2e-2, out, lse, "chunk 3")
+    pool.oracle_rows(q, slice(6 * T + T - 3, 6 * T + T), 6, prefixes[6] + T - 3, 2e-2, out, lse, "chunk 6's last columns")
+    pool.oracle_rows(q, slice(8 * T + 5, 8 * T + 6), 8 + 5, decodes[5], 2e-2, out, lse, "decode row 5")
     # a prompt token's output is the same position decoded, to the readers' rounding
     c, t = 2, 300
     one = pk.attend(q[c * T + t:c * T + t + 1], pool.k, pool.v, "bf16", pool.tables, i32([c]), i32([0]),

@@ -32,6 +32,30 @@ def test_prompt_chunks_match_float64_attention(kind, hq, hkv, d):
     _check(cache, q, out, lse, 200, (0, 37, 63, 64, 99))
 
 
+@pytest.mark.parametrize("kind", ["bf16", "fp8:row"])
+@pytest.mark.parametrize("hq,hkv,d", [(24, 4, 256), (4, 2, 32), (6, 1, 16)])
+def test_prompt_chunks_at_the_other_head_widths_go_through_window_rows(kind, hq, hkv, d):
+    # Head widths the matrix-core kernel does not take: the chunk is read as window rows of up to 64 columns by the
+    # decode reader's fused launch (what crit does with prompt_reader decode); the same contract, fresh rows included.
+    pk = kernels()
+    cache = Cache(kind, hkv, d, d, 16, [300])
+    q = rand_q(150, hq, d, 4)
+    lse = torch.empty(150, hq, device=dev)
+    out = pk.prefill(q.bfloat16(), cache.k, cache.v, kind, cache.tables[0].long(), 150, 16, key_scales=cache.ks,
+                     value_scales=cache.vs, lse=lse)
+    _check(cache, q, out, lse, 150, (0, 63, 64, 127, 128, 149))
+    position = torch.tensor([150], dtype=torch.int64, device=dev)
+    assert torch.equal(pk.prefill(q.bfloat16(), cache.k, cache.v, kind, cache.tables[0], position, 16,
+                                  key_scales=cache.ks, value_scales=cache.vs), out)
+    g = torch.Generator().manual_seed(8)
+    fk, fv = torch.randn(150, hkv, d, generator=g).bfloat16().to(dev), torch.randn(150, hkv, d, generator=g).bfloat16().to(dev)
+    got = pk.prefill(q.bfloat16(), cache.k, cache.v, kind, cache.tables[0], 150, 16, key_scales=cache.ks,
+                     value_scales=cache.vs, fresh=(fk, fv, 200))
+    for t in (0, 49, 50, 149):
+        want, _ = cache.want(q[t:t + 1], 0, 150 + t, 1, fresh=(fk.cpu(), fv.cpu(), 150, 200))
+        torch.testing.assert_close(got[t:t + 1].double().cpu(), want, atol=ATOL, rtol=RTOL, msg=f"fresh token {t}")
+
+
 @pytest.mark.parametrize("position,T", [(0, 1), (0, 512), (1, 17), (1000, 512), (8191, 33)])
 def test_chunks_at_any_position_and_length(position, T):
     pk = kernels()

@@ -213,7 +213,7 @@ def test_bad_arguments_are_refused():
     x = torch.zeros(2, 1, 64, device=dev)
     with pytest.raises(ValueError):
         pk.write(None, None, torch.zeros(2, dtype=torch.int64, device=dev), None, None, "bf16")
-    with pytest.raises(ValueError, match="page kinds"):
+    with pytest.raises(ValueError, match="page kind"):
         pk.write(x, None, torch.zeros(2, dtype=torch.int64, device=dev), k, None, "fp4")
     with pytest.raises(ValueError, match="scales"):
         pk.write(x, None, torch.zeros(2, dtype=torch.int64, device=dev), k, None, "int8")
