@@ -11,6 +11,10 @@ int crit_pkv_attend(const crit_pkv_attend_params* p, void* stream) {
     return pkv::launch_attend(p, reinterpret_cast<hipStream_t>(stream));
 }
 
+int crit_pkv_attend_static(const crit_pkv_attend_params* p, void* stream) {
+    return pkv::launch_attend_static(p, reinterpret_cast<hipStream_t>(stream));
+}
+
 int crit_pkv_merge(const crit_pkv_merge_params* p, void* stream) {
     return pkv::launch_merge(p, reinterpret_cast<hipStream_t>(stream));
 }
@@ -73,6 +77,7 @@ const char* crit_pkv_error(int code) {
         case CRIT_PKV_E_NULL: return "crit_pkv: a required pointer is NULL";
         case CRIT_PKV_E_WORKSPACE: return "crit_pkv: partitions, piece or the partial arrays do not fit the launch";
     }
+    if (code == CRIT_PKV_E_SCRATCH) return "crit_pkv: the launch's partials (rows x columns x heads x partitions x (value_dim + 2) floats) do not fit the library's static scratch (CRIT_PKV_STATIC_SCRATCH_BYTES), or its address could not be had: use crit_pkv_attend with a workspace";
     if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
     return "crit_pkv: unknown error";
 }

@@ -353,4 +353,54 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     return hip_code(hipGetLastError());
 }
 
+// -- the entry point that allocates nothing ------------------------------------------------------------------------------
+// The split launch's partials and its two counters in memory the library itself holds: a file-scope device array, one
+// copy per GPU at its own address (looked up once per device, with that device current). Every call on a GPU shares
+// that GPU's array.
+static __device__ __align__(256) unsigned char scratch[CRIT_PKV_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int64_t kScratchHead = 256;      // the counters' share of the array; the partials follow
+std::atomic<unsigned char*> g_scratch[kMaxDevices];
+
+unsigned char* scratch_of_current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    unsigned char* ptr = g_scratch[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        void* found = nullptr;
+        if (hipGetSymbolAddress(&found, HIP_SYMBOL(scratch)) != hipSuccess || !found) return nullptr;
+        ptr = static_cast<unsigned char*>(found);
+        g_scratch[dev].store(ptr, std::memory_order_release);
+    }
+    return ptr;
+}
+}   // namespace
+
+__global__ __launch_bounds__(64) void clear_counters_kernel(unsigned* counters) {
+    if (threadIdx.x < 2) counters[threadIdx.x] = 0u;
+}
+
+int launch_attend_static(const crit_pkv_attend_params* p, hipStream_t stream) {
+    if (!p) return CRIT_PKV_E_NULL;
+    if (p->n_rows < 1 || p->columns < 1 || p->heads < 1 || p->partitions < 1 || p->value_dim < 1) return CRIT_PKV_E_GEOMETRY;
+    // The partial rows a launch may write: every row's columns (rows packed by offsets take fewer).
+    const int64_t states = (int64_t)p->n_rows * p->columns * p->heads * p->partitions;
+    const int64_t need = p->fused ? 0 : states * ((int64_t)p->value_dim + 2) * (int64_t)sizeof(float);
+    if (states > (int64_t)1 << 40 || kScratchHead + need > (int64_t)CRIT_PKV_STATIC_SCRATCH_BYTES) return CRIT_PKV_E_SCRATCH;
+    unsigned char* base = scratch_of_current_device();
+    if (!base) return CRIT_PKV_E_SCRATCH;
+    crit_pkv_attend_params q = *p;
+    q.launch_state = reinterpret_cast<uint32_t*>(base);
+    float* partials = reinterpret_cast<float*>(base + kScratchHead);
+    q.partial_out = p->fused ? nullptr : partials;
+    q.partial_max = p->fused ? nullptr : partials + states * p->value_dim;
+    q.partial_sum = p->fused ? nullptr : partials + states * ((int64_t)p->value_dim + 1);
+    // The counters start at zero whatever the last call left (a fill kernel: a captured graph replays it as it is).
+    hipLaunchKernelGGL(clear_counters_kernel, dim3(1), dim3(64), 0, stream, reinterpret_cast<unsigned*>(base));
+    const int rc = hip_code(hipGetLastError());
+    if (rc) return rc;
+    return launch_attend(&q, stream);
+}
+
 }   // namespace pkv

@@ -7,6 +7,7 @@
 namespace pkv {
 int launch_write(const crit_pkv_write_params* p, hipStream_t stream);
 int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream);
+int launch_attend_static(const crit_pkv_attend_params* p, hipStream_t stream);
 int launch_merge(const crit_pkv_merge_params* p, hipStream_t stream);
 int launch_prefill(const crit_pkv_prefill_params* p, hipStream_t stream);
 int launch_slots_at(const crit_pkv_slots_params* p, hipStream_t stream);

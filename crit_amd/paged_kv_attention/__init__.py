@@ -431,7 +431,7 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
            offsets=None, tokens=None, key_scales=None, value_scales=None, multipliers=(1.0, 1.0), scale=None,
            partitions=None, parents=None, blocks=None, block_size=None, out=None, lse=None, workspace=None, piece=None,
            fused=False, fresh=None, vsplit=None, tile=None, num_warps=None, num_stages=None, maxnreg=None,
-           flash=False, chunk=None, ramp=None, sinks=None, sliding=0, derive=None, phases=0):
+           flash=False, chunk=None, ramp=None, sinks=None, sliding=0, derive=None, phases=0, static=False):
     """Decode and verify windows over paged KV (see the module's description).
 
     q [tokens][heads][dim] BF16 or FP16 (FP16 for "fp16" pages); key_pages/value_pages one layer's pages, key_scales/
@@ -457,7 +457,9 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
     prompt chunk's own keys and values as the projections gave them, unscaled), shift and first int64 device tensors
     of one element a row, or of one element for every row; not with block lists; such launches take the generic
     kernel, split or fused, the same bits either way. derive is not served. phases (a measurement's): 1 runs the split
-    launch only, 2 the merge only."""
+    launch only, 2 the merge only. static: the launch takes its partials and counters from the library's static device
+    array (crit_pkv_attend_static: for callers that cannot allocate; the same bits; launches that overlap on one GPU
+    race there; refused past _abi.STATIC_SCRATCH_BYTES of partials); no workspace is read."""
     if derive is not None:
         raise _unsupported("derive= (keys derived from value rows)")
     if parents is not None:
@@ -524,7 +526,7 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
         # a step at narrow heads is up to 128 positions) is read as the next multiple. Still one piece per cache.
         piece = -(-piece // block) * block
     scale = float(scale if scale is not None else d ** -0.5)
-    if fused:
+    if fused or static:
         po = pm = pl = None
     else:
         po, pm, pl = _workspace(device, partial_rows, hq, parts, dv, workspace)
@@ -573,6 +575,9 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
         p.fresh_shifts, p.fresh_firsts = fshift.data_ptr(), ffirst.data_ptr()
         p.fresh_stride_k, p.fresh_stride_v, p.fresh_rows = fk.stride(0), fv.stride(0), int(fk.shape[0])
         p.fresh_per_row = int(fshift.numel() != 1)
+    if static:
+        _launch(device, "crit_pkv_attend_static", "paged_kv_attention.attend", p)
+        return out
     stream = _stream_of(device)
     p.launch_state = _launch_state(device, stream)
     _launch(device, "crit_pkv_attend", "paged_kv_attention.attend", p, stream=stream)

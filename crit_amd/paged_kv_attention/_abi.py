@@ -97,7 +97,9 @@ class ReadParams(ctypes.Structure):
                 ("page_dtype", _i32), ("out_dtype", _i32), ("key_multiplier", _f32), ("value_multiplier", _f32)]
 
 
-SYMBOLS = ("crit_pkv_write", "crit_pkv_attend", "crit_pkv_merge", "crit_pkv_prefill", "crit_pkv_slots_at",
+STATIC_SCRATCH_BYTES = 32 << 20
+
+SYMBOLS = ("crit_pkv_write", "crit_pkv_attend", "crit_pkv_attend_static", "crit_pkv_merge", "crit_pkv_prefill", "crit_pkv_slots_at",
            "crit_pkv_compact", "crit_pkv_copy_pages", "crit_pkv_read_rows", "crit_pkv_abi_version", "crit_pkv_params_size", "crit_pkv_error",
            "crit_pkv_stream_read", "crit_pkv_stream_capture")
 
@@ -144,6 +146,7 @@ def load():
     lib.crit_pkv_error.argtypes = [ctypes.c_int]
     lib.crit_pkv_params_size.argtypes = [ctypes.c_int]
     for name, struct in (("crit_pkv_write", WriteParams), ("crit_pkv_attend", AttendParams),
+                         ("crit_pkv_attend_static", AttendParams),
                          ("crit_pkv_merge", MergeParams), ("crit_pkv_prefill", PrefillParams),
                          ("crit_pkv_slots_at", SlotsParams), ("crit_pkv_compact", CompactParams),
                          ("crit_pkv_copy_pages", CopyPagesParams), ("crit_pkv_read_rows", ReadParams)):

@@ -41,6 +41,7 @@ extern "C" {
 #define CRIT_PKV_E_DTYPE (-2)       /* a dtype/kind combination the kernels do not take */
 #define CRIT_PKV_E_NULL (-3)        /* a required pointer is NULL */
 #define CRIT_PKV_E_WORKSPACE (-4)   /* partitions/piece/workspace pointers inconsistent */
+#define CRIT_PKV_E_SCRATCH (-5)     /* crit_pkv_attend_static: the launch needs more than the static scratch holds */
 
 #define CRIT_PKV_MAX_COLUMNS 64
 
@@ -162,6 +163,19 @@ typedef struct crit_pkv_attend_params {
 } crit_pkv_attend_params;
 
 int crit_pkv_attend(const crit_pkv_attend_params* p, void* stream);
+
+/* crit_pkv_attend for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): no counterpart in the reference, whose module allocates its workspaces itself.
+ * The same launches and the same bits as crit_pkv_attend, with the partial arrays and the launch counters taken from
+ * a static device array of CRIT_PKV_STATIC_SCRATCH_BYTES that the library holds on every GPU it runs on until the
+ * process ends; partial_out, partial_max, partial_sum and launch_state of `p` are not read. Inputs and outputs are
+ * the caller's as before. Calls nothing that allocates. Refused with CRIT_PKV_E_SCRATCH when 256 + n_rows * columns *
+ * heads * partitions * (value_dim + 2) * 4 bytes exceed the array (fused launches need the 256 only). With offsets,
+ * offsets[r] - offsets[0] + columns <= n_rows * columns for every row (rows packed by their counts are).
+ * Every call on one GPU uses that GPU's one array: calls that may overlap there (two streams, two threads, a graph
+ * replaying beside eager calls) race on the partials and the counters; run them one after another. */
+#define CRIT_PKV_STATIC_SCRATCH_BYTES (32 * 1024 * 1024)
+int crit_pkv_attend_static(const crit_pkv_attend_params* p, void* stream);
 
 /* ---- merge of shard partials ---------------------------------------------------------------------------------------
  * Replaces PartitionedAttention.merge (inference/partitioned-attention/plugin.py:52-64): outs [parts][n][value_dim]
