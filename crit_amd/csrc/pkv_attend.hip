@@ -303,7 +303,6 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
         for (int q : {2, 4, 5, 6, 8})
             if (a.g % q == 0) qr = q;
     }
-    a.tiles = (live_rows + qr - 1) / qr;
     // The 128-wide kernel serves two adjacent KV heads per wavefront where the head count is even, so every position
     // is read in segments of two rows (512 bytes of 16-bit pages, 256 of 8-bit ones): measured best on MI355X against
     // one and four heads. Fixed by the cache's geometry, never by the launch: a column's bits depend on it.
@@ -312,8 +311,15 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     const bool fast_lists = p->blocks && wide128 && p->page % 16 == 0 && p->block_size % 16 == 0;
     const bool page16 = p->page % 16 == 0 && !p->blocks && !fresh;      // (rows with fresh positions take the generic kernel)
     a.heads_per_wave = 1;
-    a.fast128 = wide128 && (page16 || fast_lists);
+    // The bandwidth kernel walks pages that are powers of two from 16 positions up, in positions below 2^31; other
+    // multiples of 16 take the generic kernel. (block lists of blocks that are a multiple of 16: their own variant)
+    const bool pow2_page = a.page_shift >= 4 && (int64_t)p->partitions * p->piece <= 0x3fffffff;
+    a.fast128 = wide128 && ((page16 && pow2_page) || fast_lists);
     if (a.fast128 && p->kv_heads % 2 == 0) a.heads_per_wave = 2;
+    // Query rows a tile holds: the generic and block-list kernels' tile height; 16 a wavefront's heads share in the
+    // bandwidth kernel (matrix tiles of 16 columns).
+    const int tile_rows = a.fast128 && !p->blocks ? 16 / a.heads_per_wave : qr;
+    a.tiles = (live_rows + tile_rows - 1) / tile_rows;
     const int64_t gx = (int64_t)p->n_rows * (p->kv_heads / a.heads_per_wave) * a.tiles;
     if (gx > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
     // Positions past the page tables do not exist: partitions that could only hold such pieces are not launched.

@@ -27,11 +27,6 @@
 
 namespace pkv {
 
-// A workgroup barrier that orders the shared arrays only: a wavefront waits for its own LDS traffic, then for the
-// others. __syncthreads() would also wait until the wavefront's global stores (a unit's partials, which only the next
-// kernel reads) have drained, a memory round trip at every barrier of a unit's end.
-PKV_DEV void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-
 // DPP controls inside a row of 16 lanes.
 constexpr int kXor1 = 0xB1, kXor2 = 0x4E, kRor4 = 0x124, kRor8 = 0x128, kRor12 = 0x12C;
 

@@ -53,6 +53,11 @@ struct AttendArgs {
     int f_per_row;
 };
 
+// A workgroup barrier that orders the shared arrays only: a wavefront waits for its own LDS traffic, then for the
+// others. __syncthreads() would also wait until the wavefront's global stores (a unit's partials, which only the next
+// kernel reads) have drained, a memory round trip at every barrier of a unit's end.
+PKV_DEV void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // A 16-byte (or 8-byte) load of value rows, which are read once: nontemporal, so the caches do not keep them (measured
 // +4 % on the decode launch; the same hint on the key rows measured -1 %, so those stay plain loads).
 PKV_DEV uint4 load_once16(const uint8_t* p) {

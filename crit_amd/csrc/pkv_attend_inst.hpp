@@ -1,6 +1,7 @@
 // Launch of the split (or fused) kernels for ONE page kind; each pkv_attend_k*.hip instantiates one kind so the
 // kinds compile in parallel.
 #pragma once
+#include "pkv_attend_mfma.hpp"
 #include "pkv_attend128.hpp"
 #include "pkv_attend_generic.hpp"
 #include "pkv_launch.hpp"
@@ -37,20 +38,7 @@ static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipS
             return hip_code(hipGetLastError());
         }
     }
-    if (a.fast128 && !a.blocks) {       // 128-wide heads, pages of a multiple of 16 positions: the bandwidth path, resident workgroups pulling units
-        AttendArgs u = a;
-        // (a split launch lists a row's last partition twice, for the one of two size classes it falls in)
-        u.units_x = (int)grid.x, u.units_y = FUSED ? (int)grid.y : (int)grid.y + kTailClasses - 1;
-        const int64_t units = (int64_t)u.units_x * u.units_y;
-        if (units > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
-        const int64_t resident = (int64_t)compute_units() * attend_waves(KIND, QR);
-        const dim3 pgrid((unsigned)(units < resident ? units : resident));
-        switch (a.heads_per_wave) {
-            case 1: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 1, FUSED>), pgrid, dim3(256), 0, stream, u); break;
-            case 2: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 2, FUSED>), pgrid, dim3(256), 0, stream, u); break;
-            default: return CRIT_PKV_E_GEOMETRY;
-        }
-    } else if (a.fk) {       // fresh rows beside the pages: the generic kernel's variant that reads both (any head width)
+    if (a.fk) {       // fresh rows beside the pages: the generic kernel's variant that reads both (any head width)
         switch (lpr) {
             case 2: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 2, QR, FUSED, false, true>), grid, dim3(256), 0, stream, a); break;
             case 4: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 4, QR, FUSED, false, true>), grid, dim3(256), 0, stream, a); break;
@@ -75,8 +63,31 @@ static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipS
     return hip_code(hipGetLastError());
 }
 
+// 128-wide heads over pages of a multiple of 16 positions: the bandwidth path, resident workgroups pulling units.
+template <int KIND, bool F16>
+static int launch_mfma(const AttendArgs& a, bool fused, dim3 grid, hipStream_t stream) {
+    AttendArgs u = a;
+    // (a split launch lists a row's last partition once more for each size class it may fall in)
+    u.units_x = (int)grid.x, u.units_y = fused ? (int)grid.y : (int)grid.y + kTailClasses - 1;
+    const int64_t units = (int64_t)u.units_x * u.units_y;
+    if (units > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
+    const int64_t resident = (int64_t)compute_units() * kMfmaWaves;
+    const dim3 pgrid((unsigned)(units < resident ? units : resident));
+    const bool masked = a.parents != nullptr || a.parents64 != nullptr || a.sliding > 0;
+    const int which = (a.heads_per_wave == 2 ? 4 : 0) + (fused ? 2 : 0) + (masked ? 1 : 0);
+    switch (which) {
+#define PKV_MFMA(W, HWV, FU, MA) \
+    case W: hipLaunchKernelGGL((attend_mfma_kernel<KIND, F16, HWV, FU, MA>), pgrid, dim3(256), 0, stream, u); break;
+        PKV_MFMA(0, 1, false, false) PKV_MFMA(1, 1, false, true) PKV_MFMA(2, 1, true, false) PKV_MFMA(3, 1, true, true)
+        PKV_MFMA(4, 2, false, false) PKV_MFMA(5, 2, false, true) PKV_MFMA(6, 2, true, false) PKV_MFMA(7, 2, true, true)
+#undef PKV_MFMA
+    }
+    return hip_code(hipGetLastError());
+}
+
 template <int KIND, bool F16>
 static int launch_kind_impl(const AttendArgs& a, int lpr, int qr, bool fused, bool page16, dim3 grid, hipStream_t stream) {
+    if (a.fast128 && !a.blocks) return launch_mfma<KIND, F16>(a, fused, grid, stream);
     switch (qr) {
 #define PKV_CASE(Q)                                                                               \
     case Q:                                                                                       \
