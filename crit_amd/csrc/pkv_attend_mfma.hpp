@@ -103,96 +103,179 @@ struct Tile {
 };
 
 constexpr int kTileRows = 16;      // query rows (columns of S^T) a tile holds
+constexpr int kLdsRows = 512;      // batch rows whose descriptors a workgroup keeps in LDS (the others are read from memory)
 
-// One unit of work: (ux, uy) of a units_x x units_y list. MASKED: draft trees and sliding windows.
-template <int KIND, bool F16, int HW, bool FUSED, bool MASKED, int NT>
-PKV_DEV void attend_mfma_unit(const AttendArgs& a, const int ux, const int uy, float (&s_acc)[4][kTileRows][128],
-                              float (&s_m)[4][kTileRows], float (&s_l)[4][kTileRows]) {
+#ifndef PKV_MFMA_WAVES
+#define PKV_MFMA_WAVES 2
+#endif
+constexpr int kMfmaWaves = PKV_MFMA_WAVES;      // wavefronts a SIMD holds (workgroups a compute unit)
+#ifndef PKV_MFMA_TILES
+#define PKV_MFMA_TILES 2
+#endif
+constexpr int kMfmaTiles = PKV_MFMA_TILES;      // steps a wavefront keeps in flight
+
+// The launch: as many workgroups as the card holds at once, each working through units of the list (row, KV head
+// group, query tile, partition) until it is exhausted. The hardware's own dispatcher binds a workgroup to an XCD by its
+// id and starts workgroups strictly in order, so with units as uneven as ragged contexts make them it leaves slots
+// idle behind a busy one; resident workgroups that pull the next unit themselves from the launch's counter (the
+// caller's memory) keep every slot busy to the end. A workgroup knows its next unit while it works on the current one
+// (its first two units are its index and that plus the grid; a ticket names the unit after the next): the next unit's
+// page table entries are requested before the current unit's steps, its first keys, values and queries right after the
+// current unit's last step, so the current unit's fold, its partials' stores and the draw of the following ticket
+// happen while the next unit's rows are already on their way. A drawn unit without work (the list is a grid over rows
+// of different lengths) is passed over by the drawing thread at once. The last workgroup to finish zeroes the counters
+// for the next launch that uses them. Without counters the units are dealt in turn.
+// MASKED: draft trees and sliding windows.
+template <int KIND, bool F16, int HW, bool FUSED, bool MASKED>
+__global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs a) {
+    constexpr int NT = kMfmaTiles;
     constexpr int D = 128;
     constexpr int EB = KIND == 0 ? 2 : 1;
     constexpr int CPH = kTileRows / HW;      // tile columns a KV head holds
     constexpr int SPW = kTileRows / HW;      // positions a wavefront's step covers (tile rows a KV head holds)
     constexpr int EPT = kTileRows * D / 256; // output elements a thread folds
+    __shared__ __align__(16) float s_acc[4][kTileRows][128];
+    __shared__ float s_m[4][kTileRows], s_l[4][kTileRows];
+    __shared__ int s_rows[kLdsRows][5];      // count, first position, table row, first token, first partial row
+    __shared__ unsigned s_unit;
+
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int c16 = lane & 15, u = lane >> 4;
-    int bx = ux;
-    const int tile = bx % a.tiles;
-    bx /= a.tiles;
+    const int c16 = lane & 15, u4 = lane >> 4;
+    const unsigned total = (unsigned)a.units_x * (unsigned)a.units_y, grid = gridDim.x;
+    const bool pulled = a.ticket != nullptr;
     const int hgroups = a.hkv / HW;
-    const int kvh0 = (bx % hgroups) * HW;      // the first of the wavefront's KV heads
-    const int r = bx / hgroups;
-    int b = uy;
-    // The row's descriptors are read together, ahead of every test that could end the unit: one memory round trip.
-    int count_raw = *(a.counts ? a.counts + r : a.starts + r);      // (no load under a condition)
-    int64_t first64 = a.firsts[r];
-    int table_row = a.rows[(int64_t)r * a.rows_step];
-    int start = a.starts[r];
-    int off_r = *(a.offsets ? a.offsets + r : a.starts + r), off_0 = *(a.offsets ? a.offsets : a.starts);
-    asm volatile("" : "+v"(count_raw), "+v"(first64), "+v"(table_row), "+v"(start), "+v"(off_r), "+v"(off_0));
-    count_raw = __builtin_amdgcn_readfirstlane(count_raw), table_row = __builtin_amdgcn_readfirstlane(table_row);
-    start = __builtin_amdgcn_readfirstlane(start), off_r = __builtin_amdgcn_readfirstlane(off_r), off_0 = __builtin_amdgcn_readfirstlane(off_0);
-    first64 = (int64_t)(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(first64 >> 32)) << 32) |
-                        (uint32_t)__builtin_amdgcn_readfirstlane((int)first64));
-    const int64_t prow = a.offsets ? (int64_t)(off_r - off_0) : (int64_t)r * a.columns;      // the row's first partial row
-    const int count = min(a.counts ? count_raw : a.columns, a.columns);
-    const int64_t trow = (int64_t)table_row * a.tab_stride;
-    const int j0 = tile * CPH;                  // the tile's first row of the flattened (column, group head) list
-    if (j0 >= count * a.g) return;
-    const int c_lo = j0 / a.g;
-    const int c_hi = min(count, (j0 + CPH - 1) / a.g + 1);
-    int64_t nk64 = first64 + c_hi;
-    nk64 = nk64 < 0 ? 0 : (nk64 > (int64_t)a.max_keys ? (int64_t)a.max_keys : nk64);
-    const int n_keys = (int)nk64;
-    const int first = (int)(first64 < 0 ? 0 : (first64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first64));
-    const int n_pieces = (n_keys + a.piece - 1) / a.piece;
-    if constexpr (!FUSED) {
-        // Units are taken in list order, y slowest, and a launch's tail is as long as its last units: the row's last
-        // partition (usually a partial piece, the smallest unit of work) is listed after every other partition, in
-        // kTailClasses rows of y by its size (a whole piece or more first, the smallest remainders last).
-        const int np = min(n_pieces, a.parts);
-        if (np <= 0) return;
-        int cls = 0;
-        if (np == n_pieces) cls = min(kTailClasses - 1, (np * a.piece - n_keys) * kTailClasses / a.piece);
-        if (b >= a.units_y - kTailClasses) {
-            if (b - (a.units_y - kTailClasses) != cls) return;
-            b = np - 1;
-        } else if (b >= np - 1) {
-            return;
-        }
-    }
-
-    // This lane's tile column: which of the wavefront's heads it belongs to, its row of the list, its token's column
-    // and the last position that column sees.
-    const int hsel = c16 / CPH;
-    const int jr = j0 + c16 % CPH;
-    const int col = jr / a.g;
-    const bool live = col < count;
-    const int qhead = (kvh0 + hsel) * a.g + jr % a.g;
-    const int lim = live ? min(first + col, n_keys - 1) : -1;
-    const bool tree = MASKED && (a.parents != nullptr || a.parents64 != nullptr);
-    const unsigned long long anc = (tree && live) ? ancestors(a, start, col) : 0ull;
-    const int win = MASKED ? a.sliding : 0;
-    // Tile rows: row i is position i % SPW of the step, of head i / SPW. This lane's places in the three layouts:
-    //   keys    its row c16;  values and scores  rows 4 u .. 4 u + 3.
-    const int k_head = c16 / SPW, k_pos = c16 % SPW;
-    const int r_head = (4 * u) / SPW, r_pos = (4 * u) % SPW;      // (SPW is 8 or 16: a lane's four rows lie in one head)
-    const bool mine = hsel == r_head;                               // this lane's scores are of its own column's head
-    float sscale = a.sscale;
-    if constexpr (KIND == 1) sscale *= a.hm ? a.hm[kvh0 + hsel] : a.k_mult;
-
-    // Byte offsets of what this lane reads in a step, from the step's first slot; the same in every step.
     const int slot_bytes = a.hkv * D * EB;
-    const uint32_t kvo = (uint32_t)(k_pos * slot_bytes + (kvh0 + k_head) * D * EB + u * 16);
+    const bool tree = MASKED && (a.parents != nullptr || a.parents64 != nullptr);
+    const int win = MASKED ? a.sliding : 0;
+
+    // -- every row's descriptors, once per workgroup
+    auto row_from_memory = [&](int r, int (&d)[5]) __attribute__((always_inline)) {
+        const int count = a.counts ? a.counts[r] : a.columns;
+        const int64_t first64 = a.firsts[r];
+        d[0] = min(count, a.columns);
+        d[1] = (int)(first64 < 0 ? 0 : (first64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first64));
+        d[2] = a.rows[(int64_t)r * a.rows_step];
+        d[3] = a.starts[r];
+        d[4] = a.offsets ? a.offsets[r] - a.offsets[0] : r * a.columns;
+    };
+    for (int r = tid; r < min(a.n_rows, kLdsRows); r += 256) {
+        int d[5];
+        row_from_memory(r, d);
+#pragma unroll
+        for (int i = 0; i < 5; ++i) s_rows[r][i] = d[i];
+    }
+    lds_barrier();
+
+    // -- a unit of the list, decoded (everything uniform over the workgroup)
+    struct Unit {
+        bool valid;
+        int kvh0, j0, b, count, first, n_keys, n_pieces, start, c_lo, prow;
+        int64_t trow;
+    };
+    auto decode = [&](unsigned unit) __attribute__((always_inline)) -> Unit {
+        Unit un;
+        un.valid = false;
+        if (unit >= total) return un;
+        int bx = (int)(unit % (unsigned)a.units_x);
+        int b = (int)(unit / (unsigned)a.units_x);
+        const int tile = bx % a.tiles;
+        bx /= a.tiles;
+        un.kvh0 = (bx % hgroups) * HW;      // the first of the wavefronts' KV heads
+        const int r = bx / hgroups;
+        int d[5];
+        if (r < kLdsRows) {
+#pragma unroll
+            for (int i = 0; i < 5; ++i) d[i] = s_rows[r][i];
+        } else {
+            row_from_memory(r, d);
+        }
+#pragma unroll
+        for (int i = 0; i < 5; ++i) d[i] = __builtin_amdgcn_readfirstlane(d[i]);
+        un.count = d[0], un.first = d[1], un.start = d[3], un.prow = d[4];
+        un.trow = (int64_t)d[2] * a.tab_stride;
+        un.j0 = tile * CPH;                  // the tile's first row of the flattened (column, group head) list
+        if (un.j0 >= un.count * a.g) return un;
+        un.c_lo = un.j0 / a.g;
+        const int c_hi = min(un.count, (un.j0 + CPH - 1) / a.g + 1);
+        un.n_keys = min(un.first + c_hi, a.max_keys);
+        un.n_pieces = (un.n_keys + a.piece - 1) / a.piece;
+        if constexpr (!FUSED) {
+            // Units are taken in list order, y slowest, and a launch's tail is as long as its last units: the row's
+            // last partition (usually a partial piece, the smallest unit of work) is listed after every other
+            // partition, in kTailClasses rows of y by its size (a whole piece or more first, the smallest last).
+            const int np = min(un.n_pieces, a.parts);
+            if (np <= 0) return un;
+            int cls = 0;
+            if (np == un.n_pieces) cls = min(kTailClasses - 1, (np * a.piece - un.n_keys) * kTailClasses / a.piece);
+            if (b >= a.units_y - kTailClasses) {
+                if (b - (a.units_y - kTailClasses) != cls) return un;
+                b = np - 1;
+            } else if (b >= np - 1) {
+                return un;
+            }
+        }
+        un.b = b;
+        un.valid = true;
+        return un;
+    };
+
+    // -- what a lane holds for the whole launch
+    // Tile rows: row i is position i % SPW of the step, of head i / SPW. This lane's places in the three layouts:
+    //   keys    its row c16;  values and scores  rows 4 u4 .. 4 u4 + 3.
+    const int hsel = c16 / CPH;                                     // the head (of the wavefront's HW) of this lane's tile column
+    const int k_head = c16 / SPW, k_pos = c16 % SPW;
+    const int r_head = (4 * u4) / SPW, r_pos = (4 * u4) % SPW;      // (SPW is 8 or 16: a lane's four rows lie in one head)
+    const bool mine = hsel == r_head;                               // this lane's scores are of its own column's head
+    // Byte offsets of what this lane reads in a step, from the step's first slot and the unit's first head.
+    const uint32_t kvo = (uint32_t)(k_pos * slot_bytes + k_head * D * EB + u4 * 16);
     uint32_t vvo[4];
 #pragma unroll
-    for (int p = 0; p < 4; ++p) vvo[p] = (uint32_t)((r_pos + p) * slot_bytes + (kvh0 + r_head) * D * EB + c16 * 8 * EB);
-    const uint32_t svo = (uint32_t)(r_pos * a.hkv + kvh0 + r_head);      // row-scaled kinds: the lane's first score row's scale
+    for (int p = 0; p < 4; ++p) vvo[p] = (uint32_t)((r_pos + p) * slot_bytes + r_head * D * EB + c16 * 8 * EB);
+    const uint32_t svo = (uint32_t)(r_pos * a.hkv + r_head);      // row-scaled kinds: the lane's first score row's scale
 
-    auto entry = [&](int base) __attribute__((always_inline)) -> int {     // the page table entry of a step (uniform over the wavefront)
+    // -- a wavefront's walk over a partition's steps: steps wave, wave + 4, ... of pieces part, part + parts, ...
+    // (positions stay below 2^31: the launcher bounds partitions x piece)
+    struct Walk {
+        int pi, st;
+    };
+    auto walk_base = [&](const Unit& un, const Walk& w) __attribute__((always_inline)) -> int {
+        if (w.st * SPW >= a.piece) return -1;
+        const int base = w.pi * a.piece + w.st * SPW;
+        return base < un.n_keys ? base : -1;
+    };
+    auto walk_advance = [&](const Unit& un, Walk& w) __attribute__((always_inline)) -> int {
+        w.st += 4;
+        if (w.st * SPW >= a.piece) w.pi += a.parts, w.st = wave;
+        return walk_base(un, w);
+    };
+    auto entry = [&](const Unit& un, int base) __attribute__((always_inline)) -> int {     // the page table entry of a step (uniform over the wavefront)
         int pidx = base >> a.page_shift;
         pidx = pidx < a.tab_width ? pidx : a.tab_width - 1;
-        return a.tables[trow + pidx];
+        return a.tables[un.trow + pidx];
+    };
+    // The first steps of a partition with their page table entries: NT steps to fill the buffers and the NT after them.
+    struct Lead {
+        int base[2 * NT], e[2 * NT];
+        Walk w;
+    };
+    auto lead_of = [&](const Unit& un, int part) __attribute__((always_inline)) -> Lead {
+        Lead f;
+        f.w.pi = part, f.w.st = wave;
+        if (win > 0) {      // pieces wholly below the tile's window are skipped (no row sees them)
+            const int wlo = un.first + un.c_lo - win + 1;
+            const int below = (wlo > 0 ? wlo : 0) / a.piece - part;
+            if (below > 0) f.w.pi = part + (below + a.parts - 1) / a.parts * a.parts;
+        }
+        f.base[0] = walk_base(un, f.w);
+        const int again = f.base[0] >= 0 ? f.base[0] : 0;      // (a wavefront without a step reads position 0's entry)
+        f.e[0] = entry(un, again);
+#pragma unroll
+        for (int i = 1; i < 2 * NT; ++i) {
+            f.base[i] = f.base[i - 1] >= 0 ? walk_advance(un, f.w) : -1;
+            f.e[i] = entry(un, f.base[i] >= 0 ? f.base[i] : again);
+        }
+        return f;
     };
     // A step's positions lie in one page (pages are powers of two from 16 up): its first slot, uniform.
     auto first_slot = [&](int base, int e) __attribute__((always_inline)) -> int64_t {
@@ -201,8 +284,8 @@ PKV_DEV void attend_mfma_unit(const AttendArgs& a, const int ux, const int uy, f
     // Loads of one step from its first slot. Every lane loads its place of the step whether the row holds that
     // position or not (the page does; a step past the row's keys is never listed): what such a place holds is dropped
     // where it is used (keys: the score is masked; values and scales: zeroed, see sanitize()).
-    auto fetch_k = [&](int64_t slot0, Tile<KIND>& t) __attribute__((always_inline)) {
-        const uint8_t* sbase = a.kp + slot0 * slot_bytes;
+    auto fetch_k = [&](const Unit& un, int64_t slot0, Tile<KIND>& t) __attribute__((always_inline)) {
+        const uint8_t* sbase = a.kp + slot0 * slot_bytes + un.kvh0 * D * EB;
         if constexpr (KIND == 0) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) t.k[c] = *reinterpret_cast<const u32x4*>(sbase + kvo + 64 * c);
@@ -211,305 +294,313 @@ PKV_DEV void attend_mfma_unit(const AttendArgs& a, const int ux, const int uy, f
             t.k[1] = *reinterpret_cast<const u32x4*>(sbase + kvo + 64);
         }
         if constexpr (KIND >= 2) {
-            const float* ks = a.ks + slot0 * a.hkv;
-            const float* vs = a.vs + slot0 * a.hkv;
+            const float* ks = a.ks + slot0 * a.hkv + un.kvh0;
+            const float* vs = a.vs + slot0 * a.hkv + un.kvh0;
 #pragma unroll
             for (int i = 0; i < 4; ++i) t.ks[i] = ks[svo + i * a.hkv], t.vs[i] = vs[svo + i * a.hkv];
         }
     };
-    auto fetch_v = [&](int64_t slot0, Tile<KIND>& t) __attribute__((always_inline)) {
-        const uint8_t* sbase = a.vp + slot0 * slot_bytes;
+    auto fetch_v = [&](const Unit& un, int64_t slot0, Tile<KIND>& t) __attribute__((always_inline)) {
+        const uint8_t* sbase = a.vp + slot0 * slot_bytes + un.kvh0 * D * EB;
 #pragma unroll
         for (int p = 0; p < 4; ++p)
             t.v[p] = __builtin_nontemporal_load(reinterpret_cast<const typename Tile<KIND>::VVec*>(sbase + vvo[p]));
     };
-    // The row's last step: what lies past its keys may be anything, and a probability of zero times a NaN is a NaN.
-    auto sanitize = [&](int base, Tile<KIND>& t) __attribute__((always_inline)) {
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            if (base + r_pos + p >= n_keys) {
-                if constexpr (KIND == 0) t.v[p] = u32x4{0, 0, 0, 0};
-                else t.v[p] = u32x2{0, 0};
-                if constexpr (KIND >= 2) t.vs[p] = 0.0f;
-            }
-        }
-    };
 
-    // A wavefront's walk over a partition's steps: steps wave, wave + 4, ... of pieces part, part + parts, ...
-    // (positions stay below 2^31: the launcher bounds partitions x piece)
-    int pi, st;
-    auto start_part = [&](int part) __attribute__((always_inline)) {
-        pi = part, st = wave;
-        if (win > 0) {      // pieces wholly below the tile's window are skipped (no row sees them)
-            const int wlo = first + c_lo - win + 1;
-            const int below = (wlo > 0 ? wlo : 0) / a.piece - part;
-            if (below > 0) pi = part + (below + a.parts - 1) / a.parts * a.parts;
-        }
-    };
-    auto base_of = [&]() __attribute__((always_inline)) -> int {
-        if (st * SPW >= a.piece) return -1;
-        const int base = pi * a.piece + st * SPW;
-        return base < n_keys ? base : -1;
-    };
-    auto advance = [&]() __attribute__((always_inline)) -> int {
-        st += 4;
-        if (st * SPW >= a.piece) pi += a.parts, st = wave;
-        return base_of();
-    };
-    // The first steps of a partition with their page table entries: NT steps to fill the buffers and one ahead.
-    struct Lead {
-        int base[NT + 1], e[NT + 1];
-    };
-    auto lead_of = [&](int part) __attribute__((always_inline)) -> Lead {
-        Lead f;
-        start_part(part);
-        f.base[0] = base_of();
-        const int again = f.base[0] >= 0 ? f.base[0] : 0;      // (a wavefront without a step reads position 0's entry)
-        f.e[0] = entry(again);
-#pragma unroll
-        for (int i = 1; i <= NT; ++i) {
-            f.base[i] = f.base[i - 1] >= 0 ? advance() : -1;
-            f.e[i] = entry(f.base[i] >= 0 ? f.base[i] : again);
-        }
-        return f;
-    };
-    const int part_lo = FUSED ? 0 : b;
-    const int part_hi = FUSED ? min(a.parts, n_pieces) : b + 1;
-    const Lead lead_first = lead_of(part_lo);
-
-    // The query operand: this lane's column's row, piece c = the dims the keys' piece c holds (zeros in a dead column).
+    // -- what a lane holds for one unit: its tile column's token, query head, last visible position, ancestors, scale,
+    // and the query operand (its column's row, piece c = the dims the keys' piece c holds; zeros in a dead column)
+    int col = 0, lim = -1;
+    unsigned long long anc = 0ull;
+    float sscale = a.sscale;
     u32x4 qb[4];
-    {
-        const uint8_t* row = a.q + ((int64_t)(start + col) * a.q_st + (int64_t)qhead * a.q_sh) * 2;
+    auto lane_values = [&](const Unit& un) __attribute__((always_inline)) {
+        const int jr = un.j0 + c16 % CPH;
+        col = jr / a.g;
+        const bool live = col < un.count;
+        const int qhead = (un.kvh0 + hsel) * a.g + jr % a.g;
+        lim = live ? min(un.first + col, un.n_keys - 1) : -1;
+        anc = (tree && live) ? ancestors(a, un.start, col) : 0ull;
+        if constexpr (KIND == 1) sscale = a.sscale * (a.hm ? a.hm[un.kvh0 + hsel] : a.k_mult);
+        const uint8_t* row = a.q + ((int64_t)(un.start + col) * a.q_st + (int64_t)qhead * a.q_sh) * 2;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            // 16-bit pages: dims 32 c + 8 u ..; 8-bit pages: dims 64 (c / 2) + 16 u + 8 (c % 2) .. (the codes a lane's two loads hold)
-            const int dim = KIND == 0 ? 32 * c + 8 * u : 64 * (c / 2) + 16 * u + 8 * (c % 2);
+            // 16-bit pages: dims 32 c + 8 u4 ..; 8-bit pages: dims 64 (c / 2) + 16 u4 + 8 (c % 2) .. (the codes a lane's two loads hold)
+            const int dim = KIND == 0 ? 32 * c + 8 * u4 : 64 * (c / 2) + 16 * u4 + 8 * (c % 2);
             qb[c] = u32x4{0, 0, 0, 0};
             if (live) qb[c] = *reinterpret_cast<const u32x4*>(row + dim * 2);
         }
+    };
+
+    Tile<KIND> t[NT];
+    auto fill = [&](const Unit& un, const Lead& f) __attribute__((always_inline)) {      // a partition's first NT steps
+        const int again = f.base[0] >= 0 ? f.base[0] : 0;
+#pragma unroll
+        for (int i = 0; i < NT; ++i) {
+            const int64_t slot = first_slot(f.base[i] >= 0 ? f.base[i] : again, f.e[i]);
+            fetch_k(un, slot, t[i]), fetch_v(un, slot, t[i]);
+        }
+    };
+
+    unsigned u_next = blockIdx.x + grid;
+    Unit cur = decode(blockIdx.x);
+    Lead lead_cur;
+    if (cur.valid) {
+        lead_cur = lead_of(cur, FUSED ? 0 : cur.b);
+        fill(cur, lead_cur);
+        lane_values(cur);
     }
-    float run_m[FUSED ? EPT : 1], run_l[FUSED ? EPT : 1], run_a[FUSED ? EPT : 1];
-#pragma unroll
-    for (int e = 0; e < (FUSED ? EPT : 1); ++e) run_m[e] = -INFINITY, run_l[e] = 0.0f, run_a[e] = 0.0f;
-
-    for (int part = part_lo; part < part_hi; ++part) {
-        float m = -INFINITY, l = 0.0f;      // the lane's column: running maximum (the same in its four lanes), the lane's share of the sum
-        f32x4 acc[8];                        // O^T: acc[j][i] = dim 32 u + 8 i + j of the lane's column
-#pragma unroll
-        for (int j = 0; j < 8; ++j) acc[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-
-        auto step = [&](int base, Tile<KIND>& t, auto&& refill_k, auto&& refill_v) __attribute__((always_inline)) {
-            if (base + SPW > n_keys) sanitize(base, t);
-            // -- scores
-            u32x4 ka[4];
-            if constexpr (KIND == 0) {
-#pragma unroll
-                for (int c = 0; c < 4; ++c) ka[c] = t.k[c];
-            } else {
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const uint32_t w0 = c % 2 ? t.k[c / 2].z : t.k[c / 2].x, w1 = c % 2 ? t.k[c / 2].w : t.k[c / 2].y;
-                    const u32x2 lo = codes4_to_pairs<KIND>(w0), hi = codes4_to_pairs<KIND>(w1);
-                    ka[c] = u32x4{lo.x, lo.y, hi.x, hi.y};
-                }
+    for (;;) {
+        // The next unit: its first steps' page table entries are requested now and wait in registers.
+        const Unit nxt = decode(u_next);
+        Lead lead_nxt = {};
+        if (nxt.valid) lead_nxt = lead_of(nxt, FUSED ? 0 : nxt.b);
+        // The ticket of the unit after the next is drawn when the current unit's steps are done (a returning atomic
+        // in flight beside a unit's loads makes the waits on them coarser) and looked at after its fold.
+        unsigned drawn = 0;
+        bool sent = false;      // the next unit's first loads are out, the ticket is drawn
+        auto hand_over = [&]() __attribute__((always_inline)) {
+            if (pulled && tid == 0) drawn = atomicAdd(a.ticket, 1u);
+            if (nxt.valid) {
+                fill(nxt, lead_nxt);
+                lane_values(nxt);
             }
-            f32x4 s0 = mfma_k32<F16>(ka[0], qb[0], f32x4{0.0f, 0.0f, 0.0f, 0.0f});
-            f32x4 s1 = mfma_k32<F16>(ka[1], qb[1], f32x4{0.0f, 0.0f, 0.0f, 0.0f});
-            s0 = mfma_k32<F16>(ka[2], qb[2], s0);
-            s1 = mfma_k32<F16>(ka[3], qb[3], s1);
-            float ks4[4], vs4[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) ks4[i] = KIND >= 2 ? t.ks[i] : 1.0f, vs4[i] = KIND >= 2 ? t.vs[i] : 1.0f;
-            refill_k();      // (the keys' registers are free: the loads of NT steps ahead go out)
-            // the lane's scores: its column at positions base + r_pos + i of head r_head; another head's column sees nothing
-            const int room = lim - (base + r_pos);      // visible while i <= room
-            float x[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                x[i] = (s0[i] + s1[i]) * (KIND >= 2 ? sscale * ks4[i] : sscale);
-                bool vis = mine && i <= room;
-                if constexpr (MASKED) {
-                    const int n = base + r_pos + i;
-                    if (tree) vis = vis && (n < first || ((anc >> ((n - first) & 63)) & 1ull) != 0);
-                    if (win > 0) vis = vis && n > first + col - win;
-                }
-                x[i] = vis ? x[i] : -INFINITY;
-            }
-            const float top = max_across_quarters(__builtin_fmaxf(__builtin_fmaxf(x[0], x[1]), __builtin_fmaxf(x[2], x[3])));
-            const float m_new = __builtin_fmaxf(m, top);
-            const float sub = m_new == -INFINITY ? 0.0f : m_new;
-            const float alpha = m == -INFINITY ? 1.0f : exp2_fast(m - sub);      // (nothing summed yet: nothing to rescale)
-            float p[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) p[i] = exp2_fast(x[i] - sub);
-            l = __builtin_fmaf(l, alpha, (p[0] + p[1]) + (p[2] + p[3]));
-            m = m_new;
-            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {     // some row's maximum moved: rescale
-#pragma unroll
-                for (int j = 0; j < 8; ++j) acc[j] *= alpha;
-            }
-            const u32x2 pb = {pair16<F16>(p[0] * vs4[0], p[1] * vs4[1]), pair16<F16>(p[2] * vs4[2], p[3] * vs4[3])};
-            // -- values: dims {8 i + j} of the lane's four rows as two 16-bit pairs (one v_perm each), then O^T += V^T P^T
-            if constexpr (KIND == 0) {
-#pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    const u32x2 lo = {__builtin_amdgcn_perm(t.v[1][w], t.v[0][w], 0x05040100), __builtin_amdgcn_perm(t.v[3][w], t.v[2][w], 0x05040100)};
-                    const u32x2 hi = {__builtin_amdgcn_perm(t.v[1][w], t.v[0][w], 0x07060302), __builtin_amdgcn_perm(t.v[3][w], t.v[2][w], 0x07060302)};
-                    acc[2 * w] = mfma_k16<F16>(lo, pb, acc[2 * w]);
-                    acc[2 * w + 1] = mfma_k16<F16>(hi, pb, acc[2 * w + 1]);
-                }
-            } else {
-#pragma unroll
-                for (int w = 0; w < 2; ++w) {
-                    // bytes (a0 b0 a1 b1) and (a2 b2 a3 b3): two rows' codes of one dim side by side
-                    const uint32_t lo01 = __builtin_amdgcn_perm(t.v[1][w], t.v[0][w], 0x05010400), hi01 = __builtin_amdgcn_perm(t.v[1][w], t.v[0][w], 0x07030602);
-                    const uint32_t lo23 = __builtin_amdgcn_perm(t.v[3][w], t.v[2][w], 0x05010400), hi23 = __builtin_amdgcn_perm(t.v[3][w], t.v[2][w], 0x07030602);
-                    // (dims 4 w + 0, 1 from the low halves, 2, 3 from the high ones; .x: rows 0, 1; .y: rows 2, 3)
-                    const u32x2 a01 = codes4_to_pairs<KIND>(lo01), a23 = codes4_to_pairs<KIND>(lo23);
-                    const u32x2 b01 = codes4_to_pairs<KIND>(hi01), b23 = codes4_to_pairs<KIND>(hi23);
-                    const u32x2 va[4] = {u32x2{a01.x, a23.x}, u32x2{a01.y, a23.y}, u32x2{b01.x, b23.x}, u32x2{b01.y, b23.y}};
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) acc[4 * w + j] = mfma_k16<F16>(va[j], pb, acc[4 * w + j]);
-                }
-            }
-            refill_v();
+            sent = true;
         };
 
-        // Software pipeline over NT steps: a step's keys are reloaded (for NT steps ahead) as soon as its scores are
-        // issued, its values as soon as its second product is; the page table entries run one step further ahead.
-        // Past the wavefront's last step the loads re-read its first step (the caches hold it).
-        Tile<KIND> t[NT];
-        const Lead f = part == part_lo ? lead_first : lead_of(part);
-        if (f.base[0] >= 0) {
-            const int again = f.base[0];
-            auto safe = [&](int base) __attribute__((always_inline)) { return base >= 0 ? base : again; };
-            int cur[NT], next = f.base[NT], e_next = f.e[NT];
+        if (cur.valid) {
+            const int part_lo = FUSED ? 0 : cur.b;
+            const int part_hi = FUSED ? min(a.parts, cur.n_pieces) : cur.b + 1;
+            float run_m[FUSED ? EPT : 1], run_l[FUSED ? EPT : 1], run_a[FUSED ? EPT : 1];
 #pragma unroll
-            for (int i = 0; i < NT; ++i) {
-                cur[i] = f.base[i];
-                const int64_t slot = first_slot(safe(cur[i]), f.e[i]);
-                fetch_k(slot, t[i]), fetch_v(slot, t[i]);
+            for (int e = 0; e < (FUSED ? EPT : 1); ++e) run_m[e] = -INFINITY, run_l[e] = 0.0f, run_a[e] = 0.0f;
+            for (int part = part_lo; part < part_hi; ++part) {
+                float m = -INFINITY, l = 0.0f;      // the lane's column: running maximum (the same in its four lanes), the lane's share of the sum
+                f32x4 acc[8];                        // O^T: acc[j][i] = dim 32 u4 + 8 i + j of the lane's column
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+                auto step = [&](int base, Tile<KIND>& tl, auto&& refill_k, auto&& refill_v) __attribute__((always_inline)) {
+                    if (base + SPW > cur.n_keys) {
+                        // The row's last step: what lies past its keys may be anything, and a probability of zero
+                        // times a NaN is a NaN.
+#pragma unroll
+                        for (int p = 0; p < 4; ++p) {
+                            if (base + r_pos + p >= cur.n_keys) {
+                                if constexpr (KIND == 0) tl.v[p] = u32x4{0, 0, 0, 0};
+                                else tl.v[p] = u32x2{0, 0};
+                                if constexpr (KIND >= 2) tl.vs[p] = 0.0f;
+                            }
+                        }
+                    }
+                    // -- scores
+                    u32x4 ka[4];
+                    if constexpr (KIND == 0) {
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) ka[c] = tl.k[c];
+                    } else {
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            const uint32_t w0 = c % 2 ? tl.k[c / 2].z : tl.k[c / 2].x, w1 = c % 2 ? tl.k[c / 2].w : tl.k[c / 2].y;
+                            const u32x2 lo = codes4_to_pairs<KIND>(w0), hi = codes4_to_pairs<KIND>(w1);
+                            ka[c] = u32x4{lo.x, lo.y, hi.x, hi.y};
+                        }
+                    }
+                    f32x4 s0 = mfma_k32<F16>(ka[0], qb[0], f32x4{0.0f, 0.0f, 0.0f, 0.0f});
+                    f32x4 s1 = mfma_k32<F16>(ka[1], qb[1], f32x4{0.0f, 0.0f, 0.0f, 0.0f});
+                    s0 = mfma_k32<F16>(ka[2], qb[2], s0);
+                    s1 = mfma_k32<F16>(ka[3], qb[3], s1);
+                    float ks4[4], vs4[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) ks4[i] = KIND >= 2 ? tl.ks[i] : 1.0f, vs4[i] = KIND >= 2 ? tl.vs[i] : 1.0f;
+                    refill_k();      // (the keys' registers are free: the loads of NT steps ahead go out)
+                    // the lane's scores: its column at positions base + r_pos + i of head r_head; another head's column sees nothing
+                    const int room = lim - (base + r_pos);      // visible while i <= room
+                    float x[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        x[i] = (s0[i] + s1[i]) * (KIND >= 2 ? sscale * ks4[i] : sscale);
+                        bool vis = mine && i <= room;
+                        if constexpr (MASKED) {
+                            const int n = base + r_pos + i;
+                            if (tree) vis = vis && (n < cur.first || ((anc >> ((n - cur.first) & 63)) & 1ull) != 0);
+                            if (win > 0) vis = vis && n > cur.first + col - win;
+                        }
+                        x[i] = vis ? x[i] : -INFINITY;
+                    }
+                    const float top = max_across_quarters(__builtin_fmaxf(__builtin_fmaxf(x[0], x[1]), __builtin_fmaxf(x[2], x[3])));
+                    const float m_new = __builtin_fmaxf(m, top);
+                    const float sub = m_new == -INFINITY ? 0.0f : m_new;
+                    const float alpha = m == -INFINITY ? 1.0f : exp2_fast(m - sub);      // (nothing summed yet: nothing to rescale)
+                    float p[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) p[i] = exp2_fast(x[i] - sub);
+                    l = __builtin_fmaf(l, alpha, (p[0] + p[1]) + (p[2] + p[3]));
+                    m = m_new;
+                    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {     // some row's maximum moved: rescale
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) acc[j] *= alpha;
+                    }
+                    const u32x2 pb = {pair16<F16>(p[0] * vs4[0], p[1] * vs4[1]), pair16<F16>(p[2] * vs4[2], p[3] * vs4[3])};
+                    // -- values: dims {8 i + j} of the lane's four rows as two 16-bit pairs (one v_perm each), then O^T += V^T P^T
+                    if constexpr (KIND == 0) {
+#pragma unroll
+                        for (int w = 0; w < 4; ++w) {
+                            const u32x2 lo = {__builtin_amdgcn_perm(tl.v[1][w], tl.v[0][w], 0x05040100), __builtin_amdgcn_perm(tl.v[3][w], tl.v[2][w], 0x05040100)};
+                            const u32x2 hi = {__builtin_amdgcn_perm(tl.v[1][w], tl.v[0][w], 0x07060302), __builtin_amdgcn_perm(tl.v[3][w], tl.v[2][w], 0x07060302)};
+                            acc[2 * w] = mfma_k16<F16>(lo, pb, acc[2 * w]);
+                            acc[2 * w + 1] = mfma_k16<F16>(hi, pb, acc[2 * w + 1]);
+                        }
+                    } else {
+#pragma unroll
+                        for (int w = 0; w < 2; ++w) {
+                            // bytes (a0 b0 a1 b1) and (a2 b2 a3 b3): two rows' codes of one dim side by side
+                            const uint32_t lo01 = __builtin_amdgcn_perm(tl.v[1][w], tl.v[0][w], 0x05010400), hi01 = __builtin_amdgcn_perm(tl.v[1][w], tl.v[0][w], 0x07030602);
+                            const uint32_t lo23 = __builtin_amdgcn_perm(tl.v[3][w], tl.v[2][w], 0x05010400), hi23 = __builtin_amdgcn_perm(tl.v[3][w], tl.v[2][w], 0x07030602);
+                            // (dims 4 w + 0, 1 from the low halves, 2, 3 from the high ones; .x: rows 0, 1; .y: rows 2, 3)
+                            const u32x2 a01 = codes4_to_pairs<KIND>(lo01), a23 = codes4_to_pairs<KIND>(lo23);
+                            const u32x2 b01 = codes4_to_pairs<KIND>(hi01), b23 = codes4_to_pairs<KIND>(hi23);
+                            const u32x2 va[4] = {u32x2{a01.x, a23.x}, u32x2{a01.y, a23.y}, u32x2{b01.x, b23.x}, u32x2{b01.y, b23.y}};
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) acc[4 * w + j] = mfma_k16<F16>(va[j], pb, acc[4 * w + j]);
+                        }
+                    }
+                    refill_v();
+                };
+
+                // Software pipeline over NT steps: a step's keys are reloaded (for NT steps ahead) as soon as its
+                // scores are issued, its values as soon as its second product is; the page table entries run NT steps
+                // further ahead. While the NT steps ahead all exist the loop's loads are unconditional (exact waits);
+                // the wavefront's last steps are peeled: no step is loaded that is not used (a re-read of an earlier
+                // step would come from HBM again: the caches have long turned over).
+                Lead f = lead_cur;
+                if (part != part_lo) {
+                    f = lead_of(cur, part);
+                    fill(cur, f);
+                }
+                if (f.base[0] >= 0) {
+                    const int again = f.base[0];
+                    int at[NT], ahead[NT], e_ahead[NT];
+#pragma unroll
+                    for (int i = 0; i < NT; ++i) at[i] = f.base[i], ahead[i] = f.base[NT + i], e_ahead[i] = f.e[NT + i];
+                    while (ahead[NT - 1] >= 0) {
+#pragma unroll
+                        for (int i = 0; i < NT; ++i) {
+                            const int after = walk_advance(cur, f.w);      // NT steps past the one this buffer is refilled with
+                            const int e_after = entry(cur, after >= 0 ? after : again);
+                            const int64_t slot = first_slot(ahead[i], e_ahead[i]);
+                            step(at[i], t[i], [&]() __attribute__((always_inline)) { fetch_k(cur, slot, t[i]); },
+                                 [&]() __attribute__((always_inline)) { fetch_v(cur, slot, t[i]); });
+                            at[i] = ahead[i], ahead[i] = after, e_ahead[i] = e_after;
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < NT; ++i) {
+                        if (at[i] >= 0) {
+                            const bool again_i = ahead[i] >= 0;
+                            const int64_t slot = first_slot(again_i ? ahead[i] : again, e_ahead[i]);
+                            step(at[i], t[i], [&]() __attribute__((always_inline)) { if (again_i) fetch_k(cur, slot, t[i]); },
+                                 [&]() __attribute__((always_inline)) { if (again_i) fetch_v(cur, slot, t[i]); });
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < NT; ++i) {
+                        if (ahead[i] >= 0) step(ahead[i], t[i], []() {}, []() {});
+                    }
+                }
+                // The unit's steps are done: the next unit's first keys, values and queries go out before the fold.
+                const int fold_col_j0 = cur.j0, fold_kvh0 = cur.kvh0;
+                if (part == part_hi - 1) hand_over();
+
+                // The column's sum over its four lanes, then the four wavefronts through LDS, in wavefront order.
+                const float l_col = sum_across_quarters(l);
+                if (part != part_lo) lds_barrier();      // the previous partition's fold has read the LDS
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    *reinterpret_cast<f32x4*>(&s_acc[wave][c16][32 * u4 + 8 * i]) = f32x4{acc[0][i], acc[1][i], acc[2][i], acc[3][i]};
+                    *reinterpret_cast<f32x4*>(&s_acc[wave][c16][32 * u4 + 8 * i + 4]) = f32x4{acc[4][i], acc[5][i], acc[6][i], acc[7][i]};
+                }
+                if (u4 == 0) s_m[wave][c16] = m, s_l[wave][c16] = l_col;
+                lds_barrier();
+#pragma unroll
+                for (int e = 0; e < EPT; ++e) {
+                    const int idx = tid + e * 256;
+                    const int cc = idx / D, d = idx % D;
+                    const int head_i = cc / CPH;
+                    const int j = fold_col_j0 + cc % CPH;
+                    const int c = j / a.g;
+                    float M = s_m[0][cc];
+#pragma unroll
+                    for (int w = 1; w < 4; ++w) M = __builtin_fmaxf(M, s_m[w][cc]);
+                    const float sub = M == -INFINITY ? 0.0f : M;
+                    float L = 0.0f, A = 0.0f;
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        const float fw = exp2_fast(s_m[w][cc] - sub);
+                        L = __builtin_fmaf(s_l[w][cc], fw, L);
+                        A = __builtin_fmaf(s_acc[w][cc][d], fw, A);
+                    }
+                    if constexpr (KIND == 1) A *= a.hm ? a.hm[a.hkv + fold_kvh0 + head_i] : a.v_mult;
+                    if (c < cur.count) {
+                        if constexpr (FUSED) {
+                            // A column folds the partitions that hold its positions, as the merge does.
+                            const int held = min(a.parts, (min(cur.first + c + 1, a.max_keys) + a.piece - 1) / a.piece);
+                            if (part < held) {
+                                const Fold fo = fold(run_m[e], run_l[e], M, L);
+                                run_a[e] = __builtin_fmaf(run_a[e], fo.keep, A * fo.take);
+                                run_m[e] = fo.m, run_l[e] = fo.l;
+                            }
+                        } else {
+                            const int64_t at = ((int64_t)(cur.prow + c) * a.hq + (fold_kvh0 + head_i) * a.g + j % a.g) * a.parts + cur.b;
+                            a.po[at * D + d] = A;
+                            if (d == 0) a.pm[at] = M, a.pl[at] = L;
+                        }
+                    }
+                }
             }
-            for (bool more = true; more;) {
+            if constexpr (FUSED) {
 #pragma unroll
-                for (int i = 0; i < NT; ++i) {
-                    if (more && cur[i] < 0) more = false;
-                    if (more) {
-                        const int after = next >= 0 ? advance() : -1;      // the step after the one this buffer is refilled with
-                        const int e_after = entry(safe(after));
-                        const int64_t slot = first_slot(safe(next), e_next);
-                        step(cur[i], t[i], [&]() __attribute__((always_inline)) { fetch_k(slot, t[i]); },
-                             [&]() __attribute__((always_inline)) { fetch_v(slot, t[i]); });
-                        cur[i] = next, next = after, e_next = e_after;
+                for (int e = 0; e < EPT; ++e) {
+                    const int idx = tid + e * 256;
+                    const int cc = idx / D, d = idx % D;
+                    const int j = cur.j0 + cc % CPH;
+                    const int c = j / a.g;
+                    if (c < cur.count) {
+                        const int head = (cur.kvh0 + cc / CPH) * a.g + j % a.g;
+                        float M = run_m[e], L = run_l[e], A = run_a[e];
+                        if (a.sinks) {
+                            const Fold fo = fold(M, L, a.sinks[head] * kLog2e, 1.0f);
+                            A *= fo.keep, M = fo.m, L = fo.l;
+                        }
+                        const float o = L != 0.0f ? A / L : 0.0f;
+                        store_out(a.out, a.out_dtype, (int64_t)(cur.start + c) * a.o_st + (int64_t)head * a.o_sh + d, o);
+                        if (a.lse && d == 0) a.lse[(int64_t)(cur.start + c) * a.hq + head] = L != 0.0f ? __builtin_fmaf(M, kLn2, __logf(L)) : -INFINITY;
                     }
                 }
             }
         }
+        if (!sent) hand_over();      // (nothing to do in this round: the next unit's first rows go out all the same)
 
-        // The column's sum over its four lanes, then the four wavefronts through LDS, in wavefront order.
-        const float l_col = sum_across_quarters(l);
-        if (FUSED) lds_barrier();      // the previous partition's fold has read the LDS
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<f32x4*>(&s_acc[wave][c16][32 * u + 8 * i]) = f32x4{acc[0][i], acc[1][i], acc[2][i], acc[3][i]};
-            *reinterpret_cast<f32x4*>(&s_acc[wave][c16][32 * u + 8 * i + 4]) = f32x4{acc[4][i], acc[5][i], acc[6][i], acc[7][i]};
-        }
-        if (u == 0) s_m[wave][c16] = m, s_l[wave][c16] = l_col;
-        lds_barrier();
-#pragma unroll
-        for (int e = 0; e < EPT; ++e) {
-            const int idx = tid + e * 256;
-            const int cc = idx / D, d = idx % D;
-            const int head_i = cc / CPH;
-            const int j = j0 + cc % CPH;
-            const int c = j / a.g;
-            float M = s_m[0][cc];
-#pragma unroll
-            for (int w = 1; w < 4; ++w) M = __builtin_fmaxf(M, s_m[w][cc]);
-            const float sub = M == -INFINITY ? 0.0f : M;
-            float L = 0.0f, A = 0.0f;
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                const float fw = exp2_fast(s_m[w][cc] - sub);
-                L = __builtin_fmaf(s_l[w][cc], fw, L);
-                A = __builtin_fmaf(s_acc[w][cc][d], fw, A);
-            }
-            if constexpr (KIND == 1) A *= a.hm ? a.hm[a.hkv + kvh0 + head_i] : a.v_mult;
-            if (c < count) {
-                if constexpr (FUSED) {
-                    // A column folds the partitions that hold its positions, as the merge does.
-                    const int held = min(a.parts, (min(first + c + 1, a.max_keys) + a.piece - 1) / a.piece);
-                    if (part < held) {
-                        const Fold fo = fold(run_m[e], run_l[e], M, L);
-                        run_a[e] = __builtin_fmaf(run_a[e], fo.keep, A * fo.take);
-                        run_m[e] = fo.m, run_l[e] = fo.l;
-                    }
-                } else {
-                    const int64_t at = ((prow + c) * a.hq + (kvh0 + head_i) * a.g + j % a.g) * a.parts + b;
-                    a.po[at * D + d] = A;
-                    if (d == 0) a.pm[at] = M, a.pl[at] = L;
-                }
-            }
-        }
-    }
-    if constexpr (FUSED) {
-#pragma unroll
-        for (int e = 0; e < EPT; ++e) {
-            const int idx = tid + e * 256;
-            const int cc = idx / D, d = idx % D;
-            const int j = j0 + cc % CPH;
-            const int c = j / a.g;
-            if (c < count) {
-                const int head = (kvh0 + cc / CPH) * a.g + j % a.g;
-                float M = run_m[e], L = run_l[e], A = run_a[e];
-                if (a.sinks) {
-                    const Fold fo = fold(M, L, a.sinks[head] * kLog2e, 1.0f);
-                    A *= fo.keep, M = fo.m, L = fo.l;
-                }
-                const float o = L != 0.0f ? A / L : 0.0f;
-                store_out(a.out, a.out_dtype, (int64_t)(start + c) * a.o_st + (int64_t)head * a.o_sh + d, o);
-                if (a.lse && d == 0) a.lse[(int64_t)(start + c) * a.hq + head] = L != 0.0f ? __builtin_fmaf(M, kLn2, __logf(L)) : -INFINITY;
-            }
-        }
-    }
-}
-
-// The launch: as many workgroups as the card holds at once, each taking units from the launch's counter (the caller's
-// memory) until the list is exhausted. The hardware's own dispatcher binds a workgroup to an XCD by its id and starts
-// workgroups strictly in order, so with units as uneven as ragged contexts make them it leaves slots idle behind a
-// busy one; resident workgroups that pull the next unit themselves keep every slot busy to the end. The last workgroup
-// to finish zeroes the counters for the next launch that uses them. Without counters the units are dealt in turn.
-constexpr int kMfmaWaves = 2;      // wavefronts a SIMD holds (two workgroups a compute unit)
-#ifndef PKV_MFMA_TILES
-#define PKV_MFMA_TILES 2
-#endif
-constexpr int kMfmaTiles = PKV_MFMA_TILES;      // steps a wavefront keeps in flight
-
-template <int KIND, bool F16, int HW, bool FUSED, bool MASKED>
-__global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs a) {
-    __shared__ __align__(16) float s_acc[4][kTileRows][128];
-    __shared__ float s_m[4][kTileRows], s_l[4][kTileRows];
-    __shared__ unsigned s_unit;
-    const unsigned total = (unsigned)a.units_x * (unsigned)a.units_y;
-    unsigned unit = blockIdx.x;      // the first gridDim.x units need no ticket: tickets number the units after them
-    const bool pulled = a.ticket != nullptr;
-    while (unit < total) {
-        // (the next ticket is drawn after the unit, not during it: a returning atomic in flight makes every wait on
-        // the unit's loads a wait for all of them, which costs more than the ticket's round trip)
-        attend_mfma_unit<KIND, F16, HW, FUSED, MASKED, kMfmaTiles>(a, (int)(unit % (unsigned)a.units_x), (int)(unit / (unsigned)a.units_x), s_acc, s_m, s_l);
-        lds_barrier();      // the unit is done with the shared arrays, and every thread has read s_unit
+        // The unit after the next: the ticket drawn above, or, while it names a unit without work, the ones after it.
+        unsigned u_after = u_next + grid;
         if (pulled) {
-            if (threadIdx.x == 0) s_unit = gridDim.x + atomicAdd(a.ticket, 1u);
-            lds_barrier();
-            unit = s_unit;
+            if (tid == 0) {
+                unsigned found = 2 * grid + drawn;
+                while (found < total && !decode(found).valid) found = 2 * grid + atomicAdd(a.ticket, 1u);
+                s_unit = found;
+            }
+            lds_barrier();      // (and every thread is done with the fold's shared arrays)
+            u_after = s_unit;
         } else {
-            unit += gridDim.x;
+            lds_barrier();
         }
+        if (!nxt.valid && u_next >= total && u_after >= total) break;
+        cur = nxt, lead_cur = lead_nxt;
+        u_next = u_after;
+        lds_barrier();      // every thread has read s_unit before the next round's draw is published
     }
     if (!pulled) return;
     if (threadIdx.x == 0) {
-        if (atomicAdd(a.ticket + 1, 1u) == gridDim.x - 1) {
+        if (atomicAdd(a.ticket + 1, 1u) == grid - 1) {
             atomicExch(a.ticket, 0u);
             atomicExch(a.ticket + 1, 0u);
         }
