@@ -105,14 +105,11 @@ struct Tile {
 constexpr int kTileRows = 16;      // query rows (columns of S^T) a tile holds
 constexpr int kLdsRows = 512;      // batch rows whose descriptors a workgroup keeps in LDS (the others are read from memory)
 
-#ifndef PKV_MFMA_WAVES
-#define PKV_MFMA_WAVES 2
-#endif
-constexpr int kMfmaWaves = PKV_MFMA_WAVES;      // wavefronts a SIMD holds (workgroups a compute unit)
-#ifndef PKV_MFMA_TILES
-#define PKV_MFMA_TILES 2
-#endif
-constexpr int kMfmaTiles = PKV_MFMA_TILES;      // steps a wavefront keeps in flight
+// Wavefronts a SIMD holds (workgroups a compute unit) and steps a wavefront keeps in flight. Measured on MI355X: three
+// workgroups a unit (fewer registers each) and four steps in flight both stream less (the memory system is saturated by
+// two and two; more concurrent streams cost DRAM locality).
+constexpr int kMfmaWaves = 2;
+constexpr int kMfmaTiles = 2;
 
 // The launch: as many workgroups as the card holds at once, each working through units of the list (row, KV head
 // group, query tile, partition) until it is exhausted. The hardware's own dispatcher binds a workgroup to an XCD by its
@@ -137,14 +134,23 @@ __global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs
     __shared__ __align__(16) float s_acc[4][kTileRows][128];
     __shared__ float s_m[4][kTileRows], s_l[4][kTileRows];
     __shared__ int s_rows[kLdsRows][5];      // count, first position, table row, first token, first partial row
+    __shared__ int s_before[kLdsRows + 1];   // the dense list: partitions but the last of the rows before row r
+    __shared__ int s_wave_sum[4];
+    __shared__ int s_key[kLdsRows], s_order[kLdsRows];      // the dense list: the rows by the size of their last partition
     __shared__ unsigned s_unit;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c16 = lane & 15, u4 = lane >> 4;
-    const unsigned total = (unsigned)a.units_x * (unsigned)a.units_y, grid = gridDim.x;
+    const unsigned grid = gridDim.x;
     const bool pulled = a.ticket != nullptr;
     const int hgroups = a.hkv / HW;
+    // The list of units. Launches of up to kLdsRows rows take the dense list: every row's partitions but its last, row
+    // by row (each for every head group and tile), then every row's last partition (usually a partial piece: the
+    // smallest units go last) - no unit without work beyond tiles a short window row does not fill. Larger launches
+    // take the grid units_x x units_y, whose units without work are passed over as they are drawn.
+    const bool dense = a.n_rows <= kLdsRows;
+    const unsigned per_row = (unsigned)(hgroups * a.tiles);
     const int slot_bytes = a.hkv * D * EB;
     const bool tree = MASKED && (a.parents != nullptr || a.parents64 != nullptr);
     const int win = MASKED ? a.sliding : 0;
@@ -166,6 +172,60 @@ __global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs
         for (int i = 0; i < 5; ++i) s_rows[r][i] = d[i];
     }
     lds_barrier();
+    // Partitions that hold positions of row r (of its last column): what its units divide.
+    auto row_partitions = [&](int r) __attribute__((always_inline)) -> int {
+        const int count = s_rows[r][0];
+        if (count <= 0) return 0;
+        if constexpr (FUSED) return 1;
+        const int n_keys = min(s_rows[r][1] + count, a.max_keys);
+        return min((n_keys + a.piece - 1) / a.piece, a.parts);
+    };
+    if (dense) {      // s_before[r] = sum over r' < r of max(partitions(r') - 1, 0): thread i sums rows 2 i and 2 i + 1
+        const int r0 = 2 * tid, r1 = 2 * tid + 1;
+        const int c0 = r0 < a.n_rows ? max(row_partitions(r0) - 1, 0) : 0, c1 = r1 < a.n_rows ? max(row_partitions(r1) - 1, 0) : 0;
+        int run = c0 + c1;      // inclusive prefix over the threads
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int other = __shfl_up(run, o);
+            if (lane >= o) run += other;
+        }
+        if (lane == 63) s_wave_sum[wave] = run;
+        lds_barrier();
+        int base = 0;
+        for (int w = 0; w < wave; ++w) base += s_wave_sum[w];
+        const int upto = base + run - (c0 + c1);      // rows before 2 i
+        if (r0 <= a.n_rows) s_before[r0] = upto;
+        if (r1 <= a.n_rows) s_before[r1] = upto + c0;
+        if (tid == 255 && kLdsRows <= a.n_rows) s_before[kLdsRows] = upto + c0 + c1;
+        // The rows' last partitions are taken largest first (a launch's tail is as long as its last units): positions
+        // the last partition holds (more than a piece where partitions hold several pieces), ties by row.
+        for (int r = tid; r < a.n_rows; r += 256) {
+            const int count = s_rows[r][0];
+            int key = -1;
+            if (count > 0) {
+                const int n_keys = min(s_rows[r][1] + count, a.max_keys);
+                const int n_pieces = (n_keys + a.piece - 1) / a.piece;
+                key = FUSED ? n_keys : (n_pieces > a.parts ? a.piece + 1 : n_keys - (n_pieces - 1) * a.piece);
+            }
+            s_key[r] = key;
+        }
+        lds_barrier();
+        for (int r = tid; r < a.n_rows; r += 256) {
+            int rank = r;
+            if (a.n_rows <= 256) {      // (larger launches keep the rows' order: ranking them costs more than it returns)
+                const int key = s_key[r];
+                rank = 0;
+                for (int o = 0; o < a.n_rows; ++o) {
+                    const int other = s_key[o];
+                    rank += (other > key || (other == key && o < r)) ? 1 : 0;
+                }
+            }
+            s_order[rank] = r;
+        }
+        lds_barrier();
+    }
+    const unsigned phase1 = dense ? (unsigned)__builtin_amdgcn_readfirstlane(s_before[a.n_rows]) * per_row : 0u;
+    const unsigned total = dense ? phase1 + (unsigned)a.n_rows * per_row : (unsigned)a.units_x * (unsigned)a.units_y;
 
     // -- a unit of the list, decoded (everything uniform over the workgroup)
     struct Unit {
@@ -177,12 +237,31 @@ __global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs
         Unit un;
         un.valid = false;
         if (unit >= total) return un;
-        int bx = (int)(unit % (unsigned)a.units_x);
-        int b = (int)(unit / (unsigned)a.units_x);
+        int bx, b, r;
+        bool last = false;      // dense list: the row's last partition
+        if (dense) {
+            if (unit < phase1) {
+                const int q = (int)(unit / per_row);      // the q-th of all rows' partitions but their last
+                bx = (int)(unit % per_row);
+                int lo = 0, hi = a.n_rows;                // the row: s_before[r] <= q < s_before[r + 1]
+                while (hi - lo > 1) {
+                    const int mid = (lo + hi) >> 1;
+                    if (__builtin_amdgcn_readfirstlane(s_before[mid]) <= q) lo = mid;
+                    else hi = mid;
+                }
+                r = lo, b = q - __builtin_amdgcn_readfirstlane(s_before[lo]);
+            } else {
+                const unsigned rest = unit - phase1;
+                r = __builtin_amdgcn_readfirstlane(s_order[rest / per_row]), bx = (int)(rest % per_row), b = 0, last = true;
+            }
+        } else {
+            bx = (int)(unit % (unsigned)a.units_x);
+            b = (int)(unit / (unsigned)a.units_x);
+            r = bx / (int)per_row;
+            bx %= (int)per_row;
+        }
         const int tile = bx % a.tiles;
-        bx /= a.tiles;
-        un.kvh0 = (bx % hgroups) * HW;      // the first of the wavefronts' KV heads
-        const int r = bx / hgroups;
+        un.kvh0 = (bx / a.tiles) * HW;      // the first of the wavefronts' KV heads
         int d[5];
         if (r < kLdsRows) {
 #pragma unroll
@@ -206,14 +285,21 @@ __global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs
             // partition, in kTailClasses rows of y by its size (a whole piece or more first, the smallest last).
             const int np = min(un.n_pieces, a.parts);
             if (np <= 0) return un;
-            int cls = 0;
-            if (np == un.n_pieces) cls = min(kTailClasses - 1, (np * a.piece - un.n_keys) * kTailClasses / a.piece);
-            if (b >= a.units_y - kTailClasses) {
-                if (b - (a.units_y - kTailClasses) != cls) return un;
-                b = np - 1;
-            } else if (b >= np - 1) {
-                return un;
+            if (dense) {
+                if (last) b = np - 1;
+                else if (b >= np - 1) return un;      // (a tile of earlier columns that holds fewer pieces than the row's last)
+            } else {
+                int cls = 0;
+                if (np == un.n_pieces) cls = min(kTailClasses - 1, (np * a.piece - un.n_keys) * kTailClasses / a.piece);
+                if (b >= a.units_y - kTailClasses) {
+                    if (b - (a.units_y - kTailClasses) != cls) return un;
+                    b = np - 1;
+                } else if (b >= np - 1) {
+                    return un;
+                }
             }
+        } else if (dense && !last) {
+            return un;
         }
         un.b = b;
         un.valid = true;
@@ -312,7 +398,16 @@ __global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs
     int col = 0, lim = -1;
     unsigned long long anc = 0ull;
     float sscale = a.sscale;
+    float vm_cur[HW], vm_nxt[HW];      // FP8 pages: the value multipliers of the unit's heads (requested with its queries, not in its fold)
+#pragma unroll
+    for (int h = 0; h < HW; ++h) vm_cur[h] = vm_nxt[h] = 1.0f;
     u32x4 qb[4];
+    auto value_multipliers = [&](const Unit& un) __attribute__((always_inline)) {      // (requested with the unit's page table entries)
+        if constexpr (KIND == 1) {
+#pragma unroll
+            for (int h = 0; h < HW; ++h) vm_nxt[h] = a.hm ? a.hm[a.hkv + un.kvh0 + h] : a.v_mult;
+        }
+    };
     auto lane_values = [&](const Unit& un) __attribute__((always_inline)) {
         const int jr = un.j0 + c16 % CPH;
         col = jr / a.g;
@@ -346,14 +441,20 @@ __global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs
     Lead lead_cur;
     if (cur.valid) {
         lead_cur = lead_of(cur, FUSED ? 0 : cur.b);
+        value_multipliers(cur);
         fill(cur, lead_cur);
         lane_values(cur);
+#pragma unroll
+        for (int h = 0; h < HW; ++h) vm_cur[h] = vm_nxt[h];
     }
     for (;;) {
         // The next unit: its first steps' page table entries are requested now and wait in registers.
         const Unit nxt = decode(u_next);
         Lead lead_nxt = {};
-        if (nxt.valid) lead_nxt = lead_of(nxt, FUSED ? 0 : nxt.b);
+        if (nxt.valid) {
+            lead_nxt = lead_of(nxt, FUSED ? 0 : nxt.b);
+            value_multipliers(nxt);
+        }
         // The ticket of the unit after the next is drawn when the current unit's steps are done (a returning atomic
         // in flight beside a unit's loads makes the waits on them coarser) and looked at after its fold.
         unsigned drawn = 0;
@@ -539,7 +640,7 @@ __global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs
                         L = __builtin_fmaf(s_l[w][cc], fw, L);
                         A = __builtin_fmaf(s_acc[w][cc][d], fw, A);
                     }
-                    if constexpr (KIND == 1) A *= a.hm ? a.hm[a.hkv + fold_kvh0 + head_i] : a.v_mult;
+                    if constexpr (KIND == 1) A *= HW == 1 ? vm_cur[0] : (head_i == 0 ? vm_cur[0] : vm_cur[HW - 1]);
                     if (c < cur.count) {
                         if constexpr (FUSED) {
                             // A column folds the partitions that hold its positions, as the merge does.
@@ -595,6 +696,8 @@ __global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs
         }
         if (!nxt.valid && u_next >= total && u_after >= total) break;
         cur = nxt, lead_cur = lead_nxt;
+#pragma unroll
+        for (int h = 0; h < HW; ++h) vm_cur[h] = vm_nxt[h];
         u_next = u_after;
         lds_barrier();      // every thread has read s_unit before the next round's draw is published
     }

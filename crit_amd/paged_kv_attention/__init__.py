@@ -39,7 +39,7 @@ __all__ = ["KINDS", "PIECE", "MAX_COLUMNS", "Derive", "attend", "derive", "cuda_
            "tile_for", "workspace_floats", "write"]
 
 KINDS = {"bf16": 0, "fp16": 0, "fp8": 1, "fp8:row": 2, "int8": 3}
-PIECE = 2048         # positions per piece of FP8 or INT8 pages at a 128-wide head (piece_size)
+PIECE = 1536         # positions per piece of FP8 or INT8 pages at a 128-wide head (piece_size)
 MAX_COLUMNS = 64     # columns of one row a launch reads
 MAX_LISTED_BLOCKS = 1024      # block ids a token's list holds at most (attend's blocks=)
 MAX_QUERY_ROWS = 8   # query rows (columns x group heads) one workgroup holds; wider windows take more tiles
@@ -259,20 +259,22 @@ def partitions(device, kv_heads, kind, head_dim=None, value_dim=None):
     are never launched, so a large count costs short rows nothing). A column's bits depend on it: one count per
     cache."""
     if kind not in KINDS:
-        raise ValueError(f"page kinds are {', '.join(KINDS)}, not {kind!r}")
+        raise ValueError(f"{kind!r} is no page kind ({', '.join(KINDS)})")
     programs = 2 * _cus(torch.device(device))
     wanted = max(1, programs // max(1, int(kv_heads) // 2))
     return max(8, min(64, 1 << (wanted - 1).bit_length()))
 
 
 def piece_size(head_dim, value_dim, kind="bf16", kv_heads=None):
-    """Positions per piece: 128 Ki head values for 16-bit pages, 256 Ki for 8-bit ones (512 KiB of keys and values of
-    one KV head either way: measured on MI355X, a workgroup's start-up is then a few percent of its streaming),
-    within 256..2048. A column's bits depend on it; it follows the cache's geometry and page kind only."""
+    """Positions per piece: 64 Ki head values for 16-bit pages (512 positions at 128-wide heads), 192 Ki for 8-bit ones
+    (1,536), within 256..2048, a multiple of 16. Measured on MI355X: the smallest pieces large batches still stream at
+    their best rate with (a unit's fixed costs are hidden behind the next unit's rows), so a batch that does not fill
+    the chip is cut into as many units as that allows. A column's bits depend on it; it follows the cache's geometry
+    and page kind only."""
     if kind not in KINDS:
-        raise ValueError(f"page kinds are {', '.join(KINDS)}, not {kind!r}")
-    values = 131072 if KINDS[kind] == 0 else 262144
-    return max(256, min(2048, values // max(int(head_dim), int(value_dim))))
+        raise ValueError(f"{kind!r} is no page kind ({', '.join(KINDS)})")
+    values = 65536 if KINDS[kind] == 0 else 196608
+    return max(256, min(2048, values // max(int(head_dim), int(value_dim)) // 16 * 16))
 
 
 def tile_for(columns, group, capability, fused=False):
