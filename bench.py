@@ -24,10 +24,23 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, vendor figure
 
-# HBM bytes one split launch moves, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this file (each counter in
-# a run of its own, scaled by what it reads for the stream-read probe and for a 262,144-token append, kernels of
-# known size: factors 0.5000 and 1.000).
-MEASURED_TRAFFIC_BYTES = {"c2": 1_453_522_329, "c3": 2_661_386_240}
+DECODE_KERNEL = "attend_mfma_kernel"      # the split launch's kernel (the dominant one)
+
+
+def profiled_traffic(workload, piece):
+    """HBM bytes one split launch of `workload` moves, from the counter runs summarised under profiles/ (rocprofv3 --pmc
+    FETCH_SIZE and WRITE_SIZE of this file, each scaled by what it reads for a kernel of known size), or None when
+    no summary covers this kernel at this piece: the figure belongs to the kernel and the launch shape it was taken on."""
+    import re
+    path = os.path.join(ROOT, "profiles", f"{DECODE_KERNEL}_{workload}_decode.md")
+    try:
+        text = open(path, encoding="utf-8").read()
+    except OSError:
+        return None, None
+    found = re.search(r"HBM traffic per launch \(piece (\d+)\): ([\d,]+) B", text)
+    if not found or int(found.group(1)) != int(piece) or DECODE_KERNEL not in text:
+        return None, None
+    return int(found.group(2).replace(",", "")), os.path.relpath(path, ROOT)
 
 
 def log(*a):
@@ -191,8 +204,24 @@ def cpu_baseline(spec, seconds=20.0):
             "host_cpus": os.cpu_count()}
 
 
+def graph_timed(fn, launches=20, reps=5):
+    """Average milliseconds of one fn() launch replayed from a captured HIP graph of `launches` of them: the host's cost
+    of a call drops out, what is left is the kernels' own time and the gaps the hardware leaves between them."""
+    fn()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(launches):
+            fn()
+    ms = timed(graph.replay, reps, 2) / launches
+    del graph
+    return ms
+
+
 def append_sweep(pk, device, kind):
-    """KV append GB/s against the token count (algorithmic bytes: page bytes written + bf16 inputs read)."""
+    """KV append GB/s against the token count (algorithmic bytes: page bytes written + bf16 inputs read): `us` is
+    call to call through the Python module (the host's 7 us a call bound the small sizes), `kernel_us` the same launch
+    replayed from a captured graph (the kernel's own time)."""
     hkv, d, found = 8, 128, {}
     store = torch.bfloat16 if kind == "bf16" else torch.float8_e4m3fn
     e = 2 if kind == "bf16" else 1
@@ -200,13 +229,17 @@ def append_sweep(pk, device, kind):
     k = torch.zeros(n_slots, hkv, d, dtype=store, device=device)
     v = torch.zeros_like(k)
     g = torch.Generator(device=device).manual_seed(1)
-    for T in (64, 1024, 4152, 65536, 262144):
+    for T in (64, 1024, 4152, 16384, 65536, 262144):
         keys = torch.randn(T, hkv, d, device=device, generator=g).to(torch.bfloat16)
         values = torch.randn(T, hkv, d, device=device, generator=g).to(torch.bfloat16)
         slots = torch.randperm(n_slots, device=device, generator=g)[:T]
-        ms = timed(lambda: pk.write(keys, values, slots, k, v, kind, multipliers=(0.02, 0.03)), 20, 3)
+        call = lambda: pk.write(keys, values, slots, k, v, kind, multipliers=(0.02, 0.03))
+        ms = timed(call, 20, 3)
+        kernel = graph_timed(call)
         nbytes = T * hkv * 2 * d * (e + 2)
-        found[str(T)] = {"us": round(ms * 1e3, 2), "GB/s": round(nbytes / ms / 1e6, 1)}
+        found[str(T)] = {"us": round(ms * 1e3, 2), "GB/s": round(nbytes / ms / 1e6, 1),
+                         "kernel_us": round(kernel * 1e3, 2), "kernel_GB/s": round(nbytes / kernel / 1e6, 1),
+                         "kernel_frac_of_peak": round(nbytes / kernel / 1e6 / HBM_PEAK_GBPS, 4)}
     return found
 
 
@@ -485,7 +518,7 @@ def small_batches(pk, device):
     """What a piece costs a batch that does not fill the chip: one layer's decode launch (split + merge, 8B shape) for
     4 sequences of about 2,000 positions and for one of 8,000, at the default piece and at pieces of 256 positions
     (attend's piece=, the plugin's `piece` option: fixed per pool either way). Microseconds a launch over four layers of
-    different memory; the launches are queued without waits, so a figure near the host's cost of a call is bound by it."""
+    different memory, replayed from a captured graph (the host's cost of a call is not in the figure)."""
     hq, hkv, d, page, found = 32, 8, 128, 16, {}
     g = torch.Generator(device=device).manual_seed(3)
     for kind in ("bf16", "fp8"):
@@ -508,8 +541,8 @@ def small_batches(pk, device):
                 pk.attend(q, k[at[0]], v[at[0]], kind, tables, rows, rows, firsts, 1, page, out=out, piece=piece,
                           multipliers=(0.02, 0.03))
             default = pk.piece_size(d, d, kind, hkv)
-            found[f"{kind}_{name}"] = {f"piece_{default}_us": round(timed(lambda: launch(default), 40, 4) * 1e3, 1),
-                                       "piece_256_us": round(timed(lambda: launch(256), 40, 4) * 1e3, 1)}
+            found[f"{kind}_{name}"] = {f"piece_{default}_us": round(graph_timed(lambda: launch(default), 16) * 1e3, 1),
+                                       "piece_256_us": round(graph_timed(lambda: launch(256), 16) * 1e3, 1)}
     return found
 
 
@@ -647,6 +680,7 @@ def main():
     merge_ms = kernel_ms(w, 2)
     append_ms = timed(lambda: w.append(0), 50, 5)
     achieved = w.decode_bytes / split_ms / 1e6
+    traffic, traffic_source = profiled_traffic(args.workload, w.piece)
     sink = torch.zeros(64, device=device)
     read_ms, read_bytes = None, 0
     for layer in range(min(4, w.layers)):
@@ -661,9 +695,9 @@ def main():
         "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if w.kind == "bf16" else "fp8_e4m3 KV, bf16 q, f32 accumulate", "data": "synthetic",
         "config": {"workload": spec["name"], "positions": w.tokens, "partitions": w.parts, "piece": w.piece},
-        "roofline": {"bound": "hbm", "kernel": "attend_kernel (split launch)", "achieved": round(achieved, 1),
+        "roofline": {"bound": "hbm", "kernel": f"{DECODE_KERNEL} (split launch)", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "launch_ms": round(split_ms, 4), "merge_ms": round(merge_ms, 4),
                      "algorithmic_bytes_per_launch": w.decode_bytes,
                      "stream_read_GB/s": round(stream_gbps, 1)},
@@ -692,17 +726,25 @@ def main():
         extras = {}
         other = "c3" if args.workload == "c2" else "c2"
         ospec = WORKLOADS[other]
-        log(f"[bench] extra: {other} on 8 layers")
-        ow = Workload(ospec, device, layers=8)
+        log(f"[bench] the other decode workload at its full size: {other}, {ospec['layers']} layers")
+        ow = Workload(ospec, device)
         for _ in range(2):
             ow.step()
         ms = timed(ow.step, 3, 0)
         osplit = kernel_ms(ow, 1)
-        extras[other] = {"workload": ospec["name"] + " (8 of 32 layers resident; per-layer figures)",
-                         "ms_per_layer": round(ms / ow.layers, 4),
+        otraffic, osource = profiled_traffic(other, ow.piece)
+        extras[other] = {"workload": ospec["name"], "layers": ow.layers, "positions": ow.tokens, "piece": ow.piece,
+                         "ms_per_step": round(ms, 3), "ms_per_layer": round(ms / ow.layers, 4),
                          "GB/s": round((ow.decode_bytes + ow.append_bytes) * ow.layers / ms / 1e6, 1),
+                         "fraction_of_peak": round((ow.decode_bytes + ow.append_bytes) * ow.layers / ms / 1e6 / HBM_PEAK_GBPS, 4),
                          "split_launch_ms": round(osplit, 4), "split_launch_GB/s": round(ow.decode_bytes / osplit / 1e6, 1),
                          "frac": round(ow.decode_bytes / osplit / 1e6 / HBM_PEAK_GBPS, 4)}
+        # the other workload's dominant kernel against its roofline, beside the default workload's
+        result[f"roofline_{other}"] = {"bound": "hbm", "kernel": f"{DECODE_KERNEL} (split launch)",
+                                       "achieved": round(ow.decode_bytes / osplit / 1e6, 1), "peak": HBM_PEAK_GBPS,
+                                       "unit": "GB/s", "frac": round(ow.decode_bytes / osplit / 1e6 / HBM_PEAK_GBPS, 4),
+                                       "traffic": otraffic, "traffic_source": osource, "launch_ms": round(osplit, 4),
+                                       "algorithmic_bytes_per_launch": ow.decode_bytes, "workload": ospec["name"]}
         # the same launches with pieces twice as long (attend's piece=, a deployment's choice through the plugin's
         # `piece` option: fixed per pool like the default; halves the units' fixed costs, and a small batch's units)
         ow.piece *= 2
