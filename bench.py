@@ -244,14 +244,16 @@ def append_sweep(pk, device, kind):
 
 
 def append_rope(pk, device):
-    """KV append with the keys' rotary embedding fused in (write's rope=) beside the plain append of the same rows:
-    8 KV heads x 128, bf16 inputs; bytes as the plain append's (the table's rows are read besides: 512 B a token)."""
+    """KV append with the keys' rotary embedding fused in (write's rope=), and with their RMS norm in front of it as
+    well (norm=), beside the plain append of the same rows: 8 KV heads x 128, bf16 inputs; bytes as the plain append's
+    (the table's rows are read besides: 512 B a token; the norm's 128 weights stay in cache)."""
     hkv, d, found = 8, 128, {}
     n_slots = 1 << 20
     g = torch.Generator(device=device).manual_seed(2)
     angle = torch.arange(8192, dtype=torch.float64, device=device)[:, None] / \
         (10000.0 ** (torch.arange(d // 2, dtype=torch.float64, device=device) / (d // 2)))[None, :]
     table = torch.cat([angle.cos(), angle.sin()], 1).float().contiguous()
+    weight = torch.rand(d, device=device, generator=g) + 0.5
     for kind in ("bf16", "fp8"):
         store = torch.bfloat16 if kind == "bf16" else torch.float8_e4m3fn
         e = 2 if kind == "bf16" else 1
@@ -266,9 +268,13 @@ def append_rope(pk, device):
             plain = timed(lambda: pk.write(keys, values, slots, k, v, kind, multipliers=(0.02, 0.03)), 20, 3)
             fused = timed(lambda: pk.write(keys, values, slots, k, v, kind, multipliers=(0.02, 0.03),
                                            rope=(table, positions)), 20, 3)
+            normed = timed(lambda: pk.write(keys, values, slots, k, v, kind, multipliers=(0.02, 0.03),
+                                            rope=(table, positions), norm=(weight, 1e-6)), 20, 3)
             nbytes = T * hkv * 2 * d * (e + 2)
             found[kind][str(T)] = {"plain_us": round(plain * 1e3, 2), "with_rope_us": round(fused * 1e3, 2),
-                                   "with_rope_GB/s": round(nbytes / fused / 1e6, 1)}
+                                   "with_rope_GB/s": round(nbytes / fused / 1e6, 1),
+                                   "with_norm_and_rope_us": round(normed * 1e3, 2),
+                                   "with_norm_and_rope_GB/s": round(nbytes / normed / 1e6, 1)}
         del k, v
     return found
 

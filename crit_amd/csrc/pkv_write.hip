@@ -26,6 +26,10 @@ struct WriteArgs {
     int64_t rope_rows;
     int rope_interleaved;
     float rope_scale;
+    // RMS norm of each key head in front of the rotation (norm_weight null: none): x / sqrt(mean(x^2) + eps) times
+    // (norm_weight[i] + norm_offset), FP32 [dim[0]].
+    const float* norm_weight;
+    float norm_eps, norm_offset;
 };
 
 template <int IN>
@@ -205,6 +209,42 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
         float mine[EPL], other[EPL], y[EPL];
         raw[0].widen(mine);
         raw[0].across(LPR / 2).widen(other);
+        if (a.norm_weight) {
+            // The reference's rms_norm_rope (inference/fused-norms/code/torch_norms.py:149-176): each head normalised
+            // in FP32, times its weight, rotated, one rounding at the end. The sum of squares in a fixed order, the same
+            // for every page kind: squares rounded one by one, groups of 8 consecutive elements summed in order, the
+            // groups by a balanced tree of adjacent pairs (a lane of 16 elements adds its two groups first; then the
+            // row's lanes 1, 2, 4 ... apart); mean, square root and reciprocal correctly rounded.
+            float sq = 0.0f;
+#pragma unroll
+            for (int g8 = 0; g8 < EPL / 8; ++g8) {
+                float s8 = mine[8 * g8] * mine[8 * g8];
+#pragma unroll
+                for (int j = 1; j < 8; ++j) s8 = s8 + mine[8 * g8 + j] * mine[8 * g8 + j];
+                sq = g8 == 0 ? s8 : sq + s8;
+            }
+#pragma unroll
+            for (int o = 1; o < LPR; o <<= 1) sq = sq + __shfl_xor(sq, o);
+            const float mean = __fdiv_rn(sq, (float)a.dim[0]);
+            // __builtin_sqrtf is the correctly rounded root (hipcc's default for sqrtf and "/"); __fsqrt_rn is not,
+            // unless OCML_BASIC_ROUNDED_OPERATIONS is defined: it is the hardware's approximate one.
+            const float r = __fdiv_rn(1.0f, __builtin_sqrtf(mean + a.norm_eps));
+            const int i_other = (lane_in_row ^ (LPR / 2)) * EPL;      // the partner lane's first element (style half)
+            const float4* w_mine = reinterpret_cast<const float4*>(a.norm_weight + i0);
+            const float4* w_other = reinterpret_cast<const float4*>(a.norm_weight + i_other);
+#pragma unroll
+            for (int j = 0; j < EPL / 4; ++j) {
+                const float4 wm = w_mine[j], wo = w_other[j];
+                const float m4[4] = {wm.x, wm.y, wm.z, wm.w}, o4[4] = {wo.x, wo.y, wo.z, wo.w};
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const float fm = a.norm_offset != 0.0f ? m4[k] + a.norm_offset : m4[k];
+                    const float fo = a.norm_offset != 0.0f ? o4[k] + a.norm_offset : o4[k];
+                    mine[4 * j + k] = (mine[4 * j + k] * r) * fm;
+                    other[4 * j + k] = (other[4 * j + k] * r) * fo;
+                }
+            }
+        }
         if (a.rope_interleaved) {
 #pragma unroll
             for (int j = 0; j < EPL / 2; ++j) {
@@ -441,6 +481,8 @@ int launch_write(const crit_pkv_write_params* p, hipStream_t stream) {
     a.mult[0] = p->key_multiplier, a.mult[1] = p->value_multiplier;
     a.rope_table = p->rope_table, a.positions = p->rope_positions, a.rope_rows = p->rope_rows;
     a.rope_interleaved = p->rope_interleaved ? 1 : 0, a.rope_scale = p->rope_scale;
+    a.norm_weight = p->norm_weight, a.norm_eps = p->norm_eps, a.norm_offset = p->norm_offset;
+    if (p->norm_weight && (!p->rope_table || (reinterpret_cast<uintptr_t>(p->norm_weight) % 16))) return CRIT_PKV_E_GEOMETRY;
     if (p->rope_table) {
         // the whole head width rotates, a power of two of whole lanes; the lanes of a values' row of another width
         // would not line up with the keys' in the exchange

@@ -307,7 +307,7 @@ def _workspace(device, tokens, heads, parts, dv, given=None):
 
 # -- writes ----------------------------------------------------------------------------------------------------------------
 def write(keys, values, slots, key_pages, value_pages, kind, key_scales=None, value_scales=None,
-          multipliers=(1.0, 1.0), *, rope=None):
+          multipliers=(1.0, 1.0), *, rope=None, norm=None):
     """A step's keys [tokens][kv_heads][dim] and values [tokens][kv_heads][value_dim] (FP32, BF16 or FP16) into their
     slots ([tokens] int64; a slot below 0 is skipped) of one layer's pages (any view whose storage is
     [slots][kv_heads][dim]), encoded for the page kind, in one launch; the bytes torch's own casts would store
@@ -317,7 +317,11 @@ def write(keys, values, slots, key_pages, value_pages, kind, key_scales=None, va
     inference/fused-norms/code/torch_norms.py:89-147, fused into this launch): (table, positions) or (table, positions,
     style, scale): table FP32 [rows][dim] (cos of every pair, then sin), positions [tokens] int64 (clamped to the table's
     rows), style "half" (pairs j, j + dim / 2) or "interleaved" (2j, 2j + 1), scale on cos and sin; the keys go in as
-    rope() would have returned them in their own dtype. Head widths 64, 128, 256, values no wider than keys."""
+    rope() would have returned them in their own dtype. Head widths 64, 128, 256, values no wider than keys.
+    norm, with rope: (weight, eps) or (weight, eps, offset): each key head's RMS norm in front of the rotation, the
+    reference's rms_norm_rope() (torch_norms.py:149-176; what rms_norm_rope_pair does to the keys, blocks.py:160-170)
+    fused in as well: x / sqrt(mean(x^2) + eps) * (weight + offset) in FP32, rotated in FP32, rounded once to the keys'
+    dtype. weight: [dim], any float dtype (read as FP32)."""
     if keys is None:
         if rope is not None:
             raise ValueError("rope rotates keys")
@@ -378,6 +382,20 @@ def write(keys, values, slots, key_pages, value_pages, kind, key_scales=None, va
             raise ValueError("rope in the append takes head widths 64, 128 and 256, values no wider than keys")
         p.rope_table, p.rope_positions, p.rope_rows = table.data_ptr(), positions.data_ptr(), table.shape[0]
         p.rope_interleaved, p.rope_scale = int(style == "interleaved"), float(scale)
+    if norm is not None:
+        if rope is None:
+            raise ValueError("norm is the RMS norm in front of the keys' rotation: it comes with rope")
+        if not 2 <= len(norm) <= 3:
+            raise ValueError("norm is (weight, eps) or (weight, eps, offset)")
+        weight, eps, offset = tuple(norm) + (0.0,)[len(norm) - 2:]
+        if not torch.is_tensor(weight) or tuple(weight.shape) != (d,) or weight.device != keys.device or \
+                not weight.is_floating_point():
+            raise ValueError(f"norm's weight is a float [{d}] tensor on the keys' device")
+        if weight.dtype != torch.float32 or not weight.is_contiguous() or weight.data_ptr() % 16:
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError("paged_kv_attention.write: a captured append takes norm's weight as contiguous FP32")
+            weight = weight.float().contiguous().clone()
+        p.norm_weight, p.norm_eps, p.norm_offset = weight.data_ptr(), float(eps), float(offset)
     _launch(keys.device, "crit_pkv_write", "paged_kv_attention.write", p)
 
 

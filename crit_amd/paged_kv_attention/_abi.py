@@ -10,7 +10,7 @@ import shutil
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 NAME = "libcrit_pkv.so"
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 KIND_16BIT, KIND_FP8, KIND_FP8_ROW, KIND_INT8 = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
@@ -26,7 +26,7 @@ class WriteParams(ctypes.Structure):
                 ("kv_heads", _i32), ("head_dim", _i32), ("value_dim", _i32), ("kind", _i32), ("page_dtype", _i32),
                 ("in_dtype", _i32), ("key_multiplier", _f32), ("value_multiplier", _f32),
                 ("rope_table", _p), ("rope_positions", _p), ("rope_rows", _i64), ("rope_interleaved", _i32),
-                ("rope_scale", _f32)]
+                ("rope_scale", _f32), ("norm_weight", _p), ("norm_eps", _f32), ("norm_offset", _f32)]
 
 
 class AttendParams(ctypes.Structure):

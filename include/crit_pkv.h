@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 12
+#define CRIT_PKV_ABI_VERSION 13
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -81,6 +81,15 @@ typedef struct crit_pkv_write_params {
     int64_t rope_rows;
     int32_t rope_interleaved;
     float rope_scale;
+    /* RMS norm of each key head in front of the rotation: the reference's rms_norm_rope() (inference/fused-norms/code/
+     * torch_norms.py:149-176; the keys' half of rms_norm_rope_pair, :307-316, called at inference/model-template/code/
+     * blocks.py:160-170). norm_weight NULL: none. Else FP32 [head_dim], 16-byte aligned, with rope_table: each key head
+     * becomes x / sqrt(mean(x^2) + norm_eps) * (norm_weight[i] + norm_offset) in FP32, is rotated in FP32 and rounded
+     * once to in_dtype, then appended. The sum of squares is taken in a fixed order (squares rounded one by one, groups
+     * of 8 consecutive elements in order, the groups by a balanced tree of adjacent pairs); division, square root and
+     * reciprocal are correctly rounded. */
+    const float* norm_weight;
+    float norm_eps, norm_offset;
 } crit_pkv_write_params;
 
 int crit_pkv_write(const crit_pkv_write_params* p, void* stream);

@@ -140,3 +140,38 @@ def rope(x, positions, table, style="half", scale=1.0):
     else:
         raise ValueError(style)
     return turned.to(x.dtype)
+
+
+def sum_of_squares(x32):
+    """The FP32 sum of squares of each last-dimension row (a multiple of 8 wide, that many groups a power of two) in
+    the fixed order the fused append takes it in: every square rounded to FP32, groups of 8 consecutive elements summed
+    in order, the groups by a balanced tree of adjacent pairs. Plain FP32 additions, no fused multiply-add."""
+    import numpy as np
+    sq = x32.numpy().astype(np.float32)
+    sq = sq * sq
+    groups = sq.reshape(*sq.shape[:-1], sq.shape[-1] // 8, 8)
+    s = groups[..., 0].copy()
+    for j in range(1, 8):
+        s = s + groups[..., j]
+    while s.shape[-1] > 1:
+        s = s[..., 0::2] + s[..., 1::2]
+    return torch.from_numpy(s[..., 0].astype(np.float32))
+
+
+def rms_norm_rope(x, weight, eps, positions, table, offset=0.0, style="half", scale=1.0):
+    """Each token's heads [tokens][heads][dim] RMS-normalised, weighted and rotated at its position, as the reference's
+    rms_norm_rope() (inference/fused-norms/code/torch_norms.py:149-176: rms_norm of each head in FP32, times weight (+
+    offset), then rope, FP32 between them, one rounding to x's dtype) over the whole head width with a
+    [positions][dim] table. The reference's mean of squares is torch's (its order of summation is the library's own);
+    here it is sum_of_squares() / dim, so that a kernel can reproduce the bytes; 1 / sqrt(mean + eps) by an IEEE square
+    root and an IEEE division (what torch's CPU rsqrt does), (x * r) * (weight + offset) as two FP32 products."""
+    import numpy as np
+    x32 = x.float()
+    dim = x.shape[-1]
+    mean = (sum_of_squares(x32).numpy() / np.float32(dim)).astype(np.float32)
+    r = (np.float32(1.0) / np.sqrt(mean + np.float32(eps), dtype=np.float32)).astype(np.float32)
+    factor = weight.float()
+    if offset:
+        factor = factor + offset
+    normed = (x32 * torch.from_numpy(r)[..., None]) * factor
+    return rope(normed, positions, table, style, scale).to(x.dtype)

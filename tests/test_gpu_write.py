@@ -264,3 +264,46 @@ def test_keys_rotated_on_their_way_in_are_the_bytes_of_rope_then_write(kind, d, 
             pk.write(keys.to(dev), None, slots.to(dev), k, None, kind, rope=(table.to(dev), positions[:5].to(dev)))
         with pytest.raises(ValueError):
             pk.write(keys.to(dev), None, slots.to(dev), k, None, kind, rope=(table.to(dev), positions.to(dev), "pairs"))
+
+
+@pytest.mark.parametrize("kind,d,dv,in_dtype", [("bf16", 128, 128, torch.bfloat16), ("fp8", 128, 128, torch.bfloat16),
+                                           ("fp8:row", 128, 128, torch.float32), ("int8", 64, 64, torch.bfloat16),
+                                           ("fp16", 256, 256, torch.float16), ("fp8", 256, 128, torch.float32),
+                                           ("bf16", 64, 64, torch.float32)])
+@pytest.mark.parametrize("style", ["half", "interleaved"])
+def test_keys_normed_and_rotated_on_their_way_in_are_the_bytes_of_rms_norm_rope_then_write(kind, d, dv, in_dtype, style):
+    # write(rope=..., norm=(weight, eps, offset)): the reference's rms_norm_rope() on the keys (inference/fused-norms/
+    # code/torch_norms.py:149-176; the keys' half of rms_norm_rope_pair, what model-template runs before the append,
+    # blocks.py:160-170) fused into the launch: every stored byte and row scale equals the oracle's rms_norm_rope()
+    # followed by its write(); the values are neither normed nor rotated. With and without an offset, with a scale on
+    # the rotation, a weight in the keys' dtype.
+    pk = kernels()
+    g = torch.Generator().manual_seed(53)
+    T, hkv, P = 70, 3, 200
+    keys = (torch.randn(T, hkv, d, generator=g) * 3).to(in_dtype)
+    keys[5] = 0                       # a row of zeros: eps alone under the root
+    values = torch.randn(T, hkv, dv, generator=g).to(in_dtype)
+    half = d // 2
+    angle = torch.arange(P, dtype=torch.float64)[:, None] / (10000.0 ** (torch.arange(half, dtype=torch.float64) / half))[None, :]
+    table = torch.cat([angle.cos(), angle.sin()], 1).float()
+    positions = torch.randint(0, P, (T,), generator=g)
+    slots = torch.randperm(96, generator=g)[:T]
+    slots[11] = -1
+    mult = (0.05, 0.07)
+    weight = torch.randn(d, generator=g) * 0.3 + 1
+    for eps, offset, scale, w in ((1e-6, 0.0, 1.0, weight), (1e-5, 1.0, 0.75, (weight - 1).to(in_dtype))):
+        k = torch.zeros(96, hkv, d, dtype=STORE[kind], device=dev)
+        v = torch.zeros(96, hkv, dv, dtype=STORE[kind], device=dev)
+        ks = vs = None
+        if kind in ("fp8:row", "int8"):
+            ks, vs = torch.zeros(96, hkv, device=dev), torch.zeros(96, hkv, device=dev)
+        pk.write(keys.to(dev), values.to(dev), slots.to(dev), k, v, kind, ks, vs, multipliers=mult,
+                 rope=(table.to(dev), positions.to(dev), style, scale), norm=(w.to(dev), eps, offset))
+        turned = oracle_append.rms_norm_rope(keys, w, eps, positions, table, offset, style, scale)
+        want = expected_pages(kind, turned, values, slots, 96, mult)
+        _check(kind, (k, v, ks, vs), want)
+    with pytest.raises(ValueError, match="rope"):
+        pk.write(keys.to(dev), values.to(dev), slots.to(dev), k, v, kind, ks, vs, norm=(weight.to(dev), 1e-6))
+    with pytest.raises(ValueError):
+        pk.write(keys.to(dev), values.to(dev), slots.to(dev), k, v, kind, ks, vs,
+                 rope=(table.to(dev), positions.to(dev), style), norm=(weight[:8].to(dev), 1e-6))

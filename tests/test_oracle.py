@@ -683,3 +683,66 @@ def test_rope_turns_each_pair_by_its_positions_angle(style):
     torch.testing.assert_close(scaled, got * 0.5, atol=1e-6, rtol=1e-6)
     low = append.rope(x.bfloat16(), positions, table, style)
     assert low.dtype == torch.bfloat16 and torch.equal(low, append.rope(x.bfloat16().float(), positions, table, style).bfloat16())
+
+
+@pytest.mark.parametrize("style", ["half", "interleaved"])
+def test_rms_norm_rope_normalises_weighs_and_turns(style):
+    # Pins append.rms_norm_rope(): against the closed form in float64 (x / sqrt(mean(x^2) + eps) * (w + offset), then
+    # the rotation as complex numbers) to FP32 rounding; against a scalar loop in numpy float32 taking the sum of
+    # squares in the stated order (bit for bit); against torch's own rms_norm followed by the rotation (the reference's
+    # text, torch_norms.py:60-68, 149-176: its summation order is the library's, so a few outputs may round the other
+    # way); by what the norm fixes (mean square 1 before the weight when eps = 0; c x normalises to what x does for a
+    # power of two c, bit for bit); and at position 0 with weight 1 it is the plain norm.
+    g = torch.Generator().manual_seed(43)
+    T, H, D, P = 6, 3, 64, 40
+    half = D // 2
+    freqs = 1.0 / (10000.0 ** (torch.arange(half, dtype=torch.float64) / half))
+    angle = torch.arange(P, dtype=torch.float64)[:, None] * freqs[None, :]
+    table = torch.cat([angle.cos(), angle.sin()], 1).float()
+    x = torch.randn(T, H, D, generator=g) * 3
+    weight = torch.randn(D, generator=g) * 0.2 + 1
+    positions = torch.tensor([0, 3, 39, 17, 5, 44])
+    eps, offset = 1e-6, 0.5
+    got = append.rms_norm_rope(x, weight, eps, positions, table, offset, style)
+    at = positions.clamp(0, P - 1)
+    xd = x.double()
+    normed = xd / (xd.pow(2).mean(-1, keepdim=True) + eps).sqrt() * (weight.double() + offset)
+    pair = (lambda t: (t[..., :half], t[..., half:])) if style == "half" else (lambda t: (t[..., 0::2], t[..., 1::2]))
+    a, b = pair(normed)
+    turned = torch.complex(a, b) * torch.polar(torch.ones(T, 1, half, dtype=torch.float64), angle[at][:, None, :])
+    ga, gb = pair(got.double())
+    torch.testing.assert_close(ga, turned.real, atol=5e-6, rtol=5e-6)
+    torch.testing.assert_close(gb, turned.imag, atol=5e-6, rtol=5e-6)
+    # the scalar loop, the same order of every operation
+    xn, wn, tn = x.numpy(), weight.numpy(), table.numpy()
+    for t in range(T):
+        for h in range(H):
+            groups = []
+            for g8 in range(D // 8):
+                s8 = np.float32(xn[t, h, 8 * g8] * xn[t, h, 8 * g8])
+                for j in range(1, 8):
+                    s8 = np.float32(s8 + np.float32(xn[t, h, 8 * g8 + j] * xn[t, h, 8 * g8 + j]))
+                groups.append(s8)
+            while len(groups) > 1:
+                groups = [np.float32(groups[i] + groups[i + 1]) for i in range(0, len(groups), 2)]
+            r = np.float32(np.float32(1.0) / np.sqrt(np.float32(np.float32(groups[0] / np.float32(D)) + np.float32(eps))))
+            n = [np.float32(np.float32(xn[t, h, i] * r) * np.float32(wn[i] + np.float32(offset))) for i in range(D)]
+            for j in range(half):
+                ia, ib = (j, j + half) if style == "half" else (2 * j, 2 * j + 1)
+                c, s = tn[int(at[t]), j], tn[int(at[t]), half + j]
+                assert np.float32(np.float32(n[ia] * c) - np.float32(n[ib] * s)) == got[t, h, ia].item(), (t, h, j)
+                assert np.float32(np.float32(n[ib] * c) + np.float32(n[ia] * s)) == got[t, h, ib].item(), (t, h, j)
+    # torch's own norm (another summation order) then the oracle's rotation: equal but for the last place of a few
+    theirs = torch.nn.functional.rms_norm(x.float(), (D,), eps=eps) * (weight.float() + offset)
+    theirs = append.rope(theirs, positions, table, style)
+    torch.testing.assert_close(got, theirs, atol=1e-6, rtol=1e-6)
+    # invariants
+    plain = append.rms_norm_rope(x, torch.ones(D), 0.0, torch.zeros(T, dtype=torch.int64), table, 0.0, style)
+    torch.testing.assert_close(plain.double().pow(2).mean(-1), torch.ones(T, H, dtype=torch.float64), atol=1e-6, rtol=1e-6)
+    assert torch.equal(append.rms_norm_rope(4 * x, weight, 0.0, positions, table, offset, style),
+                       append.rms_norm_rope(x, weight, 0.0, positions, table, offset, style))
+    # 16-bit inputs come back in their dtype, rounded once
+    xb = x.bfloat16()
+    gb16 = append.rms_norm_rope(xb, weight, eps, positions, table, offset, style)
+    assert gb16.dtype == torch.bfloat16
+    assert torch.equal(gb16, append.rms_norm_rope(xb.float(), weight, eps, positions, table, offset, style).bfloat16())
