@@ -70,8 +70,11 @@ def test_the_module_keeps_the_reference_interface():
     write = inspect.signature(pk.write).parameters
     assert list(write)[:9] == [
         "keys", "values", "slots", "key_pages", "value_pages", "kind", "key_scales", "value_scales", "multipliers"]
-    # (beyond the reference's: the keys' rotary embedding fused into the append, by keyword only)
-    assert list(write)[9:] == ["rope"] and write["rope"].kind is inspect.Parameter.KEYWORD_ONLY and write["rope"].default is None
+    # (beyond the reference's: the keys' rotary embedding, and their RMS norm in front of it, fused into the append, by
+    # keyword only)
+    assert list(write)[9:] == ["rope", "norm"]
+    for extra in ("rope", "norm"):
+        assert write[extra].kind is inspect.Parameter.KEYWORD_ONLY and write[extra].default is None
     attend = inspect.signature(pk.attend).parameters
     assert list(attend)[:10] == ["q", "key_pages", "value_pages", "kind", "tables", "rows", "starts", "firsts", "columns",
                                  "page"]
