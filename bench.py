@@ -467,6 +467,36 @@ def pool_bookkeeping(pk, device):
     rows = torch.randint(0, B, (4152,), device=device, generator=g)
     ms = timed(lambda: pk.slots_at(tables, capacity, slot_ids, many, page, pages, rows=rows), 50, 3)
     found["slots_at_4152_positions_us"] = round(ms * 1e3, 2)
+    # a decode step's buffers (slots, window entries, tables) and the round's lengths, on the device, beside the host's
+    # way of building the same step (Python lists -> pinned tensors -> six copies: pages.py:359-397)
+    buffers = pk.StepBuffers(B, B, table_pages, pages, device)
+    start = torch.zeros(B, dtype=torch.int64, device=device)
+    ones = torch.ones(B, dtype=torch.int64, device=device)
+    ms = timed(lambda: pk.step_buffers(buffers, tables, capacity, lengths, slot_ids, page, 16), 50, 3)
+    found["step_buffers_64_rows"] = {"us": round(ms * 1e3, 2)}
+    ms = graph_timed(lambda: pk.step_buffers(buffers, tables, capacity, lengths, slot_ids, page, 16))
+    found["step_buffers_64_rows"]["kernel_us"] = round(ms * 1e3, 2)
+    ms = timed(lambda: pk.commit_round(lengths, start, ones, lengths), 50, 3)
+    found["commit_round_64_rows_us"] = round(ms * 1e3, 2)
+    host_tables, host_lengths = tables.tolist(), lengths.tolist()
+    h_slots = torch.zeros(B, dtype=torch.int64, pin_memory=True)
+    h_meta = torch.zeros(B, 4, dtype=torch.int64, pin_memory=True)
+    h_tables = torch.zeros(B, table_pages, dtype=torch.int32, pin_memory=True)
+
+    def host_step():
+        slots_l = [host_tables[r][host_lengths[r] // page] * page + host_lengths[r] % page for r in range(B)]
+        h_slots.copy_(torch.tensor(slots_l, dtype=torch.int64))
+        for r in range(B):
+            h_meta[r] = torch.tensor([r, 1, host_lengths[r], r], dtype=torch.int64)
+            h_tables[r] = torch.tensor(host_tables[r], dtype=torch.int32)
+        buffers.d_slots.copy_(h_slots, non_blocking=True)
+        buffers.d_starts.copy_(h_meta[:, 0], non_blocking=True)
+        buffers.d_counts.copy_(h_meta[:, 1], non_blocking=True)
+        buffers.d_firsts.copy_(h_meta[:, 2], non_blocking=True)
+        buffers.d_offsets.copy_(h_meta[:, 3], non_blocking=True)
+        buffers.d_tables.copy_(h_tables, non_blocking=True)
+    ms = timed(host_step, 10, 2)
+    found["step_buffers_64_rows"]["host_lists_and_copies_us"] = round(ms * 1e3, 2)
     path = torch.tensor([0, 2, 3, 5, 6, -1, -1, -1], device=device).repeat(B, 1)
     emitted = torch.full((B,), 5, dtype=torch.int64, device=device)
     moved = torch.zeros(B, dtype=torch.int64, device=device)

@@ -35,6 +35,14 @@ int crit_pkv_copy_pages(const crit_pkv_copy_pages_params* p, void* stream) {
     return pkv::launch_copy_pages(p, reinterpret_cast<hipStream_t>(stream));
 }
 
+int crit_pkv_round(const crit_pkv_round_params* p, void* stream) {
+    return pkv::launch_round(p, reinterpret_cast<hipStream_t>(stream));
+}
+
+int crit_pkv_step_buffers(const crit_pkv_step_params* p, void* stream) {
+    return pkv::launch_step_buffers(p, reinterpret_cast<hipStream_t>(stream));
+}
+
 int crit_pkv_read_rows(const crit_pkv_read_params* p, void* stream) {
     return pkv::launch_read_rows(p, reinterpret_cast<hipStream_t>(stream));
 }
@@ -65,6 +73,8 @@ int crit_pkv_params_size(int which) {
         case 5: return (int)sizeof(crit_pkv_compact_params);
         case 6: return (int)sizeof(crit_pkv_copy_pages_params);
         case 7: return (int)sizeof(crit_pkv_read_params);
+        case 8: return (int)sizeof(crit_pkv_round_params);
+        case 9: return (int)sizeof(crit_pkv_step_params);
     }
     return -1;
 }

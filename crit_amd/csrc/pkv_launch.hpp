@@ -13,6 +13,8 @@ int launch_prefill(const crit_pkv_prefill_params* p, hipStream_t stream);
 int launch_slots_at(const crit_pkv_slots_params* p, hipStream_t stream);
 int launch_compact(const crit_pkv_compact_params* p, hipStream_t stream);
 int launch_copy_pages(const crit_pkv_copy_pages_params* p, hipStream_t stream);
+int launch_round(const crit_pkv_round_params* p, hipStream_t stream);
+int launch_step_buffers(const crit_pkv_step_params* p, hipStream_t stream);
 int launch_read_rows(const crit_pkv_read_params* p, hipStream_t stream);
 int launch_stream_read(const void* data, int64_t bytes, float* sink, hipStream_t stream);
 // Compute units of the current device (cached per device), or 0 if the query fails.

@@ -1,5 +1,5 @@
 // Pool bookkeeping on the device (gfx950): the slots of positions through the bound page tables, the move of an accepted
-// draft-tree path's rows to consecutive positions, and the copy of whole pages. Integer and byte work, HBM-bound where
+// draft-tree path's rows to consecutive positions, the copy of whole pages, a round's lengths and a step's buffers. Integer and byte work, HBM-bound where
 // it is bound by anything: what the reference does with torch indexing (inference/attention-state/code/pages.py:646-684,
 // 861-869), one launch each, nothing read on the host.
 #include "pkv_launch.hpp"
@@ -119,6 +119,97 @@ __global__ __launch_bounds__(256) void set_moved_kernel(int64_t* moved, int64_t 
     if (i < rows) moved[i] = 1;
 }
 
+// KVPool.start_round / the end of commit_round (pages.py:623-644), one thread a round row.
+__global__ __launch_bounds__(256) void round_kernel(int64_t* lengths, int64_t* start, int64_t* moved, const int64_t* emitted,
+                                                    const int64_t* frontier, int64_t rows, int commit) {
+    const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (r >= rows) return;
+    if (commit) {
+        lengths[r] = emitted[r] > 0 ? frontier[r] : start[r];
+    } else {
+        start[r] = lengths[r];
+        if (moved) moved[r] = 0;
+    }
+}
+
+struct StepArgs {
+    const int64_t *lengths, *slot, *counts, *firsts;
+    int64_t *d_slots, *positions_t, *rows_t;
+    int32_t *starts_t, *d_rows, *d_starts, *d_counts;
+    int64_t* d_firsts;
+    int32_t *d_offsets, *d_tables;
+    int64_t* totals;
+    int64_t rows, d_tables_stride, step_tokens, step_rows, count_each, window;
+    int dump;
+};
+
+__device__ __forceinline__ int64_t count_of(const StepArgs& a, int64_t r) {
+    const int64_t c = a.counts ? a.counts[r] : a.count_each;
+    return c < 0 ? 0 : c;
+}
+
+// A step's buffers. Workgroup b < rows is row b; workgroup rows + w is window entry w, which it empties if fewer window
+// rows exist. Every workgroup adds up the rows before its own (all rows, for an entry): the counts are a few KiB that
+// stay in cache, and no workgroup waits for another.
+__global__ __launch_bounds__(256) void step_kernel(Tables t, StepArgs a) {
+    __shared__ int64_t s_sum[4][3];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const bool is_row = (int64_t)blockIdx.x < a.rows;
+    const int64_t r = is_row ? (int64_t)blockIdx.x : a.rows;      // rows before r are added up
+    int64_t tokens = 0, windows = 0, window_tokens = 0;
+    for (int64_t i = tid; i < r; i += 256) {
+        const int64_t c = count_of(a, i);
+        tokens += c;
+        if (c <= a.window) windows += 1, window_tokens += c;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        tokens += __shfl_xor(tokens, o);
+        windows += __shfl_xor(windows, o);
+        window_tokens += __shfl_xor(window_tokens, o);
+    }
+    if (lane == 0) s_sum[wave][0] = tokens, s_sum[wave][1] = windows, s_sum[wave][2] = window_tokens;
+    __syncthreads();
+    tokens = s_sum[0][0] + s_sum[1][0] + s_sum[2][0] + s_sum[3][0];
+    windows = s_sum[0][1] + s_sum[1][1] + s_sum[2][1] + s_sum[3][1];
+    window_tokens = s_sum[0][2] + s_sum[1][2] + s_sum[2][2] + s_sum[3][2];
+    if (!is_row) {
+        const int64_t w = (int64_t)blockIdx.x - a.rows;
+        if (w == 0 && tid == 0) {
+            a.totals[0] = tokens, a.totals[1] = windows, a.totals[2] = window_tokens;
+            a.totals[3] = tokens > a.step_tokens || windows > a.step_rows ? 1 : 0;
+            if (a.starts_t) a.starts_t[a.rows] = (int32_t)tokens;
+        }
+        if (w < windows || w >= a.step_rows) return;
+        if (tid == 0) {
+            if (a.d_rows) a.d_rows[w] = (int32_t)w;
+            a.d_starts[w] = 0, a.d_counts[w] = 0, a.d_firsts[w] = 0, a.d_offsets[w] = (int32_t)window_tokens;
+        }
+        for (int e = tid; e < t.table_pages; e += 256) a.d_tables[w * a.d_tables_stride + e] = a.dump;
+        return;
+    }
+    const int64_t s = a.slot[r], count = count_of(a, r);
+    const bool bound = s >= 0 && s < t.round_slots;
+    const int64_t first = a.firsts ? a.firsts[r] : (bound ? a.lengths[s] : 0);
+    if (tid == 0 && a.starts_t) a.starts_t[r] = (int32_t)tokens;
+    for (int64_t j = tid; j < count; j += 256) {
+        const int64_t i = tokens + j;
+        if (i >= a.step_tokens) break;
+        a.d_slots[i] = slot_at(t, s, first + j);
+        if (a.positions_t) a.positions_t[i] = first + j;
+        if (a.rows_t) a.rows_t[i] = r;
+    }
+    if (count > a.window || windows >= a.step_rows) return;
+    const int64_t w = windows;
+    if (tid == 0) {
+        if (a.d_rows) a.d_rows[w] = (int32_t)w;
+        a.d_starts[w] = (int32_t)tokens, a.d_counts[w] = (int32_t)count, a.d_firsts[w] = first;
+        a.d_offsets[w] = (int32_t)window_tokens;
+    }
+    for (int e = tid; e < t.table_pages; e += 256)
+        a.d_tables[w * a.d_tables_stride + e] = bound ? t.tables[s * t.table_stride + e] : a.dump;
+}
+
 // One workgroup: a piece of one page of one layer of one store; every load of a thread issued before its stores.
 template <typename G>
 __device__ __forceinline__ void copy_piece(uint8_t* base, int64_t page_bytes, int64_t from, int64_t to, int piece) {
@@ -230,6 +321,38 @@ int launch_copy_pages(const crit_pkv_copy_pages_params* p, hipStream_t stream) {
     const dim3 grid((unsigned)(pieces * p->n), (unsigned)p->layers, (unsigned)p->n_stores);
     hipLaunchKernelGGL(copy_pages_kernel, grid, dim3(256), 0, stream, stores, p->source, p->target, p->page, (int)pieces,
                        p->pool_pages);
+    return (int)hipGetLastError();
+}
+
+int launch_round(const crit_pkv_round_params* p, hipStream_t stream) {
+    if (!p) return CRIT_PKV_E_NULL;
+    if (p->rows == 0) return 0;
+    if (!p->round_lengths || !p->start || (p->commit && (!p->emitted || !p->frontier))) return CRIT_PKV_E_NULL;
+    if (p->rows < 0 || p->rows > ((int64_t)1 << 31) * 255) return CRIT_PKV_E_GEOMETRY;
+    hipLaunchKernelGGL(round_kernel, dim3((unsigned)((p->rows + 255) / 256)), dim3(256), 0, stream, p->round_lengths, p->start,
+                       p->moved, p->emitted, p->frontier, p->rows, p->commit);
+    return (int)hipGetLastError();
+}
+
+int launch_step_buffers(const crit_pkv_step_params* p, hipStream_t stream) {
+    if (!p) return CRIT_PKV_E_NULL;
+    if (!p->slot || !p->d_slots || !p->d_starts || !p->d_counts || !p->d_firsts || !p->d_offsets || !p->d_tables || !p->totals ||
+        (!p->round_lengths && !p->firsts))
+        return CRIT_PKV_E_NULL;
+    if (const int bad = check_tables(p->round_tables, p->round_capacity, p->round_slots, p->table_stride, p->table_pages,
+                                     p->page, p->dump))
+        return bad;
+    if (p->rows < 0 || p->rows > 32768 || p->step_rows < 0 || p->step_rows > 32768 || p->step_tokens < 0 ||
+        p->step_tokens > 0x7fffffff || p->d_tables_stride < p->table_pages || p->window < 0 || (!p->counts && p->count_each < 0))
+        return CRIT_PKV_E_GEOMETRY;
+    const Tables t{p->round_tables, p->round_capacity, p->round_slots, p->table_stride, p->table_pages, p->page,
+                   (int64_t)p->dump * p->page};
+    const StepArgs a{p->round_lengths, p->slot, p->counts, p->firsts, p->d_slots, p->positions_t, p->rows_t, p->starts_t,
+                     p->d_rows, p->d_starts, p->d_counts, p->d_firsts, p->d_offsets, p->d_tables, p->totals, p->rows,
+                     p->d_tables_stride, p->step_tokens, p->step_rows, p->count_each, p->window, p->dump};
+    // (one workgroup a row, one a window entry, and at least the one that writes the totals)
+    const int64_t grid = p->rows + (p->step_rows > 0 ? p->step_rows : 1);
+    hipLaunchKernelGGL(step_kernel, dim3((unsigned)grid), dim3(256), 0, stream, t, a);
     return (int)hipGetLastError();
 }
 

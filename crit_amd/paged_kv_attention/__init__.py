@@ -946,6 +946,102 @@ def copy_pages(stores, slots, source, target, page):
     _launch(device, "crit_pkv_copy_pages", "paged_kv_attention.copy_pages", p)
 
 
+def start_round(round_lengths, start, moved, rows):
+    """A round begins, KVPool.start_round (pages.py:623-628) in one launch: start[:rows] = round_lengths[:rows] (each
+    row's valid length as the round finds it) and moved[:rows] = 0 (no row's tree path moved yet; moved may be None).
+    int64 tensors on one device; capture-safe."""
+    _require_device(round_lengths, "the round lengths")
+    device, rows = round_lengths.device, int(rows)
+    if rows < 0:
+        raise ValueError("a round has zero rows or more")
+    p = _abi.RoundParams()
+    p.round_lengths = _i64_on(round_lengths, device, "the round lengths", rows).data_ptr()
+    p.start = _i64_on(start, device, "start", rows).data_ptr()
+    p.moved = None if moved is None else _i64_on(moved, device, "moved", rows).data_ptr()
+    p.rows, p.commit = rows, 0
+    _launch(device, "crit_pkv_round", "paged_kv_attention.start_round", p)
+
+
+def commit_round(round_lengths, start, emitted, frontier, *, tree=None):
+    """After a round's acceptance, KVPool.commit_round (pages.py:630-644) without the host: with tree=(stores, slots,
+    round_tables, round_capacity, path, moved, page, dump) the accepted draft-tree path's rows move to consecutive
+    positions first (compact(), once a round); then round_lengths[r] = frontier[r] where emitted[r] > 0, start[r] (the
+    length the round found) where the row emitted nothing, for r < len(emitted). A second commit from the same start
+    (a truncation) finds the path moved and sets the lengths again. int64 tensors on one device; capture-safe."""
+    _require_device(round_lengths, "the round lengths")
+    device = round_lengths.device
+    rows = _i64_on(emitted, device, "emitted").numel()
+    if tree is not None:
+        stores, slots, round_tables, round_capacity, path, moved, page, dump = tree
+        compact(stores, slots, round_tables, round_capacity, start, emitted, path[:rows], moved, page, dump)
+    p = _abi.RoundParams()
+    p.round_lengths = _i64_on(round_lengths, device, "the round lengths", rows).data_ptr()
+    p.start = _i64_on(start, device, "start", rows).data_ptr()
+    p.emitted, p.frontier = emitted.data_ptr(), _i64_on(frontier, device, "frontier", rows).data_ptr()
+    p.rows, p.commit = rows, 1
+    _launch(device, "crit_pkv_round", "paged_kv_attention.commit_round", p)
+
+
+class StepBuffers:
+    """A pool's step buffers at fixed device addresses, as KVPool holds them (pages.py:200-217): d_slots [step_tokens]
+    int64; d_rows, d_starts, d_counts, d_offsets [step_rows] int32; d_firsts [step_rows] int64; d_tables [step_rows]
+    [table_pages] int32; and a StepBatch's device tensors beside them (core/python/crit_plugins/device.py:590-616):
+    starts_t [step_rows + 1] int32, positions_t and rows_t [step_tokens] int64. totals [4] int64: the step's tokens,
+    window rows, window tokens and whether it overflowed the buffers. Made outside a capture; step_buffers() fills them."""
+
+    def __init__(self, step_rows, step_tokens, table_pages, dump, device):
+        if step_rows < 1 or step_tokens < step_rows or table_pages < 1:
+            raise ValueError("step buffers hold one row or more, a token a row or more, and tables of one page or more")
+        long, int32 = dict(dtype=torch.int64, device=device), dict(dtype=torch.int32, device=device)
+        self.step_rows, self.step_tokens, self.table_pages, self.dump = int(step_rows), int(step_tokens), int(table_pages), int(dump)
+        self.d_slots = torch.zeros(step_tokens, **long)
+        self.positions_t, self.rows_t = torch.zeros(step_tokens, **long), torch.zeros(step_tokens, **long)
+        self.starts_t = torch.zeros(step_rows + 1, **int32)
+        self.d_rows, self.d_starts = torch.arange(step_rows, **int32), torch.zeros(step_rows, **int32)
+        self.d_counts, self.d_offsets = torch.zeros(step_rows, **int32), torch.zeros(step_rows, **int32)
+        self.d_firsts = torch.zeros(step_rows, **long)
+        self.d_tables = torch.full((step_rows, table_pages), dump, **int32)
+        self.totals = torch.zeros(4, **long)
+
+
+def step_buffers(buffers, round_tables, round_capacity, round_lengths, slot, page, window, *, counts=None, count=1,
+                 firsts=None):
+    """A step over sequences bound to round slots, built on the device in one launch: what StepBatch.build
+    (core/python/crit_plugins/device.py:600-616), reserve()'s slots (pages.py:337-349) and KVPool._step_buffers
+    (pages.py:359-397) make on the host. Row r is `counts[r]` tokens (`count` each without counts) of the sequence in
+    round slot slot[r] from position firsts[r] (without firsts: round_lengths[slot[r]], the first position without KV).
+    Fills `buffers` (a StepBuffers): every token's slot, position and row, the rows' first tokens, and for the rows of
+    up to `window` tokens their window entries (first token, count, first position, first partial row, page table);
+    entries past the window rows are emptied, so attend() over all step_rows entries reads nothing for them.
+    buffers.totals says afterwards whether the step fitted (the host does not wait for it). int64 tensors on the tables'
+    device; capture-safe. Returns buffers."""
+    _tables(round_tables, round_capacity)
+    device = round_tables.device
+    rows = _i64_on(slot, device, "step_buffers' slot").numel()
+    if rows > buffers.step_rows or round_tables.shape[1] != buffers.table_pages or buffers.d_tables.device != device:
+        raise ValueError(f"the step buffers hold {buffers.step_rows} rows of {buffers.table_pages} table pages on "
+                         f"{buffers.d_tables.device}: {rows} rows of {round_tables.shape[1]} pages on {device} do not fit")
+    p = _abi.StepParams()
+    p.round_tables, p.round_capacity = round_tables.data_ptr(), round_capacity.data_ptr()
+    p.round_lengths = None if round_lengths is None else \
+        _i64_on(round_lengths, device, "the round lengths", round_tables.shape[0]).data_ptr()
+    if round_lengths is None and firsts is None:
+        raise ValueError("rows start at firsts or at the round lengths")
+    p.slot = slot.data_ptr()
+    p.counts = None if counts is None else _i64_on(counts, device, "step_buffers' counts", rows).data_ptr()
+    p.firsts = None if firsts is None else _i64_on(firsts, device, "step_buffers' firsts", rows).data_ptr()
+    p.d_slots, p.positions_t, p.rows_t = buffers.d_slots.data_ptr(), buffers.positions_t.data_ptr(), buffers.rows_t.data_ptr()
+    p.starts_t, p.d_rows, p.d_starts = buffers.starts_t.data_ptr(), buffers.d_rows.data_ptr(), buffers.d_starts.data_ptr()
+    p.d_counts, p.d_firsts, p.d_offsets = buffers.d_counts.data_ptr(), buffers.d_firsts.data_ptr(), buffers.d_offsets.data_ptr()
+    p.d_tables, p.totals = buffers.d_tables.data_ptr(), buffers.totals.data_ptr()
+    p.rows, p.round_slots, p.table_stride = rows, round_tables.shape[0], round_tables.stride(0)
+    p.d_tables_stride, p.step_tokens, p.step_rows = buffers.d_tables.stride(0), buffers.step_tokens, buffers.step_rows
+    p.count_each, p.window = int(count), int(window)
+    p.table_pages, p.page, p.dump = buffers.table_pages, int(page), buffers.dump
+    _launch(device, "crit_pkv_step_buffers", "paged_kv_attention.step_buffers", p)
+    return buffers
+
+
 # -- rows read back (reference: inference/attention-state/code/pages.py:455-493) -----------------------------------------
 def _read(key_pages, value_pages, kind, n, shape, dtype, key_scales, value_scales, multipliers, slots=None, table=None,
           page=0, out=None):

@@ -10,7 +10,7 @@ import shutil
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 NAME = "libcrit_pkv.so"
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 KIND_16BIT, KIND_FP8, KIND_FP8_ROW, KIND_INT8 = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
@@ -90,6 +90,20 @@ class CopyPagesParams(ctypes.Structure):
                 ("n_stores", _i32), ("layers", _i32), ("page", _i32)]
 
 
+class RoundParams(ctypes.Structure):
+    _fields_ = [("round_lengths", _p), ("start", _p), ("moved", _p), ("emitted", _p), ("frontier", _p), ("rows", _i64),
+                ("commit", _i32)]
+
+
+class StepParams(ctypes.Structure):
+    _fields_ = [("round_tables", _p), ("round_capacity", _p), ("round_lengths", _p), ("slot", _p), ("counts", _p),
+                ("firsts", _p), ("d_slots", _p), ("positions_t", _p), ("rows_t", _p), ("starts_t", _p), ("d_rows", _p),
+                ("d_starts", _p), ("d_counts", _p), ("d_firsts", _p), ("d_offsets", _p), ("d_tables", _p), ("totals", _p),
+                ("rows", _i64), ("round_slots", _i64), ("table_stride", _i64), ("d_tables_stride", _i64),
+                ("step_tokens", _i64), ("step_rows", _i64), ("count_each", _i64), ("window", _i64),
+                ("table_pages", _i32), ("page", _i32), ("dump", _i32)]
+
+
 class ReadParams(ctypes.Structure):
     _fields_ = [("key_pages", _p), ("value_pages", _p), ("key_scales", _p), ("value_scales", _p), ("head_multipliers", _p),
                 ("slots", _p), ("table", _p), ("table64", _p), ("out_keys", _p), ("out_values", _p), ("n", _i64), ("pool_slots", _i64),
@@ -100,7 +114,7 @@ class ReadParams(ctypes.Structure):
 STATIC_SCRATCH_BYTES = 32 << 20
 
 SYMBOLS = ("crit_pkv_write", "crit_pkv_attend", "crit_pkv_attend_static", "crit_pkv_merge", "crit_pkv_prefill", "crit_pkv_slots_at",
-           "crit_pkv_compact", "crit_pkv_copy_pages", "crit_pkv_read_rows", "crit_pkv_abi_version", "crit_pkv_params_size", "crit_pkv_error",
+           "crit_pkv_compact", "crit_pkv_copy_pages", "crit_pkv_round", "crit_pkv_step_buffers", "crit_pkv_read_rows", "crit_pkv_abi_version", "crit_pkv_params_size", "crit_pkv_error",
            "crit_pkv_stream_read", "crit_pkv_stream_capture")
 
 _lib = None
@@ -149,7 +163,8 @@ def load():
                          ("crit_pkv_attend_static", AttendParams),
                          ("crit_pkv_merge", MergeParams), ("crit_pkv_prefill", PrefillParams),
                          ("crit_pkv_slots_at", SlotsParams), ("crit_pkv_compact", CompactParams),
-                         ("crit_pkv_copy_pages", CopyPagesParams), ("crit_pkv_read_rows", ReadParams)):
+                         ("crit_pkv_copy_pages", CopyPagesParams), ("crit_pkv_round", RoundParams),
+                         ("crit_pkv_step_buffers", StepParams), ("crit_pkv_read_rows", ReadParams)):
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(struct), ctypes.c_void_p]
@@ -160,7 +175,7 @@ def load():
     if lib.crit_pkv_abi_version() != ABI_VERSION:
         raise RuntimeError(f"{path} speaks ABI {lib.crit_pkv_abi_version()}, this package {ABI_VERSION}: rebuild it")
     for which, struct in enumerate((WriteParams, AttendParams, MergeParams, PrefillParams, SlotsParams, CompactParams,
-                                    CopyPagesParams, ReadParams)):
+                                    CopyPagesParams, ReadParams, RoundParams, StepParams)):
         if lib.crit_pkv_params_size(which) != ctypes.sizeof(struct):
             raise RuntimeError(f"{path}: parameter struct {which} is {lib.crit_pkv_params_size(which)} bytes, the "
                                f"Python mirror {ctypes.sizeof(struct)}: rebuild the library")

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 13
+#define CRIT_PKV_ABI_VERSION 14
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -319,6 +319,64 @@ typedef struct crit_pkv_copy_pages_params {
 
 int crit_pkv_copy_pages(const crit_pkv_copy_pages_params* p, void* stream);
 
+/* Replaces KVPool.start_round and the length update that ends KVPool.commit_round (pages.py:623-644), for round rows
+ * 0 .. rows - 1 (round slot r is row r), one launch, nothing read on the host:
+ *   commit == 0 (a round begins):  start[r] = round_lengths[r];  moved[r] = 0 (moved may be NULL)
+ *   commit != 0 (after acceptance): round_lengths[r] = emitted[r] > 0 ? frontier[r] : start[r]
+ * A held row (it emitted nothing) keeps the length the round found; a second commit from the same start (a truncation)
+ * sets the lengths again from it. The tree path's move (crit_pkv_compact) comes before a commit, as in the reference. */
+typedef struct crit_pkv_round_params {
+    int64_t* round_lengths;         /* [>= rows] */
+    int64_t* start;                 /* [>= rows] */
+    int64_t* moved;                 /* [>= rows], commit == 0 only; optional */
+    const int64_t* emitted;         /* [rows], commit != 0 */
+    const int64_t* frontier;        /* [rows], commit != 0 */
+    int64_t rows;
+    int32_t commit;
+} crit_pkv_round_params;
+
+int crit_pkv_round(const crit_pkv_round_params* p, void* stream);
+
+/* Replaces, for rows of sequences bound to round slots, what the host builds every step: StepBatch.build's starts,
+ * positions and rows (core/python/crit_plugins/device.py:600-616), the slots reserve() finds (pages.py:337-349) and
+ * KVPool._step_buffers' window rows (pages.py:359-397). Row r holds counts[r] tokens (count_each without counts; a
+ * negative count reads as 0) of the sequence in round slot slot[r], the first at firsts[r] (without firsts: at
+ * round_lengths[slot[r]], the sequence's first position without KV). With tokens_before(r) the tokens of the rows
+ * before r, for each token j of row r, at i = tokens_before(r) + j:
+ *   positions_t[i] = first + j;  rows_t[i] = r;  d_slots[i] = the slot of first + j as crit_pkv_slots_at finds it
+ *   starts_t[r] = tokens_before(r);  starts_t[rows] = the tokens of all rows
+ * and for the w-th row whose count is at most `window` (a window row, in row order):
+ *   d_rows[w] = w; d_starts[w] = tokens_before(r); d_counts[w] = count; d_firsts[w] = first;
+ *   d_offsets[w] = the tokens of the window rows before it; d_tables[w][:] = round_tables[slot[r]][:] (the dump page's
+ *   id for a slot outside 0 .. round_slots - 1 and past table_pages)
+ * Window entries from the number of window rows up to step_rows - 1 are set empty (count 0, table all dump page), so a
+ * launch over all step_rows entries reads nothing for them. totals[0..3] = tokens, window rows, window tokens, and 1
+ * if the tokens exceed step_tokens or the window rows step_rows (what exceeds is not written; the reference raises
+ * ValueError on the host there, pages.py:365-368), else 0. One launch; capture-safe. rows <= 32768. */
+typedef struct crit_pkv_step_params {
+    const int32_t* round_tables;    /* [round_slots][table_stride >= table_pages] */
+    const int64_t* round_capacity;  /* [round_slots] */
+    const int64_t* round_lengths;   /* [round_slots]; may be NULL with firsts */
+    const int64_t* slot;            /* [rows] */
+    const int64_t* counts;          /* optional [rows] */
+    const int64_t* firsts;          /* optional [rows] */
+    int64_t* d_slots;               /* [step_tokens] */
+    int64_t* positions_t;           /* optional [step_tokens] */
+    int64_t* rows_t;                /* optional [step_tokens] */
+    int32_t* starts_t;              /* optional [rows + 1] */
+    int32_t* d_rows;                /* optional [step_rows] */
+    int32_t* d_starts;              /* [step_rows] */
+    int32_t* d_counts;              /* [step_rows] */
+    int64_t* d_firsts;              /* [step_rows] */
+    int32_t* d_offsets;             /* [step_rows] */
+    int32_t* d_tables;              /* [step_rows][d_tables_stride >= table_pages] */
+    int64_t* totals;                /* [4] */
+    int64_t rows, round_slots, table_stride, d_tables_stride, step_tokens, step_rows, count_each, window;
+    int32_t table_pages, page, dump;
+} crit_pkv_step_params;
+
+int crit_pkv_step_buffers(const crit_pkv_step_params* p, void* stream);
+
 /* ---- rows read back ----------------------------------------------------------------------------------------------
  * Replaces the index_select, cast and multiply of KVPool.gather and KVPool.rows_at (pages.py:455-493): row i of the
  * output is the pool's row at slots[i], or, with a page table instead (exactly one of slots, table, table64), at
@@ -349,7 +407,7 @@ int crit_pkv_read_rows(const crit_pkv_read_params* p, void* stream);
 /* ---- housekeeping ------------------------------------------------------------------------------------------------- */
 int crit_pkv_abi_version(void);
 /* sizeof() of the parameter structs as the library was compiled, for the host's mirror to cross-check
- * (which: 0 write, 1 attend, 2 merge, 3 prefill, 4 slots_at, 5 compact, 6 copy_pages, 7 read_rows), as crit_cw_params_size() does (cuda_window.cu:1502). */
+ * (which: 0 write, 1 attend, 2 merge, 3 prefill, 4 slots_at, 5 compact, 6 copy_pages, 7 read_rows, 8 round, 9 step_buffers), as crit_cw_params_size() does (cuda_window.cu:1502). */
 int crit_pkv_params_size(int which);
 const char* crit_pkv_error(int code);
 /* *id = the id of the capture `stream` is recording into (never 0), or 0 when it is not capturing; returns 0 or a HIP

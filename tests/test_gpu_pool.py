@@ -235,3 +235,203 @@ def test_a_decode_step_from_positions_on_the_device_replays_from_one_graph():
                                                      page, d ** -0.5)
             torch.testing.assert_close(out_g[1, s:s + 1].double().cpu(), want, atol=2e-2, rtol=2e-2)
         lengths += torch.tensor([1, 16, 3], device=dev)      # the sequences grow on the device
+
+
+def test_a_rounds_lengths_start_and_commit_on_the_device():
+    # KVPool.start_round / commit_round's lengths (pages.py:623-644) against the oracle on random rounds, and the
+    # reference's known answers (tests/test_rounds.py:66-72, 113-133).
+    pk = kernels()
+    g = torch.Generator().manual_seed(21)
+    slots, rows = 700, 613
+    lengths = torch.randint(0, 5000, (slots,), generator=g)
+    start, moved = torch.full((slots,), -1), torch.ones(slots, dtype=torch.int64)
+    d_lengths, d_start, d_moved = lengths.to(dev), start.to(dev), moved.to(dev)
+    for _ in range(3):
+        emitted = torch.randint(0, 3, (rows,), generator=g)
+        frontier = torch.randint(0, 6000, (rows,), generator=g)
+        oracle_pool.start_round(lengths, start, moved, rows)
+        pk.start_round(d_lengths, d_start, d_moved, rows)
+        assert torch.equal(d_start.cpu(), start) and torch.equal(d_moved.cpu(), moved)
+        moved[:rows] = 1
+        d_moved[:rows] = 1
+        oracle_pool.commit_round(lengths, start, emitted, frontier)
+        pk.commit_round(d_lengths, d_start, emitted.to(dev), frontier.to(dev))
+        assert torch.equal(d_lengths.cpu(), lengths)
+    lengths, start = torch.tensor([20, 30, 7], device=dev), torch.tensor([-1, -1, -1], device=dev)
+    pk.start_round(lengths, start, None, 2)
+    pk.commit_round(lengths, start, torch.tensor([3, 0], device=dev), torch.tensor([23, 30], device=dev))
+    pk.commit_round(lengths, start, torch.tensor([2, 0], device=dev), torch.tensor([22, 30], device=dev))
+    assert lengths.tolist() == [22, 30, 7] and start.tolist() == [20, 30, -1]
+    lengths[1] = 27
+    pk.start_round(lengths, start, None, 2)
+    pk.commit_round(lengths, start, torch.tensor([2, 0], device=dev), torch.tensor([24, 31], device=dev))
+    assert lengths.tolist() == [24, 27, 7]
+    pk.start_round(lengths, start, None, 0)      # no rows: nothing launched
+    with pytest.raises(ValueError):
+        pk.commit_round(lengths, start, torch.zeros(4, dtype=torch.int64, device=dev), torch.zeros(4, dtype=torch.int64, device=dev))
+
+
+def _bound(page, table_pages, held, round_slots, seed):
+    """Round tables of sequences bound with all the pages they hold, and the same tables as the host's lists."""
+    tables, capacity, dump = _round_pool(page, table_pages, held, round_slots, seed)
+    lists = {s: tables[s, :-(-n // page)].tolist() for s, n in held}
+    return tables, capacity, dump, lists
+
+
+@pytest.mark.parametrize("rows_n,window", [(1, 1), (7, 4), (300, 16), (1000, 3)])
+def test_a_steps_buffers_built_on_the_device_are_the_ones_the_host_builds(rows_n, window):
+    # StepBatch.build + reserve()'s slots + _step_buffers (device.py:600-616, pages.py:337-397) for bound sequences.
+    pk = kernels()
+    page, table_pages, round_slots = 16, 24, rows_n + 3
+    g = torch.Generator().manual_seed(rows_n)
+    held = [(s, int(torch.randint(40, table_pages * page + 1, (1,), generator=g))) for s in range(round_slots) if s % 5 != 4]
+    tables, capacity, dump, lists = _bound(page, table_pages, held, round_slots, seed=rows_n + 1)
+    bound = torch.tensor([s for s, _ in held])
+    slot = bound[torch.randperm(len(bound), generator=g)[:rows_n]]
+    rows_n = slot.numel()
+    counts = torch.randint(1, 2 * window + 1, (rows_n,), generator=g)
+    counts[::3] = 1
+    lengths = torch.zeros(round_slots, dtype=torch.int64)
+    for s, n in held:
+        lengths[s] = int(torch.randint(0, n - 2 * window + 1, (1,), generator=g))      # every token inside the capacity
+    rows = [(int(s), int(lengths[s]), int(c)) for s, c in zip(slot, counts)]
+    starts, positions, row_of = oracle_pool.step_batch(rows)
+    slots, d_starts, d_counts, d_firsts, d_offsets, d_tables = oracle_pool.step_buffers(lists, rows, page, dump, window, table_pages)
+    n, k = len(d_starts), len(slots)
+    step_rows, step_tokens = rows_n + 5, k + 9
+    buffers = pk.StepBuffers(step_rows, step_tokens, table_pages, dump, dev)
+    for t in (buffers.d_slots, buffers.positions_t, buffers.rows_t, buffers.starts_t, buffers.d_starts, buffers.d_counts,
+              buffers.d_firsts, buffers.d_offsets, buffers.d_tables):
+        t.fill_(-77)
+    found = pk.step_buffers(buffers, tables.to(dev), capacity.to(dev), lengths.to(dev), slot.to(dev), page, window,
+                            counts=counts.to(dev))
+    assert found is buffers and buffers.totals.tolist() == [k, n, sum(d_counts), 0]
+    assert buffers.d_slots[:k].tolist() == slots and buffers.positions_t[:k].tolist() == positions
+    assert buffers.rows_t[:k].tolist() == row_of and buffers.starts_t[:rows_n + 1].tolist() == starts
+    assert buffers.d_slots[k:].eq(-77).all() and buffers.positions_t[k:].eq(-77).all()
+    assert buffers.d_starts[:n].tolist() == d_starts and buffers.d_counts[:n].tolist() == d_counts
+    assert buffers.d_firsts[:n].tolist() == d_firsts and buffers.d_offsets[:n].tolist() == d_offsets
+    assert buffers.d_tables[:n].tolist() == d_tables and buffers.d_rows.tolist() == list(range(step_rows))
+    # entries past the window rows are empty: no tokens, every page the dump page
+    assert buffers.d_counts[n:].eq(0).all() and buffers.d_tables[n:].eq(dump).all() and buffers.d_starts[n:].eq(0).all()
+    assert buffers.d_offsets[n:].eq(sum(d_counts)).all()
+    # one count for every row, first positions given, buffers that are too small
+    firsts = torch.tensor([r[1] for r in rows])
+    pk.step_buffers(buffers, tables.to(dev), capacity.to(dev), None, slot.to(dev), page, window, count=window, firsts=firsts.to(dev))
+    same = [(s, f, window) for s, f, _ in rows]
+    slots2, d_starts2, _, d_firsts2, d_offsets2, _ = oracle_pool.step_buffers(lists, same, page, dump, window, table_pages)
+    if len(slots2) <= step_tokens:
+        assert buffers.totals.tolist() == [len(slots2), rows_n, len(slots2), 0]
+        assert buffers.d_slots[:len(slots2)].tolist() == slots2 and buffers.d_starts[:rows_n].tolist() == d_starts2
+        assert buffers.d_firsts[:rows_n].tolist() == d_firsts2 and buffers.d_offsets[:rows_n].tolist() == d_offsets2
+    small = pk.StepBuffers(max(1, n - 1), max(1, n - 1, k // 2), table_pages, dump, dev) if rows_n > 1 else None
+    if small is not None and rows_n <= small.step_rows:
+        pk.step_buffers(small, tables.to(dev), capacity.to(dev), lengths.to(dev), slot.to(dev), page, window, counts=counts.to(dev))
+        assert small.totals.tolist() == [k, n, sum(d_counts), 1]
+        assert small.d_slots.tolist() == slots[:small.step_tokens]
+
+
+def test_a_step_row_of_an_unbound_slot_lands_on_the_dump_page():
+    pk = kernels()
+    page, table_pages = 16, 4
+    tables, capacity, dump, _ = _bound(page, table_pages, [(0, 64), (2, 20)], 3, seed=5)
+    buffers = pk.StepBuffers(4, 16, table_pages, dump, dev)
+    lengths = torch.tensor([10, 3, 19], device=dev)
+    slot = torch.tensor([2, 1, 7, 0], device=dev)      # slot 1 holds nothing, slot 7 does not exist
+    pk.step_buffers(buffers, tables.to(dev), capacity.to(dev), lengths, slot, page, 2, count=2)
+    t = tables.tolist()
+    assert buffers.d_slots[:8].tolist() == [t[2][1] * 16 + 3, dump * 16, dump * 16, dump * 16, dump * 16, dump * 16,
+                                            t[0][0] * 16 + 10, t[0][0] * 16 + 11]      # (position 20 of slot 2: past its capacity)
+    assert buffers.d_firsts.tolist() == [19, 3, 0, 10] and buffers.d_tables[2].tolist() == [dump] * 4
+    assert buffers.d_tables[1].tolist() == t[1] and buffers.totals.tolist() == [8, 4, 8, 0]
+    with pytest.raises(ValueError):
+        pk.step_buffers(buffers, tables.to(dev), capacity.to(dev), lengths, torch.zeros(5, dtype=torch.int64, device=dev), page, 2)
+    with pytest.raises(ValueError):
+        pk.step_buffers(buffers, tables.to(dev), capacity.to(dev), None, slot, page, 2)
+
+
+def test_a_whole_step_buffers_append_attention_commit_replays_from_one_graph():
+    # A decode step with nothing built on the host: the step's buffers from the bound tables and the lengths on the
+    # device, the tokens' keys and values appended at the buffers' slots, attention over the buffers' window entries (two
+    # of the six entries stay empty), the lengths committed; captured once. Every replay equals the same step built the
+    # reference's way on the host (oracle lists -> tensors) and launched eagerly, bit for bit.
+    pk = kernels()
+    page, layers, hq, hkv, d, B, width = 16, 2, 8, 2, 128, 4, 2
+    table_pages = 32
+    tables, capacity, dump, lists = _bound(page, table_pages, [(0, 500), (1, 500), (2, 500), (3, 500)], 5, seed=30)
+    tables_d, capacity_d = tables.contiguous().to(dev), capacity.to(dev)
+    g = torch.Generator().manual_seed(31)
+
+    def fresh_pool():
+        g2 = torch.Generator().manual_seed(32)
+        k = (torch.randn(layers, dump + 1, page, hkv, d, generator=g2) * 0.5).bfloat16().to(dev)
+        v = (torch.randn(layers, dump + 1, page, hkv, d, generator=g2) * 0.5).bfloat16().to(dev)
+        return k, v
+    pools = {"graph": fresh_pool(), "eager": fresh_pool()}
+    lengths = torch.tensor([40, 333, 7, 90, 0], dtype=torch.int64, device=dev)
+    host_lengths = lengths.tolist()
+    slot = torch.tensor([3, 0, 2, 1], dtype=torch.int64, device=dev)
+    counts = torch.tensor([1, 2, 2, 1], dtype=torch.int64, device=dev)
+    T = int(counts.sum())
+    step_rows, step_tokens = 6, 8
+    buffers = pk.StepBuffers(step_rows, step_tokens, table_pages, dump, dev)
+    start, emitted, frontier = torch.zeros(5, dtype=torch.int64, device=dev), torch.ones(B, dtype=torch.int64, device=dev), \
+        torch.zeros(step_rows, dtype=torch.int64, device=dev)
+    keys = torch.randn(layers, step_tokens, hkv, d, generator=g).bfloat16().to(dev)
+    values = torch.randn(layers, step_tokens, hkv, d, generator=g).bfloat16().to(dev)
+    q = torch.randn(layers, step_tokens, hq, d, generator=g).bfloat16().to(dev)
+    parts = pk.partitions(torch.device(dev), hkv, "bf16")
+    workspace = torch.empty(pk.workspace_floats(step_tokens, hq, parts, d), dtype=torch.float32, device=dev)
+    out_g = torch.zeros(layers, step_tokens, hq, d, dtype=torch.bfloat16, device=dev)
+    out_e = torch.zeros_like(out_g)
+
+    def device_step():
+        k, v = pools["graph"]
+        pk.step_buffers(buffers, tables_d, capacity_d, lengths, slot, page, width, counts=counts)
+        # (tokens past the step's are appended nowhere: their slots are set below zero once, outside the capture)
+        for layer in range(layers):
+            pk.write(keys[layer], values[layer], buffers.d_slots, k[layer], v[layer], "bf16")
+            pk.attend(q[layer], k[layer], v[layer], "bf16", buffers.d_tables, buffers.d_rows, buffers.d_starts, buffers.d_firsts,
+                      width, page, counts=buffers.d_counts, offsets=buffers.d_offsets, tokens=step_tokens, out=out_g[layer],
+                      workspace=workspace)
+        torch.add(buffers.d_firsts, buffers.d_counts, out=frontier)
+        pk.commit_round(lengths, start, emitted, frontier[:B])      # (round slot r is row r: see below)
+
+    def host_step(at):
+        k, v = pools["eager"]
+        rows = [(int(s), at[int(s)], int(c)) for s, c in zip(slot.tolist(), counts.tolist())]
+        slots, d_starts, d_counts, d_firsts, d_offsets, d_tables = oracle_pool.step_buffers(lists, rows, page, dump, width, table_pages)
+        i32 = dict(dtype=torch.int32, device=dev)
+        slots_t = torch.tensor(slots + [-1] * (step_tokens - T), device=dev)
+        for layer in range(layers):
+            pk.write(keys[layer], values[layer], slots_t, k[layer], v[layer], "bf16")
+            pk.attend(q[layer], k[layer], v[layer], "bf16", torch.tensor(d_tables, **i32), torch.arange(B, **i32),
+                      torch.tensor(d_starts, **i32), torch.tensor(d_firsts, device=dev), width, page,
+                      counts=torch.tensor(d_counts, **i32), offsets=torch.tensor(d_offsets, **i32), tokens=step_tokens,
+                      out=out_e[layer], workspace=workspace)
+        return slots
+    # The commit writes round row r's length: with the rows in round-slot order the frontier of row r is slot r's. Here the
+    # rows are a permutation of the slots, so the lengths are committed through the same permutation on the host side of
+    # the comparison: round_lengths[r] = frontier[r] for r < B.
+    buffers.d_slots.fill_(-1)
+    device_step()      # (the first launches on a device look addresses up: outside the capture)
+    torch.cuda.synchronize()
+    pools["graph"] = fresh_pool()
+    lengths.copy_(torch.tensor(host_lengths))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        device_step()
+    pools["graph"][0].copy_(pools["eager"][0]), pools["graph"][1].copy_(pools["eager"][1])
+    lengths.copy_(torch.tensor(host_lengths))
+    for n in range(5):
+        at = lengths.tolist()
+        graph.replay()
+        torch.cuda.synchronize()
+        slots = host_step(at)
+        torch.cuda.synchronize()
+        assert buffers.d_slots[:T].tolist() == slots and buffers.totals.tolist() == [T, B, T, 0], n
+        assert torch.equal(out_g[:, :T], out_e[:, :T]), n
+        assert torch.equal(pools["graph"][0], pools["eager"][0]) and torch.equal(pools["graph"][1], pools["eager"][1]), n
+        want = [at[int(s)] + int(c) for s, c in zip(slot.tolist(), counts.tolist())]      # row r's frontier
+        assert lengths[:B].tolist() == want, n
+        # (the next step reads the lengths by slot: any values below the capacity do, the comparison builds from the same)

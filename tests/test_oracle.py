@@ -598,6 +598,51 @@ def test_copy_pages_copies_whole_pages_in_every_layer_and_store():
         assert torch.equal(paged[:, rest], old[:, rest])
 
 
+def test_a_rounds_lengths_follow_the_references_known_answers():
+    from oracle import pool
+    # tests/test_rounds.py:66-72: bound at 20, a round emits 3 up to frontier 23
+    lengths, start, moved = torch.tensor([20, 0]), torch.tensor([20, 0]), torch.tensor([1, 1])
+    pool.commit_round(lengths, start, torch.tensor([3]), torch.tensor([23]))
+    assert lengths.tolist() == [23, 0]
+    # tests/test_rounds.py:113-133: b held (it emitted nothing) keeps what the round found, its frontier stale or not; a
+    # truncation commits again from the round's start; a keep between rounds stands
+    lengths, start, moved = torch.tensor([20, 30, 7]), torch.tensor([-1, -1, -1]), torch.tensor([1, 1, 1])
+    pool.start_round(lengths, start, moved, 2)
+    assert start.tolist() == [20, 30, -1] and moved.tolist() == [0, 0, 1]
+    pool.commit_round(lengths, start, torch.tensor([3, 0]), torch.tensor([23, 30]))
+    assert lengths.tolist() == [23, 30, 7]
+    pool.commit_round(lengths, start, torch.tensor([2, 0]), torch.tensor([22, 30]))
+    assert lengths.tolist() == [22, 30, 7]
+    lengths[1] = 27                                            # keep("b", 27) on the host
+    pool.start_round(lengths, start, moved, 2)
+    pool.commit_round(lengths, start, torch.tensor([2, 0]), torch.tensor([24, 31]))
+    assert lengths.tolist() == [24, 27, 7]
+
+
+def test_a_steps_buffers_are_the_ones_worked_out_by_hand():
+    from oracle import pool
+    page, dump, window, table_pages = 4, 9, 3, 5
+    tables = {"a": [6, 2, 5], "b": [1], "c": [7, 0, 3, 8]}
+    rows = [("a", 9, 2), ("c", 3, 5), ("b", 2, 1), ("a", 4, 3)]      # (sequence, first position, count); c is a prompt row
+    starts, positions, row_of = pool.step_batch(rows)
+    assert starts == [0, 2, 7, 8, 11]
+    assert positions == [9, 10, 3, 4, 5, 6, 7, 2, 4, 5, 6]
+    assert row_of == [0, 0, 1, 1, 1, 1, 1, 2, 3, 3, 3]
+    slots, d_starts, d_counts, d_firsts, d_offsets, d_tables = pool.step_buffers(tables, rows, page, dump, window, table_pages)
+    #            a@9  a@10  c@3   c@4  c@5  c@6  c@7  b@2  a@4  a@5  a@6
+    assert slots == [21, 22, 31, 0, 1, 2, 3, 6, 8, 9, 10]
+    assert (d_starts, d_counts, d_firsts, d_offsets) == ([0, 7, 8], [2, 1, 3], [9, 2, 4], [0, 2, 3])
+    assert d_tables == [[6, 2, 5, 9, 9], [1, 9, 9, 9, 9], [6, 2, 5, 9, 9]]
+    # the same slots through the round tables' closed form, where the sequences are bound to round slots
+    round_tables = torch.tensor([t + [dump] * (table_pages - len(t)) for t in tables.values()], dtype=torch.int32)
+    capacity = torch.tensor([len(t) * page for t in tables.values()])
+    slot_of = {"a": 0, "b": 1, "c": 2}
+    at = pool.slots_at(round_tables, capacity, torch.tensor([slot_of[rows[r][0]] for r in row_of]), torch.tensor(positions), page, dump)
+    assert at.tolist() == slots
+    # offsets are the window rows' running token count, starts every row's
+    assert d_offsets == [sum(d_counts[:i]) for i in range(len(d_counts))]
+
+
 # -- rows read back ------------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("kind", ["bf16", "fp16", "fp8", "fp8:row", "int8"])
 def test_rows_read_back_are_the_codes_times_their_scale_one_fp32_product(kind):
