@@ -12,6 +12,7 @@ import torch
 
 from oracle import append as oracle_append
 from oracle import attend as oracle_attend
+from tests import harness
 from tests.support import kernels
 
 pytestmark = pytest.mark.gpu
@@ -29,7 +30,7 @@ class Pool:
         g = torch.Generator(device=dev).manual_seed(seed)
         held = [math.ceil((n + room) / PAGE) for n in lengths]
         self.width = (max(held) + 15) // 16 * 16
-        self.pages = int(sum(held) * 1.25) + 1
+        self.pages, self.held = int(sum(held) * 1.25) + 1, held
         order = torch.randperm(self.pages, device=dev, generator=g).to(torch.int32)
         self.tables = torch.full((len(lengths), self.width), self.pages, dtype=torch.int32, device=dev)      # (the dump page)
         at = 0
@@ -61,6 +62,12 @@ class Pool:
         for s, n in enumerate(lengths):
             keys, values = rows_of(s, n)
             self.pk.write(keys, values, self.slots(s, 0, n), self.k, self.v, kind, multipliers=self.mult)
+
+    def view(self, window=16):
+        """The pool as crit's attention plugin reads it: each sequence's page ids on the host, the dump page, the window."""
+        host = self.tables.cpu()
+        tables = {s: host[s, :w].tolist() for s, w in enumerate(self.held)}
+        return harness.PoolView(self.kind, PAGE, self.pages, window, tables, (self.k, self.v), self.mult, dev)
 
     def slots(self, s, start, n):
         p = torch.arange(start, start + n, device=dev)
@@ -139,7 +146,16 @@ def test_a_decode_step_of_the_8b_shape_at_its_batch_and_lengths(kind, B, low, hi
         assert torch.equal(got.view(torch.uint8), want.view(torch.uint8)), "appended bytes"
     q = torch.randn(B, hq, D, device=dev, generator=g).bfloat16()
     firsts = torch.tensor(lengths, dtype=torch.int64, device=dev)
-    out, lse = decode_all(pool, q, firsts)
+    # the launch crit's plugin makes of this step: a StepBatch of one token a sequence, every row a window row, tables cut
+    # at the rows' pages in widths of sixteen, partials packed by the tokens
+    batch = harness.StepBatch.build([(s, n, 1) for s, n in enumerate(lengths)], dev)
+    out, lse = harness.forward(pk, q, pool.view(), batch, lse=True)
+    assert harness.forward.launched == {"attend": 1, "prefill": 0}
+    # the same rows over the pool's whole tables, laid out by columns, and in three launches where the partials run out
+    plain, plain_lse = decode_all(pool, q, firsts)
+    assert torch.equal(out, plain) and torch.equal(lse, plain_lse)
+    cut, cut_lse = harness.forward(pk, q, pool.view(), batch, lse=True, partial_rows=B // 3 + 1)
+    assert harness.forward.launched == {"attend": 3, "prefill": 0} and torch.equal(out, cut) and torch.equal(lse, cut_lse)
     scale = D ** -0.5
     for s, n in enumerate(lengths):
         k, v = pool.stored(s, n + 1)
@@ -189,14 +205,20 @@ def test_prompt_chunks_on_prefixes_mixed_with_decode_rows():
     g = torch.Generator(device=dev).manual_seed(14)
     tokens = 8 * T + 56
     q = torch.randn(tokens, hq, D, device=dev, generator=g).bfloat16()
-    out = torch.empty(tokens, hq, D, dtype=torch.bfloat16, device=dev)
-    lse = torch.empty(tokens, hq, device=dev)
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    # the step as crit's plugin launches it: the rows of up to the pool's window (the decode rows) in one attend(), each
+    # prompt row through prefill() over its sequence's own table
+    batch = harness.StepBatch.build([(c, p, T) for c, p in enumerate(prefixes)] + [(8 + r, n, 1) for r, n in enumerate(decodes)], dev)
+    out, lse = harness.forward(pk, q, pool.view(), batch, lse=True)
+    assert harness.forward.launched == {"attend": 1, "prefill": 8}
+    # every chunk in one launch (prefill_rows) and the decode rows over the pool's whole tables give the same bits
+    once, once_lse = torch.empty_like(out), torch.empty_like(lse)
     pk.prefill_rows(q, pool.k, pool.v, "bf16", pool.tables, i32(list(range(8))), i32([c * T for c in range(8)]),
-                    i32([T] * 8), torch.tensor(prefixes, dtype=torch.int64, device=dev), T, PAGE, out=out, lse=lse)
+                    i32([T] * 8), torch.tensor(prefixes, dtype=torch.int64, device=dev), T, PAGE, out=once, lse=once_lse)
     rows = i32(list(range(8, 64)))
     pk.attend(q, pool.k, pool.v, "bf16", pool.tables, rows, i32([8 * T + r for r in range(56)]),
-              torch.tensor(decodes, dtype=torch.int64, device=dev), 1, PAGE, out=out, lse=lse)
+              torch.tensor(decodes, dtype=torch.int64, device=dev), 1, PAGE, out=once, lse=once_lse)
+    assert torch.equal(out, once) and torch.equal(lse, once_lse)
     scale = D ** -0.5
     for c, p in enumerate(prefixes):
         k, v = pool.stored(c, p + T)
