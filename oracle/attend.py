@@ -206,6 +206,66 @@ def windows_dense(q, keys, values, position, scale, sliding=0, sinks=None):
     return out, lse
 
 
+# -- the torch fallback over page tables (device_attention.py:1204-1288) ------------------------------------------------
+CHUNK = 1024      # positions a pass (device_attention.py:53)
+
+
+def windows_online(q, key_pages, value_pages, kind, tables, rows, starts, counts, firsts, columns, page, scale,
+                   key_scales=None, value_scales=None, multipliers=(1.0, 1.0), extent=None, sliding=0, sinks=None,
+                   chunk=CHUNK):
+    """Window rows in FP32 as the reference's fallback computes them (windows_torch, device_attention.py:1204-1288,
+    without trees, block lists and fresh rows): row by row and column by column, a masked online softmax over passes of
+    `chunk` positions of the row's page table (a position past the table's last page reads that page's) up to `extent`
+    (None: every position the tables hold), the rows read back dequantised to FP32 (rows_at); a sink logit folded in
+    after the passes. q [tokens][HQ][D]; tables [S][width] int32; rows, starts, counts (None: `columns` each), firsts one
+    a row. Returns (out [tokens][HQ][DV] FP32, lse [tokens][HQ] FP32), rows no window holds left zero / -inf."""
+    tokens, hq, d = q.shape
+    hkv, dv = key_pages.shape[-2], value_pages.shape[-1]
+    g = hq // hkv
+    width = tables.shape[1]
+    limit = width * page
+    extent = limit if extent is None else extent
+    extent = max(chunk, math.ceil(min(extent, limit) / chunk) * chunk)
+    out = torch.zeros(tokens, hq, dv)
+    found = torch.full((tokens, hq), float("-inf"))
+    for r in range(len(rows)):
+        table = tables[int(rows[r])]
+        count = min(int(counts[r]), columns) if counts is not None else columns
+        first = int(firsts[r])
+        for c in range(count):
+            qq = q[int(starts[r]) + c].float().view(hkv, g, d)
+            m = torch.full((hkv, g), float("-inf"))
+            l = torch.zeros(hkv, g)
+            acc = torch.zeros(hkv, g, dv)
+            for s0 in range(0, extent, chunk):
+                n = torch.arange(s0, s0 + chunk)
+                entry = table[(n // page).clamp(max=width - 1)]
+                keys, values = rows_at(key_pages, value_pages, entry.long() * page + n % page, kind, key_scales,
+                                       value_scales, multipliers)
+                seen = n <= first + c
+                if sliding:
+                    seen = seen & (n > first + c - sliding)
+                s = torch.einsum("kgd,nkd->kgn", qq, keys) * scale
+                s = s.masked_fill(~seen[None, None, :], float("-inf"))
+                top = torch.maximum(m, s.amax(-1))
+                sub = torch.where(top == float("-inf"), 0.0, top)
+                p = torch.exp(s - sub[..., None])
+                alpha = torch.exp(m - sub)
+                l = l * alpha + p.sum(-1)
+                acc = acc * alpha[..., None] + torch.einsum("kgn,nkd->kgd", p, values)
+                m = top
+            if sinks is not None:      # _sink_fold (device_attention.py:1291-1298): one more position with no value
+                sink = sinks.float().view(hkv, g)
+                top = torch.maximum(m, sink)
+                sub = torch.where(top == float("-inf"), 0.0, top)
+                keep = torch.exp(m - sub)
+                m, l, acc = top, l * keep + torch.exp(sink - sub), acc * keep[..., None]
+            t = int(starts[r]) + c
+            out[t] = torch.where(l[..., None] > 0, acc / l.clamp(min=1e-30)[..., None], 0.0).view(hq, dv)
+            found[t] = torch.where(l > 0, m + torch.log(l.clamp(min=1e-30)), float("-inf")).view(hq)
+    return out, found
+
+
 # -- online softmax steps (kernels/core/python/crit_kcore/attention_softmax.py:37-101), natural base --------------------
 def step(s, m):
     """One block of scores s [rows][positions] (masked ones -inf) against running maxima m [rows] -> (p, alpha,

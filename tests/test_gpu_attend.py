@@ -699,3 +699,27 @@ def test_a_round_hands_its_slots_over_as_int64_rows(kind):
             assert torch.equal(got, want)
         ref, _ = cache.want(q[cols:2 * cols], 0, 640, cols)
         _close(got[cols:2 * cols], ref)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("sliding,sinks", [(0, False), (40, False), (0, True)])
+def test_window_rows_equal_the_references_torch_fallback_over_the_same_tables(kind, sliding, sinks):
+    # The reader against the arithmetic the reference tests its own reader with: windows_torch's FP32 online softmax in
+    # passes of 1,024 positions over the page tables (device_attention.py:1204-1288; oracle.attend.windows_online), the
+    # same Windows metadata into both.
+    from oracle import attend as oracle_attend
+    hq, hkv, d, page = 8, 2, 128, 16
+    cache = Cache(kind, hkv, d, d, page, [1100, 64, 2300])
+    rows, starts, counts, firsts = [2, 0, 1], [0, 4, 6], [4, 2, 1], [2290, 1098, 63]
+    q = rand_q(7, hq, d, 5)
+    q_dtype = torch.float16 if kind == "fp16" else torch.bfloat16
+    sink = torch.tensor([0.5, -1.0, float("-inf"), 2.0, 0.0, 1.5, -3.0, 0.25]) if sinks else None
+    lse = torch.empty(7, hq, device=dev)
+    out = cache.attend(q, rows, starts, firsts, 4, lse=lse, counts=torch.tensor(counts, dtype=torch.int32, device=dev),
+                       sliding=sliding, sinks=None if sink is None else sink.to(dev))
+    k, v, ks, vs, tables = cache.cpu()
+    want, want_lse = oracle_attend.windows_online(q.to(q_dtype).float().cpu(), k, v, kind, tables, rows, starts, counts, firsts, 4,
+                                                  page, d ** -0.5, ks, vs, cache.multipliers, extent=2300, sliding=sliding,
+                                                  sinks=sink)
+    _close(out, want.double(), (kind, sliding, sinks))
+    _close_lse(lse, want_lse.double(), (kind, sliding, sinks))

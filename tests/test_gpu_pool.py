@@ -435,3 +435,64 @@ def test_a_whole_step_buffers_append_attention_commit_replays_from_one_graph():
         want = [at[int(s)] + int(c) for s, c in zip(slot.tolist(), counts.tolist())]      # row r's frontier
         assert lengths[:B].tolist() == want, n
         # (the next step reads the lengths by slot: any values below the capacity do, the comparison builds from the same)
+
+
+def test_the_transactional_state_is_a_sequences_length_on_the_device():
+    # KVState (inference/attention-state/code/implementation.py:5-50; oracle.state) beside the device pool: staged rows are
+    # appended past the sequence's valid length, a commit of n moves the length by n (the rest is dropped: the next rows
+    # overwrite it), a rollback leaves it; attend() over the committed rows, or with the pending ones, is one decode row.
+    from oracle.state import KVState
+    pk = kernels()
+    page, width, hd = 16, 4, 16
+    tables, capacity, dump, _ = _bound(page, width, [(0, 64)], 1, seed=40)
+    tables_d, capacity_d = tables.to(dev), capacity.to(dev)
+    k = torch.zeros(dump + 1, page, 1, hd, dtype=torch.bfloat16, device=dev)
+    v = torch.zeros_like(k)
+    lengths, start = torch.zeros(1, dtype=torch.int64, device=dev), torch.zeros(1, dtype=torch.int64, device=dev)
+    state = KVState(64, hd, hd)
+    g = torch.Generator().manual_seed(41)
+    slot0 = torch.zeros(1, dtype=torch.int64, device=dev)
+    pending = 0
+
+    def stage(n):
+        nonlocal pending
+        keys, values = torch.randn(n, 1, hd, generator=g).bfloat16(), torch.randn(n, 1, hd, generator=g).bfloat16()
+        for key, value in zip(keys[:, 0].float().tolist(), values[:, 0].float().tolist()):
+            state.stage(key, value)
+        at = int(lengths[0]) + pending + torch.arange(n, device=dev)
+        slots = pk.slots_at(tables_d, capacity_d, slot0.expand(n).contiguous(), at, page, dump)
+        pk.write(keys.to(dev), values.to(dev), slots, k, v, "bf16")
+        pending += n
+
+    def commit(n):
+        nonlocal pending
+        state.commit(n)
+        pk.start_round(lengths, start, None, 1)
+        frontier = lengths + n
+        pk.commit_round(lengths, start, torch.tensor([n], device=dev), frontier)
+        pending = 0
+
+    def check(include_pending):
+        q = torch.randn(1, 1, hd, generator=g).bfloat16()
+        want = state.attend(q[0, 0].float().tolist(), include_pending=include_pending)
+        rows = int(lengths[0]) + (pending if include_pending else 0)
+        got = pk.attend(q.to(dev), k, v, "bf16", tables_d, torch.zeros(1, dtype=torch.int32, device=dev),
+                        torch.zeros(1, dtype=torch.int32, device=dev), torch.tensor([rows - 1], device=dev), 1, page)
+        torch.testing.assert_close(got[0, 0].double().cpu(), torch.tensor(want, dtype=torch.float64), atol=2e-2, rtol=2e-2)
+    stage(5)
+    check(True)
+    commit(3)                      # two speculative rows rejected
+    assert int(lengths[0]) == len(state.committed) == 3
+    check(False)
+    stage(4)
+    check(True)
+    check(False)                   # the committed prefix alone, the staged rows lying past it
+    state.rollback()
+    pending = 0                    # (nothing to do on the device: the length did not move)
+    check(False)
+    stage(20)
+    commit(20)
+    assert int(lengths[0]) == len(state.committed) == 23
+    check(False)
+    commit(0)                      # a held row: the length stays
+    assert int(lengths[0]) == 23

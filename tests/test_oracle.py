@@ -277,6 +277,78 @@ def test_the_sdpa_cpu_path_and_the_dense_window_agree_with_float64_over_the_stor
         assert torch.allclose(dense_lse.double(), want_lse, atol=1e-4, rtol=1e-5)
 
 
+@pytest.mark.parametrize("kind", ["bf16", "fp8:row"])
+def test_the_online_fallback_over_page_tables_is_float64_attention_whatever_its_passes(kind):
+    # windows_online (the reference's windows_torch) against float64 attention over the stored values: a row whose
+    # positions span three passes, verify windows, a sliding window, sinks; passes of another size agree to FP32
+    # rounding, and passes past a column's positions leave its sums bit for bit as they were.
+    hq, hkv, d, page = 4, 2, 32, 16
+    lengths = [40, 700, 333]
+    k, v, ks, vs, tables, _ = _pool(kind, hkv, d, d, page, lengths)
+    g = torch.Generator().manual_seed(13)
+    q = torch.randn(8, hq, d, generator=g).bfloat16().float()
+    rows, starts, counts, firsts = [2, 0, 1], [0, 3, 5], [3, 1, 2], [330, 39, 698]
+    scale = d ** -0.5
+    sinks = torch.tensor([0.5, -1.0, float("-inf"), 2.0])
+    for sliding, sink in ((0, None), (24, None), (0, sinks)):
+        out, lse = attend.windows_online(q, k, v, kind, tables, rows, starts, counts, firsts, 4, page, scale, ks, vs,
+                                         sliding=sliding, sinks=sink, chunk=256)
+        for r in range(3):
+            span = slice(starts[r], starts[r] + counts[r])
+            want, want_lse = attend.window_reference(q[span], k, v, kind, tables[rows[r]], firsts[r], counts[r], page, scale,
+                                                     ks, vs, sliding=sliding)
+            if sink is not None:      # a sink is one more position with no value: out shrinks by e^lse / (e^lse + e^sink)
+                total = torch.logaddexp(want_lse, sink.double()[None, :])
+                want, want_lse = want * torch.exp(want_lse - total)[..., None], total
+            torch.testing.assert_close(out[span].double(), want, atol=2e-5, rtol=1e-4)
+            torch.testing.assert_close(lse[span].double(), want_lse, atol=2e-5, rtol=1e-5)
+        assert out[7].eq(0).all() and lse[7].eq(float("-inf")).all()      # a token no window holds
+        other, other_lse = attend.windows_online(q, k, v, kind, tables, rows, starts, counts, firsts, 4, page, scale, ks, vs,
+                                                 sliding=sliding, sinks=sink, chunk=64)
+        torch.testing.assert_close(other, out, atol=2e-5, rtol=1e-4)
+        short, short_lse = attend.windows_online(q, k, v, kind, tables, rows[1:2], starts[1:2], counts[1:2], firsts[1:2], 4,
+                                                 page, scale, ks, vs, sliding=sliding, sinks=sink, chunk=64, extent=40)
+        assert torch.equal(short[3], other[3]) and torch.equal(short_lse[3], other_lse[3])
+
+
+def test_the_transactional_state_follows_the_references_known_answers():
+    from oracle.state import KVState
+    state = KVState(capacity=3, key_width=2, value_width=1)      # README.md:224-238, test_techniques.py:471-482
+    state.stage((1.0, 0.0), (2.0,))
+    state.stage((0.0, 1.0), (10.0,))
+    assert state.attend((0.0, 0.0), include_pending=True) == (6.0,)
+    state.commit(1)
+    assert state.attend((0.0, 0.0)) == (2.0,) and state.pending == []
+    state.stage((1.0, 1.0), (99.0,))
+    state.rollback()
+    assert len(state.committed) == 1 and state.attend((0.0, 0.0)) == (2.0,)
+    one = KVState(1, 1, 1)                                         # test_techniques.py:484-494
+    with pytest.raises(ValueError):
+        one.attend((1,))
+    one.stage((1,), (2,))
+    with pytest.raises(ValueError):
+        one.stage((2,), (3,))
+    with pytest.raises(ValueError):
+        one.commit(2)
+    assert len(one.pending) == 1
+    for bad in ((0, 1, 1), (1, 1.0, 1)):
+        with pytest.raises(ValueError):
+            KVState(*bad)
+    with pytest.raises(ValueError):
+        one.stage((float("nan"),), (1,))
+    # its softmax is float64 attention over the rows it holds
+    g = torch.Generator().manual_seed(17)
+    keys, values = torch.randn(9, 4, generator=g, dtype=torch.float64), torch.randn(9, 3, generator=g, dtype=torch.float64)
+    query = torch.randn(4, generator=g, dtype=torch.float64)
+    state = KVState(16, 4, 3)
+    for key, value in zip(keys.tolist(), values.tolist()):
+        state.stage(key, value)
+    state.commit(6)
+    want, _ = attend.reference(query[None], keys[:6, None], values[:6, None], torch.ones(6, dtype=torch.bool), 0.5)
+    torch.testing.assert_close(torch.tensor(state.attend(query.tolist()), dtype=torch.float64), want[0], atol=1e-12, rtol=1e-12)
+    assert state.pending == [] and len(state.committed) == 6      # the rejected suffix is gone
+
+
 def test_a_sliding_window_sees_only_its_last_positions():
     k, v, ks, vs, tables, _ = _pool("bf16", 1, 16, 16, 16, [100])
     q = torch.randn(2, 2, 16, generator=torch.Generator().manual_seed(4))
