@@ -232,10 +232,11 @@ int compute_units() {
 }
 
 int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
-    if (!p || !p->q || !p->key_pages || !p->value_pages || !p->tables || !p->rows || !p->starts || !p->firsts || !p->out)
-        return CRIT_PKV_E_NULL;
+    if (!p || !p->q || !p->value_pages || !p->tables || !p->rows || !p->starts || !p->firsts || !p->out) return CRIT_PKV_E_NULL;
+    const bool derive = p->derive_table != nullptr;      // keys derived from the value rows: no key pages, no key scales
+    if (!derive && !p->key_pages) return CRIT_PKV_E_NULL;
     if (p->kind < 0 || p->kind > 3) return CRIT_PKV_E_DTYPE;
-    if (p->kind >= 2 && (!p->key_scales || !p->value_scales)) return CRIT_PKV_E_NULL;
+    if (p->kind >= 2 && ((!derive && !p->key_scales) || !p->value_scales)) return CRIT_PKV_E_NULL;
     const bool f16 = p->page_dtype == CRIT_PKV_F16;
     if (f16 && p->kind != 0) return CRIT_PKV_E_DTYPE;
     if (p->out_dtype != CRIT_PKV_F32 && p->out_dtype != CRIT_PKV_BF16 && p->out_dtype != CRIT_PKV_F16) return CRIT_PKV_E_DTYPE;
@@ -247,6 +248,12 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     if (p->q_stride_t % 8 || p->q_stride_h % 8 || (reinterpret_cast<uintptr_t>(p->q) % 16) ||
         (reinterpret_cast<uintptr_t>(p->key_pages) % 16) || (reinterpret_cast<uintptr_t>(p->value_pages) % 16))
         return CRIT_PKV_E_GEOMETRY;
+    if (derive) {      // one row is key and value: one width (64 or 128), halves of the rotation in whole lanes
+        if (p->head_dim != p->value_dim || (p->head_dim != 64 && p->head_dim != 128) || p->derive_rot < 16 ||
+            p->derive_rot % 16 || p->derive_rot > p->head_dim || !(p->derive_eps >= 0.0f) || p->blocks || p->fresh_keys ||
+            p->fresh_values)
+            return CRIT_PKV_E_GEOMETRY;
+    }
     const int lpr = (p->head_dim > p->value_dim ? p->head_dim : p->value_dim) / 8;      // lanes that hold the wider row
     const bool wide128 = p->head_dim == 128 && p->value_dim == 128;
     const int sp = 4 * (64 / lpr);
@@ -284,6 +291,8 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     a.f_shifts = p->fresh_shifts, a.f_firsts = p->fresh_firsts;
     a.f_stride_k = p->fresh_stride_k, a.f_stride_v = p->fresh_stride_v, a.f_rows = p->fresh_rows;
     a.f_per_row = p->fresh_per_row ? 1 : 0;
+    a.derive_table = p->derive_table, a.derive_eps = p->derive_eps, a.derive_rot = p->derive_rot;
+    a.derive_weighted = p->derive_weighted ? 1 : 0;
     a.listed_keys = p->blocks ? p->blocks_k * p->block_size : 0;
     a.block_div = make_div32(p->blocks ? (uint32_t)p->block_size : 1u);
     a.q_st = p->q_stride_t, a.q_sh = p->q_stride_h, a.o_st = p->out_stride_t, a.o_sh = p->out_stride_h, a.tab_stride = p->table_stride;
@@ -314,7 +323,7 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     // The bandwidth kernel walks pages that are powers of two from 16 positions up, in positions below 2^31; other
     // multiples of 16 take the generic kernel. (block lists of blocks that are a multiple of 16: their own variant)
     const bool pow2_page = a.page_shift >= 4 && (int64_t)p->partitions * p->piece <= 0x3fffffff;
-    a.fast128 = wide128 && ((page16 && pow2_page) || fast_lists);
+    a.fast128 = wide128 && !derive && ((page16 && pow2_page) || fast_lists);      // (derived keys: the generic kernel)
     if (a.fast128 && p->kv_heads % 2 == 0) a.heads_per_wave = 2;
     // Query rows a tile holds: the generic and block-list kernels' tile height; 16 a wavefront's heads share in the
     // bandwidth kernel (matrix tiles of 16 columns).

@@ -51,6 +51,11 @@ struct AttendArgs {
     const int64_t* f_firsts;
     int64_t f_stride_k, f_stride_v, f_rows;
     int f_per_row;
+    // Derived keys: the inverse frequencies [derive_rot / 2], then the norm's weight [dk] when derive_weighted; null:
+    // keys from their pages.
+    const float* derive_table;
+    float derive_eps;
+    int derive_rot, derive_weighted;
 };
 
 // A workgroup barrier that orders the shared arrays only: a wavefront waits for its own LDS traffic, then for the

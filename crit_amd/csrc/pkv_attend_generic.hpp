@@ -42,10 +42,18 @@ struct StepBuf {
 // the row's shift), unscaled: a score times the softmax scale only, a probability times 1 (_kernels.py:272-274, 291-345).
 // A lane holds the same 8 elements of a row either way (16 bytes of a fresh row, 8 or 16 of a page's), so both rows are
 // loaded for every position and the position picks one.
-template <int KIND, bool F16, int LPR, int QR, bool FUSED, bool SPARSE = false, bool FRESH = false>
+//
+// DERIVE: the pool holds value rows only and a position's key is derived from its value row on read
+// (paged_kv_attention/__init__.py:52-58 of the reference): k = rope(rms_norm(r) * weight, position), r the row as stored
+// (codes times their scale or multiplier), rms_norm(r) = r / sqrt(mean(r * r) + eps), the "half" rotation over the
+// first rotary_dim values (value i with value i + rotary_dim / 2) at the angle fp32(position) * freqs[i], all in FP32;
+// the scores are FP32 products of the queries with these keys (the reference multiplies the FP32 key as two parts in
+// the queries' type: the same value to about 2^-16). rotary_dim is a multiple of 16, so a half is whole lanes.
+template <int KIND, bool F16, int LPR, int QR, bool FUSED, bool SPARSE = false, bool FRESH = false, bool DERIVE = false>
 __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
     static_assert(!(SPARSE && FUSED), "block lists are read by the split launch");
     static_assert(!(SPARSE && FRESH), "block lists read the pages only");
+    static_assert(!(DERIVE && (SPARSE || FRESH)), "derived keys: windows over the pages, without block lists or fresh rows");
     constexpr int D = LPR * 8;         // the wider of the key and value rows
     constexpr int PPI = 64 / LPR;      // positions one load instruction of a wavefront covers
     constexpr int SP = 4 * PPI;        // positions a wavefront's step covers
@@ -120,7 +128,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
     for (int rr = 0; rr < QR; ++rr) anc[rr] = (tree && live[rr]) ? ancestors(a, start, col[rr]) : 0ull;
     // The lane's slice of each query row: packed 16-bit pairs for 16-bit pages, FP32 for 8-bit pages.
     uint32_t qp[QR][4];
-    float qf[KIND == 0 ? 1 : QR][8];
+    float qf[(KIND == 0 && !DERIVE) ? 1 : QR][8];
 #pragma unroll
     for (int rr = 0; rr < QR; ++rr) {
         uint4 w = make_uint4(0, 0, 0, 0);
@@ -128,7 +136,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
             w = *reinterpret_cast<const uint4*>(a.q + ((int64_t)(start + col[rr]) * a.q_st + (int64_t)qhead[rr] * a.q_sh + li * 8) * 2);
         }
         qp[rr][0] = w.x, qp[rr][1] = w.y, qp[rr][2] = w.z, qp[rr][3] = w.w;
-        if constexpr (KIND != 0) {
+        if constexpr (KIND != 0 || DERIVE) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 qf[rr][2 * j] = F16 ? f16_lo(qp[rr][j]) : bf16_lo(qp[rr][j]);
@@ -173,11 +181,11 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
             }
             const int in_page = a.page_shift >= 0 ? (n & (a.page - 1)) : (n % a.page);
             const int64_t slot = (int64_t)tab[k] * a.page + in_page;
-            buf.k[k] = *reinterpret_cast<const typename StepBuf<KIND>::Vec*>(kbase + slot * slot_bytes_k);
+            if constexpr (!DERIVE) buf.k[k] = *reinterpret_cast<const typename StepBuf<KIND>::Vec*>(kbase + slot * slot_bytes_k);
             if constexpr (KIND == 0) buf.v[k] = load_once16(vbase + slot * slot_bytes_v);
             else buf.v[k] = load_once8(vbase + slot * slot_bytes_v);
             if constexpr (KIND >= 2) {
-                buf.ks[k] = a.ks[slot * a.hkv + kvh];
+                if constexpr (!DERIVE) buf.ks[k] = a.ks[slot * a.hkv + kvh];
                 buf.vs[k] = a.vs[slot * a.hkv + kvh];
             }
             if constexpr (FRESH) {      // (unconditional too: a position below the first fresh one reads row 0 or its own clamped)
@@ -222,6 +230,55 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
             return base_of();
         };
 
+        // The lane's 8 values of position k's value row as the page holds them (codes, not yet times their scale).
+        auto stored_values = [&](const StepBuf<KIND, FRESH>& buf, int k, float (&vf)[8]) __attribute__((always_inline)) {
+            if constexpr (KIND == 0) {
+                const uint32_t vw[4] = {buf.v[k].x, buf.v[k].y, buf.v[k].z, buf.v[k].w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    vf[2 * j] = F16 ? f16_lo(vw[j]) : bf16_lo(vw[j]);
+                    vf[2 * j + 1] = F16 ? f16_hi(vw[j]) : bf16_hi(vw[j]);
+                }
+            } else if constexpr (KIND == 3) {
+                const uint32_t w2[2] = {buf.v[k].x, buf.v[k].y};
+#pragma unroll
+                for (int j = 0; j < 8; ++j) vf[j] = (float)(int8_t)(w2[j / 4] >> (8 * (j % 4)));
+            } else {
+                const f32x2 a0 = e4m3_pair<false>(buf.v[k].x), a1 = e4m3_pair<true>(buf.v[k].x);
+                const f32x2 a2 = e4m3_pair<false>(buf.v[k].y), a3 = e4m3_pair<true>(buf.v[k].y);
+                vf[0] = a0.x, vf[1] = a0.y, vf[2] = a1.x, vf[3] = a1.y;
+                vf[4] = a2.x, vf[5] = a2.y, vf[6] = a3.x, vf[7] = a3.y;
+            }
+        };
+        // DERIVE: position n's key from its value row.
+        auto derived_key = [&](const StepBuf<KIND, FRESH>& buf, int k, int n, float (&kf)[8]) __attribute__((always_inline)) {
+            stored_values(buf, k, kf);
+            const float rs = KIND >= 2 ? buf.vs[k] : (KIND == 1 ? v_mult : 1.0f);
+            float ss = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                kf[j] *= rs;
+                ss = __builtin_fmaf(kf[j], kf[j], ss);
+            }
+            ss = group_sum<LPR>(ss);
+            const float rn = 1.0f / __builtin_sqrtf(ss / (float)D + a.derive_eps);
+            const int half = a.derive_rot >> 4;      // lanes a half of the rotated values takes
+            const float* weight = a.derive_table + (a.derive_rot >> 1);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) kf[j] = kf[j] * rn * (a.derive_weighted ? weight[li * 8 + j] : 1.0f);
+            const bool low = li < half, turns = li < 2 * half;
+            const int from = turns ? (low ? lane + half : lane - half) : lane;
+            const int fi = (low ? li : li - half) * 8;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float other = __shfl(kf[j], from);
+                float sn, cs;
+                sincosf((float)n * a.derive_table[turns ? fi + j : 0], &sn, &cs);
+                const float turned = low ? kf[j] * cs - other * sn : kf[j] * cs + other * sn;
+                kf[j] = turns ? turned : kf[j];
+            }
+        };
+
         auto compute = [&](int base, const StepBuf<KIND, FRESH>& buf) __attribute__((always_inline)) {
             float s[4][QR];
             bool isf[4];      // FRESH: the position's row is a fresh one
@@ -231,7 +288,10 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
             for (int k = 0; k < 4; ++k) {
                 uint32_t kw[4];
                 float kf[8];
-                if constexpr (KIND == 0) {
+                if constexpr (DERIVE) {
+                    const int n = base + k * PPI + lg;
+                    derived_key(buf, k, n < n_keys ? n : n_keys - 1, kf);
+                } else if constexpr (KIND == 0) {
                     kw[0] = buf.k[k].x, kw[1] = buf.k[k].y, kw[2] = buf.k[k].z, kw[3] = buf.k[k].w;
                 } else if constexpr (KIND == 3) {
                     const uint32_t w2[2] = {buf.k[k].x, buf.k[k].y};
@@ -258,7 +318,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
 #pragma unroll
                 for (int rr = 0; rr < QR; ++rr) {
                     float d = 0.0f;
-                    if constexpr (KIND == 0) {
+                    if constexpr (KIND == 0 && !DERIVE) {
 #pragma unroll
                         for (int j = 0; j < 4; ++j) {
                             if constexpr (F16) {
@@ -281,7 +341,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const int n = SPARSE ? buf.pos[k] : base + k * PPI + lg;
-                    float x = s[k][rr] * (isf[k] ? a.sscale : (KIND >= 2 ? sscale * buf.ks[k] : sscale));
+                    float x = s[k][rr] * ((isf[k] || DERIVE) ? a.sscale : (KIND >= 2 ? sscale * buf.ks[k] : sscale));
                     bool vis = n <= lim[rr] && n < n_keys;
                     if constexpr (SPARSE) vis = vis && n >= 0;
                     if (tree) vis = vis && (n < first || ((anc[rr] >> ((n - first) & 63)) & 1ull) != 0);
@@ -312,23 +372,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 float vf[8];
-                if constexpr (KIND == 0) {
-                    const uint32_t vw[4] = {buf.v[k].x, buf.v[k].y, buf.v[k].z, buf.v[k].w};
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        vf[2 * j] = F16 ? f16_lo(vw[j]) : bf16_lo(vw[j]);
-                        vf[2 * j + 1] = F16 ? f16_hi(vw[j]) : bf16_hi(vw[j]);
-                    }
-                } else if constexpr (KIND == 3) {
-                    const uint32_t w2[2] = {buf.v[k].x, buf.v[k].y};
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) vf[j] = (float)(int8_t)(w2[j / 4] >> (8 * (j % 4)));
-                } else {
-                    const f32x2 a0 = e4m3_pair<false>(buf.v[k].x), a1 = e4m3_pair<true>(buf.v[k].x);
-                    const f32x2 a2 = e4m3_pair<false>(buf.v[k].y), a3 = e4m3_pair<true>(buf.v[k].y);
-                    vf[0] = a0.x, vf[1] = a0.y, vf[2] = a1.x, vf[3] = a1.y;
-                    vf[4] = a2.x, vf[5] = a2.y, vf[6] = a3.x, vf[7] = a3.y;
-                }
+                stored_values(buf, k, vf);
                 if constexpr (FRESH) {
                     const uint32_t fw[4] = {buf.f.v[k].x, buf.f.v[k].y, buf.f.v[k].z, buf.f.v[k].w};
 #pragma unroll

@@ -49,8 +49,10 @@ _DTYPE = {torch.float32: _abi.F32, torch.bfloat16: _abi.BF16, torch.float16: _ab
 
 
 class Derive(NamedTuple):
-    """Keys derived from the value rows on read (the reference's derive=). Not served by these kernels: attend() and
-    prefill() refuse it."""
+    """Keys derived from the value rows on read (attend's and prefill's derive=, reference __init__.py:82-121): weight
+    FP32 [dim] (or None: all ones), eps, freqs FP32 [rotary_dim / 2] inverse frequencies, rotary_dim. One made by
+    derive() holds its table (the freqs, then the weight) packed on the device, so a call allocates nothing; a plain
+    tuple of the four is packed at each call."""
     weight: object
     eps: float
     freqs: object
@@ -59,7 +61,36 @@ class Derive(NamedTuple):
 
 
 def derive(weight, eps, freqs, rotary_dim):
-    return Derive(weight, float(eps), freqs, int(rotary_dim))
+    """A Derive with its table packed once, for every call over the layer."""
+    return _derived(Derive(weight, eps, freqs, rotary_dim), None, None)[0]
+
+
+def _derived(given, d, device):
+    """`given` (a Derive or a tuple of its four fields) checked for heads of width d (None: not known yet) on `device`:
+    (the Derive with its packed table, whether it has a weight). The checks and their messages are the reference's
+    (__init__.py:99-121); past them these kernels take rotary widths in multiples of 16 over heads of 64 or 128."""
+    found = given if isinstance(given, Derive) else Derive(*given)
+    weight, eps, freqs, rot = found.weight, float(found.eps), found.freqs, int(found.rotary_dim)
+    if rot < 2 or rot % 2 or (d is not None and rot > d):
+        raise ValueError(f"derive's rotary_dim is even, 2 up to the head width {d}, not {rot}")
+    device = device if device is not None else (freqs.device if torch.is_tensor(freqs) else None)
+    if not torch.is_tensor(freqs) or freqs.dtype != torch.float32 or tuple(freqs.shape) != (rot // 2,) or freqs.device != device:
+        raise ValueError(f"derive's freqs are FP32 [{rot // 2}] (rotary_dim / 2 inverse frequencies) on q's device")
+    if weight is not None and (not torch.is_tensor(weight) or weight.dtype != torch.float32 or weight.dim() != 1 or
+                               (d is not None and weight.shape[0] != d) or weight.device != device):
+        raise ValueError(f"derive's weight is FP32 [{d}] (the head width) on q's device, or None")
+    if not eps >= 0:
+        raise ValueError("derive's eps is 0 or more")
+    table = found.table
+    if table is None:
+        if device is not None and device.type == "cuda" and torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("paged_kv_attention: a captured call takes a Derive made by derive() (its table packed)")
+        table = freqs.contiguous() if weight is None else torch.cat([freqs, weight.contiguous()])
+    elif table.numel() != rot // 2 + (0 if weight is None else weight.shape[0]):
+        raise ValueError("a Derive's packed table does not fit its freqs and weight")
+    if rot % 16 or (d is not None and d not in (64, 128)):
+        raise _unsupported(f"derive= with a rotary width of {rot} over heads of {d} (multiples of 16 over heads of 64 or 128 are)")
+    return found._replace(eps=eps, rotary_dim=rot, table=table), weight is not None
 
 
 def _unsupported(what):
@@ -476,12 +507,24 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
     each row's positions from `first` on are read from those rows instead of the pages (row = position - shift; a
     prompt chunk's own keys and values as the projections gave them, unscaled), shift and first int64 device tensors
     of one element a row, or of one element for every row; not with block lists; such launches take the generic
-    kernel, split or fused, the same bits either way. derive is not served. phases (a measurement's): 1 runs the split
+    kernel, split or fused, the same bits either way. derive: a Derive (or the tuple (weight, eps, freqs, rotary_dim)):
+    the keys derived from the value pages on read (key_pages None: the layer keeps value rows only), k = rope(rms_norm(r)
+    * weight, position) in FP32 from the row as stored; head widths 64 and 128, rotary widths in multiples of 16; not
+    with block lists, fresh rows or flash. phases (a measurement's): 1 runs the split
     launch only, 2 the merge only. static: the launch takes its partials and counters from the library's static device
     array (crit_pkv_attend_static: for callers that cannot allocate; the same bits; launches that overlap on one GPU
     race there; refused past _abi.STATIC_SCRATCH_BYTES of partials); no workspace is read."""
     if derive is not None:
-        raise _unsupported("derive= (keys derived from value rows)")
+        if flash:
+            raise ValueError("derive= reads keys from the value rows on the split and fused launches and prefill's "
+                             "default one: the flash structures (flash=True, flash='cuda') take key pages")
+        if blocks is not None:
+            raise ValueError("derive= reads windows without block lists")
+        if key_pages is not None:
+            raise ValueError("derive= reads the value pages as keys too: key_pages None")
+        if fresh is not None:
+            raise _unsupported("derive= with fresh rows")
+        key_pages = value_pages
     if parents is not None:
         _require_device(parents, "attend's parents")
         parents = parents.reshape(-1)
@@ -504,9 +547,12 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
         flash = False      # (block lists: the split launch, as in the reference)
     if fresh is not None and blocks is not None:
         raise ValueError("fresh rows are not read through block lists")
-    k_kind = _check_kind(kind, key_scales)
+    k_kind = _check_kind(kind, value_scales if derive is not None else key_scales)
     _require_device(q, "attend's q")
     T, hq, d = q.shape
+    derived, has_weight = (None, False) if derive is None else _derived(derive, d, q.device)
+    if derived is not None and d != value_pages.shape[-1]:
+        raise ValueError("derive= reads one row as key and value: one head width")
     _check_sinks(sinks, q)
     sliding = _check_sliding(sliding, blocks)
     hkv, dv = key_pages.shape[-2], value_pages.shape[-1]
@@ -560,6 +606,10 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
     p = _abi.AttendParams()
     p.q, p.key_pages, p.value_pages = q.data_ptr(), key_pages.data_ptr(), value_pages.data_ptr()
     p.key_scales, p.value_scales, p.head_multipliers = _ptr(key_scales), _ptr(value_scales), _ptr(per_head)
+    if derived is not None:
+        p.key_pages = p.key_scales = None
+        p.derive_table, p.derive_eps = derived.table.data_ptr(), derived.eps
+        p.derive_rot, p.derive_weighted = derived.rotary_dim, int(has_weight)
     p.tables, p.rows, p.starts, p.counts = tables.data_ptr(), rows.data_ptr(), starts.data_ptr(), _ptr(counts)
     p.rows_are_64 = int(rows.dtype == torch.int64)
     p.firsts, p.offsets = firsts.data_ptr(), _ptr(offsets)
@@ -720,8 +770,9 @@ def _prefill_launch(q, key_pages, value_pages, kind, tables, table_rows, starts,
 
 def _prefill_as_windows(q, key_pages, value_pages, kind, tables, table_rows, starts, counts, positions, max_count,
                         chunks, page, key_scales, value_scales, multipliers, scale, out, lse, sinks, sliding, fresh,
-                        int8_qk):
-    """Prompt chunks at the head widths the matrix-core kernel does not take (16, 32, 256): every chunk cut into window
+                        int8_qk, derive=None):
+    """Prompt chunks at the head widths the matrix-core kernel does not take (16, 32, 256), and those whose keys are
+    derived from the value rows: every chunk cut into window
     rows of up to MAX_COLUMNS tokens and read by attend()'s fused launch, as crit itself reads prompt rows with
     prompt_reader decode (device_attention.py:751-783). The rows' metadata is computed on the device from the chunks'
     (no length is read on the host)."""
@@ -753,7 +804,7 @@ def _prefill_as_windows(q, key_pages, value_pages, kind, tables, table_rows, sta
         out = torch.empty(q.shape[0], hq, value_pages.shape[-1], dtype=q.dtype, device=device)
     return attend(q, key_pages, value_pages, kind, tables, w_rows, w_starts, w_firsts, MAX_COLUMNS, page,
                   counts=w_counts, key_scales=key_scales, value_scales=value_scales, multipliers=multipliers,
-                  scale=scale, out=out, lse=lse, fused=True, fresh=given, sinks=sinks, sliding=sliding)
+                  scale=scale, out=out, lse=lse, fused=True, fresh=given, sinks=sinks, sliding=sliding, derive=derive)
 
 
 def prefill(q, key_pages, value_pages, kind, table, position, page, *, key_scales=None, value_scales=None,
@@ -770,9 +821,19 @@ def prefill(q, key_pages, value_pages, kind, table, position, page, *, key_scale
     grown outside a capture); a token's bits follow its own positions and `first`. int8_qk (INT8 pages): each query
     row rounded to INT8 codes at its own scale (amax / 127, half away from zero) and the scores taken as exact integer
     products of the codes on the matrix cores (v_mfma_i32_32x32x32_i8) times the row's and the keys' scales; fresh rows
-    are still read in q's type. derive is not served."""
+    are still read in q's type. derive: a Derive (or its tuple), as attend() takes it: the keys derived from the value
+    pages (key_pages None); such a chunk is read as window rows of up to MAX_COLUMNS tokens by attend()'s fused launch
+    (a prompt token's bits are those of the same position decoded); not with fresh rows, flash or int8_qk."""
     if derive is not None:
-        raise _unsupported("derive= (keys derived from value rows)")
+        if flash:
+            raise ValueError("derive= reads keys from the value rows on the split and fused launches and prefill's "
+                             "default one: the flash structures (flash=True, flash='cuda') take key pages")
+        if int8_qk:
+            raise ValueError("derive= derives 16-bit keys: not with int8_qk")
+        if key_pages is not None:
+            raise ValueError("derive= reads the value pages as keys too: key_pages None")
+        if fresh is not None:
+            raise _unsupported("derive= with fresh rows")
     _check_sinks(sinks, q)
     sliding = _check_sliding(sliding, None)
     T = q.shape[0]
@@ -798,6 +859,9 @@ def prefill(q, key_pages, value_pages, kind, table, position, page, *, key_scale
         elif first is not None:
             first = first.reshape(1)
         fresh = (fresh[0], fresh[1], first)
+    if derive is not None:
+        return _prefill_as_windows(q, None, value_pages, kind, table.reshape(1, -1), None, None, None, positions, T, 1, page,
+                                   None, value_scales, multipliers, scale, out, lse, sinks, sliding, None, False, derive)
     return _prefill_launch(q, key_pages, value_pages, kind, table.reshape(1, -1), None, None, None, positions, T, 1,
                            page, key_scales, value_scales, multipliers, scale, out, lse, sinks, sliding, fresh,
                            workspace, int8_qk)

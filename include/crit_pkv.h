@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 14
+#define CRIT_PKV_ABI_VERSION 15
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -169,6 +169,18 @@ typedef struct crit_pkv_attend_params {
      * (__init__.py:141-171); here it is the caller's, like every other buffer. NULL: units are dealt to the
      * workgroups in turn, no counters (the same bits; slower on ragged batches). */
     uint32_t* launch_state;
+    /* Keys derived from the value rows on read (the reference's derive=, paged_kv_attention/__init__.py:52-58, 82-121):
+     * a layer that caches one row a position and KV head reads it as its value and, normed and rotated, as its key:
+     * k = rope(rms_norm(r) * weight, position), r the row as stored (codes times their scale or multiplier),
+     * rms_norm(r) = r / sqrt(mean(r * r) + derive_eps), the "half" rotation over the first derive_rot values at the
+     * angle fp32(position) * freqs[i], all in FP32. derive_table: FP32 freqs [derive_rot / 2], then, with
+     * derive_weighted, the weight [head_dim]; NULL: keys from key_pages. With it key_pages and key_scales are not
+     * read (may be NULL); head_dim == value_dim, 64 or 128; derive_rot a multiple of 16 up to head_dim (the reference
+     * takes any even width); no blocks, no fresh rows. */
+    const float* derive_table;
+    float derive_eps;
+    int32_t derive_rot;
+    int32_t derive_weighted;
 } crit_pkv_attend_params;
 
 int crit_pkv_attend(const crit_pkv_attend_params* p, void* stream);

@@ -206,6 +206,23 @@ def windows_dense(q, keys, values, position, scale, sliding=0, sinks=None):
     return out, lse
 
 
+# -- keys derived from the value rows (kernels/.../paged_kv_attention/__init__.py:52-58) --------------------------------
+def derived_keys(rows, weight, eps, freqs, rotary_dim, start=0):
+    """float64 keys of the stored rows [n][HKV][D] (float64) at positions start..: rope(rms_norm(r) * weight, p) with
+    rms_norm(r) = r / sqrt(mean(r * r) + eps), weight [D] or None, the "half" rotation over the first rotary_dim values
+    (value i with value i + rotary_dim / 2, the rest kept) at the angle fp32(p) * freqs[i] taken as an FP32 product, as
+    the kernels take it (tests/test_derived_keys.py:68-81 of the reference)."""
+    y = rows / torch.sqrt((rows * rows).mean(-1, keepdim=True) + eps)
+    if weight is not None:
+        y = y * weight.double()
+    pos = torch.arange(start, start + rows.shape[0], dtype=torch.float32)
+    angle = (pos[:, None] * freqs.float()[None, :]).double()[:, None, :]
+    half = rotary_dim // 2
+    a, b = y[..., :half], y[..., half:rotary_dim]
+    turned = torch.cat([a * angle.cos() - b * angle.sin(), b * angle.cos() + a * angle.sin()], -1)
+    return torch.cat([turned, y[..., rotary_dim:]], -1)
+
+
 # -- the torch fallback over page tables (device_attention.py:1204-1288) ------------------------------------------------
 CHUNK = 1024      # positions a pass (device_attention.py:53)
 

@@ -1,0 +1,189 @@
+"""Keys derived from the value rows on read (attend's and prefill's derive=): a pool of value pages only, each row read as
+its value and, normed and rotated, as its key. Against float64 attention whose keys are derived in float64 on the host
+(oracle.attend.derived_keys) from the rows as the pages store them: every page kind, heads of 128 and 64, GQA, a rotation
+over part of the head and no norm weight, positions at page boundaries, a long row, a sliding window, sinks, trees; a
+column's bits the same alone, in any window, fused or split; a prompt chunk's tokens the same positions decoded; what the
+reference refuses is refused. Mirrors the reference's tests/test_derived_keys.py at its tolerances (8e-3 + 2e-2 |ref|,
+log-sum-exp 1e-3)."""
+import pytest
+import torch
+
+from oracle import attend as oracle_attend
+from tests.support import KINDS, STORE, kernels, rand_q
+
+pytestmark = pytest.mark.gpu
+dev = "cuda"
+EPS = 1e-6
+
+
+class Rows:
+    """One layer's value pages for several sequences over shuffled pages, written values only."""
+
+    def __init__(self, kind, hkv, d, page, lengths, seed=0, multiplier=0.03):
+        self.pk = kernels()
+        g = torch.Generator().manual_seed(seed)
+        self.kind, self.hkv, self.d, self.page = kind, hkv, d, page
+        self.multipliers = (1.0, multiplier) if kind == "fp8" else (1.0, 1.0)
+        width = max(-(-n // page) for n in lengths) + 1
+        n_pages = width * len(lengths) + 3
+        self.v = torch.zeros(n_pages, page, hkv, d, dtype=STORE[kind], device=dev)
+        self.vs = torch.zeros(n_pages, page, hkv, dtype=torch.float32, device=dev) if kind in ("fp8:row", "int8") else None
+        order = torch.randperm(n_pages, generator=g)
+        self.tables = order[:width * len(lengths)].view(len(lengths), width).to(torch.int32).to(dev)
+        for s, n in enumerate(lengths):
+            # rows of several magnitudes (the norm takes them to one): the derived keys are not the rows
+            rows = torch.randn(n, hkv, d, generator=g) * (0.5 + 3 * torch.rand(n, hkv, 1, generator=g))
+            self.pk.write(None, rows.to(dev), self.slots(s, torch.arange(n, device=dev)), None, self.v, kind, None, self.vs,
+                          multipliers=self.multipliers)
+
+    def slots(self, s, positions):
+        return self.tables[s][positions // self.page].long() * self.page + positions % self.page
+
+    def stored(self, s, n):
+        """Positions 0 .. n - 1 of sequence s as the pages hold them, float64 [n][hkv][d], on the CPU."""
+        slots = self.slots(s, torch.arange(n, device=dev))
+        v = self.v.view(-1, self.hkv, self.d)[slots].double()
+        if self.kind == "fp8":
+            v = v * self.multipliers[1]
+        if self.vs is not None:
+            v = v * self.vs.view(-1, self.hkv)[slots].double()[..., None]
+        return v.cpu()
+
+    def attend(self, q, rows, starts, firsts, columns, derive, **kw):
+        i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+        return self.pk.attend(q.to(self.q_dtype), None, self.v, self.kind, self.tables, i32(rows), i32(starts),
+                              torch.tensor(firsts, dtype=torch.int64, device=dev), columns, self.page, value_scales=self.vs,
+                              multipliers=self.multipliers, derive=derive, **kw)
+
+    @property
+    def q_dtype(self):
+        return torch.float16 if self.kind == "fp16" else torch.bfloat16
+
+    def check(self, q, out, lse, derive, s, start, first, count, sliding=0, sinks=None, seen_of=None):
+        weight, eps, freqs, rot = derive[:4]
+        values = self.stored(s, first + count)
+        keys = oracle_attend.derived_keys(values, None if weight is None else weight.cpu(), eps, freqs.cpu(), rot)
+        qd = q.to(self.q_dtype).double().cpu()
+        for c in range(count):
+            n = torch.arange(first + count)
+            seen = n <= first + c if seen_of is None else seen_of(c, n)
+            if sliding:
+                seen = seen & (n > first + c - sliding)
+            want, want_lse = oracle_attend.reference(qd[start + c], keys, values, seen, self.d ** -0.5)
+            if sinks is not None:
+                total = torch.logaddexp(want_lse, sinks.double().cpu())
+                want, want_lse = want * torch.exp(want_lse - total)[:, None], total
+            torch.testing.assert_close(out[start + c].double().cpu(), want, atol=8e-3, rtol=2e-2)
+            if lse is not None:
+                torch.testing.assert_close(lse[start + c].double().cpu(), want_lse, atol=1e-3, rtol=1e-4)
+
+
+def derive_for(pk, d, rotary_dim, weighted=True, seed=5, packed=True):
+    g = torch.Generator().manual_seed(seed)
+    freqs = (10000.0 ** (-torch.arange(0, rotary_dim, 2, dtype=torch.float64) / rotary_dim)).float().to(dev)
+    weight = (1.0 + 0.3 * torch.randn(d, generator=g)).to(dev) if weighted else None
+    return pk.derive(weight, EPS, freqs, rotary_dim) if packed else (weight, EPS, freqs, rotary_dim)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("hq,hkv,d,rot,weighted", [(8, 2, 128, 128, True), (12, 2, 64, 64, True), (8, 4, 128, 64, False),
+                                                   (16, 2, 64, 32, True), (3, 1, 128, 16, True)])
+@pytest.mark.parametrize("fused", [False, True])
+def test_windows_with_derived_keys_match_float64_attention(kind, hq, hkv, d, rot, weighted, fused):
+    # rows whose windows start and end at page boundaries (15/16, 31/32) and one of a single position
+    cache = Rows(kind, hkv, d, 16, [140, 64, 1, 517])
+    derive = derive_for(cache.pk, d, rot, weighted)
+    rows, starts, firsts, counts = [0, 1, 2, 3], [0, 5, 10, 15], [127, 31, 0, 400], [5, 5, 1, 3]
+    q = rand_q(20, hq, d, 3)
+    lse = torch.empty(20, hq, device=dev)
+    out = cache.attend(q, rows, starts, firsts, 5, derive, lse=lse, fused=fused,
+                       counts=torch.tensor(counts, dtype=torch.int32, device=dev))
+    for s, start, first, count in zip(rows, starts, firsts, counts):
+        cache.check(q, out, lse, derive, s, start, first, count)
+
+
+@pytest.mark.parametrize("kind", ["bf16", "fp8:row", "int8", "fp8"])
+def test_a_long_row_and_a_sliding_windows_edges_with_sinks(kind):
+    hq, hkv, d, n = 8, 2, 128, 4096
+    cache = Rows(kind, hkv, d, 64, [n + 4], seed=2)
+    derive = derive_for(cache.pk, d, 128, packed=False)      # (a plain tuple is packed at the call)
+    q = rand_q(4, hq, d, 7)
+    sinks = torch.tensor([0.5, -1.0, float("-inf"), 2.0, 0.0, 1.5, -3.0, 0.25], device=dev)
+    lse = torch.empty(4, hq, device=dev)
+    out = cache.attend(q, [0], [0], [n], 4, derive, lse=lse, sinks=sinks)
+    cache.check(q, out, lse, derive, 0, 0, n, 4, sinks=sinks)
+    out = cache.attend(q, [0], [0], [n], 4, derive, lse=lse, sliding=130)
+    cache.check(q, out, lse, derive, 0, 0, n, 4, sliding=130)
+
+
+@pytest.mark.parametrize("kind", ["bf16", "fp8:row"])
+def test_a_columns_bits_are_its_own_alone_in_any_window_fused_or_split(kind):
+    hq, hkv, d = 8, 2, 128
+    cache = Rows(kind, hkv, d, 16, [300, 90], seed=3)
+    derive = derive_for(cache.pk, d, 64)
+    q = rand_q(8, hq, d, 9)
+    out = cache.attend(q, [0, 1], [0, 4], [290, 80], 4, derive)
+    fused = cache.attend(q, [0, 1], [0, 4], [290, 80], 4, derive, fused=True)
+    assert torch.equal(out, fused)
+    for start, s, first in ((2, 0, 292), (4, 1, 80), (7, 1, 83)):
+        alone = cache.attend(q[start:start + 1], [s], [0], [first], 1, derive)
+        assert torch.equal(alone[0], out[start])
+    wider = cache.attend(q, [1, 0], [4, 0], [80, 290], 8, derive, counts=torch.tensor([4, 4], dtype=torch.int32, device=dev))
+    assert torch.equal(wider, out)
+
+
+def test_a_tree_with_derived_keys_sees_its_ancestors():
+    hq, hkv, d = 4, 1, 64
+    cache = Rows("bf16", hkv, d, 16, [70], seed=4)
+    derive = derive_for(cache.pk, d, 64)
+    q = rand_q(5, hq, d, 11)
+    parents = torch.tensor([-1, 0, 0, 1, 2], dtype=torch.int32, device=dev)
+    lse = torch.empty(5, hq, device=dev)
+    out = cache.attend(q, [0], [0], [65], 5, derive, lse=lse, parents=parents)
+    paths = {0: {0}, 1: {0, 1}, 2: {0, 2}, 3: {0, 1, 3}, 4: {0, 2, 4}}
+    cache.check(q, out, lse, derive, 0, 0, 65, 5,
+                seen_of=lambda c, n: (n < 65) | torch.tensor([int(x) - 65 in paths[c] for x in n]))
+
+
+@pytest.mark.parametrize("kind,d", [("bf16", 128), ("fp8", 64)])
+def test_a_prompt_chunk_with_derived_keys_is_its_positions_decoded(kind, d):
+    pk = kernels()
+    hq, hkv, T, prefix = 8, 2, 150, 37
+    cache = Rows(kind, hkv, d, 16, [prefix + T], seed=6)
+    derive = derive_for(pk, d, d)
+    q = rand_q(T, hq, d, 13).to(cache.q_dtype)
+    lse = torch.empty(T, hq, device=dev)
+    out = pk.prefill(q, None, cache.v, kind, cache.tables[0], prefix, 16, value_scales=cache.vs, multipliers=cache.multipliers,
+                     lse=lse, derive=derive)
+    for t in (0, 63, 64, 149):
+        cache.check(q, out, lse, derive, 0, t, prefix + t, 1)
+        one = cache.attend(q[t:t + 1], [0], [0], [prefix + t], 1, derive)
+        assert torch.equal(one[0], out[t])
+    on_device = pk.prefill(q, None, cache.v, kind, cache.tables[0], torch.tensor([prefix], device=dev), 16,
+                           value_scales=cache.vs, multipliers=cache.multipliers, derive=derive)
+    assert torch.equal(on_device, out)
+
+
+def test_what_derived_keys_do_not_take_is_refused():
+    pk = kernels()
+    cache = Rows("bf16", 2, 128, 16, [40])
+    derive = derive_for(pk, 128, 128)
+    q = rand_q(1, 8, 128, 1)
+    with pytest.raises(ValueError, match="flash structures"):
+        cache.attend(q, [0], [0], [39], 1, derive, flash=True)
+    with pytest.raises(ValueError, match="block lists"):
+        cache.attend(q, [0], [0], [39], 1, derive, blocks=torch.zeros(1, 1, dtype=torch.int32, device=dev), block_size=16)
+    with pytest.raises(ValueError, match="key_pages None"):
+        pk.attend(q.bfloat16(), cache.v, cache.v, "bf16", cache.tables, torch.zeros(1, dtype=torch.int32, device=dev),
+                  torch.zeros(1, dtype=torch.int32, device=dev), torch.tensor([39], device=dev), 1, 16, derive=derive)
+    with pytest.raises(ValueError, match="int8_qk"):
+        pk.prefill(q.bfloat16(), None, cache.v, "bf16", cache.tables[0], 39, 16, derive=derive, int8_qk=True)
+    freqs = derive.freqs
+    for bad, match in (((None, EPS, freqs, 130), "rotary_dim"), ((None, EPS, freqs[:3], 128), "freqs"),
+                       ((torch.ones(64, device=dev), EPS, freqs, 128), "weight"), ((None, -1.0, freqs, 128), "eps")):
+        with pytest.raises(ValueError, match=match):
+            cache.attend(q, [0], [0], [39], 1, bad)
+    with pytest.raises(NotImplementedError):      # (the reference takes any even width)
+        cache.attend(q, [0], [0], [39], 1, (None, EPS, freqs[:4], 8))
+    # a plain tuple needs packing, which a capture cannot do; a Derive made by derive() holds its table
+    assert derive.table.numel() == 64 + 128

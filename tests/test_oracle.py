@@ -311,6 +311,34 @@ def test_the_online_fallback_over_page_tables_is_float64_attention_whatever_its_
         assert torch.equal(short[3], other[3]) and torch.equal(short_lse[3], other_lse[3])
 
 
+def test_derived_keys_are_the_normed_weighted_rows_turned_by_their_positions():
+    # against rms_norm_rope (pinned above by a scalar loop and torch's rms_norm) where the rotation spans the head, by a
+    # scalar float64 loop where it does not, and by what a rotation keeps: each pair's length, and position 0 turns nothing
+    g = torch.Generator().manual_seed(23)
+    rows = torch.randn(6, 2, 32, generator=g, dtype=torch.float64) * 3
+    weight = 1.0 + 0.3 * torch.randn(32, generator=g)
+    freqs = (10000.0 ** (-torch.arange(0, 32, 2, dtype=torch.float64) / 32)).float()
+    keys = attend.derived_keys(rows, weight, 1e-6, freqs, 32, start=7)
+    angle = (torch.arange(7, 13, dtype=torch.float32)[:, None] * freqs[None, :])
+    table = torch.cat([angle.double().cos(), angle.double().sin()], 1).float()
+    want = append.rms_norm_rope(rows.float(), weight, 1e-6, torch.arange(6), table)
+    torch.testing.assert_close(keys.float(), want, atol=2e-6, rtol=2e-6)
+    part = attend.derived_keys(rows, None, 1e-6, freqs[:4] * 3, 8, start=2)
+    for n in range(6):
+        for h in range(2):
+            r = rows[n, h]
+            y = r / math.sqrt(float((r * r).mean()) + 1e-6)
+            for i in range(4):
+                t = float(torch.tensor(float(n + 2), dtype=torch.float32) * (freqs[i] * 3))
+                assert abs(float(part[n, h, i]) - (float(y[i]) * math.cos(t) - float(y[i + 4]) * math.sin(t))) < 1e-12
+                assert abs(float(part[n, h, i + 4]) - (float(y[i + 4]) * math.cos(t) + float(y[i]) * math.sin(t))) < 1e-12
+            assert torch.equal(part[n, h, 8:], y[8:])
+    still = attend.derived_keys(rows, weight, 0.0, freqs, 32, start=0)
+    normed = rows / torch.sqrt((rows * rows).mean(-1, keepdim=True)) * weight.double()
+    torch.testing.assert_close(still[0], normed[0], atol=1e-14, rtol=1e-14)
+    torch.testing.assert_close(still[..., :16] ** 2 + still[..., 16:] ** 2, normed[..., :16] ** 2 + normed[..., 16:] ** 2, atol=1e-12, rtol=1e-12)
+
+
 def test_the_transactional_state_follows_the_references_known_answers():
     from oracle.state import KVState
     state = KVState(capacity=3, key_width=2, value_width=1)      # README.md:224-238, test_techniques.py:471-482
