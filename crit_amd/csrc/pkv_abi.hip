@@ -35,6 +35,10 @@ int crit_pkv_copy_pages(const crit_pkv_copy_pages_params* p, void* stream) {
     return pkv::launch_copy_pages(p, reinterpret_cast<hipStream_t>(stream));
 }
 
+int crit_pkv_latent_attend(const crit_pkv_latent_params* p, void* stream) {
+    return pkv::launch_latent(p, reinterpret_cast<hipStream_t>(stream));
+}
+
 int crit_pkv_round(const crit_pkv_round_params* p, void* stream) {
     return pkv::launch_round(p, reinterpret_cast<hipStream_t>(stream));
 }
@@ -75,6 +79,7 @@ int crit_pkv_params_size(int which) {
         case 7: return (int)sizeof(crit_pkv_read_params);
         case 8: return (int)sizeof(crit_pkv_round_params);
         case 9: return (int)sizeof(crit_pkv_step_params);
+        case 10: return (int)sizeof(crit_pkv_latent_params);
     }
     return -1;
 }

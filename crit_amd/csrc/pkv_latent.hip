@@ -1,0 +1,377 @@
+// Latent attention (multi-head latent attention, absorbed) over a paged cache of compressed rows, for gfx950: decode
+// tokens and verify windows of every query head over rows that hold a position's latent (rank R) and then its rotary
+// key (width P); the latent is the position's value too. What the reference's latent-attention kernels module computes
+// (kernels/techniques/attention/latent-attention/torch-ext/latent_attention/__init__.py:153-229, _kernels.py), split
+// over KV partitions and merged in partition order.
+//
+// A workgroup of four wavefronts serves one unit: 16 query rows (a batch row's columns times its heads, flattened
+// column-major) over pieces b, b + parts, ... of the row's positions, 32 positions a step. The step's cache rows go
+// through LDS once ([position][value], 16-bit) and feed both products on the matrix pipe:
+//   S^T = K Q^T   v_mfma_f32_16x16x32: A = cache rows as they lie (a lane: one position, 8 adjacent values), B = the
+//                 query tile (kept in LDS for the unit). The (R + P) / 32 k-steps are dealt to the four wavefronts,
+//                 whose partial tiles are added through LDS in a fixed order, so every wavefront holds the same scores.
+//   O^T += V^T P^T  v_mfma_f32_16x16x32: B = the probabilities straight from the score tiles' registers (the D layout
+//                 of two 16-position tiles is the B layout of one 32-position k-step, k-slot e of quarter g being
+//                 position 4 g + e of tile 0 for e < 4, of tile 1 else); A = V^T read from the same LDS rows by
+//                 ds_read_b64_tr_b16, which hands a lane 4 consecutive positions of one value. Each wavefront owns R / 4
+//                 of the output values.
+// The online softmax runs in base 2 on scores times scale * log2(e). A query row's bits depend on its own query and
+// positions, `piece` and `partitions` only: the matrix pipe computes each output element from its own row and column,
+// positions past a row's own contribute exact zeros, every sum has a fixed order.
+//
+// Arithmetic intensity: one position is (R + P) * e bytes and 2 * (2 R + P) * rows flops; at 16 heads a launch is
+// HBM-bound, at 128 heads (8 tiles a row) the tiles of one (row, partition) are placed on one XCD so that its L2 serves
+// the cache rows to all of them.
+#include "pkv_attend_mfma.hpp"
+#include "pkv_launch.hpp"
+
+namespace pkv {
+namespace {
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+struct LatentArgs {
+    const uint8_t* q;
+    const uint8_t* cache;
+    const float* scales;
+    const int32_t* tables;
+    const int32_t* rows;
+    int rows_step;
+    const int32_t* starts;
+    const int32_t* counts;
+    const int64_t* firsts;
+    float* po;
+    float* pm;
+    float* pl;
+    void* out;
+    float* lse;
+    const float* sinks;
+    int64_t q_st, q_sh, o_st, o_sh, tab_stride, pairs;
+    int tab_width, n_rows, columns, heads, page, page_shift, parts, gy, piece, tiles, max_keys, scales_per_row, out_dtype;
+    float sscale;
+};
+
+// 4 consecutive positions (rows of the LDS tile) of one value, transposed on the way out of LDS: lane 4 j + c of a
+// 16-lane group points at row j's values 4 c .. 4 c + 3; lane i of the group receives value i of rows 0 .. 3.
+PKV_DEV u32x2 lds_transposed(const uint8_t* p) {
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p));
+    return __builtin_bit_cast(u32x2, v);
+}
+
+template <int R, int P, bool F16, bool FP8>
+__global__ __launch_bounds__(256, 2) void latent_kernel(LatentArgs a) {
+    constexpr int W = R + P;                   // values a cache row holds
+    constexpr int ROWB = W * 2 + 32;           // bytes between rows in LDS: 32 mod 64 words apart, so that 16 rows' 32-byte
+                                               // reads fall on different banks
+    constexpr int KS = W / 32, KSL = R / 32;   // k-steps of the scores; the first KSL are the latent's
+    constexpr int TPW = R / 64;                // 16-value output tiles a wavefront owns
+    constexpr int EB = FP8 ? 1 : 2;
+    constexpr int CPR = W * EB / 16;           // 16-byte chunks of a cache row
+    constexpr int NL = (32 * CPR + 255) / 256; // chunks a thread moves a step
+    constexpr int QCH = W * 2 / 16;
+    constexpr int NPART = FP8 ? 16 : 8;        // floats a lane's partial score tiles take (latent and rotary apart for E4M3)
+    __shared__ __align__(16) uint8_t s_k[32 * ROWB];
+    __shared__ __align__(16) uint8_t s_q[16 * ROWB];
+    __shared__ float s_part[4][NPART][64];
+    __shared__ float s_scale[FP8 ? 32 : 1][2];
+
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 4, li = lane & 15;
+    // Workgroups go to the XCDs in turn: the tiles of one (row, partition) take consecutive places of one XCD.
+    const int64_t bid = blockIdx.x;
+    const int64_t place = bid >> 3;
+    const int64_t pair = (place / a.tiles) * 8 + (bid & 7);
+    const int tile = (int)(place % a.tiles);
+    if (pair >= a.pairs) return;
+    const int r = (int)(pair / a.gy), b = (int)(pair % a.gy);
+    int count = a.columns;
+    if (a.counts) count = min(a.counts[r], a.columns);
+    const int H = a.heads;
+    const int j0 = tile * 16;
+    if (j0 >= count * H) return;
+    const int64_t first64 = a.firsts[r];
+    const int first = (int)(first64 < 0 ? 0 : (first64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first64));
+    const int c_hi = min(count, (j0 + 15) / H + 1);
+    const int n_keys = min(first + c_hi, a.max_keys);
+    const int n_pieces = (n_keys + a.piece - 1) / a.piece;
+    if (b >= n_pieces) return;
+    const int64_t trow = (int64_t)a.rows[(int64_t)r * a.rows_step] * a.tab_stride;
+    const int start = a.starts[r];
+
+    // The lane's query row (column li of the score tiles).
+    const int jq = j0 + li, colq = jq / H, headq = jq - colq * H;
+    const bool liveq = colq < count;
+    const int lim = liveq ? first + colq : -1;
+
+    for (int i = tid; i < 16 * QCH; i += 256) {
+        const int row = i / QCH, ch = i - row * QCH;
+        const int j = j0 + row, col = j / H, head = j - col * H;
+        uint4 w = make_uint4(0, 0, 0, 0);
+        if (col < count) w = *reinterpret_cast<const uint4*>(a.q + ((int64_t)(start + col) * a.q_st + (int64_t)head * a.q_sh) * 2 + ch * 16);
+        *reinterpret_cast<uint4*>(s_q + row * ROWB + ch * 16) = w;
+    }
+
+    uint4 held[NL];
+    float held_scale[2] = {1.0f, 1.0f};
+    auto slot_of = [&](int n) __attribute__((always_inline)) -> int64_t {
+        n = n < n_keys ? n : n_keys - 1;
+        int pidx = a.page_shift >= 0 ? (n >> a.page_shift) : (n / a.page);
+        pidx = pidx < a.tab_width ? pidx : a.tab_width - 1;
+        const int in_page = a.page_shift >= 0 ? (n & (a.page - 1)) : (n - (n / a.page) * a.page);
+        return (int64_t)a.tables[trow + pidx] * a.page + in_page;
+    };
+    auto fetch = [&](int base) __attribute__((always_inline)) {
+#pragma unroll
+        for (int l = 0; l < NL; ++l) {
+            const int i = tid + l * 256;
+            if (32 * CPR % 256 == 0 || i < 32 * CPR) {
+                const int row = i / CPR, ch = i - row * CPR;
+                held[l] = *reinterpret_cast<const uint4*>(a.cache + slot_of(base + row) * (W * EB) + ch * 16);
+            }
+        }
+        if constexpr (FP8) {
+            if (tid < 32) {
+                const float* s = a.scales + slot_of(base + tid) * a.scales_per_row;
+                held_scale[0] = s[0];
+                held_scale[1] = a.scales_per_row > 1 ? s[1] : s[0];
+            }
+        }
+    };
+    auto stage = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int l = 0; l < NL; ++l) {
+            const int i = tid + l * 256;
+            if (32 * CPR % 256 == 0 || i < 32 * CPR) {
+                const int row = i / CPR, ch = i - row * CPR;
+                if constexpr (FP8) {      // 16 codes: 16 values of the queries' type, exactly
+                    const uint32_t w[4] = {held[l].x, held[l].y, held[l].z, held[l].w};
+                    uint32_t o[8];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const f32x2 lo = e4m3_pair<false>(w[k]), hi = e4m3_pair<true>(w[k]);
+                        o[2 * k] = pair16<F16>(lo.x, lo.y), o[2 * k + 1] = pair16<F16>(hi.x, hi.y);
+                    }
+                    uint4* at = reinterpret_cast<uint4*>(s_k + row * ROWB + ch * 32);
+                    at[0] = make_uint4(o[0], o[1], o[2], o[3]);
+                    at[1] = make_uint4(o[4], o[5], o[6], o[7]);
+                } else {
+                    *reinterpret_cast<uint4*>(s_k + row * ROWB + ch * 16) = held[l];
+                }
+            }
+        }
+        if constexpr (FP8) {
+            if (tid < 32) s_scale[tid][0] = held_scale[0], s_scale[tid][1] = held_scale[1];
+        }
+    };
+
+    // The wavefront's steps are the unit's: steps 0 .. of pieces b, b + parts, ...
+    const int steps_per_piece = a.piece / 32;
+    int pi = b, st = 0;
+    auto base_of = [&]() __attribute__((always_inline)) -> int {
+        const int64_t base = (int64_t)pi * a.piece + st * 32;
+        return base < n_keys ? (int)base : -1;
+    };
+    auto advance = [&]() __attribute__((always_inline)) -> int {
+        if (++st >= steps_per_piece) pi += a.parts, st = 0;
+        return base_of();
+    };
+
+    float m = -INFINITY, l = 0.0f;
+    f32x4 acc[TPW];
+#pragma unroll
+    for (int t = 0; t < TPW; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    int base = base_of();      // (>= 0: b < n_pieces)
+    fetch(base);
+    while (base >= 0) {
+        stage();
+        __syncthreads();
+        const int next = advance();
+        if (next >= 0) fetch(next);
+        // -- the step's scores: this wavefront's k-steps of both 16-position tiles
+        f32x4 sl0 = {0.0f, 0.0f, 0.0f, 0.0f}, sl1 = sl0, sr0 = sl0, sr1 = sl0;
+        const uint8_t* qrow = s_q + li * ROWB + g * 16;
+        const uint8_t* krow = s_k + li * ROWB + g * 16;
+#pragma unroll
+        for (int k4 = 0; k4 < (KS + 3) / 4; ++k4) {
+            const int ks = k4 * 4 + wave;
+            if (ks < KS) {
+                const u32x4 bq = *reinterpret_cast<const u32x4*>(qrow + ks * 64);
+                const u32x4 a0 = *reinterpret_cast<const u32x4*>(krow + ks * 64);
+                const u32x4 a1 = *reinterpret_cast<const u32x4*>(krow + 16 * ROWB + ks * 64);
+                if (FP8 && ks >= KSL) {
+                    sr0 = mfma_k32<F16>(a0, bq, sr0);
+                    sr1 = mfma_k32<F16>(a1, bq, sr1);
+                } else {
+                    sl0 = mfma_k32<F16>(a0, bq, sl0);
+                    sl1 = mfma_k32<F16>(a1, bq, sl1);
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            s_part[wave][i][lane] = sl0[i], s_part[wave][4 + i][lane] = sl1[i];
+            if constexpr (FP8) s_part[wave][8 + i][lane] = sr0[i], s_part[wave][12 + i][lane] = sr1[i];
+        }
+        __syncthreads();
+        float x[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float latent = ((s_part[0][e][lane] + s_part[1][e][lane]) + s_part[2][e][lane]) + s_part[3][e][lane];
+            const int at = (e >> 2) * 16 + 4 * g + (e & 3);      // the value's position in the step
+            float v = latent;
+            if constexpr (FP8) {
+                const float rotary = ((s_part[0][8 + e][lane] + s_part[1][8 + e][lane]) + s_part[2][8 + e][lane]) + s_part[3][8 + e][lane];
+                v = __builtin_fmaf(latent, s_scale[at][0], rotary * s_scale[at][1]);
+            }
+            const int n = base + at;
+            x[e] = (n <= lim && n < n_keys) ? v * a.sscale : -INFINITY;
+        }
+        float top = __builtin_fmaxf(__builtin_fmaxf(__builtin_fmaxf(x[0], x[1]), __builtin_fmaxf(x[2], x[3])),
+                                    __builtin_fmaxf(__builtin_fmaxf(x[4], x[5]), __builtin_fmaxf(x[6], x[7])));
+        top = max_across_quarters(top);
+        const float m_new = __builtin_fmaxf(m, top);
+        const float sub = m_new == -INFINITY ? 0.0f : m_new;
+        const float alpha = exp2_fast(m - sub);
+        float p[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) p[e] = exp2_fast(x[e] - sub);
+        const float sum = sum_across_quarters(((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7])));
+        l = __builtin_fmaf(l, alpha, sum);
+        m = m_new;
+        if constexpr (FP8) {      // a value is its code times its position's latent scale: the scale rides on the probability
+#pragma unroll
+            for (int e = 0; e < 8; ++e) p[e] *= s_scale[(e >> 2) * 16 + 4 * g + (e & 3)][0];
+        }
+        const u32x4 bp = {pair16<F16>(p[0], p[1]), pair16<F16>(p[2], p[3]), pair16<F16>(p[4], p[5]), pair16<F16>(p[6], p[7])};
+        // -- the wavefront's quarter of the values
+        const uint8_t* vrow = s_k + (4 * g + (li >> 2)) * ROWB + (li & 3) * 8;
+#pragma unroll
+        for (int t = 0; t < TPW; ++t) {
+            const int ftile = wave * TPW + t;
+            const u32x2 lo = lds_transposed(vrow + ftile * 32);
+            const u32x2 hi = lds_transposed(vrow + 16 * ROWB + ftile * 32);
+            acc[t] *= alpha;
+            acc[t] = mfma_k32<F16>(u32x4{lo.x, lo.y, hi.x, hi.y}, bp, acc[t]);
+        }
+        __syncthreads();
+        base = next;
+    }
+    if (!liveq) return;
+    const int64_t index = ((int64_t)((int64_t)r * a.columns + colq) * H + headq) * a.parts + b;
+#pragma unroll
+    for (int t = 0; t < TPW; ++t)
+        *reinterpret_cast<f32x4*>(a.po + index * R + (wave * TPW + t) * 16 + 4 * g) = acc[t];
+    if (wave == 0 && g == 0) a.pm[index] = m, a.pl[index] = l;
+}
+
+// One workgroup of 64 threads a (batch row, column, head): the partitions' states folded in partition order, the sink
+// last; R / 64 values a thread.
+template <int R>
+__global__ __launch_bounds__(64) void latent_merge_kernel(LatentArgs a) {
+    const int prow = blockIdx.x, head = blockIdx.y;
+    const int r = prow / a.columns, col = prow - r * a.columns;
+    int count = a.columns;
+    if (a.counts) count = min(a.counts[r], a.columns);
+    if (col >= count) return;
+    const int64_t first64 = a.firsts[r];
+    const int first = (int)(first64 < 0 ? 0 : (first64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first64));
+    const int n_keys = min(first + col + 1, a.max_keys);
+    const int n_pieces = (n_keys + a.piece - 1) / a.piece;
+    const int np = min(a.parts, n_pieces);
+    const int64_t index = ((int64_t)prow * a.heads + head) * a.parts;
+    float M = -INFINITY, L = 0.0f, acc[R / 64];
+#pragma unroll
+    for (int i = 0; i < R / 64; ++i) acc[i] = 0.0f;
+    for (int b = 0; b < np; ++b) {
+        const Fold f = fold(M, L, a.pm[index + b], a.pl[index + b]);
+        const float* po = a.po + (index + b) * R;
+#pragma unroll
+        for (int i = 0; i < R / 64; ++i) acc[i] = __builtin_fmaf(acc[i], f.keep, po[i * 64 + threadIdx.x] * f.take);
+        M = f.m, L = f.l;
+    }
+    if (a.sinks) {      // one more position with no value
+        const float sink = a.sinks[head] * kLog2e;
+        const float top = __builtin_fmaxf(M, sink);
+        const float sub = top == -INFINITY ? 0.0f : top;
+        const float keep = exp2_fast(M - sub);
+        L = __builtin_fmaf(L, keep, exp2_fast(sink - sub));
+#pragma unroll
+        for (int i = 0; i < R / 64; ++i) acc[i] *= keep;
+        M = top;
+    }
+    const int64_t token = (int64_t)a.starts[r] + col;
+    const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+#pragma unroll
+    for (int i = 0; i < R / 64; ++i)
+        store_out(a.out, a.out_dtype, token * a.o_st + (int64_t)head * a.o_sh + i * 64 + threadIdx.x, acc[i] * inv);
+    if (a.lse && threadIdx.x == 0) a.lse[token * a.heads + head] = L > 0.0f ? (M + __builtin_log2f(L)) * kLn2 : -INFINITY;
+}
+
+template <int R, int P>
+int launch_shape(const LatentArgs& a, bool f16, bool fp8, int phases, hipStream_t stream) {
+    const int64_t blocks = (a.pairs + 7) / 8 * 8 * a.tiles;
+    if (blocks > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
+    if (phases != 2) {
+        const dim3 grid((unsigned)blocks);
+        if (fp8) {
+            if (f16) hipLaunchKernelGGL((latent_kernel<R, P, true, true>), grid, dim3(256), 0, stream, a);
+            else hipLaunchKernelGGL((latent_kernel<R, P, false, true>), grid, dim3(256), 0, stream, a);
+        } else {
+            if (f16) hipLaunchKernelGGL((latent_kernel<R, P, true, false>), grid, dim3(256), 0, stream, a);
+            else hipLaunchKernelGGL((latent_kernel<R, P, false, false>), grid, dim3(256), 0, stream, a);
+        }
+        if (const hipError_t e = hipGetLastError()) return (int)e;
+    }
+    if (phases != 1) {
+        hipLaunchKernelGGL((latent_merge_kernel<R>), dim3((unsigned)(a.n_rows * a.columns), (unsigned)a.heads), dim3(64), 0, stream, a);
+        return hip_code(hipGetLastError());
+    }
+    return 0;
+}
+
+}   // namespace
+
+int launch_latent(const crit_pkv_latent_params* p, hipStream_t stream) {
+    if (!p || !p->q || !p->cache || !p->tables || !p->rows || !p->starts || !p->firsts || !p->out || !p->partial_out ||
+        !p->partial_max || !p->partial_sum)
+        return CRIT_PKV_E_NULL;
+    const bool fp8 = p->cache_dtype == 2;
+    if (p->cache_dtype < 0 || p->cache_dtype > 2 || (p->q_dtype != CRIT_PKV_BF16 && p->q_dtype != CRIT_PKV_F16)) return CRIT_PKV_E_DTYPE;
+    if (!fp8 && p->cache_dtype != (p->q_dtype == CRIT_PKV_F16 ? 1 : 0)) return CRIT_PKV_E_DTYPE;      // 16-bit rows in the queries' type
+    if (fp8 && (!p->scales || (p->scales_per_row != 1 && p->scales_per_row != 2))) return CRIT_PKV_E_NULL;
+    if (p->out_dtype != CRIT_PKV_F32 && p->out_dtype != CRIT_PKV_BF16 && p->out_dtype != CRIT_PKV_F16) return CRIT_PKV_E_DTYPE;
+    if (p->n_rows < 1 || p->columns < 1 || p->columns > CRIT_PKV_MAX_COLUMNS || p->heads < 1 || p->page < 1 || p->table_width < 1 ||
+        (int64_t)p->n_rows * p->columns > 0x7fffffff || p->heads > 65535)
+        return CRIT_PKV_E_GEOMETRY;
+    if (p->q_stride_t % 8 || p->q_stride_h % 8 || (reinterpret_cast<uintptr_t>(p->q) % 16) || (reinterpret_cast<uintptr_t>(p->cache) % 16))
+        return CRIT_PKV_E_GEOMETRY;
+    if (p->partitions < 1 || p->partitions > 65535 || p->piece < 32 || p->piece % 32) return CRIT_PKV_E_WORKSPACE;
+    LatentArgs a;
+    a.q = reinterpret_cast<const uint8_t*>(p->q), a.cache = reinterpret_cast<const uint8_t*>(p->cache), a.scales = p->scales;
+    a.tables = p->tables, a.rows = reinterpret_cast<const int32_t*>(p->rows), a.rows_step = p->rows_are_64 ? 2 : 1;
+    a.starts = p->starts, a.counts = p->counts, a.firsts = p->firsts;
+    a.po = p->partial_out, a.pm = p->partial_max, a.pl = p->partial_sum;
+    a.out = p->out, a.lse = p->lse, a.sinks = p->sinks;
+    a.q_st = p->q_stride_t, a.q_sh = p->q_stride_h, a.o_st = p->out_stride_t, a.o_sh = p->out_stride_h, a.tab_stride = p->table_stride;
+    a.tab_width = p->table_width, a.n_rows = p->n_rows, a.columns = p->columns, a.heads = p->heads, a.page = p->page;
+    a.page_shift = -1;
+    for (int s = 0; s < 31; ++s)
+        if ((1 << s) == p->page) a.page_shift = s;
+    a.parts = p->partitions, a.piece = p->piece, a.scales_per_row = p->scales_per_row, a.out_dtype = p->out_dtype;
+    a.sscale = p->scale * kLog2e;
+    a.tiles = (p->columns * p->heads + 15) / 16;
+    const int64_t table_keys = (int64_t)p->table_width * p->page;
+    a.max_keys = (int)(table_keys < 0x3fffffff ? table_keys : 0x3fffffff);
+    if ((int64_t)p->partitions * p->piece > 0x3fffffff) return CRIT_PKV_E_WORKSPACE;
+    const int64_t live_parts = ((int64_t)a.max_keys + p->piece - 1) / p->piece;
+    a.gy = (int)(live_parts < p->partitions ? live_parts : p->partitions);
+    a.pairs = (int64_t)p->n_rows * a.gy;
+    const bool f16 = p->q_dtype == CRIT_PKV_F16;
+#define PKV_LATENT(RANK, ROPE) \
+    if (p->rank == RANK && p->rope == ROPE) return launch_shape<RANK, ROPE>(a, f16, fp8, p->phases, stream);
+    PKV_LATENT(512, 64) PKV_LATENT(256, 64) PKV_LATENT(128, 64) PKV_LATENT(128, 32) PKV_LATENT(64, 64) PKV_LATENT(64, 32)
+#undef PKV_LATENT
+    return CRIT_PKV_E_GEOMETRY;
+}
+
+}   // namespace pkv

@@ -10,7 +10,7 @@ import shutil
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 NAME = "libcrit_pkv.so"
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 KIND_16BIT, KIND_FP8, KIND_FP8_ROW, KIND_INT8 = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
@@ -105,6 +105,16 @@ class StepParams(ctypes.Structure):
                 ("table_pages", _i32), ("page", _i32), ("dump", _i32)]
 
 
+class LatentParams(ctypes.Structure):
+    _fields_ = [("q", _p), ("cache", _p), ("scales", _p), ("tables", _p), ("rows", _p), ("starts", _p), ("counts", _p),
+                ("firsts", _p), ("partial_out", _p), ("partial_max", _p), ("partial_sum", _p), ("out", _p), ("lse", _p),
+                ("sinks", _p),
+                ("q_stride_t", _i64), ("q_stride_h", _i64), ("out_stride_t", _i64), ("out_stride_h", _i64), ("table_stride", _i64),
+                ("table_width", _i32), ("n_rows", _i32), ("columns", _i32), ("heads", _i32), ("rank", _i32), ("rope", _i32),
+                ("page", _i32), ("cache_dtype", _i32), ("q_dtype", _i32), ("out_dtype", _i32), ("scales_per_row", _i32),
+                ("partitions", _i32), ("piece", _i32), ("rows_are_64", _i32), ("phases", _i32), ("scale", _f32)]
+
+
 class ReadParams(ctypes.Structure):
     _fields_ = [("key_pages", _p), ("value_pages", _p), ("key_scales", _p), ("value_scales", _p), ("head_multipliers", _p),
                 ("slots", _p), ("table", _p), ("table64", _p), ("out_keys", _p), ("out_values", _p), ("n", _i64), ("pool_slots", _i64),
@@ -115,7 +125,7 @@ class ReadParams(ctypes.Structure):
 STATIC_SCRATCH_BYTES = 32 << 20
 
 SYMBOLS = ("crit_pkv_write", "crit_pkv_attend", "crit_pkv_attend_static", "crit_pkv_merge", "crit_pkv_prefill", "crit_pkv_slots_at",
-           "crit_pkv_compact", "crit_pkv_copy_pages", "crit_pkv_round", "crit_pkv_step_buffers", "crit_pkv_read_rows", "crit_pkv_abi_version", "crit_pkv_params_size", "crit_pkv_error",
+           "crit_pkv_compact", "crit_pkv_copy_pages", "crit_pkv_round", "crit_pkv_step_buffers", "crit_pkv_latent_attend", "crit_pkv_read_rows", "crit_pkv_abi_version", "crit_pkv_params_size", "crit_pkv_error",
            "crit_pkv_stream_read", "crit_pkv_stream_capture")
 
 _lib = None
@@ -165,7 +175,8 @@ def load():
                          ("crit_pkv_merge", MergeParams), ("crit_pkv_prefill", PrefillParams),
                          ("crit_pkv_slots_at", SlotsParams), ("crit_pkv_compact", CompactParams),
                          ("crit_pkv_copy_pages", CopyPagesParams), ("crit_pkv_round", RoundParams),
-                         ("crit_pkv_step_buffers", StepParams), ("crit_pkv_read_rows", ReadParams)):
+                         ("crit_pkv_step_buffers", StepParams), ("crit_pkv_latent_attend", LatentParams),
+                         ("crit_pkv_read_rows", ReadParams)):
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(struct), ctypes.c_void_p]
@@ -176,7 +187,7 @@ def load():
     if lib.crit_pkv_abi_version() != ABI_VERSION:
         raise RuntimeError(f"{path} speaks ABI {lib.crit_pkv_abi_version()}, this package {ABI_VERSION}: rebuild it")
     for which, struct in enumerate((WriteParams, AttendParams, MergeParams, PrefillParams, SlotsParams, CompactParams,
-                                    CopyPagesParams, ReadParams, RoundParams, StepParams)):
+                                    CopyPagesParams, ReadParams, RoundParams, StepParams, LatentParams)):
         if lib.crit_pkv_params_size(which) != ctypes.sizeof(struct):
             raise RuntimeError(f"{path}: parameter struct {which} is {lib.crit_pkv_params_size(which)} bytes, the "
                                f"Python mirror {ctypes.sizeof(struct)}: rebuild the library")

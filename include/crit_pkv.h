@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 15
+#define CRIT_PKV_ABI_VERSION 16
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -389,6 +389,45 @@ typedef struct crit_pkv_step_params {
 
 int crit_pkv_step_buffers(const crit_pkv_step_params* p, void* stream);
 
+/* ---- latent attention ---------------------------------------------------------------------------------------------
+ * Replaces attend() of crit's latent-attention kernels module (kernels/techniques/attention/latent-attention/torch-ext/
+ * latent_attention/__init__.py:153-229 and its _window_kernel / _merge_kernel), which crit's attention plugin calls for
+ * pools of keys only with one KV head (inference/attention-state/code/device_attention.py:444-519): multi-head latent
+ * attention, absorbed. cache [pages][page][rank + rope]: a position's latent, then its rotary key; the latent is the
+ * position's value too. q [tokens][heads][rank + rope]; out [tokens][heads][rank]. Batch rows, tables, rows, starts,
+ * counts, firsts and columns as crit_pkv_attend_params; causal inside the window:
+ *   s[n] = scale * (q_latent . latent[n] + q_rope . rope[n]);  out = sum_n softmax(s)[n] * latent[n]
+ * 16-bit products on the matrix pipe with FP32 sums, the probabilities rounded to q's type for the value product, the
+ * softmax in FP32. A row's positions are cut into pieces of `piece` positions (a multiple of 32), piece i to partition
+ * i mod partitions; partials [n_rows * columns][heads][partitions] x (rank floats, a maximum, a sum) are merged in
+ * partition order, the sink logit (sinks [heads], natural log, -inf: none) folded in last; lse [tokens][heads] the
+ * natural log-sum-exp (the sink counted). cache_dtype: 0 BF16, 1 FP16 (q in the same type), 2 E4M3 with `scales`
+ * [pages][page][scales_per_row] FP32 (2: the latent's and the rotary key's, 1: one for the row) and BF16 or FP16 q.
+ * (rank, rope) is one of (512, 64), (256, 64), (128, 64), (128, 32), (64, 64), (64, 32). phases: 0 both launches, 1
+ * the partitions only, 2 the merge only. */
+typedef struct crit_pkv_latent_params {
+    const void* q;
+    const void* cache;
+    const float* scales;
+    const int32_t* tables;
+    const void* rows;               /* int32, or int64 with rows_are_64 */
+    const int32_t* starts;
+    const int32_t* counts;          /* optional */
+    const int64_t* firsts;
+    float* partial_out;
+    float* partial_max;
+    float* partial_sum;
+    void* out;
+    float* lse;                     /* optional */
+    const float* sinks;             /* optional */
+    int64_t q_stride_t, q_stride_h, out_stride_t, out_stride_h, table_stride;
+    int32_t table_width, n_rows, columns, heads, rank, rope, page, cache_dtype, q_dtype, out_dtype, scales_per_row,
+        partitions, piece, rows_are_64, phases;
+    float scale;
+} crit_pkv_latent_params;
+
+int crit_pkv_latent_attend(const crit_pkv_latent_params* p, void* stream);
+
 /* ---- rows read back ----------------------------------------------------------------------------------------------
  * Replaces the index_select, cast and multiply of KVPool.gather and KVPool.rows_at (pages.py:455-493): row i of the
  * output is the pool's row at slots[i], or, with a page table instead (exactly one of slots, table, table64), at
@@ -419,7 +458,7 @@ int crit_pkv_read_rows(const crit_pkv_read_params* p, void* stream);
 /* ---- housekeeping ------------------------------------------------------------------------------------------------- */
 int crit_pkv_abi_version(void);
 /* sizeof() of the parameter structs as the library was compiled, for the host's mirror to cross-check
- * (which: 0 write, 1 attend, 2 merge, 3 prefill, 4 slots_at, 5 compact, 6 copy_pages, 7 read_rows, 8 round, 9 step_buffers), as crit_cw_params_size() does (cuda_window.cu:1502). */
+ * (which: 0 write, 1 attend, 2 merge, 3 prefill, 4 slots_at, 5 compact, 6 copy_pages, 7 read_rows, 8 round, 9 step_buffers, 10 latent_attend), as crit_cw_params_size() does (cuda_window.cu:1502). */
 int crit_pkv_params_size(int which);
 const char* crit_pkv_error(int code);
 /* *id = the id of the capture `stream` is recording into (never 0), or 0 when it is not capturing; returns 0 or a HIP

@@ -1,0 +1,210 @@
+"""Latent attention on the GPU against the float64 oracle (oracle.latent, the reference's latent_attention.py) over the
+rows as the cache stores them: decode tokens and verify windows over shuffled pages at the ranks and heads of the models
+that use it, sinks and log-sum-exps, BF16, FP16 and E4M3 caches (two scales a position, or one); a token's bits the same
+alone, in a verify window, beside other rows, fused or not and in a prompt chunk; one graph replayed at other lengths;
+what the module refuses. Mirrors the reference's kernels/techniques/attention/latent-attention/tests/
+test_latent_attention.py at its tolerances (8e-3 + 2e-2 |ref|; log-sum-exp 1e-3). Calls go through the module, which
+reaches the HIP kernels through the C ABI."""
+import pytest
+import torch
+
+from oracle import latent as oracle_latent
+
+pytestmark = pytest.mark.gpu
+dev = "cuda"
+
+
+def module():
+    import crit_amd.latent_attention as la
+    return la
+
+
+class Cache:
+    """Sequences of compressed rows (latent R, rotary key P) over shuffled pages, written by the module's write()."""
+
+    def __init__(self, rank, rope, page, lengths, seed=0, dtype=torch.bfloat16, scales=0):
+        self.la = module()
+        g = torch.Generator().manual_seed(seed)
+        self.rank, self.rope, self.page = rank, rope, page
+        width = max(-(-n // page) for n in lengths) + 1
+        n_pages = width * len(lengths) + 2
+        self.cache = torch.zeros(n_pages, page, rank + rope, dtype=dtype, device=dev)
+        self.scales = torch.zeros(n_pages, page, 2, device=dev) if scales else None
+        order = torch.randperm(n_pages, generator=g)
+        self.tables = order[:width * len(lengths)].view(len(lengths), width).to(torch.int32).to(dev)
+        for s, n in enumerate(lengths):
+            latent = torch.randn(n, rank, generator=g).to(dev)
+            rope_k = torch.randn(n, rope, generator=g).to(dev) * (3 if scales else 1)
+            self.la.write(latent, rope_k, self.slots(s, torch.arange(n, device=dev)), self.cache, self.scales)
+        if scales == 1:      # one scale a row (a KV pool's fp8:row pages of one head): recode each row at one scale
+            rows = self.cache.view(-1, rank + rope).float() * torch.cat(
+                [self.scales.view(-1, 2)[:, :1].expand(-1, rank), self.scales.view(-1, 2)[:, 1:].expand(-1, rope)], 1)
+            one = (rows.abs().amax(-1) / 448.0).clamp(min=1e-30)
+            self.cache = (rows / one[:, None]).clamp(-448, 448).to(torch.float8_e4m3fn).view(n_pages, page, rank + rope)
+            self.scales = one.view(n_pages, page, 1).contiguous()
+
+    def slots(self, s, positions):
+        return self.tables[s][positions // self.page].long() * self.page + positions % self.page
+
+    def rows(self, s, n):
+        return oracle_latent.stored(self.cache.cpu(), None if self.scales is None else self.scales.cpu(), self.tables[s].cpu(),
+                                    n, self.page, self.rank)
+
+    def attend(self, q, rows, starts, firsts, columns, **kw):
+        return self.la.attend(q, self.cache, self.tables, torch.tensor(rows, dtype=torch.int32, device=dev),
+                              torch.tensor(starts, dtype=torch.int32, device=dev),
+                              torch.tensor(firsts, dtype=torch.int64, device=dev), columns, self.page, rank=self.rank,
+                              scales=self.scales, **kw)
+
+    def check(self, q, out, lse, s, start, first, count, scale, sinks=None, lse_tol=1e-3):
+        latent, rope_k = self.rows(s, first + count)
+        seen = torch.arange(first + count)[None, :] <= first + torch.arange(count)[:, None]
+        span = slice(start, start + count)
+        qc = q[span].double().cpu()
+        want, want_lse = oracle_latent.latent_attention(qc[:, :, :self.rank], qc[:, :, self.rank:], latent, rope_k, seen, scale,
+                                                        None if sinks is None else sinks.cpu())
+        torch.testing.assert_close(out[span].double().cpu(), want, atol=8e-3, rtol=2e-2)
+        if lse is not None:
+            torch.testing.assert_close(lse[span].double().cpu(), want_lse, atol=lse_tol, rtol=1e-4)
+
+
+def _q(tokens, heads, width, seed, dtype=torch.bfloat16):
+    return (torch.randn(tokens, heads, width, generator=torch.Generator().manual_seed(seed)) * 0.5).to(dev, dtype)
+
+
+@pytest.mark.parametrize("rank,rope,heads,page", [(512, 64, 16, 64), (512, 64, 128, 16), (256, 64, 8, 32), (128, 32, 20, 16),
+                                                 (64, 32, 3, 48), (128, 64, 5, 16), (64, 64, 40, 16)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_windows_match_float64_latent_attention(rank, rope, heads, page, dtype):
+    cache = Cache(rank, rope, page, [130, 64, 1, 517], dtype=dtype)
+    rows, starts, firsts, counts = [0, 1, 2, 3], [0, 5, 10, 15], [125, 59, 0, 400], [5, 5, 1, 3]
+    q = _q(20, heads, rank + rope, 3, dtype)
+    scale = 192 ** -0.5
+    sinks = torch.randn(heads, generator=torch.Generator().manual_seed(9)).to(dev)
+    sinks[0] = float("-inf")
+    for given in (None, sinks):
+        lse = torch.full((20, heads), 7.0, device=dev)
+        out = cache.attend(q, rows, starts, firsts, 5, scale=scale, lse=lse,
+                           counts=torch.tensor(counts, dtype=torch.int32, device=dev), sinks=given)
+        for s, start, first, count in zip(rows, starts, firsts, counts):
+            cache.check(q, out, lse, s, start, first, count, scale, given)
+        assert bool((lse[11:15] == 7.0).all()) and bool((lse[18:] == 7.0).all())      # only the rows' tokens are written
+
+
+def test_a_tokens_bits_are_its_own_alone_in_a_window_and_beside_other_rows():
+    cache = Cache(512, 64, 64, [700, 300, 2100], seed=2)
+    q = _q(24, 16, 576, 5)
+    together = cache.attend(q, [0, 1, 2], [0, 8, 16], [690, 290, 2090], 8)
+    for r, (start, first) in enumerate(zip([0, 8, 16], [690, 290, 2090])):
+        for c in range(8):
+            alone = cache.attend(q[start + c:start + c + 1], [r], [0], [first + c], 1)
+            assert torch.equal(alone[0], together[start + c]), (r, c)
+        window = cache.attend(q[start:start + 8], [r], [0], [first], 8)
+        assert torch.equal(window, together[start:start + 8]), r
+    # rows launched a few at a time (their partials bounded) and a round's int64 rows: the same bits
+    la = cache.la
+    limit = la.PARTIAL_BYTES
+    try:
+        la.PARTIAL_BYTES = 8 * 16 * la.partitions(torch.device(dev), 16, 512, 64, 64) * 514 * 4      # one row's
+        sliced = cache.attend(q, [0, 1, 2], [0, 8, 16], [690, 290, 2090], 8, fused=True)
+    finally:
+        la.PARTIAL_BYTES = limit
+    assert torch.equal(sliced, together)
+    as_slots = la.attend(q, cache.cache, cache.tables, torch.tensor([0, 1, 2], device=dev), torch.tensor([0, 8, 16], dtype=torch.int32, device=dev),
+                         torch.tensor([690, 290, 2090], device=dev), 8, 64, rank=512)
+    assert torch.equal(as_slots, together)
+
+
+def test_one_graph_replays_at_every_length():
+    cache = Cache(512, 64, 64, [4000], seed=3)
+    la = cache.la
+    q = _q(1, 16, 576, 7)
+    first = torch.tensor([10], dtype=torch.int64, device=dev)
+    args = (cache.cache, cache.tables, torch.zeros(1, dtype=torch.int32, device=dev), torch.zeros(1, dtype=torch.int32, device=dev),
+            first, 1, 64)
+    out = torch.empty(1, 16, 512, dtype=torch.bfloat16, device=dev)
+    la.attend(q, *args, rank=512, out=out)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        la.attend(q, *args, rank=512, out=out)
+    for at in (0, 63, 64, 1000, 3999):
+        first.fill_(at)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, cache.attend(q, [0], [0], [at], 1)), at
+
+
+def test_what_it_cannot_read_is_refused():
+    cache = Cache(512, 64, 64, [10])
+    la = cache.la
+    q = _q(1, 16, 576, 1)
+    some = lambda: (torch.zeros(1, dtype=t, device=dev) for t in (torch.int32, torch.int32, torch.int64))
+    with pytest.raises(ValueError, match="BF16 or FP16 in the cache's dtype"):
+        cache.attend(q.float(), [0], [0], [5], 1)
+    with pytest.raises(ValueError, match="powers of two"):
+        la.attend(q, cache.cache, cache.tables, *some(), 1, 64, rank=500)
+    with pytest.raises(ValueError, match="columns a row"):
+        cache.attend(q, [0], [0], [5], 65)
+    with pytest.raises(ValueError, match="sinks are contiguous FP32"):
+        cache.attend(q, [0], [0], [5], 1, sinks=torch.zeros(3, device=dev))
+    with pytest.raises(NotImplementedError, match="is not built"):      # (the reference takes every power of two)
+        la.attend(q[:, :, :48].contiguous(), torch.zeros(4, 64, 48, dtype=torch.bfloat16, device=dev), cache.tables, *some(), 1, 64, rank=32)
+    codes = torch.zeros(4, 64, 576, dtype=torch.float8_e4m3fn, device=dev)
+    with pytest.raises(ValueError, match="E4M3 cache takes its scales"):
+        la.attend(q, codes, cache.tables, *some(), 1, 64, rank=512)
+    with pytest.raises(ValueError, match="multiple of 32"):
+        cache.attend(q, [0], [0], [5], 1, piece=48)
+
+
+@pytest.mark.parametrize("scales", [2, 1])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_an_e4m3_cache_matches_float64_over_its_stored_values_and_keeps_a_tokens_bits(scales, dtype):
+    cache = Cache(512, 64, 64, [130, 517], seed=6, dtype=torch.float8_e4m3fn, scales=scales)
+    q = _q(8, 16, 576, 8, dtype)
+    lse = torch.empty(8, 16, device=dev)
+    scale = 192 ** -0.5
+    out = cache.attend(q, [0, 1], [0, 4], [126, 513], 4, scale=scale, lse=lse)
+    for s, start, first in ((0, 0, 126), (1, 4, 513)):
+        cache.check(q, out, lse, s, start, first, 4, scale)
+        for c in range(4):
+            alone = cache.attend(q[start + c:start + c + 1], [s], [0], [first + c], 1, scale=scale)
+            assert torch.equal(alone[0], out[start + c]), (s, c)
+
+
+@pytest.mark.parametrize("rank,rope,heads,page", [(512, 64, 16, 64), (512, 64, 128, 16), (128, 32, 20, 16)])
+def test_prompt_chunks_match_float64_and_are_their_positions_decoded(rank, rope, heads, page):
+    cache = Cache(rank, rope, page, [900], seed=11)
+    la = cache.la
+    sinks = torch.randn(heads, generator=torch.Generator().manual_seed(12)).to(dev)
+    scale = 192 ** -0.5
+    for position, T in ((0, 70), (400, 133), (899 - 37, 38)):
+        q = _q(T, heads, rank + rope, position + 1)
+        for given in (None, sinks):
+            lse = torch.empty(T, heads, device=dev)
+            out = la.prefill(q, cache.cache, cache.tables[0], position, page, rank=rank, scale=scale, lse=lse, sinks=given)
+            cache.check(q, out, lse, 0, 0, position, T, scale, given, lse_tol=2e-3)
+        for t in (0, T // 2, T - 1):
+            alone = cache.attend(q[t:t + 1], [0], [0], [position + t], 1, scale=scale, sinks=sinks)
+            assert torch.equal(alone[0], out[t]), (position, t)
+
+
+def test_a_prompt_tokens_bits_do_not_follow_its_chunks_length_and_a_graph_replays_at_device_positions():
+    cache = Cache(512, 64, 64, [3000], seed=13)
+    la = cache.la
+    q = _q(200, 16, 576, 14)
+    full = la.prefill(q, cache.cache, cache.tables[0], 2000, 64, rank=512)
+    for T in (1, 37, 64, 129):
+        assert torch.equal(la.prefill(q[:T], cache.cache, cache.tables[0], 2000, 64, rank=512), full[:T]), T
+    position = torch.tensor([0], dtype=torch.int64, device=dev)
+    out = torch.empty(200, 16, 512, dtype=torch.bfloat16, device=dev)
+    la.prefill(q, cache.cache, cache.tables[0], position, 64, rank=512, out=out)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        la.prefill(q, cache.cache, cache.tables[0], position, 64, rank=512, out=out)
+    for at in (0, 700, 2799):
+        position.fill_(at)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, la.prefill(q, cache.cache, cache.tables[0], at, 64, rank=512)), at

@@ -339,6 +339,64 @@ def test_derived_keys_are_the_normed_weighted_rows_turned_by_their_positions():
     torch.testing.assert_close(still[..., :16] ** 2 + still[..., 16:] ** 2, normed[..., :16] ** 2 + normed[..., 16:] ** 2, atol=1e-12, rtol=1e-12)
 
 
+def test_latent_attention_is_attention_over_latent_and_rotary_keys_with_the_latent_as_value():
+    from oracle import latent as oracle_latent
+    g = torch.Generator().manual_seed(29)
+    T, H, R, P, N = 3, 4, 8, 4, 11
+    ql, qr = torch.randn(T, H, R, generator=g, dtype=torch.float64), torch.randn(T, H, P, generator=g, dtype=torch.float64)
+    c, k = torch.randn(N, R, generator=g, dtype=torch.float64), torch.randn(N, P, generator=g, dtype=torch.float64)
+    seen = torch.arange(N)[None, :] <= torch.tensor([4, 10, 0])[:, None]
+    seen[2, 0] = False                                       # a token that sees nothing
+    scale = 0.3
+    out, lse = oracle_latent.latent_attention(ql, qr, c, k, seen, scale)
+    for t in range(T):
+        # ordinary attention with one KV head: keys the whole rows, values their latents
+        want, want_lse = attend.reference(torch.cat([ql[t], qr[t]], -1), torch.cat([c, k], -1)[:, None], c[:, None], seen[t], scale)
+        torch.testing.assert_close(out[t], want, atol=1e-12, rtol=1e-12)
+        torch.testing.assert_close(lse[t], want_lse, atol=1e-12, rtol=1e-12)
+    # a scalar loop
+    t, h = 1, 2
+    scores = [scale * (sum(float(ql[t, h, i]) * float(c[n, i]) for i in range(R)) + sum(float(qr[t, h, i]) * float(k[n, i]) for i in range(P)))
+              for n in range(N)]
+    top = max(scores)
+    w = [math.exp(x - top) for x in scores]
+    for i in range(R):
+        assert abs(float(out[t, h, i]) - sum(wn * float(c[n, i]) for n, wn in enumerate(w)) / sum(w)) < 1e-12
+    assert abs(float(lse[t, h]) - (top + math.log(sum(w)))) < 1e-12
+    assert out[2].eq(0).all() and lse[2].eq(float("-inf")).all()
+    # a sink is one more position with no value: out shrinks by e^lse / (e^lse + e^sink), lse grows to their logaddexp
+    sinks = torch.tensor([0.5, float("-inf"), -2.0, 3.0], dtype=torch.float64)
+    with_sinks, sink_lse = oracle_latent.latent_attention(ql, qr, c, k, seen, scale, sinks)
+    total = torch.logaddexp(lse, sinks[None, :])
+    torch.testing.assert_close(sink_lse, total, atol=1e-12, rtol=1e-12)
+    torch.testing.assert_close(with_sinks[:2], (out * torch.exp(lse - total)[..., None])[:2], atol=1e-12, rtol=1e-12)
+    assert with_sinks[2].eq(0).all() and sink_lse[2, 1] == float("-inf") and sink_lse[2, 0] == 0.5
+
+
+def test_a_latent_caches_rows_are_the_latent_then_the_rotary_key_each_part_coded_at_its_own_scale():
+    from oracle import latent as oracle_latent
+    g = torch.Generator().manual_seed(31)
+    n, R, P, page = 9, 16, 8, 4
+    latent, rope = torch.randn(n, R, generator=g), torch.randn(n, P, generator=g) * 5
+    latent[3] = 0                                            # a row of zeros: the floor of 1e-30
+    table = torch.tensor([2, 0, 3])
+    slots = table[torch.arange(n) // page] * page + torch.arange(n) % page
+    cache = torch.zeros(4, page, R + P, dtype=torch.bfloat16)
+    oracle_latent.write(latent, rope, slots, cache)
+    got_l, got_r = oracle_latent.stored(cache, None, table, n, page, R)
+    assert torch.equal(got_l, latent.bfloat16().double()) and torch.equal(got_r, rope.bfloat16().double())
+    codes, scales = torch.zeros(4, page, R + P, dtype=torch.float8_e4m3fn), torch.zeros(4, page, 2)
+    oracle_latent.write(latent, rope, slots, codes, scales)
+    flat, sc = codes.view(-1, R + P).view(torch.uint8), scales.view(-1, 2)
+    for i, s in enumerate(slots.tolist()):
+        for part, lo, hi, which in ((latent[i], 0, R, 0), (rope[i], R, R + P, 1)):
+            want, scale = append.encode(part[None, None, :], "fp8:row")      # the pool's rule for a row: amax / 448, IEEE
+            assert torch.equal(flat[s, lo:hi], want.view(torch.uint8)[0, 0]) and float(sc[s, which]) == float(scale[0, 0])
+    assert float(sc[slots[3], 0]) == 1e-30 or abs(float(sc[slots[3], 0]) - 1e-30) < 1e-37
+    got_l, got_r = oracle_latent.stored(codes, scales, table, n, page, R)
+    torch.testing.assert_close(got_l.float(), latent, atol=0.07, rtol=0.07)
+
+
 def test_the_transactional_state_follows_the_references_known_answers():
     from oracle.state import KVState
     state = KVState(capacity=3, key_width=2, value_width=1)      # README.md:224-238, test_techniques.py:471-482
