@@ -8,8 +8,9 @@
 // column-major) over pieces b, b + parts, ... of the row's positions, 32 positions a step. The step's cache rows go
 // through LDS once ([position][value], 16-bit) and feed both products on the matrix pipe:
 //   S^T = K Q^T   v_mfma_f32_16x16x32: A = cache rows as they lie (a lane: one position, 8 adjacent values), B = the
-//                 query tile (kept in LDS for the unit). The (R + P) / 32 k-steps are dealt to the four wavefronts,
-//                 whose partial tiles are added through LDS in a fixed order, so every wavefront holds the same scores.
+//                 query tile. The (R + P) / 32 k-steps are dealt to the four wavefronts (each keeps its k-steps of the
+//                 queries in registers for the unit), whose partial tiles are added through LDS in a fixed order, so
+//                 every wavefront holds the same scores.
 //   O^T += V^T P^T  v_mfma_f32_16x16x32: B = the probabilities straight from the score tiles' registers (the D layout
 //                 of two 16-position tiles is the B layout of one 32-position k-step, k-slot e of quarter g being
 //                 position 4 g + e of tile 0 for e < 4, of tile 1 else); A = V^T read from the same LDS rows by
@@ -47,7 +48,8 @@ struct LatentArgs {
     float* lse;
     const float* sinks;
     int64_t q_st, q_sh, o_st, o_sh, tab_stride, pairs;
-    int tab_width, n_rows, columns, heads, page, page_shift, parts, gy, piece, tiles, max_keys, scales_per_row, out_dtype;
+    int tab_width, n_rows, columns, heads, page, parts, gy, piece, tiles, max_keys, scales_per_row, out_dtype;
+    Div32 page_div;
     float sscale;
 };
 
@@ -59,7 +61,7 @@ PKV_DEV u32x2 lds_transposed(const uint8_t* p) {
 }
 
 template <int R, int P, bool F16, bool FP8>
-__global__ __launch_bounds__(256, 2) void latent_kernel(LatentArgs a) {
+__global__ __launch_bounds__(256, 3) void latent_kernel(LatentArgs a) {
     constexpr int W = R + P;                   // values a cache row holds
     constexpr int ROWB = W * 2 + 32;           // bytes between rows in LDS: 32 mod 64 words apart, so that 16 rows' 32-byte
                                                // reads fall on different banks
@@ -67,11 +69,10 @@ __global__ __launch_bounds__(256, 2) void latent_kernel(LatentArgs a) {
     constexpr int TPW = R / 64;                // 16-value output tiles a wavefront owns
     constexpr int EB = FP8 ? 1 : 2;
     constexpr int CPR = W * EB / 16;           // 16-byte chunks of a cache row
-    constexpr int NL = (32 * CPR + 255) / 256; // chunks a thread moves a step
-    constexpr int QCH = W * 2 / 16;
+    constexpr int NL = (CPR + 7) / 8;          // chunks a thread moves a step
+    constexpr int KPW = (KS + 3) / 4;          // k-steps a wavefront takes
     constexpr int NPART = FP8 ? 16 : 8;        // floats a lane's partial score tiles take (latent and rotary apart for E4M3)
     __shared__ __align__(16) uint8_t s_k[32 * ROWB];
-    __shared__ __align__(16) uint8_t s_q[16 * ROWB];
     __shared__ float s_part[4][NPART][64];
     __shared__ float s_scale[FP8 ? 32 : 1][2];
 
@@ -102,46 +103,50 @@ __global__ __launch_bounds__(256, 2) void latent_kernel(LatentArgs a) {
     const bool liveq = colq < count;
     const int lim = liveq ? first + colq : -1;
 
-    for (int i = tid; i < 16 * QCH; i += 256) {
-        const int row = i / QCH, ch = i - row * QCH;
-        const int j = j0 + row, col = j / H, head = j - col * H;
-        uint4 w = make_uint4(0, 0, 0, 0);
-        if (col < count) w = *reinterpret_cast<const uint4*>(a.q + ((int64_t)(start + col) * a.q_st + (int64_t)head * a.q_sh) * 2 + ch * 16);
-        *reinterpret_cast<uint4*>(s_q + row * ROWB + ch * 16) = w;
+    // The wavefront's k-steps of the lane's query row, as the matrix pipe takes them (a dead row: zeros).
+    u32x4 bq[KPW];
+#pragma unroll
+    for (int k4 = 0; k4 < KPW; ++k4) {
+        const int ks = k4 * 4 + wave;
+        bq[k4] = u32x4{0u, 0u, 0u, 0u};
+        if (liveq && ks < KS)
+            bq[k4] = *reinterpret_cast<const u32x4*>(a.q + ((int64_t)(start + colq) * a.q_st + (int64_t)headq * a.q_sh) * 2 + ks * 64 + g * 16);
     }
 
-    uint4 held[NL];
+    // A step's cache rows: eight threads move one row (thread t: row t / 8, its 16-byte chunks t % 8, t % 8 + 8, ...), so
+    // a thread looks up one slot a step. The page table entry is read a step ahead of the row itself, which is read a
+    // step ahead of its use: no load waits for another inside a step.
+    const int my_row = tid >> 3, my_ch = tid & 7;
+    u32x4 held[NL];
+    int entry = 0;
     float held_scale[2] = {1.0f, 1.0f};
-    auto slot_of = [&](int n) __attribute__((always_inline)) -> int64_t {
+    auto fetch_entry = [&](int base) __attribute__((always_inline)) {
+        int n = base + my_row;
         n = n < n_keys ? n : n_keys - 1;
-        int pidx = a.page_shift >= 0 ? (n >> a.page_shift) : (n / a.page);
-        pidx = pidx < a.tab_width ? pidx : a.tab_width - 1;
-        const int in_page = a.page_shift >= 0 ? (n & (a.page - 1)) : (n - (n / a.page) * a.page);
-        return (int64_t)a.tables[trow + pidx] * a.page + in_page;
+        const int pidx = (int)div32(a.page_div, (uint32_t)n);
+        entry = a.tables[trow + (pidx < a.tab_width ? pidx : a.tab_width - 1)];
     };
     auto fetch = [&](int base) __attribute__((always_inline)) {
+        int n = base + my_row;
+        n = n < n_keys ? n : n_keys - 1;
+        const int64_t slot = (int64_t)entry * a.page + (n - (int)div32(a.page_div, (uint32_t)n) * a.page);
+        const uint8_t* row = a.cache + slot * (W * EB) + my_ch * 16;
 #pragma unroll
-        for (int l = 0; l < NL; ++l) {
-            const int i = tid + l * 256;
-            if (32 * CPR % 256 == 0 || i < 32 * CPR) {
-                const int row = i / CPR, ch = i - row * CPR;
-                held[l] = *reinterpret_cast<const uint4*>(a.cache + slot_of(base + row) * (W * EB) + ch * 16);
-            }
-        }
+        for (int l = 0; l < NL; ++l)
+            if (CPR % 8 == 0 || my_ch + 8 * l < CPR) held[l] = *reinterpret_cast<const u32x4*>(row + l * 128);
         if constexpr (FP8) {
-            if (tid < 32) {
-                const float* s = a.scales + slot_of(base + tid) * a.scales_per_row;
-                held_scale[0] = s[0];
-                held_scale[1] = a.scales_per_row > 1 ? s[1] : s[0];
+            if (my_ch == 0) {
+                const float* sc = a.scales + slot * a.scales_per_row;
+                held_scale[0] = sc[0];
+                held_scale[1] = a.scales_per_row > 1 ? sc[1] : sc[0];
             }
         }
     };
     auto stage = [&]() __attribute__((always_inline)) {
+        uint8_t* row = s_k + my_row * ROWB + my_ch * (FP8 ? 32 : 16);
 #pragma unroll
         for (int l = 0; l < NL; ++l) {
-            const int i = tid + l * 256;
-            if (32 * CPR % 256 == 0 || i < 32 * CPR) {
-                const int row = i / CPR, ch = i - row * CPR;
+            if (CPR % 8 == 0 || my_ch + 8 * l < CPR) {
                 if constexpr (FP8) {      // 16 codes: 16 values of the queries' type, exactly
                     const uint32_t w[4] = {held[l].x, held[l].y, held[l].z, held[l].w};
                     uint32_t o[8];
@@ -150,16 +155,16 @@ __global__ __launch_bounds__(256, 2) void latent_kernel(LatentArgs a) {
                         const f32x2 lo = e4m3_pair<false>(w[k]), hi = e4m3_pair<true>(w[k]);
                         o[2 * k] = pair16<F16>(lo.x, lo.y), o[2 * k + 1] = pair16<F16>(hi.x, hi.y);
                     }
-                    uint4* at = reinterpret_cast<uint4*>(s_k + row * ROWB + ch * 32);
-                    at[0] = make_uint4(o[0], o[1], o[2], o[3]);
-                    at[1] = make_uint4(o[4], o[5], o[6], o[7]);
+                    u32x4* at = reinterpret_cast<u32x4*>(row + l * 256);
+                    at[0] = u32x4{o[0], o[1], o[2], o[3]};
+                    at[1] = u32x4{o[4], o[5], o[6], o[7]};
                 } else {
-                    *reinterpret_cast<uint4*>(s_k + row * ROWB + ch * 16) = held[l];
+                    *reinterpret_cast<u32x4*>(row + l * 128) = held[l];
                 }
             }
         }
         if constexpr (FP8) {
-            if (tid < 32) s_scale[tid][0] = held_scale[0], s_scale[tid][1] = held_scale[1];
+            if (my_ch == 0) s_scale[my_row][0] = held_scale[0], s_scale[my_row][1] = held_scale[1];
         }
     };
 
@@ -181,29 +186,34 @@ __global__ __launch_bounds__(256, 2) void latent_kernel(LatentArgs a) {
     for (int t = 0; t < TPW; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
     int base = base_of();      // (>= 0: b < n_pieces)
+    fetch_entry(base);
     fetch(base);
+    int next = advance();
+    if (next >= 0) fetch_entry(next);
     while (base >= 0) {
         stage();
-        __syncthreads();
-        const int next = advance();
-        if (next >= 0) fetch(next);
+        lds_barrier();
+        int after = -1;
+        if (next >= 0) {
+            fetch(next);
+            after = advance();
+            if (after >= 0) fetch_entry(after);
+        }
         // -- the step's scores: this wavefront's k-steps of both 16-position tiles
         f32x4 sl0 = {0.0f, 0.0f, 0.0f, 0.0f}, sl1 = sl0, sr0 = sl0, sr1 = sl0;
-        const uint8_t* qrow = s_q + li * ROWB + g * 16;
         const uint8_t* krow = s_k + li * ROWB + g * 16;
 #pragma unroll
-        for (int k4 = 0; k4 < (KS + 3) / 4; ++k4) {
+        for (int k4 = 0; k4 < KPW; ++k4) {
             const int ks = k4 * 4 + wave;
             if (ks < KS) {
-                const u32x4 bq = *reinterpret_cast<const u32x4*>(qrow + ks * 64);
                 const u32x4 a0 = *reinterpret_cast<const u32x4*>(krow + ks * 64);
                 const u32x4 a1 = *reinterpret_cast<const u32x4*>(krow + 16 * ROWB + ks * 64);
                 if (FP8 && ks >= KSL) {
-                    sr0 = mfma_k32<F16>(a0, bq, sr0);
-                    sr1 = mfma_k32<F16>(a1, bq, sr1);
+                    sr0 = mfma_k32<F16>(a0, bq[k4], sr0);
+                    sr1 = mfma_k32<F16>(a1, bq[k4], sr1);
                 } else {
-                    sl0 = mfma_k32<F16>(a0, bq, sl0);
-                    sl1 = mfma_k32<F16>(a1, bq, sl1);
+                    sl0 = mfma_k32<F16>(a0, bq[k4], sl0);
+                    sl1 = mfma_k32<F16>(a1, bq[k4], sl1);
                 }
             }
         }
@@ -212,7 +222,7 @@ __global__ __launch_bounds__(256, 2) void latent_kernel(LatentArgs a) {
             s_part[wave][i][lane] = sl0[i], s_part[wave][4 + i][lane] = sl1[i];
             if constexpr (FP8) s_part[wave][8 + i][lane] = sr0[i], s_part[wave][12 + i][lane] = sr1[i];
         }
-        __syncthreads();
+        lds_barrier();
         float x[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -253,8 +263,8 @@ __global__ __launch_bounds__(256, 2) void latent_kernel(LatentArgs a) {
             acc[t] *= alpha;
             acc[t] = mfma_k32<F16>(u32x4{lo.x, lo.y, hi.x, hi.y}, bp, acc[t]);
         }
-        __syncthreads();
-        base = next;
+        lds_barrier();      // (the barriers order LDS only: the next step's loads stay in flight across them)
+        base = next, next = after;
     }
     if (!liveq) return;
     const int64_t index = ((int64_t)((int64_t)r * a.columns + colq) * H + headq) * a.parts + b;
@@ -354,9 +364,7 @@ int launch_latent(const crit_pkv_latent_params* p, hipStream_t stream) {
     a.out = p->out, a.lse = p->lse, a.sinks = p->sinks;
     a.q_st = p->q_stride_t, a.q_sh = p->q_stride_h, a.o_st = p->out_stride_t, a.o_sh = p->out_stride_h, a.tab_stride = p->table_stride;
     a.tab_width = p->table_width, a.n_rows = p->n_rows, a.columns = p->columns, a.heads = p->heads, a.page = p->page;
-    a.page_shift = -1;
-    for (int s = 0; s < 31; ++s)
-        if ((1 << s) == p->page) a.page_shift = s;
+    a.page_div = make_div32((uint32_t)p->page);
     a.parts = p->partitions, a.piece = p->piece, a.scales_per_row = p->scales_per_row, a.out_dtype = p->out_dtype;
     a.sscale = p->scale * kLog2e;
     a.tiles = (p->columns * p->heads + 15) / 16;

@@ -28,7 +28,7 @@ __all__ = ["MAX_COLUMNS", "PARTIAL_BYTES", "PIECE", "SHAPES", "attend", "partiti
 
 MAX_COLUMNS = 64
 PARTIAL_BYTES = 512 << 20   # a launch's partials: rows whose partials would take more are launched a few at a time
-PIECE = 128                 # positions a piece (an order knob: one value for every launch)
+PIECE = 256                 # positions a piece (an order knob: one value for every launch)
 MAX_PARTS = 64
 SHAPES = ((512, 64), (256, 64), (128, 64), (128, 32), (64, 64), (64, 32))   # (rank, rotary width) the kernels are built for
 FP8 = torch.float8_e4m3fn
@@ -45,9 +45,10 @@ def _cus(device):
 
 
 def partitions(device, heads, rank, rope, page, kind=0):
-    """The partitions a launch over this geometry splits a row's positions into: about two workgroups a compute unit
-    for one decode token (2 x CUs over the heads' 16-row tiles), 1 to MAX_PARTS, from the heads and the device only."""
-    return max(1, min(MAX_PARTS, (2 * _cus(device)) // max(1, -(-int(heads) // 16))))
+    """The partitions a launch over this geometry splits a row's positions into: about one workgroup a compute unit
+    for one decode token (the CUs over the heads' 16-row tiles), 1 to MAX_PARTS, from the heads and the device only
+    (every partition's state is a partial the merge reads: more of them cost a batch more than they give a lone row)."""
+    return max(1, min(MAX_PARTS, _cus(device) // max(1, -(-int(heads) // 16))))
 
 
 def write(latent, rope, slots, cache, scales=None):
