@@ -13,6 +13,7 @@ index_copy append, FP32, restated in oracle/) timed on this host on a bounded sa
 """
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -550,6 +551,54 @@ def pool_bookkeeping(pk, device):
     return found
 
 
+def latent_decode(device):
+    """Latent-attention (MLA) decode at DeepSeek's geometry (rank 512, rotary 64, page 64): 64 rows of one token at
+    contexts ~U[1024, 8192], for the 16 heads a GPU of eight holds and for all 128, BF16 and E4M3 (one scale a row: a
+    KV pool's fp8:row pages) caches. Bytes: the cache rows read once (the algorithmic figure; at 128 heads the 8 tiles
+    of a row read them again from L2); flops: 2 (2 R + P) a position and head. The split launch alone (phases=1) and
+    with its merge, replayed from a captured graph."""
+    import crit_amd.latent_attention as la
+    R, P, page, B = 512, 64, 64, 64
+    lengths = torch.randint(1024, 8193, (B,), generator=torch.Generator().manual_seed(7)).tolist()
+    held = [math.ceil((n + 1) / page) for n in lengths]
+    width = (max(held) + 15) // 16 * 16
+    pages = sum(held) + 1
+    g = torch.Generator(device=device).manual_seed(21)
+    order = torch.randperm(pages - 1, device=device, generator=g).to(torch.int32)
+    tables = torch.full((B, width), pages - 1, dtype=torch.int32, device=device)
+    at = 0
+    for s, w in enumerate(held):
+        tables[s, :w] = order[at:at + w]
+        at += w
+    rows = torch.arange(B, dtype=torch.int32, device=device)
+    firsts = torch.tensor(lengths, dtype=torch.int64, device=device)
+    total = sum(n + 1 for n in lengths)
+    found = {"positions": total, "piece": la.PIECE}
+    values = torch.randn(pages, page, R + P, device=device, generator=g) * 0.5
+    for kind in ("bf16", "fp8_row_scales"):
+        if kind == "bf16":
+            cache, scales, e = values.to(torch.bfloat16), None, 2
+        else:
+            scales = (values.abs().amax(-1, keepdim=True) / 448.0).clamp(min=1e-30).contiguous()
+            cache, e = (values / scales).clamp(-448, 448).to(torch.float8_e4m3fn), 1
+        for heads in (16, 128):
+            q = (torch.randn(B, heads, R + P, device=device, generator=g) * 0.5).to(torch.bfloat16)
+            out = torch.empty(B, heads, R, dtype=torch.bfloat16, device=device)
+            call = lambda phases=0: la.attend(q, cache, tables, rows, rows, firsts, 1, page, rank=R, out=out, scales=scales,
+                                              phases=phases)
+            call()
+            split = graph_timed(lambda: call(1), 10)
+            both = graph_timed(call, 10)
+            nbytes, flops = total * (R + P) * e, total * heads * 2 * (2 * R + P)
+            found[f"{kind}_{heads}_heads"] = {
+                "partitions": la.partitions(device, heads, R, P, page), "split_us": round(split * 1e3, 1),
+                "with_merge_us": round(both * 1e3, 1), "split_GB/s": round(nbytes / split / 1e6, 1),
+                "split_frac_of_hbm_peak": round(nbytes / split / 1e6 / HBM_PEAK_GBPS, 4),
+                "split_TFLOP/s": round(flops / split / 1e9, 1),
+                "split_frac_of_bf16_mfma_peak": round(flops / split / 1e9 / 2500.0, 4)}
+    return found
+
+
 def small_batches(pk, device):
     """What a piece costs a batch that does not fill the chip: one layer's decode launch (split + merge, 8B shape) for
     4 sequences of about 2,000 positions and for one of 8,000, at the default piece and at pieces of 256 positions
@@ -675,6 +724,7 @@ def main():
                     help="run only the mixed prefill + decode batch of the extras (for counter runs on prefill_kernel)")
     ap.add_argument("--pool-only", action="store_true",
                     help="run only the pool bookkeeping of the extras (slots, the move of accepted rows, page copies)")
+    ap.add_argument("--latent-only", action="store_true", help="run only the latent-attention decode of the extras")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch one KV append of 262,144 tokens: with the stream-read probe, two kernels of known "
                          "read and write sizes against which FETCH_SIZE / WRITE_SIZE counters are scaled")
@@ -690,6 +740,11 @@ def main():
         found = mixed_prefill(pk, device)
         log(f"[bench] mixed prefill + decode: {found}")
         print(json.dumps({"mixed_prefill_decode_bf16": found}), flush=True)
+        return
+    if args.latent_only:
+        found = latent_decode(device)
+        log(f"[bench] latent-attention decode: {found}")
+        print(json.dumps({"latent_attention_decode": found}), flush=True)
         return
     if args.pool_only:
         found = pool_bookkeeping(pk, device)
@@ -811,6 +866,9 @@ def main():
         log(f"[bench] a small batch's decode step, eager and from one graph: {extras['captured_decode_step_bf16']}")
         extras["pool_bookkeeping_bf16"] = pool_bookkeeping(pk, device)
         log(f"[bench] pool bookkeeping: {extras['pool_bookkeeping_bf16']}")
+        torch.cuda.empty_cache()
+        extras["latent_attention_decode"] = latent_decode(device)
+        log(f"[bench] latent-attention decode: {extras['latent_attention_decode']}")
         result["extra"] = extras
     if not args.no_cpu:
         log("[bench] timing the CPU reference path (about 20 s)")
