@@ -60,57 +60,68 @@ PKV_DEV u32x2 lds_transposed(const uint8_t* p) {
     return __builtin_bit_cast(u32x2, v);
 }
 
-template <int R, int P, bool F16, bool FP8>
-__global__ __launch_bounds__(256, 3) void latent_kernel(LatentArgs a) {
+// NT: query tiles (of 16 rows) a workgroup serves over one staging of the cache rows: 1 where a row's columns times
+// heads fit one tile, else 2 (each tile is then two wavefronts' work: the staging, the barriers and half of the softmax
+// are shared by twice the rows). A tile's score is the sum of four chains of k-steps (chain c: k-steps c, c + 4, ...)
+// added as ((0 + 1) + 2) + 3 whichever wavefront computed them, so a row's bits do not depend on NT.
+template <int R, int P, bool F16, bool FP8, int NT>
+__global__ __launch_bounds__(256, NT == 1 ? 3 : 2) void latent_kernel(LatentArgs a) {
     constexpr int W = R + P;                   // values a cache row holds
     constexpr int ROWB = W * 2 + 32;           // bytes between rows in LDS: 32 mod 64 words apart, so that 16 rows' 32-byte
                                                // reads fall on different banks
     constexpr int KS = W / 32, KSL = R / 32;   // k-steps of the scores; the first KSL are the latent's
-    constexpr int TPW = R / 64;                // 16-value output tiles a wavefront owns
+    constexpr int WPT = 4 / NT;                // wavefronts a query tile
+    constexpr int FT = (R / 16) / WPT;         // 16-value output tiles a wavefront owns
     constexpr int EB = FP8 ? 1 : 2;
     constexpr int CPR = W * EB / 16;           // 16-byte chunks of a cache row
     constexpr int NL = (CPR + 7) / 8;          // chunks a thread moves a step
-    constexpr int KPW = (KS + 3) / 4;          // k-steps a wavefront takes
+    constexpr int KPC = (KS + 3) / 4;          // k-steps a chain holds
     constexpr int NPART = FP8 ? 16 : 8;        // floats a lane's partial score tiles take (latent and rotary apart for E4M3)
     __shared__ __align__(16) uint8_t s_k[32 * ROWB];
-    __shared__ float s_part[4][NPART][64];
+    __shared__ float s_part[NT][4][NPART][64];
     __shared__ float s_scale[FP8 ? 32 : 1][2];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 4, li = lane & 15;
-    // Workgroups go to the XCDs in turn: the tiles of one (row, partition) take consecutive places of one XCD.
+    const int wt = wave / WPT, sub = wave % WPT;      // the wavefront's tile of the workgroup's, and its place among that tile's
+    // Workgroups go to the XCDs in turn: the tile groups of one (row, partition) take consecutive places of one XCD.
     const int64_t bid = blockIdx.x;
     const int64_t place = bid >> 3;
     const int64_t pair = (place / a.tiles) * 8 + (bid & 7);
-    const int tile = (int)(place % a.tiles);
+    const int group = (int)(place % a.tiles);
     if (pair >= a.pairs) return;
     const int r = (int)(pair / a.gy), b = (int)(pair % a.gy);
     int count = a.columns;
     if (a.counts) count = min(a.counts[r], a.columns);
     const int H = a.heads;
-    const int j0 = tile * 16;
-    if (j0 >= count * H) return;
+    const int live_rows = count * H;
+    if (group * NT * 16 >= live_rows) return;
     const int64_t first64 = a.firsts[r];
     const int first = (int)(first64 < 0 ? 0 : (first64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first64));
-    const int c_hi = min(count, (j0 + 15) / H + 1);
+    const int c_hi = (min((group + 1) * NT * 16, live_rows) - 1) / H + 1;      // columns the group's rows reach
     const int n_keys = min(first + c_hi, a.max_keys);
     const int n_pieces = (n_keys + a.piece - 1) / a.piece;
     if (b >= n_pieces) return;
     const int64_t trow = (int64_t)a.rows[(int64_t)r * a.rows_step] * a.tab_stride;
     const int start = a.starts[r];
 
-    // The lane's query row (column li of the score tiles).
+    // The lane's query row (column li of its wavefront's score tiles).
+    const int j0 = (group * NT + wt) * 16;
     const int jq = j0 + li, colq = jq / H, headq = jq - colq * H;
     const bool liveq = colq < count;
     const int lim = liveq ? first + colq : -1;
+    const int unmasked = min(first + j0 / H + 1, n_keys);      // positions below it are seen by every live row of the tile
 
-    // The wavefront's k-steps of the lane's query row, as the matrix pipe takes them (a dead row: zeros).
-    u32x4 bq[KPW];
+    // The wavefront's chains of the lane's query row, as the matrix pipe takes them (a dead row: zeros).
+    u32x4 bq[NT][KPC];
 #pragma unroll
-    for (int k4 = 0; k4 < KPW; ++k4) {
-        const int ks = k4 * 4 + wave;
-        bq[k4] = u32x4{0u, 0u, 0u, 0u};
-        if (liveq && ks < KS)
-            bq[k4] = *reinterpret_cast<const u32x4*>(a.q + ((int64_t)(start + colq) * a.q_st + (int64_t)headq * a.q_sh) * 2 + ks * 64 + g * 16);
+    for (int c = 0; c < NT; ++c) {
+#pragma unroll
+        for (int k4 = 0; k4 < KPC; ++k4) {
+            const int ks = k4 * 4 + sub + c * WPT;
+            bq[c][k4] = u32x4{0u, 0u, 0u, 0u};
+            if (liveq && ks < KS)
+                bq[c][k4] = *reinterpret_cast<const u32x4*>(a.q + ((int64_t)(start + colq) * a.q_st + (int64_t)headq * a.q_sh) * 2 + ks * 64 + g * 16);
+        }
     }
 
     // A step's cache rows: eight threads move one row (thread t: row t / 8, its 16-byte chunks t % 8, t % 8 + 8, ...), so
@@ -168,7 +179,7 @@ __global__ __launch_bounds__(256, 3) void latent_kernel(LatentArgs a) {
         }
     };
 
-    // The wavefront's steps are the unit's: steps 0 .. of pieces b, b + parts, ...
+    // The workgroup's steps: steps 0 .. of pieces b, b + parts, ...
     const int steps_per_piece = a.piece / 32;
     int pi = b, st = 0;
     auto base_of = [&]() __attribute__((always_inline)) -> int {
@@ -181,9 +192,9 @@ __global__ __launch_bounds__(256, 3) void latent_kernel(LatentArgs a) {
     };
 
     float m = -INFINITY, l = 0.0f;
-    f32x4 acc[TPW];
+    f32x4 acc[FT];
 #pragma unroll
-    for (int t = 0; t < TPW; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int t = 0; t < FT; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
     int base = base_of();      // (>= 0: b < n_pieces)
     fetch_entry(base);
@@ -199,52 +210,60 @@ __global__ __launch_bounds__(256, 3) void latent_kernel(LatentArgs a) {
             after = advance();
             if (after >= 0) fetch_entry(after);
         }
-        // -- the step's scores: this wavefront's k-steps of both 16-position tiles
-        f32x4 sl0 = {0.0f, 0.0f, 0.0f, 0.0f}, sl1 = sl0, sr0 = sl0, sr1 = sl0;
+        // -- the step's scores: this wavefront's chains of its tile, both 16-position halves of the step
         const uint8_t* krow = s_k + li * ROWB + g * 16;
 #pragma unroll
-        for (int k4 = 0; k4 < KPW; ++k4) {
-            const int ks = k4 * 4 + wave;
-            if (ks < KS) {
-                const u32x4 a0 = *reinterpret_cast<const u32x4*>(krow + ks * 64);
-                const u32x4 a1 = *reinterpret_cast<const u32x4*>(krow + 16 * ROWB + ks * 64);
-                if (FP8 && ks >= KSL) {
-                    sr0 = mfma_k32<F16>(a0, bq[k4], sr0);
-                    sr1 = mfma_k32<F16>(a1, bq[k4], sr1);
-                } else {
-                    sl0 = mfma_k32<F16>(a0, bq[k4], sl0);
-                    sl1 = mfma_k32<F16>(a1, bq[k4], sl1);
+        for (int c = 0; c < NT; ++c) {
+            f32x4 sl0 = {0.0f, 0.0f, 0.0f, 0.0f}, sl1 = sl0, sr0 = sl0, sr1 = sl0;
+#pragma unroll
+            for (int k4 = 0; k4 < KPC; ++k4) {
+                const int ks = k4 * 4 + sub + c * WPT;
+                if (ks < KS) {
+                    const u32x4 a0 = *reinterpret_cast<const u32x4*>(krow + ks * 64);
+                    const u32x4 a1 = *reinterpret_cast<const u32x4*>(krow + 16 * ROWB + ks * 64);
+                    if (FP8 && ks >= KSL) {
+                        sr0 = mfma_k32<F16>(a0, bq[c][k4], sr0);
+                        sr1 = mfma_k32<F16>(a1, bq[c][k4], sr1);
+                    } else {
+                        sl0 = mfma_k32<F16>(a0, bq[c][k4], sl0);
+                        sl1 = mfma_k32<F16>(a1, bq[c][k4], sl1);
+                    }
                 }
             }
-        }
+            float (&mine)[NPART][64] = s_part[wt][sub + c * WPT];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            s_part[wave][i][lane] = sl0[i], s_part[wave][4 + i][lane] = sl1[i];
-            if constexpr (FP8) s_part[wave][8 + i][lane] = sr0[i], s_part[wave][12 + i][lane] = sr1[i];
+            for (int i = 0; i < 4; ++i) {
+                mine[i][lane] = sl0[i], mine[4 + i][lane] = sl1[i];
+                if constexpr (FP8) mine[8 + i][lane] = sr0[i], mine[12 + i][lane] = sr1[i];
+            }
         }
         lds_barrier();
         float x[8];
+        const bool masked = base + 32 > unmasked;      // (the same for the whole wavefront)
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            const float latent = ((s_part[0][e][lane] + s_part[1][e][lane]) + s_part[2][e][lane]) + s_part[3][e][lane];
+            const float latent = ((s_part[wt][0][e][lane] + s_part[wt][1][e][lane]) + s_part[wt][2][e][lane]) + s_part[wt][3][e][lane];
             const int at = (e >> 2) * 16 + 4 * g + (e & 3);      // the value's position in the step
             float v = latent;
             if constexpr (FP8) {
-                const float rotary = ((s_part[0][8 + e][lane] + s_part[1][8 + e][lane]) + s_part[2][8 + e][lane]) + s_part[3][8 + e][lane];
+                const float rotary = ((s_part[wt][0][8 + e][lane] + s_part[wt][1][8 + e][lane]) + s_part[wt][2][8 + e][lane]) + s_part[wt][3][8 + e][lane];
                 v = __builtin_fmaf(latent, s_scale[at][0], rotary * s_scale[at][1]);
             }
-            const int n = base + at;
-            x[e] = (n <= lim && n < n_keys) ? v * a.sscale : -INFINITY;
+            x[e] = v * a.sscale;
+            if (masked) {
+                const int n = base + at;
+                x[e] = (n <= lim && n < n_keys) ? x[e] : -INFINITY;
+            }
         }
         float top = __builtin_fmaxf(__builtin_fmaxf(__builtin_fmaxf(x[0], x[1]), __builtin_fmaxf(x[2], x[3])),
                                     __builtin_fmaxf(__builtin_fmaxf(x[4], x[5]), __builtin_fmaxf(x[6], x[7])));
         top = max_across_quarters(top);
         const float m_new = __builtin_fmaxf(m, top);
-        const float sub = m_new == -INFINITY ? 0.0f : m_new;
-        const float alpha = exp2_fast(m - sub);
+        const float sub2 = m_new == -INFINITY ? 0.0f : m_new;
+        const float alpha = exp2_fast(m - sub2);
         float p[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) p[e] = exp2_fast(x[e] - sub);
+        for (int e = 0; e < 8; ++e) p[e] = exp2_fast(x[e] - sub2);
         const float sum = sum_across_quarters(((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7])));
         l = __builtin_fmaf(l, alpha, sum);
         m = m_new;
@@ -253,14 +272,15 @@ __global__ __launch_bounds__(256, 3) void latent_kernel(LatentArgs a) {
             for (int e = 0; e < 8; ++e) p[e] *= s_scale[(e >> 2) * 16 + 4 * g + (e & 3)][0];
         }
         const u32x4 bp = {pair16<F16>(p[0], p[1]), pair16<F16>(p[2], p[3]), pair16<F16>(p[4], p[5]), pair16<F16>(p[6], p[7])};
-        // -- the wavefront's quarter of the values
+        // -- the wavefront's share of the values (the accumulators move only when some row's maximum did: x 1 is exact)
+        const bool rescale = __ballot(alpha != 1.0f) != 0ull;
         const uint8_t* vrow = s_k + (4 * g + (li >> 2)) * ROWB + (li & 3) * 8;
 #pragma unroll
-        for (int t = 0; t < TPW; ++t) {
-            const int ftile = wave * TPW + t;
+        for (int t = 0; t < FT; ++t) {
+            const int ftile = sub * FT + t;
             const u32x2 lo = lds_transposed(vrow + ftile * 32);
             const u32x2 hi = lds_transposed(vrow + 16 * ROWB + ftile * 32);
-            acc[t] *= alpha;
+            if (rescale) acc[t] *= alpha;
             acc[t] = mfma_k32<F16>(u32x4{lo.x, lo.y, hi.x, hi.y}, bp, acc[t]);
         }
         lds_barrier();      // (the barriers order LDS only: the next step's loads stay in flight across them)
@@ -269,9 +289,9 @@ __global__ __launch_bounds__(256, 3) void latent_kernel(LatentArgs a) {
     if (!liveq) return;
     const int64_t index = ((int64_t)((int64_t)r * a.columns + colq) * H + headq) * a.parts + b;
 #pragma unroll
-    for (int t = 0; t < TPW; ++t)
-        *reinterpret_cast<f32x4*>(a.po + index * R + (wave * TPW + t) * 16 + 4 * g) = acc[t];
-    if (wave == 0 && g == 0) a.pm[index] = m, a.pl[index] = l;
+    for (int t = 0; t < FT; ++t)
+        *reinterpret_cast<f32x4*>(a.po + index * R + (sub * FT + t) * 16 + 4 * g) = acc[t];
+    if (sub == 0 && g == 0) a.pm[index] = m, a.pl[index] = l;
 }
 
 // One workgroup of 64 threads a (batch row, column, head): the partitions' states folded in partition order, the sink
@@ -317,20 +337,30 @@ __global__ __launch_bounds__(64) void latent_merge_kernel(LatentArgs a) {
     if (a.lse && threadIdx.x == 0) a.lse[token * a.heads + head] = L > 0.0f ? (M + __builtin_log2f(L)) * kLn2 : -INFINITY;
 }
 
-template <int R, int P>
-int launch_shape(const LatentArgs& a, bool f16, bool fp8, int phases, hipStream_t stream) {
+template <int R, int P, int NT>
+int launch_tiles(const LatentArgs& a, bool f16, bool fp8, hipStream_t stream) {
     const int64_t blocks = (a.pairs + 7) / 8 * 8 * a.tiles;
     if (blocks > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
+    const dim3 grid((unsigned)blocks);
+    if (fp8) {
+        if (f16) hipLaunchKernelGGL((latent_kernel<R, P, true, true, NT>), grid, dim3(256), 0, stream, a);
+        else hipLaunchKernelGGL((latent_kernel<R, P, false, true, NT>), grid, dim3(256), 0, stream, a);
+    } else {
+        if (f16) hipLaunchKernelGGL((latent_kernel<R, P, true, false, NT>), grid, dim3(256), 0, stream, a);
+        else hipLaunchKernelGGL((latent_kernel<R, P, false, false, NT>), grid, dim3(256), 0, stream, a);
+    }
+    return hip_code(hipGetLastError());
+}
+
+template <int R, int P>
+int launch_shape(const LatentArgs& a, bool f16, bool fp8, int phases, hipStream_t stream) {
     if (phases != 2) {
-        const dim3 grid((unsigned)blocks);
-        if (fp8) {
-            if (f16) hipLaunchKernelGGL((latent_kernel<R, P, true, true>), grid, dim3(256), 0, stream, a);
-            else hipLaunchKernelGGL((latent_kernel<R, P, false, true>), grid, dim3(256), 0, stream, a);
-        } else {
-            if (f16) hipLaunchKernelGGL((latent_kernel<R, P, true, false>), grid, dim3(256), 0, stream, a);
-            else hipLaunchKernelGGL((latent_kernel<R, P, false, false>), grid, dim3(256), 0, stream, a);
-        }
-        if (const hipError_t e = hipGetLastError()) return (int)e;
+        // (a launch whose rows fit one tile each takes the one-tile workgroups: three a compute unit)
+        LatentArgs u = a;
+        const int tiles = (a.columns * a.heads + 15) / 16;
+        u.tiles = tiles > 1 ? (tiles + 1) / 2 : 1;
+        const int bad = tiles > 1 ? launch_tiles<R, P, 2>(u, f16, fp8, stream) : launch_tiles<R, P, 1>(u, f16, fp8, stream);
+        if (bad) return bad;
     }
     if (phases != 1) {
         hipLaunchKernelGGL((latent_merge_kernel<R>), dim3((unsigned)(a.n_rows * a.columns), (unsigned)a.heads), dim3(64), 0, stream, a);
