@@ -39,6 +39,14 @@ int crit_pkv_latent_attend(const crit_pkv_latent_params* p, void* stream) {
     return pkv::launch_latent(p, reinterpret_cast<hipStream_t>(stream));
 }
 
+int crit_pkv_index_scores(const crit_pkv_index_scores_params* p, void* stream) {
+    return pkv::launch_index_scores(p, reinterpret_cast<hipStream_t>(stream));
+}
+
+int crit_pkv_index_topk(const crit_pkv_index_topk_params* p, void* stream) {
+    return pkv::launch_index_topk(p, reinterpret_cast<hipStream_t>(stream));
+}
+
 int crit_pkv_round(const crit_pkv_round_params* p, void* stream) {
     return pkv::launch_round(p, reinterpret_cast<hipStream_t>(stream));
 }
@@ -80,6 +88,8 @@ int crit_pkv_params_size(int which) {
         case 8: return (int)sizeof(crit_pkv_round_params);
         case 9: return (int)sizeof(crit_pkv_step_params);
         case 10: return (int)sizeof(crit_pkv_latent_params);
+        case 11: return (int)sizeof(crit_pkv_index_scores_params);
+        case 12: return (int)sizeof(crit_pkv_index_topk_params);
     }
     return -1;
 }

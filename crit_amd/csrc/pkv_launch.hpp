@@ -16,6 +16,8 @@ int launch_copy_pages(const crit_pkv_copy_pages_params* p, hipStream_t stream);
 int launch_round(const crit_pkv_round_params* p, hipStream_t stream);
 int launch_step_buffers(const crit_pkv_step_params* p, hipStream_t stream);
 int launch_latent(const crit_pkv_latent_params* p, hipStream_t stream);
+int launch_index_scores(const crit_pkv_index_scores_params* p, hipStream_t stream);
+int launch_index_topk(const crit_pkv_index_topk_params* p, hipStream_t stream);
 int launch_read_rows(const crit_pkv_read_params* p, hipStream_t stream);
 int launch_stream_read(const void* data, int64_t bytes, float* sink, hipStream_t stream);
 // Compute units of the current device (cached per device), or 0 if the query fails.

@@ -10,7 +10,7 @@ import shutil
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 NAME = "libcrit_pkv.so"
-ABI_VERSION = 16
+ABI_VERSION = 17
 
 KIND_16BIT, KIND_FP8, KIND_FP8_ROW, KIND_INT8 = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
@@ -115,6 +115,19 @@ class LatentParams(ctypes.Structure):
                 ("partitions", _i32), ("piece", _i32), ("rows_are_64", _i32), ("phases", _i32), ("scale", _f32)]
 
 
+class IndexScoresParams(ctypes.Structure):
+    _fields_ = [("q", _p), ("keys", _p), ("key_scales", _p), ("weights", _p), ("ends", _p), ("slots", _p), ("out", _p),
+                ("q_stride_t", _i64), ("q_stride_h", _i64), ("key_stride", _i64), ("weights_stride", _i64),
+                ("out_stride", _i64), ("slots_stride", _i64),
+                ("tokens", _i32), ("n", _i32), ("group", _i32), ("heads", _i32), ("dim", _i32), ("key_dtype", _i32),
+                ("q_dtype", _i32), ("slots_are_64", _i32), ("scale", _f32)]
+
+
+class IndexTopkParams(ctypes.Structure):
+    _fields_ = [("scores", _p), ("ends", _p), ("out", _p), ("scores_stride", _i64), ("out_stride", _i64),
+                ("tokens", _i32), ("n", _i32), ("k", _i32)]
+
+
 class ReadParams(ctypes.Structure):
     _fields_ = [("key_pages", _p), ("value_pages", _p), ("key_scales", _p), ("value_scales", _p), ("head_multipliers", _p),
                 ("slots", _p), ("table", _p), ("table64", _p), ("out_keys", _p), ("out_values", _p), ("n", _i64), ("pool_slots", _i64),
@@ -125,7 +138,7 @@ class ReadParams(ctypes.Structure):
 STATIC_SCRATCH_BYTES = 32 << 20
 
 SYMBOLS = ("crit_pkv_write", "crit_pkv_attend", "crit_pkv_attend_static", "crit_pkv_merge", "crit_pkv_prefill", "crit_pkv_slots_at",
-           "crit_pkv_compact", "crit_pkv_copy_pages", "crit_pkv_round", "crit_pkv_step_buffers", "crit_pkv_latent_attend", "crit_pkv_read_rows", "crit_pkv_abi_version", "crit_pkv_params_size", "crit_pkv_error",
+           "crit_pkv_compact", "crit_pkv_copy_pages", "crit_pkv_round", "crit_pkv_step_buffers", "crit_pkv_latent_attend", "crit_pkv_index_scores", "crit_pkv_index_topk", "crit_pkv_read_rows", "crit_pkv_abi_version", "crit_pkv_params_size", "crit_pkv_error",
            "crit_pkv_stream_read", "crit_pkv_stream_capture")
 
 _lib = None
@@ -176,6 +189,7 @@ def load():
                          ("crit_pkv_slots_at", SlotsParams), ("crit_pkv_compact", CompactParams),
                          ("crit_pkv_copy_pages", CopyPagesParams), ("crit_pkv_round", RoundParams),
                          ("crit_pkv_step_buffers", StepParams), ("crit_pkv_latent_attend", LatentParams),
+                         ("crit_pkv_index_scores", IndexScoresParams), ("crit_pkv_index_topk", IndexTopkParams),
                          ("crit_pkv_read_rows", ReadParams)):
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
@@ -187,7 +201,8 @@ def load():
     if lib.crit_pkv_abi_version() != ABI_VERSION:
         raise RuntimeError(f"{path} speaks ABI {lib.crit_pkv_abi_version()}, this package {ABI_VERSION}: rebuild it")
     for which, struct in enumerate((WriteParams, AttendParams, MergeParams, PrefillParams, SlotsParams, CompactParams,
-                                    CopyPagesParams, ReadParams, RoundParams, StepParams, LatentParams)):
+                                    CopyPagesParams, ReadParams, RoundParams, StepParams, LatentParams,
+                                    IndexScoresParams, IndexTopkParams)):
         if lib.crit_pkv_params_size(which) != ctypes.sizeof(struct):
             raise RuntimeError(f"{path}: parameter struct {which} is {lib.crit_pkv_params_size(which)} bytes, the "
                                f"Python mirror {ctypes.sizeof(struct)}: rebuild the library")

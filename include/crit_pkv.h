@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 16
+#define CRIT_PKV_ABI_VERSION 17
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -428,6 +428,45 @@ typedef struct crit_pkv_latent_params {
 
 int crit_pkv_latent_attend(const crit_pkv_latent_params* p, void* stream);
 
+/* ---- sparse index selection ---------------------------------------------------------------------------------------
+ * Replaces scores() and topk() of crit's sparse-indexer kernels module (kernels/techniques/attention/sparse-indexer/
+ * torch-ext/sparse_indexer/__init__.py:83-139 and its score_kernel / topk_kernel / cuda_select.cu; the operation:
+ * inference/attention-state/code/sparse_index.py): for each query token a score over every compressed key it may see,
+ *   out[t][s] = sum_h weights[t][h] * scale * max(0, q[t][h] . keys[s])   for s < ends[t], -inf at or past it,
+ * 16-bit products on the matrix pipe with FP32 sums, ReLU, the head's factor and the sum over the heads (a fixed tree)
+ * in FP32. q [tokens][heads][dim] BF16 or FP16 (heads up to 128, dim 64, 128 or 256); keys [rows][dim] in q's type
+ * (key_dtype 0 BF16, 1 FP16) or E4M3 codes (2) with key_scales FP32 [rows], a key's value its code times its scale;
+ * key_stride in elements. slots (optional, int32 or int64 [groups][n], slots_stride apart): key j of token t is row
+ * slots[t / group][j] of keys (keys read in place where a pool stores them; group = tokens a group); without slots key
+ * j is row j. A token's bits are its own. */
+typedef struct crit_pkv_index_scores_params {
+    const void* q;
+    const void* keys;
+    const float* key_scales;        /* E4M3 keys */
+    const float* weights;           /* [tokens][weights_stride >= heads] */
+    const int32_t* ends;            /* [tokens] */
+    const void* slots;              /* optional */
+    float* out;                     /* [tokens][out_stride >= n] */
+    int64_t q_stride_t, q_stride_h, key_stride, weights_stride, out_stride, slots_stride;
+    int32_t tokens, n, group, heads, dim, key_dtype, q_dtype, slots_are_64;
+    float scale;
+} crit_pkv_index_scores_params;
+
+int crit_pkv_index_scores(const crit_pkv_index_scores_params* p, void* stream);
+
+/* out[t][0 .. k - 1] (int32) = the positions of token t's k largest scores below ends[t], ascending, then -1 (all of
+ * them where ends[t] <= k): ties to the lower position, -0 = +0, a NaN below every number (sparse_index.py:24-40). One
+ * launch, a workgroup a token: an 8-bit radix select for the k-th score, then one pass in position order. */
+typedef struct crit_pkv_index_topk_params {
+    const float* scores;            /* [tokens][scores_stride >= n] */
+    const int32_t* ends;
+    int32_t* out;                   /* [tokens][out_stride >= k] */
+    int64_t scores_stride, out_stride;
+    int32_t tokens, n, k;
+} crit_pkv_index_topk_params;
+
+int crit_pkv_index_topk(const crit_pkv_index_topk_params* p, void* stream);
+
 /* ---- rows read back ----------------------------------------------------------------------------------------------
  * Replaces the index_select, cast and multiply of KVPool.gather and KVPool.rows_at (pages.py:455-493): row i of the
  * output is the pool's row at slots[i], or, with a page table instead (exactly one of slots, table, table64), at
@@ -458,7 +497,7 @@ int crit_pkv_read_rows(const crit_pkv_read_params* p, void* stream);
 /* ---- housekeeping ------------------------------------------------------------------------------------------------- */
 int crit_pkv_abi_version(void);
 /* sizeof() of the parameter structs as the library was compiled, for the host's mirror to cross-check
- * (which: 0 write, 1 attend, 2 merge, 3 prefill, 4 slots_at, 5 compact, 6 copy_pages, 7 read_rows, 8 round, 9 step_buffers, 10 latent_attend), as crit_cw_params_size() does (cuda_window.cu:1502). */
+ * (which: 0 write, 1 attend, 2 merge, 3 prefill, 4 slots_at, 5 compact, 6 copy_pages, 7 read_rows, 8 round, 9 step_buffers, 10 latent_attend, 11 index_scores, 12 index_topk), as crit_cw_params_size() does (cuda_window.cu:1502). */
 int crit_pkv_params_size(int which);
 const char* crit_pkv_error(int code);
 /* *id = the id of the capture `stream` is recording into (never 0), or 0 when it is not capturing; returns 0 or a HIP

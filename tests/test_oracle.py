@@ -949,3 +949,87 @@ def test_rms_norm_rope_normalises_weighs_and_turns(style):
     gb16 = append.rms_norm_rope(xb, weight, eps, positions, table, offset, style)
     assert gb16.dtype == torch.bfloat16
     assert torch.equal(gb16, append.rms_norm_rope(xb.float(), weight, eps, positions, table, offset, style).bfloat16())
+
+
+# -- sparse index selection ---------------------------------------------------------------------------------------------
+def test_sparse_scores_are_the_sum_written_out_term_by_term():
+    from oracle import indexer
+    rng = np.random.default_rng(5)
+    t, h, d, n = 3, 4, 5, 7
+    q, keys, w = rng.standard_normal((t, h, d)), rng.standard_normal((n, d)), rng.standard_normal((t, h))
+    ends = np.array([7, 3, 0])
+    got = indexer.sparse_scores(q, keys, w, ends, 0.37)
+    for i in range(t):
+        for s in range(n):
+            if s >= ends[i]:
+                assert got[i, s] == -math.inf
+                continue
+            total = 0.0
+            for j in range(h):
+                dot = sum(float(q[i, j, c]) * float(keys[s, c]) for c in range(d))
+                total += float(w[i, j]) * 0.37 * max(0.0, dot)
+            assert abs(got[i, s] - total) <= 1e-12 * max(1.0, abs(total))
+
+
+def test_sparse_scores_closed_forms_one_hot_queries_relus_sign_and_linear_weights():
+    from oracle import indexer
+    rng = np.random.default_rng(6)
+    keys = rng.standard_normal((9, 4))
+    q = np.zeros((1, 2, 4))
+    q[0, 0, 1], q[0, 1, 3] = 1.0, -1.0      # head 0 reads component 1, head 1 minus component 3
+    w = np.array([[2.0, 3.0]])
+    got = indexer.sparse_scores(q, keys, w, [9], 0.5)[0]
+    want = 2.0 * 0.5 * np.maximum(keys[:, 1], 0.0) + 3.0 * 0.5 * np.maximum(-keys[:, 3], 0.0)
+    assert np.allclose(got, want, rtol=0, atol=1e-15)
+    # a transposed operand or a ReLU after the head sum would fail these: heads that cancel before the ReLU do not after
+    q2 = np.stack([np.ones((1, 4)), -np.ones((1, 4))], 1)      # two opposite heads
+    both = indexer.sparse_scores(q2, keys, np.ones((1, 2)), [9], 1.0)[0]
+    assert np.allclose(both, np.abs(keys.sum(1)), atol=1e-14)
+    a, b = rng.standard_normal((1, 2)), rng.standard_normal((1, 2))
+    qq = rng.standard_normal((1, 2, 4))
+    lin = indexer.sparse_scores(qq, keys, 2 * a - 3 * b, [9], 0.25)
+    assert np.allclose(lin, 2 * indexer.sparse_scores(qq, keys, a, [9], 0.25) - 3 * indexer.sparse_scores(qq, keys, b, [9], 0.25))
+
+
+def _select_by_taking_the_best(row, end, k):
+    """The rule without a sort: k times, the best remaining score (a number beats a NaN, the larger number wins, the
+    lower position on a tie)."""
+    left = list(range(end))
+    if end <= k:
+        return left
+    taken = []
+    for _ in range(k):
+        best = None
+        for at in left:
+            x = row[at]
+            if best is None:
+                best = at
+                continue
+            y = row[best]
+            if (y != y and x == x) or (x == x and y == y and x > y):
+                best = at
+        taken.append(best)
+        left.remove(best)
+    return sorted(taken)
+
+
+def test_sparse_index_takes_the_best_remaining_score_k_times_and_holds_the_references_known_answers():
+    from oracle import indexer
+    nan, inf = float("nan"), float("inf")
+    s = np.array([[1.0, nan, -inf, 2.0, nan]])
+    assert indexer.sparse_index(s, [5], 4).tolist() == [[0, 1, 2, 3]]      # 2, 1, -inf, then the first NaN
+    assert indexer.sparse_index(s, [5], 3).tolist() == [[0, 2, 3]]
+    assert indexer.sparse_index(s, [2], 4).tolist() == [[0, 1, -1, -1]]    # fewer valid keys than k: all of them
+    assert indexer.sparse_index(s, [0], 2).tolist() == [[-1, -1]]
+    assert indexer.sparse_index(np.array([[0.0, -0.0, 0.0, -0.0]]), [4], 2).tolist() == [[0, 1]]      # the zeros tie
+    rng = np.random.default_rng(8)
+    for case in range(40):
+        n, k = int(rng.integers(1, 40)), int(rng.integers(1, 12))
+        row = np.round(rng.standard_normal(n) * 2) / 2      # many ties
+        row[rng.integers(0, n, n // 5)] = nan
+        row[rng.integers(0, n, n // 7)] = -inf
+        row[rng.integers(0, n, n // 9)] = -0.0
+        end = int(rng.integers(0, n + 1))
+        got = indexer.sparse_index(row[None], [end], k)[0]
+        want = _select_by_taking_the_best(row, end, k)
+        assert got[:len(want)].tolist() == want and (got[len(want):] == -1).all(), case
