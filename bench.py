@@ -603,6 +603,37 @@ def latent_decode(device):
     return found
 
 
+def index_selection(device):
+    """Sparse index selection at DeepSeek-V3.2's indexer geometry (64 heads of 128, the 2,048 best keys): scores and
+    top-k over 8,192 and 50,000 keys for 1, 4, 256 and 2,048 tokens near the end of the keys, BF16 and E4M3 keys, each
+    call replayed from a captured graph. Scores: 2 H D flops a token and key on the matrix pipe; top-k: a token's scores
+    read five times (4 digit passes and the ordered pass), from L2 after the first."""
+    import crit_amd.sparse_indexer as si
+    H, D, K = 64, 128, 2048
+    g = torch.Generator(device=device).manual_seed(17)
+    found = {"heads": H, "dim": D, "k": K}
+    for n in (8192, 50000):
+        keys = (torch.randn(n, D, device=device, generator=g) * 0.5).to(torch.bfloat16)
+        key_scales = (keys.float().abs().amax(1) / 448.0).clamp_min(1e-30)
+        codes = (keys.float() / key_scales[:, None]).to(torch.float8_e4m3fn)
+        for tokens in (1, 4, 256, 2048):
+            q = (torch.randn(tokens, H, D, device=device, generator=g) * 0.5).to(torch.bfloat16)
+            w = torch.randn(tokens, H, device=device, generator=g) * H ** -0.5
+            ends = (n - torch.randint(0, 64, (tokens,), device=device, generator=g)).to(torch.int32)
+            s = torch.empty(tokens, n, dtype=torch.float32, device=device)
+            picked = torch.empty(tokens, K, dtype=torch.int32, device=device)
+            launches = 20 if tokens <= 4 else 3
+            bf16 = graph_timed(lambda: si.scores(q, keys, w, ends, out=s), launches)
+            fp8 = graph_timed(lambda: si.scores(q, codes, w, ends, key_scales=key_scales, out=s), launches)
+            top = graph_timed(lambda: si.topk(s, ends, K, out=picked), launches)
+            flops = 2.0 * tokens * n * H * D
+            found[f"{n}_keys_{tokens}_tokens"] = {
+                "scores_bf16_us": round(bf16 * 1e3, 1), "scores_e4m3_us": round(fp8 * 1e3, 1),
+                "scores_bf16_TFLOP/s": round(flops / bf16 / 1e9, 1), "topk_us": round(top * 1e3, 1),
+                "topk_GB/s_of_scores_read_once": round(tokens * n * 4 / top / 1e6, 1)}
+    return found
+
+
 def small_batches(pk, device):
     """What a piece costs a batch that does not fill the chip: one layer's decode launch (split + merge, 8B shape) for
     4 sequences of about 2,000 positions and for one of 8,000, at the default piece and at pieces of 256 positions
@@ -729,6 +760,7 @@ def main():
     ap.add_argument("--pool-only", action="store_true",
                     help="run only the pool bookkeeping of the extras (slots, the move of accepted rows, page copies)")
     ap.add_argument("--latent-only", action="store_true", help="run only the latent-attention decode of the extras")
+    ap.add_argument("--index-only", action="store_true", help="run only the sparse index selection of the extras")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch one KV append of 262,144 tokens: with the stream-read probe, two kernels of known "
                          "read and write sizes against which FETCH_SIZE / WRITE_SIZE counters are scaled")
@@ -749,6 +781,11 @@ def main():
         found = latent_decode(device)
         log(f"[bench] latent-attention decode: {found}")
         print(json.dumps({"latent_attention_decode": found}), flush=True)
+        return
+    if args.index_only:
+        found = index_selection(device)
+        log(f"[bench] sparse index selection: {found}")
+        print(json.dumps({"sparse_index_selection": found}), flush=True)
         return
     if args.pool_only:
         found = pool_bookkeeping(pk, device)
@@ -872,6 +909,7 @@ def main():
         log(f"[bench] pool bookkeeping: {extras['pool_bookkeeping_bf16']}")
         torch.cuda.empty_cache()
         extras["latent_attention_decode"] = latent_decode(device)
+        extras["sparse_index_selection"] = index_selection(device)
         log(f"[bench] latent-attention decode: {extras['latent_attention_decode']}")
         result["extra"] = extras
     if not args.no_cpu:

@@ -47,6 +47,8 @@ int crit_pkv_index_topk(const crit_pkv_index_topk_params* p, void* stream) {
     return pkv::launch_index_topk(p, reinterpret_cast<hipStream_t>(stream));
 }
 
+int64_t crit_pkv_index_topk_work_bytes(int32_t tokens, int32_t n, int32_t k) { return pkv::index_topk_work_bytes(tokens, n, k); }
+
 int crit_pkv_round(const crit_pkv_round_params* p, void* stream) {
     return pkv::launch_round(p, reinterpret_cast<hipStream_t>(stream));
 }

@@ -6,16 +6,24 @@
 //   picked[t]   = the positions of the k largest scores below ends[t], ascending, then -1; ties to the lower position,
 //                 a NaN below every number
 //
-// index_scores_kernel: a workgroup is one token and a block of keys; each of its four wavefronts takes tiles of 16 keys.
-// The token's queries sit in LDS (heads x dim, 16-bit); a tile's key rows are loaded as they lie (a lane: one key, 8
-// adjacent values per k-step: the A operand of v_mfma_f32_16x16x32), from their slots where the keys are read in place.
-// S^T = K Q^T per tile of 16 heads leaves a lane one head's products with 4 keys: ReLU, the head's factor, then the sum
-// over the 16 heads as a fixed tree of lane exchanges, the head tiles added in order. So a token's bits are its own:
-// not its neighbours', not the launch's shape.
+// Scores. A token's queries stay in registers as A operands of v_mfma_f32_16x16x32 (a lane: one head of a tile of 16,
+// 8 adjacent values per k-step), a tile of 16 keys is the B operand (a lane: one key), so a lane is left 4 heads'
+// products with one key: ReLU, the head's factor, the lane's heads added in order, the tiles of heads in order, then
+// the four quarters of the wavefront as (0 + 1) + (2 + 3). That order is the same in both kernels, so a token's bits
+// are its own: not its neighbours', not the launch's shape.
+//   index_scores_kernel: a workgroup is one token and a block of keys, its four wavefronts take tiles of 16 keys in
+//     turn and load them where they lie (from their slots where the keys are read in place): calls of few tokens.
+//   index_scores_tokens_kernel: a workgroup is 4 or 8 tokens (one or two a wavefront) and a block of keys; 64 keys a
+//     step go through LDS once for all of them (two buffers, one barrier a step, the next step's loads in flight
+//     under the products), so the keys cross the L2 once per 4 or 8 tokens.
 //
-// index_topk_kernel: a workgroup a token. The scores map to 32-bit keys that order as the rule does (NaN lowest, -0 = +0),
-// an 8-bit radix select from the top finds the k-th key and how many of its equals are taken, and one pass in position
-// order writes the positions of everything above it and of its first equals: ascending by construction.
+// Top-k. index_topk_kernel: a workgroup a token (or a slice of its positions). The scores map to 32-bit keys that order
+// as the rule does (NaN lowest, -0 = +0); an 8-bit radix select from the top finds the k-th key and how many of its
+// equals are taken (histograms in 16 copies a bin, so the lanes of a wavefront that meet in a bin meet 4 to an address,
+// and a scan over the bins instead of one thread's walk); then each wavefront takes a quarter of the positions, counts
+// what it will write, and writes the positions of everything above the k-th key and of its first equals in order:
+// ascending by construction. Calls of few tokens over many positions select in slices (the k best of each, positions
+// and scores) and then among the slices' picks: a token's k best are among its slices', in the same order.
 #include "pkv_attend_mfma.hpp"
 #include "pkv_launch.hpp"
 
@@ -31,96 +39,235 @@ struct ScoreArgs {
     const void* slots;
     float* out;
     int64_t q_st, q_sh, key_stride, w_stride, out_stride, slots_stride;
-    int tokens, n, group, heads, dim, slots_are_64, block;
+    int tokens, n, group, heads, slots_are_64, block;
     float scale;
 };
 
-template <bool F16, bool FP8>
-__global__ __launch_bounds__(256) void index_scores_kernel(ScoreArgs a) {
-    extern __shared__ __align__(16) uint8_t s_q[];      // [heads padded to 16][dim * 2 + 32 bytes]
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 4, li = lane & 15;
-    const int t = blockIdx.y;
-    const int d = a.dim, H = a.heads;
-    const int rowb = d * 2 + 32;
-    const int hp = (H + 15) / 16 * 16;
-    // the token's queries, heads past the last as zeros
-    const int chunks = d / 8;
-    for (int i = tid; i < hp * chunks; i += 256) {
-        const int h = i / chunks, c = i - h * chunks;
-        u32x4 w = {0u, 0u, 0u, 0u};
-        if (h < H) w = *reinterpret_cast<const u32x4*>(a.q + ((int64_t)t * a.q_st + (int64_t)h * a.q_sh) * 2 + c * 16);
-        *reinterpret_cast<u32x4*>(s_q + h * rowb + c * 16) = w;
-    }
-    __syncthreads();
-    const int end = min(max(a.ends[t], 0), a.n);
-    const int ksteps = d / 32;
-    const int64_t srow = (int64_t)(t / a.group) * a.slots_stride;
-    const int first = blockIdx.x * a.block;
-    const int last = min(first + a.block, a.n);
-    for (int k0 = first + wave * 16; k0 < last; k0 += 64) {
-        float* out = a.out + (int64_t)t * a.out_stride;
-        if (k0 >= end) {      // nothing of the tile is seen
-            if (g == 0 && k0 + li < last) out[k0 + li] = -INFINITY;
-            continue;
-        }
-        // the lane's key (the tile's row li), a key past the last reads the last
-        const int key = min(k0 + li, a.n - 1);
-        int64_t at = key;
-        if (a.slots) at = a.slots_are_64 ? reinterpret_cast<const int64_t*>(a.slots)[srow + key] : (int64_t) reinterpret_cast<const int32_t*>(a.slots)[srow + key];
-        const uint8_t* krow = a.keys + at * a.key_stride * (FP8 ? 1 : 2) + g * (FP8 ? 8 : 16);
-        u32x4 ka[8];      // up to 8 k-steps (dim 256)
+// One token's queries: qa[ht][ks] the lane's A operand (head ht * 16 + li, values ks * 32 + 8 g .. + 7), heads past the
+// last as zeros.
+template <int HT, int KS>
+struct TokenQ {
+    u32x4 qa[HT][KS];
+};
+
+template <int HT, int KS>
+PKV_DEV void load_token(const ScoreArgs& a, int t, int g, int li, TokenQ<HT, KS>& q) {
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-            if (ks < ksteps) {
-                if constexpr (FP8) {
-                    const u32x2 c = *reinterpret_cast<const u32x2*>(krow + ks * 32);
-                    const f32x2 a0 = e4m3_pair<false>(c.x), a1 = e4m3_pair<true>(c.x), a2 = e4m3_pair<false>(c.y), a3 = e4m3_pair<true>(c.y);
-                    ka[ks] = u32x4{pair16<F16>(a0.x, a0.y), pair16<F16>(a1.x, a1.y), pair16<F16>(a2.x, a2.y), pair16<F16>(a3.x, a3.y)};
-                } else {
-                    ka[ks] = *reinterpret_cast<const u32x4*>(krow + ks * 64);
-                }
-            }
-        }
-        float total[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        for (int ht = 0; ht < hp / 16; ++ht) {
-            f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-            const uint8_t* qrow = s_q + (ht * 16 + li) * rowb + g * 16;
+    for (int ht = 0; ht < HT; ++ht) {
+        const int h = ht * 16 + li;
+        const uint8_t* row = a.q + ((int64_t)t * a.q_st + (int64_t)h * a.q_sh) * 2 + g * 16;
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks)
-                if (ks < ksteps) acc = mfma_k32<F16>(ka[ks], *reinterpret_cast<const u32x4*>(qrow + ks * 64), acc);
-            const int h = ht * 16 + li;
-            const float factor = h < H ? a.weights[(int64_t)t * a.w_stride + h] * a.scale : 0.0f;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                float v = __builtin_fmaxf(acc[i], 0.0f) * factor;
-                // the 16 heads of the tile: a tree over the lanes 1, 2, 4, 8 apart
-                v += __shfl_xor(v, 1);
-                v += __shfl_xor(v, 2);
-                v += __shfl_xor(v, 4);
-                v += __shfl_xor(v, 8);
-                total[i] += v;
-            }
-        }
-        if (li < 4) {      // lane li of quarter g writes key 4 g + li
-            const int kk = k0 + 4 * g + li;
-            float v = li == 0 ? total[0] : (li == 1 ? total[1] : (li == 2 ? total[2] : total[3]));
-            if constexpr (FP8) {
-                const int key2 = min(kk, a.n - 1);
-                int64_t at2 = key2;
-                if (a.slots) at2 = a.slots_are_64 ? reinterpret_cast<const int64_t*>(a.slots)[srow + key2] : (int64_t) reinterpret_cast<const int32_t*>(a.slots)[srow + key2];
-                v *= a.key_scales[at2];
-            }
-            if (kk < last) out[kk] = kk < end ? v : -INFINITY;
+        for (int ks = 0; ks < KS; ++ks) {
+            u32x4 w = {0u, 0u, 0u, 0u};
+            if (h < a.heads) w = *reinterpret_cast<const u32x4*>(row + ks * 64);
+            q.qa[ht][ks] = w;
         }
     }
 }
 
+// The factor of head h of token t (0 past the last head).
+PKV_DEV float head_factor(const ScoreArgs& a, int t, int h) {
+    return h < a.heads ? a.weights[(int64_t)t * a.w_stride + h] * a.scale : 0.0f;
+}
+
+// A key's lane operand from what was loaded: 16-bit values as they are, E4M3 codes as their 16-bit values (exact).
+template <bool F16, bool FP8>
+PKV_DEV u32x4 key_operand(u32x4 raw16, u32x2 raw8) {
+    if constexpr (FP8) {
+        const f32x2 a0 = e4m3_pair<false>(raw8.x), a1 = e4m3_pair<true>(raw8.x), a2 = e4m3_pair<false>(raw8.y), a3 = e4m3_pair<true>(raw8.y);
+        return u32x4{pair16<F16>(a0.x, a0.y), pair16<F16>(a1.x, a1.y), pair16<F16>(a2.x, a2.y), pair16<F16>(a3.x, a3.y)};
+    } else {
+        return raw16;
+    }
+}
+
+// max(x, 0) as one instruction: the bits of a float order as a signed integer's do where it is positive, and every
+// negative float (and -0) is a negative integer (fmaxf comes with a second instruction that quiets a signalling NaN).
+PKV_DEV float relu(float x) { return u2f((uint32_t)max((int)f2u(x), 0)); }
+
+// A token's score with the lane's key (the tile's key li), the same bits in the four lanes of the key: f(ht) gives the
+// factors of heads ht * 16 + 4 g .. + 3.
+template <bool F16, int HT, int KS, typename Factors>
+PKV_DEV float tile_score(const TokenQ<HT, KS>& q, const u32x4 (&kb)[KS], Factors&& f) {
+    f32x4 acc[HT];
+#pragma unroll
+    for (int ht = 0; ht < HT; ++ht) acc[ht] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int ht = 0; ht < HT; ++ht) acc[ht] = mfma_k32<F16>(q.qa[ht][ks], kb[ks], acc[ht]);
+    float total = 0.0f;
+#pragma unroll
+    for (int ht = 0; ht < HT; ++ht) {
+        const f32x4 w = f(ht);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) total = __builtin_fmaf(relu(acc[ht][i]), w[i], total);      // (one rounding a head)
+    }
+    return sum_across_quarters(total);
+}
+
+PKV_DEV int64_t slot_of(const ScoreArgs& a, int64_t srow, int key) {
+    if (!a.slots) return key;
+    return a.slots_are_64 ? reinterpret_cast<const int64_t*>(a.slots)[srow + key] : (int64_t) reinterpret_cast<const int32_t*>(a.slots)[srow + key];
+}
+
+template <bool F16, bool FP8, int HT, int KS>
+__global__ __launch_bounds__(256) void index_scores_kernel(ScoreArgs a) {
+    constexpr int QROWB = KS * 64 + (HT * KS == 64 ? 0 : 16);      // a head's row in LDS (padded where that keeps it within 64 KB)
+    __shared__ __align__(16) uint8_t s_q[HT * 16 * QROWB];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 4, li = lane & 15;
+    const int t = blockIdx.y;
+    // the token's queries: loaded once a workgroup, then each wavefront's operands from LDS (heads past the last: zeros)
+    for (int i = tid; i < HT * 16 * KS * 4; i += 256) {
+        const int h = i / (KS * 4), c = i % (KS * 4);
+        u32x4 w = {0u, 0u, 0u, 0u};
+        if (h < a.heads) w = *reinterpret_cast<const u32x4*>(a.q + ((int64_t)t * a.q_st + (int64_t)h * a.q_sh) * 2 + c * 16);
+        *reinterpret_cast<u32x4*>(s_q + h * QROWB + c * 16) = w;
+    }
+    f32x4 fac[HT];
+#pragma unroll
+    for (int ht = 0; ht < HT; ++ht)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) fac[ht][i] = head_factor(a, t, ht * 16 + 4 * g + i);
+    const int end = min(max(a.ends[t], 0), a.n);
+    const int64_t srow = (int64_t)(t / a.group) * a.slots_stride;
+    const int first = blockIdx.x * a.block;
+    const int last = min(first + a.block, a.n);
+    float* out = a.out + (int64_t)t * a.out_stride;
+    using Raw = typename std::conditional<FP8, u32x2, u32x4>::type;
+    Raw held[KS];
+    int64_t held_at = 0;
+    auto fetch = [&](int k0) {      // the lane's key of the tile (a key past the last reads the last)
+        held_at = slot_of(a, srow, min(k0 + li, a.n - 1));
+        const uint8_t* krow = a.keys + held_at * a.key_stride * (FP8 ? 1 : 2) + g * (FP8 ? 8 : 16);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) held[ks] = *reinterpret_cast<const Raw*>(krow + ks * (FP8 ? 32 : 64));
+    };
+    int k0 = first + wave * 16;
+    if (k0 < last && k0 < end) fetch(k0);
+    __syncthreads();
+    TokenQ<HT, KS> q;
+#pragma unroll
+    for (int ht = 0; ht < HT; ++ht)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) q.qa[ht][ks] = *reinterpret_cast<const u32x4*>(s_q + (ht * 16 + li) * QROWB + ks * 64 + g * 16);
+    for (; k0 < last; k0 += 64) {
+        const int kk = k0 + li;
+        if (k0 >= end) {      // nothing of the tile is seen (nor of the wavefront's later ones)
+            if (g == 0 && kk < last) out[kk] = -INFINITY;
+            continue;
+        }
+        u32x4 kb[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            if constexpr (FP8) kb[ks] = key_operand<F16, true>(u32x4{}, held[ks]);
+            else kb[ks] = held[ks];
+        }
+        const int64_t at = held_at;
+        if (k0 + 64 < last && k0 + 64 < end) fetch(k0 + 64);
+        float v = tile_score<F16>(q, kb, [&](int ht) { return fac[ht]; });
+        if constexpr (FP8) v *= a.key_scales[at];
+        if (g == 0 && kk < last) out[kk] = kk < end ? v : -INFINITY;
+    }
+}
+
+template <bool F16, bool FP8, int HT, int KS, int TW>
+__global__ __launch_bounds__(256, HT * KS * TW <= 32 ? 2 : 1) void index_scores_tokens_kernel(ScoreArgs a) {
+    constexpr int E = FP8 ? 1 : 2;
+    constexpr int ROWB = KS * 32 * E + 16;            // a key's row in LDS
+    constexpr int CH = KS * 32 * E / 16;              // its 16-byte pieces
+    constexpr int PER = 64 * CH / 256;                // pieces a thread stages a step
+    constexpr int HP = HT * 16;
+    extern __shared__ __align__(16) uint8_t s_mem[];  // the heads' factors [4 TW][HP], then two buffers of 64 key rows
+    float* s_f = reinterpret_cast<float*>(s_mem);
+    uint8_t* s_k = s_mem + 4 * TW * HP * 4;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 4, li = lane & 15;
+    const int wg_first = blockIdx.y * (4 * TW);
+    TokenQ<HT, KS> q[TW];
+    int ends[TW];
+    bool live[TW];
+    int wave_end = 0;
+#pragma unroll
+    for (int j = 0; j < TW; ++j) {
+        const int t = wg_first + wave * TW + j;
+        live[j] = t < a.tokens;
+        const int tt = live[j] ? t : a.tokens - 1;
+        load_token(a, tt, g, li, q[j]);
+        ends[j] = live[j] ? min(max(a.ends[tt], 0), a.n) : 0;
+        wave_end = max(wave_end, ends[j]);
+    }
+    for (int i = tid; i < 4 * TW * HP; i += 256) {
+        const int t = wg_first + i / HP;
+        s_f[i] = t < a.tokens ? head_factor(a, t, i % HP) : 0.0f;
+    }
+    const int64_t srow = (int64_t)(wg_first / a.group) * a.slots_stride;      // (a workgroup's tokens are of one group)
+    const int first = blockIdx.x * a.block;
+    const int last = min(first + a.block, a.n);
+    u32x4 held[PER];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int c = tid + 256 * j;
+            const int64_t at = slot_of(a, srow, min(k0 + c / CH, a.n - 1));
+            held[j] = *reinterpret_cast<const u32x4*>(a.keys + at * a.key_stride * E + (c % CH) * 16);
+        }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int c = tid + 256 * j;
+            *reinterpret_cast<u32x4*>(s_k + buf * (64 * ROWB) + (c / CH) * ROWB + (c % CH) * 16) = held[j];
+        }
+    };
+    fetch(first);
+    int buf = 0;
+    for (int k0 = first; k0 < last; k0 += 64, buf ^= 1) {
+        stage(buf);
+        lds_barrier();      // (one a step: a buffer is written again two steps on, past the barrier every wavefront reaches after its reads)
+        if (k0 + 64 < last) fetch(k0 + 64);
+        const int kk = k0 + lane;
+        float mine[TW];
+#pragma unroll
+        for (int j = 0; j < TW; ++j) mine[j] = 0.0f;
+        if (k0 < wave_end) {
+            f32x4 fac[TW][HT];
+#pragma unroll
+            for (int j = 0; j < TW; ++j)
+#pragma unroll
+                for (int ht = 0; ht < HT; ++ht) fac[j][ht] = *reinterpret_cast<const f32x4*>(s_f + (wave * TW + j) * HP + ht * 16 + 4 * g);
+#pragma unroll
+            for (int T = 0; T < 4; ++T) {
+                const uint8_t* krow = s_k + buf * (64 * ROWB) + (T * 16 + li) * ROWB + g * (8 * E);
+                u32x4 kb[KS];
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    if constexpr (FP8) kb[ks] = key_operand<F16, true>(u32x4{}, *reinterpret_cast<const u32x2*>(krow + ks * 32));
+                    else kb[ks] = *reinterpret_cast<const u32x4*>(krow + ks * 64);
+                }
+#pragma unroll
+                for (int j = 0; j < TW; ++j) {
+                    const float v = tile_score<F16>(q[j], kb, [&](int ht) { return fac[j][ht]; });
+                    if (g == T) mine[j] = v;      // the quarter g keeps tile g: a lane's key is k0 + lane
+                }
+            }
+        }
+        float key_scale = 1.0f;
+        if constexpr (FP8) key_scale = a.key_scales[slot_of(a, srow, min(kk, a.n - 1))];
+#pragma unroll
+        for (int j = 0; j < TW; ++j)
+            if (live[j] && kk < last)
+                a.out[(int64_t)(wg_first + wave * TW + j) * a.out_stride + kk] = kk < ends[j] ? mine[j] * key_scale : -INFINITY;
+    }
+}
+
 struct TopkArgs {
-    const float* s;
+    const float* s;          // scores [tokens][s_stride]; the candidates' where LEVEL is 2
+    const int32_t* pos;      // the candidates' positions [tokens][s_stride] (LEVEL 2)
     const int32_t* ends;
     int32_t* out;
+    float* out_scores;       // the picks' scores beside their positions (LEVEL 1)
     int64_t s_stride, out_stride;
-    int tokens, n, k;
+    int tokens, n, k, width, parts;
 };
 
 // The key a score is ranked by: larger first; -0 and +0 the same; -inf below every finite; a NaN below everything.
@@ -130,77 +277,325 @@ PKV_DEV uint32_t rank_key(float x) {
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
+// LEVEL 0: a token's row, to its picks. 1: a slice of its row (blockIdx.y), to the slice's candidates (positions and
+// scores, [parts][k] a token). 2: a token's candidates (those with a position), to its picks.
+template <int LEVEL>
 __global__ __launch_bounds__(256) void index_topk_kernel(TopkArgs a) {
-    __shared__ unsigned s_hist[256];
+    __shared__ unsigned s_hist[256 * 16];
+    __shared__ unsigned s_wave[4];
     __shared__ unsigned s_pick[2];
-    __shared__ int s_scan[2][4];
+    __shared__ int s_cnt[4][2];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int t = blockIdx.x;
-    const float* row = a.s + (int64_t)t * a.s_stride;
-    int32_t* out = a.out + (int64_t)t * a.out_stride;
+    const int t = blockIdx.x, part = LEVEL == 1 ? blockIdx.y : 0;
     const int end = min(max(a.ends[t], 0), a.n);
     const int k = a.k;
-    if (end <= k) {
-        for (int i = tid; i < k; i += 256) out[i] = i < end ? i : -1;
-        return;
+    const float* row = a.s + (int64_t)t * a.s_stride;
+    const int32_t* pos = LEVEL == 2 ? a.pos + (int64_t)t * a.s_stride : nullptr;
+    int32_t* out = a.out + (int64_t)t * a.out_stride + (int64_t)part * k;
+    float* out_scores = LEVEL == 1 ? a.out_scores + (int64_t)t * a.out_stride + (int64_t)part * k : nullptr;
+    int lo = 0, m, valid;      // the elements lo .. lo + m - 1 of the row, `valid` of them candidates
+    if constexpr (LEVEL == 2) {
+        m = a.parts * k, valid = 0;
+        for (int p = 0; p < a.parts; ++p) valid += min(max(min(end - p * a.width, a.width), 0), k);
+    } else {
+        lo = LEVEL == 1 ? part * a.width : 0;
+        m = max(min(LEVEL == 1 ? a.width : a.n, end - lo), 0), valid = m;
     }
-    // radix select: the k-th largest key, 8 bits at a time from the top
-    uint32_t prefix = 0u, mask = 0u;
-    unsigned want = (unsigned)k;      // of the keys that match the prefix, the `want` largest are taken
-    for (int shift = 24; shift >= 0; shift -= 8) {
-        s_hist[tid] = 0u;
-        __syncthreads();
-        for (int i = tid; i < end; i += 256) {
-            const uint32_t key = rank_key(row[i]);
-            if ((key & mask) == prefix) atomicAdd(&s_hist[(key >> shift) & 255u], 1u);
+    row += lo;
+    auto take = [&](int i, float& x) -> bool {      // element i: its score; whether it is a candidate
+        if constexpr (LEVEL == 2) {
+            if (pos[i] < 0) return false;
         }
-        __syncthreads();
-        if (tid == 0) {
-            unsigned above = 0u;
-            int b = 255;
-            for (; b > 0; --b) {
-                if (above + s_hist[b] >= want) break;
-                above += s_hist[b];
+        x = row[i];
+        return true;
+    };
+    const bool all = valid <= k;      // everything is picked
+    uint32_t prefix = 0u;
+    unsigned want = 0u;               // of the keys equal to the k-th, the `want` first are taken
+    if (!all) {
+        // radix select: the k-th largest key, 8 bits at a time from the top
+        uint32_t mask = 0u;
+        want = (unsigned)k;
+        for (int shift = 24; shift >= 0; shift -= 8) {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) s_hist[tid + 256 * j] = 0u;
+            __syncthreads();
+            for (int i0 = 0; i0 < m; i0 += 1024) {
+                float x[4];
+                bool ok[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int i = i0 + j * 256 + tid;
+                    x[j] = 0.0f;
+                    ok[j] = i < m && take(i, x[j]);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t key = rank_key(x[j]);
+                    if (ok[j] && (key & mask) == prefix) atomicAdd(&s_hist[((key >> shift) & 255u) * 16 + (lane & 15)], 1u);
+                }
             }
-            s_pick[0] = (unsigned)b, s_pick[1] = want - above;
+            __syncthreads();
+            // thread tid: bin 255 - tid; the count of keys in it and in the bins above it
+            const int bin = 255 - tid;
+            unsigned h = 0u;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) h += s_hist[bin * 16 + j];
+            unsigned incl = h;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const unsigned y = __shfl_up(incl, off);
+                if (lane >= off) incl += y;
+            }
+            if (lane == 63) s_wave[wave] = incl;
+            __syncthreads();
+            for (int w = 0; w < wave; ++w) incl += s_wave[w];
+            if (incl >= want && incl - h < want) s_pick[0] = (unsigned)bin, s_pick[1] = want - (incl - h);
+            __syncthreads();
+            prefix |= s_pick[0] << shift;
+            mask |= 255u << shift;
+            want = s_pick[1];
         }
+    }
+    // In position order: everything above the k-th key, and its first `want` equals. A wavefront takes a quarter of the
+    // elements: what it will write first, then the writes.
+    const int per = (m + 255) / 256 * 64;
+    const int w_lo = min(wave * per, m), w_hi = min(w_lo + per, m);
+    const unsigned long long below = (1ull << lane) - 1ull;
+    int n_above = 0, n_equal = 0;
+    for (int i0 = w_lo; i0 < w_hi; i0 += 64) {
+        const int i = i0 + lane;
+        float x = 0.0f;
+        const bool ok = i < w_hi && take(i, x);
+        const uint32_t key = rank_key(x);
+        n_above += __popcll(__ballot(ok && (all || key > prefix)));
+        n_equal += __popcll(__ballot(ok && !all && key == prefix));
+    }
+    if (lane == 0) s_cnt[wave][0] = n_above, s_cnt[wave][1] = n_equal;
+    __syncthreads();
+    int above_seen = 0, equal_seen = 0;
+    for (int w = 0; w < wave; ++w) above_seen += s_cnt[w][0], equal_seen += s_cnt[w][1];
+    for (int i0 = w_lo; i0 < w_hi; i0 += 64) {
+        const int i = i0 + lane;
+        float x = 0.0f;
+        const bool ok = i < w_hi && take(i, x);
+        const uint32_t key = rank_key(x);
+        const bool above = ok && (all || key > prefix), equal = ok && !all && key == prefix;
+        const unsigned long long above_mask = __ballot(above), equal_mask = __ballot(equal);
+        const int rank = equal_seen + __popcll(equal_mask & below);      // the equals before this one
+        if (above || (equal && rank < (int)want)) {
+            const int place = above_seen + __popcll(above_mask & below) + min(rank, (int)want);
+            if constexpr (LEVEL == 2) out[place] = pos[i];
+            else out[place] = lo + i;
+            if constexpr (LEVEL == 1) out_scores[place] = x;
+        }
+        above_seen += __popcll(above_mask), equal_seen += __popcll(equal_mask);
+    }
+    for (int i = min(valid, k) + tid; i < k; i += 256) out[i] = -1;
+}
+
+
+// The same selection with a workgroup's elements held in registers (up to 1,024 x EPT of them): loaded once, every
+// load in flight at once, where the streaming kernel above pays a round trip to the L2 per 1,024 elements and pass.
+// Element i = j * 1,024 + tid (coalesced loads); for the writes in position order, every 64 consecutive elements (a
+// wavefront's of one j) count what they will write, a scan over those counts gives each its first place.
+template <int LEVEL, int EPT>
+__global__ __launch_bounds__(1024) void index_topk_held_kernel(TopkArgs a) {
+    __shared__ unsigned s_hist[256 * 16];
+    __shared__ unsigned s_wave[16];
+    __shared__ unsigned s_pick[2];
+    __shared__ unsigned s_chunk[EPT * 16];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int t = blockIdx.x, part = LEVEL == 1 ? blockIdx.y : 0;
+    const int end = min(max(a.ends[t], 0), a.n);
+    const int k = a.k;
+    const float* row = a.s + (int64_t)t * a.s_stride;
+    const int32_t* pos = LEVEL == 2 ? a.pos + (int64_t)t * a.s_stride : nullptr;
+    int32_t* out = a.out + (int64_t)t * a.out_stride + (int64_t)part * k;
+    float* out_scores = LEVEL == 1 ? a.out_scores + (int64_t)t * a.out_stride + (int64_t)part * k : nullptr;
+    int lo = 0, m, valid;
+    if constexpr (LEVEL == 2) {
+        m = a.parts * k, valid = 0;
+        for (int p = 0; p < a.parts; ++p) valid += min(max(min(end - p * a.width, a.width), 0), k);
+    } else {
+        lo = LEVEL == 1 ? part * a.width : 0;
+        m = max(min(LEVEL == 1 ? a.width : a.n, end - lo), 0), valid = m;
+    }
+    row += lo;
+    uint32_t key[EPT];
+    uint32_t ok = 0u;      // bit j: element j is a candidate
+    {
+        float x[EPT];
+        int at[EPT];
+#pragma unroll
+        for (int j = 0; j < EPT; ++j) {
+            const int i = j * 1024 + tid;
+            x[j] = i < m ? row[i] : 0.0f;
+            at[j] = 0;
+            if constexpr (LEVEL == 2) at[j] = i < m ? pos[i] : -1;
+        }
+#pragma unroll
+        for (int j = 0; j < EPT; ++j) {
+            key[j] = rank_key(x[j]);
+            if (j * 1024 + tid < m && at[j] >= 0) ok |= 1u << j;
+        }
+    }
+    const bool all = valid <= k;
+    uint32_t prefix = 0u;
+    unsigned want = 0u;
+    if (!all) {
+        uint32_t mask = 0u;
+        want = (unsigned)k;
+        for (int shift = 24; shift >= 0; shift -= 8) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) s_hist[tid + 1024 * j] = 0u;
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < EPT; ++j)
+                if (((ok >> j) & 1u) && (key[j] & mask) == prefix) atomicAdd(&s_hist[((key[j] >> shift) & 255u) * 16 + (lane & 15)], 1u);
+            __syncthreads();
+            unsigned h = 0u, incl = 0u;
+            const int bin = 255 - tid;
+            if (tid < 256) {      // (wavefronts 0 .. 3, whole)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) h += s_hist[bin * 16 + j];
+                incl = h;
+#pragma unroll
+                for (int off = 1; off < 64; off <<= 1) {
+                    const unsigned y = __shfl_up(incl, off);
+                    if (lane >= off) incl += y;
+                }
+                if (lane == 63) s_wave[wave] = incl;
+            }
+            __syncthreads();
+            if (tid < 256) {
+                for (int w = 0; w < wave; ++w) incl += s_wave[w];
+                if (incl >= want && incl - h < want) s_pick[0] = (unsigned)bin, s_pick[1] = want - (incl - h);
+            }
+            __syncthreads();
+            prefix |= s_pick[0] << shift;
+            mask |= 255u << shift;
+            want = s_pick[1];
+        }
+    }
+    // what each run of 64 elements writes (above the k-th key | equal to it << 16), then the places before each run
+    const unsigned long long below = (1ull << lane) - 1ull;
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+        const bool is = (ok >> j) & 1u;
+        const unsigned n_above = __popcll(__ballot(is && (all || key[j] > prefix)));
+        const unsigned n_equal = __popcll(__ballot(is && !all && key[j] == prefix));
+        if (lane == 0) s_chunk[j * 16 + wave] = n_above | (n_equal << 16);
+    }
+    __syncthreads();
+    {
+        const unsigned v = tid < EPT * 16 ? s_chunk[tid] : 0u;
+        unsigned incl = v;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const unsigned y = __shfl_up(incl, off);
+            if (lane >= off) incl += y;
+        }
+        if (lane == 63) s_wave[wave] = incl;
         __syncthreads();
-        prefix |= s_pick[0] << shift;
-        mask |= 255u << shift;
-        want = s_pick[1];
+        for (int w = 0; w < wave; ++w) incl += s_wave[w];
+        if (tid < EPT * 16) s_chunk[tid] = incl - v;
         __syncthreads();
     }
-    // positions in order: everything above the k-th key, and its first `want` equals
-    int taken = 0, equals = 0;      // before this pass of 256 positions
-    for (int i0 = 0; i0 < end; i0 += 256) {
-        const int i = i0 + tid;
-        const uint32_t key = i < end ? rank_key(row[i]) : 0u;
-        const bool above = i < end && key > prefix, equal = i < end && key == prefix;
-        const unsigned long long eq_mask = __ballot(equal), ab_mask = __ballot(above);
-        const unsigned long long below = (1ull << lane) - 1ull;
-        if (lane == 0) s_scan[0][wave] = __popcll(eq_mask), s_scan[1][wave] = __popcll(ab_mask);
-        __syncthreads();
-        int eq_before = equals, eq_total = equals;
-        for (int w = 0; w < 4; ++w) {
-            if (w < wave) eq_before += s_scan[0][w];
-            eq_total += s_scan[0][w];
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+        const bool is = (ok >> j) & 1u;
+        const bool above = is && (all || key[j] > prefix), equal = is && !all && key[j] == prefix;
+        const unsigned long long above_mask = __ballot(above), equal_mask = __ballot(equal);
+        const unsigned before = s_chunk[j * 16 + wave];
+        const int rank = (int)(before >> 16) + __popcll(equal_mask & below);
+        if (above || (equal && rank < (int)want)) {
+            const int i = j * 1024 + tid;
+            const int place = (int)(before & 0xffffu) + __popcll(above_mask & below) + min(rank, (int)want);
+            if constexpr (LEVEL == 2) out[place] = pos[i];
+            else out[place] = lo + i;
+            if constexpr (LEVEL == 1) out_scores[place] = row[i];
         }
-        const int eq_rank = eq_before + __popcll(eq_mask & below);
-        const bool pick = above || (equal && eq_rank < (int)want);
-        // the picked ones of this pass, in order: the above, and the equals still wanted
-        const int eq_picked_before_wave = min(eq_before, (int)want) - min(equals, (int)want);
-        int ab_before = 0, ab_total = 0;
-        for (int w = 0; w < 4; ++w) {
-            if (w < wave) ab_before += s_scan[1][w];
-            ab_total += s_scan[1][w];
-        }
-        const int eq_in_wave = min(eq_rank, (int)want) - min(eq_before, (int)want);
-        const int place = taken + ab_before + eq_picked_before_wave + __popcll(ab_mask & below) + eq_in_wave;
-        if (pick) out[place] = i;
-        taken += ab_total + (min(eq_total, (int)want) - min(equals, (int)want));
-        equals = eq_total;
-        __syncthreads();
     }
+    for (int i = min(valid, k) + tid; i < k; i += 1024) out[i] = -1;
+}
+
+template <bool F16, bool FP8, int HT, int KS>
+int launch_scores_shape(ScoreArgs a, bool many, int cus, hipStream_t stream) {
+    if (!many) {
+        // a block of keys a workgroup: enough workgroups for the chip
+        int block = 64;
+        while (block < 4096 && (int64_t)a.tokens * ((a.n + block - 1) / block) > (int64_t)cus * 6) block *= 2;
+        a.block = block;
+        const dim3 grid((unsigned)((a.n + block - 1) / block), (unsigned)a.tokens);
+        hipLaunchKernelGGL((index_scores_kernel<F16, FP8, HT, KS>), grid, dim3(256), 0, stream, a);
+        return hip_code(hipGetLastError());
+    }
+    constexpr int TW = HT * KS <= 16 && HT <= 4 ? 2 : 1;      // two tokens a wavefront where their queries fit its registers
+    constexpr int E = FP8 ? 1 : 2;
+    constexpr size_t lds = (size_t)4 * TW * HT * 16 * 4 + 2 * 64 * (KS * 32 * E + 16);
+    const int wgs_t = (a.tokens + 4 * TW - 1) / (4 * TW);
+    int block = 256;
+    while (block < 8192 && (int64_t)wgs_t * ((a.n + block - 1) / block) > (int64_t)cus * 16) block *= 2;
+    a.block = block;
+    if (lds > 48 * 1024) {
+        static bool raised[16] = {};      // per device: the kernel's LDS limit
+        int device = 0;
+        if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 16) return CRIT_PKV_E_GEOMETRY;
+        if (!raised[device]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&index_scores_tokens_kernel<F16, FP8, HT, KS, TW>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+                return CRIT_PKV_E_GEOMETRY;
+            raised[device] = true;
+        }
+    }
+    const dim3 grid((unsigned)((a.n + block - 1) / block), (unsigned)wgs_t);
+    hipLaunchKernelGGL((index_scores_tokens_kernel<F16, FP8, HT, KS, TW>), grid, dim3(256), lds, stream, a);
+    return hip_code(hipGetLastError());
+}
+
+template <bool F16, bool FP8>
+int launch_scores_kind(const ScoreArgs& a, int dim, bool many, int cus, hipStream_t stream) {
+    const int ht = (a.heads + 15) / 16;
+#define PKV_SHAPE(H, K) if (ht == H && dim == K * 32) return launch_scores_shape<F16, FP8, H, K>(a, many, cus, stream);
+    PKV_SHAPE(1, 2) PKV_SHAPE(1, 4) PKV_SHAPE(1, 8)
+    PKV_SHAPE(2, 2) PKV_SHAPE(2, 4) PKV_SHAPE(2, 8)
+    PKV_SHAPE(4, 2) PKV_SHAPE(4, 4) PKV_SHAPE(4, 8)
+    PKV_SHAPE(8, 2) PKV_SHAPE(8, 4) PKV_SHAPE(8, 8)
+#undef PKV_SHAPE
+    return CRIT_PKV_E_GEOMETRY;
+}
+
+// How a call selects. held: the elements a workgroup holds in registers (1,024 threads x 8, 16 or 32). A row that fits
+// is one workgroup's; a longer row goes in slices of `width` positions (each a workgroup's), then the slices' picks
+// (parts x k candidates, which must fit a workgroup too), where the candidates' room stays within kSliceRoom; everything
+// else streams, a workgroup a row.
+constexpr int kHeld = 32768;
+constexpr int64_t kSliceRoom = (int64_t)512 << 20;
+struct TopkPlan {
+    int parts;      // 0: one pass a row
+    int width;
+};
+TopkPlan topk_plan(int tokens, int n, int k, int cus) {
+    TopkPlan plan = {0, n};
+    (void)cus;
+    if (n <= kHeld || tokens > 65535) return plan;
+    for (int width = 8192; width <= kHeld; width *= 2) {
+        const int64_t parts = ((int64_t)n + width - 1) / width;
+        if (parts * k <= kHeld && parts <= 65535 && (int64_t)tokens * parts * k * 8 <= kSliceRoom) {
+            plan.parts = (int)parts, plan.width = width;
+            return plan;
+        }
+    }
+    return plan;
+}
+
+template <int LEVEL>
+void launch_topk_level(const TopkArgs& a, int elements, dim3 grid, hipStream_t stream) {
+    if (elements <= 8192) hipLaunchKernelGGL((index_topk_held_kernel<LEVEL, 8>), grid, dim3(1024), 0, stream, a);
+    else if (elements <= 16384) hipLaunchKernelGGL((index_topk_held_kernel<LEVEL, 16>), grid, dim3(1024), 0, stream, a);
+    else if (elements <= kHeld) hipLaunchKernelGGL((index_topk_held_kernel<LEVEL, 32>), grid, dim3(1024), 0, stream, a);
+    else hipLaunchKernelGGL(index_topk_kernel<LEVEL>, grid, dim3(256), 0, stream, a);
 }
 
 }   // namespace
@@ -212,51 +607,58 @@ int launch_index_scores(const crit_pkv_index_scores_params* p, hipStream_t strea
     if (p->key_dtype < 0 || p->key_dtype > 2 || (p->q_dtype != CRIT_PKV_BF16 && p->q_dtype != CRIT_PKV_F16)) return CRIT_PKV_E_DTYPE;
     if (!fp8 && p->key_dtype != (p->q_dtype == CRIT_PKV_F16 ? 1 : 0)) return CRIT_PKV_E_DTYPE;
     if (fp8 && !p->key_scales) return CRIT_PKV_E_NULL;
-    if (p->tokens < 0 || p->tokens > 65535 || p->n < 0 || p->heads < 1 || p->heads > 128 || (p->dim != 64 && p->dim != 128 && p->dim != 256) ||
-        p->group < 1 || p->q_stride_t % 8 || p->q_stride_h % 8 || (reinterpret_cast<uintptr_t>(p->q) % 16) ||
-        (reinterpret_cast<uintptr_t>(p->keys) % 16) || p->key_stride % (fp8 ? 16 : 8) || p->out_stride < p->n)
+    if (p->tokens < 0 || p->tokens > 65535 || p->n < 0 || p->n > (1 << 30) || p->heads < 1 || p->heads > 128 ||
+        (p->dim != 64 && p->dim != 128 && p->dim != 256) || p->group < 1 || p->q_stride_t % 8 || p->q_stride_h % 8 ||
+        (reinterpret_cast<uintptr_t>(p->q) % 16) || (reinterpret_cast<uintptr_t>(p->keys) % 16) || p->key_stride % (fp8 ? 16 : 8) ||
+        p->out_stride < p->n)
         return CRIT_PKV_E_GEOMETRY;
     ScoreArgs a;
     a.q = reinterpret_cast<const uint8_t*>(p->q), a.keys = reinterpret_cast<const uint8_t*>(p->keys);
     a.key_scales = p->key_scales, a.weights = p->weights, a.ends = p->ends, a.slots = p->slots, a.out = p->out;
     a.q_st = p->q_stride_t, a.q_sh = p->q_stride_h, a.key_stride = p->key_stride, a.w_stride = p->weights_stride;
     a.out_stride = p->out_stride, a.slots_stride = p->slots_stride;
-    a.tokens = p->tokens, a.n = p->n, a.group = p->group, a.heads = p->heads, a.dim = p->dim, a.slots_are_64 = p->slots_are_64;
-    a.scale = p->scale;
-    // a block of keys a workgroup: enough workgroups for the chip where the tokens are few, long blocks where they are many
-    const int cus = compute_units();
-    int block = 64;
-    while (block < 4096 && (int64_t)p->tokens * ((p->n + block - 1) / block) > (int64_t)(cus > 0 ? cus : 256) * 16) block *= 2;
-    a.block = block;
-    const int hp = (p->heads + 15) / 16 * 16;
-    const size_t lds = (size_t)hp * (p->dim * 2 + 32);
-    const dim3 grid((unsigned)((p->n + block - 1) / block), (unsigned)p->tokens);
+    a.tokens = p->tokens, a.n = p->n, a.group = p->group, a.heads = p->heads, a.slots_are_64 = p->slots_are_64;
+    a.scale = p->scale, a.block = 64;
+    const int cus = compute_units() > 0 ? compute_units() : 256;
+    // many tokens share their keys through LDS, 4 or 8 to a workgroup: where the keys are read in place, a group's
+    // tokens (they share the slots) must fill workgroups
+    const int ht = (p->heads + 15) / 16;
+    const int wg_tokens = ht * (p->dim / 32) <= 16 && ht <= 4 ? 8 : 4;
+    const bool many = p->tokens >= 16 && (!p->slots || p->group % wg_tokens == 0);
     const bool f16 = p->q_dtype == CRIT_PKV_F16;
-#define PKV_SCORES(F, E)                                                                                              \
-    {                                                                                                                  \
-        if (lds > 48 * 1024)                                                                                           \
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&index_scores_kernel<F, E>),                         \
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)               \
-                return CRIT_PKV_E_GEOMETRY;                                                                            \
-        hipLaunchKernelGGL((index_scores_kernel<F, E>), grid, dim3(256), lds, stream, a);                              \
-    }
-    if (fp8) {
-        if (f16) PKV_SCORES(true, true) else PKV_SCORES(false, true)
-    } else {
-        if (f16) PKV_SCORES(true, false) else PKV_SCORES(false, false)
-    }
-#undef PKV_SCORES
-    return hip_code(hipGetLastError());
+    if (fp8) return f16 ? launch_scores_kind<true, true>(a, p->dim, many, cus, stream) : launch_scores_kind<false, true>(a, p->dim, many, cus, stream);
+    return f16 ? launch_scores_kind<true, false>(a, p->dim, many, cus, stream) : launch_scores_kind<false, false>(a, p->dim, many, cus, stream);
+}
+
+int64_t index_topk_work_bytes(int tokens, int n, int k) {
+    if (tokens <= 0 || n <= 0 || k <= 0) return 0;
+    const TopkPlan plan = topk_plan(tokens, n, k, compute_units() > 0 ? compute_units() : 256);
+    return (int64_t)tokens * plan.parts * k * 8;
 }
 
 int launch_index_topk(const crit_pkv_index_topk_params* p, hipStream_t stream) {
     if (!p || !p->scores || !p->ends || !p->out) return CRIT_PKV_E_NULL;
     if (p->tokens == 0) return 0;
-    if (p->tokens < 0 || p->n < 0 || p->k < 1 || p->scores_stride < p->n || p->out_stride < p->k) return CRIT_PKV_E_GEOMETRY;
+    if (p->tokens < 0 || p->n < 0 || p->n > (1 << 30) || p->k < 1 || p->scores_stride < p->n || p->out_stride < p->k) return CRIT_PKV_E_GEOMETRY;
     TopkArgs a;
-    a.s = p->scores, a.ends = p->ends, a.out = p->out, a.s_stride = p->scores_stride, a.out_stride = p->out_stride;
-    a.tokens = p->tokens, a.n = p->n, a.k = p->k;
-    hipLaunchKernelGGL(index_topk_kernel, dim3((unsigned)p->tokens), dim3(256), 0, stream, a);
+    a.s = p->scores, a.pos = nullptr, a.ends = p->ends, a.out = p->out, a.out_scores = nullptr;
+    a.s_stride = p->scores_stride, a.out_stride = p->out_stride;
+    a.tokens = p->tokens, a.n = p->n, a.k = p->k, a.width = p->n, a.parts = 1;
+    const TopkPlan plan = topk_plan(p->tokens, p->n, p->k, compute_units() > 0 ? compute_units() : 256);
+    const int64_t need = (int64_t)p->tokens * plan.parts * p->k * 8;
+    if (plan.parts > 1 && p->work && p->work_bytes >= need) {
+        // the slices' k best (positions, then scores: [tokens][parts][k] each), then the k best of those
+        int32_t* cand = reinterpret_cast<int32_t*>(p->work);
+        float* cand_scores = reinterpret_cast<float*>(cand + (int64_t)p->tokens * plan.parts * p->k);
+        TopkArgs s1 = a;
+        s1.out = cand, s1.out_scores = cand_scores, s1.out_stride = (int64_t)plan.parts * p->k, s1.width = plan.width, s1.parts = plan.parts;
+        launch_topk_level<1>(s1, plan.width, dim3((unsigned)p->tokens, (unsigned)plan.parts), stream);
+        TopkArgs s2 = a;
+        s2.s = cand_scores, s2.pos = cand, s2.s_stride = (int64_t)plan.parts * p->k, s2.width = plan.width, s2.parts = plan.parts;
+        launch_topk_level<2>(s2, plan.parts * p->k, dim3((unsigned)p->tokens), stream);
+        return hip_code(hipGetLastError());
+    }
+    launch_topk_level<0>(a, p->n, dim3((unsigned)p->tokens), stream);
     return hip_code(hipGetLastError());
 }
 

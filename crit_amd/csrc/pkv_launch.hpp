@@ -18,6 +18,7 @@ int launch_step_buffers(const crit_pkv_step_params* p, hipStream_t stream);
 int launch_latent(const crit_pkv_latent_params* p, hipStream_t stream);
 int launch_index_scores(const crit_pkv_index_scores_params* p, hipStream_t stream);
 int launch_index_topk(const crit_pkv_index_topk_params* p, hipStream_t stream);
+int64_t index_topk_work_bytes(int tokens, int n, int k);
 int launch_read_rows(const crit_pkv_read_params* p, hipStream_t stream);
 int launch_stream_read(const void* data, int64_t bytes, float* sink, hipStream_t stream);
 // Compute units of the current device (cached per device), or 0 if the query fails.

@@ -124,8 +124,8 @@ class IndexScoresParams(ctypes.Structure):
 
 
 class IndexTopkParams(ctypes.Structure):
-    _fields_ = [("scores", _p), ("ends", _p), ("out", _p), ("scores_stride", _i64), ("out_stride", _i64),
-                ("tokens", _i32), ("n", _i32), ("k", _i32)]
+    _fields_ = [("scores", _p), ("ends", _p), ("out", _p), ("work", _p), ("scores_stride", _i64), ("out_stride", _i64),
+                ("work_bytes", _i64), ("tokens", _i32), ("n", _i32), ("k", _i32)]
 
 
 class ReadParams(ctypes.Structure):
@@ -138,7 +138,7 @@ class ReadParams(ctypes.Structure):
 STATIC_SCRATCH_BYTES = 32 << 20
 
 SYMBOLS = ("crit_pkv_write", "crit_pkv_attend", "crit_pkv_attend_static", "crit_pkv_merge", "crit_pkv_prefill", "crit_pkv_slots_at",
-           "crit_pkv_compact", "crit_pkv_copy_pages", "crit_pkv_round", "crit_pkv_step_buffers", "crit_pkv_latent_attend", "crit_pkv_index_scores", "crit_pkv_index_topk", "crit_pkv_read_rows", "crit_pkv_abi_version", "crit_pkv_params_size", "crit_pkv_error",
+           "crit_pkv_compact", "crit_pkv_copy_pages", "crit_pkv_round", "crit_pkv_step_buffers", "crit_pkv_latent_attend", "crit_pkv_index_scores", "crit_pkv_index_topk", "crit_pkv_index_topk_work_bytes", "crit_pkv_read_rows", "crit_pkv_abi_version", "crit_pkv_params_size", "crit_pkv_error",
            "crit_pkv_stream_read", "crit_pkv_stream_capture")
 
 _lib = None
@@ -194,6 +194,8 @@ def load():
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(struct), ctypes.c_void_p]
+    lib.crit_pkv_index_topk_work_bytes.restype = ctypes.c_int64
+    lib.crit_pkv_index_topk_work_bytes.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
     lib.crit_pkv_stream_capture.restype = ctypes.c_int
     lib.crit_pkv_stream_capture.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_ulonglong)]
     lib.crit_pkv_stream_read.restype = ctypes.c_int

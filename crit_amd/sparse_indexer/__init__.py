@@ -111,6 +111,12 @@ def topk(s, ends, k, *, out: Optional[torch.Tensor] = None):
         return out
     p = _abi.IndexTopkParams()
     p.scores, p.ends, p.out = s.data_ptr(), ends.data_ptr(), out.data_ptr()
+    # long rows: the slices' k best, then the k best of those (the same picks); their room is the caching allocator's,
+    # as the reference's is, so a graph captures the call once its shape has run
+    with torch.cuda.device(s.device):
+        room = int(_abi.load().crit_pkv_index_topk_work_bytes(t, n, int(k)))
+    work = torch.empty(room // 4, dtype=torch.int32, device=s.device) if room else None
+    p.work, p.work_bytes = _ptr(work), room
     p.scores_stride, p.out_stride, p.tokens, p.n, p.k = s.stride(0), out.stride(0), t, n, int(k)
     _launch(s.device, "crit_pkv_index_topk", "sparse_indexer.topk", p)
     return out

@@ -456,16 +456,23 @@ int crit_pkv_index_scores(const crit_pkv_index_scores_params* p, void* stream);
 
 /* out[t][0 .. k - 1] (int32) = the positions of token t's k largest scores below ends[t], ascending, then -1 (all of
  * them where ends[t] <= k): ties to the lower position, -0 = +0, a NaN below every number (sparse_index.py:24-40). One
- * launch, a workgroup a token: an 8-bit radix select for the k-th score, then one pass in position order. */
+ * workgroup a token: an 8-bit radix select for the k-th score, then the positions in order. */
 typedef struct crit_pkv_index_topk_params {
     const float* scores;            /* [tokens][scores_stride >= n] */
     const int32_t* ends;
     int32_t* out;                   /* [tokens][out_stride >= k] */
-    int64_t scores_stride, out_stride;
+    void* work;                     /* optional: crit_pkv_index_topk_work_bytes() bytes of device memory (16-aligned) */
+    int64_t scores_stride, out_stride, work_bytes;
     int32_t tokens, n, k;
 } crit_pkv_index_topk_params;
 
 int crit_pkv_index_topk(const crit_pkv_index_topk_params* p, void* stream);
+
+/* Rows past 32,768 positions select faster in slices (each slice's k best in parallel, then the k best of those: the
+ * same picks, sparse_indexer/__init__.py:152-170): the bytes of `work` a call of this shape takes, 0 where one pass a
+ * row is the way (rows a workgroup holds, or candidates past 512 MiB). Without `work` (or with less) the call selects
+ * in one pass a row. */
+int64_t crit_pkv_index_topk_work_bytes(int32_t tokens, int32_t n, int32_t k);
 
 /* ---- rows read back ----------------------------------------------------------------------------------------------
  * Replaces the index_select, cast and multiply of KVPool.gather and KVPool.rows_at (pages.py:455-493): row i of the

@@ -451,8 +451,8 @@ def test_bad_geometry_is_refused():
         cache.attend(q[:, :7], [0], [0], [99], 1)
     with pytest.raises(ValueError, match="offsets"):
         cache.attend(q, [0], [0], [99], 1, offsets=torch.zeros(1, dtype=torch.int32, device=dev))
-    with pytest.raises(NotImplementedError):
-        cache.attend(q, [0], [0], [99], 1, derive=(q, 0))
+    with pytest.raises(ValueError):
+        cache.attend(q, [0], [0], [99], 1, derive=(q, 0))      # (not a Derive: derive() makes one)
 
 
 def test_launches_that_overlap_on_two_streams_do_not_share_counters():
