@@ -525,7 +525,7 @@ int launch_scores_shape(ScoreArgs a, bool many, int cus, hipStream_t stream) {
     if (!many) {
         // a block of keys a workgroup: enough workgroups for the chip
         int block = 64;
-        while (block < 4096 && (int64_t)a.tokens * ((a.n + block - 1) / block) > (int64_t)cus * 6) block *= 2;
+        while (block < 4096 && (int64_t)a.tokens * ((a.n + block - 1) / block) > (int64_t)cus * 2) block *= 2;
         a.block = block;
         const dim3 grid((unsigned)((a.n + block - 1) / block), (unsigned)a.tokens);
         hipLaunchKernelGGL((index_scores_kernel<F16, FP8, HT, KS>), grid, dim3(256), 0, stream, a);
