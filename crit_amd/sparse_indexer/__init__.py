@@ -25,6 +25,7 @@ from ..paged_kv_attention import _launch, _ptr, _require_device
 __all__ = ["scores", "select", "topk"]
 
 FP8 = torch.float8_e4m3fn
+_LAUNCH_TOKENS = 65535
 
 
 def _check_slots(slots, tokens, rows):
@@ -74,8 +75,19 @@ def scores(q, keys, weights, ends, *, key_scales=None, scale=None, out: Optional
         raise ValueError(f"out is FP32 [{t}][{n}] or wider, rows contiguous")
     if t == 0 or n == 0:
         return out
-    if t > 65535:
-        raise ValueError(f"a call scores up to 65,535 tokens, not {t}: cut it (select() does)")
+    if t > _LAUNCH_TOKENS:      # a launch takes that many: longer calls go in runs of whole groups
+        if slots is None or slots.dim() == 1:
+            runs = [(t0, min(t0 + _LAUNCH_TOKENS, t), slots) for t0 in range(0, t, _LAUNCH_TOKENS)]
+        elif group <= _LAUNCH_TOKENS:
+            per = _LAUNCH_TOKENS // group
+            runs = [(g0 * group, min(g0 + per, t // group) * group, slots[g0:g0 + per]) for g0 in range(0, t // group, per)]
+        else:
+            runs = [(g0 * group + t0, g0 * group + min(t0 + _LAUNCH_TOKENS, group), slots[g0])
+                    for g0 in range(t // group) for t0 in range(0, group, _LAUNCH_TOKENS)]
+        for first, last, these in runs:
+            scores(q[first:last], keys, weights[first:last], ends[first:last], key_scales=key_scales, scale=scale,
+                   out=out[first:last], slots=these)
+        return out
     p = _abi.IndexScoresParams()
     p.q, p.keys, p.key_scales, p.weights, p.ends = q.data_ptr(), keys.data_ptr(), _ptr(key_scales) if fp8 else None, \
         weights.data_ptr(), ends.data_ptr()

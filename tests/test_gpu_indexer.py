@@ -177,6 +177,44 @@ def test_keys_read_in_place_score_as_their_gathered_copy(fp8, kind):
         si.scores(q, store, w, ends, key_scales=scales, slots=slots.float())
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("each", [16, 12])
+def test_a_rounds_rows_share_their_keys_in_place(fp8, each):
+    # Many tokens in groups (a round's rows, each a sequence with its own slots): groups of 16 fill the workgroups that
+    # share keys through LDS, groups of 12 do not and go a token a workgroup; either way the gathered keys' bits.
+    rows, n = 4, 900
+    q, _, _, _, w, ends = problem(rows * each, 64, 128, n, seed=13)
+    g = torch.Generator().manual_seed(6)
+    store = (torch.randn(4000, 128, generator=g) * 0.5).to(dev).to(torch.bfloat16)
+    scales = None
+    if fp8:
+        scales = (store.float().abs().amax(1) / 448.0).clamp_min(1e-30)
+        store = (store.float() / scales[:, None]).to(torch.float8_e4m3fn)
+    slots = torch.stack([torch.randperm(4000, generator=g)[:n] for _ in range(rows)]).to(dev)
+    got = si.scores(q, store, w, ends, key_scales=scales, slots=slots)
+    for r in range(rows):
+        span = slice(r * each, (r + 1) * each)
+        want = si.scores(q[span], store[slots[r]], w[span], ends[span], key_scales=None if scales is None else scales[slots[r]])
+        assert torch.equal(got[span].view(torch.int32), want.view(torch.int32)), r
+        alone = si.scores(q[span][:1], store, w[span][:1], ends[span][:1], key_scales=scales, slots=slots[r].to(torch.int32))
+        assert torch.equal(alone[0].view(torch.int32), got[span][0].view(torch.int32)), r
+
+
+def test_calls_past_a_launchs_tokens_go_in_runs(monkeypatch):
+    monkeypatch.setattr(si, "_LAUNCH_TOKENS", 40)
+    q, keys, _, _, w, ends = problem(100, 8, 64, 300, seed=17)
+    runs = si.scores(q, keys, w, ends)
+    g = torch.Generator().manual_seed(7)
+    slots = torch.stack([torch.randperm(300, generator=g)[:200] for _ in range(5)]).to(dev)      # 5 groups of 20
+    ends2 = ends.clamp(max=200)
+    grouped = si.scores(q, keys, w, ends2, slots=slots)
+    wide = si.scores(q, keys, w, ends2, slots=slots[:2].repeat_interleave(1, 0)[:2])            # 2 groups of 50: past 40 each
+    monkeypatch.setattr(si, "_LAUNCH_TOKENS", 65535)
+    assert torch.equal(runs, si.scores(q, keys, w, ends))
+    assert torch.equal(grouped, si.scores(q, keys, w, ends2, slots=slots))
+    assert torch.equal(wide, si.scores(q, keys, w, ends2, slots=slots[:2]))
+
+
 def test_graphs_capture_a_select():
     q, keys, scales, _, w, ends = problem(4, 64, 128, 2048, seed=4)
     out = torch.empty(4, 512, dtype=torch.int32, device=dev)
