@@ -1,7 +1,12 @@
-"""Assembles the folder crit's kernel loader expects for kernel id `paged-kv-attention`:
+"""Assembles the folders crit's kernel loader expects for the kernel ids `paged-kv-attention`, `latent-attention` and
+`sparse-indexer`:
 
     <dest>/paged-kv-attention/kernel.json
     <dest>/paged-kv-attention/torch-ext/paged_kv_attention/{__init__.py, _abi.py, libcrit_pkv.so}
+    <dest>/latent-attention/kernel.json
+    <dest>/latent-attention/torch-ext/latent_attention/{__init__.py, _pkv/{__init__.py, _abi.py, libcrit_pkv.so}}
+    <dest>/sparse-indexer/kernel.json
+    <dest>/sparse-indexer/torch-ext/sparse_indexer/{__init__.py, _pkv/...}
 
     python -m crit_amd.dropin <dest>          # then: export CRIT_KERNEL_PATH=<dest>  (or replace crit's own folder)
 
@@ -58,6 +63,36 @@ def assemble(dest, library=None):
     for name in ("__init__.py", "_abi.py"):
         shutil.copy(os.path.join(PACKAGE, name), os.path.join(package, name))
     shutil.copy(library, os.path.join(package, "libcrit_pkv.so"))
+    for folder, module in SIBLINGS.items():
+        assemble_sibling(dest, folder, module, library)
+    return root
+
+
+SIBLINGS = {"latent-attention": "latent_attention", "sparse-indexer": "sparse_indexer"}
+
+
+def assemble_sibling(dest, folder, module, library):
+    """The folder of a kernels module that launches through the paged-KV package's binding (its launch helper, its
+    ctypes mirrors, the one library): the loader imports a staged package under another name with nothing beside it,
+    so the package carries a copy of that binding as its subpackage `_pkv` and imports it from there."""
+    source = os.path.join(HERE, module)
+    manifest = json.load(open(os.path.join(source, "kernel.json"), encoding="utf-8"))
+    problems = check_manifest(manifest, folder)
+    if problems:
+        raise ValueError("; ".join(problems))
+    root = os.path.join(dest, folder)
+    package = os.path.join(root, "torch-ext", module)
+    binding = os.path.join(package, "_pkv")
+    os.makedirs(binding, exist_ok=True)
+    shutil.copy(os.path.join(source, "kernel.json"), os.path.join(root, "kernel.json"))
+    text = open(os.path.join(source, "__init__.py"), encoding="utf-8").read()
+    if "from ..paged_kv_attention import" not in text:
+        raise ValueError(f"{module}: no import of the paged-KV binding to stage")
+    with open(os.path.join(package, "__init__.py"), "w", encoding="utf-8") as f:
+        f.write(text.replace("from ..paged_kv_attention import", "from ._pkv import"))
+    for name in ("__init__.py", "_abi.py"):
+        shutil.copy(os.path.join(PACKAGE, name), os.path.join(binding, name))
+    shutil.copy(library, os.path.join(binding, "libcrit_pkv.so"))
     return root
 
 
