@@ -909,8 +909,9 @@ def main():
         log(f"[bench] pool bookkeeping: {extras['pool_bookkeeping_bf16']}")
         torch.cuda.empty_cache()
         extras["latent_attention_decode"] = latent_decode(device)
-        extras["sparse_index_selection"] = index_selection(device)
         log(f"[bench] latent-attention decode: {extras['latent_attention_decode']}")
+        extras["sparse_index_selection"] = index_selection(device)
+        log(f"[bench] sparse index selection: {extras['sparse_index_selection']}")
         result["extra"] = extras
     if not args.no_cpu:
         log("[bench] timing the CPU reference path (about 20 s)")
