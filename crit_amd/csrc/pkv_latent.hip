@@ -334,7 +334,8 @@ __global__ __launch_bounds__(64) void latent_merge_kernel(LatentArgs a) {
 #pragma unroll
     for (int i = 0; i < R / 64; ++i)
         store_out(a.out, a.out_dtype, token * a.o_st + (int64_t)head * a.o_sh + i * 64 + threadIdx.x, acc[i] * inv);
-    if (a.lse && threadIdx.x == 0) a.lse[token * a.heads + head] = L > 0.0f ? (M + __builtin_log2f(L)) * kLn2 : -INFINITY;
+    // (a NaN sum, from a NaN query, stays a NaN: a fault upstream shows in the log-sum-exp as it does in the output)
+    if (a.lse && threadIdx.x == 0) a.lse[token * a.heads + head] = (L > 0.0f || L != L) ? (M + __builtin_log2f(L)) * kLn2 : -INFINITY;
 }
 
 template <int R, int P, int NT>

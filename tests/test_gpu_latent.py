@@ -115,6 +115,20 @@ def test_a_tokens_bits_are_its_own_alone_in_a_window_and_beside_other_rows():
     assert torch.equal(as_slots, together)
 
 
+@pytest.mark.parametrize("heads", [16, 128])
+def test_a_nan_query_reaches_its_own_rows_output_only(heads):
+    cache = Cache(512, 64, 64, [700, 300], seed=4)
+    q = _q(2, heads, 576, 6)
+    clean = cache.attend(q, [0, 1], [0, 1], [650, 250], 1)
+    q[0, 3, 5] = float("nan")
+    lse = torch.empty(2, heads, device=dev)
+    out = cache.attend(q, [0, 1], [0, 1], [650, 250], 1, lse=lse)
+    assert bool(torch.isnan(out[0, 3]).all()) and bool(torch.isnan(lse[0, 3]))
+    keep = torch.ones(heads, dtype=torch.bool, device=dev)
+    keep[3] = False
+    assert torch.equal(out[0][keep], clean[0][keep]) and torch.equal(out[1], clean[1])
+
+
 def test_one_graph_replays_at_every_length():
     cache = Cache(512, 64, 64, [4000], seed=3)
     la = cache.la

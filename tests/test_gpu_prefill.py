@@ -386,6 +386,21 @@ def test_int8_queries_in_a_launch_that_fills_the_chip_equal_one_launch_per_chunk
         assert torch.equal(out[rows], pk.prefill(q[rows], cache.k, cache.v, "int8", cache.tables[s], prefixes[s], 16, **kw)), s
 
 
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 128), (12, 2, 64), (8, 2, 256)])
+def test_a_nan_query_in_a_prompt_chunk_reaches_its_own_tokens_output_only(hq, hkv, d):
+    # a fault upstream shows instead of turning into zeros, and in its own row only (the reference's test_nonfinite.py),
+    # on the matrix-core path (128, 64) and through window rows (256)
+    pk = kernels()
+    cache = Cache("bf16", hkv, d, d, 16, [300])
+    q = rand_q(4, hq, d, 2).bfloat16()
+    lse = torch.empty(4, hq, device=dev)
+    clean = pk.prefill(q, cache.k, cache.v, "bf16", cache.tables[0], 200, 16)
+    q[1, 0, 0] = float("nan")
+    out = pk.prefill(q, cache.k, cache.v, "bf16", cache.tables[0], 200, 16, lse=lse)
+    assert bool(torch.isnan(out[1, 0]).all()) and bool(torch.isnan(lse[1, 0]))
+    assert torch.equal(out[0], clean[0]) and torch.equal(out[2:], clean[2:]) and torch.equal(out[1, 1:], clean[1, 1:])
+
+
 def test_what_the_prompt_reader_does_not_take_is_refused():
     pk = kernels()
     cache = Cache("int8", 2, 128, 128, 16, [40])
