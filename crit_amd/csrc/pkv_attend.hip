@@ -250,9 +250,8 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
         return CRIT_PKV_E_GEOMETRY;
     if (derive) {      // one row is key and value: one width (64 or 128), halves of the rotation in whole lanes
         if (p->head_dim != p->value_dim || (p->head_dim != 64 && p->head_dim != 128) || p->derive_rot < 16 ||
-            p->derive_rot % 16 || p->derive_rot > p->head_dim || !(p->derive_eps >= 0.0f) || p->blocks || p->fresh_keys ||
-            p->fresh_values)
-            return CRIT_PKV_E_GEOMETRY;
+            p->derive_rot % 16 || p->derive_rot > p->head_dim || !(p->derive_eps >= 0.0f) || p->blocks || p->fresh_keys)
+            return CRIT_PKV_E_GEOMETRY;      // (fresh rows come as values only: their keys are derived too)
     }
     const int lpr = (p->head_dim > p->value_dim ? p->head_dim : p->value_dim) / 8;      // lanes that hold the wider row
     const bool wide128 = p->head_dim == 128 && p->value_dim == 128;
@@ -269,11 +268,12 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     if ((p->parents || p->parents64) && p->columns > 64) return CRIT_PKV_E_GEOMETRY;      // an ancestor set is a 64-bit mask
     const bool fresh = p->fresh_keys != nullptr || p->fresh_values != nullptr;
     if (fresh) {
-        if (!p->fresh_keys || !p->fresh_values || !p->fresh_shifts || !p->fresh_firsts) return CRIT_PKV_E_NULL;
+        if ((!p->fresh_keys && !derive) || !p->fresh_values || !p->fresh_shifts || !p->fresh_firsts) return CRIT_PKV_E_NULL;
         if (p->blocks) return CRIT_PKV_E_GEOMETRY;      // (block lists read the pages only, as the reference's)
         const int64_t row = (int64_t)p->kv_heads * p->head_dim, row_v = (int64_t)p->kv_heads * p->value_dim;
-        if (p->fresh_rows < 1 || p->fresh_stride_k < row || p->fresh_stride_v < row_v || p->fresh_stride_k % 8 || p->fresh_stride_v % 8 ||
-            (reinterpret_cast<uintptr_t>(p->fresh_keys) % 16) || (reinterpret_cast<uintptr_t>(p->fresh_values) % 16))
+        if (p->fresh_rows < 1 || p->fresh_stride_v < row_v || p->fresh_stride_v % 8 || (reinterpret_cast<uintptr_t>(p->fresh_values) % 16))
+            return CRIT_PKV_E_GEOMETRY;
+        if (!derive && (p->fresh_stride_k < row || p->fresh_stride_k % 8 || (reinterpret_cast<uintptr_t>(p->fresh_keys) % 16)))
             return CRIT_PKV_E_GEOMETRY;
     }
     AttendArgs a;

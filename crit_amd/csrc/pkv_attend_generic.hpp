@@ -53,7 +53,7 @@ template <int KIND, bool F16, int LPR, int QR, bool FUSED, bool SPARSE = false, 
 __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
     static_assert(!(SPARSE && FUSED), "block lists are read by the split launch");
     static_assert(!(SPARSE && FRESH), "block lists read the pages only");
-    static_assert(!(DERIVE && (SPARSE || FRESH)), "derived keys: windows over the pages, without block lists or fresh rows");
+    static_assert(!(DERIVE && SPARSE), "derived keys: windows without block lists");
     constexpr int D = LPR * 8;         // the wider of the key and value rows
     constexpr int PPI = 64 / LPR;      // positions one load instruction of a wavefront covers
     constexpr int SP = 4 * PPI;        // positions a wavefront's step covers
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
             if constexpr (FRESH) {      // (unconditional too: a position below the first fresh one reads row 0 or its own clamped)
                 int64_t row = (int64_t)n - f_shift;
                 row = row < 0 ? 0 : (row >= a.f_rows ? a.f_rows - 1 : row);
-                buf.f.k[k] = *reinterpret_cast<const uint4*>(a.fk + (row * a.f_stride_k + (int64_t)kvh * dk + lik) * 2);
+                if constexpr (!DERIVE) buf.f.k[k] = *reinterpret_cast<const uint4*>(a.fk + (row * a.f_stride_k + (int64_t)kvh * dk + lik) * 2);
                 buf.f.v[k] = load_once16(a.fv + (row * a.f_stride_v + (int64_t)kvh * dv + liv) * 2);
             }
         }
@@ -250,16 +250,23 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
                 vf[4] = a2.x, vf[5] = a2.y, vf[6] = a3.x, vf[7] = a3.y;
             }
         };
-        // DERIVE: position n's key from its value row.
-        auto derived_key = [&](const StepBuf<KIND, FRESH>& buf, int k, int n, float (&kf)[8]) __attribute__((always_inline)) {
+        // DERIVE: position n's key from its value row (a fresh position's from its fresh value row, as it is given).
+        auto derived_key = [&](const StepBuf<KIND, FRESH>& buf, int k, int n, bool is_fresh, float (&kf)[8]) __attribute__((always_inline)) {
             stored_values(buf, k, kf);
             const float rs = KIND >= 2 ? buf.vs[k] : (KIND == 1 ? v_mult : 1.0f);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) kf[j] *= rs;
+            if constexpr (FRESH) {
+                const uint32_t fw[4] = {buf.f.v[k].x, buf.f.v[k].y, buf.f.v[k].z, buf.f.v[k].w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    kf[2 * j] = is_fresh ? (F16 ? f16_lo(fw[j]) : bf16_lo(fw[j])) : kf[2 * j];
+                    kf[2 * j + 1] = is_fresh ? (F16 ? f16_hi(fw[j]) : bf16_hi(fw[j])) : kf[2 * j + 1];
+                }
+            }
             float ss = 0.0f;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                kf[j] *= rs;
-                ss = __builtin_fmaf(kf[j], kf[j], ss);
-            }
+            for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(kf[j], kf[j], ss);
             ss = group_sum<LPR>(ss);
             const float rn = 1.0f / __builtin_sqrtf(ss / (float)D + a.derive_eps);
             const int half = a.derive_rot >> 4;      // lanes a half of the rotated values takes
@@ -290,7 +297,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
                 float kf[8];
                 if constexpr (DERIVE) {
                     const int n = base + k * PPI + lg;
-                    derived_key(buf, k, n < n_keys ? n : n_keys - 1, kf);
+                    derived_key(buf, k, n < n_keys ? n : n_keys - 1, isf[k], kf);
                 } else if constexpr (KIND == 0) {
                     kw[0] = buf.k[k].x, kw[1] = buf.k[k].y, kw[2] = buf.k[k].z, kw[3] = buf.k[k].w;
                 } else if constexpr (KIND == 3) {
@@ -303,7 +310,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
                     kf[0] = a0.x, kf[1] = a0.y, kf[2] = a1.x, kf[3] = a1.y;
                     kf[4] = a2.x, kf[5] = a2.y, kf[6] = a3.x, kf[7] = a3.y;
                 }
-                if constexpr (FRESH) {
+                if constexpr (FRESH && !DERIVE) {
                     const uint32_t fw[4] = {buf.f.k[k].x, buf.f.k[k].y, buf.f.k[k].z, buf.f.k[k].w};
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {

@@ -38,13 +38,19 @@ static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipS
             return hip_code(hipGetLastError());
         }
     }
-    if (a.derive_table) {      // keys derived from the value rows: the generic kernel's variant for 64- and 128-wide heads
+    if (a.derive_table && a.fv) {      // derived keys over pages and fresh value rows
+        switch (lpr) {
+            case 8: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 8, QR, FUSED, false, true, true>), grid, dim3(256), 0, stream, a); break;
+            case 16: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 16, QR, FUSED, false, true, true>), grid, dim3(256), 0, stream, a); break;
+            default: return CRIT_PKV_E_GEOMETRY;
+        }
+    } else if (a.derive_table) {      // keys derived from the value rows: the generic kernel's variant for 64- and 128-wide heads
         switch (lpr) {
             case 8: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 8, QR, FUSED, false, false, true>), grid, dim3(256), 0, stream, a); break;
             case 16: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 16, QR, FUSED, false, false, true>), grid, dim3(256), 0, stream, a); break;
             default: return CRIT_PKV_E_GEOMETRY;
         }
-    } else if (a.fk) {       // fresh rows beside the pages: the generic kernel's variant that reads both (any head width)
+    } else if (a.fv) {       // fresh rows beside the pages: the generic kernel's variant that reads both (any head width)
         switch (lpr) {
             case 2: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 2, QR, FUSED, false, true>), grid, dim3(256), 0, stream, a); break;
             case 4: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 4, QR, FUSED, false, true>), grid, dim3(256), 0, stream, a); break;

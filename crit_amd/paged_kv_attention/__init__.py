@@ -522,8 +522,8 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
             raise ValueError("derive= reads windows without block lists")
         if key_pages is not None:
             raise ValueError("derive= reads the value pages as keys too: key_pages None")
-        if fresh is not None:
-            raise _unsupported("derive= with fresh rows")
+        if fresh is not None and fresh[0] is not None:
+            raise ValueError("derive= derives the fresh rows' keys from their values too: fresh keys None")
         key_pages = value_pages
     if parents is not None:
         _require_device(parents, "attend's parents")
@@ -628,6 +628,8 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
     p.scale, p.key_multiplier, p.value_multiplier = scale, km, vm
     if fresh is not None:
         fk, fv, fshift, ffirst = fresh
+        if derive is not None:      # (checked as the keys the values stand for: one width)
+            fk = fv
         if not (torch.is_tensor(fk) and torch.is_tensor(fv)) or fk.dim() != 3 or fk.shape[1:] != (hkv, d) or \
                 fv.shape[1:] != (hkv, dv) or fk.shape[0] != fv.shape[0] or fk.shape[0] < 1 or fk.stride(-1) != 1 or \
                 fv.stride(-1) != 1 or fk.stride(1) != d or fv.stride(1) != dv or not torch.is_tensor(fshift) or \
@@ -641,7 +643,7 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
             raise ValueError("a fresh row's shift and first are contiguous int64 tensors on q's device")
         if fk.stride(0) % 8 or fv.stride(0) % 8 or fk.data_ptr() % 16 or fv.data_ptr() % 16:
             raise ValueError("fresh rows 16-byte aligned, their token stride a multiple of 8 elements")
-        p.fresh_keys, p.fresh_values = fk.data_ptr(), fv.data_ptr()
+        p.fresh_keys, p.fresh_values = None if derive is not None else fk.data_ptr(), fv.data_ptr()
         p.fresh_shifts, p.fresh_firsts = fshift.data_ptr(), ffirst.data_ptr()
         p.fresh_stride_k, p.fresh_stride_v, p.fresh_rows = fk.stride(0), fv.stride(0), int(fk.shape[0])
         p.fresh_per_row = int(fshift.numel() != 1)
@@ -694,12 +696,15 @@ def _prefill_state(device, tokens, heads, dim, given):
     return given
 
 
-def _check_fresh(fresh, q, hkv, d, chunks):
+def _check_fresh(fresh, q, hkv, d, chunks, derived=False):
     """(keys, values, firsts or None) of a prompt launch's fresh rows, checked as the reference checks them
-    (__init__.py:1301-1308): [tokens][kv_heads][dim] each in q's dtype, head rows contiguous."""
+    (__init__.py:1301-1308): [tokens][kv_heads][dim] each in q's dtype, head rows contiguous. derived: the keys are
+    derived from the values (keys None)."""
     fk, fv, firsts = fresh
     T = q.shape[0]
-    for name, x in (("keys", fk), ("values", fv)):
+    if derived and fk is not None:
+        raise ValueError("derive= derives the fresh rows' keys from their values too: fresh keys None")
+    for name, x in ((("values", fv),) if derived else (("keys", fk), ("values", fv))):
         if not torch.is_tensor(x) or x.shape != (T, hkv, d) or x.stride(-1) != 1 or x.stride(1) != d:
             raise ValueError(f"fresh keys and values are [{T}][{hkv}][{d}], each head row contiguous")
         if x.dtype != q.dtype or x.device != q.device:
@@ -793,7 +798,7 @@ def _prefill_as_windows(q, key_pages, value_pages, kind, tables, table_rows, sta
     w_rows = table_of[:, None].expand(chunks, per).reshape(-1).to(torch.int32)
     given = None
     if fresh is not None:      # a chunk's own rows sit beside q's tokens: row = position - (chunk position - first token)
-        fk, fv, firsts = _check_fresh(fresh, q, key_pages.shape[-2], q.shape[-1], chunks)
+        fk, fv, firsts = _check_fresh(fresh, q, value_pages.shape[-2], q.shape[-1], chunks, derive is not None)
         shift = positions - first_token
         own = positions if firsts is None else torch.maximum(firsts, positions)
         given = (fk, fv, shift[:, None].expand(chunks, per).reshape(-1).contiguous(),
@@ -832,8 +837,6 @@ def prefill(q, key_pages, value_pages, kind, table, position, page, *, key_scale
             raise ValueError("derive= derives 16-bit keys: not with int8_qk")
         if key_pages is not None:
             raise ValueError("derive= reads the value pages as keys too: key_pages None")
-        if fresh is not None:
-            raise _unsupported("derive= with fresh rows")
     _check_sinks(sinks, q)
     sliding = _check_sliding(sliding, None)
     T = q.shape[0]
@@ -861,7 +864,7 @@ def prefill(q, key_pages, value_pages, kind, table, position, page, *, key_scale
         fresh = (fresh[0], fresh[1], first)
     if derive is not None:
         return _prefill_as_windows(q, None, value_pages, kind, table.reshape(1, -1), None, None, None, positions, T, 1, page,
-                                   None, value_scales, multipliers, scale, out, lse, sinks, sliding, None, False, derive)
+                                   None, value_scales, multipliers, scale, out, lse, sinks, sliding, fresh, False, derive)
     return _prefill_launch(q, key_pages, value_pages, kind, table.reshape(1, -1), None, None, None, positions, T, 1,
                            page, key_scales, value_scales, multipliers, scale, out, lse, sinks, sliding, fresh,
                            workspace, int8_qk)

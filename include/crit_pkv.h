@@ -176,7 +176,8 @@ typedef struct crit_pkv_attend_params {
      * angle fp32(position) * freqs[i], all in FP32. derive_table: FP32 freqs [derive_rot / 2], then, with
      * derive_weighted, the weight [head_dim]; NULL: keys from key_pages. With it key_pages and key_scales are not
      * read (may be NULL); head_dim == value_dim, 64 or 128; derive_rot a multiple of 16 up to head_dim (the reference
-     * takes any even width); no blocks, no fresh rows. */
+     * takes any even width); no blocks. Fresh rows come as values only (fresh_keys NULL): a fresh position's key is
+     * derived from its fresh value row. */
     const float* derive_table;
     float derive_eps;
     int32_t derive_rot;

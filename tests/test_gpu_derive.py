@@ -164,6 +164,70 @@ def test_a_prompt_chunk_with_derived_keys_is_its_positions_decoded(kind, d):
     assert torch.equal(on_device, out)
 
 
+def _check_with_fresh(cache, q, out, lse, derive, fv, at, split, tokens, window=0):
+    """Tokens of a chunk at position `at` whose positions from at + split on are the fresh value rows fv[split:]: float64
+    attention over the stored rows then the fresh ones, every key derived from its row."""
+    weight, eps, freqs, rot = derive[:4]
+    values = torch.cat([cache.stored(0, at + split), fv[split:].double().cpu()])
+    keys = oracle_attend.derived_keys(values, None if weight is None else weight.cpu(), eps, freqs.cpu(), rot)
+    qd = q.double().cpu()
+    n = torch.arange(at + fv.shape[0])
+    for t in tokens:
+        seen = n <= at + t
+        if window:
+            seen = seen & (n > at + t - window)
+        want, want_lse = oracle_attend.reference(qd[t], keys, values, seen, cache.d ** -0.5)
+        torch.testing.assert_close(out[t].double().cpu(), want, atol=8e-3, rtol=2e-2, msg=f"{at} {split} {window} {t}")
+        torch.testing.assert_close(lse[t].double().cpu(), want_lse, atol=1e-3, rtol=1e-4, msg=f"lse {at} {split} {window} {t}")
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_a_fused_chunk_derives_its_fresh_rows_keys(kind):
+    # a chunk's own positions come as fresh value rows (keys None): their keys are derived as the stored rows' are
+    # (the reference's test of the same name): two window rows of one chunk, the frontier and first on the device
+    cache = Rows(kind, 2, 128, 16, [700], multiplier=0.04)
+    pk = cache.pk
+    derive = derive_for(pk, 128, 128)
+    g = torch.Generator().manual_seed(21)
+    T = 100
+    q = rand_q(T, 8, 128, 22).to(cache.q_dtype)
+    fv = torch.randn(T, 2, 128, generator=g).to(dev).to(cache.q_dtype)
+    frontier = torch.zeros(1, dtype=torch.int64, device=dev)
+    first = torch.zeros(1, dtype=torch.int64, device=dev)
+    starts = torch.tensor([0, 64], dtype=torch.int32, device=dev)
+    counts = torch.tensor([64, T - 64], dtype=torch.int32, device=dev)
+    rows = torch.zeros(2, dtype=torch.int32, device=dev)
+    for at in (0, 200, 600):
+        for split in (0, 37, 100):
+            frontier.fill_(at)
+            first.fill_(at + split)
+            lse = torch.empty(T, 8, device=dev)
+            out = pk.attend(q, None, cache.v, kind, cache.tables, rows, starts,
+                            torch.tensor([at, at + 64], dtype=torch.int64, device=dev), 64, 16, counts=counts,
+                            value_scales=cache.vs, multipliers=cache.multipliers, lse=lse, fused=True,
+                            fresh=(None, fv, frontier, first), derive=derive)
+            _check_with_fresh(cache, q, out, lse, derive, fv, at, split, (0, 41, 99))
+    with pytest.raises(ValueError, match="fresh keys None"):
+        pk.attend(q, None, cache.v, kind, cache.tables, rows, starts, torch.tensor([0, 64], dtype=torch.int64, device=dev), 64,
+                  16, counts=counts, value_scales=cache.vs, multipliers=cache.multipliers, fused=True,
+                  fresh=(fv, fv, frontier, first), derive=derive)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_a_prompt_chunk_derives_its_fresh_rows_keys_with_a_sliding_window(kind):
+    cache = Rows(kind, 2, 128, 16, [700])
+    pk = cache.pk
+    derive = derive_for(pk, 128, 64)
+    g = torch.Generator().manual_seed(21)
+    q = rand_q(100, 8, 128, 22).to(cache.q_dtype)
+    fv = torch.randn(100, 2, 128, generator=g).to(dev).to(cache.q_dtype)
+    for at, split, window in ((0, 0, 0), (200, 37, 0), (600, 100, 0), (200, 37, 50)):
+        lse = torch.empty(100, 8, device=dev)
+        out = pk.prefill(q, None, cache.v, kind, cache.tables[0], at, 16, value_scales=cache.vs, multipliers=cache.multipliers,
+                         lse=lse, fresh=(None, fv, at + split), derive=derive, sliding=window)
+        _check_with_fresh(cache, q, out, lse, derive, fv, at, split, (0, 41, 99), window)
+
+
 def test_what_derived_keys_do_not_take_is_refused():
     pk = kernels()
     cache = Rows("bf16", 2, 128, 16, [40])
