@@ -146,6 +146,8 @@ def select(q, keys, weights, ends, k, *, key_scales=None, scale=None, out: Optio
     n = keys.shape[0] if slots is None else slots.shape[0]
     if out is None:
         out = torch.empty(t, k, dtype=torch.int32, device=q.device)
+    if out.shape != (t, k) or out.dtype != torch.int32 or out.stride(-1) != 1:
+        raise ValueError(f"out is int32 [{t}][{k}]")
     if t == 0:
         return out
     if n == 0:
