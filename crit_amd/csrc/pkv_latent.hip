@@ -210,31 +210,59 @@ __global__ __launch_bounds__(256, NT == 1 ? 3 : 2) void latent_kernel(LatentArgs
             after = advance();
             if (after >= 0) fetch_entry(after);
         }
-        // -- the step's scores: this wavefront's chains of its tile, both 16-position halves of the step
+        // -- the step's scores: this wavefront's chains of its tile, both 16-position halves of the step. The operands are
+        // read from LDS a few products ahead (a ring), so a read's latency is not waited for before every product. A
+        // chain's k-step past the last (the wavefronts do not all have as many) multiplies the last one's rows by the
+        // zeros its queries hold there.
         const uint8_t* krow = s_k + li * ROWB + g * 16;
+        {
+            constexpr int NOPS = NT * KPC;
+            constexpr int RING = NOPS < 4 ? NOPS : 4;
+            u32x4 ka[RING][2];
+            f32x4 sl[NT][2], sr[NT][2];
 #pragma unroll
-        for (int c = 0; c < NT; ++c) {
-            f32x4 sl0 = {0.0f, 0.0f, 0.0f, 0.0f}, sl1 = sl0, sr0 = sl0, sr1 = sl0;
+            for (int c = 0; c < NT; ++c)
 #pragma unroll
-            for (int k4 = 0; k4 < KPC; ++k4) {
-                const int ks = k4 * 4 + sub + c * WPT;
-                if (ks < KS) {
-                    const u32x4 a0 = *reinterpret_cast<const u32x4*>(krow + ks * 64);
-                    const u32x4 a1 = *reinterpret_cast<const u32x4*>(krow + 16 * ROWB + ks * 64);
-                    if (FP8 && ks >= KSL) {
-                        sr0 = mfma_k32<F16>(a0, bq[c][k4], sr0);
-                        sr1 = mfma_k32<F16>(a1, bq[c][k4], sr1);
-                    } else {
-                        sl0 = mfma_k32<F16>(a0, bq[c][k4], sl0);
-                        sl1 = mfma_k32<F16>(a1, bq[c][k4], sl1);
-                    }
+                for (int hh = 0; hh < 2; ++hh) sl[c][hh] = f32x4{0.0f, 0.0f, 0.0f, 0.0f}, sr[c][hh] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            auto read_k = [&](auto ic) __attribute__((always_inline)) {
+                constexpr int i = decltype(ic)::value;
+                constexpr int c = i / KPC, k4 = i % KPC;
+                int ks = k4 * 4 + sub + c * WPT;
+                ks = ks < KS ? ks : KS - 1;
+                ka[i % RING][0] = *reinterpret_cast<const u32x4*>(krow + ks * 64);
+                ka[i % RING][1] = *reinterpret_cast<const u32x4*>(krow + 16 * ROWB + ks * 64);
+            };
+            static_for<RING - 1>([&](auto ic) __attribute__((always_inline)) { read_k(ic); });
+            static_for<NOPS>([&](auto ic) __attribute__((always_inline)) {
+                constexpr int i = decltype(ic)::value;
+                constexpr int c = i / KPC, k4 = i % KPC;
+                if constexpr (i + RING - 1 < NOPS) read_k(std::integral_constant<int, i + RING - 1>{});
+                // (k-steps from KSL on are the rotary key's: a chain's k4 decides where the latent's k-steps come in fours)
+                const bool rotary = FP8 && (KSL % 4 == 0 ? k4 * 4 >= KSL : k4 * 4 + sub + c * WPT >= KSL);
+                if (rotary) {
+                    sr[c][0] = mfma_k32<F16>(ka[i % RING][0], bq[c][k4], sr[c][0]);
+                    sr[c][1] = mfma_k32<F16>(ka[i % RING][1], bq[c][k4], sr[c][1]);
+                } else {
+                    sl[c][0] = mfma_k32<F16>(ka[i % RING][0], bq[c][k4], sl[c][0]);
+                    sl[c][1] = mfma_k32<F16>(ka[i % RING][1], bq[c][k4], sl[c][1]);
                 }
-            }
-            float (&mine)[NPART][64] = s_part[wt][sub + c * WPT];
+            });
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 * (RING - 1), 0);
+            static_for<NOPS>([&](auto) __attribute__((always_inline)) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            });
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                mine[i][lane] = sl0[i], mine[4 + i][lane] = sl1[i];
-                if constexpr (FP8) mine[8 + i][lane] = sr0[i], mine[12 + i][lane] = sr1[i];
+            for (int c = 0; c < NT; ++c) {
+                float (&mine)[NPART][64] = s_part[wt][sub + c * WPT];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    mine[i][lane] = sl[c][0][i], mine[4 + i][lane] = sl[c][1][i];
+                    if constexpr (FP8) mine[8 + i][lane] = sr[c][0][i], mine[12 + i][lane] = sr[c][1][i];
+                }
             }
         }
         lds_barrier();
@@ -274,14 +302,31 @@ __global__ __launch_bounds__(256, NT == 1 ? 3 : 2) void latent_kernel(LatentArgs
         const u32x4 bp = {pair16<F16>(p[0], p[1]), pair16<F16>(p[2], p[3]), pair16<F16>(p[4], p[5]), pair16<F16>(p[6], p[7])};
         // -- the wavefront's share of the values (the accumulators move only when some row's maximum did: x 1 is exact)
         const bool rescale = __ballot(alpha != 1.0f) != 0ull;
-        const uint8_t* vrow = s_k + (4 * g + (li >> 2)) * ROWB + (li & 3) * 8;
+        const uint8_t* vrow = s_k + (4 * g + (li >> 2)) * ROWB + (li & 3) * 8 + sub * FT * 32;
+        if (rescale) {
 #pragma unroll
-        for (int t = 0; t < FT; ++t) {
-            const int ftile = sub * FT + t;
-            const u32x2 lo = lds_transposed(vrow + ftile * 32);
-            const u32x2 hi = lds_transposed(vrow + 16 * ROWB + ftile * 32);
-            if (rescale) acc[t] *= alpha;
-            acc[t] = mfma_k32<F16>(u32x4{lo.x, lo.y, hi.x, hi.y}, bp, acc[t]);
+            for (int t = 0; t < FT; ++t) acc[t] *= alpha;
+        }
+        {
+            constexpr int VR = FT < 5 ? FT : 5;      // value operands read ahead, as the keys' are
+            u32x2 va[VR][2];
+            auto read_v = [&](auto ic) __attribute__((always_inline)) {
+                constexpr int t = decltype(ic)::value;
+                va[t % VR][0] = lds_transposed(vrow + t * 32);
+                va[t % VR][1] = lds_transposed(vrow + 16 * ROWB + t * 32);
+            };
+            static_for<VR - 1>([&](auto ic) __attribute__((always_inline)) { read_v(ic); });
+            static_for<FT>([&](auto ic) __attribute__((always_inline)) {
+                constexpr int t = decltype(ic)::value;
+                if constexpr (t + VR - 1 < FT) read_v(std::integral_constant<int, t + VR - 1>{});
+                acc[t] = mfma_k32<F16>(u32x4{va[t % VR][0].x, va[t % VR][0].y, va[t % VR][1].x, va[t % VR][1].y}, bp, acc[t]);
+            });
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 * (VR - 1), 0);
+            static_for<FT>([&](auto) __attribute__((always_inline)) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            });
+            __builtin_amdgcn_sched_barrier(0);
         }
         lds_barrier();      // (the barriers order LDS only: the next step's loads stay in flight across them)
         base = next, next = after;
