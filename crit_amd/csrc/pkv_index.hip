@@ -43,23 +43,32 @@ struct ScoreArgs {
     float scale;
 };
 
-// One token's queries: qa[ht][ks] the lane's A operand (head ht * 16 + li, values ks * 32 + 8 g .. + 7), heads past the
-// last as zeros.
+// One token's queries: qa[ht][ks] the lane's A operand (head ht * 16 + li, 8 adjacent values per k-step), heads past
+// the last as zeros. Which 8 values: the ones the lane's key operand holds at that step. 16-bit keys: values
+// ks * 32 + 8 g .. + 7 (a lane loads 16 bytes of its key a step). E4M3 keys: a lane loads 16 bytes, 16 values, for a
+// pair of steps, so steps 2 j and 2 j + 1 take values 64 j + 16 g .. + 7 and + 8 .. + 15 (a sum over the values in
+// another order; both kernels use the same one).
 template <int HT, int KS>
 struct TokenQ {
     u32x4 qa[HT][KS];
 };
 
-template <int HT, int KS>
+// Where in a head's row of 16-bit queries (in bytes) the lane's operand of step ks starts.
+template <bool FP8>
+PKV_DEV constexpr int q_offset(int ks, int g) {
+    return FP8 ? (ks >> 1) * 128 + g * 32 + (ks & 1) * 16 : ks * 64 + g * 16;
+}
+
+template <bool FP8, int HT, int KS>
 PKV_DEV void load_token(const ScoreArgs& a, int t, int g, int li, TokenQ<HT, KS>& q) {
 #pragma unroll
     for (int ht = 0; ht < HT; ++ht) {
         const int h = ht * 16 + li;
-        const uint8_t* row = a.q + ((int64_t)t * a.q_st + (int64_t)h * a.q_sh) * 2 + g * 16;
+        const uint8_t* row = a.q + ((int64_t)t * a.q_st + (int64_t)h * a.q_sh) * 2;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             u32x4 w = {0u, 0u, 0u, 0u};
-            if (h < a.heads) w = *reinterpret_cast<const u32x4*>(row + ks * 64);
+            if (h < a.heads) w = *reinterpret_cast<const u32x4*>(row + q_offset<FP8>(ks, g));
             q.qa[ht][ks] = w;
         }
     }
@@ -111,7 +120,7 @@ PKV_DEV int64_t slot_of(const ScoreArgs& a, int64_t srow, int key) {
     return a.slots_are_64 ? reinterpret_cast<const int64_t*>(a.slots)[srow + key] : (int64_t) reinterpret_cast<const int32_t*>(a.slots)[srow + key];
 }
 
-template <bool F16, bool FP8, int HT, int KS>
+template <bool F16, bool FP8, int HT, int KS, int PD>
 __global__ __launch_bounds__(256) void index_scores_kernel(ScoreArgs a) {
     constexpr int QROWB = KS * 64 + (HT * KS == 64 ? 0 : 16);      // a head's row in LDS (padded where that keeps it within 64 KB)
     __shared__ __align__(16) uint8_t s_q[HT * 16 * QROWB];
@@ -134,41 +143,71 @@ __global__ __launch_bounds__(256) void index_scores_kernel(ScoreArgs a) {
     const int first = blockIdx.x * a.block;
     const int last = min(first + a.block, a.n);
     float* out = a.out + (int64_t)t * a.out_stride;
-    using Raw = typename std::conditional<FP8, u32x2, u32x4>::type;
-    Raw held[KS];
-    int64_t held_at = 0;
-    auto fetch = [&](int k0) {      // the lane's key of the tile (a key past the last reads the last)
-        held_at = slot_of(a, srow, min(k0 + li, a.n - 1));
-        const uint8_t* krow = a.keys + held_at * a.key_stride * (FP8 ? 1 : 2) + g * (FP8 ? 8 : 16);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) held[ks] = *reinterpret_cast<const Raw*>(krow + ks * (FP8 ? 32 : 64));
+    constexpr int LD = FP8 ? KS / 2 : KS;      // 16-byte loads a key a lane
+    // The wavefront's tiles (wave, wave + 4, ... of the block's tiles of 16 keys) that hold a key the token sees go
+    // through a pipeline of PD stages: a tile's key row is requested PD tiles before its products and its slot is
+    // looked up PD tiles before that (loads return in order: a slot wanted sooner would wait for every row requested
+    // after it), and every load of the loop is issued whether or not its tile exists (past the last one it repeats
+    // the last), so the waits are exact counts. Tiles wholly past the token's end are only written. PD: 3 where a
+    // wavefront has tiles enough, else 1.
+    const int seen_last = min(last, end);      // keys below it are seen
+    const int n_tiles = seen_last > first + wave * 16 ? (seen_last - first - wave * 16 + 63) / 64 : 0;
+    auto tile_k0 = [&](int i) { return first + (wave + 4 * i) * 16; };
+    auto slot_load = [&](int i) -> int64_t {
+        const int ii = i < n_tiles ? i : n_tiles - 1;
+        return slot_of(a, srow, min(tile_k0(ii) + li, a.n - 1));
     };
-    int k0 = first + wave * 16;
-    if (k0 < last && k0 < end) fetch(k0);
+    u32x4 held[PD][LD];
+    int64_t at_s[PD];
+    float ksc[PD];
+    auto row_load = [&](auto sc, int64_t at) __attribute__((always_inline)) {
+        constexpr int st = decltype(sc)::value;
+        at_s[st] = at;
+        const uint8_t* krow = a.keys + at * a.key_stride * (FP8 ? 1 : 2) + g * 16;
+#pragma unroll
+        for (int j = 0; j < LD; ++j) held[st][j] = *reinterpret_cast<const u32x4*>(krow + j * 64);
+        if constexpr (FP8) ksc[st] = a.key_scales[at];
+    };
+    int64_t ahead[PD];      // the slots of the tiles PD past the ones whose rows are in flight
+    if (n_tiles > 0) {
+        static_for<PD>([&](auto sc) __attribute__((always_inline)) { row_load(sc, slot_load(decltype(sc)::value)); });
+        static_for<PD>([&](auto sc) __attribute__((always_inline)) { ahead[decltype(sc)::value] = slot_load(PD + decltype(sc)::value); });
+    }
     __syncthreads();
     TokenQ<HT, KS> q;
 #pragma unroll
     for (int ht = 0; ht < HT; ++ht)
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) q.qa[ht][ks] = *reinterpret_cast<const u32x4*>(s_q + (ht * 16 + li) * QROWB + ks * 64 + g * 16);
-    for (; k0 < last; k0 += 64) {
-        const int kk = k0 + li;
-        if (k0 >= end) {      // nothing of the tile is seen (nor of the wavefront's later ones)
-            if (g == 0 && kk < last) out[kk] = -INFINITY;
-            continue;
-        }
-        u32x4 kb[KS];
+        for (int ks = 0; ks < KS; ++ks) q.qa[ht][ks] = *reinterpret_cast<const u32x4*>(s_q + (ht * 16 + li) * QROWB + q_offset<FP8>(ks, g));
+    for (int i = 0; i < n_tiles; i += PD) {
+        static_for<PD>([&](auto sc) __attribute__((always_inline)) {
+            constexpr int st = decltype(sc)::value;
+            const int ii = i + st;
+            u32x4 kb[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            if constexpr (FP8) kb[ks] = key_operand<F16, true>(u32x4{}, held[ks]);
-            else kb[ks] = held[ks];
-        }
-        const int64_t at = held_at;
-        if (k0 + 64 < last && k0 + 64 < end) fetch(k0 + 64);
-        float v = tile_score<F16>(q, kb, [&](int ht) { return fac[ht]; });
-        if constexpr (FP8) v *= a.key_scales[at];
-        if (g == 0 && kk < last) out[kk] = kk < end ? v : -INFINITY;
+            for (int ks = 0; ks < KS; ++ks) {
+                if constexpr (FP8) {
+                    const u32x4 w = held[st][ks >> 1];
+                    kb[ks] = key_operand<F16, true>(u32x4{}, (ks & 1) ? u32x2{w.z, w.w} : u32x2{w.x, w.y});
+                } else {
+                    kb[ks] = held[st][ks];
+                }
+            }
+            float scale_of_key = 1.0f;
+            if constexpr (FP8) scale_of_key = ksc[st];
+            if (PD > 1 || ii + PD < n_tiles) {      // (one stage: only the tiles there are; more: every load, see above)
+                row_load(sc, ahead[st]);            // tile ii + PD's row (a tile past the last: the last one's again)
+                ahead[st] = slot_load(ii + 2 * PD);
+            }
+            float v = tile_score<F16>(q, kb, [&](int ht) { return fac[ht]; });
+            if constexpr (FP8) v *= scale_of_key;
+            const int kk = tile_k0(ii) + li;
+            if (ii < n_tiles && g == 0 && kk < last) out[kk] = kk < end ? v : -INFINITY;
+        });
     }
+    // the wavefront's tiles wholly at or past the token's end
+    for (int k0 = tile_k0(n_tiles); k0 < last; k0 += 64)
+        if (g == 0 && k0 + li < last) out[k0 + li] = -INFINITY;
 }
 
 template <bool F16, bool FP8, int HT, int KS, int TW>
@@ -192,7 +231,7 @@ __global__ __launch_bounds__(256, HT * KS * TW <= 32 ? 2 : 1) void index_scores_
         const int t = wg_first + wave * TW + j;
         live[j] = t < a.tokens;
         const int tt = live[j] ? t : a.tokens - 1;
-        load_token(a, tt, g, li, q[j]);
+        load_token<FP8>(a, tt, g, li, q[j]);
         ends[j] = live[j] ? min(max(a.ends[tt], 0), a.n) : 0;
         wave_end = max(wave_end, ends[j]);
     }
@@ -237,12 +276,18 @@ __global__ __launch_bounds__(256, HT * KS * TW <= 32 ? 2 : 1) void index_scores_
                 for (int ht = 0; ht < HT; ++ht) fac[j][ht] = *reinterpret_cast<const f32x4*>(s_f + (wave * TW + j) * HP + ht * 16 + 4 * g);
 #pragma unroll
             for (int T = 0; T < 4; ++T) {
-                const uint8_t* krow = s_k + buf * (64 * ROWB) + (T * 16 + li) * ROWB + g * (8 * E);
+                const uint8_t* krow = s_k + buf * (64 * ROWB) + (T * 16 + li) * ROWB + g * 16;
                 u32x4 kb[KS];
+                if constexpr (FP8) {
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    if constexpr (FP8) kb[ks] = key_operand<F16, true>(u32x4{}, *reinterpret_cast<const u32x2*>(krow + ks * 32));
-                    else kb[ks] = *reinterpret_cast<const u32x4*>(krow + ks * 64);
+                    for (int j = 0; j < KS / 2; ++j) {
+                        const u32x4 w = *reinterpret_cast<const u32x4*>(krow + j * 64);
+                        kb[2 * j] = key_operand<F16, true>(u32x4{}, u32x2{w.x, w.y});
+                        kb[2 * j + 1] = key_operand<F16, true>(u32x4{}, u32x2{w.z, w.w});
+                    }
+                } else {
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) kb[ks] = *reinterpret_cast<const u32x4*>(krow + ks * 64);
                 }
 #pragma unroll
                 for (int j = 0; j < TW; ++j) {
@@ -523,12 +568,34 @@ __global__ __launch_bounds__(1024) void index_topk_held_kernel(TopkArgs a) {
 template <bool F16, bool FP8, int HT, int KS>
 int launch_scores_shape(ScoreArgs a, bool many, int cus, hipStream_t stream) {
     if (!many) {
-        // a block of keys a workgroup: enough workgroups for the chip
-        int block = 64;
-        while (block < 4096 && (int64_t)a.tokens * ((a.n + block - 1) / block) > (int64_t)cus * 2) block *= 2;
+        // A block of keys a workgroup, sized so that the workgroups are as many as the chip holds at once (or a whole
+        // number of times that many): every one runs from the start and they end together. Three tiles in flight a
+        // wavefront where it has six or more and the queries leave the registers room.
+        static int held_at_once[2] = {0, 0};      // workgroups a compute unit holds, by kernel (the chips of a process are alike)
+        auto resident = [&](int deep) -> int {
+            if (!held_at_once[deep]) {
+                int count = 0;
+                const hipError_t e = deep ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&count, index_scores_kernel<F16, FP8, HT, KS, 3>, 256, 0)
+                                          : hipOccupancyMaxActiveBlocksPerMultiprocessor(&count, index_scores_kernel<F16, FP8, HT, KS, 1>, 256, 0);
+                held_at_once[deep] = e == hipSuccess && count > 0 ? count : 1;
+            }
+            return held_at_once[deep];
+        };
+        auto block_for = [&](int deep) -> int {
+            const int64_t room = (int64_t)cus * resident(deep);
+            const int64_t fewest = ((int64_t)a.n + 8191) / 8192;      // blocks a token: none above 8,192 keys
+            const int64_t rounds = max((fewest * a.tokens + room - 1) / room, (int64_t)1);
+            const int64_t blocks = max(room * rounds / a.tokens, fewest);
+            return (int)(((a.n + blocks - 1) / blocks + 63) / 64 * 64);
+        };
+        const bool room_for_three = HT * KS <= 32;
+        int block = block_for(room_for_three ? 1 : 0);
+        const bool deep = room_for_three && block >= 384;
+        if (room_for_three && !deep) block = block_for(0);
         a.block = block;
         const dim3 grid((unsigned)((a.n + block - 1) / block), (unsigned)a.tokens);
-        hipLaunchKernelGGL((index_scores_kernel<F16, FP8, HT, KS>), grid, dim3(256), 0, stream, a);
+        if (deep) hipLaunchKernelGGL((index_scores_kernel<F16, FP8, HT, KS, 3>), grid, dim3(256), 0, stream, a);
+        else hipLaunchKernelGGL((index_scores_kernel<F16, FP8, HT, KS, 1>), grid, dim3(256), 0, stream, a);
         return hip_code(hipGetLastError());
     }
     constexpr int TW = HT * KS <= 16 && HT <= 4 ? 2 : 1;      // two tokens a wavefront where their queries fit its registers
