@@ -248,3 +248,53 @@ def test_it_refuses_what_it_does_not_take():
         si.topk(torch.zeros(2, 10, device=dev), ends, 0)
     with pytest.raises(ValueError):
         si.scores(q.cpu(), keys.cpu(), w.cpu(), ends.cpu())              # there is no CPU path
+
+
+@pytest.mark.parametrize("kind,fp8_keys", [("bf16", False), ("fp8", True)])
+def test_a_sparse_decode_step_reads_the_blocks_the_index_selects(kind, fp8_keys):
+    # What the reference's sparse reader does with the two modules (inference/attention-state/code/sparse_index.py, then
+    # paged_kv_attention.attend(blocks=)): four decode tokens of one sequence of 4,000 positions, one index key per
+    # block of 64 positions; each token scores the blocks it may see, its 8 best become its block list, and the
+    # attention reads those blocks only. The picks against the oracle's, the attention against float64 attention over
+    # the listed blocks.
+    from tests.support import Cache, rand_q
+    block, n_pos, k = 64, 4000, 8
+    n_blocks = -(-n_pos // block)
+    cache = Cache(kind, 2, 128, 128, 16, [n_pos])
+    q, keys, scales, values, w, _ = problem(4, 16, 64, n_blocks, seed=21, fp8=fp8_keys)
+    firsts = n_pos - 4
+    ends = torch.tensor([(firsts + t) // block + 1 for t in range(4)], dtype=torch.int32, device=dev)   # the blocks a token may see
+    picked = si.select(q, keys, w, ends, k, key_scales=scales)
+    assert picked.dtype == torch.int32 and picked.shape == (4, k)
+    want_scores = oracle_scores(q, values, w, ends, 64 ** -0.5)
+    exact = ref.sparse_index(want_scores, ends.cpu().numpy(), k)
+    for t in range(4):
+        a, b = set(picked[t].tolist()), set(exact[t].tolist())
+        if a != b:      # a pick that differs scores within the products' error of the k-th
+            assert float(want_scores[t][list(a - b)].min()) >= float(want_scores[t][list(b)].min()) - 1e-3, t
+    qa = rand_q(4, 8, 128, 5)
+    lse = torch.empty(4, 8, device=dev)
+    zero = torch.zeros(1, dtype=torch.int32, device=dev)
+    at = torch.tensor([firsts], dtype=torch.int64, device=dev)
+    out = cache.attend(qa, zero, zero, at, 4, blocks=picked, block_size=block, lse=lse, partitions=4)
+    want, want_lse = cache.want(qa.to(torch.bfloat16), 0, firsts, 4, blocks=picked.cpu(), block_size=block)
+    torch.testing.assert_close(out.double().cpu(), want, atol=8e-3, rtol=2e-2)
+    torch.testing.assert_close(lse.double().cpu(), want_lse, atol=1e-3, rtol=1e-4)
+    # the same step as one captured graph: no host work between the index and the attention
+    graph = torch.cuda.CUDAGraph()
+    again, picked_again = torch.empty_like(out), torch.empty_like(picked)
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        si.select(q, keys, w, ends, k, key_scales=scales, out=picked_again)
+        cache.attend(qa, zero, zero, at, 4, blocks=picked_again, block_size=block, partitions=4, out=again)
+        torch.cuda.synchronize()
+        picked_again.fill_(-1), again.zero_()
+        with torch.cuda.graph(graph, stream=stream):
+            si.select(q, keys, w, ends, k, key_scales=scales, out=picked_again)
+            cache.attend(qa, zero, zero, at, 4, blocks=picked_again, block_size=block, partitions=4, out=again)
+    for _ in range(2):
+        picked_again.fill_(-1), again.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(picked_again, picked) and torch.equal(again, out)
