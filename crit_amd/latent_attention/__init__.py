@@ -24,6 +24,11 @@ import torch
 from ..paged_kv_attention import _abi
 from ..paged_kv_attention import _launch, _ptr, _require_device
 
+try:        # crit's kernel build writes the engine's tuned knobs beside the module (kernels/crit_kernels/build.py:255-313)
+    from . import _crit_tuning
+except ImportError:
+    _crit_tuning = None
+
 __all__ = ["MAX_COLUMNS", "PARTIAL_BYTES", "PIECE", "SHAPES", "attend", "partitions", "prefill", "write"]
 
 MAX_COLUMNS = 64
@@ -44,11 +49,27 @@ def _cus(device):
     return _CUS[index]
 
 
+def _knob(name, heads, rank, rope, page, kind):
+    """The engine's tuned value of a knob of the "window" structure for this geometry, 0 where it has none (the
+    reference's _knobs(), __init__.py:44-50)."""
+    if _crit_tuning is None:
+        return 0
+    key = {"R": int(rank), "P": int(rope), "H": int(heads), "PAGE": int(page), "KIND": int(kind)}
+    return int(_crit_tuning.knobs("window", key, 1).get(name, 0) or 0)
+
+
 def partitions(device, heads, rank, rope, page, kind=0):
-    """The partitions a launch over this geometry splits a row's positions into: about one workgroup a compute unit
-    for one decode token (the CUs over the heads' 16-row tiles), 1 to MAX_PARTS, from the heads and the device only
-    (every partition's state is a partial the merge reads: more of them cost a batch more than they give a lone row)."""
-    return max(1, min(MAX_PARTS, _cus(device) // max(1, -(-int(heads) // 16))))
+    """The partitions a launch over this geometry splits a row's positions into: the tuning's PARTS, else the rule:
+    the CUs over twice the heads' 16-row tiles, 1 to MAX_PARTS, from the heads and the device only (the reference's:
+    2 x SMs over the tiles, __init__.py:65-71). Every partition's state is a partial the merge reads again, and a
+    row's tiles all write theirs: measured on MI355X (64 rows of 1,024 to 8,192 positions, R 512, P 64) 128 heads
+    take 356 / 294 / 261 us with 32 / 16 / 8 partitions and a lone row of 8,192 positions 34 / 42 / 67 us; 16 heads
+    102 / 97 / 89 us with 64 / 16 / 8 and a lone row 28 / 36 / 57 us. The rule gives 64, 64, 32, 16 for 16, 32, 64
+    and 128 heads; an engine that serves batches only sets PARTS lower."""
+    tuned = _knob("PARTS", heads, rank, rope, page, kind)
+    if tuned:
+        return max(1, min(MAX_PARTS, tuned))
+    return max(1, min(MAX_PARTS, _cus(device) // (2 * max(1, -(-int(heads) // 16)))))
 
 
 def write(latent, rope, slots, cache, scales=None):
@@ -115,7 +136,7 @@ def _workspace(device, floats):
 def attend(q, cache, tables, rows, starts, firsts, columns, page, *, rank, counts=None, scale=None,
            out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
            sinks: Optional[torch.Tensor] = None, scales: Optional[torch.Tensor] = None,
-           fused: Optional[bool] = None, piece=None, phases=0) -> torch.Tensor:
+           fused: Optional[bool] = None, piece=None, partitions=None, phases=0) -> torch.Tensor:
     """Decode tokens and verify windows over the latent cache (see the module's description). q [tokens][heads][R + P]
     BF16 or FP16 in the cache's dtype, the last dimension contiguous; cache [pages][page][R + P] contiguous; tables
     [S][width] int32; rows, starts [B] int32 (rows int64 too: a round's slots as they are); firsts [B] int64; counts [B]
@@ -124,8 +145,9 @@ def attend(q, cache, tables, rows, starts, firsts, columns, page, *, rank, count
     [heads]. scale defaults to (R + P) ** -0.5 (pass the model's). An E4M3 cache takes its scales, with BF16 or FP16
     queries: write()'s two a position, or one a position for the whole row ([pages][page][1], a KV pool's fp8:row pages
     of one head). fused: the same bits whatever it says; the rows are launched a few at a time where their partials
-    would take more than PARTIAL_BYTES. piece: positions a piece (a multiple of 32; default PIECE; a token's bits
-    depend on it). phases (a measurement's): 1 the partitions' launch only, 2 the merge only."""
+    would take more than PARTIAL_BYTES. piece: positions a piece (a multiple of 32; default the tuning's PIECE, else
+    PIECE), partitions: 1 to MAX_PARTS (default partitions()); a token's bits depend on both, so a caller keeps one
+    value of each for a geometry. phases (a measurement's): 1 the partitions' launch only, 2 the merge only."""
     R, P, fp8 = _check(q, cache, page, rank, sinks, scales)
     T, H, width = q.shape
     B = int(starts.shape[0])
@@ -135,10 +157,12 @@ def attend(q, cache, tables, rows, starts, firsts, columns, page, *, rank, count
             starts.dtype != torch.int32 or firsts.dtype != torch.int64 or (counts is not None and counts.dtype != torch.int32):
         raise ValueError("tables, starts and counts are int32, rows int32 or int64 and firsts int64")
     device = q.device
-    piece = int(piece or PIECE)
+    piece = int(piece or _knob("PIECE", H, R, P, page, int(fp8)) or PIECE)
     if piece < 32 or piece % 32:
         raise ValueError(f"a piece is a multiple of 32 positions, not {piece}")
-    parts = partitions(device, H, R, P, page, int(fp8))
+    parts = globals()["partitions"](device, H, R, P, page, int(fp8)) if partitions is None else int(partitions)
+    if not 1 <= parts <= MAX_PARTS:
+        raise ValueError(f"1..{MAX_PARTS} partitions, not {parts}")
     if out is None:
         out = torch.empty(T, H, R, dtype=q.dtype, device=device)
     if out.dtype not in _DTYPE or out.stride(-1) != 1 or out.shape[-1] != R:

@@ -222,3 +222,38 @@ def test_a_prompt_tokens_bits_do_not_follow_its_chunks_length_and_a_graph_replay
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, la.prefill(q, cache.cache, cache.tables[0], at, 64, rank=512)), at
+
+
+def test_the_partitions_are_a_knob_the_caller_or_the_tuning_sets():
+    # Fewer partitions: the same attention (other sums), fewer partials; the engine's tuned PARTS and PIECE (what crit's
+    # kernel build writes beside the module) are what a call without arguments takes, decode and prompt alike.
+    cache = Cache(512, 64, 64, [3000, 900], seed=6)
+    la = cache.la
+    q = _q(16, 128, 576, 8)
+    scale = 192 ** -0.5
+    default = cache.attend(q, [0, 1], [0, 8], [2990, 890], 8, scale=scale)
+    for parts in (1, 4, 16):
+        lse = torch.empty(16, 128, device=dev)
+        out = cache.attend(q, [0, 1], [0, 8], [2990, 890], 8, scale=scale, lse=lse, partitions=parts)
+        for s, start, first in ((0, 0, 2990), (1, 8, 890)):
+            cache.check(q, out, lse, s, start, first, 8, scale)
+
+    class Tuning:      # the generated accessor's shape (kernels/crit_kernels/build.py:255-313)
+        @staticmethod
+        def knobs(structure, key, rows):
+            assert structure == "window" and key == {"R": 512, "P": 64, "H": 128, "PAGE": 64, "KIND": 0}
+            return {"PARTS": 4, "PIECE": 512}
+
+    four = cache.attend(q, [0, 1], [0, 8], [2990, 890], 8, scale=scale, partitions=4, piece=512)
+    la._crit_tuning = Tuning
+    try:
+        assert la.partitions(torch.device(dev), 128, 512, 64, 64) == 4
+        tuned = cache.attend(q, [0, 1], [0, 8], [2990, 890], 8, scale=scale)
+        chunk = la.prefill(q[:8], cache.cache, cache.tables[0], 2990, 64, rank=512, scale=scale)
+    finally:
+        la._crit_tuning = None
+    assert torch.equal(tuned, four) and torch.equal(chunk, four[:8])
+    assert torch.equal(cache.attend(q, [0, 1], [0, 8], [2990, 890], 8, scale=scale), default)
+    for bad in (0, 65):
+        with pytest.raises(ValueError):
+            cache.attend(q, [0, 1], [0, 8], [2990, 890], 8, partitions=bad)
