@@ -32,6 +32,11 @@ import torch
 
 from . import _abi
 
+try:        # crit's kernel build writes the engine's tuned knobs beside the module (kernels/crit_kernels/build.py:255-313)
+    from . import _crit_tuning
+except ImportError:
+    _crit_tuning = None
+
 __all__ = ["KINDS", "PIECE", "MAX_COLUMNS", "Derive", "attend", "derive", "cuda_block", "cuda_chunk", "cuda_parts",
            "cuda_prompt", "cuda_ramp", "cuda_splits", "flash_block", "flash_chunk", "flash_parts", "flash_tile",
            "merge_shards", "owner", "partitions", "piece_size", "prefill", "prefill_rows", "prefill_state_floats", "release",
@@ -284,13 +289,25 @@ def _cus(device):
 
 
 # -- the split's order knobs -----------------------------------------------------------------------------------------------
+def _tuned(name, head_dim, value_dim, kv_heads, kind):
+    """The engine's tuned value of an order knob of the split launch (the "split" structure, keyed by the cache's
+    geometry as the reference keys it, __init__.py:262-286), 0 where it has none."""
+    if _crit_tuning is None or head_dim is None or value_dim is None or kv_heads is None:
+        return 0
+    key = {"D": int(head_dim), "DV": int(value_dim), "HKV": int(kv_heads), "KIND": KINDS[kind]}
+    return int(_crit_tuning.knobs("split", key, 1).get(name, 0) or 0)
+
+
 def partitions(device, kv_heads, kind, head_dim=None, value_dim=None):
-    """The partition count for a cache of `kv_heads` heads on `device`: about two workgroups per compute unit for one
-    long row, a workgroup serving two KV heads (a power of two within 8..64; partitions past a launch's page tables
-    are never launched, so a large count costs short rows nothing). A column's bits depend on it: one count per
-    cache."""
+    """The partition count for a cache of `kv_heads` heads on `device`: the tuning's PARTS, else about two workgroups
+    per compute unit for one long row, a workgroup serving two KV heads (a power of two within 8..64; partitions past
+    a launch's page tables are never launched, so a large count costs short rows nothing). A column's bits depend on
+    it: one count per cache."""
     if kind not in KINDS:
         raise ValueError(f"{kind!r} is no page kind ({', '.join(KINDS)})")
+    tuned = _tuned("PARTS", head_dim, value_dim, kv_heads, kind)
+    if tuned:
+        return tuned
     programs = 2 * _cus(torch.device(device))
     wanted = max(1, programs // max(1, int(kv_heads) // 2))
     return max(8, min(64, 1 << (wanted - 1).bit_length()))
@@ -300,10 +317,15 @@ def piece_size(head_dim, value_dim, kind="bf16", kv_heads=None):
     """Positions per piece: 64 Ki head values for 16-bit pages (512 positions at 128-wide heads), 192 Ki for 8-bit ones
     (1,536), within 256..2048, a multiple of 16. Measured on MI355X: the smallest pieces large batches still stream at
     their best rate with (a unit's fixed costs are hidden behind the next unit's rows), so a batch that does not fill
-    the chip is cut into as many units as that allows. A column's bits depend on it; it follows the cache's geometry
+    the chip is cut into as many units as that allows; the tuning's PIECE where the engine has one for the cache's
+    geometry (an engine of small batches gains from shorter pieces: 4 rows of 2,000 positions over FP8 pages take 36 us
+    a layer at 1,536 and 19 us at 256). A column's bits depend on it; it follows the cache's geometry
     and page kind only."""
     if kind not in KINDS:
         raise ValueError(f"{kind!r} is no page kind ({', '.join(KINDS)})")
+    tuned = _tuned("PIECE", head_dim, value_dim, kv_heads, kind)
+    if tuned:
+        return tuned
     values = 65536 if KINDS[kind] == 0 else 196608
     return max(256, min(2048, values // max(int(head_dim), int(value_dim)) // 16 * 16))
 

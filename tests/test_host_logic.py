@@ -1,3 +1,6 @@
+"""The modules' order knobs on the host (no GPU): the rules for pieces and partitions, and the engine's tuned values
+where crit's kernel build has written them beside a module (the generated _crit_tuning accessor, kernels/crit_kernels/
+build.py:255-313, stood in for by a class with the same knobs() call)."""
 
 
 def test_latent_partitions_follow_the_rule_or_the_engines_tuning():
@@ -19,3 +22,22 @@ def test_latent_partitions_follow_the_rule_or_the_engines_tuning():
     finally:
         la._crit_tuning = None
         la._CUS.clear(), la._CUS.update(held)
+
+
+def test_the_split_launchs_order_knobs_follow_the_rule_or_the_engines_tuning():
+    import crit_amd.paged_kv_attention as pk
+    assert pk.piece_size(128, 128, "bf16", 8) == 512 and pk.piece_size(128, 128, "fp8", 8) == 1536
+
+    class Tuning:
+        @staticmethod
+        def knobs(structure, key, rows):
+            assert structure == "split" and set(key) == {"D", "DV", "HKV", "KIND"}
+            return {"PIECE": 768 if key["KIND"] == 1 else 0, "PARTS": 16 if key["HKV"] == 4 else 0}
+
+    pk._crit_tuning = Tuning
+    try:
+        assert pk.piece_size(128, 128, "fp8", 8) == 768 and pk.piece_size(128, 128, "bf16", 8) == 512
+        assert pk.piece_size(128, 128, "fp8") == 1536                      # no geometry, no tuning
+        assert pk.partitions("cpu", 4, "bf16", 128, 128) == 16
+    finally:
+        pk._crit_tuning = None
