@@ -631,6 +631,30 @@ def index_selection(device):
                 "scores_bf16_us": round(bf16 * 1e3, 1), "scores_e4m3_us": round(fp8 * 1e3, 1),
                 "scores_bf16_TFLOP/s": round(flops / bf16 / 1e9, 1), "topk_us": round(top * 1e3, 1),
                 "topk_GB/s_of_scores_read_once": round(tokens * n * 4 / top / 1e6, 1)}
+    # A decode step's shape: every sequence's one token over its own keys, read in place from a store of pages of 64
+    # rows at random places (slots [sequences][n]): HBM-bound, a key row read once.
+    n, page = 49984, 64
+    for sequences in (16, 64):
+        rows = sequences * n
+        store = (torch.randn(rows, D, device=device, generator=g) * 0.5).to(torch.bfloat16)
+        store_scales = (store.float().abs().amax(1) / 448.0).clamp_min(1e-30)
+        codes = (store.float() / store_scales[:, None]).to(torch.float8_e4m3fn)
+        pages = torch.randperm(rows // page, device=device, generator=g)[:sequences * (n // page)].view(sequences, -1)
+        slots = (pages[:, :, None] * page + torch.arange(page, device=device)[None, None, :]).reshape(sequences, n)
+        slots = slots.to(torch.int32).contiguous()
+        q = (torch.randn(sequences, H, D, device=device, generator=g) * 0.5).to(torch.bfloat16)
+        w = torch.randn(sequences, H, device=device, generator=g) * H ** -0.5
+        ends = (n - torch.randint(0, 64, (sequences,), device=device, generator=g)).to(torch.int32)
+        s = torch.empty(sequences, n, dtype=torch.float32, device=device)
+        picked = torch.empty(sequences, K, dtype=torch.int32, device=device)
+        bf16 = graph_timed(lambda: si.scores(q, store, w, ends, out=s, slots=slots), 5)
+        fp8 = graph_timed(lambda: si.scores(q, codes, w, ends, key_scales=store_scales, out=s, slots=slots), 5)
+        top = graph_timed(lambda: si.topk(s, ends, K, out=picked), 5)
+        found[f"decode_step_{sequences}_sequences_of_{n}_keys_in_place"] = {
+            "scores_bf16_us": round(bf16 * 1e3, 1), "scores_bf16_GB/s_of_key_rows": round(rows * D * 2 / bf16 / 1e6, 1),
+            "scores_e4m3_us": round(fp8 * 1e3, 1), "scores_e4m3_GB/s_of_key_rows": round(rows * D / fp8 / 1e6, 1),
+            "topk_us": round(top * 1e3, 1)}
+        del store, codes, slots
     return found
 
 

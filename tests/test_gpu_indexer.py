@@ -298,3 +298,34 @@ def test_a_sparse_decode_step_reads_the_blocks_the_index_selects(kind, fp8_keys)
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(picked_again, picked) and torch.equal(again, out)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_a_decode_steps_sequences_score_their_own_keys_in_place(fp8):
+    # 64 sequences of one token, each over its own 50,000 keys where a store holds them (pages of 64 rows at random
+    # places): blocks of thousands of keys a workgroup, the launch whose wavefronts keep three tiles of key rows in
+    # flight. A sequence's scores are bit for bit those of the sequence alone over a gathered copy of its keys.
+    groups, n, page = 64, 50000, 64
+    q, _, _, _, w, _ = problem(groups, 64, 128, 8, seed=31)
+    g = torch.Generator(device=dev).manual_seed(6)
+    rows = groups * (n // page + 1) * page
+    store = (torch.randn(rows, 128, device=dev, generator=g) * 0.5).to(torch.bfloat16)
+    scales = None
+    if fp8:
+        scales = (store.float().abs().amax(1) / 448.0).clamp_min(1e-30)
+        store = (store.float() / scales[:, None]).to(torch.float8_e4m3fn)
+    pages = torch.randperm(rows // page, device=dev, generator=g).view(groups, -1)
+    slots = (pages[:, :, None] * page + torch.arange(page, device=dev)[None, None, :]).reshape(groups, -1)[:, :n]
+    slots = slots.to(torch.int32).contiguous()
+    ends = torch.randint(n - 5000, n + 1, (groups,), generator=torch.Generator().manual_seed(2)).to(torch.int32).to(dev)
+    ends[0], ends[1], ends[2], ends[3] = n, 0, 17, 4160
+    got = si.scores(q, store, w, ends, key_scales=scales, slots=slots)
+    assert bool((got[1] == float("-inf")).all())
+    for s in (0, 2, 3, 4, 33, 63):
+        keys = store[slots[s].long()]
+        alone = si.scores(q[s:s + 1], keys, w[s:s + 1], ends[s:s + 1], key_scales=None if scales is None else scales[slots[s].long()])
+        assert torch.equal(got[s], alone[0]), s
+        seen = int(ends[s])
+        assert bool(torch.isfinite(got[s, :seen]).all()) and bool((got[s, seen:] == float("-inf")).all())
+    picked = si.topk(got, ends, 64)
+    assert torch.equal(picked[0], oracle_index(got[:1], ends[:1], 64)[0].to(dev))
