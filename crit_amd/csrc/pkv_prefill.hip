@@ -482,7 +482,11 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
             }
         }
         if constexpr (KIND < 2) top = top == -INFINITY ? -INFINITY : top * sabs;
-        top = __builtin_fmaxf(top, __shfl_xor(top, 32));
+        {      // the two half-waves meet by one lane swap in the vector pipe (a shuffle is a round trip through the LDS crossbar)
+            const int w = (int)f2u(top);
+            const auto both = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+            top = __builtin_fmaxf(u2f((uint32_t)both[0]), u2f((uint32_t)both[1]));
+        }
         const float m_new = top > m + kMaxSlack ? top : m;
         sub = m_new == -INFINITY ? 0.0f : m_new;
         alpha = exp2_fast(m - sub);
