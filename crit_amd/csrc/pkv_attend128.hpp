@@ -527,12 +527,7 @@ PKV_DEV void attend128_unit(const AttendArgs& a, const int ux, const int uy) {
             if constexpr (PB > 1) {
                 const float w = exp2_fast(s_rm[wave][rho][rr] - sub);
 #pragma unroll
-                for (int d = 0; d < 8; ++d) {
-                    float x = acc[rr][d] * w;
-#pragma unroll
-                    for (int o = 16 * HW; o < 64; o <<= 1) x += __shfl_xor(x, o);
-                    acc[rr][d] = x;
-                }
+                for (int d = 0; d < 8; ++d) acc[rr][d] = sum_over_groups<16 * HW>(acc[rr][d] * w);
             }
             wm[rr] = top, wl[rr] = lsum;
         }

@@ -428,21 +428,12 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
         // through LDS in wavefront order.
 #pragma unroll
         for (int rr = 0; rr < QR; ++rr) {
-            float top = m[rr];
-#pragma unroll
-            for (int o = LPR; o < 64; o <<= 1) top = __builtin_fmaxf(top, __shfl_xor(top, o));
+            const float top = max_over_groups<LPR>(m[rr]);
             const float sub = top == -INFINITY ? 0.0f : top;
             const float w = exp2_fast(m[rr] - sub);
-            float lw = l[rr] * w;
+            const float lw = sum_over_groups<LPR>(l[rr] * w);
 #pragma unroll
-            for (int o = LPR; o < 64; o <<= 1) lw += __shfl_xor(lw, o);
-#pragma unroll
-            for (int d = 0; d < 8; ++d) {
-                float x = acc[rr][d] * w;
-#pragma unroll
-                for (int o = LPR; o < 64; o <<= 1) x += __shfl_xor(x, o);
-                acc[rr][d] = x;
-            }
+            for (int d = 0; d < 8; ++d) acc[rr][d] = sum_over_groups<LPR>(acc[rr][d] * w);
             m[rr] = top, l[rr] = lw;
         }
         if (FUSED) __syncthreads();      // the previous partition's fold has read the LDS

@@ -133,6 +133,53 @@ PKV_DEV float dpp(float x) {
     return u2f((uint32_t)__builtin_amdgcn_update_dpp(0, (int)f2u(x), CTRL, 0xf, 0xf, true));
 }
 
+// A lane's value and that of lane ^ 16 (ROWS false) or lane ^ 32 (true), in an order that depends on the lane: for
+// operations that commute. One lane swap in the vector pipe (v_permlane16_swap / v_permlane32_swap), where a shuffle
+// is a round trip through the LDS crossbar.
+struct Met {
+    float a, b;
+};
+template <bool HALVES>
+PKV_DEV Met meet(float x) {
+    const int v = (int)f2u(x);
+    if constexpr (HALVES) {
+        const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+        return Met{u2f((uint32_t)r[0]), u2f((uint32_t)r[1])};
+    } else {
+        const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+        return Met{u2f((uint32_t)r[0]), u2f((uint32_t)r[1])};
+    }
+}
+
+// The same for lane ^ O, any power of two: a rotation inside the row of 16 for 8, a shuffle below that.
+template <int O>
+PKV_DEV Met meet_at(float x) {
+    if constexpr (O == 32) return meet<true>(x);
+    else if constexpr (O == 16) return meet<false>(x);
+    else if constexpr (O == 8) return Met{x, u2f((uint32_t)__builtin_amdgcn_update_dpp(0, (int)f2u(x), 0x128, 0xf, 0xf, true))};      // row_ror:8
+    else return Met{x, __shfl_xor(x, O)};
+}
+// Sum / maximum over the lanes that hold the same place in each group of LPR lanes of the wavefront (a butterfly: every
+// lane ends with the same bits).
+template <int LPR>
+PKV_DEV float sum_over_groups(float x) {
+    if constexpr (LPR < 64) {
+        const Met m = meet_at<LPR>(x);
+        return sum_over_groups<LPR * 2>(m.a + m.b);
+    } else {
+        return x;
+    }
+}
+template <int LPR>
+PKV_DEV float max_over_groups(float x) {
+    if constexpr (LPR < 64) {
+        const Met m = meet_at<LPR>(x);
+        return max_over_groups<LPR * 2>(__builtin_fmaxf(m.a, m.b));
+    } else {
+        return x;
+    }
+}
+
 // Sum over the LANES (2 to 64, a power of two) lanes of each aligned group; every lane gets the same bits.
 template <int LANES>
 PKV_DEV float group_sum(float x) {
@@ -140,8 +187,14 @@ PKV_DEV float group_sum(float x) {
     if constexpr (LANES >= 4) x += dpp<0x4E>(x);
     if constexpr (LANES >= 8) x += dpp<0x141>(x);
     if constexpr (LANES >= 16) x += dpp<0x140>(x);
-    if constexpr (LANES >= 32) x += __shfl_xor(x, 16);
-    if constexpr (LANES >= 64) x += __shfl_xor(x, 32);
+    if constexpr (LANES >= 32) {
+        const Met m = meet<false>(x);
+        x = m.a + m.b;
+    }
+    if constexpr (LANES >= 64) {
+        const Met m = meet<true>(x);
+        x = m.a + m.b;
+    }
     return x;
 }
 template <int LANES>
@@ -150,8 +203,14 @@ PKV_DEV float group_max(float x) {
     if constexpr (LANES >= 4) x = __builtin_fmaxf(x, dpp<0x4E>(x));
     if constexpr (LANES >= 8) x = __builtin_fmaxf(x, dpp<0x141>(x));
     if constexpr (LANES >= 16) x = __builtin_fmaxf(x, dpp<0x140>(x));
-    if constexpr (LANES >= 32) x = __builtin_fmaxf(x, __shfl_xor(x, 16));
-    if constexpr (LANES >= 64) x = __builtin_fmaxf(x, __shfl_xor(x, 32));
+    if constexpr (LANES >= 32) {
+        const Met m = meet<false>(x);
+        x = __builtin_fmaxf(m.a, m.b);
+    }
+    if constexpr (LANES >= 64) {
+        const Met m = meet<true>(x);
+        x = __builtin_fmaxf(m.a, m.b);
+    }
     return x;
 }
 
