@@ -73,8 +73,15 @@ struct RawRow {
         RawRow r;
 #pragma unroll
         for (int j = 0; j < N; ++j) {
-            r.v[j] = u32x4{(unsigned)__shfl_xor((int)v[j].x, delta), (unsigned)__shfl_xor((int)v[j].y, delta),
-                           (unsigned)__shfl_xor((int)v[j].z, delta), (unsigned)__shfl_xor((int)v[j].w, delta)};
+            if (delta == 8) {      // (uniform) a rotation by 8 inside the row of 16 lanes: no trip through the LDS crossbar
+                r.v[j] = u32x4{(unsigned)__builtin_amdgcn_update_dpp(0, (int)v[j].x, 0x128, 0xf, 0xf, true),
+                               (unsigned)__builtin_amdgcn_update_dpp(0, (int)v[j].y, 0x128, 0xf, 0xf, true),
+                               (unsigned)__builtin_amdgcn_update_dpp(0, (int)v[j].z, 0x128, 0xf, 0xf, true),
+                               (unsigned)__builtin_amdgcn_update_dpp(0, (int)v[j].w, 0x128, 0xf, 0xf, true)};
+            } else {
+                r.v[j] = u32x4{(unsigned)__shfl_xor((int)v[j].x, delta), (unsigned)__shfl_xor((int)v[j].y, delta),
+                               (unsigned)__shfl_xor((int)v[j].z, delta), (unsigned)__shfl_xor((int)v[j].w, delta)};
+            }
         }
         return r;
     }
@@ -223,8 +230,7 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
                 for (int j = 1; j < 8; ++j) s8 = s8 + mine[8 * g8 + j] * mine[8 * g8 + j];
                 sq = g8 == 0 ? s8 : sq + s8;
             }
-#pragma unroll
-            for (int o = 1; o < LPR; o <<= 1) sq = sq + __shfl_xor(sq, o);
+            sq = LPR > 1 ? group_sum<(LPR > 1 ? LPR : 2)>(sq) : sq;      // (the butterfly's sums, lane pairs met in the vector pipe)
             const float mean = __fdiv_rn(sq, (float)a.dim[0]);
             // __builtin_sqrtf is the correctly rounded root (hipcc's default for sqrtf and "/"); __fsqrt_rn is not,
             // unless OCML_BASIC_ROUNDED_OPERATIONS is defined: it is the hardware's approximate one.
