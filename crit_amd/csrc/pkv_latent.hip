@@ -357,12 +357,27 @@ __global__ __launch_bounds__(64) void latent_merge_kernel(LatentArgs a) {
     float M = -INFINITY, L = 0.0f, acc[R / 64];
 #pragma unroll
     for (int i = 0; i < R / 64; ++i) acc[i] = 0.0f;
-    for (int b = 0; b < np; ++b) {
-        const Fold f = fold(M, L, a.pm[index + b], a.pl[index + b]);
-        const float* po = a.po + (index + b) * R;
+    // Four partitions' states are requested together (past the last one the last again, so every load is issued) and
+    // folded one by one in partition order: a fold waits for its own state only once in four.
+    constexpr int AHEAD = 4;
+    for (int b0 = 0; b0 < np; b0 += AHEAD) {
+        float pm[AHEAD], pl[AHEAD], po[AHEAD][R / 64];
 #pragma unroll
-        for (int i = 0; i < R / 64; ++i) acc[i] = __builtin_fmaf(acc[i], f.keep, po[i * 64 + threadIdx.x] * f.take);
-        M = f.m, L = f.l;
+        for (int j = 0; j < AHEAD; ++j) {
+            const int64_t at = index + min(b0 + j, np - 1);
+            pm[j] = a.pm[at], pl[j] = a.pl[at];
+#pragma unroll
+            for (int i = 0; i < R / 64; ++i) po[j][i] = a.po[at * R + i * 64 + threadIdx.x];
+        }
+#pragma unroll
+        for (int j = 0; j < AHEAD; ++j) {
+            if (b0 + j < np) {
+                const Fold f = fold(M, L, pm[j], pl[j]);
+#pragma unroll
+                for (int i = 0; i < R / 64; ++i) acc[i] = __builtin_fmaf(acc[i], f.keep, po[j][i] * f.take);
+                M = f.m, L = f.l;
+            }
+        }
     }
     if (a.sinks) {      // one more position with no value
         const float sink = a.sinks[head] * kLog2e;
