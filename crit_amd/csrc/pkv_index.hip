@@ -661,8 +661,12 @@ TopkPlan topk_plan(int tokens, int n, int k, int cus) {
 
 template <int LEVEL>
 void launch_topk_level(const TopkArgs& a, int elements, dim3 grid, hipStream_t stream) {
+    // (elements a thread: every one costs the same in each pass whether it is there or not, so the count is cut close)
     if (elements <= 8192) hipLaunchKernelGGL((index_topk_held_kernel<LEVEL, 8>), grid, dim3(1024), 0, stream, a);
+    else if (elements <= 12288) hipLaunchKernelGGL((index_topk_held_kernel<LEVEL, 12>), grid, dim3(1024), 0, stream, a);
+    else if (elements <= 14336) hipLaunchKernelGGL((index_topk_held_kernel<LEVEL, 14>), grid, dim3(1024), 0, stream, a);
     else if (elements <= 16384) hipLaunchKernelGGL((index_topk_held_kernel<LEVEL, 16>), grid, dim3(1024), 0, stream, a);
+    else if (elements <= 24576) hipLaunchKernelGGL((index_topk_held_kernel<LEVEL, 24>), grid, dim3(1024), 0, stream, a);
     else if (elements <= kHeld) hipLaunchKernelGGL((index_topk_held_kernel<LEVEL, 32>), grid, dim3(1024), 0, stream, a);
     else hipLaunchKernelGGL(index_topk_kernel<LEVEL>, grid, dim3(256), 0, stream, a);
 }
