@@ -183,12 +183,7 @@ __global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs
     if (dense) {      // s_before[r] = sum over r' < r of max(partitions(r') - 1, 0): thread i sums rows 2 i and 2 i + 1
         const int r0 = 2 * tid, r1 = 2 * tid + 1;
         const int c0 = r0 < a.n_rows ? max(row_partitions(r0) - 1, 0) : 0, c1 = r1 < a.n_rows ? max(row_partitions(r1) - 1, 0) : 0;
-        int run = c0 + c1;      // inclusive prefix over the threads
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            const int other = __shfl_up(run, o);
-            if (lane >= o) run += other;
-        }
+        const int run = (int)wave_inclusive_sum((unsigned)(c0 + c1));      // inclusive prefix over the threads
         if (lane == 63) s_wave_sum[wave] = run;
         lds_barrier();
         int base = 0;

@@ -180,6 +180,20 @@ PKV_DEV float max_over_groups(float x) {
     }
 }
 
+// The sum of x over the lanes up to and including this one of the wavefront, by data-parallel-primitive adds (shifts
+// of 1, 2, 4, 8 inside each row of 16 lanes, then lane 15 of a row to the next row, lane 31 to the upper half): six
+// vector instructions where a shuffle through the LDS crossbar is a round trip each.
+PKV_DEV unsigned wave_inclusive_sum(unsigned x) {
+    int v = (int)x;
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);      // row_shr:1 (zeros shifted in)
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);      // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, true);      // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, true);      // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);     // row_bcast:15 into rows 1 and 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);     // row_bcast:31 into rows 2 and 3
+    return (unsigned)v;
+}
+
 // Sum over the LANES (2 to 64, a power of two) lanes of each aligned group; every lane gets the same bits.
 template <int LANES>
 PKV_DEV float group_sum(float x) {

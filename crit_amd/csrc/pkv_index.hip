@@ -322,20 +322,6 @@ PKV_DEV uint32_t rank_key(float x) {
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
-// The sum of x over the lanes up to and including this one of the wavefront, by data-parallel-primitive adds (shifts
-// of 1, 2, 4, 8 inside each row of 16 lanes, then lane 15 of a row to the next row, lane 31 to the upper half): six
-// vector instructions where a shuffle through the LDS crossbar is a round trip each.
-PKV_DEV unsigned wave_inclusive_sum(unsigned x) {
-    int v = (int)x;
-    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);      // row_shr:1 (zeros shifted in)
-    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);      // row_shr:2
-    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, true);      // row_shr:4
-    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, true);      // row_shr:8
-    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);     // row_bcast:15 into rows 1 and 3
-    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);     // row_bcast:31 into rows 2 and 3
-    return (unsigned)v;
-}
-
 // LEVEL 0: a token's row, to its picks. 1: a slice of its row (blockIdx.y), to the slice's candidates (positions and
 // scores, [parts][k] a token). 2: a token's candidates (those with a position), to its picks.
 template <int LEVEL>
