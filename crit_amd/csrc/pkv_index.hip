@@ -463,21 +463,29 @@ __global__ __launch_bounds__(1024) void index_topk_held_kernel(TopkArgs a) {
     }
     row += lo;
     uint32_t key[EPT];
-    uint32_t ok = 0u;      // bit j: element j is a candidate
-    {
-        float x[EPT];
-        int at[EPT];
+    using Bits = typename std::conditional<(EPT > 32), uint64_t, uint32_t>::type;
+    Bits ok = 0;      // bit j: element j is a candidate
+    // (loaded 16 at a time: the loads in flight and the keys held share a thread's 128 registers)
+    constexpr int AT_ONCE = EPT > 16 ? 16 : EPT;
 #pragma unroll
-        for (int j = 0; j < EPT; ++j) {
+    for (int j0 = 0; j0 < EPT; j0 += AT_ONCE) {
+        float x[AT_ONCE];
+        int at[AT_ONCE];
+#pragma unroll
+        for (int jj = 0; jj < AT_ONCE; ++jj) {
+            const int j = j0 + jj;
             const int i = j * 1024 + tid;
-            x[j] = i < m ? row[i] : 0.0f;
-            at[j] = 0;
-            if constexpr (LEVEL == 2) at[j] = i < m ? pos[i] : -1;
+            x[jj] = (j < EPT && i < m) ? row[i] : 0.0f;
+            at[jj] = 0;
+            if constexpr (LEVEL == 2) at[jj] = (j < EPT && i < m) ? pos[i] : -1;
         }
 #pragma unroll
-        for (int j = 0; j < EPT; ++j) {
-            key[j] = rank_key(x[j]);
-            if (j * 1024 + tid < m && at[j] >= 0) ok |= 1u << j;
+        for (int jj = 0; jj < AT_ONCE; ++jj) {
+            const int j = j0 + jj;
+            if (j < EPT) {
+                key[j] = rank_key(x[jj]);
+                if (j * 1024 + tid < m && at[jj] >= 0) ok |= (Bits)1 << j;
+            }
         }
     }
     const bool all = valid <= k;
@@ -626,6 +634,12 @@ int launch_scores_kind(const ScoreArgs& a, int dim, bool many, int cus, hipStrea
 // (parts x k candidates, which must fit a workgroup too), where the candidates' room stays within kSliceRoom; everything
 // else streams, a workgroup a row.
 constexpr int kHeld = 32768;
+// Calls of many rows hold rows of up to kHeldWide elements whole, a workgroup a row (no slices, no candidates' pass:
+// measured for rows of 50,000 and k = 2,048: 320 against 432 us in slices for 2,048 rows, 43 against 58 for 256, 39
+// against 40 for 128; 64 rows take 30 us in slices, which spread a row over compute units, and 38 whole). Short of 65,536 so that the counts of equal keys before a
+// run of 64 elements fit their 16 bits.
+constexpr int kHeldWide = 64512;
+constexpr int kManyRows = 128;
 constexpr int64_t kSliceRoom = (int64_t)512 << 20;
 struct TopkPlan {
     int parts;      // 0: one pass a row
@@ -634,7 +648,7 @@ struct TopkPlan {
 TopkPlan topk_plan(int tokens, int n, int k, int cus) {
     TopkPlan plan = {0, n};
     (void)cus;
-    if (n <= kHeld || tokens > 65535) return plan;
+    if (n <= kHeld || tokens > 65535 || (n <= kHeldWide && tokens >= kManyRows)) return plan;
     for (int width = 8192; width <= kHeld; width *= 2) {
         const int64_t parts = ((int64_t)n + width - 1) / width;
         if (parts * k <= kHeld && parts <= 65535 && (int64_t)tokens * parts * k * 8 <= kSliceRoom) {
@@ -654,6 +668,10 @@ void launch_topk_level(const TopkArgs& a, int elements, dim3 grid, hipStream_t s
     else if (elements <= 16384) hipLaunchKernelGGL((index_topk_held_kernel<LEVEL, 16>), grid, dim3(1024), 0, stream, a);
     else if (elements <= 24576) hipLaunchKernelGGL((index_topk_held_kernel<LEVEL, 24>), grid, dim3(1024), 0, stream, a);
     else if (elements <= kHeld) hipLaunchKernelGGL((index_topk_held_kernel<LEVEL, 32>), grid, dim3(1024), 0, stream, a);
+    else if (LEVEL == 0 && elements <= 40960 && (int)grid.x >= kManyRows) hipLaunchKernelGGL((index_topk_held_kernel<0, 40>), grid, dim3(1024), 0, stream, a);
+    else if (LEVEL == 0 && elements <= 49152 && (int)grid.x >= kManyRows) hipLaunchKernelGGL((index_topk_held_kernel<0, 48>), grid, dim3(1024), 0, stream, a);
+    else if (LEVEL == 0 && elements <= 57344 && (int)grid.x >= kManyRows) hipLaunchKernelGGL((index_topk_held_kernel<0, 56>), grid, dim3(1024), 0, stream, a);
+    else if (LEVEL == 0 && elements <= kHeldWide && (int)grid.x >= kManyRows) hipLaunchKernelGGL((index_topk_held_kernel<0, 63>), grid, dim3(1024), 0, stream, a);
     else hipLaunchKernelGGL(index_topk_kernel<LEVEL>, grid, dim3(256), 0, stream, a);
 }
 

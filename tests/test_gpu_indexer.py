@@ -99,10 +99,12 @@ def test_a_nan_ranks_below_every_number():
     assert si.topk(z, end, 2).tolist() == [[0, 1]]          # the zeros tie
 
 
-# (rows of 9,000, 13,000, 20,000 and 30,000: each of the element counts a thread of the kernel that holds a row is built for)
+# (rows of 9,000, 13,000, 20,000 and 30,000: each of the element counts a thread of the kernel that holds a row is built
+# for; 128 rows or more of up to 64,512: a workgroup holds such a row whole)
 @pytest.mark.parametrize("n,k,t", [(200000, 512, 1), (60000, 4096, 2), (8192, 512, 3), (5, 512, 1), (33000, 16, 4),
                                    (4096, 1, 2), (9000, 2048, 2), (13000, 64, 2), (20000, 2048, 2), (30000, 300, 2),
-                                   (50000, 2048, 2)])
+                                   (50000, 2048, 2), (36000, 2048, 130), (50000, 2048, 130), (57000, 100, 128),
+                                   (64512, 2048, 129), (64513, 700, 128)])
 def test_long_rows_with_ties_nans_and_rows_cut_short(n, k, t):
     g = torch.Generator().manual_seed(n * 7 + k)
     s = torch.randn(t, n, generator=g)
