@@ -645,16 +645,31 @@ struct TopkPlan {
     int parts;      // 0: one pass a row
     int width;
 };
+// Elements a thread of the holding kernel for `elements` of a row (what launch_topk_level picks).
+int held_elements(int elements) {
+    const int steps[] = {8, 12, 14, 16, 24, 32};
+    for (int e : steps)
+        if (elements <= e * 1024) return e;
+    return 0;
+}
 TopkPlan topk_plan(int tokens, int n, int k, int cus) {
     TopkPlan plan = {0, n};
     (void)cus;
     if (n <= kHeld || tokens > 65535 || (n <= kHeldWide && tokens >= kManyRows)) return plan;
-    for (int width = 8192; width <= kHeld; width *= 2) {
-        const int64_t parts = ((int64_t)n + width - 1) / width;
-        if (parts * k <= kHeld && parts <= 65535 && (int64_t)tokens * parts * k * 8 <= kSliceRoom) {
-            plan.parts = (int)parts, plan.width = width;
-            return plan;
-        }
+    // Slices: the fewest microseconds by what the holding kernel was measured to take, 4.2 us and 0.53 us an element
+    // a thread (the candidates' pass, which also loads positions, 1.3 times that): for a few rows the two launches one
+    // after the other, for many rows every slice's workgroup counts. (50,000 positions, k = 2,048: 4 slices of 12,544
+    // and 8,192 candidates, 22 us where 7 slices of 8,192 and 14,336 candidates took 25.)
+    const int64_t fewest = ((int64_t)n + kHeld - 1) / kHeld;
+    const int64_t most = min((int64_t)kHeld / k, min((int64_t)65535, max(fewest * 8, (int64_t)16)));
+    float best = 0.0f;
+    for (int64_t parts = max(fewest, (int64_t)2); parts <= most; ++parts) {
+        const int width = (int)((((int64_t)n + parts - 1) / parts + 63) / 64 * 64);
+        const int e1 = held_elements(width), e2 = held_elements((int)(parts * k));
+        if (!e1 || !e2 || (int64_t)tokens * parts * k * 8 > kSliceRoom) continue;
+        const float slices = 4.2f + 0.53f * e1, candidates = 1.3f * (4.2f + 0.53f * e2);
+        const float cost = (tokens >= kManyRows ? (float)parts : 1.0f) * slices + candidates;
+        if (plan.parts == 0 || cost < best) best = cost, plan.parts = (int)parts, plan.width = width;
     }
     return plan;
 }
