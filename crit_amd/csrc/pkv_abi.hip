@@ -39,6 +39,10 @@ int crit_pkv_latent_attend(const crit_pkv_latent_params* p, void* stream) {
     return pkv::launch_latent(p, reinterpret_cast<hipStream_t>(stream));
 }
 
+int crit_pkv_latent_write(const crit_pkv_latent_write_params* p, void* stream) {
+    return pkv::launch_latent_write(p, reinterpret_cast<hipStream_t>(stream));
+}
+
 int crit_pkv_index_scores(const crit_pkv_index_scores_params* p, void* stream) {
     return pkv::launch_index_scores(p, reinterpret_cast<hipStream_t>(stream));
 }
@@ -92,6 +96,7 @@ int crit_pkv_params_size(int which) {
         case 10: return (int)sizeof(crit_pkv_latent_params);
         case 11: return (int)sizeof(crit_pkv_index_scores_params);
         case 12: return (int)sizeof(crit_pkv_index_topk_params);
+        case 13: return (int)sizeof(crit_pkv_latent_write_params);
     }
     return -1;
 }

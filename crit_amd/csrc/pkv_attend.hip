@@ -231,7 +231,8 @@ int compute_units() {
     return n;
 }
 
-int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
+// check_only: every refusal the launch can make is made, nothing is queued on the stream.
+static int launch_attend_checked(const crit_pkv_attend_params* p, hipStream_t stream, bool check_only) {
     if (!p || !p->q || !p->value_pages || !p->tables || !p->rows || !p->starts || !p->firsts || !p->out) return CRIT_PKV_E_NULL;
     const bool derive = p->derive_table != nullptr;      // keys derived from the value rows: no key pages, no key scales
     if (!derive && !p->key_pages) return CRIT_PKV_E_NULL;
@@ -352,11 +353,12 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
         }
         return CRIT_PKV_E_DTYPE;
     };
+    if (!p->fused && p->phases != 1 && (p->heads > 65535 || p->n_rows > 65535)) return CRIT_PKV_E_GEOMETRY;      // (the merge's grid)
+    if (check_only) return 0;
     int rc = 0;
     if (p->fused) return split(true);
     if (p->phases != 2) rc = split(false);
     if (rc || p->phases == 1) return rc;
-    if (p->heads > 65535 || p->n_rows > 65535) return CRIT_PKV_E_GEOMETRY;
     const dim3 mgrid((unsigned)p->columns, (unsigned)p->heads, (unsigned)p->n_rows);
     switch (p->value_dim) {
         case 16: hipLaunchKernelGGL((merge_kernel<16>), mgrid, dim3(64), 0, stream, a); break;
@@ -367,6 +369,8 @@ int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) {
     }
     return hip_code(hipGetLastError());
 }
+
+int launch_attend(const crit_pkv_attend_params* p, hipStream_t stream) { return launch_attend_checked(p, stream, false); }
 
 // -- the entry point that allocates nothing ------------------------------------------------------------------------------
 // The split launch's partials and its two counters in memory the library itself holds: a file-scope device array, one
@@ -411,6 +415,10 @@ int launch_attend_static(const crit_pkv_attend_params* p, hipStream_t stream) {
     q.partial_out = p->fused ? nullptr : partials;
     q.partial_max = p->fused ? nullptr : partials + states * p->value_dim;
     q.partial_sum = p->fused ? nullptr : partials + states * ((int64_t)p->value_dim + 1);
+    // A launch that would be refused queues nothing: the clear below touches counters that every stream of this GPU
+    // shares, so it must not run for a call that is not going to launch.
+    const int refused = launch_attend_checked(&q, stream, true);
+    if (refused) return refused;
     // The counters start at zero whatever the last call left (a fill kernel: a captured graph replays it as it is).
     hipLaunchKernelGGL(clear_counters_kernel, dim3(1), dim3(64), 0, stream, reinterpret_cast<unsigned*>(base));
     const int rc = hip_code(hipGetLastError());

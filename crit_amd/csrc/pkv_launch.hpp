@@ -16,6 +16,7 @@ int launch_copy_pages(const crit_pkv_copy_pages_params* p, hipStream_t stream);
 int launch_round(const crit_pkv_round_params* p, hipStream_t stream);
 int launch_step_buffers(const crit_pkv_step_params* p, hipStream_t stream);
 int launch_latent(const crit_pkv_latent_params* p, hipStream_t stream);
+int launch_latent_write(const crit_pkv_latent_write_params* p, hipStream_t stream);
 int launch_index_scores(const crit_pkv_index_scores_params* p, hipStream_t stream);
 int launch_index_topk(const crit_pkv_index_topk_params* p, hipStream_t stream);
 int64_t index_topk_work_bytes(int tokens, int n, int k);

@@ -1,28 +1,33 @@
-"""Latent attention (multi-head latent attention, absorbed) on MI355X: the host side of crit's latent-attention kernels
-module (reference kernels/techniques/attention/latent-attention/torch-ext/latent_attention/__init__.py), same names,
-arguments and errors, over the gfx950 kernels of libcrit_pkv.so (crit_pkv_latent_attend). crit's attention plugin calls
-it for pools of keys only with one KV head (inference/attention-state/code/device_attention.py:444-519).
+"""Latent attention (multi-head latent attention with the key up-projection absorbed) on MI355X: the host side of crit's
+latent-attention kernels module (reference kernels/techniques/attention/latent-attention/torch-ext/latent_attention/
+__init__.py: `write` :74-97, `prefill` :121-152, `attend` :155-229, `partitions` :65-71), with the same calls, keyword
+arguments and error types, over the gfx950 kernels of libcrit_pkv.so (crit_pkv_latent_attend, crit_pkv_latent_write).
+crit's attention plugin calls it for keys-only pools of one KV head (inference/attention-state/code/
+device_attention.py:444-519). There is no other implementation behind this module: without the library every call fails.
 
-    write(latent, rope, slots, cache)                  # rows into their page slots: cache [pages][page][R + P]
-    out = attend(q, cache, tables, rows, starts, firsts, columns, page, rank=R)
-    # q [tokens][heads][R + P]: the query's latent part (the key up-projection absorbed) then its rotary part;
-    # out [tokens][heads][R]: the attention output in the latent space
+The cache is [pages][page][R + P]: position n of a sequence keeps its latent (R values) and then its rotary key (P
+values) in one row at slot table[n // page] * page + n % page. A query is [R + P] too, its latent part already
+multiplied through the key up-projection, so for every head
 
-Row b of a launch is table row rows[b]'s sequence; its columns are tokens starts[b] .. starts[b] + counts[b] - 1 at
-positions firsts[b] + column, each seeing the positions up to its own. A row's positions are cut into pieces of PIECE
-positions, piece i to partition i mod partitions(); the partitions' states are merged in partition order. A token's bits
-depend on its own query and positions, the piece and the partition count, never on the rows or columns beside it.
-fused=True gives the same bits (here: the same launches over the module's bounded partials, a few rows at a time);
-prefill() reads a prompt chunk as windows of MAX_COLUMNS columns, so a prompt token has the bits of the same position
-decoded (what the reference's plugin does with prompt_reader "decode"). There is no other implementation behind this
-module: without the library every call fails.
+    score[n] = scale * (q[:R] . row[n][:R] + q[R:] . row[n][R:])      out = sum_n softmax(score)[n] * row[n][:R]
+
+write()    puts rows into their slots (one launch, any float input type).
+attend()   decode tokens and verify windows: batch row b is the sequence of table row rows[b]; its counts[b] columns are
+           tokens starts[b].. of q at positions firsts[b] + column, each seeing positions up to its own.
+prefill()  a prompt chunk of one sequence, causal.
+
+Order of the sums. A row's positions are cut into pieces of `piece` positions, piece i going to partition i mod
+partitions; each partition's running state is folded into the result in partition order, the sink last. A token's bits
+depend on its own query and positions, `piece` and the partition count only, never on the batch it rode in, so
+fused=True / False and any row batching give equal bits, and prefill() (which reads a chunk as windows of MAX_COLUMNS
+columns) gives each prompt token the bits it would have decoded.
 """
 from typing import Optional
 
 import torch
 
 from ..paged_kv_attention import _abi
-from ..paged_kv_attention import _launch, _ptr, _require_device
+from ..paged_kv_attention import _grown, _holding, _launch, _ptr, _require_device
 
 try:        # crit's kernel build writes the engine's tuned knobs beside the module (kernels/crit_kernels/build.py:255-313)
     from . import _crit_tuning
@@ -32,14 +37,14 @@ except ImportError:
 __all__ = ["MAX_COLUMNS", "PARTIAL_BYTES", "PIECE", "SHAPES", "attend", "partitions", "prefill", "write"]
 
 MAX_COLUMNS = 64
-PARTIAL_BYTES = 512 << 20   # a launch's partials: rows whose partials would take more are launched a few at a time
-PIECE = 256                 # positions a piece (an order knob: one value for every launch)
+PARTIAL_BYTES = 512 << 20   # the most partials one launch may take; a larger batch goes in several launches of rows
+PIECE = 256                 # default positions a piece
 MAX_PARTS = 64
-SHAPES = ((512, 64), (256, 64), (128, 64), (128, 32), (64, 64), (64, 32))   # (rank, rotary width) the kernels are built for
+SHAPES = ((512, 64), (256, 64), (128, 64), (128, 32), (64, 64), (64, 32))   # (R, P) pairs the kernels are built for
 FP8 = torch.float8_e4m3fn
 _DTYPE = {torch.float32: _abi.F32, torch.bfloat16: _abi.BF16, torch.float16: _abi.F16}
+_CACHE_DTYPE = {torch.bfloat16: 0, torch.float16: 1, FP8: 2}
 _CUS = {}
-_partials = {}      # device index -> the module's partials (FP32), grown outside a capture
 
 
 def _cus(device):
@@ -50,8 +55,8 @@ def _cus(device):
 
 
 def _knob(name, heads, rank, rope, page, kind):
-    """The engine's tuned value of a knob of the "window" structure for this geometry, 0 where it has none (the
-    reference's _knobs(), __init__.py:44-50)."""
+    """The engine's tuned value of knob `name` for this geometry (structure "window", keyed as the reference keys it,
+    __init__.py:44-50), or 0."""
     if _crit_tuning is None:
         return 0
     key = {"R": int(rank), "P": int(rope), "H": int(heads), "PAGE": int(page), "KIND": int(kind)}
@@ -59,140 +64,175 @@ def _knob(name, heads, rank, rope, page, kind):
 
 
 def partitions(device, heads, rank, rope, page, kind=0):
-    """The partitions a launch over this geometry splits a row's positions into: the tuning's PARTS, else the rule:
-    the CUs over twice the heads' 16-row tiles, 1 to MAX_PARTS, from the heads and the device only (the reference's:
-    2 x SMs over the tiles, __init__.py:65-71). Every partition's state is a partial the merge reads again, and a
-    row's tiles all write theirs: measured on MI355X (64 rows of 1,024 to 8,192 positions, R 512, P 64) 128 heads
-    take 356 / 294 / 261 us with 32 / 16 / 8 partitions and a lone row of 8,192 positions 34 / 42 / 67 us; 16 heads
-    102 / 97 / 89 us with 64 / 16 / 8 and a lone row 28 / 36 / 57 us. The rule gives 64, 64, 32, 16 for 16, 32, 64
-    and 128 heads; an engine that serves batches only sets PARTS lower."""
+    """How many partitions a row's pieces are dealt to for this geometry on `device`: the tuned PARTS if the engine has
+    one, else one workgroup's worth of work for every second compute unit per 16 heads, between 1 and MAX_PARTS (64 for
+    16 and 32 heads, 32 for 64, 16 for 128 on 256 compute units). It depends on the heads and the device only, because a
+    token's bits depend on it. (The reference's rule is the same idea for its tiles: __init__.py:65-71.)"""
     tuned = _knob("PARTS", heads, rank, rope, page, kind)
-    if tuned:
-        return max(1, min(MAX_PARTS, tuned))
-    return max(1, min(MAX_PARTS, _cus(device) // (2 * max(1, -(-int(heads) // 16)))))
+    wanted = tuned if tuned else _cus(device) // (2 * max(1, -(-int(heads) // 16)))
+    return min(MAX_PARTS, max(1, wanted))
 
 
 def write(latent, rope, slots, cache, scales=None):
-    """latent [N][R] and rope [N][P] into their slots (int64 [N], page * page_size + offset) of cache
-    [pages][page][R + P], in the cache's dtype (device work only; capture-safe). An E4M3 cache takes scales FP32
-    [pages][page][2]: each position's latent and rotary key coded at their own scale, max |x| / 448 (at least 1e-30),
-    the codes the nearest E4M3 values of x / scale (IEEE divisions). Plain torch indexing, as the reference's."""
-    rank = latent.shape[-1]
-    if cache.shape[-1] != rank + rope.shape[-1] or latent.shape[0] != rope.shape[0] or slots.shape[0] != latent.shape[0]:
-        raise ValueError("a cache row is the latent then the rotary key, one row a slot")
-    slots = slots.long()
-    if cache.dtype == FP8:
-        if scales is None or tuple(scales.shape) != (*cache.shape[:2], 2) or scales.dtype != torch.float32:
-            raise ValueError("an E4M3 cache takes scales FP32 [pages][page][2] (the latent's, the rotary key's)")
-        codes, found = [], []
-        for x in (latent.float(), rope.float()):
-            amax = x.abs().amax(-1)
-            s = (amax / torch.full_like(amax, 448.0)).clamp(min=1e-30)
-            codes.append((x / s[:, None]).clamp(-448.0, 448.0).to(FP8).view(torch.uint8))
-            found.append(s)
-        cache.view(torch.uint8).view(-1, cache.shape[-1]).index_copy_(0, slots, torch.cat(codes, dim=-1))
-        scales.view(-1, 2).index_copy_(0, slots, torch.stack(found, dim=-1))
+    """Append rows: token t's latent[t] ([N][R]) and rope[t] ([N][P]) side by side into row slots[t] (int64 [N]) of
+    cache [pages][page][R + P], converted to the cache's dtype. A float8_e4m3fn cache also takes scales FP32
+    [pages][page][2]: each part is coded at its own scale max|x| / 448 (not below 1e-30) and the two scales are stored
+    at the row's place. One kernel launch, nothing allocated when the inputs are contiguous rows of one float type."""
+    if latent.dim() != 2 or rope.dim() != 2 or cache.dim() != 3:
+        raise ValueError("write: latent [N][R], rope [N][P] and cache [pages][page][R + P]")
+    n, rank = latent.shape
+    width = rope.shape[1]
+    if rope.shape[0] != n or slots.shape != (n,) or cache.shape[2] != rank + width:
+        raise ValueError(f"write: {n} latents of {rank} need {n} rotary keys, {n} slots and cache rows of "
+                         f"{rank} + {width}, not {tuple(rope.shape)}, {tuple(slots.shape)}, {cache.shape[2]}")
+    _require_device(cache, "the latent cache")
+    if cache.dtype not in _CACHE_DTYPE or not cache.is_contiguous():
+        raise ValueError("write: the cache is contiguous BF16, FP16 or float8_e4m3fn")
+    coded = cache.dtype == FP8
+    if coded and (scales is None or scales.dtype != torch.float32 or tuple(scales.shape) != (*cache.shape[:2], 2)
+                  or not scales.is_contiguous()):
+        raise ValueError(f"write: an E4M3 cache keeps two FP32 scales a row, [{cache.shape[0]}][{cache.shape[1]}][2]")
+    if n == 0:
         return
-    cache.view(-1, cache.shape[-1]).index_copy_(0, slots, torch.cat([latent.to(cache.dtype), rope.to(cache.dtype)], dim=-1))
+    if latent.dtype not in _DTYPE:
+        latent = latent.float()
+    if rope.dtype != latent.dtype:
+        rope = rope.to(latent.dtype)
+    if latent.stride(1) != 1:
+        latent = latent.contiguous()
+    if rope.stride(1) != 1:
+        rope = rope.contiguous()
+    if slots.dtype != torch.int64 or not slots.is_contiguous():
+        slots = slots.long().contiguous()
+    p = _abi.LatentWriteParams()
+    p.latent, p.rope, p.slots, p.cache, p.scales = latent.data_ptr(), rope.data_ptr(), slots.data_ptr(), cache.data_ptr(), \
+        _ptr(scales) if coded else None
+    p.tokens, p.latent_stride, p.rope_stride = n, latent.stride(0), rope.stride(0)
+    p.rank, p.rope_width, p.in_dtype, p.cache_dtype = rank, width, _DTYPE[latent.dtype], _CACHE_DTYPE[cache.dtype]
+    _launch(cache.device, "crit_pkv_latent_write", "latent_attention.write", p)
 
 
-def _check(q, cache, page, rank, sinks, scales):
-    """(R, P, fp8) of a call, its inputs checked (the reference's checks and messages, __init__.py:96-117)."""
-    _require_device(q, "latent attention's q")
-    T, H, width = q.shape
-    R, P = int(rank), width - int(rank)
-    if cache.dim() != 3 or cache.shape[-1] != width or cache.shape[1] != page or not cache.is_contiguous():
-        raise ValueError(f"the cache is contiguous [pages][{page}][{width}]: the latent then the rotary key")
-    fp8 = cache.dtype == FP8
-    if (q.dtype != cache.dtype and not fp8) or q.dtype not in (torch.bfloat16, torch.float16) or q.stride(-1) != 1:
-        raise ValueError("q is BF16 or FP16 in the cache's dtype (either over an E4M3 cache), its last dimension "
-                         "contiguous")
-    if fp8 and (scales is None or tuple(scales.shape) not in ((*cache.shape[:2], 2), (*cache.shape[:2], 1)) or
-                scales.dtype != torch.float32 or not scales.is_contiguous()):
-        raise ValueError("an E4M3 cache takes its scales FP32 [pages][page][2] (or [pages][page][1]: one a row)")
-    if R < 16 or P < 16 or R & (R - 1) or P & (P - 1) or R > 1024 or P > 256:
-        raise ValueError("the rank and the rotary width are powers of two (16 to 1024 and 16 to 256)")
-    if sinks is not None and (sinks.dtype != torch.float32 or tuple(sinks.shape) != (H,) or not sinks.is_contiguous()
-                              or sinks.device != q.device):
-        raise ValueError(f"sinks are contiguous FP32 [{H}] on q's device")
-    if (R, P) not in SHAPES:
-        raise NotImplementedError(f"latent_attention (gfx950): rank {R} with a rotary width of {P} is not built; "
-                                  f"(rank, rotary width) is one of {SHAPES}")
-    if cache.device != q.device:
-        raise ValueError("q and the cache live on one device")
-    return R, P, fp8
+class _Call:
+    """The operands every reading call shares, validated once: q, the cache, its scales and the sinks."""
+    __slots__ = ("tokens", "heads", "rank", "rope", "coded")
+
+    def __init__(self, q, cache, page, rank, sinks, scales):
+        if q.dim() != 3:
+            raise ValueError("q: [tokens][heads][R + P]")
+        _require_device(q, "latent attention's q")
+        self.tokens, self.heads, width = q.shape
+        self.rank, self.rope = int(rank), width - int(rank)
+        self.coded = cache.dtype == FP8
+        if cache.dim() != 3 or tuple(cache.shape[1:]) != (page, width) or not cache.is_contiguous():
+            raise ValueError(f"cache: contiguous [pages][{page}][{width}] (a row is R latent values, then P rotary), "
+                             f"not {tuple(cache.shape)}")
+        if q.dtype not in (torch.bfloat16, torch.float16) or q.stride(-1) != 1 or not (self.coded or q.dtype == cache.dtype):
+            raise ValueError("q: BF16 or FP16 in the cache's dtype (either of the two over an E4M3 cache), unit stride "
+                             "along its last dimension")
+        if self.coded:
+            ok = scales is not None and scales.dtype == torch.float32 and scales.is_contiguous() and \
+                scales.dim() == 3 and tuple(scales.shape[:2]) == tuple(cache.shape[:2]) and scales.shape[2] in (1, 2)
+            if not ok:
+                raise ValueError("scales: an E4M3 cache takes its scales, contiguous FP32 [pages][page][2] (latent, rotary "
+                                 "key) or [pages][page][1] (one for the row)")
+
+        def power_of_two(n, low, high):
+            return low <= n <= high and n & (n - 1) == 0
+
+        if not power_of_two(self.rank, 16, 1024) or not power_of_two(self.rope, 16, 256):
+            raise ValueError(f"rank {self.rank} / rotary width {self.rope}: both are powers of two, 16..1024 and 16..256")
+        if sinks is not None:
+            if sinks.dtype != torch.float32 or tuple(sinks.shape) != (self.heads,) or not sinks.is_contiguous() or \
+                    sinks.device != q.device:
+                raise ValueError(f"sinks: one FP32 logit a head, contiguous [{self.heads}] on q's device")
+        if (self.rank, self.rope) not in SHAPES:
+            raise NotImplementedError(f"latent_attention (gfx950): rank {self.rank} with a rotary width of {self.rope} is "
+                                      f"not built; (rank, rotary width) is one of {SHAPES}")
+        if cache.device != q.device:
+            raise ValueError(f"cache is on {cache.device}, q on {q.device}")
 
 
-def _workspace(device, floats):
-    index = device.index if device.index is not None else torch.cuda.current_device()
-    held = _partials.get(index)
-    if held is None or held.numel() < floats:
-        if torch.cuda.is_current_stream_capturing():
-            raise RuntimeError("latent_attention: the partials grow outside a capture: run the launch's shape eagerly first")
-        held = _partials[index] = torch.empty(floats, dtype=torch.float32, device=device)
-    return held
+def _partials(device, floats):
+    """The current owner's partials buffer on `device` (paged_kv_attention.owner()), at least `floats` long. It grows
+    outside a capture only, and a buffer it outgrew is kept alive, because a captured graph may still replay into it."""
+    return _grown(_holding(device), "latent", floats, device, 1 << 16,
+                  "latent attend: run a launch of this shape once before capturing it")
 
 
 def attend(q, cache, tables, rows, starts, firsts, columns, page, *, rank, counts=None, scale=None,
            out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
            sinks: Optional[torch.Tensor] = None, scales: Optional[torch.Tensor] = None,
-           fused: Optional[bool] = None, piece=None, partitions=None, phases=0) -> torch.Tensor:
-    """Decode tokens and verify windows over the latent cache (see the module's description). q [tokens][heads][R + P]
-    BF16 or FP16 in the cache's dtype, the last dimension contiguous; cache [pages][page][R + P] contiguous; tables
-    [S][width] int32; rows, starts [B] int32 (rows int64 too: a round's slots as they are); firsts [B] int64; counts [B]
-    int32 (None: `columns` each); columns the widest row (a Python int, 1 to MAX_COLUMNS). Returns out
-    [tokens][heads][R] in q's dtype (written at the rows' tokens); lse [tokens][heads] FP32 when given; sinks FP32
-    [heads]. scale defaults to (R + P) ** -0.5 (pass the model's). An E4M3 cache takes its scales, with BF16 or FP16
-    queries: write()'s two a position, or one a position for the whole row ([pages][page][1], a KV pool's fp8:row pages
-    of one head). fused: the same bits whatever it says; the rows are launched a few at a time where their partials
-    would take more than PARTIAL_BYTES. piece: positions a piece (a multiple of 32; default the tuning's PIECE, else
-    PIECE), partitions: 1 to MAX_PARTS (default partitions()); a token's bits depend on both, so a caller keeps one
-    value of each for a geometry. phases (a measurement's): 1 the partitions' launch only, 2 the merge only."""
-    R, P, fp8 = _check(q, cache, page, rank, sinks, scales)
-    T, H, width = q.shape
-    B = int(starts.shape[0])
-    if not 1 <= columns <= MAX_COLUMNS or B == 0:
-        raise ValueError(f"1..{MAX_COLUMNS} columns a row, one row or more")
-    if tables.dtype != torch.int32 or tables.stride(-1) != 1 or rows.dtype not in (torch.int32, torch.int64) or \
-            starts.dtype != torch.int32 or firsts.dtype != torch.int64 or (counts is not None and counts.dtype != torch.int32):
-        raise ValueError("tables, starts and counts are int32, rows int32 or int64 and firsts int64")
+           fused: Optional[bool] = None, piece=None, partitions=None, workspace: Optional[torch.Tensor] = None,
+           phases=0) -> torch.Tensor:
+    """Decode tokens and verify windows (see the module text). q [tokens][heads][R + P]; tables [S][width] int32; rows
+    and starts [B] int32 (rows may be int64); firsts [B] int64; counts [B] int32 or None (every row has `columns`);
+    columns: the widest row, a Python int within 1..MAX_COLUMNS. Returns out [tokens][heads][R] (q's dtype unless `out`
+    is given as BF16, FP16 or FP32), written at the rows' tokens only. lse: FP32 [tokens][heads], the natural
+    log-sum-exp of a token's scaled scores, its sink included. sinks: FP32 [heads] logits of one extra position that has
+    no value. scale: default (R + P) ** -0.5. scales: an E4M3 cache's, as write() stores them, or one a row.
+
+    fused is accepted for the reference's signature and changes nothing: the bits are the same either way and the
+    partials stay bounded (PARTIAL_BYTES; a larger batch is launched a few rows at a time). piece (a multiple of 32)
+    and partitions (1..MAX_PARTS) default to the tuned values or PIECE and partitions(); keep one value of each per
+    geometry, since a token's bits depend on them. workspace: FP32 scratch for the partials; without it the module uses
+    a buffer held per owner (paged_kv_attention.owner) and device, so launches of two owners on two streams never share
+    partials. phases is for timing: 1 runs the partitions' launch alone, 2 the merge alone."""
+    call = _Call(q, cache, page, rank, sinks, scales)
+    heads, R, P = call.heads, call.rank, call.rope
+    batch = int(starts.shape[0])
+    if batch < 1 or not 1 <= int(columns) <= MAX_COLUMNS:
+        raise ValueError(f"a launch has at least one row and 1..{MAX_COLUMNS} columns a row, not {batch} x {columns}")
+    columns = int(columns)
+    if tables.dtype != torch.int32 or tables.dim() != 2 or tables.stride(1) != 1:
+        raise ValueError("tables: int32 [sequences][pages], unit stride along pages")
+    if rows.dtype not in (torch.int32, torch.int64) or starts.dtype != torch.int32 or firsts.dtype != torch.int64 or \
+            (counts is not None and counts.dtype != torch.int32):
+        raise ValueError("rows: int32 or int64; starts and counts: int32; firsts: int64")
     device = q.device
-    piece = int(piece or _knob("PIECE", H, R, P, page, int(fp8)) or PIECE)
+    coded = int(call.coded)
+    piece = int(piece or _knob("PIECE", heads, R, P, page, coded) or PIECE)
     if piece < 32 or piece % 32:
-        raise ValueError(f"a piece is a multiple of 32 positions, not {piece}")
-    parts = globals()["partitions"](device, H, R, P, page, int(fp8)) if partitions is None else int(partitions)
+        raise ValueError(f"piece: {piece}; a multiple of 32 positions")
+    parts = int(partitions) if partitions is not None else globals()["partitions"](device, heads, R, P, page, coded)
     if not 1 <= parts <= MAX_PARTS:
-        raise ValueError(f"1..{MAX_PARTS} partitions, not {parts}")
+        raise ValueError(f"partitions: {parts}; within 1..{MAX_PARTS}")
     if out is None:
-        out = torch.empty(T, H, R, dtype=q.dtype, device=device)
-    if out.dtype not in _DTYPE or out.stride(-1) != 1 or out.shape[-1] != R:
-        raise ValueError("out is [tokens][heads][rank] BF16, FP16 or FP32, its last dimension contiguous")
+        out = torch.empty(call.tokens, heads, R, dtype=q.dtype, device=device)
+    elif out.dtype not in _DTYPE or out.dim() != 3 or out.shape[2] != R or out.stride(2) != 1:
+        raise ValueError(f"out: BF16, FP16 or FP32 [tokens][heads][{R}], unit stride along its last dimension")
     if lse is not None and (lse.dtype != torch.float32 or not lse.is_contiguous()):
-        raise ValueError("lse is contiguous FP32 [tokens][heads]")
-    per_row = int(columns) * H * parts                    # partial states a batch row takes
-    rows_a_launch = max(1, min(B, (PARTIAL_BYTES // 4) // (per_row * (R + 2))))
-    work = _workspace(device, rows_a_launch * per_row * (R + 2))
+        raise ValueError("lse: contiguous FP32 [tokens][heads]")
+    states_a_row = columns * heads * parts
+    floats_a_row = states_a_row * (R + 2)
+    if workspace is None:
+        rows_a_launch = max(1, min(batch, (PARTIAL_BYTES // 4) // floats_a_row))
+        work = _partials(device, rows_a_launch * floats_a_row)
+    else:
+        if workspace.dtype != torch.float32 or not workspace.is_contiguous() or workspace.numel() < floats_a_row:
+            raise ValueError(f"workspace: contiguous FP32 with room for one row's partials at least ({floats_a_row})")
+        rows_a_launch = min(batch, workspace.numel() // floats_a_row)
+        work = workspace
     p = _abi.LatentParams()
-    p.q, p.cache, p.scales, p.tables = q.data_ptr(), cache.data_ptr(), _ptr(scales) if fp8 else None, tables.data_ptr()
+    p.q, p.cache, p.tables = q.data_ptr(), cache.data_ptr(), tables.data_ptr()
+    p.scales = _ptr(scales) if coded else None
     p.out, p.lse, p.sinks = out.data_ptr(), _ptr(lse), _ptr(sinks)
     p.q_stride_t, p.q_stride_h, p.out_stride_t, p.out_stride_h = q.stride(0), q.stride(1), out.stride(0), out.stride(1)
     p.table_stride, p.table_width = tables.stride(0), tables.shape[1]
-    p.columns, p.heads, p.rank, p.rope, p.page = int(columns), H, R, P, int(page)
-    p.cache_dtype = 2 if fp8 else (1 if cache.dtype == torch.float16 else 0)
+    p.columns, p.heads, p.rank, p.rope, p.page = columns, heads, R, P, int(page)
+    p.cache_dtype = _CACHE_DTYPE[cache.dtype]
     p.q_dtype, p.out_dtype = _DTYPE[q.dtype], _DTYPE[out.dtype]
-    p.scales_per_row = int(scales.shape[-1]) if fp8 else 0
+    p.scales_per_row = int(scales.shape[2]) if coded else 0
     p.partitions, p.piece, p.rows_are_64, p.phases = parts, piece, int(rows.dtype == torch.int64), int(phases)
-    p.scale = float(scale if scale is not None else width ** -0.5)
-    for at in range(0, B, rows_a_launch):
-        n = min(rows_a_launch, B - at)
-        states = n * per_row
-        p.partial_out = work.data_ptr()
-        p.partial_max = work.data_ptr() + states * R * 4
-        p.partial_sum = work.data_ptr() + states * (R + 1) * 4
+    p.scale = float((R + P) ** -0.5 if scale is None else scale)
+    base = work.data_ptr()
+    for first in range(0, batch, rows_a_launch):
+        n = min(rows_a_launch, batch - first)
+        states = n * states_a_row
+        p.partial_out, p.partial_max, p.partial_sum = base, base + 4 * states * R, base + 4 * states * (R + 1)
         p.n_rows = n
-        p.rows = rows.data_ptr() + at * rows.element_size()
-        p.starts, p.firsts = starts.data_ptr() + at * 4, firsts.data_ptr() + at * 8
-        p.counts = None if counts is None else counts.data_ptr() + at * 4
+        p.rows = rows.data_ptr() + first * rows.element_size()
+        p.starts, p.firsts = starts.data_ptr() + 4 * first, firsts.data_ptr() + 8 * first
+        p.counts = None if counts is None else counts.data_ptr() + 4 * first
         _launch(device, "crit_pkv_latent_attend", "latent_attention.attend", p)
     return out
 
@@ -200,31 +240,29 @@ def attend(q, cache, tables, rows, starts, firsts, columns, page, *, rank, count
 def prefill(q, cache, table, position, page, *, rank, scale=None, out: Optional[torch.Tensor] = None,
             lse: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None,
             scales: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """A prompt chunk of one sequence over the latent cache: q [T][heads][R + P] at positions position .. position +
-    T - 1 (their rows written), table [pages] int32 its page table, position an int or a one-element int64 device
-    tensor read on the device (one graph for every position) -> out [T][heads][R] in q's dtype (and lse [T][heads] when
-    given), causal. Read as windows of MAX_COLUMNS columns through attend(): a token's bits do not depend on the
-    chunk's length and are those of the same position decoded. Sinks, lse, scale and an E4M3 cache's scales as
-    attend()."""
-    T = q.shape[0]
-    _check(q, cache, page, rank, sinks, scales)
-    if T < 1 or table.dim() != 1:
-        raise ValueError("a prompt chunk is one token or more over one page table [pages]")
+    """A prompt chunk of one sequence, causal: q [T][heads][R + P] are the tokens at positions position .. position +
+    T - 1 (their rows already written), table [pages] int32 the sequence's page table; position is an int, or a
+    one-element int64 device tensor that is read on the device so that one captured graph serves every position.
+    Returns out [T][heads][R] (and fills lse [T][heads] when given). The chunk is read as windows of MAX_COLUMNS
+    columns through attend(), so a token's bits are those of the same position decoded and do not depend on T. scale,
+    sinks, lse and an E4M3 cache's scales as attend() takes them."""
+    _Call(q, cache, page, rank, sinks, scales)
+    count = q.shape[0]
+    if count < 1 or table.dim() != 1:
+        raise ValueError("prefill: at least one token, over one page table [pages]")
     device = q.device
     if torch.is_tensor(position):
-        first = position.reshape(1)
-        if first.dtype != torch.int64 or first.device != device:
-            raise ValueError("a device position is a one-element int64 tensor on q's device")
+        if position.numel() != 1 or position.dtype != torch.int64 or position.device != device:
+            raise ValueError("position: an int, or a one-element int64 tensor on q's device")
+        origin = position.reshape(1)
+    elif torch.cuda.is_current_stream_capturing():
+        raise RuntimeError("latent_attention.prefill: under capture pass `position` as a device tensor")
     else:
-        if torch.cuda.is_current_stream_capturing():
-            raise RuntimeError("latent_attention.prefill: a captured chunk takes its position as a device tensor")
-        first = torch.tensor([int(position)], dtype=torch.int64, device=device)
-    n = -(-T // MAX_COLUMNS)
-    step = torch.arange(n, dtype=torch.int64, device=device) * MAX_COLUMNS
-    counts = (T - step).clamp(max=MAX_COLUMNS).to(torch.int32)
-    tables = table.reshape(1, -1)
-    if tables.dtype != torch.int32:
-        tables = tables.to(torch.int32)
-    return attend(q, cache, tables, torch.zeros(n, dtype=torch.int32, device=device), step.to(torch.int32), first + step,
-                  min(MAX_COLUMNS, T), page, rank=rank, counts=counts, scale=scale, out=out, lse=lse, sinks=sinks,
-                  scales=scales, fused=True)
+        origin = torch.tensor([int(position)], dtype=torch.int64, device=device)
+    windows = -(-count // MAX_COLUMNS)
+    offsets = torch.arange(0, windows * MAX_COLUMNS, MAX_COLUMNS, dtype=torch.int64, device=device)
+    widths = torch.clamp(count - offsets, max=MAX_COLUMNS).to(torch.int32)
+    one_table = table.reshape(1, -1) if table.dtype == torch.int32 else table.reshape(1, -1).to(torch.int32)
+    return attend(q, cache, one_table, torch.zeros(windows, dtype=torch.int32, device=device), offsets.to(torch.int32),
+                  origin + offsets, min(MAX_COLUMNS, count), page, rank=rank, counts=widths, scale=scale, out=out, lse=lse,
+                  sinks=sinks, scales=scales, fused=True)

@@ -104,17 +104,18 @@ def _unsupported(what):
 
 # -- owners: what the module itself keeps on a device (reference __init__.py:129-171 keeps its workspaces the same way) --
 class _Holding:
-    """One owner's memory on one device: the partials of its split launches, the row states of its prompt chunks with
-    fresh rows, and the counters its unit-pulling launches draw from. Buffers a launch outgrew stay in `kept`: a
+    """One owner's memory on one device: the partials of its split launches (`latent`: those of its latent-attention
+    launches), the row states of its prompt chunks with fresh rows, and the counters its unit-pulling launches draw from. Buffers a launch outgrew stay in `kept`: a
     captured graph may still replay into them."""
-    __slots__ = ("partials", "states", "counters", "pairs_used", "pair_of", "kept")
+    __slots__ = ("partials", "states", "latent", "counters", "pairs_used", "pair_of", "kept")
 
     def __init__(self):
-        self.partials = self.states = self.counters = None
+        self.partials = self.states = self.latent = self.counters = None
         self.pairs_used, self.pair_of, self.kept = 0, {}, []
 
 
 COUNTER_PAIRS = 512      # counter pairs an owner's block holds (one a stream that launches, one a capture)
+COUNTER_HEADROOM = 384   # pairs an eager launch leaves free for captures: it starts a new block when fewer are left
 _holdings = {}           # (device index, owner key) -> _Holding
 _local = threading.local()
 
@@ -178,15 +179,21 @@ def _launch_state(device, stream):
     The pairs come from a zeroed block the owner holds; a launch leaves its pair zero."""
     holding = _holding(device)
     capture = _abi.capture_id(stream)
+    if not capture and (holding.counters is None or holding.pairs_used > COUNTER_PAIRS - COUNTER_HEADROOM):
+        # An eager launch tops the block up while there is still room for the captures that may follow it: a block is
+        # zeroed memory, which a capture cannot allocate. The pairs handed out stay where they are (`kept`).
+        if holding.counters is not None:
+            holding.kept.append(holding.counters)
+        holding.counters, holding.pairs_used = torch.zeros(2 * COUNTER_PAIRS, dtype=torch.int32, device=device), 0
     at = holding.pair_of.get((stream, capture))
     if at is None:
-        if holding.counters is None or holding.pairs_used == COUNTER_PAIRS:
-            if capture:
-                raise RuntimeError("paged_kv_attention.attend: run a launch once on this device before capturing one "
-                                   "(its launch counters are allocated, zeroed, outside a capture)")
-            if holding.counters is not None:
-                holding.kept.append(holding.counters)
-            holding.counters, holding.pairs_used = torch.zeros(2 * COUNTER_PAIRS, dtype=torch.int32, device=device), 0
+        if holding.counters is None:
+            raise RuntimeError("paged_kv_attention.attend: run a launch once on this device before capturing one "
+                               "(its launch counters are allocated, zeroed, outside a capture)")
+        if holding.pairs_used == COUNTER_PAIRS:
+            raise RuntimeError(f"paged_kv_attention.attend: {COUNTER_HEADROOM} captures in a row have used up this "
+                               "owner's launch counters; run one launch outside a capture (it allocates the next "
+                               "block) and capture again")
         at = holding.pair_of[(stream, capture)] = holding.counters.data_ptr() + 8 * holding.pairs_used
         holding.pairs_used += 1
     return at
@@ -292,9 +299,10 @@ def _cus(device):
 def _tuned(name, head_dim, value_dim, kv_heads, kind):
     """The engine's tuned value of an order knob of the split launch (the "split" structure, keyed by the cache's
     geometry as the reference keys it, __init__.py:262-286), 0 where it has none."""
-    if _crit_tuning is None or head_dim is None or value_dim is None or kv_heads is None:
+    if _crit_tuning is None or head_dim is None or kv_heads is None:
         return 0
-    key = {"D": int(head_dim), "DV": int(value_dim), "HKV": int(kv_heads), "KIND": KINDS[kind]}
+    # (a cache described by its key width alone has values of that width: the reference's _split_key, __init__.py:255-257)
+    key = {"D": int(head_dim), "DV": int(value_dim or head_dim), "HKV": int(kv_heads), "KIND": KINDS[kind]}
     return int(_crit_tuning.knobs("split", key, 1).get(name, 0) or 0)
 
 
@@ -850,7 +858,8 @@ def prefill(q, key_pages, value_pages, kind, table, position, page, *, key_scale
     products of the codes on the matrix cores (v_mfma_i32_32x32x32_i8) times the row's and the keys' scales; fresh rows
     are still read in q's type. derive: a Derive (or its tuple), as attend() takes it: the keys derived from the value
     pages (key_pages None); such a chunk is read as window rows of up to MAX_COLUMNS tokens by attend()'s fused launch
-    (a prompt token's bits are those of the same position decoded); not with fresh rows, flash or int8_qk."""
+    (a prompt token's bits are those of the same position decoded), with fresh rows too (a chunk's own value rows, their
+    keys derived the same way); not with flash or int8_qk."""
     if derive is not None:
         if flash:
             raise ValueError("derive= reads keys from the value rows on the split and fused launches and prefill's "

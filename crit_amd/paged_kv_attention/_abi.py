@@ -10,7 +10,7 @@ import shutil
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 NAME = "libcrit_pkv.so"
-ABI_VERSION = 17
+ABI_VERSION = 18
 
 KIND_16BIT, KIND_FP8, KIND_FP8_ROW, KIND_INT8 = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
@@ -115,6 +115,12 @@ class LatentParams(ctypes.Structure):
                 ("partitions", _i32), ("piece", _i32), ("rows_are_64", _i32), ("phases", _i32), ("scale", _f32)]
 
 
+class LatentWriteParams(ctypes.Structure):
+    _fields_ = [("latent", _p), ("rope", _p), ("slots", _p), ("cache", _p), ("scales", _p),
+                ("tokens", _i64), ("latent_stride", _i64), ("rope_stride", _i64),
+                ("rank", _i32), ("rope_width", _i32), ("in_dtype", _i32), ("cache_dtype", _i32)]
+
+
 class IndexScoresParams(ctypes.Structure):
     _fields_ = [("q", _p), ("keys", _p), ("key_scales", _p), ("weights", _p), ("ends", _p), ("slots", _p), ("out", _p),
                 ("q_stride_t", _i64), ("q_stride_h", _i64), ("key_stride", _i64), ("weights_stride", _i64),
@@ -138,7 +144,7 @@ class ReadParams(ctypes.Structure):
 STATIC_SCRATCH_BYTES = 32 << 20
 
 SYMBOLS = ("crit_pkv_write", "crit_pkv_attend", "crit_pkv_attend_static", "crit_pkv_merge", "crit_pkv_prefill", "crit_pkv_slots_at",
-           "crit_pkv_compact", "crit_pkv_copy_pages", "crit_pkv_round", "crit_pkv_step_buffers", "crit_pkv_latent_attend", "crit_pkv_index_scores", "crit_pkv_index_topk", "crit_pkv_index_topk_work_bytes", "crit_pkv_read_rows", "crit_pkv_abi_version", "crit_pkv_params_size", "crit_pkv_error",
+           "crit_pkv_compact", "crit_pkv_copy_pages", "crit_pkv_round", "crit_pkv_step_buffers", "crit_pkv_latent_attend", "crit_pkv_latent_write", "crit_pkv_index_scores", "crit_pkv_index_topk", "crit_pkv_index_topk_work_bytes", "crit_pkv_read_rows", "crit_pkv_abi_version", "crit_pkv_params_size", "crit_pkv_error",
            "crit_pkv_stream_read", "crit_pkv_stream_capture")
 
 _lib = None
@@ -189,6 +195,7 @@ def load():
                          ("crit_pkv_slots_at", SlotsParams), ("crit_pkv_compact", CompactParams),
                          ("crit_pkv_copy_pages", CopyPagesParams), ("crit_pkv_round", RoundParams),
                          ("crit_pkv_step_buffers", StepParams), ("crit_pkv_latent_attend", LatentParams),
+                         ("crit_pkv_latent_write", LatentWriteParams),
                          ("crit_pkv_index_scores", IndexScoresParams), ("crit_pkv_index_topk", IndexTopkParams),
                          ("crit_pkv_read_rows", ReadParams)):
         fn = getattr(lib, name)
@@ -204,7 +211,7 @@ def load():
         raise RuntimeError(f"{path} speaks ABI {lib.crit_pkv_abi_version()}, this package {ABI_VERSION}: rebuild it")
     for which, struct in enumerate((WriteParams, AttendParams, MergeParams, PrefillParams, SlotsParams, CompactParams,
                                     CopyPagesParams, ReadParams, RoundParams, StepParams, LatentParams,
-                                    IndexScoresParams, IndexTopkParams)):
+                                    IndexScoresParams, IndexTopkParams, LatentWriteParams)):
         if lib.crit_pkv_params_size(which) != ctypes.sizeof(struct):
             raise RuntimeError(f"{path}: parameter struct {which} is {lib.crit_pkv_params_size(which)} bytes, the "
                                f"Python mirror {ctypes.sizeof(struct)}: rebuild the library")
@@ -213,15 +220,15 @@ def load():
     return lib
 
 
-_capture = ctypes.c_ulonglong()
-
-
 def capture_id(stream):
-    """The id of the capture `stream` (a handle) is recording into, 0 when it is not capturing."""
-    code = load().crit_pkv_stream_capture(stream, ctypes.byref(_capture))
+    """The id of the capture `stream` (a handle) is recording into, 0 when it is not capturing. The cell the library
+    writes the id into is the call's own: ctypes lets other threads run during the call, and each owner launches from
+    its own thread."""
+    cell = ctypes.c_ulonglong()
+    code = load().crit_pkv_stream_capture(stream, ctypes.byref(cell))
     if code:
         check(code, "crit_pkv_stream_capture")
-    return _capture.value
+    return cell.value
 
 
 def check(code, what):

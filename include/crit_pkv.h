@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 17
+#define CRIT_PKV_ABI_VERSION 18
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -192,8 +192,10 @@ int crit_pkv_attend(const crit_pkv_attend_params* p, void* stream);
  * a static device array of CRIT_PKV_STATIC_SCRATCH_BYTES that the library holds on every GPU it runs on until the
  * process ends; partial_out, partial_max, partial_sum and launch_state of `p` are not read. Inputs and outputs are
  * the caller's as before. Calls nothing that allocates. Refused with CRIT_PKV_E_SCRATCH when 256 + n_rows * columns *
- * heads * partitions * (value_dim + 2) * 4 bytes exceed the array (fused launches need the 256 only). With offsets,
- * offsets[r] - offsets[0] + columns <= n_rows * columns for every row (rows packed by their counts are).
+ * heads * partitions * (value_dim + 2) * 4 bytes exceed the array (fused launches need the 256 only). A launch
+ * that any check refuses queues nothing on the stream. Precondition the library cannot check (offsets are device
+ * memory): with offsets, offsets[r] - offsets[0] + columns <= n_rows * columns for every row, as rows packed by
+ * their counts have it; a row past that bound would write its partials beyond the array.
  * Every call on one GPU uses that GPU's one array: calls that may overlap there (two streams, two threads, a graph
  * replaying beside eager calls) race on the partials and the counters; run them one after another. */
 #define CRIT_PKV_STATIC_SCRATCH_BYTES (32 * 1024 * 1024)
@@ -429,6 +431,25 @@ typedef struct crit_pkv_latent_params {
 
 int crit_pkv_latent_attend(const crit_pkv_latent_params* p, void* stream);
 
+/* ---- append to a latent cache ----------------------------------------------------------------------------------------
+ * Replaces write() of the latent-attention kernels module (latent_attention/__init__.py:74-97, torch indexing there):
+ * token t's latent [rank] and rotary key [rope_width] (in_dtype: CRIT_PKV_F32, _BF16 or _F16; rows latent_stride and
+ * rope_stride elements apart, each contiguous) go side by side into row slots[t] of cache [slots][rank + rope_width];
+ * a slot below 0 is skipped. cache_dtype 0 BF16 / 1 FP16: values rounded to nearest even. cache_dtype 2 E4M3: each of
+ * the two parts coded at its own scale, scale = max(max|x| / 448, 1e-30), code = e4m3(clamp(x / scale, -448, 448)) with
+ * IEEE divisions, the scales stored at scales[slot][0] (latent) and [slot][1] (rotary key). One launch. */
+typedef struct crit_pkv_latent_write_params {
+    const void* latent;
+    const void* rope;
+    const int64_t* slots;           /* [tokens] */
+    void* cache;
+    float* scales;                  /* [slots][2] FP32, cache_dtype 2; else NULL */
+    int64_t tokens, latent_stride, rope_stride;
+    int32_t rank, rope_width, in_dtype, cache_dtype;
+} crit_pkv_latent_write_params;
+
+int crit_pkv_latent_write(const crit_pkv_latent_write_params* p, void* stream);
+
 /* ---- sparse index selection ---------------------------------------------------------------------------------------
  * Replaces scores() and topk() of crit's sparse-indexer kernels module (kernels/techniques/attention/sparse-indexer/
  * torch-ext/sparse_indexer/__init__.py:83-139 and its score_kernel / topk_kernel / cuda_select.cu; the operation:
@@ -505,7 +526,7 @@ int crit_pkv_read_rows(const crit_pkv_read_params* p, void* stream);
 /* ---- housekeeping ------------------------------------------------------------------------------------------------- */
 int crit_pkv_abi_version(void);
 /* sizeof() of the parameter structs as the library was compiled, for the host's mirror to cross-check
- * (which: 0 write, 1 attend, 2 merge, 3 prefill, 4 slots_at, 5 compact, 6 copy_pages, 7 read_rows, 8 round, 9 step_buffers, 10 latent_attend, 11 index_scores, 12 index_topk), as crit_cw_params_size() does (cuda_window.cu:1502). */
+ * (which: 0 write, 1 attend, 2 merge, 3 prefill, 4 slots_at, 5 compact, 6 copy_pages, 7 read_rows, 8 round, 9 step_buffers, 10 latent_attend, 11 index_scores, 12 index_topk, 13 latent_write), as crit_cw_params_size() does (cuda_window.cu:1502). */
 int crit_pkv_params_size(int which);
 const char* crit_pkv_error(int code);
 /* *id = the id of the capture `stream` is recording into (never 0), or 0 when it is not capturing; returns 0 or a HIP

@@ -160,7 +160,7 @@ def test_what_it_cannot_read_is_refused():
         la.attend(q, cache.cache, cache.tables, *some(), 1, 64, rank=500)
     with pytest.raises(ValueError, match="columns a row"):
         cache.attend(q, [0], [0], [5], 65)
-    with pytest.raises(ValueError, match="sinks are contiguous FP32"):
+    with pytest.raises(ValueError, match="sinks: one FP32 logit a head"):
         cache.attend(q, [0], [0], [5], 1, sinks=torch.zeros(3, device=dev))
     with pytest.raises(NotImplementedError, match="is not built"):      # (the reference takes every power of two)
         la.attend(q[:, :, :48].contiguous(), torch.zeros(4, 64, 48, dtype=torch.bfloat16, device=dev), cache.tables, *some(), 1, 64, rank=32)
@@ -257,3 +257,102 @@ def test_the_partitions_are_a_knob_the_caller_or_the_tuning_sets():
     for bad in (0, 65):
         with pytest.raises(ValueError):
             cache.attend(q, [0, 1], [0, 8], [2990, 890], 8, partitions=bad)
+
+
+@pytest.mark.parametrize("source", [torch.float32, torch.bfloat16, torch.float16])
+def test_write_stores_the_bytes_and_scales_of_the_reference_rule(source):
+    # oracle.latent.write is the reference's torch rule (latent_attention/__init__.py:74-97); the module's write is one
+    # HIP launch and must leave the same bytes: rows of zeros (the 1e-30 floor), NaN and infinite inputs, values that
+    # saturate, an untouched row, and a skipped slot.
+    la = module()
+    g = torch.Generator().manual_seed(21)
+    n, R, P, page, pages = 37, 128, 32, 16, 6
+    latent = torch.randn(n, R, generator=g) * 3
+    rope_k = torch.randn(n, P, generator=g) * 40
+    latent[3] = 0
+    rope_k[4] = 0
+    latent[5, 7] = float("nan")
+    rope_k[6, 1] = float("inf")
+    latent[8, 0] = -0.0
+    latent, rope_k = latent.to(source), rope_k.to(source)
+    slots = torch.randperm(pages * page, generator=g)[:n]
+    for dtype in (torch.bfloat16, torch.float16, torch.float8_e4m3fn):
+        coded = dtype == torch.float8_e4m3fn
+        want = torch.zeros(pages, page, R + P, dtype=dtype)
+        want_scales = torch.zeros(pages, page, 2) if coded else None
+        oracle_latent.write(latent, rope_k, slots, want, want_scales)
+        got = torch.zeros(pages, page, R + P, dtype=dtype, device=dev)
+        got_scales = torch.zeros(pages, page, 2, device=dev) if coded else None
+        dropped = slots.clone().to(dev)
+        la.write(latent.to(dev), rope_k.to(dev), dropped, got, got_scales)
+        raw = torch.uint8 if coded else torch.int16
+
+        def same(a, b):      # bit for bit; a 16-bit NaN only as a NaN (its payload differs between torch's own casts)
+            if coded:
+                return torch.equal(a.view(raw), b.view(raw))
+            nan = torch.isnan(b.float())
+            return torch.equal(torch.isnan(a.float()), nan) and torch.equal(a.view(raw)[~nan], b.view(raw)[~nan])
+        assert same(got.cpu(), want), dtype
+        if coded:
+            found, nan = got_scales.cpu(), torch.isnan(want_scales)      # (a NaN row's scale is a NaN, whatever its payload)
+            assert torch.equal(torch.isnan(found), nan) and torch.equal(found.view(torch.int32)[~nan], want_scales.view(torch.int32)[~nan])
+        # a token whose slot is negative is skipped; strided inputs are read where they lie
+        got.zero_()
+        dropped[0] = -1
+        wide = torch.zeros(n, R + 8, dtype=source, device=dev)
+        wide[:, :R] = latent.to(dev)
+        la.write(wide[:, :R], rope_k.to(dev), dropped, got, got_scales)
+        kept = want.clone().view(-1, R + P)
+        kept[slots[0]] = 0
+        assert same(got.cpu(), kept.view(pages, page, R + P)), dtype
+
+
+def test_two_owners_launch_on_two_streams_without_sharing_partials_and_an_outgrown_buffer_outlives_its_graph():
+    import crit_amd.paged_kv_attention as pk
+    cache = Cache(512, 64, 64, [3000, 900, 2000], seed=31)
+    la = cache.la
+    q = _q(3, 16, 576, 32)
+    rows = torch.tensor([0, 1, 2], dtype=torch.int32, device=dev)
+    starts = torch.tensor([0, 1, 2], dtype=torch.int32, device=dev)
+    firsts = torch.tensor([2990, 890, 1990], dtype=torch.int64, device=dev)
+    args = (cache.cache, cache.tables, rows, starts, firsts, 1, 64)
+    serial = la.attend(q, *args, rank=512)
+    torch.cuda.synchronize()
+    one, two = torch.cuda.Stream(), torch.cuda.Stream()
+    out_a = torch.empty_like(serial)
+    out_b = [torch.empty_like(serial) for _ in range(6)]
+    try:
+        with pk.owner("a"), torch.cuda.stream(one):
+            la.attend(q, *args, rank=512, out=out_a)      # (the owner's partials exist before the capture)
+            one.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=one):
+                la.attend(q, *args, rank=512, out=out_a)
+        held = pk._holdings[(torch.cuda.current_device(), "a")].latent
+        for i in range(6):      # owner a's graph replays on one stream while owner b launches on another
+            out_a.zero_()
+            with torch.cuda.stream(one):
+                graph.replay()
+            with pk.owner("b"), torch.cuda.stream(two):
+                la.attend(q, *args, rank=512, out=out_b[i])
+        torch.cuda.synchronize()
+        assert torch.equal(out_a, serial)
+        assert all(torch.equal(o, serial) for o in out_b)
+        assert pk._holdings[(torch.cuda.current_device(), "b")].latent.data_ptr() != held.data_ptr()
+        # owner a outgrows its buffer with a larger eager launch: the graph still replays into the old one, which is
+        # kept, so memory allocated afterwards is not what the replay writes
+        wide_q = _q(24, 128, 576, 33)
+        with pk.owner("a"):
+            cache.attend(wide_q, [0, 1, 2], [0, 8, 16], [2990, 890, 1990], 8)
+            grown = pk._holdings[(torch.cuda.current_device(), "a")].latent
+        assert grown.data_ptr() != held.data_ptr() and grown.numel() > held.numel()
+        fresh = [torch.full((held.numel(),), 5.0, device=dev) for _ in range(4)]
+        out_a.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_a, serial)
+        assert all(bool((t == 5.0).all()) for t in fresh)
+        del graph
+    finally:
+        pk.release("a")
+        pk.release("b")
