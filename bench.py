@@ -658,6 +658,74 @@ def index_selection(device):
     return found
 
 
+def reference_shapes(pk, device):
+    """The shapes the reference publishes its decode and append rows on (its paged-kv-attention README: 24 query / 4 KV
+    heads x 256 over `fp8:row` pages of 64, 24 / 2 x 256 bf16, 56 / 8 x 128 int8 row-scaled; 1 and 8 rows; 1, 5 and 8
+    columns; 4K, 16K and 200K positions; `write` of 1 / 256 / 4,096 tokens into 8,192 shuffled slots), one layer,
+    replayed from a captured graph over four caches read in turn (each launch cold), each with its fraction of the
+    8 TB/s HBM peak. The reference's own figures are for another card (RTX 5090) and are context, not a target. Widths
+    other than 128 x 128 take attend_generic_kernel; 56 / 8 x 128 the matrix-core kernel."""
+    found = {}
+    g = torch.Generator(device=device).manual_seed(11)
+    shapes = (("24q_4kv_x256_fp8row_page64", 24, 4, 256, 64, "fp8:row"), ("24q_2kv_x256_bf16_page16", 24, 2, 256, 16, "bf16"),
+              ("56q_8kv_x128_int8_page16", 56, 8, 128, 16, "int8"))
+    for name, hq, hkv, d, page, kind in shapes:
+        e = 2 if kind == "bf16" else 1
+        store = torch.bfloat16 if kind == "bf16" else (torch.int8 if kind == "int8" else torch.float8_e4m3fn)
+        for ctx, rows_cases in ((4096, ((1, 1), (8, 1))), (16384, ((1, 1), (8, 1))), (200_000, ((1, 1), (1, 5), (1, 8), (8, 1)))):
+            most = max(b for b, _ in rows_cases)
+            width = ((ctx + 8 + page - 1) // page + 15) // 16 * 16
+            pages = most * width
+            layers = 4 if pages * page * hkv * d * e * 2 < (1 << 30) else 2      # (caches read in turn: every launch cold)
+            caches = []
+            for _ in range(layers):
+                if kind == "bf16":
+                    k = torch.randn(pages + 1, page, hkv, d, device=device, dtype=torch.bfloat16, generator=g)
+                    v = torch.randn(pages + 1, page, hkv, d, device=device, dtype=torch.bfloat16, generator=g)
+                    caches.append((k, v, None, None))
+                else:
+                    if kind == "int8":
+                        k = torch.randint(-100, 100, (pages + 1, page, hkv, d), device=device, dtype=torch.int8, generator=g)
+                        v = torch.randint(-100, 100, (pages + 1, page, hkv, d), device=device, dtype=torch.int8, generator=g)
+                    else:
+                        k = (torch.randn(pages + 1, page, hkv, d, device=device, dtype=torch.bfloat16, generator=g) * 50).to(store)
+                        v = (torch.randn(pages + 1, page, hkv, d, device=device, dtype=torch.bfloat16, generator=g) * 50).to(store)
+                    ks = torch.rand(pages + 1, page, hkv, device=device, generator=g) * 0.01 + 0.001
+                    caches.append((k, v, ks, ks.clone()))
+            tables = torch.randperm(pages, device=device, generator=g).to(torch.int32).view(most, width).contiguous()
+            for batch, columns in rows_cases:
+                rows = torch.arange(batch, dtype=torch.int32, device=device)
+                starts = rows * columns
+                firsts = torch.full((batch,), ctx - columns, dtype=torch.int64, device=device)
+                q = torch.randn(batch * columns, hq, d, device=device, generator=g).to(torch.bfloat16)
+                out = torch.empty_like(q)
+                at = [0]
+
+                def launch():
+                    at[0] = (at[0] + 1) % layers
+                    k, v, ks, vs = caches[at[0]]
+                    pk.attend(q, k, v, kind, tables, rows, starts, firsts, columns, page, out=out, key_scales=ks,
+                              value_scales=vs)
+                ms = graph_timed(launch, 8)
+                nbytes = batch * ctx * hkv * (2 * d * e + (8 if kind != "bf16" else 0))
+                found[f"{name}_{batch}_rows_{columns}_cols_ctx{ctx}"] = {
+                    "us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1),
+                    "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+            del caches
+            torch.cuda.empty_cache()
+    # write(): tokens into 8,192 shuffled slots, bf16 24 / 2 x 256 (the reference's append row)
+    hkv, d = 2, 256
+    k = torch.zeros(8192, hkv, d, dtype=torch.bfloat16, device=device)
+    v = torch.zeros_like(k)
+    for T in (1, 256, 4096):
+        keys = torch.randn(T, hkv, d, device=device, generator=g).to(torch.bfloat16)
+        values = torch.randn(T, hkv, d, device=device, generator=g).to(torch.bfloat16)
+        slots = torch.randperm(8192, device=device, generator=g)[:T]
+        ms = graph_timed(lambda: pk.write(keys, values, slots, k, v, "bf16"), 20)
+        found[f"write_{T}_tokens_into_8192_slots_bf16_2kv_x256"] = {"us": round(ms * 1e3, 2), "GB/s": round(T * hkv * 2 * d * 4 / ms / 1e6, 1)}
+    return found
+
+
 def small_batches(pk, device):
     """What a piece costs a batch that does not fill the chip: one layer's decode launch (split + merge, 8B shape) for
     4 sequences of about 2,000 positions and for one of 8,000, at the default piece and at pieces of 256 positions
@@ -785,6 +853,8 @@ def main():
                     help="run only the pool bookkeeping of the extras (slots, the move of accepted rows, page copies)")
     ap.add_argument("--latent-only", action="store_true", help="run only the latent-attention decode of the extras")
     ap.add_argument("--index-only", action="store_true", help="run only the sparse index selection of the extras")
+    ap.add_argument("--shapes-only", action="store_true",
+                    help="run only the decode and append rows at the shapes the reference publishes its own on")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch one KV append of 262,144 tokens: with the stream-read probe, two kernels of known "
                          "read and write sizes against which FETCH_SIZE / WRITE_SIZE counters are scaled")
@@ -810,6 +880,11 @@ def main():
         found = index_selection(device)
         log(f"[bench] sparse index selection: {found}")
         print(json.dumps({"sparse_index_selection": found}), flush=True)
+        return
+    if args.shapes_only:
+        found = reference_shapes(pk, device)
+        log(f"[bench] the reference's published shapes: {found}")
+        print(json.dumps({"reference_published_shapes": found}), flush=True)
         return
     if args.pool_only:
         found = pool_bookkeeping(pk, device)
@@ -925,6 +1000,9 @@ def main():
         log(f"[bench] prefill over 8-bit pages: {extras['prefill_8bit_pages']}")
         extras["prefill_fp8_pages_fresh_rows"] = prefill_fresh(pk, device)
         log(f"[bench] prefill over FP8 pages, with fresh rows: {extras['prefill_fp8_pages_fresh_rows']}")
+        torch.cuda.empty_cache()
+        extras["reference_published_shapes"] = reference_shapes(pk, device)
+        log(f"[bench] the reference's published shapes: {extras['reference_published_shapes']}")
         torch.cuda.empty_cache()
         extras["small_batches_by_piece"] = small_batches(pk, device)
         log(f"[bench] small batches, default piece and 256: {extras['small_batches_by_piece']}")

@@ -207,8 +207,10 @@ int launch_merge(const crit_pkv_merge_params* p, hipStream_t stream) {
     return hip_code(hipGetLastError());
 }
 
+// The tile heights the kernels are built for. A tile taller than a launch's rows computes rows nobody stores; a row's
+// bits do not depend on the height of the tile it sits in.
 static int pick_qr(int live_rows) {
-    static const int choices[] = {1, 2, 4, 5, 6, 8};
+    static const int choices[] = {1, 2, 4, 8};
     for (int c : choices)
         if (live_rows <= c) return c;
     return 8;
@@ -309,10 +311,10 @@ static int launch_attend_checked(const crit_pkv_attend_params* p, hipStream_t st
     const int live_rows = p->columns * a.g;
     int qr = pick_qr(live_rows);
     if (p->blocks) {      // a tile of one column's rows: the largest tile height that divides the group
-        qr = 1;
-        for (int q : {2, 4, 5, 6, 8})
-            if (a.g % q == 0) qr = q;
+        qr = a.g % 4 == 0 ? 4 : 1;      // (the block-list kernels are built for tiles of 1 and 4 rows)
     }
+    // The generic kernel's variants that read fresh rows or derive their keys are built for tiles of 2 and 8 rows.
+    if (fresh || derive) qr = qr <= 2 ? 2 : 8;
     // The 128-wide kernel serves two adjacent KV heads per wavefront where the head count is even, so every position
     // is read in segments of two rows (512 bytes of 16-bit pages, 256 of 8-bit ones): measured best on MI355X against
     // one and four heads. Fixed by the cache's geometry, never by the launch: a column's bits depend on it.

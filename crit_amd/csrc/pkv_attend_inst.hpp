@@ -10,7 +10,11 @@ namespace pkv {
 
 template <int KIND, bool F16, int QR, bool FUSED>
 static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipStream_t stream) {
-    if constexpr (!FUSED) {
+    // (which tile heights each variant is built for: launch_attend picks among them)
+    constexpr bool LISTS = QR == 1 || QR == 4, SPECIAL = QR == 2 || QR == 8;
+    if (a.blocks && (FUSED || !LISTS)) return CRIT_PKV_E_GEOMETRY;
+    if ((a.derive_table || a.fv) && !SPECIAL) return CRIT_PKV_E_GEOMETRY;
+    if constexpr (!FUSED && LISTS) {
         if (a.blocks && a.fast128) {
             // block lists whose steps lie in one block and one page: the bandwidth path walking each column's list
             AttendArgs u = a;
@@ -38,6 +42,7 @@ static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipS
             return hip_code(hipGetLastError());
         }
     }
+    if constexpr (SPECIAL) {
     if (a.derive_table && a.fv) {      // derived keys over pages and fresh value rows
         switch (lpr) {
             case 8: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 8, QR, FUSED, false, true, true>), grid, dim3(256), 0, stream, a); break;
@@ -59,7 +64,10 @@ static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipS
             case 32: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 32, QR, FUSED, false, true>), grid, dim3(256), 0, stream, a); break;
             default: return CRIT_PKV_E_GEOMETRY;
         }
-    } else if (lpr == 16) {
+    }
+    if (a.derive_table || a.fv) return hip_code(hipGetLastError());
+    }
+    if (lpr == 16) {
         hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 16, QR, FUSED>), grid, dim3(256), 0, stream, a);
     } else if (lpr == 8) {
         hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 8, QR, FUSED>), grid, dim3(256), 0, stream, a);
@@ -105,7 +113,7 @@ static int launch_kind_impl(const AttendArgs& a, int lpr, int qr, bool fused, bo
     case Q:                                                                                       \
         return fused ? launch_one<KIND, F16, Q, true>(a, lpr, page16, grid, stream)               \
                      : launch_one<KIND, F16, Q, false>(a, lpr, page16, grid, stream);
-        PKV_CASE(1) PKV_CASE(2) PKV_CASE(4) PKV_CASE(5) PKV_CASE(6) PKV_CASE(8)
+        PKV_CASE(1) PKV_CASE(2) PKV_CASE(4) PKV_CASE(8)
 #undef PKV_CASE
     }
     return CRIT_PKV_E_GEOMETRY;

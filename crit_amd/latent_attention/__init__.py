@@ -40,7 +40,7 @@ MAX_COLUMNS = 64
 PARTIAL_BYTES = 512 << 20   # the most partials one launch may take; a larger batch goes in several launches of rows
 PIECE = 256                 # default positions a piece
 MAX_PARTS = 64
-SHAPES = ((512, 64), (256, 64), (128, 64), (128, 32), (64, 64), (64, 32))   # (R, P) pairs the kernels are built for
+SHAPES = ((1024, 64), (512, 128), (512, 64), (256, 64), (128, 64), (128, 32), (64, 64), (64, 32))   # (R, P) the kernels are built for
 FP8 = torch.float8_e4m3fn
 _DTYPE = {torch.float32: _abi.F32, torch.bfloat16: _abi.BF16, torch.float16: _abi.F16}
 _CACHE_DTYPE = {torch.bfloat16: 0, torch.float16: 1, FP8: 2}

@@ -406,7 +406,7 @@ int crit_pkv_step_buffers(const crit_pkv_step_params* p, void* stream);
  * partition order, the sink logit (sinks [heads], natural log, -inf: none) folded in last; lse [tokens][heads] the
  * natural log-sum-exp (the sink counted). cache_dtype: 0 BF16, 1 FP16 (q in the same type), 2 E4M3 with `scales`
  * [pages][page][scales_per_row] FP32 (2: the latent's and the rotary key's, 1: one for the row) and BF16 or FP16 q.
- * (rank, rope) is one of (512, 64), (256, 64), (128, 64), (128, 32), (64, 64), (64, 32). phases: 0 both launches, 1
+ * (rank, rope) is one of (1024, 64), (512, 128), (512, 64), (256, 64), (128, 64), (128, 32), (64, 64), (64, 32). phases: 0 both launches, 1
  * the partitions only, 2 the merge only. */
 typedef struct crit_pkv_latent_params {
     const void* q;

@@ -73,7 +73,8 @@ def _q(tokens, heads, width, seed, dtype=torch.bfloat16):
 
 
 @pytest.mark.parametrize("rank,rope,heads,page", [(512, 64, 16, 64), (512, 64, 128, 16), (256, 64, 8, 32), (128, 32, 20, 16),
-                                                 (64, 32, 3, 48), (128, 64, 5, 16), (64, 64, 40, 16)])
+                                                 (64, 32, 3, 48), (128, 64, 5, 16), (64, 64, 40, 16), (1024, 64, 16, 64),
+                                                 (512, 128, 24, 16)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_windows_match_float64_latent_attention(rank, rope, heads, page, dtype):
     cache = Cache(rank, rope, page, [130, 64, 1, 517], dtype=dtype)
