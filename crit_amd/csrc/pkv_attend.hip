@@ -258,6 +258,7 @@ static int launch_attend_checked(const crit_pkv_attend_params* p, hipStream_t st
     }
     const int lpr = (p->head_dim > p->value_dim ? p->head_dim : p->value_dim) / 8;      // lanes that hold the wider row
     const bool wide128 = p->head_dim == 128 && p->value_dim == 128;
+    const bool wide256 = p->head_dim == 256 && p->value_dim == 256;      // (the matrix-core kernel's second width: two halves of 128)
     const int sp = 4 * (64 / lpr);
     if (p->partitions < 1 || p->partitions > 65535 || p->piece < 1 || p->piece % sp) return CRIT_PKV_E_WORKSPACE;
     if (!p->fused && (!p->partial_out || !p->partial_max || !p->partial_sum)) return CRIT_PKV_E_WORKSPACE;
@@ -326,8 +327,8 @@ static int launch_attend_checked(const crit_pkv_attend_params* p, hipStream_t st
     // The bandwidth kernel walks pages that are powers of two from 16 positions up, in positions below 2^31; other
     // multiples of 16 take the generic kernel. (block lists of blocks that are a multiple of 16: their own variant)
     const bool pow2_page = a.page_shift >= 4 && (int64_t)p->partitions * p->piece <= 0x3fffffff;
-    a.fast128 = wide128 && !derive && ((page16 && pow2_page) || fast_lists);      // (derived keys: the generic kernel)
-    if (a.fast128 && p->kv_heads % 2 == 0) a.heads_per_wave = 2;
+    a.fast128 = !derive && (((wide128 || wide256) && page16 && pow2_page && p->piece % 16 == 0) || fast_lists);      // (derived keys: the generic kernel)
+    if (a.fast128 && wide128 && p->kv_heads % 2 == 0) a.heads_per_wave = 2;
     // Query rows a tile holds: the generic and block-list kernels' tile height; 16 a wavefront's heads share in the
     // bandwidth kernel (matrix tiles of 16 columns).
     const int tile_rows = a.fast128 && !p->blocks ? 16 / a.heads_per_wave : qr;

@@ -83,7 +83,7 @@ static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipS
     return hip_code(hipGetLastError());
 }
 
-// 128-wide heads over pages of a multiple of 16 positions: the bandwidth path, resident workgroups pulling units.
+// 128- and 256-wide heads over pages of a multiple of 16 positions: the bandwidth path, resident workgroups pulling units.
 template <int KIND, bool F16>
 static int launch_mfma(const AttendArgs& a, bool fused, dim3 grid, hipStream_t stream) {
     AttendArgs u = a;
@@ -91,15 +91,16 @@ static int launch_mfma(const AttendArgs& a, bool fused, dim3 grid, hipStream_t s
     u.units_x = (int)grid.x, u.units_y = fused ? (int)grid.y : (int)grid.y + kTailClasses - 1;
     const int64_t units = (int64_t)u.units_x * u.units_y;
     if (units > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
-    const int64_t resident = (int64_t)compute_units() * kMfmaWaves;
+    const int64_t resident = (int64_t)compute_units() * (a.dk == 256 ? 1 : kMfmaWaves);
     const dim3 pgrid((unsigned)(units < resident ? units : resident));
     const bool masked = a.parents != nullptr || a.parents64 != nullptr || a.sliding > 0;
-    const int which = (a.heads_per_wave == 2 ? 4 : 0) + (fused ? 2 : 0) + (masked ? 1 : 0);
+    const int which = (a.dk == 256 ? 8 : (a.heads_per_wave == 2 ? 4 : 0)) + (fused ? 2 : 0) + (masked ? 1 : 0);
     switch (which) {
-#define PKV_MFMA(W, HWV, FU, MA) \
-    case W: hipLaunchKernelGGL((attend_mfma_kernel<KIND, F16, HWV, FU, MA>), pgrid, dim3(256), 0, stream, u); break;
-        PKV_MFMA(0, 1, false, false) PKV_MFMA(1, 1, false, true) PKV_MFMA(2, 1, true, false) PKV_MFMA(3, 1, true, true)
-        PKV_MFMA(4, 2, false, false) PKV_MFMA(5, 2, false, true) PKV_MFMA(6, 2, true, false) PKV_MFMA(7, 2, true, true)
+#define PKV_MFMA(W, HWV, FU, MA, DH) \
+    case W: hipLaunchKernelGGL((attend_mfma_kernel<KIND, F16, HWV, FU, MA, DH>), pgrid, dim3(256), 0, stream, u); break;
+        PKV_MFMA(0, 1, false, false, 1) PKV_MFMA(1, 1, false, true, 1) PKV_MFMA(2, 1, true, false, 1) PKV_MFMA(3, 1, true, true, 1)
+        PKV_MFMA(4, 2, false, false, 1) PKV_MFMA(5, 2, false, true, 1) PKV_MFMA(6, 2, true, false, 1) PKV_MFMA(7, 2, true, true, 1)
+        PKV_MFMA(8, 1, false, false, 2) PKV_MFMA(9, 1, false, true, 2) PKV_MFMA(10, 1, true, false, 2) PKV_MFMA(11, 1, true, true, 2)
 #undef PKV_MFMA
     }
     return hip_code(hipGetLastError());

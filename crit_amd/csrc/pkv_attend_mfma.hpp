@@ -94,11 +94,11 @@ PKV_DEV float sum_across_quarters(float x) {      // (row 0 + row 1) + (row 2 + 
     return u2f((uint32_t)b[0]) + u2f((uint32_t)b[1]);
 }
 
-template <int KIND>
+template <int KIND, int DH>
 struct Tile {
     using VVec = typename std::conditional<KIND == 0, u32x4, u32x2>::type;
-    u32x4 k[KIND == 0 ? 4 : 2];      // the lane's pieces of its position's K row
-    VVec v[4];                        // the lane's 8 dims of the V rows of its quarter's four positions
+    u32x4 k[(KIND == 0 ? 4 : 2) * DH];      // the lane's pieces of its position's K row
+    VVec v[4][DH];                           // the lane's 8 dims (of each 128-wide half) of the V rows of its quarter's four positions
     float ks[KIND >= 2 ? 4 : 1], vs[KIND >= 2 ? 4 : 1];      // row-scaled kinds: the scales of positions 4 u .. 4 u + 3
 };
 
@@ -122,16 +122,20 @@ constexpr int kMfmaTiles = 2;
 // happen while the next unit's rows are already on their way. A drawn unit without work (the list is a grid over rows
 // of different lengths) is passed over by the drawing thread at once. The last workgroup to finish zeroes the counters
 // for the next launch that uses them. Without counters the units are dealt in turn.
-// MASKED: draft trees and sliding windows.
-template <int KIND, bool F16, int HW, bool FUSED, bool MASKED>
-__global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs a) {
+// MASKED: draft trees and sliding windows. DH: 128-wide halves of a head (1: heads of 128; 2: heads of 256, whose rows
+// are 512 bytes of 16-bit pages by themselves, so a wavefront serves one KV head: HW 1): twice the key pieces, query
+// pieces, score products and output tiles, the same layouts otherwise; twice the registers too, so one workgroup a
+// compute unit, which keeps as many bytes in flight as two of the narrower ones (a step's rows are twice as long).
+template <int KIND, bool F16, int HW, bool FUSED, bool MASKED, int DH = 1>
+__global__ __launch_bounds__(256, DH == 2 ? 1 : kMfmaWaves) void attend_mfma_kernel(AttendArgs a) {
     constexpr int NT = kMfmaTiles;
-    constexpr int D = 128;
+    constexpr int D = 128 * DH;
+    static_assert(DH == 1 || (DH == 2 && HW == 1), "heads of 128 or 256; one KV head a wavefront at 256");
     constexpr int EB = KIND == 0 ? 2 : 1;
     constexpr int CPH = kTileRows / HW;      // tile columns a KV head holds
     constexpr int SPW = kTileRows / HW;      // positions a wavefront's step covers (tile rows a KV head holds)
     constexpr int EPT = kTileRows * D / 256; // output elements a thread folds
-    __shared__ __align__(16) float s_acc[4][kTileRows][128];
+    __shared__ __align__(16) float s_acc[4][kTileRows][D];
     __shared__ float s_m[4][kTileRows], s_l[4][kTileRows];
     __shared__ int s_rows[kLdsRows][5];      // count, first position, table row, first token, first partial row
     __shared__ int s_before[kLdsRows + 1];   // the dense list: partitions but the last of the rows before row r
@@ -365,15 +369,10 @@ __global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs
     // Loads of one step from its first slot. Every lane loads its place of the step whether the row holds that
     // position or not (the page does; a step past the row's keys is never listed): what such a place holds is dropped
     // where it is used (keys: the score is masked; values and scales: zeroed, see sanitize()).
-    auto fetch_k = [&](const Unit& un, int64_t slot0, Tile<KIND>& t) __attribute__((always_inline)) {
+    auto fetch_k = [&](const Unit& un, int64_t slot0, Tile<KIND, DH>& t) __attribute__((always_inline)) {
         const uint8_t* sbase = a.kp + slot0 * slot_bytes + un.kvh0 * D * EB;
-        if constexpr (KIND == 0) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) t.k[c] = *reinterpret_cast<const u32x4*>(sbase + kvo + 64 * c);
-        } else {
-            t.k[0] = *reinterpret_cast<const u32x4*>(sbase + kvo);
-            t.k[1] = *reinterpret_cast<const u32x4*>(sbase + kvo + 64);
-        }
+        for (int c = 0; c < (KIND == 0 ? 4 : 2) * DH; ++c) t.k[c] = *reinterpret_cast<const u32x4*>(sbase + kvo + 64 * c);
         if constexpr (KIND >= 2) {
             const float* ks = a.ks + slot0 * a.hkv + un.kvh0;
             const float* vs = a.vs + slot0 * a.hkv + un.kvh0;
@@ -381,11 +380,14 @@ __global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs
             for (int i = 0; i < 4; ++i) t.ks[i] = ks[svo + i * a.hkv], t.vs[i] = vs[svo + i * a.hkv];
         }
     };
-    auto fetch_v = [&](const Unit& un, int64_t slot0, Tile<KIND>& t) __attribute__((always_inline)) {
+    auto fetch_v = [&](const Unit& un, int64_t slot0, Tile<KIND, DH>& t) __attribute__((always_inline)) {
         const uint8_t* sbase = a.vp + slot0 * slot_bytes + un.kvh0 * D * EB;
 #pragma unroll
-        for (int p = 0; p < 4; ++p)
-            t.v[p] = __builtin_nontemporal_load(reinterpret_cast<const typename Tile<KIND>::VVec*>(sbase + vvo[p]));
+        for (int p = 0; p < 4; ++p) {
+#pragma unroll
+            for (int h = 0; h < DH; ++h)
+                t.v[p][h] = __builtin_nontemporal_load(reinterpret_cast<const typename Tile<KIND, DH>::VVec*>(sbase + vvo[p] + h * 128 * EB));
+        }
     };
 
     // -- what a lane holds for one unit: its tile column's token, query head, last visible position, ancestors, scale,
@@ -396,7 +398,7 @@ __global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs
     float vm_cur[HW], vm_nxt[HW];      // FP8 pages: the value multipliers of the unit's heads (requested with its queries, not in its fold)
 #pragma unroll
     for (int h = 0; h < HW; ++h) vm_cur[h] = vm_nxt[h] = 1.0f;
-    u32x4 qb[4];
+    u32x4 qb[4 * DH];
     auto value_multipliers = [&](const Unit& un) __attribute__((always_inline)) {      // (requested with the unit's page table entries)
         if constexpr (KIND == 1) {
 #pragma unroll
@@ -413,7 +415,7 @@ __global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs
         if constexpr (KIND == 1) sscale = a.sscale * (a.hm ? a.hm[un.kvh0 + hsel] : a.k_mult);
         const uint8_t* row = a.q + ((int64_t)(un.start + col) * a.q_st + (int64_t)qhead * a.q_sh) * 2;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
+        for (int c = 0; c < 4 * DH; ++c) {
             // 16-bit pages: dims 32 c + 8 u4 ..; 8-bit pages: dims 64 (c / 2) + 16 u4 + 8 (c % 2) .. (the codes a lane's two loads hold)
             const int dim = KIND == 0 ? 32 * c + 8 * u4 : 64 * (c / 2) + 16 * u4 + 8 * (c % 2);
             qb[c] = u32x4{0, 0, 0, 0};
@@ -421,7 +423,7 @@ __global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs
         }
     };
 
-    Tile<KIND> t[NT];
+    Tile<KIND, DH> t[NT];
     auto fill = [&](const Unit& un, const Lead& f) __attribute__((always_inline)) {      // a partition's first NT steps
         const int again = f.base[0] >= 0 ? f.base[0] : 0;
 #pragma unroll
@@ -471,31 +473,34 @@ __global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs
             for (int e = 0; e < (FUSED ? EPT : 1); ++e) run_m[e] = -INFINITY, run_l[e] = 0.0f, run_a[e] = 0.0f;
             for (int part = part_lo; part < part_hi; ++part) {
                 float m = -INFINITY, l = 0.0f;      // the lane's column: running maximum (the same in its four lanes), the lane's share of the sum
-                f32x4 acc[8];                        // O^T: acc[j][i] = dim 32 u4 + 8 i + j of the lane's column
+                f32x4 acc[8 * DH];                   // O^T: acc[8 h + j][i] = dim 128 h + 32 u4 + 8 i + j of the lane's column
 #pragma unroll
-                for (int j = 0; j < 8; ++j) acc[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                for (int j = 0; j < 8 * DH; ++j) acc[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-                auto step = [&](int base, Tile<KIND>& tl, auto&& refill_k, auto&& refill_v) __attribute__((always_inline)) {
+                auto step = [&](int base, Tile<KIND, DH>& tl, auto&& refill_k, auto&& refill_v) __attribute__((always_inline)) {
                     if (base + SPW > cur.n_keys) {
                         // The row's last step: what lies past its keys may be anything, and a probability of zero
                         // times a NaN is a NaN.
 #pragma unroll
                         for (int p = 0; p < 4; ++p) {
                             if (base + r_pos + p >= cur.n_keys) {
-                                if constexpr (KIND == 0) tl.v[p] = u32x4{0, 0, 0, 0};
-                                else tl.v[p] = u32x2{0, 0};
+#pragma unroll
+                                for (int h = 0; h < DH; ++h) {
+                                    if constexpr (KIND == 0) tl.v[p][h] = u32x4{0, 0, 0, 0};
+                                    else tl.v[p][h] = u32x2{0, 0};
+                                }
                                 if constexpr (KIND >= 2) tl.vs[p] = 0.0f;
                             }
                         }
                     }
                     // -- scores
-                    u32x4 ka[4];
+                    u32x4 ka[4 * DH];
                     if constexpr (KIND == 0) {
 #pragma unroll
-                        for (int c = 0; c < 4; ++c) ka[c] = tl.k[c];
+                        for (int c = 0; c < 4 * DH; ++c) ka[c] = tl.k[c];
                     } else {
 #pragma unroll
-                        for (int c = 0; c < 4; ++c) {
+                        for (int c = 0; c < 4 * DH; ++c) {
                             const uint32_t w0 = c % 2 ? tl.k[c / 2].z : tl.k[c / 2].x, w1 = c % 2 ? tl.k[c / 2].w : tl.k[c / 2].y;
                             const u32x2 lo = codes4_to_pairs<KIND>(w0), hi = codes4_to_pairs<KIND>(w1);
                             ka[c] = u32x4{lo.x, lo.y, hi.x, hi.y};
@@ -503,8 +508,11 @@ __global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs
                     }
                     f32x4 s0 = mfma_k32<F16>(ka[0], qb[0], f32x4{0.0f, 0.0f, 0.0f, 0.0f});
                     f32x4 s1 = mfma_k32<F16>(ka[1], qb[1], f32x4{0.0f, 0.0f, 0.0f, 0.0f});
-                    s0 = mfma_k32<F16>(ka[2], qb[2], s0);
-                    s1 = mfma_k32<F16>(ka[3], qb[3], s1);
+#pragma unroll
+                    for (int c = 2; c < 4 * DH; c += 2) {      // (two chains, the even pieces and the odd ones)
+                        s0 = mfma_k32<F16>(ka[c], qb[c], s0);
+                        s1 = mfma_k32<F16>(ka[c + 1], qb[c + 1], s1);
+                    }
                     float ks4[4], vs4[4];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) ks4[i] = KIND >= 2 ? tl.ks[i] : 1.0f, vs4[i] = KIND >= 2 ? tl.vs[i] : 1.0f;
@@ -534,31 +542,34 @@ __global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs
                     m = m_new;
                     if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {     // some row's maximum moved: rescale
 #pragma unroll
-                        for (int j = 0; j < 8; ++j) acc[j] *= alpha;
+                        for (int j = 0; j < 8 * DH; ++j) acc[j] *= alpha;
                     }
                     const u32x2 pb = {pair16<F16>(p[0] * vs4[0], p[1] * vs4[1]), pair16<F16>(p[2] * vs4[2], p[3] * vs4[3])};
                     // -- values: dims {8 i + j} of the lane's four rows as two 16-bit pairs (one v_perm each), then O^T += V^T P^T
+#pragma unroll
+                    for (int h = 0; h < DH; ++h) {
                     if constexpr (KIND == 0) {
 #pragma unroll
                         for (int w = 0; w < 4; ++w) {
-                            const u32x2 lo = {__builtin_amdgcn_perm(tl.v[1][w], tl.v[0][w], 0x05040100), __builtin_amdgcn_perm(tl.v[3][w], tl.v[2][w], 0x05040100)};
-                            const u32x2 hi = {__builtin_amdgcn_perm(tl.v[1][w], tl.v[0][w], 0x07060302), __builtin_amdgcn_perm(tl.v[3][w], tl.v[2][w], 0x07060302)};
-                            acc[2 * w] = mfma_k16<F16>(lo, pb, acc[2 * w]);
-                            acc[2 * w + 1] = mfma_k16<F16>(hi, pb, acc[2 * w + 1]);
+                            const u32x2 lo = {__builtin_amdgcn_perm(tl.v[1][h][w], tl.v[0][h][w], 0x05040100), __builtin_amdgcn_perm(tl.v[3][h][w], tl.v[2][h][w], 0x05040100)};
+                            const u32x2 hi = {__builtin_amdgcn_perm(tl.v[1][h][w], tl.v[0][h][w], 0x07060302), __builtin_amdgcn_perm(tl.v[3][h][w], tl.v[2][h][w], 0x07060302)};
+                            acc[8 * h + 2 * w] = mfma_k16<F16>(lo, pb, acc[8 * h + 2 * w]);
+                            acc[8 * h + 2 * w + 1] = mfma_k16<F16>(hi, pb, acc[8 * h + 2 * w + 1]);
                         }
                     } else {
 #pragma unroll
                         for (int w = 0; w < 2; ++w) {
                             // bytes (a0 b0 a1 b1) and (a2 b2 a3 b3): two rows' codes of one dim side by side
-                            const uint32_t lo01 = __builtin_amdgcn_perm(tl.v[1][w], tl.v[0][w], 0x05010400), hi01 = __builtin_amdgcn_perm(tl.v[1][w], tl.v[0][w], 0x07030602);
-                            const uint32_t lo23 = __builtin_amdgcn_perm(tl.v[3][w], tl.v[2][w], 0x05010400), hi23 = __builtin_amdgcn_perm(tl.v[3][w], tl.v[2][w], 0x07030602);
+                            const uint32_t lo01 = __builtin_amdgcn_perm(tl.v[1][h][w], tl.v[0][h][w], 0x05010400), hi01 = __builtin_amdgcn_perm(tl.v[1][h][w], tl.v[0][h][w], 0x07030602);
+                            const uint32_t lo23 = __builtin_amdgcn_perm(tl.v[3][h][w], tl.v[2][h][w], 0x05010400), hi23 = __builtin_amdgcn_perm(tl.v[3][h][w], tl.v[2][h][w], 0x07030602);
                             // (dims 4 w + 0, 1 from the low halves, 2, 3 from the high ones; .x: rows 0, 1; .y: rows 2, 3)
                             const u32x2 a01 = codes4_to_pairs<KIND>(lo01), a23 = codes4_to_pairs<KIND>(lo23);
                             const u32x2 b01 = codes4_to_pairs<KIND>(hi01), b23 = codes4_to_pairs<KIND>(hi23);
                             const u32x2 va[4] = {u32x2{a01.x, a23.x}, u32x2{a01.y, a23.y}, u32x2{b01.x, b23.x}, u32x2{b01.y, b23.y}};
 #pragma unroll
-                            for (int j = 0; j < 4; ++j) acc[4 * w + j] = mfma_k16<F16>(va[j], pb, acc[4 * w + j]);
+                            for (int j = 0; j < 4; ++j) acc[8 * h + 4 * w + j] = mfma_k16<F16>(va[j], pb, acc[8 * h + 4 * w + j]);
                         }
+                    }
                     }
                     refill_v();
                 };
@@ -611,9 +622,12 @@ __global__ __launch_bounds__(256, kMfmaWaves) void attend_mfma_kernel(AttendArgs
                 const float l_col = sum_across_quarters(l);
                 if (part != part_lo) lds_barrier();      // the previous partition's fold has read the LDS
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    *reinterpret_cast<f32x4*>(&s_acc[wave][c16][32 * u4 + 8 * i]) = f32x4{acc[0][i], acc[1][i], acc[2][i], acc[3][i]};
-                    *reinterpret_cast<f32x4*>(&s_acc[wave][c16][32 * u4 + 8 * i + 4]) = f32x4{acc[4][i], acc[5][i], acc[6][i], acc[7][i]};
+                for (int h = 0; h < DH; ++h) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        *reinterpret_cast<f32x4*>(&s_acc[wave][c16][128 * h + 32 * u4 + 8 * i]) = f32x4{acc[8 * h][i], acc[8 * h + 1][i], acc[8 * h + 2][i], acc[8 * h + 3][i]};
+                        *reinterpret_cast<f32x4*>(&s_acc[wave][c16][128 * h + 32 * u4 + 8 * i + 4]) = f32x4{acc[8 * h + 4][i], acc[8 * h + 5][i], acc[8 * h + 6][i], acc[8 * h + 7][i]};
+                    }
                 }
                 if (u4 == 0) s_m[wave][c16] = m, s_l[wave][c16] = l_col;
                 lds_barrier();
