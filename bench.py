@@ -713,6 +713,20 @@ def reference_shapes(pk, device):
                     "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
             del caches
             torch.cuda.empty_cache()
+    # prefill(): one chunk of 16 / 256 / 2,048 tokens after 1,024 positions, bf16 24 / 2 x 256 (the reference's prefill rows)
+    hq, hkv, d, page = 24, 2, 256, 16
+    pages = (1024 + 2048) // page + 16
+    k = torch.randn(pages + 1, page, hkv, d, device=device, dtype=torch.bfloat16, generator=g)
+    v = torch.randn(pages + 1, page, hkv, d, device=device, dtype=torch.bfloat16, generator=g)
+    table = torch.randperm(pages, device=device, generator=g).to(torch.int32)
+    for T in (16, 256, 2048):
+        q = torch.randn(T, hq, d, device=device, generator=g).to(torch.bfloat16)
+        out = torch.empty_like(q)
+        position = torch.tensor([1024], dtype=torch.int64, device=device)
+        ms = graph_timed(lambda: pk.prefill(q, k, v, "bf16", table, position, page, out=out), 8)
+        flops = 4 * hq * d * sum(1024 + t + 1 for t in range(T))
+        found[f"prefill_{T}_tokens_after_1024_bf16_24q_2kv_x256"] = {
+            "us": round(ms * 1e3, 1), "TFLOP/s": round(flops / ms / 1e9, 1), "frac_of_bf16_mfma_peak": round(flops / ms / 1e9 / 2500.0, 4)}
     # write(): tokens into 8,192 shuffled slots, bf16 24 / 2 x 256 (the reference's append row)
     hkv, d = 2, 256
     k = torch.zeros(8192, hkv, d, dtype=torch.bfloat16, device=device)
