@@ -21,10 +21,11 @@ namespace pkv {
 // IQK: INT8 pages with the first product in integers (the reference's int8_qk): each query row becomes INT8 codes at its
 // own scale, the keys' codes go to LDS as they are, and S^T = K Q^T is v_mfma_i32_32x32x32_i8 (32 dims a step).
 template <int KIND, bool F16, int D, int WAVES, bool RESUME = false, bool IQK = false>
-__global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillArgs a) {
+__global__ __launch_bounds__(64 * WAVES, D == 256 ? 1 : 8 / WAVES) void prefill_kernel(PrefillArgs a) {
     static_assert(!RESUME || KIND == 0, "fresh rows are 16-bit");
     static_assert(!IQK || KIND == 3, "integer scores: INT8 pages");
     constexpr int KSTR8 = D + 16;       // IQK: K row stride in LDS (bytes)
+    static_assert(D == 64 || D == 128 || D == 256, "head widths 64, 128, 256");
     static_assert(WAVES == 4 || (WAVES == 8 && D == 128), "eight wavefronts: 128-wide heads only");
     constexpr int NT = 64 * WAVES;      // threads of the workgroup
     constexpr int BMW = 32 * WAVES;     // query rows it holds
@@ -39,6 +40,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
     constexpr int DPT = WAVES == 8 ? 4 : 8;
     constexpr int VC = D / DPT;         // pieces of one V row
     constexpr int VGROUPS = 16 * VC;    // (group of four keys, piece) pairs of a V block: the workgroup's threads, or half of them (D = 64)
+    constexpr int VPASS = (VGROUPS + NT - 1) / NT;      // ... or twice them (D = 256): a thread then takes two pairs, NT apart
     // K blocks alternate between two buffers. V blocks too with four wavefronts; with eight, half of the wavefronts
     // multiply by a block's values one iteration after the other half (below), so V blocks go round three buffers.
     constexpr int VBUFS = WAVES == 8 ? 3 : 2;
@@ -169,7 +171,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
     // stores them transposed as eight 8-byte groups (8-bit codes become 16-bit values on the way, exactly).
     // The page table entries of a block are fetched one block before its rows (load_entries, then take_slots, then load_k and load_v): a
     // row's address depends on its entry, and a wait on an entry would also wait on every row load issued before it.
-    u32x4 kreg[KPASS], vreg[4];      // vreg[i]: key 4 kg + i; 8-bit pages fill .x and .y only
+    u32x4 kreg[KPASS], vreg[VPASS][4];      // vreg[vp][i]: key 4 kg + i of pass vp; 8-bit pages fill .x and .y only
     int ent = 0, inp = 0;
     float ksreg = 1.0f, vsreg = 1.0f;
     constexpr bool direct = RESUME;      // fresh rows: the chunk's tokens in order, no table (the launcher sets page = 1)
@@ -186,7 +188,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
     // take_slots turns the entries into slots and hands every thread the slots of its rows; it runs during the second
     // product of the iteration before the loads that use them, so the exchange's latency passes behind the products
     // and load_k / load_v issue their row loads back to back.
-    constexpr int NROW = KPASS + 4;
+    constexpr int NROW = KPASS + 4 * VPASS;
     uint32_t rowslot[NROW], myslot = 0;
     auto take_slots = [&]() __attribute__((always_inline)) {
         myslot = (uint32_t)ent * (uint32_t)a.page + (uint32_t)inp;
@@ -194,10 +196,10 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
             constexpr int p = decltype(pc)::value;
             rowslot[p] = (uint32_t)__builtin_amdgcn_ds_bpermute(((p * NT + tid) / CH) << 2, (int)myslot);
         });
-        const int kg = tid % VGROUPS / VC;      // D = 64: the upper half of the workgroup repeats the lower
-        static_for<4>([&](auto ic) __attribute__((always_inline)) {
-            constexpr int i = decltype(ic)::value;
-            rowslot[KPASS + i] = (uint32_t)__builtin_amdgcn_ds_bpermute((4 * kg + i) << 2, (int)myslot);
+        static_for<4 * VPASS>([&](auto ic) __attribute__((always_inline)) {
+            constexpr int vp = decltype(ic)::value / 4, i = decltype(ic)::value % 4;
+            const int kg = (vp * NT + tid) % VGROUPS / VC;      // D = 64: the upper half of the workgroup repeats the lower
+            rowslot[KPASS + 4 * vp + i] = (uint32_t)__builtin_amdgcn_ds_bpermute((4 * kg + i) << 2, (int)myslot);
         });
     };
     auto load_k = [&]() __attribute__((always_inline)) {
@@ -209,17 +211,17 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
         if constexpr (KIND >= 2) ksreg = a.ks[(uint64_t)myslot * a.hkv + kvh];
     };
     auto load_v = [&]() __attribute__((always_inline)) {
-        const uint8_t* vthread = vbase + (tid % VGROUPS % VC) * (DPT * EB);
-        static_for<4>([&](auto ic) __attribute__((always_inline)) {
-            constexpr int i = decltype(ic)::value;
-            const uint8_t* row = vthread + (uint64_t)rowslot[KPASS + i] * v_slot_bytes;
+        static_for<4 * VPASS>([&](auto ic) __attribute__((always_inline)) {
+            constexpr int vp = decltype(ic)::value / 4, i = decltype(ic)::value % 4;
+            const uint8_t* vthread = vbase + ((vp * NT + tid) % VGROUPS % VC) * (DPT * EB);
+            const uint8_t* row = vthread + (uint64_t)rowslot[KPASS + 4 * vp + i] * v_slot_bytes;
             if constexpr (DPT * EB == 16) {
-                vreg[i] = *reinterpret_cast<const u32x4*>(row);
+                vreg[vp][i] = *reinterpret_cast<const u32x4*>(row);
             } else if constexpr (DPT * EB == 8) {
                 const u32x2 w = *reinterpret_cast<const u32x2*>(row);
-                vreg[i].x = w.x, vreg[i].y = w.y;
+                vreg[vp][i].x = w.x, vreg[vp][i].y = w.y;
             } else {
-                vreg[i].x = *reinterpret_cast<const uint32_t*>(row);
+                vreg[vp][i].x = *reinterpret_cast<const uint32_t*>(row);
             }
         });
         if constexpr (KIND >= 2) vsreg = a.vs[(uint64_t)myslot * a.hkv + kvh];
@@ -250,13 +252,15 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
         // transposed: dim row 8 c + i gets the four keys' values as one 8-byte group at the place v_place gives, byte
         // offset v_place(kg, 8 c) ^ (16 i), plus 128 i. A thread with four dims holds i = 4 up + 0 .. 3 of them: 64 up
         // goes into the XOR and 512 up into the sum (bits 7 to 9 of the first term are clear, so the sum carries nothing).
-        const int idx = tid % VGROUPS;      // repeated pairs store the same bytes twice
-        const int kg = idx / VC, piece = idx % VC;
-        const int c = piece / (8 / DPT), up = piece % (8 / DPT);
         uint8_t* vb = reinterpret_cast<uint8_t*>(v_lds[buf]);
         if constexpr (KIND >= 2) {
             if (tid < BN) vs_lds[buf][tid] = vsreg;
         }
+        static_for<VPASS>([&](auto vpc) __attribute__((always_inline)) {
+        constexpr int vp = decltype(vpc)::value;
+        const int idx = (vp * NT + tid) % VGROUPS;      // repeated pairs store the same bytes twice
+        const int kg = idx / VC, piece = idx % VC;
+        const int c = piece / (8 / DPT), up = piece % (8 / DPT);
         const uint32_t v_write = ((uint32_t)v_place(kg, 8 * c) ^ (64u * (uint32_t)up)) + 512u * (uint32_t)up;
         static_for<DPT / 2>([&](auto jc) __attribute__((always_inline)) {
             constexpr int j = decltype(jc)::value;      // dims 2 j and 2 j + 1 of the thread's eight
@@ -264,9 +268,9 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 if constexpr (KIND == 0) {
-                    w[k] = vreg[k][j];
+                    w[k] = vreg[vp][k][j];
                 } else {
-                    w[k] = code_pair<KIND, j % 2 == 1>(vreg[k][j / 2]);
+                    w[k] = code_pair<KIND, j % 2 == 1>(vreg[vp][k][j / 2]);
                 }
             }
 #pragma unroll
@@ -277,6 +281,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
                 *reinterpret_cast<u32x2*>(vb + (v_write ^ (16u * i)) + 128 * i) = u32x2{k01, k23};
             }
             if constexpr (KIND != 0) PKV_SB();      // (as in store_k)
+        });
         });
     };
     // Operand reads, two operands a step. K, step i: k-step i of both 32-key halves. V, step i: keys
@@ -408,7 +413,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
         }
         // one product, then a share of the staging work (LDS reads of later operands, the stores' permutes and
         // writes, the row loads) in its shadow
-        if constexpr (KIND == 0) {      // (8-bit pages: the conversions' temporaries make this order spill)
+        if constexpr (KIND == 0 && D != 256) {      // (8-bit pages: the conversions' temporaries make this order spill)
             __builtin_amdgcn_sched_group_barrier(0x100, 2 * (RING - 1), 0);
             static_for<2 * KS>([&](auto) __attribute__((always_inline)) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -518,7 +523,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void prefill_kernel(PrefillA
             o[nb + 1] = mfma<F16>(va[i % RING][1], pop[g], o[nb + 1]);
             // steps 0 .. 5 take the pairs of pop[1], pop[2], pop[3] in order, each a step (D = 128) or more (D = 64:
             // two at a time) before the step that multiplies by them
-            if constexpr (NB == 4) {
+            if constexpr (NB >= 4) {
                 if constexpr (i < 6) pairs(vbuf, std::integral_constant<int, 1 + i / 2>{}, std::integral_constant<int, i % 2>{});
             } else {
                 if constexpr (i == 0) pairs(vbuf, c1, c0), pairs(vbuf, c1, c1);
@@ -663,6 +668,10 @@ template <int KIND, bool F16, bool RESUME = false, bool IQK = false>
 static int launch_d(const PrefillArgs& a, int d, bool wide, dim3 grid, hipStream_t stream) {
     switch (d) {
         case 64: hipLaunchKernelGGL((prefill_kernel<KIND, F16, 64, 4, RESUME, IQK>), grid, dim3(256), 0, stream, a); break;
+        case 256:      // (one workgroup a compute unit: 133 KB of LDS, about 300 registers; integer scores at 64 and 128 only)
+            if constexpr (IQK) return CRIT_PKV_E_GEOMETRY;
+            else hipLaunchKernelGGL((prefill_kernel<KIND, F16, 256, 4, RESUME, false>), grid, dim3(256), 0, stream, a);
+            break;
         case 128:
             if constexpr (!RESUME) {
                 if (wide) {
@@ -717,7 +726,8 @@ int launch_prefill(const crit_pkv_prefill_params* p, hipStream_t stream) {
     if (p->chunks < 1 || p->chunks > 65535 || p->max_count < 1 || p->max_count > (1 << 30) || p->kv_heads < 1 || p->kv_heads > 65535 || p->heads < 1 ||
         p->heads % p->kv_heads || p->page < 1 || p->table_width < 1 || p->sliding < 0)
         return CRIT_PKV_E_GEOMETRY;
-    if (p->head_dim != 64 && p->head_dim != 128) return CRIT_PKV_E_GEOMETRY;
+    if (p->head_dim != 64 && p->head_dim != 128 && p->head_dim != 256) return CRIT_PKV_E_GEOMETRY;
+    if (p->head_dim == 256 && p->int8_qk) return CRIT_PKV_E_GEOMETRY;
     const int out_align = p->out_dtype == CRIT_PKV_F32 ? 4 : 4;      // 4 elements per store either way
     if (p->q_stride_t % 8 || p->q_stride_h % 8 || p->out_stride_t % out_align || p->out_stride_h % out_align ||
         (reinterpret_cast<uintptr_t>(p->q) % 16) || (reinterpret_cast<uintptr_t>(p->out) % 16) ||

@@ -764,7 +764,7 @@ def _prefill_launch(q, key_pages, value_pages, kind, tables, table_rows, starts,
     if q.dtype != want_q:
         raise ValueError(f"q is {want_q} over {kind} pages, not {q.dtype}")
     device = q.device
-    if d not in (64, 128):
+    if d not in (64, 128, 256) or (d == 256 and k_kind == 3):      # (INT8 pages at 256 would spill: window rows)
         return _prefill_as_windows(q, key_pages, value_pages, kind, tables, table_rows, starts, counts, positions,
                                    max_count, chunks, page, key_scales, value_scales, multipliers, scale, out, lse,
                                    sinks, sliding, fresh, int8_qk)
@@ -806,7 +806,7 @@ def _prefill_launch(q, key_pages, value_pages, kind, tables, table_rows, starts,
 def _prefill_as_windows(q, key_pages, value_pages, kind, tables, table_rows, starts, counts, positions, max_count,
                         chunks, page, key_scales, value_scales, multipliers, scale, out, lse, sinks, sliding, fresh,
                         int8_qk, derive=None):
-    """Prompt chunks at the head widths the matrix-core kernel does not take (16, 32, 256), and those whose keys are
+    """Prompt chunks at the head widths the matrix-core kernel does not take (16, 32; 256 over INT8 pages), and those whose keys are
     derived from the value rows: every chunk cut into window
     rows of up to MAX_COLUMNS tokens and read by attend()'s fused launch, as crit itself reads prompt rows with
     prompt_reader decode (device_attention.py:751-783). The rows' metadata is computed on the device from the chunks'

@@ -20,8 +20,9 @@ def _check(cache, q, out, lse, position, tokens, sliding=0):
 
 
 @pytest.mark.parametrize("kind", KINDS)
-@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 128), (32, 8, 128), (40, 8, 128), (12, 2, 64)])
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 128), (32, 8, 128), (40, 8, 128), (12, 2, 64), (24, 2, 256), (24, 4, 256)])
 def test_prompt_chunks_match_float64_attention(kind, hq, hkv, d):
+    # (256-wide heads: the matrix-core kernel with one workgroup a compute unit; INT8 pages there go through window rows)
     pk = kernels()
     cache = Cache(kind, hkv, d, d, 16, [300])
     q = rand_q(100, hq, d, 4)
@@ -34,9 +35,10 @@ def test_prompt_chunks_match_float64_attention(kind, hq, hkv, d):
 
 @pytest.mark.parametrize("kind", ["bf16", "fp8:row"])
 @pytest.mark.parametrize("hq,hkv,d", [(24, 4, 256), (4, 2, 32), (6, 1, 16)])
-def test_prompt_chunks_at_the_other_head_widths_go_through_window_rows(kind, hq, hkv, d):
-    # Head widths the matrix-core kernel does not take: the chunk is read as window rows of up to 64 columns by the
-    # decode reader's fused launch (what crit does with prompt_reader decode); the same contract, fresh rows included.
+def test_prompt_chunks_at_the_other_head_widths(kind, hq, hkv, d):
+    # 256-wide heads on the matrix-core kernel; 16 and 32, which it does not take, as window rows of up to 64 columns
+    # read by the decode reader's fused launch (what crit does with prompt_reader decode); the same contract, fresh
+    # rows included.
     pk = kernels()
     cache = Cache(kind, hkv, d, d, 16, [300])
     q = rand_q(150, hq, d, 4)
@@ -389,7 +391,7 @@ def test_int8_queries_in_a_launch_that_fills_the_chip_equal_one_launch_per_chunk
 @pytest.mark.parametrize("hq,hkv,d", [(8, 2, 128), (12, 2, 64), (8, 2, 256)])
 def test_a_nan_query_in_a_prompt_chunk_reaches_its_own_tokens_output_only(hq, hkv, d):
     # a fault upstream shows instead of turning into zeros, and in its own row only (the reference's test_nonfinite.py),
-    # on the matrix-core path (128, 64) and through window rows (256)
+    # at every head width of the matrix-core path
     pk = kernels()
     cache = Cache("bf16", hkv, d, d, 16, [300])
     q = rand_q(4, hq, d, 2).bfloat16()
