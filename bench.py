@@ -554,9 +554,10 @@ def pool_bookkeeping(pk, device):
 def latent_decode(device):
     """Latent-attention (MLA) decode at DeepSeek's geometry (rank 512, rotary 64, page 64): 64 rows of one token at
     contexts ~U[1024, 8192], for the 16 heads a GPU of eight holds and for all 128, BF16 and E4M3 (one scale a row: a
-    KV pool's fp8:row pages) caches. Bytes: the cache rows read once (the algorithmic figure; at 128 heads the 8 tiles
-    of a row read them again from L2); flops: 2 (2 R + P) a position and head. The split launch alone (phases=1) and
-    with its merge, replayed from a captured graph."""
+    KV pool's fp8:row pages) caches. Bytes: the cache rows read once (the algorithmic figure); flops: 2 (2 R + P) a
+    position and head. The split launch alone (phases=1) and with its merge, replayed from a captured graph. At 128
+    heads of a BF16 cache the many-heads kernel reads (tile_rows 128); the row `bf16_128_heads_by_tile_rows` sets it
+    against the small tiles at 64, 8 and 1 batch rows, which is the trade its default makes."""
     import crit_amd.latent_attention as la
     R, P, page, B = 512, 64, 64, 64
     lengths = torch.randint(1024, 8193, (B,), generator=torch.Generator().manual_seed(7)).tolist()
@@ -593,12 +594,25 @@ def latent_decode(device):
             split = graph_timed(lambda: call(1), 3) / layers
             both = graph_timed(call, 3) / layers
             nbytes, flops = total * (R + P) * e, total * heads * 2 * (2 * R + P)
+            tiles = la.tile_rows(heads, R, P, page, int(kind != "bf16"))
             found[f"{kind}_{heads}_heads"] = {
-                "partitions": la.partitions(device, heads, R, P, page), "split_us": round(split * 1e3, 1),
+                "tile_rows": tiles, "piece": la.PIECE_MANY_HEADS if tiles == 128 else la.PIECE,
+                "partitions": la.partitions(device, heads, R, P, page, int(kind != "bf16")), "split_us": round(split * 1e3, 1),
                 "with_merge_us": round(both * 1e3, 1), "split_GB/s": round(nbytes / split / 1e6, 1),
                 "split_frac_of_hbm_peak": round(nbytes / split / 1e6 / HBM_PEAK_GBPS, 4),
                 "split_TFLOP/s": round(flops / split / 1e9, 1),
                 "split_frac_of_bf16_mfma_peak": round(flops / split / 1e9 / 2500.0, 4)}
+            if kind == "bf16" and heads == 128:
+                trade = {}
+                for n in (64, 8, 1):
+                    for tiles in (128, 16):
+                        def some(phases=0):
+                            for cache in caches:
+                                la.attend(q[:n], cache, tables, rows[:n], rows[:n], firsts[:n], 1, page, rank=R, out=out[:n],
+                                          phases=phases, tile_rows=tiles)
+                        some()
+                        trade[f"{n}_rows_tile_rows_{tiles}_us"] = round(graph_timed(some, 3) / layers * 1e3, 1)
+                found["bf16_128_heads_by_tile_rows"] = trade
         del caches, scales
     return found
 

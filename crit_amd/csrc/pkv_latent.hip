@@ -51,6 +51,7 @@ struct LatentArgs {
     int tab_width, n_rows, columns, heads, page, parts, gy, piece, tiles, max_keys, scales_per_row, out_dtype;
     Div32 page_div;
     float sscale;
+    int tile_rows;      // the caller's choice: 0 (the geometry decides), 16, 128
 };
 
 // 4 consecutive positions (rows of the LDS tile) of one value, transposed on the way out of LDS: lane 4 j + c of a
@@ -339,6 +340,485 @@ __global__ __launch_bounds__(256, NT == 1 ? 3 : 2) void latent_kernel(LatentArgs
     if (sub == 0 && g == 0) a.pm[index] = m, a.pl[index] = l;
 }
 
+// -- many heads: 128 query rows a workgroup -----------------------------------------------------------------------------
+// With 128 heads a launch spends 2 (2 R + P) flops a query row and position on (R + P) e bytes: it is bound by the matrix
+// pipe and by what LDS can feed it as much as by HBM. The kernel above reads a step's cache rows from LDS once for every
+// 16 query rows, and every workgroup of a (row, partition) stages them again. This one holds 128 query rows in a
+// workgroup of four wavefronts, one a SIMD with 512 registers each, on v_mfma_f32_32x32x16:
+//   scores  S^T = K Q^T      wavefront w takes rows 32 w .. 32 w + 31: A = cache rows (a lane: position n32, 8 values
+//                            of half h of the k-step), B = its queries, all (R + P) / 16 k-steps in 144 registers. Two
+//                            chains of 18 products: a product every 32 clocks cannot wait for the one before it.
+//   softmax                  the wavefront's own 32 rows; the probabilities (16-bit, [row][position]) and each row's
+//                            factor on its accumulators go to LDS for the others.
+//   values  O^T += V^T P^T   wavefront w takes values 128 w .. 128 w + 127 of ALL 128 rows (256 accumulators): A = V^T
+//                            by two ds_read_b64_tr_b16 an operand (4 positions of one value each), read once for four
+//                            products; B = the four row blocks' probabilities from LDS. Splitting the values rather
+//                            than the rows quarters the transposing reads, the slowest the LDS serves.
+// The cache rows reach LDS without passing through registers (global_load_lds_dwordx4: there are none to spare) into a
+// ring of four tiles of 32 positions, three in flight while one is multiplied; a wavefront sends nine loads a tile,
+// spread between the products, because each holds the wavefront until the memory pipe has taken it. Two barriers a
+// step: the tile has landed; the probabilities are written.
+//
+// A tile in LDS: the latents as [32 positions][R values] (rows of 2 R bytes, no padding) and behind them the rotary keys
+// as [32][P]. The DMA writes lane i's 16 bytes at byte 16 i of what an instruction fills, but a lane may fetch any 16
+// bytes, so the 16-byte chunks of a row are stored permuted: chunk c of position n at place c ^ (4 (n & 3) + ((n >> 2)
+// & 3)) of the latent row (c ^ ((n >> 1) & 7) of the rotary row). The score product's operand read (16 lanes: 16
+// positions, one chunk each) and the transposing read of the values (a half-wave: 4 positions x 64 bytes) then both
+// fall on all 64 banks once (the bank-conflict counter reads zero).
+//
+// The softmax keeps a row's reference maximum until the running maximum exceeds it by more than kLazyHeads (base 2), so
+// the 256 accumulators are rescaled on few steps; the decision is the row's own, from its own scores in step order.
+// A row's bits depend on its query, its positions, `piece` and `partitions` only, as above (they differ from the
+// kernel above: which of the two serves a launch follows from tile_rows, the heads, the shape and the page alone, never
+// from the batch). The partials are stored as the registers hold them (whole kilobytes a store) and merged by a kernel
+// of their own, below.
+//
+// Measured on MI355X, 64 rows of one token at contexts ~U[1024, 8192], 128 heads, BF16: 142 us (the kernel above: 259
+// us); a step of 32 positions takes about 4,600 clocks against 2,176 of matrix instructions (scores 1,800, softmax and
+// the probabilities' way through LDS 750, values 1,900, barriers 300), and a unit's start (ranking the rows, the table,
+// the queries: 36 gathers of 32 rows x 32 bytes a wavefront) and end (256 KB of partials) another 38,000. With one
+// workgroup a compute unit nothing hides either, so launches of a few rows are slower than with the small tiles (1 row:
+// 80 us against 40): tile_rows = 16 asks for those.
+constexpr float kLazyHeads = 8.0f;
+constexpr int kHeadsRows = 128;      // query rows a workgroup of the many-heads kernel holds
+
+template <bool F16>
+PKV_DEV f32x16 mfma_32(u32x4 a, u32x4 b, f32x16 c) {
+    if constexpr (F16) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+}
+// (The loads are spelled in assembly so that the compiler neither counts them nor waits for them: the waits are the
+// kernel's own, and those and the barrier are "memory" clobbers, which keeps a tile's LDS reads behind them.)
+// 64 lanes x 16 bytes from base + offset (a lane's own) to LDS bytes lds .. lds + 1023.
+PKV_DEV void dma_row(uint32_t offset, const uint8_t* base, unsigned lds) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(offset), "s"(base), "s"(lds));
+}
+PKV_DEV void dma_any(const uint8_t* from, unsigned lds) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(from), "s"(lds));
+}
+template <int N>
+PKV_DEV void wait_loads() {
+    static_assert(N >= 0 && N < 64, "vmcnt is six bits");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+// The score products and their operand reads are spelled out too, with the accumulators in ordinary registers (the
+// compiler would put them where the value accumulators are and move 16 of those out and back every step) and the waits
+// counted by hand: `ahead` reads are in flight behind the one a product needs.
+template <bool F16>
+PKV_DEV void score_product(f32x16& c, const u32x4& a, const u32x4& b) {
+    if constexpr (F16) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+    else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+}
+template <int OFFSET>
+PKV_DEV void lds_read16(u32x4& to, uint32_t at) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(to) : "v"(at), "n"(OFFSET));
+}
+template <int AHEAD>
+PKV_DEV void lds_arrived(u32x4& x) {      // (the operand is named so that its use cannot move above the wait)
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(AHEAD));
+}
+
+template <int R, int P, bool F16>
+__global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
+    static_assert(R == 512 && P == 64, "rows of 1,024 + 128 bytes");
+    constexpr int W = R + P, KS = W / 16, KSL = R / 16, NB = R / 32;      // k-steps of the scores (the first KSL the latent's); value blocks
+    constexpr int MAIN = 32 * R * 2, TILE = MAIN + 32 * P * 2, NSTAGE = 4;
+    constexpr int LPT = 9;      // loads a wavefront issues a tile: its 8 latent rows, and the rotary keys of the same rows
+    __shared__ __align__(1024) uint8_t ring[NSTAGE * TILE];
+    __shared__ __align__(16) uint8_t s_prob[kHeadsRows * 64];      // the step's probabilities, 16-bit [row][position]
+    __shared__ float s_alpha[kHeadsRows];                           // the step's factor on each row's accumulators
+
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, n32 = lane & 31, h = lane >> 5;
+    // Workgroups go to the XCDs in turn (workgroup i to XCD i mod 8), and all units of one batch row go to one XCD: they
+    // read the same queries, which its L2 then fetches once. Within an XCD the order is row, partition, tile group.
+    // Workgroups start in grid order and a compute unit holds one: a launch ends when the last one does, so the longest
+    // rows go first (ranked here, lane i holding row i: launches of up to 64 rows; larger ones keep the caller's order).
+    const int64_t place = blockIdx.x >> 3;
+    const int group = (int)(place % a.tiles);
+    const int64_t pair = place / a.tiles;
+    const int b = (int)(pair % a.gy);
+    int r = (int)(pair / a.gy) * 8 + (int)(blockIdx.x & 7);
+    if (r >= a.n_rows) return;
+    if (a.n_rows <= 64 && a.n_rows > 1) {
+        // (keys are distinct: the length, then the lower index first)
+        uint64_t mine = 0;
+        if (lane < a.n_rows) {
+            const int c = a.counts ? min(a.counts[lane], a.columns) : a.columns;
+            const int64_t f = a.firsts[lane];
+            mine = ((uint64_t)((f < 0 ? 0 : (f > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : f)) + c) << 8) + (uint64_t)(64 - lane);
+        }
+        const uint32_t lo = (uint32_t)mine, hi = (uint32_t)(mine >> 32);
+        int rank = 0;
+        for (int j = 0; j < a.n_rows; ++j) {
+            const uint64_t other = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)hi, j) << 32) | (uint32_t)__builtin_amdgcn_readlane((int)lo, j);
+            rank += other > mine ? 1 : 0;
+        }
+        r = __builtin_ctzll(__ballot(lane < a.n_rows && rank == r));
+    }
+    int count = a.columns;
+    if (a.counts) count = min(a.counts[r], a.columns);
+    const int H = a.heads;
+    const int live_rows = count * H;
+    if (group * kHeadsRows >= live_rows) return;
+    const int64_t first64 = a.firsts[r];
+    const int first = (int)(first64 < 0 ? 0 : (first64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first64));
+    const int c_hi = (min((group + 1) * kHeadsRows, live_rows) - 1) / H + 1;      // columns the group's rows reach
+    const int n_keys = min(first + c_hi, a.max_keys);
+    const int n_pieces = (n_keys + a.piece - 1) / a.piece;
+    if (b >= n_pieces) return;
+    const int64_t trow = (int64_t)a.rows[(int64_t)r * a.rows_step] * a.tab_stride;
+    const int start = a.starts[r];
+
+    // The unit's tiles: tile t is step t % spp of piece b + (t / spp) parts.
+    const int spp = a.piece / 32;
+    int n_tiles;
+    {
+        const int whole = (n_pieces - 1 - b) / a.parts;      // the unit's pieces before its last
+        const int last_piece = b + whole * a.parts;
+        const int left = n_keys - last_piece * a.piece;      // positions of the last piece (>= 1)
+        n_tiles = whole * spp + min(spp, (left + 31) / 32);
+    }
+
+    // -- staging. Wavefront w fills rows 8 w .. 8 w + 7 of a tile: one load a latent row (lane i: the chunk that belongs
+    // at place i), one for the rotary keys of the eight rows (lane i: row i / 8, the chunk that belongs at place i % 8).
+    // A wavefront's eight rows are neighbours in one page (pages are multiples of 16 positions), so it needs one page
+    // table entry a tile: the lanes hold, for 64 tiles at a time, each tile's first position and the slot that
+    // position 0 would have in the page of the wavefront's rows, and a step takes its own by v_readlane: no load inside
+    // the loop waits on the table.
+    const unsigned ring_at = (unsigned)(uintptr_t)ring;
+    const int half_row = 16 * (wave >> 1);
+    // (What a lane derives from its number is derived again in every step, from a copy of the number the compiler cannot
+    // see through: kept across the loop, the few dozen addresses below would push the queries out of the registers.)
+    int ln = lane;
+    int tile_pos = 0, tile_slot = 0, held_from = 0;
+    auto hold_tiles = [&](int from) __attribute__((always_inline)) {
+        const int tt = min(from + lane, n_tiles - 1);
+        const int pc = tt / spp;
+        const int base = (b + pc * a.parts) * a.piece + (tt - pc * spp) * 32;
+        const int p0 = min(base + half_row, n_keys - 1);
+        const int page_index = (int)div32(a.page_div, (uint32_t)p0);
+        const int entry = a.tables[trow + (page_index < a.tab_width ? page_index : a.tab_width - 1)];
+        tile_pos = base, tile_slot = (entry - page_index) * a.page, held_from = from;
+    };
+    hold_tiles(0);
+    // plan: where tile t comes from and goes to (past the unit's last tile: that one again, so that every wait counts the
+    // same loads); returns its first position. send: load k of the planned tile's nine. Inside the loop the loads go out
+    // between the score products, a few products apart: issued back to back they would hold the wavefront, and its SIMD's
+    // matrix pipe with it, until the memory pipe has taken them all.
+    const uint8_t* plan_row0 = a.cache;
+    int plan_room = 0;
+    unsigned plan_to = 0;
+    auto plan = [&](int t, int stage) __attribute__((always_inline)) -> int {
+        t = t < n_tiles ? t : n_tiles - 1;
+        if (t - held_from >= 64) hold_tiles(held_from + 64);
+        const int base = __builtin_amdgcn_readlane(tile_pos, t - held_from);
+        const int page_slot = __builtin_amdgcn_readlane(tile_slot, t - held_from);
+        const int n0 = min(base + 8 * wave, n_keys - 1);
+        plan_room = n_keys - 1 - n0;      // rows after the wavefront's first that are their own (the others repeat the last position)
+        plan_row0 = a.cache + (int64_t)(page_slot + n0) * (W * 2);
+        plan_to = ring_at + (unsigned)(stage * TILE);
+        return base;
+    };
+    auto send = [&](auto kc) __attribute__((always_inline)) {
+        constexpr int k = decltype(kc)::value;
+        if constexpr (k < 8) {
+            const uint32_t place = (uint32_t)(ln ^ ((2 * wave + k / 4) & 3)) * 16u;
+            dma_row(place ^ (uint32_t)(64 * (k & 3)), plan_row0 + min(k, plan_room) * (W * 2), plan_to + (unsigned)((8 * wave + k) * (R * 2)));
+        } else {
+            const int tail_row = ln >> 3;
+            const uint32_t tail_at = (uint32_t)(R * 2 + 16 * ((ln & 7) ^ (((8 * wave + tail_row) >> 1) & 7)));
+            dma_any(plan_row0 + (uint32_t)(min(tail_row, plan_room) * (W * 2)) + tail_at, plan_to + (unsigned)(MAIN + wave * 1024));
+        }
+    };
+    auto issue = [&](int t, int stage) __attribute__((always_inline)) -> int {
+        const int base = plan(t, stage);
+        static_for<LPT>(send);
+        return base;
+    };
+
+    // The lane's query row: column n32 of its wavefront's score tile.
+    const int j0 = group * kHeadsRows + wave * 32;
+    const int jq = j0 + n32, colq = jq / H, headq = jq - colq * H;
+    const bool liveq = colq < count;
+    const int lim = liveq ? first + colq : -1;
+    const int unmasked = min(first + j0 / H + 1, n_keys);      // positions below it are seen by every live row of the wavefront
+
+    int base = issue(0, 0);
+    u32x4 bq[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        bq[ks] = u32x4{0u, 0u, 0u, 0u};
+        if (liveq) bq[ks] = *reinterpret_cast<const u32x4*>(a.q + ((int64_t)(start + colq) * a.q_st + (int64_t)headq * a.q_sh) * 2 + ks * 32 + h * 16);
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(bq[ks].x), "v"(bq[ks].y), "v"(bq[ks].z), "v"(bq[ks].w));
+    // (the queries are waited for here, with the first tile; the next two tiles go out behind them)
+    int base1 = issue(1, 1), base2 = issue(2, 2);
+
+    float m = -INFINITY, l = 0.0f;
+    f32x16 acc[4][4];      // [block of 32 values][block of 32 query rows]
+#pragma unroll
+    for (int vb = 0; vb < 4; ++vb)
+#pragma unroll
+        for (int hb = 0; hb < 4; ++hb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[vb][hb][v] = 0.0f;
+
+    for (int t = 0; t < n_tiles; ++t) {
+        const int stage = t & (NSTAGE - 1);
+        wait_loads<2 * LPT>();      // the tile's loads of this wavefront have landed: those of the next two may be in flight
+        lds_barrier();              // everybody's have, and nobody reads the tile before any more, nor the last probabilities
+        const int base3 = plan(t + 3, (t + 3) & (NSTAGE - 1));
+        const uint8_t* tile = ring + stage * TILE;
+        // Operand addresses inside a tile (see the layout above), from the opaque copy of the number of the lane.
+        asm volatile("" : "+v"(ln));
+        const int n32 = ln & 31, h = ln >> 5;
+        const int fk = 4 * (n32 & 3) + ((n32 >> 2) & 3);
+        const uint32_t k_lane = (uint32_t)(n32 * (R * 2) + 16 * ((fk ^ h) & 15));                       // ^ 32 i for k-step i of the latent
+        const uint32_t t_lane = (uint32_t)(MAIN + n32 * (P * 2) + 16 * ((h ^ (n32 >> 1)) & 7));         // ^ 32 i for k-step i of the rotary key
+        // The values: the wavefront's 128 of them. For block vb of 32 values and k-step g of 16 positions the lane's operand
+        // is positions 16 g + 8 h + 4 e + (0 .. 3), e = 0, 1: two transposing reads, lane 4 j + c of a 16-lane group pointing
+        // at position j's values 4 c .. 4 c + 3.
+        const int i16 = ln & 15, mh = (ln >> 4) & 1;
+        const uint32_t v_lane = (uint32_t)((8 * h + (i16 >> 2)) * (R * 2) + 256 * wave + 8 * (i16 & 1));
+        const uint32_t v_low = (uint32_t)(2 * mh + ((i16 & 3) >> 1));      // the chunk's low two bits, ^ ((2 h + e) & 3)
+        uint8_t* p_mine = s_prob + (wave * 32 + n32) * 64 + 8 * h;           // + 16 (q ^ p_turn): positions 8 q + 4 h .. + 3
+        const uint32_t p_turn = (uint32_t)((n32 >> 2) & 3);
+        const uint8_t* p_read = s_prob + n32 * 64;                           // + 2048 hb + 16 ((2 g + h) ^ p_turn)
+
+        // -- scores of the wavefront's 32 rows: 36 products in two chains (even and odd ones: a product every 32 clocks
+        // cannot wait for the one before it), the operand of each read RING - 1 products ahead, five of the tile's loads
+        // sent out in between
+        f32x16 s, s2;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[v] = 0.0f, s2[v] = 0.0f;
+        {
+            constexpr int RING = 6;
+            u32x4 ka[RING];
+            const uint32_t tile_at = (uint32_t)(uintptr_t)tile;
+            // k-steps in the order 0, 8, 16, 24, 1, 9, ...: four share an address register
+            uint32_t k_at = 0;
+            auto read_k = [&](auto ic) __attribute__((always_inline)) {
+                constexpr int i = decltype(ic)::value;
+                if constexpr (i < KSL) {
+                    constexpr int lo = i / 4, hi = i % 4;      // k-step lo + 8 hi
+                    if constexpr (hi == 0) k_at = tile_at + (k_lane ^ (uint32_t)(32 * lo));
+                    lds_read16<256 * hi>(ka[i % RING], k_at);
+                } else {
+                    lds_read16<0>(ka[i % RING], tile_at + (t_lane ^ (uint32_t)(32 * (i - KSL))));
+                }
+            };
+            static_for<RING - 1>([&](auto ic) __attribute__((always_inline)) { read_k(ic); });
+            asm volatile("s_nop 1" : "+v"(s), "+v"(s2));
+            static_for<KS>([&](auto ic) __attribute__((always_inline)) {
+                constexpr int i = decltype(ic)::value;
+                if constexpr (i + RING - 1 < KS) read_k(std::integral_constant<int, i + RING - 1>{});
+                if constexpr (i % 8 == 2) send(std::integral_constant<int, i / 8>{});
+                constexpr int ahead = KS - 1 - i < RING - 1 ? KS - 1 - i : RING - 1;
+                lds_arrived<ahead>(ka[i % RING]);
+                constexpr int ks = i < KSL ? i / 4 + 8 * (i % 4) : i;
+                if constexpr (i % 2 == 0) score_product<F16>(s, ka[i % RING], bq[ks]);
+                else score_product<F16>(s2, ka[i % RING], bq[ks]);
+            });
+            asm volatile("s_nop 15\n\ts_nop 15" : "+v"(s), "+v"(s2));      // (the products' results are read by vector instructions next)
+        }
+        // -- softmax of the lane's row over its 16 positions of the tile (the other half-wave holds the other 16): the
+        // lane holds positions 8 (v / 4) + 4 h + v % 4
+        const bool masked = base + 32 > unmasked;      // (the same for the whole wavefront)
+        float x[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) x[v] = (s[v] + s2[v]) * a.sscale;
+        if (masked) {
+            const int seen = min(lim, n_keys - 1) - base - 4 * h;      // position 8 (v / 4) + v % 4 of the lane's is seen up to this
+#pragma unroll
+            for (int v = 0; v < 16; ++v) x[v] = 8 * (v / 4) + v % 4 <= seen ? x[v] : -INFINITY;
+        }
+        float top = x[0];
+#pragma unroll
+        for (int v = 1; v < 16; ++v) top = __builtin_fmaxf(top, x[v]);
+        {
+            const int w = (int)f2u(top);
+            const auto both = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+            top = __builtin_fmaxf(u2f((uint32_t)both[0]), u2f((uint32_t)both[1]));
+        }
+        const float m_new = top > m + kLazyHeads ? top : m;      // (a NaN score: the comparison fails, the NaN reaches the sum)
+        const float sub = m_new == -INFINITY ? 0.0f : m_new;
+        const float alpha = exp2_fast(m - sub);
+        m = m_new;
+        float p[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) p[v] = exp2_fast(x[v] - sub);
+        const float sum = (((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]))) +
+                          (((p[8] + p[9]) + (p[10] + p[11])) + ((p[12] + p[13]) + (p[14] + p[15])));
+        l = __builtin_fmaf(l, alpha, sum);
+        // The probabilities and the row's factor go to the other wavefronts through LDS: each multiplies the values it
+        // owns by the probabilities of all 128 rows.
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            *reinterpret_cast<u32x2*>(p_mine + 16 * ((uint32_t)q ^ p_turn)) =
+                u32x2{pair16<F16>(p[4 * q], p[4 * q + 1]), pair16<F16>(p[4 * q + 2], p[4 * q + 3])};
+        if (h == 0) s_alpha[wave * 32 + n32] = alpha;
+        lds_barrier();
+        float factor[4];
+#pragma unroll
+        for (int hb = 0; hb < 4; ++hb) factor[hb] = s_alpha[hb * 32 + n32];
+        if (__ballot(factor[0] != 1.0f || factor[1] != 1.0f || factor[2] != 1.0f || factor[3] != 1.0f) != 0ull) {
+            // (x 1 is exact: the accumulators move only when some row's reference did; spelled out so that they stay
+            // where the matrix pipe keeps them, and the last product that wrote them is a whole score phase back)
+            static_for<16>([&](auto bc) __attribute__((always_inline)) {
+                constexpr int vb = decltype(bc)::value / 4, hb = decltype(bc)::value % 4;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    float e = acc[vb][hb][v], tmp;
+                    asm volatile("v_accvgpr_read_b32 %0, %1\n\tv_mul_f32 %0, %0, %2\n\tv_accvgpr_write_b32 %1, %0" : "=&v"(tmp), "+a"(e) : "v"(factor[hb]));
+                    acc[vb][hb][v] = e;
+                }
+            });
+        }
+        // -- values: operand i = (k-step g = i / 4, block vb = i % 4) of V^T against the four row blocks' probabilities
+        {
+            constexpr int RING = 4, NOPS = 8;
+            u32x4 pb[4];      // the four row blocks' probabilities of the k-step being multiplied
+            u32x2 va[RING][2];
+            auto read_p = [&](auto gc) __attribute__((always_inline)) {
+                constexpr int g = decltype(gc)::value;
+#pragma unroll
+                for (int hb = 0; hb < 4; ++hb)
+                    pb[hb] = *reinterpret_cast<const u32x4*>(p_read + 2048 * hb + 16 * ((uint32_t)(2 * g + h) ^ p_turn));
+            };
+            read_p(std::integral_constant<int, 0>{});
+            auto read_v = [&](auto ic) __attribute__((always_inline)) {
+                constexpr int i = decltype(ic)::value;
+                constexpr int g = i / 4, vb = i % 4;
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const uint32_t at = v_lane + 64u * (uint32_t)(vb ^ (i16 >> 2)) + 16u * (v_low ^ (uint32_t)((2 * h + e) & 3));
+                    va[i % RING][e] = lds_transposed(tile + at + (16 * g + 4 * e) * (R * 2));
+                }
+            };
+            static_for<RING - 1>([&](auto ic) __attribute__((always_inline)) { read_v(ic); });
+            __builtin_amdgcn_sched_group_barrier(0x100, 4 + 2 * (RING - 1), 0);
+            __builtin_amdgcn_sched_barrier(0);
+            static_for<NOPS / 2>([&](auto sc) __attribute__((always_inline)) {
+                constexpr int sec = decltype(sc)::value;
+                send(std::integral_constant<int, 5 + sec>{});
+                if constexpr (sec == 2) {      // (the first k-step's products have been issued: their operands were read at issue)
+                    read_p(std::integral_constant<int, 1>{});
+                    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                static_for<2>([&](auto jc) __attribute__((always_inline)) {
+                    constexpr int i = 2 * sec + decltype(jc)::value;
+                    constexpr int g = i / 4, vb = i % 4;
+                    if constexpr (i + RING - 1 < NOPS) read_v(std::integral_constant<int, i + RING - 1>{});
+                    const u32x4 av = {va[i % RING][0].x, va[i % RING][0].y, va[i % RING][1].x, va[i % RING][1].y};
+#pragma unroll
+                    for (int hb = 0; hb < 4; ++hb) acc[vb][hb] = mfma_32<F16>(av, pb[hb], acc[vb][hb]);
+                });
+                static_for<2>([&](auto jc) __attribute__((always_inline)) {
+                    constexpr int i = 2 * sec + decltype(jc)::value;
+                    if constexpr (i + RING - 1 < NOPS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                });
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        }
+        base = base1, base1 = base2, base2 = base3;
+    }
+    wait_loads<0>();      // (the loads past the last tile: LDS must not be written for a workgroup that has gone)
+    {
+        const int w = (int)f2u(l);
+        const auto both = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+        l = u2f((uint32_t)both[0]) + u2f((uint32_t)both[1]);
+    }
+    // The partial output as the registers hold it, a lane's four values side by side and the lanes in order (whole
+    // kilobytes a store): [unit][partition][wavefront][value block][row block][v / 4][lane][4]; the merge below reads the
+    // same way. (A tile of 128 rows is one column's: the heads are a multiple of 128.)
+    if (h == 0 && liveq) {
+        const int64_t index = ((int64_t)((int64_t)r * a.columns + colq) * H + headq) * a.parts + b;
+        a.pm[index] = m, a.pl[index] = l;
+    }
+    float* slab = a.po + ((((int64_t)r * a.tiles + group) * a.parts + b) * 4 + wave) * (int64_t)(kHeadsRows * R / 4) + lane * 4;
+#pragma unroll
+    for (int vb = 0; vb < 4; ++vb)
+#pragma unroll
+        for (int hb = 0; hb < 4; ++hb)
+#pragma unroll
+            for (int v4 = 0; v4 < 4; ++v4)
+                *reinterpret_cast<float4*>(slab + ((vb * 4 + hb) * 4 + v4) * 256) =
+                    make_float4(acc[vb][hb][4 * v4], acc[vb][hb][4 * v4 + 1], acc[vb][hb][4 * v4 + 2], acc[vb][hb][4 * v4 + 3]);
+}
+
+// The many-heads kernel's partitions merged: a workgroup of 64 threads folds, in partition order, one (value block, row
+// block) pair of one wavefront's share of a unit, reading the partials as that wavefront stored them; the sink last.
+template <int R>
+__global__ __launch_bounds__(64) void latent_heads_merge_kernel(LatentArgs a) {
+    const int lane = threadIdx.x, n32 = lane & 31, h = lane >> 5;
+    const int wave = blockIdx.x & 3, unit = blockIdx.x >> 2, vb = blockIdx.y >> 2, hb = blockIdx.y & 3;
+    const int r = unit / a.tiles, group = unit - r * a.tiles;
+    const int H = a.heads;
+    const int j = group * kHeadsRows + hb * 32 + n32, col = j / H, head = j - col * H;
+    int count = a.columns;
+    if (a.counts) count = min(a.counts[r], a.columns);
+    if (col >= count) return;
+    const int64_t first64 = a.firsts[r];
+    const int first = (int)(first64 < 0 ? 0 : (first64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first64));
+    const int n_keys = min(first + col + 1, a.max_keys);
+    const int n_pieces = (n_keys + a.piece - 1) / a.piece;
+    const int np = min(a.parts, n_pieces);
+    const int64_t index = ((int64_t)((int64_t)r * a.columns + col) * H + head) * a.parts;
+    const float* slab = a.po + ((int64_t)unit * a.parts * 4 + wave) * (int64_t)(kHeadsRows * R / 4) + (vb * 4 + hb) * 1024 + lane * 4;
+    float M = -INFINITY, L = 0.0f, acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+    constexpr int AHEAD = 4;      // partitions requested together (past the last one the last again, so every load is issued)
+    for (int b0 = 0; b0 < np; b0 += AHEAD) {
+        float pm[AHEAD], pl[AHEAD];
+        float4 po[AHEAD][4];
+#pragma unroll
+        for (int k = 0; k < AHEAD; ++k) {
+            const int b = min(b0 + k, np - 1);
+            pm[k] = a.pm[index + b], pl[k] = a.pl[index + b];
+#pragma unroll
+            for (int v4 = 0; v4 < 4; ++v4)
+                po[k][v4] = *reinterpret_cast<const float4*>(slab + (int64_t)b * 4 * (kHeadsRows * R / 4) + v4 * 256);
+        }
+#pragma unroll
+        for (int k = 0; k < AHEAD; ++k) {
+            if (b0 + k < np) {
+                const Fold f = fold(M, L, pm[k], pl[k]);
+#pragma unroll
+                for (int v4 = 0; v4 < 4; ++v4) {
+                    acc[4 * v4] = __builtin_fmaf(acc[4 * v4], f.keep, po[k][v4].x * f.take);
+                    acc[4 * v4 + 1] = __builtin_fmaf(acc[4 * v4 + 1], f.keep, po[k][v4].y * f.take);
+                    acc[4 * v4 + 2] = __builtin_fmaf(acc[4 * v4 + 2], f.keep, po[k][v4].z * f.take);
+                    acc[4 * v4 + 3] = __builtin_fmaf(acc[4 * v4 + 3], f.keep, po[k][v4].w * f.take);
+                }
+                M = f.m, L = f.l;
+            }
+        }
+    }
+    if (a.sinks) {      // one more position with no value
+        const float sink = a.sinks[head] * kLog2e;
+        const float top = __builtin_fmaxf(M, sink);
+        const float sub = top == -INFINITY ? 0.0f : top;
+        const float keep = exp2_fast(M - sub);
+        L = __builtin_fmaf(L, keep, exp2_fast(sink - sub));
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] *= keep;
+        M = top;
+    }
+    const int64_t token = (int64_t)a.starts[r] + col;
+    const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+        store_out(a.out, a.out_dtype, token * a.o_st + (int64_t)head * a.o_sh + wave * 128 + vb * 32 + 8 * (i / 4) + 4 * h + i % 4, acc[i] * inv);
+    if (a.lse && wave == 0 && vb == 0 && h == 0) a.lse[token * a.heads + head] = (L > 0.0f || L != L) ? (M + __builtin_log2f(L)) * kLn2 : -INFINITY;
+}
+
 // One workgroup of 64 threads a (batch row, column, head): the partitions' states folded in partition order, the sink
 // last; R / 64 values a thread.
 template <int R>
@@ -413,8 +893,35 @@ int launch_tiles(const LatentArgs& a, bool f16, bool fp8, hipStream_t stream) {
     return hip_code(hipGetLastError());
 }
 
+// Which launches the many-heads kernel can serve: 16-bit caches of the one shape it is built for, heads in 128s, pages
+// of a multiple of 16 positions. It serves them unless the caller asks for the small tiles. (Nothing else decides, the
+// batch least of all: a token's bits follow the kernel that reads it.)
+template <int R, int P>
+bool many_heads(const LatentArgs& a, bool fp8) {
+    return R == 512 && P == 64 && !fp8 && a.heads % kHeadsRows == 0 && a.page % 16 == 0;
+}
+
 template <int R, int P>
 int launch_shape(const LatentArgs& a, bool f16, bool fp8, int phases, hipStream_t stream) {
+    if constexpr (R == 512 && P == 64) {
+        if (a.tile_rows != 16 && many_heads<R, P>(a, fp8)) {
+            LatentArgs u = a;
+            u.tiles = a.columns * a.heads / kHeadsRows;
+            const int64_t blocks = (int64_t)((a.n_rows + 7) / 8) * 8 * a.gy * u.tiles, merges = (int64_t)a.n_rows * u.tiles * 4;
+            if (blocks > 0x7fffffff || merges > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
+            if (phases != 2) {
+                if (f16) hipLaunchKernelGGL((latent_heads_kernel<R, P, true>), dim3((unsigned)blocks), dim3(256), 0, stream, u);
+                else hipLaunchKernelGGL((latent_heads_kernel<R, P, false>), dim3((unsigned)blocks), dim3(256), 0, stream, u);
+                const int bad = hip_code(hipGetLastError());
+                if (bad) return bad;
+            }
+            if (phases != 1) {
+                hipLaunchKernelGGL((latent_heads_merge_kernel<R>), dim3((unsigned)merges, 16), dim3(64), 0, stream, u);
+                return hip_code(hipGetLastError());
+            }
+            return 0;
+        }
+    }
     if (phases != 2) {
         // (a launch whose rows fit one tile each takes the one-tile workgroups: three a compute unit)
         LatentArgs u = a;
@@ -458,6 +965,11 @@ int launch_latent(const crit_pkv_latent_params* p, hipStream_t stream) {
     a.page_div = make_div32((uint32_t)p->page);
     a.parts = p->partitions, a.piece = p->piece, a.scales_per_row = p->scales_per_row, a.out_dtype = p->out_dtype;
     a.sscale = p->scale * kLog2e;
+    a.tile_rows = p->tile_rows;
+    if (p->tile_rows != 0 && p->tile_rows != 16 && p->tile_rows != kHeadsRows) return CRIT_PKV_E_GEOMETRY;
+    if (p->tile_rows == kHeadsRows &&
+        !(p->rank == 512 && p->rope == 64 && !fp8 && p->heads % kHeadsRows == 0 && p->page % 16 == 0))
+        return CRIT_PKV_E_GEOMETRY;
     a.tiles = (p->columns * p->heads + 15) / 16;
     const int64_t table_keys = (int64_t)p->table_width * p->page;
     a.max_keys = (int)(table_keys < 0x3fffffff ? table_keys : 0x3fffffff);
@@ -467,7 +979,7 @@ int launch_latent(const crit_pkv_latent_params* p, hipStream_t stream) {
     a.pairs = (int64_t)p->n_rows * a.gy;
     const bool f16 = p->q_dtype == CRIT_PKV_F16;
 #define PKV_LATENT(RANK, ROPE) \
-    if (p->rank == RANK && p->rope == ROPE) return launch_shape<RANK, ROPE>(a, f16, fp8, p->phases, stream);
+    if (p->rank == RANK && p->rope == ROPE) return launch_shape<RANK, ROPE>(a, f16, fp8, p->phases , stream);
     PKV_LATENT(512, 64) PKV_LATENT(256, 64) PKV_LATENT(128, 64) PKV_LATENT(128, 32) PKV_LATENT(64, 64) PKV_LATENT(64, 32)
     PKV_LATENT(1024, 64) PKV_LATENT(512, 128)
 #undef PKV_LATENT

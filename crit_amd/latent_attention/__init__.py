@@ -34,11 +34,13 @@ try:        # crit's kernel build writes the engine's tuned knobs beside the mod
 except ImportError:
     _crit_tuning = None
 
-__all__ = ["MAX_COLUMNS", "PARTIAL_BYTES", "PIECE", "SHAPES", "attend", "partitions", "prefill", "write"]
+__all__ = ["MAX_COLUMNS", "PARTIAL_BYTES", "PIECE", "PIECE_MANY_HEADS", "SHAPES", "attend", "partitions", "prefill",
+           "tile_rows", "write"]
 
 MAX_COLUMNS = 64
 PARTIAL_BYTES = 512 << 20   # the most partials one launch may take; a larger batch goes in several launches of rows
 PIECE = 256                 # default positions a piece
+PIECE_MANY_HEADS = 512      # ... where the many-heads kernel reads (TILE_ROWS 128)
 MAX_PARTS = 64
 SHAPES = ((1024, 64), (512, 128), (512, 64), (256, 64), (128, 64), (128, 32), (64, 64), (64, 32))   # (R, P) the kernels are built for
 FP8 = torch.float8_e4m3fn
@@ -63,14 +65,35 @@ def _knob(name, heads, rank, rope, page, kind):
     return int(_crit_tuning.knobs("window", key, 1).get(name, 0) or 0)
 
 
-def partitions(device, heads, rank, rope, page, kind=0):
+def partitions(device, heads, rank, rope, page, kind=0, tile_rows=None):
     """How many partitions a row's pieces are dealt to for this geometry on `device`: the tuned PARTS if the engine has
     one, else one workgroup's worth of work for every second compute unit per 16 heads, between 1 and MAX_PARTS (64 for
-    16 and 32 heads, 32 for 64, 16 for 128 on 256 compute units). It depends on the heads and the device only, because a
-    token's bits depend on it. (The reference's rule is the same idea for its tiles: __init__.py:65-71.)"""
+    16 and 32 heads, 32 for 64, 16 for 128 on 256 compute units); where the many-heads kernel reads (tile_rows(...) ==
+    128), whose workgroups take a compute unit each and 128 query rows, one for every 32 compute units (8). It depends
+    on the geometry and the device only, because a token's bits depend on it. (The reference's rule is the same idea
+    for its tiles: __init__.py:65-71.)"""
     tuned = _knob("PARTS", heads, rank, rope, page, kind)
-    wanted = tuned if tuned else _cus(device) // (2 * max(1, -(-int(heads) // 16)))
-    return min(MAX_PARTS, max(1, wanted))
+    if tuned:
+        return min(MAX_PARTS, max(1, tuned))
+    if globals()["tile_rows"](heads, rank, rope, page, kind, tile_rows) == 128:
+        return min(MAX_PARTS, max(1, _cus(device) // 32))
+    return min(MAX_PARTS, max(1, _cus(device) // (2 * max(1, -(-int(heads) // 16)))))
+
+
+def tile_rows(heads, rank, rope, page, kind=0, asked=None):
+    """The query rows a workgroup holds for this geometry, 16 or 128, which names the kernel that reads it (and a token's
+    bits follow the kernel). 128, the many-heads kernel (32 x 32 matrix tiles, the cache rows by DMA into LDS, one
+    workgroup a compute unit), takes 16-bit caches of DeepSeek's shape (512, 64) with heads in 128s and pages of a
+    multiple of 16 positions, and is what such a geometry gets unless `asked` (attend's tile_rows=) or the engine's tuned
+    TILE_ROWS says 16: it reads a batch of 64 rows about twice as fast as the small tiles, and a single row three times
+    slower (one workgroup a partition instead of four). Everything else gets 16."""
+    able = (int(rank), int(rope)) == (512, 64) and not int(kind) and int(heads) % 128 == 0 and int(page) % 16 == 0
+    want = int(asked or _knob("TILE_ROWS", heads, rank, rope, page, kind) or 0)
+    if want not in (0, 16, 128):
+        raise ValueError(f"tile_rows: {want}; 16 or 128 (or 0: by the geometry)")
+    if want == 128 and not able:
+        raise ValueError("tile_rows 128 reads 16-bit caches of (512, 64) with heads in 128s and pages of a multiple of 16")
+    return 128 if able and want != 16 else 16
 
 
 def write(latent, rope, slots, cache, scales=None):
@@ -163,7 +186,7 @@ def attend(q, cache, tables, rows, starts, firsts, columns, page, *, rank, count
            out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
            sinks: Optional[torch.Tensor] = None, scales: Optional[torch.Tensor] = None,
            fused: Optional[bool] = None, piece=None, partitions=None, workspace: Optional[torch.Tensor] = None,
-           phases=0) -> torch.Tensor:
+           phases=0, tile_rows=None) -> torch.Tensor:
     """Decode tokens and verify windows (see the module text). q [tokens][heads][R + P]; tables [S][width] int32; rows
     and starts [B] int32 (rows may be int64); firsts [B] int64; counts [B] int32 or None (every row has `columns`);
     columns: the widest row, a Python int within 1..MAX_COLUMNS. Returns out [tokens][heads][R] (q's dtype unless `out`
@@ -176,7 +199,8 @@ def attend(q, cache, tables, rows, starts, firsts, columns, page, *, rank, count
     and partitions (1..MAX_PARTS) default to the tuned values or PIECE and partitions(); keep one value of each per
     geometry, since a token's bits depend on them. workspace: FP32 scratch for the partials; without it the module uses
     a buffer held per owner (paged_kv_attention.owner) and device, so launches of two owners on two streams never share
-    partials. phases is for timing: 1 runs the partitions' launch alone, 2 the merge alone."""
+    partials. phases is for timing: 1 runs the partitions' launch alone, 2 the merge alone. tile_rows: 16 or 128, the
+    kernel that reads (see tile_rows()); default: the tuned TILE_ROWS, else by the geometry."""
     call = _Call(q, cache, page, rank, sinks, scales)
     heads, R, P = call.heads, call.rank, call.rope
     batch = int(starts.shape[0])
@@ -190,10 +214,11 @@ def attend(q, cache, tables, rows, starts, firsts, columns, page, *, rank, count
         raise ValueError("rows: int32 or int64; starts and counts: int32; firsts: int64")
     device = q.device
     coded = int(call.coded)
-    piece = int(piece or _knob("PIECE", heads, R, P, page, coded) or PIECE)
+    tiles = globals()["tile_rows"](heads, R, P, page, coded, tile_rows)
+    piece = int(piece or _knob("PIECE", heads, R, P, page, coded) or (PIECE_MANY_HEADS if tiles == 128 else PIECE))
     if piece < 32 or piece % 32:
         raise ValueError(f"piece: {piece}; a multiple of 32 positions")
-    parts = int(partitions) if partitions is not None else globals()["partitions"](device, heads, R, P, page, coded)
+    parts = int(partitions) if partitions is not None else globals()["partitions"](device, heads, R, P, page, coded, tiles)
     if not 1 <= parts <= MAX_PARTS:
         raise ValueError(f"partitions: {parts}; within 1..{MAX_PARTS}")
     if out is None:
@@ -223,6 +248,7 @@ def attend(q, cache, tables, rows, starts, firsts, columns, page, *, rank, count
     p.q_dtype, p.out_dtype = _DTYPE[q.dtype], _DTYPE[out.dtype]
     p.scales_per_row = int(scales.shape[2]) if coded else 0
     p.partitions, p.piece, p.rows_are_64, p.phases = parts, piece, int(rows.dtype == torch.int64), int(phases)
+    p.tile_rows = tiles
     p.scale = float((R + P) ** -0.5 if scale is None else scale)
     base = work.data_ptr()
     for first in range(0, batch, rows_a_launch):
@@ -239,7 +265,7 @@ def attend(q, cache, tables, rows, starts, firsts, columns, page, *, rank, count
 
 def prefill(q, cache, table, position, page, *, rank, scale=None, out: Optional[torch.Tensor] = None,
             lse: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None,
-            scales: Optional[torch.Tensor] = None) -> torch.Tensor:
+            scales: Optional[torch.Tensor] = None, tile_rows=None) -> torch.Tensor:
     """A prompt chunk of one sequence, causal: q [T][heads][R + P] are the tokens at positions position .. position +
     T - 1 (their rows already written), table [pages] int32 the sequence's page table; position is an int, or a
     one-element int64 device tensor that is read on the device so that one captured graph serves every position.
@@ -265,4 +291,4 @@ def prefill(q, cache, table, position, page, *, rank, scale=None, out: Optional[
     one_table = table.reshape(1, -1) if table.dtype == torch.int32 else table.reshape(1, -1).to(torch.int32)
     return attend(q, cache, one_table, torch.zeros(windows, dtype=torch.int32, device=device), offsets.to(torch.int32),
                   origin + offsets, min(MAX_COLUMNS, count), page, rank=rank, counts=widths, scale=scale, out=out, lse=lse,
-                  sinks=sinks, scales=scales, fused=True)
+                  sinks=sinks, scales=scales, fused=True, tile_rows=tile_rows)

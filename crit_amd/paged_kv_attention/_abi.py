@@ -10,7 +10,7 @@ import shutil
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 NAME = "libcrit_pkv.so"
-ABI_VERSION = 18
+ABI_VERSION = 19
 
 KIND_16BIT, KIND_FP8, KIND_FP8_ROW, KIND_INT8 = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
@@ -112,7 +112,8 @@ class LatentParams(ctypes.Structure):
                 ("q_stride_t", _i64), ("q_stride_h", _i64), ("out_stride_t", _i64), ("out_stride_h", _i64), ("table_stride", _i64),
                 ("table_width", _i32), ("n_rows", _i32), ("columns", _i32), ("heads", _i32), ("rank", _i32), ("rope", _i32),
                 ("page", _i32), ("cache_dtype", _i32), ("q_dtype", _i32), ("out_dtype", _i32), ("scales_per_row", _i32),
-                ("partitions", _i32), ("piece", _i32), ("rows_are_64", _i32), ("phases", _i32), ("scale", _f32)]
+                ("partitions", _i32), ("piece", _i32), ("rows_are_64", _i32), ("phases", _i32), ("tile_rows", _i32),
+                ("scale", _f32)]
 
 
 class LatentWriteParams(ctypes.Structure):

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 18
+#define CRIT_PKV_ABI_VERSION 19
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -407,7 +407,13 @@ int crit_pkv_step_buffers(const crit_pkv_step_params* p, void* stream);
  * natural log-sum-exp (the sink counted). cache_dtype: 0 BF16, 1 FP16 (q in the same type), 2 E4M3 with `scales`
  * [pages][page][scales_per_row] FP32 (2: the latent's and the rotary key's, 1: one for the row) and BF16 or FP16 q.
  * (rank, rope) is one of (1024, 64), (512, 128), (512, 64), (256, 64), (128, 64), (128, 32), (64, 64), (64, 32). phases: 0 both launches, 1
- * the partitions only, 2 the merge only. */
+ * the partitions only, 2 the merge only.
+ * tile_rows: the query rows a workgroup holds, which decides the kernel and with it a token's bits. 16: tiles of 16 rows
+ * (two a workgroup from 32 rows on), every geometry, the fastest for a few batch rows. 128: 128 rows a workgroup on
+ * 32 x 32 matrix tiles, the cache rows by DMA into LDS, one workgroup a compute unit (16-bit caches of (512, 64), heads a
+ * multiple of 128, pages a multiple of 16 positions; anything else: CRIT_PKV_E_GEOMETRY), about twice the throughput of
+ * the other from a few dozen batch rows on and slower below ten. 0: 128 where the geometry allows, else 16. The
+ * partials of the two are laid out differently (same size): phases 1 and 2 of one call take the same tile_rows. */
 typedef struct crit_pkv_latent_params {
     const void* q;
     const void* cache;
@@ -425,7 +431,7 @@ typedef struct crit_pkv_latent_params {
     const float* sinks;             /* optional */
     int64_t q_stride_t, q_stride_h, out_stride_t, out_stride_h, table_stride;
     int32_t table_width, n_rows, columns, heads, rank, rope, page, cache_dtype, q_dtype, out_dtype, scales_per_row,
-        partitions, piece, rows_are_64, phases;
+        partitions, piece, rows_are_64, phases, tile_rows;
     float scale;
 } crit_pkv_latent_params;
 

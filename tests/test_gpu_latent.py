@@ -116,6 +116,44 @@ def test_a_tokens_bits_are_its_own_alone_in_a_window_and_beside_other_rows():
     assert torch.equal(as_slots, together)
 
 
+@pytest.mark.parametrize("tile_rows", [128, 16])
+def test_many_heads_either_kernel_matches_float64_and_a_tokens_bits_follow_the_kernel_alone(tile_rows):
+    # 128 heads of DeepSeek's shape: the many-heads kernel (128 query rows a workgroup; the default here) or, asked for,
+    # the small tiles. Either way a token's bits are its own: alone, in a verify window, beside other rows (the longest
+    # rows go first inside the launch), in launches of a few rows at a time; and the lengths straddle pieces, tiles of 32
+    # positions and pages.
+    cache = Cache(512, 64, 16, [1500, 33, 2100, 600], seed=31)
+    la = cache.la
+    assert la.tile_rows(128, 512, 64, 16) == 128 and la.tile_rows(128, 512, 64, 16, asked=16) == 16
+    assert la.tile_rows(64, 512, 64, 16) == 16 and la.tile_rows(128, 512, 64, 24) == 16 and la.tile_rows(128, 512, 64, 16, 1) == 16
+    q = _q(16, 128, 576, 32)
+    rows, starts, firsts = [0, 1, 2, 3], [0, 4, 8, 12], [1496, 29, 2096, 511]
+    sinks = torch.randn(128, generator=torch.Generator().manual_seed(33)).to(dev)
+    lse = torch.empty(16, 128, device=dev)
+    together = cache.attend(q, rows, starts, firsts, 4, lse=lse, sinks=sinks, tile_rows=tile_rows)
+    for s_, start, first in zip(rows, starts, firsts):
+        cache.check(q, together, lse, s_, start, first, 4, 576 ** -0.5, sinks)
+        window = cache.attend(q[start:start + 4], [s_], [0], [first], 4, sinks=sinks, tile_rows=tile_rows)
+        assert torch.equal(window, together[start:start + 4]), s_
+        for c in (0, 3):
+            alone = cache.attend(q[start + c:start + c + 1], [s_], [0], [first + c], 1, sinks=sinks, tile_rows=tile_rows)
+            assert torch.equal(alone[0], together[start + c]), (s_, c)
+    limit = la.PARTIAL_BYTES
+    try:
+        la.PARTIAL_BYTES = 4 * 128 * la.partitions(torch.device(dev), 128, 512, 64, 16, 0, tile_rows) * 514 * 4      # one row's
+        sliced = cache.attend(q, rows, starts, firsts, 4, sinks=sinks, tile_rows=tile_rows)
+    finally:
+        la.PARTIAL_BYTES = limit
+    assert torch.equal(sliced, together)
+    other = cache.attend(q, rows, starts, firsts, 4, sinks=sinks, tile_rows=144 - tile_rows)
+    torch.testing.assert_close(other.float(), together.float(), atol=8e-3, rtol=2e-2)      # the same attention, other sums
+    with pytest.raises(ValueError):
+        cache.attend(q, rows, starts, firsts, 4, tile_rows=64)
+    small = Cache(512, 64, 16, [40], seed=34)
+    with pytest.raises(ValueError):      # 16 heads: not the many-heads kernel's
+        small.attend(_q(1, 16, 576, 35), [0], [0], [39], 1, tile_rows=128)
+
+
 @pytest.mark.parametrize("heads", [16, 128])
 def test_a_nan_query_reaches_its_own_rows_output_only(heads):
     cache = Cache(512, 64, 64, [700, 300], seed=4)

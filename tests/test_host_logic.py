@@ -10,15 +10,22 @@ def test_latent_partitions_follow_the_rule_or_the_engines_tuning():
     held = dict(la._CUS)
     la._CUS[0] = 256                                   # an MI355X's compute units (no device is asked)
     try:
-        assert [la.partitions(device, h, 512, 64, 64) for h in (1, 16, 32, 64, 128)] == [64, 64, 64, 32, 16]
+        # (128 heads of a 16-bit (512, 64) cache: the many-heads kernel, a workgroup a compute unit; an E4M3 cache, pages
+        # of no multiple of 16 or the small tiles asked for: the rule of the small tiles)
+        assert [la.partitions(device, h, 512, 64, 64) for h in (1, 16, 32, 64, 128)] == [64, 64, 64, 32, 8]
+        assert la.partitions(device, 128, 512, 64, 64, 1) == 16 and la.partitions(device, 128, 512, 64, 24) == 16
+        assert la.partitions(device, 128, 512, 64, 64, 0, 16) == 16 and la.partitions(device, 128, 256, 64, 64) == 16
+        assert la.tile_rows(128, 512, 64, 64) == 128 and la.tile_rows(256, 512, 64, 16) == 128
+        assert la.tile_rows(64, 512, 64, 64) == 16 and la.tile_rows(128, 512, 64, 64, asked=16) == 16
 
         class Tuning:
             @staticmethod
             def knobs(structure, key, rows):
-                return {"PARTS": 8 if key["H"] == 128 else 0, "PIECE": 0}
+                return {"PARTS": 12 if key["H"] == 128 else 0, "PIECE": 0, "TILE_ROWS": 16 if key["PAGE"] == 32 else 0}
 
         la._crit_tuning = Tuning
-        assert la.partitions(device, 128, 512, 64, 64) == 8 and la.partitions(device, 16, 512, 64, 64) == 64
+        assert la.partitions(device, 128, 512, 64, 64) == 12 and la.partitions(device, 16, 512, 64, 64) == 64
+        assert la.tile_rows(128, 512, 64, 32) == 16 and la.tile_rows(128, 512, 64, 64) == 128
     finally:
         la._crit_tuning = None
         la._CUS.clear(), la._CUS.update(held)
