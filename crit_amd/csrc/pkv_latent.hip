@@ -381,6 +381,7 @@ __global__ __launch_bounds__(256, NT == 1 ? 3 : 2) void latent_kernel(LatentArgs
 // 80 us against 40): tile_rows = 16 asks for those.
 constexpr float kLazyHeads = 8.0f;
 constexpr int kHeadsRows = 128;      // query rows a workgroup of the many-heads kernel holds
+constexpr int kRowsToAnXcd = 16;     // launches of that many batch rows or more keep a row's units on one XCD
 
 template <bool F16>
 PKV_DEV f32x16 mfma_32(u32x4 a, u32x4 b, f32x16 c) {
@@ -432,16 +433,24 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
     __shared__ float s_alpha[kHeadsRows];                           // the step's factor on each row's accumulators
 
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, n32 = lane & 31, h = lane >> 5;
-    // Workgroups go to the XCDs in turn (workgroup i to XCD i mod 8), and all units of one batch row go to one XCD: they
-    // read the same queries, which its L2 then fetches once. Within an XCD the order is row, partition, tile group.
+    // Workgroups go to the XCDs in turn (workgroup i to XCD i mod 8), and the tile groups of one (row, partition) pair
+    // take consecutive places of one XCD, whose L2 then serves the pair's cache rows to all of them. Launches of 16 batch
+    // rows or more deal whole rows to the XCDs (a row's partitions read the same queries, which one L2 then fetches
+    // once: 142 against 165 us for 64 rows of 128 heads); smaller ones deal the pairs, or XCDs would idle.
     // Workgroups start in grid order and a compute unit holds one: a launch ends when the last one does, so the longest
     // rows go first (ranked here, lane i holding row i: launches of up to 64 rows; larger ones keep the caller's order).
     const int64_t place = blockIdx.x >> 3;
     const int group = (int)(place % a.tiles);
-    const int64_t pair = place / a.tiles;
-    const int b = (int)(pair % a.gy);
-    int r = (int)(pair / a.gy) * 8 + (int)(blockIdx.x & 7);
-    if (r >= a.n_rows) return;
+    int b, r;
+    if (a.n_rows >= kRowsToAnXcd) {
+        const int64_t pair = place / a.tiles;
+        b = (int)(pair % a.gy), r = (int)(pair / a.gy) * 8 + (int)(blockIdx.x & 7);
+        if (r >= a.n_rows) return;
+    } else {
+        const int64_t pair = (place / a.tiles) * 8 + (int64_t)(blockIdx.x & 7);
+        if (pair >= a.pairs) return;
+        b = (int)(pair % a.gy), r = (int)(pair / a.gy);
+    }
     if (a.n_rows <= 64 && a.n_rows > 1) {
         // (keys are distinct: the length, then the lower index first)
         uint64_t mine = 0;
@@ -736,7 +745,7 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
     }
     // The partial output as the registers hold it, a lane's four values side by side and the lanes in order (whole
     // kilobytes a store): [unit][partition][wavefront][value block][row block][v / 4][lane][4]; the merge below reads the
-    // same way. (A tile of 128 rows is one column's: the heads are a multiple of 128.)
+    // same way. (Rows past a window's last are stored too, and never read.)
     if (h == 0 && liveq) {
         const int64_t index = ((int64_t)((int64_t)r * a.columns + colq) * H + headq) * a.parts + b;
         a.pm[index] = m, a.pl[index] = l;
@@ -893,21 +902,24 @@ int launch_tiles(const LatentArgs& a, bool f16, bool fp8, hipStream_t stream) {
     return hip_code(hipGetLastError());
 }
 
-// Which launches the many-heads kernel can serve: 16-bit caches of the one shape it is built for, heads in 128s, pages
-// of a multiple of 16 positions. It serves them unless the caller asks for the small tiles. (Nothing else decides, the
-// batch least of all: a token's bits follow the kernel that reads it.)
+// Which launches the many-heads kernel serves: 16-bit caches of the one shape it is built for with pages of a multiple
+// of 16 positions, where the caller asks for it (any number of heads: a tile of 128 rows is then 128 / heads columns of
+// a window, which is how a prompt chunk of few heads fills it) or, left to the library, where the heads come in 128s.
+// (Nothing else decides, the batch least of all: a token's bits follow the kernel that reads it.)
 template <int R, int P>
 bool many_heads(const LatentArgs& a, bool fp8) {
-    return R == 512 && P == 64 && !fp8 && a.heads % kHeadsRows == 0 && a.page % 16 == 0;
+    if (!(R == 512 && P == 64 && !fp8 && a.page % 16 == 0)) return false;
+    return a.tile_rows == kHeadsRows || (a.tile_rows == 0 && a.heads % kHeadsRows == 0);
 }
 
 template <int R, int P>
 int launch_shape(const LatentArgs& a, bool f16, bool fp8, int phases, hipStream_t stream) {
     if constexpr (R == 512 && P == 64) {
-        if (a.tile_rows != 16 && many_heads<R, P>(a, fp8)) {
+        if (many_heads<R, P>(a, fp8)) {
             LatentArgs u = a;
-            u.tiles = a.columns * a.heads / kHeadsRows;
-            const int64_t blocks = (int64_t)((a.n_rows + 7) / 8) * 8 * a.gy * u.tiles, merges = (int64_t)a.n_rows * u.tiles * 4;
+            u.tiles = (a.columns * a.heads + kHeadsRows - 1) / kHeadsRows;
+            const int64_t blocks = (a.n_rows >= kRowsToAnXcd ? (int64_t)((a.n_rows + 7) / 8) * 8 * a.gy : (u.pairs + 7) / 8 * 8) * u.tiles;
+            const int64_t merges = (int64_t)a.n_rows * u.tiles * 4;
             if (blocks > 0x7fffffff || merges > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
             if (phases != 2) {
                 if (f16) hipLaunchKernelGGL((latent_heads_kernel<R, P, true>), dim3((unsigned)blocks), dim3(256), 0, stream, u);
@@ -967,9 +979,7 @@ int launch_latent(const crit_pkv_latent_params* p, hipStream_t stream) {
     a.sscale = p->scale * kLog2e;
     a.tile_rows = p->tile_rows;
     if (p->tile_rows != 0 && p->tile_rows != 16 && p->tile_rows != kHeadsRows) return CRIT_PKV_E_GEOMETRY;
-    if (p->tile_rows == kHeadsRows &&
-        !(p->rank == 512 && p->rope == 64 && !fp8 && p->heads % kHeadsRows == 0 && p->page % 16 == 0))
-        return CRIT_PKV_E_GEOMETRY;
+    if (p->tile_rows == kHeadsRows && !(p->rank == 512 && p->rope == 64 && !fp8 && p->page % 16 == 0)) return CRIT_PKV_E_GEOMETRY;
     a.tiles = (p->columns * p->heads + 15) / 16;
     const int64_t table_keys = (int64_t)p->table_width * p->page;
     a.max_keys = (int)(table_keys < 0x3fffffff ? table_keys : 0x3fffffff);

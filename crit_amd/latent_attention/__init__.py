@@ -83,17 +83,18 @@ def partitions(device, heads, rank, rope, page, kind=0, tile_rows=None):
 def tile_rows(heads, rank, rope, page, kind=0, asked=None):
     """The query rows a workgroup holds for this geometry, 16 or 128, which names the kernel that reads it (and a token's
     bits follow the kernel). 128, the many-heads kernel (32 x 32 matrix tiles, the cache rows by DMA into LDS, one
-    workgroup a compute unit), takes 16-bit caches of DeepSeek's shape (512, 64) with heads in 128s and pages of a
-    multiple of 16 positions, and is what such a geometry gets unless `asked` (attend's tile_rows=) or the engine's tuned
-    TILE_ROWS says 16: it reads a batch of 64 rows about twice as fast as the small tiles, and a single row three times
-    slower (one workgroup a partition instead of four). Everything else gets 16."""
-    able = (int(rank), int(rope)) == (512, 64) and not int(kind) and int(heads) % 128 == 0 and int(page) % 16 == 0
+    workgroup a compute unit), takes 16-bit caches of DeepSeek's shape (512, 64) with pages of a multiple of 16
+    positions. Heads in 128s get it unless `asked` (attend's tile_rows=) or the engine's tuned TILE_ROWS says 16: it
+    reads a batch of 64 rows about twice as fast as the small tiles, and a single row twice slower (one workgroup a
+    partition instead of four). With fewer heads it is there for the asking (a tile is then 128 / heads columns of a
+    window: prompt chunks, prefill's packed=True); left alone they get 16, as does everything else."""
+    able = (int(rank), int(rope)) == (512, 64) and not int(kind) and int(page) % 16 == 0
     want = int(asked or _knob("TILE_ROWS", heads, rank, rope, page, kind) or 0)
     if want not in (0, 16, 128):
         raise ValueError(f"tile_rows: {want}; 16 or 128 (or 0: by the geometry)")
     if want == 128 and not able:
-        raise ValueError("tile_rows 128 reads 16-bit caches of (512, 64) with heads in 128s and pages of a multiple of 16")
-    return 128 if able and want != 16 else 16
+        raise ValueError("tile_rows 128 reads 16-bit caches of (512, 64) with pages of a multiple of 16 positions")
+    return 128 if able and (want == 128 or (want == 0 and int(heads) % 128 == 0)) else 16
 
 
 def write(latent, rope, slots, cache, scales=None):
@@ -227,7 +228,8 @@ def attend(q, cache, tables, rows, starts, firsts, columns, page, *, rank, count
         raise ValueError(f"out: BF16, FP16 or FP32 [tokens][heads][{R}], unit stride along its last dimension")
     if lse is not None and (lse.dtype != torch.float32 or not lse.is_contiguous()):
         raise ValueError("lse: contiguous FP32 [tokens][heads]")
-    states_a_row = columns * heads * parts
+    # (the many-heads kernel stores whole tiles of 128 rows)
+    states_a_row = (-(-columns * heads // 128) * 128 if tiles == 128 else columns * heads) * parts
     floats_a_row = states_a_row * (R + 2)
     if workspace is None:
         rows_a_launch = max(1, min(batch, (PARTIAL_BYTES // 4) // floats_a_row))
@@ -265,14 +267,22 @@ def attend(q, cache, tables, rows, starts, firsts, columns, page, *, rank, count
 
 def prefill(q, cache, table, position, page, *, rank, scale=None, out: Optional[torch.Tensor] = None,
             lse: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None,
-            scales: Optional[torch.Tensor] = None, tile_rows=None) -> torch.Tensor:
+            scales: Optional[torch.Tensor] = None, tile_rows=None, packed=False) -> torch.Tensor:
     """A prompt chunk of one sequence, causal: q [T][heads][R + P] are the tokens at positions position .. position +
     T - 1 (their rows already written), table [pages] int32 the sequence's page table; position is an int, or a
     one-element int64 device tensor that is read on the device so that one captured graph serves every position.
     Returns out [T][heads][R] (and fills lse [T][heads] when given). The chunk is read as windows of MAX_COLUMNS
     columns through attend(), so a token's bits are those of the same position decoded and do not depend on T. scale,
-    sinks, lse and an E4M3 cache's scales as attend() takes them."""
+    sinks, lse and an E4M3 cache's scales as attend() takes them.
+
+    packed=True reads the chunk with the many-heads kernel whatever the heads (tile_rows 128: a tile of 128 query rows
+    is 128 / heads tokens, the cache rows staged once for all of them), which a chunk of some hundred tokens fills where
+    a decode step of few heads does not: several times the small tiles' speed at 16 heads. A token's bits are then the
+    many-heads kernel's, not those of the same position decoded with the small tiles (the same attention, other sums:
+    within the tolerance either has against the exact result); they still do not depend on T or on its neighbours."""
     _Call(q, cache, page, rank, sinks, scales)
+    if packed:
+        tile_rows = 128
     count = q.shape[0]
     if count < 1 or table.dim() != 1:
         raise ValueError("prefill: at least one token, over one page table [pages]")

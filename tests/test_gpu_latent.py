@@ -126,6 +126,7 @@ def test_many_heads_either_kernel_matches_float64_and_a_tokens_bits_follow_the_k
     la = cache.la
     assert la.tile_rows(128, 512, 64, 16) == 128 and la.tile_rows(128, 512, 64, 16, asked=16) == 16
     assert la.tile_rows(64, 512, 64, 16) == 16 and la.tile_rows(128, 512, 64, 24) == 16 and la.tile_rows(128, 512, 64, 16, 1) == 16
+    assert la.tile_rows(64, 512, 64, 16, asked=128) == 128
     q = _q(16, 128, 576, 32)
     rows, starts, firsts = [0, 1, 2, 3], [0, 4, 8, 12], [1496, 29, 2096, 511]
     sinks = torch.randn(128, generator=torch.Generator().manual_seed(33)).to(dev)
@@ -149,9 +150,10 @@ def test_many_heads_either_kernel_matches_float64_and_a_tokens_bits_follow_the_k
     torch.testing.assert_close(other.float(), together.float(), atol=8e-3, rtol=2e-2)      # the same attention, other sums
     with pytest.raises(ValueError):
         cache.attend(q, rows, starts, firsts, 4, tile_rows=64)
-    small = Cache(512, 64, 16, [40], seed=34)
-    with pytest.raises(ValueError):      # 16 heads: not the many-heads kernel's
-        small.attend(_q(1, 16, 576, 35), [0], [0], [39], 1, tile_rows=128)
+    odd = Cache(512, 64, 24, [40], seed=34)
+    with pytest.raises(ValueError):      # pages of no multiple of 16 positions: not the many-heads kernel's
+        odd.attend(_q(1, 128, 576, 35), [0], [0], [39], 1, tile_rows=128)
+    assert torch.equal(odd.attend(_q(1, 128, 576, 35), [0], [0], [39], 1), odd.attend(_q(1, 128, 576, 35), [0], [0], [39], 1, tile_rows=16))
 
 
 @pytest.mark.parametrize("heads", [16, 128])
@@ -240,6 +242,28 @@ def test_prompt_chunks_match_float64_and_are_their_positions_decoded(rank, rope,
         for t in (0, T // 2, T - 1):
             alone = cache.attend(q[t:t + 1], [0], [0], [position + t], 1, scale=scale, sinks=sinks)
             assert torch.equal(alone[0], out[t]), (position, t)
+
+
+@pytest.mark.parametrize("heads", [16, 24, 64])
+def test_packed_prompt_chunks_of_few_heads_match_float64_and_a_tokens_bits_do_not_follow_the_chunk(heads):
+    # packed=True: the many-heads kernel reads the chunk, a tile of 128 query rows being 128 / heads tokens (with 24
+    # heads a token straddles two tiles). Against the exact result at the module's tolerance; a token's bits are those of
+    # the same position read alone by the same kernel (tile_rows=128), whatever the chunk's length; against the small
+    # tiles' decode bits they are another rounding of the same sums, inside the same tolerance.
+    cache = Cache(512, 64, 16, [1200], seed=41)
+    la = cache.la
+    sinks = torch.randn(heads, generator=torch.Generator().manual_seed(42)).to(dev)
+    for position, T in ((0, 70), (500, 133), (1199 - 300, 301)):
+        q = _q(T, heads, 576, position + 3)
+        lse = torch.empty(T, heads, device=dev)
+        out = la.prefill(q, cache.cache, cache.tables[0], position, 16, rank=512, lse=lse, sinks=sinks, packed=True)
+        cache.check(q, out, lse, 0, 0, position, T, 576 ** -0.5, sinks, lse_tol=2e-3)
+        for t in (0, T // 2, T - 1):
+            alone = cache.attend(q[t:t + 1], [0], [0], [position + t], 1, sinks=sinks, tile_rows=128)
+            assert torch.equal(alone[0], out[t]), (position, t)
+        assert torch.equal(la.prefill(q[:T // 2], cache.cache, cache.tables[0], position, 16, rank=512, sinks=sinks, packed=True), out[:T // 2])
+        decoded = la.prefill(q, cache.cache, cache.tables[0], position, 16, rank=512, sinks=sinks)
+        torch.testing.assert_close(out.float(), decoded.float(), atol=8e-3, rtol=2e-2)
 
 
 def test_a_prompt_tokens_bits_do_not_follow_its_chunks_length_and_a_graph_replays_at_device_positions():
