@@ -672,13 +672,14 @@ def index_selection(device):
     return found
 
 
-def reference_shapes(pk, device):
+def reference_shapes(pk, device, only=None):
     """The shapes the reference publishes its decode and append rows on (its paged-kv-attention README: 24 query / 4 KV
     heads x 256 over `fp8:row` pages of 64, 24 / 2 x 256 bf16, 56 / 8 x 128 int8 row-scaled; 1 and 8 rows; 1, 5 and 8
     columns; 4K, 16K and 200K positions; `write` of 1 / 256 / 4,096 tokens into 8,192 shuffled slots), one layer,
     replayed from a captured graph over four caches read in turn (each launch cold), each with its fraction of the
     8 TB/s HBM peak. The reference's own figures are for another card (RTX 5090) and are context, not a target. Widths
-    other than 128 x 128 take attend_generic_kernel; 56 / 8 x 128 the matrix-core kernel."""
+    256-wide heads take the matrix-core kernel in two 128-wide halves, 56 / 8 x 128 as the 128-wide pools do. `only`
+    (--shape): run just the rows whose name contains it, for a profile of one shape."""
     found = {}
     g = torch.Generator(device=device).manual_seed(11)
     shapes = (("24q_4kv_x256_fp8row_page64", 24, 4, 256, 64, "fp8:row"), ("24q_2kv_x256_bf16_page16", 24, 2, 256, 16, "bf16"),
@@ -687,6 +688,10 @@ def reference_shapes(pk, device):
         e = 2 if kind == "bf16" else 1
         store = torch.bfloat16 if kind == "bf16" else (torch.int8 if kind == "int8" else torch.float8_e4m3fn)
         for ctx, rows_cases in ((4096, ((1, 1), (8, 1))), (16384, ((1, 1), (8, 1))), (200_000, ((1, 1), (1, 5), (1, 8), (8, 1)))):
+            if only:
+                rows_cases = tuple(c for c in rows_cases if only in f"{name}_{c[0]}_rows_{c[1]}_cols_ctx{ctx}")
+                if not rows_cases:
+                    continue
             most = max(b for b, _ in rows_cases)
             width = ((ctx + 8 + page - 1) // page + 15) // 16 * 16
             pages = most * width
@@ -734,6 +739,8 @@ def reference_shapes(pk, device):
     v = torch.randn(pages + 1, page, hkv, d, device=device, dtype=torch.bfloat16, generator=g)
     table = torch.randperm(pages, device=device, generator=g).to(torch.int32)
     for T in (16, 256, 2048):
+        if only and only not in f"prefill_{T}_tokens_after_1024_bf16_24q_2kv_x256":
+            continue
         q = torch.randn(T, hq, d, device=device, generator=g).to(torch.bfloat16)
         out = torch.empty_like(q)
         position = torch.tensor([1024], dtype=torch.int64, device=device)
@@ -746,6 +753,8 @@ def reference_shapes(pk, device):
     k = torch.zeros(8192, hkv, d, dtype=torch.bfloat16, device=device)
     v = torch.zeros_like(k)
     for T in (1, 256, 4096):
+        if only and only not in f"write_{T}_tokens_into_8192_slots_bf16_2kv_x256":
+            continue
         keys = torch.randn(T, hkv, d, device=device, generator=g).to(torch.bfloat16)
         values = torch.randn(T, hkv, d, device=device, generator=g).to(torch.bfloat16)
         slots = torch.randperm(8192, device=device, generator=g)[:T]
@@ -881,6 +890,7 @@ def main():
                     help="run only the pool bookkeeping of the extras (slots, the move of accepted rows, page copies)")
     ap.add_argument("--latent-only", action="store_true", help="run only the latent-attention decode of the extras")
     ap.add_argument("--index-only", action="store_true", help="run only the sparse index selection of the extras")
+    ap.add_argument("--shape", default=None, help="with --shapes-only: only the rows whose name contains this")
     ap.add_argument("--shapes-only", action="store_true",
                     help="run only the decode and append rows at the shapes the reference publishes its own on")
     ap.add_argument("--calibrate", action="store_true",
@@ -910,7 +920,7 @@ def main():
         print(json.dumps({"sparse_index_selection": found}), flush=True)
         return
     if args.shapes_only:
-        found = reference_shapes(pk, device)
+        found = reference_shapes(pk, device, args.shape)
         log(f"[bench] the reference's published shapes: {found}")
         print(json.dumps({"reference_published_shapes": found}), flush=True)
         return

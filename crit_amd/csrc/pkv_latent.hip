@@ -364,7 +364,8 @@ __global__ __launch_bounds__(256, NT == 1 ? 3 : 2) void latent_kernel(LatentArgs
 // bytes, so the 16-byte chunks of a row are stored permuted: chunk c of position n at place c ^ (4 (n & 3) + ((n >> 2)
 // & 3)) of the latent row (c ^ ((n >> 1) & 7) of the rotary row). The score product's operand read (16 lanes: 16
 // positions, one chunk each) and the transposing read of the values (a half-wave: 4 positions x 64 bytes) then both
-// fall on all 64 banks once (the bank-conflict counter reads zero).
+// fall on all 64 banks once (the bank-conflict counter read zero while the tiles were all the LDS traffic; the 8-byte
+// writes of the probabilities meet two to a bank).
 //
 // The softmax keeps a row's reference maximum until the running maximum exceeds it by more than kLazyHeads (base 2), so
 // the 256 accumulators are rescaled on few steps; the decision is the row's own, from its own scores in step order.
