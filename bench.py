@@ -1068,7 +1068,7 @@ def main():
                      "frac": mixed["prefill_frac_of_bf16_mfma_peak"]})
         for name, found in extras["latent_attention_decode"].items():
             if isinstance(found, dict) and "split_us" in found:
-                also.append({"kernel": "latent_kernel", "workload": f"64 rows ctx~U[1024,8192] rank 512 + rope 64, {name}",
+                also.append({"kernel": "latent_heads_kernel" if found.get("tile_rows") == 128 else "latent_kernel", "workload": f"64 rows ctx~U[1024,8192] rank 512 + rope 64, {name}",
                              "us": found["split_us"], "with_merge_us": found["with_merge_us"], "bound": "hbm",
                              "frac": found["split_frac_of_hbm_peak"], "mfma_frac": found["split_frac_of_bf16_mfma_peak"]})
         result["roofline"]["also"] = also

@@ -713,10 +713,10 @@ int launch_index_scores(const crit_pkv_index_scores_params* p, hipStream_t strea
     a.scale = p->scale, a.block = 64;
     const int cus = compute_units() > 0 ? compute_units() : 256;
     // many tokens share their keys through LDS, 4 or 8 to a workgroup: where the keys are read in place, a group's
-    // tokens (they share the slots) must fill workgroups
+    // tokens (they share the slots) must fill workgroups, unless one list serves every token (slots_stride 0)
     const int ht = (p->heads + 15) / 16;
     const int wg_tokens = ht * (p->dim / 32) <= 16 && ht <= 4 ? 8 : 4;
-    const bool many = p->tokens >= 16 && (!p->slots || p->group % wg_tokens == 0);
+    const bool many = p->tokens >= 16 && (!p->slots || p->slots_stride == 0 || p->group % wg_tokens == 0);
     const bool f16 = p->q_dtype == CRIT_PKV_F16;
     if (fp8) return f16 ? launch_scores_kind<true, true>(a, p->dim, many, cus, stream) : launch_scores_kind<false, true>(a, p->dim, many, cus, stream);
     return f16 ? launch_scores_kind<true, false>(a, p->dim, many, cus, stream) : launch_scores_kind<false, false>(a, p->dim, many, cus, stream);

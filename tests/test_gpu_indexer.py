@@ -181,6 +181,21 @@ def test_keys_read_in_place_score_as_their_gathered_copy(fp8, kind):
         si.scores(q, store, w, ends, key_scales=scales, slots=slots.float())
 
 
+def test_one_list_for_many_tokens_takes_the_shared_kernel_whatever_their_count():
+    # One slot list [n] for every token (a prompt chunk of one sequence): 19 or 21 tokens fill no whole workgroups of 4
+    # or 8, and share their keys through LDS all the same; every token scores as it does alone.
+    n = 900
+    g = torch.Generator().manual_seed(15)
+    store = (torch.randn(4000, 128, generator=g) * 0.5).to(dev).to(torch.bfloat16)
+    slots = torch.randperm(4000, generator=g)[:n].to(dev)
+    for tokens in (19, 21):
+        q, _, _, _, w, ends = problem(tokens, 64, 128, n, seed=16 + tokens)
+        got = si.scores(q, store, w, ends, slots=slots)
+        assert torch.equal(got, si.scores(q, store[slots], w, ends))
+        for t in (0, 7, tokens - 1):
+            assert torch.equal(got[t], si.scores(q[t:t + 1], store, w[t:t + 1], ends[t:t + 1], slots=slots)[0]), t
+
+
 @pytest.mark.parametrize("fp8", [False, True])
 @pytest.mark.parametrize("each", [16, 12])
 def test_a_rounds_rows_share_their_keys_in_place(fp8, each):
