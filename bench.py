@@ -891,6 +891,8 @@ def main():
     ap.add_argument("--latent-only", action="store_true", help="run only the latent-attention decode of the extras")
     ap.add_argument("--index-only", action="store_true", help="run only the sparse index selection of the extras")
     ap.add_argument("--shape", default=None, help="with --shapes-only: only the rows whose name contains this")
+    ap.add_argument("--append-only", action="store_true",
+                    help="run only the KV append with rope and norm fused in beside the plain append (for counter runs on write_rows)")
     ap.add_argument("--shapes-only", action="store_true",
                     help="run only the decode and append rows at the shapes the reference publishes its own on")
     ap.add_argument("--calibrate", action="store_true",
@@ -923,6 +925,11 @@ def main():
         found = reference_shapes(pk, device, args.shape)
         log(f"[bench] the reference's published shapes: {found}")
         print(json.dumps({"reference_published_shapes": found}), flush=True)
+        return
+    if args.append_only:
+        found = append_rope(pk, device)
+        log(f"[bench] append with rope and norm: {found}")
+        print(json.dumps({"append_with_rope_and_norm": found}), flush=True)
         return
     if args.pool_only:
         found = pool_bookkeeping(pk, device)
