@@ -29,7 +29,7 @@ struct WriteArgs {
     // RMS norm of each key head in front of the rotation (norm_weight null: none): x / sqrt(mean(x^2) + eps) times
     // (norm_weight[i] + norm_offset), FP32 [dim[0]].
     const float* norm_weight;
-    float norm_eps, norm_offset;
+    float norm_eps, norm_offset, norm_inv_dim;
 };
 
 template <int IN>
@@ -162,6 +162,7 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
     int head[U];
     bool second[U], in[U], live[U];      // second: a row of the values; live: this lane holds elements of the row
     float mult[U];                       // "fp8" pages: the row's divisor, fetched with its inputs
+    int64_t rope_pos = 0;                // ROPE: the token's position, fetched with its inputs (the table's row waits for it)
     // Every load of the U rows is issued before anything waits for one: no load sits under a condition (a row past the
     // end reads row 0, a lane past a narrow row's width reads the row's start) and nothing indexes the launch arguments
     // by a value a lane computes (which would fetch them from memory): the choice between the keys' and the values'
@@ -184,13 +185,12 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
         const void* src = second[u] ? a.src[1] : a.src[0];
         const int64_t st = second[u] ? a.stride_t[1] : a.stride_t[0], sh = second[u] ? a.stride_h[1] : a.stride_h[0];
         raw[u].load(src, (int64_t)t * st + head[u] * sh + (live[u] ? i0 : 0));
+        if constexpr (ROPE) rope_pos = a.positions[t];
     }
     __builtin_amdgcn_sched_barrier(0);      // (nothing that waits for a load moves up among the loads)
     if constexpr (ROPE) {
         static_assert(U == 1 && LPR >= 2, "one row a thread, a row over two lanes or more");
-        const uint32_t rowc = in[0] ? row0 : 0;
-        const uint32_t t = div32(a.heads_div, rowc);
-        int64_t pos = a.positions[t];
+        int64_t pos = rope_pos;
         pos = pos < 0 ? 0 : (pos > a.rope_rows - 1 ? a.rope_rows - 1 : pos);
         const int half = a.dim[0] >> 1;
         const bool upper = lane_in_row >= LPR / 2;
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
         }
         float mine[EPL], other[EPL], y[EPL];
         raw[0].widen(mine);
-        raw[0].across(LPR / 2).widen(other);
+        if (!a.norm_weight) raw[0].across(LPR / 2).widen(other);
         if (a.norm_weight) {
             // The reference's rms_norm_rope (inference/fused-norms/code/torch_norms.py:149-176): each head normalised
             // in FP32, times its weight, rotated, one rounding at the end. The sum of squares in a fixed order, the same
@@ -231,24 +231,27 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
                 sq = g8 == 0 ? s8 : sq + s8;
             }
             sq = LPR > 1 ? group_sum<(LPR > 1 ? LPR : 2)>(sq) : sq;      // (the butterfly's sums, lane pairs met in the vector pipe)
-            const float mean = __fdiv_rn(sq, (float)a.dim[0]);
+            const float mean = sq * a.norm_inv_dim;      // (the width is a power of two: the product is the quotient, exactly)
             // __builtin_sqrtf is the correctly rounded root (hipcc's default for sqrtf and "/"); __fsqrt_rn is not,
             // unless OCML_BASIC_ROUNDED_OPERATIONS is defined: it is the hardware's approximate one.
             const float r = __fdiv_rn(1.0f, __builtin_sqrtf(mean + a.norm_eps));
-            const int i_other = (lane_in_row ^ (LPR / 2)) * EPL;      // the partner lane's first element (style half)
             const float4* w_mine = reinterpret_cast<const float4*>(a.norm_weight + i0);
-            const float4* w_other = reinterpret_cast<const float4*>(a.norm_weight + i_other);
 #pragma unroll
             for (int j = 0; j < EPL / 4; ++j) {
-                const float4 wm = w_mine[j], wo = w_other[j];
-                const float m4[4] = {wm.x, wm.y, wm.z, wm.w}, o4[4] = {wo.x, wo.y, wo.z, wo.w};
+                const float4 wm = w_mine[j];
+                const float m4[4] = {wm.x, wm.y, wm.z, wm.w};
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const float fm = a.norm_offset != 0.0f ? m4[k] + a.norm_offset : m4[k];
-                    const float fo = a.norm_offset != 0.0f ? o4[k] + a.norm_offset : o4[k];
                     mine[4 * j + k] = (mine[4 * j + k] * r) * fm;
-                    other[4 * j + k] = (other[4 * j + k] * r) * fo;
                 }
+            }
+            // the partner lane's elements (style half) as that lane normalised them: the same operations on the same
+            // numbers as normalising them here, without doing it twice
+#pragma unroll
+            for (int j = 0; j < EPL; ++j) {
+                if (LPR / 2 == 8) other[j] = u2f((uint32_t)__builtin_amdgcn_update_dpp(0, (int)f2u(mine[j]), 0x128, 0xf, 0xf, true));
+                else other[j] = __shfl_xor(mine[j], LPR / 2);
             }
         }
         if (a.rope_interleaved) {
@@ -488,6 +491,7 @@ int launch_write(const crit_pkv_write_params* p, hipStream_t stream) {
     a.rope_table = p->rope_table, a.positions = p->rope_positions, a.rope_rows = p->rope_rows;
     a.rope_interleaved = p->rope_interleaved ? 1 : 0, a.rope_scale = p->rope_scale;
     a.norm_weight = p->norm_weight, a.norm_eps = p->norm_eps, a.norm_offset = p->norm_offset;
+    a.norm_inv_dim = 1.0f / (float)p->head_dim;
     if (p->norm_weight && (!p->rope_table || (reinterpret_cast<uintptr_t>(p->norm_weight) % 16))) return CRIT_PKV_E_GEOMETRY;
     if (p->rope_table) {
         // the whole head width rotates, a power of two of whole lanes; the lanes of a values' row of another width
