@@ -91,6 +91,25 @@ PKV_DEV uint32_t bf16_rne(float x) {
     return (x != x) ? 0x7fc0u : r;
 }
 PKV_DEV uint32_t pack_bf16(float a, float b) { return bf16_rne(a) | (bf16_rne(b) << 16); }
+// Eight FP32 values as four BF16 pairs with the same bits as pack_bf16, by the hardware's conversion (v_cvt_pk_bf16_f32:
+// round to nearest even, like bf16_rne, for every number) where no value is a NaN, which one test over the packed
+// words decides (a 16-bit half above 0x7F80 in magnitude): a NaN comes out of the hardware quiet but with its payload,
+// and torch's cast stores 0x7FC0, so then the words are made again one value at a time.
+PKV_DEV u32x4 pack8_bf16(const float (&x)[8]) {
+    typedef __attribute__((ext_vector_type(2))) __bf16 pair_t;
+    uint32_t w[4], any = 0u;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const pair_t r = {(__bf16)x[2 * j], (__bf16)x[2 * j + 1]};
+        w[j] = __builtin_bit_cast(uint32_t, r);
+        any |= (w[j] & 0x7fff7fffu) + 0x007f007fu;
+    }
+    if (any & 0x80008000u) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) w[j] = pack_bf16(x[2 * j], x[2 * j + 1]);
+    }
+    return u32x4{w[0], w[1], w[2], w[3]};
+}
 
 PKV_DEV float f16_lo(uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu)); }
 PKV_DEV float f16_hi(uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16)); }

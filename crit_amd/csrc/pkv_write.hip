@@ -91,8 +91,8 @@ struct RawRow {
             static_for<N>([&](auto j) { v[j] = u32x4{f2u(x[4 * j]), f2u(x[4 * j + 1]), f2u(x[4 * j + 2]), f2u(x[4 * j + 3])}; });
         } else if constexpr (IN == CRIT_PKV_BF16) {
             static_for<N>([&](auto j) {
-                v[j] = u32x4{pack_bf16(x[8 * j], x[8 * j + 1]), pack_bf16(x[8 * j + 2], x[8 * j + 3]),
-                             pack_bf16(x[8 * j + 4], x[8 * j + 5]), pack_bf16(x[8 * j + 6], x[8 * j + 7])};
+                const float x8[8] = {x[8 * j], x[8 * j + 1], x[8 * j + 2], x[8 * j + 3], x[8 * j + 4], x[8 * j + 5], x[8 * j + 6], x[8 * j + 7]};
+                v[j] = pack8_bf16(x8);
             });
         } else {
             static_for<N>([&](auto j) {
@@ -262,8 +262,13 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
                 y[2 * j + 1] = x1 * cs[j] + x0 * sn[j];
             }
         } else {
+            {
+                // (a - b is a + (-b), bit for bit: the lower half's sign goes into its sines, one XOR an element, and
+                // the two halves run the same three operations)
+                const uint32_t flip = upper ? 0u : 0x80000000u;
 #pragma unroll
-            for (int j = 0; j < EPL; ++j) y[j] = upper ? mine[j] * cs[j] + other[j] * sn[j] : mine[j] * cs[j] - other[j] * sn[j];
+                for (int j = 0; j < EPL; ++j) y[j] = mine[j] * cs[j] + other[j] * u2f(f2u(sn[j]) ^ flip);
+            }
         }
         if (!second[0]) raw[0].pack(y);
     }
@@ -285,7 +290,8 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
             if constexpr (F16) {
                 v = make_uint4(pack_f16(x[0], x[1]), pack_f16(x[2], x[3]), pack_f16(x[4], x[5]), pack_f16(x[6], x[7]));
             } else {
-                v = make_uint4(pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]), pack_bf16(x[6], x[7]));
+                const u32x4 packed = pack8_bf16(x);
+                v = make_uint4(packed.x, packed.y, packed.z, packed.w);
             }
             if (live[u]) __builtin_nontemporal_store(u32x4{v.x, v.y, v.z, v.w}, reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(pages) + dst));
         } else {
