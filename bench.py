@@ -556,8 +556,8 @@ def latent_decode(device):
     contexts ~U[1024, 8192], for the 16 heads a GPU of eight holds and for all 128, BF16 and E4M3 (one scale a row: a
     KV pool's fp8:row pages) caches. Bytes: the cache rows read once (the algorithmic figure); flops: 2 (2 R + P) a
     position and head. The split launch alone (phases=1) and with its merge, replayed from a captured graph. At 128
-    heads of a BF16 cache the many-heads kernel reads (tile_rows 128); the row `bf16_128_heads_by_tile_rows` sets it
-    against the small tiles at 64, 8 and 1 batch rows, which is the trade its default makes."""
+    heads the many-heads kernel reads (tile_rows 128); the rows `*_128_heads_by_tile_rows` set it against the small
+    tiles at 64, 8 and 1 batch rows, which is the trade its default makes."""
     import crit_amd.latent_attention as la
     R, P, page, B = 512, 64, 64, 64
     lengths = torch.randint(1024, 8193, (B,), generator=torch.Generator().manual_seed(7)).tolist()
@@ -602,17 +602,17 @@ def latent_decode(device):
                 "split_frac_of_hbm_peak": round(nbytes / split / 1e6 / HBM_PEAK_GBPS, 4),
                 "split_TFLOP/s": round(flops / split / 1e9, 1),
                 "split_frac_of_bf16_mfma_peak": round(flops / split / 1e9 / 2500.0, 4)}
-            if kind == "bf16" and heads == 128:
+            if heads == 128:
                 trade = {}
                 for n in (64, 8, 1):
                     for tiles in (128, 16):
                         def some(phases=0):
-                            for cache in caches:
+                            for cache, sc in zip(caches, scales):
                                 la.attend(q[:n], cache, tables, rows[:n], rows[:n], firsts[:n], 1, page, rank=R, out=out[:n],
-                                          phases=phases, tile_rows=tiles)
+                                          scales=sc, phases=phases, tile_rows=tiles)
                         some()
                         trade[f"{n}_rows_tile_rows_{tiles}_us"] = round(graph_timed(some, 3) / layers * 1e3, 1)
-                found["bf16_128_heads_by_tile_rows"] = trade
+                found[f"{kind}_128_heads_by_tile_rows"] = trade
         del caches, scales
     return found
 

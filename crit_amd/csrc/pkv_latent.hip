@@ -379,7 +379,7 @@ __global__ __launch_bounds__(256, NT == 1 ? 3 : 2) void latent_kernel(LatentArgs
 // the probabilities' way through LDS 750, values 1,900, barriers 300), and a unit's start (ranking the rows, the table,
 // the queries: 36 gathers of 32 rows x 32 bytes a wavefront) and end (256 KB of partials) another 38,000. With one
 // workgroup a compute unit nothing hides either, so launches of a few rows are slower than with the small tiles (1 row:
-// 80 us against 40): tile_rows = 16 asks for those.
+// 80 us against 40): tile_rows = 16 asks for those. E4M3 rows (see the kernel's constants): 171 us.
 constexpr float kLazyHeads = 8.0f;
 constexpr int kHeadsRows = 128;      // query rows a workgroup of the many-heads kernel holds
 constexpr int kRowsToAnXcd = 16;     // launches of that many batch rows or more keep a row's units on one XCD
@@ -400,6 +400,9 @@ PKV_DEV void dma_row(uint32_t offset, const uint8_t* base, unsigned lds) {
 }
 PKV_DEV void dma_any(const uint8_t* from, unsigned lds) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(from), "s"(lds));
+}
+PKV_DEV void dma_word(const float* from, unsigned lds) {      // 4 bytes a lane, to LDS bytes lds + 4 lane
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(from), "s"(lds));
 }
 template <int N>
 PKV_DEV void wait_loads() {
@@ -423,13 +426,22 @@ PKV_DEV void lds_arrived(u32x4& x) {      // (the operand is named so that its u
     asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(AHEAD));
 }
 
-template <int R, int P, bool F16>
+template <int R, int P, bool F16, bool FP8>
 __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
     static_assert(R == 512 && P == 64, "rows of 1,024 + 128 bytes");
     constexpr int W = R + P, KS = W / 16, KSL = R / 16, NB = R / 32;      // k-steps of the scores (the first KSL the latent's); value blocks
-    constexpr int MAIN = 32 * R * 2, TILE = MAIN + 32 * P * 2, NSTAGE = 4;
-    constexpr int LPT = 9;      // loads a wavefront issues a tile: its 8 latent rows, and the rotary keys of the same rows
+    // E4M3 caches: the codes land in a ring of three raw tiles (a wavefront's eight rows side by side, as they lie in
+    // HBM) and the wavefront that fetched them writes them out as 16-bit values, exactly, into one of two tiles of the
+    // layout the products read, one step ahead of its use; a row's scales travel the same way.
+    constexpr int MAIN = 32 * R * 2, TILE = MAIN + 32 * P * 2, NSTAGE = FP8 ? 2 : 4;
+    constexpr int RAW = 32 * W, NRAW = 3, CPR = W / 16;      // a raw tile's bytes; raw tiles; 16-byte chunks of a row of codes
+    // loads a wavefront issues a tile: its 8 latent rows and the rotary keys of the same rows (16-bit); 4.5 KB of codes
+    // and the rows' scales (E4M3)
+    constexpr int LPT = FP8 ? 6 : 9;
     __shared__ __align__(1024) uint8_t ring[NSTAGE * TILE];
+    __shared__ __align__(1024) uint8_t raw[FP8 ? NRAW * RAW : 16];
+    __shared__ float s_raw_scale[FP8 ? NRAW : 1][4][16];             // [raw tile][wavefront][latent, rotary][its row]
+    __shared__ __align__(16) float s_scale[FP8 ? 2 : 1][2][32];      // [tile][latent, rotary][position]
     __shared__ __align__(16) uint8_t s_prob[kHeadsRows * 64];      // the step's probabilities, 16-bit [row][position]
     __shared__ float s_alpha[kHeadsRows];                           // the step's factor on each row's accumulators
 
@@ -519,8 +531,10 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
     // between the score products, a few products apart: issued back to back they would hold the wavefront, and its SIMD's
     // matrix pipe with it, until the memory pipe has taken them all.
     const uint8_t* plan_row0 = a.cache;
+    const float* plan_scale0 = a.scales;
     int plan_room = 0;
-    unsigned plan_to = 0;
+    unsigned plan_to = 0, plan_scale_to = 0;
+    const unsigned raw_at = (unsigned)(uintptr_t)raw, raw_scale_at = (unsigned)(uintptr_t)&s_raw_scale[0][0][0];
     auto plan = [&](int t, int stage) __attribute__((always_inline)) -> int {
         t = t < n_tiles ? t : n_tiles - 1;
         if (t - held_from >= 64) hold_tiles(held_from + 64);
@@ -528,13 +542,31 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
         const int page_slot = __builtin_amdgcn_readlane(tile_slot, t - held_from);
         const int n0 = min(base + 8 * wave, n_keys - 1);
         plan_room = n_keys - 1 - n0;      // rows after the wavefront's first that are their own (the others repeat the last position)
-        plan_row0 = a.cache + (int64_t)(page_slot + n0) * (W * 2);
-        plan_to = ring_at + (unsigned)(stage * TILE);
+        if constexpr (FP8) {
+            plan_row0 = a.cache + (int64_t)(page_slot + n0) * W;
+            plan_scale0 = a.scales + (int64_t)(page_slot + n0) * a.scales_per_row;
+            plan_to = raw_at + (unsigned)(stage * RAW + wave * (8 * W));
+            plan_scale_to = raw_scale_at + (unsigned)((stage * 4 + wave) * 64);
+        } else {
+            plan_row0 = a.cache + (int64_t)(page_slot + n0) * (W * 2);
+            plan_to = ring_at + (unsigned)(stage * TILE);
+        }
         return base;
     };
     auto send = [&](auto kc) __attribute__((always_inline)) {
         constexpr int k = decltype(kc)::value;
-        if constexpr (k < 8) {
+        if constexpr (FP8) {
+            // (chunk c of the wavefront's 288: row c / 36 of its eight; the last load fills half a kilobyte)
+            if constexpr (k < 5) {
+                const int c = 64 * k + ln;
+                if (k < 4 || ln < 32) {
+                    const int row = c / CPR;
+                    dma_any(plan_row0 + (uint32_t)(min(row, plan_room) * W + (c - row * CPR) * 16), plan_to + (unsigned)(k * 1024));
+                }
+            } else if constexpr (k == 5) {
+                if (ln < 16) dma_word(plan_scale0 + min(ln & 7, plan_room) * a.scales_per_row + (ln >> 3) * (a.scales_per_row - 1), plan_scale_to);
+            }
+        } else if constexpr (k < 8) {
             const uint32_t place = (uint32_t)(ln ^ ((2 * wave + k / 4) & 3)) * 16u;
             dma_row(place ^ (uint32_t)(64 * (k & 3)), plan_row0 + min(k, plan_room) * (W * 2), plan_to + (unsigned)((8 * wave + k) * (R * 2)));
         } else {
@@ -567,6 +599,47 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
     for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(bq[ks].x), "v"(bq[ks].y), "v"(bq[ks].z), "v"(bq[ks].w));
     // (the queries are waited for here, with the first tile; the next two tiles go out behind them)
     int base1 = issue(1, 1), base2 = issue(2, 2);
+    // E4M3: the wavefront's rows of raw tile `from`, as 16-bit values in tile `to` (a lane: 16 codes a turn).
+    auto convert = [&](int from, int to) __attribute__((always_inline)) {
+        if constexpr (FP8) {
+            asm volatile("" : "+v"(ln));
+            const uint8_t* codes_at = raw + from * RAW + wave * (8 * W);
+            uint8_t* tile_to = ring + to * TILE;
+#pragma unroll
+            for (int j = 0; j < 5; ++j) {
+                const int c = 64 * j + ln;
+                if (j < 4 || ln < 32) {
+                    const int row = c / CPR, cj = c - row * CPR, n = 8 * wave + row;
+                    const u32x4 codes = *reinterpret_cast<const u32x4*>(codes_at + c * 16);
+                    const uint32_t w[4] = {codes.x, codes.y, codes.z, codes.w};
+                    uint32_t o[8];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        if constexpr (F16) {
+                            const f32x2 lo = e4m3_pair<false>(w[k]), hi = e4m3_pair<true>(w[k]);
+                            o[2 * k] = pair16<true>(lo.x, lo.y), o[2 * k + 1] = pair16<true>(hi.x, hi.y);
+                        } else {
+                            const u32x2 both = codes4_to_pairs<1>(w[k]);
+                            o[2 * k] = both.x, o[2 * k + 1] = both.y;
+                        }
+                    }
+                    // (16-bit chunks 2 cj and 2 cj + 1 of position n, each at its permuted place)
+                    const bool latent = cj < KSL;
+                    const uint32_t turn = latent ? (uint32_t)(4 * (n & 3) + ((n >> 2) & 3)) : (uint32_t)((n >> 1) & 7);
+                    uint8_t* row_at = tile_to + (latent ? n * (R * 2) : MAIN + n * (P * 2));
+                    const uint32_t chunk = (uint32_t)(latent ? 2 * cj : 2 * (cj - KSL));
+                    *reinterpret_cast<u32x4*>(row_at + 16 * (chunk ^ turn)) = u32x4{o[0], o[1], o[2], o[3]};
+                    *reinterpret_cast<u32x4*>(row_at + 16 * ((chunk + 1) ^ turn)) = u32x4{o[4], o[5], o[6], o[7]};
+                }
+            }
+            if (ln < 16) s_scale[to][ln >> 3][8 * wave + (ln & 7)] = s_raw_scale[from][wave][ln];
+        }
+    };
+    if constexpr (FP8) {
+        wait_loads<2 * LPT>();      // (its own rows of the first tile are all a wavefront converts: no barrier)
+        convert(0, 0);
+    }
+    int raw_stage = 0;      // E4M3: the raw tile that held tile t (tile t + 3 goes there)
 
     float m = -INFINITY, l = 0.0f;
     f32x16 acc[4][4];      // [block of 32 values][block of 32 query rows]
@@ -579,9 +652,11 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
 
     for (int t = 0; t < n_tiles; ++t) {
         const int stage = t & (NSTAGE - 1);
-        wait_loads<2 * LPT>();      // the tile's loads of this wavefront have landed: those of the next two may be in flight
+        // 16-bit: the tile's loads of this wavefront have landed, those of the next two may be in flight. E4M3: the next
+        // tile's have (it is converted at the end of this step), the one after may be in flight.
+        wait_loads<FP8 ? LPT : 2 * LPT>();
         lds_barrier();              // everybody's have, and nobody reads the tile before any more, nor the last probabilities
-        const int base3 = plan(t + 3, (t + 3) & (NSTAGE - 1));
+        const int base3 = plan(t + 3, FP8 ? raw_stage : (t + 3) & (NSTAGE - 1));
         const uint8_t* tile = ring + stage * TILE;
         // Operand addresses inside a tile (see the layout above), from the opaque copy of the number of the lane.
         asm volatile("" : "+v"(ln));
@@ -602,45 +677,69 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
         // -- scores of the wavefront's 32 rows: 36 products in two chains (even and odd ones: a product every 32 clocks
         // cannot wait for the one before it), the operand of each read RING - 1 products ahead, five of the tile's loads
         // sent out in between
-        f32x16 s, s2;
+        // (E4M3: the rotary keys' products, which take a scale of their own, in a chain of their own, every ninth)
+        f32x16 s, s2, s3;
 #pragma unroll
         for (int v = 0; v < 16; ++v) s[v] = 0.0f, s2[v] = 0.0f;
+        if constexpr (FP8) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) s3[v] = 0.0f;
+        }
         {
-            constexpr int RING = 6;
+            constexpr int RING = FP8 ? 5 : 6;
             u32x4 ka[RING];
             const uint32_t tile_at = (uint32_t)(uintptr_t)tile;
-            // k-steps in the order 0, 8, 16, 24, 1, 9, ...: four share an address register
+            // the latent's k-steps in the order 0, 8, 16, 24, 1, 9, ...: four share an address register
             uint32_t k_at = 0;
             auto read_k = [&](auto ic) __attribute__((always_inline)) {
                 constexpr int i = decltype(ic)::value;
-                if constexpr (i < KSL) {
-                    constexpr int lo = i / 4, hi = i % 4;      // k-step lo + 8 hi
+                constexpr bool rotary = FP8 ? i % 9 == 8 : i >= KSL;
+                constexpr int at = FP8 ? (rotary ? i / 9 : i - i / 9) : (rotary ? i - KSL : i);
+                if constexpr (!rotary) {
+                    constexpr int lo = at / 4, hi = at % 4;      // k-step lo + 8 hi
                     if constexpr (hi == 0) k_at = tile_at + (k_lane ^ (uint32_t)(32 * lo));
                     lds_read16<256 * hi>(ka[i % RING], k_at);
                 } else {
-                    lds_read16<0>(ka[i % RING], tile_at + (t_lane ^ (uint32_t)(32 * (i - KSL))));
+                    lds_read16<0>(ka[i % RING], tile_at + (t_lane ^ (uint32_t)(32 * at)));
                 }
             };
             static_for<RING - 1>([&](auto ic) __attribute__((always_inline)) { read_k(ic); });
-            asm volatile("s_nop 1" : "+v"(s), "+v"(s2));
+            if constexpr (FP8) asm volatile("s_nop 1" : "+v"(s), "+v"(s2), "+v"(s3));
+            else asm volatile("s_nop 1" : "+v"(s), "+v"(s2));
             static_for<KS>([&](auto ic) __attribute__((always_inline)) {
                 constexpr int i = decltype(ic)::value;
                 if constexpr (i + RING - 1 < KS) read_k(std::integral_constant<int, i + RING - 1>{});
                 if constexpr (i % 8 == 2) send(std::integral_constant<int, i / 8>{});
                 constexpr int ahead = KS - 1 - i < RING - 1 ? KS - 1 - i : RING - 1;
                 lds_arrived<ahead>(ka[i % RING]);
-                constexpr int ks = i < KSL ? i / 4 + 8 * (i % 4) : i;
-                if constexpr (i % 2 == 0) score_product<F16>(s, ka[i % RING], bq[ks]);
+                constexpr bool rotary = FP8 ? i % 9 == 8 : i >= KSL;
+                constexpr int at = FP8 ? (rotary ? i / 9 : i - i / 9) : (rotary ? i - KSL : i);
+                constexpr int ks = rotary ? KSL + at : at / 4 + 8 * (at % 4);
+                if constexpr (FP8 && rotary) score_product<F16>(s3, ka[i % RING], bq[ks]);
+                else if constexpr ((FP8 ? at : i) % 2 == 0) score_product<F16>(s, ka[i % RING], bq[ks]);
                 else score_product<F16>(s2, ka[i % RING], bq[ks]);
             });
-            asm volatile("s_nop 15\n\ts_nop 15" : "+v"(s), "+v"(s2));      // (the products' results are read by vector instructions next)
+            // (the products' results are read by vector instructions next)
+            if constexpr (FP8) asm volatile("s_nop 15\n\ts_nop 15" : "+v"(s), "+v"(s2), "+v"(s3));
+            else asm volatile("s_nop 15\n\ts_nop 15" : "+v"(s), "+v"(s2));
         }
         // -- softmax of the lane's row over its 16 positions of the tile (the other half-wave holds the other 16): the
         // lane holds positions 8 (v / 4) + 4 h + v % 4
         const bool masked = base + 32 > unmasked;      // (the same for the whole wavefront)
         float x[16];
+        if constexpr (FP8) {      // (the scales of the lane's positions: the latent's, the rotary key's)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) x[v] = (s[v] + s2[v]) * a.sscale;
+            for (int q = 0; q < 4; ++q) {
+                const f32x4 scale0 = *reinterpret_cast<const f32x4*>(&s_scale[stage][0][8 * q + 4 * h]);
+                const f32x4 scale1 = *reinterpret_cast<const f32x4*>(&s_scale[stage][1][8 * q + 4 * h]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    x[4 * q + e] = __builtin_fmaf(s[4 * q + e] + s2[4 * q + e], scale0[e], s3[4 * q + e] * scale1[e]) * a.sscale;
+            }
+        } else {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) x[v] = (s[v] + s2[v]) * a.sscale;
+        }
         if (masked) {
             const int seen = min(lim, n_keys - 1) - base - 4 * h;      // position 8 (v / 4) + v % 4 of the lane's is seen up to this
 #pragma unroll
@@ -664,6 +763,14 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
         const float sum = (((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]))) +
                           (((p[8] + p[9]) + (p[10] + p[11])) + ((p[12] + p[13]) + (p[14] + p[15])));
         l = __builtin_fmaf(l, alpha, sum);
+        if constexpr (FP8) {      // a value is its code times its position's latent scale: the scale rides on the probability
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const f32x4 scale0 = *reinterpret_cast<const f32x4*>(&s_scale[stage][0][8 * q + 4 * h]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) p[4 * q + e] *= scale0[e];
+            }
+        }
         // The probabilities and the row's factor go to the other wavefronts through LDS: each multiplies the values it
         // owns by the probabilities of all 128 rows.
 #pragma unroll
@@ -714,7 +821,7 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
             __builtin_amdgcn_sched_barrier(0);
             static_for<NOPS / 2>([&](auto sc) __attribute__((always_inline)) {
                 constexpr int sec = decltype(sc)::value;
-                send(std::integral_constant<int, 5 + sec>{});
+                if constexpr (!FP8 || sec == 0) send(std::integral_constant<int, 5 + sec>{});
                 if constexpr (sec == 2) {      // (the first k-step's products have been issued: their operands were read at issue)
                     read_p(std::integral_constant<int, 1>{});
                     __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
@@ -735,6 +842,10 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
                 });
                 __builtin_amdgcn_sched_barrier(0);
             });
+        }
+        if constexpr (FP8) {
+            if (t + 1 < n_tiles) convert(raw_stage == NRAW - 1 ? 0 : raw_stage + 1, stage ^ 1);
+            raw_stage = raw_stage == NRAW - 1 ? 0 : raw_stage + 1;
         }
         base = base1, base1 = base2, base2 = base3;
     }
@@ -903,13 +1014,13 @@ int launch_tiles(const LatentArgs& a, bool f16, bool fp8, hipStream_t stream) {
     return hip_code(hipGetLastError());
 }
 
-// Which launches the many-heads kernel serves: 16-bit caches of the one shape it is built for with pages of a multiple
-// of 16 positions, where the caller asks for it (any number of heads: a tile of 128 rows is then 128 / heads columns of
+// Which launches the many-heads kernel serves: caches of the one shape it is built for with pages of a multiple of 16
+// positions, where the caller asks for it (any number of heads: a tile of 128 rows is then 128 / heads columns of
 // a window, which is how a prompt chunk of few heads fills it) or, left to the library, where the heads come in 128s.
 // (Nothing else decides, the batch least of all: a token's bits follow the kernel that reads it.)
 template <int R, int P>
 bool many_heads(const LatentArgs& a, bool fp8) {
-    if (!(R == 512 && P == 64 && !fp8 && a.page % 16 == 0)) return false;
+    if (!(R == 512 && P == 64 && a.page % 16 == 0)) return false;
     return a.tile_rows == kHeadsRows || (a.tile_rows == 0 && a.heads % kHeadsRows == 0);
 }
 
@@ -923,8 +1034,13 @@ int launch_shape(const LatentArgs& a, bool f16, bool fp8, int phases, hipStream_
             const int64_t merges = (int64_t)a.n_rows * u.tiles * 4;
             if (blocks > 0x7fffffff || merges > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
             if (phases != 2) {
-                if (f16) hipLaunchKernelGGL((latent_heads_kernel<R, P, true>), dim3((unsigned)blocks), dim3(256), 0, stream, u);
-                else hipLaunchKernelGGL((latent_heads_kernel<R, P, false>), dim3((unsigned)blocks), dim3(256), 0, stream, u);
+                if (fp8) {
+                    if (f16) hipLaunchKernelGGL((latent_heads_kernel<R, P, true, true>), dim3((unsigned)blocks), dim3(256), 0, stream, u);
+                    else hipLaunchKernelGGL((latent_heads_kernel<R, P, false, true>), dim3((unsigned)blocks), dim3(256), 0, stream, u);
+                } else {
+                    if (f16) hipLaunchKernelGGL((latent_heads_kernel<R, P, true, false>), dim3((unsigned)blocks), dim3(256), 0, stream, u);
+                    else hipLaunchKernelGGL((latent_heads_kernel<R, P, false, false>), dim3((unsigned)blocks), dim3(256), 0, stream, u);
+                }
                 const int bad = hip_code(hipGetLastError());
                 if (bad) return bad;
             }
@@ -980,7 +1096,7 @@ int launch_latent(const crit_pkv_latent_params* p, hipStream_t stream) {
     a.sscale = p->scale * kLog2e;
     a.tile_rows = p->tile_rows;
     if (p->tile_rows != 0 && p->tile_rows != 16 && p->tile_rows != kHeadsRows) return CRIT_PKV_E_GEOMETRY;
-    if (p->tile_rows == kHeadsRows && !(p->rank == 512 && p->rope == 64 && !fp8 && p->page % 16 == 0)) return CRIT_PKV_E_GEOMETRY;
+    if (p->tile_rows == kHeadsRows && !(p->rank == 512 && p->rope == 64 && p->page % 16 == 0)) return CRIT_PKV_E_GEOMETRY;
     a.tiles = (p->columns * p->heads + 15) / 16;
     const int64_t table_keys = (int64_t)p->table_width * p->page;
     a.max_keys = (int)(table_keys < 0x3fffffff ? table_keys : 0x3fffffff);

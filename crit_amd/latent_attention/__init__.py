@@ -83,17 +83,17 @@ def partitions(device, heads, rank, rope, page, kind=0, tile_rows=None):
 def tile_rows(heads, rank, rope, page, kind=0, asked=None):
     """The query rows a workgroup holds for this geometry, 16 or 128, which names the kernel that reads it (and a token's
     bits follow the kernel). 128, the many-heads kernel (32 x 32 matrix tiles, the cache rows by DMA into LDS, one
-    workgroup a compute unit), takes 16-bit caches of DeepSeek's shape (512, 64) with pages of a multiple of 16
+    workgroup a compute unit), takes caches of DeepSeek's shape (512, 64), 16-bit or E4M3, with pages of a multiple of 16
     positions. Heads in 128s get it unless `asked` (attend's tile_rows=) or the engine's tuned TILE_ROWS says 16: it
     reads a batch of 64 rows about twice as fast as the small tiles, and a single row twice slower (one workgroup a
     partition instead of four). With fewer heads it is there for the asking (a tile is then 128 / heads columns of a
     window: prompt chunks, prefill's packed=True); left alone they get 16, as does everything else."""
-    able = (int(rank), int(rope)) == (512, 64) and not int(kind) and int(page) % 16 == 0
+    able = (int(rank), int(rope)) == (512, 64) and int(page) % 16 == 0
     want = int(asked or _knob("TILE_ROWS", heads, rank, rope, page, kind) or 0)
     if want not in (0, 16, 128):
         raise ValueError(f"tile_rows: {want}; 16 or 128 (or 0: by the geometry)")
     if want == 128 and not able:
-        raise ValueError("tile_rows 128 reads 16-bit caches of (512, 64) with pages of a multiple of 16 positions")
+        raise ValueError("tile_rows 128 reads caches of (512, 64) with pages of a multiple of 16 positions")
     return 128 if able and (want == 128 or (want == 0 and int(heads) % 128 == 0)) else 16
 
 

@@ -410,7 +410,7 @@ int crit_pkv_step_buffers(const crit_pkv_step_params* p, void* stream);
  * the partitions only, 2 the merge only.
  * tile_rows: the query rows a workgroup holds, which decides the kernel and with it a token's bits. 16: tiles of 16 rows
  * (two a workgroup from 32 rows on), every geometry, the fastest for a few batch rows. 128: 128 rows a workgroup on
- * 32 x 32 matrix tiles, the cache rows by DMA into LDS, one workgroup a compute unit (16-bit caches of (512, 64), pages a
+ * 32 x 32 matrix tiles, the cache rows by DMA into LDS, one workgroup a compute unit (caches of (512, 64) only, pages a
  * multiple of 16 positions; anything else: CRIT_PKV_E_GEOMETRY), about twice the throughput of the other from a few
  * dozen batch rows of 128 heads on and slower below ten; with fewer heads a tile takes 128 / heads columns of a window,
  * which is how prompt chunks fill it. 0: 128 where it is allowed and the heads are a multiple of 128, else 16. The

@@ -125,7 +125,7 @@ def test_many_heads_either_kernel_matches_float64_and_a_tokens_bits_follow_the_k
     cache = Cache(512, 64, 16, [1500, 33, 2100, 600], seed=31)
     la = cache.la
     assert la.tile_rows(128, 512, 64, 16) == 128 and la.tile_rows(128, 512, 64, 16, asked=16) == 16
-    assert la.tile_rows(64, 512, 64, 16) == 16 and la.tile_rows(128, 512, 64, 24) == 16 and la.tile_rows(128, 512, 64, 16, 1) == 16
+    assert la.tile_rows(64, 512, 64, 16) == 16 and la.tile_rows(128, 512, 64, 24) == 16 and la.tile_rows(128, 512, 64, 16, 1) == 128
     assert la.tile_rows(64, 512, 64, 16, asked=128) == 128
     q = _q(16, 128, 576, 32)
     rows, starts, firsts = [0, 1, 2, 3], [0, 4, 8, 12], [1496, 29, 2096, 511]
@@ -225,6 +225,33 @@ def test_an_e4m3_cache_matches_float64_over_its_stored_values_and_keeps_a_tokens
         for c in range(4):
             alone = cache.attend(q[start + c:start + c + 1], [s], [0], [first + c], 1, scale=scale)
             assert torch.equal(alone[0], out[start + c]), (s, c)
+
+
+@pytest.mark.parametrize("scales", [2, 1])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_an_e4m3_cache_under_the_many_heads_kernel_matches_float64_and_keeps_a_tokens_bits(scales, dtype):
+    # 128 heads over codes: the many-heads kernel converts each tile in LDS, one step ahead; rows that end inside a tile,
+    # a page and a piece, one tile long and many pieces long; a packed prompt chunk of few heads on the same kernel.
+    cache = Cache(512, 64, 16, [1500, 33, 2100, 600], seed=41, dtype=torch.float8_e4m3fn, scales=scales)
+    la = cache.la
+    assert la.tile_rows(128, 512, 64, 16, 1) == 128
+    q = _q(16, 128, 576, 42, dtype)
+    rows, starts, firsts = [0, 1, 2, 3], [0, 4, 8, 12], [1496, 29, 2096, 511]
+    sinks = torch.randn(128, generator=torch.Generator().manual_seed(43)).to(dev)
+    lse = torch.empty(16, 128, device=dev)
+    scale = 192 ** -0.5
+    together = cache.attend(q, rows, starts, firsts, 4, scale=scale, lse=lse, sinks=sinks)
+    for s_, start, first in zip(rows, starts, firsts):
+        cache.check(q, together, lse, s_, start, first, 4, scale, sinks)
+        for c in (0, 3):
+            alone = cache.attend(q[start + c:start + c + 1], [s_], [0], [first + c], 1, scale=scale, sinks=sinks)
+            assert torch.equal(alone[0], together[start + c]), (s_, c)
+    small = cache.attend(q, rows, starts, firsts, 4, scale=scale, sinks=sinks, tile_rows=16)
+    torch.testing.assert_close(small.float(), together.float(), atol=8e-3, rtol=2e-2)      # the same attention, other sums
+    few = _q(40, 16, 576, 44, dtype)
+    lse = torch.empty(40, 16, device=dev)
+    packed = la.prefill(few, cache.cache, cache.tables[2], 2060, 16, rank=512, scale=scale, scales=cache.scales, lse=lse, packed=True)
+    cache.check(few, packed, lse, 2, 0, 2060, 40, scale)
 
 
 @pytest.mark.parametrize("rank,rope,heads,page", [(512, 64, 16, 64), (512, 64, 128, 16), (128, 32, 20, 16)])

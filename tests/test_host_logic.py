@@ -10,10 +10,10 @@ def test_latent_partitions_follow_the_rule_or_the_engines_tuning():
     held = dict(la._CUS)
     la._CUS[0] = 256                                   # an MI355X's compute units (no device is asked)
     try:
-        # (128 heads of a 16-bit (512, 64) cache: the many-heads kernel, a workgroup a compute unit; an E4M3 cache, pages
-        # of no multiple of 16 or the small tiles asked for: the rule of the small tiles)
+        # (128 heads of a (512, 64) cache, 16-bit or E4M3: the many-heads kernel, a workgroup a compute unit; pages of no
+        # multiple of 16, another shape or the small tiles asked for: the rule of the small tiles)
         assert [la.partitions(device, h, 512, 64, 64) for h in (1, 16, 32, 64, 128)] == [64, 64, 64, 32, 8]
-        assert la.partitions(device, 128, 512, 64, 64, 1) == 16 and la.partitions(device, 128, 512, 64, 24) == 16
+        assert la.partitions(device, 128, 512, 64, 64, 1) == 8 and la.partitions(device, 128, 512, 64, 24) == 16
         assert la.partitions(device, 128, 512, 64, 64, 0, 16) == 16 and la.partitions(device, 128, 256, 64, 64) == 16
         assert la.tile_rows(128, 512, 64, 64) == 128 and la.tile_rows(256, 512, 64, 16) == 128
         assert la.tile_rows(64, 512, 64, 64) == 16 and la.tile_rows(128, 512, 64, 64, asked=16) == 16
