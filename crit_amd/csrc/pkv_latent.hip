@@ -1109,6 +1109,8 @@ int launch_latent(const crit_pkv_latent_params* p, hipStream_t stream) {
     if (p->rank == RANK && p->rope == ROPE) return launch_shape<RANK, ROPE>(a, f16, fp8, p->phases , stream);
     PKV_LATENT(512, 64) PKV_LATENT(256, 64) PKV_LATENT(128, 64) PKV_LATENT(128, 32) PKV_LATENT(64, 64) PKV_LATENT(64, 32)
     PKV_LATENT(1024, 64) PKV_LATENT(512, 128)
+    PKV_LATENT(1024, 32) PKV_LATENT(1024, 128) PKV_LATENT(1024, 256) PKV_LATENT(512, 32) PKV_LATENT(512, 256) PKV_LATENT(256, 32)
+    PKV_LATENT(256, 128) PKV_LATENT(256, 256) PKV_LATENT(128, 128) PKV_LATENT(128, 256) PKV_LATENT(64, 128) PKV_LATENT(64, 256)
 #undef PKV_LATENT
     return CRIT_PKV_E_GEOMETRY;
 }

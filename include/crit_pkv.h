@@ -406,8 +406,8 @@ int crit_pkv_step_buffers(const crit_pkv_step_params* p, void* stream);
  * partition order, the sink logit (sinks [heads], natural log, -inf: none) folded in last; lse [tokens][heads] the
  * natural log-sum-exp (the sink counted). cache_dtype: 0 BF16, 1 FP16 (q in the same type), 2 E4M3 with `scales`
  * [pages][page][scales_per_row] FP32 (2: the latent's and the rotary key's, 1: one for the row) and BF16 or FP16 q.
- * (rank, rope) is one of (1024, 64), (512, 128), (512, 64), (256, 64), (128, 64), (128, 32), (64, 64), (64, 32). phases: 0 both launches, 1
- * the partitions only, 2 the merge only.
+ * rank is one of 64, 128, 256, 512, 1024 and rope one of 32, 64, 128, 256 (anything else: CRIT_PKV_E_GEOMETRY). phases:
+ * 0 both launches, 1 the partitions only, 2 the merge only.
  * tile_rows: the query rows a workgroup holds, which decides the kernel and with it a token's bits. 16: tiles of 16 rows
  * (two a workgroup from 32 rows on), every geometry, the fastest for a few batch rows. 128: 128 rows a workgroup on
  * 32 x 32 matrix tiles, the cache rows by DMA into LDS, one workgroup a compute unit (caches of (512, 64) only, pages a

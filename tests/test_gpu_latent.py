@@ -74,7 +74,10 @@ def _q(tokens, heads, width, seed, dtype=torch.bfloat16):
 
 @pytest.mark.parametrize("rank,rope,heads,page", [(512, 64, 16, 64), (512, 64, 128, 16), (256, 64, 8, 32), (128, 32, 20, 16),
                                                  (64, 32, 3, 48), (128, 64, 5, 16), (64, 64, 40, 16), (1024, 64, 16, 64),
-                                                 (512, 128, 24, 16)])
+                                                 (512, 128, 24, 16), (1024, 32, 2, 16), (1024, 128, 4, 32), (1024, 256, 16, 16),
+                                                 (512, 32, 16, 64), (512, 256, 3, 16), (256, 32, 6, 16), (256, 128, 8, 32),
+                                                 (256, 256, 1, 16), (128, 128, 5, 16), (128, 256, 20, 16), (64, 128, 2, 48),
+                                                 (64, 256, 7, 16)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_windows_match_float64_latent_attention(rank, rope, heads, page, dtype):
     cache = Cache(rank, rope, page, [130, 64, 1, 517], dtype=dtype)
@@ -212,11 +215,12 @@ def test_what_it_cannot_read_is_refused():
         cache.attend(q, [0], [0], [5], 1, piece=48)
 
 
+@pytest.mark.parametrize("rank,rope", [(512, 64), (64, 32), (128, 32), (256, 128), (1024, 256), (64, 256)])
 @pytest.mark.parametrize("scales", [2, 1])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_an_e4m3_cache_matches_float64_over_its_stored_values_and_keeps_a_tokens_bits(scales, dtype):
-    cache = Cache(512, 64, 64, [130, 517], seed=6, dtype=torch.float8_e4m3fn, scales=scales)
-    q = _q(8, 16, 576, 8, dtype)
+def test_an_e4m3_cache_matches_float64_over_its_stored_values_and_keeps_a_tokens_bits(scales, dtype, rank, rope):
+    cache = Cache(rank, rope, 64, [130, 517], seed=6, dtype=torch.float8_e4m3fn, scales=scales)
+    q = _q(8, 16, rank + rope, 8, dtype)
     lse = torch.empty(8, 16, device=dev)
     scale = 192 ** -0.5
     out = cache.attend(q, [0, 1], [0, 4], [126, 513], 4, scale=scale, lse=lse)
