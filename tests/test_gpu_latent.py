@@ -452,18 +452,21 @@ def test_two_owners_launch_on_two_streams_without_sharing_partials_and_an_outgro
         pk.release("b")
 
 
-def test_many_heads_units_longer_than_the_lanes_hold_tiles_for_and_rows_beyond_the_ranked_launches():
+@pytest.mark.parametrize("coded", [0, 2, 1])
+def test_many_heads_units_longer_than_the_lanes_hold_tiles_for_and_rows_beyond_the_ranked_launches(coded):
     # A unit of more than 64 tiles of 32 positions refills the lanes' table of tiles on the way (one partition over
     # 9,000 positions is 282 tiles); a launch of more than 64 batch rows keeps the caller's order instead of ranking the
-    # rows by length, and one of fewer than 16 deals (row, partition) pairs, not whole rows, to the XCDs.
-    long = Cache(512, 64, 64, [9000], seed=51)
+    # rows by length, and one of fewer than 16 deals (row, partition) pairs, not whole rows, to the XCDs. 16-bit rows,
+    # and E4M3 rows with two scales a position or one.
+    kind = dict(dtype=torch.float8_e4m3fn, scales=coded) if coded else {}
+    long = Cache(512, 64, 64, [9000], seed=51, **kind)
     q = _q(1, 128, 576, 52)
     lse = torch.empty(1, 128, device=dev)
-    for parts in (1, 3):
-        out = long.attend(q, [0], [0], [8999], 1, lse=lse, partitions=parts, piece=512)
+    for parts, piece in ((1, 512), (3, 512), (5, 96)):
+        out = long.attend(q, [0], [0], [8999], 1, lse=lse, partitions=parts, piece=piece)
         long.check(q, out, lse, 0, 0, 8999, 1, 576 ** -0.5)
     lengths = [40 + 37 * (i % 9) for i in range(70)]
-    many = Cache(512, 64, 16, lengths, seed=53)
+    many = Cache(512, 64, 16, lengths, seed=53, **kind)
     q = _q(70, 128, 576, 54)
     rows, starts, firsts = list(range(70)), list(range(70)), [n - 1 for n in lengths]
     together = many.attend(q, rows, starts, firsts, 1)
