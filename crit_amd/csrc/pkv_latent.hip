@@ -417,6 +417,11 @@ PKV_DEV void score_product(f32x16& c, const u32x4& a, const u32x4& b) {
     if constexpr (F16) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
     else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
 }
+template <bool F16>
+PKV_DEV void score_product_first(f32x16& c, const u32x4& a, const u32x4& b) {      // (a chain's first: onto zeros)
+    if constexpr (F16) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+    else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+}
 template <int OFFSET>
 PKV_DEV void lds_read16(u32x4& to, uint32_t at) {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(to) : "v"(at), "n"(OFFSET));
@@ -598,7 +603,7 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(bq[ks].x), "v"(bq[ks].y), "v"(bq[ks].z), "v"(bq[ks].w));
     // (the queries are waited for here, with the first tile; the next two tiles go out behind them)
-    int base1 = issue(1, 1), base2 = issue(2, 2);
+    int base1 = issue(1, 1), base2 = FP8 ? issue(2, 2) : 0;
     // E4M3: the wavefront's rows of raw tile `from`, as 16-bit values in tile `to` (a lane: 16 codes a turn).
     auto convert = [&](int from, int to) __attribute__((always_inline)) {
         if constexpr (FP8) {
@@ -650,161 +655,332 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[vb][hb][v] = 0.0f;
 
-    for (int t = 0; t < n_tiles; ++t) {
-        const int stage = t & (NSTAGE - 1);
-        // 16-bit: the tile's loads of this wavefront have landed, those of the next two may be in flight. E4M3: the next
-        // tile's have (it is converted at the end of this step), the one after may be in flight.
-        wait_loads<FP8 ? LPT : 2 * LPT>();
-        lds_barrier();              // everybody's have, and nobody reads the tile before any more, nor the last probabilities
-        const int base3 = plan(t + 3, FP8 ? raw_stage : (t + 3) & (NSTAGE - 1));
-        const uint8_t* tile = ring + stage * TILE;
-        // Operand addresses inside a tile (see the layout above), from the opaque copy of the number of the lane.
-        asm volatile("" : "+v"(ln));
-        const int n32 = ln & 31, h = ln >> 5;
-        const int fk = 4 * (n32 & 3) + ((n32 >> 2) & 3);
-        const uint32_t k_lane = (uint32_t)(n32 * (R * 2) + 16 * ((fk ^ h) & 15));                       // ^ 32 i for k-step i of the latent
-        const uint32_t t_lane = (uint32_t)(MAIN + n32 * (P * 2) + 16 * ((h ^ (n32 >> 1)) & 7));         // ^ 32 i for k-step i of the rotary key
-        // The values: the wavefront's 128 of them. For block vb of 32 values and k-step g of 16 positions the lane's operand
-        // is positions 16 g + 8 h + 4 e + (0 .. 3), e = 0, 1: two transposing reads, lane 4 j + c of a 16-lane group pointing
-        // at position j's values 4 c .. 4 c + 3.
-        const int i16 = ln & 15, mh = (ln >> 4) & 1;
-        const uint32_t v_lane = (uint32_t)((8 * h + (i16 >> 2)) * (R * 2) + 256 * wave + 8 * (i16 & 1));
-        const uint32_t v_low = (uint32_t)(2 * mh + ((i16 & 3) >> 1));      // the chunk's low two bits, ^ ((2 h + e) & 3)
-        uint8_t* p_mine = s_prob + (wave * 32 + n32) * 64 + 8 * h;           // + 16 (q ^ p_turn): positions 8 q + 4 h .. + 3
-        const uint32_t p_turn = (uint32_t)((n32 >> 2) & 3);
-        const uint8_t* p_read = s_prob + n32 * 64;                           // + 2048 hb + 16 ((2 g + h) ^ p_turn)
+    if constexpr (FP8) {
+        for (int t = 0; t < n_tiles; ++t) {
+            const int stage = t & (NSTAGE - 1);
+            // 16-bit: the tile's loads of this wavefront have landed, those of the next two may be in flight. E4M3: the next
+            // tile's have (it is converted at the end of this step), the one after may be in flight.
+            wait_loads<FP8 ? LPT : 2 * LPT>();
+            lds_barrier();              // everybody's have, and nobody reads the tile before any more, nor the last probabilities
+            const int base3 = plan(t + 3, FP8 ? raw_stage : (t + 3) & (NSTAGE - 1));
+            const uint8_t* tile = ring + stage * TILE;
+            // Operand addresses inside a tile (see the layout above), from the opaque copy of the number of the lane.
+            asm volatile("" : "+v"(ln));
+            const int n32 = ln & 31, h = ln >> 5;
+            const int fk = 4 * (n32 & 3) + ((n32 >> 2) & 3);
+            const uint32_t k_lane = (uint32_t)(n32 * (R * 2) + 16 * ((fk ^ h) & 15));                       // ^ 32 i for k-step i of the latent
+            const uint32_t t_lane = (uint32_t)(MAIN + n32 * (P * 2) + 16 * ((h ^ (n32 >> 1)) & 7));         // ^ 32 i for k-step i of the rotary key
+            // The values: the wavefront's 128 of them. For block vb of 32 values and k-step g of 16 positions the lane's operand
+            // is positions 16 g + 8 h + 4 e + (0 .. 3), e = 0, 1: two transposing reads, lane 4 j + c of a 16-lane group pointing
+            // at position j's values 4 c .. 4 c + 3.
+            const int i16 = ln & 15, mh = (ln >> 4) & 1;
+            const uint32_t v_lane = (uint32_t)((8 * h + (i16 >> 2)) * (R * 2) + 256 * wave + 8 * (i16 & 1));
+            const uint32_t v_low = (uint32_t)(2 * mh + ((i16 & 3) >> 1));      // the chunk's low two bits, ^ ((2 h + e) & 3)
+            uint8_t* p_mine = s_prob + (wave * 32 + n32) * 64 + 8 * h;           // + 16 (q ^ p_turn): positions 8 q + 4 h .. + 3
+            const uint32_t p_turn = (uint32_t)((n32 >> 2) & 3);
+            const uint8_t* p_read = s_prob + n32 * 64;                           // + 2048 hb + 16 ((2 g + h) ^ p_turn)
 
-        // -- scores of the wavefront's 32 rows: 36 products in two chains (even and odd ones: a product every 32 clocks
-        // cannot wait for the one before it), the operand of each read RING - 1 products ahead, five of the tile's loads
-        // sent out in between
-        // (E4M3: the rotary keys' products, which take a scale of their own, in a chain of their own, every ninth)
-        f32x16 s, s2, s3;
+            // -- scores of the wavefront's 32 rows: 36 products in two chains (even and odd ones: a product every 32 clocks
+            // cannot wait for the one before it), the operand of each read RING - 1 products ahead, five of the tile's loads
+            // sent out in between
+            // (E4M3: the rotary keys' products, which take a scale of their own, in a chain of their own, every ninth)
+            f32x16 s, s2, s3;
+            {
+                constexpr int RING = 6;
+                u32x4 ka[RING];
+                const uint32_t tile_at = (uint32_t)(uintptr_t)tile;
+                // the latent's k-steps in the order 0, 8, 16, 24, 1, 9, ...: four share an address register
+                uint32_t k_at = 0;
+                auto read_k = [&](auto ic) __attribute__((always_inline)) {
+                    constexpr int i = decltype(ic)::value;
+                    constexpr bool rotary = FP8 ? i % 9 == 8 : i >= KSL;
+                    constexpr int at = FP8 ? (rotary ? i / 9 : i - i / 9) : (rotary ? i - KSL : i);
+                    if constexpr (!rotary) {
+                        constexpr int lo = at / 4, hi = at % 4;      // k-step lo + 8 hi
+                        if constexpr (hi == 0) k_at = tile_at + (k_lane ^ (uint32_t)(32 * lo));
+                        lds_read16<256 * hi>(ka[i % RING], k_at);
+                    } else {
+                        lds_read16<0>(ka[i % RING], tile_at + (t_lane ^ (uint32_t)(32 * at)));
+                    }
+                };
+                static_for<RING - 1>([&](auto ic) __attribute__((always_inline)) { read_k(ic); });
+                static_for<KS>([&](auto ic) __attribute__((always_inline)) {
+                    constexpr int i = decltype(ic)::value;
+                    if constexpr (i + RING - 1 < KS) read_k(std::integral_constant<int, i + RING - 1>{});
+                    if constexpr (i % 8 == 2) send(std::integral_constant<int, i / 8>{});
+                    constexpr int ahead = KS - 1 - i < RING - 1 ? KS - 1 - i : RING - 1;
+                    lds_arrived<ahead>(ka[i % RING]);
+                    constexpr bool rotary = FP8 ? i % 9 == 8 : i >= KSL;
+                    constexpr int at = FP8 ? (rotary ? i / 9 : i - i / 9) : (rotary ? i - KSL : i);
+                    constexpr int ks = rotary ? KSL + at : at / 4 + 8 * (at % 4);
+                    // (a chain's first product onto zeros)
+                    if constexpr (FP8 && rotary && at == 0) score_product_first<F16>(s3, ka[i % RING], bq[ks]);
+                    else if constexpr (FP8 && rotary) score_product<F16>(s3, ka[i % RING], bq[ks]);
+                    else if constexpr (i == 0) score_product_first<F16>(s, ka[i % RING], bq[ks]);
+                    else if constexpr (i == 1) score_product_first<F16>(s2, ka[i % RING], bq[ks]);
+                    else if constexpr ((FP8 ? at : i) % 2 == 0) score_product<F16>(s, ka[i % RING], bq[ks]);
+                    else score_product<F16>(s2, ka[i % RING], bq[ks]);
+                });
+                // (the products' results are read by vector instructions next)
+                if constexpr (FP8) asm volatile("s_nop 15\n\ts_nop 15" : "+v"(s), "+v"(s2), "+v"(s3));
+                else asm volatile("s_nop 15\n\ts_nop 15" : "+v"(s), "+v"(s2));
+            }
+            // -- softmax of the lane's row over its 16 positions of the tile (the other half-wave holds the other 16): the
+            // lane holds positions 8 (v / 4) + 4 h + v % 4
+            const bool masked = base + 32 > unmasked;      // (the same for the whole wavefront)
+            float x[16];
+            if constexpr (FP8) {      // (the scales of the lane's positions: the latent's, the rotary key's)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) s[v] = 0.0f, s2[v] = 0.0f;
-        if constexpr (FP8) {
+                for (int q = 0; q < 4; ++q) {
+                    const f32x4 scale0 = *reinterpret_cast<const f32x4*>(&s_scale[stage][0][8 * q + 4 * h]);
+                    const f32x4 scale1 = *reinterpret_cast<const f32x4*>(&s_scale[stage][1][8 * q + 4 * h]);
 #pragma unroll
-            for (int v = 0; v < 16; ++v) s3[v] = 0.0f;
+                    for (int e = 0; e < 4; ++e)
+                        x[4 * q + e] = __builtin_fmaf(s[4 * q + e] + s2[4 * q + e], scale0[e], s3[4 * q + e] * scale1[e]) * a.sscale;
+                }
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) x[v] = (s[v] + s2[v]) * a.sscale;
+            }
+            if (masked) {
+                const int seen = min(lim, n_keys - 1) - base - 4 * h;      // position 8 (v / 4) + v % 4 of the lane's is seen up to this
+#pragma unroll
+                for (int v = 0; v < 16; ++v) x[v] = 8 * (v / 4) + v % 4 <= seen ? x[v] : -INFINITY;
+            }
+            float top = x[0];
+#pragma unroll
+            for (int v = 1; v < 16; ++v) top = __builtin_fmaxf(top, x[v]);
+            {
+                const int w = (int)f2u(top);
+                const auto both = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+                top = __builtin_fmaxf(u2f((uint32_t)both[0]), u2f((uint32_t)both[1]));
+            }
+            const float m_new = top > m + kLazyHeads ? top : m;      // (a NaN score: the comparison fails, the NaN reaches the sum)
+            const float sub = m_new == -INFINITY ? 0.0f : m_new;
+            const float alpha = exp2_fast(m - sub);
+            m = m_new;
+            float p[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) p[v] = exp2_fast(x[v] - sub);
+            const float sum = (((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]))) +
+                              (((p[8] + p[9]) + (p[10] + p[11])) + ((p[12] + p[13]) + (p[14] + p[15])));
+            l = __builtin_fmaf(l, alpha, sum);
+            if constexpr (FP8) {      // a value is its code times its position's latent scale: the scale rides on the probability
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const f32x4 scale0 = *reinterpret_cast<const f32x4*>(&s_scale[stage][0][8 * q + 4 * h]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) p[4 * q + e] *= scale0[e];
+                }
+            }
+            // The probabilities and the row's factor go to the other wavefronts through LDS: each multiplies the values it
+            // owns by the probabilities of all 128 rows.
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                *reinterpret_cast<u32x2*>(p_mine + 16 * ((uint32_t)q ^ p_turn)) =
+                    u32x2{pair16<F16>(p[4 * q], p[4 * q + 1]), pair16<F16>(p[4 * q + 2], p[4 * q + 3])};
+            if (h == 0) s_alpha[wave * 32 + n32] = alpha;
+            lds_barrier();
+            float factor[4];
+#pragma unroll
+            for (int hb = 0; hb < 4; ++hb) factor[hb] = s_alpha[hb * 32 + n32];
+            if (__ballot(factor[0] != 1.0f || factor[1] != 1.0f || factor[2] != 1.0f || factor[3] != 1.0f) != 0ull) {
+                // (x 1 is exact: the accumulators move only when some row's reference did; spelled out so that they stay
+                // where the matrix pipe keeps them, and the last product that wrote them is a whole score phase back)
+                static_for<16>([&](auto bc) __attribute__((always_inline)) {
+                    constexpr int vb = decltype(bc)::value / 4, hb = decltype(bc)::value % 4;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        float e = acc[vb][hb][v], tmp;
+                        asm volatile("v_accvgpr_read_b32 %0, %1\n\tv_mul_f32 %0, %0, %2\n\tv_accvgpr_write_b32 %1, %0" : "=&v"(tmp), "+a"(e) : "v"(factor[hb]));
+                        acc[vb][hb][v] = e;
+                    }
+                });
+            }
+            // -- values: operand i = (k-step g = i / 4, block vb = i % 4) of V^T against the four row blocks' probabilities
+            {
+                constexpr int RING = 4, NOPS = 8;
+                u32x4 pb[4];      // the four row blocks' probabilities of the k-step being multiplied
+                u32x2 va[RING][2];
+                auto read_p = [&](auto gc) __attribute__((always_inline)) {
+                    constexpr int g = decltype(gc)::value;
+#pragma unroll
+                    for (int hb = 0; hb < 4; ++hb)
+                        pb[hb] = *reinterpret_cast<const u32x4*>(p_read + 2048 * hb + 16 * ((uint32_t)(2 * g + h) ^ p_turn));
+                };
+                read_p(std::integral_constant<int, 0>{});
+                auto read_v = [&](auto ic) __attribute__((always_inline)) {
+                    constexpr int i = decltype(ic)::value;
+                    constexpr int g = i / 4, vb = i % 4;
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) {
+                        const uint32_t at = v_lane + 64u * (uint32_t)(vb ^ (i16 >> 2)) + 16u * (v_low ^ (uint32_t)((2 * h + e) & 3));
+                        va[i % RING][e] = lds_transposed(tile + at + (16 * g + 4 * e) * (R * 2));
+                    }
+                };
+                static_for<RING - 1>([&](auto ic) __attribute__((always_inline)) { read_v(ic); });
+                __builtin_amdgcn_sched_group_barrier(0x100, 4 + 2 * (RING - 1), 0);
+                __builtin_amdgcn_sched_barrier(0);
+                static_for<NOPS / 2>([&](auto sc) __attribute__((always_inline)) {
+                    constexpr int sec = decltype(sc)::value;
+                    if constexpr (!FP8 || sec == 0) send(std::integral_constant<int, 5 + sec>{});
+                    if constexpr (sec == 2) {      // (the first k-step's products have been issued: their operands were read at issue)
+                        read_p(std::integral_constant<int, 1>{});
+                        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    static_for<2>([&](auto jc) __attribute__((always_inline)) {
+                        constexpr int i = 2 * sec + decltype(jc)::value;
+                        constexpr int g = i / 4, vb = i % 4;
+                        if constexpr (i + RING - 1 < NOPS) read_v(std::integral_constant<int, i + RING - 1>{});
+                        const u32x4 av = {va[i % RING][0].x, va[i % RING][0].y, va[i % RING][1].x, va[i % RING][1].y};
+#pragma unroll
+                        for (int hb = 0; hb < 4; ++hb) acc[vb][hb] = mfma_32<F16>(av, pb[hb], acc[vb][hb]);
+                    });
+                    static_for<2>([&](auto jc) __attribute__((always_inline)) {
+                        constexpr int i = 2 * sec + decltype(jc)::value;
+                        if constexpr (i + RING - 1 < NOPS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                    });
+                    __builtin_amdgcn_sched_barrier(0);
+                });
+            }
+            if constexpr (FP8) {
+                if (t + 1 < n_tiles) convert(raw_stage == NRAW - 1 ? 0 : raw_stage + 1, stage ^ 1);
+                raw_stage = raw_stage == NRAW - 1 ? 0 : raw_stage + 1;
+            }
+            base = base1, base1 = base2, base2 = base3;
         }
-        {
-            constexpr int RING = FP8 ? 5 : 6;
+    } else {
+        // 16-bit rows: the same operations on the same numbers in a pipeline of one step: a step's value products go out
+        // one step later, together with the next step's softmax, whose vector work then runs in their shadow instead of
+        // with the matrix pipe idle. A tile therefore stays in the ring one step longer, and two tiles are in flight
+        // instead of three. Barriers: A, the tile has landed and the last probabilities are written; B, everybody has read
+        // those probabilities, the next may be written.
+        struct Lane {
+            int h, i16;
+            uint32_t k_lane, t_lane, v_lane, v_low, p_turn;
+            uint8_t* p_mine;
+            const uint8_t* p_read;
+        };
+        auto lane_now = [&]() __attribute__((always_inline)) -> Lane {
+            asm volatile("" : "+v"(ln));
+            Lane L;
+            const int n32 = ln & 31, h = ln >> 5;
+            const int fk = 4 * (n32 & 3) + ((n32 >> 2) & 3);
+            L.h = h, L.i16 = ln & 15;
+            L.k_lane = (uint32_t)(n32 * (R * 2) + 16 * ((fk ^ h) & 15));
+            L.t_lane = (uint32_t)(MAIN + n32 * (P * 2) + 16 * ((h ^ (n32 >> 1)) & 7));
+            const int mh = (ln >> 4) & 1;
+            L.v_lane = (uint32_t)((8 * h + (L.i16 >> 2)) * (R * 2) + 256 * wave + 8 * (L.i16 & 1));
+            L.v_low = (uint32_t)(2 * mh + ((L.i16 & 3) >> 1));
+            L.p_mine = s_prob + (wave * 32 + n32) * 64 + 8 * h;
+            L.p_turn = (uint32_t)((n32 >> 2) & 3);
+            L.p_read = s_prob + n32 * 64;
+            return L;
+        };
+        f32x16 s, s2;
+        auto scores = [&](const uint8_t* tile, const Lane& L) __attribute__((always_inline)) {
+            constexpr int RING = 6;
             u32x4 ka[RING];
             const uint32_t tile_at = (uint32_t)(uintptr_t)tile;
-            // the latent's k-steps in the order 0, 8, 16, 24, 1, 9, ...: four share an address register
             uint32_t k_at = 0;
             auto read_k = [&](auto ic) __attribute__((always_inline)) {
                 constexpr int i = decltype(ic)::value;
-                constexpr bool rotary = FP8 ? i % 9 == 8 : i >= KSL;
-                constexpr int at = FP8 ? (rotary ? i / 9 : i - i / 9) : (rotary ? i - KSL : i);
-                if constexpr (!rotary) {
-                    constexpr int lo = at / 4, hi = at % 4;      // k-step lo + 8 hi
-                    if constexpr (hi == 0) k_at = tile_at + (k_lane ^ (uint32_t)(32 * lo));
+                if constexpr (i < KSL) {
+                    constexpr int lo = i / 4, hi = i % 4;      // k-step lo + 8 hi
+                    if constexpr (hi == 0) k_at = tile_at + (L.k_lane ^ (uint32_t)(32 * lo));
                     lds_read16<256 * hi>(ka[i % RING], k_at);
                 } else {
-                    lds_read16<0>(ka[i % RING], tile_at + (t_lane ^ (uint32_t)(32 * at)));
+                    lds_read16<0>(ka[i % RING], tile_at + (L.t_lane ^ (uint32_t)(32 * (i - KSL))));
                 }
             };
             static_for<RING - 1>([&](auto ic) __attribute__((always_inline)) { read_k(ic); });
-            if constexpr (FP8) asm volatile("s_nop 1" : "+v"(s), "+v"(s2), "+v"(s3));
-            else asm volatile("s_nop 1" : "+v"(s), "+v"(s2));
             static_for<KS>([&](auto ic) __attribute__((always_inline)) {
                 constexpr int i = decltype(ic)::value;
                 if constexpr (i + RING - 1 < KS) read_k(std::integral_constant<int, i + RING - 1>{});
                 if constexpr (i % 8 == 2) send(std::integral_constant<int, i / 8>{});
                 constexpr int ahead = KS - 1 - i < RING - 1 ? KS - 1 - i : RING - 1;
                 lds_arrived<ahead>(ka[i % RING]);
-                constexpr bool rotary = FP8 ? i % 9 == 8 : i >= KSL;
-                constexpr int at = FP8 ? (rotary ? i / 9 : i - i / 9) : (rotary ? i - KSL : i);
-                constexpr int ks = rotary ? KSL + at : at / 4 + 8 * (at % 4);
-                if constexpr (FP8 && rotary) score_product<F16>(s3, ka[i % RING], bq[ks]);
-                else if constexpr ((FP8 ? at : i) % 2 == 0) score_product<F16>(s, ka[i % RING], bq[ks]);
+                constexpr int ks = i < KSL ? i / 4 + 8 * (i % 4) : i;
+                if constexpr (i == 0) score_product_first<F16>(s, ka[i % RING], bq[ks]);
+                else if constexpr (i == 1) score_product_first<F16>(s2, ka[i % RING], bq[ks]);
+                else if constexpr (i % 2 == 0) score_product<F16>(s, ka[i % RING], bq[ks]);
                 else score_product<F16>(s2, ka[i % RING], bq[ks]);
             });
-            // (the products' results are read by vector instructions next)
-            if constexpr (FP8) asm volatile("s_nop 15\n\ts_nop 15" : "+v"(s), "+v"(s2), "+v"(s3));
-            else asm volatile("s_nop 15\n\ts_nop 15" : "+v"(s), "+v"(s2));
-        }
-        // -- softmax of the lane's row over its 16 positions of the tile (the other half-wave holds the other 16): the
-        // lane holds positions 8 (v / 4) + 4 h + v % 4
-        const bool masked = base + 32 > unmasked;      // (the same for the whole wavefront)
-        float x[16];
-        if constexpr (FP8) {      // (the scales of the lane's positions: the latent's, the rotary key's)
+            asm volatile("s_nop 15\n\ts_nop 15" : "+v"(s), "+v"(s2));
+        };
+        // The softmax of a step in four parts (each goes behind a quarter of the value products), on x in place.
+        float x[16], alpha = 1.0f, sub = 0.0f;
+        auto soften = [&](auto part_c, auto mask_c, int base, const Lane& L) __attribute__((always_inline)) {
+            constexpr int part = decltype(part_c)::value;
+            if constexpr (part == 0) {
+                if constexpr (decltype(mask_c)::value) {
+                    const int seen = min(lim, n_keys - 1) - base - 4 * L.h;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const f32x4 scale0 = *reinterpret_cast<const f32x4*>(&s_scale[stage][0][8 * q + 4 * h]);
-                const f32x4 scale1 = *reinterpret_cast<const f32x4*>(&s_scale[stage][1][8 * q + 4 * h]);
+                    for (int v = 0; v < 16; ++v) {
+                        const float y = (s[v] + s2[v]) * a.sscale;
+                        x[v] = 8 * (v / 4) + v % 4 <= seen ? y : -INFINITY;
+                    }
+                } else {
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    x[4 * q + e] = __builtin_fmaf(s[4 * q + e] + s2[4 * q + e], scale0[e], s3[4 * q + e] * scale1[e]) * a.sscale;
-            }
-        } else {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) x[v] = (s[v] + s2[v]) * a.sscale;
-        }
-        if (masked) {
-            const int seen = min(lim, n_keys - 1) - base - 4 * h;      // position 8 (v / 4) + v % 4 of the lane's is seen up to this
-#pragma unroll
-            for (int v = 0; v < 16; ++v) x[v] = 8 * (v / 4) + v % 4 <= seen ? x[v] : -INFINITY;
-        }
-        float top = x[0];
-#pragma unroll
-        for (int v = 1; v < 16; ++v) top = __builtin_fmaxf(top, x[v]);
-        {
-            const int w = (int)f2u(top);
-            const auto both = __builtin_amdgcn_permlane32_swap(w, w, false, false);
-            top = __builtin_fmaxf(u2f((uint32_t)both[0]), u2f((uint32_t)both[1]));
-        }
-        const float m_new = top > m + kLazyHeads ? top : m;      // (a NaN score: the comparison fails, the NaN reaches the sum)
-        const float sub = m_new == -INFINITY ? 0.0f : m_new;
-        const float alpha = exp2_fast(m - sub);
-        m = m_new;
-        float p[16];
-#pragma unroll
-        for (int v = 0; v < 16; ++v) p[v] = exp2_fast(x[v] - sub);
-        const float sum = (((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]))) +
-                          (((p[8] + p[9]) + (p[10] + p[11])) + ((p[12] + p[13]) + (p[14] + p[15])));
-        l = __builtin_fmaf(l, alpha, sum);
-        if constexpr (FP8) {      // a value is its code times its position's latent scale: the scale rides on the probability
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const f32x4 scale0 = *reinterpret_cast<const f32x4*>(&s_scale[stage][0][8 * q + 4 * h]);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) p[4 * q + e] *= scale0[e];
-            }
-        }
-        // The probabilities and the row's factor go to the other wavefronts through LDS: each multiplies the values it
-        // owns by the probabilities of all 128 rows.
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-            *reinterpret_cast<u32x2*>(p_mine + 16 * ((uint32_t)q ^ p_turn)) =
-                u32x2{pair16<F16>(p[4 * q], p[4 * q + 1]), pair16<F16>(p[4 * q + 2], p[4 * q + 3])};
-        if (h == 0) s_alpha[wave * 32 + n32] = alpha;
-        lds_barrier();
-        float factor[4];
-#pragma unroll
-        for (int hb = 0; hb < 4; ++hb) factor[hb] = s_alpha[hb * 32 + n32];
-        if (__ballot(factor[0] != 1.0f || factor[1] != 1.0f || factor[2] != 1.0f || factor[3] != 1.0f) != 0ull) {
-            // (x 1 is exact: the accumulators move only when some row's reference did; spelled out so that they stay
-            // where the matrix pipe keeps them, and the last product that wrote them is a whole score phase back)
-            static_for<16>([&](auto bc) __attribute__((always_inline)) {
-                constexpr int vb = decltype(bc)::value / 4, hb = decltype(bc)::value % 4;
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    float e = acc[vb][hb][v], tmp;
-                    asm volatile("v_accvgpr_read_b32 %0, %1\n\tv_mul_f32 %0, %0, %2\n\tv_accvgpr_write_b32 %1, %0" : "=&v"(tmp), "+a"(e) : "v"(factor[hb]));
-                    acc[vb][hb][v] = e;
+                    for (int v = 0; v < 16; ++v) x[v] = (s[v] + s2[v]) * a.sscale;
                 }
-            });
-        }
-        // -- values: operand i = (k-step g = i / 4, block vb = i % 4) of V^T against the four row blocks' probabilities
-        {
+            } else if constexpr (part == 1) {
+                float top = x[0];
+#pragma unroll
+                for (int v = 1; v < 16; ++v) top = __builtin_fmaxf(top, x[v]);
+                const int w = (int)f2u(top);
+                const auto both = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+                top = __builtin_fmaxf(u2f((uint32_t)both[0]), u2f((uint32_t)both[1]));
+                const float m_new = top > m + kLazyHeads ? top : m;
+                sub = m_new == -INFINITY ? 0.0f : m_new;
+                alpha = exp2_fast(m - sub);
+                m = m_new;
+            } else if constexpr (part == 2) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) x[v] = exp2_fast(x[v] - sub);
+            } else {
+                const float sum = (((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]))) +
+                                  (((x[8] + x[9]) + (x[10] + x[11])) + ((x[12] + x[13]) + (x[14] + x[15])));
+                l = __builtin_fmaf(l, alpha, sum);
+            }
+        };
+        auto publish = [&](const Lane& L) __attribute__((always_inline)) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                *reinterpret_cast<u32x2*>(L.p_mine + 16 * ((uint32_t)q ^ L.p_turn)) =
+                    u32x2{pair16<F16>(x[4 * q], x[4 * q + 1]), pair16<F16>(x[4 * q + 2], x[4 * q + 3])};
+            if (L.h == 0) s_alpha[wave * 32 + (ln & 31)] = alpha;
+        };
+        auto rescale = [&]() __attribute__((always_inline)) {
+            float factor[4];
+#pragma unroll
+            for (int hb = 0; hb < 4; ++hb) factor[hb] = s_alpha[hb * 32 + (ln & 31)];
+            if (__ballot(factor[0] != 1.0f || factor[1] != 1.0f || factor[2] != 1.0f || factor[3] != 1.0f) != 0ull) {
+                static_for<16>([&](auto bc) __attribute__((always_inline)) {
+                    constexpr int vb = decltype(bc)::value / 4, hb = decltype(bc)::value % 4;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        float e = acc[vb][hb][v], tmp;
+                        asm volatile("v_accvgpr_read_b32 %0, %1\n\tv_mul_f32 %0, %0, %2\n\tv_accvgpr_write_b32 %1, %0" : "=&v"(tmp), "+a"(e) : "v"(factor[hb]));
+                        acc[vb][hb][v] = e;
+                    }
+                });
+            }
+        };
+        // The value products of the tile at `tile` (its probabilities are in LDS), four of the planned tile's loads sent
+        // between them (SEND) and the softmax of the step at `base` in their shadow (SOFT).
+        auto values = [&](const uint8_t* tile, const Lane& L, auto send_c, auto soft_c, auto mask_c, int base) __attribute__((always_inline)) {
+            constexpr bool SEND = decltype(send_c)::value, SOFT = decltype(soft_c)::value;
             constexpr int RING = 4, NOPS = 8;
-            u32x4 pb[4];      // the four row blocks' probabilities of the k-step being multiplied
+            u32x4 pb[4];
             u32x2 va[RING][2];
             auto read_p = [&](auto gc) __attribute__((always_inline)) {
                 constexpr int g = decltype(gc)::value;
 #pragma unroll
                 for (int hb = 0; hb < 4; ++hb)
-                    pb[hb] = *reinterpret_cast<const u32x4*>(p_read + 2048 * hb + 16 * ((uint32_t)(2 * g + h) ^ p_turn));
+                    pb[hb] = *reinterpret_cast<const u32x4*>(L.p_read + 2048 * hb + 16 * ((uint32_t)(2 * g + L.h) ^ L.p_turn));
             };
             read_p(std::integral_constant<int, 0>{});
             auto read_v = [&](auto ic) __attribute__((always_inline)) {
@@ -812,7 +988,7 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
                 constexpr int g = i / 4, vb = i % 4;
 #pragma unroll
                 for (int e = 0; e < 2; ++e) {
-                    const uint32_t at = v_lane + 64u * (uint32_t)(vb ^ (i16 >> 2)) + 16u * (v_low ^ (uint32_t)((2 * h + e) & 3));
+                    const uint32_t at = L.v_lane + 64u * (uint32_t)(vb ^ (L.i16 >> 2)) + 16u * (L.v_low ^ (uint32_t)((2 * L.h + e) & 3));
                     va[i % RING][e] = lds_transposed(tile + at + (16 * g + 4 * e) * (R * 2));
                 }
             };
@@ -821,33 +997,75 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
             __builtin_amdgcn_sched_barrier(0);
             static_for<NOPS / 2>([&](auto sc) __attribute__((always_inline)) {
                 constexpr int sec = decltype(sc)::value;
-                if constexpr (!FP8 || sec == 0) send(std::integral_constant<int, 5 + sec>{});
-                if constexpr (sec == 2) {      // (the first k-step's products have been issued: their operands were read at issue)
+                if constexpr (SEND) send(std::integral_constant<int, 5 + sec>{});
+                if constexpr (sec == 2) {
                     read_p(std::integral_constant<int, 1>{});
                     __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 static_for<2>([&](auto jc) __attribute__((always_inline)) {
                     constexpr int i = 2 * sec + decltype(jc)::value;
-                    constexpr int g = i / 4, vb = i % 4;
+                    constexpr int vb = i % 4;
                     if constexpr (i + RING - 1 < NOPS) read_v(std::integral_constant<int, i + RING - 1>{});
                     const u32x4 av = {va[i % RING][0].x, va[i % RING][0].y, va[i % RING][1].x, va[i % RING][1].y};
 #pragma unroll
                     for (int hb = 0; hb < 4; ++hb) acc[vb][hb] = mfma_32<F16>(av, pb[hb], acc[vb][hb]);
                 });
+                if constexpr (SOFT) soften(sc, mask_c, base, L);
                 static_for<2>([&](auto jc) __attribute__((always_inline)) {
                     constexpr int i = 2 * sec + decltype(jc)::value;
                     if constexpr (i + RING - 1 < NOPS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                    static_for<4>([&](auto) __attribute__((always_inline)) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        if constexpr (SOFT) {
+                            __builtin_amdgcn_sched_group_barrier(0x002, sec == 0 && decltype(mask_c)::value ? 8 : 4, 0);
+                            if constexpr (sec == 1 || sec == 2) __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
+                        }
+                    });
                 });
                 __builtin_amdgcn_sched_barrier(0);
             });
+        };
+        const std::true_type yes;
+        const std::false_type no;
+        // step 0: no values yet
+        {
+            wait_loads<LPT>();
+            lds_barrier();
+            const int base2 = plan(2, 2);
+            const Lane L = lane_now();
+            scores(ring, L);
+            static_for<4>([&](auto sc) __attribute__((always_inline)) {
+                send(std::integral_constant<int, 5 + decltype(sc)::value>{});
+                soften(sc, yes, base, L);
+            });
+            publish(L);
+            base = base1, base1 = base2;
         }
-        if constexpr (FP8) {
-            if (t + 1 < n_tiles) convert(raw_stage == NRAW - 1 ? 0 : raw_stage + 1, stage ^ 1);
-            raw_stage = raw_stage == NRAW - 1 ? 0 : raw_stage + 1;
+        // A unit's steps come in the order of their positions: first those every row of the wavefront sees whole, then
+        // the masked ones, each kind in a loop of its own (a branch around the products inside one loop sends the
+        // accumulators to scratch).
+        auto step = [&](int t, auto mask_c) __attribute__((always_inline)) {
+            wait_loads<LPT>();      // the tile's loads of this wavefront have landed: those of the next may be in flight
+            lds_barrier();          // A
+            const int base2 = plan(t + 2, (t + 2) & (NSTAGE - 1));
+            const Lane L = lane_now();
+            scores(ring + (t & (NSTAGE - 1)) * TILE, L);
+            rescale();
+            values(ring + ((t - 1) & (NSTAGE - 1)) * TILE, L, yes, yes, mask_c, base);
+            lds_barrier();          // B
+            publish(L);
+            base = base1, base1 = base2;
+        };
+        int t = 1;
+        for (; t < n_tiles && base + 32 <= unmasked; ++t) step(t, no);
+        for (; t < n_tiles; ++t) step(t, yes);
+        lds_barrier();
+        {
+            const Lane L = lane_now();
+            rescale();
+            values(ring + ((n_tiles - 1) & (NSTAGE - 1)) * TILE, L, no, no, no, 0);
         }
-        base = base1, base1 = base2, base2 = base3;
     }
     wait_loads<0>();      // (the loads past the last tile: LDS must not be written for a workgroup that has gone)
     {
