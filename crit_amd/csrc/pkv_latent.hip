@@ -863,8 +863,7 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
             uint8_t* p_mine;
             const uint8_t* p_read;
         };
-        auto lane_now = [&]() __attribute__((always_inline)) -> Lane {
-            asm volatile("" : "+v"(ln));
+        auto lane_of = [&]() __attribute__((always_inline)) -> Lane {
             Lane L;
             const int n32 = ln & 31, h = ln >> 5;
             const int fk = 4 * (n32 & 3) + ((n32 >> 2) & 3);
@@ -877,6 +876,17 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
             L.p_mine = s_prob + (wave * 32 + n32) * 64 + 8 * h;
             L.p_turn = (uint32_t)((n32 >> 2) & 3);
             L.p_read = s_prob + n32 * 64;
+            return L;
+        };
+        // (Five of them are kept; the rest, and what a step derives from any, is derived again in every step from copies
+        // the compiler cannot see through, or it would keep all of that too and push the queries out of the registers.)
+        const Lane lane_kept = lane_of();
+        auto lane_now = [&]() __attribute__((always_inline)) -> Lane {
+            asm volatile("" : "+v"(ln));
+            Lane L = lane_of();
+            L.k_lane = lane_kept.k_lane, L.t_lane = lane_kept.t_lane, L.v_lane = lane_kept.v_lane, L.v_low = lane_kept.v_low,
+            L.p_turn = lane_kept.p_turn;
+            asm volatile("" : "+v"(L.k_lane), "+v"(L.t_lane), "+v"(L.v_lane), "+v"(L.v_low), "+v"(L.p_turn));
             return L;
         };
         f32x16 s, s2;
