@@ -605,15 +605,17 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
     // (the queries are waited for here, with the first tile; the next two tiles go out behind them)
     int base1 = issue(1, 1), base2 = FP8 ? issue(2, 2) : 0;
     // E4M3: the wavefront's rows of raw tile `from`, as 16-bit values in tile `to` (a lane: 16 codes a turn).
-    auto convert = [&](int from, int to) __attribute__((always_inline)) {
+    // (In five parts, without a branch, so that a part can go between the value products: the last part's upper lanes
+    // repeat the lower ones' chunks, and every quarter-wave copies the scales.)
+    auto convert_part = [&](auto jc, int from, int to) __attribute__((always_inline)) {
         if constexpr (FP8) {
+            constexpr int j = decltype(jc)::value;
             asm volatile("" : "+v"(ln));
             const uint8_t* codes_at = raw + from * RAW + wave * (8 * W);
             uint8_t* tile_to = ring + to * TILE;
-#pragma unroll
-            for (int j = 0; j < 5; ++j) {
-                const int c = 64 * j + ln;
-                if (j < 4 || ln < 32) {
+            {
+                const int c = 64 * j + (j < 4 ? ln : (ln & 31));
+                {
                     const int row = c / CPR, cj = c - row * CPR, n = 8 * wave + row;
                     const u32x4 codes = *reinterpret_cast<const u32x4*>(codes_at + c * 16);
                     const uint32_t w[4] = {codes.x, codes.y, codes.z, codes.w};
@@ -637,8 +639,11 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
                     *reinterpret_cast<u32x4*>(row_at + 16 * ((chunk + 1) ^ turn)) = u32x4{o[4], o[5], o[6], o[7]};
                 }
             }
-            if (ln < 16) s_scale[to][ln >> 3][8 * wave + (ln & 7)] = s_raw_scale[from][wave][ln];
+            if constexpr (j == 4) s_scale[to][(ln >> 3) & 1][8 * wave + (ln & 7)] = s_raw_scale[from][wave][ln & 15];
         }
+    };
+    auto convert = [&](int from, int to) __attribute__((always_inline)) {
+        static_for<5>([&](auto jc) __attribute__((always_inline)) { convert_part(jc, from, to); });
     };
     if constexpr (FP8) {
         wait_loads<2 * LPT>();      // (its own rows of the first tile are all a wavefront converts: no barrier)
@@ -798,6 +803,7 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
                 });
             }
             // -- values: operand i = (k-step g = i / 4, block vb = i % 4) of V^T against the four row blocks' probabilities
+            const int next_raw = raw_stage == NRAW - 1 ? 0 : raw_stage + 1;
             {
                 constexpr int RING = 4, NOPS = 8;
                 u32x4 pb[4];      // the four row blocks' probabilities of the k-step being multiplied
@@ -837,6 +843,9 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
 #pragma unroll
                         for (int hb = 0; hb < 4; ++hb) acc[vb][hb] = mfma_32<F16>(av, pb[hb], acc[vb][hb]);
                     });
+                    // (the next tile's codes become values between the products: a part a section, two in the last)
+                    convert_part(sc, next_raw, stage ^ 1);
+                    if constexpr (sec == 3) convert_part(std::integral_constant<int, 4>{}, next_raw, stage ^ 1);
                     static_for<2>([&](auto jc) __attribute__((always_inline)) {
                         constexpr int i = 2 * sec + decltype(jc)::value;
                         if constexpr (i + RING - 1 < NOPS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
@@ -845,10 +854,7 @@ __global__ __launch_bounds__(256, 1) void latent_heads_kernel(LatentArgs a) {
                     __builtin_amdgcn_sched_barrier(0);
                 });
             }
-            if constexpr (FP8) {
-                if (t + 1 < n_tiles) convert(raw_stage == NRAW - 1 ? 0 : raw_stage + 1, stage ^ 1);
-                raw_stage = raw_stage == NRAW - 1 ? 0 : raw_stage + 1;
-            }
+            raw_stage = next_raw;
             base = base1, base1 = base2, base2 = base3;
         }
     } else {
