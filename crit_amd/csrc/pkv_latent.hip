@@ -374,12 +374,14 @@ __global__ __launch_bounds__(256, NT == 1 ? 3 : 2) void latent_kernel(LatentArgs
 // from the batch). The partials are stored as the registers hold them (whole kilobytes a store) and merged by a kernel
 // of their own, below.
 //
-// Measured on MI355X, 64 rows of one token at contexts ~U[1024, 8192], 128 heads, BF16: 142 us (the kernel above: 259
-// us); a step of 32 positions takes about 4,600 clocks against 2,176 of matrix instructions (scores 1,800, softmax and
-// the probabilities' way through LDS 750, values 1,900, barriers 300), and a unit's start (ranking the rows, the table,
-// the queries: 36 gathers of 32 rows x 32 bytes a wavefront) and end (256 KB of partials) another 38,000. With one
-// workgroup a compute unit nothing hides either, so launches of a few rows are slower than with the small tiles (1 row:
-// 80 us against 40): tile_rows = 16 asks for those. E4M3 rows (see the kernel's constants): 171 us.
+// Measured on MI355X, 64 rows of one token at contexts ~U[1024, 8192], 128 heads, BF16: 127-130 us (the kernel above:
+// 259 us). With every phase after the other (142 us) a step of 32 positions took about 4,600 clocks against 2,176 of
+// matrix instructions (scores 1,800, softmax and the probabilities' way through LDS 750, values 1,900, barriers 300),
+// so 16-bit rows now send a step's value products out one step later, with the next step's softmax between them. A
+// unit's start (ranking the rows, the table, the queries: 36 gathers of 32 rows x 32 bytes a wavefront) and end (256
+// KB of partials) are another 38,000. With one workgroup a compute unit nothing hides either, so launches of a few rows
+// are slower than with the small tiles (1 row: 67 us against 40): tile_rows = 16 asks for those. E4M3 rows (see the
+// kernel's constants): 158 us.
 constexpr float kLazyHeads = 8.0f;
 constexpr int kHeadsRows = 128;      // query rows a workgroup of the many-heads kernel holds
 constexpr int kRowsToAnXcd = 16;     // launches of that many batch rows or more keep a row's units on one XCD
