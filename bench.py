@@ -720,16 +720,20 @@ def reference_shapes(pk, device, only=None):
                 out = torch.empty_like(q)
                 at = [0]
 
-                def launch():
+                def launch(piece=None):
                     at[0] = (at[0] + 1) % layers
                     k, v, ks, vs = caches[at[0]]
                     pk.attend(q, k, v, kind, tables, rows, starts, firsts, columns, page, out=out, key_scales=ks,
-                              value_scales=vs)
+                              value_scales=vs, piece=piece)
                 ms = graph_timed(launch, 8)
                 nbytes = batch * ctx * hkv * (2 * d * e + (8 if kind != "bf16" else 0))
                 found[f"{name}_{batch}_rows_{columns}_cols_ctx{ctx}"] = {
                     "us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1),
                     "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+                if batch == 1 and columns == 1 and ctx <= 16384:
+                    # (one short row: what an engine of single sequences gets with the reference's own largest piece, 128
+                    # positions, instead of the default, which is sized for full batches)
+                    found[f"{name}_{batch}_rows_{columns}_cols_ctx{ctx}"]["piece_128_us"] = round(graph_timed(lambda: launch(128), 8) * 1e3, 1)
             del caches
             torch.cuda.empty_cache()
     # prefill(): one chunk of 16 / 256 / 2,048 tokens after 1,024 positions, bf16 24 / 2 x 256 (the reference's prefill rows)

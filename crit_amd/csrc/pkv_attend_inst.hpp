@@ -23,6 +23,7 @@ static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipS
             if (units > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
             const int64_t resident = (int64_t)compute_units() * attend_waves(KIND, QR);
             const dim3 pgrid((unsigned)(units < resident ? units : resident));
+            if (units <= resident) u.ticket = nullptr;      // (a unit a workgroup: nothing to draw, no counter touched)
             switch (a.heads_per_wave) {
                 case 1: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 1, false, true>), pgrid, dim3(256), 0, stream, u); break;
                 case 2: hipLaunchKernelGGL((attend128_kernel<KIND, F16, QR, 2, false, true>), pgrid, dim3(256), 0, stream, u); break;
@@ -93,6 +94,9 @@ static int launch_mfma(const AttendArgs& a, bool fused, dim3 grid, hipStream_t s
     if (units > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
     const int64_t resident = (int64_t)compute_units() * (a.dk == 256 ? 1 : kMfmaWaves);
     const dim3 pgrid((unsigned)(units < resident ? units : resident));
+    // A unit a workgroup at most: nothing to draw, and no counter touched (a draw's round trip and the count of the
+    // finished workgroups are a few microseconds at the end of a launch that is one unit long).
+    if (units <= resident) u.ticket = nullptr;
     const bool masked = a.parents != nullptr || a.parents64 != nullptr || a.sliding > 0;
     const int which = (a.dk == 256 ? 8 : (a.heads_per_wave == 2 ? 4 : 0)) + (fused ? 2 : 0) + (masked ? 1 : 0);
     switch (which) {
