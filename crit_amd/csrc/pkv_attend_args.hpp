@@ -38,7 +38,7 @@ struct AttendArgs {
     int64_t q_st, q_sh, o_st, o_sh, tab_stride, blocks_stride;
     int dk, dv;      // key and value head widths
     int fast128;     // keys and values 128 wide: the bandwidth kernel where the pages (or block lists) allow it
-    int tab_width, n_rows, columns, hq, hkv, g, page, page_shift, parts, piece, sliding, out_dtype, tiles, max_keys, heads_per_wave, units_x, units_y;
+    int tab_width, n_rows, columns, hq, hkv, g, page, page_shift, parts, piece, sliding, out_dtype, tiles, max_keys, heads_per_wave, units_x, units_y, query_tiles;
     int blocks_k, block_size, listed_keys;      // listed_keys = blocks_k * block_size: the positions a list's run holds
     Div32 block_div;
     float sscale, k_mult, v_mult;

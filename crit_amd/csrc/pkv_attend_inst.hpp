@@ -92,13 +92,14 @@ static int launch_mfma(const AttendArgs& a, bool fused, dim3 grid, hipStream_t s
     u.units_x = (int)grid.x, u.units_y = fused ? (int)grid.y : (int)grid.y + kTailClasses - 1;
     const int64_t units = (int64_t)u.units_x * u.units_y;
     if (units > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
-    const int64_t resident = (int64_t)compute_units() * (a.dk == 256 ? 1 : kMfmaWaves);
+    const int64_t resident = (int64_t)compute_units() * (a.dk == 256 || a.query_tiles > 1 ? 1 : kMfmaWaves);
     const dim3 pgrid((unsigned)(units < resident ? units : resident));
     // A unit a workgroup at most: nothing to draw, and no counter touched (a draw's round trip and the count of the
     // finished workgroups are a few microseconds at the end of a launch that is one unit long).
     if (units <= resident) u.ticket = nullptr;
     const bool masked = a.parents != nullptr || a.parents64 != nullptr || a.sliding > 0;
-    const int which = (a.dk == 256 ? 8 : (a.heads_per_wave == 2 ? 4 : 0)) + (fused ? 2 : 0) + (masked ? 1 : 0);
+    const int which = (a.dk == 256 ? 8 : (a.heads_per_wave == 2 ? 4 : 0)) + (fused ? 2 : 0) + (masked ? 1 : 0) +
+                      (a.query_tiles > 1 ? 12 : 0);
     switch (which) {
 #define PKV_MFMA(W, HWV, FU, MA, DH) \
     case W: hipLaunchKernelGGL((attend_mfma_kernel<KIND, F16, HWV, FU, MA, DH>), pgrid, dim3(256), 0, stream, u); break;
@@ -106,6 +107,17 @@ static int launch_mfma(const AttendArgs& a, bool fused, dim3 grid, hipStream_t s
         PKV_MFMA(4, 2, false, false, 1) PKV_MFMA(5, 2, false, true, 1) PKV_MFMA(6, 2, true, false, 1) PKV_MFMA(7, 2, true, true, 1)
         PKV_MFMA(8, 1, false, false, 2) PKV_MFMA(9, 1, false, true, 2) PKV_MFMA(10, 1, true, false, 2) PKV_MFMA(11, 1, true, true, 2)
 #undef PKV_MFMA
+        // four query tiles a workgroup: split launches of 128-wide heads over 16-bit pages
+#define PKV_MFMA_QT(W, HWV, MA) \
+    case W:                                                                                                                  \
+        if constexpr (KIND == 0) {                                                                                           \
+            hipLaunchKernelGGL((attend_mfma_kernel<KIND, F16, HWV, false, MA, 1, 4>), pgrid, dim3(256), 0, stream, u);       \
+            break;                                                                                                           \
+        }                                                                                                                    \
+        return CRIT_PKV_E_GEOMETRY;
+        PKV_MFMA_QT(12, 1, false) PKV_MFMA_QT(13, 1, true) PKV_MFMA_QT(16, 2, false) PKV_MFMA_QT(17, 2, true)
+#undef PKV_MFMA_QT
+        default: return CRIT_PKV_E_GEOMETRY;
     }
     return hip_code(hipGetLastError());
 }

@@ -126,11 +126,18 @@ constexpr int kMfmaTiles = 2;
 // are 512 bytes of 16-bit pages by themselves, so a wavefront serves one KV head: HW 1): twice the key pieces, query
 // pieces, score products and output tiles, the same layouts otherwise; twice the registers too, so one workgroup a
 // compute unit, which keeps as many bytes in flight as two of the narrower ones (a step's rows are twice as long).
-template <int KIND, bool F16, int HW, bool FUSED, bool MASKED, int DH = 1>
-__global__ __launch_bounds__(256, DH == 2 ? 1 : kMfmaWaves) void attend_mfma_kernel(AttendArgs a) {
+// QT: query tiles a wavefront holds (windows of several columns, wide GQA groups): a step's keys and values, once in
+// the registers, are multiplied with each tile's queries and probabilities in turn, every tile with its own softmax
+// state and accumulators, so a tile's bits are what they are alone and the rows are read once for QT tiles instead of
+// once a tile. More than one tile takes the registers of a second workgroup on the compute unit (one stays). Built for
+// four tiles of 128-wide heads over 16-bit pages, where it measured faster (64 rows ~U[1024, 8192] of 32 / 8 heads, 8
+// columns: 676 -> 480 us); 8-bit pages and 256-wide heads measured slower and keep a tile a workgroup.
+template <int KIND, bool F16, int HW, bool FUSED, bool MASKED, int DH = 1, int QT = 1>
+__global__ __launch_bounds__(256, (DH == 2 || QT > 1) ? 1 : kMfmaWaves) void attend_mfma_kernel(AttendArgs a) {
     constexpr int NT = kMfmaTiles;
     constexpr int D = 128 * DH;
     static_assert(DH == 1 || (DH == 2 && HW == 1), "heads of 128 or 256; one KV head a wavefront at 256");
+    static_assert(QT == 1 || !FUSED, "several query tiles: the split launch");
     constexpr int EB = KIND == 0 ? 2 : 1;
     constexpr int CPH = kTileRows / HW;      // tile columns a KV head holds
     constexpr int SPW = kTileRows / HW;      // positions a wavefront's step covers (tile rows a KV head holds)
@@ -272,10 +279,10 @@ __global__ __launch_bounds__(256, DH == 2 ? 1 : kMfmaWaves) void attend_mfma_ker
         for (int i = 0; i < 5; ++i) d[i] = __builtin_amdgcn_readfirstlane(d[i]);
         un.count = d[0], un.first = d[1], un.start = d[3], un.prow = d[4];
         un.trow = (int64_t)d[2] * a.tab_stride;
-        un.j0 = tile * CPH;                  // the tile's first row of the flattened (column, group head) list
+        un.j0 = tile * (QT * CPH);           // the first row of the unit's tiles in the flattened (column, group head) list
         if (un.j0 >= un.count * a.g) return un;
         un.c_lo = un.j0 / a.g;
-        const int c_hi = min(un.count, (un.j0 + CPH - 1) / a.g + 1);
+        const int c_hi = min(un.count, (un.j0 + QT * CPH - 1) / a.g + 1);
         un.n_keys = min(un.first + c_hi, a.max_keys);
         un.n_pieces = (un.n_keys + a.piece - 1) / a.piece;
         if constexpr (!FUSED) {
@@ -392,13 +399,15 @@ __global__ __launch_bounds__(256, DH == 2 ? 1 : kMfmaWaves) void attend_mfma_ker
 
     // -- what a lane holds for one unit: its tile column's token, query head, last visible position, ancestors, scale,
     // and the query operand (its column's row, piece c = the dims the keys' piece c holds; zeros in a dead column)
-    int col = 0, lim = -1;
-    unsigned long long anc = 0ull;
+    int col[QT], lim[QT];
+    unsigned long long anc[QT];
+#pragma unroll
+    for (int q = 0; q < QT; ++q) col[q] = 0, lim[q] = -1, anc[q] = 0ull;
     float sscale = a.sscale;
     float vm_cur[HW], vm_nxt[HW];      // FP8 pages: the value multipliers of the unit's heads (requested with its queries, not in its fold)
 #pragma unroll
     for (int h = 0; h < HW; ++h) vm_cur[h] = vm_nxt[h] = 1.0f;
-    u32x4 qb[4 * DH];
+    u32x4 qb[QT][4 * DH];
     auto value_multipliers = [&](const Unit& un) __attribute__((always_inline)) {      // (requested with the unit's page table entries)
         if constexpr (KIND == 1) {
 #pragma unroll
@@ -406,20 +415,23 @@ __global__ __launch_bounds__(256, DH == 2 ? 1 : kMfmaWaves) void attend_mfma_ker
         }
     };
     auto lane_values = [&](const Unit& un) __attribute__((always_inline)) {
-        const int jr = un.j0 + c16 % CPH;
-        col = jr / a.g;
-        const bool live = col < un.count;
-        const int qhead = (un.kvh0 + hsel) * a.g + jr % a.g;
-        lim = live ? min(un.first + col, un.n_keys - 1) : -1;
-        anc = (tree && live) ? ancestors(a, un.start, col) : 0ull;
         if constexpr (KIND == 1) sscale = a.sscale * (a.hm ? a.hm[un.kvh0 + hsel] : a.k_mult);
-        const uint8_t* row = a.q + ((int64_t)(un.start + col) * a.q_st + (int64_t)qhead * a.q_sh) * 2;
 #pragma unroll
-        for (int c = 0; c < 4 * DH; ++c) {
-            // 16-bit pages: dims 32 c + 8 u4 ..; 8-bit pages: dims 64 (c / 2) + 16 u4 + 8 (c % 2) .. (the codes a lane's two loads hold)
-            const int dim = KIND == 0 ? 32 * c + 8 * u4 : 64 * (c / 2) + 16 * u4 + 8 * (c % 2);
-            qb[c] = u32x4{0, 0, 0, 0};
-            if (live) qb[c] = *reinterpret_cast<const u32x4*>(row + dim * 2);
+        for (int q = 0; q < QT; ++q) {
+            const int jr = un.j0 + q * CPH + c16 % CPH;
+            col[q] = jr / a.g;
+            const bool live = col[q] < un.count;
+            const int qhead = (un.kvh0 + hsel) * a.g + jr % a.g;
+            lim[q] = live ? min(un.first + col[q], un.n_keys - 1) : -1;
+            anc[q] = (tree && live) ? ancestors(a, un.start, col[q]) : 0ull;
+            const uint8_t* row = a.q + ((int64_t)(un.start + col[q]) * a.q_st + (int64_t)qhead * a.q_sh) * 2;
+#pragma unroll
+            for (int c = 0; c < 4 * DH; ++c) {
+                // 16-bit pages: dims 32 c + 8 u4 ..; 8-bit pages: dims 64 (c / 2) + 16 u4 + 8 (c % 2) .. (the codes a lane's two loads hold)
+                const int dim = KIND == 0 ? 32 * c + 8 * u4 : 64 * (c / 2) + 16 * u4 + 8 * (c % 2);
+                qb[q][c] = u32x4{0, 0, 0, 0};
+                if (live) qb[q][c] = *reinterpret_cast<const u32x4*>(row + dim * 2);
+            }
         }
     };
 
@@ -472,10 +484,14 @@ __global__ __launch_bounds__(256, DH == 2 ? 1 : kMfmaWaves) void attend_mfma_ker
 #pragma unroll
             for (int e = 0; e < (FUSED ? EPT : 1); ++e) run_m[e] = -INFINITY, run_l[e] = 0.0f, run_a[e] = 0.0f;
             for (int part = part_lo; part < part_hi; ++part) {
-                float m = -INFINITY, l = 0.0f;      // the lane's column: running maximum (the same in its four lanes), the lane's share of the sum
-                f32x4 acc[8 * DH];                   // O^T: acc[8 h + j][i] = dim 128 h + 32 u4 + 8 i + j of the lane's column
+                float m[QT], l[QT];                  // the lane's column of each tile: running maximum (the same in its four lanes), the lane's share of the sum
+                f32x4 acc[QT][8 * DH];               // O^T: acc[q][8 h + j][i] = dim 128 h + 32 u4 + 8 i + j of the lane's column of tile q
 #pragma unroll
-                for (int j = 0; j < 8 * DH; ++j) acc[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                for (int q = 0; q < QT; ++q) {
+                    m[q] = -INFINITY, l[q] = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < 8 * DH; ++j) acc[q][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                }
 
                 auto step = [&](int base, Tile<KIND, DH>& tl, auto&& refill_k, auto&& refill_v) __attribute__((always_inline)) {
                     if (base + SPW > cur.n_keys) {
@@ -506,45 +522,56 @@ __global__ __launch_bounds__(256, DH == 2 ? 1 : kMfmaWaves) void attend_mfma_ker
                             ka[c] = u32x4{lo.x, lo.y, hi.x, hi.y};
                         }
                     }
-                    f32x4 s0 = mfma_k32<F16>(ka[0], qb[0], f32x4{0.0f, 0.0f, 0.0f, 0.0f});
-                    f32x4 s1 = mfma_k32<F16>(ka[1], qb[1], f32x4{0.0f, 0.0f, 0.0f, 0.0f});
+                    f32x4 s0[QT], s1[QT];
+#pragma unroll
+                    for (int q = 0; q < QT; ++q) {
+                        s0[q] = mfma_k32<F16>(ka[0], qb[q][0], f32x4{0.0f, 0.0f, 0.0f, 0.0f});
+                        s1[q] = mfma_k32<F16>(ka[1], qb[q][1], f32x4{0.0f, 0.0f, 0.0f, 0.0f});
+                    }
 #pragma unroll
                     for (int c = 2; c < 4 * DH; c += 2) {      // (two chains, the even pieces and the odd ones)
-                        s0 = mfma_k32<F16>(ka[c], qb[c], s0);
-                        s1 = mfma_k32<F16>(ka[c + 1], qb[c + 1], s1);
+#pragma unroll
+                        for (int q = 0; q < QT; ++q) {
+                            s0[q] = mfma_k32<F16>(ka[c], qb[q][c], s0[q]);
+                            s1[q] = mfma_k32<F16>(ka[c + 1], qb[q][c + 1], s1[q]);
+                        }
                     }
                     float ks4[4], vs4[4];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) ks4[i] = KIND >= 2 ? tl.ks[i] : 1.0f, vs4[i] = KIND >= 2 ? tl.vs[i] : 1.0f;
                     refill_k();      // (the keys' registers are free: the loads of NT steps ahead go out)
-                    // the lane's scores: its column at positions base + r_pos + i of head r_head; another head's column sees nothing
-                    const int room = lim - (base + r_pos);      // visible while i <= room
-                    float x[4];
+                    u32x2 pb[QT];
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        x[i] = (s0[i] + s1[i]) * (KIND >= 2 ? sscale * ks4[i] : sscale);
-                        bool vis = mine && i <= room;
-                        if constexpr (MASKED) {
-                            const int n = base + r_pos + i;
-                            if (tree) vis = vis && (n < cur.first || ((anc >> ((n - cur.first) & 63)) & 1ull) != 0);
-                            if (win > 0) vis = vis && n > cur.first + col - win;
+                    for (int q = 0; q < QT; ++q) {
+                        // the lane's scores: its column at positions base + r_pos + i of head r_head; another head's column sees nothing
+                        const int room = lim[q] - (base + r_pos);      // visible while i <= room
+                        float x[4];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            x[i] = (s0[q][i] + s1[q][i]) * (KIND >= 2 ? sscale * ks4[i] : sscale);
+                            bool vis = mine && i <= room;
+                            if constexpr (MASKED) {
+                                const int n = base + r_pos + i;
+                                if (tree) vis = vis && (n < cur.first || ((anc[q] >> ((n - cur.first) & 63)) & 1ull) != 0);
+                                if (win > 0) vis = vis && n > cur.first + col[q] - win;
+                            }
+                            x[i] = vis ? x[i] : -INFINITY;
                         }
-                        x[i] = vis ? x[i] : -INFINITY;
-                    }
-                    const float top = max_across_quarters(__builtin_fmaxf(__builtin_fmaxf(x[0], x[1]), __builtin_fmaxf(x[2], x[3])));
-                    const float m_new = __builtin_fmaxf(m, top);
-                    const float sub = m_new == -INFINITY ? 0.0f : m_new;
-                    const float alpha = m == -INFINITY ? 1.0f : exp2_fast(m - sub);      // (nothing summed yet: nothing to rescale)
-                    float p[4];
+                        const float top = max_across_quarters(__builtin_fmaxf(__builtin_fmaxf(x[0], x[1]), __builtin_fmaxf(x[2], x[3])));
+                        const float m_new = __builtin_fmaxf(m[q], top);
+                        const float sub = m_new == -INFINITY ? 0.0f : m_new;
+                        const float alpha = m[q] == -INFINITY ? 1.0f : exp2_fast(m[q] - sub);      // (nothing summed yet: nothing to rescale)
+                        float p[4];
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) p[i] = exp2_fast(x[i] - sub);
-                    l = __builtin_fmaf(l, alpha, (p[0] + p[1]) + (p[2] + p[3]));
-                    m = m_new;
-                    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {     // some row's maximum moved: rescale
+                        for (int i = 0; i < 4; ++i) p[i] = exp2_fast(x[i] - sub);
+                        l[q] = __builtin_fmaf(l[q], alpha, (p[0] + p[1]) + (p[2] + p[3]));
+                        m[q] = m_new;
+                        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {     // some row's maximum moved: rescale
 #pragma unroll
-                        for (int j = 0; j < 8 * DH; ++j) acc[j] *= alpha;
+                            for (int j = 0; j < 8 * DH; ++j) acc[q][j] *= alpha;
+                        }
+                        pb[q] = u32x2{pair16<F16>(p[0] * vs4[0], p[1] * vs4[1]), pair16<F16>(p[2] * vs4[2], p[3] * vs4[3])};
                     }
-                    const u32x2 pb = {pair16<F16>(p[0] * vs4[0], p[1] * vs4[1]), pair16<F16>(p[2] * vs4[2], p[3] * vs4[3])};
                     // -- values: dims {8 i + j} of the lane's four rows as two 16-bit pairs (one v_perm each), then O^T += V^T P^T
 #pragma unroll
                     for (int h = 0; h < DH; ++h) {
@@ -553,8 +580,11 @@ __global__ __launch_bounds__(256, DH == 2 ? 1 : kMfmaWaves) void attend_mfma_ker
                         for (int w = 0; w < 4; ++w) {
                             const u32x2 lo = {__builtin_amdgcn_perm(tl.v[1][h][w], tl.v[0][h][w], 0x05040100), __builtin_amdgcn_perm(tl.v[3][h][w], tl.v[2][h][w], 0x05040100)};
                             const u32x2 hi = {__builtin_amdgcn_perm(tl.v[1][h][w], tl.v[0][h][w], 0x07060302), __builtin_amdgcn_perm(tl.v[3][h][w], tl.v[2][h][w], 0x07060302)};
-                            acc[8 * h + 2 * w] = mfma_k16<F16>(lo, pb, acc[8 * h + 2 * w]);
-                            acc[8 * h + 2 * w + 1] = mfma_k16<F16>(hi, pb, acc[8 * h + 2 * w + 1]);
+#pragma unroll
+                            for (int q = 0; q < QT; ++q) {
+                                acc[q][8 * h + 2 * w] = mfma_k16<F16>(lo, pb[q], acc[q][8 * h + 2 * w]);
+                                acc[q][8 * h + 2 * w + 1] = mfma_k16<F16>(hi, pb[q], acc[q][8 * h + 2 * w + 1]);
+                            }
                         }
                     } else {
 #pragma unroll
@@ -567,7 +597,10 @@ __global__ __launch_bounds__(256, DH == 2 ? 1 : kMfmaWaves) void attend_mfma_ker
                             const u32x2 b01 = codes4_to_pairs<KIND>(hi01), b23 = codes4_to_pairs<KIND>(hi23);
                             const u32x2 va[4] = {u32x2{a01.x, a23.x}, u32x2{a01.y, a23.y}, u32x2{b01.x, b23.x}, u32x2{b01.y, b23.y}};
 #pragma unroll
-                            for (int j = 0; j < 4; ++j) acc[8 * h + 4 * w + j] = mfma_k16<F16>(va[j], pb, acc[8 * h + 4 * w + j]);
+                            for (int q = 0; q < QT; ++q) {
+#pragma unroll
+                                for (int j = 0; j < 4; ++j) acc[q][8 * h + 4 * w + j] = mfma_k16<F16>(va[j], pb[q], acc[q][8 * h + 4 * w + j]);
+                            }
                         }
                     }
                     }
@@ -618,25 +651,28 @@ __global__ __launch_bounds__(256, DH == 2 ? 1 : kMfmaWaves) void attend_mfma_ker
                 const int fold_col_j0 = cur.j0, fold_kvh0 = cur.kvh0;
                 if (part == part_hi - 1) hand_over();
 
-                // The column's sum over its four lanes, then the four wavefronts through LDS, in wavefront order.
-                const float l_col = sum_across_quarters(l);
-                if (part != part_lo) lds_barrier();      // the previous partition's fold has read the LDS
+                // A tile's column sums over its four lanes, then the four wavefronts through LDS, in wavefront order; tile
+                // after tile through the same arrays.
+#pragma unroll
+                for (int q = 0; q < QT; ++q) {
+                const float l_col = sum_across_quarters(l[q]);
+                if (part != part_lo || q > 0) lds_barrier();      // the fold before has read the LDS
 #pragma unroll
                 for (int h = 0; h < DH; ++h) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        *reinterpret_cast<f32x4*>(&s_acc[wave][c16][128 * h + 32 * u4 + 8 * i]) = f32x4{acc[8 * h][i], acc[8 * h + 1][i], acc[8 * h + 2][i], acc[8 * h + 3][i]};
-                        *reinterpret_cast<f32x4*>(&s_acc[wave][c16][128 * h + 32 * u4 + 8 * i + 4]) = f32x4{acc[8 * h + 4][i], acc[8 * h + 5][i], acc[8 * h + 6][i], acc[8 * h + 7][i]};
+                        *reinterpret_cast<f32x4*>(&s_acc[wave][c16][128 * h + 32 * u4 + 8 * i]) = f32x4{acc[q][8 * h][i], acc[q][8 * h + 1][i], acc[q][8 * h + 2][i], acc[q][8 * h + 3][i]};
+                        *reinterpret_cast<f32x4*>(&s_acc[wave][c16][128 * h + 32 * u4 + 8 * i + 4]) = f32x4{acc[q][8 * h + 4][i], acc[q][8 * h + 5][i], acc[q][8 * h + 6][i], acc[q][8 * h + 7][i]};
                     }
                 }
-                if (u4 == 0) s_m[wave][c16] = m, s_l[wave][c16] = l_col;
+                if (u4 == 0) s_m[wave][c16] = m[q], s_l[wave][c16] = l_col;
                 lds_barrier();
 #pragma unroll
                 for (int e = 0; e < EPT; ++e) {
                     const int idx = tid + e * 256;
                     const int cc = idx / D, d = idx % D;
                     const int head_i = cc / CPH;
-                    const int j = fold_col_j0 + cc % CPH;
+                    const int j = fold_col_j0 + q * CPH + cc % CPH;
                     const int c = j / a.g;
                     float M = s_m[0][cc];
 #pragma unroll
@@ -665,6 +701,7 @@ __global__ __launch_bounds__(256, DH == 2 ? 1 : kMfmaWaves) void attend_mfma_ker
                             if (d == 0) a.pm[at] = M, a.pl[at] = L;
                         }
                     }
+                }
                 }
             }
             if constexpr (FUSED) {

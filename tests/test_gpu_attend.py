@@ -120,6 +120,27 @@ def test_rows_and_columns_are_invariant_bit_for_bit(kind, hkv, d, dv):
         assert torch.equal(packed[start:start + count], together[start:start + count])
 
 
+@pytest.mark.parametrize("hkv,sliding", [(2, 0), (3, 0), (2, 700), (3, 41)])
+def test_windows_of_many_tiles_share_a_workgroup_and_keep_each_tokens_bits(hkv, sliding):
+    # 16-bit pages of 128-wide heads: a window of three tiles or more (12 columns x 4 heads: six tiles of 8 rows with two
+    # KV heads a wavefront, three of 16 with one) is read four tiles a workgroup; a token's bits stay those of its own
+    # one-column launch and of the fused launch, with and without a sliding window, and rows of fewer columns beside it.
+    cache = Cache("bf16", hkv, 128, 128, 16, [1500, 40, 2100])
+    q = rand_q(36, 4 * hkv, 128, 21)
+    counts = torch.tensor([12, 5, 12], dtype=torch.int32, device=dev)
+    firsts = [1480, 30, 2085]
+    lse = torch.empty(36, 4 * hkv, device=dev)
+    together = cache.attend(q, [0, 1, 2], [0, 12, 24], firsts, 12, counts=counts, sliding=sliding, lse=lse)
+    assert torch.equal(together[:12], cache.attend(q, [0, 1, 2], [0, 12, 24], firsts, 12, counts=counts, sliding=sliding, fused=True)[:12])
+    for s, start, first, count in zip([0, 1, 2], [0, 12, 24], firsts, [12, 5, 12]):
+        want, want_lse = cache.want(q[start:start + count], s, first, count, sliding=sliding)
+        _close(together[start:start + count], want)
+        _close_lse(lse[start:start + count], want_lse)
+        for c in (0, count // 2, count - 1):
+            one = cache.attend(q[start + c:start + c + 1], [s], [0], [first + c], 1, sliding=sliding)
+            assert torch.equal(one[0], together[start + c]), (s, c)
+
+
 def test_a_count_past_the_columns_reads_as_the_columns():
     cache = Cache("bf16", 2, 128, 128, 16, [300, 300])
     q = rand_q(8, 8, 128, 11)
