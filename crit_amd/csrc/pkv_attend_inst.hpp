@@ -92,14 +92,14 @@ static int launch_mfma(const AttendArgs& a, bool fused, dim3 grid, hipStream_t s
     u.units_x = (int)grid.x, u.units_y = fused ? (int)grid.y : (int)grid.y + kTailClasses - 1;
     const int64_t units = (int64_t)u.units_x * u.units_y;
     if (units > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
-    const int64_t resident = (int64_t)compute_units() * (a.dk == 256 || a.query_tiles > 1 ? 1 : kMfmaWaves);
+    const int64_t resident = (int64_t)compute_units() * (a.dk == 256 || a.query_tiles > 2 ? 1 : kMfmaWaves);
     const dim3 pgrid((unsigned)(units < resident ? units : resident));
     // A unit a workgroup at most: nothing to draw, and no counter touched (a draw's round trip and the count of the
     // finished workgroups are a few microseconds at the end of a launch that is one unit long).
     if (units <= resident) u.ticket = nullptr;
     const bool masked = a.parents != nullptr || a.parents64 != nullptr || a.sliding > 0;
     const int which = (a.dk == 256 ? 8 : (a.heads_per_wave == 2 ? 4 : 0)) + (fused ? 2 : 0) + (masked ? 1 : 0) +
-                      (a.query_tiles > 1 ? 12 : 0);
+                      (a.query_tiles == 4 ? 12 : (a.query_tiles == 2 ? 24 : 0));
     switch (which) {
 #define PKV_MFMA(W, HWV, FU, MA, DH) \
     case W: hipLaunchKernelGGL((attend_mfma_kernel<KIND, F16, HWV, FU, MA, DH>), pgrid, dim3(256), 0, stream, u); break;
@@ -117,6 +117,16 @@ static int launch_mfma(const AttendArgs& a, bool fused, dim3 grid, hipStream_t s
         return CRIT_PKV_E_GEOMETRY;
         PKV_MFMA_QT(12, 1, false) PKV_MFMA_QT(13, 1, true) PKV_MFMA_QT(16, 2, false) PKV_MFMA_QT(17, 2, true)
 #undef PKV_MFMA_QT
+        // two query tiles a workgroup: FP8 pages (their registers leave room for two workgroups a compute unit still)
+#define PKV_MFMA_QT2(W, HWV, MA) \
+    case W:                                                                                                                  \
+        if constexpr (KIND == 1) {                                                                                           \
+            hipLaunchKernelGGL((attend_mfma_kernel<KIND, F16, HWV, false, MA, 1, 2>), pgrid, dim3(256), 0, stream, u);       \
+            break;                                                                                                           \
+        }                                                                                                                    \
+        return CRIT_PKV_E_GEOMETRY;
+        PKV_MFMA_QT2(24, 1, false) PKV_MFMA_QT2(25, 1, true) PKV_MFMA_QT2(28, 2, false) PKV_MFMA_QT2(29, 2, true)
+#undef PKV_MFMA_QT2
         default: return CRIT_PKV_E_GEOMETRY;
     }
     return hip_code(hipGetLastError());

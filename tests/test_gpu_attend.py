@@ -120,12 +120,14 @@ def test_rows_and_columns_are_invariant_bit_for_bit(kind, hkv, d, dv):
         assert torch.equal(packed[start:start + count], together[start:start + count])
 
 
+@pytest.mark.parametrize("kind", ["bf16", "fp8"])
 @pytest.mark.parametrize("hkv,sliding", [(2, 0), (3, 0), (2, 700), (3, 41)])
-def test_windows_of_many_tiles_share_a_workgroup_and_keep_each_tokens_bits(hkv, sliding):
-    # 16-bit pages of 128-wide heads: a window of three tiles or more (12 columns x 4 heads: six tiles of 8 rows with two
-    # KV heads a wavefront, three of 16 with one) is read four tiles a workgroup; a token's bits stay those of its own
-    # one-column launch and of the fused launch, with and without a sliding window, and rows of fewer columns beside it.
-    cache = Cache("bf16", hkv, 128, 128, 16, [1500, 40, 2100])
+def test_windows_of_many_tiles_share_a_workgroup_and_keep_each_tokens_bits(hkv, sliding, kind):
+    # Pages of 128-wide heads: a window of three tiles or more (12 columns x 4 heads: six tiles of 8 rows with two KV
+    # heads a wavefront, three of 16 with one) is read four tiles a workgroup (16-bit pages) or two (FP8 pages); a
+    # token's bits stay those of its own one-column launch and of the fused launch, with and without a sliding window,
+    # and rows of fewer columns beside it.
+    cache = Cache(kind, hkv, 128, 128, 16, [1500, 40, 2100])
     q = rand_q(36, 4 * hkv, 128, 21)
     counts = torch.tensor([12, 5, 12], dtype=torch.int32, device=dev)
     firsts = [1480, 30, 2085]
