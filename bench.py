@@ -767,6 +767,45 @@ def reference_shapes(pk, device, only=None):
     return found
 
 
+def verify_windows(pk, device):
+    """Verify windows of a draft (8B shape, 32 query / 8 KV heads x 128, pages of 16): 64 rows at contexts ~U[1024, 8192],
+    each a window of 1, 4, 5 or 8 columns, bf16 and fp8 pages; microseconds a launch (split + merge) over four layers of
+    different memory, replayed from a captured graph. The rows are read once for four tiles of 16-bit pages (two of
+    FP8 pages) a workgroup; one column is the decode step for comparison."""
+    hq, hkv, d, page, B, found = 32, 8, 128, 16, 64, {}
+    g = torch.Generator(device=device).manual_seed(5)
+    ctx = torch.randint(1024, 8193, (B,), generator=torch.Generator().manual_seed(1))
+    held = [(int(n) + 8 + page - 1) // page for n in ctx]
+    width = (max(held) + 15) // 16 * 16
+    pages = sum(held) + 1
+    order = torch.randperm(pages, device=device, generator=g).to(torch.int32)
+    tables = torch.full((B, width), pages, dtype=torch.int32, device=device)
+    at = 0
+    for s, w in enumerate(held):
+        tables[s, :w] = order[at:at + w]
+        at += w
+    rows = torch.arange(B, dtype=torch.int32, device=device)
+    for kind in ("bf16", "fp8"):
+        store = torch.bfloat16 if kind == "bf16" else torch.float8_e4m3fn
+        ks = [(torch.randn(pages + 1, page, hkv, d, device=device, dtype=torch.bfloat16, generator=g) * 0.5).to(store) for _ in range(4)]
+        vs = [(torch.randn(pages + 1, page, hkv, d, device=device, dtype=torch.bfloat16, generator=g) * 0.5).to(store) for _ in range(4)]
+        for columns in (1, 4, 5, 8):
+            starts = rows * columns
+            firsts = (ctx - columns).to(torch.int64).to(device)
+            q = torch.randn(B * columns, hq, d, device=device, generator=g).to(torch.bfloat16)
+            out = torch.empty_like(q)
+            i = [0]
+
+            def launch():
+                i[0] = (i[0] + 1) % 4
+                pk.attend(q, ks[i[0]], vs[i[0]], kind, tables, rows, starts, firsts, columns, page, out=out,
+                          multipliers=(0.02, 0.03))
+            found[f"{kind}_{columns}_columns_us"] = round(graph_timed(launch, 8) * 1e3, 1)
+        del ks, vs
+        torch.cuda.empty_cache()
+    return found
+
+
 def small_batches(pk, device):
     """What a piece costs a batch that does not fill the chip: one layer's decode launch (split + merge, 8B shape) for
     4 sequences of about 2,000 positions and for one of 8,000, at the default piece and at pieces of 256 positions
@@ -1052,6 +1091,9 @@ def main():
         torch.cuda.empty_cache()
         extras["reference_published_shapes"] = reference_shapes(pk, device)
         log(f"[bench] the reference's published shapes: {extras['reference_published_shapes']}")
+        torch.cuda.empty_cache()
+        extras["verify_windows_64_rows"] = verify_windows(pk, device)
+        log(f"[bench] verify windows, 64 rows: {extras['verify_windows_64_rows']}")
         torch.cuda.empty_cache()
         extras["small_batches_by_piece"] = small_batches(pk, device)
         log(f"[bench] small batches, default piece and 256: {extras['small_batches_by_piece']}")
