@@ -333,16 +333,17 @@ static int launch_attend_checked(const crit_pkv_attend_params* p, hipStream_t st
     // bandwidth kernel (matrix tiles of 16 columns).
     const int tile_rows = a.fast128 && !p->blocks ? 16 / a.heads_per_wave : qr;
     a.tiles = (live_rows + tile_rows - 1) / tile_rows;
-    // Windows of three tiles or more of 128-wide heads over 16-bit pages, split launch: a workgroup holds four tiles and
-    // reads the rows once for all of them. A tile's bits are the same however many share a workgroup, so this may
-    // follow the launch. Measured on MI355X (32 / 8 heads, 64 rows ~U[1024, 8192]): 5 columns 519 -> 424 us, 8 columns
-    // 676 -> 480; one row of 32,768: 72 -> 56 and 91 -> 62. Not taken where it measured slower: two tiles (one
-    // workgroup a compute unit instead of two streams as much as it saves), 8-bit pages (8 columns 376 -> 334 us but
-    // 5 columns 279 -> 302, one row 55 -> 92: the converted rows' steps are too long a chain for one wavefront a SIMD)
-    // and 256-wide heads in pairs of tiles (64 rows: 4 columns 443 -> 554 us; only rows of 100,000 positions gained).
+    // Windows of several tiles of 128-wide heads over 16-bit pages, split launch: a workgroup holds four tiles (one
+    // workgroup a compute unit), or the two of a window of two (two workgroups still, with two dozen registers in
+    // scratch outside the steps), and reads the rows once for all of them. A tile's bits are the same however many
+    // share a workgroup, so this may follow the launch. Measured on MI355X (32 / 8 heads, 64 rows ~U[1024, 8192]): 4
+    // columns 383 -> 288 us, 5 columns 519 -> 424, 8 columns 676 -> 480; one row of 32,768: 55 -> 45, 72 -> 56 and 91 ->
+    // 62. Not taken where it measured slower: four tiles of 8-bit pages (8 columns 376 -> 334 us but 5 columns 279 ->
+    // 302, one row 55 -> 92: the converted rows' steps are too long a chain for one wavefront a SIMD) and 256-wide
+    // heads in pairs of tiles (64 rows: 4 columns 443 -> 554 us; only rows of 100,000 positions gained).
     a.query_tiles = 1;
-    if (a.fast128 && !p->blocks && !p->fused && wide128 && p->kind == 0 && a.tiles >= 3) {
-        a.query_tiles = 4;
+    if (a.fast128 && !p->blocks && !p->fused && wide128 && p->kind == 0 && a.tiles >= 2) {
+        a.query_tiles = a.tiles >= 3 ? 4 : 2;
         a.tiles = (a.tiles + a.query_tiles - 1) / a.query_tiles;
     }
     // FP8 pages (whose tiles leave room for two workgroups a compute unit even in pairs): two tiles a workgroup. 64 rows,

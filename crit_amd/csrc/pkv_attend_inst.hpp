@@ -120,7 +120,7 @@ static int launch_mfma(const AttendArgs& a, bool fused, dim3 grid, hipStream_t s
         // two query tiles a workgroup: FP8 pages (their registers leave room for two workgroups a compute unit still)
 #define PKV_MFMA_QT2(W, HWV, MA) \
     case W:                                                                                                                  \
-        if constexpr (KIND == 1) {                                                                                           \
+        if constexpr (KIND <= 1) {                                                                                           \
             hipLaunchKernelGGL((attend_mfma_kernel<KIND, F16, HWV, false, MA, 1, 2>), pgrid, dim3(256), 0, stream, u);       \
             break;                                                                                                           \
         }                                                                                                                    \
