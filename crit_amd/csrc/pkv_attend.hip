@@ -346,10 +346,11 @@ static int launch_attend_checked(const crit_pkv_attend_params* p, hipStream_t st
         a.query_tiles = a.tiles >= 3 ? 4 : 2;
         a.tiles = (a.tiles + a.query_tiles - 1) / a.query_tiles;
     }
-    // FP8 pages (whose tiles leave room for two workgroups a compute unit even in pairs): two tiles a workgroup. 64 rows,
-    // 4 / 5 / 8 columns: 207 -> 147, 279 -> 214, 376 -> 230 us; one row of 32,768: 54 -> 52 and 64 -> 52 us, but a
-    // pair alone (4 columns) 40 -> 51 us, so a window of two tiles pairs them only in launches that fill the card.
-    if (a.fast128 && !p->blocks && !p->fused && wide128 && p->kind == 1 && a.tiles >= 2) {
+    // 8-bit pages: two tiles a workgroup, two workgroups a compute unit still (FP8 in 242-252 registers; the row-scaled
+    // kinds with two dozen in scratch outside the steps). 64 rows, 4 / 5 / 8 columns: FP8 207 -> 147, 279 -> 214, 376 ->
+    // 230 us, INT8 224 -> 167, 307 -> 264, 428 -> 287 us; one row of 32,768 (FP8): 54 -> 52 and 64 -> 52 us, but a pair
+    // alone (4 columns) 40 -> 51 us, so a window of two tiles pairs them only in launches that fill the card.
+    if (a.fast128 && !p->blocks && !p->fused && wide128 && p->kind >= 1 && a.tiles >= 2) {
         const int64_t apart = (int64_t)p->n_rows * (p->kv_heads / a.heads_per_wave) * a.tiles * p->partitions;
         if (a.tiles >= 3 || apart > (int64_t)compute_units() * 2) {
             a.query_tiles = 2;

@@ -117,10 +117,10 @@ static int launch_mfma(const AttendArgs& a, bool fused, dim3 grid, hipStream_t s
         return CRIT_PKV_E_GEOMETRY;
         PKV_MFMA_QT(12, 1, false) PKV_MFMA_QT(13, 1, true) PKV_MFMA_QT(16, 2, false) PKV_MFMA_QT(17, 2, true)
 #undef PKV_MFMA_QT
-        // two query tiles a workgroup: FP8 pages (their registers leave room for two workgroups a compute unit still)
+        // two query tiles a workgroup, two workgroups a compute unit still
 #define PKV_MFMA_QT2(W, HWV, MA) \
     case W:                                                                                                                  \
-        if constexpr (KIND <= 1) {                                                                                           \
+        if constexpr (KIND <= 3) {                                                                                           \
             hipLaunchKernelGGL((attend_mfma_kernel<KIND, F16, HWV, false, MA, 1, 2>), pgrid, dim3(256), 0, stream, u);       \
             break;                                                                                                           \
         }                                                                                                                    \

@@ -130,9 +130,9 @@ constexpr int kMfmaTiles = 2;
 // the registers, are multiplied with each tile's queries and probabilities in turn, every tile with its own softmax
 // state and accumulators, so a tile's bits are what they are alone and the rows are read once for QT tiles instead of
 // once a tile. More than one tile takes the registers of a second workgroup on the compute unit (one stays). Built for
-// four tiles (or a window's two) of 128-wide heads over 16-bit pages and two over FP8 pages (pairs still fit two
+// four tiles (or a window's two) of 128-wide heads over 16-bit pages and two over 8-bit pages (pairs still fit two
 // workgroups a compute unit), where it measured faster (64 rows ~U[1024, 8192] of 32 / 8 heads, 8 columns: 676 -> 480 us, FP8 376 -> 224);
-// row-scaled pages and 256-wide heads measured slower and keep a tile a workgroup.
+// four tiles of 8-bit pages and pairs of 256-wide heads measured slower.
 template <int KIND, bool F16, int HW, bool FUSED, bool MASKED, int DH = 1, int QT = 1>
 __global__ __launch_bounds__(256, (DH == 2 || QT > 2) ? 1 : kMfmaWaves) void attend_mfma_kernel(AttendArgs a) {
     constexpr int NT = kMfmaTiles;
