@@ -339,8 +339,7 @@ static int launch_attend_checked(const crit_pkv_attend_params* p, hipStream_t st
     // share a workgroup, so this may follow the launch. Measured on MI355X (32 / 8 heads, 64 rows ~U[1024, 8192]): 4
     // columns 383 -> 288 us, 5 columns 519 -> 424, 8 columns 676 -> 480; one row of 32,768: 55 -> 45, 72 -> 56 and 91 ->
     // 62. Not taken where it measured slower: four tiles of 8-bit pages (8 columns 376 -> 334 us but 5 columns 279 ->
-    // 302, one row 55 -> 92: the converted rows' steps are too long a chain for one wavefront a SIMD) and 256-wide
-    // heads in pairs of tiles (64 rows: 4 columns 443 -> 554 us; only rows of 100,000 positions gained).
+    // 302, one row 55 -> 92: the converted rows' steps are too long a chain for one wavefront a SIMD).
     a.query_tiles = 1;
     if (a.fast128 && !p->blocks && !p->fused && wide128 && p->kind == 0 && a.tiles >= 2) {
         a.query_tiles = a.tiles >= 3 ? 4 : 2;
@@ -356,6 +355,13 @@ static int launch_attend_checked(const crit_pkv_attend_params* p, hipStream_t st
             a.query_tiles = 2;
             a.tiles = (a.tiles + a.query_tiles - 1) / a.query_tiles;
         }
+    }
+    // 256-wide heads: pairs of tiles with one step in flight a wavefront instead of two (with two, 56-85 registers went
+    // to scratch and 64 rows x 4 columns took 554 us against 443 apart; with one, 24 / 2 heads x 256 bf16, 64 rows, 2 / 4
+    // / 5 / 8 columns: 287 -> 232, 445 -> 410, 569 -> 452, 856 -> 676 us; one row of 200,000: 255 -> 146 and 344 -> 237).
+    if (a.fast128 && !p->blocks && !p->fused && wide256 && a.tiles >= 2) {
+        a.query_tiles = 2;
+        a.tiles = (a.tiles + a.query_tiles - 1) / a.query_tiles;
     }
     const int64_t gx = (int64_t)p->n_rows * (p->kv_heads / a.heads_per_wave) * a.tiles;
     if (gx > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;

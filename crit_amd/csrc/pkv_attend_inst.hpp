@@ -127,6 +127,8 @@ static int launch_mfma(const AttendArgs& a, bool fused, dim3 grid, hipStream_t s
         return CRIT_PKV_E_GEOMETRY;
         PKV_MFMA_QT2(24, 1, false) PKV_MFMA_QT2(25, 1, true) PKV_MFMA_QT2(28, 2, false) PKV_MFMA_QT2(29, 2, true)
 #undef PKV_MFMA_QT2
+        case 32: hipLaunchKernelGGL((attend_mfma_kernel<KIND, F16, 1, false, false, 2, 2>), pgrid, dim3(256), 0, stream, u); break;
+        case 33: hipLaunchKernelGGL((attend_mfma_kernel<KIND, F16, 1, false, true, 2, 2>), pgrid, dim3(256), 0, stream, u); break;
         default: return CRIT_PKV_E_GEOMETRY;
     }
     return hip_code(hipGetLastError());

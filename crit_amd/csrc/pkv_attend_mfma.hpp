@@ -132,10 +132,11 @@ constexpr int kMfmaTiles = 2;
 // once a tile. More than one tile takes the registers of a second workgroup on the compute unit (one stays). Built for
 // four tiles (or a window's two) of 128-wide heads over 16-bit pages and two over 8-bit pages (pairs still fit two
 // workgroups a compute unit), where it measured faster (64 rows ~U[1024, 8192] of 32 / 8 heads, 8 columns: 676 -> 480 us, FP8 376 -> 224);
-// four tiles of 8-bit pages and pairs of 256-wide heads measured slower.
+// pairs of tiles of 256-wide heads keep one step in flight a wavefront instead of two (NT), or their registers spill;
+// four tiles of 8-bit pages measured slower.
 template <int KIND, bool F16, int HW, bool FUSED, bool MASKED, int DH = 1, int QT = 1>
 __global__ __launch_bounds__(256, (DH == 2 || QT > 2) ? 1 : kMfmaWaves) void attend_mfma_kernel(AttendArgs a) {
-    constexpr int NT = kMfmaTiles;
+    constexpr int NT = DH == 2 && QT == 2 ? 1 : kMfmaTiles;
     constexpr int D = 128 * DH;
     static_assert(DH == 1 || (DH == 2 && HW == 1), "heads of 128 or 256; one KV head a wavefront at 256");
     static_assert(QT == 1 || !FUSED, "several query tiles: the split launch");
