@@ -251,11 +251,13 @@ static int launch_attend_checked(const crit_pkv_attend_params* p, hipStream_t st
     if (p->q_stride_t % 8 || p->q_stride_h % 8 || (reinterpret_cast<uintptr_t>(p->q) % 16) ||
         (reinterpret_cast<uintptr_t>(p->key_pages) % 16) || (reinterpret_cast<uintptr_t>(p->value_pages) % 16))
         return CRIT_PKV_E_GEOMETRY;
-    if (derive) {      // one row is key and value: one width (64 or 128), halves of the rotation in whole lanes
-        if (p->head_dim != p->value_dim || (p->head_dim != 64 && p->head_dim != 128) || p->derive_rot < 16 ||
-            p->derive_rot % 16 || p->derive_rot > p->head_dim || !(p->derive_eps >= 0.0f) || p->blocks || p->fresh_keys)
+    if (derive) {      // one row is key and value: one width; any even rotary width up to it
+        if (p->head_dim != p->value_dim || p->derive_rot < 2 || p->derive_rot % 2 || p->derive_rot > p->head_dim ||
+            !(p->derive_eps >= 0.0f) || p->blocks || p->fresh_keys)
             return CRIT_PKV_E_GEOMETRY;      // (fresh rows come as values only: their keys are derived too)
     }
+    // INT8 queries against INT8 keys (prefill's int8_qk for the chunks it reads as window rows): the fused launch
+    if (p->int8_qk && (p->kind != 3 || derive || p->blocks || !p->fused)) return p->kind != 3 ? CRIT_PKV_E_DTYPE : CRIT_PKV_E_GEOMETRY;
     const int lpr = (p->head_dim > p->value_dim ? p->head_dim : p->value_dim) / 8;      // lanes that hold the wider row
     const bool wide128 = p->head_dim == 128 && p->value_dim == 128;
     const bool wide256 = p->head_dim == 256 && p->value_dim == 256;      // (the matrix-core kernel's second width: two halves of 128)
@@ -297,6 +299,7 @@ static int launch_attend_checked(const crit_pkv_attend_params* p, hipStream_t st
     a.f_per_row = p->fresh_per_row ? 1 : 0;
     a.derive_table = p->derive_table, a.derive_eps = p->derive_eps, a.derive_rot = p->derive_rot;
     a.derive_weighted = p->derive_weighted ? 1 : 0;
+    a.iqk = p->int8_qk ? 1 : 0;
     a.listed_keys = p->blocks ? p->blocks_k * p->block_size : 0;
     a.block_div = make_div32(p->blocks ? (uint32_t)p->block_size : 1u);
     a.q_st = p->q_stride_t, a.q_sh = p->q_stride_h, a.o_st = p->out_stride_t, a.o_sh = p->out_stride_h, a.tab_stride = p->table_stride;
@@ -315,7 +318,8 @@ static int launch_attend_checked(const crit_pkv_attend_params* p, hipStream_t st
         qr = a.g % 4 == 0 ? 4 : 1;      // (the block-list kernels are built for tiles of 1 and 4 rows)
     }
     // The generic kernel's variants that read fresh rows or derive their keys are built for tiles of 2 and 8 rows.
-    if (fresh || derive) qr = qr <= 2 ? 2 : 8;
+    if (fresh || derive || a.iqk) qr = qr <= 2 ? 2 : 8;      // (so is the one with INT8 queries)
+    if (derive && p->head_dim != 64 && p->head_dim != 128) qr = 8;      // (derived keys at the other widths: tiles of 8 only)
     // The 128-wide kernel serves two adjacent KV heads per wavefront where the head count is even, so every position
     // is read in segments of two rows (512 bytes of 16-bit pages, 256 of 8-bit ones): measured best on MI355X against
     // one and four heads. Fixed by the cache's geometry, never by the launch: a column's bits depend on it.
@@ -327,7 +331,7 @@ static int launch_attend_checked(const crit_pkv_attend_params* p, hipStream_t st
     // The bandwidth kernel walks pages that are powers of two from 16 positions up, in positions below 2^31; other
     // multiples of 16 take the generic kernel. (block lists of blocks that are a multiple of 16: their own variant)
     const bool pow2_page = a.page_shift >= 4 && (int64_t)p->partitions * p->piece <= 0x3fffffff;
-    a.fast128 = !derive && (((wide128 || wide256) && page16 && pow2_page && p->piece % 16 == 0) || fast_lists);      // (derived keys: the generic kernel)
+    a.fast128 = !derive && !a.iqk && (((wide128 || wide256) && page16 && pow2_page && p->piece % 16 == 0) || fast_lists);      // (derived keys: the generic kernel)
     if (a.fast128 && wide128 && p->kv_heads % 2 == 0) a.heads_per_wave = 2;
     // Query rows a tile holds: the generic and block-list kernels' tile height; 16 a wavefront's heads share in the
     // bandwidth kernel (matrix tiles of 16 columns).

@@ -56,6 +56,7 @@ struct AttendArgs {
     const float* derive_table;
     float derive_eps;
     int derive_rot, derive_weighted;
+    int iqk;      // INT8 pages: the queries as INT8 codes at each row's own scale (prefill's int8_qk read as windows)
 };
 
 // A workgroup barrier that orders the shared arrays only: a wavefront waits for its own LDS traffic, then for the

@@ -48,9 +48,18 @@ struct StepBuf {
 // (codes times their scale or multiplier), rms_norm(r) = r / sqrt(mean(r * r) + eps), the "half" rotation over the
 // first rotary_dim values (value i with value i + rotary_dim / 2) at the angle fp32(position) * freqs[i], all in FP32;
 // the scores are FP32 products of the queries with these keys (the reference multiplies the FP32 key as two parts in
-// the queries' type: the same value to about 2^-16). rotary_dim is a multiple of 16, so a half is whole lanes.
-template <int KIND, bool F16, int LPR, int QR, bool FUSED, bool SPARSE = false, bool FRESH = false, bool DERIVE = false>
+// the queries' type: the same value to about 2^-16). rotary_dim is any even width up to the head's: where it is a
+// multiple of 16 a half is whole lanes and a lane's partner elements sit in one other lane.
+//
+// IQK (INT8 pages): each query row becomes INT8 codes at its own scale (amax / 127, at least 1e-30, rounded half away
+// from zero: _kernels.py:637-643 of the reference, its int8_qk), and a page position's score is the exact integer
+// product of the two rows' codes (sums below 2^24, so FP32 holds them) times both scales; a fresh position's score
+// keeps the queries' 16 bits. What a prompt chunk read as window rows asks for where the matrix-core prompt kernel
+// is not built for the head width.
+template <int KIND, bool F16, int LPR, int QR, bool FUSED, bool SPARSE = false, bool FRESH = false, bool DERIVE = false,
+          bool IQK = false>
 __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
+    static_assert(!IQK || (KIND == 3 && !DERIVE && !SPARSE), "integer scores: INT8 pages, windows without lists");
     static_assert(!(SPARSE && FUSED), "block lists are read by the split launch");
     static_assert(!(SPARSE && FRESH), "block lists read the pages only");
     static_assert(!(DERIVE && SPARSE), "derived keys: windows without block lists");
@@ -141,6 +150,22 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
             for (int j = 0; j < 4; ++j) {
                 qf[rr][2 * j] = F16 ? f16_lo(qp[rr][j]) : bf16_lo(qp[rr][j]);
                 qf[rr][2 * j + 1] = F16 ? f16_hi(qp[rr][j]) : bf16_hi(qp[rr][j]);
+            }
+        }
+    }
+    float qi[IQK ? QR : 1][8], q_scale[IQK ? QR : 1];      // IQK: the rows' codes (as FP32 integers) and scales
+    if constexpr (IQK) {
+#pragma unroll
+        for (int rr = 0; rr < QR; ++rr) {
+            float amax = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) amax = __builtin_fmaxf(amax, __builtin_fabsf(qf[rr][j]));
+            amax = group_max<LPR>(amax);
+            q_scale[rr] = __builtin_fmaxf(__fdiv_rn(amax, 127.0f), 1e-30f);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float f = __fdiv_rn(qf[rr][j], q_scale[rr]);
+                qi[rr][j] = (float)(int)(f >= 0.0f ? f + 0.5f : f - 0.5f);      // (a NaN row gives codes of 0, as the cast does)
             }
         }
     }
@@ -269,19 +294,42 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
             for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(kf[j], kf[j], ss);
             ss = group_sum<LPR>(ss);
             const float rn = 1.0f / __builtin_sqrtf(ss / (float)D + a.derive_eps);
-            const int half = a.derive_rot >> 4;      // lanes a half of the rotated values takes
             const float* weight = a.derive_table + (a.derive_rot >> 1);
 #pragma unroll
             for (int j = 0; j < 8; ++j) kf[j] = kf[j] * rn * (a.derive_weighted ? weight[li * 8 + j] : 1.0f);
-            const bool low = li < half, turns = li < 2 * half;
-            const int from = turns ? (low ? lane + half : lane - half) : lane;
-            const int fi = (low ? li : li - half) * 8;
+            // Element e = 8 li + j turns with element e + h (e below h = rotary_dim / 2) or e - h (h <= e < rotary_dim).
+            const int h = a.derive_rot >> 1, hl = h >> 3, hs = h & 7;      // the partner: hl lanes and hs places away
+            float other[8];
+            if (hs == 0) {      // halves of whole lanes: the partner sits at the same place of the lane hl away
+                const bool low = li < hl, turns = li < 2 * hl;
+                const int from = turns ? (low ? lane + hl : lane - hl) : lane;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) other[j] = __shfl(kf[j], from);
+            } else {
+                // Any even width: place s of a lane is the partner of place (s - hs) mod 8 of the lower half's elements
+                // (in the lane hl, or hl + 1, below) and of place (s + hs) mod 8 of the upper half's (hl, or hl + 1,
+                // above); both places are the same for every lane, so each is one shuffle and a select.
+#pragma unroll
+                for (int j = 0; j < 8; ++j) other[j] = 0.0f;
+#pragma unroll
+                for (int s = 0; s < 8; ++s) {
+                    const int jl = (s - hs) & 7, ju = (s + hs) & 7;
+                    const float up = __shfl(kf[s], lane + hl + (jl + hs >= 8 ? 1 : 0));       // for an element of the lower half
+                    const float down = __shfl(kf[s], lane - hl - (ju < hs ? 1 : 0));          // for one of the upper half
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const int e = li * 8 + j;
+                        other[j] = (j == jl && e < h) ? up : ((j == ju && e >= h && e < a.derive_rot) ? down : other[j]);
+                    }
+                }
+            }
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const float other = __shfl(kf[j], from);
+                const int e = li * 8 + j;
+                const bool low = e < h, turns = e < a.derive_rot;
                 float sn, cs;
-                sincosf((float)n * a.derive_table[turns ? fi + j : 0], &sn, &cs);
-                const float turned = low ? kf[j] * cs - other * sn : kf[j] * cs + other * sn;
+                sincosf((float)n * a.derive_table[turns ? (low ? e : e - h) : 0], &sn, &cs);
+                const float turned = low ? kf[j] * cs - other[j] * sn : kf[j] * cs + other[j] * sn;
                 kf[j] = turns ? turned : kf[j];
             }
         };
@@ -336,7 +384,11 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
                         }
                     } else {
 #pragma unroll
-                        for (int j = 0; j < 8; ++j) d = __builtin_fmaf(qf[rr][j], kf[j], d);
+                        for (int j = 0; j < 8; ++j) {
+                            float qv = qf[rr][j];
+                            if constexpr (IQK) qv = (FRESH && isf[k]) ? qv : qi[rr][j];
+                            d = __builtin_fmaf(qv, kf[j], d);
+                        }
                     }
                     s[k][rr] = group_sum<LPR>(d);
                 }
@@ -349,6 +401,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(AttendArgs a) {
                 for (int k = 0; k < 4; ++k) {
                     const int n = SPARSE ? buf.pos[k] : base + k * PPI + lg;
                     float x = s[k][rr] * ((isf[k] || DERIVE) ? a.sscale : (KIND >= 2 ? sscale * buf.ks[k] : sscale));
+                    if constexpr (IQK) x = isf[k] ? x : x * q_scale[rr];
                     bool vis = n <= lim[rr] && n < n_keys;
                     if constexpr (SPARSE) vis = vis && n >= 0;
                     if (tree) vis = vis && (n < first || ((anc[rr] >> ((n - first) & 63)) & 1ull) != 0);

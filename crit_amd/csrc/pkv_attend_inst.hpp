@@ -43,20 +43,40 @@ static int launch_one(const AttendArgs& a, int lpr, bool page16, dim3 grid, hipS
             return hip_code(hipGetLastError());
         }
     }
+    if constexpr (SPECIAL && KIND == 3 && FUSED) {
+        if (a.iqk) {      // INT8 queries against INT8 keys: a prompt chunk's window rows (with or without its own fresh rows)
+            switch (a.fv ? lpr : -lpr) {
+#define PKV_IQK(L) \
+    case L: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, L, QR, true, false, true, false, true>), grid, dim3(256), 0, stream, a); break; \
+    case -L: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, L, QR, true, false, false, false, true>), grid, dim3(256), 0, stream, a); break;
+                PKV_IQK(2) PKV_IQK(4) PKV_IQK(8) PKV_IQK(16) PKV_IQK(32)
+#undef PKV_IQK
+                default: return CRIT_PKV_E_GEOMETRY;
+            }
+            return hip_code(hipGetLastError());
+        }
+    }
+    if (a.iqk) return CRIT_PKV_E_GEOMETRY;
     if constexpr (SPECIAL) {
     if (a.derive_table && a.fv) {      // derived keys over pages and fresh value rows
         switch (lpr) {
+            case 2: if constexpr (QR == 8) { hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 2, QR, FUSED, false, true, true>), grid, dim3(256), 0, stream, a); break; } return CRIT_PKV_E_GEOMETRY;
+            case 4: if constexpr (QR == 8) { hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 4, QR, FUSED, false, true, true>), grid, dim3(256), 0, stream, a); break; } return CRIT_PKV_E_GEOMETRY;
             case 8: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 8, QR, FUSED, false, true, true>), grid, dim3(256), 0, stream, a); break;
             case 16: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 16, QR, FUSED, false, true, true>), grid, dim3(256), 0, stream, a); break;
+            case 32: if constexpr (QR == 8) { hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 32, QR, FUSED, false, true, true>), grid, dim3(256), 0, stream, a); break; } return CRIT_PKV_E_GEOMETRY;
             default: return CRIT_PKV_E_GEOMETRY;
         }
-    } else if (a.derive_table) {      // keys derived from the value rows: the generic kernel's variant for 64- and 128-wide heads
+    } else if (a.derive_table) {      // keys derived from the value rows: the generic kernel's variant (any head width; the widths other than 64 and 128 in tiles of 8 rows only)
         switch (lpr) {
+            case 2: if constexpr (QR == 8) { hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 2, QR, FUSED, false, false, true>), grid, dim3(256), 0, stream, a); break; } return CRIT_PKV_E_GEOMETRY;
+            case 4: if constexpr (QR == 8) { hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 4, QR, FUSED, false, false, true>), grid, dim3(256), 0, stream, a); break; } return CRIT_PKV_E_GEOMETRY;
             case 8: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 8, QR, FUSED, false, false, true>), grid, dim3(256), 0, stream, a); break;
             case 16: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 16, QR, FUSED, false, false, true>), grid, dim3(256), 0, stream, a); break;
+            case 32: if constexpr (QR == 8) { hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 32, QR, FUSED, false, false, true>), grid, dim3(256), 0, stream, a); break; } return CRIT_PKV_E_GEOMETRY;
             default: return CRIT_PKV_E_GEOMETRY;
         }
-    } else if (a.fv) {       // fresh rows beside the pages: the generic kernel's variant that reads both (any head width)
+    } else if (a.fv) {       // fresh rows beside the pages: the generic kernel's variant that reads both (any head width; the widths other than 64 and 128 in tiles of 8 rows only)
         switch (lpr) {
             case 2: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 2, QR, FUSED, false, true>), grid, dim3(256), 0, stream, a); break;
             case 4: hipLaunchKernelGGL((attend_generic_kernel<KIND, F16, 4, QR, FUSED, false, true>), grid, dim3(256), 0, stream, a); break;

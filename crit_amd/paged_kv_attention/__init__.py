@@ -73,7 +73,7 @@ def derive(weight, eps, freqs, rotary_dim):
 def _derived(given, d, device):
     """`given` (a Derive or a tuple of its four fields) checked for heads of width d (None: not known yet) on `device`:
     (the Derive with its packed table, whether it has a weight). The checks and their messages are the reference's
-    (__init__.py:99-121); past them these kernels take rotary widths in multiples of 16 over heads of 64 or 128."""
+    (__init__.py:99-121): any even rotary width from 2 up to the head width, at every head width."""
     found = given if isinstance(given, Derive) else Derive(*given)
     weight, eps, freqs, rot = found.weight, float(found.eps), found.freqs, int(found.rotary_dim)
     if rot < 2 or rot % 2 or (d is not None and rot > d):
@@ -93,8 +93,6 @@ def _derived(given, d, device):
         table = freqs.contiguous() if weight is None else torch.cat([freqs, weight.contiguous()])
     elif table.numel() != rot // 2 + (0 if weight is None else weight.shape[0]):
         raise ValueError("a Derive's packed table does not fit its freqs and weight")
-    if rot % 16 or (d is not None and d not in (64, 128)):
-        raise _unsupported(f"derive= with a rotary width of {rot} over heads of {d} (multiples of 16 over heads of 64 or 128 are)")
     return found._replace(eps=eps, rotary_dim=rot, table=table), weight is not None
 
 
@@ -512,7 +510,8 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
            offsets=None, tokens=None, key_scales=None, value_scales=None, multipliers=(1.0, 1.0), scale=None,
            partitions=None, parents=None, blocks=None, block_size=None, out=None, lse=None, workspace=None, piece=None,
            fused=False, fresh=None, vsplit=None, tile=None, num_warps=None, num_stages=None, maxnreg=None,
-           flash=False, chunk=None, ramp=None, sinks=None, sliding=0, derive=None, phases=0, static=False):
+           flash=False, chunk=None, ramp=None, sinks=None, sliding=0, derive=None, phases=0, static=False,
+           int8_qk=False):
     """Decode and verify windows over paged KV (see the module's description).
 
     q [tokens][heads][dim] BF16 or FP16 (FP16 for "fp16" pages); key_pages/value_pages one layer's pages, key_scales/
@@ -539,8 +538,10 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
     of one element a row, or of one element for every row; not with block lists; such launches take the generic
     kernel, split or fused, the same bits either way. derive: a Derive (or the tuple (weight, eps, freqs, rotary_dim)):
     the keys derived from the value pages on read (key_pages None: the layer keeps value rows only), k = rope(rms_norm(r)
-    * weight, position) in FP32 from the row as stored; head widths 64 and 128, rotary widths in multiples of 16; not
-    with block lists, fresh rows or flash. phases (a measurement's): 1 runs the split
+    * weight, position) in FP32 from the row as stored; any head width and any even rotary width up to it; not
+    with block lists, fresh keys or flash. int8_qk (INT8 pages, fused launches; what prefill passes for the chunks it
+    reads as window rows): the queries as INT8 codes at each row's own scale, a page position's score the exact
+    product of the codes times both scales. phases (a measurement's): 1 runs the split
     launch only, 2 the merge only. static: the launch takes its partials and counters from the library's static device
     array (crit_pkv_attend_static: for callers that cannot allocate; the same bits; launches that overlap on one GPU
     race there; refused past _abi.STATIC_SCRATCH_BYTES of partials); no workspace is read."""
@@ -578,6 +579,11 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
     if fresh is not None and blocks is not None:
         raise ValueError("fresh rows are not read through block lists")
     k_kind = _check_kind(kind, value_scales if derive is not None else key_scales)
+    if int8_qk:
+        if k_kind != 3:
+            raise ValueError("int8_qk multiplies INT8 queries with INT8 keys: int8 pages only")
+        if derive is not None or blocks is not None or flash or not fused:
+            raise ValueError("int8_qk reads windows in the fused launch, without block lists, derived keys or flash")
     _require_device(q, "attend's q")
     T, hq, d = q.shape
     derived, has_weight = (None, False) if derive is None else _derived(derive, d, q.device)
@@ -656,6 +662,7 @@ def attend(q, key_pages, value_pages, kind, tables, rows, starts, firsts, column
     p.kind, p.page_dtype, p.out_dtype = k_kind, _page_dtype(key_pages, kind), _DTYPE[out.dtype]
     p.partitions, p.piece, p.fused, p.sliding, p.phases = parts, piece, int(bool(fused)), sliding, int(phases)
     p.scale, p.key_multiplier, p.value_multiplier = scale, km, vm
+    p.int8_qk = int(bool(int8_qk))
     if fresh is not None:
         fk, fv, fshift, ffirst = fresh
         if derive is not None:      # (checked as the keys the values stand for: one width)
@@ -811,8 +818,6 @@ def _prefill_as_windows(q, key_pages, value_pages, kind, tables, table_rows, sta
     rows of up to MAX_COLUMNS tokens and read by attend()'s fused launch, as crit itself reads prompt rows with
     prompt_reader decode (device_attention.py:751-783). The rows' metadata is computed on the device from the chunks'
     (no length is read on the host)."""
-    if int8_qk:
-        raise _unsupported(f"int8_qk at head width {q.shape[-1]}")
     device, hq = q.device, q.shape[1]
     if q.shape[-1] not in HEAD_WIDTHS:
         raise ValueError(f"head widths are powers of two from 16 to 256, not {q.shape[-1]}")
@@ -839,7 +844,8 @@ def _prefill_as_windows(q, key_pages, value_pages, kind, tables, table_rows, sta
         out = torch.empty(q.shape[0], hq, value_pages.shape[-1], dtype=q.dtype, device=device)
     return attend(q, key_pages, value_pages, kind, tables, w_rows, w_starts, w_firsts, MAX_COLUMNS, page,
                   counts=w_counts, key_scales=key_scales, value_scales=value_scales, multipliers=multipliers,
-                  scale=scale, out=out, lse=lse, fused=True, fresh=given, sinks=sinks, sliding=sliding, derive=derive)
+                  scale=scale, out=out, lse=lse, fused=True, fresh=given, sinks=sinks, sliding=sliding, derive=derive,
+                  int8_qk=int8_qk)
 
 
 def prefill(q, key_pages, value_pages, kind, table, position, page, *, key_scales=None, value_scales=None,

@@ -10,7 +10,7 @@ import shutil
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 NAME = "libcrit_pkv.so"
-ABI_VERSION = 19
+ABI_VERSION = 20
 
 KIND_16BIT, KIND_FP8, KIND_FP8_ROW, KIND_INT8 = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
@@ -44,7 +44,8 @@ class AttendParams(ctypes.Structure):
                 ("fresh_keys", _p), ("fresh_values", _p), ("fresh_shifts", _p), ("fresh_firsts", _p),
                 ("fresh_stride_k", _i64), ("fresh_stride_v", _i64), ("fresh_rows", _i64), ("fresh_per_row", _i32),
                 ("rows_are_64", _i32), ("launch_state", _p),
-                ("derive_table", _p), ("derive_eps", _f32), ("derive_rot", _i32), ("derive_weighted", _i32)]
+                ("derive_table", _p), ("derive_eps", _f32), ("derive_rot", _i32), ("derive_weighted", _i32),
+                ("int8_qk", _i32)]
 
 
 class MergeParams(ctypes.Structure):

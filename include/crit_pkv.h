@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define CRIT_PKV_ABI_VERSION 19
+#define CRIT_PKV_ABI_VERSION 20
 
 /* Page kinds: the values of KINDS in the reference module (__init__.py:78). */
 #define CRIT_PKV_KIND_16BIT 0   /* bf16 or fp16 pages (page_dtype says which) */
@@ -175,13 +175,18 @@ typedef struct crit_pkv_attend_params {
      * rms_norm(r) = r / sqrt(mean(r * r) + derive_eps), the "half" rotation over the first derive_rot values at the
      * angle fp32(position) * freqs[i], all in FP32. derive_table: FP32 freqs [derive_rot / 2], then, with
      * derive_weighted, the weight [head_dim]; NULL: keys from key_pages. With it key_pages and key_scales are not
-     * read (may be NULL); head_dim == value_dim, 64 or 128; derive_rot a multiple of 16 up to head_dim (the reference
-     * takes any even width); no blocks. Fresh rows come as values only (fresh_keys NULL): a fresh position's key is
-     * derived from its fresh value row. */
+     * read (may be NULL); head_dim == value_dim; derive_rot any even width from 2 up to head_dim; no blocks. Fresh rows
+     * come as values only (fresh_keys NULL): a fresh position's key is derived from its fresh value row. */
     const float* derive_table;
     float derive_eps;
     int32_t derive_rot;
     int32_t derive_weighted;
+    /* INT8 pages, fused launches: each query row read as INT8 codes at its own scale (amax / 127, at least 1e-30,
+     * rounded half away from zero) and a page position's score as the exact product of the two rows' codes times both
+     * scales (prefill's int8_qk, __init__.py:1284-1285, _kernels.py:637-643, 668-671, for the prompt chunks that are
+     * read as window rows); fresh positions keep the queries' 16 bits. Not with blocks or derive. Such launches take
+     * the generic kernel whatever the head width. */
+    int32_t int8_qk;
 } crit_pkv_attend_params;
 
 int crit_pkv_attend(const crit_pkv_attend_params* p, void* stream);

@@ -1,7 +1,7 @@
 """Keys derived from the value rows on read (attend's and prefill's derive=): a pool of value pages only, each row read as
 its value and, normed and rotated, as its key. Against float64 attention whose keys are derived in float64 on the host
-(oracle.attend.derived_keys) from the rows as the pages store them: every page kind, heads of 128 and 64, GQA, a rotation
-over part of the head and no norm weight, positions at page boundaries, a long row, a sliding window, sinks, trees; a
+(oracle.attend.derived_keys) from the rows as the pages store them: every page kind, every head width, GQA, a rotation
+over part of the head (any even width) and no norm weight, positions at page boundaries, a long row, a sliding window, sinks, trees; a
 column's bits the same alone, in any window, fused or split; a prompt chunk's tokens the same positions decoded; what the
 reference refuses is refused. Mirrors the reference's tests/test_derived_keys.py at its tolerances (8e-3 + 2e-2 |ref|,
 log-sum-exp 1e-3)."""
@@ -87,7 +87,12 @@ def derive_for(pk, d, rotary_dim, weighted=True, seed=5, packed=True):
 
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("hq,hkv,d,rot,weighted", [(8, 2, 128, 128, True), (12, 2, 64, 64, True), (8, 4, 128, 64, False),
-                                                   (16, 2, 64, 32, True), (3, 1, 128, 16, True)])
+                                                   (16, 2, 64, 32, True), (3, 1, 128, 16, True),
+                                                   # rotary widths whose halves are not whole lanes of 8 elements
+                                                   # (12, 1, 25 and 50 apart), and the other head widths
+                                                   (8, 2, 128, 24, True), (4, 2, 64, 2, False), (8, 2, 64, 50, True),
+                                                   (4, 2, 32, 32, True), (4, 1, 16, 10, False), (6, 2, 256, 100, True),
+                                                   (4, 4, 256, 256, False)])
 @pytest.mark.parametrize("fused", [False, True])
 def test_windows_with_derived_keys_match_float64_attention(kind, hq, hkv, d, rot, weighted, fused):
     # rows whose windows start and end at page boundaries (15/16, 31/32) and one of a single position
@@ -145,12 +150,12 @@ def test_a_tree_with_derived_keys_sees_its_ancestors():
                 seen_of=lambda c, n: (n < 65) | torch.tensor([int(x) - 65 in paths[c] for x in n]))
 
 
-@pytest.mark.parametrize("kind,d", [("bf16", 128), ("fp8", 64)])
-def test_a_prompt_chunk_with_derived_keys_is_its_positions_decoded(kind, d):
+@pytest.mark.parametrize("kind,d,rot", [("bf16", 128, 128), ("fp8", 64, 64), ("int8", 32, 6), ("fp8:row", 256, 200)])
+def test_a_prompt_chunk_with_derived_keys_is_its_positions_decoded(kind, d, rot):
     pk = kernels()
     hq, hkv, T, prefix = 8, 2, 150, 37
     cache = Rows(kind, hkv, d, 16, [prefix + T], seed=6)
-    derive = derive_for(pk, d, d)
+    derive = derive_for(pk, d, rot)
     q = rand_q(T, hq, d, 13).to(cache.q_dtype)
     lse = torch.empty(T, hq, device=dev)
     out = pk.prefill(q, None, cache.v, kind, cache.tables[0], prefix, 16, value_scales=cache.vs, multipliers=cache.multipliers,
@@ -247,7 +252,7 @@ def test_what_derived_keys_do_not_take_is_refused():
                        ((torch.ones(64, device=dev), EPS, freqs, 128), "weight"), ((None, -1.0, freqs, 128), "eps")):
         with pytest.raises(ValueError, match=match):
             cache.attend(q, [0], [0], [39], 1, bad)
-    with pytest.raises(NotImplementedError):      # (the reference takes any even width)
-        cache.attend(q, [0], [0], [39], 1, (None, EPS, freqs[:4], 8))
+    with pytest.raises(ValueError, match="rotary_dim"):      # (any even width is taken; an odd one is not a width)
+        cache.attend(q, [0], [0], [39], 1, (None, EPS, freqs[:4], 9))
     # a plain tuple needs packing, which a capture cannot do; a Derive made by derive() holds its table
     assert derive.table.numel() == 64 + 128

@@ -331,7 +331,7 @@ def test_several_chunks_with_fresh_rows_equal_one_launch_each(kind):
             assert torch.equal(lse[rows], one_lse), s
 
 
-@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 128), (12, 2, 64)])
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 128), (12, 2, 64), (8, 2, 32), (4, 2, 16), (8, 2, 256)])
 def test_int8_queries_against_int8_keys(hq, hkv, d):
     # int8_qk over INT8 pages: the scores are exact integer products of the query rows' INT8 codes (their own scale,
     # amax / 127, half away from zero) and the keys' codes, times both scales: against the oracle with the queries
