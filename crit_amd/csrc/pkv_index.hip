@@ -17,13 +17,14 @@
 //     step go through LDS once for all of them (two buffers, one barrier a step, the next step's loads in flight
 //     under the products), so the keys cross the L2 once per 4 or 8 tokens.
 //
-// Top-k. index_topk_kernel: a workgroup a token (or a slice of its positions). The scores map to 32-bit keys that order
-// as the rule does (NaN lowest, -0 = +0); an 8-bit radix select from the top finds the k-th key and how many of its
-// equals are taken (histograms in 16 copies a bin, so the lanes of a wavefront that meet in a bin meet 4 to an address,
-// and a scan over the bins instead of one thread's walk); then each wavefront takes a quarter of the positions, counts
-// what it will write, and writes the positions of everything above the k-th key and of its first equals in order:
-// ascending by construction. Calls of few tokens over many positions select in slices (the k best of each, positions
-// and scores) and then among the slices' picks: a token's k best are among its slices', in the same order.
+// Top-k. The scores map to 32-bit keys that order as the rule does (NaN lowest, -0 = +0); a radix select from the top
+// finds the k-th key and how many of its equals are taken; then the positions of everything above the k-th key and of
+// its first equals are written in order: ascending by construction.
+//   index_topk_runs_kernel: a workgroup holds a row (or a slice of one) in registers, a thread a run of consecutive
+//     positions: digits of 11, 11 and 10 bits, the places of a thread's picks from its own counts and one scan.
+//   index_topk_kernel: rows no workgroup can hold stream through 8-bit digits, a workgroup a row.
+// Calls of few tokens over many positions select in slices (the k best of each, positions and scores) and then among
+// the slices' picks: a token's k best are among its slices', in the same order.
 #include "pkv_attend_mfma.hpp"
 #include "pkv_launch.hpp"
 
@@ -322,6 +323,12 @@ PKV_DEV uint32_t rank_key(float x) {
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
+// A score that ranks as `key` does (the score itself but for -0, which comes back +0, and a NaN's payload).
+PKV_DEV float score_of_key(uint32_t key) {
+    if (key == 0u) return u2f(0x7fc00000u);
+    return u2f((key & 0x80000000u) ? (key ^ 0x80000000u) : ~key);
+}
+
 // LEVEL 0: a token's row, to its picks. 1: a slice of its row (blockIdx.y), to the slice's candidates (positions and
 // scores, [parts][k] a token). 2: a token's candidates (those with a position), to its picks.
 template <int LEVEL>
@@ -435,17 +442,27 @@ __global__ __launch_bounds__(256) void index_topk_kernel(TopkArgs a) {
 }
 
 
-// The same selection with a workgroup's elements held in registers (up to 1,024 x EPT of them): loaded once, every
-// load in flight at once, where the streaming kernel above pays a round trip to the L2 per 1,024 elements and pass.
-// Element i = j * 1,024 + tid (coalesced loads); for the writes in position order, every 64 consecutive elements (a
-// wavefront's of one j) count what they will write, a scan over those counts gives each its first place.
+// The sum of s_wave[0 .. wave - 1] and of all 16 entries: lane l reads entry l % 16, a scan over the lanes, and the
+// two sums are lanes wave - 1 and 15 of it (`wave` is uniform): a dozen instructions and one LDS round trip, where a
+// loop over the entries before this wavefront's is up to fifteen round trips one after another.
+PKV_DEV unsigned waves_before(const unsigned* s_wave, int wave, int lane, unsigned& total) {
+    const unsigned v = s_wave[lane & 15];
+    const unsigned incl = wave_inclusive_sum(v);
+    total = (unsigned)__builtin_amdgcn_readlane((int)incl, 15);
+    const unsigned upto = (unsigned)__builtin_amdgcn_readlane((int)incl, wave > 0 ? wave - 1 : 0);
+    return wave > 0 ? upto : 0u;
+}
+
 template <int LEVEL, int EPT>
-__global__ __launch_bounds__(1024) void index_topk_held_kernel(TopkArgs a) {
-    __shared__ unsigned s_hist[256 * 16];
-    __shared__ unsigned s_wave[16];
+__global__ __launch_bounds__(1024) void index_topk_runs_kernel(TopkArgs a) {
+    // Four copies of the histogram, a lane's by its number; a copy's bins side by side (a wavefront's lanes that fall into
+    // different bins meet in different banks, and the scan reads a thread's bins as one word or two, no two lanes in a
+    // bank), the copies 16 words out of step, so that a bin's four copies are four banks too.
+    constexpr int COPIES = 4, COPY_WORDS = 2048 + 16;
+    __shared__ __align__(16) unsigned s_hist[COPIES * COPY_WORDS];
+    __shared__ __align__(16) unsigned s_wave[16];
     __shared__ unsigned s_pick[2];
-    __shared__ unsigned s_chunk[EPT * 16];
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int t = blockIdx.x, part = LEVEL == 1 ? blockIdx.y : 0;
     const int end = min(max(a.ends[t], 0), a.n);
     const int k = a.k;
@@ -453,109 +470,166 @@ __global__ __launch_bounds__(1024) void index_topk_held_kernel(TopkArgs a) {
     const int32_t* pos = LEVEL == 2 ? a.pos + (int64_t)t * a.s_stride : nullptr;
     int32_t* out = a.out + (int64_t)t * a.out_stride + (int64_t)part * k;
     float* out_scores = LEVEL == 1 ? a.out_scores + (int64_t)t * a.out_stride + (int64_t)part * k : nullptr;
-    int lo = 0, m, valid;
+    int lo = 0, m, valid, avail;      // avail: the elements the row holds from lo on, whatever `end` says
     if constexpr (LEVEL == 2) {
-        m = a.parts * k, valid = 0;
+        m = a.parts * k, valid = 0, avail = m;
         for (int p = 0; p < a.parts; ++p) valid += min(max(min(end - p * a.width, a.width), 0), k);
     } else {
         lo = LEVEL == 1 ? part * a.width : 0;
         m = max(min(LEVEL == 1 ? a.width : a.n, end - lo), 0), valid = m;
+        avail = max(min(LEVEL == 1 ? a.width : a.n, a.n - lo), 0);
     }
     row += lo;
+    const int first = tid * EPT;
+    const bool mine = first < m;      // this thread's run holds elements of the row
     uint32_t key[EPT];
+    int held_pos[LEVEL == 2 ? EPT : 1];      // LEVEL 2: the candidates' positions, kept for the writes
     using Bits = typename std::conditional<(EPT > 32), uint64_t, uint32_t>::type;
-    Bits ok = 0;      // bit j: element j is a candidate
-    // (loaded 16 at a time: the loads in flight and the keys held share a thread's 128 registers)
-    constexpr int AT_ONCE = EPT > 16 ? 16 : EPT;
+    Bits ok = 0;      // bit j: element first + j is a candidate
 #pragma unroll
-    for (int j0 = 0; j0 < EPT; j0 += AT_ONCE) {
-        float x[AT_ONCE];
-        int at[AT_ONCE];
+    for (int j = 0; j < EPT; ++j) key[j] = 0u;
+    if (mine) {
+        const bool whole = EPT % 4 == 0 && first + EPT <= avail && (reinterpret_cast<uintptr_t>(row) & 15) == 0 &&
+                           (LEVEL != 2 || (reinterpret_cast<uintptr_t>(pos) & 15) == 0);
+        constexpr int AT_ONCE = EPT > 32 ? EPT / 2 : EPT;      // (the loads in flight and the keys held share a thread's registers)
 #pragma unroll
-        for (int jj = 0; jj < AT_ONCE; ++jj) {
-            const int j = j0 + jj;
-            const int i = j * 1024 + tid;
-            x[jj] = (j < EPT && i < m) ? row[i] : 0.0f;
-            at[jj] = 0;
-            if constexpr (LEVEL == 2) at[jj] = (j < EPT && i < m) ? pos[i] : -1;
-        }
+        for (int j0 = 0; j0 < EPT; j0 += AT_ONCE) {
+            float x[AT_ONCE];
+            int at[AT_ONCE];
+            if (whole) {
+                if constexpr (EPT % 4 == 0) {
 #pragma unroll
-        for (int jj = 0; jj < AT_ONCE; ++jj) {
-            const int j = j0 + jj;
-            if (j < EPT) {
-                key[j] = rank_key(x[jj]);
-                if (j * 1024 + tid < m && at[jj] >= 0) ok |= (Bits)1 << j;
+                    for (int q = 0; q < AT_ONCE / 4; ++q) {
+                        const f32x4 v = *reinterpret_cast<const f32x4*>(row + first + j0 + 4 * q);
+                        x[4 * q] = v.x, x[4 * q + 1] = v.y, x[4 * q + 2] = v.z, x[4 * q + 3] = v.w;
+                        if constexpr (LEVEL == 2) {
+                            const u32x4 w = *reinterpret_cast<const u32x4*>(pos + first + j0 + 4 * q);
+                            at[4 * q] = (int)w.x, at[4 * q + 1] = (int)w.y, at[4 * q + 2] = (int)w.z, at[4 * q + 3] = (int)w.w;
+                        } else {
+                            at[4 * q] = at[4 * q + 1] = at[4 * q + 2] = at[4 * q + 3] = 0;
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int jj = 0; jj < AT_ONCE; ++jj) {
+                    const int i = first + j0 + jj;
+                    x[jj] = i < m ? row[i] : 0.0f;
+                    at[jj] = 0;
+                    if constexpr (LEVEL == 2) at[jj] = i < m ? pos[i] : -1;
+                }
+            }
+#pragma unroll
+            for (int jj = 0; jj < AT_ONCE; ++jj) {
+                const int j = j0 + jj;
+                const bool is = first + j < m && at[jj] >= 0;
+                key[j] = is ? rank_key(x[jj]) : 0u;
+                if (is) ok |= (Bits)1 << j;
+                if constexpr (LEVEL == 2) held_pos[j] = at[jj];
             }
         }
     }
-    const bool all = valid <= k;
+    const bool all = valid <= k;      // everything is picked
     uint32_t prefix = 0u;
-    unsigned want = 0u;
+    unsigned want = 0u;               // of the keys equal to the k-th, the `want` first are taken
     if (!all) {
-        uint32_t mask = 0u;
         want = (unsigned)k;
-        for (int shift = 24; shift >= 0; shift -= 8) {
+        static_for<3>([&](auto pass) {
+            constexpr int p = pass;
+            constexpr int kShift[3] = {21, 10, 0}, kDigit[3] = {11, 11, 10};
+            constexpr int shift = kShift[p], bins = 1 << kDigit[p], done = shift + kDigit[p];      // `done`: the bits below the digits already chosen
+            for (int i = tid; i < COPIES * COPY_WORDS / 4; i += 1024) reinterpret_cast<u32x4*>(s_hist)[i] = u32x4{0u, 0u, 0u, 0u};
+            lds_barrier();
+            if (mine) {
+                unsigned* const copy = s_hist + (lane & (COPIES - 1)) * COPY_WORDS;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) s_hist[tid + 1024 * j] = 0u;
-            __syncthreads();
-#pragma unroll
-            for (int j = 0; j < EPT; ++j)
-                if (((ok >> j) & 1u) && (key[j] & mask) == prefix) atomicAdd(&s_hist[((key[j] >> shift) & 255u) * 16 + (lane & 15)], 1u);
-            __syncthreads();
-            unsigned h = 0u, incl = 0u;
-            const int bin = 255 - tid;
-            if (tid < 256) {      // (wavefronts 0 .. 3, whole)
-#pragma unroll
-                for (int j = 0; j < 16; ++j) h += s_hist[bin * 16 + j];
-                incl = wave_inclusive_sum(h);
-                if (lane == 63) s_wave[wave] = incl;
+                for (int j = 0; j < EPT; ++j) {
+                    if constexpr (p == 0) atomicAdd(&copy[key[j] >> 21], 1u);
+                    else if ((key[j] >> (done & 31)) == (prefix >> (done & 31))) atomicAdd(&copy[(key[j] >> shift) & (unsigned)(bins - 1)], 1u);
+                }
             }
-            __syncthreads();
-            if (tid < 256) {
-                for (int w = 0; w < wave; ++w) incl += s_wave[w];
-                if (incl >= want && incl - h < want) s_pick[0] = (unsigned)bin, s_pick[1] = want - (incl - h);
+            lds_barrier();
+            // thread tid: the bins per * tid upwards (per of them); a scan of the counts from bin 0 up, and what lies
+            // above a bin is the total less the scan up to it
+            constexpr int per = bins / 1024;
+            unsigned h[per], sum = 0u;
+#pragma unroll
+            for (int i = 0; i < per; ++i) h[i] = 0u;
+#pragma unroll
+            for (int c = 0; c < COPIES; ++c) {
+                const unsigned* mine_of = s_hist + c * COPY_WORDS + per * tid;
+                if constexpr (per % 4 == 0) {
+#pragma unroll
+                    for (int i = 0; i < per; i += 4) {
+                        const u32x4 v = *reinterpret_cast<const u32x4*>(mine_of + i);
+                        h[i] += v.x, h[i + 1] += v.y, h[i + 2] += v.z, h[i + 3] += v.w;
+                    }
+                } else if constexpr (per == 2) {
+                    const u32x2 v = *reinterpret_cast<const u32x2*>(mine_of);
+                    h[0] += v.x, h[1] += v.y;
+                } else {
+                    h[0] += mine_of[0];
+                }
             }
-            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < per; ++i) sum += h[i];
+            unsigned incl = wave_inclusive_sum(sum);
+            if (lane == 63) s_wave[wave] = incl;
+            lds_barrier();
+            unsigned total;
+            incl += waves_before(s_wave, wave, lane, total);
+            unsigned before = total - incl;      // the keys in the bins above this thread's
+#pragma unroll
+            for (int i = per - 1; i >= 0; --i) {
+                const unsigned upto = before + h[i];
+                if (upto >= want && before < want) s_pick[0] = (unsigned)(tid * per + i), s_pick[1] = want - before;
+                before = upto;
+            }
+            lds_barrier();
             prefix |= s_pick[0] << shift;
-            mask |= 255u << shift;
             want = s_pick[1];
+        });
+    }
+    // What each thread writes (above the k-th key | equal to it << 16), then the places before each thread's. A key of
+    // 0 is a NaN's or that of an element that is no candidate: only where the k-th key is 0 (or everything is picked)
+    // does an element's bit of `ok` decide.
+    const bool plain = !all && prefix != 0u;
+    auto is_above = [&](int j) __attribute__((always_inline)) -> bool {
+        return plain ? key[j] > prefix : (((ok >> j) & 1u) && (all || key[j] > prefix));
+    };
+    auto is_equal = [&](int j) __attribute__((always_inline)) -> bool {
+        return plain ? key[j] == prefix : (((ok >> j) & 1u) && !all && key[j] == prefix);
+    };
+    unsigned n_above = 0u, n_equal = 0u;
+    if (plain) {
+#pragma unroll
+        for (int j = 0; j < EPT; ++j) n_above += key[j] > prefix ? 1u : 0u, n_equal += key[j] == prefix ? 1u : 0u;
+    } else {
+#pragma unroll
+        for (int j = 0; j < EPT; ++j) n_above += is_above(j) ? 1u : 0u, n_equal += is_equal(j) ? 1u : 0u;
+    }
+    const unsigned both = n_above | (n_equal << 16);      // (a row holds fewer than 65,536 elements: no carry between the halves)
+    unsigned incl = wave_inclusive_sum(both);
+    if (lane == 63) s_wave[wave] = incl;
+    lds_barrier();
+    unsigned total;
+    incl += waves_before(s_wave, wave, lane, total);
+    int above_seen = (int)((incl - both) & 0xffffu), equal_seen = (int)((incl - both) >> 16);
+    const int picks = min(valid, k);
+    if (n_above | n_equal) {
+        int place = above_seen + min(equal_seen, (int)want);      // (one further for every element written)
+#pragma unroll
+        for (int j = 0; j < EPT; ++j) {
+            const bool above = is_above(j), equal = is_equal(j);
+            if (above || (equal && equal_seen < (int)want)) {
+                out[place] = LEVEL == 2 ? held_pos[j] : lo + first + j;
+                if constexpr (LEVEL == 1) out_scores[place] = score_of_key(key[j]);
+                ++place;
+            }
+            equal_seen += equal ? 1 : 0;
         }
     }
-    // what each run of 64 elements writes (above the k-th key | equal to it << 16), then the places before each run
-    const unsigned long long below = (1ull << lane) - 1ull;
-#pragma unroll
-    for (int j = 0; j < EPT; ++j) {
-        const bool is = (ok >> j) & 1u;
-        const unsigned n_above = __popcll(__ballot(is && (all || key[j] > prefix)));
-        const unsigned n_equal = __popcll(__ballot(is && !all && key[j] == prefix));
-        if (lane == 0) s_chunk[j * 16 + wave] = n_above | (n_equal << 16);
-    }
-    __syncthreads();
-    {
-        const unsigned v = tid < EPT * 16 ? s_chunk[tid] : 0u;
-        unsigned incl = wave_inclusive_sum(v);
-        if (lane == 63) s_wave[wave] = incl;
-        __syncthreads();
-        for (int w = 0; w < wave; ++w) incl += s_wave[w];
-        if (tid < EPT * 16) s_chunk[tid] = incl - v;
-        __syncthreads();
-    }
-#pragma unroll
-    for (int j = 0; j < EPT; ++j) {
-        const bool is = (ok >> j) & 1u;
-        const bool above = is && (all || key[j] > prefix), equal = is && !all && key[j] == prefix;
-        const unsigned long long above_mask = __ballot(above), equal_mask = __ballot(equal);
-        const unsigned before = s_chunk[j * 16 + wave];
-        const int rank = (int)(before >> 16) + __popcll(equal_mask & below);
-        if (above || (equal && rank < (int)want)) {
-            const int i = j * 1024 + tid;
-            const int place = (int)(before & 0xffffu) + __popcll(above_mask & below) + min(rank, (int)want);
-            if constexpr (LEVEL == 2) out[place] = pos[i];
-            else out[place] = lo + i;
-            if constexpr (LEVEL == 1) out_scores[place] = row[i];
-        }
-    }
-    for (int i = min(valid, k) + tid; i < k; i += 1024) out[i] = -1;
+    for (int i = picks + tid; i < k; i += 1024) out[i] = -1;
 }
 
 template <bool F16, bool FP8, int HT, int KS>
@@ -635,9 +709,9 @@ int launch_scores_kind(const ScoreArgs& a, int dim, bool many, int cus, hipStrea
 // else streams, a workgroup a row.
 constexpr int kHeld = 32768;
 // Calls of many rows hold rows of up to kHeldWide elements whole, a workgroup a row (no slices, no candidates' pass:
-// measured for rows of 50,000 and k = 2,048: 320 against 432 us in slices for 2,048 rows, 43 against 58 for 256, 39
-// against 40 for 128; 64 rows take 30 us in slices, which spread a row over compute units, and 38 whole). Short of 65,536 so that the counts of equal keys before a
-// run of 64 elements fit their 16 bits.
+// measured for rows of 50,000 and k = 2,048: 253 against 432 us in slices for 2,048 rows, 37 against 58 for 256; 64 rows
+// take 22 us in slices, which spread a row over compute units, and 38 whole). Short of 65,536 so that the counts of
+// the keys above and equal to the k-th fit 16 bits each.
 constexpr int kHeldWide = 64512;
 constexpr int kManyRows = 128;
 constexpr int64_t kSliceRoom = (int64_t)512 << 20;
@@ -647,7 +721,7 @@ struct TopkPlan {
 };
 // Elements a thread of the holding kernel for `elements` of a row (what launch_topk_level picks).
 int held_elements(int elements) {
-    const int steps[] = {8, 12, 14, 16, 24, 32};
+    const int steps[] = {8, 12, 16, 24, 32};
     for (int e : steps)
         if (elements <= e * 1024) return e;
     return 0;
@@ -656,10 +730,10 @@ TopkPlan topk_plan(int tokens, int n, int k, int cus) {
     TopkPlan plan = {0, n};
     (void)cus;
     if (n <= kHeld || tokens > 65535 || (n <= kHeldWide && tokens >= kManyRows)) return plan;
-    // Slices: the fewest microseconds by what the holding kernel was measured to take, 4.2 us and 0.53 us an element
-    // a thread (the candidates' pass, which also loads positions, 1.3 times that): for a few rows the two launches one
+    // Slices: the fewest microseconds by what the holding kernel was measured to take, 4.3 us and 0.42 us an element
+    // a thread (the candidates' pass, which also loads positions, 1.15 times that): for a few rows the two launches one
     // after the other, for many rows every slice's workgroup counts. (50,000 positions, k = 2,048: 4 slices of 12,544
-    // and 8,192 candidates, 22 us where 7 slices of 8,192 and 14,336 candidates took 25.)
+    // and 8,192 candidates, 20 us.)
     const int64_t fewest = ((int64_t)n + kHeld - 1) / kHeld;
     const int64_t most = min((int64_t)kHeld / k, min((int64_t)65535, max(fewest * 8, (int64_t)16)));
     float best = 0.0f;
@@ -667,7 +741,7 @@ TopkPlan topk_plan(int tokens, int n, int k, int cus) {
         const int width = (int)((((int64_t)n + parts - 1) / parts + 63) / 64 * 64);
         const int e1 = held_elements(width), e2 = held_elements((int)(parts * k));
         if (!e1 || !e2 || (int64_t)tokens * parts * k * 8 > kSliceRoom) continue;
-        const float slices = 4.2f + 0.53f * e1, candidates = 1.3f * (4.2f + 0.53f * e2);
+        const float slices = 4.3f + 0.42f * e1, candidates = 1.15f * (4.3f + 0.42f * e2);
         const float cost = (tokens >= kManyRows ? (float)parts : 1.0f) * slices + candidates;
         if (plan.parts == 0 || cost < best) best = cost, plan.parts = (int)parts, plan.width = width;
     }
@@ -676,18 +750,19 @@ TopkPlan topk_plan(int tokens, int n, int k, int cus) {
 
 template <int LEVEL>
 void launch_topk_level(const TopkArgs& a, int elements, dim3 grid, hipStream_t stream) {
-    // (elements a thread: every one costs the same in each pass whether it is there or not, so the count is cut close)
-    if (elements <= 8192) hipLaunchKernelGGL((index_topk_held_kernel<LEVEL, 8>), grid, dim3(1024), 0, stream, a);
-    else if (elements <= 12288) hipLaunchKernelGGL((index_topk_held_kernel<LEVEL, 12>), grid, dim3(1024), 0, stream, a);
-    else if (elements <= 14336) hipLaunchKernelGGL((index_topk_held_kernel<LEVEL, 14>), grid, dim3(1024), 0, stream, a);
-    else if (elements <= 16384) hipLaunchKernelGGL((index_topk_held_kernel<LEVEL, 16>), grid, dim3(1024), 0, stream, a);
-    else if (elements <= 24576) hipLaunchKernelGGL((index_topk_held_kernel<LEVEL, 24>), grid, dim3(1024), 0, stream, a);
-    else if (elements <= kHeld) hipLaunchKernelGGL((index_topk_held_kernel<LEVEL, 32>), grid, dim3(1024), 0, stream, a);
-    else if (LEVEL == 0 && elements <= 40960 && (int)grid.x >= kManyRows) hipLaunchKernelGGL((index_topk_held_kernel<0, 40>), grid, dim3(1024), 0, stream, a);
-    else if (LEVEL == 0 && elements <= 49152 && (int)grid.x >= kManyRows) hipLaunchKernelGGL((index_topk_held_kernel<0, 48>), grid, dim3(1024), 0, stream, a);
-    else if (LEVEL == 0 && elements <= 57344 && (int)grid.x >= kManyRows) hipLaunchKernelGGL((index_topk_held_kernel<0, 56>), grid, dim3(1024), 0, stream, a);
-    else if (LEVEL == 0 && elements <= kHeldWide && (int)grid.x >= kManyRows) hipLaunchKernelGGL((index_topk_held_kernel<0, 63>), grid, dim3(1024), 0, stream, a);
+    // (elements a thread: threads past the row's end skip the passes, so the count only has to hold the row)
+#define PKV_RUNS(L, E) hipLaunchKernelGGL((index_topk_runs_kernel<L, E>), grid, dim3(1024), 0, stream, a)
+    if (elements <= 8192) PKV_RUNS(LEVEL, 8);
+    else if (elements <= 12288) PKV_RUNS(LEVEL, 12);
+    else if (elements <= 16384) PKV_RUNS(LEVEL, 16);
+    else if (elements <= 24576) PKV_RUNS(LEVEL, 24);
+    else if (elements <= kHeld) PKV_RUNS(LEVEL, 32);
+    else if (LEVEL == 0 && elements <= 40960 && (int)grid.x >= kManyRows) PKV_RUNS(0, 40);
+    else if (LEVEL == 0 && elements <= 49152 && (int)grid.x >= kManyRows) PKV_RUNS(0, 48);
+    else if (LEVEL == 0 && elements <= 57344 && (int)grid.x >= kManyRows) PKV_RUNS(0, 56);
+    else if (LEVEL == 0 && elements <= kHeldWide && (int)grid.x >= kManyRows) PKV_RUNS(0, 64);
     else hipLaunchKernelGGL(index_topk_kernel<LEVEL>, grid, dim3(256), 0, stream, a);
+#undef PKV_RUNS
 }
 
 }   // namespace
