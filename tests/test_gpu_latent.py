@@ -2,8 +2,8 @@
 rows as the cache stores them: decode tokens and verify windows over shuffled pages at the ranks and heads of the models
 that use it, sinks and log-sum-exps, BF16, FP16 and E4M3 caches (two scales a position, or one); a token's bits the same
 alone, in a verify window, beside other rows, fused or not and in a prompt chunk; one graph replayed at other lengths;
-what the module refuses. Mirrors the reference's kernels/techniques/attention/latent-attention/tests/
-test_latent_attention.py at its tolerances (8e-3 + 2e-2 |ref|; log-sum-exp 1e-3). Calls go through the module, which
+what the module refuses. The cases cover those of the reference's kernels/techniques/attention/latent-attention/tests/
+test_latent_attention.py, at its tolerances (8e-3 + 2e-2 |ref|; log-sum-exp 1e-3). Calls go through the module, which
 reaches the HIP kernels through the C ABI."""
 import pytest
 import torch
@@ -20,56 +20,69 @@ def module():
 
 
 class Cache:
-    """Sequences of compressed rows (latent R, rotary key P) over shuffled pages, written by the module's write()."""
+    """A latent cache of several sequences: a position's row is its latent (R values) then its rotary key (P values),
+    appended by the module's own write() into pages handed out from a shuffled list, a spare page a sequence. scales: 0
+    (a 16-bit cache), 2 (E4M3 codes, the latent and the rotary key each at its own scale) or 1 (E4M3 codes at one
+    scale a row, as a KV pool's fp8:row pages of one head hold them)."""
 
     def __init__(self, rank, rope, page, lengths, seed=0, dtype=torch.bfloat16, scales=0):
         self.la = module()
-        g = torch.Generator().manual_seed(seed)
         self.rank, self.rope, self.page = rank, rope, page
-        width = max(-(-n // page) for n in lengths) + 1
-        n_pages = width * len(lengths) + 2
-        self.cache = torch.zeros(n_pages, page, rank + rope, dtype=dtype, device=dev)
-        self.scales = torch.zeros(n_pages, page, 2, device=dev) if scales else None
-        order = torch.randperm(n_pages, generator=g)
-        self.tables = order[:width * len(lengths)].view(len(lengths), width).to(torch.int32).to(dev)
+        draw = torch.Generator().manual_seed(seed)
+        each = 1 + max((n + page - 1) // page for n in lengths)
+        total = each * len(lengths) + 2
+        self.tables = torch.randperm(total, generator=draw)[:each * len(lengths)].reshape(len(lengths), each).to(
+            device=dev, dtype=torch.int32)
+        self.cache = torch.zeros(total, page, rank + rope, dtype=dtype, device=dev)
+        self.scales = torch.zeros(total, page, 2, device=dev) if scales else None
         for s, n in enumerate(lengths):
-            latent = torch.randn(n, rank, generator=g).to(dev)
-            rope_k = torch.randn(n, rope, generator=g).to(dev) * (3 if scales else 1)
-            self.la.write(latent, rope_k, self.slots(s, torch.arange(n, device=dev)), self.cache, self.scales)
-        if scales == 1:      # one scale a row (a KV pool's fp8:row pages of one head): recode each row at one scale
-            rows = self.cache.view(-1, rank + rope).float() * torch.cat(
-                [self.scales.view(-1, 2)[:, :1].expand(-1, rank), self.scales.view(-1, 2)[:, 1:].expand(-1, rope)], 1)
-            one = (rows.abs().amax(-1) / 448.0).clamp(min=1e-30)
-            self.cache = (rows / one[:, None]).clamp(-448, 448).to(torch.float8_e4m3fn).view(n_pages, page, rank + rope)
-            self.scales = one.view(n_pages, page, 1).contiguous()
+            latent = torch.randn(n, rank, generator=draw).to(dev)
+            rotary = torch.randn(n, rope, generator=draw).to(dev) * (3 if scales else 1)      # (two scales that differ)
+            self.la.write(latent, rotary, self.slot_of(s, torch.arange(n, device=dev)), self.cache, self.scales)
+        if scales == 1:
+            self._recode_at_one_scale(total)
 
-    def slots(self, s, positions):
-        return self.tables[s][positions // self.page].long() * self.page + positions % self.page
+    def _recode_at_one_scale(self, total):
+        width = self.rank + self.rope
+        two = self.scales.reshape(-1, 2)
+        by_value = torch.cat([two[:, :1].expand(-1, self.rank), two[:, 1:].expand(-1, self.rope)], dim=1)
+        values = self.cache.reshape(-1, width).float() * by_value
+        one = (values.abs().amax(dim=-1) / 448.0).clamp(min=1e-30)
+        codes = (values / one.unsqueeze(-1)).clamp(-448, 448).to(torch.float8_e4m3fn)
+        self.cache, self.scales = codes.reshape(total, self.page, width), one.reshape(total, self.page, 1).contiguous()
+
+    def slot_of(self, s, positions):
+        pages = self.tables[s].long()[torch.div(positions, self.page, rounding_mode="floor")]
+        return pages * self.page + positions % self.page
 
     def rows(self, s, n):
-        return oracle_latent.stored(self.cache.cpu(), None if self.scales is None else self.scales.cpu(), self.tables[s].cpu(),
-                                    n, self.page, self.rank)
+        """Positions 0 .. n - 1 of sequence s as the cache stores them: (latent [n][R], rotary key [n][P]), float64."""
+        scales = None if self.scales is None else self.scales.cpu()
+        return oracle_latent.stored(self.cache.cpu(), scales, self.tables[s].cpu(), n, self.page, self.rank)
 
     def attend(self, q, rows, starts, firsts, columns, **kw):
-        return self.la.attend(q, self.cache, self.tables, torch.tensor(rows, dtype=torch.int32, device=dev),
-                              torch.tensor(starts, dtype=torch.int32, device=dev),
+        ints = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+        return self.la.attend(q, self.cache, self.tables, ints(rows), ints(starts),
                               torch.tensor(firsts, dtype=torch.int64, device=dev), columns, self.page, rank=self.rank,
                               scales=self.scales, **kw)
 
     def check(self, q, out, lse, s, start, first, count, scale, sinks=None, lse_tol=1e-3):
-        latent, rope_k = self.rows(s, first + count)
-        seen = torch.arange(first + count)[None, :] <= first + torch.arange(count)[:, None]
-        span = slice(start, start + count)
-        qc = q[span].double().cpu()
-        want, want_lse = oracle_latent.latent_attention(qc[:, :, :self.rank], qc[:, :, self.rank:], latent, rope_k, seen, scale,
-                                                        None if sinks is None else sinks.cpu())
-        torch.testing.assert_close(out[span].double().cpu(), want, atol=8e-3, rtol=2e-2)
+        """Tokens start .. start + count - 1 against float64 latent attention of window row (s, first, count)."""
+        latent, rotary = self.rows(s, first + count)
+        own = first + torch.arange(count)
+        seen = torch.arange(first + count).unsqueeze(0) <= own.unsqueeze(1)
+        tokens = slice(start, start + count)
+        queries = q[tokens].double().cpu()
+        want, want_lse = oracle_latent.latent_attention(queries[..., :self.rank], queries[..., self.rank:], latent, rotary, seen,
+                                                        scale, None if sinks is None else sinks.cpu())
+        torch.testing.assert_close(out[tokens].double().cpu(), want, atol=8e-3, rtol=2e-2)
         if lse is not None:
-            torch.testing.assert_close(lse[span].double().cpu(), want_lse, atol=lse_tol, rtol=1e-4)
+            torch.testing.assert_close(lse[tokens].double().cpu(), want_lse, atol=lse_tol, rtol=1e-4)
 
 
 def _q(tokens, heads, width, seed, dtype=torch.bfloat16):
-    return (torch.randn(tokens, heads, width, generator=torch.Generator().manual_seed(seed)) * 0.5).to(dev, dtype)
+    draw = torch.Generator().manual_seed(seed)
+    return torch.randn(tokens, heads, width, generator=draw).mul_(0.5).to(dev, dtype)
 
 
 @pytest.mark.parametrize("rank,rope,heads,page", [(512, 64, 16, 64), (512, 64, 128, 16), (256, 64, 8, 32), (128, 32, 20, 16),
