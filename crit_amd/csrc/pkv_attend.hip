@@ -312,6 +312,12 @@ static int launch_attend_checked(const crit_pkv_attend_params* p, hipStream_t st
         if ((1 << s) == p->page) a.page_shift = s;
     a.parts = p->partitions, a.piece = p->piece, a.sliding = p->sliding, a.out_dtype = p->out_dtype;
     a.sscale = p->scale * kLog2e, a.k_mult = p->key_multiplier, a.v_mult = p->value_multiplier;
+    // 64-wide heads over an even number of KV heads: pairs of adjacent heads go through the bandwidth kernel as
+    // 128-wide ones (what decides is the cache's geometry and the call's kind, never the launch's size)
+    a.narrow = (p->head_dim == 64 && p->value_dim == 64 && p->kv_heads % 2 == 0 && !derive && !p->blocks && !a.iqk &&
+                !(p->fresh_keys || p->fresh_values) && p->page % 16 == 0 && a.page_shift >= 4 &&
+                (int64_t)p->partitions * p->piece <= 0x3fffffff && p->piece % 16 == 0) ? 1 : 0;
+    if (a.narrow) a.hkv = p->kv_heads / 2, a.g *= 2, a.dk = a.dv = 128;
     const int live_rows = p->columns * a.g;
     int qr = pick_qr(live_rows);
     if (p->blocks) {      // a tile of one column's rows: the largest tile height that divides the group
@@ -331,8 +337,8 @@ static int launch_attend_checked(const crit_pkv_attend_params* p, hipStream_t st
     // The bandwidth kernel walks pages that are powers of two from 16 positions up, in positions below 2^31; other
     // multiples of 16 take the generic kernel. (block lists of blocks that are a multiple of 16: their own variant)
     const bool pow2_page = a.page_shift >= 4 && (int64_t)p->partitions * p->piece <= 0x3fffffff;
-    a.fast128 = !derive && !a.iqk && (((wide128 || wide256) && page16 && pow2_page && p->piece % 16 == 0) || fast_lists);      // (derived keys: the generic kernel)
-    if (a.fast128 && wide128 && p->kv_heads % 2 == 0) a.heads_per_wave = 2;
+    a.fast128 = a.narrow || (!derive && !a.iqk && (((wide128 || wide256) && page16 && pow2_page && p->piece % 16 == 0) || fast_lists));      // (derived keys: the generic kernel)
+    if (a.fast128 && (wide128 || a.narrow) && a.hkv % 2 == 0) a.heads_per_wave = 2;
     // Query rows a tile holds: the generic and block-list kernels' tile height; 16 a wavefront's heads share in the
     // bandwidth kernel (matrix tiles of 16 columns).
     const int tile_rows = a.fast128 && !p->blocks ? 16 / a.heads_per_wave : qr;
@@ -367,7 +373,7 @@ static int launch_attend_checked(const crit_pkv_attend_params* p, hipStream_t st
         a.query_tiles = 2;
         a.tiles = (a.tiles + a.query_tiles - 1) / a.query_tiles;
     }
-    const int64_t gx = (int64_t)p->n_rows * (p->kv_heads / a.heads_per_wave) * a.tiles;
+    const int64_t gx = (int64_t)p->n_rows * (a.hkv / a.heads_per_wave) * a.tiles;
     if (gx > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
     // Positions past the page tables do not exist: partitions that could only hold such pieces are not launched.
     const int64_t table_keys = (int64_t)p->table_width * p->page;

@@ -56,6 +56,7 @@ struct AttendArgs {
     const float* derive_table;
     float derive_eps;
     int derive_rot, derive_weighted;
+    int narrow;   // 64-wide heads read in pairs as 128-wide ones: hkv, g, dk and dv above are the pairs' (half, twice, 128, 128)
     int iqk;      // INT8 pages: the queries as INT8 codes at each row's own scale (prefill's int8_qk read as windows)
 };
 

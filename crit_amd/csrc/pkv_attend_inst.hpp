@@ -118,7 +118,7 @@ static int launch_mfma(const AttendArgs& a, bool fused, dim3 grid, hipStream_t s
     // finished workgroups are a few microseconds at the end of a launch that is one unit long).
     if (units <= resident) u.ticket = nullptr;
     const bool masked = a.parents != nullptr || a.parents64 != nullptr || a.sliding > 0;
-    const int which = (a.dk == 256 ? 8 : (a.heads_per_wave == 2 ? 4 : 0)) + (fused ? 2 : 0) + (masked ? 1 : 0) +
+    const int which = (a.narrow ? 64 : 0) + (a.dk == 256 ? 8 : (a.heads_per_wave == 2 ? 4 : 0)) + (fused ? 2 : 0) + (masked ? 1 : 0) +
                       (a.query_tiles == 4 ? 12 : (a.query_tiles == 2 ? 24 : 0));
     switch (which) {
 #define PKV_MFMA(W, HWV, FU, MA, DH) \
@@ -127,6 +127,12 @@ static int launch_mfma(const AttendArgs& a, bool fused, dim3 grid, hipStream_t s
         PKV_MFMA(4, 2, false, false, 1) PKV_MFMA(5, 2, false, true, 1) PKV_MFMA(6, 2, true, false, 1) PKV_MFMA(7, 2, true, true, 1)
         PKV_MFMA(8, 1, false, false, 2) PKV_MFMA(9, 1, false, true, 2) PKV_MFMA(10, 1, true, false, 2) PKV_MFMA(11, 1, true, true, 2)
 #undef PKV_MFMA
+        // 64-wide heads in pairs
+#define PKV_MFMA_NARROW(W, HWV, FU, MA) \
+    case 64 + W: hipLaunchKernelGGL((attend_mfma_kernel<KIND, F16, HWV, FU, MA, 1, 1, true>), pgrid, dim3(256), 0, stream, u); break;
+        PKV_MFMA_NARROW(0, 1, false, false) PKV_MFMA_NARROW(1, 1, false, true) PKV_MFMA_NARROW(2, 1, true, false) PKV_MFMA_NARROW(3, 1, true, true)
+        PKV_MFMA_NARROW(4, 2, false, false) PKV_MFMA_NARROW(5, 2, false, true) PKV_MFMA_NARROW(6, 2, true, false) PKV_MFMA_NARROW(7, 2, true, true)
+#undef PKV_MFMA_NARROW
         // four query tiles a workgroup: split launches of 128-wide heads over 16-bit pages
 #define PKV_MFMA_QT(W, HWV, MA) \
     case W:                                                                                                                  \

@@ -134,8 +134,17 @@ constexpr int kMfmaTiles = 2;
 // workgroups a compute unit), where it measured faster (64 rows ~U[1024, 8192] of 32 / 8 heads, 8 columns: 676 -> 480 us, FP8 376 -> 224);
 // pairs of tiles of 256-wide heads keep one step in flight a wavefront instead of two (NT), or their registers spill;
 // four tiles of 8-bit pages measured slower.
-template <int KIND, bool F16, int HW, bool FUSED, bool MASKED, int DH = 1, int QT = 1>
+// NARROW: 64-wide heads, read as 128-wide ones. Two adjacent KV heads' rows of a position are 128 contiguous values,
+// which is what a 128-wide head's row is: the launcher hands the kernel half the KV heads at twice the width and GQA
+// groups twice as large (a group's first half the query heads of the even KV head, its second half the odd one's: the
+// query heads' own order). A query row enters the first product with zeros in the other head's 64 dims (exact: the
+// products with them are zeros), so its scores are its own head's; the second product gives it 128 output dims of
+// which its own head's 64 are kept. Twice the matrix work a byte, on a pipe this kernel leaves nine tenths idle, for
+// the 128-wide kernel's loads: 512 contiguous bytes a position and wavefront. What follows a KV head (row scales, an
+// FP8 pool's multipliers) is looked up by the column's own head.
+template <int KIND, bool F16, int HW, bool FUSED, bool MASKED, int DH = 1, int QT = 1, bool NARROW = false>
 __global__ __launch_bounds__(256, (DH == 2 || QT > 2) ? 1 : kMfmaWaves) void attend_mfma_kernel(AttendArgs a) {
+    static_assert(!NARROW || (DH == 1 && QT == 1), "64-wide heads: one 128-wide pair a tile row, one tile a workgroup");
     constexpr int NT = DH == 2 && QT == 2 ? 1 : kMfmaTiles;
     constexpr int D = 128 * DH;
     static_assert(DH == 1 || (DH == 2 && HW == 1), "heads of 128 or 256; one KV head a wavefront at 256");
@@ -378,16 +387,24 @@ __global__ __launch_bounds__(256, (DH == 2 || QT > 2) ? 1 : kMfmaWaves) void att
     // Loads of one step from its first slot. Every lane loads its place of the step whether the row holds that
     // position or not (the page does; a step past the row's keys is never listed): what such a place holds is dropped
     // where it is used (keys: the score is masked; values and scales: zeroed, see sanitize()).
-    auto fetch_k = [&](const Unit& un, int64_t slot0, Tile<KIND, DH>& t) __attribute__((always_inline)) {
+    // (NARROW: `odd`, whether this lane's column is a query row of the pair's odd KV head; the scales are per KV head)
+    auto fetch_k = [&](const Unit& un, int64_t slot0, Tile<KIND, DH>& t, int odd) __attribute__((always_inline)) {
         const uint8_t* sbase = a.kp + slot0 * slot_bytes + un.kvh0 * D * EB;
 #pragma unroll
         for (int c = 0; c < (KIND == 0 ? 4 : 2) * DH; ++c) t.k[c] = *reinterpret_cast<const u32x4*>(sbase + kvo + 64 * c);
         if constexpr (KIND >= 2) {
-            const float* ks = a.ks + slot0 * a.hkv + un.kvh0;
-            const float* vs = a.vs + slot0 * a.hkv + un.kvh0;
+            const int heads = NARROW ? 2 * a.hkv : a.hkv;      // scales a slot
+            const int first = NARROW ? (int)svo * 2 + odd : (int)svo;      // (svo = r_pos * hkv + r_head)
+            const float* ks = a.ks + slot0 * heads + (NARROW ? 2 * un.kvh0 : un.kvh0);
+            const float* vs = a.vs + slot0 * heads + (NARROW ? 2 * un.kvh0 : un.kvh0);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) t.ks[i] = ks[svo + i * a.hkv], t.vs[i] = vs[svo + i * a.hkv];
+            for (int i = 0; i < 4; ++i) t.ks[i] = ks[first + i * heads], t.vs[i] = vs[first + i * heads];
         }
+    };
+    // NARROW: whether this lane's tile column (a query row of the flattened list) belongs to the pair's odd KV head.
+    auto odd_of = [&](const Unit& un) __attribute__((always_inline)) -> int {
+        if constexpr (!NARROW) return 0;
+        return ((un.j0 + c16 % CPH) % a.g) >= (a.g >> 1) ? 1 : 0;
     };
     auto fetch_v = [&](const Unit& un, int64_t slot0, Tile<KIND, DH>& t) __attribute__((always_inline)) {
         const uint8_t* sbase = a.vp + slot0 * slot_bytes + un.kvh0 * D * EB;
@@ -417,7 +434,8 @@ __global__ __launch_bounds__(256, (DH == 2 || QT > 2) ? 1 : kMfmaWaves) void att
         }
     };
     auto lane_values = [&](const Unit& un) __attribute__((always_inline)) {
-        if constexpr (KIND == 1) sscale = a.sscale * (a.hm ? a.hm[un.kvh0 + hsel] : a.k_mult);
+        const int odd = odd_of(un);
+        if constexpr (KIND == 1) sscale = a.sscale * (a.hm ? a.hm[NARROW ? 2 * (un.kvh0 + hsel) + odd : un.kvh0 + hsel] : a.k_mult);
 #pragma unroll
         for (int q = 0; q < QT; ++q) {
             const int jr = un.j0 + q * CPH + c16 % CPH;
@@ -432,7 +450,11 @@ __global__ __launch_bounds__(256, (DH == 2 || QT > 2) ? 1 : kMfmaWaves) void att
                 // 16-bit pages: dims 32 c + 8 u4 ..; 8-bit pages: dims 64 (c / 2) + 16 u4 + 8 (c % 2) .. (the codes a lane's two loads hold)
                 const int dim = KIND == 0 ? 32 * c + 8 * u4 : 64 * (c / 2) + 16 * u4 + 8 * (c % 2);
                 qb[q][c] = u32x4{0, 0, 0, 0};
-                if (live) qb[q][c] = *reinterpret_cast<const u32x4*>(row + dim * 2);
+                if constexpr (NARROW) {      // the column's own head's 64 dims, zeros in the other head's
+                    if (live && (dim >> 6) == odd) qb[q][c] = *reinterpret_cast<const u32x4*>(row + (dim & 63) * 2);
+                } else {
+                    if (live) qb[q][c] = *reinterpret_cast<const u32x4*>(row + dim * 2);
+                }
             }
         }
     };
@@ -440,10 +462,11 @@ __global__ __launch_bounds__(256, (DH == 2 || QT > 2) ? 1 : kMfmaWaves) void att
     Tile<KIND, DH> t[NT];
     auto fill = [&](const Unit& un, const Lead& f) __attribute__((always_inline)) {      // a partition's first NT steps
         const int again = f.base[0] >= 0 ? f.base[0] : 0;
+        const int odd = odd_of(un);
 #pragma unroll
         for (int i = 0; i < NT; ++i) {
             const int64_t slot = first_slot(f.base[i] >= 0 ? f.base[i] : again, f.e[i]);
-            fetch_k(un, slot, t[i]), fetch_v(un, slot, t[i]);
+            fetch_k(un, slot, t[i], odd), fetch_v(un, slot, t[i]);
         }
     };
 
@@ -615,6 +638,7 @@ __global__ __launch_bounds__(256, (DH == 2 || QT > 2) ? 1 : kMfmaWaves) void att
                 // the wavefront's last steps are peeled: no step is loaded that is not used (a re-read of an earlier
                 // step would come from HBM again: the caches have long turned over).
                 Lead f = lead_cur;
+                const int odd_cur = odd_of(cur);
                 if (part != part_lo) {
                     f = lead_of(cur, part);
                     fill(cur, f);
@@ -630,7 +654,7 @@ __global__ __launch_bounds__(256, (DH == 2 || QT > 2) ? 1 : kMfmaWaves) void att
                             const int after = walk_advance(cur, f.w);      // NT steps past the one this buffer is refilled with
                             const int e_after = entry(cur, after >= 0 ? after : again);
                             const int64_t slot = first_slot(ahead[i], e_ahead[i]);
-                            step(at[i], t[i], [&]() __attribute__((always_inline)) { fetch_k(cur, slot, t[i]); },
+                            step(at[i], t[i], [&]() __attribute__((always_inline)) { fetch_k(cur, slot, t[i], odd_cur); },
                                  [&]() __attribute__((always_inline)) { fetch_v(cur, slot, t[i]); });
                             at[i] = ahead[i], ahead[i] = after, e_ahead[i] = e_after;
                         }
@@ -640,7 +664,7 @@ __global__ __launch_bounds__(256, (DH == 2 || QT > 2) ? 1 : kMfmaWaves) void att
                         if (at[i] >= 0) {
                             const bool again_i = ahead[i] >= 0;
                             const int64_t slot = first_slot(again_i ? ahead[i] : again, e_ahead[i]);
-                            step(at[i], t[i], [&]() __attribute__((always_inline)) { if (again_i) fetch_k(cur, slot, t[i]); },
+                            step(at[i], t[i], [&]() __attribute__((always_inline)) { if (again_i) fetch_k(cur, slot, t[i], odd_cur); },
                                  [&]() __attribute__((always_inline)) { if (again_i) fetch_v(cur, slot, t[i]); });
                         }
                     }
@@ -687,8 +711,14 @@ __global__ __launch_bounds__(256, (DH == 2 || QT > 2) ? 1 : kMfmaWaves) void att
                         L = __builtin_fmaf(s_l[w][cc], fw, L);
                         A = __builtin_fmaf(s_acc[w][cc][d], fw, A);
                     }
-                    if constexpr (KIND == 1) A *= HW == 1 ? vm_cur[0] : (head_i == 0 ? vm_cur[0] : vm_cur[HW - 1]);
-                    if (c < cur.count) {
+                    // NARROW: the element is kept where its dim lies in the 64 of its column's own KV head
+                    const int odd = NARROW ? ((j % a.g) >= (a.g >> 1) ? 1 : 0) : 0;
+                    const bool kept = !NARROW || (d >> 6) == odd;
+                    if constexpr (KIND == 1) {
+                        if constexpr (NARROW) A *= a.hm ? a.hm[2 * a.hkv + 2 * (fold_kvh0 + head_i) + odd] : a.v_mult;
+                        else A *= HW == 1 ? vm_cur[0] : (head_i == 0 ? vm_cur[0] : vm_cur[HW - 1]);
+                    }
+                    if (c < cur.count && kept) {
                         if constexpr (FUSED) {
                             // A column folds the partitions that hold its positions, as the merge does.
                             const int held = min(a.parts, (min(cur.first + c + 1, a.max_keys) + a.piece - 1) / a.piece);
@@ -699,8 +729,9 @@ __global__ __launch_bounds__(256, (DH == 2 || QT > 2) ? 1 : kMfmaWaves) void att
                             }
                         } else {
                             const int64_t at = ((int64_t)(cur.prow + c) * a.hq + (fold_kvh0 + head_i) * a.g + j % a.g) * a.parts + cur.b;
-                            a.po[at * D + d] = A;
-                            if (d == 0) a.pm[at] = M, a.pl[at] = L;
+                            if constexpr (NARROW) a.po[at * 64 + (d & 63)] = A;
+                            else a.po[at * D + d] = A;
+                            if ((d & (NARROW ? 63 : D - 1)) == 0) a.pm[at] = M, a.pl[at] = L;
                         }
                     }
                 }
@@ -713,7 +744,8 @@ __global__ __launch_bounds__(256, (DH == 2 || QT > 2) ? 1 : kMfmaWaves) void att
                     const int cc = idx / D, d = idx % D;
                     const int j = cur.j0 + cc % CPH;
                     const int c = j / a.g;
-                    if (c < cur.count) {
+                    const bool kept = !NARROW || (d >> 6) == ((j % a.g) >= (a.g >> 1) ? 1 : 0);
+                    if (c < cur.count && kept) {
                         const int head = (cur.kvh0 + cc / CPH) * a.g + j % a.g;
                         float M = run_m[e], L = run_l[e], A = run_a[e];
                         if (a.sinks) {
@@ -721,8 +753,8 @@ __global__ __launch_bounds__(256, (DH == 2 || QT > 2) ? 1 : kMfmaWaves) void att
                             A *= fo.keep, M = fo.m, L = fo.l;
                         }
                         const float o = L != 0.0f ? A / L : 0.0f;
-                        store_out(a.out, a.out_dtype, (int64_t)(cur.start + c) * a.o_st + (int64_t)head * a.o_sh + d, o);
-                        if (a.lse && d == 0) a.lse[(int64_t)(cur.start + c) * a.hq + head] = L != 0.0f ? __builtin_fmaf(M, kLn2, __logf(L)) : -INFINITY;
+                        store_out(a.out, a.out_dtype, (int64_t)(cur.start + c) * a.o_st + (int64_t)head * a.o_sh + (NARROW ? (d & 63) : d), o);
+                        if (a.lse && (d & (NARROW ? 63 : D - 1)) == 0) a.lse[(int64_t)(cur.start + c) * a.hq + head] = L != 0.0f ? __builtin_fmaf(M, kLn2, __logf(L)) : -INFINITY;
                     }
                 }
             }
