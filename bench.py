@@ -767,6 +767,60 @@ def reference_shapes(pk, device, only=None):
     return found
 
 
+def narrow_heads(pk, device):
+    """Decode over 64-wide heads (32 query / 8 KV heads x 64, the shape of the small models: a step's batch of 64 rows,
+    contexts ~U[1024, 8192], pages of 16), which the bandwidth kernel reads in pairs of KV heads as 128-wide ones: the
+    split launch alone (`phases=1`) and with its merge, replayed from a captured graph over four layers' caches read in
+    turn (each launch cold), BF16 and FP8 pages, each with its fraction of the 8 TB/s HBM peak."""
+    found = {}
+    g = torch.Generator(device=device).manual_seed(23)
+    hq, hkv, d, page, rows = 32, 8, 64, 16, 64
+    ctx = torch.randint(1024, 8193, (rows,), generator=torch.Generator().manual_seed(5))
+    width = ((8192 + 8 + page - 1) // page + 15) // 16 * 16
+    pages = width * rows
+    tables = torch.randperm(pages, device=device, generator=g).to(torch.int32).view(rows, width).contiguous()
+    r = torch.arange(rows, dtype=torch.int32, device=device)
+    firsts = (ctx - 1).to(torch.int64).to(device)
+    q = torch.randn(rows, hq, d, device=device, generator=g).to(torch.bfloat16)
+    out = torch.empty_like(q)
+    for kind, store in (("bf16", torch.bfloat16), ("fp8", torch.float8_e4m3fn)):
+        fresh = lambda: (torch.randn(pages + 1, page, hkv, d, device=device, dtype=torch.bfloat16, generator=g) * 0.5).to(store)
+        ks, vs = [fresh() for _ in range(4)], [fresh() for _ in range(4)]
+        at = [0]
+
+        def launch(phases):
+            at[0] = (at[0] + 1) % 4
+            pk.attend(q, ks[at[0]], vs[at[0]], kind, tables, r, r, firsts, 1, page, out=out, multipliers=(0.02, 0.03), phases=phases)
+        split = graph_timed(lambda: launch(1), 12)
+        both = graph_timed(lambda: launch(0), 12)
+        nbytes = int(ctx.sum()) * hkv * 2 * d * (2 if kind == "bf16" else 1)
+        found[kind] = {"piece": pk.piece_size(d, d, kind, hkv), "positions": int(ctx.sum()), "split_us": round(split * 1e3, 1),
+                       "with_merge_us": round(both * 1e3, 1), "split_GB/s": round(nbytes / split / 1e6, 1),
+                       "split_frac_of_hbm_peak": round(nbytes / split / 1e6 / HBM_PEAK_GBPS, 4)}
+        del ks, vs
+        torch.cuda.empty_cache()
+    return found
+
+
+def known_traffic(pk, device):
+    """Two launches of known HBM traffic for scaling the FETCH_SIZE and WRITE_SIZE counters of a profile of one of the
+    --*-only runs (with --calibrate): stream_read_kernel over 512 MiB, and write_rows of 262,144 tokens of 8 KV heads x
+    128 (BF16 to BF16 pages)."""
+    data = torch.zeros(512 << 20, dtype=torch.uint8, device=device)
+    sink = torch.zeros(64, device=device)
+    pk.stream_read(data, sink)
+    T, hkv, d = 262144, 8, 128
+    ck = torch.zeros(1 << 20, hkv, d, dtype=torch.bfloat16, device=device)
+    cv = torch.zeros_like(ck)
+    keys = torch.randn(T, hkv, d, device=device).to(torch.bfloat16)
+    values = torch.randn(T, hkv, d, device=device).to(torch.bfloat16)
+    slots = torch.randperm(1 << 20, device=device)[:T]
+    pk.write(keys, values, slots, ck, cv, "bf16")
+    torch.cuda.synchronize()
+    log(f"[bench] calibration: stream_read_kernel reads {data.numel()} bytes a launch; write_rows of {T} tokens reads "
+        f"{2 * T * hkv * d * 2 + T * 8} bytes and writes {2 * T * hkv * d * 2} bytes")
+
+
 def verify_windows(pk, device):
     """Verify windows of a draft (8B shape, 32 query / 8 KV heads x 128, pages of 16): 64 rows at contexts ~U[1024, 8192],
     each a window of 1, 4, 5 or 8 columns, bf16 and fp8 pages; microseconds a launch (split + merge) over four layers of
@@ -933,6 +987,7 @@ def main():
                     help="run only the pool bookkeeping of the extras (slots, the move of accepted rows, page copies)")
     ap.add_argument("--latent-only", action="store_true", help="run only the latent-attention decode of the extras")
     ap.add_argument("--index-only", action="store_true", help="run only the sparse index selection of the extras")
+    ap.add_argument("--heads64-only", action="store_true", help="run only the decode over 64-wide heads of the extras")
     ap.add_argument("--shape", default=None, help="with --shapes-only: only the rows whose name contains this")
     ap.add_argument("--append-only", action="store_true",
                     help="run only the KV append with rope and norm fused in beside the plain append (for counter runs on write_rows)")
@@ -963,6 +1018,13 @@ def main():
         found = index_selection(device)
         log(f"[bench] sparse index selection: {found}")
         print(json.dumps({"sparse_index_selection": found}), flush=True)
+        return
+    if args.heads64_only:
+        if args.calibrate:
+            known_traffic(pk, device)
+        found = narrow_heads(pk, device)
+        log(f"[bench] decode over 64-wide heads: {found}")
+        print(json.dumps({"heads_of_64_decode": found}), flush=True)
         return
     if args.shapes_only:
         found = reference_shapes(pk, device, args.shape)
@@ -1092,6 +1154,9 @@ def main():
         extras["reference_published_shapes"] = reference_shapes(pk, device)
         log(f"[bench] the reference's published shapes: {extras['reference_published_shapes']}")
         torch.cuda.empty_cache()
+        extras["heads_of_64_decode"] = narrow_heads(pk, device)
+        log(f"[bench] decode over 64-wide heads, 32q / 8kv, 64 rows: {extras['heads_of_64_decode']}")
+        torch.cuda.empty_cache()
         extras["verify_windows_64_rows"] = verify_windows(pk, device)
         log(f"[bench] verify windows, 64 rows: {extras['verify_windows_64_rows']}")
         torch.cuda.empty_cache()
@@ -1124,6 +1189,9 @@ def main():
                 also.append({"kernel": "latent_heads_kernel" if found.get("tile_rows") == 128 else "latent_kernel", "workload": f"64 rows ctx~U[1024,8192] rank 512 + rope 64, {name}",
                              "us": found["split_us"], "with_merge_us": found["with_merge_us"], "bound": "hbm",
                              "frac": found["split_frac_of_hbm_peak"], "mfma_frac": found["split_frac_of_bf16_mfma_peak"]})
+        for kind, found in extras["heads_of_64_decode"].items():
+            also.append({"kernel": f"{DECODE_KERNEL} (split launch, pairs of 64-wide heads)", "workload": f"64 rows ctx~U[1024,8192] 32q/8kv x 64, {kind}",
+                         "us": found["split_us"], "with_merge_us": found["with_merge_us"], "bound": "hbm", "frac": found["split_frac_of_hbm_peak"]})
         result["roofline"]["also"] = also
     if not args.no_cpu:
         log("[bench] timing the CPU reference path (about 20 s)")
