@@ -238,8 +238,8 @@ def append_sweep(pk, device, kind):
         ms = timed(call, 20, 3)
         kernel = graph_timed(call)
         nbytes = T * hkv * 2 * d * (e + 2)
-        found[str(T)] = {"us": round(ms * 1e3, 2), "GB/s": round(nbytes / ms / 1e6, 1),
-                         "kernel_us": round(kernel * 1e3, 2), "kernel_GB/s": round(nbytes / kernel / 1e6, 1),
+        found[str(T)] = {"us": round(ms * 1e3, 2), "kernel_us": round(kernel * 1e3, 2),
+                         "kernel_GB/s": round(nbytes / kernel / 1e6, 1),
                          "kernel_frac_of_peak": round(nbytes / kernel / 1e6 / HBM_PEAK_GBPS, 4)}
     return found
 
@@ -272,10 +272,9 @@ def append_rope(pk, device):
             normed = timed(lambda: pk.write(keys, values, slots, k, v, kind, multipliers=(0.02, 0.03),
                                             rope=(table, positions), norm=(weight, 1e-6)), 20, 3)
             nbytes = T * hkv * 2 * d * (e + 2)
-            found[kind][str(T)] = {"plain_us": round(plain * 1e3, 2), "with_rope_us": round(fused * 1e3, 2),
-                                   "with_rope_GB/s": round(nbytes / fused / 1e6, 1),
-                                   "with_norm_and_rope_us": round(normed * 1e3, 2),
-                                   "with_norm_and_rope_GB/s": round(nbytes / normed / 1e6, 1)}
+            found[kind][str(T)] = {"plain_us": round(plain * 1e3, 2), "rope_us": round(fused * 1e3, 2),
+                                   "norm_rope_us": round(normed * 1e3, 2),
+                                   "norm_rope_GB/s": round(nbytes / normed / 1e6, 1)}
         del k, v
     return found
 
@@ -307,12 +306,13 @@ def long_context(pk, device):
                                                   chunk=chunk, out=out, workspace=ws, phases=phases)
                 total = timed(call, 10, 2)
                 split = timed(lambda: call(1), 10, 2)
+                # (GB/s = algorithmic bytes / us: the fractions of the 8 TB/s peak, with the merge and of the split launch alone)
                 found[f"B{batch}_ctx{ctx}_chunk{chunk}"] = {
-                    "us": round(total * 1e3, 1), "split_us": round(split * 1e3, 1), "merge_us": round((total - split) * 1e3, 1),
-                    "GB/s": round(nbytes / total / 1e6, 1), "split_GB/s": round(nbytes / split / 1e6, 1)}
+                    "us": round(total * 1e3, 1), "split_us": round(split * 1e3, 1),
+                    "frac": round(nbytes / total / 1e6 / HBM_PEAK_GBPS, 3), "split_frac": round(nbytes / split / 1e6 / HBM_PEAK_GBPS, 3)}
             # (the default reader beside them: partitions x pieces, a partition's pieces b, b + P, ... one unit)
             total = timed(lambda: pk.attend(q, k, v, "bf16", tables, rows, rows, firsts, 1, page, out=out), 10, 2)
-            found[f"B{batch}_ctx{ctx}_default_reader"] = {"us": round(total * 1e3, 1), "GB/s": round(nbytes / total / 1e6, 1)}
+            found[f"B{batch}_ctx{ctx}_default_reader"] = {"us": round(total * 1e3, 1), "frac": round(nbytes / total / 1e6 / HBM_PEAK_GBPS, 3)}
     return found
 
 
@@ -643,8 +643,7 @@ def index_selection(device):
             flops = 2.0 * tokens * n * H * D
             found[f"{n}_keys_{tokens}_tokens"] = {
                 "scores_bf16_us": round(bf16 * 1e3, 1), "scores_e4m3_us": round(fp8 * 1e3, 1),
-                "scores_bf16_TFLOP/s": round(flops / bf16 / 1e9, 1), "topk_us": round(top * 1e3, 1),
-                "topk_GB/s_of_scores_read_once": round(tokens * n * 4 / top / 1e6, 1)}
+                "scores_bf16_TFLOP/s": round(flops / bf16 / 1e9, 1), "topk_us": round(top * 1e3, 1)}
     # A decode step's shape: every sequence's one token over its own keys, read in place from a store of pages of 64
     # rows at random places (slots [sequences][n]): HBM-bound, a key row read once.
     n, page = 49984, 64
@@ -728,8 +727,7 @@ def reference_shapes(pk, device, only=None):
                 ms = graph_timed(launch, 8)
                 nbytes = batch * ctx * hkv * (2 * d * e + (8 if kind != "bf16" else 0))
                 found[f"{name}_{batch}_rows_{columns}_cols_ctx{ctx}"] = {
-                    "us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1),
-                    "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+                    "us": round(ms * 1e3, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 3)}
                 if batch == 1 and columns == 1 and ctx <= 16384:
                     # (one short row: what an engine of single sequences gets with the reference's own largest piece, 128
                     # positions, instead of the default, which is sized for full batches)
