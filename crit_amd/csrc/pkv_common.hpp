@@ -84,17 +84,19 @@ struct Quotients {
 PKV_DEV float bf16_lo(uint32_t w) { return u2f(w << 16); }
 PKV_DEV float bf16_hi(uint32_t w) { return u2f(w & 0xffff0000u); }
 
-// FP32 -> BF16 bits, round to nearest even; NaN -> 0x7FC0 (what torch's CPU cast stores).
+// FP32 -> BF16 bits, round to nearest even; NaN -> 0xFFFF: what torch's CPU cast of a tensor stores (its vectorised
+// conversion, AVX2 and AVX-512 alike, blends 0xFFFF in for every NaN; its scalar conversion, which only a build
+// without those reaches, returns 0x7FC0: the reference's stored bytes for a NaN follow the host it runs on).
 PKV_DEV uint32_t bf16_rne(float x) {
     uint32_t u = f2u(x);
     uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-    return (x != x) ? 0x7fc0u : r;
+    return (x != x) ? 0xffffu : r;
 }
 PKV_DEV uint32_t pack_bf16(float a, float b) { return bf16_rne(a) | (bf16_rne(b) << 16); }
 // Eight FP32 values as four BF16 pairs with the same bits as pack_bf16, by the hardware's conversion (v_cvt_pk_bf16_f32:
 // round to nearest even, like bf16_rne, for every number) where no value is a NaN, which one test over the packed
 // words decides (a 16-bit half above 0x7F80 in magnitude): a NaN comes out of the hardware quiet but with its payload,
-// and torch's cast stores 0x7FC0, so then the words are made again one value at a time.
+// and torch's cast stores 0xFFFF, so then the words are made again one value at a time.
 PKV_DEV u32x4 pack8_bf16(const float (&x)[8]) {
     typedef __attribute__((ext_vector_type(2))) __bf16 pair_t;
     uint32_t w[4], any = 0u;

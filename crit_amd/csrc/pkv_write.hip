@@ -287,7 +287,11 @@ __global__ __launch_bounds__(256) void write_rows(WriteArgs a) {
         const int64_t dst = (slot[u] * a.hkv + head[u]) * dim + i0;
         if constexpr (KIND == 0) {
             uint4 v;
-            if constexpr (F16) {
+            if constexpr ((IN == CRIT_PKV_BF16 && !F16) || (IN == CRIT_PKV_F16 && F16)) {
+                // the pages' type is the inputs' own: the row as it came, bit for bit (torch's .to() of a tensor's own
+                // dtype is the tensor: a NaN keeps its payload, where a cast from another type stores the canonical one)
+                v = make_uint4(raw[u].v[0].x, raw[u].v[0].y, raw[u].v[0].z, raw[u].v[0].w);
+            } else if constexpr (F16) {
                 v = make_uint4(pack_f16(x[0], x[1]), pack_f16(x[2], x[3]), pack_f16(x[4], x[5]), pack_f16(x[6], x[7]));
             } else {
                 const u32x4 packed = pack8_bf16(x);
@@ -385,7 +389,10 @@ __global__ __launch_bounds__(256) void write_rows_scalar(WriteArgs a) {
     }
     for (int i = 0; i < dim; ++i) {
         const float x = load_in<IN>(a.src[which], src + i);
-        if constexpr (KIND == 0) {
+        if constexpr (KIND == 0 && ((IN == CRIT_PKV_BF16 && !F16) || (IN == CRIT_PKV_F16 && F16))) {
+            // (the inputs' own type: the element's bits as they came)
+            reinterpret_cast<uint16_t*>(a.pages[which])[dst + i] = reinterpret_cast<const uint16_t*>(a.src[which])[src + i];
+        } else if constexpr (KIND == 0) {
             reinterpret_cast<uint16_t*>(a.pages[which])[dst + i] = (uint16_t)(F16 ? f16_bits(x) : bf16_rne(x));
         } else {
             const float q = __fdiv_rn(x, div);

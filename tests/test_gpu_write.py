@@ -41,6 +41,37 @@ def test_writes_encode_as_torch_does_and_skip_negative_slots(kind, d, dv, in_dty
     _check(kind, (k, v, ks, vs), expected_pages(kind, keys, values, slots, 64, mult))
 
 
+@pytest.mark.parametrize("kind,dtype", [("bf16", torch.bfloat16), ("fp16", torch.float16)])
+@pytest.mark.parametrize("d", [128, 20])
+def test_sixteen_bit_rows_into_pages_of_their_own_type_keep_every_bit(kind, dtype, d):
+    # The reference's write() stores keys.to(the pages' dtype) (pages.py:439-453): for inputs of the pages' own type that
+    # is the tensor itself, so every bit pattern arrives as it is, a NaN with its payload and sign (a cast from FP32
+    # stores the canonical NaN instead: the oracle's rule, checked beside it). d = 20: the scalar kernel.
+    pk = kernels()
+    patterns = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype)
+    rows = 65536 // (4 * d) * 4
+    x = patterns[:rows * d].reshape(rows // 4, 4, d)
+    k = torch.zeros(rows // 4, 4, d, dtype=dtype, device=dev)
+    v = torch.zeros_like(k)
+    slots = torch.randperm(rows // 4, generator=torch.Generator().manual_seed(3))
+    pk.write(x.to(dev), x.flip(0).to(dev), slots.to(dev), k, v, kind)
+    assert torch.equal(k.cpu().view(torch.int16)[slots], x.view(torch.int16))
+    assert torch.equal(v.cpu().view(torch.int16)[slots], x.flip(0).view(torch.int16))
+    # The same values as FP32 inputs go through torch's cast. What it stores for a NaN follows the host (its vectorised
+    # BF16 conversion stores 0xFFFF, its scalar one 0x7FC0; FP16 keeps the payload): every other value bit for bit, a
+    # NaN as a NaN, and as the oracle's where this host casts the way the kernels do.
+    wide = x.float()
+    pk.write(wide.to(dev), wide.to(dev), slots.to(dev), k, v, kind)
+    want = expected_pages(kind, wide, wide, slots, rows // 4, (1.0, 1.0))[0]
+    got = k.cpu()
+    numbers = ~torch.isnan(want.float())
+    assert torch.equal(torch.isnan(got.float()), ~numbers)
+    assert torch.equal(got.view(torch.int16)[numbers], want.view(torch.int16)[numbers])
+    host_nan = torch.tensor([float("nan")] * 16).to(dtype).view(torch.int16)[0].item() & 0xffff
+    if dtype == torch.float16 or host_nan == 0xffff:
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
 @pytest.mark.parametrize("T", [4152, 33001])
 @pytest.mark.parametrize("kind", ["bf16", "fp8", "fp8:row", "int8"])
 def test_a_large_append_with_edge_values_is_bit_exact(kind, T):
