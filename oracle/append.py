@@ -51,9 +51,12 @@ def encode(rows, kind, multiplier=1.0):
     (the reference's per-layer scale) or a [kv_heads] tensor (one scale per KV head, broadcast over tokens and dims: a
     superset of the reference rule with the same expression). The division is tensor / tensor, which is IEEE on
     every torch backend."""
-    x = rows.float()
     if kind in ("bf16", "fp16", "fp32"):
-        return x.to(STORAGE[kind]), None
+        # rows.to(storage), the reference's own expression (pages.py:453): rows of the pages' type are stored as they
+        # are, every bit (a NaN with its payload); what a cast stores for a NaN is torch's and follows the host (FP32 to
+        # BF16: 0xFFFF by its vectorised conversion, 0x7FC0 by its scalar one; to FP16 the payload's top bits)
+        return rows.to(STORAGE[kind]), None
+    x = rows.float()
     if kind == "fp8":
         m = torch.as_tensor(multiplier, dtype=torch.float32)
         if m.dim() == 1:

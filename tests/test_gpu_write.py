@@ -72,6 +72,41 @@ def test_sixteen_bit_rows_into_pages_of_their_own_type_keep_every_bit(kind, dtyp
         assert torch.equal(got.view(torch.int16), want.view(torch.int16))
 
 
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("d", [128, 24])
+def test_every_sixteen_bit_pattern_is_encoded_as_the_oracle_encodes_it(kind, in_dtype, d):
+    # Every BF16 / FP16 bit pattern as an input (FP32 inputs: every BF16 pattern widened, and with low bits set on either
+    # side of the rounding ties), into every page kind, vector kernel (d = 128) and scalar one (d = 24): every number's
+    # stored bits and every row scale equal the oracle's; a NaN is stored as a NaN (whose bits, where a cast makes them,
+    # are its conversion instruction's: the test of the pages' own type above has the cases that are pinned).
+    pk = kernels()
+    patterns = torch.arange(65536, dtype=torch.int32).to(torch.int16)
+    if in_dtype == torch.float32:
+        wide = patterns.view(torch.bfloat16).float().view(torch.int32)
+        x = torch.cat([wide, wide | 0x8000, wide | 0x7fff, wide | 0x8001, wide | 0x0001]).view(torch.float32)
+    else:
+        x = patterns.view(in_dtype)
+    x = x[:x.numel() // (4 * d) * 4 * d].reshape(-1, 4, d)
+    T = x.shape[0]
+    k = torch.zeros(T, 4, d, dtype=STORE[kind], device=dev)
+    v = torch.zeros_like(k)
+    ks = vs = None
+    if kind in ("fp8:row", "int8"):
+        ks, vs = torch.zeros(T, 4, device=dev), torch.zeros(T, 4, device=dev)
+    slots = torch.randperm(T, generator=torch.Generator().manual_seed(3))
+    mult = (0.05, 0.07)
+    pk.write(x.to(dev), x.flip(0).to(dev), slots.to(dev), k, v, kind, ks, vs, multipliers=mult)
+    want = expected_pages(kind, x, x.flip(0), slots, T, mult)
+    for name, got, exact in zip(("keys", "values", "key scales", "value scales"), (k, v, ks, vs), want):
+        if exact is None:
+            continue
+        got = got.cpu()
+        nan = torch.isnan(exact.float())
+        assert torch.equal(torch.isnan(got.float()), nan), (name, "which are NaN")
+        assert torch.equal(bits(got)[~nan], bits(exact)[~nan]), (name, "the numbers' bits")
+
+
 @pytest.mark.parametrize("T", [4152, 33001])
 @pytest.mark.parametrize("kind", ["bf16", "fp8", "fp8:row", "int8"])
 def test_a_large_append_with_edge_values_is_bit_exact(kind, T):
