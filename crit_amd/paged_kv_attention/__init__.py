@@ -379,7 +379,8 @@ def write(keys, values, slots, key_pages, value_pages, kind, key_scales=None, va
     inference/fused-norms/code/torch_norms.py:89-147, fused into this launch): (table, positions) or (table, positions,
     style, scale): table FP32 [rows][dim] (cos of every pair, then sin), positions [tokens] int64 (clamped to the table's
     rows), style "half" (pairs j, j + dim / 2) or "interleaved" (2j, 2j + 1), scale on cos and sin; the keys go in as
-    rope() would have returned them in their own dtype. Head widths 64, 128, 256, values no wider than keys.
+    rope() would have returned them in their own dtype. Head widths 64, 128, 256 (values wider than the keys go in a
+    second launch).
     norm, with rope: (weight, eps) or (weight, eps, offset): each key head's RMS norm in front of the rotation, the
     reference's rms_norm_rope() (torch_norms.py:149-176; what rms_norm_rope_pair does to the keys, blocks.py:160-170)
     fused in as well: x / sqrt(mean(x^2) + eps) * (weight + offset) in FP32, rotated in FP32, rounded once to the keys'
@@ -399,6 +400,11 @@ def write(keys, values, slots, key_pages, value_pages, kind, key_scales=None, va
     T, hkv, d = keys.shape
     if T == 0:
         return
+    if rope is not None and values is not None and values.shape[-1] > d:
+        # (the rotating launch lays a row over the lanes of the wider of the two widths, and a key's partner lanes are
+        # counted in its own: values wider than the keys go in a launch of their own, the same bytes)
+        write(keys, None, slots, key_pages, None, kind, key_scales, None, multipliers=multipliers, rope=rope, norm=norm)
+        return write(None, values, slots, None, value_pages, kind, None, value_scales, multipliers=multipliers)
     if keys.dtype not in _DTYPE:
         keys = keys.float()
     if keys.stride(-1) != 1:
@@ -440,8 +446,8 @@ def write(keys, values, slots, key_pages, value_pages, kind, key_scales=None, va
         if not torch.is_tensor(positions) or positions.dtype != torch.int64 or tuple(positions.shape) != (T,) or \
                 not positions.is_contiguous() or positions.device != keys.device:
             raise ValueError(f"rope's positions are a contiguous int64 [{T}] tensor on the keys' device")
-        if d not in (64, 128, 256) or p.value_dim > d:
-            raise ValueError("rope in the append takes head widths 64, 128 and 256, values no wider than keys")
+        if d not in (64, 128, 256):
+            raise ValueError("rope in the append takes head widths 64, 128 and 256")
         p.rope_table, p.rope_positions, p.rope_rows = table.data_ptr(), positions.data_ptr(), table.shape[0]
         p.rope_interleaved, p.rope_scale = int(style == "interleaved"), float(scale)
     if norm is not None:

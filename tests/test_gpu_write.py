@@ -288,7 +288,7 @@ def test_bad_arguments_are_refused():
 
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("d,dv,in_dtype", [(128, 128, torch.bfloat16), (64, 64, torch.float32), (256, 128, torch.bfloat16),
-                                           (128, 64, torch.float16)])
+                                           (128, 64, torch.float16), (64, 128, torch.bfloat16)])      # (values wider than keys: two launches)
 @pytest.mark.parametrize("style", ["half", "interleaved"])
 def test_keys_rotated_on_their_way_in_are_the_bytes_of_rope_then_write(kind, d, dv, in_dtype, style):
     # write(rope=(table, positions, style, scale)): the reference's rope() on the keys (inference/fused-norms/code/
@@ -335,7 +335,7 @@ def test_keys_rotated_on_their_way_in_are_the_bytes_of_rope_then_write(kind, d, 
 @pytest.mark.parametrize("kind,d,dv,in_dtype", [("bf16", 128, 128, torch.bfloat16), ("fp8", 128, 128, torch.bfloat16),
                                            ("fp8:row", 128, 128, torch.float32), ("int8", 64, 64, torch.bfloat16),
                                            ("fp16", 256, 256, torch.float16), ("fp8", 256, 128, torch.float32),
-                                           ("bf16", 64, 64, torch.float32)])
+                                           ("bf16", 64, 64, torch.float32), ("fp8:row", 64, 256, torch.bfloat16)])
 @pytest.mark.parametrize("style", ["half", "interleaved"])
 def test_keys_normed_and_rotated_on_their_way_in_are_the_bytes_of_rms_norm_rope_then_write(kind, d, dv, in_dtype, style):
     # write(rope=..., norm=(weight, eps, offset)): the reference's rms_norm_rope() on the keys (inference/fused-norms/
