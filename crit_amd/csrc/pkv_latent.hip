@@ -1235,6 +1235,189 @@ __global__ __launch_bounds__(64) void latent_merge_kernel(LatentArgs a) {
     if (a.lse && threadIdx.x == 0) a.lse[token * a.heads + head] = (L > 0.0f || L != L) ? (M + __builtin_log2f(L)) * kLn2 : -INFINITY;
 }
 
+// -- the shapes whose rows do not fill the tiles above (ranks 16 and 32, a rotary width of 16) -----------------------------
+// A wavefront serves one query row (a batch row's column and head) over pieces b, b + parts, ... of the positions it
+// sees, 64 positions a step with a lane a position: the lane reads its position's whole cache row for the score (the
+// query's values wait in LDS as FP32), the step's softmax runs over the wavefront, and for the values the lanes turn
+// to the row's dims (lane i: values 2 i, 2 i + 1 of every 128) while the positions' probabilities and slots go round by
+// shuffle. No matrix pipe and every cache row read twice (the second time from the caches): these shapes are served,
+// not tuned. The partials have the layout and the meaning of the kernels' above.
+template <bool F16, bool FP8>
+__global__ __launch_bounds__(256) void latent_plain_kernel(LatentArgs a, int R, int P, int groups) {
+    constexpr int EB = FP8 ? 1 : 2;
+    __shared__ float s_q[4][1024 + 256];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int W = R + P;
+    const int64_t pair = blockIdx.x / groups;
+    const int group = (int)(blockIdx.x - pair * groups);
+    const int r = (int)(pair / a.gy), b = (int)(pair % a.gy);
+    const int H = a.heads;
+    int count = a.columns;
+    if (a.counts) count = min(a.counts[r], a.columns);
+    const int jq = group * 4 + wave, colq = jq / H, headq = jq - colq * H;
+    const bool liveq = colq < count;
+    if (liveq) {
+        const uint8_t* q = a.q + ((int64_t)(a.starts[r] + colq) * a.q_st + (int64_t)headq * a.q_sh) * 2;
+        for (int e = lane * 2; e < W; e += 128) {
+            const uint32_t w = *reinterpret_cast<const uint32_t*>(q + e * 2);
+            s_q[wave][e] = F16 ? f16_lo(w) : bf16_lo(w);
+            s_q[wave][e + 1] = F16 ? f16_hi(w) : bf16_hi(w);
+        }
+    }
+    __syncthreads();
+    if (!liveq) return;
+    const int64_t first64 = a.firsts[r];
+    const int first = (int)(first64 < 0 ? 0 : (first64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first64));
+    const int n_keys = min(first + colq + 1, a.max_keys);      // the positions this query row sees
+    const int n_pieces = (n_keys + a.piece - 1) / a.piece;
+    if (b >= n_pieces) return;
+    const int64_t trow = (int64_t)a.rows[(int64_t)r * a.rows_step] * a.tab_stride;
+    const float* query = s_q[wave];
+
+    float m = -INFINITY, l = 0.0f, acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+    for (int pi = b; pi < n_pieces; pi += a.parts) {
+        const int piece_end = min((pi + 1) * a.piece, n_keys);      // (partitions * piece is bounded by the launch)
+        for (int base = pi * a.piece; base < piece_end; base += 64) {
+            const bool seen = base + lane < piece_end;
+            const int n = seen ? base + lane : piece_end - 1;
+            const int pidx = (int)div32(a.page_div, (uint32_t)n);
+            const int entry = a.tables[trow + (pidx < a.tab_width ? pidx : a.tab_width - 1)];
+            const int64_t slot = (int64_t)entry * a.page + (n - pidx * a.page);
+            const uint8_t* row = a.cache + slot * (W * EB);
+            float s0 = 1.0f, s1 = 1.0f;
+            if constexpr (FP8) {
+                const float* sc = a.scales + slot * a.scales_per_row;
+                s0 = sc[0], s1 = a.scales_per_row > 1 ? sc[1] : s0;
+            }
+            float dots[2] = {0.0f, 0.0f};      // the latent's products, then the rotary key's
+#pragma unroll
+            for (int part = 0; part < 2; ++part) {
+                const int e0 = part ? R : 0, e1 = part ? W : R;
+                float dot = 0.0f;
+                for (int e = e0; e < e1; e += 16 / EB) {
+                    const u32x4 w = *reinterpret_cast<const u32x4*>(row + e * EB);
+                    const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        if constexpr (FP8) {
+                            const f32x2 lo = e4m3_pair<false>(ws[k]), hi = e4m3_pair<true>(ws[k]);
+                            dot = __builtin_fmaf(lo.x, query[e + 4 * k], dot);
+                            dot = __builtin_fmaf(lo.y, query[e + 4 * k + 1], dot);
+                            dot = __builtin_fmaf(hi.x, query[e + 4 * k + 2], dot);
+                            dot = __builtin_fmaf(hi.y, query[e + 4 * k + 3], dot);
+                        } else {
+                            dot = __builtin_fmaf(F16 ? f16_lo(ws[k]) : bf16_lo(ws[k]), query[e + 2 * k], dot);
+                            dot = __builtin_fmaf(F16 ? f16_hi(ws[k]) : bf16_hi(ws[k]), query[e + 2 * k + 1], dot);
+                        }
+                    }
+                }
+                dots[part] = dot;
+            }
+            float x = (FP8 ? __builtin_fmaf(dots[0], s0, dots[1] * s1) : dots[0] + dots[1]) * a.sscale;
+            x = seen ? x : -INFINITY;
+            const float m_new = __builtin_fmaxf(m, group_max<64>(x));
+            const float sub = m_new == -INFINITY ? 0.0f : m_new;
+            const float alpha = exp2_fast(m - sub);
+            float p = exp2_fast(x - sub);
+            l = __builtin_fmaf(l, alpha, group_sum<64>(p));
+            m = m_new;
+            if constexpr (FP8) p *= s0;      // a value is its code times its position's latent scale
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[i] *= alpha;
+            const int lo = (int)(uint32_t)slot, hi = (int)(slot >> 32);
+            const int live = min(64, piece_end - base);
+            for (int j = 0; j < live; ++j) {
+                const float pj = __shfl(p, j);
+                const int64_t at = ((int64_t)__shfl(hi, j) << 32) | (uint32_t)__shfl(lo, j);
+                const uint8_t* values = a.cache + at * (W * EB) + lane * 2 * EB;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    if (i * 128 + lane * 2 < R) {
+                        float v0, v1;
+                        if constexpr (FP8) {
+                            const f32x2 v = e4m3_pair<false>(*reinterpret_cast<const uint16_t*>(values + i * 128));
+                            v0 = v.x, v1 = v.y;
+                        } else {
+                            const uint32_t w = *reinterpret_cast<const uint32_t*>(values + i * 256);
+                            v0 = F16 ? f16_lo(w) : bf16_lo(w), v1 = F16 ? f16_hi(w) : bf16_hi(w);
+                        }
+                        acc[2 * i] = __builtin_fmaf(pj, v0, acc[2 * i]);
+                        acc[2 * i + 1] = __builtin_fmaf(pj, v1, acc[2 * i + 1]);
+                    }
+                }
+            }
+        }
+    }
+    const int64_t index = ((int64_t)((int64_t)r * a.columns + colq) * H + headq) * a.parts + b;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        if (i * 128 + lane * 2 < R)
+            *reinterpret_cast<f32x2*>(a.po + index * R + i * 128 + lane * 2) = f32x2{acc[2 * i], acc[2 * i + 1]};
+    if (lane == 0) a.pm[index] = m, a.pl[index] = l;
+}
+
+// Its merge: latent_merge_kernel with the rank at run time (a thread: values t, t + 64, ... one after another).
+__global__ __launch_bounds__(64) void latent_plain_merge_kernel(LatentArgs a, int R) {
+    const int prow = blockIdx.x, head = blockIdx.y;
+    const int r = prow / a.columns, col = prow - r * a.columns;
+    int count = a.columns;
+    if (a.counts) count = min(a.counts[r], a.columns);
+    if (col >= count) return;
+    const int64_t first64 = a.firsts[r];
+    const int first = (int)(first64 < 0 ? 0 : (first64 > (int64_t)0x3fffffff ? (int64_t)0x3fffffff : first64));
+    const int n_keys = min(first + col + 1, a.max_keys);
+    const int n_pieces = (n_keys + a.piece - 1) / a.piece;
+    const int np = min(a.parts, n_pieces);
+    const int64_t index = ((int64_t)prow * a.heads + head) * a.parts;
+    const int64_t token = (int64_t)a.starts[r] + col;
+    for (int d = threadIdx.x; d < R; d += 64) {
+        float M = -INFINITY, L = 0.0f, acc = 0.0f;
+        for (int b = 0; b < np; ++b) {
+            const Fold f = fold(M, L, a.pm[index + b], a.pl[index + b]);
+            acc = __builtin_fmaf(acc, f.keep, a.po[(index + b) * R + d] * f.take);
+            M = f.m, L = f.l;
+        }
+        if (a.sinks) {      // one more position with no value
+            const float sink = a.sinks[head] * kLog2e;
+            const float top = __builtin_fmaxf(M, sink);
+            const float sub = top == -INFINITY ? 0.0f : top;
+            const float keep = exp2_fast(M - sub);
+            L = __builtin_fmaf(L, keep, exp2_fast(sink - sub));
+            acc *= keep;
+            M = top;
+        }
+        const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+        store_out(a.out, a.out_dtype, token * a.o_st + (int64_t)head * a.o_sh + d, acc * inv);
+        if (a.lse && d == 0) a.lse[token * a.heads + head] = (L > 0.0f || L != L) ? (M + __builtin_log2f(L)) * kLn2 : -INFINITY;
+    }
+}
+
+int launch_plain(const LatentArgs& a, int R, int P, bool f16, bool fp8, int phases, hipStream_t stream) {
+    if (phases != 2) {
+        const int groups = (a.columns * a.heads + 3) / 4;
+        const int64_t blocks = a.pairs * groups;
+        if (blocks > 0x7fffffff) return CRIT_PKV_E_GEOMETRY;
+        const dim3 grid((unsigned)blocks);
+        if (fp8) {
+            if (f16) hipLaunchKernelGGL((latent_plain_kernel<true, true>), grid, dim3(256), 0, stream, a, R, P, groups);
+            else hipLaunchKernelGGL((latent_plain_kernel<false, true>), grid, dim3(256), 0, stream, a, R, P, groups);
+        } else {
+            if (f16) hipLaunchKernelGGL((latent_plain_kernel<true, false>), grid, dim3(256), 0, stream, a, R, P, groups);
+            else hipLaunchKernelGGL((latent_plain_kernel<false, false>), grid, dim3(256), 0, stream, a, R, P, groups);
+        }
+        const int bad = hip_code(hipGetLastError());
+        if (bad) return bad;
+    }
+    if (phases != 1) {
+        hipLaunchKernelGGL(latent_plain_merge_kernel, dim3((unsigned)(a.n_rows * a.columns), (unsigned)a.heads), dim3(64), 0, stream, a, R);
+        return hip_code(hipGetLastError());
+    }
+    return 0;
+}
+
+
 template <int R, int P, int NT>
 int launch_tiles(const LatentArgs& a, bool f16, bool fp8, hipStream_t stream) {
     const int64_t blocks = (a.pairs + 7) / 8 * 8 * a.tiles;
@@ -1348,6 +1531,9 @@ int launch_latent(const crit_pkv_latent_params* p, hipStream_t stream) {
     PKV_LATENT(1024, 32) PKV_LATENT(1024, 128) PKV_LATENT(1024, 256) PKV_LATENT(512, 32) PKV_LATENT(512, 256) PKV_LATENT(256, 32)
     PKV_LATENT(256, 128) PKV_LATENT(256, 256) PKV_LATENT(128, 128) PKV_LATENT(128, 256) PKV_LATENT(64, 128) PKV_LATENT(64, 256)
 #undef PKV_LATENT
+    const auto power_of_two = [](int x, int lo, int hi) { return x >= lo && x <= hi && (x & (x - 1)) == 0; };
+    if (power_of_two(p->rank, 16, 1024) && power_of_two(p->rope, 16, 256) && p->tile_rows != kHeadsRows)
+        return launch_plain(a, p->rank, p->rope, f16, fp8, p->phases, stream);
     return CRIT_PKV_E_GEOMETRY;
 }
 

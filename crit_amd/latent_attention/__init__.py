@@ -42,7 +42,8 @@ PARTIAL_BYTES = 512 << 20   # the most partials one launch may take; a larger ba
 PIECE = 256                 # default positions a piece
 PIECE_MANY_HEADS = 512      # ... where the many-heads kernel reads (TILE_ROWS 128)
 MAX_PARTS = 64
-SHAPES = tuple((r, p) for r in (1024, 512, 256, 128, 64) for p in (256, 128, 64, 32))   # (R, P) the kernels are built for
+SHAPES = tuple((r, p) for r in (1024, 512, 256, 128, 64) for p in (256, 128, 64, 32))   # (R, P) the matrix-core kernels read;
+# ranks 16 and 32 and a rotary width of 16 are served by a kernel of plain vector arithmetic
 FP8 = torch.float8_e4m3fn
 _DTYPE = {torch.float32: _abi.F32, torch.bfloat16: _abi.BF16, torch.float16: _abi.F16}
 _CACHE_DTYPE = {torch.bfloat16: 0, torch.float16: 1, FP8: 2}
@@ -169,9 +170,6 @@ class _Call:
             if sinks.dtype != torch.float32 or tuple(sinks.shape) != (self.heads,) or not sinks.is_contiguous() or \
                     sinks.device != q.device:
                 raise ValueError(f"sinks: one FP32 logit a head, contiguous [{self.heads}] on q's device")
-        if (self.rank, self.rope) not in SHAPES:
-            raise NotImplementedError(f"latent_attention (gfx950): rank {self.rank} with a rotary width of {self.rope} is "
-                                      f"not built: ranks 64 to 1024 with rotary widths 32 to 256 are")
         if cache.device != q.device:
             raise ValueError(f"cache is on {cache.device}, q on {q.device}")
 

@@ -96,10 +96,6 @@ def _derived(given, d, device):
     return found._replace(eps=eps, rotary_dim=rot, table=table), weight is not None
 
 
-def _unsupported(what):
-    return NotImplementedError(f"paged_kv_attention (gfx950): {what} is not served by these kernels")
-
-
 # -- owners: what the module itself keeps on a device (reference __init__.py:129-171 keeps its workspaces the same way) --
 class _Holding:
     """One owner's memory on one device: the partials of its split launches (`latent`: those of its latent-attention

@@ -90,7 +90,12 @@ def _q(tokens, heads, width, seed, dtype=torch.bfloat16):
                                                  (512, 128, 24, 16), (1024, 32, 2, 16), (1024, 128, 4, 32), (1024, 256, 16, 16),
                                                  (512, 32, 16, 64), (512, 256, 3, 16), (256, 32, 6, 16), (256, 128, 8, 32),
                                                  (256, 256, 1, 16), (128, 128, 5, 16), (128, 256, 20, 16), (64, 128, 2, 48),
-                                                 (64, 256, 7, 16)])
+                                                 (64, 256, 7, 16),
+                                                 # ranks and rotary widths below the matrix tiles: the vector kernel
+                                                 (16, 16, 3, 16), (32, 16, 16, 48), (16, 256, 5, 16), (32, 64, 8, 64),
+                                                 (1024, 16, 2, 16), (512, 16, 16, 32), (64, 16, 7, 16), (32, 32, 4, 16),
+                                                 (16, 64, 1, 16), (128, 16, 6, 16), (256, 16, 3, 16), (16, 32, 2, 16),
+                                                 (16, 128, 2, 16), (32, 128, 3, 16), (32, 256, 2, 16)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_windows_match_float64_latent_attention(rank, rope, heads, page, dtype):
     cache = Cache(rank, rope, page, [130, 64, 1, 517], dtype=dtype)
@@ -219,8 +224,6 @@ def test_what_it_cannot_read_is_refused():
         cache.attend(q, [0], [0], [5], 65)
     with pytest.raises(ValueError, match="sinks: one FP32 logit a head"):
         cache.attend(q, [0], [0], [5], 1, sinks=torch.zeros(3, device=dev))
-    with pytest.raises(NotImplementedError, match="is not built"):      # (the reference takes every power of two)
-        la.attend(q[:, :, :48].contiguous(), torch.zeros(4, 64, 48, dtype=torch.bfloat16, device=dev), cache.tables, *some(), 1, 64, rank=32)
     codes = torch.zeros(4, 64, 576, dtype=torch.float8_e4m3fn, device=dev)
     with pytest.raises(ValueError, match="E4M3 cache takes its scales"):
         la.attend(q, codes, cache.tables, *some(), 1, 64, rank=512)
@@ -228,7 +231,8 @@ def test_what_it_cannot_read_is_refused():
         cache.attend(q, [0], [0], [5], 1, piece=48)
 
 
-@pytest.mark.parametrize("rank,rope", [(512, 64), (64, 32), (128, 32), (256, 128), (1024, 256), (64, 256)])
+@pytest.mark.parametrize("rank,rope", [(512, 64), (64, 32), (128, 32), (256, 128), (1024, 256), (64, 256), (16, 16), (32, 64),
+                                       (512, 16), (16, 256)])
 @pytest.mark.parametrize("scales", [2, 1])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_an_e4m3_cache_matches_float64_over_its_stored_values_and_keeps_a_tokens_bits(scales, dtype, rank, rope):
@@ -242,6 +246,27 @@ def test_an_e4m3_cache_matches_float64_over_its_stored_values_and_keeps_a_tokens
         for c in range(4):
             alone = cache.attend(q[start + c:start + c + 1], [s], [0], [first + c], 1, scale=scale)
             assert torch.equal(alone[0], out[start + c]), (s, c)
+
+
+@pytest.mark.parametrize("rank,rope", [(16, 16), (32, 64), (1024, 16)])
+@pytest.mark.parametrize("coded", [0, 2])
+def test_shapes_below_the_matrix_tiles_keep_a_tokens_bits_and_deal_their_pieces_round(rank, rope, coded):
+    kind = dict(dtype=torch.float8_e4m3fn, scales=coded) if coded else {}
+    cache = Cache(rank, rope, 16, [3000, 70], seed=21, **kind)
+    q = _q(8, 6, rank + rope, 22)
+    lse = torch.empty(8, 6, device=dev)
+    scale = 0.11
+    together = cache.attend(q, [0, 1], [0, 4], [2990, 60], 4, scale=scale, lse=lse)
+    for s, start, first in ((0, 0, 2990), (1, 4, 60)):
+        cache.check(q, together, lse, s, start, first, 4, scale)
+        for c in range(4):
+            alone = cache.attend(q[start + c:start + c + 1], [s], [0], [first + c], 1, scale=scale)
+            assert torch.equal(alone[0], together[start + c]), (s, c)
+    # few partitions: partition b reads pieces b, b + partitions, ...; a piece that is no multiple of a step of 64
+    for parts, piece in ((1, 512), (3, 96), (5, 32)):
+        out = cache.attend(q, [0, 1], [0, 4], [2990, 60], 4, scale=scale, lse=lse, partitions=parts, piece=piece)
+        for s, start, first in ((0, 0, 2990), (1, 4, 60)):
+            cache.check(q, out, lse, s, start, first, 4, scale)
 
 
 @pytest.mark.parametrize("scales", [2, 1])
@@ -271,7 +296,7 @@ def test_an_e4m3_cache_under_the_many_heads_kernel_matches_float64_and_keeps_a_t
     cache.check(few, packed, lse, 2, 0, 2060, 40, scale)
 
 
-@pytest.mark.parametrize("rank,rope,heads,page", [(512, 64, 16, 64), (512, 64, 128, 16), (128, 32, 20, 16)])
+@pytest.mark.parametrize("rank,rope,heads,page", [(512, 64, 16, 64), (512, 64, 128, 16), (128, 32, 20, 16), (32, 16, 4, 16)])
 def test_prompt_chunks_match_float64_and_are_their_positions_decoded(rank, rope, heads, page):
     cache = Cache(rank, rope, page, [900], seed=11)
     la = cache.la
