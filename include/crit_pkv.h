@@ -411,7 +411,9 @@ int crit_pkv_step_buffers(const crit_pkv_step_params* p, void* stream);
  * partition order, the sink logit (sinks [heads], natural log, -inf: none) folded in last; lse [tokens][heads] the
  * natural log-sum-exp (the sink counted). cache_dtype: 0 BF16, 1 FP16 (q in the same type), 2 E4M3 with `scales`
  * [pages][page][scales_per_row] FP32 (2: the latent's and the rotary key's, 1: one for the row) and BF16 or FP16 q.
- * rank is one of 64, 128, 256, 512, 1024 and rope one of 32, 64, 128, 256 (anything else: CRIT_PKV_E_GEOMETRY). phases:
+ * rank is a power of two from 16 to 1024 and rope one from 16 to 256, as the reference's module takes them (anything
+ * else: CRIT_PKV_E_GEOMETRY); ranks from 64 with widths from 32 are read on the matrix pipe, the smaller ones by plain
+ * vector arithmetic. phases:
  * 0 both launches, 1 the partitions only, 2 the merge only.
  * tile_rows: the query rows a workgroup holds, which decides the kernel and with it a token's bits. 16: tiles of 16 rows
  * (two a workgroup from 32 rows on), every geometry, the fastest for a few batch rows. 128: 128 rows a workgroup on
