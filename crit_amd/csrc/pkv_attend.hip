@@ -66,7 +66,7 @@ __global__ __launch_bounds__(64) void merge_kernel(AttendArgs a) {
         constexpr int U = EPL > 2 ? 16 : 32;
         float po[2][U][EPL], pm_next, pl_next;
         auto load_scalars = [&](int b0) __attribute__((always_inline)) {
-            const int b = min(b0 + (lane & (U - 1)), nb - 1);
+            const int b = min(b0 + ((int)threadIdx.x & (U - 1)), nb - 1);      // (the thread's own place: `lane` is clamped to the value row)
             pm_next = a.pm[at + b], pl_next = a.pl[at + b];
         };
         auto load_values = [&](int b0, float (&dst)[U][EPL]) __attribute__((always_inline)) {
@@ -78,7 +78,7 @@ __global__ __launch_bounds__(64) void merge_kernel(AttendArgs a) {
             }
         };
         auto fold_batch = [&](int b0, float pm, float pl, const float (&val)[U][EPL]) __attribute__((always_inline)) {
-            const int u_lane = lane & (U - 1);
+            const int u_lane = (int)threadIdx.x & (U - 1);
             if (b0 + u_lane >= nb) pm = -INFINITY, pl = 0.0f;      // (lanes past the last partition are not folded below)
             float upto = pm;      // the maximum of this batch's partitions up to the lane's
 #pragma unroll

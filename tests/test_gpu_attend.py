@@ -173,16 +173,20 @@ def test_a_fused_launch_gives_a_column_the_split_launchs_bits(kind, hq, hkv, d, 
         _close_lse(lse[:3], want_lse)
 
 
-@pytest.mark.parametrize("kind,hq,hkv,d", [("bf16", 8, 2, 128), ("fp8", 24, 4, 256), ("bf16", 8, 2, 64)])
-def test_a_row_of_many_partitions_merges_to_the_fused_launchs_bits(kind, hq, hkv, d):
+@pytest.mark.parametrize("kind,hq,hkv,d,dv", [("bf16", 8, 2, 128, 128), ("fp8", 24, 4, 256, 256), ("bf16", 8, 2, 64, 64),
+                                              # value rows narrower than a wavefront: the merge's lanes past them
+                                              # still take a partition each
+                                              ("bf16", 4, 2, 16, 16), ("int8", 6, 2, 32, 32), ("fp8:row", 2, 1, 128, 16),
+                                              ("bf16", 3, 3, 32, 64)])
+def test_a_row_of_many_partitions_merges_to_the_fused_launchs_bits(kind, hq, hkv, d, dv):
     # Long rows cut into many partitions (the long-context split): the merge takes the maxima and exponentials of a
     # batch of partitions on as many lanes and keeps only the sums in order; the fused launch folds one partition
     # after another. The same bits for 9 partitions (the first count past the one-by-one merge), one batch exactly,
     # a few batches with a ragged last one, a count no row fills; with sinks; and the oracle.
     pk = kernels()
-    block = pk.flash_block(d, d, hq, hkv, 16, kind)
-    cache = Cache(kind, hkv, d, d, 16, [40 * block * 5 + 7], seed=51)
-    n = cache.lengths[0] if hasattr(cache, "lengths") else 40 * block * 5 + 7
+    block = pk.flash_block(d, dv, hq, hkv, 16, kind)
+    cache = Cache(kind, hkv, d, dv, 16, [40 * block * 5 + 7], seed=51)
+    n = cache.lengths[0]
     q = rand_q(3, hq, d, 52)
     sinks = torch.linspace(-1, 1, hq, device=dev)
     for parts, piece in ((9, block * 23), (32, block * 6), (16, block * 6), (77, block * 2), (500, block)):
