@@ -91,9 +91,13 @@ __global__ __launch_bounds__(256) void compact_kernel(Tables t, Stores stores, c
         const int64_t node = path_is_32 ? (int64_t) reinterpret_cast<const int32_t*>(path)[r * path_stride + tid]
                                         : reinterpret_cast<const int64_t*>(path)[r * path_stride + tid];
         if (node >= 0) {
-            keep = 1;
             src = slot_at(t, r, first + node);
             dst = slot_at(t, r, first + tid);
+            // A target past the slot's capacity is the dump page: nothing is moved there. The reference's index_copy_
+            // leaves one of the rows sent there, which one is not defined; what is defined is that a SOURCE past the
+            // capacity reads the dump page as it was before the move, and it stays so only if no row's workgroup
+            // writes it meanwhile.
+            keep = dst != t.dump_slot;
         }
     }
     // (a column's place in the list: the kept columns before it, counted a wavefront at a time)

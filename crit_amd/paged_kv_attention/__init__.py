@@ -1011,6 +1011,8 @@ def compact(stores, slots, round_tables, round_capacity, start, emitted, path, m
     """An accepted draft-tree path's rows to consecutive positions, KVPool._compact (pages.py:662-684) in one launch
     over every layer and store: for round row r (round slot r) where moved[r] == 0, node path[r][j] at position
     start[r] + path[r][j] moves to start[r] + j for 0 < j < emitted[r] with path[r][j] >= 0; then moved[:rows] = 1.
+    Every slot outside the dump page ends as the reference leaves it; the dump page itself is read (a node past its
+    slot's capacity) and never written (what the reference leaves there is one of several rows, undefined which).
     stores: the pool's tensors [layers][...] (keys, values, row scales; None entries skipped), each layer `slots` rows;
     path [rows][width] int64 or int32 (up to 256 columns); start, emitted, moved int64 [rows or more]."""
     _tables(round_tables, round_capacity)

@@ -309,8 +309,10 @@ int crit_pkv_slots_at(const crit_pkv_slots_params* p, void* stream);
  * r) and column 0 < j < min(width, emitted[r]) with path[r][j] >= 0, where moved[r] == 0, the row of every store and
  * layer at position start[r] + path[r][j] is copied to position start[r] + j (slots as crit_pkv_slots_at finds them:
  * a position outside the slot's capacity is the dump page's first slot). All of a row's sources are read before any
- * of its targets is written, as index_copy_(index_select()) does. Then moved[r] = 1 for every r < rows (a second
- * launch on the same stream). */
+ * of its targets is written, as index_copy_(index_select()) does. A target outside the capacity (the dump page's
+ * first slot) is not written: the reference leaves one of the rows sent there, which one is undefined, and a source
+ * outside the capacity must read the dump page as it was before the move whichever row's workgroup runs first. Then
+ * moved[r] = 1 for every r < rows (a second launch on the same stream). */
 typedef struct crit_pkv_compact_params {
     const int32_t* round_tables;
     const int64_t* round_capacity;

@@ -156,6 +156,38 @@ def test_compact_of_the_widest_path_and_of_sources_past_capacity():
                    start.to(dev), emitted.to(dev), path.to(dev), moved.to(dev), page, dump)
 
 
+def test_compact_reads_the_dump_page_as_it_was_and_leaves_it_so():
+    # Rows whose windows run past their slots' capacity: their targets there are the dump page's first slot, and so is
+    # the source of an accepted node past the capacity. index_copy_(index_select()) reads every source first, so such
+    # a node's target gets the dump page's row as it was before the move, whatever other rows send there meanwhile;
+    # what the dump page holds afterwards is one of the rows sent to it in the reference (undefined which) and the
+    # row it held here. Every other slot: equal to the reference's.
+    pk = kernels()
+    page, layers, rows = 16, 4, 9
+    lengths = [(s, 40 + 3 * s) for s in range(rows)]
+    tables, capacity, dump = _round_pool(page, 12, lengths, rows, seed=11)
+    slots = (dump + 1) * page
+    stores = _stores("fp8:row", layers, slots, 3, 16, 12)
+    start = capacity - 4                      # a window of 12 columns: 8 of them past the capacity
+    emitted = torch.full((rows,), 12)
+    path = torch.arange(12).repeat(rows, 1)
+    path[:, 1] = 9                            # column 1 (inside) takes node 9 (past the capacity: the dump page's row)
+    path[:, 2] = 3
+    path[:, 3] = 2
+    moved = torch.zeros(rows, dtype=torch.int64)
+    want = [s.clone() for s in stores]
+    oracle_pool.compact(want, slots, tables, capacity, start, emitted, path, moved.clone(), page, dump)
+    for _ in range(5):      # (which workgroup runs first differs from launch to launch)
+        got = [s.to(dev) for s in stores]
+        pk.compact(got, slots, tables.to(dev), capacity.to(dev), start.to(dev), emitted.to(dev), path.to(dev), moved.to(dev), page, dump)
+        for i, (a, b, before) in enumerate(zip(got, want, stores)):
+            a, b, before = (bits(x).cpu().reshape(layers, slots, -1) for x in (a, b, before))
+            assert torch.equal(a[:, :dump * page], b[:, :dump * page]), f"store {i}"
+            assert torch.equal(a[:, dump * page:], before[:, dump * page:]), f"store {i}: the dump page"
+            r = int(oracle_pool.slots_at(tables, capacity, torch.tensor([0]), start[:1] + 1, page, dump)[0])
+            assert torch.equal(a[:, r], before[:, dump * page]), "the dump page's row as it was"
+
+
 @pytest.mark.parametrize("kind,hkv,d,page", [("bf16", 8, 128, 16), ("fp8:row", 8, 128, 16), ("int8", 2, 64, 4), ("fp16", 1, 6, 2)])
 @pytest.mark.parametrize("interleaved", [False, True])
 def test_pages_are_copied_whole_in_every_layer_and_store(kind, hkv, d, page, interleaved):
