@@ -12,9 +12,11 @@ from . import append
 
 
 # -- the float64 reference over stored values (test_paged_kv_attention.py:71-81) ---------------------------------------
-def reference(q, keys, values, seen, scale):
+def reference(q, keys, values, seen, scale, late=None):
     """q [HQ][D] float64 over keys [n][HKV][D], values [n][HKV][DV] where seen [n] (bool) -> (out [HQ][DV], lse [HQ]).
-    A head that sees nothing gets zeros and -inf."""
+    A head that sees nothing gets zeros and -inf. late = (queries [HQ][D], position): the positions from `position` on
+    are scored with those queries instead (an int8_qk chunk's fresh rows meet the queries as they are, the pages' rows
+    their INT8 codes: _kernels.py:668-671, 708-709)."""
     hq, hkv = q.shape[0], keys.shape[1]
     group = hq // hkv
     out, lse = [], []
@@ -22,6 +24,8 @@ def reference(q, keys, values, seen, scale):
     for h in range(hq):
         k, v = keys[:, h // group], values[:, h // group]
         s = (k @ q[h]) * scale
+        if late is not None:
+            s = torch.where(torch.arange(k.shape[0]) >= late[1], (k @ late[0][h]) * scale, s)
         s = torch.where(seen, s, neg)
         if not bool(seen.any()):
             out.append(torch.zeros(values.shape[-1], dtype=torch.float64))
@@ -106,20 +110,21 @@ def window_reference(q, key_pages, value_pages, kind, table, first, count, page,
     """One window row in float64: q [count][HQ][D] (rounded to q_dtype first, as the kernels read it) at positions
     first .. first + count - 1 -> (out [count][HQ][DV], lse [count][HQ]). parents: the row's draft tree (seen_by);
     blocks [count][k] with block_size: each column's listed KV blocks (listed); fresh: with_fresh's tuple; int8_qk: the
-    queries as int8_rows gives them (pages only: not with fresh)."""
+    queries as int8_rows gives them against the pages' positions, as they are against the fresh ones."""
     n = first + count
     keys, values = stored_rows(key_pages, value_pages, table, n, page, kind, key_scales, value_scales, multipliers)
     if fresh is not None:
         keys, values = with_fresh(keys, values, fresh, q_dtype)
     qd = q.to(q_dtype).double()
+    as_given = None
     if int8_qk:
-        qd = int8_rows(q.to(q_dtype))
+        as_given, qd = (qd, max(int(fresh[3]), 0)) if fresh is not None else None, int8_rows(q.to(q_dtype))
     outs, lses = [], []
     for c in range(count):
         seen = seen_by(first, count, c, n, parents, sliding)
         if blocks is not None:
             seen = seen & listed(blocks[c], block_size, n)
-        o, l = reference(qd[c], keys, values, seen, scale)
+        o, l = reference(qd[c], keys, values, seen, scale, None if as_given is None else (as_given[0][c], as_given[1]))
         outs.append(o)
         lses.append(l)
     return torch.stack(outs), torch.stack(lses)

@@ -367,6 +367,9 @@ def test_int8_queries_against_int8_keys(hq, hkv, d):
     mixed = pk.prefill(q.bfloat16(), cache.k, cache.v, "int8", cache.tables[0], 350, 16, int8_qk=True, fresh=(fk, fv), **kw)
     plain = pk.prefill(q.bfloat16(), cache.k, cache.v, "int8", cache.tables[0], 350, 16, fresh=(fk, fv), **kw)
     assert float((mixed.float() - plain.float()).abs().max()) < 0.06
+    for t in (0, 1, 75, 149):      # (the oracle scores the pages' positions with the codes, the fresh ones with q itself)
+        want, _ = cache.want(q[t:t + 1], 0, 350 + t, 1, int8_qk=True, fresh=(fk.cpu(), fv.cpu(), 350, 350))
+        torch.testing.assert_close(mixed[t:t + 1].double().cpu(), want, atol=ATOL, rtol=RTOL, msg=f"int8_qk with fresh rows, token {t}")
     first = pk.prefill(q.bfloat16(), cache.k, cache.v, "int8", cache.tables[0], 0, 16, int8_qk=True, fresh=(fk, fv), **kw)
     assert torch.equal(first, pk.prefill(q.bfloat16(), cache.k, cache.v, "int8", cache.tables[0], 0, 16, fresh=(fk, fv), **kw))
 

@@ -641,6 +641,40 @@ def test_int8_query_rows_are_their_codes_times_their_scale():
         assert torch.allclose(out[c], want, atol=1e-12) and torch.allclose(lse[c], want_lse, atol=1e-12)
 
 
+def test_an_int8_chunks_fresh_rows_meet_the_queries_as_they_are():
+    # Pins window_reference(int8_qk=True, fresh=...) and reference(late=): the pages' positions are scored with the
+    # queries' INT8 codes times their scale, the fresh ones (from `first` on) with the 16-bit queries themselves
+    # (_kernels.py:668-671 against 708-709). Checked against a softmax written out position by position in plain Python.
+    k, v, ks, vs, tables, _ = _pool("int8", 2, 16, 16, 16, [40])
+    g = torch.Generator().manual_seed(9)
+    q = torch.randn(3, 4, 16, generator=g)
+    fk, fv = torch.randn(3, 2, 16, generator=g).bfloat16(), torch.randn(3, 2, 16, generator=g).bfloat16()
+    first = 38                                           # the chunk is positions 37..39; 38 and 39 are fresh
+    out, lse = attend.window_reference(q, k, v, "int8", tables[0], 37, 3, 16, 0.25, ks, vs, int8_qk=True,
+                                       fresh=(fk, fv, 37, first))
+    keys, values = attend.stored_rows(k, v, tables[0], 40, 16, "int8", ks, vs)
+    coded, given = attend.int8_rows(q.bfloat16()), q.bfloat16().double()
+    for c in range(3):
+        for h in range(4):
+            scores, rows = [], []
+            for n in range(37 + c + 1):
+                if n >= first:
+                    key, value, query = fk[n - 37, h // 2].double(), fv[n - 37, h // 2].double(), given[c, h]
+                else:
+                    key, value, query = keys[n, h // 2], values[n, h // 2], coded[c, h]
+                scores.append(float(key @ query) * 0.25)
+                rows.append(value)
+            top = max(scores)
+            weights = [math.exp(x - top) for x in scores]
+            total = sum(weights)
+            want = sum(w / total * r for w, r in zip(weights, rows))
+            assert torch.allclose(out[c, h], want, atol=1e-12), (c, h)
+            assert abs(float(lse[c, h]) - (top + math.log(total))) < 1e-12
+    # the difference is there to see: scoring the fresh rows with the codes too gives another answer
+    other, _ = attend.window_reference(q, k, v, "int8", tables[0], 37, 3, 16, 0.25, ks, vs, int8_qk=True)
+    assert not torch.allclose(out, other, atol=1e-4)
+
+
 # -- the pool's device-side bookkeeping ------------------------------------------------------------------------------------
 def _round_pool(page=4, table_pages=6, lengths=((0, 17), (1, 9), (3, 24)), round_slots=4, seed=0):
     """Round tables of a few bound sequences over shuffled pages; unbound slots and the entries past a sequence's pages
