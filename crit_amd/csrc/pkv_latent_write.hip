@@ -48,9 +48,15 @@ __global__ __launch_bounds__(256) void latent_write_kernel(LatentWriteArgs a) {
         const int64_t to = slot * row_width + (which ? a.width[0] : 0);
         if constexpr (CACHE < 2) {
             uint16_t* dst = reinterpret_cast<uint16_t*>(a.cache) + to;
-            for (int i = lane; i < n; i += 64) {
-                const float x = in_value<IN>(src, from + i);
-                dst[i] = (uint16_t)(CACHE == 1 ? f16_bits(x) : bf16_rne(x));
+            if constexpr ((IN == CRIT_PKV_BF16 && CACHE == 0) || (IN == CRIT_PKV_F16 && CACHE == 1)) {
+                // rows of the cache's own type are stored as they are, every bit (the reference's .to() of the same
+                // dtype is the tensor itself: a NaN keeps its payload)
+                for (int i = lane; i < n; i += 64) dst[i] = reinterpret_cast<const uint16_t*>(src)[from + i];
+            } else {
+                for (int i = lane; i < n; i += 64) {
+                    const float x = in_value<IN>(src, from + i);
+                    dst[i] = (uint16_t)(CACHE == 1 ? f16_bits(x) : bf16_rne(x));
+                }
             }
         } else {
             float amax = 0.0f;

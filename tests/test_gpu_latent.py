@@ -391,6 +391,19 @@ def test_the_partitions_are_a_knob_the_caller_or_the_tuning_sets():
             cache.attend(q, [0, 1], [0, 8], [2990, 890], 8, partitions=bad)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_write_keeps_every_bit_of_rows_of_the_caches_own_type(dtype):
+    # every 16-bit pattern once (NaNs with their payloads and signs, subnormals, both zeros) as latents and rotary keys
+    la = module()
+    patterns = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype)
+    latent, rope_k = patterns[:49152].reshape(384, 128), patterns[49152:].reshape(512, 32)[:384]
+    slots = torch.randperm(400, generator=torch.Generator().manual_seed(5))[:384]
+    cache = torch.zeros(25, 16, 160, dtype=dtype, device=dev)
+    la.write(latent.to(dev), rope_k.to(dev), slots.to(dev), cache)
+    rows = cache.cpu().view(torch.int16).reshape(400, 160)[slots]
+    assert torch.equal(rows[:, :128], latent.view(torch.int16)) and torch.equal(rows[:, 128:], rope_k.view(torch.int16))
+
+
 @pytest.mark.parametrize("source", [torch.float32, torch.bfloat16, torch.float16])
 def test_write_stores_the_bytes_and_scales_of_the_reference_rule(source):
     # oracle.latent.write is the reference's torch rule (latent_attention/__init__.py:74-97); the module's write is one
@@ -419,8 +432,8 @@ def test_write_stores_the_bytes_and_scales_of_the_reference_rule(source):
         la.write(latent.to(dev), rope_k.to(dev), dropped, got, got_scales)
         raw = torch.uint8 if coded else torch.int16
 
-        def same(a, b):      # bit for bit; a 16-bit NaN only as a NaN (its payload differs between torch's own casts)
-            if coded:
+        def same(a, b):      # bit for bit; a 16-bit NaN that went through a cast only as a NaN (its payload differs
+            if coded or source == dtype:      # between torch's own casts); rows of the cache's own type: every bit
                 return torch.equal(a.view(raw), b.view(raw))
             nan = torch.isnan(b.float())
             return torch.equal(torch.isnan(a.float()), nan) and torch.equal(a.view(raw)[~nan], b.view(raw)[~nan])
