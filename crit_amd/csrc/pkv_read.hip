@@ -45,6 +45,7 @@ __global__ __launch_bounds__(256) void read_rows_kernel(ReadArgs a) {
         slot = (a.table ? (int64_t)a.table[entry] : a.table64[entry]) * a.page + i % a.page;
     }
     float x[E];
+    u32x4 as_stored = {0u, 0u, 0u, 0u};      // 16-bit pages read back in their own type: the bits as they are
     if (slot < 0 || (a.pool_slots > 0 && slot >= a.pool_slots)) {
 #pragma unroll
         for (int j = 0; j < E; ++j) x[j] = 0.0f;
@@ -53,6 +54,7 @@ __global__ __launch_bounds__(256) void read_rows_kernel(ReadArgs a) {
         if constexpr (KIND == 0) {
             const u32x4 w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a.pages[which] + (row * a.dim[which] + c * 8) * 2));
             const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+            as_stored = w;
             if (a.f16_pages) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) x[2 * j] = f16_lo(ws[j]), x[2 * j + 1] = f16_hi(ws[j]);
@@ -96,6 +98,13 @@ __global__ __launch_bounds__(256) void read_rows_kernel(ReadArgs a) {
     } else {
         u32x4* o = reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(a.out[which]) + at);
         const bool bf = a.out_dtype == CRIT_PKV_BF16;
+        if constexpr (KIND == 0) {
+            // (the reference's .to(compute) of the pages' own dtype is the tensor itself: a NaN keeps its payload)
+            if (bf != (a.f16_pages != 0)) {
+                o[0] = as_stored;
+                return;
+            }
+        }
 #pragma unroll
         for (int j = 0; j < E / 8; ++j) {
             u32x4 w;

@@ -65,6 +65,27 @@ def test_rows_at_slots_and_a_sequences_first_positions_read_back_as_torch_does(k
     _equal(out[0], want_k, "keys only")
 
 
+@pytest.mark.parametrize("kind,dtype", [("bf16", torch.bfloat16), ("fp16", torch.float16)])
+def test_sixteen_bit_pages_read_back_in_their_own_type_keep_every_bit(kind, dtype):
+    # KVPool.gather's rows.to(compute) of the pages' own dtype is the tensor itself (pages.py:455-477): every one of
+    # the 65,536 bit patterns comes back as it is stored, a NaN with its payload and sign; read back as FP32 (rows_at)
+    # every number is exact and a NaN is a NaN.
+    pk = kernels()
+    patterns = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype)
+    k = patterns.reshape(16, 16, 2, 128)
+    v = patterns.flip(0).reshape(16, 16, 2, 128)
+    table = torch.randperm(16, generator=torch.Generator().manual_seed(2)).to(torch.int32)
+    gk, gv = pk.gather(k.to(dev), v.to(dev), kind, table.to(dev), 250, 16, dtype=dtype)
+    want_k, want_v = oracle_attend.gather(k, v, table, 250, 16, kind, dtype)
+    assert torch.equal(gk.cpu().view(torch.int16), want_k.view(torch.int16))
+    assert torch.equal(gv.cpu().view(torch.int16), want_v.view(torch.int16))
+    slots = torch.arange(256)
+    rk, _ = pk.rows_at(k.to(dev), v.to(dev), kind, slots.to(dev))
+    want = k.reshape(256, 2, 128).float()
+    numbers = ~torch.isnan(want)
+    assert torch.equal(torch.isnan(rk.cpu()), ~numbers) and torch.equal(rk.cpu()[numbers], want[numbers])
+
+
 def test_per_head_multipliers_and_what_is_refused():
     pk = kernels()
     k, v, _, _ = _pool("fp8", 8, 16, 4, 128, 128, 33)
