@@ -239,7 +239,6 @@ def append_sweep(pk, device, kind):
         kernel = graph_timed(call)
         nbytes = T * hkv * 2 * d * (e + 2)
         found[str(T)] = {"us": round(ms * 1e3, 2), "kernel_us": round(kernel * 1e3, 2),
-                         "kernel_GB/s": round(nbytes / kernel / 1e6, 1),
                          "kernel_frac_of_peak": round(nbytes / kernel / 1e6 / HBM_PEAK_GBPS, 4)}
     return found
 
@@ -1124,7 +1123,7 @@ def main():
                                        "achieved": round(ow.decode_bytes / osplit / 1e6, 1), "peak": HBM_PEAK_GBPS,
                                        "unit": "GB/s", "frac": round(ow.decode_bytes / osplit / 1e6 / HBM_PEAK_GBPS, 4),
                                        "traffic": otraffic, "traffic_source": osource, "launch_ms": round(osplit, 4),
-                                       "algorithmic_bytes_per_launch": ow.decode_bytes, "workload": ospec["name"]}
+                                       "algorithmic_bytes_per_launch": ow.decode_bytes, "workload": other}
         # the same launches with pieces twice as long (attend's piece=, a deployment's choice through the plugin's
         # `piece` option: fixed per pool like the default; halves the units' fixed costs, and a small batch's units)
         ow.piece *= 2
