@@ -298,7 +298,7 @@ def long_context(pk, device):
             firsts = torch.full((batch,), ctx - 1, dtype=torch.int64, device=device)
             out = torch.empty(batch, hq, d, dtype=torch.bfloat16, device=device)
             nbytes = batch * ctx * hkv * 2 * d * 2
-            for chunk in (512, 1024, 2048):
+            for chunk in (512, 2048):
                 parts = pk.flash_parts(tables.shape[1] * page, chunk)
                 ws = torch.empty(pk.workspace_floats(batch, hq, parts, d), dtype=torch.float32, device=device)
                 call = lambda phases=0: pk.attend(q, k, v, "bf16", tables, rows, rows, firsts, 1, page, flash=True,
