@@ -1,4 +1,5 @@
-"""Seeded sweeps over the geometry of the attention entry points: every case draws its page kind, head widths (keys' and
+"""Seeded sweeps over the geometry of the attention entry points (paged windows, block lists, prompt chunks, latent
+windows, index selection): every case draws its page kind, head widths (keys' and
 values'), KV heads and GQA group, page size (powers of two and not), rows' lengths, window widths and live columns,
 sliding window, draft tree, piece and partitions from its seed, and is checked against float64 attention over the stored
 values (2e-2, as everywhere) with the split launch and the fused launch bit for bit the same. What the hand-picked
@@ -155,3 +156,96 @@ def test_prompt_chunks_of_any_geometry(seed):
         head = pk.prefill(q[:cut].to(q_dtype), cache.k, cache.v, kind, table, position, page, **kw)
         tail = pk.prefill(q[cut:].to(q_dtype), cache.k, cache.v, kind, table, position + cut, page, **kw)
         assert torch.equal(torch.cat([head, tail]), out), (seed, cut)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_latent_windows_of_any_geometry(seed):
+    # every rank and rotary width the reference's module takes (the matrix-core kernels' shapes, the many-heads kernel
+    # where it may read, and the shapes below the tiles), 16-bit and E4M3 caches with two scales a row or one
+    from tests.test_gpu_latent import Cache as LatentCache, _q
+    draw = random.Random(seed)
+    if draw.random() < 0.4:
+        rank, rope = 512, 64
+    else:
+        rank, rope = draw.choice([16, 32, 64, 128, 256, 512, 1024]), draw.choice([16, 32, 64, 128, 256])
+    heads = draw.choice([1, 2, 3, 5, 8, 16, 16, 20, 40, 64, 128])
+    if rank * heads > 512 * 128:
+        heads = 16
+    page = draw.choice([16, 16, 32, 64, 48, 8, 1, 128])
+    coded = draw.choice([0, 0, 2, 1])
+    dtype = draw.choice([torch.bfloat16, torch.float16])
+    lengths = [draw.choice([1, 2, 31, 32, 33, 64, 255, 256, 257, 700, 1500, 3000]) + draw.randint(0, 20)
+               for _ in range(draw.randint(1, 4))]
+    cols = draw.choice([1, 1, 2, 3, 5, 8])
+    rows, starts, firsts, counts, tokens = _rows(draw, lengths, cols)
+    kw = dict(counts=torch.tensor(counts, dtype=torch.int32, device=dev))
+    if draw.random() < 0.3:
+        kw["piece"] = draw.choice([32, 64, 96, 256, 512, 1024])
+    if draw.random() < 0.3:
+        kw["partitions"] = draw.choice([1, 3, 8, 64])
+    if (rank, rope) == (512, 64) and page % 16 == 0 and draw.random() < 0.5:
+        kw["tile_rows"] = draw.choice([16, 128])
+    scale = draw.choice([None, 0.07])
+    kind = dict(dtype=torch.float8_e4m3fn, scales=coded) if coded else dict(dtype=dtype)
+    cache = LatentCache(rank, rope, page, lengths, seed=seed, **kind)
+    q = _q(tokens, heads, rank + rope, seed + 500, dtype)
+    sinks = torch.randn(heads, generator=torch.Generator().manual_seed(seed)).to(dev) if draw.random() < 0.3 else None
+    lse = torch.empty(tokens, heads, device=dev)
+    out = cache.attend(q, rows, starts, firsts, cols, lse=lse, sinks=sinks, scale=scale, **kw)
+    used = (rank + rope) ** -0.5 if scale is None else scale
+    for s, start, first, count in zip(rows, starts, firsts, counts):
+        cache.check(q, out, lse, s, start, first, count, used, sinks)
+        j = draw.randrange(count)      # a token alone in a window of one column: the same bits
+        alone = cache.attend(q[start + j:start + j + 1], [s], [0], [first + j], 1, sinks=sinks, scale=scale,
+                             **{**kw, "counts": None})
+        assert torch.equal(alone[0], out[start + j]), (seed, s, j)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_index_selection_of_any_geometry(seed):
+    import numpy as np
+
+    from crit_amd import sparse_indexer as si
+    from oracle import indexer as ref
+    from tests.test_gpu_indexer import compressed
+    draw = random.Random(seed)
+    heads, width = draw.choice([1, 2, 4, 8, 16, 32, 64, 128]), draw.choice([64, 128, 256])
+    e4m3 = draw.random() < 0.4
+    dtype = draw.choice([torch.bfloat16, torch.float16])
+    n = draw.choice([1, 5, 63, 64, 65, 200, 1000, 3000])
+    groups = draw.choice([0, 0, 1, 1, 2, 3, 5])      # 0: the keys as they lie; 1: one list of slots; more: a list a group
+    each = draw.choice([1, 2, 3, 4, 7, 8, 16, 20, 33])
+    tokens = each * max(1, groups)
+    k = draw.choice([1, 16, 64, 512])
+    store_n = n + draw.choice([0, 10, 500])
+    g = torch.Generator().manual_seed(seed)
+    rows = torch.empty(store_n, width).normal_(0.0, 0.5, generator=g).to(dev).to(dtype)
+    q = torch.empty(tokens, heads, width).normal_(0.0, 0.5, generator=g).to(dev).to(dtype)
+    w = (torch.empty(tokens, heads).normal_(generator=g) / heads ** 0.5).to(dev)
+    ends = (torch.rand(tokens, generator=g) * (n + 1)).long().clamp_(max=n).to(torch.int32).to(dev)
+    keys, scales, values = compressed(rows, e4m3)
+    kw, slots = {}, None
+    if groups == 0:
+        keys, values, scales = keys[:n], values[:n], None if scales is None else scales[:n]
+    elif groups == 1:
+        slots = torch.randperm(store_n, generator=g)[:n].to(dev)
+        kw["slots"] = slots.to(torch.int32) if draw.random() < 0.5 else slots
+    else:
+        slots = torch.stack([torch.randperm(store_n, generator=g)[:n] for _ in range(groups)]).to(dev)
+        kw["slots"] = slots
+    got = si.scores(q, keys, w, ends, key_scales=scales, **kw)
+    picks = si.topk(got, ends, k)
+    if groups <= 1:
+        assert torch.equal(si.select(q, keys, w, ends, k, key_scales=scales, **kw), picks), seed
+    f = lambda x: x.double().cpu().numpy()
+    for gi in range(max(1, groups)):
+        span = slice(gi * each, (gi + 1) * each) if groups > 1 else slice(None)
+        vals = values if slots is None else values[(slots if slots.dim() == 1 else slots[gi]).long()]
+        want = ref.sparse_scores(f(q[span]), f(vals), f(w[span]), ends[span].cpu().numpy(), width ** -0.5)
+        slack = ref.sparse_scores(f(q[span].abs()), f(vals.abs()), f(w[span].abs()), ends[span].cpu().numpy(), width ** -0.5) * 1e-4 + 1e-6
+        found = got[span].cpu().numpy()
+        seen = np.isfinite(want)
+        assert np.array_equal(seen, np.isfinite(found)) and (found[~seen] == -np.inf).all(), (seed, "the causal ends")
+        assert (np.abs(found.astype(np.float64)[seen] - want[seen]) <= slack[seen]).all(), (seed, "scores")
+        exact = torch.from_numpy(ref.sparse_index(got[span].double().cpu().numpy(), ends[span].cpu().numpy(), k))
+        assert torch.equal(picks[span].long().cpu(), exact), (seed, "picks")
