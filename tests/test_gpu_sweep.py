@@ -1,5 +1,5 @@
-"""Seeded sweeps over the geometry of the attention entry points (paged windows, block lists, prompt chunks, latent
-windows, index selection): every case draws its page kind, head widths (keys' and
+"""Seeded sweeps over the geometry of the entry points (paged windows, block lists, prompt chunks, latent windows, index
+selection against float64; appends, plain and with the keys' rope and norm fused in, byte for byte): an attention case draws its page kind, head widths (keys' and
 values'), KV heads and GQA group, page size (powers of two and not), rows' lengths, window widths and live columns,
 sliding window, draft tree, piece and partitions from its seed, and is checked against float64 attention over the stored
 values (2e-2, as everywhere) with the split launch and the fused launch bit for bit the same. What the hand-picked
@@ -249,3 +249,137 @@ def test_index_selection_of_any_geometry(seed):
         assert (np.abs(found.astype(np.float64)[seen] - want[seen]) <= slack[seen]).all(), (seed, "scores")
         exact = torch.from_numpy(ref.sparse_index(got[span].double().cpu().numpy(), ends[span].cpu().numpy(), k))
         assert torch.equal(picks[span].long().cpu(), exact), (seed, "picks")
+
+
+def _same_bytes(got, want, what):
+    """Stored tensors bit for bit; a NaN only as a NaN where `want` holds one (what a cast stores for it is the host's)."""
+    from tests.support import bits
+    got = got.cpu()
+    nan = torch.isnan(want.float())
+    assert torch.equal(torch.isnan(got.float()), nan), (what, "which are NaN")
+    assert torch.equal(bits(got)[~nan], bits(want)[~nan]), (what, int((bits(got)[~nan] != bits(want)[~nan]).sum()), "differ")
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_appends_of_any_geometry_store_the_oracles_bytes(seed):
+    # rows of any width (the scalar kernel's too), strided views of a wider projection output, keys only or values
+    # only, FP32 / BF16 / FP16 inputs into every page kind, magnitudes from 1e-2 to 1e3 and one far outlier, per-head
+    # multipliers, negative slots: every stored byte and row scale
+    from tests.support import STORE, expected_pages
+    draw = random.Random(seed)
+    pk = kernels()
+    kind = draw.choice(KINDS)
+    d = draw.choice([8, 16, 20, 32, 40, 64, 96, 128, 128, 192, 256, 512])
+    dv = d if draw.random() < 0.6 else draw.choice([8, 16, 24, 64, 128, 256])
+    hkv = draw.choice([1, 2, 3, 4, 8, 16])
+    T = draw.choice([1, 2, 3, 7, 64, 100, 257, 1000, 4152])
+    n_slots = T + draw.choice([0, 5, 100])
+    in_dtype = draw.choice([torch.float32, torch.bfloat16, torch.float16])
+    which = draw.choice(["both", "both", "both", "keys", "values"])
+    strided = draw.random() < 0.4
+    g = torch.Generator().manual_seed(seed)
+    if kind == "fp8" and draw.random() < 0.5:
+        mult = torch.rand(2, hkv, generator=g) * 0.04 + 0.01
+    else:
+        mult = (draw.choice([1.0, 0.05, 0.013]), draw.choice([1.0, 0.07]))
+    amp = draw.choice([0.01, 1.0, 30.0, 1000.0])
+    keys = (torch.randn(T, hkv, d, generator=g) * amp).to(in_dtype)
+    values = (torch.randn(T, hkv, dv, generator=g) * amp).to(in_dtype)
+    if T > 2:
+        keys[1] = 0.0
+        values[2, 0] = 0.0
+    if draw.random() < 0.3 and in_dtype != torch.float16:
+        keys[0, 0, 0] = 1e30
+    slots = torch.randperm(n_slots, generator=g)[:T]
+    for i in range(T):
+        if draw.random() < 0.05:
+            slots[i] = -1 - draw.randint(0, 3)
+
+    def on_device(x):
+        if not strided:
+            return x.to(dev)
+        width = x.shape[2]      # a view into a wider row, as a fused projection's output is
+        wide = torch.zeros(T, hkv * width + 8 * draw.randint(0, 3), dtype=x.dtype, device=dev)
+        wide[:, :hkv * width] = x.reshape(T, hkv * width).to(dev)
+        return wide[:, :hkv * width].view(T, hkv, width)
+    k = torch.zeros(n_slots, hkv, d, dtype=STORE[kind], device=dev)
+    v = torch.zeros(n_slots, hkv, dv, dtype=STORE[kind], device=dev)
+    ks = vs = None
+    if kind in ("fp8:row", "int8"):
+        ks, vs = torch.zeros(n_slots, hkv, device=dev), torch.zeros(n_slots, hkv, device=dev)
+    given = mult.to(dev) if torch.is_tensor(mult) else mult
+    if which == "both":
+        pk.write(on_device(keys), on_device(values), slots.to(dev), k, v, kind, ks, vs, multipliers=given)
+    elif which == "keys":
+        pk.write(on_device(keys), None, slots.to(dev), k, None, kind, ks, None, multipliers=given)
+    else:
+        pk.write(None, on_device(values), slots.to(dev), None, v, kind, None, vs, multipliers=given)
+    want = expected_pages(kind, keys, values, slots, n_slots, (mult[0], mult[1]) if torch.is_tensor(mult) else mult)
+    for at, (name, got, exact) in enumerate(zip(("keys", "values", "key scales", "value scales"), (k, v, ks, vs), want)):
+        if exact is None:
+            continue
+        if (which == "keys" and at in (1, 3)) or (which == "values" and at in (0, 2)):
+            exact = torch.zeros_like(exact)      # (the part not given stays untouched)
+        _same_bytes(got, exact, (seed, name))
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_appends_with_the_keys_rope_and_norm_fused_in_store_the_oracles_bytes(seed):
+    # rope() or rms_norm_rope() of the keys and then the append, against the oracle's two steps: magnitudes from 1e-20
+    # to 1e15, zeros of both signs, infinities, subnormals, NaNs, positions past the table, both pair styles, a scale
+    # on cos and sin, the weight in FP32 or in the inputs' type, values wider or narrower than the keys
+    from oracle import append as oracle_append
+    from tests.support import STORE, expected_pages
+    draw = random.Random(seed)
+    pk = kernels()
+    kind = draw.choice(KINDS)
+    d, dv = draw.choice([64, 128, 256]), draw.choice([64, 128, 256])
+    in_dtype = draw.choice([torch.float32, torch.bfloat16, torch.float16])
+    if kind == "fp16" and in_dtype == torch.bfloat16:
+        in_dtype = torch.float16
+    style = draw.choice(["half", "interleaved"])
+    normed = draw.random() < 0.6
+    g = torch.Generator().manual_seed(seed)
+    T, hkv, P = draw.choice([1, 7, 70, 300]), draw.choice([1, 2, 3, 8]), 500
+    mag = draw.choice([1e-20, 1e-3, 1.0, 30.0, 1e4, 1e15 if in_dtype != torch.float16 else 3e3])
+    keys = torch.randn(T, hkv, d, generator=g) * mag
+    flat = keys.view(-1)
+    for special in (0.0, -0.0, float("inf"), float("-inf"), 1e-40, -1e-40, 65504.0):
+        if draw.random() < 0.4:
+            flat[torch.randint(0, flat.numel(), (3,), generator=g)] = special
+    if draw.random() < 0.3:
+        flat[torch.randint(0, flat.numel(), (2,), generator=g)] = float("nan")
+    if draw.random() < 0.3:
+        keys[0] = 0
+    keys = keys.to(in_dtype)
+    values = torch.randn(T, hkv, dv, generator=g).to(in_dtype)
+    half = d // 2
+    angle = torch.arange(P, dtype=torch.float64)[:, None] / (10000.0 ** (torch.arange(half, dtype=torch.float64) / half))[None, :]
+    table = torch.cat([angle.cos(), angle.sin()], 1).float()
+    positions = torch.randint(-3, P + 10, (T,), generator=g)
+    n_slots = T + 9
+    slots = torch.randperm(n_slots, generator=g)[:T]
+    if T > 2:
+        slots[1] = -1
+    mult = (draw.choice([0.05, 1.0, 3.7e-3]), 0.07)
+    scale = draw.choice([1.0, 0.75, 1.3])
+    k = torch.zeros(n_slots, hkv, d, dtype=STORE[kind], device=dev)
+    v = torch.zeros(n_slots, hkv, dv, dtype=STORE[kind], device=dev)
+    ks = vs = None
+    if kind in ("fp8:row", "int8"):
+        ks, vs = torch.zeros(n_slots, hkv, device=dev), torch.zeros(n_slots, hkv, device=dev)
+    rope = (table.to(dev), positions.to(dev), style, scale)
+    if normed:
+        weight = torch.randn(d, generator=g) * 0.3 + 1
+        eps, offset = draw.choice([1e-6, 1e-5, 0.0 if mag >= 1e-3 else 1e-6]), draw.choice([0.0, 1.0])
+        weight = weight if draw.random() < 0.5 else weight.to(in_dtype)
+        pk.write(keys.to(dev), values.to(dev), slots.to(dev), k, v, kind, ks, vs, multipliers=mult, rope=rope,
+                 norm=(weight.to(dev), eps, offset))
+        turned = oracle_append.rms_norm_rope(keys, weight, eps, positions, table, offset, style, scale)
+    else:
+        pk.write(keys.to(dev), values.to(dev), slots.to(dev), k, v, kind, ks, vs, multipliers=mult, rope=rope)
+        turned = oracle_append.rope(keys, positions, table, style, scale)
+    want = expected_pages(kind, turned, values, slots, n_slots, mult)
+    for name, got, exact in zip(("keys", "values", "key scales", "value scales"), (k, v, ks, vs), want):
+        if exact is not None:
+            _same_bytes(got, exact, (seed, name))
