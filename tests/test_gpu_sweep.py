@@ -1,10 +1,10 @@
-"""Seeded sweeps over the geometry of the entry points (paged windows, block lists, prompt chunks, latent windows, index
-selection against float64; appends, plain and with the keys' rope and norm fused in, byte for byte): an attention case draws its page kind, head widths (keys' and
-values'), KV heads and GQA group, page size (powers of two and not), rows' lengths, window widths and live columns,
-sliding window, draft tree, piece and partitions from its seed, and is checked against float64 attention over the stored
-values (2e-2, as everywhere) with the split launch and the fused launch bit for bit the same. What the hand-picked
-shapes of the other files leave between them (a value row narrower than a wavefront under many partitions was one such
-gap) is met here by chance rather than by foresight."""
+"""Seeded sweeps over the geometry of the entry points: paged windows, block lists, prompt chunks, latent windows and
+index selection against float64; appends, plain and with the keys' rope and norm fused in, byte for byte. An attention
+case draws its page kind, head widths (keys' and values'), KV heads and GQA group, page size (powers of two and not),
+rows' lengths, window widths and live columns, sliding window, draft tree, piece and partitions from its seed, and is
+checked against float64 attention over the stored values (2e-2, as everywhere) with the split launch and the fused
+launch bit for bit the same. What the hand-picked shapes of the other files leave between them (a value row narrower
+than a wavefront under many partitions was one such gap) is met here by chance rather than by foresight."""
 import math
 import random
 
