@@ -29,6 +29,20 @@ def test_the_header_declares_the_entry_points():
         assert want in names
 
 
+def test_the_header_is_plain_c(tmp_path):
+    # what a cgo / JNI / ctypes binding includes: C99, pedantic, no warning; and the same text as C++
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    source = tmp_path / "use.c"
+    source.write_text('#include "crit_pkv.h"\nint main(void) { crit_pkv_attend_params p; (void)p; return CRIT_PKV_ABI_VERSION > 0 ? 0 : 1; }\n')
+    include = os.path.join(ROOT, "include")
+    for command in (["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror"], ["g++", "-std=c++17", "-Wall", "-Werror", "-x", "c++"]):
+        done = subprocess.run(command + ["-I", include, "-fsyntax-only", str(source)], capture_output=True, text=True)
+        assert done.returncode == 0, done.stderr
+
+
 def test_the_library_exports_every_declared_symbol(lib):
     for name in _declared():
         assert hasattr(lib, name), name
