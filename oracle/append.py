@@ -172,7 +172,8 @@ def rms_norm_rope(x, weight, eps, positions, table, offset=0.0, style="half", sc
     x32 = x.float()
     dim = x.shape[-1]
     mean = (sum_of_squares(x32).numpy() / np.float32(dim)).astype(np.float32)
-    r = (np.float32(1.0) / np.sqrt(mean + np.float32(eps), dtype=np.float32)).astype(np.float32)
+    with np.errstate(divide="ignore"):      # (a row of zeros under eps 0: 1 / 0 is the infinity torch's rsqrt gives)
+        r = (np.float32(1.0) / np.sqrt(mean + np.float32(eps), dtype=np.float32)).astype(np.float32)
     factor = weight.float()
     if offset:
         factor = factor + offset
