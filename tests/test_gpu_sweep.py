@@ -383,3 +383,52 @@ def test_appends_with_the_keys_rope_and_norm_fused_in_store_the_oracles_bytes(se
     for name, got, exact in zip(("keys", "values", "key scales", "value scales"), (k, v, ks, vs), want):
         if exact is not None:
             _same_bytes(got, exact, (seed, name))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_windows_at_the_launchs_limits(seed):
+    # launches of hundreds to 1,500 rows (past the rows a workgroup lists in LDS), windows of up to 64 columns under GQA
+    # groups of up to 32 (dozens of tiles a KV head), thousands of partitions of the shortest pieces, rows of no column
+    draw = random.Random(7000 + seed)
+    kind = draw.choice(KINDS)
+    d = draw.choice([64, 128, 128, 256, 32])
+    hkv, g = draw.choice([1, 2, 4, 8]), draw.choice([1, 4, 8, 16, 32])
+    g = min(g, 128 // hkv)
+    page = draw.choice([16, 16, 64, 256])
+    mode = ("many rows", "wide windows", "many partitions", "empty rows")[seed % 4]
+    if mode == "many rows":
+        lengths, cols = [draw.randint(1, 60) for _ in range(draw.choice([300, 700, 1500]))], draw.choice([1, 2])
+    elif mode == "wide windows":
+        lengths = [draw.choice([64, 100, 700, 3000]) + draw.randint(0, 30) for _ in range(draw.randint(1, 3))]
+        cols = draw.choice([16, 33, 64])
+    elif mode == "many partitions":
+        lengths, cols = [draw.choice([5000, 20000]) + draw.randint(0, 100) for _ in range(draw.randint(1, 2))], draw.choice([1, 3])
+    else:
+        lengths, cols = [draw.choice([1, 5, 300]) for _ in range(draw.randint(2, 6))], draw.choice([1, 4])
+    rows, starts, firsts, counts, tokens = [], [], [], [], 0
+    for s, n in enumerate(lengths):
+        c = 0 if mode == "empty rows" and draw.random() < 0.4 else draw.randint(1, min(cols, n))
+        rows.append(s), starts.append(tokens), firsts.append(n - max(c, 1)), counts.append(c)
+        tokens += cols
+    fused = draw.random() < 0.4
+    kw = dict(counts=torch.tensor(counts, dtype=torch.int32, device=dev), fused=fused)
+    if mode == "many partitions":
+        kw["partitions"], kw["piece"] = draw.choice([200, 1000, 5000]), draw.choice([16, 32, 64])
+    sliding = draw.choice([0, 0, 50])
+    if sliding:
+        kw["sliding"] = sliding
+    cache = Cache(kind, hkv, d, d, page, lengths, seed=seed)
+    q = rand_q(tokens, hkv * g, d, seed + 1000)
+    lse = torch.full((tokens, hkv * g), 7.0, device=dev)
+    out = cache.attend(q, rows, starts, firsts, cols, lse=lse, **kw)
+    other = cache.attend(q, rows, starts, firsts, cols, **{**kw, "fused": not fused})
+    for i, (start, count) in enumerate(zip(starts, counts)):
+        assert torch.equal(out[start:start + count], other[start:start + count]), (seed, i)
+        assert bool((lse[start + count:start + cols] == 7.0).all()), (seed, i, "tokens past the row's count are not written")
+    for i in (range(len(rows)) if len(rows) <= 8 else draw.sample(range(len(rows)), 8)):
+        s, start, first, count = rows[i], starts[i], firsts[i], counts[i]
+        if count:
+            some = sorted({0, count - 1, draw.randrange(count)})
+            want, want_lse = cache.want(q[start:start + count], s, first, count, sliding=sliding)
+            torch.testing.assert_close(out[start:start + count].double().cpu()[some], want[some], atol=ATOL, rtol=RTOL)
+            torch.testing.assert_close(lse[start:start + count].double().cpu()[some], want_lse[some], atol=1e-3, rtol=1e-4)
