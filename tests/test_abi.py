@@ -43,6 +43,37 @@ def test_the_header_is_plain_c(tmp_path):
         assert done.returncode == 0, done.stderr
 
 
+def test_a_c_program_links_the_library_and_is_refused_a_null_launch(tmp_path, lib):
+    # the boundary as a cgo / JNI stub meets it: a C99 program, the header, the shared library; no GPU is touched (the
+    # launch is refused for its NULL pointers before any HIP call)
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    from crit_amd.paged_kv_attention import _abi
+    library = next(path for path in _abi.candidates() if os.path.exists(path))
+    source = tmp_path / "use.c"
+    source.write_text("""#include <stdio.h>
+#include <string.h>
+#include "crit_pkv.h"
+int main(void) {
+    crit_pkv_attend_params p;
+    memset(&p, 0, sizeof p);
+    if (crit_pkv_abi_version() != CRIT_PKV_ABI_VERSION) return 2;
+    int code = crit_pkv_attend(&p, NULL);
+    printf("%d %s", code, crit_pkv_error(code));
+    return code == CRIT_PKV_E_NULL ? 0 : 3;
+}
+""")
+    where = os.path.dirname(library)
+    program = tmp_path / "use"
+    built = subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(source), "-o", str(program),
+                            "-L", where, "-lcrit_pkv", f"-Wl,-rpath,{where}", "-Wl,-rpath,/opt/rocm/lib"], capture_output=True, text=True)
+    assert built.returncode == 0, built.stderr
+    ran = subprocess.run([str(program)], capture_output=True, text=True, timeout=60)
+    assert ran.returncode == 0 and "NULL" in ran.stdout, (ran.returncode, ran.stdout, ran.stderr)
+
+
 def test_the_library_exports_every_declared_symbol(lib):
     for name in _declared():
         assert hasattr(lib, name), name
